@@ -1,0 +1,163 @@
+/*
+ * sswin3d — C ABI of the MI355X (gfx950) sparse window-attention operator library.
+ *
+ * Plain pointers and sizes only: every pointer marked "device" is a HIP device address,
+ * every other pointer is host memory.  `stream` is a hipStream_t passed as void*.
+ * No function allocates or frees device memory: scratch space is passed in by the caller
+ * (`ws`, `ws_bytes`, sized by the matching *_workspace_bytes query).  All kernels are
+ * enqueued on `stream`; functions that return a size to the host (documented below)
+ * synchronise that stream once, everything else is asynchronous.
+ *
+ * Return value: 0 on success, non-zero on error; sswin_last_error() then holds a message
+ * (thread-local).  Errors are argument errors detected on the host before any launch.
+ *
+ * Each entry point replaces one operator of the reference's pybind module `custom_ops`
+ * (sparse_swin/ops.cpp:7-18, declarations sparse_swin/ops.h:4-50); the citation beside
+ * each declaration is the reference function it stands in for.
+ */
+#ifndef SSWIN3D_H
+#define SSWIN3D_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* value dtypes */
+enum { SSWIN_F32 = 0, SSWIN_F16 = 1, SSWIN_BF16 = 2, SSWIN_F64 = 3 };
+/* key dtypes of sswin_unique_consecutive_indices */
+enum { SSWIN_I32 = 0, SSWIN_I64 = 1, SSWIN_I16 = 2, SSWIN_I8 = 3, SSWIN_U8 = 4 };
+/* block product kinds */
+enum { SSWIN_MUL_Q_K = 0, SSWIN_MUL_QK_V = 1 };
+enum { SSWIN_GRAD_RC_CR = 0, SSWIN_GRAD_RR_RC = 1, SSWIN_GRAD_CR_RR = 2 };
+enum { SSWIN_TRANSPOSE_RC = 0, SSWIN_TRANSPOSE_RR = 1 };
+
+const char* sswin_last_error(void);
+/* library ABI version, bumped on any signature change */
+int sswin_abi_version(void);
+
+/* ---- index operators -------------------------------------------------------------- */
+
+/* flatten_indices (sparse_swin/ops.cu:232-273, ops.h:38): wrapping int32 row-major hash of a
+ * contiguous [ndim, M] int32 index matrix; strides come from sizes[1:]. ndim <= 8.
+ * idx, out: device.  sizes: host, ndim entries. */
+int sswin_flatten_indices(const int32_t* idx, int ndim, int64_t M, const int32_t* sizes,
+                          int32_t* out, void* stream);
+
+/* sort_indices (sparse_swin/ops.cu:276-289, ops.h:39): stable ascending argsort of signed
+ * int32 keys.  keys, perm_out, ws: device. */
+size_t sswin_sort_indices_workspace_bytes(int64_t M);
+int sswin_sort_indices(const int32_t* keys, int64_t M, int32_t* perm_out, void* ws,
+                       size_t ws_bytes, void* stream);
+
+/* unique_consecutive_indices (sparse_swin/ops.cu:32-103, ops.h:41): 0-based rank of the run
+ * of equal consecutive keys each element belongs to.  keys, out, ws: device. */
+size_t sswin_unique_consecutive_workspace_bytes(int64_t M);
+int sswin_unique_consecutive_indices(const void* keys, int key_dtype, int64_t M, int32_t* out,
+                                     void* ws, size_t ws_bytes, void* stream);
+
+/* return_inverse (sparse_swin/ops.cu:718-730, ops.h:40): rank of x[i] among the distinct
+ * values of x, and the number of distinct values.  maxnum = -1 means max(x)+1 (costs one
+ * extra stream synchronisation).  Values of x must lie in [0, maxnum).
+ * x, out, ws: device.  count_out: host.  Synchronises `stream` to deliver count_out;
+ * pass count_out = NULL to stay asynchronous (only possible with maxnum >= 0).
+ * workspace query: pass the same maxnum you will pass to the call, or, for maxnum = -1,
+ * an upper bound of max(x)+1. */
+size_t sswin_return_inverse_workspace_bytes(int64_t M, int64_t maxnum_bound);
+int sswin_return_inverse(const int32_t* x, int64_t M, int64_t maxnum, int32_t* out,
+                         int64_t* count_out, void* ws, size_t ws_bytes, void* stream);
+
+/* qkv_sparse_indices (sparse_swin/ops.cu:206-227, 293-335, ops.h:23-28): from [N,2]
+ * (window, pos) voxel indices build the element-level COO indices of Q/V ([4,E], rows
+ * window, head, pos, channel) and of K^T ([4,E], rows window, head, channel, pos) in input
+ * voxel order, and the permutations that sort their row-major hashes (shapes
+ * {B,H,n,hd} and {B,H,hd,n}).  E = N*H*hd.  (window, pos) pairs must be distinct,
+ * window in [0,B), pos in [0,n).  The ordering is that of the exact (non-wrapping) hash.
+ * All array arguments: device.  Asynchronous. */
+size_t sswin_qkv_sparse_indices_workspace_bytes(int64_t N, int B, int n);
+int sswin_qkv_sparse_indices(const int32_t* indices, int64_t N, int B, int n, int H, int hd,
+                             int32_t* idx_qv, int32_t* sorted_qv, int32_t* idx_k,
+                             int32_t* sorted_k, void* ws, size_t ws_bytes, void* stream);
+
+/* ---- per-group offsets ("plan") ----------------------------------------------------- */
+
+/* Group structure of a coalesced 4-D COO operand whose last dimension is dense
+ * (sparse_swin/ops.cu:781-784, 836-841, 870-876: bincount_, the three cumsums and the
+ * .item() totals).  A group is a non-empty (index0, index1) = (window, head) pair;
+ * groups appear in ascending order.  `idx` is the [4, M] int32 index matrix of Q (for
+ * 'q_k') or V (for 'qk_v'); `inner` is its dense last-dimension extent (head dim), so
+ * that M / inner token rows exist.
+ *
+ * plan (device, int32, capacity 5 * g_cap entries, g_cap >= number of groups; M/inner is
+ * always enough) receives five rows of g_cap entries each:
+ *   row 0  c[g]           tokens of group g                  (the reference's `_c`)
+ *   row 1  row_start[g]   exclusive scan of c                (`idx_starts`)
+ *   row 2  sq_start[g]    exclusive scan of c*c              (`pos_starts`)
+ *   row 3  window[g]      index0 of the group
+ *   row 4  head[g]        index1 of the group
+ * totals_out (host, 4 x int64): {G, sum c, sum c*c, max c}.  Synchronises `stream`. */
+size_t sswin_plan_workspace_bytes(int64_t M, int inner);
+int sswin_plan_from_indices(const int32_t* idx, int64_t M, int inner, int32_t* plan,
+                            int64_t g_cap, int64_t* totals_out, void* ws, size_t ws_bytes,
+                            void* stream);
+
+/* Same three scans from a given `_c` (what the reference recomputes inside every
+ * matmul_grad / qkv_transpose call, sparse_swin/ops.cu:681, 697, 965-968, 986-989,
+ * 1007-1010).  c: device int32 [G].  scans: device int32 [2*G]: row 0 = exclusive scan of c,
+ * row 1 = exclusive scan of c*c.  Asynchronous. */
+size_t sswin_scan_counts_workspace_bytes(int64_t G);
+int sswin_scan_counts(const int32_t* c, int64_t G, int32_t* scans, void* ws, size_t ws_bytes,
+                      void* stream);
+
+/* ---- block products ------------------------------------------------------------------ */
+
+/* matmul_cuda_naive (sparse_swin/ops.cu:344-418, 788-943, 1034-1088, ops.h:4-12).
+ *  kind = SSWIN_MUL_Q_K : mat1 = Q values [sum c*C] (per group row-major [c x C]),
+ *                         mat2 = K^T values, per group row-major [C x c];
+ *                         out_val [sum c*c], out_idx [4, sum c*c] = (window, head, pos_i, pos_j)
+ *  kind = SSWIN_MUL_QK_V: mat1 = P values [sum c*c] (per group row-major [c x c]),
+ *                         mat2 = V values, per group row-major [c x C];
+ *                         out_val [sum c*C], out_idx [4, sum c*C] = (window, head, pos_i, channel)
+ * `plan`/`g_cap`/`G`/`c_max` come from sswin_plan_from_indices on `tok_idx`, the [4, M] index matrix
+ * of the operand that carries the token rows (Q for q_k, V for qk_v), M = sum c*C; its row 2
+ * provides pos.  All array arguments: device.  Asynchronous. */
+int sswin_block_matmul(int kind, int dtype, const void* mat1_v, const void* mat2_v,
+                       const int32_t* tok_idx, int64_t M, int C, const int32_t* plan,
+                       int64_t g_cap, int64_t G, int64_t c_max, void* out_val,
+                       int32_t* out_idx, int64_t out_nnz, void* stream);
+
+/* matmul_grad_cuda_naive (sparse_swin/ops.cu:422-515, 945-1031, 1092-1114, ops.h:15-21):
+ * value-only block products; both operands are read along their rows.
+ *  SSWIN_GRAD_RC_CR: out[c x c] = m1[c x C] . m2[c x C]^T
+ *  SSWIN_GRAD_RR_RC: out[c x C] = m1[c x c] . m2[C x c]^T
+ *  SSWIN_GRAD_CR_RR: out[C x c] = m1[C x c] . m2[c x c]^T
+ * c: device int32 [G]; scans: device, from sswin_scan_counts.  Asynchronous. */
+int sswin_block_matmul_grad(int kind, int dtype, const void* m1, const void* m2,
+                            const int32_t* c, const int32_t* scans, int64_t G, int C,
+                            void* out, void* stream);
+
+/* qkv_transpose (sparse_swin/ops.cu:518-557, 663-715, 1117-1132, ops.h:30-35):
+ *  SSWIN_TRANSPOSE_RC: per group [c x C] -> [C x c];  SSWIN_TRANSPOSE_RR: [c x c] -> transposed.
+ * Asynchronous. */
+int sswin_block_transpose(int kind, int dtype, const void* in, const int32_t* c,
+                          const int32_t* scans, int64_t G, int C, void* out, void* stream);
+
+/* ---- sparse row softmax ---------------------------------------------------------------- */
+
+/* softmax_last_dim_forward (sparse_swin/ops.cu:107-167, ops.h:43-45): rows are runs of equal
+ * consecutive ids in idx_row (sorted).  y = exp(v - max(0, rowmax)) / (rowsum + 1e-8).
+ * dtype SSWIN_F32 or SSWIN_F64.  Deterministic (no atomics).  Asynchronous. */
+int sswin_softmax_last_dim_forward(const int32_t* idx_row, const void* values, int dtype,
+                                   int64_t A, void* out, void* stream);
+
+/* softmax_last_dim_backward (sparse_swin/ops.cu:169-194, ops.h:47-50):
+ * gx = g*y - y * sum_row(g*y).  Asynchronous. */
+int sswin_softmax_last_dim_backward(const int32_t* idx_row, const void* y, const void* grad,
+                                    int dtype, int64_t A, void* out, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SSWIN3D_H */

@@ -1,0 +1,71 @@
+"""ctypes binding of ``libsswin3d.so`` (declarations in ``include/sswin3d.h``).
+
+The library is the only compute path of this package.  If it is missing, loading raises:
+there is no CPU or PyTorch fallback.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "libsswin3d.so")
+
+_vp, _i64, _i32, _sz = C.c_void_p, C.c_int64, C.c_int, C.c_size_t
+
+# name -> (restype, argtypes); mirrors include/sswin3d.h one to one
+SIGNATURES = {
+    "sswin_last_error": (C.c_char_p, []),
+    "sswin_abi_version": (_i32, []),
+    "sswin_flatten_indices": (_i32, [_vp, _i32, _i64, _vp, _vp, _vp]),
+    "sswin_sort_indices_workspace_bytes": (_sz, [_i64]),
+    "sswin_sort_indices": (_i32, [_vp, _i64, _vp, _vp, _sz, _vp]),
+    "sswin_unique_consecutive_workspace_bytes": (_sz, [_i64]),
+    "sswin_unique_consecutive_indices": (_i32, [_vp, _i32, _i64, _vp, _vp, _sz, _vp]),
+    "sswin_return_inverse_workspace_bytes": (_sz, [_i64, _i64]),
+    "sswin_return_inverse": (_i32, [_vp, _i64, _i64, _vp, _vp, _vp, _sz, _vp]),
+    "sswin_qkv_sparse_indices_workspace_bytes": (_sz, [_i64, _i32, _i32]),
+    "sswin_qkv_sparse_indices": (_i32, [_vp, _i64, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "sswin_plan_workspace_bytes": (_sz, [_i64, _i32]),
+    "sswin_plan_from_indices": (_i32, [_vp, _i64, _i32, _vp, _i64, _vp, _vp, _sz, _vp]),
+    "sswin_scan_counts_workspace_bytes": (_sz, [_i64]),
+    "sswin_scan_counts": (_i32, [_vp, _i64, _vp, _vp, _sz, _vp]),
+    "sswin_block_matmul": (_i32, [_i32, _i32, _vp, _vp, _vp, _i64, _i32, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp]),
+    "sswin_block_matmul_grad": (_i32, [_i32, _i32, _vp, _vp, _vp, _vp, _i64, _i32, _vp, _vp]),
+    "sswin_block_transpose": (_i32, [_i32, _i32, _vp, _vp, _vp, _i64, _i32, _vp, _vp]),
+    "sswin_softmax_last_dim_forward": (_i32, [_vp, _vp, _i32, _i64, _vp, _vp]),
+    "sswin_softmax_last_dim_backward": (_i32, [_vp, _vp, _vp, _i32, _i64, _vp, _vp]),
+}
+
+ABI_VERSION = 1
+_lib = None
+
+
+class LibraryMissing(RuntimeError):
+    pass
+
+
+def load():
+    """Load the HIP library once.  Raises :class:`LibraryMissing` if it has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise LibraryMissing(
+            f"{LIB_PATH} not found: build it with `python -m sparseswin3d_amd.build` "
+            "(there is no CPU fallback for the sparse window-attention operators)")
+    lib = C.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)          # AttributeError here means header and library disagree
+        fn.restype = res
+        fn.argtypes = args
+    if lib.sswin_abi_version() != ABI_VERSION:
+        raise RuntimeError(f"libsswin3d ABI {lib.sswin_abi_version()} != binding ABI {ABI_VERSION}; rebuild")
+    _lib = lib
+    return lib
+
+
+def check(status: int):
+    """Turn a non-zero status into RuntimeError carrying the library's message."""
+    if status != 0:
+        raise RuntimeError(load().sswin_last_error().decode("utf-8", "replace"))

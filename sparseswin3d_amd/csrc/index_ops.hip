@@ -1,0 +1,436 @@
+// Integer index operators: flatten_indices, sort_indices, unique_consecutive_indices,
+// return_inverse, qkv_sparse_indices.  All of them are HBM-bound integer work; the kernels
+// are laid out for coalesced 64-lane accesses and use no floating point.
+#include <cstring>
+#include <rocprim/device/device_radix_sort.hpp>
+#include <rocprim/iterator/counting_iterator.hpp>
+
+#include "scan.hpp"
+#include "sswin_common.hpp"
+
+namespace sswin {
+
+// thread-local error buffer lives here (one definition for the whole library)
+char* error_buffer() {
+    static thread_local char buf[512] = {0};
+    return buf;
+}
+int fail(const char* fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(error_buffer(), 512, fmt, ap);
+    va_end(ap);
+    return 1;
+}
+
+// ------------------------------------------------------------------------------------------
+// flatten_indices
+// ------------------------------------------------------------------------------------------
+struct Strides {
+    uint32_t s[8];
+};
+
+template <int NDIM>
+__global__ __launch_bounds__(256) void flatten_kernel(const int32_t* __restrict__ idx, int64_t M,
+                                                      Strides st, int32_t* __restrict__ out) {
+    // four consecutive columns per thread; vector path when the row pitch keeps 16-byte alignment
+    const int64_t m4 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (m4 >= M) return;
+    if ((M & 3) == 0 && m4 + 3 < M) {
+        uint32_t h0 = 0, h1 = 0, h2 = 0, h3 = 0;
+#pragma unroll
+        for (int i = 0; i < NDIM; ++i) {
+            const int4 v = *reinterpret_cast<const int4*>(idx + (int64_t)i * M + m4);
+            h0 += (uint32_t)v.x * st.s[i];
+            h1 += (uint32_t)v.y * st.s[i];
+            h2 += (uint32_t)v.z * st.s[i];
+            h3 += (uint32_t)v.w * st.s[i];
+        }
+        *reinterpret_cast<int4*>(out + m4) = make_int4((int)h0, (int)h1, (int)h2, (int)h3);
+    } else {
+        for (int64_t m = m4; m < M && m < m4 + 4; ++m) {
+            uint32_t h = 0;
+#pragma unroll
+            for (int i = 0; i < NDIM; ++i) h += (uint32_t)idx[(int64_t)i * M + m] * st.s[i];
+            out[m] = (int)h;
+        }
+    }
+}
+
+template <int NDIM>
+static void launch_flatten(const int32_t* idx, int64_t M, const Strides& st, int32_t* out,
+                           hipStream_t s) {
+    const int64_t threads = (M + 3) / 4;
+    hipLaunchKernelGGL(flatten_kernel<NDIM>, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s,
+                       idx, M, st, out);
+}
+
+// ------------------------------------------------------------------------------------------
+// unique_consecutive_indices: inclusive scan of "differs from predecessor" flags
+// ------------------------------------------------------------------------------------------
+template <typename K>
+struct RunFlagLoad {
+    const K* x;
+    __device__ int operator()(int64_t i) const { return (i > 0 && x[i] != x[i - 1]) ? 1 : 0; }
+};
+struct InclusiveStore {
+    int32_t* out;
+    __device__ void operator()(int64_t i, int ex, int item) const { out[i] = ex + item; }
+};
+
+template <typename K>
+static int unique_consecutive_t(const void* keys, int64_t M, int32_t* out, int32_t* tile_sums,
+                                hipStream_t s) {
+    RunFlagLoad<K> ld{static_cast<const K*>(keys)};
+    InclusiveStore st{out};
+    return device_exclusive_scan<int32_t>(ld, st, M, tile_sums, (int32_t*)nullptr, s, "unique_consecutive");
+}
+
+// ------------------------------------------------------------------------------------------
+// presence bitmap helpers (return_inverse, qkv_sparse_indices)
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void fill_u32_kernel(uint32_t* __restrict__ p, int64_t n, uint32_t v) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) p[i] = v;
+}
+
+__global__ __launch_bounds__(256) void set_bits_kernel(const int32_t* __restrict__ x, int64_t M,
+                                                       uint32_t* __restrict__ bits) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < M) {
+        const uint32_t v = (uint32_t)x[i];
+        atomicOr(&bits[v >> 5], 1u << (v & 31));
+    }
+}
+
+// (window, pos) pairs -> bit window*n + pos
+__global__ __launch_bounds__(256) void set_bits_pairs_kernel(const int32_t* __restrict__ ind, int64_t N,
+                                                             int n, uint32_t* __restrict__ bits) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < N) {
+        const int2 wp = *reinterpret_cast<const int2*>(ind + 2 * i);
+        const uint64_t v = (uint64_t)(uint32_t)wp.x * (uint32_t)n + (uint32_t)wp.y;
+        atomicOr(&bits[v >> 5], 1u << (v & 31));
+    }
+}
+
+struct PopcLoad {
+    const uint32_t* bits;
+    __device__ int operator()(int64_t i) const { return __popc(bits[i]); }
+};
+struct ExclusiveStore {
+    int32_t* out;
+    __device__ void operator()(int64_t i, int ex, int) const { out[i] = ex; }
+};
+
+__device__ __forceinline__ int rank_of_bit(const uint32_t* __restrict__ bits,
+                                           const int32_t* __restrict__ word_prefix, uint64_t v) {
+    const uint64_t w = v >> 5;
+    const uint32_t below = bits[w] & ((1u << (v & 31)) - 1u);
+    return word_prefix[w] + __popc(below);
+}
+
+__global__ __launch_bounds__(256) void rank_lookup_kernel(const int32_t* __restrict__ x, int64_t M,
+                                                          const uint32_t* __restrict__ bits,
+                                                          const int32_t* __restrict__ word_prefix,
+                                                          int32_t* __restrict__ out) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < M) out[i] = rank_of_bit(bits, word_prefix, (uint32_t)x[i]);
+}
+
+// max of int32 array into a single device int (one atomicMax per block)
+__global__ __launch_bounds__(256) void max_i32_kernel(const int32_t* __restrict__ x, int64_t M,
+                                                      int32_t* __restrict__ out) {
+    __shared__ int lds[4];
+    int m = INT32_MIN;
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < M; i += (int64_t)gridDim.x * 256)
+        m = max(m, x[i]);
+    m = wave_max_i32(m);
+    if ((threadIdx.x & 63) == 0) lds[threadIdx.x >> 6] = m;
+    __syncthreads();
+    if (threadIdx.x == 0) atomicMax(out, max(max(lds[0], lds[1]), max(lds[2], lds[3])));
+}
+
+// ------------------------------------------------------------------------------------------
+// qkv_sparse_indices
+// ------------------------------------------------------------------------------------------
+// Per voxel: rank r in (window, pos) order, and for rank r the source voxel, the rank T of the
+// first token of its window and the token count c of its window.
+__global__ __launch_bounds__(256) void voxel_rank_kernel(const int32_t* __restrict__ ind, int64_t N, int n,
+                                                         const uint32_t* __restrict__ bits,
+                                                         const int32_t* __restrict__ word_prefix,
+                                                         int32_t* __restrict__ order,   // [N] voxel of rank r
+                                                         int32_t* __restrict__ win_T,   // [N] by rank
+                                                         int32_t* __restrict__ win_c) { // [N] by rank
+    const int64_t v = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (v >= N) return;
+    const int2 wp = *reinterpret_cast<const int2*>(ind + 2 * v);
+    const uint64_t first = (uint64_t)(uint32_t)wp.x * (uint32_t)n;
+    const int r = rank_of_bit(bits, word_prefix, first + (uint32_t)wp.y);
+    const int T = rank_of_bit(bits, word_prefix, first);
+    const int Tn = rank_of_bit(bits, word_prefix, first + (uint32_t)n);  // bitmap has a padding word
+    order[r] = (int32_t)v;
+    win_T[r] = T;
+    win_c[r] = Tn - T;
+}
+
+// Element-level COO rows in input voxel order; four consecutive channels per thread.
+// idx_qv rows: window, head, pos, channel.  idx_k rows: window, head, channel, pos.
+__global__ __launch_bounds__(256) void expand_coo_kernel(const int32_t* __restrict__ ind, int64_t E,
+                                                         int H, int hd, int32_t* __restrict__ idx_qv,
+                                                         int32_t* __restrict__ idx_k) {
+    const int64_t e = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (e >= E) return;
+    const int D = H * hd;
+    const int64_t v = e / D;
+    const int local = (int)(e - v * D);
+    const int h = local / hd, ch = local - h * hd;
+    const int2 wp = *reinterpret_cast<const int2*>(ind + 2 * v);
+    const int4 w4 = make_int4(wp.x, wp.x, wp.x, wp.x);
+    const int4 h4 = make_int4(h, h, h, h);
+    const int4 p4 = make_int4(wp.y, wp.y, wp.y, wp.y);
+    const int4 c4 = make_int4(ch, ch + 1, ch + 2, ch + 3);
+    *reinterpret_cast<int4*>(idx_qv + e) = w4;
+    *reinterpret_cast<int4*>(idx_qv + E + e) = h4;
+    *reinterpret_cast<int4*>(idx_qv + 2 * E + e) = p4;
+    *reinterpret_cast<int4*>(idx_qv + 3 * E + e) = c4;
+    *reinterpret_cast<int4*>(idx_k + e) = w4;
+    *reinterpret_cast<int4*>(idx_k + E + e) = h4;
+    *reinterpret_cast<int4*>(idx_k + 2 * E + e) = c4;
+    *reinterpret_cast<int4*>(idx_k + 3 * E + e) = p4;
+}
+
+// sorted_qv: destination slot hd*(H*T + h*c + i) + ch holds source element v*D + h*hd + ch.
+// One thread per (rank, head, channel quad): a 16-byte store, 128 contiguous bytes per hd=32 row.
+__global__ __launch_bounds__(256) void sorted_qv_kernel(const int32_t* __restrict__ order,
+                                                        const int32_t* __restrict__ win_T,
+                                                        const int32_t* __restrict__ win_c, int64_t N,
+                                                        int H, int hd, int32_t* __restrict__ sorted_qv) {
+    const int q = hd >> 2;                                  // channel quads per head
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const int64_t total = N * H * q;
+    if (t >= total) return;
+    const int cq = (int)(t % q);
+    const int64_t rh = t / q;
+    const int h = (int)(rh % H);
+    const int64_t r = rh / H;
+    const int T = win_T[r], c = win_c[r];
+    const int i = (int)(r - T);
+    const int64_t dst = (int64_t)hd * ((int64_t)H * T + (int64_t)h * c + i) + cq * 4;
+    const int src = (int)((int64_t)order[r] * H * hd + h * hd + cq * 4);
+    *reinterpret_cast<int4*>(sorted_qv + dst) = make_int4(src, src + 1, src + 2, src + 3);
+}
+
+// sorted_k: destination slot hd*(H*T + h*c) + ch*c + i.  Lanes run over consecutive ranks, so
+// for a fixed (head, channel) a wave writes runs of c contiguous ints per window.
+__global__ __launch_bounds__(256) void sorted_k_kernel(const int32_t* __restrict__ order,
+                                                       const int32_t* __restrict__ win_T,
+                                                       const int32_t* __restrict__ win_c, int64_t N,
+                                                       int H, int hd, int32_t* __restrict__ sorted_k) {
+    const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (r >= N) return;
+    const int T = win_T[r], c = win_c[r];
+    const int i = (int)(r - T);
+    const int h = blockIdx.y;
+    const int64_t base = (int64_t)hd * ((int64_t)H * T + (int64_t)h * c) + i;
+    const int src = (int)((int64_t)order[r] * H * hd + h * hd);
+    for (int ch = 0; ch < hd; ++ch) sorted_k[base + (int64_t)ch * c] = src + ch;
+}
+
+}  // namespace sswin
+
+using namespace sswin;
+
+// ==========================================================================================
+// C ABI
+// ==========================================================================================
+extern "C" {
+
+const char* sswin_last_error(void) { return error_buffer(); }
+int sswin_abi_version(void) { return 1; }
+
+int sswin_flatten_indices(const int32_t* idx, int ndim, int64_t M, const int32_t* sizes, int32_t* out,
+                          void* stream) {
+    SSWIN_CHECK(ndim >= 1 && ndim <= 8, "flatten_indices: ndim %d not in [1, 8]", ndim);
+    SSWIN_CHECK(M >= 0, "flatten_indices: negative column count");
+    if (M == 0) return 0;
+    SSWIN_CHECK(idx && out && sizes, "flatten_indices: null pointer");
+    Strides st;
+    st.s[ndim - 1] = 1u;
+    for (int i = ndim - 2; i >= 0; --i) st.s[i] = st.s[i + 1] * (uint32_t)sizes[i + 1];
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (ndim) {
+        case 1: launch_flatten<1>(idx, M, st, out, s); break;
+        case 2: launch_flatten<2>(idx, M, st, out, s); break;
+        case 3: launch_flatten<3>(idx, M, st, out, s); break;
+        case 4: launch_flatten<4>(idx, M, st, out, s); break;
+        case 5: launch_flatten<5>(idx, M, st, out, s); break;
+        case 6: launch_flatten<6>(idx, M, st, out, s); break;
+        case 7: launch_flatten<7>(idx, M, st, out, s); break;
+        default: launch_flatten<8>(idx, M, st, out, s); break;
+    }
+    return launch_ok("flatten_indices");
+}
+
+// ---- sort_indices ---------------------------------------------------------------------------
+size_t sswin_sort_indices_workspace_bytes(int64_t M) {
+    if (M <= 0) return 256;
+    size_t tmp = 0;
+    rocprim::radix_sort_pairs(nullptr, tmp, (const int32_t*)nullptr, (int32_t*)nullptr,
+                              rocprim::counting_iterator<int32_t>(0), (int32_t*)nullptr, (size_t)M, 0, 32,
+                              (hipStream_t)0);
+    return align_up(tmp, 256) + align_up((size_t)M * sizeof(int32_t), 256) + 256;
+}
+
+int sswin_sort_indices(const int32_t* keys, int64_t M, int32_t* perm_out, void* ws, size_t ws_bytes,
+                       void* stream) {
+    SSWIN_CHECK(M >= 0 && M < (int64_t)INT32_MAX, "sort_indices: element count %lld out of range", (long long)M);
+    if (M == 0) return 0;
+    SSWIN_CHECK(keys && perm_out && ws, "sort_indices: null pointer");
+    SSWIN_CHECK(ws_bytes >= sswin_sort_indices_workspace_bytes(M), "sort_indices: workspace too small");
+    Carver cv(ws, ws_bytes);
+    int32_t* keys_sorted = cv.take<int32_t>((size_t)M);
+    size_t tmp = 0;
+    rocprim::radix_sort_pairs(nullptr, tmp, keys, keys_sorted, rocprim::counting_iterator<int32_t>(0),
+                              perm_out, (size_t)M, 0, 32, (hipStream_t)0);
+    void* tmp_ptr = cv.take<char>(tmp);
+    SSWIN_CHECK(cv.ok(), "sort_indices: workspace too small");
+    SSWIN_HIP(rocprim::radix_sort_pairs(tmp_ptr, tmp, keys, keys_sorted,
+                                        rocprim::counting_iterator<int32_t>(0), perm_out, (size_t)M, 0, 32,
+                                        static_cast<hipStream_t>(stream)));
+    return 0;
+}
+
+// ---- unique_consecutive_indices ---------------------------------------------------------------
+size_t sswin_unique_consecutive_workspace_bytes(int64_t M) {
+    return align_up((size_t)(scan_num_tiles(M > 0 ? M : 1)) * sizeof(int32_t), 256) + 256;
+}
+
+int sswin_unique_consecutive_indices(const void* keys, int key_dtype, int64_t M, int32_t* out, void* ws,
+                                     size_t ws_bytes, void* stream) {
+    SSWIN_CHECK(M >= 0, "unique_consecutive_indices: negative length");
+    if (M == 0) return 0;
+    SSWIN_CHECK(keys && out && ws, "unique_consecutive_indices: null pointer");
+    SSWIN_CHECK(ws_bytes >= sswin_unique_consecutive_workspace_bytes(M),
+                "unique_consecutive_indices: workspace too small");
+    Carver cv(ws, ws_bytes);
+    int32_t* tile_sums = cv.take<int32_t>((size_t)scan_num_tiles(M));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (key_dtype) {
+        case SSWIN_I32: return unique_consecutive_t<int32_t>(keys, M, out, tile_sums, s);
+        case SSWIN_I64: return unique_consecutive_t<int64_t>(keys, M, out, tile_sums, s);
+        case SSWIN_I16: return unique_consecutive_t<int16_t>(keys, M, out, tile_sums, s);
+        case SSWIN_I8: return unique_consecutive_t<int8_t>(keys, M, out, tile_sums, s);
+        case SSWIN_U8: return unique_consecutive_t<uint8_t>(keys, M, out, tile_sums, s);
+        default: return fail("unique_consecutive_indices: unsupported key dtype %d", key_dtype);
+    }
+}
+
+// ---- return_inverse ---------------------------------------------------------------------------
+static size_t bitmap_words(int64_t nbits) { return (size_t)((nbits + 31) / 32) + 1; }  // +1 padding word
+
+size_t sswin_return_inverse_workspace_bytes(int64_t M, int64_t maxnum_bound) {
+    (void)M;
+    if (maxnum_bound < 1) maxnum_bound = 1;
+    const size_t words = bitmap_words(maxnum_bound);
+    return align_up(words * 4, 256) * 2 + align_up((size_t)scan_num_tiles((int64_t)words) * 4, 256) + 1024;
+}
+
+int sswin_return_inverse(const int32_t* x, int64_t M, int64_t maxnum, int32_t* out, int64_t* count_out,
+                         void* ws, size_t ws_bytes, void* stream) {
+    SSWIN_CHECK(M >= 0, "return_inverse: negative length");
+    if (M == 0) {
+        if (count_out) *count_out = 0;
+        return 0;
+    }
+    SSWIN_CHECK(x && out && ws, "return_inverse: null pointer");
+    SSWIN_CHECK(maxnum >= -1, "return_inverse: maxnum %lld invalid", (long long)maxnum);
+    SSWIN_CHECK(maxnum != -1 || count_out, "return_inverse: maxnum = -1 needs count_out (synchronous call)");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    Carver cv(ws, ws_bytes);
+    int32_t* total_dev = cv.take<int32_t>(2);   // [0] distinct count, [1] max
+    SSWIN_CHECK(cv.ok(), "return_inverse: workspace too small");
+    if (maxnum == -1) {
+        int32_t* max_dev = total_dev + 1;
+        hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(256), 0, s, reinterpret_cast<uint32_t*>(max_dev),
+                           (int64_t)1, (uint32_t)INT32_MIN);
+        const unsigned blocks = (unsigned)std::min<int64_t>((M + 255) / 256, 2048);
+        hipLaunchKernelGGL(max_i32_kernel, dim3(blocks), dim3(256), 0, s, x, M, max_dev);
+        int32_t mx = 0;
+        SSWIN_HIP(hipMemcpyAsync(&mx, max_dev, sizeof(int32_t), hipMemcpyDeviceToHost, s));
+        SSWIN_HIP(hipStreamSynchronize(s));
+        SSWIN_CHECK(mx >= 0, "return_inverse: all values negative");
+        maxnum = (int64_t)mx + 1;
+    }
+    const size_t words = bitmap_words(maxnum);
+    uint32_t* bits = cv.take<uint32_t>(words);
+    int32_t* word_prefix = cv.take<int32_t>(words);
+    int32_t* tile_sums = cv.take<int32_t>((size_t)scan_num_tiles((int64_t)words));
+    SSWIN_CHECK(cv.ok(), "return_inverse: workspace too small for maxnum %lld", (long long)maxnum);
+    const unsigned fill_blocks = (unsigned)std::min<size_t>((words + 255) / 256, 4096);
+    hipLaunchKernelGGL(fill_u32_kernel, dim3(fill_blocks), dim3(256), 0, s, bits, (int64_t)words, 0u);
+    hipLaunchKernelGGL(set_bits_kernel, dim3((unsigned)((M + 255) / 256)), dim3(256), 0, s, x, M, bits);
+    PopcLoad ld{bits};
+    ExclusiveStore st{word_prefix};
+    if (device_exclusive_scan<int32_t>(ld, st, (int64_t)words, tile_sums, total_dev, s, "return_inverse scan")) return 1;
+    hipLaunchKernelGGL(rank_lookup_kernel, dim3((unsigned)((M + 255) / 256)), dim3(256), 0, s, x, M, bits,
+                       word_prefix, out);
+    if (launch_ok("return_inverse")) return 1;
+    if (count_out) {
+        int32_t cnt = 0;
+        SSWIN_HIP(hipMemcpyAsync(&cnt, total_dev, sizeof(int32_t), hipMemcpyDeviceToHost, s));
+        SSWIN_HIP(hipStreamSynchronize(s));
+        *count_out = cnt;
+    }
+    return 0;
+}
+
+// ---- qkv_sparse_indices -----------------------------------------------------------------------
+size_t sswin_qkv_sparse_indices_workspace_bytes(int64_t N, int B, int n) {
+    const size_t words = bitmap_words((int64_t)B * n + n);
+    return align_up(words * 4, 256) * 2 + align_up((size_t)scan_num_tiles((int64_t)words) * 4, 256) +
+           3 * align_up((size_t)(N > 0 ? N : 1) * 4, 256) + 1024;
+}
+
+int sswin_qkv_sparse_indices(const int32_t* indices, int64_t N, int B, int n, int H, int hd,
+                             int32_t* idx_qv, int32_t* sorted_qv, int32_t* idx_k, int32_t* sorted_k,
+                             void* ws, size_t ws_bytes, void* stream) {
+    SSWIN_CHECK(N >= 0 && B > 0 && n > 0 && H > 0 && hd > 0, "qkv_sparse_indices: bad sizes");
+    SSWIN_CHECK(hd % 4 == 0, "qkv_sparse_indices: head dim %d must be a multiple of 4", hd);
+    const int64_t E = N * H * hd;
+    SSWIN_CHECK(E < (int64_t)INT32_MAX, "qkv_sparse_indices: N*H*hd = %lld does not fit int32", (long long)E);
+    SSWIN_CHECK((int64_t)B * n + n < ((int64_t)1 << 36), "qkv_sparse_indices: B*n too large");
+    if (N == 0) return 0;
+    SSWIN_CHECK(indices && idx_qv && sorted_qv && idx_k && sorted_k && ws, "qkv_sparse_indices: null pointer");
+    SSWIN_CHECK(ws_bytes >= sswin_qkv_sparse_indices_workspace_bytes(N, B, n),
+                "qkv_sparse_indices: workspace too small");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    Carver cv(ws, ws_bytes);
+    const size_t words = bitmap_words((int64_t)B * n + n);
+    uint32_t* bits = cv.take<uint32_t>(words);
+    int32_t* word_prefix = cv.take<int32_t>(words);
+    int32_t* tile_sums = cv.take<int32_t>((size_t)scan_num_tiles((int64_t)words));
+    int32_t* order = cv.take<int32_t>((size_t)N);
+    int32_t* win_T = cv.take<int32_t>((size_t)N);
+    int32_t* win_c = cv.take<int32_t>((size_t)N);
+    SSWIN_CHECK(cv.ok(), "qkv_sparse_indices: workspace too small");
+
+    const unsigned fill_blocks = (unsigned)std::min<size_t>((words + 255) / 256, 4096);
+    hipLaunchKernelGGL(fill_u32_kernel, dim3(fill_blocks), dim3(256), 0, s, bits, (int64_t)words, 0u);
+    const unsigned nb = (unsigned)((N + 255) / 256);
+    hipLaunchKernelGGL(set_bits_pairs_kernel, dim3(nb), dim3(256), 0, s, indices, N, n, bits);
+    PopcLoad ld{bits};
+    ExclusiveStore st{word_prefix};
+    if (device_exclusive_scan<int32_t>(ld, st, (int64_t)words, tile_sums, (int32_t*)nullptr, s, "qkv_sparse_indices scan")) return 1;
+    hipLaunchKernelGGL(voxel_rank_kernel, dim3(nb), dim3(256), 0, s, indices, N, n, bits, word_prefix, order,
+                       win_T, win_c);
+    hipLaunchKernelGGL(expand_coo_kernel, dim3((unsigned)((E / 4 + 255) / 256)), dim3(256), 0, s, indices, E, H,
+                       hd, idx_qv, idx_k);
+    const int64_t qv_threads = N * H * (hd / 4);
+    hipLaunchKernelGGL(sorted_qv_kernel, dim3((unsigned)((qv_threads + 255) / 256)), dim3(256), 0, s, order,
+                       win_T, win_c, N, H, hd, sorted_qv);
+    hipLaunchKernelGGL(sorted_k_kernel, dim3(nb, (unsigned)H), dim3(256), 0, s, order, win_T, win_c, N, H, hd,
+                       sorted_k);
+    return launch_ok("qkv_sparse_indices");
+}
+
+}  // extern "C"

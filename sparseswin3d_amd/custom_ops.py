@@ -1,0 +1,359 @@
+"""Drop-in replacement of the reference's ``custom_ops`` extension module.
+
+Same ten operator names, positional signatures, return types and error behaviour as the
+pybind module built from ``sparse_swin/ops.cpp:7-18`` / ``sparse_swin/ops.h:4-50`` of the
+reference.  Every operator runs hand-written HIP kernels from ``libsswin3d.so`` on the
+current HIP stream of the tensors' device; torch is used only to allocate outputs and
+scratch space and to hand over device pointers and the stream.  There is no CPU fallback:
+tensors that are not on a GPU, or a missing library, raise ``RuntimeError``.
+
+Use in the reference's ``swin3d_base.py`` by replacing its JIT ``load(...)`` call with
+``from sparseswin3d_amd import custom_ops as ops``.
+"""
+from __future__ import annotations
+
+import ctypes as C
+from collections import OrderedDict
+
+import torch
+
+from . import _lib
+
+_DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2, torch.float64: 3}
+_KEY_CODE = {torch.int32: 0, torch.int64: 1, torch.int16: 2, torch.int8: 3, torch.uint8: 4}
+_MUL = {"q_k": 0, "qk_v": 1}
+_GRAD = {"rc_cr": 0, "rr_rc": 1, "cr_rr": 2}
+_TRANSPOSE = {"rc": 0, "rr": 1}
+
+
+def _check(cond, msg):
+    if not cond:
+        raise RuntimeError(msg)
+
+
+def _dev(*tensors):
+    d = tensors[0].device
+    _check(d.type == "cuda", "sparseswin3d_amd.custom_ops runs on the GPU only; got a tensor on "
+                             f"'{d}'. There is no CPU fallback.")
+    for t in tensors[1:]:
+        _check(t.device == d, f"tensors on different devices: {d} and {t.device}")
+    return d
+
+
+def _stream(device):
+    return C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+
+
+def _ptr(t):
+    return C.c_void_p(t.data_ptr())
+
+
+def _ws(nbytes, device):
+    return torch.empty(int(nbytes), dtype=torch.uint8, device=device)
+
+
+def _host_i32(values):
+    arr = (C.c_int32 * len(values))(*[int(v) for v in values])
+    return arr
+
+
+# --------------------------------------------------------------------------------------- #
+# index operators
+# --------------------------------------------------------------------------------------- #
+def flatten_indices(indices, sizes):
+    """Wrapping int32 row-major hash of ``indices[:len(sizes)]`` (reference ops.cu:232-273)."""
+    lib = _lib.load()
+    d = _dev(indices)
+    _check(indices.dim() == 2, "flatten_indices: indices must be 2-D [ndim, nnz]")
+    _check(indices.dtype == torch.int32, f"flatten_indices: indices must be int32, got {indices.dtype}")
+    ndim = len(sizes)
+    _check(1 <= ndim <= indices.shape[0], "flatten_indices: len(sizes) exceeds the number of index rows")
+    indices = indices.contiguous()
+    m = indices.shape[1]
+    out = torch.empty(m, dtype=torch.int32, device=d)
+    with torch.cuda.device(d):
+        _lib.check(lib.sswin_flatten_indices(_ptr(indices), ndim, m, _host_i32(sizes), _ptr(out), _stream(d)))
+    return out
+
+
+def sort_indices(flattened_indices):
+    """Stable ascending argsort of int32 keys, int32 result (reference ops.cu:276-289)."""
+    lib = _lib.load()
+    d = _dev(flattened_indices)
+    _check(flattened_indices.dtype == torch.int32, "sort_indices: keys must be int32")
+    keys = flattened_indices.contiguous().view(-1)
+    m = keys.numel()
+    out = torch.empty(m, dtype=torch.int32, device=d)
+    nbytes = lib.sswin_sort_indices_workspace_bytes(m)
+    ws = _ws(nbytes, d)
+    with torch.cuda.device(d):
+        _lib.check(lib.sswin_sort_indices(_ptr(keys), m, _ptr(out), _ptr(ws), nbytes, _stream(d)))
+    return out
+
+
+def unique_consecutive_indices(nums):
+    """Rank of the run of equal consecutive values each element belongs to (ops.cu:32-103)."""
+    lib = _lib.load()
+    d = _dev(nums)
+    _check(nums.dim() == 1, "unique_consecutive_indices: expected a 1-D tensor")
+    _check(nums.dtype in _KEY_CODE, f"unique_consecutive_indices: unsupported dtype {nums.dtype}")
+    nums = nums.contiguous()
+    m = nums.numel()
+    out = torch.empty(m, dtype=torch.int32, device=d)
+    nbytes = lib.sswin_unique_consecutive_workspace_bytes(m)
+    ws = _ws(nbytes, d)
+    with torch.cuda.device(d):
+        _lib.check(lib.sswin_unique_consecutive_indices(_ptr(nums), _KEY_CODE[nums.dtype], m, _ptr(out),
+                                                        _ptr(ws), nbytes, _stream(d)))
+    return out
+
+
+def return_inverse(x, maxnum=-1):
+    """``(rank of x[i] among the distinct values, number of distinct values)`` (ops.cu:718-730)."""
+    lib = _lib.load()
+    d = _dev(x)
+    _check(x.dtype == torch.int32, "return_inverse: x must be int32")
+    x = x.contiguous().view(-1)
+    m = x.numel()
+    out = torch.empty(m, dtype=torch.int32, device=d)
+    if m == 0:
+        return out, 0
+    maxnum = int(maxnum)
+    bound = maxnum
+    if maxnum == -1:
+        # the table size is data dependent: one read-back here, as in the reference (ops.cu:721)
+        bound = int(x.max().item()) + 1
+        _check(bound >= 1, "return_inverse: all values negative")
+        maxnum = bound
+    nbytes = lib.sswin_return_inverse_workspace_bytes(m, bound)
+    ws = _ws(nbytes, d)
+    count = C.c_int64(0)
+    with torch.cuda.device(d):
+        _lib.check(lib.sswin_return_inverse(_ptr(x), m, maxnum, _ptr(out), C.byref(count), _ptr(ws), nbytes,
+                                            _stream(d)))
+    return out, int(count.value)
+
+
+def qkv_sparse_indices(indices, batch_size, spatial_dim, num_heads, c):
+    """Element-level COO indices of Q/V and K^T plus their sorting permutations (ops.cu:293-335)."""
+    lib = _lib.load()
+    d = _dev(indices)
+    _check(indices.dim() == 2 and indices.shape[1] == 2, "qkv_sparse_indices: indices must be [N, 2]")
+    _check(indices.dtype == torch.int32, "qkv_sparse_indices: indices must be int32")
+    indices = indices.contiguous()
+    n_vox = indices.shape[0]
+    e = n_vox * num_heads * c
+    idx_qv = torch.empty((4, e), dtype=torch.int32, device=d)
+    idx_k = torch.empty((4, e), dtype=torch.int32, device=d)
+    sorted_qv = torch.empty(e, dtype=torch.int32, device=d)
+    sorted_k = torch.empty(e, dtype=torch.int32, device=d)
+    nbytes = lib.sswin_qkv_sparse_indices_workspace_bytes(n_vox, int(batch_size), int(spatial_dim))
+    ws = _ws(nbytes, d)
+    with torch.cuda.device(d):
+        _lib.check(lib.sswin_qkv_sparse_indices(_ptr(indices), n_vox, int(batch_size), int(spatial_dim),
+                                                int(num_heads), int(c), _ptr(idx_qv), _ptr(sorted_qv),
+                                                _ptr(idx_k), _ptr(sorted_k), _ptr(ws), nbytes, _stream(d)))
+    return idx_qv, sorted_qv, idx_k, sorted_k
+
+
+# --------------------------------------------------------------------------------------- #
+# per-group offsets: a small cache so that the eight backward calls that receive the `_c`
+# tensor returned by matmul_cuda_naive do not rescan it.
+# --------------------------------------------------------------------------------------- #
+class _PlanCache:
+    """Maps the storage address of a `_c` tensor handed out by :func:`matmul_cuda_naive` to
+    its scans.  Entries hold a reference to the plan tensor, so the address cannot be reused
+    while an entry is alive; the version counter guards against in-place edits."""
+
+    def __init__(self, capacity=32):
+        self.capacity = capacity
+        self.entries = OrderedDict()
+
+    def put(self, c_view, plan, g_cap, totals):
+        key = (c_view.device.index, c_view.data_ptr(), c_view.numel())
+        self.entries[key] = (plan, g_cap, totals, c_view._version)
+        self.entries.move_to_end(key)
+        while len(self.entries) > self.capacity:
+            self.entries.popitem(last=False)
+
+    def get(self, c):
+        key = (c.device.index, c.data_ptr(), c.numel())
+        hit = self.entries.get(key)
+        if hit is None or hit[3] != c._version or c.dtype != torch.int32 or not c.is_contiguous():
+            return None
+        self.entries.move_to_end(key)
+        return hit
+
+    def clear(self):
+        self.entries.clear()
+
+
+_plan_cache = _PlanCache()
+
+
+def _scans_for(c, lib, d):
+    """Return ``(scans [2,G] int32 rows: excl-scan c, excl-scan c*c; sum_c2 or None)``."""
+    hit = _plan_cache.get(c)
+    g = c.numel()
+    if hit is not None:
+        plan, g_cap, totals, _ = hit
+        rows = plan.view(5, g_cap)
+        if g_cap == g:
+            return rows[1:3].reshape(-1), totals[2]
+        return torch.stack([rows[1, :g], rows[2, :g]]).reshape(-1), totals[2]
+    scans = torch.empty(2 * max(g, 1), dtype=torch.int32, device=d)
+    nbytes = lib.sswin_scan_counts_workspace_bytes(g)
+    ws = _ws(nbytes, d)
+    _lib.check(lib.sswin_scan_counts(_ptr(c), g, _ptr(scans), _ptr(ws), nbytes, _stream(d)))
+    return scans, None
+
+
+# --------------------------------------------------------------------------------------- #
+# block products
+# --------------------------------------------------------------------------------------- #
+def matmul_cuda_naive(mat1_v, mat1_idx, mat1_shape, mat2_v, mat2_idx, mat2_shape, mul_type):
+    """Window-blocked sparse product ``'q_k'`` or ``'qk_v'`` (reference ops.cu:788-943, 1034-1088).
+
+    Returns ``(indices int32 [4, nnz], values [nnz], shape list[4], _c int32 [G])``.
+    """
+    lib = _lib.load()
+    _check(mat1_idx.dim() == 2, "Expected mat1_idx.dim() == 2 to be true, but got false.")
+    _check(mat2_idx.dim() == 2, "Expected mat2_idx.dim() == 2 to be true, but got false.")
+    _check(mat1_v.dim() == 1, "Expected mat1_v.dim() == 1 to be true, but got false.")
+    _check(mat2_v.dim() == 1, "Expected mat2_v.dim() == 1 to be true, but got false.")
+    _check(mul_type in _MUL, f"Invalid mul_type: {mul_type}. Expected 'q_k' or 'qk_v'.")
+    _check(mat1_v.dtype == mat2_v.dtype, f"mat1 dtype {mat1_v.dtype} does not match mat2 dtype {mat2_v.dtype}")
+    _check(mat1_idx.dtype == mat2_idx.dtype,
+           f"mat1 dtype {mat1_idx.dtype} does not match mat2 dtype {mat2_idx.dtype}")
+    _check(mat1_idx.dtype == torch.int32, f"mat1 dtype is not int32, but {mat1_idx.dtype}")
+    s1, s2 = [int(v) for v in mat1_shape], [int(v) for v in mat2_shape]
+    _check(len(s1) == 4 and len(s2) == 4 and s1[0] == s2[0] and s1[1] == s2[1] and s1[3] == s2[2],
+           f"Invalid shapes: mat1_shape {s1} and mat2_shape {s2}. Expected sizes: 4. Expected "
+           "mat1_shape[0] == mat2_shape[0], mat1_shape[1] == mat2_shape[1], mat1_shape[3] == mat2_shape[2].")
+    _check(mat1_v.dtype in _DTYPE_CODE, f"unsupported value dtype {mat1_v.dtype}")
+    d = _dev(mat1_v, mat1_idx, mat2_v, mat2_idx)
+    _check(mat1_idx.shape[0] == 4 and mat2_idx.shape[0] == 4, "index matrices must have 4 rows")
+    _check(mat1_idx.shape[1] == mat1_v.numel() and mat2_idx.shape[1] == mat2_v.numel(),
+           "index and value counts differ")
+    mat1_v, mat2_v = mat1_v.contiguous(), mat2_v.contiguous()
+    mat1_idx, mat2_idx = mat1_idx.contiguous(), mat2_idx.contiguous()
+
+    kind = _MUL[mul_type]
+    tok_idx = mat1_idx if kind == 0 else mat2_idx
+    inner = s1[3] if kind == 0 else s2[3]
+    m = tok_idx.shape[1]
+    out_shape = [s1[0], s1[1], s1[2], s2[3]]
+    if m == 0:
+        return (torch.empty((4, 0), dtype=torch.int32, device=d), torch.empty(0, dtype=mat1_v.dtype, device=d),
+                out_shape, torch.empty(0, dtype=torch.int32, device=d))
+    _check(m % inner == 0, f"operand nnz {m} is not a multiple of its dense last dimension {inner}")
+    rows = m // inner
+    g_cap = max(1, min(rows, s1[0] * s1[1]))
+    plan = torch.empty(5 * g_cap, dtype=torch.int32, device=d)
+    totals = (C.c_int64 * 4)()
+    stream = _stream(d)
+    with torch.cuda.device(d):
+        nbytes = lib.sswin_plan_workspace_bytes(m, inner)
+        ws = _ws(nbytes, d)
+        _lib.check(lib.sswin_plan_from_indices(_ptr(tok_idx), m, inner, _ptr(plan), g_cap, totals, _ptr(ws),
+                                               nbytes, stream))
+        g, sum_c, sum_c2, c_max = (int(totals[i]) for i in range(4))
+        if kind == 0:
+            _check(mat2_v.numel() == m, f"'q_k': mat2 holds {mat2_v.numel()} values, expected {m}")
+            nnz = sum_c2
+        else:
+            _check(mat1_v.numel() == sum_c2,
+                   f"'qk_v': mat1 holds {mat1_v.numel()} values, expected sum of c*c = {sum_c2}")
+            nnz = m
+        out_idx = torch.empty((4, nnz), dtype=torch.int32, device=d)
+        out_val = torch.empty(nnz, dtype=mat1_v.dtype, device=d)
+        _lib.check(lib.sswin_block_matmul(kind, _DTYPE_CODE[mat1_v.dtype], _ptr(mat1_v), _ptr(mat2_v),
+                                          _ptr(tok_idx), m, inner, _ptr(plan), g_cap, g, c_max,
+                                          _ptr(out_val), _ptr(out_idx), nnz, stream))
+    c_view = plan[:g]
+    _plan_cache.put(c_view, plan, g_cap, (g, sum_c, sum_c2, c_max))
+    return out_idx, out_val, out_shape, c_view
+
+
+def matmul_grad_cuda_naive(mat1_v, mat2_v, _c, C_, mul_type):
+    """Value-only block products of the backward pass (reference ops.cu:945-1031, 1092-1114)."""
+    lib = _lib.load()
+    _check(mul_type in _GRAD, f"Invalid mul_type: {mul_type}. Expected 'rc_cr', 'rr_rc' or 'cr_rr'.")
+    _check(mat1_v.dtype == mat2_v.dtype, f"mat1 dtype {mat1_v.dtype} does not match mat2 dtype {mat2_v.dtype}")
+    _check(mat1_v.dtype in _DTYPE_CODE, f"unsupported value dtype {mat1_v.dtype}")
+    _check(_c.dtype == torch.int32, "_c must be int32")
+    d = _dev(mat1_v, mat2_v, _c)
+    mat1_v, mat2_v, _c = mat1_v.contiguous(), mat2_v.contiguous(), _c.contiguous()
+    g, C_ = _c.numel(), int(C_)
+    kind = _GRAD[mul_type]
+    with torch.cuda.device(d):
+        scans, sum_c2 = _scans_for(_c, lib, d)
+        if kind == 0:
+            if sum_c2 is None:      # output size is data dependent: one read-back (reference ops.cu:968)
+                sum_c2 = int((_c.to(torch.int64) ** 2).sum().item())
+            total = sum_c2
+            _check(mat1_v.numel() == mat2_v.numel(), "'rc_cr': operands must have equal sizes")
+        elif kind == 1:
+            total = mat2_v.numel()
+        else:
+            total = mat1_v.numel()
+        out = torch.empty(total, dtype=mat1_v.dtype, device=d)
+        if g > 0 and total > 0:
+            _lib.check(lib.sswin_block_matmul_grad(kind, _DTYPE_CODE[mat1_v.dtype], _ptr(mat1_v), _ptr(mat2_v),
+                                                   _ptr(_c), _ptr(scans), g, C_, _ptr(out), _stream(d)))
+    return out
+
+
+def qkv_transpose(mat1_v, _c, C_, mul_type):
+    """Per-group transposes ``'rc'`` / ``'rr'`` (reference ops.cu:663-715, 1117-1132)."""
+    lib = _lib.load()
+    _check(mul_type in _TRANSPOSE, f"Invalid mul_type: {mul_type}. Expected 'rc', or 'rr'.")
+    _check(mat1_v.dtype in _DTYPE_CODE, f"unsupported value dtype {mat1_v.dtype}")
+    _check(_c.dtype == torch.int32, "_c must be int32")
+    d = _dev(mat1_v, _c)
+    mat1_v, _c = mat1_v.contiguous(), _c.contiguous()
+    g = _c.numel()
+    out = torch.empty_like(mat1_v)
+    with torch.cuda.device(d):
+        scans, _ = _scans_for(_c, lib, d)
+        if g > 0 and mat1_v.numel() > 0:
+            _lib.check(lib.sswin_block_transpose(_TRANSPOSE[mul_type], _DTYPE_CODE[mat1_v.dtype], _ptr(mat1_v),
+                                                 _ptr(_c), _ptr(scans), g, int(C_), _ptr(out), _stream(d)))
+    return out
+
+
+# --------------------------------------------------------------------------------------- #
+# sparse row softmax
+# --------------------------------------------------------------------------------------- #
+def _softmax_args(indices, *vals):
+    d = _dev(indices, *vals)
+    _check(indices.dtype == torch.int32, "softmax: row ids must be int32")
+    _check(all(v.dim() == 1 and v.numel() == indices.numel() for v in vals), "softmax: size mismatch")
+    dtype = vals[0].dtype
+    _check(all(v.dtype == dtype for v in vals), "softmax: dtype mismatch")
+    _check(dtype in (torch.float32, torch.float64, torch.float16, torch.bfloat16),
+           f"softmax: unsupported dtype {dtype}")
+    work = dtype if dtype in (torch.float32, torch.float64) else torch.float32
+    return d, dtype, work, indices.contiguous(), [v.contiguous().to(work) for v in vals]
+
+
+def softmax_last_dim_forward(indices, values):
+    """``exp(v - max(0, rowmax)) / (rowsum + 1e-8)`` over sorted row ids (reference ops.cu:128-167)."""
+    lib = _lib.load()
+    d, dtype, work, indices, (values,) = _softmax_args(indices, values)
+    out = torch.empty_like(values)
+    with torch.cuda.device(d):
+        _lib.check(lib.sswin_softmax_last_dim_forward(_ptr(indices), _ptr(values), _DTYPE_CODE[work],
+                                                      values.numel(), _ptr(out), _stream(d)))
+    return out.to(dtype)
+
+
+def softmax_last_dim_backward(indices, values, grad_values):
+    """``g*y - y*sum_row(g*y)`` (reference ops.cu:169-194)."""
+    lib = _lib.load()
+    d, dtype, work, indices, (values, grad_values) = _softmax_args(indices, values, grad_values)
+    out = torch.empty_like(values)
+    with torch.cuda.device(d):
+        _lib.check(lib.sswin_softmax_last_dim_backward(_ptr(indices), _ptr(values), _ptr(grad_values),
+                                                       _DTYPE_CODE[work], values.numel(), _ptr(out), _stream(d)))
+    return out.to(dtype)

@@ -1,0 +1,226 @@
+"""GPU parity of the window-blocked products, transposes and the sparse softmax against the
+CPU oracle.  Indices and offsets: bit-exact.  Values: fp32 within rel 1e-5 of the fp64 oracle,
+fp16/bf16 within rel 2e-2 (relative error measured as in helpers.close)."""
+import zlib
+
+import numpy as np
+import pytest
+import torch
+
+from helpers import close, qkv_operands, ragged_window_indices, random_window_indices
+
+pytestmark = pytest.mark.gpu
+
+RTOL = {torch.float32: 1e-5, torch.float64: 1e-12, torch.float16: 2e-2, torch.bfloat16: 2e-2}
+
+
+def seed_of(*parts):
+    return zlib.crc32(repr(parts).encode()) % 100000
+
+
+def dev(a, dtype=None):
+    t = torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    return t if dtype is None else t.to(dtype)
+
+
+def host(t):
+    return t.detach().to(torch.float64).cpu().numpy() if t.is_floating_point() else t.cpu().numpy()
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from sparseswin3d_amd import custom_ops
+    return custom_ops
+
+
+# window occupancy mixes: tiny, around the 32 / 64 tile edges, full 5^3 windows, empty slots
+MIXES = {
+    "tiny": [1, 2, 3, 1, 5, 4],
+    "edges": [31, 32, 33, 0, 63, 64, 65, 1],
+    "full": [125, 124, 100, 7],
+    "mixed": [1, 40, 2, 125, 0, 0, 17, 32, 90, 3, 3, 3, 3, 64],
+}
+
+
+def build(oracle, mix, H, hd, seed, n=125):
+    rng = np.random.default_rng(seed)
+    counts = MIXES[mix]
+    ind = ragged_window_indices(rng, counts, n)
+    B = len(counts)
+    return B, n, qkv_operands(oracle, ind, B, n, H, hd, rng, dtype=np.float64)
+
+
+def run_forward(ops, oracle, d, dtype):
+    """q_k -> softmax -> qk_v on the GPU and in the fp64 oracle; returns both sides."""
+    q, kt, v = (dev(d[k], dtype) for k in ("q", "kt", "v"))
+    qi, ki = dev(d["qi"]), dev(d["ki"])
+    s_idx, s_val, s_shape, c1 = ops.matmul_cuda_naive(q, qi, d["q_shape"], kt, ki, d["k_shape"], "q_k")
+    # oracle consumes the same (rounded) inputs in fp64
+    q64, kt64, v64 = host(q), host(kt), host(v)
+    r_idx, r_val, r_shape, r_c = oracle.matmul_cuda_naive(q64, d["qi"], d["q_shape"], kt64, d["ki"], d["k_shape"], "q_k")
+    return dict(q=q, kt=kt, v=v, qi=qi, ki=ki, s_idx=s_idx, s_val=s_val, s_shape=s_shape, c1=c1,
+                q64=q64, kt64=kt64, v64=v64, r_idx=r_idx, r_val=r_val, r_shape=r_shape, r_c=r_c)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("mix,H,hd", [("tiny", 2, 32), ("edges", 3, 32), ("full", 1, 32), ("mixed", 3, 32),
+                                      ("mixed", 2, 16), ("edges", 1, 64)])
+def test_q_k_and_qk_v(ops, oracle, mix, H, hd, dtype):
+    B, n, d = build(oracle, mix, H, hd, seed=seed_of(mix, H, hd))
+    f = run_forward(ops, oracle, d, dtype)
+    # --- q_k
+    assert f["s_idx"].dtype == torch.int32 and f["c1"].dtype == torch.int32
+    assert f["s_shape"] == f["r_shape"] == [B, H, n, n]
+    np.testing.assert_array_equal(host(f["c1"]), f["r_c"])
+    np.testing.assert_array_equal(host(f["s_idx"]), f["r_idx"])
+    close(host(f["s_val"]), f["r_val"], RTOL[dtype], "q_k values")
+    # --- qk_v, fed with the oracle's attention so both sides multiply the same numbers
+    rows = oracle.unique_consecutive_indices(oracle.flatten_indices(f["r_idx"][:3], f["r_shape"][:3]))
+    p64 = oracle.softmax_last_dim_forward(rows, f["r_val"])
+    p = dev(p64, dtype)
+    o_idx, o_val, o_shape, c2 = ops.matmul_cuda_naive(p, f["s_idx"], f["s_shape"], f["v"], f["qi"], d["q_shape"], "qk_v")
+    ro_idx, ro_val, ro_shape, ro_c = oracle.matmul_cuda_naive(host(p), f["r_idx"], f["r_shape"], f["v64"], d["qi"],
+                                                             d["q_shape"], "qk_v")
+    assert o_shape == ro_shape == [B, H, n, hd]
+    np.testing.assert_array_equal(host(c2), ro_c)
+    np.testing.assert_array_equal(host(o_idx), ro_idx)
+    close(host(o_val), ro_val, RTOL[dtype], "qk_v values")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16])
+@pytest.mark.parametrize("mix,H,hd", [("tiny", 2, 32), ("edges", 2, 32), ("mixed", 3, 32), ("full", 1, 32),
+                                      ("mixed", 1, 16), ("edges", 1, 64)])
+@pytest.mark.parametrize("kind", ["rc_cr", "rr_rc", "cr_rr"])
+def test_matmul_grad(ops, oracle, mix, H, hd, kind, dtype):
+    rng = np.random.default_rng(seed_of(mix, H, hd, kind))
+    c = np.repeat(np.array([x for x in MIXES[mix] if x > 0], np.int32), H)
+    mat = int((c.astype(np.int64) * hd).sum())
+    sq = int((c.astype(np.int64) ** 2).sum())
+    n1, n2 = {"rc_cr": (mat, mat), "rr_rc": (sq, mat), "cr_rr": (mat, sq)}[kind]
+    m1 = dev(rng.standard_normal(n1), dtype)
+    m2 = dev(rng.standard_normal(n2), dtype)
+    out = ops.matmul_grad_cuda_naive(m1, m2, dev(c), hd, kind)
+    ref = oracle.matmul_grad_cuda_naive(host(m1), host(m2), c, hd, kind)
+    assert out.dtype == dtype
+    close(host(out), ref, RTOL[dtype], kind)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.float16])
+@pytest.mark.parametrize("mix,hd", [("tiny", 32), ("edges", 32), ("mixed", 32), ("full", 16)])
+@pytest.mark.parametrize("kind", ["rc", "rr"])
+def test_qkv_transpose(ops, oracle, mix, hd, kind, dtype):
+    rng = np.random.default_rng(len(mix) + hd)
+    c = np.array([x for x in MIXES[mix] if x > 0], np.int32)
+    total = int((c.astype(np.int64) * (hd if kind == "rc" else c)).sum())
+    m = dev(rng.standard_normal(total), dtype)
+    out = ops.qkv_transpose(m, dev(c), hd, kind)
+    ref = oracle.qkv_transpose(host(m), c, hd, kind)
+    np.testing.assert_array_equal(host(out), ref)          # pure data movement: exact
+
+
+def test_backward_identities_through_transposes(ops, oracle):
+    """The backward of 'q_k' as the reference's autograd Function composes it
+    (sparse_swin/swin3d_base.py:119-126) against plain per-group matrix algebra in fp64."""
+    B, n, d = build(oracle, "mixed", 2, 32, seed=9)
+    f = run_forward(ops, oracle, d, torch.float32)
+    rng = np.random.default_rng(1)
+    g_np = rng.standard_normal(f["s_val"].numel()).astype(np.float32)
+    g = dev(g_np)
+    c, C_ = f["c1"], 32
+    dq = ops.matmul_grad_cuda_naive(g, f["kt"], c, C_, "rr_rc")
+    qt = ops.qkv_transpose(f["q"], c, C_, "rc")
+    gt = ops.qkv_transpose(g, c, C_, "rr")
+    dkt = ops.matmul_grad_cuda_naive(qt, gt, c, C_, "cr_rr")
+    # plain algebra per group
+    cs = f["r_c"]
+    q64, kt64 = f["q64"], f["kt64"]
+    dq_ref, dkt_ref = [], []
+    po = mo = 0
+    for cg in cs:
+        cg = int(cg)
+        Q = q64[mo:mo + cg * C_].reshape(cg, C_)
+        Kt = kt64[mo:mo + cg * C_].reshape(C_, cg)
+        dS = g_np[po:po + cg * cg].astype(np.float64).reshape(cg, cg)
+        dq_ref.append((dS @ Kt.T).ravel())
+        dkt_ref.append((Q.T @ dS).ravel())
+        po += cg * cg
+        mo += cg * C_
+    close(host(dq), np.concatenate(dq_ref), 1e-5, "dQ")
+    close(host(dkt), np.concatenate(dkt_ref), 1e-5, "dK^T")
+
+
+# ------------------------------------------------------------------------------------------ softmax
+def _rows(lengths):
+    return np.repeat(np.arange(len(lengths)), lengths).astype(np.int32)
+
+
+ROW_MIXES = {
+    "short": [1, 2, 3, 16, 17, 31, 32, 33, 1, 1],
+    "windows": [125] * 40 + [7] * 30 + [64] * 9,
+    "cross_tile": [2047, 1, 2048, 2049, 5000, 3, 4096 + 17],
+    "single_long": [10_000],
+}
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64])
+@pytest.mark.parametrize("mix", list(ROW_MIXES))
+def test_softmax_forward_backward(ops, oracle, mix, dtype):
+    rng = np.random.default_rng(len(mix))
+    rows = _rows(ROW_MIXES[mix])
+    v = rng.standard_normal(len(rows)) * 3.0
+    v[rng.random(len(rows)) < 0.2] -= 100.0                    # masked entries of shifted windows
+    v64 = host(dev(v, dtype))
+    y = ops.softmax_last_dim_forward(dev(rows), dev(v, dtype))
+    y_ref = oracle.softmax_last_dim_forward(rows, v64)
+    close(host(y), y_ref, RTOL[dtype] if dtype == torch.float64 else 1e-5, "softmax fwd")
+    g = rng.standard_normal(len(rows))
+    gx = ops.softmax_last_dim_backward(dev(rows), y, dev(g, dtype))
+    gx_ref = oracle.softmax_last_dim_backward(rows, host(y), host(dev(g, dtype)))
+    close(host(gx), gx_ref, RTOL[dtype] if dtype == torch.float64 else 1e-5, "softmax bwd")
+
+
+def test_softmax_all_negative_rows_keep_zero_max(ops, oracle):
+    # rows whose maximum is below zero: the subtracted maximum is 0, not the row maximum
+    rows = _rows([4, 4, 1])
+    v = np.array([-1, -2, -3, -4, -30, -31, -32, -33, -5], np.float32)
+    y = ops.softmax_last_dim_forward(dev(rows), dev(v)).cpu().numpy().astype(np.float64)
+    ref = oracle.softmax_last_dim_forward(rows, v.astype(np.float64))
+    close(y, ref, 1e-5, "negative rows")
+    assert abs(y[4:8].sum() - 1.0) > 1e-6          # the 1e-8 term is visible for exp(-30)-sized sums
+
+
+def test_softmax_deterministic(ops):
+    rng = np.random.default_rng(0)
+    rows = dev(_rows([37] * 5000))
+    v = dev(rng.standard_normal(37 * 5000).astype(np.float32))
+    a = ops.softmax_last_dim_forward(rows, v)
+    b = ops.softmax_last_dim_forward(rows, v)
+    assert torch.equal(a, b)
+
+
+# ------------------------------------------------------------------------------------------ errors
+def test_error_behaviour(ops, oracle):
+    B, n, d = build(oracle, "tiny", 1, 32, seed=3)
+    q, kt = dev(d["q"], torch.float32), dev(d["kt"], torch.float32)
+    qi, ki = dev(d["qi"]), dev(d["ki"])
+    with pytest.raises(RuntimeError, match="Invalid mul_type"):
+        ops.matmul_cuda_naive(q, qi, d["q_shape"], kt, ki, d["k_shape"], "k_q")
+    with pytest.raises(RuntimeError, match="not int32"):
+        ops.matmul_cuda_naive(q, qi.long(), d["q_shape"], kt, ki.long(), d["k_shape"], "q_k")
+    with pytest.raises(RuntimeError, match="does not match"):
+        ops.matmul_cuda_naive(q, qi, d["q_shape"], kt.double(), ki, d["k_shape"], "q_k")
+    with pytest.raises(RuntimeError, match="Invalid shapes"):
+        ops.matmul_cuda_naive(q, qi, d["q_shape"], kt, ki, [B, 1, 16, n], "q_k")
+    c = dev(np.array([1, 2], np.int32))
+    with pytest.raises(RuntimeError, match="Invalid mul_type"):
+        ops.matmul_grad_cuda_naive(q, kt, c, 32, "rc_rc")
+    with pytest.raises(RuntimeError, match="Invalid mul_type"):
+        ops.qkv_transpose(q, c, 32, "cr")
+
+
+def test_empty_operands(ops):
+    e_idx = torch.empty((4, 0), dtype=torch.int32, device="cuda")
+    e_val = torch.empty(0, dtype=torch.float32, device="cuda")
+    idx, val, shape, c = ops.matmul_cuda_naive(e_val, e_idx, [4, 2, 125, 32], e_val, e_idx, [4, 2, 32, 125], "q_k")
+    assert idx.shape == (4, 0) and val.numel() == 0 and c.numel() == 0 and shape == [4, 2, 125, 125]
+    assert ops.softmax_last_dim_forward(torch.empty(0, dtype=torch.int32, device="cuda"), e_val).numel() == 0
