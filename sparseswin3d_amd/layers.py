@@ -1,0 +1,248 @@
+"""Shifted-window block and stage built around :class:`WindowAttentionSparse`.
+
+Host-side mirror of the caller side of the reference's ``sparse_swin/swin3d_base.py``:
+window/shift clamping (ref ``:276-300``), sparse window partition / reverse (``:336-413``),
+padding and cyclic roll of voxel indices (``:501-554``), the 27-region shift mask
+(``:416-452``), ``SwinTransformerBlock`` (``:680-782``) and ``BasicLayer`` (``:785-873``).
+All of it is integer arithmetic on an [N, 4] (batch, d, h, w) int32 index tensor plus plain
+torch modules; the attention itself runs in the HIP operators.
+"""
+from __future__ import annotations
+
+from typing import List, Sequence
+
+import torch
+import torch.nn as nn
+
+from .window_attention import WindowAttentionSparse, replace_feature
+
+
+def get_window_size(x_size, window_size, shift_size=None):
+    """Clamp the window (and zero the shift) along axes where the grid is not larger."""
+    ws = list(window_size)
+    ss = list(shift_size) if shift_size is not None else None
+    for i, extent in enumerate(x_size):
+        if extent <= window_size[i]:
+            ws[i] = extent
+            if ss is not None:
+                ss[i] = 0
+    return tuple(ws) if ss is None else (tuple(ws), tuple(ss))
+
+
+def _window_grid(spatial, window_size):
+    return [s // w for s, w in zip(spatial, window_size)]
+
+
+def window_partition_sparse(x, window_size):
+    """(batch, d, h, w) voxel indices -> (window id, position inside the window); in place."""
+    d, h, w = x.spatial_shape
+    nd, nh, nw = _window_grid((d, h, w), window_size)
+    wd, wh, ww = window_size
+    i = x.indices
+    window = i[:, 0] * (nd * nh * nw) + (i[:, 1] // wd) * (nh * nw) + (i[:, 2] // wh) * nw + (i[:, 3] // ww)
+    pos = (i[:, 1] % wd) * (wh * ww) + (i[:, 2] % wh) * ww + (i[:, 3] % ww)
+    batch = x.batch_size
+    x.indices = torch.stack([window, pos], dim=1)
+    x.spatial_shape = (wd * wh * ww,)
+    x.batch_size = batch * nd * nh * nw
+    return x
+
+
+def window_reverse_sparse(x, original_shape, window_size):
+    """Inverse of :func:`window_partition_sparse`; in place."""
+    b, d, h, w, _ = original_shape
+    nd, nh, nw = _window_grid((d, h, w), window_size)
+    wd, wh, ww = window_size
+    window, pos = x.indices[:, 0], x.indices[:, 1]
+    per_batch = nd * nh * nw
+    batch, cell = window // per_batch, window % per_batch
+    zd = (cell // (nh * nw)) * wd + pos // (wh * ww)
+    zh = ((cell % (nh * nw)) // nw) * wh + (pos % (wh * ww)) // ww
+    zw = (cell % nw) * ww + pos % ww
+    x.indices = torch.stack([batch, zd, zh, zw], dim=1)
+    x.spatial_shape = [d, h, w]
+    x.batch_size = b
+    return x
+
+
+def pad_sparse_tensor(x, pad_l, pad_r, pad_t, pad_b, pad_d0=0, pad_d1=0):
+    """Grow the spatial shape; leading pads shift the indices."""
+    idx = x.indices.clone()
+    idx[:, 1] += pad_d0
+    idx[:, 2] += pad_t
+    idx[:, 3] += pad_l
+    x.indices = idx
+    x.spatial_shape = (x.spatial_shape[0] + pad_d0 + pad_d1, x.spatial_shape[1] + pad_t + pad_b,
+                       x.spatial_shape[2] + pad_l + pad_r)
+    return x
+
+
+def roll_sparse_tensor(x, shifts, dims):
+    """Cyclic shift of voxel indices along spatial dims 1..3."""
+    idx = x.indices.clone()
+    for shift, dim in zip(shifts, dims):
+        if dim < 1 or dim > 3:
+            raise ValueError("Dimension out of bounds for spatial shift. Must be 1, 2, or 3.")
+        idx[:, dim] = (idx[:, dim] + shift) % x.spatial_shape[dim - 1]
+    x.indices = idx
+    return x
+
+
+def window_partition(x: torch.Tensor, window_size: List[int]) -> torch.Tensor:
+    """Dense [b, d, h, w, c] -> [b * windows, tokens per window, c]."""
+    b, d, h, w, c = x.shape
+    wd, wh, ww = window_size
+    x = x.view(b, d // wd, wd, h // wh, wh, w // ww, ww, c)
+    return x.permute(0, 1, 3, 5, 2, 4, 6, 7).contiguous().view(-1, wd * wh * ww, c)
+
+
+def compute_mask(dims: List[int], window_size: List[int], shift_size: List[int], device) -> torch.Tensor:
+    """int8 [windows, tokens per window] region ids (27 regions) of the shifted grid."""
+    d, h, w = dims
+    img = torch.zeros((1, d, h, w, 1), device=device, dtype=torch.int8)
+    region = 0
+    for sd in (slice(-window_size[0]), slice(-window_size[0], -shift_size[0]), slice(-shift_size[0], None)):
+        for sh in (slice(-window_size[1]), slice(-window_size[1], -shift_size[1]), slice(-shift_size[1], None)):
+            for sw in (slice(-window_size[2]), slice(-window_size[2], -shift_size[2]), slice(-shift_size[2], None)):
+                img[:, sd, sh, sw, :] = region
+                region += 1
+    return window_partition(img, list(window_size)).squeeze(-1)
+
+
+_ACTIVATIONS = {"GELU": nn.GELU, "RELU": nn.ReLU, "LEAKYRELU": nn.LeakyReLU, "SILU": nn.SiLU, "SWISH": nn.SiLU,
+                "TANH": nn.Tanh, "SIGMOID": nn.Sigmoid, "ELU": nn.ELU}
+
+
+def get_act_layer(name: str):
+    try:
+        return _ACTIVATIONS[name.upper()]()
+    except KeyError:
+        raise ValueError(f"Unknown activation '{name}'.") from None
+
+
+class MLP(nn.Module):
+    """Two-layer feed-forward block: linear, activation, dropout, linear, dropout."""
+
+    def __init__(self, hidden_size: int, mlp_dim: int, dropout_rate: float = 0.0, act="GELU"):
+        super().__init__()
+        if not 0 <= dropout_rate <= 1:
+            raise ValueError("dropout_rate should be between 0 and 1.")
+        self.linear1 = nn.Linear(hidden_size, mlp_dim or hidden_size)
+        self.linear2 = nn.Linear(mlp_dim or hidden_size, hidden_size)
+        self.fn = get_act_layer(act) if isinstance(act, str) else act
+        self.drop1 = nn.Dropout(dropout_rate)
+        self.drop2 = nn.Dropout(dropout_rate)
+
+    def forward(self, x):
+        return self.drop2(self.linear2(self.drop1(self.fn(self.linear1(x)))))
+
+
+class DropPath(nn.Module):
+    """Stochastic depth: drops whole rows with probability ``drop_prob`` during training."""
+
+    def __init__(self, drop_prob: float = 0.0, scale_by_keep: bool = True):
+        super().__init__()
+        if not 0 <= drop_prob <= 1:
+            raise ValueError("Drop path prob should be between 0 and 1.")
+        self.drop_prob = drop_prob
+        self.scale_by_keep = scale_by_keep
+
+    def forward(self, x):
+        if self.drop_prob == 0.0 or not self.training:
+            return x
+        keep = 1.0 - self.drop_prob
+        mask = x.new_empty((x.shape[0],) + (1,) * (x.ndim - 1)).bernoulli_(keep)
+        if keep > 0.0 and self.scale_by_keep:
+            mask.div_(keep)
+        return x * mask
+
+
+class SwinTransformerBlock(nn.Module):
+    """norm -> (shifted) window attention -> residual -> norm -> MLP -> residual."""
+
+    def __init__(self, dim: int, num_heads: int, window_size: Sequence[int], shift_size: Sequence[int],
+                 mlp_ratio: float = 4.0, qkv_bias: bool = True, drop: float = 0.0, attn_drop: float = 0.0,
+                 drop_path: float = 0.0, act_layer: str = "GELU", norm_layer=nn.LayerNorm,
+                 use_checkpoint: bool = False) -> None:
+        super().__init__()
+        self.dim = dim
+        self.num_heads = num_heads
+        self.window_size = window_size
+        self.shift_size = shift_size
+        self.mlp_ratio = mlp_ratio
+        self.use_checkpoint = use_checkpoint
+        self.norm1 = norm_layer(dim)
+        self.attn = WindowAttentionSparse(dim, window_size=self.window_size, num_heads=num_heads,
+                                          qkv_bias=qkv_bias, attn_drop=attn_drop, proj_drop=drop)
+        self.drop_path = DropPath(drop_path) if drop_path > 0.0 else nn.Identity()
+        self.norm2 = norm_layer(dim)
+        self.mlp = MLP(hidden_size=dim, mlp_dim=int(dim * mlp_ratio), act=act_layer, dropout_rate=drop)
+
+    def forward_part1(self, x, mask_matrix):
+        x = replace_feature(x, self.norm1(x.features))
+        b, (d, h, w), c = x.batch_size, x.spatial_shape, x.features.shape[-1]
+        window_size, shift_size = get_window_size((d, h, w), self.window_size, self.shift_size)
+        pad_d1 = (window_size[0] - d % window_size[0]) % window_size[0]
+        pad_b = (window_size[1] - h % window_size[1]) % window_size[1]
+        pad_r = (window_size[2] - w % window_size[2]) % window_size[2]
+        x = pad_sparse_tensor(x, 0, pad_r, 0, pad_b, 0, pad_d1)
+        dims = [b, *x.spatial_shape, c]
+        shifted = any(s > 0 for s in shift_size)
+        if shifted:
+            x = roll_sparse_tensor(x, shifts=tuple(-s for s in shift_size), dims=(1, 2, 3))
+        x = window_partition_sparse(x, window_size)
+        x = self.attn(x, mask=mask_matrix if shifted else None)
+        x = window_reverse_sparse(x, dims, window_size)
+        if shifted:
+            x = roll_sparse_tensor(x, shifts=tuple(shift_size), dims=(1, 2, 3))
+        if pad_d1 > 0 or pad_r > 0 or pad_b > 0:
+            x.spatial_shape = [d, h, w]
+        return x
+
+    def forward_part2(self, x):
+        x = replace_feature(x, self.norm2(x.features))
+        return replace_feature(x, self.drop_path(self.mlp(x.features)))
+
+    def forward(self, x, mask_matrix):
+        shortcut = x
+        x = self.forward_part1(x, mask_matrix)
+        x = replace_feature(x, shortcut.features + self.drop_path(x.features))
+        return replace_feature(x, x.features + self.forward_part2(x).features)
+
+
+class BasicLayer(nn.Module):
+    """One stage: ``depth`` blocks alternating no shift / shift by half a window."""
+
+    def __init__(self, dim: int, depth: int, num_heads: int, window_size: Sequence[int], drop_path,
+                 mlp_ratio: float = 4.0, qkv_bias: bool = False, drop: float = 0.0, attn_drop: float = 0.0,
+                 norm_layer=nn.LayerNorm, downsample=None, use_checkpoint: bool = False,
+                 indice_key=None) -> None:
+        super().__init__()
+        self.window_size = window_size
+        self.shift_size = tuple(i // 2 for i in window_size)
+        self.no_shift = tuple(0 for _ in window_size)
+        self.depth = depth
+        self.use_checkpoint = use_checkpoint
+        self.blocks = nn.ModuleList([
+            SwinTransformerBlock(dim=dim, num_heads=num_heads, window_size=self.window_size,
+                                 shift_size=self.no_shift if i % 2 == 0 else self.shift_size,
+                                 mlp_ratio=mlp_ratio, qkv_bias=qkv_bias, drop=drop, attn_drop=attn_drop,
+                                 drop_path=drop_path[i] if isinstance(drop_path, list) else drop_path,
+                                 norm_layer=norm_layer, use_checkpoint=use_checkpoint)
+            for i in range(depth)])
+        self.downsample = downsample
+        if callable(self.downsample):
+            self.downsample = downsample(dim=dim, norm_layer=norm_layer, spatial_dims=len(self.window_size),
+                                         indice_key=indice_key)
+
+    def forward(self, x):
+        d, h, w = x.spatial_shape
+        window_size, shift_size = get_window_size((d, h, w), self.window_size, self.shift_size)
+        padded = [-(-s // ws) * ws for s, ws in zip((d, h, w), window_size)]
+        # The mask is built whenever the layer has a shift; unshifted blocks ignore it.
+        attn_mask = compute_mask(padded, window_size, shift_size, x.features.device)
+        for blk in self.blocks:
+            x = blk(x, attn_mask)
+        if self.downsample is not None:
+            x = self.downsample(x)
+        return x

@@ -1,0 +1,62 @@
+"""The C-ABI library builds, loads without a GPU and exports every symbol the header declares."""
+import ctypes
+import os
+import re
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    text = open(os.path.join(ROOT, "include", "sswin3d.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(sswin_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_declares_the_ten_operators():
+    names = declared_symbols()
+    for op in ("flatten_indices", "sort_indices", "unique_consecutive_indices", "return_inverse",
+               "qkv_sparse_indices", "block_matmul", "block_matmul_grad", "block_transpose",
+               "softmax_last_dim_forward", "softmax_last_dim_backward"):
+        assert f"sswin_{op}" in names
+
+
+def test_library_exports_every_declared_symbol():
+    from sparseswin3d_amd import _lib
+    lib = _lib.load()                                  # raises if the .so has not been built
+    for name in declared_symbols():
+        assert hasattr(lib, name), f"{name} declared in include/sswin3d.h but not exported"
+        assert name in _lib.SIGNATURES, f"{name} has no ctypes signature"
+    assert sorted(_lib.SIGNATURES) == declared_symbols()
+    assert lib.sswin_abi_version() == _lib.ABI_VERSION
+
+
+def test_argument_errors_are_reported_without_a_gpu():
+    from sparseswin3d_amd import _lib
+    lib = _lib.load()
+    # ndim out of range is rejected on the host before any launch
+    rc = lib.sswin_flatten_indices(None, 9, 10, None, None, None)
+    assert rc != 0 and b"ndim" in lib.sswin_last_error()
+    rc = lib.sswin_block_transpose(7, 0, None, None, None, 1, 32, None, None)
+    assert rc != 0 and b"Invalid mul_type" in lib.sswin_last_error()
+    rc = lib.sswin_softmax_last_dim_forward(None, None, 1, -1, None, None)
+    assert rc != 0
+
+
+def test_custom_ops_refuse_cpu_tensors():
+    import pytest
+    import torch
+    from sparseswin3d_amd import custom_ops
+    with pytest.raises(RuntimeError, match="GPU only"):
+        custom_ops.softmax_last_dim_forward(torch.zeros(3, dtype=torch.int32), torch.zeros(3))
+    with pytest.raises(RuntimeError, match="GPU only"):
+        custom_ops.sort_indices(torch.zeros(3, dtype=torch.int32))
+
+
+def test_product_does_not_import_the_oracle():
+    pkg = os.path.join(ROOT, "sparseswin3d_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for f in files:
+            if f.endswith((".py", ".hip", ".hpp", ".h")):
+                text = open(os.path.join(dirpath, f)).read()
+                assert not re.search(r"^\s*(from|import)\s+oracle\b", text, flags=re.M), f"{f} imports the oracle"
+                assert "liboracle" not in text and "cpu_path" not in text, f"{f} reaches into oracle/"
