@@ -1,0 +1,296 @@
+#!/usr/bin/env python3
+"""Benchmark of the sparse window-attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--kernels-json PATH]
+
+Workload (``config.workload``): the stage-1 block pair of the synthetic ScanNet-like room —
+``WindowAttentionSparse`` with the regular 5^3 windows, then with the windows shifted by 2,
+dim 96, 3 heads, fp32, forward + backward, about 100k voxels.  One step = forward of both
+attention modules chained, then backward from N(0,1) upstream gradients.  Inputs (features,
+window indices, mask, upstream gradients, weights) are resident in HBM before timing.
+
+``value`` = tokens/s = (attention calls per step x voxels) / step time.
+
+The JSON line also carries
+  roofline      the kernel that takes the largest share of a step, timed alone with HIP events
+                on the stream it is launched on; achieved = algorithmic bytes / duration
+  cpu_baseline  the PyTorch-CPU path (per-window torch.mm + scatter softmax + autograd) timed
+                on the host cores on a bounded sample of the same workload
+A per-kernel table goes to stderr and, with --kernels-json, to a file.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+import torch
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE) for the kernels
+# below on this workload; None = not measured.  Source summaries live in profiles/.
+MEASURED_TRAFFIC_BYTES = {}
+
+
+def log(*a):
+    print(*a, file=sys.stderr, flush=True)
+
+
+# ------------------------------------------------------------------------------------------
+def build_workload(device):
+    from sparseswin3d_amd import synth
+    from sparseswin3d_amd.window_attention import WindowAttentionSparse
+    w = synth.config2()
+    ws = w.window
+    shift = tuple(s // 2 for s in ws)
+    torch.manual_seed(2)
+    N = len(w.coords4)
+    blocks = []
+    pshape = synth.padded_shape(w.spatial_shape, ws)
+    mask = torch.from_numpy(synth.shift_region_mask(pshape, ws, shift)).to(device)
+    for sh in ((0, 0, 0), shift):
+        idx, nw, n = synth.window_indices(w.coords4, w.spatial_shape, ws, sh)
+        st = synth.scene_stats(idx, nw * w.batch_size)
+        attn = WindowAttentionSparse(w.dim, w.heads, ws, qkv_bias=True).to(device)
+        torch.nn.init.xavier_uniform_(attn.qkv.weight)
+        blocks.append(dict(attn=attn, idx=torch.from_numpy(idx).to(device), idx_np=idx, slots=nw * w.batch_size,
+                           n=n, mask=mask if any(sh) else None, stats=st.describe(w.heads), shift=sh))
+    feats = torch.randn(N, w.dim, device=device)
+    upstream = torch.randn(N, w.dim, device=device)
+    return dict(name=w.name, N=N, dim=w.dim, heads=w.heads, blocks=blocks, feats=feats, upstream=upstream,
+                mask_np=mask.cpu().numpy())
+
+
+def run_step(wl):
+    from sparseswin3d_amd.window_attention import SparseVoxelTensor
+    x = wl["feats"].detach().requires_grad_(True)
+    h = x
+    for b in wl["blocks"]:
+        t = SparseVoxelTensor(h, b["idx"], (b["n"],), b["slots"])
+        h = b["attn"](t, b["mask"]).features
+    h.backward(wl["upstream"])
+    return x.grad
+
+
+# ------------------------------------------------------------------------------------------
+def event_time_ms(fn, reps, warmup=2):
+    for _ in range(warmup):
+        fn()
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(reps):
+        fn()
+    stop.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(stop) / reps
+
+
+def kernel_table(wl, reps=20):
+    """Time every operator's kernels alone on the first block's tensors (regular windows)."""
+    from sparseswin3d_amd import _lib, custom_ops as ops
+    from sparseswin3d_amd.window_attention import qkv_sparse_cuda
+    lib = _lib.load()
+    b = wl["blocks"][0]
+    H, D = wl["heads"], wl["dim"]
+    hd = D // H
+    N = wl["N"]
+    dev = wl["feats"].device
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    ptr = lambda t: C.c_void_p(t.data_ptr())
+
+    qkv = torch.randn(N, 3, H, hd, device=dev)
+    q, kt, v = qkv_sparse_cuda(qkv, b["idx"], b["slots"], b["n"])
+    s_idx, s_val, s_shape, c = ops.matmul_cuda_naive(q.values, q.indices, q.shape, kt.values, kt.indices, kt.shape, "q_k")
+    flat = ops.flatten_indices(s_idx[:3], s_shape[:3])
+    rows = ops.unique_consecutive_indices(flat)
+    p_val = ops.softmax_last_dim_forward(rows, s_val)
+    o_idx, o_val, o_shape, c2 = ops.matmul_cuda_naive(p_val, s_idx, s_shape, v.values, v.indices, v.shape, "qk_v")
+    E, A, G = q.values.numel(), s_val.numel(), c.numel()
+    s = 4
+
+    # plan once, then the product kernels alone
+    m = E
+    g_cap = max(1, min(m // hd, b["slots"] * H))
+    plan = torch.empty(5 * g_cap, dtype=torch.int32, device=dev)
+    totals = (C.c_int64 * 4)()
+    nb = lib.sswin_plan_workspace_bytes(m, hd)
+    ws = torch.empty(nb, dtype=torch.uint8, device=dev)
+    _lib.check(lib.sswin_plan_from_indices(ptr(q.indices), m, hd, ptr(plan), g_cap, totals, ptr(ws), nb, stream))
+    c_max = int(totals[3])
+    scans = torch.stack([plan.view(5, g_cap)[1, :G], plan.view(5, g_cap)[2, :G]]).reshape(-1).contiguous()
+    cc = plan[:G].contiguous()
+    out_s = torch.empty(A, device=dev)
+    out_si = torch.empty((4, A), dtype=torch.int32, device=dev)
+    out_o = torch.empty(E, device=dev)
+    out_oi = torch.empty((4, E), dtype=torch.int32, device=dev)
+    g_s = torch.randn(A, device=dev)
+    g_o = torch.randn(E, device=dev)
+
+    def mm(kind, a, bb, tok, ov, oi, nnz):
+        return lambda: _lib.check(lib.sswin_block_matmul(kind, 0, ptr(a), ptr(bb), ptr(tok), m, hd, ptr(plan), g_cap, G,
+                                                         c_max, ptr(ov), ptr(oi), nnz, stream))
+
+    def grad(kind, a, bb, out):
+        return lambda: _lib.check(lib.sswin_block_matmul_grad(kind, 0, ptr(a), ptr(bb), ptr(cc), ptr(scans), G, hd,
+                                                              ptr(out), stream))
+
+    def tr(kind, a, out):
+        return lambda: _lib.check(lib.sswin_block_transpose(kind, 0, ptr(a), ptr(cc), ptr(scans), G, hd, ptr(out), stream))
+
+    tmp_e, tmp_a = torch.empty(E, device=dev), torch.empty(A, device=dev)
+    idxT = b["idx"].T.contiguous()
+    flat_tok = ops.flatten_indices(idxT, [b["slots"], b["n"]])
+    perm_idx = o_idx[[0, 2, 1, 3], :].contiguous()
+    flat_perm = ops.flatten_indices(perm_idx, [o_shape[0], o_shape[2], o_shape[1], o_shape[3]])
+
+    entries = [
+        # name, callable, algorithmic bytes, calls per attention fwd+bwd
+        ("qkv_sparse_indices", lambda: ops.qkv_sparse_indices(b["idx"], b["slots"], b["n"], H, hd), 8 * N + 40 * E, 1),
+        ("plan_from_indices", lambda: _lib.check(lib.sswin_plan_from_indices(ptr(q.indices), m, hd, ptr(plan), g_cap, totals, ptr(ws), nb, stream)), 0, 2),
+        ("block_matmul q_k", mm(0, q.values, kt.values, q.indices, out_s, out_si, A), 2 * s * E + (s + 16) * A + 4 * G, 1),
+        ("flatten_indices [3,A]", lambda: ops.flatten_indices(s_idx[:3], s_shape[:3]), 16 * A, 1),
+        ("unique_consecutive_indices [A]", lambda: ops.unique_consecutive_indices(flat), 8 * A, 1),
+        ("softmax_last_dim_forward", lambda: ops.softmax_last_dim_forward(rows, s_val), 12 * A, 1),
+        ("block_matmul qk_v", mm(1, p_val, v.values, v.indices, out_o, out_oi, E), s * A + s * E + (s + 16) * E + 4 * G, 1),
+        ("flatten_indices [4,E] (permute)", lambda: ops.flatten_indices(perm_idx, [o_shape[0], o_shape[2], o_shape[1], o_shape[3]]), 0, 1),
+        ("sort_indices [E] (permute)", lambda: ops.sort_indices(flat_perm), 0, 1),
+        ("return_inverse [N]", lambda: ops.return_inverse(flat_tok, -1), 0, 1),
+        ("softmax_last_dim_backward", lambda: ops.softmax_last_dim_backward(rows, p_val, g_s), 16 * A, 1),
+        ("grad rc_cr", grad(0, g_o, v.values, tmp_a), 2 * s * E + s * A, 1),
+        ("grad rr_rc", grad(1, g_s, kt.values, tmp_e), s * A + 2 * s * E, 2),
+        ("grad cr_rr", grad(2, q.values, g_s, tmp_e), s * A + 2 * s * E, 1),
+        ("transpose rc", tr(0, q.values, tmp_e), 2 * s * E, 2),
+        ("transpose rr", tr(1, g_s, tmp_a), 2 * s * A, 2),
+    ]
+    table = []
+    for name, fn, nbytes, calls in entries:
+        ms = event_time_ms(fn, reps)
+        gbps = nbytes / ms / 1e6 if nbytes else None
+        table.append(dict(kernel=name, ms=ms, algorithmic_bytes=nbytes, calls=calls,
+                          achieved_gbps=gbps, frac=(gbps / HBM_PEAK_GBPS) if gbps else None))
+    return table, dict(N=N, E=E, A=A, G=G, c_max=c_max)
+
+
+# ------------------------------------------------------------------------------------------
+def cpu_baseline(wl, target_tokens=12000):
+    """README path on the host cores, forward + backward, on the first windows of block 0."""
+    from oracle import cpu_path
+    b = wl["blocks"][0]
+    idx = b["idx_np"]
+    order = np.argsort(idx[:, 0], kind="stable")
+    take = order[:target_tokens]
+    # keep whole windows only
+    last_win = idx[take[-1], 0]
+    take = order[idx[order, 0] <= last_win]
+    sub_idx = idx[take]
+    attn = b["attn"]
+    p = {k: v.detach().float().cpu() for k, v in attn.state_dict().items()}
+    n = b["n"]
+    feats = wl["feats"][torch.from_numpy(take).to(wl["feats"].device)].cpu().requires_grad_(True)
+    up = wl["upstream"][torch.from_numpy(take).to(wl["feats"].device)].cpu()
+    table = p["relative_position_bias_table"].clone().requires_grad_(True)
+    qw = p["qkv.weight"].clone().requires_grad_(True)
+    pw = p["proj.weight"].clone().requires_grad_(True)
+    rel = attn.relative_position_index.cpu()[:n, :n].reshape(-1)
+
+    def once():
+        rpb = table[rel].reshape(n, n, -1).permute(2, 0, 1)
+        out = cpu_path.window_attention_cpu(feats, sub_idx, n, attn.num_heads, qw, p.get("qkv.bias"), pw,
+                                            p["proj.bias"], rpb, None, softmax="readme")
+        out.backward(up)
+
+    once()                                   # warm-up (allocator, thread pool)
+    t0 = time.perf_counter()
+    once()
+    dt = time.perf_counter() - t0
+    return dict(value=len(take) / dt, unit="tokens/s", cores=torch.get_num_threads(), kind="port",
+                sample=f"one WindowAttentionSparse fwd+bwd (regular windows) on the first {len(take)} voxels "
+                       f"({len(np.unique(sub_idx[:, 0]))} windows) of the workload, {dt:.1f} s, "
+                       f"host has {os.cpu_count()} logical cpus")
+
+
+# ------------------------------------------------------------------------------------------
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=10)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel table")
+    ap.add_argument("--kernels-json", default=None)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs on one GPU only (windows are independent; sharding is "
+                 "described in DESIGN.md); rerun with --gpus 1")
+    if not torch.cuda.is_available():
+        sys.exit("bench.py: no HIP GPU visible")
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+    wl = build_workload(device)
+    log(f"workload {wl['name']}: N={wl['N']}, blocks: " + "; ".join(str(b["stats"]) for b in wl["blocks"]))
+
+    for _ in range(args.warmup):
+        run_step(wl)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+        run_step(wl)
+    torch.cuda.synchronize()
+    dt = time.perf_counter() - t0
+    ms_per_step = dt / args.steps * 1e3
+    calls = len(wl["blocks"])
+    value = calls * wl["N"] / (dt / args.steps)
+
+    roofline = None
+    sizes = {}
+    if not args.no_kernels:
+        table, sizes = kernel_table(wl)
+        log(f"{'kernel':36s} {'ms':>9s} {'calls':>5s} {'alg MB':>9s} {'GB/s':>9s} {'% HBM':>7s}")
+        for r in table:
+            log(f"{r['kernel']:36s} {r['ms']:9.4f} {r['calls']:5d} {r['algorithmic_bytes'] / 1e6:9.1f} "
+                f"{(r['achieved_gbps'] or 0):9.1f} {100 * (r['frac'] or 0):7.2f}")
+        ops_ms = sum(r["ms"] * r["calls"] for r in table)
+        alg = sum(r["algorithmic_bytes"] * r["calls"] for r in table)
+        log(f"operators only, one attention fwd+bwd: {ops_ms:.3f} ms for {alg / 1e6:.1f} MB algorithmic "
+            f"= {alg / ops_ms / 1e6:.1f} GB/s = {100 * alg / ops_ms / 1e6 / HBM_PEAK_GBPS:.2f}% of HBM peak")
+        dom = max((r for r in table if r["algorithmic_bytes"]), key=lambda r: r["ms"] * r["calls"])
+        roofline = dict(bound="hbm", kernel=dom["kernel"], achieved=round(dom["achieved_gbps"], 1),
+                        peak=HBM_PEAK_GBPS, unit="GB/s", frac=round(dom["frac"], 4),
+                        traffic=MEASURED_TRAFFIC_BYTES.get(dom["kernel"]),
+                        algorithmic_bytes=dom["algorithmic_bytes"], ms=round(dom["ms"], 4),
+                        operators_only_ms=round(ops_ms, 3),
+                        operators_only_frac=round(alg / ops_ms / 1e6 / HBM_PEAK_GBPS, 4))
+        if args.kernels_json:
+            with open(args.kernels_json, "w") as f:
+                json.dump(dict(sizes=sizes, kernels=table), f, indent=1)
+
+    cpu = None
+    if not args.no_cpu:
+        cpu = cpu_baseline(wl)
+        log(f"cpu baseline: {cpu}")
+
+    line = {
+        "metric": "window-attn tokens/s fwd+bwd on 1 MI355X", "value": value, "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": f"{wl['name']}: stage-1 block pair (regular 5^3 windows, then shifted by 2) of "
+                               "WindowAttentionSparse, dim 96, 3 heads, forward+backward",
+                   "voxels": wl["N"], "attention_calls_per_step": calls, **sizes},
+        "roofline": roofline, "cpu_baseline": cpu,
+    }
+    if cpu:
+        line["speedup_vs_cpu"] = value / cpu["value"]
+    print(json.dumps(line), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -54,6 +54,13 @@ def load():
         raise LibraryMissing(
             f"{LIB_PATH} not found: build it with `python -m sparseswin3d_amd.build` "
             "(there is no CPU fallback for the sparse window-attention operators)")
+    # One HIP runtime per process: the tensors and streams handed to the library come from
+    # PyTorch, so PyTorch's own libamdhip64 must be the one already resident when the library's
+    # dependency on libamdhip64.so.7 is resolved (the loader reuses it by SONAME).
+    import torch
+    torch_hip = os.path.join(os.path.dirname(torch.__file__), "lib", "libamdhip64.so")
+    if os.path.exists(torch_hip):
+        C.CDLL(torch_hip, mode=C.RTLD_GLOBAL)
     lib = C.CDLL(LIB_PATH)
     for name, (res, args) in SIGNATURES.items():
         fn = getattr(lib, name)          # AttributeError here means header and library disagree
