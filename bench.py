@@ -181,13 +181,16 @@ def kernel_table(wl, reps=20):
 
 
 # ------------------------------------------------------------------------------------------
-def cpu_baseline(wl, target_tokens=12000):
-    """README path on the host cores, forward + backward, on the first windows of block 0."""
+def cpu_baseline(wl, target_tokens=None, repeats=2):
+    """README path on the host cores, forward + backward, on block 0 (regular windows).
+
+    Bounded sample: the whole first attention call of the workload (about 5 s per pass on 16
+    cores), timed `repeats` times after a warm-up on a small prefix."""
     from oracle import cpu_path
     b = wl["blocks"][0]
     idx = b["idx_np"]
     order = np.argsort(idx[:, 0], kind="stable")
-    take = order[:target_tokens]
+    take = order[:target_tokens or len(order)]
     # keep whole windows only
     last_win = idx[take[-1], 0]
     take = order[idx[order, 0] <= last_win]
@@ -202,19 +205,22 @@ def cpu_baseline(wl, target_tokens=12000):
     pw = p["proj.weight"].clone().requires_grad_(True)
     rel = attn.relative_position_index.cpu()[:n, :n].reshape(-1)
 
-    def once():
+    def once(f, ix, u):
         rpb = table[rel].reshape(n, n, -1).permute(2, 0, 1)
-        out = cpu_path.window_attention_cpu(feats, sub_idx, n, attn.num_heads, qw, p.get("qkv.bias"), pw,
+        out = cpu_path.window_attention_cpu(f, ix, n, attn.num_heads, qw, p.get("qkv.bias"), pw,
                                             p["proj.bias"], rpb, None, softmax="readme")
-        out.backward(up)
+        out.backward(u)
 
-    once()                                   # warm-up (allocator, thread pool)
+    warm = idx[order[:4000], 0].max()
+    wsel = idx[take, 0] < warm
+    once(feats[wsel].detach().requires_grad_(True), sub_idx[wsel], up[wsel])     # warm-up
     t0 = time.perf_counter()
-    once()
-    dt = time.perf_counter() - t0
+    for _ in range(repeats):
+        once(feats, sub_idx, up)
+    dt = (time.perf_counter() - t0) / repeats
     return dict(value=len(take) / dt, unit="tokens/s", cores=torch.get_num_threads(), kind="port",
                 sample=f"one WindowAttentionSparse fwd+bwd (regular windows) on the first {len(take)} voxels "
-                       f"({len(np.unique(sub_idx[:, 0]))} windows) of the workload, {dt:.1f} s, "
+                       f"({len(np.unique(sub_idx[:, 0]))} windows) of the workload, {dt:.1f} s per pass x {repeats}, "
                        f"host has {os.cpu_count()} logical cpus")
 
 

@@ -13,13 +13,19 @@
 //   RR_RC     m1  sq       m2  mat, j-major   mat [c x C]  c  C  c
 //   CR_RR     m1  mat[Cxc] m2  sq,  j-major   mat [C x c]  C  c  c
 //
-// Execution model (wave64, 256-thread workgroups, one workgroup per four consecutive groups):
-//   * if all four groups have I, J, K <= 32, each wavefront multiplies one group on its own
-//     (64 lanes = 8 x 8 register tiles of 4 x 4) — balanced work for the many small windows;
-//   * otherwise the four groups are processed one after another by the whole workgroup with
-//     fixed-size LDS blocks, so LDS use does not depend on the window occupancy.
-// Operands are staged in LDS k-major (At[k][i], Bs[k][j]) so that the inner loop is two 16-byte
-// LDS reads per 16 fused multiply-adds.  The work is HBM-bound (about 1.7 flop per byte).
+// Execution model (gfx950, wave64): the unit of work is one 32 x 32 output block of one group,
+// computed by ONE wavefront with v_mfma_f32_32x32x2_f32.  Operands go from global memory
+// straight into the MFMA lane layout — no LDS, no barriers, so wavefronts never wait for each
+// other and small windows cost one short task each:
+//   * lane l supplies A[i = l % 32][k] and B[k][j = l % 32]; within a 32-wide k chunk the MFMA
+//     step s pairs k = s (lanes 0-31) with k = 16 + s (lanes 32-63).  The sum over k does not
+//     care about that order, and it makes every row-contiguous operand a run of 16 consecutive
+//     values per lane (four 16-byte loads), and every k-major operand one coalesced row per step.
+//   * the accumulator of lane l holds column j = l % 32 of rows 8*(r/4) + 4*(l/32) + r%4,
+//     r = 0..15, so each store instruction writes two contiguous row segments.
+// A workgroup of four wavefronts takes four consecutive groups and deals their blocks round
+// robin.  The work is HBM-bound (about 1.7 flop per byte); MFMA is used because it removes the
+// LDS staging and the barriers, not because the arithmetic needs it.
 #include <cstdlib>
 #include <type_traits>
 
@@ -29,19 +35,11 @@ namespace sswin {
 
 enum { MODE_QK = 0, MODE_PV = 1, MODE_RC_CR = 2, MODE_RR_RC = 3, MODE_CR_RR = 4 };
 
-constexpr int KC = 32;                 // k extent of one LDS chunk
 constexpr int GROUPS_PER_WG = 4;
-constexpr int MAX_POS = 1024;          // largest supported window occupancy for index emission
+constexpr int MAX_POS = 1024;          // largest window occupancy the simple kernel's LDS table holds
 
 typedef float f32x4_u __attribute__((ext_vector_type(4), aligned(4)));
-typedef int i32x4_u __attribute__((ext_vector_type(4), aligned(4)));
-
-template <int MODE> struct BlockShape;   // workgroup-path LDS block (IB x JB), IB*JB/16 == 256
-template <> struct BlockShape<MODE_QK>    { static constexpr int IB = 64,  JB = 64;  };
-template <> struct BlockShape<MODE_RC_CR> { static constexpr int IB = 64,  JB = 64;  };
-template <> struct BlockShape<MODE_PV>    { static constexpr int IB = 128, JB = 32;  };
-template <> struct BlockShape<MODE_RR_RC> { static constexpr int IB = 128, JB = 32;  };
-template <> struct BlockShape<MODE_CR_RR> { static constexpr int IB = 32,  JB = 128; };
+typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 template <int MODE> __host__ __device__ constexpr bool b_is_kmajor() { return MODE == MODE_QK || MODE == MODE_PV; }
 
@@ -60,122 +58,6 @@ __device__ __forceinline__ GroupDims group_dims(int c, int C, int64_t rs, int64_
     return d;
 }
 
-// ------------------------------------------------------------------------------------------
-// LDS staging.  NT threads (tid in [0, NT)) fill a chunk; out-of-range elements become zero so
-// the multiply needs no bounds checks.
-// ------------------------------------------------------------------------------------------
-// source row-major [R x K] (k contiguous) -> dst[kk * P + rr], rr in [0, RB), kk in [0, KC)
-template <int NT, int RB, typename T>
-__device__ __forceinline__ void stage_transposed(const T* __restrict__ src, int R, int K, int r0, int k0,
-                                                 float* __restrict__ dst, int tid) {
-    constexpr int P = RB + 4;
-#pragma unroll 4
-    for (int f = tid; f < RB * KC; f += NT) {
-        const int rr = f / KC, kk = f % KC;
-        const int gr = r0 + rr, gk = k0 + kk;
-        float v = 0.f;
-        if (gr < R && gk < K) v = to_acc(src[(int64_t)gr * K + gk]);
-        dst[kk * P + rr] = v;
-    }
-}
-
-// source k-major [K x J] (j contiguous) -> dst[kk * P + jj], jj in [0, JB)
-template <int NT, int JB, typename T>
-__device__ __forceinline__ void stage_direct(const T* __restrict__ src, int K, int J, int k0, int j0,
-                                             float* __restrict__ dst, int tid) {
-    constexpr int P = JB + 4;
-#pragma unroll 4
-    for (int f = tid; f < JB * KC; f += NT) {
-        const int kk = f / JB, jj = f % JB;
-        const int gk = k0 + kk, gj = j0 + jj;
-        float v = 0.f;
-        if (gk < K && gj < J) v = to_acc(src[(int64_t)gk * J + gj]);
-        dst[kk * P + jj] = v;
-    }
-}
-
-template <int IB, int JB>
-__device__ __forceinline__ void multiply_chunk(const float* __restrict__ At, const float* __restrict__ Bs,
-                                               int ti, int tj, int kmax, float (&acc)[4][4]) {
-    constexpr int IP = IB + 4, JP = JB + 4;
-    const float* ap = At + 4 * ti;
-    const float* bp = Bs + 4 * tj;
-#pragma unroll 4
-    for (int kk = 0; kk < kmax; ++kk) {
-        const float4 a = *reinterpret_cast<const float4*>(ap + kk * IP);
-        const float4 b = *reinterpret_cast<const float4*>(bp + kk * JP);
-        const float av[4] = {a.x, a.y, a.z, a.w};
-        const float bv[4] = {b.x, b.y, b.z, b.w};
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-#pragma unroll
-            for (int s = 0; s < 4; ++s) acc[r][s] = fmaf(av[r], bv[s], acc[r][s]);
-    }
-}
-
-template <typename T>
-__device__ __forceinline__ void store_tile(T* __restrict__ O, int I, int J, int i0, int j0,
-                                           const float (&acc)[4][4]) {
-    if (i0 >= I || j0 >= J) return;
-#pragma unroll
-    for (int r = 0; r < 4; ++r) {
-        const int i = i0 + r;
-        if (i >= I) break;
-        T* p = O + (int64_t)i * J + j0;
-        if (sizeof(T) == 4 && j0 + 3 < J) {
-            f32x4_u v = {acc[r][0], acc[r][1], acc[r][2], acc[r][3]};
-            *reinterpret_cast<f32x4_u*>(p) = v;
-        } else {
-#pragma unroll
-            for (int s = 0; s < 4; ++s)
-                if (j0 + s < J) p[s] = from_acc<T>(acc[r][s]);
-        }
-    }
-}
-
-// ------------------------------------------------------------------------------------------
-// COO index emission for one group by NT threads.  Rows of out_idx are out_nnz apart.
-//   QK: slot ss + i*c + j      -> (window, head, pos[i], pos[j])
-//   PV: slot rs*C + i*C + ch   -> (window, head, pos[i], ch)
-// ------------------------------------------------------------------------------------------
-template <int NT, bool IS_QK>
-__device__ __forceinline__ void emit_indices(int32_t* __restrict__ out_idx, int64_t out_nnz, int64_t base,
-                                             int c, int C, int w, int h, const int* __restrict__ pos,
-                                             int tid) {
-    const int J = IS_QK ? c : C;
-    const int count = c * J;
-    int32_t* r0 = out_idx + base;
-    int32_t* r1 = r0 + out_nnz;
-    int32_t* r2 = r1 + out_nnz;
-    int32_t* r3 = r2 + out_nnz;
-    for (int f = tid * 4; f < count; f += NT * 4) {
-        int i = f / J, j = f - i * J;
-        int a[4], b[4];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int ii = i < c ? i : c - 1;              // clamp for the masked tail lanes
-            a[q] = pos[ii];
-            b[q] = IS_QK ? pos[j] : j;
-            if (++j == J) { j = 0; ++i; }
-        }
-        if (f + 3 < count) {
-            i32x4_u vw = {w, w, w, w}, vh = {h, h, h, h};
-            i32x4_u va = {a[0], a[1], a[2], a[3]}, vb = {b[0], b[1], b[2], b[3]};
-            *reinterpret_cast<i32x4_u*>(r0 + f) = vw;
-            *reinterpret_cast<i32x4_u*>(r1 + f) = vh;
-            *reinterpret_cast<i32x4_u*>(r2 + f) = va;
-            *reinterpret_cast<i32x4_u*>(r3 + f) = vb;
-        } else {
-            for (int q = 0; q < 4 && f + q < count; ++q) {
-                r0[f + q] = w; r1[f + q] = h; r2[f + q] = a[q]; r3[f + q] = b[q];
-            }
-        }
-    }
-}
-
-// ------------------------------------------------------------------------------------------
-// main kernel
-// ------------------------------------------------------------------------------------------
 struct GroupTable {
     const int32_t* c;          // [G]
     const int32_t* row_start;  // [G] exclusive scan of c
@@ -184,101 +66,140 @@ struct GroupTable {
     const int32_t* head;       // [G] or null
 };
 
-template <typename T, int MODE, bool EMIT>
-__global__ __launch_bounds__(256) void block_product_kernel(const T* __restrict__ m1, const T* __restrict__ m2,
-                                                            GroupTable gt, int64_t G, int C,
-                                                            const int32_t* __restrict__ tok_pos,
-                                                            T* __restrict__ out, int32_t* __restrict__ out_idx,
-                                                            int64_t out_nnz) {
-    using BS = BlockShape<MODE>;
-    constexpr int WG_LDS = KC * (BS::IB + 4) + KC * (BS::JB + 4);
-    constexpr int WAVE_LDS = 2 * KC * (32 + 4);
-    constexpr int LDS_FLOATS = WG_LDS > 4 * WAVE_LDS ? WG_LDS : 4 * WAVE_LDS;
-    __shared__ __attribute__((aligned(16))) float lds[LDS_FLOATS];
-    __shared__ int pos_s[EMIT ? MAX_POS : 1];
+// 16 consecutive values of one operand row, zero beyond `valid` (0..16).
+template <typename T>
+__device__ __forceinline__ void load_run16(const T* __restrict__ p, int valid, float (&x)[16]) {
+    if (valid >= 16) {
+        if (std::is_same<T, float>::value) {
+            const f32x4_u* q = reinterpret_cast<const f32x4_u*>(p);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const f32x4_u t = q[v];
+                x[4 * v] = t.x; x[4 * v + 1] = t.y; x[4 * v + 2] = t.z; x[4 * v + 3] = t.w;
+            }
+        } else {
+#pragma unroll
+            for (int s = 0; s < 16; ++s) x[s] = to_acc(p[s]);
+        }
+    } else {
+#pragma unroll
+        for (int s = 0; s < 16; ++s) x[s] = s < valid ? to_acc(p[s]) : 0.f;
+    }
+}
 
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+__device__ __forceinline__ int clamp16(int v) { return v < 0 ? 0 : (v > 16 ? 16 : v); }
+
+template <typename T, int MODE, bool EMIT>
+__global__ __launch_bounds__(256) void block_product_mfma_kernel(const T* __restrict__ m1, const T* __restrict__ m2,
+                                                                 GroupTable gt, int64_t G, int C,
+                                                                 const int32_t* __restrict__ tok_pos,
+                                                                 T* __restrict__ out, int32_t* __restrict__ out_idx,
+                                                                 int64_t out_nnz) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int half = lane >> 5, l32 = lane & 31;
     const int64_t g0 = (int64_t)blockIdx.x * GROUPS_PER_WG;
 
-    // this wave's own group (wave path) — also used to decide the path for the whole workgroup
-    const int64_t gw = g0 + wave;
-    const int cw = gw < G ? gt.c[gw] : 0;
-    int cmax = 0;
+    // blocks of the workgroup's four groups
+    int cq[GROUPS_PER_WG], nbj[GROUPS_PER_WG], first[GROUPS_PER_WG + 1];
+    first[0] = 0;
 #pragma unroll
     for (int q = 0; q < GROUPS_PER_WG; ++q) {
         const int64_t g = g0 + q;
-        const int cq = g < G ? gt.c[g] : 0;
-        cmax = cq > cmax ? cq : cmax;
+        const int c = g < G ? gt.c[g] : 0;
+        cq[q] = c;
+        const int I = MODE == MODE_CR_RR ? C : c;
+        const int J = (MODE == MODE_PV || MODE == MODE_RR_RC) ? C : c;
+        nbj[q] = (J + 31) >> 5;
+        first[q + 1] = first[q] + (c > 0 ? ((I + 31) >> 5) * nbj[q] : 0);
     }
-    const bool small = cmax <= 32 && C <= 32;
+    const int total = first[GROUPS_PER_WG];
 
-    if (small) {
-        // ---------------- one group per wavefront ----------------
-        float* At = lds + wave * WAVE_LDS;
-        float* Bs = At + KC * 36;
-        const bool active = cw > 0;
-        GroupDims d = {0, 0, 0, 0, 0, 0};
-        int64_t rs = 0, ss = 0;
-        if (active) {
-            rs = gt.row_start[gw];
-            ss = gt.sq_start[gw];
-            d = group_dims<MODE>(cw, C, rs, ss);
-        }
-        const T* A = m1 + d.a_off;
-        const T* B = m2 + d.b_off;
-        stage_transposed<64, 32, T>(A, d.I, d.K, 0, 0, At, lane);
-        if (b_is_kmajor<MODE>()) stage_direct<64, 32, T>(B, d.K, d.J, 0, 0, Bs, lane);
-        else stage_transposed<64, 32, T>(B, d.J, d.K, 0, 0, Bs, lane);
-        if (EMIT && active && lane < cw) pos_s[wave * 32 + lane] = tok_pos[(rs + lane) * C];
-        __syncthreads();
-        float acc[4][4] = {};
-        const int ti = lane >> 3, tj = lane & 7;
-        multiply_chunk<32, 32>(At, Bs, ti, tj, d.K, acc);
-        if (active) {
-            store_tile<T>(out + d.o_off, d.I, d.J, 4 * ti, 4 * tj, acc);
-            if (EMIT)
-                emit_indices<64, MODE == MODE_QK>(out_idx, out_nnz, d.o_off, cw, C, gt.window[gw], gt.head[gw],
-                                                  pos_s + wave * 32, lane);
-        }
-        return;
-    }
-
-    // ---------------- whole workgroup per group, groups one after another ----------------
-    float* At = lds;
-    float* Bs = lds + KC * (BS::IB + 4);
-    constexpr int TJ = BS::JB / 4;
-    const int ti = tid / TJ, tj = tid % TJ;
-    for (int q = 0; q < GROUPS_PER_WG; ++q) {
+    for (int t = wave; t < total; t += 4) {
+        int q = 0;
+#pragma unroll
+        for (int qq = 1; qq < GROUPS_PER_WG; ++qq) q += (t >= first[qq]) ? 1 : 0;
+        int c = cq[0], nj = nbj[0], f0 = first[0];
+#pragma unroll
+        for (int qq = 1; qq < GROUPS_PER_WG; ++qq)
+            if (q == qq) { c = cq[qq]; nj = nbj[qq]; f0 = first[qq]; }
         const int64_t g = g0 + q;
-        if (g >= G) break;                                   // uniform across the workgroup
-        const int c = gt.c[g];
+        const int local = t - f0;
+        const int bi = local / nj, bj = local - bi * nj;
         const int64_t rs = gt.row_start[g], ss = gt.sq_start[g];
         const GroupDims d = group_dims<MODE>(c, C, rs, ss);
+        const int i_a = bi * 32 + l32;           // operand row of A this lane feeds
+        const int j_b = bj * 32 + l32;           // operand column of B this lane feeds
+
+        // positions for the index rows; issued first so their latency hides behind the product
+        int pos_i[16], pos_j = 0, win = 0, hd_ = 0;
+        if (EMIT) {
+            win = gt.window[g];
+            hd_ = gt.head[g];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int i = bi * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+                pos_i[r] = i < c ? tok_pos[(rs + i) * C] : 0;
+            }
+            if (MODE == MODE_QK) pos_j = j_b < c ? tok_pos[(rs + j_b) * C] : 0;
+        }
+
         const T* A = m1 + d.a_off;
         const T* B = m2 + d.b_off;
-        T* O = out + d.o_off;
-        for (int ib = 0; ib < d.I; ib += BS::IB) {
-            for (int jb = 0; jb < d.J; jb += BS::JB) {
-                float acc[4][4] = {};
-                for (int k0 = 0; k0 < d.K; k0 += KC) {
-                    __syncthreads();                          // previous chunk fully consumed
-                    stage_transposed<256, BS::IB, T>(A, d.I, d.K, ib, k0, At, tid);
-                    if (b_is_kmajor<MODE>()) stage_direct<256, BS::JB, T>(B, d.K, d.J, k0, jb, Bs, tid);
-                    else stage_transposed<256, BS::JB, T>(B, d.J, d.K, jb, k0, Bs, tid);
-                    __syncthreads();
-                    const int kmax = d.K - k0 < KC ? d.K - k0 : KC;
-                    multiply_chunk<BS::IB, BS::JB>(At, Bs, ti, tj, kmax, acc);
+        f32x16 acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        for (int kc = 0; kc < d.K; kc += 32) {
+            const int kb = kc + half * 16;
+            const int left = d.K - kb;                          // values of k left for this lane half
+            float a[16], b[16];
+            load_run16<T>(A + (int64_t)i_a * d.K + kb, i_a < d.I ? clamp16(left) : 0, a);
+            if (b_is_kmajor<MODE>()) {
+                const T* bp = B + (int64_t)kb * d.J + j_b;
+                const bool jin = j_b < d.J;
+#pragma unroll
+                for (int s = 0; s < 16; ++s) b[s] = (jin && s < left) ? to_acc(bp[(int64_t)s * d.J]) : 0.f;
+            } else {
+                load_run16<T>(B + (int64_t)j_b * d.K + kb, j_b < d.J ? clamp16(left) : 0, b);
+            }
+            const int steps = d.K - kc;                          // uniform: steps that carry data
+#pragma unroll
+            for (int s = 0; s < 16; ++s)
+                if (s < steps) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], acc, 0, 0, 0);
+        }
+
+        if (j_b < d.J) {
+            T* O = out + d.o_off + j_b;
+            int32_t* X = EMIT ? out_idx + d.o_off + j_b : nullptr;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int i = bi * 32 + 8 * (r >> 2) + 4 * half + (r & 3);
+                if (i < d.I) {
+                    const int64_t off = (int64_t)i * d.J;
+                    O[off] = from_acc<T>(acc[r]);
+                    if (EMIT) {
+                        X[off] = win;
+                        X[off + out_nnz] = hd_;
+                        X[off + 2 * out_nnz] = pos_i[r];
+                        X[off + 3 * out_nnz] = MODE == MODE_QK ? pos_j : j_b;
+                    }
                 }
-                store_tile<T>(O, d.I, d.J, ib + 4 * ti, jb + 4 * tj, acc);
             }
         }
-        if (EMIT) {
-            __syncthreads();                                  // pos_s of the previous group consumed
-            for (int i = tid; i < c; i += 256) pos_s[i] = tok_pos[(rs + i) * C];
-            __syncthreads();
-            emit_indices<256, MODE == MODE_QK>(out_idx, out_nnz, d.o_off, c, C, gt.window[g], gt.head[g], pos_s,
-                                               tid);
-        }
+    }
+}
+
+// COO index rows for one group, written by NT threads of one workgroup (simple kernel only).
+template <int NT, bool IS_QK>
+__device__ __forceinline__ void emit_indices(int32_t* __restrict__ out_idx, int64_t out_nnz, int64_t base,
+                                             int c, int C, int w, int h, const int* __restrict__ pos,
+                                             int tid) {
+    const int J = IS_QK ? c : C;
+    const int count = c * J;
+    int32_t* r0 = out_idx + base;
+    for (int f = tid; f < count; f += NT) {
+        const int i = f / J, j = f - i * J;
+        r0[f] = w;
+        r0[f + out_nnz] = h;
+        r0[f + 2 * out_nnz] = pos[i];
+        r0[f + 3 * out_nnz] = IS_QK ? pos[j] : j;
     }
 }
 
@@ -372,7 +293,7 @@ static int launch_product(const void* m1, const void* m2, const GroupTable& gt, 
         if (!force_simple()) {
             tiled = true;
             const unsigned blocks = (unsigned)((G + GROUPS_PER_WG - 1) / GROUPS_PER_WG);
-            hipLaunchKernelGGL((block_product_kernel<T, MODE, EMIT>), dim3(blocks), dim3(256), 0, s,
+            hipLaunchKernelGGL((block_product_mfma_kernel<T, MODE, EMIT>), dim3(blocks), dim3(256), 0, s,
                                static_cast<const T*>(m1), static_cast<const T*>(m2), gt, G, C, tok_pos,
                                static_cast<T*>(out), out_idx, out_nnz);
         }
