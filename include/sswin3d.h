@@ -157,6 +157,53 @@ int sswin_softmax_last_dim_forward(const int32_t* idx_row, const void* values, i
 int sswin_softmax_last_dim_backward(const int32_t* idx_row, const void* y, const void* grad,
                                     int dtype, int64_t A, void* out, void* stream);
 
+/* ---- fused window attention (replaces Python glue of the reference, no operator of ops.h) ---- */
+
+/* Token plan: what sparse_swin/swin3d_base.py:483-498 (qkv_sparse_cuda: index expansion, two
+ * sorts, five gathers) and :673-675 (permute, return_inverse, un-sort gather) establish by
+ * sorting, derived once from the [N,2] (window, pos) voxel indices without any sort.
+ * tokens (device int32 [5*N]): five rows of N entries indexed by token rank r (rank in
+ *   (window, pos) order): voxel of rank r; rank of the first token of its window; tokens of its
+ *   window; pos; window.
+ * plan (device int32 [5*g_cap]): rows c, T (rank of the window's first token), sq_start
+ *   (exclusive scan of c*c over groups), window, head — groups ordered (window, head).
+ * totals_out (host, 4 x int64): {groups G, non-empty windows, sum over groups of c*c, max c}.
+ * (window, pos) pairs must be distinct, window in [0,B), pos in [0,n).  Synchronises `stream`. */
+size_t sswin_token_plan_workspace_bytes(int64_t N, int B, int n);
+int sswin_token_plan(const int32_t* indices, int64_t N, int B, int n, int H, int32_t* tokens,
+                     int32_t* plan, int64_t g_cap, int64_t* totals_out, void* ws, size_t ws_bytes,
+                     void* stream);
+
+/* Token tensors are dense [N, stride] arrays of `dtype`; element (voxel v, head h, channel ch) is
+ * base[v*stride + col0 + h*hd + ch].  "sq" arrays are fp32 arrays of all [c x c] blocks.
+ *
+ * tokens x tokens -> sq: out[g][i][j] = sum_ch (scale_a * A[token i, ch]) * B[token j, ch].
+ * With epilogue != 0 (the product S = Q K^T of swin3d_base.py:660-668): adds
+ * bias[h, pos_i, pos_j] (fp32 [H,n,n], :557-566) and, if mask != NULL (int8 [n_mask_windows, n]
+ * region ids, :569-581), -100 where the regions of the two tokens differ; row_ids (optional)
+ * receives the softmax row id H*T + h*c + i of every element.  Asynchronous. */
+int sswin_fused_tokens_to_sq(int dtype, int epilogue, const int32_t* plan, int64_t g_cap, int64_t G,
+                             const int32_t* tokens, int64_t N, int H, int hd, const void* a_base,
+                             int64_t a_stride, int a_col0, const void* b_base, int64_t b_stride,
+                             int b_col0, float scale_a, const float* bias, int n, const int8_t* mask,
+                             int n_mask_windows, float* out, int32_t* row_ids, void* stream);
+
+/* sq x tokens -> tokens: out[token i, ch] = scale_out * sum_k A(i,k) * B[token k, ch] with
+ * A(i,k) = sq[g][i][k] (a_kmajor = 0: O = P V, dQ = dS K) or sq[g][k][i] (a_kmajor = 1:
+ * dV = P^T dO, dK = dS^T Q).  Every (voxel, head, channel) of the output is written once.
+ * Replaces 'qk_v' + permute + un-sort (swin3d_base.py:672-675) and the backward products with
+ * their transposes (:119-134).  Asynchronous. */
+int sswin_fused_sq_to_tokens(int dtype, int a_kmajor, const int32_t* plan, int64_t g_cap, int64_t G,
+                             const int32_t* tokens, int64_t N, int hd, const float* sq,
+                             const void* b_base, int64_t b_stride, int b_col0, void* o_base,
+                             int64_t o_stride, int o_col0, float scale_out, void* stream);
+
+/* d_bias[h, pos_i, pos_j] += ds over all windows (the backward of swin3d_base.py:557-566, which
+ * autograd performs as an index_add).  d_bias: fp32 [H,n,n], zeroed by the caller.  n*n*4 bytes
+ * must fit 64 KiB of LDS.  Uses float atomics (summation order varies).  Asynchronous. */
+int sswin_fused_bias_grad(const int32_t* plan, int64_t g_cap, int64_t G, const int32_t* tokens,
+                          int64_t N, int H, int n, const float* ds, float* d_bias, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -14,7 +14,7 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libsswin3d.so")
-SOURCES = ["index_ops.hip", "plan.hip", "block_matmul.hip", "softmax.hip"]
+SOURCES = ["index_ops.hip", "plan.hip", "block_matmul.hip", "softmax.hip", "fused_attention.hip"]
 ARCH = "gfx950"
 # packed FP32 instructions are switched off for all device code on purpose
 FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}",
@@ -44,7 +44,7 @@ def build(verbose: bool = False) -> str:
             print(r.stderr, file=sys.stderr)
         return obj
 
-    with ThreadPoolExecutor(max_workers=4) as ex:
+    with ThreadPoolExecutor(max_workers=5) as ex:
         objs = list(ex.map(compile_one, SOURCES))
     cmd = [hipcc, "-shared", "-fPIC", f"--offload-arch={ARCH}", *objs, "-o", OUT]
     r = subprocess.run(cmd, capture_output=True, text=True)

@@ -29,6 +29,7 @@
 #include <cstdlib>
 #include <type_traits>
 
+#include "mfma_block.hpp"
 #include "sswin_common.hpp"
 
 namespace sswin {
@@ -37,9 +38,6 @@ enum { MODE_QK = 0, MODE_PV = 1, MODE_RC_CR = 2, MODE_RR_RC = 3, MODE_CR_RR = 4 
 
 constexpr int GROUPS_PER_WG = 4;
 constexpr int MAX_POS = 1024;          // largest window occupancy the simple kernel's LDS table holds
-
-typedef float f32x4_u __attribute__((ext_vector_type(4), aligned(4)));
-typedef float f32x16 __attribute__((ext_vector_type(16)));
 
 template <int MODE> __host__ __device__ constexpr bool b_is_kmajor() { return MODE == MODE_QK || MODE == MODE_PV; }
 
@@ -65,29 +63,6 @@ struct GroupTable {
     const int32_t* window;     // [G] or null
     const int32_t* head;       // [G] or null
 };
-
-// 16 consecutive values of one operand row, zero beyond `valid` (0..16).
-template <typename T>
-__device__ __forceinline__ void load_run16(const T* __restrict__ p, int valid, float (&x)[16]) {
-    if (valid >= 16) {
-        if (std::is_same<T, float>::value) {
-            const f32x4_u* q = reinterpret_cast<const f32x4_u*>(p);
-#pragma unroll
-            for (int v = 0; v < 4; ++v) {
-                const f32x4_u t = q[v];
-                x[4 * v] = t.x; x[4 * v + 1] = t.y; x[4 * v + 2] = t.z; x[4 * v + 3] = t.w;
-            }
-        } else {
-#pragma unroll
-            for (int s = 0; s < 16; ++s) x[s] = to_acc(p[s]);
-        }
-    } else {
-#pragma unroll
-        for (int s = 0; s < 16; ++s) x[s] = s < valid ? to_acc(p[s]) : 0.f;
-    }
-}
-
-__device__ __forceinline__ int clamp16(int v) { return v < 0 ? 0 : (v > 16 ? 16 : v); }
 
 template <typename T, int MODE, bool EMIT>
 __global__ __launch_bounds__(256) void block_product_mfma_kernel(const T* __restrict__ m1, const T* __restrict__ m2,

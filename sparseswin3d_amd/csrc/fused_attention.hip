@@ -1,0 +1,515 @@
+// Fused window-attention path used inside WindowAttentionSparse.
+//
+// The reference assembles Q, K^T and V as sorted COO copies of the dense qkv tensor
+// (sparse_swin/swin3d_base.py:483-498), multiplies them, adds bias and mask with index_select
+// passes (:557-581), and un-sorts the result with a permute + return_inverse + index_select
+// (:673-675).  Here the MFMA block products read token rows straight from the dense tensors
+// through the token order, so none of those copies exist:
+//
+//   token plan   (window, pos) voxel indices -> token order, per-group table          (sswin_token_plan)
+//   tokens -> sq S = (scale*Q) K^T + bias + mask   or   dP = dO V^T                    (fused_sq_kernel)
+//   sq -> tokens O = P V, dV = P^T dO, dQ = scale * dS K, dK = scale * dS^T Q        (fused_tok_kernel)
+//   bias grad    d_rpb[h, p_i, p_j] += dS                                             (rpb_grad_kernel)
+//
+// "sq" arrays are fp32 arrays of all [c x c] blocks in group order (group = window, head);
+// token tensors are [N, row_stride] arrays addressed as row order[T_k + i], column col0 + h*hd + ch.
+// The softmax between the two products is the ordinary sparse row softmax; its row ids are a
+// by-product of the first kernel.
+#include <algorithm>
+
+#include "mfma_block.hpp"
+#include "scan.hpp"
+#include "sswin_common.hpp"
+
+namespace sswin {
+
+constexpr int FUSED_GROUPS_PER_WG = 4;
+
+// ------------------------------------------------------------------------------------------
+// token plan
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void tp_fill_kernel(uint32_t* __restrict__ p, int64_t n, uint32_t v) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) p[i] = v;
+}
+
+__global__ __launch_bounds__(256) void tp_set_bits_kernel(const int32_t* __restrict__ ind, int64_t N, int n,
+                                                          uint32_t* __restrict__ bits) {
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < N) {
+        const int2 wp = *reinterpret_cast<const int2*>(ind + 2 * i);
+        const uint64_t v = (uint64_t)(uint32_t)wp.x * (uint32_t)n + (uint32_t)wp.y;
+        atomicOr(&bits[v >> 5], 1u << (v & 31));
+    }
+}
+
+struct TpPopcLoad {
+    const uint32_t* bits;
+    __device__ int operator()(int64_t i) const { return __popc(bits[i]); }
+};
+struct TpExclusiveStore {
+    int32_t* out;
+    __device__ void operator()(int64_t i, int ex, int) const { out[i] = ex; }
+};
+
+__device__ __forceinline__ int tp_rank_of_bit(const uint32_t* __restrict__ bits,
+                                              const int32_t* __restrict__ word_prefix, uint64_t v) {
+    const uint64_t w = v >> 5;
+    return word_prefix[w] + __popc(bits[w] & ((1u << (v & 31)) - 1u));
+}
+
+// per voxel -> entries by token rank: source voxel, first rank and size of its window, pos, window
+__global__ __launch_bounds__(256) void tp_rank_kernel(const int32_t* __restrict__ ind, int64_t N, int n,
+                                                      const uint32_t* __restrict__ bits,
+                                                      const int32_t* __restrict__ word_prefix,
+                                                      int32_t* __restrict__ order, int32_t* __restrict__ tok_T,
+                                                      int32_t* __restrict__ tok_c, int32_t* __restrict__ tok_pos,
+                                                      int32_t* __restrict__ tok_win) {
+    const int64_t v = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (v >= N) return;
+    const int2 wp = *reinterpret_cast<const int2*>(ind + 2 * v);
+    const uint64_t first = (uint64_t)(uint32_t)wp.x * (uint32_t)n;
+    const int r = tp_rank_of_bit(bits, word_prefix, first + (uint32_t)wp.y);
+    const int T = tp_rank_of_bit(bits, word_prefix, first);
+    const int Tn = tp_rank_of_bit(bits, word_prefix, first + (uint32_t)n);
+    order[r] = (int32_t)v;
+    tok_T[r] = T;
+    tok_c[r] = Tn - T;
+    tok_pos[r] = wp.y;
+    tok_win[r] = wp.x;
+}
+
+// scan over token ranks: item = 1 | c*c << 32 at the first token of a window
+struct WindowLoad {
+    const int32_t* tok_T;
+    const int32_t* tok_c;
+    __device__ int64_t operator()(int64_t r) const {
+        if (tok_T[r] != (int32_t)r) return 0;
+        const int64_t c = tok_c[r];
+        return (int64_t)1 | ((c * c) << 32);
+    }
+};
+struct WindowStore {
+    const int32_t* tok_c;
+    const int32_t* tok_win;
+    int32_t* plan;
+    int64_t g_cap;
+    int H;
+    int32_t* cmax;
+    __device__ void operator()(int64_t r, int64_t ex, int64_t item) const {
+        if (item == 0) return;
+        const int64_t k = ex & 0xffffffffll;          // rank of the window among non-empty windows
+        const int64_t q2 = ex >> 32;                  // sum of c*c over earlier windows
+        const int c = tok_c[r];
+        const int w = tok_win[r];
+        for (int h = 0; h < H; ++h) {
+            const int64_t g = k * H + h;
+            if (g >= g_cap) return;
+            plan[g] = c;
+            plan[g_cap + g] = (int32_t)r;             // T_k: rank of the window's first token
+            plan[2 * g_cap + g] = (int32_t)(q2 * H + (int64_t)h * c * c);
+            plan[3 * g_cap + g] = w;
+            plan[4 * g_cap + g] = h;
+        }
+        if (c > *cmax) atomicMax(cmax, c);
+    }
+};
+
+__global__ void tp_zero_kernel(int32_t* p, int n) {
+    if ((int)threadIdx.x < n) p[threadIdx.x] = 0;
+}
+
+// ------------------------------------------------------------------------------------------
+// group table of the fused kernels
+// ------------------------------------------------------------------------------------------
+struct FusedGroups {
+    const int32_t* c;        // tokens of the group's window
+    const int32_t* T;        // rank of the window's first token
+    const int32_t* sq;       // start of the group's [c x c] block in sq arrays
+    const int32_t* window;
+    const int32_t* head;
+    int64_t G;
+};
+
+struct TokenTensor {         // rows addressed by voxel, columns col0 + h*hd + ch
+    const void* base;
+    int64_t stride;
+    int col0;
+};
+
+// work distribution: four consecutive groups per workgroup, their 32-row x 32-column blocks dealt
+// round robin to the four wavefronts
+struct TaskSet {
+    int c[FUSED_GROUPS_PER_WG], nbj[FUSED_GROUPS_PER_WG], first[FUSED_GROUPS_PER_WG + 1];
+};
+
+__device__ __forceinline__ TaskSet make_tasks(const FusedGroups& gt, int64_t g0, bool square, int hd) {
+    TaskSet t;
+    t.first[0] = 0;
+#pragma unroll
+    for (int q = 0; q < FUSED_GROUPS_PER_WG; ++q) {
+        const int64_t g = g0 + q;
+        const int c = g < gt.G ? gt.c[g] : 0;
+        t.c[q] = c;
+        t.nbj[q] = square ? (c + 31) >> 5 : (hd + 31) >> 5;
+        t.first[q + 1] = t.first[q] + (c > 0 ? ((c + 31) >> 5) * t.nbj[q] : 0);
+    }
+    return t;
+}
+
+__device__ __forceinline__ void locate_task(const TaskSet& ts, int t, int& q, int& c, int& bi, int& bj) {
+    q = 0;
+#pragma unroll
+    for (int qq = 1; qq < FUSED_GROUPS_PER_WG; ++qq) q += (t >= ts.first[qq]) ? 1 : 0;
+    c = ts.c[0];
+    int nj = ts.nbj[0], f0 = ts.first[0];
+#pragma unroll
+    for (int qq = 1; qq < FUSED_GROUPS_PER_WG; ++qq)
+        if (q == qq) { c = ts.c[qq]; nj = ts.nbj[qq]; f0 = ts.first[qq]; }
+    const int local = t - f0;
+    bi = local / nj;
+    bj = local - bi * nj;
+}
+
+// ------------------------------------------------------------------------------------------
+// tokens x tokens -> sq :  out[i, j] = sum_ch A[token i, ch] * B[token j, ch]   (K = hd)
+//   EPI = true : S = scale*acc + bias[h, pos_i, pos_j] + (mask region differs ? -100 : 0), row ids
+//   EPI = false: plain product (dP = dO V^T)
+// ------------------------------------------------------------------------------------------
+template <typename T, bool EPI>
+__global__ __launch_bounds__(256) void fused_sq_kernel(FusedGroups gt, const int32_t* __restrict__ order,
+                                                       const int32_t* __restrict__ tok_pos, int H, int hd,
+                                                       TokenTensor ta, TokenTensor tb, float scale_a,
+                                                       const float* __restrict__ bias, int n,
+                                                       const int8_t* __restrict__ mask, int n_mask_windows,
+                                                       float* __restrict__ out, int32_t* __restrict__ row_ids) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int half = lane >> 5, l32 = lane & 31;
+    const int64_t g0 = (int64_t)blockIdx.x * FUSED_GROUPS_PER_WG;
+    const TaskSet ts = make_tasks(gt, g0, true, hd);
+    const int total = ts.first[FUSED_GROUPS_PER_WG];
+    const T* A = static_cast<const T*>(ta.base);
+    const T* B = static_cast<const T*>(tb.base);
+
+    for (int t = wave; t < total; t += 4) {
+        int q, c, bi, bj;
+        locate_task(ts, t, q, c, bi, bj);
+        const int64_t g = g0 + q;
+        const int Tk = gt.T[g], h = gt.head[g];
+        const int64_t sq0 = gt.sq[g];
+        const int i_a = bi * 32 + l32, j_b = bj * 32 + l32;
+        const bool a_in = i_a < c, b_in = j_b < c;
+        const T* pa = A + (a_in ? (int64_t)order[Tk + i_a] * ta.stride : 0) + ta.col0 + h * hd;
+        const T* pb = B + (b_in ? (int64_t)order[Tk + j_b] * tb.stride : 0) + tb.col0 + h * hd;
+
+        // epilogue inputs first: their latency hides behind the product
+        int pos_i[16], pos_j = 0, m_j = 0;
+        const int8_t* mrow = nullptr;
+        if (EPI) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int i = bi * 32 + acc_row(r, half);
+                pos_i[r] = i < c ? tok_pos[Tk + i] : 0;
+            }
+            pos_j = b_in ? tok_pos[Tk + j_b] : 0;
+            if (mask) {
+                mrow = mask + (int64_t)(gt.window[g] % n_mask_windows) * n;
+                m_j = mrow[pos_j];
+            }
+        }
+
+        f32x16 acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        for (int kc = 0; kc < hd; kc += 32) {
+            const int kb = kc + half * 16;
+            const int left = hd - kb;
+            float a[16], b[16];
+            load_run16<T>(pa + kb, a_in ? clamp16(left) : 0, a);
+            load_run16<T>(pb + kb, b_in ? clamp16(left) : 0, b);
+            if (scale_a != 1.0f) {
+#pragma unroll
+                for (int s = 0; s < 16; ++s) a[s] *= scale_a;
+            }
+            const int steps = hd - kc;
+#pragma unroll
+            for (int s = 0; s < 16; ++s)
+                if (s < steps) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], acc, 0, 0, 0);
+        }
+
+        if (b_in) {
+            float* O = out + sq0 + j_b;
+            const float* brow = EPI ? bias + (int64_t)h * n * n + pos_j : nullptr;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int i = bi * 32 + acc_row(r, half);
+                if (i < c) {
+                    float v = acc[r];
+                    if (EPI) {
+                        v += brow[(int64_t)pos_i[r] * n];
+                        if (mask && mrow[pos_i[r]] != m_j) v += -100.0f;
+                        if (row_ids) row_ids[sq0 + (int64_t)i * c + j_b] = H * Tk + h * c + i;
+                    }
+                    O[(int64_t)i * c] = v;
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// sq x tokens -> tokens :  out[token i, ch] = scale * sum_k A(i, k) * B[token k, ch]   (K = c)
+//   A_KMAJOR = false: A(i, k) = sq[i*c + k]   (O = P V, dQ = dS K)
+//   A_KMAJOR = true : A(i, k) = sq[k*c + i]   (dV = P^T dO, dK = dS^T Q)
+// ------------------------------------------------------------------------------------------
+template <typename T, bool A_KMAJOR>
+__global__ __launch_bounds__(256) void fused_tok_kernel(FusedGroups gt, const int32_t* __restrict__ order, int hd,
+                                                        const float* __restrict__ sq, TokenTensor tb,
+                                                        TokenTensor to, float scale_out) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int half = lane >> 5, l32 = lane & 31;
+    const int64_t g0 = (int64_t)blockIdx.x * FUSED_GROUPS_PER_WG;
+    const TaskSet ts = make_tasks(gt, g0, false, hd);
+    const int total = ts.first[FUSED_GROUPS_PER_WG];
+    const T* B = static_cast<const T*>(tb.base);
+    T* O = static_cast<T*>(const_cast<void*>(to.base));
+
+    for (int t = wave; t < total; t += 4) {
+        int q, c, bi, bj;
+        locate_task(ts, t, q, c, bi, bj);
+        const int64_t g = g0 + q;
+        const int Tk = gt.T[g], h = gt.head[g];
+        const float* S = sq + gt.sq[g];
+        const int i_a = bi * 32 + l32, j_b = bj * 32 + l32;
+        const bool a_in = i_a < c, b_in = j_b < hd;
+
+        // output rows of this lane half
+        int64_t orow[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int i = bi * 32 + acc_row(r, half);
+            orow[r] = i < c ? (int64_t)order[Tk + i] * to.stride : -1;
+        }
+
+        f32x16 acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        for (int kc = 0; kc < c; kc += 32) {
+            const int kb = kc + half * 16;
+            const int left = c - kb;                              // k values left for this lane half
+            float a[16], b[16];
+            if (!A_KMAJOR) {
+                load_run16<float>(S + (int64_t)i_a * c + kb, a_in ? clamp16(left) : 0, a);
+            } else {
+#pragma unroll
+                for (int s = 0; s < 16; ++s) a[s] = (a_in && s < left) ? S[(int64_t)(kb + s) * c + i_a] : 0.f;
+            }
+#pragma unroll
+            for (int s = 0; s < 16; ++s) {
+                float v = 0.f;
+                if (b_in && s < left) v = to_acc(B[(int64_t)order[Tk + kb + s] * tb.stride + tb.col0 + h * hd + j_b]);
+                b[s] = v;
+            }
+            const int steps = c - kc;
+#pragma unroll
+            for (int s = 0; s < 16; ++s)
+                if (s < steps) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], acc, 0, 0, 0);
+        }
+
+        if (b_in) {
+            const int col = to.col0 + h * hd + j_b;
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                if (orow[r] >= 0) O[orow[r] + col] = from_acc<T>(acc[r] * scale_out);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// gradient of the relative position bias: d_rpb[h, pos_i, pos_j] += dS over all windows.
+// grid (slices, H).  Each workgroup accumulates its windows into an LDS copy of one head's table
+// (LDS float atomics) and flushes the non-zero entries with one global atomic each.
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void rpb_grad_kernel(FusedGroups gt, const int32_t* __restrict__ tok_pos, int H,
+                                                       int n, const float* __restrict__ ds,
+                                                       float* __restrict__ d_rpb) {
+    extern __shared__ float table[];
+    const int h = blockIdx.y;
+    const int nn = n * n;
+    for (int e = threadIdx.x; e < nn; e += 256) table[e] = 0.f;
+    __syncthreads();
+    const int64_t windows = gt.G / H;
+    for (int64_t k = blockIdx.x; k < windows; k += gridDim.x) {
+        const int64_t g = k * H + h;
+        const int c = gt.c[g], Tk = gt.T[g];
+        const float* S = ds + gt.sq[g];
+        const int count = c * c;
+        for (int f = threadIdx.x; f < count; f += 256) {
+            const int i = f / c, j = f - i * c;
+            atomicAdd(&table[tok_pos[Tk + i] * n + tok_pos[Tk + j]], S[f]);
+        }
+    }
+    __syncthreads();
+    float* dst = d_rpb + (int64_t)h * nn;
+    for (int e = threadIdx.x; e < nn; e += 256) {
+        const float v = table[e];
+        if (v != 0.f) atomicAdd(&dst[e], v);
+    }
+}
+
+template <typename T>
+static int launch_sq(bool epi, const FusedGroups& gt, const int32_t* order, const int32_t* tok_pos, int H, int hd,
+                     const TokenTensor& ta, const TokenTensor& tb, float scale_a, const float* bias, int n,
+                     const int8_t* mask, int nmw, float* out, int32_t* row_ids, hipStream_t s) {
+    const unsigned blocks = (unsigned)((gt.G + FUSED_GROUPS_PER_WG - 1) / FUSED_GROUPS_PER_WG);
+    if (epi)
+        hipLaunchKernelGGL((fused_sq_kernel<T, true>), dim3(blocks), dim3(256), 0, s, gt, order, tok_pos, H, hd, ta,
+                           tb, scale_a, bias, n, mask, nmw, out, row_ids);
+    else
+        hipLaunchKernelGGL((fused_sq_kernel<T, false>), dim3(blocks), dim3(256), 0, s, gt, order, tok_pos, H, hd, ta,
+                           tb, scale_a, bias, n, mask, nmw, out, row_ids);
+    return launch_ok("fused tokens->sq product");
+}
+
+template <typename T>
+static int launch_tok(bool a_kmajor, const FusedGroups& gt, const int32_t* order, int hd, const float* sq,
+                      const TokenTensor& tb, const TokenTensor& to, float scale_out, hipStream_t s) {
+    const unsigned blocks = (unsigned)((gt.G + FUSED_GROUPS_PER_WG - 1) / FUSED_GROUPS_PER_WG);
+    if (a_kmajor)
+        hipLaunchKernelGGL((fused_tok_kernel<T, true>), dim3(blocks), dim3(256), 0, s, gt, order, hd, sq, tb, to,
+                           scale_out);
+    else
+        hipLaunchKernelGGL((fused_tok_kernel<T, false>), dim3(blocks), dim3(256), 0, s, gt, order, hd, sq, tb, to,
+                           scale_out);
+    return launch_ok("fused sq->tokens product");
+}
+
+static FusedGroups groups_of(const int32_t* plan, int64_t g_cap, int64_t G) {
+    return FusedGroups{plan, plan + g_cap, plan + 2 * g_cap, plan + 3 * g_cap, plan + 4 * g_cap, G};
+}
+
+}  // namespace sswin
+
+using namespace sswin;
+
+extern "C" {
+
+static size_t tp_words(int B, int n) { return (size_t)(((int64_t)B * n + n + 31) / 32) + 1; }
+
+size_t sswin_token_plan_workspace_bytes(int64_t N, int B, int n) {
+    const size_t words = tp_words(B, n);
+    const size_t tiles = (size_t)std::max<int64_t>(scan_num_tiles((int64_t)words), scan_num_tiles(N > 0 ? N : 1));
+    return align_up(words * 4, 256) * 2 + align_up(tiles * 8, 256) + 1024;
+}
+
+int sswin_token_plan(const int32_t* indices, int64_t N, int B, int n, int H, int32_t* tokens,
+                     int32_t* plan, int64_t g_cap, int64_t* totals_out, void* ws, size_t ws_bytes,
+                     void* stream) {
+    SSWIN_CHECK(N >= 0 && B > 0 && n > 0 && H > 0, "token_plan: bad sizes");
+    SSWIN_CHECK(totals_out, "token_plan: totals_out is null");
+    totals_out[0] = totals_out[1] = totals_out[2] = totals_out[3] = 0;
+    if (N == 0) return 0;
+    SSWIN_CHECK(indices && tokens && plan && ws, "token_plan: null pointer");
+    SSWIN_CHECK(N < (int64_t)INT32_MAX, "token_plan: too many voxels");
+    SSWIN_CHECK(g_cap > 0, "token_plan: g_cap must be positive");
+    SSWIN_CHECK(ws_bytes >= sswin_token_plan_workspace_bytes(N, B, n), "token_plan: workspace too small");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    Carver cv(ws, ws_bytes);
+    const size_t words = tp_words(B, n);
+    int64_t* total_dev = cv.take<int64_t>(2);
+    uint32_t* bits = cv.take<uint32_t>(words);
+    int32_t* word_prefix = cv.take<int32_t>(words);
+    int64_t* tile_sums = cv.take<int64_t>(
+        (size_t)std::max<int64_t>(scan_num_tiles((int64_t)words), scan_num_tiles(N)));
+    SSWIN_CHECK(cv.ok(), "token_plan: workspace too small");
+    int32_t* order = tokens;
+    int32_t* tok_T = tokens + N;
+    int32_t* tok_c = tokens + 2 * N;
+    int32_t* tok_pos = tokens + 3 * N;
+    int32_t* tok_win = tokens + 4 * N;
+    int32_t* cmax = reinterpret_cast<int32_t*>(total_dev + 1);
+
+    const unsigned fill_blocks = (unsigned)std::min<size_t>((words + 255) / 256, 4096);
+    hipLaunchKernelGGL(tp_fill_kernel, dim3(fill_blocks), dim3(256), 0, s, bits, (int64_t)words, 0u);
+    hipLaunchKernelGGL(tp_zero_kernel, dim3(1), dim3(64), 0, s, cmax, 2);
+    const unsigned nb = (unsigned)((N + 255) / 256);
+    hipLaunchKernelGGL(tp_set_bits_kernel, dim3(nb), dim3(256), 0, s, indices, N, n, bits);
+    TpPopcLoad pl{bits};
+    TpExclusiveStore ps{word_prefix};
+    if (device_exclusive_scan<int32_t>(pl, ps, (int64_t)words, reinterpret_cast<int32_t*>(tile_sums),
+                                       (int32_t*)nullptr, s, "token_plan bitmap scan"))
+        return 1;
+    hipLaunchKernelGGL(tp_rank_kernel, dim3(nb), dim3(256), 0, s, indices, N, n, bits, word_prefix, order, tok_T,
+                       tok_c, tok_pos, tok_win);
+    WindowLoad wl{tok_T, tok_c};
+    WindowStore wst{tok_c, tok_win, plan, g_cap, H, cmax};
+    if (device_exclusive_scan<int64_t>(wl, wst, N, tile_sums, total_dev, s, "token_plan window scan")) return 1;
+    int64_t host[2] = {0, 0};
+    SSWIN_HIP(hipMemcpyAsync(host, total_dev, sizeof(host), hipMemcpyDeviceToHost, s));
+    SSWIN_HIP(hipStreamSynchronize(s));
+    const int64_t windows = host[0] & 0xffffffffll;
+    const int64_t s2 = host[0] >> 32;
+    SSWIN_CHECK(host[0] >= 0 && s2 * H < (int64_t)INT32_MAX,
+                "token_plan: the attention matrix has 2^31 or more non-zeros, which int32 offsets cannot address");
+    totals_out[0] = windows * H;
+    totals_out[1] = windows;
+    totals_out[2] = s2 * H;
+    totals_out[3] = (int32_t)(host[1] & 0xffffffffll);
+    SSWIN_CHECK(windows * H <= g_cap, "token_plan: %lld groups exceed the plan capacity %lld",
+                (long long)(windows * H), (long long)g_cap);
+    return 0;
+}
+
+int sswin_fused_tokens_to_sq(int dtype, int epilogue, const int32_t* plan, int64_t g_cap, int64_t G,
+                             const int32_t* tokens, int64_t N, int H, int hd, const void* a_base,
+                             int64_t a_stride, int a_col0, const void* b_base, int64_t b_stride, int b_col0,
+                             float scale_a, const float* bias, int n, const int8_t* mask, int n_mask_windows,
+                             float* out, int32_t* row_ids, void* stream) {
+    SSWIN_CHECK(G >= 0 && G <= g_cap && N >= 0 && H > 0 && hd > 0, "fused_tokens_to_sq: bad sizes");
+    if (G == 0) return 0;
+    SSWIN_CHECK(plan && tokens && a_base && b_base && out, "fused_tokens_to_sq: null pointer");
+    SSWIN_CHECK(!epilogue || (bias && n > 0), "fused_tokens_to_sq: the epilogue needs the bias table");
+    SSWIN_CHECK(!mask || n_mask_windows > 0, "fused_tokens_to_sq: mask without window count");
+    const FusedGroups gt = groups_of(plan, g_cap, G);
+    const TokenTensor ta{a_base, a_stride, a_col0}, tb{b_base, b_stride, b_col0};
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int32_t* order = tokens;
+    const int32_t* tok_pos = tokens + 3 * N;
+    switch (dtype) {
+        case SSWIN_F32: return launch_sq<float>(epilogue, gt, order, tok_pos, H, hd, ta, tb, scale_a, bias, n, mask, n_mask_windows, out, row_ids, s);
+        case SSWIN_F16: return launch_sq<__half>(epilogue, gt, order, tok_pos, H, hd, ta, tb, scale_a, bias, n, mask, n_mask_windows, out, row_ids, s);
+        case SSWIN_BF16: return launch_sq<__hip_bfloat16>(epilogue, gt, order, tok_pos, H, hd, ta, tb, scale_a, bias, n, mask, n_mask_windows, out, row_ids, s);
+        default: return fail("fused_tokens_to_sq: unsupported token dtype %d", dtype);
+    }
+}
+
+int sswin_fused_sq_to_tokens(int dtype, int a_kmajor, const int32_t* plan, int64_t g_cap, int64_t G,
+                             const int32_t* tokens, int64_t N, int hd, const float* sq, const void* b_base,
+                             int64_t b_stride, int b_col0, void* o_base, int64_t o_stride, int o_col0,
+                             float scale_out, void* stream) {
+    SSWIN_CHECK(G >= 0 && G <= g_cap && N >= 0 && hd > 0, "fused_sq_to_tokens: bad sizes");
+    if (G == 0) return 0;
+    SSWIN_CHECK(plan && tokens && sq && b_base && o_base, "fused_sq_to_tokens: null pointer");
+    const FusedGroups gt = groups_of(plan, g_cap, G);
+    const TokenTensor tb{b_base, b_stride, b_col0}, to{o_base, o_stride, o_col0};
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    switch (dtype) {
+        case SSWIN_F32: return launch_tok<float>(a_kmajor, gt, tokens, hd, sq, tb, to, scale_out, s);
+        case SSWIN_F16: return launch_tok<__half>(a_kmajor, gt, tokens, hd, sq, tb, to, scale_out, s);
+        case SSWIN_BF16: return launch_tok<__hip_bfloat16>(a_kmajor, gt, tokens, hd, sq, tb, to, scale_out, s);
+        default: return fail("fused_sq_to_tokens: unsupported token dtype %d", dtype);
+    }
+}
+
+int sswin_fused_bias_grad(const int32_t* plan, int64_t g_cap, int64_t G, const int32_t* tokens, int64_t N,
+                          int H, int n, const float* ds, float* d_bias, void* stream) {
+    SSWIN_CHECK(G >= 0 && G <= g_cap && H > 0 && n > 0, "fused_bias_grad: bad sizes");
+    if (G == 0) return 0;
+    SSWIN_CHECK(plan && tokens && ds && d_bias, "fused_bias_grad: null pointer");
+    SSWIN_CHECK((size_t)n * n * sizeof(float) <= 64 * 1024,
+                "fused_bias_grad: a window of %d positions needs a %zu-byte LDS table (limit 64 KiB)", n,
+                (size_t)n * n * sizeof(float));
+    const FusedGroups gt = groups_of(plan, g_cap, G);
+    const int64_t windows = G / H;
+    const unsigned slices = (unsigned)std::min<int64_t>(windows, 128);
+    hipLaunchKernelGGL(rpb_grad_kernel, dim3(slices, (unsigned)H), dim3(256), (size_t)n * n * sizeof(float),
+                       static_cast<hipStream_t>(stream), gt, tokens + 3 * N, H, n, ds, d_bias);
+    return launch_ok("fused bias gradient");
+}
+
+}  // extern "C"

@@ -1,0 +1,44 @@
+// Building blocks shared by the MFMA block-product kernels (gfx950, wave64).
+//
+// One wavefront computes one 32 x 32 output block with v_mfma_f32_32x32x2_f32.  Lane l feeds
+// A[i = l % 32][k] and B[k][j = l % 32]; inside a 32-wide k chunk, MFMA step s pairs k = s
+// (lanes 0-31) with k = 16 + s (lanes 32-63), so a row-contiguous operand is a run of 16
+// consecutive values per lane.  Accumulator register r of lane l is output element
+// (row 8*(r/4) + 4*(l/32) + r%4, column l % 32).
+#pragma once
+
+#include <type_traits>
+
+#include "sswin_common.hpp"
+
+namespace sswin {
+
+typedef float f32x4_u __attribute__((ext_vector_type(4), aligned(4)));
+typedef float f32x16 __attribute__((ext_vector_type(16)));
+
+// 16 consecutive values of one operand row, zero beyond `valid` (0..16).
+template <typename T>
+__device__ __forceinline__ void load_run16(const T* __restrict__ p, int valid, float (&x)[16]) {
+    if (valid >= 16) {
+        if (std::is_same<T, float>::value) {
+            const f32x4_u* q = reinterpret_cast<const f32x4_u*>(p);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                const f32x4_u t = q[v];
+                x[4 * v] = t.x; x[4 * v + 1] = t.y; x[4 * v + 2] = t.z; x[4 * v + 3] = t.w;
+            }
+        } else {
+#pragma unroll
+            for (int s = 0; s < 16; ++s) x[s] = to_acc(p[s]);
+        }
+    } else {
+#pragma unroll
+        for (int s = 0; s < 16; ++s) x[s] = s < valid ? to_acc(p[s]) : 0.f;
+    }
+}
+
+__device__ __forceinline__ int clamp16(int v) { return v < 0 ? 0 : (v > 16 ? 16 : v); }
+
+__device__ __forceinline__ int acc_row(int r, int half) { return 8 * (r >> 2) + 4 * half + (r & 3); }
+
+}  // namespace sswin

@@ -2,69 +2,148 @@
 //
 // A coalesced 4-D COO operand [B, H, n, inner] with a dense last dimension is a sequence of
 // token rows (one per `inner` consecutive columns), sorted by (window, head, pos).  A group is
-// a run of token rows with equal (window, head).  One packed scan yields, per group, its index
-// and the exclusive sum of c*c; the head row of a group is its exclusive sum of c.
+// a run of token rows with equal (window, head).
+//
+// plan_tile_kernel works on tiles of PLAN_TILE token rows: the (window, head) keys of the tile
+// are staged in LDS, run heads are found with wave ballots and compacted into a start table,
+// and the token count of a group is the distance to the next head (one look-ahead past the
+// tile end for the last head of the tile).  Pass 1 reduces (number of heads, sum of c*c) per
+// tile, a single block scans the tile sums, pass 2 repeats the tile work and writes the plan.
 #include "scan.hpp"
 #include "sswin_common.hpp"
 
 namespace sswin {
 
-struct RowKeys {
-    const int32_t* i0;   // idx row 0 (window)
-    const int32_t* i1;   // idx row 1 (head)
-    int64_t R;           // token rows
-    int inner;
-    __device__ bool same(int64_t a, int64_t b) const {
-        return i0[a * inner] == i0[b * inner] && i1[a * inner] == i1[b * inner];
-    }
-    __device__ bool is_head(int64_t r) const { return r == 0 || !same(r, r - 1); }
-    // number of token rows of the group starting at r (rows are sorted, so the group is the
-    // maximal run of rows equal to r): gallop, then bisect.
-    __device__ int64_t run_length(int64_t r) const {
-        int64_t lo = r, step = 1;            // lo: last row known equal
-        int64_t hi = R;                      // hi: first row known different (or R)
-        while (true) {
-            int64_t p = lo + step;
-            if (p >= R) break;
-            if (same(r, p)) { lo = p; step <<= 1; } else { hi = p; break; }
-        }
-        while (hi - lo > 1) {
-            int64_t mid = lo + (hi - lo) / 2;
-            if (same(r, mid)) lo = mid; else hi = mid;
-        }
-        return hi - r;
-    }
-};
+constexpr int PLAN_THREADS = 256;
+constexpr int PLAN_TILE = 2048;
+constexpr int PLAN_ROUNDS = PLAN_TILE / PLAN_THREADS;
 
-// item = 1 | c*c << 32 at group heads, else 0
-struct PlanLoad {
-    RowKeys k;
-    __device__ int64_t operator()(int64_t r) const {
-        if (!k.is_head(r)) return 0;
-        const int64_t c = k.run_length(r);
-        return (int64_t)1 | ((c * c) << 32);
-    }
-};
+template <bool WRITE>
+__global__ __launch_bounds__(PLAN_THREADS) void plan_tile_kernel(const int32_t* __restrict__ i0,
+                                                                const int32_t* __restrict__ i1, int64_t R,
+                                                                int inner, int64_t* __restrict__ tile_sums,
+                                                                int32_t* __restrict__ plan, int64_t g_cap,
+                                                                int32_t* __restrict__ cmax_out) {
+    __shared__ int kw[PLAN_TILE + 1], kh[PLAN_TILE + 1];     // slot e + 1 = key of tile row e; slot 0 = predecessor
+    __shared__ int start_s[PLAN_TILE + 1];
+    __shared__ int wave_cnt_s[PLAN_THREADS / 64];
+    __shared__ long long scan_lds[PLAN_THREADS / 64];
+    __shared__ int next_head_s;
 
-struct PlanStore {
-    RowKeys k;
-    int32_t* plan;
-    int64_t g_cap;
-    int32_t* cmax;
-    __device__ void operator()(int64_t r, int64_t ex, int64_t item) const {
-        if (item == 0) return;
-        const int64_t g = ex & 0xffffffffll;
-        if (g >= g_cap) return;
-        // c*c is a perfect square below 2^31: the double square root is exact
-        const int c = (int)(sqrt((double)(item >> 32)) + 0.5);
-        plan[g] = c;
-        plan[g_cap + g] = (int32_t)r;
-        plan[2 * g_cap + g] = (int32_t)(ex >> 32);
-        plan[3 * g_cap + g] = k.i0[r * k.inner];
-        plan[4 * g_cap + g] = k.i1[r * k.inner];
-        if (c > *cmax) atomicMax(cmax, c);
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int64_t tile_base = (int64_t)blockIdx.x * PLAN_TILE;
+    const int tile_n = (int)((R - tile_base) < PLAN_TILE ? (R - tile_base) : PLAN_TILE);
+
+#pragma unroll
+    for (int j = 0; j < PLAN_ROUNDS; ++j) {
+        const int e = j * PLAN_THREADS + tid;
+        if (e < tile_n) {
+            const int64_t col = (tile_base + e) * inner;
+            kw[e + 1] = i0[col];
+            kh[e + 1] = i1[col];
+        }
     }
-};
+    if (tid == 0) {
+        if (tile_base > 0) {
+            kw[0] = i0[(tile_base - 1) * inner];
+            kh[0] = i1[(tile_base - 1) * inner];
+        } else {
+            kw[0] = ~i0[0];                                  // anything different from row 0
+            kh[0] = 0;
+        }
+    }
+    __syncthreads();
+
+    // heads, compacted in row order
+    int rnk[PLAN_ROUNDS];
+    int wave_count = 0;
+#pragma unroll
+    for (int j = 0; j < PLAN_ROUNDS; ++j) {
+        const int e = wave * (PLAN_TILE / 4) + j * 64 + lane;
+        const bool flag = e < tile_n && (kw[e + 1] != kw[e] || kh[e + 1] != kh[e]);
+        const unsigned long long mask = __ballot(flag);
+        rnk[j] = flag ? wave_count + __popcll(mask & ((1ull << lane) - 1ull)) : -1;
+        wave_count += __popcll(mask);
+    }
+    if (lane == 0) wave_cnt_s[wave] = wave_count;
+    __syncthreads();
+    int wave_base = 0, nheads = 0;
+#pragma unroll
+    for (int w = 0; w < PLAN_THREADS / 64; ++w) {
+        const int t = wave_cnt_s[w];
+        if (w < wave) wave_base += t;
+        nheads += t;
+    }
+#pragma unroll
+    for (int j = 0; j < PLAN_ROUNDS; ++j)
+        if (rnk[j] >= 0) start_s[wave_base + rnk[j]] = wave * (PLAN_TILE / 4) + j * 64 + lane;
+
+    // first head after the tile: first row whose key differs from the tile's last key
+    if (wave == 0 && nheads > 0) {
+        const int lw = kw[tile_n], lh = kh[tile_n];
+        int64_t p = tile_base + tile_n;
+        int64_t found = R;
+        while (p < R) {
+            const int64_t r = p + lane;
+            bool differs = false;
+            if (r < R) {
+                const int64_t col = r * inner;
+                differs = i0[col] != lw || i1[col] != lh;
+            }
+            const unsigned long long mask = __ballot(differs);
+            if (mask) {
+                found = p + (__ffsll((long long)mask) - 1);
+                break;
+            }
+            p += 64;
+        }
+        if (lane == 0) next_head_s = (int)(found - tile_base);
+    }
+    __syncthreads();
+    if (tid == 0 && nheads > 0) start_s[nheads] = next_head_s;
+    __syncthreads();
+
+    // per-thread heads k = tid * PLAN_ROUNDS .. (blocked, so that a block scan gives prefixes in order)
+    long long sq_local = 0;
+    int cvals[PLAN_ROUNDS];
+    int cmx = 0;
+#pragma unroll
+    for (int j = 0; j < PLAN_ROUNDS; ++j) {
+        const int k = tid * PLAN_ROUNDS + j;
+        int c = 0;
+        if (k < nheads) c = start_s[k + 1] - start_s[k];
+        cvals[j] = c;
+        sq_local += (long long)c * c;
+        cmx = c > cmx ? c : cmx;
+    }
+    long long sq_total;
+    long long sq_prefix = block_exclusive_scan<long long, PLAN_THREADS / 64>(sq_local, scan_lds, &sq_total);
+    if (!WRITE) {
+        if (tid == 0) tile_sums[blockIdx.x] = (long long)nheads | (sq_total << 32);
+        return;
+    }
+    const long long off = tile_sums[blockIdx.x];             // exclusive prefix over tiles (packed)
+    const int64_t g_base = off & 0xffffffffll;
+    long long sq = (off >> 32) + sq_prefix;
+#pragma unroll
+    for (int j = 0; j < PLAN_ROUNDS; ++j) {
+        const int k = tid * PLAN_ROUNDS + j;
+        if (k < nheads) {
+            const int64_t g = g_base + k;
+            if (g < g_cap) {
+                const int e = start_s[k];
+                plan[g] = cvals[j];
+                plan[g_cap + g] = (int32_t)(tile_base + e);
+                plan[2 * g_cap + g] = (int32_t)sq;
+                plan[3 * g_cap + g] = kw[e + 1];
+                plan[4 * g_cap + g] = kh[e + 1];
+            }
+            sq += (long long)cvals[j] * cvals[j];
+        }
+    }
+    cmx = wave_max_i32(cmx);
+    if (lane == 0 && cmx > 0) atomicMax(cmax_out, cmx);
+}
 
 __global__ void zero_i32_kernel(int32_t* p, int n) {
     if ((int)threadIdx.x < n) p[threadIdx.x] = 0;
@@ -95,7 +174,8 @@ extern "C" {
 
 size_t sswin_plan_workspace_bytes(int64_t M, int inner) {
     const int64_t R = inner > 0 ? M / inner : 0;
-    return align_up((size_t)scan_num_tiles(R > 0 ? R : 1) * sizeof(int64_t), 256) + 1024;
+    const int64_t tiles = (R + PLAN_TILE - 1) / PLAN_TILE;
+    return align_up((size_t)(tiles > 0 ? tiles : 1) * sizeof(int64_t), 256) + 1024;
 }
 
 int sswin_plan_from_indices(const int32_t* idx, int64_t M, int inner, int32_t* plan, int64_t g_cap,
@@ -110,16 +190,19 @@ int sswin_plan_from_indices(const int32_t* idx, int64_t M, int inner, int32_t* p
     SSWIN_CHECK(g_cap > 0, "plan: g_cap must be positive");
     SSWIN_CHECK(ws_bytes >= sswin_plan_workspace_bytes(M, inner), "plan: workspace too small");
     hipStream_t s = static_cast<hipStream_t>(stream);
+    const int64_t tiles = (R + PLAN_TILE - 1) / PLAN_TILE;
     Carver cv(ws, ws_bytes);
     int64_t* total_dev = cv.take<int64_t>(2);           // [0] packed total, [1] low word: c_max
-    int64_t* tile_sums = cv.take<int64_t>((size_t)scan_num_tiles(R));
+    int64_t* tile_sums = cv.take<int64_t>((size_t)tiles);
     SSWIN_CHECK(cv.ok(), "plan: workspace too small");
     int32_t* cmax = reinterpret_cast<int32_t*>(total_dev + 1);
     hipLaunchKernelGGL(zero_i32_kernel, dim3(1), dim3(64), 0, s, cmax, 2);
-    RowKeys k{idx, idx + M, R, inner};
-    PlanLoad ld{k};
-    PlanStore st{k, plan, g_cap, cmax};
-    if (device_exclusive_scan<int64_t>(ld, st, R, tile_sums, total_dev, s, "plan scan")) return 1;
+    hipLaunchKernelGGL(plan_tile_kernel<false>, dim3((unsigned)tiles), dim3(PLAN_THREADS), 0, s, idx, idx + M, R,
+                       inner, tile_sums, plan, g_cap, cmax);
+    hipLaunchKernelGGL((scan_tile_sums_kernel<int64_t>), dim3(1), dim3(1024), 0, s, tile_sums, tiles, total_dev);
+    hipLaunchKernelGGL(plan_tile_kernel<true>, dim3((unsigned)tiles), dim3(PLAN_THREADS), 0, s, idx, idx + M, R,
+                       inner, tile_sums, plan, g_cap, cmax);
+    if (launch_ok("plan")) return 1;
     int64_t host[2] = {0, 0};
     SSWIN_HIP(hipMemcpyAsync(host, total_dev, sizeof(host), hipMemcpyDeviceToHost, s));
     SSWIN_HIP(hipStreamSynchronize(s));

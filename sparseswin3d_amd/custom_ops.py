@@ -191,6 +191,44 @@ class _PlanCache:
 _plan_cache = _PlanCache()
 
 
+class _IndexPlanCache:
+    """Plans keyed by the index matrix they were derived from.  'q_k' and 'qk_v' of one forward
+    pass receive the same sorted Q/V index tensor, so the second call skips the plan kernels and
+    their host synchronisation.  Entries keep the index tensor alive (its address cannot be
+    reused) and remember its version counter (in-place edits invalidate the entry)."""
+
+    def __init__(self, capacity=4):
+        self.capacity = capacity
+        self.entries = OrderedDict()
+
+    @staticmethod
+    def _key(idx, inner):
+        return (idx.device.index, idx.data_ptr(), idx.shape[1], inner)
+
+    def get(self, idx, inner):
+        hit = self.entries.get(self._key(idx, inner))
+        if hit is None or hit[0]._version != hit[1]:
+            return None
+        return hit[2:]
+
+    def put(self, idx, inner, plan, g_cap, totals):
+        self.entries[self._key(idx, inner)] = (idx, idx._version, plan, g_cap, totals)
+        while len(self.entries) > self.capacity:
+            self.entries.popitem(last=False)
+
+    def clear(self):
+        self.entries.clear()
+
+
+_index_plan_cache = _IndexPlanCache()
+
+
+def clear_caches():
+    """Drop cached plans (and the tensors they keep alive)."""
+    _plan_cache.clear()
+    _index_plan_cache.clear()
+
+
 def _scans_for(c, lib, d):
     """Return ``(scans [2,G] int32 rows: excl-scan c, excl-scan c*c; sum_c2 or None)``."""
     hit = _plan_cache.get(c)
@@ -248,16 +286,21 @@ def matmul_cuda_naive(mat1_v, mat1_idx, mat1_shape, mat2_v, mat2_idx, mat2_shape
                 out_shape, torch.empty(0, dtype=torch.int32, device=d))
     _check(m % inner == 0, f"operand nnz {m} is not a multiple of its dense last dimension {inner}")
     rows = m // inner
-    g_cap = max(1, min(rows, s1[0] * s1[1]))
-    plan = torch.empty(5 * g_cap, dtype=torch.int32, device=d)
-    totals = (C.c_int64 * 4)()
     stream = _stream(d)
     with torch.cuda.device(d):
-        nbytes = lib.sswin_plan_workspace_bytes(m, inner)
-        ws = _ws(nbytes, d)
-        _lib.check(lib.sswin_plan_from_indices(_ptr(tok_idx), m, inner, _ptr(plan), g_cap, totals, _ptr(ws),
-                                               nbytes, stream))
-        g, sum_c, sum_c2, c_max = (int(totals[i]) for i in range(4))
+        cached = _index_plan_cache.get(tok_idx, inner)
+        if cached is not None:
+            plan, g_cap, (g, sum_c, sum_c2, c_max) = cached
+        else:
+            g_cap = max(1, min(rows, s1[0] * s1[1]))
+            plan = torch.empty(5 * g_cap, dtype=torch.int32, device=d)
+            totals = (C.c_int64 * 4)()
+            nbytes = lib.sswin_plan_workspace_bytes(m, inner)
+            ws = _ws(nbytes, d)
+            _lib.check(lib.sswin_plan_from_indices(_ptr(tok_idx), m, inner, _ptr(plan), g_cap, totals, _ptr(ws),
+                                                   nbytes, stream))
+            g, sum_c, sum_c2, c_max = (int(totals[i]) for i in range(4))
+            _index_plan_cache.put(tok_idx, inner, plan, g_cap, (g, sum_c, sum_c2, c_max))
         if kind == 0:
             _check(mat2_v.numel() == m, f"'q_k': mat2 holds {mat2_v.numel()} values, expected {m}")
             nnz = sum_c2

@@ -1,0 +1,141 @@
+"""Fused window attention: one autograd Function around the token-plan and the fused MFMA
+block products of ``libsswin3d.so``.
+
+Numerically this is the same computation as the operator-by-operator composition in
+:mod:`sparseswin3d_amd.window_attention` (reference ``sparse_swin/swin3d_base.py:654-675``):
+
+    S = (scale*Q) K^T + bias + mask  ->  P = sparse softmax(S)  ->  O = P V  (in voxel order)
+
+but Q, K, V token rows are read straight from the dense ``qkv`` tensor through the token order
+and the output is written straight into voxel order, so the sorted COO copies, the bias/mask
+gather passes, the permute and the un-sort never exist.  The attention values S and P are still
+materialised in HBM (P is needed by the backward pass).
+"""
+from __future__ import annotations
+
+import ctypes as C
+
+import torch
+from torch.autograd import Function
+from torch.autograd.function import once_differentiable
+
+from . import _lib
+from . import custom_ops as ops
+
+_DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+
+def _ptr(t):
+    return C.c_void_p(t.data_ptr() if t is not None else 0)
+
+
+class TokenPlan:
+    """Token order and per-group table of one set of (window, pos) voxel indices."""
+
+    def __init__(self, indices: torch.Tensor, batch_size: int, n: int, num_heads: int):
+        lib = _lib.load()
+        if indices.device.type != "cuda":
+            raise RuntimeError("TokenPlan runs on the GPU only; there is no CPU fallback")
+        if indices.dtype != torch.int32 or indices.dim() != 2 or indices.shape[1] != 2:
+            raise RuntimeError("TokenPlan: indices must be int32 [N, 2]")
+        indices = indices.contiguous()
+        d = indices.device
+        N = indices.shape[0]
+        self.N, self.H, self.n, self.B = N, int(num_heads), int(n), int(batch_size)
+        self.g_cap = max(1, min(N, self.B) * self.H)
+        self.tokens = torch.empty(5 * max(N, 1), dtype=torch.int32, device=d)
+        self.plan = torch.empty(5 * self.g_cap, dtype=torch.int32, device=d)
+        totals = (C.c_int64 * 4)()
+        with torch.cuda.device(d):
+            nbytes = lib.sswin_token_plan_workspace_bytes(N, self.B, self.n)
+            ws = torch.empty(int(nbytes), dtype=torch.uint8, device=d)
+            stream = C.c_void_p(torch.cuda.current_stream(d).cuda_stream)
+            _lib.check(lib.sswin_token_plan(_ptr(indices), N, self.B, self.n, self.H, _ptr(self.tokens),
+                                            _ptr(self.plan), self.g_cap, totals, _ptr(ws), nbytes, stream))
+        self.G, self.windows, self.A, self.c_max = (int(totals[i]) for i in range(4))
+        self.device = d
+
+
+def _tokens_to_sq(tp, dtype, epilogue, a, a_stride, a_col0, b, b_stride, b_col0, hd, scale, bias, mask, out, rows):
+    lib = _lib.load()
+    stream = C.c_void_p(torch.cuda.current_stream(tp.device).cuda_stream)
+    _lib.check(lib.sswin_fused_tokens_to_sq(
+        _DTYPE_CODE[dtype], 1 if epilogue else 0, _ptr(tp.plan), tp.g_cap, tp.G, _ptr(tp.tokens), tp.N, tp.H, hd,
+        _ptr(a), a_stride, a_col0, _ptr(b), b_stride, b_col0, C.c_float(scale), _ptr(bias), tp.n, _ptr(mask),
+        0 if mask is None else mask.shape[0], _ptr(out), _ptr(rows), stream))
+
+
+def _sq_to_tokens(tp, dtype, a_kmajor, sq, b, b_stride, b_col0, o, o_stride, o_col0, hd, scale):
+    lib = _lib.load()
+    stream = C.c_void_p(torch.cuda.current_stream(tp.device).cuda_stream)
+    _lib.check(lib.sswin_fused_sq_to_tokens(
+        _DTYPE_CODE[dtype], 1 if a_kmajor else 0, _ptr(tp.plan), tp.g_cap, tp.G, _ptr(tp.tokens), tp.N, hd,
+        _ptr(sq), _ptr(b), b_stride, b_col0, _ptr(o), o_stride, o_col0, C.c_float(scale), stream))
+
+
+class _FusedWindowAttention(Function):
+    @staticmethod
+    def forward(ctx, qkv, bias, indices, mask, batch_size, n, scale):
+        # qkv [N, 3, H, hd]; bias fp32 [H, n, n]; indices int32 [N, 2]; mask int8 [nW, n] or None
+        qkv = qkv.contiguous()
+        N, _, H, hd = qkv.shape
+        D = H * hd
+        dtype = qkv.dtype
+        tp = TokenPlan(indices, batch_size, n, H)
+        d = qkv.device
+        bias32 = bias.detach().to(torch.float32).contiguous()
+        if mask is not None:
+            mask = mask.to(torch.int8).contiguous()
+        with torch.cuda.device(d):
+            s = torch.empty(tp.A, dtype=torch.float32, device=d)
+            rows = torch.empty(tp.A, dtype=torch.int32, device=d)
+            _tokens_to_sq(tp, dtype, True, qkv, 3 * D, 0, qkv, 3 * D, D, hd, scale, bias32, mask, s, rows)
+            p = ops.softmax_last_dim_forward(rows, s)
+            out = torch.empty((N, D), dtype=dtype, device=d)
+            _sq_to_tokens(tp, dtype, False, p, qkv, 3 * D, 2 * D, out, D, 0, hd, 1.0)
+        ctx.save_for_backward(qkv, p, rows)
+        ctx.tp, ctx.scale, ctx.bias_meta = tp, scale, (bias.dtype, bias.shape)
+        return out
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad_out):
+        qkv, p, rows = ctx.saved_tensors
+        tp, scale = ctx.tp, ctx.scale
+        N, _, H, hd = qkv.shape
+        D = H * hd
+        dtype = qkv.dtype
+        d = qkv.device
+        grad_out = grad_out.contiguous().to(dtype)
+        lib = _lib.load()
+        with torch.cuda.device(d):
+            d_qkv = torch.empty_like(qkv)
+            d_p = torch.empty(tp.A, dtype=torch.float32, device=d)
+            # dP = dO V^T ; dV = P^T dO
+            _tokens_to_sq(tp, dtype, False, grad_out, D, 0, qkv, 3 * D, 2 * D, hd, 1.0, None, None, d_p, None)
+            _sq_to_tokens(tp, dtype, True, p, grad_out, D, 0, d_qkv, 3 * D, 2 * D, hd, 1.0)
+            d_s = ops.softmax_last_dim_backward(rows, p, d_p)
+            # dQ = scale * dS K ; dK = scale * dS^T Q
+            _sq_to_tokens(tp, dtype, False, d_s, qkv, 3 * D, D, d_qkv, 3 * D, 0, hd, scale)
+            _sq_to_tokens(tp, dtype, True, d_s, qkv, 3 * D, 0, d_qkv, 3 * D, D, hd, scale)
+            d_bias = None
+            if ctx.needs_input_grad[1]:
+                bias_dtype, bias_shape = ctx.bias_meta
+                d_bias32 = torch.zeros(bias_shape, dtype=torch.float32, device=d)
+                stream = C.c_void_p(torch.cuda.current_stream(d).cuda_stream)
+                _lib.check(lib.sswin_fused_bias_grad(_ptr(tp.plan), tp.g_cap, tp.G, _ptr(tp.tokens), tp.N, H, tp.n,
+                                                     _ptr(d_s), _ptr(d_bias32), stream))
+                d_bias = d_bias32.to(bias_dtype)
+        return d_qkv, d_bias, None, None, None, None, None
+
+
+def fused_window_attention(qkv, bias, indices, mask, batch_size, n, scale):
+    """``qkv`` [N,3,H,hd], ``bias`` [H,n,n], ``indices`` int32 [N,2] (window,pos), ``mask`` int8
+    [nW,n] or None -> attention output [N, H*hd] in the caller's voxel order."""
+    return _FusedWindowAttention.apply(qkv, bias, indices, mask, batch_size, n, scale)
+
+
+def supports(qkv: torch.Tensor, n: int) -> bool:
+    """The fused path covers fp32/fp16/bf16 on the GPU and windows of at most 128 positions
+    (bias-gradient LDS table); everything else takes the operator-by-operator path."""
+    return qkv.is_cuda and qkv.dtype in _DTYPE_CODE and n * n * 4 <= 64 * 1024

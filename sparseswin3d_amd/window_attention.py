@@ -232,7 +232,14 @@ def relative_position_index_3d(window_size: Sequence[int]) -> torch.Tensor:
 
 
 class WindowAttentionSparse(nn.Module):
-    """Window multi-head self attention with relative position bias on sparse windows."""
+    """Window multi-head self attention with relative position bias on sparse windows.
+
+    ``fused`` (class or instance attribute, default True) selects the fused HIP path of
+    :mod:`sparseswin3d_amd.fused`; with ``fused = False`` the forward pass is the
+    operator-by-operator composition of the reference.  Both give the same result.
+    """
+
+    fused = True
 
     def __init__(self, dim: int, num_heads: int, window_size: Sequence[int], qkv_bias: bool = False,
                  attn_drop: float = 0.0, proj_drop: float = 0.0) -> None:
@@ -262,6 +269,13 @@ class WindowAttentionSparse(nn.Module):
         b = x.batch_size
         c = x.features.shape[-1]
         qkv = self.qkv(x.features).reshape(-1, 3, self.num_heads, c // self.num_heads)
+        if self.fused:
+            from . import fused
+            if fused.supports(qkv, n):
+                out = fused.fused_window_attention(qkv, self.relative_position_bias(n, torch.float32), x.indices,
+                                                   mask, b, n, self.scale)
+                x = replace_feature(x, out)
+                return replace_feature(x, self.proj_drop(self.proj(x.features)))
         q, k_t, v = qkv_sparse_cuda(qkv, x.indices, b, n)
         attn = spspmm_block_naive(q * self.scale, k_t, "q_k")
         attn = sp_add_rpb(attn, self.relative_position_bias(n, attn.values.dtype))
