@@ -94,7 +94,7 @@ def event_time_ms(fn, reps, warmup=2):
     return start.elapsed_time(stop) / reps
 
 
-def kernel_table(wl, reps=20):
+def kernel_table(wl, reps=20, only=None):
     """Time every operator's kernels alone on the first block's tensors (regular windows)."""
     from sparseswin3d_amd import _lib, custom_ops as ops
     from sparseswin3d_amd.window_attention import qkv_sparse_cuda
@@ -171,12 +171,58 @@ def kernel_table(wl, reps=20):
         ("transpose rc", tr(0, q.values, tmp_e), 2 * s * E, 2),
         ("transpose rr", tr(1, g_s, tmp_a), 2 * s * A, 2),
     ]
-    table = []
-    for name, fn, nbytes, calls in entries:
-        ms = event_time_ms(fn, reps)
-        gbps = nbytes / ms / 1e6 if nbytes else None
-        table.append(dict(kernel=name, ms=ms, algorithmic_bytes=nbytes, calls=calls,
-                          achieved_gbps=gbps, frac=(gbps / HBM_PEAK_GBPS) if gbps else None))
+    # ---- the fused path (what WindowAttentionSparse.forward runs by default) ----
+    from sparseswin3d_amd import fused as F
+    tp = F.TokenPlan(b["idx"], b["slots"], b["n"], H)
+    qkv_c = qkv.contiguous()
+    bias = torch.randn(H, b["n"], b["n"], device=dev)
+    mask = wl["blocks"][1]["mask"]
+    s_f = torch.empty(tp.A, device=dev)
+    rows_f = torch.empty(tp.A, dtype=torch.int32, device=dev)
+    out_f = torch.empty(N, D, device=dev)
+    dqkv = torch.empty_like(qkv_c)
+    dbias = torch.zeros(H, b["n"], b["n"], device=dev)
+    dt = torch.float32
+    bg_bytes = lib.sswin_fused_bias_grad_workspace_bytes(tp.G, H, b["n"])
+    bg_ws = torch.empty(int(bg_bytes), dtype=torch.uint8, device=dev)
+    f_entries = [
+        ("fused token_plan", lambda: F.TokenPlan(b["idx"], b["slots"], b["n"], H), 28 * N + 20 * tp.G, 1),
+        ("fused S=QK^T+bias+mask", lambda: F._tokens_to_sq(tp, dt, True, qkv_c, 3 * D, 0, qkv_c, 3 * D, D, hd, 0.17, bias, mask, s_f, rows_f), 8 * E + 8 * A, 1),
+        ("fused softmax fwd", lambda: ops.softmax_last_dim_forward(rows_f, s_f), 12 * A, 1),
+        ("fused O=PV", lambda: F._sq_to_tokens(tp, dt, False, p_val, qkv_c, 3 * D, 2 * D, out_f, D, 0, hd, 1.0), 4 * A + 8 * E, 1),
+        ("fused dP=dO V^T", lambda: F._tokens_to_sq(tp, dt, False, out_f, D, 0, qkv_c, 3 * D, 2 * D, hd, 1.0, None, None, s_f, None), 8 * E + 4 * A, 1),
+        ("fused dV=P^T dO", lambda: F._sq_to_tokens(tp, dt, True, p_val, out_f, D, 0, dqkv, 3 * D, 2 * D, hd, 1.0), 4 * A + 8 * E, 1),
+        ("fused softmax bwd", lambda: ops.softmax_last_dim_backward(rows_f, p_val, g_s), 16 * A, 1),
+        ("fused dQ=dS K", lambda: F._sq_to_tokens(tp, dt, False, g_s, qkv_c, 3 * D, D, dqkv, 3 * D, 0, hd, 0.17), 4 * A + 8 * E, 1),
+        ("fused dK=dS^T Q", lambda: F._sq_to_tokens(tp, dt, True, g_s, qkv_c, 3 * D, 0, dqkv, 3 * D, D, hd, 0.17), 4 * A + 8 * E, 1),
+        ("fused bias grad", lambda: _lib.check(lib.sswin_fused_bias_grad(ptr(tp.plan), tp.g_cap, tp.G, ptr(tp.tokens), tp.N, H, b["n"], ptr(g_s), ptr(dbias), ptr(bg_ws), bg_bytes, stream)), 4 * A, 1),
+    ]
+
+    def measure(items, path):
+        rows_ = []
+        for name, fn, nbytes, calls in items:
+            ms = event_time_ms(fn, reps)
+            gbps = nbytes / ms / 1e6 if nbytes else None
+            rows_.append(dict(kernel=name, path=path, ms=ms, algorithmic_bytes=nbytes, calls=calls,
+                              achieved_gbps=gbps, frac=(gbps / HBM_PEAK_GBPS) if gbps else None))
+        return rows_
+
+    if only is not None:
+        # profiling mode: run the named kernels (substring match) `reps` times each, plus a plain
+        # device-to-device copy of known size that calibrates the FETCH_SIZE / WRITE_SIZE counters
+        src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device=dev)
+        dst = torch.empty_like(src)
+        picked = [e for e in f_entries + entries if only in e[0]]
+        for name, fn, nbytes, calls in picked:
+            log(f"profiling {name}: {reps} launches, algorithmic bytes {nbytes}")
+            for _ in range(reps):
+                fn()
+        for _ in range(reps):
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        log(f"calibration copy: {reps} launches of {src.numel() * 4} bytes read and written")
+        return [], dict(N=N, E=E, A=A, G=G, c_max=c_max)
+    table = measure(f_entries, "fused") + measure(entries, "operators")
     return table, dict(N=N, E=E, A=A, G=G, c_max=c_max)
 
 
@@ -233,6 +279,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel table")
     ap.add_argument("--kernels-json", default=None)
+    ap.add_argument("--profile-kernel", default=None, metavar="NAME",
+                    help="run only the kernels whose table name contains NAME (for rocprofv3) and exit")
+    ap.add_argument("--profile-reps", type=int, default=5)
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (windows are independent; sharding is "
@@ -243,6 +292,9 @@ def main():
     torch.cuda.set_device(device)
     wl = build_workload(device)
     log(f"workload {wl['name']}: N={wl['N']}, blocks: " + "; ".join(str(b["stats"]) for b in wl["blocks"]))
+    if args.profile_kernel is not None:
+        kernel_table(wl, reps=args.profile_reps, only=args.profile_kernel)
+        return
 
     for _ in range(args.warmup):
         run_step(wl)
@@ -261,20 +313,27 @@ def main():
     if not args.no_kernels:
         table, sizes = kernel_table(wl)
         log(f"{'kernel':36s} {'ms':>9s} {'calls':>5s} {'alg MB':>9s} {'GB/s':>9s} {'% HBM':>7s}")
-        for r in table:
-            log(f"{r['kernel']:36s} {r['ms']:9.4f} {r['calls']:5d} {r['algorithmic_bytes'] / 1e6:9.1f} "
-                f"{(r['achieved_gbps'] or 0):9.1f} {100 * (r['frac'] or 0):7.2f}")
-        ops_ms = sum(r["ms"] * r["calls"] for r in table)
-        alg = sum(r["algorithmic_bytes"] * r["calls"] for r in table)
-        log(f"operators only, one attention fwd+bwd: {ops_ms:.3f} ms for {alg / 1e6:.1f} MB algorithmic "
-            f"= {alg / ops_ms / 1e6:.1f} GB/s = {100 * alg / ops_ms / 1e6 / HBM_PEAK_GBPS:.2f}% of HBM peak")
-        dom = max((r for r in table if r["algorithmic_bytes"]), key=lambda r: r["ms"] * r["calls"])
+        summary = {}
+        for path in ("fused", "operators"):
+            rows_ = [r for r in table if r["path"] == path]
+            log(f"-- {path} path, one attention forward+backward --")
+            for r in rows_:
+                log(f"{r['kernel']:36s} {r['ms']:9.4f} {r['calls']:5d} {r['algorithmic_bytes'] / 1e6:9.1f} "
+                    f"{(r['achieved_gbps'] or 0):9.1f} {100 * (r['frac'] or 0):7.2f}")
+            ms_ = sum(r["ms"] * r["calls"] for r in rows_)
+            alg = sum(r["algorithmic_bytes"] * r["calls"] for r in rows_)
+            summary[path] = dict(ms=round(ms_, 4), algorithmic_bytes=alg,
+                                 frac=round(alg / ms_ / 1e6 / HBM_PEAK_GBPS, 4))
+            log(f"{path} kernels, one attention fwd+bwd: {ms_:.3f} ms for {alg / 1e6:.1f} MB algorithmic "
+                f"= {alg / ms_ / 1e6:.1f} GB/s = {100 * alg / ms_ / 1e6 / HBM_PEAK_GBPS:.2f}% of HBM peak")
+        # the step runs the fused path: its slowest kernel is the dominant one
+        dom = max((r for r in table if r["path"] == "fused" and r["algorithmic_bytes"]),
+                  key=lambda r: r["ms"] * r["calls"])
         roofline = dict(bound="hbm", kernel=dom["kernel"], achieved=round(dom["achieved_gbps"], 1),
                         peak=HBM_PEAK_GBPS, unit="GB/s", frac=round(dom["frac"], 4),
                         traffic=MEASURED_TRAFFIC_BYTES.get(dom["kernel"]),
                         algorithmic_bytes=dom["algorithmic_bytes"], ms=round(dom["ms"], 4),
-                        operators_only_ms=round(ops_ms, 3),
-                        operators_only_frac=round(alg / ops_ms / 1e6 / HBM_PEAK_GBPS, 4))
+                        path_summaries=summary)
         if args.kernels_json:
             with open(args.kernels_json, "w") as f:
                 json.dump(dict(sizes=sizes, kernels=table), f, indent=1)

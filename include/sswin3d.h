@@ -199,10 +199,13 @@ int sswin_fused_sq_to_tokens(int dtype, int a_kmajor, const int32_t* plan, int64
                              int64_t o_stride, int o_col0, float scale_out, void* stream);
 
 /* d_bias[h, pos_i, pos_j] += ds over all windows (the backward of swin3d_base.py:557-566, which
- * autograd performs as an index_add).  d_bias: fp32 [H,n,n], zeroed by the caller.  n*n*4 bytes
- * must fit 64 KiB of LDS.  Uses float atomics (summation order varies).  Asynchronous. */
+ * autograd performs as an index_add).  d_bias: fp32 [H,n,n], accumulated into (zero it first).
+ * n*n*4 bytes must fit 64 KiB of LDS.  Partial tables are built with LDS float atomics (the
+ * summation order inside a workgroup varies) and summed without global atomics.  Asynchronous. */
+size_t sswin_fused_bias_grad_workspace_bytes(int64_t G, int H, int n);
 int sswin_fused_bias_grad(const int32_t* plan, int64_t g_cap, int64_t G, const int32_t* tokens,
-                          int64_t N, int H, int n, const float* ds, float* d_bias, void* stream);
+                          int64_t N, int H, int n, const float* ds, float* d_bias, void* ws,
+                          size_t ws_bytes, void* stream);
 
 #ifdef __cplusplus
 }

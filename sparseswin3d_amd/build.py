@@ -19,6 +19,7 @@ ARCH = "gfx950"
 # packed FP32 instructions are switched off for all device code on purpose
 FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+         "-munsafe-fp-atomics",          # LDS float adds as ds_add_f32 instead of compare-and-swap loops
          "-Wno-unused-command-line-argument"]
 
 

@@ -198,21 +198,21 @@ __global__ __launch_bounds__(256) void fused_sq_kernel(FusedGroups gt, const int
         const int64_t sq0 = gt.sq[g];
         const int i_a = bi * 32 + l32, j_b = bj * 32 + l32;
         const bool a_in = i_a < c, b_in = j_b < c;
-        const T* pa = A + (a_in ? (int64_t)order[Tk + i_a] * ta.stride : 0) + ta.col0 + h * hd;
-        const T* pb = B + (b_in ? (int64_t)order[Tk + j_b] * tb.stride : 0) + tb.col0 + h * hd;
+        // rows past the end of the window are clamped to its last token: their products are finite
+        // garbage that is never stored, and no load needs a predicate
+        const int i_c = a_in ? i_a : c - 1, j_c = b_in ? j_b : c - 1;
+        const T* pa = A + (int64_t)order[Tk + i_c] * ta.stride + ta.col0 + h * hd;
+        const T* pb = B + (int64_t)order[Tk + j_c] * tb.stride + tb.col0 + h * hd;
 
-        // epilogue inputs first: their latency hides behind the product
-        int pos_i[16], pos_j = 0, m_j = 0;
-        const int8_t* mrow = nullptr;
+        // epilogue inputs: one load per lane (row token, column token); the 16 rows a lane stores
+        // are fetched from the row lanes with cross-lane reads in the epilogue
+        int pos_a = 0, pos_j = 0, m_a = 0, m_j = 0;
         if (EPI) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int i = bi * 32 + acc_row(r, half);
-                pos_i[r] = i < c ? tok_pos[Tk + i] : 0;
-            }
-            pos_j = b_in ? tok_pos[Tk + j_b] : 0;
+            pos_a = tok_pos[Tk + i_c];
+            pos_j = tok_pos[Tk + j_c];
             if (mask) {
-                mrow = mask + (int64_t)(gt.window[g] % n_mask_windows) * n;
+                const int8_t* mrow = mask + (int64_t)(gt.window[g] % n_mask_windows) * n;
+                m_a = mrow[pos_a];
                 m_j = mrow[pos_j];
             }
         }
@@ -220,32 +220,50 @@ __global__ __launch_bounds__(256) void fused_sq_kernel(FusedGroups gt, const int
         f32x16 acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
         for (int kc = 0; kc < hd; kc += 32) {
             const int kb = kc + half * 16;
-            const int left = hd - kb;
             float a[16], b[16];
-            load_run16<T>(pa + kb, a_in ? clamp16(left) : 0, a);
-            load_run16<T>(pb + kb, b_in ? clamp16(left) : 0, b);
-            if (scale_a != 1.0f) {
+            if (kc + 32 <= hd) {                                   // full chunk (uniform)
+                load_run16_full<T>(pa + kb, a);
+                load_run16_full<T>(pb + kb, b);
+                if (scale_a != 1.0f) {
 #pragma unroll
-                for (int s = 0; s < 16; ++s) a[s] *= scale_a;
+                    for (int s = 0; s < 16; ++s) a[s] *= scale_a;
+                }
+#pragma unroll
+                for (int s = 0; s < 16; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], acc, 0, 0, 0);
+            } else {
+                const int left = hd - kb;
+                load_run16<T>(pa + kb, clamp16(left), a);
+                load_run16<T>(pb + kb, clamp16(left), b);
+                if (scale_a != 1.0f) {
+#pragma unroll
+                    for (int s = 0; s < 16; ++s) a[s] *= scale_a;
+                }
+                const int steps = hd - kc;
+#pragma unroll
+                for (int s = 0; s < 16; ++s)
+                    if (s < steps) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], acc, 0, 0, 0);
             }
-            const int steps = hd - kc;
-#pragma unroll
-            for (int s = 0; s < 16; ++s)
-                if (s < steps) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], acc, 0, 0, 0);
         }
 
-        if (b_in) {
+        {
             float* O = out + sq0 + j_b;
             const float* brow = EPI ? bias + (int64_t)h * n * n + pos_j : nullptr;
+            const int rid0 = H * Tk + h * c;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int i = bi * 32 + acc_row(r, half);
-                if (i < c) {
+                const int il = acc_row(r, half);                    // row inside the block
+                const int i = bi * 32 + il;
+                int p_i = 0, m_i = 0;
+                if (EPI) {                                          // all lanes take part in the shuffles
+                    p_i = __shfl(pos_a, il, 64);
+                    if (mask) m_i = __shfl(m_a, il, 64);
+                }
+                if (b_in && i < c) {
                     float v = acc[r];
                     if (EPI) {
-                        v += brow[(int64_t)pos_i[r] * n];
-                        if (mask && mrow[pos_i[r]] != m_j) v += -100.0f;
-                        if (row_ids) row_ids[sq0 + (int64_t)i * c + j_b] = H * Tk + h * c + i;
+                        v += brow[p_i * n];
+                        if (mask && m_i != m_j) v += -100.0f;
+                        if (row_ids) row_ids[sq0 + (int64_t)i * c + j_b] = rid0 + i;
                     }
                     O[(int64_t)i * c] = v;
                 }
@@ -279,77 +297,156 @@ __global__ __launch_bounds__(256) void fused_tok_kernel(FusedGroups gt, const in
         const float* S = sq + gt.sq[g];
         const int i_a = bi * 32 + l32, j_b = bj * 32 + l32;
         const bool a_in = i_a < c, b_in = j_b < hd;
+        const int i_c = a_in ? i_a : c - 1, j_c = b_in ? j_b : hd - 1;     // clamped: loads need no predicate
 
-        // output rows of this lane half
-        int64_t orow[16];
-#pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int i = bi * 32 + acc_row(r, half);
-            orow[r] = i < c ? (int64_t)order[Tk + i] * to.stride : -1;
-        }
+        // voxel of this lane's row token; the 16 rows a lane stores are fetched with cross-lane reads
+        const int vox_a = a_in ? order[Tk + i_a] : -1;
+        const T* bcol = B + tb.col0 + h * hd + j_c;
 
         f32x16 acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
         for (int kc = 0; kc < c; kc += 32) {
             const int kb = kc + half * 16;
-            const int left = c - kb;                              // k values left for this lane half
+            // voxels of the 32 tokens of this k chunk: one coalesced load, then cross-lane reads
+            const int kt = kc + l32;
+            const int ord_l = order[Tk + (kt < c ? kt : c - 1)];
             float a[16], b[16];
-            if (!A_KMAJOR) {
-                load_run16<float>(S + (int64_t)i_a * c + kb, a_in ? clamp16(left) : 0, a);
-            } else {
-#pragma unroll
-                for (int s = 0; s < 16; ++s) a[s] = (a_in && s < left) ? S[(int64_t)(kb + s) * c + i_a] : 0.f;
-            }
 #pragma unroll
             for (int s = 0; s < 16; ++s) {
-                float v = 0.f;
-                if (b_in && s < left) v = to_acc(B[(int64_t)order[Tk + kb + s] * tb.stride + tb.col0 + h * hd + j_b]);
-                b[s] = v;
+                const int vox = __shfl(ord_l, half * 16 + s, 64);
+                b[s] = to_acc(bcol[(int64_t)vox * tb.stride]);
             }
-            const int steps = c - kc;
+            if (kc + 32 <= c) {                                    // full chunk (uniform)
+                if (!A_KMAJOR) {
+                    load_run16_full<float>(S + (int64_t)i_c * c + kb, a);
+                } else {
 #pragma unroll
-            for (int s = 0; s < 16; ++s)
-                if (s < steps) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], acc, 0, 0, 0);
+                    for (int s = 0; s < 16; ++s) a[s] = S[(int64_t)(kb + s) * c + i_c];
+                }
+#pragma unroll
+                for (int s = 0; s < 16; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], acc, 0, 0, 0);
+            } else {
+                const int left = c - kb;                           // k values left for this lane half
+#pragma unroll
+                for (int s = 0; s < 16; ++s) {
+                    const int k = kb + s < c ? kb + s : c - 1;
+                    const float v = A_KMAJOR ? S[(int64_t)k * c + i_c] : S[(int64_t)i_c * c + k];
+                    a[s] = s < left ? v : 0.f;                     // zero A kills the clamped B rows
+                }
+                const int steps = c - kc;
+#pragma unroll
+                for (int s = 0; s < 16; ++s)
+                    if (s < steps) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], acc, 0, 0, 0);
+            }
         }
 
-        if (b_in) {
+        {
             const int col = to.col0 + h * hd + j_b;
 #pragma unroll
-            for (int r = 0; r < 16; ++r)
-                if (orow[r] >= 0) O[orow[r] + col] = from_acc<T>(acc[r] * scale_out);
+            for (int r = 0; r < 16; ++r) {
+                const int vox = __shfl(vox_a, acc_row(r, half), 64);
+                if (b_in && vox >= 0) O[(int64_t)vox * to.stride + col] = from_acc<T>(acc[r] * scale_out);
+            }
         }
     }
 }
 
 // ------------------------------------------------------------------------------------------
-// gradient of the relative position bias: d_rpb[h, pos_i, pos_j] += dS over all windows.
-// grid (slices, H).  Each workgroup accumulates its windows into an LDS copy of one head's table
-// (LDS float atomics) and flushes the non-zero entries with one global atomic each.
+// gradient of the relative position bias: d_rpb[h, pos_i, pos_j] = sum of dS over all windows.
+// Stage 1, grid (slices, H): a workgroup of 16 wavefronts walks its share of the windows and
+// accumulates into an LDS copy of one head's [n x n] table.  All wavefronts look at the same
+// window; wavefront r owns the table rows [r*RB, (r+1)*RB), i.e. the rows of dS whose token
+// position falls into that range (a contiguous run of rows, positions being sorted inside a
+// window).  Table rows are therefore private to a wavefront: plain LDS read-add-write, no
+// atomics, and a fixed summation order.  The next window's header and positions are fetched
+// while the current one is processed.  Stage 2 sums the per-slice tables in slice order.
 // ------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void rpb_grad_kernel(FusedGroups gt, const int32_t* __restrict__ tok_pos, int H,
-                                                       int n, const float* __restrict__ ds,
-                                                       float* __restrict__ d_rpb) {
+constexpr int RPB_THREADS = 1024;
+
+struct RpbWindow {
+    int c, Tk, pos0, pos1;
+    int64_t sq;
+};
+
+__device__ __forceinline__ RpbWindow rpb_fetch(const FusedGroups& gt, const int32_t* __restrict__ tok_pos,
+                                               int64_t k, int64_t windows, int H, int h, int lane) {
+    RpbWindow w{0, 0, 0, 0, 0};
+    if (k < windows) {
+        const int64_t g = k * H + h;
+        w.c = gt.c[g];
+        w.Tk = gt.T[g];
+        w.sq = gt.sq[g];
+        w.pos0 = lane < w.c ? tok_pos[w.Tk + lane] : -1;
+        w.pos1 = 64 + lane < w.c ? tok_pos[w.Tk + 64 + lane] : -1;
+    }
+    return w;
+}
+
+__global__ __launch_bounds__(RPB_THREADS) void rpb_grad_partial_kernel(FusedGroups gt,
+                                                                       const int32_t* __restrict__ tok_pos, int H,
+                                                                       int n, const float* __restrict__ ds,
+                                                                       float* __restrict__ partial) {
     extern __shared__ float table[];
     const int h = blockIdx.y;
     const int nn = n * n;
-    for (int e = threadIdx.x; e < nn; e += 256) table[e] = 0.f;
+    constexpr int WAVES = RPB_THREADS / 64;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int rb = (n + WAVES - 1) / WAVES;
+    const int lo = wave * rb, hi = lo + rb;                        // table rows owned by this wavefront
+    for (int e = threadIdx.x; e < nn; e += RPB_THREADS) table[e] = 0.f;
     __syncthreads();
     const int64_t windows = gt.G / H;
+    RpbWindow next = rpb_fetch(gt, tok_pos, blockIdx.x, windows, H, h, lane);
     for (int64_t k = blockIdx.x; k < windows; k += gridDim.x) {
-        const int64_t g = k * H + h;
-        const int c = gt.c[g], Tk = gt.T[g];
-        const float* S = ds + gt.sq[g];
-        const int count = c * c;
-        for (int f = threadIdx.x; f < count; f += 256) {
-            const int i = f / c, j = f - i * c;
-            atomicAdd(&table[tok_pos[Tk + i] * n + tok_pos[Tk + j]], S[f]);
+        const RpbWindow w = next;
+        next = rpb_fetch(gt, tok_pos, k + gridDim.x, windows, H, h, lane);
+        const int c = w.c;
+        // rows of this window whose position lies in [lo, hi): a contiguous run i_lo .. i_lo+cnt-1
+        const unsigned long long m0 = __ballot(w.pos0 >= lo && w.pos0 < hi);
+        const unsigned long long m1 = __ballot(w.pos1 >= lo && w.pos1 < hi);
+        const int cnt = __popcll(m0) + __popcll(m1);
+        if (cnt == 0) continue;                                     // wave-uniform
+        const int i_lo = m0 ? __ffsll((long long)m0) - 1 : 64 + __ffsll((long long)m1) - 1;
+        const int count = cnt * c;                                  // contiguous values of dS
+        const float* S = ds + w.sq + (int64_t)i_lo * c;
+        const uint32_t magic = (uint32_t)((0x100000000ull + (uint32_t)c - 1) / (uint32_t)c);
+        for (int f0 = 0; f0 < count; f0 += 64 * 4) {
+            float v[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int f = f0 + u * 64 + lane;
+                v[u] = f < count ? S[f] : 0.f;
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                const int f = f0 + u * 64 + lane;
+                const int fc = f < count ? f : 0;
+                const int il = (int)__umulhi((uint32_t)fc, magic);
+                const int j = fc - il * c;
+                const int i = i_lo + il;
+                const int pi0 = __shfl(w.pos0, i & 63, 64), pi1 = __shfl(w.pos1, i & 63, 64);
+                const int pj0 = __shfl(w.pos0, j & 63, 64), pj1 = __shfl(w.pos1, j & 63, 64);
+                const int pi = i < 64 ? pi0 : pi1, pj = j < 64 ? pj0 : pj1;
+                if (f < count) table[pi * n + pj] += v[u];
+            }
         }
     }
     __syncthreads();
-    float* dst = d_rpb + (int64_t)h * nn;
-    for (int e = threadIdx.x; e < nn; e += 256) {
-        const float v = table[e];
-        if (v != 0.f) atomicAdd(&dst[e], v);
+    float* dst = partial + ((int64_t)blockIdx.x * H + h) * nn;
+    for (int e = threadIdx.x; e < nn; e += RPB_THREADS) dst[e] = table[e];
+}
+
+__global__ __launch_bounds__(256) void rpb_grad_reduce_kernel(const float* __restrict__ partial, int slices,
+                                                              int64_t table_elems, float* __restrict__ d_rpb) {
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= table_elems) return;
+    float sum[4] = {0.f, 0.f, 0.f, 0.f};
+    int s = 0;
+    for (; s + 4 <= slices; s += 4) {
+#pragma unroll
+        for (int u = 0; u < 4; ++u) sum[u] += partial[(int64_t)(s + u) * table_elems + e];
     }
+    for (; s < slices; ++s) sum[0] += partial[(int64_t)s * table_elems + e];
+    d_rpb[e] += (sum[0] + sum[1]) + (sum[2] + sum[3]);
 }
 
 template <typename T>
@@ -496,19 +593,37 @@ int sswin_fused_sq_to_tokens(int dtype, int a_kmajor, const int32_t* plan, int64
     }
 }
 
+static int bias_grad_slices(int64_t windows, int H) {
+    // about two 1024-thread workgroups per CU over all heads, at least eight windows per slice
+    const int64_t want = std::max<int64_t>(1, 512 / std::max(H, 1));
+    const int64_t useful = std::max<int64_t>(1, (windows + 7) / 8);
+    return (int)std::min<int64_t>(want, useful);
+}
+
+size_t sswin_fused_bias_grad_workspace_bytes(int64_t G, int H, int n) {
+    const int64_t windows = H > 0 ? G / H : 0;
+    return (size_t)bias_grad_slices(windows, H) * H * n * n * sizeof(float) + 256;
+}
+
 int sswin_fused_bias_grad(const int32_t* plan, int64_t g_cap, int64_t G, const int32_t* tokens, int64_t N,
-                          int H, int n, const float* ds, float* d_bias, void* stream) {
+                          int H, int n, const float* ds, float* d_bias, void* ws, size_t ws_bytes,
+                          void* stream) {
     SSWIN_CHECK(G >= 0 && G <= g_cap && H > 0 && n > 0, "fused_bias_grad: bad sizes");
     if (G == 0) return 0;
-    SSWIN_CHECK(plan && tokens && ds && d_bias, "fused_bias_grad: null pointer");
-    SSWIN_CHECK((size_t)n * n * sizeof(float) <= 64 * 1024,
-                "fused_bias_grad: a window of %d positions needs a %zu-byte LDS table (limit 64 KiB)", n,
-                (size_t)n * n * sizeof(float));
+    SSWIN_CHECK(plan && tokens && ds && d_bias && ws, "fused_bias_grad: null pointer");
+    SSWIN_CHECK((size_t)n * n * sizeof(float) <= 64 * 1024 && n <= 128,
+                "fused_bias_grad: a window of %d positions needs a %zu-byte LDS table (limit 64 KiB, 128 positions)",
+                n, (size_t)n * n * sizeof(float));
+    SSWIN_CHECK(ws_bytes >= sswin_fused_bias_grad_workspace_bytes(G, H, n), "fused_bias_grad: workspace too small");
     const FusedGroups gt = groups_of(plan, g_cap, G);
-    const int64_t windows = G / H;
-    const unsigned slices = (unsigned)std::min<int64_t>(windows, 128);
-    hipLaunchKernelGGL(rpb_grad_kernel, dim3(slices, (unsigned)H), dim3(256), (size_t)n * n * sizeof(float),
-                       static_cast<hipStream_t>(stream), gt, tokens + 3 * N, H, n, ds, d_bias);
+    const int slices = bias_grad_slices(G / H, H);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    float* partial = static_cast<float*>(ws);
+    hipLaunchKernelGGL(rpb_grad_partial_kernel, dim3((unsigned)slices, (unsigned)H), dim3(RPB_THREADS),
+                       (size_t)n * n * sizeof(float), s, gt, tokens + 3 * N, H, n, ds, partial);
+    const int64_t elems = (int64_t)H * n * n;
+    hipLaunchKernelGGL(rpb_grad_reduce_kernel, dim3((unsigned)((elems + 255) / 256)), dim3(256), 0, s, partial, slices,
+                       elems, d_bias);
     return launch_ok("fused bias gradient");
 }
 

@@ -37,6 +37,22 @@ __device__ __forceinline__ void load_run16(const T* __restrict__ p, int valid, f
     }
 }
 
+// 16 consecutive values, all valid
+template <typename T>
+__device__ __forceinline__ void load_run16_full(const T* __restrict__ p, float (&x)[16]) {
+    if (std::is_same<T, float>::value) {
+        const f32x4_u* q = reinterpret_cast<const f32x4_u*>(p);
+#pragma unroll
+        for (int v = 0; v < 4; ++v) {
+            const f32x4_u t = q[v];
+            x[4 * v] = t.x; x[4 * v + 1] = t.y; x[4 * v + 2] = t.z; x[4 * v + 3] = t.w;
+        }
+    } else {
+#pragma unroll
+        for (int s = 0; s < 16; ++s) x[s] = to_acc(p[s]);
+    }
+}
+
 __device__ __forceinline__ int clamp16(int v) { return v < 0 ? 0 : (v > 16 ? 16 : v); }
 
 __device__ __forceinline__ int acc_row(int r, int half) { return 8 * (r >> 2) + 4 * half + (r & 3); }

@@ -123,8 +123,10 @@ class _FusedWindowAttention(Function):
                 bias_dtype, bias_shape = ctx.bias_meta
                 d_bias32 = torch.zeros(bias_shape, dtype=torch.float32, device=d)
                 stream = C.c_void_p(torch.cuda.current_stream(d).cuda_stream)
+                nbytes = lib.sswin_fused_bias_grad_workspace_bytes(tp.G, H, tp.n)
+                ws = torch.empty(int(nbytes), dtype=torch.uint8, device=d)
                 _lib.check(lib.sswin_fused_bias_grad(_ptr(tp.plan), tp.g_cap, tp.G, _ptr(tp.tokens), tp.N, H, tp.n,
-                                                     _ptr(d_s), _ptr(d_bias32), stream))
+                                                     _ptr(d_s), _ptr(d_bias32), _ptr(ws), nbytes, stream))
                 d_bias = d_bias32.to(bias_dtype)
         return d_qkv, d_bias, None, None, None, None, None
 
