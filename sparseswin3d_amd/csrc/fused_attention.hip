@@ -249,20 +249,28 @@ __global__ __launch_bounds__(256) void fused_sq_kernel(FusedGroups gt, const int
             float* O = out + sq0 + j_b;
             const float* brow = EPI ? bias + (int64_t)h * n * n + pos_j : nullptr;
             const int rid0 = H * Tk + h * c;
+            // bias values of the 16 rows are gathered before any of them is used, so that the
+            // gather latencies overlap instead of adding up
+            float bv[16];
+            int m_i[16];
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const int il = acc_row(r, half);                    // row inside the block
-                const int i = bi * 32 + il;
-                int p_i = 0, m_i = 0;
+                bv[r] = 0.f;
+                m_i[r] = 0;
                 if (EPI) {                                          // all lanes take part in the shuffles
-                    p_i = __shfl(pos_a, il, 64);
-                    if (mask) m_i = __shfl(m_a, il, 64);
+                    const int il = acc_row(r, half);
+                    bv[r] = brow[__shfl(pos_a, il, 64) * n];
+                    if (mask) m_i[r] = __shfl(m_a, il, 64);
                 }
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int i = bi * 32 + acc_row(r, half);
                 if (b_in && i < c) {
                     float v = acc[r];
                     if (EPI) {
-                        v += brow[p_i * n];
-                        if (mask && m_i != m_j) v += -100.0f;
+                        v += bv[r];
+                        if (mask && m_i[r] != m_j) v += -100.0f;
                         if (row_ids) row_ids[sq0 + (int64_t)i * c + j_b] = rid0 + i;
                     }
                     O[(int64_t)i * c] = v;
