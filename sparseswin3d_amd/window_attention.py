@@ -217,6 +217,54 @@ def trunc_normal_(tensor, mean=0.0, std=1.0, a=-2.0, b=2.0):
         return tensor.clamp_(min=a, max=b)
 
 
+class _TallLinear(Function):
+    """``x @ W^T + b`` for a very tall ``x`` [N, in] (N = number of voxels).
+
+    Forward and input gradient are ordinary GEMMs.  The weight gradient ``dY^T x`` is an
+    [out x in] result reduced over N rows; a single GEMM call maps it onto out*in/tile
+    workgroups only (27 for 288 x 96), which leaves most of the 256 CUs idle.  Splitting the
+    reduction into batches (one bmm, then a sum over the batch) fills the chip.
+    """
+
+    SPLITS = 64
+
+    @staticmethod
+    def forward(ctx, x, weight, bias):
+        ctx.save_for_backward(x, weight)
+        ctx.has_bias = bias is not None
+        return torch.nn.functional.linear(x, weight, bias)
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad_out):
+        x, weight = ctx.saved_tensors
+        grad_out = grad_out.contiguous()
+        grad_x = grad_out @ weight if ctx.needs_input_grad[0] else None
+        grad_w = grad_b = None
+        if ctx.needs_input_grad[1]:
+            n = x.shape[0]
+            s = _TallLinear.SPLITS
+            rows = n // s
+            if rows >= 256:
+                main = rows * s
+                part = torch.bmm(grad_out[:main].view(s, rows, -1).transpose(1, 2), x[:main].view(s, rows, -1))
+                grad_w = part.sum(0)
+                if main < n:
+                    grad_w = grad_w + grad_out[main:].t() @ x[main:]
+            else:
+                grad_w = grad_out.t() @ x
+        if ctx.has_bias and ctx.needs_input_grad[2]:
+            grad_b = grad_out.sum(0)
+        return grad_x, grad_w, grad_b
+
+
+def tall_linear(x, layer: nn.Linear):
+    """Apply an ``nn.Linear`` to a tall 2-D input with the split-reduction weight gradient."""
+    if x.dim() == 2 and x.is_cuda:
+        return _TallLinear.apply(x, layer.weight, layer.bias)
+    return layer(x)
+
+
 def relative_position_index_3d(window_size: Sequence[int]) -> torch.Tensor:
     """[n, n] index into the (2w-1)^3 relative position bias table for a 3-D window."""
     wd, wh, ww = window_size
@@ -268,14 +316,14 @@ class WindowAttentionSparse(nn.Module):
         n = x.spatial_shape[0]
         b = x.batch_size
         c = x.features.shape[-1]
-        qkv = self.qkv(x.features).reshape(-1, 3, self.num_heads, c // self.num_heads)
+        qkv = tall_linear(x.features, self.qkv).reshape(-1, 3, self.num_heads, c // self.num_heads)
         if self.fused:
             from . import fused
             if fused.supports(qkv, n):
                 out = fused.fused_window_attention(qkv, self.relative_position_bias(n, torch.float32), x.indices,
                                                    mask, b, n, self.scale)
                 x = replace_feature(x, out)
-                return replace_feature(x, self.proj_drop(self.proj(x.features)))
+                return replace_feature(x, self.proj_drop(tall_linear(x.features, self.proj)))
         q, k_t, v = qkv_sparse_cuda(qkv, x.indices, b, n)
         attn = spspmm_block_naive(q * self.scale, k_t, "q_k")
         attn = sp_add_rpb(attn, self.relative_position_bias(n, attn.values.dtype))
@@ -285,4 +333,4 @@ class WindowAttentionSparse(nn.Module):
         out = spspmm_block_naive(attn, v, "qk_v").permute((0, 2, 1, 3))      # (window, pos, head, ch)
         unsort = ops.return_inverse(ops.flatten_indices(x.indices.T.contiguous(), [b, n]), -1)[0]
         x = replace_feature(x, out.values.reshape(x.features.shape).index_select(0, unsort))
-        return replace_feature(x, self.proj_drop(self.proj(x.features)))
+        return replace_feature(x, self.proj_drop(tall_linear(x.features, self.proj)))
