@@ -309,7 +309,9 @@ class WindowAttentionSparse(nn.Module):
 
     def relative_position_bias(self, n: int, dtype) -> torch.Tensor:
         index = self.relative_position_index[:n, :n].reshape(-1)
-        bias = self.relative_position_bias_table[index].reshape(n, n, -1)
+        # index_select: its backward is one index_add over n*n rows (advanced indexing would
+        # sort the indices on every backward pass)
+        bias = self.relative_position_bias_table.index_select(0, index).reshape(n, n, -1)
         return bias.permute(2, 0, 1).contiguous().to(dtype)
 
     def forward(self, x, mask):
