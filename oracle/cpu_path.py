@@ -66,17 +66,22 @@ def window_attention_cpu(features: torch.Tensor, win_idx: np.ndarray, n: int, nu
     pos = torch.from_numpy(win_idx[perm, 1].astype(np.int64))
     mask_t = None if mask is None else torch.from_numpy(np.asarray(mask)).to(torch.int64)
 
+    # one split per operand: its backward is a single concatenation, whereas slicing
+    # q[start:start+c] per window would make autograd build a full-size zero tensor per slice
+    sizes = [int(c) for c in counts]
+    q_w, k_w, v_w = q.split(sizes), k.split(sizes), v.split(sizes)
+
     scores, row_ids = [], []
     start = 0
     row_base = 0
-    for w, c in zip(wins, counts):
+    for k_win, (w, c) in enumerate(zip(wins, counts)):
         c = int(c)
         p = pos[start:start + c]
         if mask_t is not None:
             region = mask_t[int(w) % mask_t.shape[0]].index_select(0, p)
             penalty = (region[None, :] != region[:, None]).to(features.dtype) * -100.0
         for h in range(H):
-            s = torch.mm(q[start:start + c, h], k[start:start + c, h].t())
+            s = torch.mm(q_w[k_win][:, h], k_w[k_win][:, h].t())
             s = s + rpb[h].index_select(0, p).index_select(1, p)
             if mask_t is not None:
                 s = s + penalty
@@ -90,17 +95,10 @@ def window_attention_cpu(features: torch.Tensor, win_idx: np.ndarray, n: int, nu
     attn = sm(vals, idx_row, row_base)
 
     outs = []
-    start = 0
-    off = 0
-    for c in counts:
-        c = int(c)
-        per_head = []
-        for h in range(H):
-            p_block = attn[off:off + c * c].reshape(c, c)
-            per_head.append(torch.mm(p_block, v[start:start + c, h]))
-            off += c * c
+    blocks = attn.split([c * c for c in sizes for _ in range(H)])
+    for k_win, c in enumerate(sizes):
+        per_head = [torch.mm(blocks[k_win * H + h].reshape(c, c), v_w[k_win][:, h]) for h in range(H)]
         outs.append(torch.stack(per_head, 1).reshape(c, D))      # (token, head, channel)
-        start += c
     out_sorted = torch.cat(outs, 0)
     inv = np.empty_like(perm)
     inv[perm] = np.arange(N)

@@ -265,6 +265,38 @@ def tall_linear(x, layer: nn.Linear):
     return layer(x)
 
 
+class _BiasTableGather(Function):
+    """``table.index_select(0, index)`` whose backward adds the rows of each table entry in a
+    fixed order (``bins[t]`` lists the positions of ``index`` equal to ``t``, padded with
+    ``len(index)``), so the table gradient is the same bit pattern on every run; an
+    index_add with atomics is not."""
+
+    @staticmethod
+    def forward(ctx, table, index, bins):
+        ctx.save_for_backward(bins)
+        return table.index_select(0, index)
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad):
+        (bins,) = ctx.saved_tensors
+        padded = torch.cat([grad, grad.new_zeros(1, grad.shape[1])], 0)
+        rows = padded.index_select(0, bins.reshape(-1)).reshape(bins.shape[0], bins.shape[1], -1)
+        return rows.sum(1), None, None
+
+
+def _index_bins(index: torch.Tensor, table_rows: int) -> torch.Tensor:
+    """[table_rows, m] positions of ``index`` per table row, padded with ``len(index)``."""
+    order = torch.argsort(index, stable=True)
+    counts = torch.bincount(index, minlength=table_rows)
+    starts = torch.cumsum(counts, 0) - counts
+    m = max(int(counts.max()), 1)
+    slot = torch.arange(m, device=index.device)[None, :]
+    take = (starts[:, None] + slot).clamp_(max=max(len(index) - 1, 0))
+    bins = order[take] if len(index) else take
+    return torch.where(slot < counts[:, None], bins, torch.full_like(bins, len(index)))
+
+
 def relative_position_index_3d(window_size: Sequence[int]) -> torch.Tensor:
     """[n, n] index into the (2w-1)^3 relative position bias table for a 3-D window."""
     wd, wh, ww = window_size
@@ -306,12 +338,15 @@ class WindowAttentionSparse(nn.Module):
         self.proj = nn.Linear(dim, dim)
         self.proj_drop = nn.Dropout(proj_drop)
         trunc_normal_(self.relative_position_bias_table, std=0.02)
+        self._bias_bins = {}        # (n, device) -> (index, bins) of the deterministic bias gather
 
     def relative_position_bias(self, n: int, dtype) -> torch.Tensor:
-        index = self.relative_position_index[:n, :n].reshape(-1)
-        # index_select: its backward is one index_add over n*n rows (advanced indexing would
-        # sort the indices on every backward pass)
-        bias = self.relative_position_bias_table.index_select(0, index).reshape(n, n, -1)
+        table = self.relative_position_bias_table
+        cached = self._bias_bins.get((n, table.device))
+        if cached is None:
+            index = self.relative_position_index[:n, :n].reshape(-1)
+            cached = self._bias_bins[(n, table.device)] = (index, _index_bins(index, table.shape[0]))
+        bias = _BiasTableGather.apply(table, *cached).reshape(n, n, -1)
         return bias.permute(2, 0, 1).contiguous().to(dtype)
 
     def forward(self, x, mask):
