@@ -203,6 +203,32 @@ def kernel_table(wl, reps=20, only=None):
         ("fused bias grad", lambda: _lib.check(lib.sswin_fused_bias_grad(ptr(tp.plan), tp.g_cap, tp.G, ptr(tp.tokens), tp.N, H, b["n"], ptr(g_s), ptr(dbias), ptr(bg_ws), bg_bytes, stream)), 4 * A, 1),
     ]
 
+    # ---- the window-resident kernels (what the step runs for heads of 32 channels) ----
+    lse = torch.empty(H * N, device=dev)
+    mask_p, nmw = ptr(mask), (0 if mask is None else mask.shape[0])
+    qa = (ptr(qkv_c), 3 * D, 0, ptr(qkv_c), 3 * D, D, ptr(qkv_c), 3 * D, 2 * D)
+    da = (ptr(dqkv), 3 * D, 0, ptr(dqkv), 3 * D, D, ptr(dqkv), 3 * D, 2 * D)
+    up_r = torch.randn(N, D, device=dev)
+
+    def r_fwd():
+        _lib.check(lib.sswin_window_attention_forward(0, ptr(tp.tasks), tp.g_cap, tp.bucket_counts, ptr(tp.tokens), N, H,
+                                                      hd, *qa, C.c_float(0.17), ptr(bias), b["n"], mask_p, nmw,
+                                                      ptr(out_f), D, 0, ptr(lse), stream))
+
+    def r_bwd(sides):
+        return lambda: _lib.check(lib.sswin_window_attention_backward(
+            0, ptr(tp.tasks), tp.g_cap, tp.bucket_counts, ptr(tp.tokens), N, H, hd, *qa, C.c_float(0.17), ptr(bias),
+            b["n"], mask_p, nmw, ptr(out_f), D, 0, ptr(up_r), D, 0, ptr(lse), *da, ptr(s_f), sides, stream))
+
+    r_fwd()                                       # lse and out_f must hold a real forward for the backward timings
+    r_entries = [
+        ("resident token_plan", lambda: F.TokenPlan(b["idx"], b["slots"], b["n"], H), 28 * N + 36 * tp.G, 1),
+        ("resident forward", r_fwd, 16 * E + 4 * H * N, 1),
+        ("resident backward dQ", r_bwd(1), 24 * E + 4 * H * N, 1),
+        ("resident backward dK,dV,dS", r_bwd(2), 28 * E + 4 * A + 4 * H * N, 1),
+        ("resident bias grad", lambda: _lib.check(lib.sswin_fused_bias_grad(ptr(tp.plan), tp.g_cap, tp.G, ptr(tp.tokens), tp.N, H, b["n"], ptr(s_f), ptr(dbias), ptr(bg_ws), bg_bytes, stream)), 4 * A, 1),
+    ]
+
     def measure(items, path):
         rows_ = []
         for name, fn, nbytes, calls in items:
@@ -217,7 +243,7 @@ def kernel_table(wl, reps=20, only=None):
         # device-to-device copy of known size that calibrates the FETCH_SIZE / WRITE_SIZE counters
         src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device=dev)
         dst = torch.empty_like(src)
-        picked = [e for e in f_entries + entries if only in e[0]]
+        picked = [e for e in r_entries + f_entries + entries if only in e[0]]
         for name, fn, nbytes, calls in picked:
             log(f"profiling {name}: {reps} launches, algorithmic bytes {nbytes}")
             for _ in range(reps):
@@ -227,7 +253,7 @@ def kernel_table(wl, reps=20, only=None):
         torch.cuda.synchronize()
         log(f"calibration copy: {reps} launches of {src.numel() * 4} bytes read and written")
         return [], dict(N=N, E=E, A=A, G=G, c_max=c_max)
-    table = measure(f_entries, "fused") + measure(entries, "operators")
+    table = measure(r_entries, "resident") + measure(f_entries, "fused") + measure(entries, "operators")
     return table, dict(N=N, E=E, A=A, G=G, c_max=c_max)
 
 
@@ -322,7 +348,7 @@ def main():
         table, sizes = kernel_table(wl)
         log(f"{'kernel':36s} {'ms':>9s} {'calls':>5s} {'alg MB':>9s} {'GB/s':>9s} {'% HBM':>7s}")
         summary = {}
-        for path in ("fused", "operators"):
+        for path in ("resident", "fused", "operators"):
             rows_ = [r for r in table if r["path"] == path]
             log(f"-- {path} path, one attention forward+backward --")
             for r in rows_:
@@ -334,9 +360,9 @@ def main():
                                  frac=round(alg / ms_ / 1e6 / HBM_PEAK_GBPS, 4))
             log(f"{path} kernels, one attention fwd+bwd: {ms_:.3f} ms for {alg / 1e6:.1f} MB algorithmic "
                 f"= {alg / ms_ / 1e6:.1f} GB/s = {100 * alg / ms_ / 1e6 / HBM_PEAK_GBPS:.2f}% of HBM peak")
-        # the step runs the fused path: its slowest single-launch kernel is the dominant one
+        # the step runs the window-resident path: its slowest kernel is the dominant one
         # (the token plan is a sequence of small launches, not a kernel)
-        dom = max((r for r in table if r["path"] == "fused" and r["kernel"] != "fused token_plan"),
+        dom = max((r for r in table if r["path"] == "resident" and "token_plan" not in r["kernel"]),
                   key=lambda r: r["ms"] * r["calls"])
         roofline = dict(bound="hbm", kernel=dom["kernel"], achieved=round(dom["achieved_gbps"], 1),
                         peak=HBM_PEAK_GBPS, unit="GB/s", frac=round(dom["frac"], 4),

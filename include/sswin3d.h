@@ -167,12 +167,16 @@ int sswin_softmax_last_dim_backward(const int32_t* idx_row, const void* y, const
  *   window; pos; window.
  * plan (device int32 [5*g_cap]): rows c, T (rank of the window's first token), sq_start
  *   (exclusive scan of c*c over groups), window, head — groups ordered (window, head).
- * totals_out (host, 4 x int64): {groups G, non-empty windows, sum over groups of c*c, max c}.
+ * tasks (device int32 [4][g_cap][4], or NULL): group descriptors {T, c | head << 8, window,
+ *   sq_start} bucketed by ceil(c/32) = 1..4 for sswin_window_attention_*; the order of the
+ *   descriptors inside a bucket is unspecified.
+ * totals_out (host, 9 x int64): {groups G, non-empty windows, sum over groups of c*c, max c,
+ *   groups in bucket 1..4, groups with c > 128 (no descriptor)}; the last five are 0 without tasks.
  * (window, pos) pairs must be distinct, window in [0,B), pos in [0,n).  Synchronises `stream`. */
 size_t sswin_token_plan_workspace_bytes(int64_t N, int B, int n);
 int sswin_token_plan(const int32_t* indices, int64_t N, int B, int n, int H, int32_t* tokens,
-                     int32_t* plan, int64_t g_cap, int64_t* totals_out, void* ws, size_t ws_bytes,
-                     void* stream);
+                     int32_t* plan, int64_t g_cap, int32_t* tasks, int64_t* totals_out, void* ws,
+                     size_t ws_bytes, void* stream);
 
 /* Token tensors are dense [N, stride] arrays of `dtype`; element (voxel v, head h, channel ch) is
  * base[v*stride + col0 + h*hd + ch].  "sq" arrays are fp32 arrays of all [c x c] blocks.
@@ -200,12 +204,47 @@ int sswin_fused_sq_to_tokens(int dtype, int a_kmajor, const int32_t* plan, int64
 
 /* d_bias[h, pos_i, pos_j] += ds over all windows (the backward of swin3d_base.py:557-566, which
  * autograd performs as an index_add).  d_bias: fp32 [H,n,n], accumulated into (zero it first).
- * n*n*4 bytes must fit 64 KiB of LDS.  Partial tables are built with LDS float atomics (the
- * summation order inside a workgroup varies) and summed without global atomics.  Asynchronous. */
+ * n*n*4 bytes must fit 64 KiB of LDS.  No atomics: every table row is owned by one wavefront
+ * and partial tables are summed in a fixed order, so the result is reproducible.  Asynchronous. */
 size_t sswin_fused_bias_grad_workspace_bytes(int64_t G, int H, int n);
 int sswin_fused_bias_grad(const int32_t* plan, int64_t g_cap, int64_t G, const int32_t* tokens,
                           int64_t N, int H, int n, const float* ds, float* d_bias, void* ws,
                           size_t ws_bytes, void* stream);
+
+/* ---- window-resident attention (whole forward / backward of the attention core) ---------- */
+
+/* Forward of sparse_swin/swin3d_base.py:660-672 for every (window, head) group in one pass:
+ * O = softmax((scale*Q) K^T + bias + mask) V with the operator's softmax semantics
+ * (ops.cu:128-167: max(0,rowmax), sum + 1e-8).  The attention matrix stays in registers.
+ * tasks / bucket_counts (host, 4 x int64) come from sswin_token_plan; q, k, v, o are token
+ * tensors as above with hd = 32; lse (fp32 [H*N]) receives m + log(sum) of attention row
+ * H*T + h*c + i (the row id of the sparse softmax).  Windows of at most 128 tokens.  Asynchronous. */
+int sswin_window_attention_forward(int dtype, const int32_t* tasks, int64_t g_cap,
+                                   const int64_t* bucket_counts, const int32_t* tokens, int64_t N,
+                                   int H, int hd, const void* q_base, int64_t q_stride, int q_col0,
+                                   const void* k_base, int64_t k_stride, int k_col0,
+                                   const void* v_base, int64_t v_stride, int v_col0, float scale,
+                                   const float* bias, int n, const int8_t* mask, int n_mask_windows,
+                                   void* o_base, int64_t o_stride, int o_col0, float* lse,
+                                   void* stream);
+
+/* Backward of the same (swin3d_base.py:106-138 and :177-188 composed): from O, dO and lse,
+ * recomputes P per tile and writes dQ = scale dS K, dK = scale dS^T Q, dV = P^T dO with
+ * dS = P (dP - rowsum(dO o O)).  ds_out (fp32 "sq" array in plan order, or NULL) receives dS
+ * for sswin_fused_bias_grad.  sides: 1 = dQ only, 2 = dK and dV (and dS) only, 3 = all.
+ * Asynchronous. */
+int sswin_window_attention_backward(int dtype, const int32_t* tasks, int64_t g_cap,
+                                    const int64_t* bucket_counts, const int32_t* tokens, int64_t N,
+                                    int H, int hd, const void* q_base, int64_t q_stride, int q_col0,
+                                    const void* k_base, int64_t k_stride, int k_col0,
+                                    const void* v_base, int64_t v_stride, int v_col0, float scale,
+                                    const float* bias, int n, const int8_t* mask, int n_mask_windows,
+                                    const void* o_base, int64_t o_stride, int o_col0,
+                                    const void* do_base, int64_t do_stride, int do_col0,
+                                    const float* lse, void* dq_base, int64_t dq_stride, int dq_col0,
+                                    void* dk_base, int64_t dk_stride, int dk_col0, void* dv_base,
+                                    int64_t dv_stride, int dv_col0, float* ds_out, int sides,
+                                    void* stream);
 
 #ifdef __cplusplus
 }

@@ -16,6 +16,7 @@
 // The softmax between the two products is the ordinary sparse row softmax; its row ids are a
 // by-product of the first kernel.
 #include <algorithm>
+#include <cstring>
 
 #include "mfma_block.hpp"
 #include "scan.hpp"
@@ -116,6 +117,36 @@ struct WindowStore {
 
 __global__ void tp_zero_kernel(int32_t* p, int n) {
     if ((int)threadIdx.x < n) p[threadIdx.x] = 0;
+}
+
+// Groups bucketed by their number of 32-token tiles (bucket b: 32*b < c <= 32*(b+1), b = 0..3;
+// counts[4] counts larger groups, which have no descriptor).  Descriptor = {T, c | head << 8,
+// window, sq_start}.  Slots inside a bucket are handed out with one atomic per wavefront and
+// bucket, so the order inside a bucket varies from run to run; consumers treat the groups of a
+// bucket as an unordered set.
+__global__ __launch_bounds__(256) void tp_tasks_kernel(const int32_t* __restrict__ plan, int64_t g_cap, int H,
+                                                       const int64_t* __restrict__ scan_total,
+                                                       int4* __restrict__ tasks, int32_t* __restrict__ counts) {
+    const int64_t G = (scan_total[0] & 0xffffffffll) * H;
+    const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    const bool live = g < G && g < g_cap;
+    const int c = live ? plan[g] : 0;
+    const int b = live ? min((c - 1) >> 5, 4) : -1;
+    const int lane = threadIdx.x & 63;
+    int slot = 0;
+#pragma unroll
+    for (int q = 0; q < 5; ++q) {
+        const unsigned long long mine = __ballot(b == q);
+        if (mine == 0) continue;
+        const int leader = __ffsll((long long)mine) - 1;
+        int base = 0;
+        if (lane == leader) base = atomicAdd(&counts[q], __popcll(mine));
+        base = __shfl(base, leader, 64);
+        if (b == q) slot = base + __popcll(mine & ((1ull << lane) - 1ull));
+    }
+    if (live && b < 4)
+        tasks[(int64_t)b * g_cap + slot] =
+            make_int4(plan[g_cap + g], c | (plan[4 * g_cap + g] << 8), plan[3 * g_cap + g], plan[2 * g_cap + g]);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -503,11 +534,11 @@ size_t sswin_token_plan_workspace_bytes(int64_t N, int B, int n) {
 }
 
 int sswin_token_plan(const int32_t* indices, int64_t N, int B, int n, int H, int32_t* tokens,
-                     int32_t* plan, int64_t g_cap, int64_t* totals_out, void* ws, size_t ws_bytes,
-                     void* stream) {
+                     int32_t* plan, int64_t g_cap, int32_t* tasks, int64_t* totals_out, void* ws,
+                     size_t ws_bytes, void* stream) {
     SSWIN_CHECK(N >= 0 && B > 0 && n > 0 && H > 0, "token_plan: bad sizes");
     SSWIN_CHECK(totals_out, "token_plan: totals_out is null");
-    totals_out[0] = totals_out[1] = totals_out[2] = totals_out[3] = 0;
+    for (int i = 0; i < 9; ++i) totals_out[i] = 0;
     if (N == 0) return 0;
     SSWIN_CHECK(indices && tokens && plan && ws, "token_plan: null pointer");
     SSWIN_CHECK(N < (int64_t)INT32_MAX, "token_plan: too many voxels");
@@ -516,7 +547,7 @@ int sswin_token_plan(const int32_t* indices, int64_t N, int B, int n, int H, int
     hipStream_t s = static_cast<hipStream_t>(stream);
     Carver cv(ws, ws_bytes);
     const size_t words = tp_words(B, n);
-    int64_t* total_dev = cv.take<int64_t>(2);
+    int64_t* total_dev = cv.take<int64_t>(8);        // scan total, {c_max, -}, five bucket counters, -
     uint32_t* bits = cv.take<uint32_t>(words);
     int32_t* word_prefix = cv.take<int32_t>(words);
     int64_t* tile_sums = cv.take<int64_t>(
@@ -528,10 +559,11 @@ int sswin_token_plan(const int32_t* indices, int64_t N, int B, int n, int H, int
     int32_t* tok_pos = tokens + 3 * N;
     int32_t* tok_win = tokens + 4 * N;
     int32_t* cmax = reinterpret_cast<int32_t*>(total_dev + 1);
+    int32_t* bucket_counts = reinterpret_cast<int32_t*>(total_dev + 2);
 
     const unsigned fill_blocks = (unsigned)std::min<size_t>((words + 255) / 256, 4096);
     hipLaunchKernelGGL(tp_fill_kernel, dim3(fill_blocks), dim3(256), 0, s, bits, (int64_t)words, 0u);
-    hipLaunchKernelGGL(tp_zero_kernel, dim3(1), dim3(64), 0, s, cmax, 2);
+    hipLaunchKernelGGL(tp_zero_kernel, dim3(1), dim3(64), 0, s, cmax, 8);
     const unsigned nb = (unsigned)((N + 255) / 256);
     hipLaunchKernelGGL(tp_set_bits_kernel, dim3(nb), dim3(256), 0, s, indices, N, n, bits);
     TpPopcLoad pl{bits};
@@ -544,7 +576,10 @@ int sswin_token_plan(const int32_t* indices, int64_t N, int B, int n, int H, int
     WindowLoad wl{tok_T, tok_c};
     WindowStore wst{tok_c, tok_win, plan, g_cap, H, cmax};
     if (device_exclusive_scan<int64_t>(wl, wst, N, tile_sums, total_dev, s, "token_plan window scan")) return 1;
-    int64_t host[2] = {0, 0};
+    if (tasks)
+        hipLaunchKernelGGL(tp_tasks_kernel, dim3((unsigned)((g_cap + 255) / 256)), dim3(256), 0, s, plan, g_cap, H,
+                           total_dev, reinterpret_cast<int4*>(tasks), bucket_counts);
+    int64_t host[5] = {0, 0, 0, 0, 0};
     SSWIN_HIP(hipMemcpyAsync(host, total_dev, sizeof(host), hipMemcpyDeviceToHost, s));
     SSWIN_HIP(hipStreamSynchronize(s));
     const int64_t windows = host[0] & 0xffffffffll;
@@ -555,6 +590,11 @@ int sswin_token_plan(const int32_t* indices, int64_t N, int B, int n, int H, int
     totals_out[1] = windows;
     totals_out[2] = s2 * H;
     totals_out[3] = (int32_t)(host[1] & 0xffffffffll);
+    if (tasks) {
+        int32_t counts[6];
+        memcpy(counts, host + 2, sizeof(counts));
+        for (int b = 0; b < 5; ++b) totals_out[4 + b] = counts[b];
+    }
     SSWIN_CHECK(windows * H <= g_cap, "token_plan: %lld groups exceed the plan capacity %lld",
                 (long long)(windows * H), (long long)g_cap);
     return 0;

@@ -45,14 +45,19 @@ class TokenPlan:
         self.g_cap = max(1, min(N, self.B) * self.H)
         self.tokens = torch.empty(5 * max(N, 1), dtype=torch.int32, device=d)
         self.plan = torch.empty(5 * self.g_cap, dtype=torch.int32, device=d)
-        totals = (C.c_int64 * 4)()
+        # group descriptors of the window-resident kernels, bucketed by ceil(c / 32)
+        self.tasks = torch.empty(16 * self.g_cap, dtype=torch.int32, device=d)
+        totals = (C.c_int64 * 9)()
         with torch.cuda.device(d):
             nbytes = lib.sswin_token_plan_workspace_bytes(N, self.B, self.n)
             ws = torch.empty(int(nbytes), dtype=torch.uint8, device=d)
             stream = C.c_void_p(torch.cuda.current_stream(d).cuda_stream)
             _lib.check(lib.sswin_token_plan(_ptr(indices), N, self.B, self.n, self.H, _ptr(self.tokens),
-                                            _ptr(self.plan), self.g_cap, totals, _ptr(ws), nbytes, stream))
+                                            _ptr(self.plan), self.g_cap, _ptr(self.tasks), totals, _ptr(ws),
+                                            nbytes, stream))
         self.G, self.windows, self.A, self.c_max = (int(totals[i]) for i in range(4))
+        self.bucket_counts = (C.c_int64 * 4)(*(int(totals[4 + b]) for b in range(4)))
+        self.oversize_groups = int(totals[8])
         self.device = d
 
 
@@ -131,10 +136,90 @@ class _FusedWindowAttention(Function):
         return d_qkv, d_bias, None, None, None, None, None
 
 
-def fused_window_attention(qkv, bias, indices, mask, batch_size, n, scale):
+def _token_args(t, stride, col0):
+    return _ptr(t), stride, col0
+
+
+class _ResidentWindowAttention(Function):
+    """Window-resident kernels: the attention matrix never reaches HBM.  Saved for backward:
+    qkv, the attention output and one log-sum-exp per attention row."""
+
+    @staticmethod
+    def forward(ctx, qkv, bias, indices, mask, batch_size, n, scale):
+        qkv = qkv.contiguous()
+        N, _, H, hd = qkv.shape
+        D = H * hd
+        dtype = qkv.dtype
+        d = qkv.device
+        tp = TokenPlan(indices, batch_size, n, H)
+        if tp.oversize_groups:
+            raise RuntimeError(f"window-resident attention: {tp.oversize_groups} groups hold more than 128 tokens")
+        bias32 = bias.detach().to(torch.float32).contiguous()
+        if mask is not None:
+            mask = mask.to(torch.int8).contiguous()
+        lib = _lib.load()
+        with torch.cuda.device(d):
+            out = torch.empty((N, D), dtype=dtype, device=d)
+            lse = torch.empty(max(H * N, 1), dtype=torch.float32, device=d)
+            stream = C.c_void_p(torch.cuda.current_stream(d).cuda_stream)
+            _lib.check(lib.sswin_window_attention_forward(
+                _DTYPE_CODE[dtype], _ptr(tp.tasks), tp.g_cap, tp.bucket_counts, _ptr(tp.tokens), N, H, hd,
+                *_token_args(qkv, 3 * D, 0), *_token_args(qkv, 3 * D, D), *_token_args(qkv, 3 * D, 2 * D),
+                C.c_float(scale), _ptr(bias32), n, _ptr(mask), 0 if mask is None else mask.shape[0],
+                *_token_args(out, D, 0), _ptr(lse), stream))
+        ctx.save_for_backward(qkv, out, lse, bias32, mask)
+        ctx.tp, ctx.scale, ctx.bias_meta = tp, scale, (bias.dtype, bias.shape)
+        return out
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad_out):
+        qkv, out, lse, bias32, mask = ctx.saved_tensors
+        tp, scale = ctx.tp, ctx.scale
+        N, _, H, hd = qkv.shape
+        D = H * hd
+        dtype = qkv.dtype
+        d = qkv.device
+        grad_out = grad_out.contiguous().to(dtype)
+        lib = _lib.load()
+        with torch.cuda.device(d):
+            d_qkv = torch.empty_like(qkv)
+            want_bias = ctx.needs_input_grad[1]
+            d_s = torch.empty(max(tp.A, 1), dtype=torch.float32, device=d) if want_bias else None
+            stream = C.c_void_p(torch.cuda.current_stream(d).cuda_stream)
+            _lib.check(lib.sswin_window_attention_backward(
+                _DTYPE_CODE[dtype], _ptr(tp.tasks), tp.g_cap, tp.bucket_counts, _ptr(tp.tokens), N, H, hd,
+                *_token_args(qkv, 3 * D, 0), *_token_args(qkv, 3 * D, D), *_token_args(qkv, 3 * D, 2 * D),
+                C.c_float(scale), _ptr(bias32), tp.n, _ptr(mask), 0 if mask is None else mask.shape[0],
+                *_token_args(out, D, 0), *_token_args(grad_out, D, 0), _ptr(lse),
+                *_token_args(d_qkv, 3 * D, 0), *_token_args(d_qkv, 3 * D, D), *_token_args(d_qkv, 3 * D, 2 * D),
+                _ptr(d_s), 3, stream))
+            d_bias = None
+            if want_bias:
+                bias_dtype, bias_shape = ctx.bias_meta
+                d_bias32 = torch.zeros(bias_shape, dtype=torch.float32, device=d)
+                nbytes = lib.sswin_fused_bias_grad_workspace_bytes(tp.G, H, tp.n)
+                ws = torch.empty(int(nbytes), dtype=torch.uint8, device=d)
+                _lib.check(lib.sswin_fused_bias_grad(_ptr(tp.plan), tp.g_cap, tp.G, _ptr(tp.tokens), tp.N, H, tp.n,
+                                                     _ptr(d_s), _ptr(d_bias32), _ptr(ws), nbytes, stream))
+                d_bias = d_bias32.to(bias_dtype)
+        return d_qkv, d_bias, None, None, None, None, None
+
+
+def fused_window_attention(qkv, bias, indices, mask, batch_size, n, scale, resident=None):
     """``qkv`` [N,3,H,hd], ``bias`` [H,n,n], ``indices`` int32 [N,2] (window,pos), ``mask`` int8
-    [nW,n] or None -> attention output [N, H*hd] in the caller's voxel order."""
-    return _FusedWindowAttention.apply(qkv, bias, indices, mask, batch_size, n, scale)
+    [nW,n] or None -> attention output [N, H*hd] in the caller's voxel order.
+
+    ``resident`` selects the window-resident kernels (default: whenever they apply, i.e. heads
+    of 32 channels); otherwise the block products with the attention matrix in HBM are used."""
+    if resident is None:
+        resident = supports_resident(qkv, n)
+    fn = _ResidentWindowAttention if resident else _FusedWindowAttention
+    return fn.apply(qkv, bias, indices, mask, batch_size, n, scale)
+
+
+def supports_resident(qkv: torch.Tensor, n: int) -> bool:
+    return supports(qkv, n) and qkv.shape[-1] == 32 and n <= 128
 
 
 def supports(qkv: torch.Tensor, n: int) -> bool:

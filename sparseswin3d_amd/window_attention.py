@@ -316,10 +316,14 @@ class WindowAttentionSparse(nn.Module):
 
     ``fused`` (class or instance attribute, default True) selects the fused HIP path of
     :mod:`sparseswin3d_amd.fused`; with ``fused = False`` the forward pass is the
-    operator-by-operator composition of the reference.  Both give the same result.
+    operator-by-operator composition of the reference.  ``resident`` picks between the two
+    fused variants: True = window-resident kernels (attention matrix kept in registers, heads
+    of 32 channels only), False = block products with the attention matrix in HBM, None =
+    resident whenever it applies.  All paths give the same result.
     """
 
     fused = True
+    resident = None
 
     def __init__(self, dim: int, num_heads: int, window_size: Sequence[int], qkv_bias: bool = False,
                  attn_drop: float = 0.0, proj_drop: float = 0.0) -> None:
@@ -358,7 +362,7 @@ class WindowAttentionSparse(nn.Module):
             from . import fused
             if fused.supports(qkv, n):
                 out = fused.fused_window_attention(qkv, self.relative_position_bias(n, torch.float32), x.indices,
-                                                   mask, b, n, self.scale)
+                                                   mask, b, n, self.scale, self.resident)
                 x = replace_feature(x, out)
                 return replace_feature(x, self.proj_drop(tall_linear(x.features, self.proj)))
         q, k_t, v = qkv_sparse_cuda(qkv, x.indices, b, n)

@@ -50,3 +50,14 @@ def close(out, ref, rtol, what=""):
     worst = np.argmax(err - bound)
     assert (err <= bound).all(), (f"{what}: worst element {worst}: out={out.flat[worst]!r} "
                                   f"ref={ref.flat[worst]!r} err={err.flat[worst]:.3e} bound={bound.flat[worst]:.3e}")
+
+
+PATHS = ["resident", "fused", "operators"]
+
+
+def set_path(attn, path):
+    """Select the implementation behind WindowAttentionSparse.forward: "resident" = window-resident
+    kernels, "fused" = block products with the attention matrix in memory, "operators" = the
+    operator-by-operator composition of the reference."""
+    attn.fused = path != "operators"
+    attn.resident = {"resident": True, "fused": False, "operators": None}[path]

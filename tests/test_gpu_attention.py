@@ -8,7 +8,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import close
+from helpers import PATHS, close, set_path
 
 pytestmark = pytest.mark.gpu
 
@@ -33,10 +33,10 @@ def _cpu_attention(attn, feats64, win_idx, n, mask, softmax="ops"):
     return out, leaves
 
 
-@pytest.mark.parametrize("fused", [True, False], ids=["fused", "operators"])
+@pytest.mark.parametrize("path", PATHS)
 @pytest.mark.parametrize("shift", [(0, 0, 0), (2, 2, 2)])
 @pytest.mark.parametrize("dim,heads", [(96, 3), (64, 2)])
-def test_window_attention_forward_backward(shift, dim, heads, fused):
+def test_window_attention_forward_backward(shift, dim, heads, path):
     from sparseswin3d_amd import synth
     from sparseswin3d_amd.window_attention import SparseVoxelTensor, WindowAttentionSparse
     torch.manual_seed(0)
@@ -44,7 +44,7 @@ def test_window_attention_forward_backward(shift, dim, heads, fused):
     win_idx, nw, n = synth.window_indices(c4, grid, (5, 5, 5), shift)
     N = len(win_idx)
     attn = WindowAttentionSparse(dim, heads, (5, 5, 5), qkv_bias=True).cuda()
-    attn.fused = fused
+    set_path(attn, path)
     with torch.no_grad():
         attn.relative_position_bias_table.normal_(0, 0.5)       # make the bias matter
     mask_np = synth.shift_region_mask(synth.padded_shape(grid, (5, 5, 5)), (5, 5, 5), (2, 2, 2)) if any(shift) else None

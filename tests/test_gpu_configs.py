@@ -13,7 +13,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import close, qkv_operands
+from helpers import PATHS, close, qkv_operands, set_path
 
 pytestmark = pytest.mark.gpu
 
@@ -164,13 +164,13 @@ def _gpu(attn, feats, idx, B, n, mask, upstream=None):
     return out.detach(), f.grad
 
 
-@pytest.mark.parametrize("fused", [True, False], ids=["fused", "operators"])
-def test_cfg1_forward_against_cpu_path(fused):
+@pytest.mark.parametrize("path", PATHS)
+def test_cfg1_forward_against_cpu_path(path):
     """Configuration 1: one forward, regular windows, fp32, ~22k voxels."""
     w = _workload("cfg1")
     idx, B, n, _ = _windows(w, (0, 0, 0))
     attn = _attention(w.dim, w.heads, torch.float32)
-    attn.fused = fused
+    set_path(attn, path)
     torch.manual_seed(1)
     feats = torch.randn(len(idx), w.dim)
     out, _ = _gpu(attn, feats, idx, B, n, None)
@@ -179,15 +179,15 @@ def test_cfg1_forward_against_cpu_path(fused):
     close(host(out), ref.numpy(), 1e-5, "cfg1 forward")
 
 
-@pytest.mark.parametrize("cfg,fused", [("cfg2", True), ("cfg3", True), ("cfg3", False)],
-                         ids=["cfg2-fused", "cfg3-fused", "cfg3-operators"])
-def test_shifted_forward_backward_against_cpu_path(cfg, fused):
+@pytest.mark.parametrize("cfg,path", [("cfg2", "resident"), ("cfg2", "fused"), ("cfg3", "resident"), ("cfg3", "fused"),
+                                      ("cfg3", "operators")])
+def test_shifted_forward_backward_against_cpu_path(cfg, path):
     """Configurations 2 (second block of the pair) and 3: shifted windows with the region mask,
     fp32 forward + backward with N(0,1) upstream gradients."""
     w = _workload(cfg)
     idx, B, n, mask = _windows(w, (2, 2, 2))
     attn = _attention(w.dim, w.heads, torch.float32)
-    attn.fused = fused
+    set_path(attn, path)
     torch.manual_seed(2)
     feats = torch.randn(len(idx), w.dim)
     up = torch.randn(len(idx), w.dim)
@@ -204,13 +204,13 @@ def test_shifted_forward_backward_against_cpu_path(cfg, fused):
           "d bias table")
 
 
-@pytest.mark.parametrize("fused", [True, False], ids=["fused", "operators"])
-def test_cfg4_bf16_dense_windows_against_cpu_fp64(fused):
+@pytest.mark.parametrize("path", PATHS)
+def test_cfg4_bf16_dense_windows_against_cpu_fp64(path):
     """Configuration 4: ~8k voxels in windows of 100-125 tokens, dim 768, 24 heads, bf16."""
     w = _workload("cfg4")
     idx, B, n, mask = _windows(w, (2, 2, 2))
     attn = _attention(w.dim, w.heads, torch.bfloat16)
-    attn.fused = fused
+    set_path(attn, path)
     torch.manual_seed(3)
     feats = (torch.randn(len(idx), w.dim) * 0.5).to(torch.bfloat16)
     up = torch.randn(len(idx), w.dim).to(torch.bfloat16)
@@ -230,8 +230,8 @@ def test_cfg5_four_stage_encoder_bf16_forward():
     Each stage's attention is checked against the fp64 CPU path fed with the same stage input.
 
     Stage 1 has 216 320 window slots: slots*125*96 exceeds 2^31, where the reference's int32
-    row-major hash (ops.cu:264) wraps and its own ordering is undefined; the fused path orders
-    by the exact key, so stage 1 is run on it.  The later stages also run the operator path."""
+    row-major hash (ops.cu:264) wraps and its own ordering is undefined; the fused paths order
+    by the exact key, so stage 1 is run on them.  The later stages also run the operator path."""
     from sparseswin3d_amd import synth
     w = _workload("cfg5")
     coords = w.coords4
@@ -244,13 +244,16 @@ def test_cfg5_four_stage_encoder_bf16_forward():
         B = nw * w.batch_size
         mask = synth.shift_region_mask(synth.padded_shape(shape, (5, 5, 5)), (5, 5, 5), (2, 2, 2))
         attn = _attention(dim, H, torch.bfloat16, seed=10 + stage)
-        attn.fused = True
+        set_path(attn, "resident")
         out, _ = _gpu(attn, feats, idx, B, n, mask)
         with torch.no_grad():
             ref, _ = _cpu(attn, feats.double(), idx, n, mask)
-        close(host(out), ref.numpy(), 2e-2, f"stage {stage + 1} fused")
+        close(host(out), ref.numpy(), 2e-2, f"stage {stage + 1} resident")
+        set_path(attn, "fused")
+        out_f, _ = _gpu(attn, feats, idx, B, n, mask)
+        close(host(out_f), ref.numpy(), 2e-2, f"stage {stage + 1} fused")
         if B * n * dim < 2 ** 31:
-            attn.fused = False
+            set_path(attn, "operators")
             out_ops, _ = _gpu(attn, feats, idx, B, n, mask)
             close(host(out_ops), ref.numpy(), 2e-2, f"stage {stage + 1} operators")
         else:
@@ -306,7 +309,8 @@ def test_cfg2_properties_voxel_order_and_linearity():
     out2, _ = _gpu(attn, feats, idx, B, n, mask, up1)
     assert torch.equal(out2, out)
     assert torch.equal(attn.relative_position_bias_table.grad, tg1)      # fixed-order table gradient
-    attn.fused = False
-    out_ops, g_ops = _gpu(attn, feats, idx, B, n, mask, up1)
-    close(host(out_ops), host(out), 1e-5, "operator path forward")
-    close(host(g_ops), host(g1), 1e-5, "operator path backward")
+    for path in ("fused", "operators"):
+        set_path(attn, path)
+        out_o, g_o = _gpu(attn, feats, idx, B, n, mask, up1)
+        close(host(out_o), host(out), 1e-5, f"{path} path forward")
+        close(host(g_o), host(g1), 1e-5, f"{path} path backward")

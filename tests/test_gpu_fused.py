@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import close, ragged_window_indices, random_window_indices
+from helpers import PATHS, close, ragged_window_indices, random_window_indices, set_path
 
 pytestmark = pytest.mark.gpu
 
@@ -69,20 +69,22 @@ def test_fused_equals_operator_path(shift):
     feats = torch.randn(len(idx), 96, device="cuda")
     up = torch.randn(len(idx), 96, device="cuda")
     res = {}
-    for fused in (True, False):
-        attn.fused = fused
+    for path in PATHS:
+        set_path(attn, path)
         attn.zero_grad()
         f = feats.clone().requires_grad_(True)
         out = attn(SparseVoxelTensor(f, torch.from_numpy(idx).cuda(), (n,), nw), mask).features
         out.backward(up)
-        res[fused] = [t.detach().cpu().numpy() for t in
+        res[path] = [t.detach().cpu().numpy() for t in
                       (out, f.grad, attn.qkv.weight.grad, attn.relative_position_bias_table.grad)]
-    for a, b, what in zip(res[True], res[False], ("out", "d feats", "d qkv.w", "d bias table")):
-        close(a, b, 1e-5, what)
+    for path in ("resident", "fused"):
+        for a, b, what in zip(res[path], res["operators"], ("out", "d feats", "d qkv.w", "d bias table")):
+            close(a, b, 1e-5, f"{path}: {what}")
 
 
+@pytest.mark.parametrize("path", ["resident", "fused"])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
-def test_fused_16bit_against_cpu_fp64(dtype):
+def test_fused_16bit_against_cpu_fp64(dtype, path):
     from oracle import cpu_path
     from sparseswin3d_amd import synth
     from sparseswin3d_amd.window_attention import SparseVoxelTensor
@@ -90,6 +92,7 @@ def test_fused_16bit_against_cpu_fp64(dtype):
     idx, nw, n = synth.window_indices(c4, (10, 10, 10), (5, 5, 5), (2, 2, 2))
     mask_np = synth.shift_region_mask((10, 10, 10), (5, 5, 5), (2, 2, 2))
     attn = _modules(64, 2, dtype)
+    set_path(attn, path)
     feats = (torch.randn(len(idx), 64) * 0.5).to(dtype)
     x = SparseVoxelTensor(feats.cuda(), torch.from_numpy(idx).cuda(), (n,), nw)
     out = attn(x, torch.from_numpy(mask_np).cuda()).features
@@ -97,4 +100,82 @@ def test_fused_16bit_against_cpu_fp64(dtype):
     rpb = p["relative_position_bias_table"][p["relative_position_index"].reshape(-1).long()].reshape(n, n, -1).permute(2, 0, 1)
     ref = cpu_path.window_attention_cpu(feats.double(), idx, n, 2, p["qkv.weight"], p["qkv.bias"], p["proj.weight"],
                                         p["proj.bias"], rpb, mask_np)
-    close(out.detach().double().cpu().numpy(), ref.numpy(), 2e-2, f"fused {dtype}")
+    close(out.detach().double().cpu().numpy(), ref.numpy(), 2e-2, f"{path} {dtype}")
+
+
+@pytest.mark.parametrize("mix", ["tiny", "edges", "full", "mixed"])
+@pytest.mark.parametrize("use_mask", [False, True], ids=["nomask", "mask"])
+def test_resident_kernels_on_ragged_windows(mix, use_mask):
+    """Window-resident forward/backward through the C ABI on hand-picked occupancies (1 token,
+    around the 32/64/96 tile edges, full 125-token windows, empty slots) against dense fp64
+    attention per window; also checks the bucket counts of the task list."""
+    import ctypes as C
+    from sparseswin3d_amd import _lib
+    from sparseswin3d_amd.fused import TokenPlan, _ptr
+    mixes = {"tiny": [1, 2, 3, 1, 5, 4], "edges": [31, 32, 33, 0, 63, 64, 65, 1, 95, 96, 97],
+             "full": [125, 124, 100, 7], "mixed": [1, 40, 2, 125, 0, 0, 17, 32, 90, 3, 3, 3, 3, 64]}
+    counts = mixes[mix]
+    rng = np.random.default_rng(len(mix) + use_mask)
+    n, H, hd = 125, 3, 32
+    D = H * hd
+    ind = ragged_window_indices(rng, counts, n)
+    N, B = len(ind), len(counts)
+    tp = TokenPlan(torch.from_numpy(ind).cuda(), B, n, H)
+    want = [sum(1 for c in counts if 32 * b < c <= 32 * (b + 1)) * H for b in range(4)]
+    assert list(tp.bucket_counts) == want and tp.oversize_groups == 0
+    qkv = torch.randn(N, 3 * D, dtype=torch.float64)
+    bias = torch.randn(H, n, n, dtype=torch.float64)
+    d_out = torch.randn(N, D, dtype=torch.float64)
+    mask = torch.from_numpy(rng.integers(0, 3, size=(4, n)).astype(np.int8)) if use_mask else None
+    scale = hd ** -0.5
+
+    lib = _lib.load()
+    q32 = qkv.float().cuda()
+    b32 = bias.float().cuda()
+    do32 = d_out.float().cuda()
+    m_dev = None if mask is None else mask.cuda()
+    out = torch.full((N, D), float("nan"), device="cuda")
+    lse = torch.empty(H * N, device="cuda")
+    dqkv = torch.full((N, 3 * D), float("nan"), device="cuda")
+    ds = torch.full((tp.A,), float("nan"), device="cuda")
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    nmw = 0 if mask is None else mask.shape[0]
+    _lib.check(lib.sswin_window_attention_forward(
+        0, _ptr(tp.tasks), tp.g_cap, tp.bucket_counts, _ptr(tp.tokens), N, H, hd, _ptr(q32), 3 * D, 0, _ptr(q32), 3 * D, D,
+        _ptr(q32), 3 * D, 2 * D, C.c_float(scale), _ptr(b32), n, _ptr(m_dev), nmw, _ptr(out), D, 0, _ptr(lse), stream))
+    _lib.check(lib.sswin_window_attention_backward(
+        0, _ptr(tp.tasks), tp.g_cap, tp.bucket_counts, _ptr(tp.tokens), N, H, hd, _ptr(q32), 3 * D, 0, _ptr(q32), 3 * D, D,
+        _ptr(q32), 3 * D, 2 * D, C.c_float(scale), _ptr(b32), n, _ptr(m_dev), nmw, _ptr(out), D, 0, _ptr(do32), D, 0,
+        _ptr(lse), _ptr(dqkv), 3 * D, 0, _ptr(dqkv), 3 * D, D, _ptr(dqkv), 3 * D, 2 * D, _ptr(ds), 3, stream))
+
+    # dense fp64 reference per window with autograd
+    qkv_r = q32.double().cpu().requires_grad_(True)
+    bias_r = b32.double().cpu().requires_grad_(True)
+    ref = torch.zeros(N, D, dtype=torch.float64)
+    order = np.lexsort((ind[:, 1], ind[:, 0]))
+    pieces = []
+    for w in np.unique(ind[:, 0]):
+        vox = torch.from_numpy(order[ind[order, 0] == w])
+        pos = torch.from_numpy(ind[vox.numpy(), 1].astype(np.int64))
+        x = qkv_r[vox].reshape(len(vox), 3, H, hd)
+        s = torch.einsum("ihc,jhc->hij", x[:, 0] * scale, x[:, 1]) + bias_r[:, pos][:, :, pos]
+        if mask is not None:
+            r = mask[int(w) % mask.shape[0]].long()[pos]
+            s = s + (r[None, :] != r[:, None]).double() * -100.0
+        m = s.max(-1, keepdim=True).values.clamp(min=0)
+        e = (s - m).exp()
+        p = e / (e.sum(-1, keepdim=True) + 1e-8)
+        pieces.append((vox, torch.einsum("hij,jhc->ihc", p, x[:, 2]).reshape(len(vox), D)))
+    ref = torch.zeros(N, D, dtype=torch.float64).index_put((torch.cat([v for v, _ in pieces]),),
+                                                            torch.cat([o for _, o in pieces]))
+    ref.backward(do32.double().cpu())
+    close(out.cpu().numpy(), ref.detach().numpy(), 1e-5, "O")
+    close(dqkv.cpu().numpy(), qkv_r.grad.numpy(), 1e-5, "d qkv")
+    # bias gradient from the stored dS
+    d_bias = torch.zeros(H, n, n, device="cuda")
+    nbytes = lib.sswin_fused_bias_grad_workspace_bytes(tp.G, H, n)
+    ws = torch.empty(int(nbytes), dtype=torch.uint8, device="cuda")
+    _lib.check(lib.sswin_fused_bias_grad(_ptr(tp.plan), tp.g_cap, tp.G, _ptr(tp.tokens), N, H, n, _ptr(ds), _ptr(d_bias),
+                                         _ptr(ws), nbytes, stream))
+    assert not torch.isnan(ds).any()
+    close(d_bias.cpu().numpy(), bias_r.grad.numpy(), 1e-5, "d bias")
