@@ -21,6 +21,7 @@ ARCH = "gfx950"
 FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
          "-munsafe-fp-atomics",          # LDS float adds as ds_add_f32 instead of compare-and-swap loops
+         "-mllvm", "-amdgpu-mfma-vgpr-form",   # MFMA accumulators in VGPRs: no copies to and from AGPRs
          "-Wno-unused-command-line-argument"]
 
 

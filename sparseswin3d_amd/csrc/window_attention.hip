@@ -27,6 +27,7 @@
 // first and the short ones fill the tail; the loop over tiles is a run-time loop with a register
 // budget that does not depend on the tile count.
 #include <math.h>
+#include <stdint.h>
 
 #include "mfma_block.hpp"
 #include "sswin_common.hpp"
@@ -81,25 +82,141 @@ __device__ __forceinline__ GroupCtx load_group(const int4* __restrict__ tasks, i
     return g;
 }
 
-// the head's 16-channel half of one token row as an MFMA operand run
+// ------------------------------------------------------------------------------------------
+// Addressing.  Every token tensor is reached as  uniform byte base (tensor base + head columns)
+// + 32-bit byte offset of the row: one full-rate 24-bit multiply per token and no 64-bit vector
+// arithmetic.  The host checks that row offsets fit 32 bits and that rows are 16-byte aligned.
+// ------------------------------------------------------------------------------------------
+typedef float f32x4_a __attribute__((ext_vector_type(4)));               // naturally aligned
+typedef uint32_t u32x4_a __attribute__((ext_vector_type(4)));
+
+constexpr float LOG2E = 1.4426950408889634f;
+constexpr float LN2 = 0.6931471805599453f;
+
 template <typename T>
-__device__ __forceinline__ void load_slice(const TokenTensor32& t, int vox, int h, int half, float (&x)[16]) {
-    const T* p = static_cast<const T*>(t.base) + (int64_t)vox * t.stride + t.col0 + h * 32 + half * 16;
-    load_run16_full<T>(p, x);
+__device__ __forceinline__ const char* head_base(const TokenTensor32& t, int h) {
+    return static_cast<const char*>(t.base) + (int64_t)(t.col0 + h * 32) * sizeof(T);
+}
+template <typename T>
+__device__ __forceinline__ uint32_t pitch_of(const TokenTensor32& t) { return (uint32_t)t.stride * (uint32_t)sizeof(T); }
+
+// 16 consecutive channels of one token row -> fp32
+template <typename T>
+__device__ __forceinline__ void load_slice(const char* __restrict__ base, uint32_t off, float (&x)[16]);
+template <>
+__device__ __forceinline__ void load_slice<float>(const char* __restrict__ base, uint32_t off, float (&x)[16]) {
+    const f32x4_a* p = reinterpret_cast<const f32x4_a*>(base + off);
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        const f32x4_a t = p[v];
+        x[4 * v] = t.x; x[4 * v + 1] = t.y; x[4 * v + 2] = t.z; x[4 * v + 3] = t.w;
+    }
+}
+__device__ __forceinline__ void unpack2(uint32_t u, float& lo, float& hi, __half) {
+    const __half2 h2 = __builtin_bit_cast(__half2, u);
+    lo = __low2float(h2);
+    hi = __high2float(h2);
+}
+__device__ __forceinline__ void unpack2(uint32_t u, float& lo, float& hi, __hip_bfloat16) {
+    lo = __builtin_bit_cast(float, u << 16);
+    hi = __builtin_bit_cast(float, u & 0xffff0000u);
+}
+template <typename T>
+__device__ __forceinline__ void load_slice(const char* __restrict__ base, uint32_t off, float (&x)[16]) {
+    const u32x4_a* p = reinterpret_cast<const u32x4_a*>(base + off);
+#pragma unroll
+    for (int v = 0; v < 2; ++v) {
+        const u32x4_a t = p[v];
+        unpack2(t.x, x[8 * v], x[8 * v + 1], T());
+        unpack2(t.y, x[8 * v + 2], x[8 * v + 3], T());
+        unpack2(t.z, x[8 * v + 4], x[8 * v + 5], T());
+        unpack2(t.w, x[8 * v + 6], x[8 * v + 7], T());
+    }
 }
 
 template <typename T>
-__device__ __forceinline__ const T* column_ptr(const TokenTensor32& t, int h, int l32) {
-    return static_cast<const T*>(t.base) + t.col0 + h * 32 + l32;
+__device__ __forceinline__ void store_slice(char* __restrict__ base, uint32_t off, const float (&x)[16]);
+template <>
+__device__ __forceinline__ void store_slice<float>(char* __restrict__ base, uint32_t off, const float (&x)[16]) {
+    f32x4_a* p = reinterpret_cast<f32x4_a*>(base + off);
+#pragma unroll
+    for (int v = 0; v < 4; ++v) p[v] = f32x4_a{x[4 * v], x[4 * v + 1], x[4 * v + 2], x[4 * v + 3]};
 }
+__device__ __forceinline__ uint32_t pack2(float lo, float hi, __half) {
+    return __builtin_bit_cast(uint32_t, __floats2half2_rn(lo, hi));
+}
+__device__ __forceinline__ uint32_t pack2(float lo, float hi, __hip_bfloat16) {
+    const uint32_t a = __builtin_bit_cast(uint16_t, __float2bfloat16(lo));
+    const uint32_t b = __builtin_bit_cast(uint16_t, __float2bfloat16(hi));
+    return a | (b << 16);
+}
+template <typename T>
+__device__ __forceinline__ void store_slice(char* __restrict__ base, uint32_t off, const float (&x)[16]) {
+    u32x4_a* p = reinterpret_cast<u32x4_a*>(base + off);
+#pragma unroll
+    for (int v = 0; v < 2; ++v)
+        p[v] = u32x4_a{pack2(x[8 * v], x[8 * v + 1], T()), pack2(x[8 * v + 2], x[8 * v + 3], T()),
+                       pack2(x[8 * v + 4], x[8 * v + 5], T()), pack2(x[8 * v + 6], x[8 * v + 7], T())};
+}
+
+// ------------------------------------------------------------------------------------------
+// Wave-private LDS.  A "tile" holds 32 token rows of 32 fp32 channels at a pitch of 36 dwords
+// (16-byte rows stay aligned, and 16-byte accesses of neighbouring rows fall into different
+// banks); it turns the row-major global loads into the column-major MFMA operand of the second
+// product and the accumulators back into rows for wide stores.  A "table" holds one 32-bit value
+// per token of the tile; the 16 entries a lane needs (rows acc_row(r, half)) are four runs of
+// four, fetched with four 16-byte reads.  Only the owning wavefront touches its tiles and tables;
+// LDS operations of one wavefront execute in order, so no barrier is involved.
+// ------------------------------------------------------------------------------------------
+constexpr int TILE_LD = 36;
+constexpr int TILE_WORDS = 32 * TILE_LD;
+
+__device__ __forceinline__ void tile_put_rows(float* tile, int l32, int half, const float (&x)[16]) {
+    f32x4_a* p = reinterpret_cast<f32x4_a*>(tile + l32 * TILE_LD + half * 16);
+#pragma unroll
+    for (int v = 0; v < 4; ++v) p[v] = f32x4_a{x[4 * v], x[4 * v + 1], x[4 * v + 2], x[4 * v + 3]};
+}
+__device__ __forceinline__ void tile_get_rows(const float* tile, int l32, int half, float (&x)[16]) {
+    const f32x4_a* p = reinterpret_cast<const f32x4_a*>(tile + l32 * TILE_LD + half * 16);
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        const f32x4_a t = p[v];
+        x[4 * v] = t.x; x[4 * v + 1] = t.y; x[4 * v + 2] = t.z; x[4 * v + 3] = t.w;
+    }
+}
+// x[r] = tile[row acc_row(r, half)][column l32]
+__device__ __forceinline__ void tile_get_cols(const float* tile, int l32, int half, float (&x)[16]) {
+    const float* p = tile + 4 * half * TILE_LD + l32;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) x[r] = p[(8 * (r >> 2) + (r & 3)) * TILE_LD];
+}
+__device__ __forceinline__ void tile_put_acc(float* tile, int l32, int half, const f32x16& acc) {
+    float* p = tile + 4 * half * TILE_LD + l32;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) p[(8 * (r >> 2) + (r & 3)) * TILE_LD] = acc[r];
+}
+__device__ __forceinline__ void table_put(uint32_t* tab, int l32, uint32_t v) { tab[l32] = v; }
+__device__ __forceinline__ void table_get(const uint32_t* tab, int half, uint32_t (&x)[16]) {
+    const u32x4_a* p = reinterpret_cast<const u32x4_a*>(tab + 4 * half);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const u32x4_a t = p[2 * q];
+        x[4 * q] = t.x; x[4 * q + 1] = t.y; x[4 * q + 2] = t.z; x[4 * q + 3] = t.w;
+    }
+}
+__device__ __forceinline__ uint32_t f2u(float v) { return __builtin_bit_cast(uint32_t, v); }
+__device__ __forceinline__ float u2f(uint32_t v) { return __builtin_bit_cast(float, v); }
+__device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // ------------------------------------------------------------------------------------------
 // forward
 // ------------------------------------------------------------------------------------------
-template <typename T>
+template <typename T, bool MASK>
 __global__ __launch_bounds__(256) void wattn_fwd_kernel(WAttnCommon a, TokenTensor32 tq, TokenTensor32 tk,
                                                         TokenTensor32 tv, TokenTensor32 to,
                                                         float* __restrict__ lse) {
+    __shared__ __attribute__((aligned(16))) float tiles[4][TILE_WORDS];
+    __shared__ __attribute__((aligned(16))) uint32_t tabs[4][2][32];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int half = lane >> 5, l32 = lane & 31;
     int64_t d;
@@ -108,94 +225,116 @@ __global__ __launch_bounds__(256) void wattn_fwd_kernel(WAttnCommon a, TokenTens
     const GroupCtx g = load_group(a.tasks, d);
     const int c = g.c, h = g.h;
     const int nt = (c + 31) >> 5;
+    float* tile = tiles[wave];
+    uint32_t* tab_key = tabs[wave][0];
+    uint32_t* tab_alpha = tabs[wave][1];
+    const int32_t* order = a.order + g.Tk;
+    const int32_t* tok_pos = a.tok_pos + g.Tk;
+    const int8_t* mrow = MASK ? a.mask + (int64_t)(g.w % a.nmw) * a.n : nullptr;
+    const uint32_t slice = half * 16 * sizeof(T);
+    const char* qbase = head_base<T>(tq, h);
+    const char* kbase = head_base<T>(tk, h);
+    const char* vbase = head_base<T>(tv, h);
+    const uint32_t qpitch = pitch_of<T>(tq), kpitch = pitch_of<T>(tk), vpitch = pitch_of<T>(tv);
 
     // query side: lane l32 owns query bi*32 + l32 (both halves), clamped to the last token
     const int i_q = bi * 32 + l32;
     const int i_c = i_q < c ? i_q : c - 1;
-    const int vox_i = a.order[g.Tk + i_c];
-    const int pos_i = a.tok_pos[g.Tk + i_c];
-    const int8_t* mrow = a.mask ? a.mask + (int64_t)(g.w % a.nmw) * a.n : nullptr;
-    const int reg_i = mrow ? mrow[pos_i] : 0;
+    const uint32_t vox_i = order[i_c];
+    const int pos_i = tok_pos[i_c];
+    const int reg_i = MASK ? mrow[pos_i] : 0;
     float qb[16];
-    load_slice<T>(tq, vox_i, h, half, qb);
+    load_slice<T>(qbase, __umul24(vox_i, qpitch) + slice, qb);
+    const float qscale = a.scale * LOG2E;                    // scores are kept in units of log 2
 #pragma unroll
-    for (int s = 0; s < 16; ++s) qb[s] *= a.scale;
+    for (int s = 0; s < 16; ++s) qb[s] *= qscale;
+    const char* bias_h = reinterpret_cast<const char*>(a.bias + (int64_t)h * a.n * a.n);
+    const uint32_t brow = (uint32_t)(pos_i * a.n) * 4u;
 
-    const float* brow = a.bias + ((int64_t)h * a.n + pos_i) * a.n;
-    const T* vcol = column_ptr<T>(tv, h, l32);
     float m = 0.f;                                           // the operator's max(0, rowmax)
     float l = 0.f;                                           // this lane half's share of the row sum
     f32x16 o = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll 1
     for (int t = 0; t < nt; ++t) {
-        // S^T tile: rows = keys of tile t, columns = queries
+        // key side of tile t: lane l32 owns key t*32 + l32
         const int j = t * 32 + l32;
         const int j_c = j < c ? j : c - 1;
-        const int vox_j = a.order[g.Tk + j_c];
-        const int p = a.tok_pos[g.Tk + j_c];
-        const int pj = p | ((mrow ? (int)mrow[p] : 0) << 8);
+        const uint32_t vox_j = order[j_c];
+        const int pos_j = tok_pos[j_c];
+        float ka[16], va[16];
+        load_slice<T>(kbase, __umul24(vox_j, kpitch) + slice, ka);
+        load_slice<T>(vbase, __umul24(vox_j, vpitch) + slice, va);
+        uint32_t pk = (uint32_t)pos_j * 4u;
+        if (MASK) pk |= (uint32_t)mrow[pos_j] << 16;
+        table_put(tab_key, l32, pk);
+        // S^T tile: rows = keys, columns = queries
         f32x16 S = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-        {
-            float ka[16];
-            load_slice<T>(tk, vox_j, h, half, ka);
 #pragma unroll
-            for (int s = 0; s < 16; ++s) S = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[s], qb[s], S, 0, 0, 0);
-        }
-        // V in B layout: lane (ch, half) reads V[key acc_row(r, half)][ch]; bias row entries
-        float vb[16], bv[16];
-        int pk[16];
+        for (int s = 0; s < 16; ++s) S = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[s], qb[s], S, 0, 0, 0);
+        tile_put_rows(tile, l32, half, va);
+        __builtin_amdgcn_wave_barrier();
+        uint32_t pkr[16];
+        table_get(tab_key, half, pkr);
+        float bv[16];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int jl = acc_row(r, half);
-            vb[r] = to_acc(vcol[(int64_t)__shfl(vox_j, jl, 64) * tv.stride]);
-            pk[r] = __shfl(pj, jl, 64);
-            bv[r] = brow[pk[r] & 0xff];
-        }
+        for (int r = 0; r < 16; ++r)
+            bv[r] = *reinterpret_cast<const float*>(bias_h + (brow + (MASK ? (pkr[r] & 0xffffu) : pkr[r])));
+        float vb[16];
+        tile_get_cols(tile, l32, half, vb);                  // V[key acc_row(r, half)][channel l32]
+
+        const int jlim = c - t * 32 - 4 * half;              // keys acc_row(r, 0) >= jlim are padding
         float mt = m;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            float s = S[r] + bv[r];
-            if (mrow && (pk[r] >> 8) != reg_i) s += -100.0f;
-            s = t * 32 + acc_row(r, half) < c ? s : -INFINITY;
+            float s = fmaf(bv[r], LOG2E, S[r]);
+            if (MASK && (int)(pkr[r] >> 16) != reg_i) s += -100.0f * LOG2E;
+            s = (8 * (r >> 2) + (r & 3)) < jlim ? s : -INFINITY;
             S[r] = s;
             mt = fmaxf(mt, s);
         }
         mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
         if (t > 0) {                                         // rescale what earlier tiles accumulated
-            const float alpha = expf(m - mt);
+            const float alpha = exp2_fast(m - mt);
             l *= alpha;
+            table_put(tab_alpha, l32, f2u(alpha));
+            __builtin_amdgcn_wave_barrier();
+            uint32_t ar[16];
+            table_get(tab_alpha, half, ar);
 #pragma unroll
-            for (int r = 0; r < 16; ++r) o[r] *= __shfl(alpha, acc_row(r, half), 64);
+            for (int r = 0; r < 16; ++r) o[r] *= u2f(ar[r]);
         }
         m = mt;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const float e = expf(S[r] - m);
+            const float e = exp2_fast(S[r] - m);
             l += e;
             o = __builtin_amdgcn_mfma_f32_32x32x2f32(e, vb[r], o, 0, 0, 0);
         }
     }
     l += __shfl_xor(l, 32, 64);
     l += 1e-8f;
-    if (half == 0 && i_q < c) lse[(int64_t)a.H * g.Tk + h * c + i_q] = m + logf(l);
+    if (half == 0 && i_q < c) lse[(int64_t)a.H * g.Tk + h * c + i_q] = (m + __builtin_amdgcn_logf(l)) * LN2;
+    // accumulators (rows = queries by register) -> rows by lane, normalise, wide stores
+    tile_put_acc(tile, l32, half, o);
+    __builtin_amdgcn_wave_barrier();
+    float orow[16];
+    tile_get_rows(tile, l32, half, orow);
     const float inv_l = 1.0f / l;
-    T* ocol = const_cast<T*>(column_ptr<T>(to, h, l32));
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        const int il = acc_row(r, half);
-        const int vox = __shfl(vox_i, il, 64);
-        const float w = __shfl(inv_l, il, 64);
-        if (bi * 32 + il < c) ocol[(int64_t)vox * to.stride] = from_acc<T>(o[r] * w);
-    }
+    for (int s = 0; s < 16; ++s) orow[s] *= inv_l;
+    if (i_q < c)
+        store_slice<T>(const_cast<char*>(head_base<T>(to, h)), __umul24(vox_i, pitch_of<T>(to)) + slice, orow);
 }
 
 // ------------------------------------------------------------------------------------------
 // backward, query side: dQ
 // ------------------------------------------------------------------------------------------
-template <typename T>
+template <typename T, bool MASK>
 __global__ __launch_bounds__(256) void wattn_bwd_q_kernel(WAttnCommon a, TokenTensor32 tq, TokenTensor32 tk,
                                                           TokenTensor32 tv, TokenTensor32 to, TokenTensor32 tdo,
                                                           const float* __restrict__ lse, TokenTensor32 tdq) {
+    __shared__ __attribute__((aligned(16))) float tiles[4][TILE_WORDS];
+    __shared__ __attribute__((aligned(16))) uint32_t tabs[4][32];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int half = lane >> 5, l32 = lane & 31;
     int64_t d;
@@ -204,85 +343,98 @@ __global__ __launch_bounds__(256) void wattn_bwd_q_kernel(WAttnCommon a, TokenTe
     const GroupCtx g = load_group(a.tasks, d);
     const int c = g.c, h = g.h;
     const int nt = (c + 31) >> 5;
+    float* tile = tiles[wave];
+    uint32_t* tab_key = tabs[wave];
+    const int32_t* order = a.order + g.Tk;
+    const int32_t* tok_pos = a.tok_pos + g.Tk;
+    const int8_t* mrow = MASK ? a.mask + (int64_t)(g.w % a.nmw) * a.n : nullptr;
+    const uint32_t slice = half * 16 * sizeof(T);
+    const char* kbase = head_base<T>(tk, h);
+    const char* vbase = head_base<T>(tv, h);
+    const uint32_t kpitch = pitch_of<T>(tk), vpitch = pitch_of<T>(tv);
 
     const int i_q = bi * 32 + l32;
     const int i_c = i_q < c ? i_q : c - 1;
-    const int vox_i = a.order[g.Tk + i_c];
-    const int pos_i = a.tok_pos[g.Tk + i_c];
-    const int8_t* mrow = a.mask ? a.mask + (int64_t)(g.w % a.nmw) * a.n : nullptr;
-    const int reg_i = mrow ? mrow[pos_i] : 0;
-    const float L = lse[(int64_t)a.H * g.Tk + h * c + i_c];
+    const uint32_t vox_i = order[i_c];
+    const int pos_i = tok_pos[i_c];
+    const int reg_i = MASK ? mrow[pos_i] : 0;
+    const float L2 = lse[(int64_t)a.H * g.Tk + h * c + i_c] * LOG2E;
     float qb[16], dob[16];
-    load_slice<T>(tq, vox_i, h, half, qb);
-    load_slice<T>(tdo, vox_i, h, half, dob);
+    load_slice<T>(head_base<T>(tq, h), __umul24(vox_i, pitch_of<T>(tq)) + slice, qb);
+    load_slice<T>(head_base<T>(tdo, h), __umul24(vox_i, pitch_of<T>(tdo)) + slice, dob);
     float D = 0.f;
     {
         float ob[16];
-        load_slice<T>(to, vox_i, h, half, ob);
+        load_slice<T>(head_base<T>(to, h), __umul24(vox_i, pitch_of<T>(to)) + slice, ob);
 #pragma unroll
-        for (int s = 0; s < 16; ++s) D += dob[s] * ob[s];
+        for (int s = 0; s < 16; ++s) D = fmaf(dob[s], ob[s], D);
     }
     D += __shfl_xor(D, 32, 64);
+    const float qscale = a.scale * LOG2E;
 #pragma unroll
-    for (int s = 0; s < 16; ++s) qb[s] *= a.scale;
+    for (int s = 0; s < 16; ++s) qb[s] *= qscale;
+    const char* bias_h = reinterpret_cast<const char*>(a.bias + (int64_t)h * a.n * a.n);
+    const uint32_t brow = (uint32_t)(pos_i * a.n) * 4u;
 
-    const float* brow = a.bias + ((int64_t)h * a.n + pos_i) * a.n;
-    const T* kcol = column_ptr<T>(tk, h, l32);
     f32x16 dq = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll 1
     for (int t = 0; t < nt; ++t) {
         const int j = t * 32 + l32;
         const int j_c = j < c ? j : c - 1;
-        const int vox_j = a.order[g.Tk + j_c];
-        const int p = a.tok_pos[g.Tk + j_c];
-        const int pj = p | ((mrow ? (int)mrow[p] : 0) << 8);
+        const uint32_t vox_j = order[j_c];
+        const int pos_j = tok_pos[j_c];
+        float ka[16], va[16];
+        load_slice<T>(kbase, __umul24(vox_j, kpitch) + slice, ka);
+        load_slice<T>(vbase, __umul24(vox_j, vpitch) + slice, va);
+        uint32_t pk = (uint32_t)pos_j * 4u;
+        if (MASK) pk |= (uint32_t)mrow[pos_j] << 16;
+        table_put(tab_key, l32, pk);
         f32x16 St = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
         f32x16 dPt = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-        {
-            float ka[16], va[16];
-            load_slice<T>(tk, vox_j, h, half, ka);
-            load_slice<T>(tv, vox_j, h, half, va);
 #pragma unroll
-            for (int s = 0; s < 16; ++s) St = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[s], qb[s], St, 0, 0, 0);
+        for (int s = 0; s < 16; ++s) St = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[s], qb[s], St, 0, 0, 0);
+        tile_put_rows(tile, l32, half, ka);                  // K rows, read back by column for dQ
 #pragma unroll
-            for (int s = 0; s < 16; ++s) dPt = __builtin_amdgcn_mfma_f32_32x32x2f32(va[s], dob[s], dPt, 0, 0, 0);
-        }
-        int pk[16];
-        float bv[16], kb[16];
+        for (int s = 0; s < 16; ++s) dPt = __builtin_amdgcn_mfma_f32_32x32x2f32(va[s], dob[s], dPt, 0, 0, 0);
+        __builtin_amdgcn_wave_barrier();
+        uint32_t pkr[16];
+        table_get(tab_key, half, pkr);
+        float bv[16];
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const int jl = acc_row(r, half);
-            pk[r] = __shfl(pj, jl, 64);
-            bv[r] = brow[pk[r] & 0xff];
-            kb[r] = to_acc(kcol[(int64_t)__shfl(vox_j, jl, 64) * tk.stride]);
-        }
+        for (int r = 0; r < 16; ++r)
+            bv[r] = *reinterpret_cast<const float*>(bias_h + (brow + (MASK ? (pkr[r] & 0xffffu) : pkr[r])));
+        float kb[16];
+        tile_get_cols(tile, l32, half, kb);                  // K[key acc_row(r, half)][channel l32]
+        const int jlim = c - t * 32 - 4 * half;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const int jg = t * 32 + acc_row(r, half);
-            float s = St[r] + bv[r];
-            if (mrow && (pk[r] >> 8) != reg_i) s += -100.0f;
-            const float pr = jg < c ? expf(s - L) : 0.f;
+            float s = fmaf(bv[r], LOG2E, St[r]);
+            if (MASK && (int)(pkr[r] >> 16) != reg_i) s += -100.0f * LOG2E;
+            const float pr = (8 * (r >> 2) + (r & 3)) < jlim ? exp2_fast(s - L2) : 0.f;
             const float ds = pr * (dPt[r] - D);
             dq = __builtin_amdgcn_mfma_f32_32x32x2f32(ds, kb[r], dq, 0, 0, 0);
         }
     }
-    T* ocol = const_cast<T*>(column_ptr<T>(tdq, h, l32));
+    tile_put_acc(tile, l32, half, dq);
+    __builtin_amdgcn_wave_barrier();
+    float row[16];
+    tile_get_rows(tile, l32, half, row);
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        const int il = acc_row(r, half);
-        const int vox = __shfl(vox_i, il, 64);
-        if (bi * 32 + il < c) ocol[(int64_t)vox * tdq.stride] = from_acc<T>(dq[r] * a.scale);
-    }
+    for (int s = 0; s < 16; ++s) row[s] *= a.scale;
+    if (i_q < c)
+        store_slice<T>(const_cast<char*>(head_base<T>(tdq, h)), __umul24(vox_i, pitch_of<T>(tdq)) + slice, row);
 }
 
 // ------------------------------------------------------------------------------------------
 // backward, key side: dK, dV (and dS for the bias gradient)
 // ------------------------------------------------------------------------------------------
-template <typename T>
+template <typename T, bool MASK>
 __global__ __launch_bounds__(256) void wattn_bwd_kv_kernel(WAttnCommon a, TokenTensor32 tq, TokenTensor32 tk,
                                                            TokenTensor32 tv, TokenTensor32 to, TokenTensor32 tdo,
                                                            const float* __restrict__ lse, TokenTensor32 tdk,
                                                            TokenTensor32 tdv, float* __restrict__ ds_out) {
+    __shared__ __attribute__((aligned(16))) float tiles[4][2][TILE_WORDS];
+    __shared__ __attribute__((aligned(16))) uint32_t tabs[4][3][32];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int half = lane >> 5, l32 = lane & 31;
     int64_t d;
@@ -291,21 +443,37 @@ __global__ __launch_bounds__(256) void wattn_bwd_kv_kernel(WAttnCommon a, TokenT
     const GroupCtx g = load_group(a.tasks, d);
     const int c = g.c, h = g.h;
     const int nt = (c + 31) >> 5;
+    float* tile_q = tiles[wave][0];
+    float* tile_do = tiles[wave][1];
+    uint32_t* tab_pos = tabs[wave][0];
+    uint32_t* tab_L = tabs[wave][1];
+    uint32_t* tab_D = tabs[wave][2];
+    const int32_t* order = a.order + g.Tk;
+    const int32_t* tok_pos = a.tok_pos + g.Tk;
+    const int8_t* mrow = MASK ? a.mask + (int64_t)(g.w % a.nmw) * a.n : nullptr;
+    const uint32_t slice = half * 16 * sizeof(T);
+    const char* qbase = head_base<T>(tq, h);
+    const char* obase = head_base<T>(to, h);
+    const char* dobase = head_base<T>(tdo, h);
+    const uint32_t qpitch = pitch_of<T>(tq), opitch = pitch_of<T>(to), dopitch = pitch_of<T>(tdo);
+    const float* lse_g = lse + (int64_t)a.H * g.Tk + h * c;
 
     // key side: lane l32 owns key bj*32 + l32
     const int j_k = bj * 32 + l32;
     const int j_c = j_k < c ? j_k : c - 1;
-    const int vox_j = a.order[g.Tk + j_c];
-    const int pos_j = a.tok_pos[g.Tk + j_c];
-    const int8_t* mrow = a.mask ? a.mask + (int64_t)(g.w % a.nmw) * a.n : nullptr;
-    const int reg_j = mrow ? mrow[pos_j] : 0;
+    const uint32_t vox_j = order[j_c];
+    const int pos_j = tok_pos[j_c];
+    const int reg_j = MASK ? mrow[pos_j] : 0;
     float kb[16], vb[16];
-    load_slice<T>(tk, vox_j, h, half, kb);
-    load_slice<T>(tv, vox_j, h, half, vb);
+    load_slice<T>(head_base<T>(tk, h), __umul24(vox_j, pitch_of<T>(tk)) + slice, kb);
+    load_slice<T>(head_base<T>(tv, h), __umul24(vox_j, pitch_of<T>(tv)) + slice, vb);
+    const float kscale = a.scale * LOG2E;                    // scores in units of log 2
+#pragma unroll
+    for (int s = 0; s < 16; ++s) kb[s] *= kscale;
+    const char* bias_h = reinterpret_cast<const char*>(a.bias + (int64_t)h * a.n * a.n);
+    const uint32_t bcol = (uint32_t)pos_j * 4u;
+    float* ds_g = ds_out ? ds_out + g.sq + j_k : nullptr;
 
-    const float* bcol = a.bias + (int64_t)h * a.n * a.n + pos_j;
-    const T* docol = column_ptr<T>(tdo, h, l32);
-    const T* qcol = column_ptr<T>(tq, h, l32);
     f32x16 dk = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     f32x16 dv = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll 1
@@ -313,72 +481,74 @@ __global__ __launch_bounds__(256) void wattn_bwd_kv_kernel(WAttnCommon a, TokenT
         // query side of tile t: lane l32 owns query t*32 + l32
         const int i = t * 32 + l32;
         const int i_c = i < c ? i : c - 1;
-        const int vox_i = a.order[g.Tk + i_c];
-        const int p = a.tok_pos[g.Tk + i_c];
-        const int pi = p | ((mrow ? (int)mrow[p] : 0) << 8);
-        const float L_i = lse[(int64_t)a.H * g.Tk + h * c + i_c];
-        f32x16 St = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-        f32x16 dPt = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        const uint32_t vox_i = order[i_c];
+        const int pos_i = tok_pos[i_c];
+        // padding queries get L = +inf, which makes their P and dS exactly zero
+        const float L2_i = i < c ? lse_g[i_c] * LOG2E : INFINITY;
+        float qa[16], doa[16];
+        load_slice<T>(qbase, __umul24(vox_i, qpitch) + slice, qa);
+        load_slice<T>(dobase, __umul24(vox_i, dopitch) + slice, doa);
         float D_i = 0.f;
         {
-            float qa[16], doa[16], oa[16];
-            load_slice<T>(tq, vox_i, h, half, qa);
-            load_slice<T>(tdo, vox_i, h, half, doa);
-            load_slice<T>(to, vox_i, h, half, oa);
+            float oa[16];
+            load_slice<T>(obase, __umul24(vox_i, opitch) + slice, oa);
 #pragma unroll
-            for (int s = 0; s < 16; ++s) D_i += doa[s] * oa[s];
-#pragma unroll
-            for (int s = 0; s < 16; ++s)
-                St = __builtin_amdgcn_mfma_f32_32x32x2f32(qa[s] * a.scale, kb[s], St, 0, 0, 0);
-#pragma unroll
-            for (int s = 0; s < 16; ++s) dPt = __builtin_amdgcn_mfma_f32_32x32x2f32(doa[s], vb[s], dPt, 0, 0, 0);
+            for (int s = 0; s < 16; ++s) D_i = fmaf(doa[s], oa[s], D_i);
         }
         D_i += __shfl_xor(D_i, 32, 64);
+        uint32_t pi = (uint32_t)(pos_i * a.n) * 4u;          // byte offset of bias row pos_i (< 2^16)
+        if (MASK) pi |= (uint32_t)mrow[pos_i] << 16;
+        table_put(tab_pos, l32, pi);
+        table_put(tab_L, l32, f2u(L2_i));
+        table_put(tab_D, l32, f2u(D_i));
+        f32x16 St = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        f32x16 dPt = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+        for (int s = 0; s < 16; ++s) St = __builtin_amdgcn_mfma_f32_32x32x2f32(qa[s], kb[s], St, 0, 0, 0);
+        tile_put_rows(tile_q, l32, half, qa);
+#pragma unroll
+        for (int s = 0; s < 16; ++s) dPt = __builtin_amdgcn_mfma_f32_32x32x2f32(doa[s], vb[s], dPt, 0, 0, 0);
+        tile_put_rows(tile_do, l32, half, doa);
+        __builtin_amdgcn_wave_barrier();
 
-        // the B-layout rows of dO and Q for the two products below
+        // P and dS of the tile: rows = queries acc_row(r, half), column = this lane's key
+        uint32_t pir[16];
+        table_get(tab_pos, half, pir);
+        float bv[16];
+#pragma unroll
+        for (int r = 0; r < 16; ++r)
+            bv[r] = *reinterpret_cast<const float*>(bias_h + (bcol + (MASK ? (pir[r] & 0xffffu) : pir[r])));
+        uint32_t Lr[16], Dr[16];
+        table_get(tab_L, half, Lr);
+        table_get(tab_D, half, Dr);
         float dob[16], qbr[16];
+        tile_get_cols(tile_do, l32, half, dob);              // dO[query acc_row(r, half)][channel l32]
+        tile_get_cols(tile_q, l32, half, qbr);               // Q[query acc_row(r, half)][channel l32]
+        float* ds_t = ds_g ? ds_g + (int64_t)(t * 32 + 4 * half) * c : nullptr;
+        const int ilim = c - t * 32 - 4 * half;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            const int64_t vox = __shfl(vox_i, acc_row(r, half), 64);
-            dob[r] = to_acc(docol[vox * tdo.stride]);
-            qbr[r] = to_acc(qcol[vox * tq.stride]);
-        }
-        // P and dS of the tile: rows = queries acc_row(r, half), column = this lane's key
-        {
-            int pk[16];
-            float bv[16];
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                pk[r] = __shfl(pi, acc_row(r, half), 64);
-                bv[r] = bcol[(int64_t)(pk[r] & 0xff) * a.n];
-            }
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int il = acc_row(r, half);
-                const int ig = t * 32 + il;
-                const bool valid = ig < c && j_k < c;
-                // cross-lane reads stay outside the predicated code: every lane must take part
-                const float Lr = __shfl(L_i, il, 64), Dr = __shfl(D_i, il, 64);
-                float s = St[r] + bv[r];
-                if (mrow && (pk[r] >> 8) != reg_j) s += -100.0f;
-                const float pr = valid ? expf(s - Lr) : 0.f;
-                const float ds = pr * (dPt[r] - Dr);
-                if (ds_out && valid) ds_out[(int64_t)g.sq + (int64_t)ig * c + j_k] = ds;
-                dv = __builtin_amdgcn_mfma_f32_32x32x2f32(pr, dob[r], dv, 0, 0, 0);     // dV += P^T dO
-                dk = __builtin_amdgcn_mfma_f32_32x32x2f32(ds, qbr[r], dk, 0, 0, 0);     // dK += dS^T Q
-            }
+            float s = fmaf(bv[r], LOG2E, St[r]);
+            if (MASK && (int)(pir[r] >> 16) != reg_j) s += -100.0f * LOG2E;
+            const float pr = exp2_fast(s - u2f(Lr[r]));
+            const float ds = pr * (dPt[r] - u2f(Dr[r]));
+            const int row = 8 * (r >> 2) + (r & 3);
+            if (ds_t && row < ilim && j_k < c) ds_t[row * c] = ds;
+            dv = __builtin_amdgcn_mfma_f32_32x32x2f32(pr, dob[r], dv, 0, 0, 0);     // dV += P^T dO
+            dk = __builtin_amdgcn_mfma_f32_32x32x2f32(ds, qbr[r], dk, 0, 0, 0);     // dK += dS^T Q
         }
     }
-    T* dkcol = const_cast<T*>(column_ptr<T>(tdk, h, l32));
-    T* dvcol = const_cast<T*>(column_ptr<T>(tdv, h, l32));
+    tile_put_acc(tile_q, l32, half, dk);
+    tile_put_acc(tile_do, l32, half, dv);
+    __builtin_amdgcn_wave_barrier();
+    float krow[16], vrow[16];
+    tile_get_rows(tile_q, l32, half, krow);
+    tile_get_rows(tile_do, l32, half, vrow);
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        const int jl = acc_row(r, half);
-        const int vox = __shfl(vox_j, jl, 64);
-        if (bj * 32 + jl < c) {
-            dkcol[(int64_t)vox * tdk.stride] = from_acc<T>(dk[r] * a.scale);
-            dvcol[(int64_t)vox * tdv.stride] = from_acc<T>(dv[r]);
-        }
+    for (int s = 0; s < 16; ++s) krow[s] *= a.scale;
+    if (j_k < c) {
+        store_slice<T>(const_cast<char*>(head_base<T>(tdk, h)), __umul24(vox_j, pitch_of<T>(tdk)) + slice, krow);
+        store_slice<T>(const_cast<char*>(head_base<T>(tdv, h)), __umul24(vox_j, pitch_of<T>(tdv)) + slice, vrow);
     }
 }
 
@@ -391,21 +561,48 @@ template <typename T>
 static int run_forward(const WAttnCommon& a, const TokenTensor32& q, const TokenTensor32& k, const TokenTensor32& v,
                        const TokenTensor32& o, float* lse, hipStream_t s) {
     const unsigned blocks = (unsigned)((a.first[4] + 3) / 4);
-    hipLaunchKernelGGL((wattn_fwd_kernel<T>), dim3(blocks), dim3(256), 0, s, a, q, k, v, o, lse);
+    if (a.mask)
+        hipLaunchKernelGGL((wattn_fwd_kernel<T, true>), dim3(blocks), dim3(256), 0, s, a, q, k, v, o, lse);
+    else
+        hipLaunchKernelGGL((wattn_fwd_kernel<T, false>), dim3(blocks), dim3(256), 0, s, a, q, k, v, o, lse);
     return launch_ok("window attention forward");
+}
+
+template <typename T, bool MASK>
+static void launch_backward(const WAttnCommon& a, const TokenTensor32& q, const TokenTensor32& k,
+                            const TokenTensor32& v, const TokenTensor32& o, const TokenTensor32& d_o, const float* lse,
+                            const TokenTensor32& dq, const TokenTensor32& dk, const TokenTensor32& dv, float* ds_out,
+                            int sides, hipStream_t s) {
+    const unsigned blocks = (unsigned)((a.first[4] + 3) / 4);
+    if (sides & 1)
+        hipLaunchKernelGGL((wattn_bwd_q_kernel<T, MASK>), dim3(blocks), dim3(256), 0, s, a, q, k, v, o, d_o, lse, dq);
+    if (sides & 2)
+        hipLaunchKernelGGL((wattn_bwd_kv_kernel<T, MASK>), dim3(blocks), dim3(256), 0, s, a, q, k, v, o, d_o, lse, dk,
+                           dv, ds_out);
 }
 
 template <typename T>
 static int run_backward(const WAttnCommon& a, const TokenTensor32& q, const TokenTensor32& k, const TokenTensor32& v,
                         const TokenTensor32& o, const TokenTensor32& d_o, const float* lse, const TokenTensor32& dq,
                         const TokenTensor32& dk, const TokenTensor32& dv, float* ds_out, int sides, hipStream_t s) {
-    const unsigned blocks = (unsigned)((a.first[4] + 3) / 4);
-    if (sides & 1)
-        hipLaunchKernelGGL((wattn_bwd_q_kernel<T>), dim3(blocks), dim3(256), 0, s, a, q, k, v, o, d_o, lse, dq);
-    if (sides & 2)
-        hipLaunchKernelGGL((wattn_bwd_kv_kernel<T>), dim3(blocks), dim3(256), 0, s, a, q, k, v, o, d_o, lse, dk, dv,
-                           ds_out);
+    if (a.mask)
+        launch_backward<T, true>(a, q, k, v, o, d_o, lse, dq, dk, dv, ds_out, sides, s);
+    else
+        launch_backward<T, false>(a, q, k, v, o, d_o, lse, dq, dk, dv, ds_out, sides, s);
     return launch_ok("window attention backward");
+}
+
+// rows must be reachable with 32-bit byte offsets and 16-byte vector accesses
+static int check_tensor(const char* who, const char* name, const void* base, int64_t stride, int col0, int64_t N,
+                        int H, int dtype) {
+    const int64_t esz = dtype == SSWIN_F32 ? 4 : 2;
+    SSWIN_CHECK(stride >= (int64_t)H * 32 + col0 && col0 >= 0, "%s: %s has %lld columns per row, fewer than col0 + H*32",
+                who, name, (long long)stride);
+    SSWIN_CHECK(N * stride * esz < ((int64_t)1 << 32) && stride * esz < (1 << 24) && N < (1 << 24),
+                "%s: %s is too large for 32-bit row offsets", who, name);
+    SSWIN_CHECK(((uintptr_t)base % 16) == 0 && (stride * esz) % 16 == 0 && (col0 * esz) % 16 == 0,
+                "%s: %s rows are not 16-byte aligned", who, name);
+    return 0;
 }
 
 static WAttnCommon make_common(const int32_t* tasks, int64_t g_cap, const int64_t* counts, const int32_t* tokens,
@@ -426,10 +623,11 @@ static WAttnCommon make_common(const int32_t* tasks, int64_t g_cap, const int64_
     return a;
 }
 
-static int check_common(const char* who, const int32_t* tasks, int64_t g_cap, const int64_t* counts,
+static int check_common(const char* who, int dtype, const int32_t* tasks, int64_t g_cap, const int64_t* counts,
                         const int32_t* tokens, int64_t N, int H, int hd, const float* bias, int n, const int8_t* mask,
                         int nmw, int64_t* total) {
     SSWIN_CHECK(hd == 32, "%s: head dimension %d is not supported (32 only)", who, hd);
+    SSWIN_CHECK(dtype == SSWIN_F32 || dtype == SSWIN_F16 || dtype == SSWIN_BF16, "%s: unsupported token dtype %d", who, dtype);
     SSWIN_CHECK(N >= 0 && H > 0 && H < (1 << 23) && g_cap > 0, "%s: bad sizes", who);
     SSWIN_CHECK(n > 0 && n <= 128, "%s: windows of %d positions are not supported (128 at most)", who, n);
     SSWIN_CHECK(counts, "%s: bucket counts are null", who);
@@ -458,11 +656,16 @@ int sswin_window_attention_forward(int dtype, const int32_t* tasks, int64_t g_ca
                                    int n, const int8_t* mask, int n_mask_windows, void* o_base, int64_t o_stride,
                                    int o_col0, float* lse, void* stream) {
     int64_t total = 0;
-    if (check_common("window_attention_forward", tasks, g_cap, bucket_counts, tokens, N, H, hd, bias, n, mask,
+    if (check_common("window_attention_forward", dtype, tasks, g_cap, bucket_counts, tokens, N, H, hd, bias, n, mask,
                      n_mask_windows, &total))
         return 1;
     if (total == 0) return 0;
     SSWIN_CHECK(q_base && k_base && v_base && o_base && lse, "window_attention_forward: null pointer");
+    if (check_tensor("window_attention_forward", "q", q_base, q_stride, q_col0, N, H, dtype) ||
+        check_tensor("window_attention_forward", "k", k_base, k_stride, k_col0, N, H, dtype) ||
+        check_tensor("window_attention_forward", "v", v_base, v_stride, v_col0, N, H, dtype) ||
+        check_tensor("window_attention_forward", "o", o_base, o_stride, o_col0, N, H, dtype))
+        return 1;
     const WAttnCommon a = make_common(tasks, g_cap, bucket_counts, tokens, N, H, n, scale, bias, mask, n_mask_windows);
     const TokenTensor32 q{q_base, q_stride, q_col0}, k{k_base, k_stride, k_col0}, v{v_base, v_stride, v_col0},
         o{o_base, o_stride, o_col0};
@@ -485,7 +688,7 @@ int sswin_window_attention_backward(int dtype, const int32_t* tasks, int64_t g_c
                                     void* dk_base, int64_t dk_stride, int dk_col0, void* dv_base, int64_t dv_stride,
                                     int dv_col0, float* ds_out, int sides, void* stream) {
     int64_t total = 0;
-    if (check_common("window_attention_backward", tasks, g_cap, bucket_counts, tokens, N, H, hd, bias, n, mask,
+    if (check_common("window_attention_backward", dtype, tasks, g_cap, bucket_counts, tokens, N, H, hd, bias, n, mask,
                      n_mask_windows, &total))
         return 1;
     if (total == 0) return 0;
@@ -493,6 +696,19 @@ int sswin_window_attention_backward(int dtype, const int32_t* tasks, int64_t g_c
     SSWIN_CHECK(q_base && k_base && v_base && o_base && do_base && lse, "window_attention_backward: null pointer");
     SSWIN_CHECK(!(sides & 1) || dq_base, "window_attention_backward: dq is null");
     SSWIN_CHECK(!(sides & 2) || (dk_base && dv_base), "window_attention_backward: dk or dv is null");
+    {
+        const char* who = "window_attention_backward";
+        if (check_tensor(who, "q", q_base, q_stride, q_col0, N, H, dtype) ||
+            check_tensor(who, "k", k_base, k_stride, k_col0, N, H, dtype) ||
+            check_tensor(who, "v", v_base, v_stride, v_col0, N, H, dtype) ||
+            check_tensor(who, "o", o_base, o_stride, o_col0, N, H, dtype) ||
+            check_tensor(who, "do", do_base, do_stride, do_col0, N, H, dtype))
+            return 1;
+        if ((sides & 1) && check_tensor(who, "dq", dq_base, dq_stride, dq_col0, N, H, dtype)) return 1;
+        if ((sides & 2) && (check_tensor(who, "dk", dk_base, dk_stride, dk_col0, N, H, dtype) ||
+                            check_tensor(who, "dv", dv_base, dv_stride, dv_col0, N, H, dtype)))
+            return 1;
+    }
     const WAttnCommon a = make_common(tasks, g_cap, bucket_counts, tokens, N, H, n, scale, bias, mask, n_mask_windows);
     const TokenTensor32 q{q_base, q_stride, q_col0}, k{k_base, k_stride, k_col0}, v{v_base, v_stride, v_col0},
         o{o_base, o_stride, o_col0}, d_o{do_base, do_stride, do_col0}, dq{dq_base, dq_stride, dq_col0},
