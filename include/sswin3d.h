@@ -172,11 +172,16 @@ int sswin_softmax_last_dim_backward(const int32_t* idx_row, const void* y, const
  *   descriptors inside a bucket is unspecified.
  * totals_out (host, 9 x int64): {groups G, non-empty windows, sum over groups of c*c, max c,
  *   groups in bucket 1..4, groups with c > 128 (no descriptor)}; the last five are 0 without tasks.
- * (window, pos) pairs must be distinct, window in [0,B), pos in [0,n).  Synchronises `stream`. */
+ * (window, pos) pairs must be distinct, window in [0,B), pos in [0,n).
+ * synchronize != 0: waits for `stream` and decodes the totals.  synchronize == 0: only enqueues
+ * the work and a copy of the raw totals into totals_out (pinned host memory); once the caller
+ * has waited for the stream, sswin_token_plan_totals(totals_out, H, g_cap) decodes them in place
+ * and performs the capacity checks. */
 size_t sswin_token_plan_workspace_bytes(int64_t N, int B, int n);
 int sswin_token_plan(const int32_t* indices, int64_t N, int B, int n, int H, int32_t* tokens,
                      int32_t* plan, int64_t g_cap, int32_t* tasks, int64_t* totals_out, void* ws,
-                     size_t ws_bytes, void* stream);
+                     size_t ws_bytes, int synchronize, void* stream);
+int sswin_token_plan_totals(int64_t* totals, int H, int64_t g_cap);
 
 /* Token tensors are dense [N, stride] arrays of `dtype`; element (voxel v, head h, channel ch) is
  * base[v*stride + col0 + h*hd + ch].  "sq" arrays are fp32 arrays of all [c x c] blocks.

@@ -36,7 +36,8 @@ SIGNATURES = {
     "sswin_softmax_last_dim_forward": (_i32, [_vp, _vp, _i32, _i64, _vp, _vp]),
     "sswin_softmax_last_dim_backward": (_i32, [_vp, _vp, _vp, _i32, _i64, _vp, _vp]),
     "sswin_token_plan_workspace_bytes": (_sz, [_i64, _i32, _i32]),
-    "sswin_token_plan": (_i32, [_vp, _i64, _i32, _i32, _i32, _vp, _vp, _i64, _vp, _vp, _vp, _sz, _vp]),
+    "sswin_token_plan": (_i32, [_vp, _i64, _i32, _i32, _i32, _vp, _vp, _i64, _vp, _vp, _vp, _sz, _i32, _vp]),
+    "sswin_token_plan_totals": (_i32, [_vp, _i32, _i64]),
     "sswin_fused_tokens_to_sq": (_i32, [_i32, _i32, _vp, _i64, _i64, _vp, _i64, _i32, _i32, _vp, _i64, _i32,
                                         _vp, _i64, _i32, C.c_float, _vp, _i32, _vp, _i32, _vp, _vp, _vp]),
     "sswin_fused_sq_to_tokens": (_i32, [_i32, _i32, _vp, _i64, _i64, _vp, _i64, _i32, _vp, _vp, _i64, _i32,
@@ -52,7 +53,7 @@ SIGNATURES = {
                                                _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i32, _vp]),
 }
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 _lib = None
 
 

@@ -28,111 +28,126 @@ constexpr int FUSED_GROUPS_PER_WG = 4;
 
 // ------------------------------------------------------------------------------------------
 // token plan
+//
+// Five launches, no sort:
+//   1. clear the presence bitmap (W = ceil(n/32) words per window slot) and the counters
+//   2. one atomicOr per voxel
+//   3. per block of 256 window slots: sums of (tokens, tokens^2, non-empty windows)
+//   4. per block: prefix of the earlier blocks' sums, scan inside the block; every non-empty
+//      window learns the rank T of its first token, its rank k among the non-empty windows and
+//      the sum of c*c before it, and writes its H plan rows and task descriptors
+//   5. per voxel: rank = T(window) + number of occupied positions below its own
+// Reduce-then-scan (3, 4) instead of a chained scan: no block waits for another block.
 // ------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(256) void tp_fill_kernel(uint32_t* __restrict__ p, int64_t n, uint32_t v) {
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) p[i] = v;
+constexpr int TP_BLOCK = 256;
+
+__global__ __launch_bounds__(256) void tp_clear_kernel(uint32_t* __restrict__ p, int64_t n, int64_t* counters) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) p[i] = 0u;
+    if (blockIdx.x == 0 && threadIdx.x < 8) counters[threadIdx.x] = 0;
 }
 
-__global__ __launch_bounds__(256) void tp_set_bits_kernel(const int32_t* __restrict__ ind, int64_t N, int n,
+__global__ __launch_bounds__(256) void tp_set_bits_kernel(const int32_t* __restrict__ ind, int64_t N, int W,
                                                           uint32_t* __restrict__ bits) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i < N) {
         const int2 wp = *reinterpret_cast<const int2*>(ind + 2 * i);
-        const uint64_t v = (uint64_t)(uint32_t)wp.x * (uint32_t)n + (uint32_t)wp.y;
-        atomicOr(&bits[v >> 5], 1u << (v & 31));
+        atomicOr(&bits[(int64_t)wp.x * W + (wp.y >> 5)], 1u << (wp.y & 31));
     }
 }
 
-struct TpPopcLoad {
-    const uint32_t* bits;
-    __device__ int operator()(int64_t i) const { return __popc(bits[i]); }
-};
-struct TpExclusiveStore {
-    int32_t* out;
-    __device__ void operator()(int64_t i, int ex, int) const { out[i] = ex; }
-};
-
-__device__ __forceinline__ int tp_rank_of_bit(const uint32_t* __restrict__ bits,
-                                              const int32_t* __restrict__ word_prefix, uint64_t v) {
-    const uint64_t w = v >> 5;
-    return word_prefix[w] + __popc(bits[w] & ((1u << (v & 31)) - 1u));
-}
-
-// per voxel -> entries by token rank: source voxel, first rank and size of its window, pos, window
-__global__ __launch_bounds__(256) void tp_rank_kernel(const int32_t* __restrict__ ind, int64_t N, int n,
-                                                      const uint32_t* __restrict__ bits,
-                                                      const int32_t* __restrict__ word_prefix,
-                                                      int32_t* __restrict__ order, int32_t* __restrict__ tok_T,
-                                                      int32_t* __restrict__ tok_c, int32_t* __restrict__ tok_pos,
-                                                      int32_t* __restrict__ tok_win) {
-    const int64_t v = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (v >= N) return;
-    const int2 wp = *reinterpret_cast<const int2*>(ind + 2 * v);
-    const uint64_t first = (uint64_t)(uint32_t)wp.x * (uint32_t)n;
-    const int r = tp_rank_of_bit(bits, word_prefix, first + (uint32_t)wp.y);
-    const int T = tp_rank_of_bit(bits, word_prefix, first);
-    const int Tn = tp_rank_of_bit(bits, word_prefix, first + (uint32_t)n);
-    order[r] = (int32_t)v;
-    tok_T[r] = T;
-    tok_c[r] = Tn - T;
-    tok_pos[r] = wp.y;
-    tok_win[r] = wp.x;
-}
-
-// scan over token ranks: item = 1 | c*c << 32 at the first token of a window
-struct WindowLoad {
-    const int32_t* tok_T;
-    const int32_t* tok_c;
-    __device__ int64_t operator()(int64_t r) const {
-        if (tok_T[r] != (int32_t)r) return 0;
-        const int64_t c = tok_c[r];
-        return (int64_t)1 | ((c * c) << 32);
+__device__ __forceinline__ int tp_window_count(const uint32_t* __restrict__ bits, int64_t w, int W) {
+    int c = 0;
+    if (W == 4) {
+        const uint4 v = *reinterpret_cast<const uint4*>(bits + w * 4);
+        c = __popc(v.x) + __popc(v.y) + __popc(v.z) + __popc(v.w);
+    } else {
+        for (int k = 0; k < W; ++k) c += __popc(bits[w * W + k]);
     }
-};
-struct WindowStore {
-    const int32_t* tok_c;
-    const int32_t* tok_win;
-    int32_t* plan;
-    int64_t g_cap;
-    int H;
-    int32_t* cmax;
-    __device__ void operator()(int64_t r, int64_t ex, int64_t item) const {
-        if (item == 0) return;
-        const int64_t k = ex & 0xffffffffll;          // rank of the window among non-empty windows
-        const int64_t q2 = ex >> 32;                  // sum of c*c over earlier windows
-        const int c = tok_c[r];
-        const int w = tok_win[r];
+    return c;
+}
+
+// block sums: partial_a[blk] = sum c | sum c*c << 32, partial_b[blk] = non-empty windows
+__global__ __launch_bounds__(TP_BLOCK) void tp_block_sums_kernel(const uint32_t* __restrict__ bits, int64_t B, int W,
+                                                                 int64_t* __restrict__ partial_a,
+                                                                 int32_t* __restrict__ partial_b) {
+    __shared__ int64_t lds_a[TP_BLOCK / 64];
+    __shared__ int32_t lds_b[TP_BLOCK / 64];
+    const int64_t w = (int64_t)blockIdx.x * TP_BLOCK + threadIdx.x;
+    const int64_t c = w < B ? tp_window_count(bits, w, W) : 0;
+    int64_t ta;
+    int32_t tb;
+    (void)block_exclusive_scan<int64_t, TP_BLOCK / 64>(c | ((c * c) << 32), lds_a, &ta);
+    (void)block_exclusive_scan<int32_t, TP_BLOCK / 64>(c > 0 ? 1 : 0, lds_b, &tb);
+    if (threadIdx.x == 0) {
+        partial_a[blockIdx.x] = ta;
+        partial_b[blockIdx.x] = tb;
+    }
+}
+
+// Groups are bucketed by their number of 32-token tiles (bucket b: 32*b < c <= 32*(b+1), b = 0..3;
+// counters[4] counts larger groups, which get no descriptor).  Descriptor = {T, c | head << 8,
+// window, sq_start}.  Slots inside a bucket are handed out with one atomic per wavefront and
+// bucket, so the order of the windows inside a bucket varies from run to run; consumers treat a
+// bucket as an unordered set.
+__global__ __launch_bounds__(TP_BLOCK) void tp_windows_kernel(const uint32_t* __restrict__ bits, int64_t B, int W,
+                                                              int H, const int64_t* __restrict__ partial_a,
+                                                              const int32_t* __restrict__ partial_b,
+                                                              int32_t* __restrict__ win_T, int32_t* __restrict__ plan,
+                                                              int64_t g_cap, int4* __restrict__ tasks,
+                                                              int64_t* __restrict__ totals,
+                                                              int32_t* __restrict__ counters) {
+    __shared__ int64_t lds_a[TP_BLOCK / 64];
+    __shared__ int32_t lds_b[TP_BLOCK / 64];
+    __shared__ int64_t base_a_s;
+    __shared__ int32_t base_b_s;
+    // prefix of the earlier blocks
+    int64_t pa = 0;
+    int32_t pb = 0;
+    for (int64_t i = threadIdx.x; i < blockIdx.x; i += TP_BLOCK) {
+        pa += partial_a[i];
+        pb += partial_b[i];
+    }
+    int64_t ta;
+    int32_t tb;
+    (void)block_exclusive_scan<int64_t, TP_BLOCK / 64>(pa, lds_a, &ta);
+    (void)block_exclusive_scan<int32_t, TP_BLOCK / 64>(pb, lds_b, &tb);
+    if (threadIdx.x == 0) {
+        base_a_s = ta;
+        base_b_s = tb;
+    }
+    __syncthreads();
+    const int64_t base_a = base_a_s;
+    const int32_t base_b = base_b_s;
+
+    const int64_t w = (int64_t)blockIdx.x * TP_BLOCK + threadIdx.x;
+    const int64_t c = w < B ? tp_window_count(bits, w, W) : 0;
+    const int64_t ea = block_exclusive_scan<int64_t, TP_BLOCK / 64>(c | ((c * c) << 32), lds_a, &ta) + base_a;
+    const int32_t k = block_exclusive_scan<int32_t, TP_BLOCK / 64>(c > 0 ? 1 : 0, lds_b, &tb) + base_b;
+    if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) {
+        totals[0] = (int64_t)(base_b + tb);                     // non-empty windows
+        totals[1] = base_a + ta;                                // sum c | sum c*c << 32
+    }
+    const int32_t T = (int32_t)(ea & 0xffffffffll);
+    const int64_t q2 = ea >> 32;
+    if (w < B) win_T[w] = T;
+
+    const int lane = threadIdx.x & 63;
+    const bool live = c > 0 && ((int64_t)k + 1) * H <= g_cap;
+    if (live) {
         for (int h = 0; h < H; ++h) {
-            const int64_t g = k * H + h;
-            if (g >= g_cap) return;
-            plan[g] = c;
-            plan[g_cap + g] = (int32_t)r;             // T_k: rank of the window's first token
+            const int64_t g = (int64_t)k * H + h;
+            plan[g] = (int32_t)c;
+            plan[g_cap + g] = T;
             plan[2 * g_cap + g] = (int32_t)(q2 * H + (int64_t)h * c * c);
-            plan[3 * g_cap + g] = w;
+            plan[3 * g_cap + g] = (int32_t)w;
             plan[4 * g_cap + g] = h;
         }
-        if (c > *cmax) atomicMax(cmax, c);
     }
-};
-
-__global__ void tp_zero_kernel(int32_t* p, int n) {
-    if ((int)threadIdx.x < n) p[threadIdx.x] = 0;
-}
-
-// Groups bucketed by their number of 32-token tiles (bucket b: 32*b < c <= 32*(b+1), b = 0..3;
-// counts[4] counts larger groups, which have no descriptor).  Descriptor = {T, c | head << 8,
-// window, sq_start}.  Slots inside a bucket are handed out with one atomic per wavefront and
-// bucket, so the order inside a bucket varies from run to run; consumers treat the groups of a
-// bucket as an unordered set.
-__global__ __launch_bounds__(256) void tp_tasks_kernel(const int32_t* __restrict__ plan, int64_t g_cap, int H,
-                                                       const int64_t* __restrict__ scan_total,
-                                                       int4* __restrict__ tasks, int32_t* __restrict__ counts) {
-    const int64_t G = (scan_total[0] & 0xffffffffll) * H;
-    const int64_t g = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    const bool live = g < G && g < g_cap;
-    const int c = live ? plan[g] : 0;
-    const int b = live ? min((c - 1) >> 5, 4) : -1;
-    const int lane = threadIdx.x & 63;
+    // wave maximum of c, one atomic per wavefront
+    const int cm = wave_max_i32((int)c);
+    if (lane == 0 && cm > 0) atomicMax(&counters[5], cm);
+    if (tasks == nullptr) return;
+    const int b = live ? min(((int)c - 1) >> 5, 4) : -1;
     int slot = 0;
 #pragma unroll
     for (int q = 0; q < 5; ++q) {
@@ -140,13 +155,54 @@ __global__ __launch_bounds__(256) void tp_tasks_kernel(const int32_t* __restrict
         if (mine == 0) continue;
         const int leader = __ffsll((long long)mine) - 1;
         int base = 0;
-        if (lane == leader) base = atomicAdd(&counts[q], __popcll(mine));
+        if (lane == leader) base = atomicAdd(&counters[q], H * __popcll(mine));
         base = __shfl(base, leader, 64);
-        if (b == q) slot = base + __popcll(mine & ((1ull << lane) - 1ull));
+        if (b == q) slot = base + H * __popcll(mine & ((1ull << lane) - 1ull));
     }
-    if (live && b < 4)
-        tasks[(int64_t)b * g_cap + slot] =
-            make_int4(plan[g_cap + g], c | (plan[4 * g_cap + g] << 8), plan[3 * g_cap + g], plan[2 * g_cap + g]);
+    if (live && b < 4) {
+        for (int h = 0; h < H; ++h)
+            tasks[(int64_t)b * g_cap + slot + h] =
+                make_int4(T, (int)c | (h << 8), (int)w, (int32_t)(q2 * H + (int64_t)h * c * c));
+    }
+}
+
+// per voxel -> entries by token rank: source voxel, first rank and size of its window, pos, window
+__global__ __launch_bounds__(256) void tp_rank_kernel(const int32_t* __restrict__ ind, int64_t N, int W,
+                                                      const uint32_t* __restrict__ bits,
+                                                      const int32_t* __restrict__ win_T,
+                                                      int32_t* __restrict__ order, int32_t* __restrict__ tok_T,
+                                                      int32_t* __restrict__ tok_c, int32_t* __restrict__ tok_pos,
+                                                      int32_t* __restrict__ tok_win) {
+    const int64_t v = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (v >= N) return;
+    const int2 wp = *reinterpret_cast<const int2*>(ind + 2 * v);
+    const int T = win_T[wp.x];
+    const int word = wp.y >> 5;
+    const uint32_t below_mask = (1u << (wp.y & 31)) - 1u;
+    int below = 0, c = 0;
+    if (W == 4) {
+        const uint4 q = *reinterpret_cast<const uint4*>(bits + (int64_t)wp.x * 4);
+        const uint32_t b[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int pc = __popc(b[k]);
+            c += pc;
+            below += k < word ? pc : (k == word ? __popc(b[k] & below_mask) : 0);
+        }
+    } else {
+        for (int k = 0; k < W; ++k) {
+            const uint32_t x = bits[(int64_t)wp.x * W + k];
+            const int pc = __popc(x);
+            c += pc;
+            below += k < word ? pc : (k == word ? __popc(x & below_mask) : 0);
+        }
+    }
+    const int r = T + below;
+    order[r] = (int32_t)v;
+    tok_T[r] = T;
+    tok_c[r] = c;
+    tok_pos[r] = wp.y;
+    tok_win[r] = wp.x;
 }
 
 // ------------------------------------------------------------------------------------------
@@ -525,18 +581,21 @@ using namespace sswin;
 
 extern "C" {
 
-static size_t tp_words(int B, int n) { return (size_t)(((int64_t)B * n + n + 31) / 32) + 1; }
+static int tp_words_per_window(int n) { return (n + 31) / 32; }
+static int64_t tp_blocks(int B) { return ((int64_t)B + TP_BLOCK - 1) / TP_BLOCK; }
 
 size_t sswin_token_plan_workspace_bytes(int64_t N, int B, int n) {
-    const size_t words = tp_words(B, n);
-    const size_t tiles = (size_t)std::max<int64_t>(scan_num_tiles((int64_t)words), scan_num_tiles(N > 0 ? N : 1));
-    return align_up(words * 4, 256) * 2 + align_up(tiles * 8, 256) + 1024;
+    (void)N;
+    const size_t words = (size_t)B * tp_words_per_window(n);
+    const size_t blocks = (size_t)tp_blocks(B);
+    return align_up(words * 4, 256) + align_up((size_t)B * 4, 256) + align_up(blocks * 8, 256) +
+           align_up(blocks * 4, 256) + 1024;
 }
 
 int sswin_token_plan(const int32_t* indices, int64_t N, int B, int n, int H, int32_t* tokens,
                      int32_t* plan, int64_t g_cap, int32_t* tasks, int64_t* totals_out, void* ws,
-                     size_t ws_bytes, void* stream) {
-    SSWIN_CHECK(N >= 0 && B > 0 && n > 0 && H > 0, "token_plan: bad sizes");
+                     size_t ws_bytes, int synchronize, void* stream) {
+    SSWIN_CHECK(N >= 0 && B > 0 && n > 0 && H > 0 && H < 256, "token_plan: bad sizes");
     SSWIN_CHECK(totals_out, "token_plan: totals_out is null");
     for (int i = 0; i < 9; ++i) totals_out[i] = 0;
     if (N == 0) return 0;
@@ -546,57 +605,57 @@ int sswin_token_plan(const int32_t* indices, int64_t N, int B, int n, int H, int
     SSWIN_CHECK(ws_bytes >= sswin_token_plan_workspace_bytes(N, B, n), "token_plan: workspace too small");
     hipStream_t s = static_cast<hipStream_t>(stream);
     Carver cv(ws, ws_bytes);
-    const size_t words = tp_words(B, n);
-    int64_t* total_dev = cv.take<int64_t>(8);        // scan total, {c_max, -}, five bucket counters, -
+    const int W = tp_words_per_window(n);
+    const size_t words = (size_t)B * W;
+    const int64_t blocks = tp_blocks(B);
+    int64_t* totals_dev = cv.take<int64_t>(8);       // [0] windows, [1] sum c | sum c*c << 32, [2..7] counters
     uint32_t* bits = cv.take<uint32_t>(words);
-    int32_t* word_prefix = cv.take<int32_t>(words);
-    int64_t* tile_sums = cv.take<int64_t>(
-        (size_t)std::max<int64_t>(scan_num_tiles((int64_t)words), scan_num_tiles(N)));
+    int32_t* win_T = cv.take<int32_t>((size_t)B);
+    int64_t* partial_a = cv.take<int64_t>((size_t)blocks);
+    int32_t* partial_b = cv.take<int32_t>((size_t)blocks);
     SSWIN_CHECK(cv.ok(), "token_plan: workspace too small");
+    int32_t* counters = reinterpret_cast<int32_t*>(totals_dev + 2);   // five buckets, c_max
     int32_t* order = tokens;
     int32_t* tok_T = tokens + N;
     int32_t* tok_c = tokens + 2 * N;
     int32_t* tok_pos = tokens + 3 * N;
     int32_t* tok_win = tokens + 4 * N;
-    int32_t* cmax = reinterpret_cast<int32_t*>(total_dev + 1);
-    int32_t* bucket_counts = reinterpret_cast<int32_t*>(total_dev + 2);
 
-    const unsigned fill_blocks = (unsigned)std::min<size_t>((words + 255) / 256, 4096);
-    hipLaunchKernelGGL(tp_fill_kernel, dim3(fill_blocks), dim3(256), 0, s, bits, (int64_t)words, 0u);
-    hipLaunchKernelGGL(tp_zero_kernel, dim3(1), dim3(64), 0, s, cmax, 8);
+    const unsigned clear_blocks = (unsigned)std::min<size_t>((words + 255) / 256, 2048);
+    hipLaunchKernelGGL(tp_clear_kernel, dim3(clear_blocks), dim3(256), 0, s, bits, (int64_t)words, totals_dev);
     const unsigned nb = (unsigned)((N + 255) / 256);
-    hipLaunchKernelGGL(tp_set_bits_kernel, dim3(nb), dim3(256), 0, s, indices, N, n, bits);
-    TpPopcLoad pl{bits};
-    TpExclusiveStore ps{word_prefix};
-    if (device_exclusive_scan<int32_t>(pl, ps, (int64_t)words, reinterpret_cast<int32_t*>(tile_sums),
-                                       (int32_t*)nullptr, s, "token_plan bitmap scan"))
-        return 1;
-    hipLaunchKernelGGL(tp_rank_kernel, dim3(nb), dim3(256), 0, s, indices, N, n, bits, word_prefix, order, tok_T,
-                       tok_c, tok_pos, tok_win);
-    WindowLoad wl{tok_T, tok_c};
-    WindowStore wst{tok_c, tok_win, plan, g_cap, H, cmax};
-    if (device_exclusive_scan<int64_t>(wl, wst, N, tile_sums, total_dev, s, "token_plan window scan")) return 1;
-    if (tasks)
-        hipLaunchKernelGGL(tp_tasks_kernel, dim3((unsigned)((g_cap + 255) / 256)), dim3(256), 0, s, plan, g_cap, H,
-                           total_dev, reinterpret_cast<int4*>(tasks), bucket_counts);
-    int64_t host[5] = {0, 0, 0, 0, 0};
-    SSWIN_HIP(hipMemcpyAsync(host, total_dev, sizeof(host), hipMemcpyDeviceToHost, s));
+    hipLaunchKernelGGL(tp_set_bits_kernel, dim3(nb), dim3(256), 0, s, indices, N, W, bits);
+    hipLaunchKernelGGL(tp_block_sums_kernel, dim3((unsigned)blocks), dim3(TP_BLOCK), 0, s, bits, (int64_t)B, W,
+                       partial_a, partial_b);
+    hipLaunchKernelGGL(tp_windows_kernel, dim3((unsigned)blocks), dim3(TP_BLOCK), 0, s, bits, (int64_t)B, W, H,
+                       partial_a, partial_b, win_T, plan, g_cap, reinterpret_cast<int4*>(tasks), totals_dev, counters);
+    hipLaunchKernelGGL(tp_rank_kernel, dim3(nb), dim3(256), 0, s, indices, N, W, bits, win_T, order, tok_T, tok_c,
+                       tok_pos, tok_win);
+    if (launch_ok("token plan")) return 1;
+    // raw totals: the caller decodes them with sswin_token_plan_totals once the copy has landed
+    SSWIN_HIP(hipMemcpyAsync(totals_out, totals_dev, 8 * sizeof(int64_t), hipMemcpyDeviceToHost, s));
+    if (!synchronize) return 0;
     SSWIN_HIP(hipStreamSynchronize(s));
-    const int64_t windows = host[0] & 0xffffffffll;
-    const int64_t s2 = host[0] >> 32;
-    SSWIN_CHECK(host[0] >= 0 && s2 * H < (int64_t)INT32_MAX,
+    return sswin_token_plan_totals(totals_out, H, g_cap);
+}
+
+int sswin_token_plan_totals(int64_t* totals, int H, int64_t g_cap) {
+    SSWIN_CHECK(totals && H > 0, "token_plan_totals: bad arguments");
+    int64_t raw[8];
+    memcpy(raw, totals, sizeof(raw));
+    int32_t counters[12];
+    memcpy(counters, raw + 2, sizeof(counters));
+    const int64_t windows = raw[0];
+    const int64_t s2 = raw[1] >> 32;
+    SSWIN_CHECK(raw[1] >= 0 && s2 * H < (int64_t)INT32_MAX,
                 "token_plan: the attention matrix has 2^31 or more non-zeros, which int32 offsets cannot address");
-    totals_out[0] = windows * H;
-    totals_out[1] = windows;
-    totals_out[2] = s2 * H;
-    totals_out[3] = (int32_t)(host[1] & 0xffffffffll);
-    if (tasks) {
-        int32_t counts[6];
-        memcpy(counts, host + 2, sizeof(counts));
-        for (int b = 0; b < 5; ++b) totals_out[4 + b] = counts[b];
-    }
     SSWIN_CHECK(windows * H <= g_cap, "token_plan: %lld groups exceed the plan capacity %lld",
                 (long long)(windows * H), (long long)g_cap);
+    totals[0] = windows * H;
+    totals[1] = windows;
+    totals[2] = s2 * H;
+    totals[3] = counters[5];
+    for (int b = 0; b < 5; ++b) totals[4 + b] = counters[b];
     return 0;
 }
 

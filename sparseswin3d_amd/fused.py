@@ -30,9 +30,13 @@ def _ptr(t):
 
 
 class TokenPlan:
-    """Token order and per-group table of one set of (window, pos) voxel indices."""
+    """Token order and per-group table of one set of (window, pos) voxel indices.
 
-    def __init__(self, indices: torch.Tensor, batch_size: int, n: int, num_heads: int):
+    With ``defer=True`` the constructor only enqueues the kernels and the copy of the totals;
+    work enqueued afterwards (the qkv projection) overlaps the host round trip, and
+    :meth:`finish` waits for the totals when they are needed."""
+
+    def __init__(self, indices: torch.Tensor, batch_size: int, n: int, num_heads: int, defer: bool = False):
         lib = _lib.load()
         if indices.device.type != "cuda":
             raise RuntimeError("TokenPlan runs on the GPU only; there is no CPU fallback")
@@ -47,18 +51,35 @@ class TokenPlan:
         self.plan = torch.empty(5 * self.g_cap, dtype=torch.int32, device=d)
         # group descriptors of the window-resident kernels, bucketed by ceil(c / 32)
         self.tasks = torch.empty(16 * self.g_cap, dtype=torch.int32, device=d)
-        totals = (C.c_int64 * 9)()
+        self.device = d
+        self._totals = torch.zeros(9, dtype=torch.int64, pin_memory=True)
+        self._indices = indices                      # kept alive until the kernels have run
         with torch.cuda.device(d):
             nbytes = lib.sswin_token_plan_workspace_bytes(N, self.B, self.n)
-            ws = torch.empty(int(nbytes), dtype=torch.uint8, device=d)
+            self._ws = torch.empty(int(nbytes), dtype=torch.uint8, device=d)
             stream = C.c_void_p(torch.cuda.current_stream(d).cuda_stream)
             _lib.check(lib.sswin_token_plan(_ptr(indices), N, self.B, self.n, self.H, _ptr(self.tokens),
-                                            _ptr(self.plan), self.g_cap, _ptr(self.tasks), totals, _ptr(ws),
-                                            nbytes, stream))
+                                            _ptr(self.plan), self.g_cap, _ptr(self.tasks),
+                                            C.c_void_p(self._totals.data_ptr()), _ptr(self._ws), nbytes, 0, stream))
+            self._event = torch.cuda.Event()
+            self._event.record(torch.cuda.current_stream(d))
+        if not defer:
+            self.finish()
+
+    def finish(self):
+        """Wait for the totals (once) and decode them."""
+        if self._event is None:
+            return self
+        self._event.synchronize()
+        self._event = None
+        if self.N > 0:
+            _lib.check(_lib.load().sswin_token_plan_totals(C.c_void_p(self._totals.data_ptr()), self.H, self.g_cap))
+        totals = self._totals.tolist()
         self.G, self.windows, self.A, self.c_max = (int(totals[i]) for i in range(4))
         self.bucket_counts = (C.c_int64 * 4)(*(int(totals[4 + b]) for b in range(4)))
         self.oversize_groups = int(totals[8])
-        self.device = d
+        self._ws = self._indices = None
+        return self
 
 
 def _tokens_to_sq(tp, dtype, epilogue, a, a_stride, a_col0, b, b_stride, b_col0, hd, scale, bias, mask, out, rows):
@@ -80,13 +101,13 @@ def _sq_to_tokens(tp, dtype, a_kmajor, sq, b, b_stride, b_col0, o, o_stride, o_c
 
 class _FusedWindowAttention(Function):
     @staticmethod
-    def forward(ctx, qkv, bias, indices, mask, batch_size, n, scale):
+    def forward(ctx, qkv, bias, indices, mask, batch_size, n, scale, plan):
         # qkv [N, 3, H, hd]; bias fp32 [H, n, n]; indices int32 [N, 2]; mask int8 [nW, n] or None
         qkv = qkv.contiguous()
         N, _, H, hd = qkv.shape
         D = H * hd
         dtype = qkv.dtype
-        tp = TokenPlan(indices, batch_size, n, H)
+        tp = (plan or TokenPlan(indices, batch_size, n, H)).finish()
         d = qkv.device
         bias32 = bias.detach().to(torch.float32).contiguous()
         if mask is not None:
@@ -133,7 +154,7 @@ class _FusedWindowAttention(Function):
                 _lib.check(lib.sswin_fused_bias_grad(_ptr(tp.plan), tp.g_cap, tp.G, _ptr(tp.tokens), tp.N, H, tp.n,
                                                      _ptr(d_s), _ptr(d_bias32), _ptr(ws), nbytes, stream))
                 d_bias = d_bias32.to(bias_dtype)
-        return d_qkv, d_bias, None, None, None, None, None
+        return d_qkv, d_bias, None, None, None, None, None, None
 
 
 def _token_args(t, stride, col0):
@@ -145,13 +166,13 @@ class _ResidentWindowAttention(Function):
     qkv, the attention output and one log-sum-exp per attention row."""
 
     @staticmethod
-    def forward(ctx, qkv, bias, indices, mask, batch_size, n, scale):
+    def forward(ctx, qkv, bias, indices, mask, batch_size, n, scale, plan):
         qkv = qkv.contiguous()
         N, _, H, hd = qkv.shape
         D = H * hd
         dtype = qkv.dtype
         d = qkv.device
-        tp = TokenPlan(indices, batch_size, n, H)
+        tp = (plan or TokenPlan(indices, batch_size, n, H)).finish()
         if tp.oversize_groups:
             raise RuntimeError(f"window-resident attention: {tp.oversize_groups} groups hold more than 128 tokens")
         bias32 = bias.detach().to(torch.float32).contiguous()
@@ -203,19 +224,20 @@ class _ResidentWindowAttention(Function):
                 _lib.check(lib.sswin_fused_bias_grad(_ptr(tp.plan), tp.g_cap, tp.G, _ptr(tp.tokens), tp.N, H, tp.n,
                                                      _ptr(d_s), _ptr(d_bias32), _ptr(ws), nbytes, stream))
                 d_bias = d_bias32.to(bias_dtype)
-        return d_qkv, d_bias, None, None, None, None, None
+        return d_qkv, d_bias, None, None, None, None, None, None
 
 
-def fused_window_attention(qkv, bias, indices, mask, batch_size, n, scale, resident=None):
+def fused_window_attention(qkv, bias, indices, mask, batch_size, n, scale, resident=None, plan=None):
     """``qkv`` [N,3,H,hd], ``bias`` [H,n,n], ``indices`` int32 [N,2] (window,pos), ``mask`` int8
     [nW,n] or None -> attention output [N, H*hd] in the caller's voxel order.
 
     ``resident`` selects the window-resident kernels (default: whenever they apply, i.e. heads
-    of 32 channels); otherwise the block products with the attention matrix in HBM are used."""
+    of 32 channels); otherwise the block products with the attention matrix in HBM are used.
+    ``plan``: a :class:`TokenPlan` of ``indices`` made earlier (possibly still in flight)."""
     if resident is None:
         resident = supports_resident(qkv, n)
     fn = _ResidentWindowAttention if resident else _FusedWindowAttention
-    return fn.apply(qkv, bias, indices, mask, batch_size, n, scale)
+    return fn.apply(qkv, bias, indices, mask, batch_size, n, scale, plan)
 
 
 def supports_resident(qkv: torch.Tensor, n: int) -> bool:

@@ -357,14 +357,18 @@ class WindowAttentionSparse(nn.Module):
         n = x.spatial_shape[0]
         b = x.batch_size
         c = x.features.shape[-1]
-        qkv = tall_linear(x.features, self.qkv).reshape(-1, 3, self.num_heads, c // self.num_heads)
+        plan = None
         if self.fused:
             from . import fused
-            if fused.supports(qkv, n):
-                out = fused.fused_window_attention(qkv, self.relative_position_bias(n, torch.float32), x.indices,
-                                                   mask, b, n, self.scale, self.resident)
-                x = replace_feature(x, out)
-                return replace_feature(x, self.proj_drop(tall_linear(x.features, self.proj)))
+            if fused.supports(x.features, n):
+                # the token plan is enqueued first; the projection below runs while its totals travel
+                plan = fused.TokenPlan(x.indices, b, n, self.num_heads, defer=True)
+        qkv = tall_linear(x.features, self.qkv).reshape(-1, 3, self.num_heads, c // self.num_heads)
+        if plan is not None:
+            out = fused.fused_window_attention(qkv, self.relative_position_bias(n, torch.float32), x.indices,
+                                               mask, b, n, self.scale, self.resident, plan)
+            x = replace_feature(x, out)
+            return replace_feature(x, self.proj_drop(tall_linear(x.features, self.proj)))
         q, k_t, v = qkv_sparse_cuda(qkv, x.indices, b, n)
         attn = spspmm_block_naive(q * self.scale, k_t, "q_k")
         attn = sp_add_rpb(attn, self.relative_position_bias(n, attn.values.dtype))
