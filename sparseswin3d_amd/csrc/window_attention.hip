@@ -330,7 +330,7 @@ __global__ __launch_bounds__(256) void wattn_fwd_kernel(WAttnCommon a, TokenTens
 // backward, query side: dQ
 // ------------------------------------------------------------------------------------------
 template <typename T, bool MASK>
-__global__ __launch_bounds__(256) void wattn_bwd_q_kernel(WAttnCommon a, TokenTensor32 tq, TokenTensor32 tk,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void wattn_bwd_q_kernel(WAttnCommon a, TokenTensor32 tq, TokenTensor32 tk,
                                                           TokenTensor32 tv, TokenTensor32 to, TokenTensor32 tdo,
                                                           const float* __restrict__ lse, TokenTensor32 tdq) {
     __shared__ __attribute__((aligned(16))) float tiles[4][TILE_WORDS];
@@ -429,7 +429,7 @@ __global__ __launch_bounds__(256) void wattn_bwd_q_kernel(WAttnCommon a, TokenTe
 // backward, key side: dK, dV (and dS for the bias gradient)
 // ------------------------------------------------------------------------------------------
 template <typename T, bool MASK>
-__global__ __launch_bounds__(256) void wattn_bwd_kv_kernel(WAttnCommon a, TokenTensor32 tq, TokenTensor32 tk,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void wattn_bwd_kv_kernel(WAttnCommon a, TokenTensor32 tq, TokenTensor32 tk,
                                                            TokenTensor32 tv, TokenTensor32 to, TokenTensor32 tdo,
                                                            const float* __restrict__ lse, TokenTensor32 tdk,
                                                            TokenTensor32 tdv, float* __restrict__ ds_out) {
@@ -511,31 +511,46 @@ __global__ __launch_bounds__(256) void wattn_bwd_kv_kernel(WAttnCommon a, TokenT
         tile_put_rows(tile_do, l32, half, doa);
         __builtin_amdgcn_wave_barrier();
 
-        // P and dS of the tile: rows = queries acc_row(r, half), column = this lane's key
+        // P and dS of the tile: rows = queries acc_row(r, half), column = this lane's key.
+        // The bias gathers of all 16 rows are issued first; everything else is fetched from
+        // LDS four rows at a time, right before it is used, to keep the register footprint low.
         uint32_t pir[16];
         table_get(tab_pos, half, pir);
         float bv[16];
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-            bv[r] = *reinterpret_cast<const float*>(bias_h + (bcol + (MASK ? (pir[r] & 0xffffu) : pir[r])));
-        uint32_t Lr[16], Dr[16];
-        table_get(tab_L, half, Lr);
-        table_get(tab_D, half, Dr);
-        float dob[16], qbr[16];
-        tile_get_cols(tile_do, l32, half, dob);              // dO[query acc_row(r, half)][channel l32]
-        tile_get_cols(tile_q, l32, half, qbr);               // Q[query acc_row(r, half)][channel l32]
-        float* ds_t = ds_g ? ds_g + (int64_t)(t * 32 + 4 * half) * c : nullptr;
-        const int ilim = c - t * 32 - 4 * half;
+        uint32_t differ = 0;                                  // bit r: regions of the row and the key differ
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
-            float s = fmaf(bv[r], LOG2E, St[r]);
-            if (MASK && (int)(pir[r] >> 16) != reg_j) s += -100.0f * LOG2E;
-            const float pr = exp2_fast(s - u2f(Lr[r]));
-            const float ds = pr * (dPt[r] - u2f(Dr[r]));
-            const int row = 8 * (r >> 2) + (r & 3);
-            if (ds_t && row < ilim && j_k < c) ds_t[row * c] = ds;
-            dv = __builtin_amdgcn_mfma_f32_32x32x2f32(pr, dob[r], dv, 0, 0, 0);     // dV += P^T dO
-            dk = __builtin_amdgcn_mfma_f32_32x32x2f32(ds, qbr[r], dk, 0, 0, 0);     // dK += dS^T Q
+            bv[r] = *reinterpret_cast<const float*>(bias_h + (bcol + (MASK ? (pir[r] & 0xffffu) : pir[r])));
+            if (MASK) differ |= ((int)(pir[r] >> 16) != reg_j ? 1u : 0u) << r;
+        }
+        float* ds_t = ds_g ? ds_g + (int64_t)(t * 32 + 4 * half) * c : nullptr;
+        const int ilim = c - t * 32 - 4 * half;
+        const u32x4_a* L4 = reinterpret_cast<const u32x4_a*>(tab_L + 4 * half);
+        const u32x4_a* D4 = reinterpret_cast<const u32x4_a*>(tab_D + 4 * half);
+        const float* do_col = tile_do + 4 * half * TILE_LD + l32;
+        const float* q_col = tile_q + 4 * half * TILE_LD + l32;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const u32x4_a Lq = L4[2 * q], Dq = D4[2 * q];
+            const uint32_t Lr[4] = {Lq.x, Lq.y, Lq.z, Lq.w}, Dr[4] = {Dq.x, Dq.y, Dq.z, Dq.w};
+            float dob[4], qbr[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                dob[k] = do_col[(8 * q + k) * TILE_LD];      // dO[query acc_row(r, half)][channel l32]
+                qbr[k] = q_col[(8 * q + k) * TILE_LD];       // Q [query acc_row(r, half)][channel l32]
+            }
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const int r = 4 * q + k;
+                float s = fmaf(bv[r], LOG2E, St[r]);
+                if (MASK && (differ >> r & 1u)) s += -100.0f * LOG2E;
+                const float pr = exp2_fast(s - u2f(Lr[k]));
+                const float ds = pr * (dPt[r] - u2f(Dr[k]));
+                const int row = 8 * q + k;
+                if (ds_t && row < ilim && j_k < c) ds_t[row * c] = ds;
+                dv = __builtin_amdgcn_mfma_f32_32x32x2f32(pr, dob[k], dv, 0, 0, 0);     // dV += P^T dO
+                dk = __builtin_amdgcn_mfma_f32_32x32x2f32(ds, qbr[k], dk, 0, 0, 0);     // dK += dS^T Q
+            }
         }
     }
     tile_put_acc(tile_q, l32, half, dk);
