@@ -38,7 +38,11 @@ HBM_PEAK_GBPS = 8000.0
 # HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE) for the kernels
 # below on this workload; None = not measured.  Source summaries live in profiles/.
 MEASURED_TRAFFIC_BYTES = {
-    # profiles/fused_tok_kernel_cfg2_pmc.txt: FETCH_SIZE x 2.0 KiB + WRITE_SIZE x 1.0 KiB
+    # profiles/wattn_kernels_cfg2_pmc.txt and profiles/fused_tok_kernel_cfg2_pmc.txt:
+    # FETCH_SIZE x 2.0 KiB + WRITE_SIZE x 1.0 KiB per launch
+    "resident forward": 174.2e6,
+    "resident backward dQ": 258.0e6,
+    "resident backward dK,dV,dS": 348.1e6,
     "fused dV=P^T dO": 128.1e6,
     "fused dK=dS^T Q": 128.1e6,      # same kernel instantiation and operand shapes as dV
     "fused O=PV": 135.4e6,
