@@ -224,13 +224,24 @@ def kernel_table(wl, reps=20, only=None):
             0, ptr(tp.tasks), tp.g_cap, tp.bucket_counts, ptr(tp.tokens), N, H, hd, *qa, C.c_float(0.17), ptr(bias),
             b["n"], mask_p, nmw, ptr(out_f), D, 0, ptr(up_r), D, 0, ptr(lse), *da, ptr(s_f), sides, stream))
 
+    from sparseswin3d_amd.window_attention import relative_position_index_3d
+    ti = F.BiasTableIndex.build(relative_position_index_3d(wl["blocks"][0]["attn"].window_size).to(dev), 729)
+    d_table = torch.empty(729, H, device=dev)
+    tg_bytes = lib.sswin_bias_table_grad_workspace_bytes(tp.G, H, 729)
+    tg_ws = torch.empty(int(tg_bytes), dtype=torch.uint8, device=dev)
+
+    def r_table_grad():
+        _lib.check(lib.sswin_bias_table_grad(ptr(tp.plan), tp.g_cap, tp.G, ptr(tp.tokens), tp.N, H, b["n"], ptr(ti.code),
+                                             ti.offset0, 729, ptr(s_f), ptr(d_table), ptr(tg_ws), tg_bytes, stream))
+
     r_fwd()                                       # lse and out_f must hold a real forward for the backward timings
     r_entries = [
         ("resident token_plan", lambda: F.TokenPlan(b["idx"], b["slots"], b["n"], H), 28 * N + 36 * tp.G, 1),
         ("resident forward", r_fwd, 16 * E + 4 * H * N, 1),
         ("resident backward dQ", r_bwd(1), 24 * E + 4 * H * N, 1),
         ("resident backward dK,dV,dS", r_bwd(2), 28 * E + 4 * A + 4 * H * N, 1),
-        ("resident bias grad", lambda: _lib.check(lib.sswin_fused_bias_grad(ptr(tp.plan), tp.g_cap, tp.G, ptr(tp.tokens), tp.N, H, b["n"], ptr(s_f), ptr(dbias), ptr(bg_ws), bg_bytes, stream)), 4 * A, 1),
+        ("resident bias table grad", r_table_grad, 4 * A, 1),
+        ("resident bias grad [H,n,n]", lambda: _lib.check(lib.sswin_fused_bias_grad(ptr(tp.plan), tp.g_cap, tp.G, ptr(tp.tokens), tp.N, H, b["n"], ptr(s_f), ptr(dbias), ptr(bg_ws), bg_bytes, stream)), 4 * A, 1),
     ]
 
     def measure(items, path):
@@ -312,8 +323,8 @@ def cpu_baseline(wl, target_tokens=None, budget_s=15.0, max_repeats=3):
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=10)
-    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel table")
     ap.add_argument("--kernels-json", default=None)

@@ -216,6 +216,16 @@ int sswin_fused_bias_grad(const int32_t* plan, int64_t g_cap, int64_t G, const i
                           int64_t N, int H, int n, const float* ds, float* d_bias, void* ws,
                           size_t ws_bytes, void* stream);
 
+/* Gradient of the relative position bias table itself (swin3d_base.py:624-652 gathers the
+ * [H,n,n] bias from a [(2w-1)^3, H] table by relative_position_index; autograd scatters back with
+ * an index_add).  The index is linear in the two positions: rel(p_i,p_j) = code[p_i] - code[p_j]
+ * + offset0 (code: device int32 [n]).  d_table (fp32 [table_rows, H]) is overwritten.
+ * table_rows <= 1024, n <= 128.  No atomics, fixed summation order.  Asynchronous (the G == 0 case records a memset: do not capture it). */
+size_t sswin_bias_table_grad_workspace_bytes(int64_t G, int H, int table_rows);
+int sswin_bias_table_grad(const int32_t* plan, int64_t g_cap, int64_t G, const int32_t* tokens,
+                          int64_t N, int H, int n, const int32_t* code, int offset0, int table_rows,
+                          const float* ds, float* d_table, void* ws, size_t ws_bytes, void* stream);
+
 /* ---- window-resident attention (whole forward / backward of the attention core) ---------- */
 
 /* Forward of sparse_swin/swin3d_base.py:660-672 for every (window, head) group in one pass:

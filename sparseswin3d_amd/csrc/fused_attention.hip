@@ -544,6 +544,111 @@ __global__ __launch_bounds__(256) void rpb_grad_reduce_kernel(const float* __res
     d_rpb[e] += (sum[0] + sum[1]) + (sum[2] + sum[3]);
 }
 
+// ------------------------------------------------------------------------------------------
+// Gradient of the relative position bias *table*: d_table[rel(p_i, p_j), h] = sum of dS over all
+// windows, where rel(p_i, p_j) = code[p_i] - code[p_j] + offset0 (the index arithmetic of
+// sparse_swin/swin3d_base.py:630-647 is linear in the two positions).  A table has (2w-1)^3 rows
+// (729 for 5^3 windows), so every wavefront keeps a private copy of one head's column in LDS:
+// wavefront (h, s) walks its slice of the windows in plan order, reads the [c x c] blocks of dS
+// row by row: the entries of one row of dS go to different table rows, so a half wavefront adds a
+// row chunk with plain read-add-write, and the two halves work on alternate rows with a copy of
+// the column each (LDS float atomics would be an order of magnitude slower).  Partial columns are
+// summed in slice order by rpb_table_reduce_kernel.
+// ------------------------------------------------------------------------------------------
+constexpr int RPBT_MAX_ROWS = 1024;
+
+__global__ __launch_bounds__(256) void rpb_table_partial_kernel(FusedGroups gt, const int32_t* __restrict__ tok_pos,
+                                                                int H, const int32_t* __restrict__ code, int offset0,
+                                                                int rows, const float* __restrict__ ds,
+                                                                int64_t windows, int slices, int64_t per_slice,
+                                                                float* __restrict__ partial) {
+    __shared__ float tables[4][2][RPBT_MAX_ROWS];
+    __shared__ int32_t codes[4][128];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int half = lane >> 5, l32 = lane & 31;
+    const int64_t p = (int64_t)blockIdx.x * 4 + wave;           // wavefront id = s * H + h
+    if (p >= (int64_t)slices * H) return;
+    const int h = (int)(p % H);
+    const int64_t sl = p / H;
+    float* mine = tables[wave][half];
+    int32_t* cw = codes[wave];
+    for (int e = l32; e < rows; e += 32) mine[e] = 0.f;
+    // slice sl takes the windows sl, sl + slices, ...: crowded windows are neighbours in plan order,
+    // so dealing them out evens the load.  The next window's header is fetched early.
+    (void)per_slice;
+    int c_n = 0, T_n = 0, sq_n = 0;
+    if (sl < windows) {
+        const int64_t g = sl * H + h;
+        c_n = gt.c[g];
+        T_n = gt.T[g];
+        sq_n = gt.sq[g];
+    }
+    for (int64_t k = sl; k < windows; k += slices) {
+        const int c = c_n, Tk = T_n;
+        const float* blk = ds + sq_n;
+        if (k + slices < windows) {
+            const int64_t g = (k + slices) * H + h;
+            c_n = gt.c[g];
+            T_n = gt.T[g];
+            sq_n = gt.sq[g];
+        }
+        __builtin_amdgcn_wave_barrier();
+        for (int t = lane; t < c; t += 64) cw[t] = code[tok_pos[Tk + t]];
+        __builtin_amdgcn_wave_barrier();
+        // item = (row i, chunk of 32 columns): all lanes of an item hit different table rows.
+        // The two halves of the wavefront take alternate items and add into separate copies of
+        // the table, so plain read-add-write is enough.  Eight items per half are loaded first.
+        const int nch = (c + 31) >> 5, items = c * nch;
+        int i = half / nch, ch = half - i * nch;
+        for (int q0 = 0; q0 < items; q0 += 16) {
+            float v[8];
+            int row[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int q = q0 + 2 * u + half;
+                const int j = ch * 32 + l32;
+                const bool live = q < items && j < c;
+                v[u] = live ? blk[i * c + j] : 0.f;
+                const unsigned r = live ? (unsigned)(cw[i] - cw[j] + offset0) : 0xffffffffu;
+                row[u] = r < (unsigned)rows ? (int)r : -1;
+                ch += 2;
+                if (ch >= nch) { ch -= nch; i += 1; }
+                if (ch >= nch) { ch -= nch; i += 1; }
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (row[u] >= 0) mine[row[u]] += v[u];
+        }
+    }
+    __builtin_amdgcn_wave_barrier();
+    float* out = partial + ((int64_t)h * slices + sl) * rows;
+    for (int e = lane; e < rows; e += 64) out[e] = tables[wave][0][e] + tables[wave][1][e];
+}
+
+// d_table[row, h] = sum over slices of partial[h][slice][row].  One workgroup per 32 table rows
+// of one head: thread (q, r) adds the slices q, q+32, ... of row r (short independent chains),
+// then the 32 partial sums of a row are added in the order of q: a fixed order altogether.
+__global__ __launch_bounds__(1024) void rpb_table_reduce_kernel(const float* __restrict__ partial, int slices, int rows,
+                                                                int H, float* __restrict__ d_table) {
+    __shared__ float part[32][33];
+    const int r = threadIdx.x & 31, q = threadIdx.x >> 5;
+    const int h = blockIdx.y;
+    const int row = blockIdx.x * 32 + r;
+    float sum = 0.f;
+    if (row < rows) {
+        const float* src = partial + (int64_t)h * slices * rows + row;
+        for (int s = q; s < slices; s += 32) sum += src[(int64_t)s * rows];
+    }
+    part[q][r] = sum;
+    __syncthreads();
+    if (q == 0 && row < rows) {
+        float total = 0.f;
+#pragma unroll
+        for (int k = 0; k < 32; ++k) total += part[k][r];
+        d_table[(int64_t)row * H + h] = total;
+    }
+}
+
 template <typename T>
 static int launch_sq(bool epi, const FusedGroups& gt, const int32_t* order, const int32_t* tok_pos, int H, int hd,
                      const TokenTensor& ta, const TokenTensor& tb, float scale_a, const float* bias, int n,
@@ -732,6 +837,45 @@ int sswin_fused_bias_grad(const int32_t* plan, int64_t g_cap, int64_t G, const i
     hipLaunchKernelGGL(rpb_grad_reduce_kernel, dim3((unsigned)((elems + 255) / 256)), dim3(256), 0, s, partial, slices,
                        elems, d_bias);
     return launch_ok("fused bias gradient");
+}
+
+static int table_grad_slices(int64_t windows, int H) {
+    // about sixteen wavefronts per CU over all heads, at least two windows per slice
+    const int64_t want = std::max<int64_t>(1, 4096 / std::max(H, 1));
+    const int64_t useful = std::max<int64_t>(1, (windows + 1) / 2);
+    return (int)std::min<int64_t>(want, useful);
+}
+
+size_t sswin_bias_table_grad_workspace_bytes(int64_t G, int H, int table_rows) {
+    const int64_t windows = H > 0 ? G / H : 0;
+    return (size_t)table_grad_slices(windows, H) * H * table_rows * sizeof(float) + 256;
+}
+
+int sswin_bias_table_grad(const int32_t* plan, int64_t g_cap, int64_t G, const int32_t* tokens, int64_t N, int H,
+                          int n, const int32_t* code, int offset0, int table_rows, const float* ds, float* d_table,
+                          void* ws, size_t ws_bytes, void* stream) {
+    SSWIN_CHECK(G >= 0 && G <= g_cap && H > 0 && n > 0 && n <= 128, "bias_table_grad: bad sizes");
+    SSWIN_CHECK(table_rows > 0 && table_rows <= RPBT_MAX_ROWS, "bias_table_grad: a table of %d rows is not supported (%d at most)",
+                table_rows, RPBT_MAX_ROWS);
+    SSWIN_CHECK(d_table, "bias_table_grad: null pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (G == 0) {
+        SSWIN_HIP(hipMemsetAsync(d_table, 0, (size_t)table_rows * H * sizeof(float), s));
+        return 0;
+    }
+    SSWIN_CHECK(plan && tokens && code && ds && ws, "bias_table_grad: null pointer");
+    SSWIN_CHECK(ws_bytes >= sswin_bias_table_grad_workspace_bytes(G, H, table_rows), "bias_table_grad: workspace too small");
+    const FusedGroups gt = groups_of(plan, g_cap, G);
+    const int64_t windows = G / H;
+    const int slices = table_grad_slices(windows, H);
+    const int64_t per_slice = (windows + slices - 1) / slices;
+    float* partial = static_cast<float*>(ws);
+    const int64_t waves = (int64_t)slices * H;
+    hipLaunchKernelGGL(rpb_table_partial_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, s, gt, tokens + 3 * N, H,
+                       code, offset0, table_rows, ds, windows, slices, per_slice, partial);
+    hipLaunchKernelGGL(rpb_table_reduce_kernel, dim3((unsigned)((table_rows + 31) / 32), (unsigned)H), dim3(1024), 0, s,
+                       partial, slices, table_rows, H, d_table);
+    return launch_ok("bias table gradient");
 }
 
 }  // extern "C"

@@ -166,7 +166,9 @@ class _ResidentWindowAttention(Function):
     qkv, the attention output and one log-sum-exp per attention row."""
 
     @staticmethod
-    def forward(ctx, qkv, bias, indices, mask, batch_size, n, scale, plan):
+    def forward(ctx, qkv, bias, indices, mask, batch_size, n, scale, plan, table_index):
+        # ``bias`` is the gathered [H, n, n] bias, or, with ``table_index`` (a BiasTableIndex), the
+        # [rows, H] bias table itself: then the backward returns the table's gradient directly
         qkv = qkv.contiguous()
         N, _, H, hd = qkv.shape
         D = H * hd
@@ -175,7 +177,11 @@ class _ResidentWindowAttention(Function):
         tp = (plan or TokenPlan(indices, batch_size, n, H)).finish()
         if tp.oversize_groups:
             raise RuntimeError(f"window-resident attention: {tp.oversize_groups} groups hold more than 128 tokens")
-        bias32 = bias.detach().to(torch.float32).contiguous()
+        if table_index is None:
+            bias32 = bias.detach().to(torch.float32).contiguous()
+        else:
+            bias32 = (bias.detach().to(torch.float32).index_select(0, table_index.flat).reshape(n, n, H)
+                      .permute(2, 0, 1).contiguous())
         if mask is not None:
             mask = mask.to(torch.int8).contiguous()
         lib = _lib.load()
@@ -189,7 +195,7 @@ class _ResidentWindowAttention(Function):
                 C.c_float(scale), _ptr(bias32), n, _ptr(mask), 0 if mask is None else mask.shape[0],
                 *_token_args(out, D, 0), _ptr(lse), stream))
         ctx.save_for_backward(qkv, out, lse, bias32, mask)
-        ctx.tp, ctx.scale, ctx.bias_meta = tp, scale, (bias.dtype, bias.shape)
+        ctx.tp, ctx.scale, ctx.bias_meta, ctx.table_index = tp, scale, (bias.dtype, bias.shape), table_index
         return out
 
     @staticmethod
@@ -218,26 +224,68 @@ class _ResidentWindowAttention(Function):
             d_bias = None
             if want_bias:
                 bias_dtype, bias_shape = ctx.bias_meta
-                d_bias32 = torch.zeros(bias_shape, dtype=torch.float32, device=d)
-                nbytes = lib.sswin_fused_bias_grad_workspace_bytes(tp.G, H, tp.n)
-                ws = torch.empty(int(nbytes), dtype=torch.uint8, device=d)
-                _lib.check(lib.sswin_fused_bias_grad(_ptr(tp.plan), tp.g_cap, tp.G, _ptr(tp.tokens), tp.N, H, tp.n,
-                                                     _ptr(d_s), _ptr(d_bias32), _ptr(ws), nbytes, stream))
+                ti = ctx.table_index
+                if ti is None:
+                    d_bias32 = torch.zeros(bias_shape, dtype=torch.float32, device=d)
+                    nbytes = lib.sswin_fused_bias_grad_workspace_bytes(tp.G, H, tp.n)
+                    ws = torch.empty(int(nbytes), dtype=torch.uint8, device=d)
+                    _lib.check(lib.sswin_fused_bias_grad(_ptr(tp.plan), tp.g_cap, tp.G, _ptr(tp.tokens), tp.N, H,
+                                                         tp.n, _ptr(d_s), _ptr(d_bias32), _ptr(ws), nbytes, stream))
+                else:
+                    rows = bias_shape[0]
+                    d_bias32 = torch.empty(bias_shape, dtype=torch.float32, device=d)
+                    nbytes = lib.sswin_bias_table_grad_workspace_bytes(tp.G, H, rows)
+                    ws = torch.empty(int(nbytes), dtype=torch.uint8, device=d)
+                    _lib.check(lib.sswin_bias_table_grad(_ptr(tp.plan), tp.g_cap, tp.G, _ptr(tp.tokens), tp.N, H, tp.n,
+                                                         _ptr(ti.code), ti.offset0, rows, _ptr(d_s), _ptr(d_bias32),
+                                                         _ptr(ws), nbytes, stream))
                 d_bias = d_bias32.to(bias_dtype)
-        return d_qkv, d_bias, None, None, None, None, None, None
+        return d_qkv, d_bias, None, None, None, None, None, None, None
 
 
-def fused_window_attention(qkv, bias, indices, mask, batch_size, n, scale, resident=None, plan=None):
+class BiasTableIndex:
+    """The relative position index [n, n] of a bias table in the form the library uses:
+    ``index[p, q] = code[p] - code[q] + offset0`` (true for the index arithmetic of
+    sparse_swin/swin3d_base.py:630-647).  :meth:`build` returns None if an index is not of
+    that form or the table is too large for the table-gradient kernel."""
+
+    def __init__(self, flat, code, offset0):
+        self.flat, self.code, self.offset0 = flat, code, offset0
+
+    @staticmethod
+    def build(index: torch.Tensor, table_rows: int):
+        n = index.shape[0]
+        if index.dim() != 2 or index.shape[1] != n or n > 128 or table_rows > 1024 or n == 0:
+            return None
+        idx = index.to(torch.int64)
+        code = idx[:, 0]
+        offset0 = int(idx[0, 0]) - 0
+        # index[p, q] = code[p] - code[q] + offset0 with code[0] carrying offset0 out again
+        code = code - int(code[0])
+        if not torch.equal(idx, code[:, None] - code[None, :] + offset0):
+            return None
+        if int(idx.min()) < 0 or int(idx.max()) >= table_rows:
+            return None
+        return BiasTableIndex(idx.reshape(-1).contiguous(), code.to(torch.int32).contiguous(), offset0)
+
+
+def fused_window_attention(qkv, bias, indices, mask, batch_size, n, scale, resident=None, plan=None,
+                           table_index=None):
     """``qkv`` [N,3,H,hd], ``bias`` [H,n,n], ``indices`` int32 [N,2] (window,pos), ``mask`` int8
     [nW,n] or None -> attention output [N, H*hd] in the caller's voxel order.
 
     ``resident`` selects the window-resident kernels (default: whenever they apply, i.e. heads
     of 32 channels); otherwise the block products with the attention matrix in HBM are used.
-    ``plan``: a :class:`TokenPlan` of ``indices`` made earlier (possibly still in flight)."""
+    ``plan``: a :class:`TokenPlan` of ``indices`` made earlier (possibly still in flight).
+    ``table_index`` (resident path only): a :class:`BiasTableIndex`; ``bias`` is then the
+    [rows, H] bias table and its gradient is computed without the [H, n, n] detour."""
     if resident is None:
         resident = supports_resident(qkv, n)
-    fn = _ResidentWindowAttention if resident else _FusedWindowAttention
-    return fn.apply(qkv, bias, indices, mask, batch_size, n, scale, plan)
+    if resident:
+        return _ResidentWindowAttention.apply(qkv, bias, indices, mask, batch_size, n, scale, plan, table_index)
+    if table_index is not None:
+        raise ValueError("table_index needs the window-resident kernels")
+    return _FusedWindowAttention.apply(qkv, bias, indices, mask, batch_size, n, scale, plan)
 
 
 def supports_resident(qkv: torch.Tensor, n: int) -> bool:

@@ -348,6 +348,15 @@ class WindowAttentionSparse(nn.Module):
         trunc_normal_(self.relative_position_bias_table, std=0.02)
         self._bias_bins = {}        # (n, device) -> (index, bins) of the deterministic bias gather
 
+    def _table_index(self, n: int):
+        """BiasTableIndex of the first n positions on the table's device (cached), or None."""
+        from . import fused
+        table = self.relative_position_bias_table
+        key = ("table", n, table.device)
+        if key not in self._bias_bins:
+            self._bias_bins[key] = fused.BiasTableIndex.build(self.relative_position_index[:n, :n], table.shape[0])
+        return self._bias_bins[key]
+
     def relative_position_bias(self, n: int, dtype) -> torch.Tensor:
         table = self.relative_position_bias_table
         cached = self._bias_bins.get((n, table.device))
@@ -369,8 +378,14 @@ class WindowAttentionSparse(nn.Module):
                 plan = fused.TokenPlan(x.indices, b, n, self.num_heads, defer=True)
         qkv = tall_linear(x.features, self.qkv).reshape(-1, 3, self.num_heads, c // self.num_heads)
         if plan is not None:
-            out = fused.fused_window_attention(qkv, self.relative_position_bias(n, torch.float32), x.indices,
-                                               mask, b, n, self.scale, self.resident, plan)
+            resident = fused.supports_resident(qkv, n) if self.resident is None else self.resident
+            table_index = self._table_index(n) if resident else None
+            if table_index is not None:
+                out = fused.fused_window_attention(qkv, self.relative_position_bias_table, x.indices, mask, b, n,
+                                                   self.scale, True, plan, table_index)
+            else:
+                out = fused.fused_window_attention(qkv, self.relative_position_bias(n, torch.float32), x.indices,
+                                                   mask, b, n, self.scale, resident, plan)
             x = replace_feature(x, out)
             return replace_feature(x, self.proj_drop(tall_linear(x.features, self.proj)))
         q, k_t, v = qkv_sparse_cuda(qkv, x.indices, b, n)

@@ -179,3 +179,45 @@ def test_resident_kernels_on_ragged_windows(mix, use_mask):
                                          _ptr(ws), nbytes, stream))
     assert not torch.isnan(ds).any()
     close(d_bias.cpu().numpy(), bias_r.grad.numpy(), 1e-5, "d bias")
+
+
+@pytest.mark.parametrize("mix,H", [("tiny", 1), ("mixed", 3), ("full", 2), ("many", 3)])
+def test_bias_table_gradient(mix, H):
+    """d_table[rel(p_i, p_j), h] = sum of dS: the table-gradient kernel against a numpy scatter."""
+    import ctypes as C
+    from sparseswin3d_amd import _lib
+    from sparseswin3d_amd.fused import BiasTableIndex, TokenPlan, _ptr
+    from sparseswin3d_amd.window_attention import relative_position_index_3d
+    rng = np.random.default_rng(len(mix) + H)
+    mixes = {"tiny": [1, 2, 3, 1, 5, 4], "mixed": [1, 40, 2, 125, 0, 0, 17, 32, 90, 3, 3, 3, 3, 64, 65, 70],
+             "full": [125, 124, 100, 7], "many": list(rng.integers(0, 60, size=700))}
+    counts = [int(c) for c in mixes[mix]]
+    n, rows = 125, 729
+    ind = ragged_window_indices(rng, counts, n)
+    tp = TokenPlan(torch.from_numpy(ind).cuda(), len(counts), n, H)
+    rel = relative_position_index_3d((5, 5, 5))
+    ti = BiasTableIndex.build(rel.cuda(), rows)
+    assert ti is not None
+    ds = rng.standard_normal(tp.A).astype(np.float32)
+    lib = _lib.load()
+    out = torch.full((rows, H), float("nan"), device="cuda")
+    nbytes = lib.sswin_bias_table_grad_workspace_bytes(tp.G, H, rows)
+    ws = torch.empty(int(nbytes), dtype=torch.uint8, device="cuda")
+    ds_d = torch.from_numpy(ds).cuda()
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    _lib.check(lib.sswin_bias_table_grad(_ptr(tp.plan), tp.g_cap, tp.G, _ptr(tp.tokens), tp.N, H, n, _ptr(ti.code),
+                                         ti.offset0, rows, _ptr(ds_d), _ptr(out), _ptr(ws), nbytes, stream))
+    # reference: walk the plan on the host
+    plan = tp.plan.view(5, -1)[:, :tp.G].cpu().numpy()
+    pos = tp.tokens.view(5, -1)[3].cpu().numpy()
+    ref = np.zeros((rows, H))
+    reln = rel.numpy()
+    for g in range(tp.G):
+        c, T, sq, _, h = (int(v) for v in plan[:, g])
+        p = pos[T:T + c]
+        np.add.at(ref[:, h], reln[p][:, p].reshape(-1), ds[sq:sq + c * c].astype(np.float64))
+    close(out.cpu().numpy(), ref, 1e-5, "d table")
+    out2 = torch.empty_like(out)
+    _lib.check(lib.sswin_bias_table_grad(_ptr(tp.plan), tp.g_cap, tp.G, _ptr(tp.tokens), tp.N, H, n, _ptr(ti.code),
+                                         ti.offset0, rows, _ptr(ds_d), _ptr(out2), _ptr(ws), nbytes, stream))
+    assert torch.equal(out, out2)                       # same bits on every run
