@@ -44,6 +44,8 @@ SIGNATURES = {
                                         _vp, _i64, _i32, C.c_float, _vp]),
     "sswin_fused_bias_grad_workspace_bytes": (_sz, [_i64, _i32, _i32]),
     "sswin_fused_bias_grad": (_i32, [_vp, _i64, _i64, _vp, _i64, _i32, _i32, _vp, _vp, _vp, _sz, _vp]),
+    "sswin_column_sum_workspace_bytes": (_sz, [_i64, _i32]),
+    "sswin_column_sum": (_i32, [_vp, _i64, _i32, _vp, _vp, _sz, _vp]),
     "sswin_bias_table_grad_workspace_bytes": (_sz, [_i64, _i32, _i32]),
     "sswin_bias_table_grad": (_i32, [_vp, _i64, _i64, _vp, _i64, _i32, _i32, _vp, _i32, _i32, _vp, _vp, _vp, _sz, _vp]),
     "sswin_window_attention_forward": (_i32, [_i32, _vp, _i64, _vp, _vp, _i64, _i32, _i32,
@@ -55,7 +57,7 @@ SIGNATURES = {
                                                _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i32, _vp]),
 }
 
-ABI_VERSION = 5
+ABI_VERSION = 6
 _lib = None
 
 

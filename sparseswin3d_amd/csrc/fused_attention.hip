@@ -625,26 +625,33 @@ __global__ __launch_bounds__(256) void rpb_table_partial_kernel(FusedGroups gt, 
     for (int e = lane; e < rows; e += 64) out[e] = tables[wave][0][e] + tables[wave][1][e];
 }
 
-// d_table[row, h] = sum over slices of partial[h][slice][row].  One workgroup per 32 table rows
-// of one head: thread (q, r) adds the slices q, q+32, ... of row r (short independent chains),
-// then the 32 partial sums of a row are added in the order of q: a fixed order altogether.
+// d_table[row, h] = sum over slices of partial[h][slice][row].  One workgroup per 16 table rows
+// of one head: thread (q, r) adds the slices q, q+64, ... of row r (short chains, four loads in
+// flight each), then the 64 chain sums of a row are added in the order of q: a fixed order.
 __global__ __launch_bounds__(1024) void rpb_table_reduce_kernel(const float* __restrict__ partial, int slices, int rows,
                                                                 int H, float* __restrict__ d_table) {
-    __shared__ float part[32][33];
-    const int r = threadIdx.x & 31, q = threadIdx.x >> 5;
+    __shared__ float part[64][17];
+    const int r = threadIdx.x & 15, q = threadIdx.x >> 4;
     const int h = blockIdx.y;
-    const int row = blockIdx.x * 32 + r;
-    float sum = 0.f;
+    const int row = blockIdx.x * 16 + r;
+    float s0 = 0.f, s1 = 0.f, s2 = 0.f, s3 = 0.f;
     if (row < rows) {
         const float* src = partial + (int64_t)h * slices * rows + row;
-        for (int s = q; s < slices; s += 32) sum += src[(int64_t)s * rows];
+        int s = q;
+        for (; s + 192 < slices; s += 256) {
+            s0 += src[(int64_t)s * rows];
+            s1 += src[(int64_t)(s + 64) * rows];
+            s2 += src[(int64_t)(s + 128) * rows];
+            s3 += src[(int64_t)(s + 192) * rows];
+        }
+        for (; s < slices; s += 64) s0 += src[(int64_t)s * rows];
     }
-    part[q][r] = sum;
+    part[q][r] = (s0 + s1) + (s2 + s3);
     __syncthreads();
     if (q == 0 && row < rows) {
         float total = 0.f;
 #pragma unroll
-        for (int k = 0; k < 32; ++k) total += part[k][r];
+        for (int k = 0; k < 64; ++k) total += part[k][r];
         d_table[(int64_t)row * H + h] = total;
     }
 }
@@ -873,7 +880,7 @@ int sswin_bias_table_grad(const int32_t* plan, int64_t g_cap, int64_t G, const i
     const int64_t waves = (int64_t)slices * H;
     hipLaunchKernelGGL(rpb_table_partial_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, s, gt, tokens + 3 * N, H,
                        code, offset0, table_rows, ds, windows, slices, per_slice, partial);
-    hipLaunchKernelGGL(rpb_table_reduce_kernel, dim3((unsigned)((table_rows + 31) / 32), (unsigned)H), dim3(1024), 0, s,
+    hipLaunchKernelGGL(rpb_table_reduce_kernel, dim3((unsigned)((table_rows + 15) / 16), (unsigned)H), dim3(1024), 0, s,
                        partial, slices, table_rows, H, d_table);
     return launch_ok("bias table gradient");
 }

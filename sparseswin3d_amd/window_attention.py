@@ -234,6 +234,26 @@ def _rocblas_gemm():
         torch.backends.cuda.preferred_blas_library(prev)
 
 
+def _column_sum(t: torch.Tensor) -> torch.Tensor:
+    """``t.sum(0)`` of a tall [N, P] matrix; fp32 on the GPU goes through the library's two-stage
+    kernel (about twice as fast as the generic reduction on [10^5 x 288], fixed order)."""
+    p = t.shape[1]
+    if not (t.is_cuda and t.dtype == torch.float32 and t.dim() == 2 and p % 4 == 0 and p <= 1024 and t.shape[0] > 0):
+        return t.sum(0)
+    import ctypes as C
+    from . import _lib
+    lib = _lib.load()
+    t = t.contiguous()
+    with torch.cuda.device(t.device):
+        out = torch.empty(p, dtype=t.dtype, device=t.device)
+        nbytes = lib.sswin_column_sum_workspace_bytes(t.shape[0], p)
+        ws = torch.empty(int(nbytes), dtype=torch.uint8, device=t.device)
+        _lib.check(lib.sswin_column_sum(C.c_void_p(t.data_ptr()), t.shape[0], p, C.c_void_p(out.data_ptr()),
+                                        C.c_void_p(ws.data_ptr()), nbytes,
+                                        C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)))
+    return out
+
+
 class _TallLinear(Function):
     """``x @ W^T + b`` for a very tall ``x`` [N, in] (N = number of voxels): forward, input
     gradient and weight gradient are three library GEMMs, routed to the BLAS backend that
@@ -258,7 +278,7 @@ class _TallLinear(Function):
             if ctx.needs_input_grad[1]:
                 grad_w = grad_out.t() @ x
         if ctx.has_bias and ctx.needs_input_grad[2]:
-            grad_b = grad_out.sum(0)
+            grad_b = _column_sum(grad_out)
         return grad_x, grad_w, grad_b
 
 
