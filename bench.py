@@ -54,10 +54,11 @@ def log(*a):
 
 
 # ------------------------------------------------------------------------------------------
-def build_workload(device):
+def build_workload(device, name="cfg2"):
     from sparseswin3d_amd import synth
     from sparseswin3d_amd.window_attention import WindowAttentionSparse
-    w = synth.config2()
+    w = {"cfg1": synth.config1, "cfg2": synth.config2, "cfg3": synth.config3, "cfg4": synth.config4}[name]()
+    dtype = torch.bfloat16 if w.dtype == "bf16" else torch.float32
     ws = w.window
     shift = tuple(s // 2 for s in ws)
     torch.manual_seed(2)
@@ -70,11 +71,12 @@ def build_workload(device):
         st = synth.scene_stats(idx, nw * w.batch_size)
         attn = WindowAttentionSparse(w.dim, w.heads, ws, qkv_bias=True).to(device)
         torch.nn.init.xavier_uniform_(attn.qkv.weight)
+        attn = attn.to(dtype)
         blocks.append(dict(attn=attn, idx=torch.from_numpy(idx).to(device), idx_np=idx, slots=nw * w.batch_size,
                            n=n, mask=mask if any(sh) else None, stats=st.describe(w.heads), shift=sh))
-    feats = torch.randn(N, w.dim, device=device)
-    upstream = torch.randn(N, w.dim, device=device)
-    return dict(name=w.name, N=N, dim=w.dim, heads=w.heads, blocks=blocks, feats=feats, upstream=upstream,
+    feats = torch.randn(N, w.dim, device=device).to(dtype)
+    upstream = torch.randn(N, w.dim, device=device).to(dtype)
+    return dict(name=w.name, dtype=dtype, N=N, dim=w.dim, heads=w.heads, blocks=blocks, feats=feats, upstream=upstream,
                 mask_np=mask.cpu().numpy())
 
 
@@ -325,6 +327,8 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4"],
+                    help="cfg2 is the benchmark; the others report the step time only")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel table")
     ap.add_argument("--kernels-json", default=None)
@@ -339,7 +343,9 @@ def main():
         sys.exit("bench.py: no HIP GPU visible")
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
-    wl = build_workload(device)
+    wl = build_workload(device, args.workload)
+    if args.workload != "cfg2":
+        args.no_cpu = args.no_kernels = True
     log(f"workload {wl['name']}: N={wl['N']}, blocks: " + "; ".join(str(b["stats"]) for b in wl["blocks"]))
     if args.profile_kernel is not None:
         kernel_table(wl, reps=args.profile_reps, only=args.profile_kernel)
@@ -396,9 +402,9 @@ def main():
     line = {
         "metric": "window-attn tokens/s fwd+bwd on 1 MI355X", "value": value, "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": f"{wl['name']}: stage-1 block pair (regular 5^3 windows, then shifted by 2) of "
-                               "WindowAttentionSparse, dim 96, 3 heads, forward+backward",
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if wl["dtype"] == torch.bfloat16 else "f32", "data": "synthetic",
+        "config": {"workload": f"{wl['name']}: block pair (regular 5^3 windows, then shifted by 2) of "
+                               f"WindowAttentionSparse, dim {wl['dim']}, {wl['heads']} heads, forward+backward",
                    "voxels": wl["N"], "attention_calls_per_step": calls, **sizes},
         "roofline": roofline, "cpu_baseline": cpu,
     }

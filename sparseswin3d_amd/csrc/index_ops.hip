@@ -78,6 +78,93 @@ struct InclusiveStore {
     __device__ void operator()(int64_t i, int ex, int item) const { out[i] = ex + item; }
 };
 
+// int32 keys: 16-byte loads and stores.  A tile is 256 threads x 4 rounds x 4 keys; round v of
+// thread t covers keys (v*256 + t)*4 .. +3 of the tile, so every access is fully coalesced.  The
+// four per-round counts of a thread are scanned at once, packed 16 bits apiece into an int64.
+constexpr int UC_TILE = 4096;
+
+__device__ __forceinline__ void uc_flags(const int32_t* __restrict__ x, int64_t M, int64_t tile0, int v, int4& key,
+                                         int (&f)[4]) {
+    const int lane = threadIdx.x & 63;
+    const int64_t i0 = tile0 + ((int64_t)v * 256 + threadIdx.x) * 4;
+    key = make_int4(0, 0, 0, 0);
+    if (i0 + 3 < M) {
+        key = *reinterpret_cast<const int4*>(x + i0);
+    } else {
+        if (i0 < M) key.x = x[i0];
+        if (i0 + 1 < M) key.y = x[i0 + 1];
+        if (i0 + 2 < M) key.z = x[i0 + 2];
+    }
+    int prev = __shfl_up(key.w, 1, 64);                       // last key of the left neighbour
+    if (lane == 0) prev = (i0 > 0 && i0 < M) ? x[i0 - 1] : key.x;
+    f[0] = (i0 > 0 && i0 < M && key.x != prev) ? 1 : 0;
+    f[1] = (i0 + 1 < M && key.y != key.x) ? 1 : 0;
+    f[2] = (i0 + 2 < M && key.z != key.y) ? 1 : 0;
+    f[3] = (i0 + 3 < M && key.w != key.z) ? 1 : 0;
+}
+
+__global__ __launch_bounds__(256) void uc_reduce_kernel(const int32_t* __restrict__ x, int64_t M,
+                                                        int32_t* __restrict__ tile_sums) {
+    __shared__ int32_t lds[4];
+    const int64_t tile0 = (int64_t)blockIdx.x * UC_TILE;
+    int cnt = 0;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        int4 key;
+        int f[4];
+        uc_flags(x, M, tile0, v, key, f);
+        cnt += f[0] + f[1] + f[2] + f[3];
+    }
+    int32_t total;
+    (void)block_exclusive_scan<int32_t, 4>(cnt, lds, &total);
+    if (threadIdx.x == 0) tile_sums[blockIdx.x] = total;
+}
+
+__global__ __launch_bounds__(256) void uc_scan_kernel(const int32_t* __restrict__ x, int64_t M,
+                                                      const int32_t* __restrict__ tile_offs,
+                                                      int32_t* __restrict__ out) {
+    __shared__ int64_t lds[4];
+    const int64_t tile0 = (int64_t)blockIdx.x * UC_TILE;
+    int f[4][4];
+    int64_t packed = 0;
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        int4 key;
+        uc_flags(x, M, tile0, v, key, f[v]);
+        packed |= (int64_t)(f[v][0] + f[v][1] + f[v][2] + f[v][3]) << (16 * v);
+    }
+    int64_t total;
+    const int64_t ex = block_exclusive_scan<int64_t, 4>(packed, lds, &total);
+    int base = tile_offs[blockIdx.x];                          // flags before this tile
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        int r = base + (int)((ex >> (16 * v)) & 0xffff);      // flags before this thread's keys of round v
+        const int64_t i0 = tile0 + ((int64_t)v * 256 + threadIdx.x) * 4;
+        int4 o;
+        r += f[v][0]; o.x = r;
+        r += f[v][1]; o.y = r;
+        r += f[v][2]; o.z = r;
+        r += f[v][3]; o.w = r;
+        if (i0 + 3 < M) {
+            *reinterpret_cast<int4*>(out + i0) = o;
+        } else {
+            if (i0 < M) out[i0] = o.x;
+            if (i0 + 1 < M) out[i0 + 1] = o.y;
+            if (i0 + 2 < M) out[i0 + 2] = o.z;
+        }
+        base += (int)((total >> (16 * v)) & 0xffff);          // all flags of round v
+    }
+}
+
+static int unique_consecutive_i32(const int32_t* keys, int64_t M, int32_t* out, int32_t* tile_sums, hipStream_t s) {
+    if (M <= 0) return 0;
+    const int64_t tiles = (M + UC_TILE - 1) / UC_TILE;
+    hipLaunchKernelGGL(uc_reduce_kernel, dim3((unsigned)tiles), dim3(256), 0, s, keys, M, tile_sums);
+    hipLaunchKernelGGL((scan_tile_sums_kernel<int32_t>), dim3(1), dim3(1024), 0, s, tile_sums, tiles, (int32_t*)nullptr);
+    hipLaunchKernelGGL(uc_scan_kernel, dim3((unsigned)tiles), dim3(256), 0, s, keys, M, tile_sums, out);
+    return launch_ok("unique_consecutive");
+}
+
 template <typename K>
 static int unique_consecutive_t(const void* keys, int64_t M, int32_t* out, int32_t* tile_sums,
                                 hipStream_t s) {
@@ -316,7 +403,10 @@ int sswin_unique_consecutive_indices(const void* keys, int key_dtype, int64_t M,
     int32_t* tile_sums = cv.take<int32_t>((size_t)scan_num_tiles(M));
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (key_dtype) {
-        case SSWIN_I32: return unique_consecutive_t<int32_t>(keys, M, out, tile_sums, s);
+        case SSWIN_I32:
+            if (((uintptr_t)keys % 16) == 0 && ((uintptr_t)out % 16) == 0)
+                return unique_consecutive_i32(static_cast<const int32_t*>(keys), M, out, tile_sums, s);
+            return unique_consecutive_t<int32_t>(keys, M, out, tile_sums, s);
         case SSWIN_I64: return unique_consecutive_t<int64_t>(keys, M, out, tile_sums, s);
         case SSWIN_I16: return unique_consecutive_t<int16_t>(keys, M, out, tile_sums, s);
         case SSWIN_I8: return unique_consecutive_t<int8_t>(keys, M, out, tile_sums, s);

@@ -62,14 +62,24 @@ def test_sort_indices_full_range(ops, oracle):
     np.testing.assert_array_equal(ops.sort_indices(dev(keys)).cpu().numpy(), oracle.sort_indices(keys))
 
 
-@pytest.mark.parametrize("m,dtype", [(1, np.int32), (2, np.int32), (2048, np.int32), (2049, np.int32),
-                                     (100_003, np.int32), (50_000, np.int64)])
+@pytest.mark.parametrize("m,dtype", [(1, np.int32), (2, np.int32), (3, np.int32), (5, np.int32), (2048, np.int32),
+                                     (2049, np.int32), (4095, np.int32), (4096, np.int32), (4097, np.int32),
+                                     (100_003, np.int32), (1_000_001, np.int32), (50_000, np.int64)])
 def test_unique_consecutive_indices(ops, oracle, m, dtype):
     rng = np.random.default_rng(m)
     x = np.cumsum(rng.random(m) < 0.3).astype(dtype)            # sorted with runs
     out = ops.unique_consecutive_indices(dev(x)).cpu().numpy()
     assert out.dtype == np.int32
     np.testing.assert_array_equal(out, oracle.unique_consecutive_indices(x))
+
+
+def test_unique_consecutive_unaligned_view(ops, oracle):
+    """A view that starts 4 bytes into an allocation takes the generic (unvectorised) kernel."""
+    rng = np.random.default_rng(3)
+    x = np.cumsum(rng.random(10_001) < 0.5).astype(np.int32)
+    t = dev(x)[1:]
+    np.testing.assert_array_equal(ops.unique_consecutive_indices(t).cpu().numpy(),
+                                  oracle.unique_consecutive_indices(x[1:]))
 
 
 def test_unique_consecutive_unsorted_runs(ops, oracle):
