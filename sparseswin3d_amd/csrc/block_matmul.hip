@@ -258,6 +258,63 @@ static bool force_simple() {
     return v;
 }
 
+// COO index rows of a product, streamed by their own kernel: one wavefront per group, four
+// consecutive entries per lane and 16-byte stores (a row of the index matrix is a pure function
+// of the plan and the token positions, so the MFMA kernel does not have to carry it).
+// rows: window, head, pos_i, and pos_j ('q_k', J = c) or the channel ('qk_v', J = C).
+typedef int i32x4_u __attribute__((ext_vector_type(4), aligned(4)));
+
+template <bool IS_QK>
+__global__ __launch_bounds__(256) void emit_coo_kernel(GroupTable gt, int64_t G, int C,
+                                                       const int32_t* __restrict__ tok_pos,
+                                                       int32_t* __restrict__ out_idx, int64_t out_nnz) {
+    __shared__ int pos_s[GROUPS_PER_WG][MAX_POS];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int64_t g = (int64_t)blockIdx.x * GROUPS_PER_WG + wave;
+    if (g >= G) return;
+    const int c = gt.c[g];
+    const int64_t rs = gt.row_start[g];
+    const int w = gt.window[g], h = gt.head[g];
+    int* pos = pos_s[wave];
+    for (int i = lane; i < c; i += 64) pos[i] = tok_pos[(rs + i) * C];
+    __builtin_amdgcn_wave_barrier();
+    const int J = IS_QK ? c : C;
+    const int count = c * J;
+    const int64_t base = IS_QK ? (int64_t)gt.sq_start[g] : rs * C;
+    int32_t* r0 = out_idx + base;
+    int32_t* r1 = r0 + out_nnz;
+    int32_t* r2 = r1 + out_nnz;
+    int32_t* r3 = r2 + out_nnz;
+    const i32x4_u wv = {w, w, w, w}, hv = {h, h, h, h};
+    for (int f = 4 * lane; f < count; f += 256) {
+        int i = f / J, j = f - i * J;
+        int pi[4], pj[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const int ic = i < c ? i : c - 1;                 // entries past the end are not stored
+            pi[k] = pos[ic];
+            pj[k] = IS_QK ? pos[j] : j;
+            if (++j == J) {
+                j = 0;
+                ++i;
+            }
+        }
+        if (f + 3 < count) {
+            *reinterpret_cast<i32x4_u*>(r0 + f) = wv;
+            *reinterpret_cast<i32x4_u*>(r1 + f) = hv;
+            *reinterpret_cast<i32x4_u*>(r2 + f) = i32x4_u{pi[0], pi[1], pi[2], pi[3]};
+            *reinterpret_cast<i32x4_u*>(r3 + f) = i32x4_u{pj[0], pj[1], pj[2], pj[3]};
+        } else {
+            for (int k = 0; k < 4 && f + k < count; ++k) {
+                r0[f + k] = w;
+                r1[f + k] = h;
+                r2[f + k] = pi[k];
+                r3[f + k] = pj[k];
+            }
+        }
+    }
+}
+
 template <typename T, int MODE, bool EMIT>
 static int launch_product(const void* m1, const void* m2, const GroupTable& gt, int64_t G, int C,
                           const int32_t* tok_pos, void* out, int32_t* out_idx, int64_t out_nnz,
@@ -268,9 +325,15 @@ static int launch_product(const void* m1, const void* m2, const GroupTable& gt, 
         if (!force_simple()) {
             tiled = true;
             const unsigned blocks = (unsigned)((G + GROUPS_PER_WG - 1) / GROUPS_PER_WG);
-            hipLaunchKernelGGL((block_product_mfma_kernel<T, MODE, EMIT>), dim3(blocks), dim3(256), 0, s,
+            // 'q_k' writes its four index rows from a streaming kernel (measured faster than carrying
+            // them through the MFMA kernel); 'qk_v' keeps them in the product kernel
+            constexpr bool split = EMIT && MODE == MODE_QK;
+            hipLaunchKernelGGL((block_product_mfma_kernel<T, MODE, EMIT && !split>), dim3(blocks), dim3(256), 0, s,
                                static_cast<const T*>(m1), static_cast<const T*>(m2), gt, G, C, tok_pos,
                                static_cast<T*>(out), out_idx, out_nnz);
+            if (split)
+                hipLaunchKernelGGL((emit_coo_kernel<true>), dim3(blocks), dim3(256), 0, s, gt, G, C, tok_pos, out_idx,
+                                   out_nnz);
         }
     }
     if (!tiled) {
