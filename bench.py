@@ -82,6 +82,8 @@ def build_workload(device, name="cfg2"):
 
 def run_step(wl):
     from sparseswin3d_amd.window_attention import SparseVoxelTensor
+    for blk in wl["blocks"]:                                  # as a training step does: fresh gradients
+        blk["attn"].zero_grad(set_to_none=True)
     x = wl["feats"].detach().requires_grad_(True)
     h = x
     for b in wl["blocks"]:
@@ -243,7 +245,7 @@ def kernel_table(wl, reps=20, only=None):
         ("resident backward dQ", r_bwd(1), 24 * E + 4 * H * N, 1),
         ("resident backward dK,dV,dS", r_bwd(2), 28 * E + 4 * A + 4 * H * N, 1),
         ("resident bias table grad", r_table_grad, 4 * A, 1),
-        ("resident bias grad [H,n,n]", lambda: _lib.check(lib.sswin_fused_bias_grad(ptr(tp.plan), tp.g_cap, tp.G, ptr(tp.tokens), tp.N, H, b["n"], ptr(s_f), ptr(dbias), ptr(bg_ws), bg_bytes, stream)), 4 * A, 1),
+        ("resident bias grad [H,n,n]", lambda: _lib.check(lib.sswin_fused_bias_grad(ptr(tp.plan), tp.g_cap, tp.G, ptr(tp.tokens), tp.N, H, b["n"], ptr(s_f), ptr(dbias), ptr(bg_ws), bg_bytes, stream)), 4 * A, 0),
     ]
 
     def measure(items, path):

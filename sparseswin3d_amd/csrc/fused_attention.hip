@@ -560,34 +560,37 @@ constexpr int RPBT_MAX_ROWS = 1024;
 __global__ __launch_bounds__(256) void rpb_table_partial_kernel(FusedGroups gt, const int32_t* __restrict__ tok_pos,
                                                                 int H, const int32_t* __restrict__ code, int offset0,
                                                                 int rows, const float* __restrict__ ds,
-                                                                int64_t windows, int slices, int64_t per_slice,
+                                                                int64_t windows, int wslices, int rsplit,
                                                                 float* __restrict__ partial) {
     __shared__ float tables[4][2][RPBT_MAX_ROWS];
     __shared__ int32_t codes[4][128];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int half = lane >> 5, l32 = lane & 31;
     const int64_t p = (int64_t)blockIdx.x * 4 + wave;           // wavefront id = s * H + h
+    const int slices = wslices * rsplit;
     if (p >= (int64_t)slices * H) return;
     const int h = (int)(p % H);
     const int64_t sl = p / H;
+    const int64_t ws = sl % wslices;                            // windows ws, ws + wslices, ...
+    const int rs = (int)(sl / wslices);                         // rows rs, rs + rsplit, ... of each of them
     float* mine = tables[wave][half];
     int32_t* cw = codes[wave];
     for (int e = l32; e < rows; e += 32) mine[e] = 0.f;
-    // slice sl takes the windows sl, sl + slices, ...: crowded windows are neighbours in plan order,
-    // so dealing them out evens the load.  The next window's header is fetched early.
-    (void)per_slice;
+    // A slice takes every wslices-th window (crowded windows are neighbours in plan order, so
+    // dealing them out evens the load) and, when windows are few and large, every rsplit-th row of
+    // them.  The next window's header is fetched early.
     int c_n = 0, T_n = 0, sq_n = 0;
-    if (sl < windows) {
-        const int64_t g = sl * H + h;
+    if (ws < windows) {
+        const int64_t g = ws * H + h;
         c_n = gt.c[g];
         T_n = gt.T[g];
         sq_n = gt.sq[g];
     }
-    for (int64_t k = sl; k < windows; k += slices) {
+    for (int64_t k = ws; k < windows; k += wslices) {
         const int c = c_n, Tk = T_n;
         const float* blk = ds + sq_n;
-        if (k + slices < windows) {
-            const int64_t g = (k + slices) * H + h;
+        if (k + wslices < windows) {
+            const int64_t g = (k + wslices) * H + h;
             c_n = gt.c[g];
             T_n = gt.T[g];
             sq_n = gt.sq[g];
@@ -598,8 +601,10 @@ __global__ __launch_bounds__(256) void rpb_table_partial_kernel(FusedGroups gt, 
         // item = (row i, chunk of 32 columns): all lanes of an item hit different table rows.
         // The two halves of the wavefront take alternate items and add into separate copies of
         // the table, so plain read-add-write is enough.  Eight items per half are loaded first.
-        const int nch = (c + 31) >> 5, items = c * nch;
-        int i = half / nch, ch = half - i * nch;
+        const int nch = (c + 31) >> 5;
+        const int my_rows = c > rs ? (c - rs + rsplit - 1) / rsplit : 0;
+        const int items = my_rows * nch;
+        int ir = half / nch, ch = half - ir * nch;            // ir counts this slice's rows
         for (int q0 = 0; q0 < items; q0 += 16) {
             float v[8];
             int row[8];
@@ -607,13 +612,14 @@ __global__ __launch_bounds__(256) void rpb_table_partial_kernel(FusedGroups gt, 
             for (int u = 0; u < 8; ++u) {
                 const int q = q0 + 2 * u + half;
                 const int j = ch * 32 + l32;
+                const int i = rs + rsplit * ir;
                 const bool live = q < items && j < c;
                 v[u] = live ? blk[i * c + j] : 0.f;
                 const unsigned r = live ? (unsigned)(cw[i] - cw[j] + offset0) : 0xffffffffu;
                 row[u] = r < (unsigned)rows ? (int)r : -1;
                 ch += 2;
-                if (ch >= nch) { ch -= nch; i += 1; }
-                if (ch >= nch) { ch -= nch; i += 1; }
+                if (ch >= nch) { ch -= nch; ir += 1; }
+                if (ch >= nch) { ch -= nch; ir += 1; }
             }
 #pragma unroll
             for (int u = 0; u < 8; ++u)
@@ -846,16 +852,21 @@ int sswin_fused_bias_grad(const int32_t* plan, int64_t g_cap, int64_t G, const i
     return launch_ok("fused bias gradient");
 }
 
-static int table_grad_slices(int64_t windows, int H) {
-    // about sixteen wavefronts per CU over all heads, at least two windows per slice
+// slices = window slices x row split: about sixteen wavefronts per CU over all heads, at least two
+// windows per window slice; few large windows are also split by rows (up to 8 ways)
+static void table_grad_slices(int64_t windows, int H, int* wslices, int* rsplit) {
     const int64_t want = std::max<int64_t>(1, 4096 / std::max(H, 1));
     const int64_t useful = std::max<int64_t>(1, (windows + 1) / 2);
-    return (int)std::min<int64_t>(want, useful);
+    *wslices = (int)std::min<int64_t>(want, useful);
+    const int64_t waves = (int64_t)*wslices * H;
+    *rsplit = (int)std::max<int64_t>(1, std::min<int64_t>(8, 2048 / std::max<int64_t>(waves, 1)));
 }
 
 size_t sswin_bias_table_grad_workspace_bytes(int64_t G, int H, int table_rows) {
     const int64_t windows = H > 0 ? G / H : 0;
-    return (size_t)table_grad_slices(windows, H) * H * table_rows * sizeof(float) + 256;
+    int wslices, rsplit;
+    table_grad_slices(windows, H, &wslices, &rsplit);
+    return (size_t)wslices * rsplit * H * table_rows * sizeof(float) + 256;
 }
 
 int sswin_bias_table_grad(const int32_t* plan, int64_t g_cap, int64_t G, const int32_t* tokens, int64_t N, int H,
@@ -874,12 +885,13 @@ int sswin_bias_table_grad(const int32_t* plan, int64_t g_cap, int64_t G, const i
     SSWIN_CHECK(ws_bytes >= sswin_bias_table_grad_workspace_bytes(G, H, table_rows), "bias_table_grad: workspace too small");
     const FusedGroups gt = groups_of(plan, g_cap, G);
     const int64_t windows = G / H;
-    const int slices = table_grad_slices(windows, H);
-    const int64_t per_slice = (windows + slices - 1) / slices;
+    int wslices, rsplit;
+    table_grad_slices(windows, H, &wslices, &rsplit);
+    const int slices = wslices * rsplit;
     float* partial = static_cast<float*>(ws);
     const int64_t waves = (int64_t)slices * H;
     hipLaunchKernelGGL(rpb_table_partial_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, s, gt, tokens + 3 * N, H,
-                       code, offset0, table_rows, ds, windows, slices, per_slice, partial);
+                       code, offset0, table_rows, ds, windows, wslices, rsplit, partial);
     hipLaunchKernelGGL(rpb_table_reduce_kernel, dim3((unsigned)((table_rows + 15) / 16), (unsigned)H), dim3(1024), 0, s,
                        partial, slices, table_rows, H, d_table);
     return launch_ok("bias table gradient");
