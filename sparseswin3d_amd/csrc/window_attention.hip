@@ -25,7 +25,15 @@
 // Groups are bucketed by their number of 32-token tiles (1..4).  One launch covers all buckets:
 // tasks (group, 32-row block) are numbered with the heaviest bucket first, so the long tasks start
 // first and the short ones fill the tail; the loop over tiles is a run-time loop with a register
-// budget that does not depend on the tile count.
+// budget that does not depend on the tile count.  Groups of one tile get their whole backward
+// from one wavefront (wattn_bwd_one_kernel).
+//
+// Global memory is touched in whole row slices only: eight (fp32) or four (16-bit) neighbouring
+// lanes read or write the 128 or 64 contiguous bytes a head occupies in a token row, and a
+// wave-private LDS tile turns these pieces into the row-per-lane MFMA operands (RowLoad,
+// rows_to_tile, tile_store_rows).  A row-per-lane load would touch 64 different cache lines per
+// instruction for 16 bytes each; the vector memory pipeline of a compute unit is shared by all
+// its waves and was the busiest unit of these kernels before.
 #include <math.h>
 #include <stdint.h>
 
@@ -100,18 +108,6 @@ __device__ __forceinline__ const char* head_base(const TokenTensor32& t, int h) 
 template <typename T>
 __device__ __forceinline__ uint32_t pitch_of(const TokenTensor32& t) { return (uint32_t)t.stride * (uint32_t)sizeof(T); }
 
-// 16 consecutive channels of one token row -> fp32
-template <typename T>
-__device__ __forceinline__ void load_slice(const char* __restrict__ base, uint32_t off, float (&x)[16]);
-template <>
-__device__ __forceinline__ void load_slice<float>(const char* __restrict__ base, uint32_t off, float (&x)[16]) {
-    const f32x4_a* p = reinterpret_cast<const f32x4_a*>(base + off);
-#pragma unroll
-    for (int v = 0; v < 4; ++v) {
-        const f32x4_a t = p[v];
-        x[4 * v] = t.x; x[4 * v + 1] = t.y; x[4 * v + 2] = t.z; x[4 * v + 3] = t.w;
-    }
-}
 __device__ __forceinline__ void unpack2(uint32_t u, float& lo, float& hi, __half) {
     const __half2 h2 = __builtin_bit_cast(__half2, u);
     lo = __low2float(h2);
@@ -121,27 +117,6 @@ __device__ __forceinline__ void unpack2(uint32_t u, float& lo, float& hi, __hip_
     lo = __builtin_bit_cast(float, u << 16);
     hi = __builtin_bit_cast(float, u & 0xffff0000u);
 }
-template <typename T>
-__device__ __forceinline__ void load_slice(const char* __restrict__ base, uint32_t off, float (&x)[16]) {
-    const u32x4_a* p = reinterpret_cast<const u32x4_a*>(base + off);
-#pragma unroll
-    for (int v = 0; v < 2; ++v) {
-        const u32x4_a t = p[v];
-        unpack2(t.x, x[8 * v], x[8 * v + 1], T());
-        unpack2(t.y, x[8 * v + 2], x[8 * v + 3], T());
-        unpack2(t.z, x[8 * v + 4], x[8 * v + 5], T());
-        unpack2(t.w, x[8 * v + 6], x[8 * v + 7], T());
-    }
-}
-
-template <typename T>
-__device__ __forceinline__ void store_slice(char* __restrict__ base, uint32_t off, const float (&x)[16]);
-template <>
-__device__ __forceinline__ void store_slice<float>(char* __restrict__ base, uint32_t off, const float (&x)[16]) {
-    f32x4_a* p = reinterpret_cast<f32x4_a*>(base + off);
-#pragma unroll
-    for (int v = 0; v < 4; ++v) p[v] = f32x4_a{x[4 * v], x[4 * v + 1], x[4 * v + 2], x[4 * v + 3]};
-}
 __device__ __forceinline__ uint32_t pack2(float lo, float hi, __half) {
     return __builtin_bit_cast(uint32_t, __floats2half2_rn(lo, hi));
 }
@@ -149,14 +124,6 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi, __hip_bfloat16) {
     const uint32_t a = __builtin_bit_cast(uint16_t, __float2bfloat16(lo));
     const uint32_t b = __builtin_bit_cast(uint16_t, __float2bfloat16(hi));
     return a | (b << 16);
-}
-template <typename T>
-__device__ __forceinline__ void store_slice(char* __restrict__ base, uint32_t off, const float (&x)[16]) {
-    u32x4_a* p = reinterpret_cast<u32x4_a*>(base + off);
-#pragma unroll
-    for (int v = 0; v < 2; ++v)
-        p[v] = u32x4_a{pack2(x[8 * v], x[8 * v + 1], T()), pack2(x[8 * v + 2], x[8 * v + 3], T()),
-                       pack2(x[8 * v + 4], x[8 * v + 5], T()), pack2(x[8 * v + 6], x[8 * v + 7], T())};
 }
 
 // ------------------------------------------------------------------------------------------
@@ -209,13 +176,128 @@ __device__ __forceinline__ float u2f(uint32_t v) { return __builtin_bit_cast(flo
 __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
 
 // ------------------------------------------------------------------------------------------
-// forward
+// Coalesced token rows.  A head's slice of a token row is 32 channels = CH chunks of 16 bytes
+// (8 for fp32, 4 for 16-bit values).  One load instruction fetches 64 / CH whole slices: lane l
+// reads chunk l % CH of the row l / CH of its group, so the lanes of a slice read one contiguous
+// 128- or 64-byte piece and the memory pipeline sees a quarter of the requests a row-per-lane
+// load makes.  The pieces are turned into the row-per-lane MFMA operand through an LDS tile.
+// ------------------------------------------------------------------------------------------
+template <typename T>
+struct RowLoad {
+    static constexpr int CH = 32 * (int)sizeof(T) / 16;      // chunks per row slice
+    static constexpr int ROWS = 64 / CH;                     // rows per instruction
+    static constexpr int NI = 32 / ROWS;                     // instructions per 32 rows
+    u32x4_a v[NI];
+};
+
+// vox_lane: voxel of row l32, held by lanes l32 and l32 + 32
+template <typename T>
+__device__ __forceinline__ void rows_load(const char* __restrict__ base, uint32_t pitch, uint32_t vox_lane, int lane,
+                                          RowLoad<T>& r) {
+    constexpr int CH = RowLoad<T>::CH, ROWS = RowLoad<T>::ROWS;
+#pragma unroll
+    for (int v = 0; v < RowLoad<T>::NI; ++v) {
+        const uint32_t vox = (uint32_t)__shfl((int)vox_lane, v * ROWS + lane / CH, 64);
+        r.v[v] = *reinterpret_cast<const u32x4_a*>(base + (__umul24(vox, pitch) + (uint32_t)(lane % CH) * 16u));
+    }
+}
+template <typename T>
+__device__ __forceinline__ void rows_to_tile(float* tile, int lane, const RowLoad<T>& r);
+template <>
+__device__ __forceinline__ void rows_to_tile<float>(float* tile, int lane, const RowLoad<float>& r) {
+#pragma unroll
+    for (int v = 0; v < RowLoad<float>::NI; ++v)
+        *reinterpret_cast<u32x4_a*>(tile + (v * 8 + lane / 8) * TILE_LD + (lane % 8) * 4) = r.v[v];
+}
+template <typename T>
+__device__ __forceinline__ void rows_to_tile(float* tile, int lane, const RowLoad<T>& r) {
+#pragma unroll
+    for (int v = 0; v < RowLoad<T>::NI; ++v) {
+        float x[8];
+        unpack2(r.v[v].x, x[0], x[1], T());
+        unpack2(r.v[v].y, x[2], x[3], T());
+        unpack2(r.v[v].z, x[4], x[5], T());
+        unpack2(r.v[v].w, x[6], x[7], T());
+        f32x4_a* p = reinterpret_cast<f32x4_a*>(tile + (v * 16 + lane / 4) * TILE_LD + (lane % 4) * 8);
+        p[0] = f32x4_a{x[0], x[1], x[2], x[3]};
+        p[1] = f32x4_a{x[4], x[5], x[6], x[7]};
+    }
+}
+// tile rows -> global rows, the same lane assignment; rows at or beyond `rows` are padding
+template <typename T>
+__device__ __forceinline__ void tile_store_rows(const float* tile, char* __restrict__ base, uint32_t pitch,
+                                                uint32_t vox_lane, int rows, int lane);
+template <>
+__device__ __forceinline__ void tile_store_rows<float>(const float* tile, char* __restrict__ base, uint32_t pitch,
+                                                       uint32_t vox_lane, int rows, int lane) {
+#pragma unroll
+    for (int v = 0; v < 4; ++v) {
+        const int R = v * 8 + lane / 8;
+        const uint32_t vox = (uint32_t)__shfl((int)vox_lane, R, 64);
+        const u32x4_a x = *reinterpret_cast<const u32x4_a*>(tile + R * TILE_LD + (lane % 8) * 4);
+        if (R < rows) *reinterpret_cast<u32x4_a*>(base + (__umul24(vox, pitch) + (uint32_t)(lane % 8) * 16u)) = x;
+    }
+}
+template <typename T>
+__device__ __forceinline__ void tile_store_rows(const float* tile, char* __restrict__ base, uint32_t pitch,
+                                                uint32_t vox_lane, int rows, int lane) {
+#pragma unroll
+    for (int v = 0; v < 2; ++v) {
+        const int R = v * 16 + lane / 4;
+        const uint32_t vox = (uint32_t)__shfl((int)vox_lane, R, 64);
+        const f32x4_a* p = reinterpret_cast<const f32x4_a*>(tile + R * TILE_LD + (lane % 4) * 8);
+        const f32x4_a lo = p[0], hi = p[1];
+        const u32x4_a x = {pack2(lo.x, lo.y, T()), pack2(lo.z, lo.w, T()), pack2(hi.x, hi.y, T()), pack2(hi.z, hi.w, T())};
+        if (R < rows) *reinterpret_cast<u32x4_a*>(base + (__umul24(vox, pitch) + (uint32_t)(lane % 4) * 16u)) = x;
+    }
+}
+
+// table[row] = x_row . y_row for the 32 rows two loads hold: per-chunk dot products, summed over
+// the CH lanes of a row by DPP steps inside groups of 4 and 8 lanes
+template <typename T>
+__device__ __forceinline__ float chunk_dot(const u32x4_a& x, const u32x4_a& y);
+template <>
+__device__ __forceinline__ float chunk_dot<float>(const u32x4_a& x, const u32x4_a& y) {
+    float d = u2f(x.x) * u2f(y.x);
+    d = fmaf(u2f(x.y), u2f(y.y), d);
+    d = fmaf(u2f(x.z), u2f(y.z), d);
+    return fmaf(u2f(x.w), u2f(y.w), d);
+}
+template <typename T>
+__device__ __forceinline__ float chunk_dot(const u32x4_a& x, const u32x4_a& y) {
+    const uint32_t xs[4] = {x.x, x.y, x.z, x.w}, ys[4] = {y.x, y.y, y.z, y.w};
+    float d = 0.f;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        float a0, a1, b0, b1;
+        unpack2(xs[k], a0, a1, T());
+        unpack2(ys[k], b0, b1, T());
+        d = fmaf(a0, b0, d);
+        d = fmaf(a1, b1, d);
+    }
+    return d;
+}
+template <typename T>
+__device__ __forceinline__ void rows_dot_to_table(uint32_t* tab, int lane, const RowLoad<T>& x, const RowLoad<T>& y) {
+    constexpr int CH = RowLoad<T>::CH, ROWS = RowLoad<T>::ROWS;
+#pragma unroll
+    for (int v = 0; v < RowLoad<T>::NI; ++v) {
+        float d = chunk_dot<T>(x.v[v], y.v[v]);
+        d += dpp_f32<0xB1>(d);                               // lanes 0..3 of a quad
+        d += dpp_f32<0x4E>(d);
+        if (CH == 8) d += dpp_f32<0x141>(d);                 // the two quads of 8 lanes
+        if (lane % CH == 0) tab[v * ROWS + lane / CH] = f2u(d);
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// forward: rows = 32 queries of a group, tiles = its keys
 // ------------------------------------------------------------------------------------------
 template <typename T, bool MASK>
-__global__ __launch_bounds__(256) void wattn_fwd_kernel(WAttnCommon a, TokenTensor32 tq, TokenTensor32 tk,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void wattn_fwd_kernel(WAttnCommon a, TokenTensor32 tq, TokenTensor32 tk,
                                                         TokenTensor32 tv, TokenTensor32 to,
                                                         float* __restrict__ lse) {
-    __shared__ __attribute__((aligned(16))) float tiles[4][TILE_WORDS];
+    __shared__ __attribute__((aligned(16))) float tiles[4][2][TILE_WORDS];
     __shared__ __attribute__((aligned(16))) uint32_t tabs[4][2][32];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int half = lane >> 5, l32 = lane & 31;
@@ -225,13 +307,13 @@ __global__ __launch_bounds__(256) void wattn_fwd_kernel(WAttnCommon a, TokenTens
     const GroupCtx g = load_group(a.tasks, d);
     const int c = g.c, h = g.h;
     const int nt = (c + 31) >> 5;
-    float* tile = tiles[wave];
+    float* tile = tiles[wave][0];
+    float* tile_x = tiles[wave][1];
     uint32_t* tab_key = tabs[wave][0];
     uint32_t* tab_alpha = tabs[wave][1];
     const int32_t* order = a.order + g.Tk;
     const int32_t* tok_pos = a.tok_pos + g.Tk;
     const int8_t* mrow = MASK ? a.mask + (int64_t)(g.w % a.nmw) * a.n : nullptr;
-    const uint32_t slice = half * 16 * sizeof(T);
     const char* qbase = head_base<T>(tq, h);
     const char* kbase = head_base<T>(tk, h);
     const char* vbase = head_base<T>(tv, h);
@@ -244,7 +326,13 @@ __global__ __launch_bounds__(256) void wattn_fwd_kernel(WAttnCommon a, TokenTens
     const int pos_i = tok_pos[i_c];
     const int reg_i = MASK ? mrow[pos_i] : 0;
     float qb[16];
-    load_slice<T>(qbase, __umul24(vox_i, qpitch) + slice, qb);
+    {
+        RowLoad<T> rq;
+        rows_load<T>(qbase, qpitch, vox_i, lane, rq);
+        rows_to_tile<T>(tile_x, lane, rq);
+        __builtin_amdgcn_wave_barrier();
+        tile_get_rows(tile_x, l32, half, qb);
+    }
     const float qscale = a.scale * LOG2E;                    // scores are kept in units of log 2
 #pragma unroll
     for (int s = 0; s < 16; ++s) qb[s] *= qscale;
@@ -261,18 +349,22 @@ __global__ __launch_bounds__(256) void wattn_fwd_kernel(WAttnCommon a, TokenTens
         const int j_c = j < c ? j : c - 1;
         const uint32_t vox_j = order[j_c];
         const int pos_j = tok_pos[j_c];
-        float ka[16], va[16];
-        load_slice<T>(kbase, __umul24(vox_j, kpitch) + slice, ka);
-        load_slice<T>(vbase, __umul24(vox_j, vpitch) + slice, va);
+        RowLoad<T> rk, rv;
+        rows_load<T>(kbase, kpitch, vox_j, lane, rk);
+        rows_load<T>(vbase, vpitch, vox_j, lane, rv);
         uint32_t pk = (uint32_t)pos_j * 4u;
         if (MASK) pk |= (uint32_t)mrow[pos_j] << 16;
+        __builtin_amdgcn_wave_barrier();
         table_put(tab_key, l32, pk);
+        rows_to_tile<T>(tile_x, lane, rk);
+        rows_to_tile<T>(tile, lane, rv);
+        __builtin_amdgcn_wave_barrier();
+        float ka[16];
+        tile_get_rows(tile_x, l32, half, ka);
         // S^T tile: rows = keys, columns = queries
         f32x16 S = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
         for (int s = 0; s < 16; ++s) S = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[s], qb[s], S, 0, 0, 0);
-        tile_put_rows(tile, l32, half, va);
-        __builtin_amdgcn_wave_barrier();
         uint32_t pkr[16];
         table_get(tab_key, half, pkr);
         float bv[16];
@@ -314,16 +406,17 @@ __global__ __launch_bounds__(256) void wattn_fwd_kernel(WAttnCommon a, TokenTens
     l += __shfl_xor(l, 32, 64);
     l += 1e-8f;
     if (half == 0 && i_q < c) lse[(int64_t)a.H * g.Tk + h * c + i_q] = (m + __builtin_amdgcn_logf(l)) * LN2;
-    // accumulators (rows = queries by register) -> rows by lane, normalise, wide stores
+    // normalise (one factor per query row, through the table), accumulators -> LDS rows -> coalesced stores
+    __builtin_amdgcn_wave_barrier();
+    table_put(tab_alpha, l32, f2u(1.0f / l));
+    __builtin_amdgcn_wave_barrier();
+    uint32_t ir[16];
+    table_get(tab_alpha, half, ir);
+#pragma unroll
+    for (int r = 0; r < 16; ++r) o[r] *= u2f(ir[r]);
     tile_put_acc(tile, l32, half, o);
     __builtin_amdgcn_wave_barrier();
-    float orow[16];
-    tile_get_rows(tile, l32, half, orow);
-    const float inv_l = 1.0f / l;
-#pragma unroll
-    for (int s = 0; s < 16; ++s) orow[s] *= inv_l;
-    if (i_q < c)
-        store_slice<T>(const_cast<char*>(head_base<T>(to, h)), __umul24(vox_i, pitch_of<T>(to)) + slice, orow);
+    tile_store_rows<T>(tile, const_cast<char*>(head_base<T>(to, h)), pitch_of<T>(to), vox_i, c - bi * 32, lane);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -333,8 +426,8 @@ template <typename T, bool MASK>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void wattn_bwd_q_kernel(WAttnCommon a, TokenTensor32 tq, TokenTensor32 tk,
                                                           TokenTensor32 tv, TokenTensor32 to, TokenTensor32 tdo,
                                                           const float* __restrict__ lse, TokenTensor32 tdq) {
-    __shared__ __attribute__((aligned(16))) float tiles[4][TILE_WORDS];
-    __shared__ __attribute__((aligned(16))) uint32_t tabs[4][32];
+    __shared__ __attribute__((aligned(16))) float tiles[4][2][TILE_WORDS];
+    __shared__ __attribute__((aligned(16))) uint32_t tabs[4][2][32];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int half = lane >> 5, l32 = lane & 31;
     int64_t d;
@@ -343,12 +436,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     const GroupCtx g = load_group(a.tasks, d);
     const int c = g.c, h = g.h;
     const int nt = (c + 31) >> 5;
-    float* tile = tiles[wave];
-    uint32_t* tab_key = tabs[wave];
+    float* tile = tiles[wave][0];                            // K of the tile (read back by column)
+    float* tile_x = tiles[wave][1];                          // rows in transit to the operand layout, dQ
+    uint32_t* tab_key = tabs[wave][0];
+    uint32_t* tab_D = tabs[wave][1];
     const int32_t* order = a.order + g.Tk;
     const int32_t* tok_pos = a.tok_pos + g.Tk;
     const int8_t* mrow = MASK ? a.mask + (int64_t)(g.w % a.nmw) * a.n : nullptr;
-    const uint32_t slice = half * 16 * sizeof(T);
     const char* kbase = head_base<T>(tk, h);
     const char* vbase = head_base<T>(tv, h);
     const uint32_t kpitch = pitch_of<T>(tk), vpitch = pitch_of<T>(tv);
@@ -360,16 +454,21 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     const int reg_i = MASK ? mrow[pos_i] : 0;
     const float L2 = lse[(int64_t)a.H * g.Tk + h * c + i_c] * LOG2E;
     float qb[16], dob[16];
-    load_slice<T>(head_base<T>(tq, h), __umul24(vox_i, pitch_of<T>(tq)) + slice, qb);
-    load_slice<T>(head_base<T>(tdo, h), __umul24(vox_i, pitch_of<T>(tdo)) + slice, dob);
-    float D = 0.f;
     {
-        float ob[16];
-        load_slice<T>(head_base<T>(to, h), __umul24(vox_i, pitch_of<T>(to)) + slice, ob);
-#pragma unroll
-        for (int s = 0; s < 16; ++s) D = fmaf(dob[s], ob[s], D);
+        RowLoad<T> rq, rdo, ro;
+        rows_load<T>(head_base<T>(tq, h), pitch_of<T>(tq), vox_i, lane, rq);
+        rows_load<T>(head_base<T>(tdo, h), pitch_of<T>(tdo), vox_i, lane, rdo);
+        rows_load<T>(head_base<T>(to, h), pitch_of<T>(to), vox_i, lane, ro);
+        rows_to_tile<T>(tile_x, lane, rq);
+        __builtin_amdgcn_wave_barrier();
+        tile_get_rows(tile_x, l32, half, qb);
+        __builtin_amdgcn_wave_barrier();
+        rows_to_tile<T>(tile_x, lane, rdo);
+        rows_dot_to_table<T>(tab_D, lane, rdo, ro);          // D_i = dO_i . O_i
+        __builtin_amdgcn_wave_barrier();
+        tile_get_rows(tile_x, l32, half, dob);
     }
-    D += __shfl_xor(D, 32, 64);
+    const float D = u2f(tab_D[l32]);
     const float qscale = a.scale * LOG2E;
 #pragma unroll
     for (int s = 0; s < 16; ++s) qb[s] *= qscale;
@@ -383,26 +482,31 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         const int j_c = j < c ? j : c - 1;
         const uint32_t vox_j = order[j_c];
         const int pos_j = tok_pos[j_c];
-        float ka[16], va[16];
-        load_slice<T>(kbase, __umul24(vox_j, kpitch) + slice, ka);
-        load_slice<T>(vbase, __umul24(vox_j, vpitch) + slice, va);
+        RowLoad<T> rk, rv;
+        rows_load<T>(kbase, kpitch, vox_j, lane, rk);
+        rows_load<T>(vbase, vpitch, vox_j, lane, rv);
         uint32_t pk = (uint32_t)pos_j * 4u;
         if (MASK) pk |= (uint32_t)mrow[pos_j] << 16;
-        table_put(tab_key, l32, pk);
-        f32x16 St = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-        f32x16 dPt = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll
-        for (int s = 0; s < 16; ++s) St = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[s], qb[s], St, 0, 0, 0);
-        tile_put_rows(tile, l32, half, ka);                  // K rows, read back by column for dQ
-#pragma unroll
-        for (int s = 0; s < 16; ++s) dPt = __builtin_amdgcn_mfma_f32_32x32x2f32(va[s], dob[s], dPt, 0, 0, 0);
         __builtin_amdgcn_wave_barrier();
+        table_put(tab_key, l32, pk);
+        rows_to_tile<T>(tile, lane, rk);                     // K rows, read back by column for dQ
+        rows_to_tile<T>(tile_x, lane, rv);
+        __builtin_amdgcn_wave_barrier();
+        float ka[16], va[16];
+        tile_get_rows(tile, l32, half, ka);
+        tile_get_rows(tile_x, l32, half, va);
         uint32_t pkr[16];
         table_get(tab_key, half, pkr);
         float bv[16];
 #pragma unroll
         for (int r = 0; r < 16; ++r)
             bv[r] = *reinterpret_cast<const float*>(bias_h + (brow + (MASK ? (pkr[r] & 0xffffu) : pkr[r])));
+        f32x16 St = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        f32x16 dPt = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+        for (int s = 0; s < 16; ++s) St = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[s], qb[s], St, 0, 0, 0);
+#pragma unroll
+        for (int s = 0; s < 16; ++s) dPt = __builtin_amdgcn_mfma_f32_32x32x2f32(va[s], dob[s], dPt, 0, 0, 0);
         float kb[16];
         tile_get_cols(tile, l32, half, kb);                  // K[key acc_row(r, half)][channel l32]
         const int jlim = c - t * 32 - 4 * half;
@@ -415,14 +519,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             dq = __builtin_amdgcn_mfma_f32_32x32x2f32(ds, kb[r], dq, 0, 0, 0);
         }
     }
-    tile_put_acc(tile, l32, half, dq);
-    __builtin_amdgcn_wave_barrier();
-    float row[16];
-    tile_get_rows(tile, l32, half, row);
 #pragma unroll
-    for (int s = 0; s < 16; ++s) row[s] *= a.scale;
-    if (i_q < c)
-        store_slice<T>(const_cast<char*>(head_base<T>(tdq, h)), __umul24(vox_i, pitch_of<T>(tdq)) + slice, row);
+    for (int r = 0; r < 16; ++r) dq[r] *= a.scale;
+    __builtin_amdgcn_wave_barrier();
+    tile_put_acc(tile_x, l32, half, dq);
+    __builtin_amdgcn_wave_barrier();
+    tile_store_rows<T>(tile_x, const_cast<char*>(head_base<T>(tdq, h)), pitch_of<T>(tdq), vox_i, c - bi * 32, lane);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -451,7 +553,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     const int32_t* order = a.order + g.Tk;
     const int32_t* tok_pos = a.tok_pos + g.Tk;
     const int8_t* mrow = MASK ? a.mask + (int64_t)(g.w % a.nmw) * a.n : nullptr;
-    const uint32_t slice = half * 16 * sizeof(T);
     const char* qbase = head_base<T>(tq, h);
     const char* obase = head_base<T>(to, h);
     const char* dobase = head_base<T>(tdo, h);
@@ -465,8 +566,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     const int pos_j = tok_pos[j_c];
     const int reg_j = MASK ? mrow[pos_j] : 0;
     float kb[16], vb[16];
-    load_slice<T>(head_base<T>(tk, h), __umul24(vox_j, pitch_of<T>(tk)) + slice, kb);
-    load_slice<T>(head_base<T>(tv, h), __umul24(vox_j, pitch_of<T>(tv)) + slice, vb);
+    {
+        RowLoad<T> rk, rv;
+        rows_load<T>(head_base<T>(tk, h), pitch_of<T>(tk), vox_j, lane, rk);
+        rows_load<T>(head_base<T>(tv, h), pitch_of<T>(tv), vox_j, lane, rv);
+        rows_to_tile<T>(tile_q, lane, rk);
+        rows_to_tile<T>(tile_do, lane, rv);
+        __builtin_amdgcn_wave_barrier();
+        tile_get_rows(tile_q, l32, half, kb);
+        tile_get_rows(tile_do, l32, half, vb);
+    }
     const float kscale = a.scale * LOG2E;                    // scores in units of log 2
 #pragma unroll
     for (int s = 0; s < 16; ++s) kb[s] *= kscale;
@@ -485,31 +594,28 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
         const int pos_i = tok_pos[i_c];
         // padding queries get L = +inf, which makes their P and dS exactly zero
         const float L2_i = i < c ? lse_g[i_c] * LOG2E : INFINITY;
-        float qa[16], doa[16];
-        load_slice<T>(qbase, __umul24(vox_i, qpitch) + slice, qa);
-        load_slice<T>(dobase, __umul24(vox_i, dopitch) + slice, doa);
-        float D_i = 0.f;
-        {
-            float oa[16];
-            load_slice<T>(obase, __umul24(vox_i, opitch) + slice, oa);
-#pragma unroll
-            for (int s = 0; s < 16; ++s) D_i = fmaf(doa[s], oa[s], D_i);
-        }
-        D_i += __shfl_xor(D_i, 32, 64);
+        RowLoad<T> rq, rdo, ro;
+        rows_load<T>(qbase, qpitch, vox_i, lane, rq);
+        rows_load<T>(dobase, dopitch, vox_i, lane, rdo);
+        rows_load<T>(obase, opitch, vox_i, lane, ro);
         uint32_t pi = (uint32_t)(pos_i * a.n) * 4u;          // byte offset of bias row pos_i (< 2^16)
         if (MASK) pi |= (uint32_t)mrow[pos_i] << 16;
+        __builtin_amdgcn_wave_barrier();
         table_put(tab_pos, l32, pi);
         table_put(tab_L, l32, f2u(L2_i));
-        table_put(tab_D, l32, f2u(D_i));
+        rows_dot_to_table<T>(tab_D, lane, rdo, ro);          // D_i = dO_i . O_i
+        rows_to_tile<T>(tile_q, lane, rq);                   // both are read back by row and by column
+        rows_to_tile<T>(tile_do, lane, rdo);
+        __builtin_amdgcn_wave_barrier();
+        float qa[16], doa[16];
+        tile_get_rows(tile_q, l32, half, qa);
+        tile_get_rows(tile_do, l32, half, doa);
         f32x16 St = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
         f32x16 dPt = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
         for (int s = 0; s < 16; ++s) St = __builtin_amdgcn_mfma_f32_32x32x2f32(qa[s], kb[s], St, 0, 0, 0);
-        tile_put_rows(tile_q, l32, half, qa);
 #pragma unroll
         for (int s = 0; s < 16; ++s) dPt = __builtin_amdgcn_mfma_f32_32x32x2f32(doa[s], vb[s], dPt, 0, 0, 0);
-        tile_put_rows(tile_do, l32, half, doa);
-        __builtin_amdgcn_wave_barrier();
 
         // P and dS of the tile: rows = queries acc_row(r, half), column = this lane's key.
         // The bias gathers of all 16 rows are issued first; everything else is fetched from
@@ -553,18 +659,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
             }
         }
     }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dk[r] *= a.scale;
+    __builtin_amdgcn_wave_barrier();
     tile_put_acc(tile_q, l32, half, dk);
     tile_put_acc(tile_do, l32, half, dv);
     __builtin_amdgcn_wave_barrier();
-    float krow[16], vrow[16];
-    tile_get_rows(tile_q, l32, half, krow);
-    tile_get_rows(tile_do, l32, half, vrow);
-#pragma unroll
-    for (int s = 0; s < 16; ++s) krow[s] *= a.scale;
-    if (j_k < c) {
-        store_slice<T>(const_cast<char*>(head_base<T>(tdk, h)), __umul24(vox_j, pitch_of<T>(tdk)) + slice, krow);
-        store_slice<T>(const_cast<char*>(head_base<T>(tdv, h)), __umul24(vox_j, pitch_of<T>(tdv)) + slice, vrow);
-    }
+    tile_store_rows<T>(tile_q, const_cast<char*>(head_base<T>(tdk, h)), pitch_of<T>(tdk), vox_j, c - bj * 32, lane);
+    tile_store_rows<T>(tile_do, const_cast<char*>(head_base<T>(tdv, h)), pitch_of<T>(tdv), vox_j, c - bj * 32, lane);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -592,7 +694,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     uint32_t* tab_L = tabs[wave][2];
     uint32_t* tab_D = tabs[wave][3];
     const int8_t* mrow = MASK ? a.mask + (int64_t)(g.w % a.nmw) * a.n : nullptr;
-    const uint32_t slice = half * 16 * sizeof(T);
 
     // lane l32 owns token l32 as a query and as a key, clamped to the last token
     const int t_c = l32 < c ? l32 : c - 1;
@@ -602,27 +703,35 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     // padding queries get L = +inf, which makes their P and dS exactly zero
     const float L2 = l32 < c ? lse[(int64_t)a.H * g.Tk + h * c + t_c] * LOG2E : INFINITY;
     float qa[16], ka[16], va[16], doa[16];
-    load_slice<T>(head_base<T>(tq, h), __umul24(vox, pitch_of<T>(tq)) + slice, qa);
-    load_slice<T>(head_base<T>(tk, h), __umul24(vox, pitch_of<T>(tk)) + slice, ka);
-    load_slice<T>(head_base<T>(tv, h), __umul24(vox, pitch_of<T>(tv)) + slice, va);
-    load_slice<T>(head_base<T>(tdo, h), __umul24(vox, pitch_of<T>(tdo)) + slice, doa);
-    float D = 0.f;
     {
-        float oa[16];
-        load_slice<T>(head_base<T>(to, h), __umul24(vox, pitch_of<T>(to)) + slice, oa);
-#pragma unroll
-        for (int s = 0; s < 16; ++s) D = fmaf(doa[s], oa[s], D);
+        RowLoad<T> rq, rk, rv, rdo, ro;
+        rows_load<T>(head_base<T>(tk, h), pitch_of<T>(tk), vox, lane, rk);
+        rows_load<T>(head_base<T>(tv, h), pitch_of<T>(tv), vox, lane, rv);
+        rows_load<T>(head_base<T>(tq, h), pitch_of<T>(tq), vox, lane, rq);
+        rows_load<T>(head_base<T>(tdo, h), pitch_of<T>(tdo), vox, lane, rdo);
+        rows_load<T>(head_base<T>(to, h), pitch_of<T>(to), vox, lane, ro);
+        rows_to_tile<T>(tile_a, lane, rk);
+        rows_to_tile<T>(tile_b, lane, rv);
+        __builtin_amdgcn_wave_barrier();
+        tile_get_rows(tile_a, l32, half, ka);
+        tile_get_rows(tile_b, l32, half, va);
+        __builtin_amdgcn_wave_barrier();
+        rows_to_tile<T>(tile_a, lane, rq);
+        rows_to_tile<T>(tile_b, lane, rdo);                  // dO stays there for the second half
+        rows_dot_to_table<T>(tab_D, lane, rdo, ro);          // D_i = dO_i . O_i
+        __builtin_amdgcn_wave_barrier();
+        tile_get_rows(tile_a, l32, half, qa);
+        tile_get_rows(tile_b, l32, half, doa);
+        __builtin_amdgcn_wave_barrier();
     }
-    D += __shfl_xor(D, 32, 64);
+    const float D = u2f(tab_D[l32]);
     const uint32_t region_bits = MASK ? (uint32_t)reg << 16 : 0u;
     const uint32_t bcol = (uint32_t)pos * 4u;                // byte offset of bias column pos
     const uint32_t brow = (uint32_t)(pos * a.n) * 4u;        // byte offset of bias row pos (< 2^16)
     table_put(tab_key, l32, bcol | region_bits);
     table_put(tab_row, l32, brow | region_bits);
     table_put(tab_L, l32, f2u(L2));
-    table_put(tab_D, l32, f2u(D));
-    tile_put_rows(tile_a, l32, half, ka);
-    tile_put_rows(tile_b, l32, half, doa);
+    tile_put_rows(tile_a, l32, half, ka);                    // K rows, read back by column for dQ
     const float qscale = a.scale * LOG2E;                    // scores in units of log 2
     const char* bias_h = reinterpret_cast<const char*>(a.bias + (int64_t)h * a.n * a.n);
 
@@ -659,15 +768,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
                 dq = __builtin_amdgcn_mfma_f32_32x32x2f32(ds, kb[k], dq, 0, 0, 0);
             }
         }
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dq[r] *= a.scale;
         __builtin_amdgcn_wave_barrier();
         tile_put_acc(tile_a, l32, half, dq);
         __builtin_amdgcn_wave_barrier();
-        float row[16];
-        tile_get_rows(tile_a, l32, half, row);
-#pragma unroll
-        for (int s = 0; s < 16; ++s) row[s] *= a.scale;
-        if (l32 < c)
-            store_slice<T>(const_cast<char*>(head_base<T>(tdq, h)), __umul24(vox, pitch_of<T>(tdq)) + slice, row);
+        tile_store_rows<T>(tile_a, const_cast<char*>(head_base<T>(tdq, h)), pitch_of<T>(tdq), vox, c, lane);
     }
 
     // ---- queries by register, keys by lane: dK, dV, dS ----
@@ -720,19 +826,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
             dk = __builtin_amdgcn_mfma_f32_32x32x2f32(ds, qbr[k], dk, 0, 0, 0);     // dK += dS^T Q
         }
     }
+#pragma unroll
+    for (int r = 0; r < 16; ++r) dk[r] *= a.scale;
     __builtin_amdgcn_wave_barrier();
     tile_put_acc(tile_a, l32, half, dk);
     tile_put_acc(tile_b, l32, half, dv);
     __builtin_amdgcn_wave_barrier();
-    float krow[16], vrow[16];
-    tile_get_rows(tile_a, l32, half, krow);
-    tile_get_rows(tile_b, l32, half, vrow);
-#pragma unroll
-    for (int s = 0; s < 16; ++s) krow[s] *= a.scale;
-    if (l32 < c) {
-        store_slice<T>(const_cast<char*>(head_base<T>(tdk, h)), __umul24(vox, pitch_of<T>(tdk)) + slice, krow);
-        store_slice<T>(const_cast<char*>(head_base<T>(tdv, h)), __umul24(vox, pitch_of<T>(tdv)) + slice, vrow);
-    }
+    tile_store_rows<T>(tile_a, const_cast<char*>(head_base<T>(tdk, h)), pitch_of<T>(tdk), vox, c, lane);
+    tile_store_rows<T>(tile_b, const_cast<char*>(head_base<T>(tdv, h)), pitch_of<T>(tdv), vox, c, lane);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -828,6 +929,7 @@ static int check_common(const char* who, int dtype, const int32_t* tasks, int64_
                     (long long)counts[b], (long long)g_cap);
         *total += counts[b];
     }
+    SSWIN_CHECK(*total < ((int64_t)1 << 29), "%s: %lld groups are too many for one launch", who, (long long)*total);
     if (*total == 0) return 0;
     SSWIN_CHECK(tasks && tokens && bias, "%s: null pointer", who);
     SSWIN_CHECK(!mask || nmw > 0, "%s: mask without window count", who);
