@@ -42,7 +42,7 @@ MEASURED_TRAFFIC_BYTES = {
     # FETCH_SIZE x 2.0 KiB + WRITE_SIZE x 1.0 KiB per launch
     "resident forward": 174.2e6,
     "resident backward dQ": 258.0e6,
-    "resident backward dK,dV,dS": 348.1e6,
+    "resident backward dK,dV,dS": 344.5e6,
     "fused dV=P^T dO": 128.1e6,
     "fused dK=dS^T Q": 128.1e6,      # same kernel instantiation and operand shapes as dV
     "fused O=PV": 135.4e6,

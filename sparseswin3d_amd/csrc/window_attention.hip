@@ -25,8 +25,7 @@
 // Groups are bucketed by their number of 32-token tiles (1..4).  One launch covers all buckets:
 // tasks (group, 32-row block) are numbered with the heaviest bucket first, so the long tasks start
 // first and the short ones fill the tail; the loop over tiles is a run-time loop with a register
-// budget that does not depend on the tile count.  Groups of one tile get their whole backward
-// from one wavefront (wattn_bwd_one_kernel).
+// budget that does not depend on the tile count.
 //
 // Global memory is touched in whole row slices only: eight (fp32) or four (16-bit) neighbouring
 // lanes read or write the 128 or 64 contiguous bytes a head occupies in a token row, and a
@@ -138,11 +137,6 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi, __hip_bfloat16) {
 constexpr int TILE_LD = 36;
 constexpr int TILE_WORDS = 32 * TILE_LD;
 
-__device__ __forceinline__ void tile_put_rows(float* tile, int l32, int half, const float (&x)[16]) {
-    f32x4_a* p = reinterpret_cast<f32x4_a*>(tile + l32 * TILE_LD + half * 16);
-#pragma unroll
-    for (int v = 0; v < 4; ++v) p[v] = f32x4_a{x[4 * v], x[4 * v + 1], x[4 * v + 2], x[4 * v + 3]};
-}
 __device__ __forceinline__ void tile_get_rows(const float* tile, int l32, int half, float (&x)[16]) {
     const f32x4_a* p = reinterpret_cast<const f32x4_a*>(tile + l32 * TILE_LD + half * 16);
 #pragma unroll
@@ -670,173 +664,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
 }
 
 // ------------------------------------------------------------------------------------------
-// backward of a group of at most 32 tokens: dQ, dK, dV (and dS) from one wavefront.  The two
-// orientations of the score tile are both recomputed from one set of operand registers (lane l32
-// is query l32 and key l32 at once), so q, k, v, dO and O are read once instead of twice.
-// ------------------------------------------------------------------------------------------
-template <typename T, bool MASK>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void wattn_bwd_one_kernel(
-    WAttnCommon a, int64_t groups, TokenTensor32 tq, TokenTensor32 tk, TokenTensor32 tv, TokenTensor32 to,
-    TokenTensor32 tdo, const float* __restrict__ lse, TokenTensor32 tdq, TokenTensor32 tdk, TokenTensor32 tdv,
-    float* __restrict__ ds_out) {
-    __shared__ __attribute__((aligned(16))) float tiles[4][2][TILE_WORDS];
-    __shared__ __attribute__((aligned(16))) uint32_t tabs[4][4][32];
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-    const int half = lane >> 5, l32 = lane & 31;
-    const int64_t task = (int64_t)blockIdx.x * 4 + wave;
-    if (task >= groups) return;
-    const GroupCtx g = load_group(a.tasks, task);            // one-tile groups are bucket 0
-    const int c = g.c, h = g.h;
-    float* tile_a = tiles[wave][0];                          // K rows, then dQ, then Q rows, then dK
-    float* tile_b = tiles[wave][1];                          // dO rows, then dV
-    uint32_t* tab_key = tabs[wave][0];
-    uint32_t* tab_row = tabs[wave][1];
-    uint32_t* tab_L = tabs[wave][2];
-    uint32_t* tab_D = tabs[wave][3];
-    const int8_t* mrow = MASK ? a.mask + (int64_t)(g.w % a.nmw) * a.n : nullptr;
-
-    // lane l32 owns token l32 as a query and as a key, clamped to the last token
-    const int t_c = l32 < c ? l32 : c - 1;
-    const uint32_t vox = a.order[g.Tk + t_c];
-    const int pos = a.tok_pos[g.Tk + t_c];
-    const int reg = MASK ? mrow[pos] : 0;
-    // padding queries get L = +inf, which makes their P and dS exactly zero
-    const float L2 = l32 < c ? lse[(int64_t)a.H * g.Tk + h * c + t_c] * LOG2E : INFINITY;
-    float qa[16], ka[16], va[16], doa[16];
-    {
-        RowLoad<T> rq, rk, rv, rdo, ro;
-        rows_load<T>(head_base<T>(tk, h), pitch_of<T>(tk), vox, lane, rk);
-        rows_load<T>(head_base<T>(tv, h), pitch_of<T>(tv), vox, lane, rv);
-        rows_load<T>(head_base<T>(tq, h), pitch_of<T>(tq), vox, lane, rq);
-        rows_load<T>(head_base<T>(tdo, h), pitch_of<T>(tdo), vox, lane, rdo);
-        rows_load<T>(head_base<T>(to, h), pitch_of<T>(to), vox, lane, ro);
-        rows_to_tile<T>(tile_a, lane, rk);
-        rows_to_tile<T>(tile_b, lane, rv);
-        __builtin_amdgcn_wave_barrier();
-        tile_get_rows(tile_a, l32, half, ka);
-        tile_get_rows(tile_b, l32, half, va);
-        __builtin_amdgcn_wave_barrier();
-        rows_to_tile<T>(tile_a, lane, rq);
-        rows_to_tile<T>(tile_b, lane, rdo);                  // dO stays there for the second half
-        rows_dot_to_table<T>(tab_D, lane, rdo, ro);          // D_i = dO_i . O_i
-        __builtin_amdgcn_wave_barrier();
-        tile_get_rows(tile_a, l32, half, qa);
-        tile_get_rows(tile_b, l32, half, doa);
-        __builtin_amdgcn_wave_barrier();
-    }
-    const float D = u2f(tab_D[l32]);
-    const uint32_t region_bits = MASK ? (uint32_t)reg << 16 : 0u;
-    const uint32_t bcol = (uint32_t)pos * 4u;                // byte offset of bias column pos
-    const uint32_t brow = (uint32_t)(pos * a.n) * 4u;        // byte offset of bias row pos (< 2^16)
-    table_put(tab_key, l32, bcol | region_bits);
-    table_put(tab_row, l32, brow | region_bits);
-    table_put(tab_L, l32, f2u(L2));
-    tile_put_rows(tile_a, l32, half, ka);                    // K rows, read back by column for dQ
-    const float qscale = a.scale * LOG2E;                    // scores in units of log 2
-    const char* bias_h = reinterpret_cast<const char*>(a.bias + (int64_t)h * a.n * a.n);
-
-    // ---- keys by register, queries by lane: dQ ----
-    {
-        f32x16 St = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-        f32x16 dPt = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll
-        for (int s = 0; s < 16; ++s) St = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[s], qa[s] * qscale, St, 0, 0, 0);
-#pragma unroll
-        for (int s = 0; s < 16; ++s) dPt = __builtin_amdgcn_mfma_f32_32x32x2f32(va[s], doa[s], dPt, 0, 0, 0);
-        __builtin_amdgcn_wave_barrier();
-        uint32_t pkr[16];
-        table_get(tab_key, half, pkr);
-        float bv[16];
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-            bv[r] = *reinterpret_cast<const float*>(bias_h + (brow + (MASK ? (pkr[r] & 0xffffu) : pkr[r])));
-        const int jlim = c - 4 * half;                       // keys acc_row(r, 0) >= jlim are padding
-        const float* k_col = tile_a + 4 * half * TILE_LD + l32;
-        f32x16 dq = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            float kb[4];
-#pragma unroll
-            for (int k = 0; k < 4; ++k) kb[k] = k_col[(8 * q + k) * TILE_LD];   // K[key acc_row(r, half)][channel l32]
-#pragma unroll
-            for (int k = 0; k < 4; ++k) {
-                const int r = 4 * q + k;
-                float s = fmaf(bv[r], LOG2E, St[r]);
-                if (MASK && (int)(pkr[r] >> 16) != reg) s += -100.0f * LOG2E;
-                const float pr = (8 * q + k) < jlim ? exp2_fast(s - L2) : 0.f;
-                const float ds = pr * (dPt[r] - D);
-                dq = __builtin_amdgcn_mfma_f32_32x32x2f32(ds, kb[k], dq, 0, 0, 0);
-            }
-        }
-#pragma unroll
-        for (int r = 0; r < 16; ++r) dq[r] *= a.scale;
-        __builtin_amdgcn_wave_barrier();
-        tile_put_acc(tile_a, l32, half, dq);
-        __builtin_amdgcn_wave_barrier();
-        tile_store_rows<T>(tile_a, const_cast<char*>(head_base<T>(tdq, h)), pitch_of<T>(tdq), vox, c, lane);
-    }
-
-    // ---- queries by register, keys by lane: dK, dV, dS ----
-    __builtin_amdgcn_wave_barrier();
-    tile_put_rows(tile_a, l32, half, qa);
-    f32x16 S = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-    f32x16 dP = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll
-    for (int s = 0; s < 16; ++s) S = __builtin_amdgcn_mfma_f32_32x32x2f32(qa[s] * qscale, ka[s], S, 0, 0, 0);
-#pragma unroll
-    for (int s = 0; s < 16; ++s) dP = __builtin_amdgcn_mfma_f32_32x32x2f32(doa[s], va[s], dP, 0, 0, 0);
-    __builtin_amdgcn_wave_barrier();
-    uint32_t pir[16];
-    table_get(tab_row, half, pir);
-    float bv[16];
-    uint32_t differ = 0;                                     // bit r: regions of the row and the key differ
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-        bv[r] = *reinterpret_cast<const float*>(bias_h + (bcol + (MASK ? (pir[r] & 0xffffu) : pir[r])));
-        if (MASK) differ |= ((int)(pir[r] >> 16) != reg ? 1u : 0u) << r;
-    }
-    float* ds_t = ds_out ? ds_out + g.sq + l32 + (int64_t)(4 * half) * c : nullptr;
-    const int ilim = c - 4 * half;
-    const u32x4_a* L4 = reinterpret_cast<const u32x4_a*>(tab_L + 4 * half);
-    const u32x4_a* D4 = reinterpret_cast<const u32x4_a*>(tab_D + 4 * half);
-    const float* do_col = tile_b + 4 * half * TILE_LD + l32;
-    const float* q_col = tile_a + 4 * half * TILE_LD + l32;
-    f32x16 dk = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-    f32x16 dv = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        const u32x4_a Lq = L4[2 * q], Dq = D4[2 * q];
-        const uint32_t Lr[4] = {Lq.x, Lq.y, Lq.z, Lq.w}, Dr[4] = {Dq.x, Dq.y, Dq.z, Dq.w};
-        float dob[4], qbr[4];
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            dob[k] = do_col[(8 * q + k) * TILE_LD];          // dO[query acc_row(r, half)][channel l32]
-            qbr[k] = q_col[(8 * q + k) * TILE_LD];           // Q [query acc_row(r, half)][channel l32]
-        }
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            const int r = 4 * q + k;
-            float s = fmaf(bv[r], LOG2E, S[r]);
-            if (MASK && (differ >> r & 1u)) s += -100.0f * LOG2E;
-            const float pr = exp2_fast(s - u2f(Lr[k]));
-            const float ds = pr * (dP[r] - u2f(Dr[k]));
-            const int row = 8 * q + k;
-            if (ds_t && row < ilim && l32 < c) ds_t[row * c] = ds;
-            dv = __builtin_amdgcn_mfma_f32_32x32x2f32(pr, dob[k], dv, 0, 0, 0);     // dV += P^T dO
-            dk = __builtin_amdgcn_mfma_f32_32x32x2f32(ds, qbr[k], dk, 0, 0, 0);     // dK += dS^T Q
-        }
-    }
-#pragma unroll
-    for (int r = 0; r < 16; ++r) dk[r] *= a.scale;
-    __builtin_amdgcn_wave_barrier();
-    tile_put_acc(tile_a, l32, half, dk);
-    tile_put_acc(tile_b, l32, half, dv);
-    __builtin_amdgcn_wave_barrier();
-    tile_store_rows<T>(tile_a, const_cast<char*>(head_base<T>(tdk, h)), pitch_of<T>(tdk), vox, c, lane);
-    tile_store_rows<T>(tile_b, const_cast<char*>(head_base<T>(tdv, h)), pitch_of<T>(tdv), vox, c, lane);
-}
-
-// ------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------
 constexpr int WATTN_BUCKETS = 4;
@@ -857,20 +684,12 @@ static void launch_backward(const WAttnCommon& a, const TokenTensor32& q, const 
                             const TokenTensor32& v, const TokenTensor32& o, const TokenTensor32& d_o, const float* lse,
                             const TokenTensor32& dq, const TokenTensor32& dk, const TokenTensor32& dv, float* ds_out,
                             int sides, hipStream_t s) {
-    // With both sides wanted, groups of one tile go to the kernel that produces all three
-    // gradients from one wavefront; the per-side kernels cover the larger groups.
-    WAttnCommon big = a;
-    const int64_t one_tile = sides == 3 ? a.first[4] - a.first[3] : 0;
-    if (one_tile) big.first[4] = a.first[3];
-    const unsigned blocks = (unsigned)((big.first[4] + 3) / 4);
-    if (blocks && (sides & 1))
-        hipLaunchKernelGGL((wattn_bwd_q_kernel<T, MASK>), dim3(blocks), dim3(256), 0, s, big, q, k, v, o, d_o, lse, dq);
-    if (blocks && (sides & 2))
-        hipLaunchKernelGGL((wattn_bwd_kv_kernel<T, MASK>), dim3(blocks), dim3(256), 0, s, big, q, k, v, o, d_o, lse, dk,
+    const unsigned blocks = (unsigned)((a.first[4] + 3) / 4);
+    if (sides & 1)
+        hipLaunchKernelGGL((wattn_bwd_q_kernel<T, MASK>), dim3(blocks), dim3(256), 0, s, a, q, k, v, o, d_o, lse, dq);
+    if (sides & 2)
+        hipLaunchKernelGGL((wattn_bwd_kv_kernel<T, MASK>), dim3(blocks), dim3(256), 0, s, a, q, k, v, o, d_o, lse, dk,
                            dv, ds_out);
-    if (one_tile)
-        hipLaunchKernelGGL((wattn_bwd_one_kernel<T, MASK>), dim3((unsigned)((one_tile + 3) / 4)), dim3(256), 0, s, a,
-                           one_tile, q, k, v, o, d_o, lse, dq, dk, dv, ds_out);
 }
 
 template <typename T>
