@@ -77,7 +77,9 @@ def build_workload(device, name="cfg2"):
     feats = torch.randn(N, w.dim, device=device).to(dtype)
     upstream = torch.randn(N, w.dim, device=device).to(dtype)
     return dict(name=w.name, dtype=dtype, N=N, dim=w.dim, heads=w.heads, blocks=blocks, feats=feats, upstream=upstream,
-                mask_np=mask.cpu().numpy())
+                mask_np=mask.cpu().numpy(), coords4=torch.from_numpy(w.coords4).to(device),
+                spatial_shape=tuple(w.spatial_shape), batch_size=w.batch_size, window=tuple(ws), shift=shift,
+                padded=tuple(pshape))
 
 
 def run_step(wl):
@@ -273,7 +275,41 @@ def kernel_table(wl, reps=20, only=None):
         log(f"calibration copy: {reps} launches of {src.numel() * 4} bytes read and written")
         return [], dict(N=N, E=E, A=A, G=G, c_max=c_max)
     table = measure(r_entries, "resident") + measure(f_entries, "fused") + measure(entries, "operators")
+    table += measure(stage_entries(wl), "stage")
     return table, dict(N=N, E=E, A=A, G=G, c_max=c_max)
+
+
+def stage_entries(wl):
+    """Index glue of a stage (block and stage level callers of the attention): the kernels, and
+    the tensor-op chains of the reference's formulation they replace (calls = 0)."""
+    from sparseswin3d_amd import layers
+    from sparseswin3d_amd.window_attention import SparseVoxelTensor
+    N, D = wl["N"], wl["dim"]
+    c4, ws, sh, pd = wl["coords4"], wl["window"], wl["shift"], wl["padded"]
+    n = ws[0] * ws[1] * ws[2]
+    windows = (pd[0] // ws[0]) * (pd[1] // ws[1]) * (pd[2] // ws[2])
+    x = SparseVoxelTensor(wl["feats"].float(), c4, wl["spatial_shape"], wl["batch_size"])
+    plan, coords, _ = layers.downsample_plan(x, 2)
+    M = plan.windows
+
+    def torch_partition():
+        t = SparseVoxelTensor(x.features, c4, pd, wl["batch_size"])
+        t = layers.roll_sparse_tensor(t, tuple(-s for s in sh), (1, 2, 3))
+        return layers.window_partition_sparse(t, ws)
+
+    def torch_pool():
+        inv = torch.repeat_interleave(torch.arange(M, device=c4.device), plan.plan[:M].long())
+        out = torch.zeros(M, D, device=c4.device).index_add_(0, inv, x.features[plan.tokens[:N].long()])
+        return out / plan.plan[:M, None]
+
+    return [
+        ("stage window indices (pad+roll+partition)", lambda: layers.sparse_window_indices(c4, wl["batch_size"], pd, ws, sh), 24 * N, 1),
+        ("stage shift mask", lambda: layers.compute_mask(list(pd), list(ws), list(sh), c4.device), windows * n, 1),
+        ("stage merge plan (2x2x2 cells, coords)", lambda: layers.downsample_plan(x, 2), 16 * N + 20 * N + 16 * M, 1),
+        ("stage merge mean pool", lambda: layers._PoolWindows.apply(x.features, plan, True), 4 * D * (N + M), 1),
+        ("torch roll + partition (reference form)", torch_partition, 24 * N, 0),
+        ("torch index_add mean pool", torch_pool, 4 * D * (N + M), 0),
+    ]
 
 
 # ------------------------------------------------------------------------------------------
@@ -371,9 +407,10 @@ def main():
         table, sizes = kernel_table(wl)
         log(f"{'kernel':36s} {'ms':>9s} {'calls':>5s} {'alg MB':>9s} {'GB/s':>9s} {'% HBM':>7s}")
         summary = {}
-        for path in ("resident", "fused", "operators"):
+        for path in ("resident", "fused", "operators", "stage"):
             rows_ = [r for r in table if r["path"] == path]
-            log(f"-- {path} path, one attention forward+backward --")
+            log(f"-- {path} path, one attention forward+backward --" if path != "stage" else
+                "-- index glue of one stage (window indices, mask, stride-2 merge) --")
             for r in rows_:
                 log(f"{r['kernel']:36s} {r['ms']:9.4f} {r['calls']:5d} {r['algorithmic_bytes'] / 1e6:9.1f} "
                     f"{(r['achieved_gbps'] or 0):9.1f} {100 * (r['frac'] or 0):7.2f}")
@@ -381,7 +418,7 @@ def main():
             alg = sum(r["algorithmic_bytes"] * r["calls"] for r in rows_)
             summary[path] = dict(ms=round(ms_, 4), algorithmic_bytes=alg,
                                  frac=round(alg / ms_ / 1e6 / HBM_PEAK_GBPS, 4))
-            log(f"{path} kernels, one attention fwd+bwd: {ms_:.3f} ms for {alg / 1e6:.1f} MB algorithmic "
+            log(f"{path} kernels, {'one attention fwd+bwd' if path != 'stage' else 'once per stage'}: {ms_:.3f} ms for {alg / 1e6:.1f} MB algorithmic "
                 f"= {alg / ms_ / 1e6:.1f} GB/s = {100 * alg / ms_ / 1e6 / HBM_PEAK_GBPS:.2f}% of HBM peak")
         # the step runs the window-resident path: its slowest kernel is the dominant one
         # (the token plan is a sequence of small launches, not a kernel)

@@ -268,6 +268,43 @@ int sswin_window_attention_backward(int dtype, const int32_t* tasks, int64_t g_c
                                     int64_t dv_stride, int dv_col0, float* ds_out, int sides,
                                     void* stream);
 
+/* ---- voxel grid glue of a stage (callers of the attention: block and stage level) ---------- */
+
+/* (batch, d, h, w) voxel coordinates -> (window slot, position inside the window) of the grid
+ * shifted cyclically by -shift: pad_sparse_tensor + roll_sparse_tensor + window_partition_sparse
+ * (sparse_swin/swin3d_base.py:501-554, 336-372) in one pass.  coords: device int32 [N,4]
+ * (16-byte aligned); dims: host int32[3] padded extents (multiples of window); window, shift: host
+ * int32[3], 0 <= shift < extent; indices: device int32 [N,2].  window slot =
+ * ((batch*nd + wz)*nh + wy)*nw + wx.  With window = {2,2,2} and no shift the result is (merged
+ * voxel, child slot) of the floor(coord/2) down-sampling between stages.  Asynchronous. */
+int sswin_window_indices(const int32_t* coords, int64_t N, int batch_size, const int32_t* dims,
+                         const int32_t* window, const int32_t* shift, int32_t* indices,
+                         void* stream);
+
+/* Region ids of the shifted-window attention mask, int8 [windows per batch item, positions]:
+ * compute_mask (swin3d_base.py:416-452: 27 slice assignments into a dense volume, then
+ * window_partition) evaluated per element.  A shift of 0 along an axis gives region 2 on that
+ * axis, as the reference's slices do.  Asynchronous. */
+int sswin_shift_mask(const int32_t* dims, const int32_t* window, const int32_t* shift, int8_t* mask,
+                     void* stream);
+
+/* (batch, wz, wy, wx) of the M non-empty windows of a token plan made with H = 1, in plan order
+ * (ascending window slot): the output coordinates of the stride-2 down-sampling
+ * (swin3d_base.py:950-976, spconv SparseConv3d kernel 2 stride 2: out = floor(coord/2), deduped).
+ * coords_out: device int32 [M,4], 16-byte aligned.  Asynchronous. */
+int sswin_window_coords(const int32_t* plan, int64_t g_cap, int64_t M, const int32_t* dims,
+                        const int32_t* window, int32_t* coords_out, void* stream);
+
+/* Rows of the voxels of each non-empty window reduced to one row, in (window, position) order and
+ * therefore in a fixed order without atomics: dst[m] = sum (mean != 0: average) of src[voxel] over
+ * the voxels of window m (plan / tokens from sswin_token_plan with H = 1).  backward != 0 is the
+ * gradient: src = [M, C] gradient of the pooled rows, dst[voxel] = src[m] (/ count).  C a multiple of
+ * 4; src, dst dense rows of `dtype` with the given strides.  Stands where the reference uses the
+ * strided sparse convolution between stages (swin3d_base.py:950-976).  Asynchronous. */
+int sswin_pool_windows(int dtype, int backward, int mean, const int32_t* plan, int64_t g_cap,
+                       int64_t M, const int32_t* tokens, int64_t N, const void* src,
+                       int64_t src_stride, int C, void* dst, int64_t dst_stride, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -36,7 +36,8 @@ class TokenPlan:
     work enqueued afterwards (the qkv projection) overlaps the host round trip, and
     :meth:`finish` waits for the totals when they are needed."""
 
-    def __init__(self, indices: torch.Tensor, batch_size: int, n: int, num_heads: int, defer: bool = False):
+    def __init__(self, indices: torch.Tensor, batch_size: int, n: int, num_heads: int, defer: bool = False,
+                 tasks: bool = True):
         lib = _lib.load()
         if indices.device.type != "cuda":
             raise RuntimeError("TokenPlan runs on the GPU only; there is no CPU fallback")
@@ -50,7 +51,7 @@ class TokenPlan:
         self.tokens = torch.empty(5 * max(N, 1), dtype=torch.int32, device=d)
         self.plan = torch.empty(5 * self.g_cap, dtype=torch.int32, device=d)
         # group descriptors of the window-resident kernels, bucketed by ceil(c / 32)
-        self.tasks = torch.empty(16 * self.g_cap, dtype=torch.int32, device=d)
+        self.tasks = torch.empty(16 * self.g_cap, dtype=torch.int32, device=d) if tasks else None
         self.device = d
         self._totals = torch.zeros(9, dtype=torch.int64, pin_memory=True)
         self._indices = indices                      # kept alive until the kernels have run

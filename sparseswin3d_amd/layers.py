@@ -9,12 +9,31 @@ torch modules; the attention itself runs in the HIP operators.
 """
 from __future__ import annotations
 
+import copy
+import ctypes as C
 from typing import List, Sequence
 
 import torch
 import torch.nn as nn
+from torch.autograd import Function
+from torch.autograd.function import once_differentiable
 
+from . import _lib
 from .window_attention import WindowAttentionSparse, replace_feature
+
+_DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+
+def _ptr(t):
+    return C.c_void_p(t.data_ptr()) if t is not None else None
+
+
+def _i32x3(v):
+    return (C.c_int32 * 3)(*(int(e) for e in v))
+
+
+def _stream(device):
+    return C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
 
 
 def get_window_size(x_size, window_size, shift_size=None):
@@ -97,16 +116,111 @@ def window_partition(x: torch.Tensor, window_size: List[int]) -> torch.Tensor:
 
 
 def compute_mask(dims: List[int], window_size: List[int], shift_size: List[int], device) -> torch.Tensor:
-    """int8 [windows, tokens per window] region ids (27 regions) of the shifted grid."""
-    d, h, w = dims
-    img = torch.zeros((1, d, h, w, 1), device=device, dtype=torch.int8)
-    region = 0
-    for sd in (slice(-window_size[0]), slice(-window_size[0], -shift_size[0]), slice(-shift_size[0], None)):
-        for sh in (slice(-window_size[1]), slice(-window_size[1], -shift_size[1]), slice(-shift_size[1], None)):
-            for sw in (slice(-window_size[2]), slice(-window_size[2], -shift_size[2]), slice(-shift_size[2], None)):
-                img[:, sd, sh, sw, :] = region
-                region += 1
-    return window_partition(img, list(window_size)).squeeze(-1)
+    """int8 [windows, tokens per window] region ids (27 regions) of the shifted grid.
+
+    The reference assigns 27 slices of a dense volume and partitions it (ref ``:416-452``);
+    here one kernel evaluates the region of every (window, position) directly."""
+    device = torch.device(device)
+    if device.type != "cuda":
+        raise RuntimeError("compute_mask runs on the GPU only; there is no CPU fallback")
+    windows = 1
+    for extent, w in zip(dims, window_size):
+        windows *= extent // w
+    n = window_size[0] * window_size[1] * window_size[2]
+    mask = torch.empty((windows, n), dtype=torch.int8, device=device)
+    with torch.cuda.device(device):
+        _lib.check(_lib.load().sswin_shift_mask(_i32x3(dims), _i32x3(window_size), _i32x3(shift_size), _ptr(mask),
+                                                _stream(device)))
+    return mask
+
+
+def sparse_window_indices(indices: torch.Tensor, batch_size: int, dims: Sequence[int], window_size: Sequence[int],
+                          shift_size: Sequence[int] = (0, 0, 0)) -> torch.Tensor:
+    """int32 [N, 4] (batch, d, h, w) -> int32 [N, 2] (window slot, position) of the grid of
+    padded extents ``dims`` rolled by ``-shift_size``: :func:`pad_sparse_tensor` (trailing pads),
+    :func:`roll_sparse_tensor` and :func:`window_partition_sparse` in one kernel."""
+    if indices.device.type != "cuda":
+        raise RuntimeError("sparse_window_indices runs on the GPU only; there is no CPU fallback")
+    if indices.dtype != torch.int32 or indices.dim() != 2 or indices.shape[1] != 4:
+        raise RuntimeError("sparse_window_indices: indices must be int32 [N, 4]")
+    indices = indices.contiguous()
+    out = torch.empty((indices.shape[0], 2), dtype=torch.int32, device=indices.device)
+    with torch.cuda.device(indices.device):
+        _lib.check(_lib.load().sswin_window_indices(_ptr(indices), indices.shape[0], int(batch_size), _i32x3(dims),
+                                                    _i32x3(window_size), _i32x3(shift_size), _ptr(out),
+                                                    _stream(indices.device)))
+    return out
+
+
+class _PoolWindows(Function):
+    """Sum or mean of the feature rows of every non-empty window, in (window, position) order."""
+
+    @staticmethod
+    def forward(ctx, features, plan, mean):
+        features = features.contiguous()
+        M, channels = plan.windows, features.shape[1]
+        out = torch.empty((M, channels), dtype=features.dtype, device=features.device)
+        with torch.cuda.device(features.device):
+            _lib.check(_lib.load().sswin_pool_windows(
+                _DTYPE_CODE[features.dtype], 0, 1 if mean else 0, _ptr(plan.plan), plan.g_cap, M, _ptr(plan.tokens),
+                plan.N, _ptr(features), channels, channels, _ptr(out), channels, _stream(features.device)))
+        ctx.plan, ctx.mean = plan, mean
+        return out
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad):
+        plan = ctx.plan
+        grad = grad.contiguous()
+        channels = grad.shape[1]
+        g_in = torch.empty((plan.N, channels), dtype=grad.dtype, device=grad.device)
+        with torch.cuda.device(grad.device):
+            _lib.check(_lib.load().sswin_pool_windows(
+                _DTYPE_CODE[grad.dtype], 1, 1 if ctx.mean else 0, _ptr(plan.plan), plan.g_cap, plan.windows,
+                _ptr(plan.tokens), plan.N, _ptr(grad), channels, channels, _ptr(g_in), channels, _stream(grad.device)))
+        return g_in, None, None
+
+
+def downsample_plan(x, factor: int = 2):
+    """Token plan of the ``floor(coord / factor)`` merge: windows of ``factor``^3 cells, one head.
+    Returns ``(plan, merged coordinates int32 [M, 4], merged spatial shape)``."""
+    from .fused import TokenPlan
+    f = int(factor)
+    dims = [-(-int(e) // f) * f for e in x.spatial_shape]
+    win = (f, f, f)
+    idx = sparse_window_indices(x.indices, x.batch_size, dims, win)
+    slots = x.batch_size * (dims[0] // f) * (dims[1] // f) * (dims[2] // f)
+    plan = TokenPlan(idx, slots, f * f * f, 1, tasks=False)
+    coords = torch.empty((plan.windows, 4), dtype=torch.int32, device=x.indices.device)
+    with torch.cuda.device(coords.device):
+        _lib.check(_lib.load().sswin_window_coords(_ptr(plan.plan), plan.g_cap, plan.windows, _i32x3(dims), _i32x3(win),
+                                                   _ptr(coords), _stream(coords.device)))
+    return plan, coords, [e // f for e in dims]
+
+
+class PoolDownsample(nn.Module):
+    """Stride-2 merge between stages: voxels with the same ``floor(coord / 2)`` become one voxel.
+
+    Stands where the reference builds ``spconv.SparseConv3d(dim, 2*dim, kernel_size=2, stride=2)``
+    (ref ``:950-976``; spconv is not available here): same output coordinates (deduplicated
+    ``floor(coord/2)``, ascending (batch, d, h, w)), the children's rows averaged instead of
+    weighted per tap, then ``norm`` and a bias-free ``Linear(dim, 2*dim)``."""
+
+    def __init__(self, dim: int, norm_layer=nn.LayerNorm, spatial_dims: int = 3, indice_key=None) -> None:
+        super().__init__()
+        if spatial_dims != 3:
+            raise ValueError("PoolDownsample handles three spatial dimensions")
+        self.dim = dim
+        self.norm = norm_layer(dim) if norm_layer is not None else nn.Identity()
+        self.reduction = nn.Linear(dim, 2 * dim, bias=False)
+
+    def forward(self, x):
+        plan, coords, shape = downsample_plan(x, 2)
+        pooled = _PoolWindows.apply(x.features, plan, True)
+        out = copy.copy(x)
+        out.indices, out.spatial_shape = coords, shape
+        out.features = self.reduction(self.norm(pooled))
+        return out
 
 
 _ACTIVATIONS = {"GELU": nn.GELU, "RELU": nn.ReLU, "LEAKYRELU": nn.LeakyReLU, "SILU": nn.SiLU, "SWISH": nn.SiLU,
@@ -180,24 +294,29 @@ class SwinTransformerBlock(nn.Module):
 
     def forward_part1(self, x, mask_matrix):
         x = replace_feature(x, self.norm1(x.features))
-        b, (d, h, w), c = x.batch_size, x.spatial_shape, x.features.shape[-1]
+        d, h, w = x.spatial_shape
         window_size, shift_size = get_window_size((d, h, w), self.window_size, self.shift_size)
-        pad_d1 = (window_size[0] - d % window_size[0]) % window_size[0]
-        pad_b = (window_size[1] - h % window_size[1]) % window_size[1]
-        pad_r = (window_size[2] - w % window_size[2]) % window_size[2]
-        x = pad_sparse_tensor(x, 0, pad_r, 0, pad_b, 0, pad_d1)
-        dims = [b, *x.spatial_shape, c]
         shifted = any(s > 0 for s in shift_size)
-        if shifted:
-            x = roll_sparse_tensor(x, shifts=tuple(-s for s in shift_size), dims=(1, 2, 3))
-        x = window_partition_sparse(x, window_size)
-        x = self.attn(x, mask=mask_matrix if shifted else None)
-        x = window_reverse_sparse(x, dims, window_size)
-        if shifted:
-            x = roll_sparse_tensor(x, shifts=tuple(shift_size), dims=(1, 2, 3))
-        if pad_d1 > 0 or pad_r > 0 or pad_b > 0:
-            x.spatial_shape = [d, h, w]
-        return x
+        # pad (trailing), roll by -shift and partition in one pass; the voxel list itself keeps its
+        # (batch, d, h, w) indices, so the reverse / roll back / un-pad of the reference
+        # (ref :760-771) has nothing left to do.  Blocks of a stage with the same shift share the
+        # window indices and the token plan through ``x.window_cache``.
+        cache = getattr(x, "window_cache", None)
+        key = (tuple(window_size), tuple(shift_size))
+        view = cache.get(key) if cache is not None else None
+        if view is None:
+            dims = [-(-e // ws) * ws for e, ws in zip((d, h, w), window_size)]
+            view = copy.copy(x)
+            view.window_cache = None
+            view.indices = sparse_window_indices(x.indices, x.batch_size, dims, window_size, shift_size)
+            view.spatial_shape = (window_size[0] * window_size[1] * window_size[2],)
+            view.batch_size = x.batch_size * (dims[0] // window_size[0]) * (dims[1] // window_size[1]) * (dims[2] // window_size[2])
+            view.plan_cache = {}
+            if cache is not None:
+                cache[key] = view
+        view = replace_feature(view, x.features)
+        out = self.attn(view, mask=mask_matrix if shifted else None)
+        return replace_feature(x, out.features)
 
     def forward_part2(self, x):
         x = replace_feature(x, self.norm2(x.features))
@@ -241,8 +360,11 @@ class BasicLayer(nn.Module):
         padded = [-(-s // ws) * ws for s, ws in zip((d, h, w), window_size)]
         # The mask is built whenever the layer has a shift; unshifted blocks ignore it.
         attn_mask = compute_mask(padded, window_size, shift_size, x.features.device)
+        x = copy.copy(x)
+        x.window_cache = {}                      # (window, shift) -> window indices and token plans of this stage
         for blk in self.blocks:
             x = blk(x, attn_mask)
+        x.window_cache = None
         if self.downsample is not None:
             x = self.downsample(x)
         return x

@@ -394,8 +394,14 @@ class WindowAttentionSparse(nn.Module):
         if self.fused:
             from . import fused
             if fused.supports(x.features, n):
-                # the token plan is enqueued first; the projection below runs while its totals travel
-                plan = fused.TokenPlan(x.indices, b, n, self.num_heads, defer=True)
+                # the token plan is enqueued first; the projection below runs while its totals travel.
+                # A stage hands the same window indices to several blocks: they share one plan.
+                cache = getattr(x, "plan_cache", None)
+                plan = cache.get(self.num_heads) if cache is not None else None
+                if plan is None:
+                    plan = fused.TokenPlan(x.indices, b, n, self.num_heads, defer=True)
+                    if cache is not None:
+                        cache[self.num_heads] = plan
         qkv = tall_linear(x.features, self.qkv).reshape(-1, 3, self.num_heads, c // self.num_heads)
         if plan is not None:
             resident = fused.supports_resident(qkv, n) if self.resident is None else self.resident

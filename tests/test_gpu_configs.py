@@ -243,6 +243,12 @@ def test_cfg5_four_stage_encoder_bf16_forward():
         idx, nw, n = synth.window_indices(coords, shape, (5, 5, 5), (2, 2, 2))
         B = nw * w.batch_size
         mask = synth.shift_region_mask(synth.padded_shape(shape, (5, 5, 5)), (5, 5, 5), (2, 2, 2))
+        # the same indices and mask from the grid kernels, at the stage's full size
+        from sparseswin3d_amd.layers import compute_mask, sparse_window_indices
+        pdims = synth.padded_shape(shape, (5, 5, 5))
+        np.testing.assert_array_equal(
+            sparse_window_indices(torch.from_numpy(coords).cuda(), w.batch_size, pdims, (5, 5, 5), (2, 2, 2)).cpu().numpy(), idx)
+        np.testing.assert_array_equal(compute_mask(list(pdims), [5, 5, 5], [2, 2, 2], "cuda").cpu().numpy(), mask)
         attn = _attention(dim, H, torch.bfloat16, seed=10 + stage)
         set_path(attn, "resident")
         out, _ = _gpu(attn, feats, idx, B, n, mask)
@@ -260,22 +266,20 @@ def test_cfg5_four_stage_encoder_bf16_forward():
             assert stage == 0
         if stage == 3:
             break
-        # between stages: merge voxels by floor(coord/2), average their features, widen channels
-        merged, inverse = synth.downsample_coords(coords[:, 1:], 2)          # batch-blind: redo per room
-        rooms, inv_all, base = [], np.empty(len(coords), np.int64), 0
-        for b in range(w.batch_size):
-            sel = np.nonzero(coords[:, 0] == b)[0]
-            m, inv = synth.downsample_coords(coords[sel, 1:], 2)
-            rooms.append(m)
-            inv_all[sel] = inv + base
-            base += len(m)
-        new_coords, _ = synth.with_batch(rooms)
-        pooled = torch.zeros(base, dim, dtype=torch.float32, device="cuda")
-        pooled.index_add_(0, torch.from_numpy(inv_all).cuda(), out.float())
-        cnt = torch.bincount(torch.from_numpy(inv_all).cuda(), minlength=base).clamp_(min=1)
-        pooled = pooled / cnt[:, None]
-        np.testing.assert_allclose(pooled.cpu().numpy(), synth.mean_pool(out.float().cpu().numpy(), inv_all, base),
-                                   rtol=1e-5, atol=1e-6)
+        # between stages: merge voxels by floor(coord/2), average their features, widen channels;
+        # the merge runs on the GPU (window indices of 2x2x2 cells -> token plan -> pooling kernel)
+        # and is checked against the CPU restatement at full size
+        from oracle import grid as og
+        from sparseswin3d_amd.layers import _PoolWindows, downsample_plan
+        from sparseswin3d_amd.window_attention import SparseVoxelTensor
+        xs = SparseVoxelTensor(out.float(), torch.from_numpy(coords).cuda(), shape, w.batch_size)
+        plan, new_coords_d, new_shape = downsample_plan(xs, 2)
+        pooled = _PoolWindows.apply(xs.features, plan, True)
+        ref_coords, ref_pooled, _ = og.downsample(coords, out.float().cpu().numpy())
+        new_coords = new_coords_d.cpu().numpy()
+        np.testing.assert_array_equal(new_coords, ref_coords)
+        np.testing.assert_allclose(pooled.cpu().numpy(), ref_pooled, rtol=1e-5, atol=1e-6)
+        assert tuple(new_shape) == tuple((s_ + 1) // 2 for s_ in shape)
         feats = torch.cat([pooled, pooled], 1).to(torch.bfloat16).cpu()       # dim -> 2*dim
         coords = new_coords
         shape = tuple((s + 1) // 2 for s in shape)

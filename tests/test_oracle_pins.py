@@ -286,12 +286,73 @@ def test_cpu_path_equals_dense_window_attention():
         np.testing.assert_allclose(a.numpy(), b.numpy(), rtol=1e-10, atol=1e-12)
 
 
-def test_shift_mask_matches_dense_swin_construction():
+def _region_brute_force(dims, ws, ss):
+    """Region of every cell of the shifted grid, one cell at a time: along each axis the three
+    slices [:-ws], [-ws:-s], [-s:] are applied in this order and the last one that holds the
+    coordinate wins (Python slice semantics: s == 0 makes the middle slice empty and the last
+    one the whole axis)."""
+    def axis(v, extent, w, s):
+        r = None
+        for k, sl in enumerate((slice(-w), slice(-w, -s), slice(-s, None))):
+            if v in range(extent)[sl]:
+                r = k
+        return r
+    nd, nh, nw = (dims[a] // ws[a] for a in range(3))
+    out = np.zeros((nd * nh * nw, ws[0] * ws[1] * ws[2]), np.int8)
+    for z in range(dims[0]):
+        for y in range(dims[1]):
+            for x in range(dims[2]):
+                win = ((z // ws[0]) * nh + y // ws[1]) * nw + x // ws[2]
+                pos = ((z % ws[0]) * ws[1] + y % ws[1]) * ws[2] + x % ws[2]
+                out[win, pos] = 9 * axis(z, dims[0], ws[0], ss[0]) + 3 * axis(y, dims[1], ws[1], ss[1]) \
+                    + axis(x, dims[2], ws[2], ss[2])
+    return out
+
+
+@pytest.mark.parametrize("dims,ws,ss", [((15, 10, 20), (5, 5, 5), (2, 2, 2)), ((6, 8, 4), (3, 4, 2), (1, 2, 1)),
+                                        ((5, 10, 5), (5, 5, 5), (0, 2, 0)), ((4, 4, 4), (2, 2, 2), (0, 0, 0))])
+def test_shift_mask_matches_cell_by_cell_construction(dims, ws, ss):
+    from oracle import grid
     from sparseswin3d_amd import synth
-    from sparseswin3d_amd.layers import compute_mask
-    m = compute_mask([15, 10, 20], [5, 5, 5], [2, 2, 2], "cpu").numpy()
-    np.testing.assert_array_equal(m, synth.shift_region_mask((15, 10, 20), (5, 5, 5), (2, 2, 2)))
-    assert m.shape == (3 * 2 * 4, 125) and m.max() == 26
+    ref = _region_brute_force(dims, ws, ss)
+    np.testing.assert_array_equal(grid.shift_mask(dims, ws, ss), ref)
+    np.testing.assert_array_equal(synth.shift_region_mask(dims, ws, ss), ref)
+    if all(ss) and all(d > w for d, w in zip(dims, ws)):
+        assert ref.max() == 26
+
+
+def test_oracle_window_indices_match_dense_roll_and_partition():
+    """The step-by-step pad / roll / partition of the oracle against torch.roll + reshape on a
+    dense volume of voxel ids, with a grid that needs padding and two batch items."""
+    from oracle import grid as og
+    grid, ws, shift = (9, 13, 5), (5, 5, 5), (2, 2, 2)
+    padded = (10, 15, 5)
+    vol = torch.arange(2 * int(np.prod(padded))).reshape(2, *padded)
+    rolled = torch.roll(vol, shifts=tuple(-s for s in shift), dims=(1, 2, 3))
+    parts = rolled.reshape(2, 2, 5, 3, 5, 1, 5).permute(0, 1, 3, 5, 2, 4, 6).reshape(-1, 125)   # [window, pos] -> id
+    bb, zz, yy, xx = np.meshgrid(np.arange(2), *[np.arange(g) for g in grid], indexing="ij")
+    c4 = np.stack([bb.ravel(), zz.ravel(), yy.ravel(), xx.ravel()], 1).astype(np.int32)
+    idx, nw, n = og.window_indices(c4, grid, ws, shift)
+    assert (nw, n) == (6, 125)
+    vox_id = ((c4[:, 0] * padded[0] + c4[:, 1]) * padded[1] + c4[:, 2]) * padded[2] + c4[:, 3]
+    np.testing.assert_array_equal(parts.numpy()[idx[:, 0], idx[:, 1]], vox_id)
+
+
+def test_oracle_downsample_against_dictionary_brute_force():
+    from oracle import grid as og
+    rng = np.random.default_rng(8)
+    c4 = np.unique(np.stack([rng.integers(0, 2, 400), rng.integers(0, 9, 400), rng.integers(0, 7, 400),
+                             rng.integers(0, 11, 400)], 1), axis=0).astype(np.int32)
+    c4 = c4[rng.permutation(len(c4))]
+    f = rng.standard_normal((len(c4), 8))
+    coords, pooled, inverse = og.downsample(c4, f)
+    cells = {}
+    for row, feat in zip(c4, f):
+        cells.setdefault((row[0], row[1] // 2, row[2] // 2, row[3] // 2), []).append(feat)
+    keys = sorted(cells)
+    np.testing.assert_array_equal(coords, np.array(keys, np.int32))
+    np.testing.assert_allclose(pooled, np.stack([np.mean(cells[k], 0) for k in keys]), rtol=1e-12)
+    assert all(tuple(coords[inverse[i]]) == (c4[i, 0], c4[i, 1] // 2, c4[i, 2] // 2, c4[i, 3] // 2) for i in range(len(c4)))
 
 
 def test_window_indices_match_dense_roll_and_partition():
