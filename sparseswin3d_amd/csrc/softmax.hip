@@ -16,6 +16,7 @@ namespace sswin {
 constexpr int SM_THREADS = 256;
 constexpr int SM_TILE = 2048;
 constexpr int SM_ROUNDS = SM_TILE / SM_THREADS;   // 8 ballot rounds of 64 per wave
+constexpr int VEC_PAD = 4;
 
 __device__ __forceinline__ float exp_t(float x) { return expf(x); }
 __device__ __forceinline__ double exp_t(double x) { return exp(x); }
@@ -27,8 +28,8 @@ __global__ __launch_bounds__(SM_THREADS) void softmax_rows_kernel(const int32_t*
                                                                   const T* __restrict__ v,   // values (fwd) / y (bwd)
                                                                   const T* __restrict__ g,   // upstream grad (bwd)
                                                                   int64_t A, T* __restrict__ out) {
-    __shared__ T val_s[SM_TILE];
-    __shared__ T g_s[BWD ? SM_TILE : 1];
+    __shared__ __attribute__((aligned(16))) T val_s[SM_TILE];
+    __shared__ __attribute__((aligned(16))) T g_s[BWD ? SM_TILE : VEC_PAD];
     __shared__ int rid_s[SM_TILE + 1];      // rid_s[e + 1] = id of tile element e; rid_s[0] = predecessor
     __shared__ int start_s[SM_TILE + 1];
     __shared__ int wave_cnt_s[SM_THREADS / 64];
@@ -37,14 +38,33 @@ __global__ __launch_bounds__(SM_THREADS) void softmax_rows_kernel(const int32_t*
     const int64_t tile_base = (int64_t)blockIdx.x * SM_TILE;
     const int tile_n = (int)((A - tile_base) < SM_TILE ? (A - tile_base) : SM_TILE);
 
-    // 1. stage the tile
+    // 1. stage the tile: 16-byte loads for a whole tile (tile_base is a multiple of the tile and
+    // the arrays are 16-byte aligned; the host checks), element loads for the last, partial tile
+    constexpr int VEC = 16 / (int)sizeof(T);                 // values per 16 bytes
+    typedef T vec_t __attribute__((ext_vector_type(VEC)));
+    typedef int ivec_t __attribute__((ext_vector_type(4)));
+    if (tile_n == SM_TILE) {
 #pragma unroll
-    for (int j = 0; j < SM_ROUNDS; ++j) {
-        const int e = j * SM_THREADS + tid;
-        if (e < tile_n) {
-            val_s[e] = v[tile_base + e];
-            rid_s[e + 1] = idx_row[tile_base + e];
-            if (BWD) g_s[e] = g[tile_base + e];
+        for (int j = 0; j < SM_TILE / (SM_THREADS * VEC); ++j) {
+            const int e = (j * SM_THREADS + tid) * VEC;
+            *reinterpret_cast<vec_t*>(val_s + e) = *reinterpret_cast<const vec_t*>(v + tile_base + e);
+            if (BWD) *reinterpret_cast<vec_t*>(g_s + e) = *reinterpret_cast<const vec_t*>(g + tile_base + e);
+        }
+#pragma unroll
+        for (int j = 0; j < SM_TILE / (SM_THREADS * 4); ++j) {
+            const int e = (j * SM_THREADS + tid) * 4;
+            const ivec_t r = *reinterpret_cast<const ivec_t*>(idx_row + tile_base + e);
+            rid_s[e + 1] = r.x; rid_s[e + 2] = r.y; rid_s[e + 3] = r.z; rid_s[e + 4] = r.w;
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < SM_ROUNDS; ++j) {
+            const int e = j * SM_THREADS + tid;
+            if (e < tile_n) {
+                val_s[e] = v[tile_base + e];
+                rid_s[e + 1] = idx_row[tile_base + e];
+                if (BWD) g_s[e] = g[tile_base + e];
+            }
         }
     }
     if (tid == 0) rid_s[0] = tile_base > 0 ? idx_row[tile_base - 1] : idx_row[0] - 1;
@@ -108,7 +128,7 @@ __global__ __launch_bounds__(SM_THREADS) void softmax_rows_kernel(const int32_t*
             }
             for (int64_t p = tile_end + l; p < ext_end; p += 16) sum += exp_t(v[p] - m);
             sum = row16_sum(sum) + (T)1e-8;
-            for (int e = s + l; e < e_end; e += 16) out[tile_base + e] = val_s[e] / sum;
+            for (int e = s + l; e < e_end; e += 16) val_s[e] = val_s[e] / sum;
             for (int64_t p = tile_end + l; p < ext_end; p += 16) out[p] = exp_t(v[p] - m) / sum;
         } else {
             T dot = 0;
@@ -117,12 +137,28 @@ __global__ __launch_bounds__(SM_THREADS) void softmax_rows_kernel(const int32_t*
             dot = row16_sum(dot);
             for (int e = s + l; e < e_end; e += 16) {
                 const T y = val_s[e];
-                out[tile_base + e] = g_s[e] * y - y * dot;
+                val_s[e] = g_s[e] * y - y * dot;
             }
             for (int64_t p = tile_end + l; p < ext_end; p += 16) {
                 const T y = v[p];
                 out[p] = g[p] * y - y * dot;
             }
+        }
+    }
+    // 4. the tile's results leave LDS with 16-byte stores.  Elements before the first row start
+    // belong to a row of an earlier workgroup, which writes them itself.
+    __syncthreads();
+    if (nrows == 0) return;
+    const int s0 = start_s[0];
+#pragma unroll
+    for (int j = 0; j < SM_TILE / (SM_THREADS * VEC); ++j) {
+        const int e = (j * SM_THREADS + tid) * VEC;
+        if (e >= s0 && e + VEC <= tile_n) {
+            *reinterpret_cast<vec_t*>(out + tile_base + e) = *reinterpret_cast<const vec_t*>(val_s + e);
+        } else {
+#pragma unroll
+            for (int k = 0; k < VEC; ++k)
+                if (e + k >= s0 && e + k < tile_n) out[tile_base + e + k] = val_s[e + k];
         }
     }
 }
@@ -147,6 +183,7 @@ int sswin_softmax_last_dim_forward(const int32_t* idx_row, const void* values, i
     SSWIN_CHECK(A >= 0, "softmax forward: negative length");
     if (A == 0) return 0;
     SSWIN_CHECK(idx_row && values && out, "softmax forward: null pointer");
+    SSWIN_CHECK(((uintptr_t)idx_row | (uintptr_t)values | (uintptr_t)out) % 16 == 0, "softmax forward: arrays must be 16-byte aligned");
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == SSWIN_F32) return launch_softmax<float, false>(idx_row, values, nullptr, A, out, s);
     if (dtype == SSWIN_F64) return launch_softmax<double, false>(idx_row, values, nullptr, A, out, s);
@@ -158,6 +195,8 @@ int sswin_softmax_last_dim_backward(const int32_t* idx_row, const void* y, const
     SSWIN_CHECK(A >= 0, "softmax backward: negative length");
     if (A == 0) return 0;
     SSWIN_CHECK(idx_row && y && grad && out, "softmax backward: null pointer");
+    SSWIN_CHECK(((uintptr_t)idx_row | (uintptr_t)y | (uintptr_t)grad | (uintptr_t)out) % 16 == 0,
+                "softmax backward: arrays must be 16-byte aligned");
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (dtype == SSWIN_F32) return launch_softmax<float, true>(idx_row, y, grad, A, out, s);
     if (dtype == SSWIN_F64) return launch_softmax<double, true>(idx_row, y, grad, A, out, s);

@@ -377,7 +377,11 @@ def _softmax_args(indices, *vals):
     _check(dtype in (torch.float32, torch.float64, torch.float16, torch.bfloat16),
            f"softmax: unsupported dtype {dtype}")
     work = dtype if dtype in (torch.float32, torch.float64) else torch.float32
-    return d, dtype, work, indices.contiguous(), [v.contiguous().to(work) for v in vals]
+    def aligned(t):
+        # the kernels move 16 bytes at a time: a view that starts inside an allocation is copied
+        t = t.contiguous()
+        return t if t.data_ptr() % 16 == 0 else t.clone()
+    return d, dtype, work, aligned(indices), [aligned(v.to(work)) for v in vals]
 
 
 def softmax_last_dim_forward(indices, values):

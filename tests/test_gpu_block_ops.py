@@ -189,6 +189,19 @@ def test_softmax_all_negative_rows_keep_zero_max(ops, oracle):
     assert abs(y[4:8].sum() - 1.0) > 1e-6          # the 1e-8 term is visible for exp(-30)-sized sums
 
 
+def test_softmax_views_inside_an_allocation(ops, oracle):
+    """Row ids and values that start 4 bytes into their allocations (the kernels use 16-byte moves)."""
+    rng = np.random.default_rng(21)
+    rows = _rows([5, 1, 2047, 40, 3000])
+    v = rng.standard_normal(len(rows) + 1).astype(np.float32)
+    rows_d = dev(np.concatenate([[0], rows]).astype(np.int32))[1:]
+    y = ops.softmax_last_dim_forward(rows_d, dev(v)[1:])
+    close(host(y), oracle.softmax_last_dim_forward(rows, v[1:].astype(np.float64)), 1e-5, "views fwd")
+    g = rng.standard_normal(len(rows) + 1).astype(np.float32)
+    gx = ops.softmax_last_dim_backward(rows_d, y, dev(g)[1:])
+    close(host(gx), oracle.softmax_last_dim_backward(rows, host(y), g[1:].astype(np.float64)), 1e-5, "views bwd")
+
+
 def test_softmax_deterministic(ops):
     rng = np.random.default_rng(0)
     rows = dev(_rows([37] * 5000))
