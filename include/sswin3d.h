@@ -226,12 +226,12 @@ int sswin_bias_table_grad(const int32_t* plan, int64_t g_cap, int64_t G, const i
                           int64_t N, int H, int n, const int32_t* code, int offset0, int table_rows,
                           const float* ds, float* d_table, void* ws, size_t ws_bytes, void* stream);
 
-/* Column sums of a dense fp32 [N, P] matrix (P a multiple of 4, at most 1024): the bias gradient
- * of the qkv / proj nn.Linear (swin3d_base.py:606-610; autograd's grad_out.sum(0)).  Fixed
- * summation order.  Asynchronous (N == 0 records a memset). */
+/* Column sums (fp32) of a dense [N, P] matrix of `dtype` (fp32 / fp16 / bf16; P a multiple of 4,
+ * rows contiguous): the bias gradient of the qkv / proj nn.Linear (swin3d_base.py:606-610;
+ * autograd's grad_out.sum(0)).  Fixed summation order.  Asynchronous (N == 0 records a memset). */
 size_t sswin_column_sum_workspace_bytes(int64_t N, int P);
-int sswin_column_sum(const float* x, int64_t N, int P, float* out, void* ws, size_t ws_bytes,
-                     void* stream);
+int sswin_column_sum(const void* x, int dtype, int64_t N, int P, float* out, void* ws,
+                     size_t ws_bytes, void* stream);
 
 /* ---- window-resident attention (whole forward / backward of the attention core) ---------- */
 

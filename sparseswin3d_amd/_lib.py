@@ -45,7 +45,7 @@ SIGNATURES = {
     "sswin_fused_bias_grad_workspace_bytes": (_sz, [_i64, _i32, _i32]),
     "sswin_fused_bias_grad": (_i32, [_vp, _i64, _i64, _vp, _i64, _i32, _i32, _vp, _vp, _vp, _sz, _vp]),
     "sswin_column_sum_workspace_bytes": (_sz, [_i64, _i32]),
-    "sswin_column_sum": (_i32, [_vp, _i64, _i32, _vp, _vp, _sz, _vp]),
+    "sswin_column_sum": (_i32, [_vp, _i32, _i64, _i32, _vp, _vp, _sz, _vp]),
     "sswin_bias_table_grad_workspace_bytes": (_sz, [_i64, _i32, _i32]),
     "sswin_bias_table_grad": (_i32, [_vp, _i64, _i64, _vp, _i64, _i32, _i32, _vp, _i32, _i32, _vp, _vp, _vp, _sz, _vp]),
     "sswin_window_indices": (_i32, [_vp, _i64, _i32, _vp, _vp, _vp, _vp, _vp]),
@@ -61,7 +61,7 @@ SIGNATURES = {
                                                _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i32, _vp]),
 }
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 _lib = None
 
 

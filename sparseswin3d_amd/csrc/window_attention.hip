@@ -36,6 +36,8 @@
 #include <math.h>
 #include <stdint.h>
 
+#include <type_traits>
+
 #include "mfma_block.hpp"
 #include "sswin_common.hpp"
 
@@ -168,6 +170,59 @@ __device__ __forceinline__ void table_get(const uint32_t* tab, int half, uint32_
 __device__ __forceinline__ uint32_t f2u(float v) { return __builtin_bit_cast(uint32_t, v); }
 __device__ __forceinline__ float u2f(uint32_t v) { return __builtin_bit_cast(float, v); }
 __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// ------------------------------------------------------------------------------------------
+// One MFMA product step over the reduction slots a lane holds.  fp32 tokens: one
+// v_mfma_f32_32x32x2_f32 per slot (the lane pair l, l + 32 supplies k = 2 values).  16-bit tokens:
+// the operands are rounded to the token type and eight slots go into one v_mfma_f32_32x32x16
+// (k = 16: eight slots of lanes 0-31, eight of lanes 32-63) - an eighth of the matrix-core
+// passes.  A and B use the same slot -> reduction index mapping, which is all a product needs.
+// ------------------------------------------------------------------------------------------
+template <typename T> struct LowPrec;
+template <> struct LowPrec<__hip_bfloat16> {
+    typedef __bf16 elem;
+    typedef __bf16 vec __attribute__((ext_vector_type(8)));
+    static __device__ __forceinline__ f32x16 mma(vec a, vec b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
+    }
+};
+template <> struct LowPrec<__half> {
+    typedef _Float16 elem;
+    typedef _Float16 vec __attribute__((ext_vector_type(8)));
+    static __device__ __forceinline__ f32x16 mma(vec a, vec b, f32x16 c) {
+        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
+    }
+};
+// eight slots: a[OFF .. OFF + 8) against b[0 .. 8)
+template <typename T, int OFF, typename A, typename B>
+__device__ __forceinline__ void mma_slots8_off(const A& a, const B& b, f32x16& acc) {
+    typename LowPrec<T>::vec va, vb;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        va[i] = (typename LowPrec<T>::elem)a[OFF + i];
+        vb[i] = (typename LowPrec<T>::elem)b[i];
+    }
+    acc = LowPrec<T>::mma(va, vb, acc);
+}
+template <typename T, int OFF, int N, typename A, typename B>
+__device__ __forceinline__ void mma_slots(const A& a, const B& b, f32x16& acc) {
+    if constexpr (std::is_same<T, float>::value) {
+#pragma unroll
+        for (int s = 0; s < N; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[OFF + s], b[OFF + s], acc, 0, 0, 0);
+    } else {
+        static_assert(N % 8 == 0, "16-bit products take eight slots per step");
+#pragma unroll
+        for (int m = 0; m < N / 8; ++m) {
+            typename LowPrec<T>::vec va, vb;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                va[i] = (typename LowPrec<T>::elem)a[OFF + 8 * m + i];
+                vb[i] = (typename LowPrec<T>::elem)b[OFF + 8 * m + i];
+            }
+            acc = LowPrec<T>::mma(va, vb, acc);
+        }
+    }
+}
 
 // ------------------------------------------------------------------------------------------
 // Coalesced token rows.  A head's slice of a token row is 32 channels = CH chunks of 16 bytes
@@ -357,8 +412,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         tile_get_rows(tile_x, l32, half, ka);
         // S^T tile: rows = keys, columns = queries
         f32x16 S = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll
-        for (int s = 0; s < 16; ++s) S = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[s], qb[s], S, 0, 0, 0);
+        mma_slots<T, 0, 16>(ka, qb, S);
         uint32_t pkr[16];
         table_get(tab_key, half, pkr);
         float bv[16];
@@ -390,11 +444,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             for (int r = 0; r < 16; ++r) o[r] *= u2f(ar[r]);
         }
         m = mt;
+        if constexpr (std::is_same<T, float>::value) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            const float e = exp2_fast(S[r] - m);
-            l += e;
-            o = __builtin_amdgcn_mfma_f32_32x32x2f32(e, vb[r], o, 0, 0, 0);
+            for (int r = 0; r < 16; ++r) {
+                const float e = exp2_fast(S[r] - m);
+                l += e;
+                o = __builtin_amdgcn_mfma_f32_32x32x2f32(e, vb[r], o, 0, 0, 0);
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                S[r] = exp2_fast(S[r] - m);
+                l += S[r];
+            }
+            mma_slots<T, 0, 16>(S, vb, o);
         }
     }
     l += __shfl_xor(l, 32, 64);
@@ -497,10 +560,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             bv[r] = *reinterpret_cast<const float*>(bias_h + (brow + (MASK ? (pkr[r] & 0xffffu) : pkr[r])));
         f32x16 St = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
         f32x16 dPt = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll
-        for (int s = 0; s < 16; ++s) St = __builtin_amdgcn_mfma_f32_32x32x2f32(ka[s], qb[s], St, 0, 0, 0);
-#pragma unroll
-        for (int s = 0; s < 16; ++s) dPt = __builtin_amdgcn_mfma_f32_32x32x2f32(va[s], dob[s], dPt, 0, 0, 0);
+        mma_slots<T, 0, 16>(ka, qb, St);
+        mma_slots<T, 0, 16>(va, dob, dPt);
         float kb[16];
         tile_get_cols(tile, l32, half, kb);                  // K[key acc_row(r, half)][channel l32]
         const int jlim = c - t * 32 - 4 * half;
@@ -510,8 +571,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             if (MASK && (int)(pkr[r] >> 16) != reg_i) s += -100.0f * LOG2E;
             const float pr = (8 * (r >> 2) + (r & 3)) < jlim ? exp2_fast(s - L2) : 0.f;
             const float ds = pr * (dPt[r] - D);
-            dq = __builtin_amdgcn_mfma_f32_32x32x2f32(ds, kb[r], dq, 0, 0, 0);
+            if constexpr (std::is_same<T, float>::value)
+                dq = __builtin_amdgcn_mfma_f32_32x32x2f32(ds, kb[r], dq, 0, 0, 0);
+            else
+                St[r] = ds;
         }
+        if constexpr (!std::is_same<T, float>::value) mma_slots<T, 0, 16>(St, kb, dq);
     }
 #pragma unroll
     for (int r = 0; r < 16; ++r) dq[r] *= a.scale;
@@ -606,10 +671,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
         tile_get_rows(tile_do, l32, half, doa);
         f32x16 St = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
         f32x16 dPt = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll
-        for (int s = 0; s < 16; ++s) St = __builtin_amdgcn_mfma_f32_32x32x2f32(qa[s], kb[s], St, 0, 0, 0);
-#pragma unroll
-        for (int s = 0; s < 16; ++s) dPt = __builtin_amdgcn_mfma_f32_32x32x2f32(doa[s], vb[s], dPt, 0, 0, 0);
+        mma_slots<T, 0, 16>(qa, kb, St);
+        mma_slots<T, 0, 16>(doa, vb, dPt);
 
         // P and dS of the tile: rows = queries acc_row(r, half), column = this lane's key.
         // The bias gathers of all 16 rows are issued first; everything else is fetched from
@@ -629,6 +692,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
         const u32x4_a* D4 = reinterpret_cast<const u32x4_a*>(tab_D + 4 * half);
         const float* do_col = tile_do + 4 * half * TILE_LD + l32;
         const float* q_col = tile_q + 4 * half * TILE_LD + l32;
+        float dob8[8], qbr8[8];                              // 16-bit tokens: operands of eight slots
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
             const u32x4_a Lq = L4[2 * q], Dq = D4[2 * q];
@@ -648,8 +712,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
                 const float ds = pr * (dPt[r] - u2f(Dr[k]));
                 const int row = 8 * q + k;
                 if (ds_t && row < ilim && j_k < c) ds_t[row * c] = ds;
-                dv = __builtin_amdgcn_mfma_f32_32x32x2f32(pr, dob[k], dv, 0, 0, 0);     // dV += P^T dO
-                dk = __builtin_amdgcn_mfma_f32_32x32x2f32(ds, qbr[k], dk, 0, 0, 0);     // dK += dS^T Q
+                if constexpr (std::is_same<T, float>::value) {
+                    dv = __builtin_amdgcn_mfma_f32_32x32x2f32(pr, dob[k], dv, 0, 0, 0);     // dV += P^T dO
+                    dk = __builtin_amdgcn_mfma_f32_32x32x2f32(ds, qbr[k], dk, 0, 0, 0);     // dK += dS^T Q
+                } else {                                     // collected: eight slots per 16-bit step
+                    St[r] = pr;
+                    dPt[r] = ds;
+                    dob8[4 * (q & 1) + k] = dob[k];
+                    qbr8[4 * (q & 1) + k] = qbr[k];
+                }
+            }
+            if constexpr (!std::is_same<T, float>::value) {
+                if (q & 1) {
+                    if (q == 1) {
+                        mma_slots<T, 0, 8>(St, dob8, dv);
+                        mma_slots<T, 0, 8>(dPt, qbr8, dk);
+                    } else {
+                        mma_slots8_off<T, 8>(St, dob8, dv);
+                        mma_slots8_off<T, 8>(dPt, qbr8, dk);
+                    }
+                }
             }
         }
     }

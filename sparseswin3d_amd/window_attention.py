@@ -234,24 +234,27 @@ def _rocblas_gemm():
         torch.backends.cuda.preferred_blas_library(prev)
 
 
+_SUM_DTYPE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+
 def _column_sum(t: torch.Tensor) -> torch.Tensor:
-    """``t.sum(0)`` of a tall [N, P] matrix; fp32 on the GPU goes through the library's two-stage
-    kernel (about twice as fast as the generic reduction on [10^5 x 288], fixed order)."""
-    p = t.shape[1]
-    if not (t.is_cuda and t.dtype == torch.float32 and t.dim() == 2 and p % 4 == 0 and p <= 1024 and t.shape[0] > 0):
+    """``t.sum(0)`` of a tall [N, P] matrix on the GPU through the library's two-stage kernel (sums
+    in fp32, fixed order; about twice as fast as the generic reduction on [10^5 x 288])."""
+    p = t.shape[1] if t.dim() == 2 else 0
+    if not (t.is_cuda and t.dtype in _SUM_DTYPE and t.dim() == 2 and p % 4 == 0 and t.shape[0] > 0):
         return t.sum(0)
     import ctypes as C
     from . import _lib
     lib = _lib.load()
     t = t.contiguous()
     with torch.cuda.device(t.device):
-        out = torch.empty(p, dtype=t.dtype, device=t.device)
+        out = torch.empty(p, dtype=torch.float32, device=t.device)
         nbytes = lib.sswin_column_sum_workspace_bytes(t.shape[0], p)
         ws = torch.empty(int(nbytes), dtype=torch.uint8, device=t.device)
-        _lib.check(lib.sswin_column_sum(C.c_void_p(t.data_ptr()), t.shape[0], p, C.c_void_p(out.data_ptr()),
-                                        C.c_void_p(ws.data_ptr()), nbytes,
+        _lib.check(lib.sswin_column_sum(C.c_void_p(t.data_ptr()), _SUM_DTYPE[t.dtype], t.shape[0], p,
+                                        C.c_void_p(out.data_ptr()), C.c_void_p(ws.data_ptr()), nbytes,
                                         C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)))
-    return out
+    return out.to(t.dtype)
 
 
 class _TallLinear(Function):

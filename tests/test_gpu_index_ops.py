@@ -128,22 +128,26 @@ def test_ops_reject_cpu_tensors(ops):
         ops.flatten_indices(torch.zeros((2, 4), dtype=torch.int32), [3, 3])
 
 
-@pytest.mark.parametrize("N,P", [(1, 96), (7, 288), (1000, 96), (107500, 288), (4099, 4), (5000, 1024)])
-def test_column_sum(N, P):
-    """Bias gradient of the projections: column sums of a tall matrix, fixed order."""
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-5), (torch.bfloat16, 1e-5), (torch.float16, 1e-5)])
+@pytest.mark.parametrize("N,P", [(1, 96), (7, 288), (1000, 96), (107500, 288), (4099, 4), (5000, 1024), (8200, 2304),
+                                 (300, 1100)])
+def test_column_sum(N, P, dtype, tol):
+    """Bias gradient of the projections: column sums of a tall matrix in fp32, fixed order."""
     import ctypes as C
     from sparseswin3d_amd import _lib
     lib = _lib.load()
     g = torch.Generator().manual_seed(N + P)
-    x = torch.randn(N, P, generator=g)
+    x = torch.randn(N, P, generator=g).to(dtype)
     xd = x.cuda()
     out = torch.full((P,), float("nan"), device="cuda")
     nbytes = lib.sswin_column_sum_workspace_bytes(N, P)
     ws = torch.empty(int(nbytes), dtype=torch.uint8, device="cuda")
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    code = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}[dtype]
     for _ in range(2):
-        _lib.check(lib.sswin_column_sum(C.c_void_p(xd.data_ptr()), N, P, C.c_void_p(out.data_ptr()),
+        _lib.check(lib.sswin_column_sum(C.c_void_p(xd.data_ptr()), code, N, P, C.c_void_p(out.data_ptr()),
                                         C.c_void_p(ws.data_ptr()), nbytes, stream))
-    ref = x.double().sum(0).numpy()
+    ref = x.double().sum(0).numpy()                      # the rounded inputs, summed exactly
     got = out.cpu().numpy().astype(np.float64)
-    assert np.all(np.abs(got - ref) <= 1e-5 * (np.abs(ref) + np.abs(x.double()).sum(0).numpy() / max(N, 1) ** 0.5 + 1e-6))
+    scale = np.abs(x.double()).sum(0).numpy() / max(N, 1) ** 0.5
+    assert np.all(np.abs(got - ref) <= tol * (np.abs(ref) + scale + 1e-6))
