@@ -41,8 +41,8 @@ MEASURED_TRAFFIC_BYTES = {
     # profiles/wattn_kernels_cfg2_pmc.txt and profiles/fused_tok_kernel_cfg2_pmc.txt:
     # FETCH_SIZE x 2.0 KiB + WRITE_SIZE x 1.0 KiB per launch
     "resident forward": 174.2e6,
-    "resident backward dQ": 258.0e6,
-    "resident backward dK,dV,dS": 344.5e6,
+    "resident backward dQ, all groups": 258.0e6,
+    "resident backward dK,dV,dS only": 344.5e6,
     "fused dV=P^T dO": 128.1e6,
     "fused dK=dS^T Q": 128.1e6,      # same kernel instantiation and operand shapes as dV
     "fused O=PV": 135.4e6,
@@ -225,9 +225,18 @@ def kernel_table(wl, reps=20, only=None):
                                                       hd, *qa, C.c_float(0.17), ptr(bias), b["n"], mask_p, nmw,
                                                       ptr(out_f), D, 0, ptr(lse), stream))
 
-    def r_bwd(sides):
+    # The step asks for both sides (3): groups of at most 32 tokens then get dQ from the key-side
+    # kernel and the query-side kernel runs for the larger groups only.  6 times that key-side
+    # launch alone; restricted bucket counts time the query-side launch of the larger groups.
+    bc = [int(x) for x in tp.bucket_counts]
+    cg = tp.plan[:tp.G].to(torch.int64)                                  # plan row 0: tokens of each group
+    rows1, rowsL = int(cg[cg <= 32].sum()), int(cg[cg > 32].sum())       # token-head rows of small / large groups
+    only_large = [0, bc[1], bc[2], bc[3]]
+
+    def r_bwd(sides, counts=None):
+        counts = tp.bucket_counts if counts is None else (C.c_int64 * 4)(*counts)
         return lambda: _lib.check(lib.sswin_window_attention_backward(
-            0, ptr(tp.tasks), tp.g_cap, tp.bucket_counts, ptr(tp.tokens), N, H, hd, *qa, C.c_float(0.17), ptr(bias),
+            0, ptr(tp.tasks), tp.g_cap, counts, ptr(tp.tokens), N, H, hd, *qa, C.c_float(0.17), ptr(bias),
             b["n"], mask_p, nmw, ptr(out_f), D, 0, ptr(up_r), D, 0, ptr(lse), *da, ptr(s_f), sides, stream))
 
     from sparseswin3d_amd.window_attention import relative_position_index_3d
@@ -244,8 +253,10 @@ def kernel_table(wl, reps=20, only=None):
     r_entries = [
         ("resident token_plan", lambda: F.TokenPlan(b["idx"], b["slots"], b["n"], H), 28 * N + 36 * tp.G, 1),
         ("resident forward", r_fwd, 16 * E + 4 * H * N, 1),
-        ("resident backward dQ", r_bwd(1), 24 * E + 4 * H * N, 1),
-        ("resident backward dK,dV,dS", r_bwd(2), 28 * E + 4 * A + 4 * H * N, 1),
+        ("resident backward dQ, groups > 32 tokens", r_bwd(1, only_large), (24 * hd + 4) * rowsL, 1 if rowsL else 0),
+        ("resident backward dK,dV,dS + dQ of small groups", r_bwd(6), 28 * E + 4 * A + 4 * H * N + 4 * hd * rows1, 1),
+        ("resident backward dQ, all groups", r_bwd(1), 24 * E + 4 * H * N, 0),
+        ("resident backward dK,dV,dS only", r_bwd(2), 28 * E + 4 * A + 4 * H * N, 0),
         ("resident bias table grad", r_table_grad, 4 * A, 1),
         ("resident bias grad [H,n,n]", lambda: _lib.check(lib.sswin_fused_bias_grad(ptr(tp.plan), tp.g_cap, tp.G, ptr(tp.tokens), tp.N, H, b["n"], ptr(s_f), ptr(dbias), ptr(bg_ws), bg_bytes, stream)), 4 * A, 0),
     ]

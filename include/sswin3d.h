@@ -253,8 +253,10 @@ int sswin_window_attention_forward(int dtype, const int32_t* tasks, int64_t g_ca
 /* Backward of the same (swin3d_base.py:106-138 and :177-188 composed): from O, dO and lse,
  * recomputes P per tile and writes dQ = scale dS K, dK = scale dS^T Q, dV = P^T dO with
  * dS = P (dP - rowsum(dO o O)).  ds_out (fp32 "sq" array in plan order, or NULL) receives dS
- * for sswin_fused_bias_grad.  sides: 1 = dQ only, 2 = dK and dV (and dS) only, 3 = all.
- * Asynchronous. */
+ * for the bias gradient.  sides: 1 = dQ only (query-side kernel), 2 = dK and dV (and dS) only
+ * (key-side kernel), 3 = all: the key-side kernel then also writes dQ of the groups of at most 32
+ * tokens (their dS is already in its registers) and the query-side kernel runs for the larger
+ * groups only; 6 = the key-side launch of 3 alone (for profiling).  Asynchronous. */
 int sswin_window_attention_backward(int dtype, const int32_t* tasks, int64_t g_cap,
                                     const int64_t* bucket_counts, const int32_t* tokens, int64_t N,
                                     int H, int hd, const void* q_base, int64_t q_stride, int q_col0,

@@ -139,6 +139,11 @@ __device__ __forceinline__ uint32_t pack2(float lo, float hi, __hip_bfloat16) {
 constexpr int TILE_LD = 36;
 constexpr int TILE_WORDS = 32 * TILE_LD;
 
+__device__ __forceinline__ void tile_put_rows(float* tile, int l32, int half, const float (&x)[16]) {
+    f32x4_a* p = reinterpret_cast<f32x4_a*>(tile + l32 * TILE_LD + half * 16);
+#pragma unroll
+    for (int v = 0; v < 4; ++v) p[v] = f32x4_a{x[4 * v], x[4 * v + 1], x[4 * v + 2], x[4 * v + 3]};
+}
 __device__ __forceinline__ void tile_get_rows(const float* tile, int l32, int half, float (&x)[16]) {
     const f32x4_a* p = reinterpret_cast<const f32x4_a*>(tile + l32 * TILE_LD + half * 16);
 #pragma unroll
@@ -193,6 +198,35 @@ template <> struct LowPrec<__half> {
         return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
     }
 };
+// the same, starting from the instruction's zero operand instead of a cleared accumulator
+template <typename T, int N, typename A, typename B>
+__device__ __forceinline__ f32x16 mma_slots_first(const A& a, const B& b) {
+    const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    f32x16 acc;
+    if constexpr (std::is_same<T, float>::value) {
+        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[0], b[0], zero, 0, 0, 0);
+#pragma unroll
+        for (int s = 1; s < N; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], acc, 0, 0, 0);
+    } else {
+        typename LowPrec<T>::vec va, vb;
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            va[i] = (typename LowPrec<T>::elem)a[i];
+            vb[i] = (typename LowPrec<T>::elem)b[i];
+        }
+        acc = LowPrec<T>::mma(va, vb, zero);
+#pragma unroll
+        for (int m = 1; m < N / 8; ++m) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                va[i] = (typename LowPrec<T>::elem)a[8 * m + i];
+                vb[i] = (typename LowPrec<T>::elem)b[8 * m + i];
+            }
+            acc = LowPrec<T>::mma(va, vb, acc);
+        }
+    }
+    return acc;
+}
 // eight slots: a[OFF .. OFF + 8) against b[0 .. 8)
 template <typename T, int OFF, typename A, typename B>
 __device__ __forceinline__ void mma_slots8_off(const A& a, const B& b, f32x16& acc) {
@@ -390,9 +424,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 
     float m = 0.f;                                           // the operator's max(0, rowmax)
     float l = 0.f;                                           // this lane half's share of the row sum
-    f32x16 o = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll 1
-    for (int t = 0; t < nt; ++t) {
+    f32x16 o;
+    // one tile of keys.  The first tile is a separate instantiation: its accumulators start from the
+    // instruction's zero operand and nothing has to be rescaled (most groups have one tile only).
+    auto tile_step = [&](auto first_tag, const int t) {
+        constexpr bool FIRST = decltype(first_tag)::value;
         // key side of tile t: lane l32 owns key t*32 + l32
         const int j = t * 32 + l32;
         const int j_c = j < c ? j : c - 1;
@@ -411,8 +447,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         float ka[16];
         tile_get_rows(tile_x, l32, half, ka);
         // S^T tile: rows = keys, columns = queries
-        f32x16 S = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-        mma_slots<T, 0, 16>(ka, qb, S);
+        f32x16 S = mma_slots_first<T, 16>(ka, qb);
         uint32_t pkr[16];
         table_get(tab_key, half, pkr);
         float bv[16];
@@ -433,7 +468,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             mt = fmaxf(mt, s);
         }
         mt = fmaxf(mt, __shfl_xor(mt, 32, 64));
-        if (t > 0) {                                         // rescale what earlier tiles accumulated
+        if constexpr (!FIRST) {                              // rescale what earlier tiles accumulated
             const float alpha = exp2_fast(m - mt);
             l *= alpha;
             table_put(tab_alpha, l32, f2u(alpha));
@@ -444,22 +479,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             for (int r = 0; r < 16; ++r) o[r] *= u2f(ar[r]);
         }
         m = mt;
-        if constexpr (std::is_same<T, float>::value) {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const float e = exp2_fast(S[r] - m);
-                l += e;
-                o = __builtin_amdgcn_mfma_f32_32x32x2f32(e, vb[r], o, 0, 0, 0);
-            }
-        } else {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                S[r] = exp2_fast(S[r] - m);
-                l += S[r];
-            }
-            mma_slots<T, 0, 16>(S, vb, o);
+        for (int r = 0; r < 16; ++r) {
+            S[r] = exp2_fast(S[r] - m);
+            l += S[r];
         }
-    }
+        if constexpr (FIRST)
+            o = mma_slots_first<T, 16>(S, vb);
+        else
+            mma_slots<T, 0, 16>(S, vb, o);
+    };
+    tile_step(std::true_type{}, 0);
+#pragma unroll 1
+    for (int t = 1; t < nt; ++t) tile_step(std::false_type{}, t);
     l += __shfl_xor(l, 32, 64);
     l += 1e-8f;
     if (half == 0 && i_q < c) lse[(int64_t)a.H * g.Tk + h * c + i_q] = (m + __builtin_amdgcn_logf(l)) * LN2;
@@ -589,11 +621,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 // ------------------------------------------------------------------------------------------
 // backward, key side: dK, dV (and dS for the bias gradient)
 // ------------------------------------------------------------------------------------------
-template <typename T, bool MASK>
+// DQ1: groups of one tile also get their dQ here (dS is already in registers; transposed through
+// LDS it is the A operand of dQ = dS K), which saves them the whole query-side kernel
+template <typename T, bool MASK, bool DQ1>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void wattn_bwd_kv_kernel(WAttnCommon a, TokenTensor32 tq, TokenTensor32 tk,
                                                            TokenTensor32 tv, TokenTensor32 to, TokenTensor32 tdo,
                                                            const float* __restrict__ lse, TokenTensor32 tdk,
-                                                           TokenTensor32 tdv, float* __restrict__ ds_out) {
+                                                           TokenTensor32 tdv, float* __restrict__ ds_out,
+                                                           TokenTensor32 tdq) {
     __shared__ __attribute__((aligned(16))) float tiles[4][2][TILE_WORDS];
     __shared__ __attribute__((aligned(16))) uint32_t tabs[4][3][32];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
@@ -715,6 +750,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
                 if constexpr (std::is_same<T, float>::value) {
                     dv = __builtin_amdgcn_mfma_f32_32x32x2f32(pr, dob[k], dv, 0, 0, 0);     // dV += P^T dO
                     dk = __builtin_amdgcn_mfma_f32_32x32x2f32(ds, qbr[k], dk, 0, 0, 0);     // dK += dS^T Q
+                    if (DQ1) dPt[r] = ds;
                 } else {                                     // collected: eight slots per 16-bit step
                     St[r] = pr;
                     dPt[r] = ds;
@@ -733,6 +769,30 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
                     }
                 }
             }
+        }
+        if (DQ1 && nt == 1) {
+            // dS of the only tile (rows = queries by register, column = this lane's key; padding keys
+            // zeroed) -> LDS -> one query row per lane; K rows (still scaled by scale * log2 e) go back
+            // to LDS for the column reads.  dQ = scale dS K = (dS K_scaled) ln 2.
+#pragma unroll
+            for (int r = 0; r < 16; ++r) dPt[r] = j_k < c ? dPt[r] : 0.f;
+            __builtin_amdgcn_wave_barrier();
+            tile_put_acc(tile_do, l32, half, dPt);
+            tile_put_rows(tile_q, l32, half, kb);
+            __builtin_amdgcn_wave_barrier();
+            float dsr[16], kc[16];
+            tile_get_rows(tile_do, l32, half, dsr);              // dS[query l32][keys 16 * half + s]
+            const float* k_col = tile_q + 16 * half * TILE_LD + l32;
+#pragma unroll
+            for (int s = 0; s < 16; ++s) kc[s] = k_col[s * TILE_LD];  // K[key 16 * half + s][channel l32]
+            f32x16 dq = mma_slots_first<T, 16>(dsr, kc);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) dq[r] *= LN2;
+            __builtin_amdgcn_wave_barrier();
+            tile_put_acc(tile_do, l32, half, dq);
+            __builtin_amdgcn_wave_barrier();
+            tile_store_rows<T>(tile_do, const_cast<char*>(head_base<T>(tdq, h)), pitch_of<T>(tdq), vox_j, c, lane);
+            __builtin_amdgcn_wave_barrier();
         }
     }
 #pragma unroll
@@ -767,11 +827,22 @@ static void launch_backward(const WAttnCommon& a, const TokenTensor32& q, const 
                             const TokenTensor32& dq, const TokenTensor32& dk, const TokenTensor32& dv, float* ds_out,
                             int sides, hipStream_t s) {
     const unsigned blocks = (unsigned)((a.first[4] + 3) / 4);
+    if (sides == 3 || sides == 6) {
+        // groups of one tile get dQ from the key-side kernel; the query-side kernel takes the rest
+        WAttnCommon big = a;
+        big.first[4] = a.first[3];
+        const unsigned big_blocks = (unsigned)((big.first[4] + 3) / 4);
+        if (big_blocks && sides == 3)
+            hipLaunchKernelGGL((wattn_bwd_q_kernel<T, MASK>), dim3(big_blocks), dim3(256), 0, s, big, q, k, v, o, d_o, lse, dq);
+        hipLaunchKernelGGL((wattn_bwd_kv_kernel<T, MASK, true>), dim3(blocks), dim3(256), 0, s, a, q, k, v, o, d_o, lse,
+                           dk, dv, ds_out, dq);
+        return;
+    }
     if (sides & 1)
         hipLaunchKernelGGL((wattn_bwd_q_kernel<T, MASK>), dim3(blocks), dim3(256), 0, s, a, q, k, v, o, d_o, lse, dq);
     if (sides & 2)
-        hipLaunchKernelGGL((wattn_bwd_kv_kernel<T, MASK>), dim3(blocks), dim3(256), 0, s, a, q, k, v, o, d_o, lse, dk,
-                           dv, ds_out);
+        hipLaunchKernelGGL((wattn_bwd_kv_kernel<T, MASK, false>), dim3(blocks), dim3(256), 0, s, a, q, k, v, o, d_o, lse,
+                           dk, dv, ds_out, dq);
 }
 
 template <typename T>
@@ -886,9 +957,10 @@ int sswin_window_attention_backward(int dtype, const int32_t* tasks, int64_t g_c
                      n_mask_windows, &total))
         return 1;
     if (total == 0) return 0;
-    SSWIN_CHECK(sides >= 1 && sides <= 3, "window_attention_backward: sides must be 1 (dQ), 2 (dK, dV) or 3");
+    SSWIN_CHECK(sides == 1 || sides == 2 || sides == 3 || sides == 6,
+                "window_attention_backward: sides must be 1 (dQ), 2 (dK, dV), 3 (all) or 6 (key-side kernel of 3)");
     SSWIN_CHECK(q_base && k_base && v_base && o_base && do_base && lse, "window_attention_backward: null pointer");
-    SSWIN_CHECK(!(sides & 1) || dq_base, "window_attention_backward: dq is null");
+    SSWIN_CHECK(!(sides & 5) || dq_base, "window_attention_backward: dq is null");
     SSWIN_CHECK(!(sides & 2) || (dk_base && dv_base), "window_attention_backward: dk or dv is null");
     {
         const char* who = "window_attention_backward";
@@ -898,7 +970,7 @@ int sswin_window_attention_backward(int dtype, const int32_t* tasks, int64_t g_c
             check_tensor(who, "o", o_base, o_stride, o_col0, N, H, dtype) ||
             check_tensor(who, "do", do_base, do_stride, do_col0, N, H, dtype))
             return 1;
-        if ((sides & 1) && check_tensor(who, "dq", dq_base, dq_stride, dq_col0, N, H, dtype)) return 1;
+        if ((sides & 5) && check_tensor(who, "dq", dq_base, dq_stride, dq_col0, N, H, dtype)) return 1;
         if ((sides & 2) && (check_tensor(who, "dk", dk_base, dk_stride, dk_col0, N, H, dtype) ||
                             check_tensor(who, "dv", dv_base, dv_stride, dv_col0, N, H, dtype)))
             return 1;
