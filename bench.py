@@ -225,9 +225,10 @@ def kernel_table(wl, reps=20, only=None):
                                                       hd, *qa, C.c_float(0.17), ptr(bias), b["n"], mask_p, nmw,
                                                       ptr(out_f), D, 0, ptr(lse), stream))
 
-    # The step asks for both sides (3): groups of at most 32 tokens then get dQ from the key-side
-    # kernel and the query-side kernel runs for the larger groups only.  6 times that key-side
-    # launch alone; restricted bucket counts time the query-side launch of the larger groups.
+    # The step asks for all gradients at once (sides = 3): one launch in which groups of at most
+    # 32 tokens get dQ from their key-side task and only the larger groups have query-side tasks.
+    # The parts are timed alone for comparison: 6 = the key-side tasks of that launch, restricted
+    # bucket counts = the query-side kernel on the larger groups, 1 / 2 = the per-side kernels.
     bc = [int(x) for x in tp.bucket_counts]
     cg = tp.plan[:tp.G].to(torch.int64)                                  # plan row 0: tokens of each group
     rows1, rowsL = int(cg[cg <= 32].sum()), int(cg[cg > 32].sum())       # token-head rows of small / large groups
@@ -253,8 +254,9 @@ def kernel_table(wl, reps=20, only=None):
     r_entries = [
         ("resident token_plan", lambda: F.TokenPlan(b["idx"], b["slots"], b["n"], H), 28 * N + 36 * tp.G, 1),
         ("resident forward", r_fwd, 16 * E + 4 * H * N, 1),
-        ("resident backward dQ, groups > 32 tokens", r_bwd(1, only_large), (24 * hd + 4) * rowsL, 1 if rowsL else 0),
-        ("resident backward dK,dV,dS + dQ of small groups", r_bwd(6), 28 * E + 4 * A + 4 * H * N + 4 * hd * rows1, 1),
+        ("resident backward (dQ,dK,dV,dS)", r_bwd(3), 32 * E + 4 * A + 4 * H * N, 1),
+        ("resident backward dQ, groups > 32 tokens", r_bwd(1, only_large), (24 * hd + 4) * rowsL, 0),
+        ("resident backward dK,dV,dS + dQ of small groups", r_bwd(6), 28 * E + 4 * A + 4 * H * N + 4 * hd * rows1, 0),
         ("resident backward dQ, all groups", r_bwd(1), 24 * E + 4 * H * N, 0),
         ("resident backward dK,dV,dS only", r_bwd(2), 28 * E + 4 * A + 4 * H * N, 0),
         ("resident bias table grad", r_table_grad, 4 * A, 1),

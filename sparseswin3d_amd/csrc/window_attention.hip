@@ -511,24 +511,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 // ------------------------------------------------------------------------------------------
 // backward, query side: dQ
 // ------------------------------------------------------------------------------------------
+// One task of the query side on one wavefront.  tile: K of the tile (read back by column); tile_x:
+// rows in transit to the operand layout, then dQ; two 32-entry tables.
 template <typename T, bool MASK>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void wattn_bwd_q_kernel(WAttnCommon a, TokenTensor32 tq, TokenTensor32 tk,
-                                                          TokenTensor32 tv, TokenTensor32 to, TokenTensor32 tdo,
-                                                          const float* __restrict__ lse, TokenTensor32 tdq) {
-    __shared__ __attribute__((aligned(16))) float tiles[4][2][TILE_WORDS];
-    __shared__ __attribute__((aligned(16))) uint32_t tabs[4][2][32];
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+__device__ __forceinline__ void bwd_q_task(const WAttnCommon& a, int64_t task, float* tile, float* tile_x,
+                                           uint32_t* tab_key, uint32_t* tab_D, const TokenTensor32& tq,
+                                           const TokenTensor32& tk, const TokenTensor32& tv, const TokenTensor32& to,
+                                           const TokenTensor32& tdo, const float* __restrict__ lse,
+                                           const TokenTensor32& tdq) {
+    const int lane = threadIdx.x & 63;
     const int half = lane >> 5, l32 = lane & 31;
     int64_t d;
     int bi;
-    if (!locate(a, (int64_t)blockIdx.x * 4 + wave, d, bi)) return;
+    if (!locate(a, task, d, bi)) return;
     const GroupCtx g = load_group(a.tasks, d);
     const int c = g.c, h = g.h;
     const int nt = (c + 31) >> 5;
-    float* tile = tiles[wave][0];                            // K of the tile (read back by column)
-    float* tile_x = tiles[wave][1];                          // rows in transit to the operand layout, dQ
-    uint32_t* tab_key = tabs[wave][0];
-    uint32_t* tab_D = tabs[wave][1];
     const int32_t* order = a.order + g.Tk;
     const int32_t* tok_pos = a.tok_pos + g.Tk;
     const int8_t* mrow = MASK ? a.mask + (int64_t)(g.w % a.nmw) * a.n : nullptr;
@@ -618,32 +616,38 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     tile_store_rows<T>(tile_x, const_cast<char*>(head_base<T>(tdq, h)), pitch_of<T>(tdq), vox_i, c - bi * 32, lane);
 }
 
+template <typename T, bool MASK>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void wattn_bwd_q_kernel(
+    WAttnCommon a, TokenTensor32 tq, TokenTensor32 tk, TokenTensor32 tv, TokenTensor32 to, TokenTensor32 tdo,
+    const float* __restrict__ lse, TokenTensor32 tdq) {
+    __shared__ __attribute__((aligned(16))) float tiles[4][2][TILE_WORDS];
+    __shared__ __attribute__((aligned(16))) uint32_t tabs[4][2][32];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    bwd_q_task<T, MASK>(a, (int64_t)blockIdx.x * 4 + wave, tiles[wave][0], tiles[wave][1], tabs[wave][0], tabs[wave][1],
+                        tq, tk, tv, to, tdo, lse, tdq);
+}
+
 // ------------------------------------------------------------------------------------------
 // backward, key side: dK, dV (and dS for the bias gradient)
 // ------------------------------------------------------------------------------------------
 // DQ1: groups of one tile also get their dQ here (dS is already in registers; transposed through
 // LDS it is the A operand of dQ = dS K), which saves them the whole query-side kernel
 template <typename T, bool MASK, bool DQ1>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void wattn_bwd_kv_kernel(WAttnCommon a, TokenTensor32 tq, TokenTensor32 tk,
-                                                           TokenTensor32 tv, TokenTensor32 to, TokenTensor32 tdo,
-                                                           const float* __restrict__ lse, TokenTensor32 tdk,
-                                                           TokenTensor32 tdv, float* __restrict__ ds_out,
-                                                           TokenTensor32 tdq) {
-    __shared__ __attribute__((aligned(16))) float tiles[4][2][TILE_WORDS];
-    __shared__ __attribute__((aligned(16))) uint32_t tabs[4][3][32];
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+__device__ __forceinline__ void bwd_kv_task(const WAttnCommon& a, int64_t task, float* tile_q, float* tile_do,
+                                            uint32_t* tab_pos, uint32_t* tab_L, uint32_t* tab_D,
+                                            const TokenTensor32& tq, const TokenTensor32& tk, const TokenTensor32& tv,
+                                            const TokenTensor32& to, const TokenTensor32& tdo,
+                                            const float* __restrict__ lse, const TokenTensor32& tdk,
+                                            const TokenTensor32& tdv, float* __restrict__ ds_out,
+                                            const TokenTensor32& tdq) {
+    const int lane = threadIdx.x & 63;
     const int half = lane >> 5, l32 = lane & 31;
     int64_t d;
     int bj;
-    if (!locate(a, (int64_t)blockIdx.x * 4 + wave, d, bj)) return;
+    if (!locate(a, task, d, bj)) return;
     const GroupCtx g = load_group(a.tasks, d);
     const int c = g.c, h = g.h;
     const int nt = (c + 31) >> 5;
-    float* tile_q = tiles[wave][0];
-    float* tile_do = tiles[wave][1];
-    uint32_t* tab_pos = tabs[wave][0];
-    uint32_t* tab_L = tabs[wave][1];
-    uint32_t* tab_D = tabs[wave][2];
     const int32_t* order = a.order + g.Tk;
     const int32_t* tok_pos = a.tok_pos + g.Tk;
     const int8_t* mrow = MASK ? a.mask + (int64_t)(g.w % a.nmw) * a.n : nullptr;
@@ -805,6 +809,38 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     tile_store_rows<T>(tile_do, const_cast<char*>(head_base<T>(tdv, h)), pitch_of<T>(tdv), vox_j, c - bj * 32, lane);
 }
 
+template <typename T, bool MASK>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void wattn_bwd_kv_kernel(
+    WAttnCommon a, TokenTensor32 tq, TokenTensor32 tk, TokenTensor32 tv, TokenTensor32 to, TokenTensor32 tdo,
+    const float* __restrict__ lse, TokenTensor32 tdk, TokenTensor32 tdv, float* __restrict__ ds_out) {
+    __shared__ __attribute__((aligned(16))) float tiles[4][2][TILE_WORDS];
+    __shared__ __attribute__((aligned(16))) uint32_t tabs[4][3][32];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    bwd_kv_task<T, MASK, false>(a, (int64_t)blockIdx.x * 4 + wave, tiles[wave][0], tiles[wave][1], tabs[wave][0],
+                                tabs[wave][1], tabs[wave][2], tq, tk, tv, to, tdo, lse, tdk, tdv, ds_out, tdk);
+}
+
+// The whole backward in one launch: the query-side tasks of the groups of more than 32 tokens
+// first (tasks 0 .. first[3]), then the key-side tasks of all groups; groups of at most 32 tokens
+// get dQ from their key-side task.  One launch keeps the chip filled while the long tasks run.
+template <typename T, bool MASK>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void wattn_bwd_all_kernel(
+    WAttnCommon a, TokenTensor32 tq, TokenTensor32 tk, TokenTensor32 tv, TokenTensor32 to, TokenTensor32 tdo,
+    const float* __restrict__ lse, TokenTensor32 tdq, TokenTensor32 tdk, TokenTensor32 tdv,
+    float* __restrict__ ds_out, int key_side_only) {
+    __shared__ __attribute__((aligned(16))) float tiles[4][2][TILE_WORDS];
+    __shared__ __attribute__((aligned(16))) uint32_t tabs[4][3][32];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+    const int64_t task = (int64_t)blockIdx.x * 4 + wave;
+    const int64_t nq = key_side_only ? 0 : a.first[3];       // query-side tasks of the larger groups
+    if (task < nq)
+        bwd_q_task<T, MASK>(a, task, tiles[wave][0], tiles[wave][1], tabs[wave][0], tabs[wave][1], tq, tk, tv, to, tdo,
+                            lse, tdq);
+    else
+        bwd_kv_task<T, MASK, true>(a, task - nq, tiles[wave][0], tiles[wave][1], tabs[wave][0], tabs[wave][1],
+                                   tabs[wave][2], tq, tk, tv, to, tdo, lse, tdk, tdv, ds_out, tdq);
+}
+
 // ------------------------------------------------------------------------------------------
 // host side
 // ------------------------------------------------------------------------------------------
@@ -826,23 +862,18 @@ static void launch_backward(const WAttnCommon& a, const TokenTensor32& q, const 
                             const TokenTensor32& v, const TokenTensor32& o, const TokenTensor32& d_o, const float* lse,
                             const TokenTensor32& dq, const TokenTensor32& dk, const TokenTensor32& dv, float* ds_out,
                             int sides, hipStream_t s) {
-    const unsigned blocks = (unsigned)((a.first[4] + 3) / 4);
     if (sides == 3 || sides == 6) {
-        // groups of one tile get dQ from the key-side kernel; the query-side kernel takes the rest
-        WAttnCommon big = a;
-        big.first[4] = a.first[3];
-        const unsigned big_blocks = (unsigned)((big.first[4] + 3) / 4);
-        if (big_blocks && sides == 3)
-            hipLaunchKernelGGL((wattn_bwd_q_kernel<T, MASK>), dim3(big_blocks), dim3(256), 0, s, big, q, k, v, o, d_o, lse, dq);
-        hipLaunchKernelGGL((wattn_bwd_kv_kernel<T, MASK, true>), dim3(blocks), dim3(256), 0, s, a, q, k, v, o, d_o, lse,
-                           dk, dv, ds_out, dq);
+        const int64_t tasks = a.first[4] + (sides == 3 ? a.first[3] : 0);
+        hipLaunchKernelGGL((wattn_bwd_all_kernel<T, MASK>), dim3((unsigned)((tasks + 3) / 4)), dim3(256), 0, s, a, q, k, v,
+                           o, d_o, lse, dq, dk, dv, ds_out, sides == 6 ? 1 : 0);
         return;
     }
+    const unsigned blocks = (unsigned)((a.first[4] + 3) / 4);
     if (sides & 1)
         hipLaunchKernelGGL((wattn_bwd_q_kernel<T, MASK>), dim3(blocks), dim3(256), 0, s, a, q, k, v, o, d_o, lse, dq);
     if (sides & 2)
-        hipLaunchKernelGGL((wattn_bwd_kv_kernel<T, MASK, false>), dim3(blocks), dim3(256), 0, s, a, q, k, v, o, d_o, lse,
-                           dk, dv, ds_out, dq);
+        hipLaunchKernelGGL((wattn_bwd_kv_kernel<T, MASK>), dim3(blocks), dim3(256), 0, s, a, q, k, v, o, d_o, lse, dk,
+                           dv, ds_out);
 }
 
 template <typename T>
