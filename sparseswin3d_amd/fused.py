@@ -13,6 +13,7 @@ materialised in HBM (P is needed by the backward pass).
 """
 from __future__ import annotations
 
+import contextlib
 import ctypes as C
 
 import torch
@@ -27,6 +28,23 @@ _DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 
 def _ptr(t):
     return C.c_void_p(t.data_ptr() if t is not None else 0)
+
+
+launch_timer = None      # a list turns on timing: entries (name, start event, stop event) of the attention launches
+
+
+@contextlib.contextmanager
+def _timed(name, device):
+    """Brackets one library launch with events on the stream it is enqueued on (only while
+    ``launch_timer`` is a list; a benchmark uses it to time the kernels inside a real step)."""
+    if launch_timer is None:
+        yield
+        return
+    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    start.record(torch.cuda.current_stream(device))
+    yield
+    stop.record(torch.cuda.current_stream(device))
+    launch_timer.append((name, start, stop))
 
 
 class TokenPlan:
@@ -190,11 +208,12 @@ class _ResidentWindowAttention(Function):
             out = torch.empty((N, D), dtype=dtype, device=d)
             lse = torch.empty(max(H * N, 1), dtype=torch.float32, device=d)
             stream = C.c_void_p(torch.cuda.current_stream(d).cuda_stream)
-            _lib.check(lib.sswin_window_attention_forward(
-                _DTYPE_CODE[dtype], _ptr(tp.tasks), tp.g_cap, tp.bucket_counts, _ptr(tp.tokens), N, H, hd,
-                *_token_args(qkv, 3 * D, 0), *_token_args(qkv, 3 * D, D), *_token_args(qkv, 3 * D, 2 * D),
-                C.c_float(scale), _ptr(bias32), n, _ptr(mask), 0 if mask is None else mask.shape[0],
-                *_token_args(out, D, 0), _ptr(lse), stream))
+            with _timed("window_attention_forward", d):
+                _lib.check(lib.sswin_window_attention_forward(
+                    _DTYPE_CODE[dtype], _ptr(tp.tasks), tp.g_cap, tp.bucket_counts, _ptr(tp.tokens), N, H, hd,
+                    *_token_args(qkv, 3 * D, 0), *_token_args(qkv, 3 * D, D), *_token_args(qkv, 3 * D, 2 * D),
+                    C.c_float(scale), _ptr(bias32), n, _ptr(mask), 0 if mask is None else mask.shape[0],
+                    *_token_args(out, D, 0), _ptr(lse), stream))
         ctx.save_for_backward(qkv, out, lse, bias32, mask)
         ctx.tp, ctx.scale, ctx.bias_meta, ctx.table_index = tp, scale, (bias.dtype, bias.shape), table_index
         return out
@@ -215,13 +234,14 @@ class _ResidentWindowAttention(Function):
             want_bias = ctx.needs_input_grad[1]
             d_s = torch.empty(max(tp.A, 1), dtype=torch.float32, device=d) if want_bias else None
             stream = C.c_void_p(torch.cuda.current_stream(d).cuda_stream)
-            _lib.check(lib.sswin_window_attention_backward(
-                _DTYPE_CODE[dtype], _ptr(tp.tasks), tp.g_cap, tp.bucket_counts, _ptr(tp.tokens), N, H, hd,
-                *_token_args(qkv, 3 * D, 0), *_token_args(qkv, 3 * D, D), *_token_args(qkv, 3 * D, 2 * D),
-                C.c_float(scale), _ptr(bias32), tp.n, _ptr(mask), 0 if mask is None else mask.shape[0],
-                *_token_args(out, D, 0), *_token_args(grad_out, D, 0), _ptr(lse),
-                *_token_args(d_qkv, 3 * D, 0), *_token_args(d_qkv, 3 * D, D), *_token_args(d_qkv, 3 * D, 2 * D),
-                _ptr(d_s), 3, stream))
+            with _timed("window_attention_backward", d):
+                _lib.check(lib.sswin_window_attention_backward(
+                    _DTYPE_CODE[dtype], _ptr(tp.tasks), tp.g_cap, tp.bucket_counts, _ptr(tp.tokens), N, H, hd,
+                    *_token_args(qkv, 3 * D, 0), *_token_args(qkv, 3 * D, D), *_token_args(qkv, 3 * D, 2 * D),
+                    C.c_float(scale), _ptr(bias32), tp.n, _ptr(mask), 0 if mask is None else mask.shape[0],
+                    *_token_args(out, D, 0), *_token_args(grad_out, D, 0), _ptr(lse),
+                    *_token_args(d_qkv, 3 * D, 0), *_token_args(d_qkv, 3 * D, D), *_token_args(d_qkv, 3 * D, 2 * D),
+                    _ptr(d_s), 3, stream))
             d_bias = None
             if want_bias:
                 bias_dtype, bias_shape = ctx.bias_meta
