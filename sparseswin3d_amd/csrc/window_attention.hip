@@ -10,10 +10,12 @@
 //   forward    per (group, 32 queries): S^T tiles = K Q^T on MFMA, + bias + mask, softmax in
 //              registers, O = P V with P fed to the MFMA straight from the accumulators;
 //              writes O rows in voxel order and one log-sum-exp per attention row.
-//   backward Q per (group, 32 queries): recomputes S^T, dP^T = V dO^T, dS = P (dP - D) with
-//              D_i = dO_i . O_i, dQ = scale dS K.
-//   backward KV per (group, 32 keys): recomputes S and dP = dO V^T in the other orientation,
-//              dV = P^T dO, dK = scale dS^T Q; optionally stores dS for the bias gradient.
+//   backward, query side, per (group, 32 queries): recomputes S^T, dP^T = V dO^T, dS = P (dP - D)
+//              with D_i = dO_i . O_i, dQ = scale dS K.
+//   backward, key side, per (group, 32 keys): recomputes S and dP = dO V^T in the other orientation,
+//              dV = P^T dO, dK = scale dS^T Q; optionally stores dS for the bias gradient.  For a
+//              group of at most 32 tokens it also produces dQ from the dS it already holds.
+//   The whole backward is one launch: query-side tasks of the larger groups, then key-side tasks.
 //
 // Orientation trick: v_mfma_f32_32x32x2_f32 leaves output column l%32 in lane l and 16 rows in
 // its registers.  Computing S transposed (keys as rows, queries as columns) puts a whole
