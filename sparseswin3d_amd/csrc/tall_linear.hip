@@ -1,0 +1,260 @@
+// Y = X W^T + b for a very tall fp32 X [N, K] (N = voxels, K = channels <= 192) and a small weight
+// W [P, K]: the qkv and proj projections of the window attention (nn.Linear of
+// sparse_swin/swin3d_base.py:606-610, applied at :658 and :676).
+//
+// On gfx950 the fp32 matrix instruction runs on the vector ALU's own multipliers (64 FLOP per clock
+// and SIMD, and it blocks the ALU while it runs), so an fp32 GEMM cannot get past the packed-FMA rate;
+// the bf16 matrix cores are sixteen times faster and sit idle.  This kernel uses them without giving
+// up fp32 accuracy: every fp32 operand is split exactly into three bf16 pieces (x = h + m + l, 8 + 8 +
+// 8 significant bits, by truncation and exact subtraction) and a product is the sum of the six
+// piece products whose weight is at least 2^-16 of the leading one (hh, hm, mh, mm, hl, lh), all
+// accumulated in fp32 by v_mfma_f32_32x32x16_bf16.  What is dropped (ml, lm, ll) is below 2^-23 of
+// the product, i.e. at the level of fp32 rounding itself.
+//
+// Layout: a workgroup (4 waves) owns one group of 96 output columns and keeps the three bf16 planes
+// of those columns of W in LDS in MFMA operand order (prepared once per call by a small kernel); it
+// walks over blocks of 128 rows, one 32-row tile per wave.  Per 16-wide k step a lane reads its
+// 8 fp32 of X (row l % 32, k group l / 32), splits them, and feeds 3 column tiles x 6 products.
+#include <stdint.h>
+
+#include <algorithm>
+
+#include "mfma_block.hpp"
+#include "sswin_common.hpp"
+
+namespace sswin {
+
+typedef __bf16 tl_bf16x8 __attribute__((ext_vector_type(8)));
+typedef uint32_t tl_u32x4 __attribute__((ext_vector_type(4)));
+typedef float tl_f32x4 __attribute__((ext_vector_type(4)));
+
+constexpr int TL_COLS = 96;          // output columns per workgroup (3 MFMA tiles)
+constexpr int TL_MAX_K = 192;
+
+// exact split of two fp32 values into bf16 pieces, packed (low half = first value)
+struct Split2 {
+    uint32_t h, m, l;
+};
+__device__ __forceinline__ Split2 split2(float x0, float x1) {
+    const uint32_t u0 = __builtin_bit_cast(uint32_t, x0), u1 = __builtin_bit_cast(uint32_t, x1);
+    const float r0 = x0 - __builtin_bit_cast(float, u0 & 0xffff0000u);
+    const float r1 = x1 - __builtin_bit_cast(float, u1 & 0xffff0000u);
+    const uint32_t v0 = __builtin_bit_cast(uint32_t, r0), v1 = __builtin_bit_cast(uint32_t, r1);
+    const float s0 = r0 - __builtin_bit_cast(float, v0 & 0xffff0000u);
+    const float s1 = r1 - __builtin_bit_cast(float, v1 & 0xffff0000u);
+    Split2 o;
+    o.h = __builtin_amdgcn_perm(u1, u0, 0x07060302u);       // {u1.hi16, u0.hi16}
+    o.m = __builtin_amdgcn_perm(v1, v0, 0x07060302u);
+    o.l = __builtin_amdgcn_perm(__builtin_bit_cast(uint32_t, s1), __builtin_bit_cast(uint32_t, s0), 0x07060302u);
+    return o;
+}
+
+// planes of W in operand order: [column group][k step][column tile][plane][lane 64][8 bf16]
+__global__ __launch_bounds__(256) void tall_linear_prepare_kernel(const float* __restrict__ w, int P, int K,
+                                                                  tl_u32x4* __restrict__ planes) {
+    const int ksteps = K / 16;
+    const int64_t total = (int64_t)(P / TL_COLS) * ksteps * 3 * 64;     // (group, k step, tile, lane)
+    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= total) return;
+    const int lane = (int)(i & 63);
+    int64_t rest = i >> 6;
+    const int ct = (int)(rest % 3);
+    rest /= 3;
+    const int ks = (int)(rest % ksteps);
+    const int cg = (int)(rest / ksteps);
+    const int col = cg * TL_COLS + ct * 32 + (lane & 31);
+    const float* src = w + (int64_t)col * K + ks * 16 + (lane >> 5) * 8;
+    uint32_t h[4], m[4], l[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        const Split2 s = split2(src[2 * e], src[2 * e + 1]);
+        h[e] = s.h; m[e] = s.m; l[e] = s.l;
+    }
+    tl_u32x4* dst = planes + (((int64_t)(cg * ksteps + ks) * 3 + ct) * 3) * 64 + lane;
+    dst[0] = tl_u32x4{h[0], h[1], h[2], h[3]};
+    dst[64] = tl_u32x4{m[0], m[1], m[2], m[3]};
+    dst[128] = tl_u32x4{l[0], l[1], l[2], l[3]};
+}
+
+__device__ __forceinline__ tl_bf16x8 as_bf16x8(const tl_u32x4& v) { return __builtin_bit_cast(tl_bf16x8, v); }
+
+struct APlanes {
+    tl_bf16x8 h, m, l;
+};
+__device__ __forceinline__ APlanes split8(const tl_f32x4& c0, const tl_f32x4& c1) {
+    const Split2 s0 = split2(c0.x, c0.y), s1 = split2(c0.z, c0.w), s2 = split2(c1.x, c1.y), s3 = split2(c1.z, c1.w);
+    APlanes a;
+    a.h = as_bf16x8(tl_u32x4{s0.h, s1.h, s2.h, s3.h});
+    a.m = as_bf16x8(tl_u32x4{s0.m, s1.m, s2.m, s3.m});
+    a.l = as_bf16x8(tl_u32x4{s0.l, s1.l, s2.l, s3.l});
+    return a;
+}
+
+// one 16-wide k step of a 32-row tile against the workgroup's 96 columns: 3 tiles x 6 products
+__device__ __forceinline__ void k_step(const APlanes& a, const tl_u32x4* wk, f32x16 (&acc)[3]) {
+    tl_bf16x8 bh[3], bm[3], bl[3];
+#pragma unroll
+    for (int ct = 0; ct < 3; ++ct) {
+        bh[ct] = as_bf16x8(wk[(ct * 3 + 0) * 64]);
+        bm[ct] = as_bf16x8(wk[(ct * 3 + 1) * 64]);
+        bl[ct] = as_bf16x8(wk[(ct * 3 + 2) * 64]);
+    }
+    // small terms first; the three column tiles alternate so that no product waits for the previous
+    // one into the same accumulator
+#pragma unroll
+    for (int ct = 0; ct < 3; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.l, bh[ct], acc[ct], 0, 0, 0);
+#pragma unroll
+    for (int ct = 0; ct < 3; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.h, bl[ct], acc[ct], 0, 0, 0);
+#pragma unroll
+    for (int ct = 0; ct < 3; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.m, bm[ct], acc[ct], 0, 0, 0);
+#pragma unroll
+    for (int ct = 0; ct < 3; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.m, bh[ct], acc[ct], 0, 0, 0);
+#pragma unroll
+    for (int ct = 0; ct < 3; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.h, bm[ct], acc[ct], 0, 0, 0);
+#pragma unroll
+    for (int ct = 0; ct < 3; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.h, bh[ct], acc[ct], 0, 0, 0);
+}
+
+// KS > 0: K = 16 KS known at compile time and the rows of the next block are requested before the
+// current block is multiplied (two workgroups per CU leave the registers for it).  KS = 0: any
+// supported K, with the next k step's 8 values in flight during the current one.
+template <int KS>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void tall_linear_forward_kernel(const float* __restrict__ x, int64_t N, int K,
+                                                                  const tl_u32x4* __restrict__ planes, int groups,
+                                                                  const float* __restrict__ bias, float* __restrict__ y,
+                                                                  int P, int64_t row_blocks) {
+    extern __shared__ __attribute__((aligned(16))) tl_u32x4 w_s[];      // [k step][tile][plane][lane]
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int half = lane >> 5, l32 = lane & 31;
+    const int ksteps = KS > 0 ? KS : K / 16;
+    const int cg = blockIdx.x % groups;
+    const int64_t wg = blockIdx.x / groups, wgs = gridDim.x / groups;
+    // this group's planes: global -> LDS, once
+    const int n16 = ksteps * 9 * 64;
+    const tl_u32x4* src = planes + (int64_t)cg * n16;
+    for (int e = threadIdx.x; e < n16; e += 256) w_s[e] = src[e];
+    __syncthreads();
+    float bcol[3];
+#pragma unroll
+    for (int ct = 0; ct < 3; ++ct) bcol[ct] = bias ? bias[cg * TL_COLS + ct * 32 + l32] : 0.f;
+
+    auto row_ptr = [&](int64_t rb) {
+        int64_t row = rb * 128 + wave * 32 + l32;
+        row = row < N ? row : N - 1;                                     // padding rows read the last row
+        return reinterpret_cast<const tl_f32x4*>(x + row * K + half * 8);
+    };
+    constexpr int NX = KS > 0 ? KS : 1;
+    tl_f32x4 xn[NX][2];                                                  // rows of the block to come
+    if (KS > 0 && wg < row_blocks) {
+        const tl_f32x4* xp = row_ptr(wg);
+#pragma unroll
+        for (int ks = 0; ks < NX; ++ks) xn[ks][0] = xp[ks * 4], xn[ks][1] = xp[ks * 4 + 1];
+    }
+    for (int64_t rb = wg; rb < row_blocks; rb += wgs) {
+        const int64_t row0 = rb * 128 + wave * 32;
+        f32x16 acc[3];
+#pragma unroll
+        for (int ct = 0; ct < 3; ++ct) acc[ct] = f32x16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        if constexpr (KS > 0) {
+            tl_f32x4 xc[NX][2];
+#pragma unroll
+            for (int ks = 0; ks < NX; ++ks) xc[ks][0] = xn[ks][0], xc[ks][1] = xn[ks][1];
+            if (rb + wgs < row_blocks) {
+                const tl_f32x4* xp = row_ptr(rb + wgs);
+#pragma unroll
+                for (int ks = 0; ks < NX; ++ks) xn[ks][0] = xp[ks * 4], xn[ks][1] = xp[ks * 4 + 1];
+            }
+#pragma unroll
+            for (int ks = 0; ks < NX; ++ks) {
+                k_step(split8(xc[ks][0], xc[ks][1]), w_s + ks * 9 * 64 + lane, acc);
+                __builtin_amdgcn_sched_barrier(0);                       // keeps the operands of later steps out of registers
+            }
+        } else {
+            const tl_f32x4* xp = row_ptr(rb);
+            tl_f32x4 c0 = xp[0], c1 = xp[1];
+            for (int ks = 0; ks < ksteps; ++ks) {
+                const APlanes a = split8(c0, c1);
+                if (ks + 1 < ksteps) c0 = xp[(ks + 1) * 4], c1 = xp[(ks + 1) * 4 + 1];
+                k_step(a, w_s + ks * 9 * 64 + lane, acc);
+            }
+        }
+        if (row0 >= N) continue;
+        // accumulator register r of lane l: row acc_row(r, half), column l % 32
+#pragma unroll
+        for (int ct = 0; ct < 3; ++ct) {
+            float* yp = y + (int64_t)cg * TL_COLS + ct * 32 + l32;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int64_t orow = row0 + acc_row(r, half);
+                if (orow < N) yp[orow * P] = acc[ct][r] + bcol[ct];
+            }
+        }
+    }
+}
+
+}  // namespace sswin
+
+using namespace sswin;
+
+extern "C" {
+
+size_t sswin_tall_linear_workspace_bytes(int P, int K) {
+    if (P <= 0 || K <= 0 || (P % TL_COLS) || (K % 16) || K > TL_MAX_K) return 0;
+    return (size_t)(P / TL_COLS) * (K / 16) * 9 * 64 * sizeof(tl_u32x4) + 256;
+}
+
+int sswin_tall_linear_forward(const float* x, int64_t N, int K, const float* w, const float* bias, int P, float* y,
+                              void* ws, size_t ws_bytes, void* stream) {
+    SSWIN_CHECK(N >= 0 && K > 0 && P > 0, "tall_linear_forward: bad sizes");
+    SSWIN_CHECK(K % 16 == 0 && K <= TL_MAX_K, "tall_linear_forward: %d input channels are not supported (a multiple of 16, at most %d)",
+                K, TL_MAX_K);
+    SSWIN_CHECK(P % TL_COLS == 0, "tall_linear_forward: %d output channels are not a multiple of %d", P, TL_COLS);
+    if (N == 0) return 0;
+    SSWIN_CHECK(x && w && y && ws, "tall_linear_forward: null pointer");
+    SSWIN_CHECK(((uintptr_t)x % 16) == 0 && ((uintptr_t)ws % 16) == 0, "tall_linear_forward: x and the workspace must be 16-byte aligned");
+    SSWIN_CHECK(ws_bytes >= sswin_tall_linear_workspace_bytes(P, K), "tall_linear_forward: workspace too small");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int groups = P / TL_COLS, ksteps = K / 16;
+    tl_u32x4* planes = static_cast<tl_u32x4*>(ws);
+    const int64_t prep = (int64_t)groups * ksteps * 3 * 64;
+    hipLaunchKernelGGL(tall_linear_prepare_kernel, dim3((unsigned)((prep + 255) / 256)), dim3(256), 0, s, w, P, K, planes);
+    const size_t lds = (size_t)ksteps * 9 * 64 * sizeof(tl_u32x4);
+    const int64_t row_blocks = (N + 127) / 128;
+    int cus = 256;
+    {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
+            cus = n;
+    }
+    const int per_cu = lds <= 64 * 1024 ? 2 : 1;                          // workgroups that fit a CU's LDS
+    int64_t per_group = std::min<int64_t>(row_blocks, std::max<int64_t>(1, (int64_t)cus * per_cu / groups));
+    static bool configured = false;
+    if (!configured) {
+        const int max_lds = TL_MAX_K / 16 * 9 * 64 * (int)sizeof(tl_u32x4);
+        const void* all[] = {reinterpret_cast<const void*>(tall_linear_forward_kernel<0>),
+                             reinterpret_cast<const void*>(tall_linear_forward_kernel<2>),
+                             reinterpret_cast<const void*>(tall_linear_forward_kernel<3>),
+                             reinterpret_cast<const void*>(tall_linear_forward_kernel<4>),
+                             reinterpret_cast<const void*>(tall_linear_forward_kernel<6>)};
+        for (const void* k : all) SSWIN_HIP(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, max_lds));
+        configured = true;
+    }
+    auto launch = [&](auto kernel) -> int {
+        hipLaunchKernelGGL(kernel, dim3((unsigned)(per_group * groups)), dim3(256), lds, s, x, N, K, planes, groups, bias, y, P,
+                           row_blocks);
+        return 0;
+    };
+    int rc;
+    switch (ksteps) {
+        case 6: rc = launch(tall_linear_forward_kernel<6>); break;       // 96 channels (stage 1)
+        case 4: rc = launch(tall_linear_forward_kernel<4>); break;
+        case 3: rc = launch(tall_linear_forward_kernel<3>); break;
+        case 2: rc = launch(tall_linear_forward_kernel<2>); break;
+        default: rc = launch(tall_linear_forward_kernel<0>); break;
+    }
+    if (rc) return rc;
+    return launch_ok("tall_linear_forward");
+}
+
+}  // extern "C"
