@@ -115,18 +115,14 @@ __device__ __forceinline__ void k_step(const APlanes& a, const tl_u32x4* wk, f32
     for (int ct = 0; ct < 3; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.h, bh[ct], acc[ct], 0, 0, 0);
 }
 
-// KS > 0: K = 16 KS known at compile time and the rows of the next block are requested before the
-// current block is multiplied (two workgroups per CU leave the registers for it).  KS = 0: any
-// supported K, with the next k step's 8 values in flight during the current one.
-template <int KS>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void tall_linear_forward_kernel(const float* __restrict__ x, int64_t N, int K,
-                                                                  const tl_u32x4* __restrict__ planes, int groups,
-                                                                  const float* __restrict__ bias, float* __restrict__ y,
-                                                                  int P, int64_t row_blocks) {
+// any supported K; the next k step's 8 values are in flight during the current one
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void tall_linear_forward_kernel(
+    const float* __restrict__ x, int64_t N, int K, const tl_u32x4* __restrict__ planes, int groups, const float* __restrict__ bias,
+    float* __restrict__ y, int P, int64_t row_blocks) {
     extern __shared__ __attribute__((aligned(16))) tl_u32x4 w_s[];      // [k step][tile][plane][lane]
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int half = lane >> 5, l32 = lane & 31;
-    const int ksteps = KS > 0 ? KS : K / 16;
+    const int ksteps = K / 16;
     const int cg = blockIdx.x % groups;
     const int64_t wg = blockIdx.x / groups, wgs = gridDim.x / groups;
     // this group's planes: global -> LDS, once
@@ -138,45 +134,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
     for (int ct = 0; ct < 3; ++ct) bcol[ct] = bias ? bias[cg * TL_COLS + ct * 32 + l32] : 0.f;
 
-    auto row_ptr = [&](int64_t rb) {
-        int64_t row = rb * 128 + wave * 32 + l32;
-        row = row < N ? row : N - 1;                                     // padding rows read the last row
-        return reinterpret_cast<const tl_f32x4*>(x + row * K + half * 8);
-    };
-    constexpr int NX = KS > 0 ? KS : 1;
-    tl_f32x4 xn[NX][2];                                                  // rows of the block to come
-    if (KS > 0 && wg < row_blocks) {
-        const tl_f32x4* xp = row_ptr(wg);
-#pragma unroll
-        for (int ks = 0; ks < NX; ++ks) xn[ks][0] = xp[ks * 4], xn[ks][1] = xp[ks * 4 + 1];
-    }
     for (int64_t rb = wg; rb < row_blocks; rb += wgs) {
         const int64_t row0 = rb * 128 + wave * 32;
         f32x16 acc[3];
 #pragma unroll
         for (int ct = 0; ct < 3; ++ct) acc[ct] = f32x16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-        if constexpr (KS > 0) {
-            tl_f32x4 xc[NX][2];
-#pragma unroll
-            for (int ks = 0; ks < NX; ++ks) xc[ks][0] = xn[ks][0], xc[ks][1] = xn[ks][1];
-            if (rb + wgs < row_blocks) {
-                const tl_f32x4* xp = row_ptr(rb + wgs);
-#pragma unroll
-                for (int ks = 0; ks < NX; ++ks) xn[ks][0] = xp[ks * 4], xn[ks][1] = xp[ks * 4 + 1];
-            }
-#pragma unroll
-            for (int ks = 0; ks < NX; ++ks) {
-                k_step(split8(xc[ks][0], xc[ks][1]), w_s + ks * 9 * 64 + lane, acc);
-                __builtin_amdgcn_sched_barrier(0);                       // keeps the operands of later steps out of registers
-            }
-        } else {
-            const tl_f32x4* xp = row_ptr(rb);
-            tl_f32x4 c0 = xp[0], c1 = xp[1];
-            for (int ks = 0; ks < ksteps; ++ks) {
-                const APlanes a = split8(c0, c1);
-                if (ks + 1 < ksteps) c0 = xp[(ks + 1) * 4], c1 = xp[(ks + 1) * 4 + 1];
-                k_step(a, w_s + ks * 9 * 64 + lane, acc);
-            }
+        int64_t row = row0 + l32;
+        row = row < N ? row : N - 1;                                     // padding rows read the last row
+        const tl_f32x4* xp = reinterpret_cast<const tl_f32x4*>(x + row * K + half * 8);
+        tl_f32x4 c0 = xp[0], c1 = xp[1];
+        for (int ks = 0; ks < ksteps; ++ks) {
+            const APlanes a = split8(c0, c1);
+            if (ks + 1 < ksteps) c0 = xp[(ks + 1) * 4], c1 = xp[(ks + 1) * 4 + 1];
+            k_step(a, w_s + ks * 9 * 64 + lane, acc);
         }
         if (row0 >= N) continue;
         // accumulator register r of lane l: row acc_row(r, half), column l % 32
@@ -192,9 +162,83 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 }
 
+// The same product with the rows of X read the way they lie in memory.  The kernel above reads a
+// row per lane, 16 bytes at a time: every such instruction touches 64 cache lines and the texture
+// path, not the matrix cores, sets its pace.  Here a wave reads its 32 x K tile as one contiguous
+// run (16 bytes per lane, 8 lines per instruction), one block ahead, parks it in a private LDS tile
+// (pitch K + 4 floats, so 8 rows hit 8 different bank groups) and takes its operands from there.
+// One workgroup of 8 waves per CU shares the planes of W: K <= 96 fits 160 KB of LDS.
+constexpr int TL_STAGED_MAX_KS = 6;
+template <int KS>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void tall_linear_forward_staged_kernel(
+    const float* __restrict__ x, int64_t N, const tl_u32x4* __restrict__ planes, int groups, const float* __restrict__ bias,
+    float* __restrict__ y, int P, int64_t row_tiles) {
+    constexpr int K = KS * 16, PITCH = K + 4, C4 = K / 4, NI = 2 * KS;   // 16-byte chunks per row; loads per lane and tile
+    extern __shared__ __attribute__((aligned(16))) tl_u32x4 w_s[];      // [k step][tile][plane][lane], then the X tiles
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int half = lane >> 5, l32 = lane & 31;
+    const int cg = blockIdx.x % groups;
+    const int64_t first = (int64_t)(blockIdx.x / groups) * 8 + wave, stride = (int64_t)(gridDim.x / groups) * 8;
+    constexpr int n16 = KS * 9 * 64;
+    const tl_u32x4* src = planes + (int64_t)cg * n16;
+    for (int e = threadIdx.x; e < n16; e += 512) w_s[e] = src[e];
+    float* xs = reinterpret_cast<float*>(w_s + n16) + wave * 32 * PITCH;
+    __syncthreads();
+    float bcol[3];
+#pragma unroll
+    for (int ct = 0; ct < 3; ++ct) bcol[ct] = bias ? bias[cg * TL_COLS + ct * 32 + l32] : 0.f;
+
+    tl_f32x4 xn[NI];
+    auto fetch = [&](int64_t t) {
+        const int64_t e0 = t * 32 * K, end = N * K;                      // the tile is 32 K consecutive floats
+        const tl_f32x4* xp = reinterpret_cast<const tl_f32x4*>(x + e0);
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const int q = i * 64 + lane;
+            xn[i] = e0 + q * 4 < end ? xp[q] : tl_f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+    };
+    if (first < row_tiles) fetch(first);
+    for (int64_t t = first; t < row_tiles; t += stride) {
+        const int64_t row0 = t * 32;
+        __builtin_amdgcn_wave_barrier();                                 // the previous tile's operand reads are done
+#pragma unroll
+        for (int i = 0; i < NI; ++i) {
+            const int q = i * 64 + lane;
+            *reinterpret_cast<tl_f32x4*>(xs + (q / C4) * PITCH + (q % C4) * 4) = xn[i];
+        }
+        __builtin_amdgcn_wave_barrier();
+        if (t + stride < row_tiles) fetch(t + stride);
+        f32x16 acc[3];
+#pragma unroll
+        for (int ct = 0; ct < 3; ++ct) acc[ct] = f32x16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        const float* xr = xs + l32 * PITCH + half * 8;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+            const tl_f32x4 c0 = *reinterpret_cast<const tl_f32x4*>(xr + ks * 16);
+            const tl_f32x4 c1 = *reinterpret_cast<const tl_f32x4*>(xr + ks * 16 + 4);
+            k_step(split8(c0, c1), w_s + ks * 9 * 64 + lane, acc);
+            __builtin_amdgcn_sched_barrier(0);                           // keeps the operands of later steps out of registers
+        }
+#pragma unroll
+        for (int ct = 0; ct < 3; ++ct) {
+            float* yp = y + (int64_t)cg * TL_COLS + ct * 32 + l32;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int64_t orow = row0 + acc_row(r, half);
+                if (orow < N) yp[orow * P] = acc[ct][r] + bcol[ct];
+            }
+        }
+    }
+}
+
 }  // namespace sswin
 
 using namespace sswin;
+
+static int staged_lds_bytes(int ksteps) {
+    return ksteps * 9 * 64 * (int)sizeof(tl_u32x4) + 8 * 32 * (ksteps * 16 + 4) * (int)sizeof(float);
+}
 
 extern "C" {
 
@@ -218,8 +262,6 @@ int sswin_tall_linear_forward(const float* x, int64_t N, int K, const float* w, 
     tl_u32x4* planes = static_cast<tl_u32x4*>(ws);
     const int64_t prep = (int64_t)groups * ksteps * 3 * 64;
     hipLaunchKernelGGL(tall_linear_prepare_kernel, dim3((unsigned)((prep + 255) / 256)), dim3(256), 0, s, w, P, K, planes);
-    const size_t lds = (size_t)ksteps * 9 * 64 * sizeof(tl_u32x4);
-    const int64_t row_blocks = (N + 127) / 128;
     int cus = 256;
     {
         int dev = 0, n = 0;
@@ -227,33 +269,43 @@ int sswin_tall_linear_forward(const float* x, int64_t N, int K, const float* w, 
             hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0)
             cus = n;
     }
-    const int per_cu = lds <= 64 * 1024 ? 2 : 1;                          // workgroups that fit a CU's LDS
-    int64_t per_group = std::min<int64_t>(row_blocks, std::max<int64_t>(1, (int64_t)cus * per_cu / groups));
     static bool configured = false;
     if (!configured) {
         const int max_lds = TL_MAX_K / 16 * 9 * 64 * (int)sizeof(tl_u32x4);
-        const void* all[] = {reinterpret_cast<const void*>(tall_linear_forward_kernel<0>),
-                             reinterpret_cast<const void*>(tall_linear_forward_kernel<2>),
-                             reinterpret_cast<const void*>(tall_linear_forward_kernel<3>),
-                             reinterpret_cast<const void*>(tall_linear_forward_kernel<4>),
-                             reinterpret_cast<const void*>(tall_linear_forward_kernel<6>)};
-        for (const void* k : all) SSWIN_HIP(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, max_lds));
+        SSWIN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(tall_linear_forward_kernel),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, max_lds));
+        const void* staged[] = {reinterpret_cast<const void*>(tall_linear_forward_staged_kernel<1>),
+                                reinterpret_cast<const void*>(tall_linear_forward_staged_kernel<2>),
+                                reinterpret_cast<const void*>(tall_linear_forward_staged_kernel<3>),
+                                reinterpret_cast<const void*>(tall_linear_forward_staged_kernel<4>),
+                                reinterpret_cast<const void*>(tall_linear_forward_staged_kernel<5>),
+                                reinterpret_cast<const void*>(tall_linear_forward_staged_kernel<6>)};
+        for (int ks = 1; ks <= TL_STAGED_MAX_KS; ++ks)
+            SSWIN_HIP(hipFuncSetAttribute(staged[ks - 1], hipFuncAttributeMaxDynamicSharedMemorySize, staged_lds_bytes(ks)));
         configured = true;
     }
-    auto launch = [&](auto kernel) -> int {
-        hipLaunchKernelGGL(kernel, dim3((unsigned)(per_group * groups)), dim3(256), lds, s, x, N, K, planes, groups, bias, y, P,
-                           row_blocks);
-        return 0;
-    };
-    int rc;
-    switch (ksteps) {
-        case 6: rc = launch(tall_linear_forward_kernel<6>); break;       // 96 channels (stage 1)
-        case 4: rc = launch(tall_linear_forward_kernel<4>); break;
-        case 3: rc = launch(tall_linear_forward_kernel<3>); break;
-        case 2: rc = launch(tall_linear_forward_kernel<2>); break;
-        default: rc = launch(tall_linear_forward_kernel<0>); break;
+    if (ksteps <= TL_STAGED_MAX_KS) {
+        const int64_t row_tiles = (N + 31) / 32;
+        const int64_t per_group = std::min<int64_t>((row_tiles + 7) / 8, std::max<int64_t>(1, cus / groups));
+        const dim3 grid((unsigned)(per_group * groups)), block(512);
+        const size_t lds = staged_lds_bytes(ksteps);
+#define SSWIN_TL_STAGED(KS)                                                                                                  \
+    case KS:                                                                                                                 \
+        hipLaunchKernelGGL(tall_linear_forward_staged_kernel<KS>, grid, block, lds, s, x, N, planes, groups, bias, y, P,     \
+                           row_tiles);                                                                                       \
+        break;
+        switch (ksteps) {
+            SSWIN_TL_STAGED(1) SSWIN_TL_STAGED(2) SSWIN_TL_STAGED(3) SSWIN_TL_STAGED(4) SSWIN_TL_STAGED(5) SSWIN_TL_STAGED(6)
+        }
+#undef SSWIN_TL_STAGED
+        return launch_ok("tall_linear_forward");
     }
-    if (rc) return rc;
+    const size_t lds = (size_t)ksteps * 9 * 64 * sizeof(tl_u32x4);
+    const int64_t row_blocks = (N + 127) / 128;
+    const int per_cu = lds <= 64 * 1024 ? 2 : 1;                          // workgroups that fit a CU's LDS
+    int64_t per_group = std::min<int64_t>(row_blocks, std::max<int64_t>(1, (int64_t)cus * per_cu / groups));
+    hipLaunchKernelGGL(tall_linear_forward_kernel, dim3((unsigned)(per_group * groups)), dim3(256), lds, s, x, N, K, planes,
+                       groups, bias, y, P, row_blocks);
     return launch_ok("tall_linear_forward");
 }
 

@@ -257,15 +257,48 @@ def _column_sum(t: torch.Tensor) -> torch.Tensor:
     return out.to(t.dtype)
 
 
+def _split_linear_forward(x: torch.Tensor, weight: torch.Tensor, bias):
+    """``x @ W^T + b`` through the library's matrix-core kernel for fp32 (operands split into bf16
+    pieces, fp32 accuracy), or None when the shape or dtype is outside what that kernel takes."""
+    if not (x.is_cuda and x.dtype == torch.float32 and weight.dtype == torch.float32 and x.dim() == 2
+            and x.shape[0] > 0 and (bias is None or bias.dtype == torch.float32)):
+        return None
+    import ctypes as C
+    from . import _lib
+    lib = _lib.load()
+    n, k = x.shape
+    p = weight.shape[0]
+    nbytes = int(lib.sswin_tall_linear_workspace_bytes(p, k))
+    if nbytes == 0:
+        return None
+    x = x.contiguous()
+    weight = weight.contiguous()
+    if x.data_ptr() % 16:
+        x = x.clone()
+    with torch.cuda.device(x.device):
+        y = torch.empty(n, p, dtype=torch.float32, device=x.device)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+        b = bias.contiguous() if bias is not None else None
+        _lib.check(lib.sswin_tall_linear_forward(C.c_void_p(x.data_ptr()), n, k, C.c_void_p(weight.data_ptr()),
+                                                 C.c_void_p(b.data_ptr() if b is not None else None), p,
+                                                 C.c_void_p(y.data_ptr()), C.c_void_p(ws.data_ptr()), nbytes,
+                                                 C.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)))
+    return y
+
+
 class _TallLinear(Function):
-    """``x @ W^T + b`` for a very tall ``x`` [N, in] (N = number of voxels): forward, input
-    gradient and weight gradient are three library GEMMs, routed to the BLAS backend that
-    handles tall-skinny shapes best (see :func:`_rocblas_gemm`)."""
+    """``x @ W^T + b`` for a very tall ``x`` [N, in] (N = number of voxels).  The fp32 forward runs on
+    the bf16 matrix cores with exactly split operands where the shape allows; input gradient and
+    weight gradient are library GEMMs, routed to the BLAS backend that handles tall-skinny shapes
+    best (see :func:`_rocblas_gemm`)."""
 
     @staticmethod
     def forward(ctx, x, weight, bias):
         ctx.save_for_backward(x, weight)
         ctx.has_bias = bias is not None
+        y = _split_linear_forward(x, weight, bias)
+        if y is not None:
+            return y
         with _rocblas_gemm():
             return torch.nn.functional.linear(x, weight, bias)
 
