@@ -11,8 +11,8 @@
 // accumulated in fp32 by v_mfma_f32_32x32x16_bf16.  What is dropped (ml, lm, ll) is below 2^-23 of
 // the product, i.e. at the level of fp32 rounding itself.
 //
-// Layout: a workgroup (4 waves) owns one group of 96 output columns and keeps the three bf16 planes
-// of those columns of W in LDS in MFMA operand order (prepared once per call by a small kernel); it
+// Layout: a workgroup owns one group of 96 output columns and keeps the three bf16 planes of those
+// columns of W in LDS in MFMA operand order (split by the workgroup itself when it starts); it
 // walks over blocks of 128 rows, one 32-row tile per wave.  Per 16-wide k step a lane reads its
 // 8 fp32 of X (row l % 32, k group l / 32), splits them, and feeds 3 column tiles x 6 products.
 #include <stdint.h>
@@ -49,33 +49,6 @@ __device__ __forceinline__ Split2 split2(float x0, float x1) {
     return o;
 }
 
-// planes of W in operand order: [column group][k step][column tile][plane][lane 64][8 bf16]
-__global__ __launch_bounds__(256) void tall_linear_prepare_kernel(const float* __restrict__ w, int P, int K,
-                                                                  tl_u32x4* __restrict__ planes) {
-    const int ksteps = K / 16;
-    const int64_t total = (int64_t)(P / TL_COLS) * ksteps * 3 * 64;     // (group, k step, tile, lane)
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i >= total) return;
-    const int lane = (int)(i & 63);
-    int64_t rest = i >> 6;
-    const int ct = (int)(rest % 3);
-    rest /= 3;
-    const int ks = (int)(rest % ksteps);
-    const int cg = (int)(rest / ksteps);
-    const int col = cg * TL_COLS + ct * 32 + (lane & 31);
-    const float* src = w + (int64_t)col * K + ks * 16 + (lane >> 5) * 8;
-    uint32_t h[4], m[4], l[4];
-#pragma unroll
-    for (int e = 0; e < 4; ++e) {
-        const Split2 s = split2(src[2 * e], src[2 * e + 1]);
-        h[e] = s.h; m[e] = s.m; l[e] = s.l;
-    }
-    tl_u32x4* dst = planes + (((int64_t)(cg * ksteps + ks) * 3 + ct) * 3) * 64 + lane;
-    dst[0] = tl_u32x4{h[0], h[1], h[2], h[3]};
-    dst[64] = tl_u32x4{m[0], m[1], m[2], m[3]};
-    dst[128] = tl_u32x4{l[0], l[1], l[2], l[3]};
-}
-
 __device__ __forceinline__ tl_bf16x8 as_bf16x8(const tl_u32x4& v) { return __builtin_bit_cast(tl_bf16x8, v); }
 
 struct APlanes {
@@ -90,45 +63,85 @@ __device__ __forceinline__ APlanes split8(const tl_f32x4& c0, const tl_f32x4& c1
     return a;
 }
 
-// one 16-wide k step of a 32-row tile against the workgroup's 96 columns: 3 tiles x 6 products
-__device__ __forceinline__ void k_step(const APlanes& a, const tl_u32x4* wk, f32x16 (&acc)[3]) {
-    tl_bf16x8 bh[3], bm[3], bl[3];
+// The workgroup's 96 columns of W, split and laid out in LDS in operand order:
+// [k step][column tile 3][plane 3][lane 64][8 bf16]
+template <int THREADS>
+__device__ __forceinline__ void fill_w_planes(const float* __restrict__ w, int K, int ksteps, int cg, tl_u32x4* w_s) {
+    for (int it = threadIdx.x; it < ksteps * 3 * 64; it += THREADS) {
+        const int lane = it & 63, ct = (it >> 6) % 3, ks = (it >> 6) / 3;
+        const int col = cg * TL_COLS + ct * 32 + (lane & 31);
+        const tl_f32x4* src = reinterpret_cast<const tl_f32x4*>(w + (int64_t)col * K + ks * 16 + (lane >> 5) * 8);
+        const tl_f32x4 c0 = src[0], c1 = src[1];
+        const Split2 s0 = split2(c0.x, c0.y), s1 = split2(c0.z, c0.w), s2 = split2(c1.x, c1.y), s3 = split2(c1.z, c1.w);
+        tl_u32x4* dst = w_s + (ks * 3 + ct) * 3 * 64 + lane;
+        dst[0] = tl_u32x4{s0.h, s1.h, s2.h, s3.h};
+        dst[64] = tl_u32x4{s0.m, s1.m, s2.m, s3.m};
+        dst[128] = tl_u32x4{s0.l, s1.l, s2.l, s3.l};
+    }
+}
+
+// Workgroups b, b + 8, b + 16 ... run on the same XCD and share its L2: the column groups of one set
+// of rows are dealt to such workgroups, so X comes from HBM once.  Returns the column group and the
+// row slot (0 .. gridDim.x / groups - 1) of this workgroup.
+__device__ __forceinline__ void group_and_slot(int groups, int& cg, int& slot) {
+    const int b = blockIdx.x, chunk = 8 * groups, full = gridDim.x / chunk * chunk;
+    if (b < full) {
+        cg = (b / 8) % groups;
+        slot = b / chunk * 8 + b % 8;
+    } else {
+        cg = (b - full) % groups;
+        slot = full / groups + (b - full) / groups;
+    }
+}
+
+// the three planes of the workgroup's three column tiles for one k step, as read from LDS
+struct BPlanes {
+    tl_bf16x8 h[3], m[3], l[3];
+};
+__device__ __forceinline__ BPlanes read_b(const tl_u32x4* wk) {
+    BPlanes b;
 #pragma unroll
     for (int ct = 0; ct < 3; ++ct) {
-        bh[ct] = as_bf16x8(wk[(ct * 3 + 0) * 64]);
-        bm[ct] = as_bf16x8(wk[(ct * 3 + 1) * 64]);
-        bl[ct] = as_bf16x8(wk[(ct * 3 + 2) * 64]);
+        b.h[ct] = as_bf16x8(wk[(ct * 3 + 0) * 64]);
+        b.m[ct] = as_bf16x8(wk[(ct * 3 + 1) * 64]);
+        b.l[ct] = as_bf16x8(wk[(ct * 3 + 2) * 64]);
     }
-    // small terms first; the three column tiles alternate so that no product waits for the previous
-    // one into the same accumulator
+    return b;
+}
+
+// one 16-wide k step of a 32-row tile against the workgroup's 96 columns: 3 tiles x 6 products.
+// Small terms first; the three column tiles alternate so that no product waits for the previous one
+// into the same accumulator.
+__device__ __forceinline__ void k_products(const APlanes& a, const BPlanes& b, f32x16 (&acc)[3]) {
 #pragma unroll
-    for (int ct = 0; ct < 3; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.l, bh[ct], acc[ct], 0, 0, 0);
+    for (int ct = 0; ct < 3; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.l, b.h[ct], acc[ct], 0, 0, 0);
 #pragma unroll
-    for (int ct = 0; ct < 3; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.h, bl[ct], acc[ct], 0, 0, 0);
+    for (int ct = 0; ct < 3; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.h, b.l[ct], acc[ct], 0, 0, 0);
 #pragma unroll
-    for (int ct = 0; ct < 3; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.m, bm[ct], acc[ct], 0, 0, 0);
+    for (int ct = 0; ct < 3; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.m, b.m[ct], acc[ct], 0, 0, 0);
 #pragma unroll
-    for (int ct = 0; ct < 3; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.m, bh[ct], acc[ct], 0, 0, 0);
+    for (int ct = 0; ct < 3; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.m, b.h[ct], acc[ct], 0, 0, 0);
 #pragma unroll
-    for (int ct = 0; ct < 3; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.h, bm[ct], acc[ct], 0, 0, 0);
+    for (int ct = 0; ct < 3; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.h, b.m[ct], acc[ct], 0, 0, 0);
 #pragma unroll
-    for (int ct = 0; ct < 3; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.h, bh[ct], acc[ct], 0, 0, 0);
+    for (int ct = 0; ct < 3; ++ct) acc[ct] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.h, b.h[ct], acc[ct], 0, 0, 0);
+}
+__device__ __forceinline__ void k_step(const APlanes& a, const tl_u32x4* wk, f32x16 (&acc)[3]) {
+    k_products(a, read_b(wk), acc);
 }
 
 // any supported K; the next k step's 8 values are in flight during the current one
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) void tall_linear_forward_kernel(
-    const float* __restrict__ x, int64_t N, int K, const tl_u32x4* __restrict__ planes, int groups, const float* __restrict__ bias,
+    const float* __restrict__ x, int64_t N, int K, const float* __restrict__ w, int groups, const float* __restrict__ bias,
     float* __restrict__ y, int P, int64_t row_blocks) {
     extern __shared__ __attribute__((aligned(16))) tl_u32x4 w_s[];      // [k step][tile][plane][lane]
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int half = lane >> 5, l32 = lane & 31;
     const int ksteps = K / 16;
-    const int cg = blockIdx.x % groups;
-    const int64_t wg = blockIdx.x / groups, wgs = gridDim.x / groups;
-    // this group's planes: global -> LDS, once
-    const int n16 = ksteps * 9 * 64;
-    const tl_u32x4* src = planes + (int64_t)cg * n16;
-    for (int e = threadIdx.x; e < n16; e += 256) w_s[e] = src[e];
+    int cg, slot;
+    group_and_slot(groups, cg, slot);
+    const int64_t wg = slot, wgs = gridDim.x / groups;
+    fill_w_planes<256>(w, K, ksteps, cg, w_s);
     __syncthreads();
     float bcol[3];
 #pragma unroll
@@ -171,17 +184,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 constexpr int TL_STAGED_MAX_KS = 6;
 template <int KS>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void tall_linear_forward_staged_kernel(
-    const float* __restrict__ x, int64_t N, const tl_u32x4* __restrict__ planes, int groups, const float* __restrict__ bias,
+    const float* __restrict__ x, int64_t N, const float* __restrict__ w, int groups, const float* __restrict__ bias,
     float* __restrict__ y, int P, int64_t row_tiles) {
     constexpr int K = KS * 16, PITCH = K + 4, C4 = K / 4, NI = 2 * KS;   // 16-byte chunks per row; loads per lane and tile
     extern __shared__ __attribute__((aligned(16))) tl_u32x4 w_s[];      // [k step][tile][plane][lane], then the X tiles
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int half = lane >> 5, l32 = lane & 31;
-    const int cg = blockIdx.x % groups;
-    const int64_t first = (int64_t)(blockIdx.x / groups) * 8 + wave, stride = (int64_t)(gridDim.x / groups) * 8;
+    int cg, slot;
+    group_and_slot(groups, cg, slot);
+    const int64_t first = (int64_t)slot * 8 + wave, stride = (int64_t)(gridDim.x / groups) * 8;
     constexpr int n16 = KS * 9 * 64;
-    const tl_u32x4* src = planes + (int64_t)cg * n16;
-    for (int e = threadIdx.x; e < n16; e += 512) w_s[e] = src[e];
+    fill_w_planes<512>(w, K, KS, cg, w_s);
     float* xs = reinterpret_cast<float*>(w_s + n16) + wave * 32 * PITCH;
     __syncthreads();
     float bcol[3];
@@ -213,11 +226,19 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
         for (int ct = 0; ct < 3; ++ct) acc[ct] = f32x16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
         const float* xr = xs + l32 * PITCH + half * 8;
+        // the operands of step ks + 1 are read and split while the products of step ks run
+        APlanes a[2];
+        BPlanes b[2];
+        a[0] = split8(*reinterpret_cast<const tl_f32x4*>(xr), *reinterpret_cast<const tl_f32x4*>(xr + 4));
+        b[0] = read_b(w_s + lane);
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            const tl_f32x4 c0 = *reinterpret_cast<const tl_f32x4*>(xr + ks * 16);
-            const tl_f32x4 c1 = *reinterpret_cast<const tl_f32x4*>(xr + ks * 16 + 4);
-            k_step(split8(c0, c1), w_s + ks * 9 * 64 + lane, acc);
+            if (ks + 1 < KS) {
+                b[(ks + 1) & 1] = read_b(w_s + (ks + 1) * 9 * 64 + lane);
+                a[(ks + 1) & 1] = split8(*reinterpret_cast<const tl_f32x4*>(xr + (ks + 1) * 16),
+                                         *reinterpret_cast<const tl_f32x4*>(xr + (ks + 1) * 16 + 4));
+            }
+            k_products(a[ks & 1], b[ks & 1], acc);
             __builtin_amdgcn_sched_barrier(0);                           // keeps the operands of later steps out of registers
         }
 #pragma unroll
@@ -242,26 +263,21 @@ static int staged_lds_bytes(int ksteps) {
 
 extern "C" {
 
-size_t sswin_tall_linear_workspace_bytes(int P, int K) {
-    if (P <= 0 || K <= 0 || (P % TL_COLS) || (K % 16) || K > TL_MAX_K) return 0;
-    return (size_t)(P / TL_COLS) * (K / 16) * 9 * 64 * sizeof(tl_u32x4) + 256;
+int sswin_tall_linear_supported(int P, int K) {
+    return P > 0 && K > 0 && (P % TL_COLS) == 0 && (K % 16) == 0 && K <= TL_MAX_K;
 }
 
 int sswin_tall_linear_forward(const float* x, int64_t N, int K, const float* w, const float* bias, int P, float* y,
-                              void* ws, size_t ws_bytes, void* stream) {
+                              void* stream) {
     SSWIN_CHECK(N >= 0 && K > 0 && P > 0, "tall_linear_forward: bad sizes");
     SSWIN_CHECK(K % 16 == 0 && K <= TL_MAX_K, "tall_linear_forward: %d input channels are not supported (a multiple of 16, at most %d)",
                 K, TL_MAX_K);
     SSWIN_CHECK(P % TL_COLS == 0, "tall_linear_forward: %d output channels are not a multiple of %d", P, TL_COLS);
     if (N == 0) return 0;
-    SSWIN_CHECK(x && w && y && ws, "tall_linear_forward: null pointer");
-    SSWIN_CHECK(((uintptr_t)x % 16) == 0 && ((uintptr_t)ws % 16) == 0, "tall_linear_forward: x and the workspace must be 16-byte aligned");
-    SSWIN_CHECK(ws_bytes >= sswin_tall_linear_workspace_bytes(P, K), "tall_linear_forward: workspace too small");
+    SSWIN_CHECK(x && w && y, "tall_linear_forward: null pointer");
+    SSWIN_CHECK(((uintptr_t)x % 16) == 0 && ((uintptr_t)w % 16) == 0, "tall_linear_forward: x and w must be 16-byte aligned");
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int groups = P / TL_COLS, ksteps = K / 16;
-    tl_u32x4* planes = static_cast<tl_u32x4*>(ws);
-    const int64_t prep = (int64_t)groups * ksteps * 3 * 64;
-    hipLaunchKernelGGL(tall_linear_prepare_kernel, dim3((unsigned)((prep + 255) / 256)), dim3(256), 0, s, w, P, K, planes);
     int cus = 256;
     {
         int dev = 0, n = 0;
@@ -291,7 +307,7 @@ int sswin_tall_linear_forward(const float* x, int64_t N, int K, const float* w, 
         const size_t lds = staged_lds_bytes(ksteps);
 #define SSWIN_TL_STAGED(KS)                                                                                                  \
     case KS:                                                                                                                 \
-        hipLaunchKernelGGL(tall_linear_forward_staged_kernel<KS>, grid, block, lds, s, x, N, planes, groups, bias, y, P,     \
+        hipLaunchKernelGGL(tall_linear_forward_staged_kernel<KS>, grid, block, lds, s, x, N, w, groups, bias, y, P,          \
                            row_tiles);                                                                                       \
         break;
         switch (ksteps) {
@@ -304,8 +320,8 @@ int sswin_tall_linear_forward(const float* x, int64_t N, int K, const float* w, 
     const int64_t row_blocks = (N + 127) / 128;
     const int per_cu = lds <= 64 * 1024 ? 2 : 1;                          // workgroups that fit a CU's LDS
     int64_t per_group = std::min<int64_t>(row_blocks, std::max<int64_t>(1, (int64_t)cus * per_cu / groups));
-    hipLaunchKernelGGL(tall_linear_forward_kernel, dim3((unsigned)(per_group * groups)), dim3(256), lds, s, x, N, K, planes,
-                       groups, bias, y, P, row_blocks);
+    hipLaunchKernelGGL(tall_linear_forward_kernel, dim3((unsigned)(per_group * groups)), dim3(256), lds, s, x, N, K, w, groups,
+                       bias, y, P, row_blocks);
     return launch_ok("tall_linear_forward");
 }
 

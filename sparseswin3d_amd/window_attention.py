@@ -268,20 +268,20 @@ def _split_linear_forward(x: torch.Tensor, weight: torch.Tensor, bias):
     lib = _lib.load()
     n, k = x.shape
     p = weight.shape[0]
-    nbytes = int(lib.sswin_tall_linear_workspace_bytes(p, k))
-    if nbytes == 0:
+    if not lib.sswin_tall_linear_supported(p, k):
         return None
     x = x.contiguous()
     weight = weight.contiguous()
     if x.data_ptr() % 16:
         x = x.clone()
+    if weight.data_ptr() % 16:
+        weight = weight.clone()
     with torch.cuda.device(x.device):
         y = torch.empty(n, p, dtype=torch.float32, device=x.device)
-        ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
         b = bias.contiguous() if bias is not None else None
         _lib.check(lib.sswin_tall_linear_forward(C.c_void_p(x.data_ptr()), n, k, C.c_void_p(weight.data_ptr()),
                                                  C.c_void_p(b.data_ptr() if b is not None else None), p,
-                                                 C.c_void_p(y.data_ptr()), C.c_void_p(ws.data_ptr()), nbytes,
+                                                 C.c_void_p(y.data_ptr()),
                                                  C.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)))
     return y
 

@@ -19,15 +19,12 @@ TOL = 1e-6          # of sum_k |x_ik w_jk|
 def _run(lib, _lib, x, w, b):
     N, K = x.shape
     P = w.shape[0]
-    nb = int(lib.sswin_tall_linear_workspace_bytes(P, K))
-    assert nb > 0
-    ws = torch.empty(nb, dtype=torch.uint8, device="cuda")
+    assert lib.sswin_tall_linear_supported(P, K)
     y = torch.full((N, P), float("nan"), device="cuda")
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
-    for _ in range(2):                                  # a second call over the same workspace
-        _lib.check(lib.sswin_tall_linear_forward(C.c_void_p(x.data_ptr()), N, K, C.c_void_p(w.data_ptr()),
-                                                 C.c_void_p(b.data_ptr() if b is not None else None), P,
-                                                 C.c_void_p(y.data_ptr()), C.c_void_p(ws.data_ptr()), nb, stream))
+    _lib.check(lib.sswin_tall_linear_forward(C.c_void_p(x.data_ptr()), N, K, C.c_void_p(w.data_ptr()),
+                                             C.c_void_p(b.data_ptr() if b is not None else None), P,
+                                             C.c_void_p(y.data_ptr()), stream))
     torch.cuda.synchronize()
     return y
 
@@ -80,15 +77,15 @@ def test_tall_linear_exact_cases():
 def test_tall_linear_rejects_unsupported_shapes():
     from sparseswin3d_amd import _lib
     lib = _lib.load()
-    assert lib.sswin_tall_linear_workspace_bytes(100, 96) == 0       # columns not a multiple of 96
-    assert lib.sswin_tall_linear_workspace_bytes(96, 100) == 0       # channels not a multiple of 16
-    assert lib.sswin_tall_linear_workspace_bytes(96, 384) == 0       # too many channels
+    assert lib.sswin_tall_linear_supported(288, 96) == 1
+    assert lib.sswin_tall_linear_supported(100, 96) == 0             # columns not a multiple of 96
+    assert lib.sswin_tall_linear_supported(96, 100) == 0             # channels not a multiple of 16
+    assert lib.sswin_tall_linear_supported(96, 384) == 0             # too many channels
     x = torch.zeros(8, 100, device="cuda")
     w = torch.zeros(96, 100, device="cuda")
     y = torch.zeros(8, 96, device="cuda")
-    ws = torch.zeros(1024, dtype=torch.uint8, device="cuda")
     rc = lib.sswin_tall_linear_forward(C.c_void_p(x.data_ptr()), 8, 100, C.c_void_p(w.data_ptr()), None, 96,
-                                       C.c_void_p(y.data_ptr()), C.c_void_p(ws.data_ptr()), 1024, None)
+                                       C.c_void_p(y.data_ptr()), None)
     assert rc != 0
     with pytest.raises(RuntimeError, match="input channels"):
         _lib.check(rc)
