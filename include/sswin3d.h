@@ -243,6 +243,15 @@ int sswin_tall_linear_supported(int P, int K);
 int sswin_tall_linear_forward(const float* x, int64_t N, int K, const float* w, const float* bias,
                               int P, float* y, void* stream);
 
+/* dw[P,K] = dy[N,P]^T x[N,K] and, when db is not NULL, db[P] = column sums of dy: weight and bias
+ * gradient of the same layers (autograd of nn.Linear, swin3d_base.py:606-610).  fp32, P a multiple
+ * of 96, K = 32, 64 or 96 (the workspace size is 0 for anything else).  Same split-operand
+ * arithmetic as the forward; partial sums per workgroup are added in a fixed order, so the result
+ * is the same on every run.  dw, db and ws 16-byte aligned.  Asynchronous. */
+size_t sswin_tall_linear_weight_grad_workspace_bytes(int64_t N, int P, int K);
+int sswin_tall_linear_weight_grad(const float* dy, const float* x, int64_t N, int P, int K, float* dw,
+                                  float* db, void* ws, size_t ws_bytes, void* stream);
+
 /* ---- window-resident attention (whole forward / backward of the attention core) ---------- */
 
 /* Forward of sparse_swin/swin3d_base.py:660-672 for every (window, head) group in one pass:

@@ -253,6 +253,171 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     }
 }
 
+// ------------------------------------------------------------------------------------------
+// Weight and bias gradient of the same layers: dW[P,K] = dY^T X, db[P] = column sums of dY, for
+// dY [N,P] and X [N,K] (autograd of the nn.Linear at swin3d_base.py:606-610).
+//
+// The reduction runs over the rows, so both operands carry rows in their k slots: a lane reads 8 rows
+// of one column with 8 dword loads (32 lanes = 128 contiguous bytes of a row) and splits them in
+// registers.  A workgroup has 12 waves = 4 row quarters x 3 waves; a wave owns one 32-column tile of dY
+// (within the workgroup's group of 96 columns of dY) against all of X's column tiles.  The split planes
+// of X are shared among the 3 waves of a quarter through LDS (each wave splits one tile of X), double
+// buffered with one barrier per 16-row step.  The quarters are added through LDS at the end in a
+// fixed order, every workgroup writes one partial dW / db, and a second kernel adds the partials in
+// workgroup order: no atomics, the same bits on every run.
+// ------------------------------------------------------------------------------------------
+constexpr int WG_QUARTERS = 4, WG_WAVES = 12, WG_STEP_ROWS = 16 * WG_QUARTERS;
+
+struct Raw8 {
+    float v[8];
+};
+// 8 rows (slot e of k group kg = row r0 + 8 kg + e) of column `col`; rows past N read as zero
+__device__ __forceinline__ Raw8 load_rows8(const float* __restrict__ base, int64_t pitch, int64_t r0, int64_t N, int col,
+                                           int half) {
+    Raw8 o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        const int64_t row = r0 + half * 8 + e;
+        o.v[e] = row < N ? base[row * pitch + col] : 0.f;
+    }
+    return o;
+}
+__device__ __forceinline__ APlanes split_raw8(const Raw8& r) {
+    const Split2 s0 = split2(r.v[0], r.v[1]), s1 = split2(r.v[2], r.v[3]), s2 = split2(r.v[4], r.v[5]), s3 = split2(r.v[6], r.v[7]);
+    APlanes a;
+    a.h = as_bf16x8(tl_u32x4{s0.h, s1.h, s2.h, s3.h});
+    a.m = as_bf16x8(tl_u32x4{s0.m, s1.m, s2.m, s3.m});
+    a.l = as_bf16x8(tl_u32x4{s0.l, s1.l, s2.l, s3.l});
+    return a;
+}
+
+// XT = K / 32 column tiles of X (1..3)
+template <int XT>
+__global__ __launch_bounds__(WG_WAVES * 64) __attribute__((amdgpu_waves_per_eu(3, 3))) void tall_linear_wgrad_kernel(
+    const float* __restrict__ dy, const float* __restrict__ x, int64_t N, int P, int groups, int64_t rows_per_chunk,
+    float* __restrict__ part_w, float* __restrict__ part_b) {
+    constexpr int K = XT * 32;
+    // X planes: [buffer 2][quarter 4][tile XT][plane 3][lane 64] x 16 bytes; reused for the final sums
+    extern __shared__ __attribute__((aligned(16))) tl_u32x4 lds[];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int half = lane >> 5, l32 = lane & 31;
+    const int quarter = wave / 3, t = wave % 3;                          // t: this wave's column tile of dY (and of X)
+    int g, chunk;
+    group_and_slot(groups, g, chunk);                                    // the groups of one row chunk share an XCD's L2
+    const int64_t row_begin = (int64_t)chunk * rows_per_chunk;
+    const int64_t row_end = row_begin + rows_per_chunk < N ? row_begin + rows_per_chunk : N;
+    const int steps = (int)((row_end - row_begin + WG_STEP_ROWS - 1) / WG_STEP_ROWS);
+    const int ycol = g * 96 + t * 32 + l32, xcol = t * 32 + l32;
+    constexpr int BUF = WG_QUARTERS * XT * 3 * 64;                       // 16-byte units per buffer
+
+    f32x16 acc[XT];
+#pragma unroll
+    for (int xt = 0; xt < XT; ++xt) acc[xt] = f32x16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    float bsum = 0.f;
+    // rows are requested two steps ahead (loaded HBM latency is about two steps of products)
+    Raw8 ry[2], rx[2];
+    auto fetch = [&](int s, Raw8& y8, Raw8& x8) {
+        const int64_t r0 = row_begin + (int64_t)s * WG_STEP_ROWS + quarter * 16;
+        y8 = load_rows8(dy, P, r0, row_end, ycol, half);
+        if (t < XT) x8 = load_rows8(x, K, r0, row_end, xcol, half);
+    };
+    auto step = [&](int s, Raw8& y8, Raw8& x8) {
+        tl_u32x4* buf = lds + (s & 1) * BUF + quarter * XT * 3 * 64;
+        if (t < XT) {
+            const APlanes xp = split_raw8(x8);
+            tl_u32x4* dst = buf + t * 3 * 64 + lane;
+            dst[0] = __builtin_bit_cast(tl_u32x4, xp.h);
+            dst[64] = __builtin_bit_cast(tl_u32x4, xp.m);
+            dst[128] = __builtin_bit_cast(tl_u32x4, xp.l);
+        }
+        const APlanes a = split_raw8(y8);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) bsum += y8.v[e];
+        if (s + 2 < steps) fetch(s + 2, y8, x8);
+        __syncthreads();
+#pragma unroll
+        for (int xt = 0; xt < XT; ++xt) {
+            const tl_bf16x8 bh = as_bf16x8(buf[(xt * 3 + 0) * 64 + lane]);
+            const tl_bf16x8 bm = as_bf16x8(buf[(xt * 3 + 1) * 64 + lane]);
+            const tl_bf16x8 bl = as_bf16x8(buf[(xt * 3 + 2) * 64 + lane]);
+            acc[xt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.l, bh, acc[xt], 0, 0, 0);
+            acc[xt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.h, bl, acc[xt], 0, 0, 0);
+            acc[xt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.m, bm, acc[xt], 0, 0, 0);
+            acc[xt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.m, bh, acc[xt], 0, 0, 0);
+            acc[xt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.h, bm, acc[xt], 0, 0, 0);
+            acc[xt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.h, bh, acc[xt], 0, 0, 0);
+        }
+    };
+    fetch(0, ry[0], rx[0]);
+    if (steps > 1) fetch(1, ry[1], rx[1]);
+    for (int s = 0; s < steps; s += 2) {
+        step(s, ry[0], rx[0]);
+        if (s + 1 < steps) step(s + 1, ry[1], rx[1]);
+    }
+    // quarters: (0 + 2) + (1 + 3), through LDS; values of a wave at [slot][value][lane]
+    float* red = reinterpret_cast<float*>(lds);
+    constexpr int VALS = XT * 16 + 1;                                    // accumulators and the bias sum
+    auto put = [&](int slot) {
+        float* dst = red + (slot * VALS) * 64 + lane;
+#pragma unroll
+        for (int xt = 0; xt < XT; ++xt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) dst[(xt * 16 + r) * 64] = acc[xt][r];
+        dst[XT * 16 * 64] = bsum;
+    };
+    auto add = [&](int slot) {
+        const float* src = red + (slot * VALS) * 64 + lane;
+#pragma unroll
+        for (int xt = 0; xt < XT; ++xt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[xt][r] += src[(xt * 16 + r) * 64];
+        bsum += src[XT * 16 * 64];
+    };
+    __syncthreads();
+    if (quarter >= 2) put((quarter - 2) * 3 + t);
+    __syncthreads();
+    if (quarter < 2) add(quarter * 3 + t);
+    __syncthreads();
+    if (quarter == 1) put(t);
+    __syncthreads();
+    if (quarter == 0) {
+        add(t);
+        float* pw = part_w + (int64_t)chunk * P * K + (int64_t)(g * 96 + t * 32) * K + l32;
+#pragma unroll
+        for (int xt = 0; xt < XT; ++xt)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) pw[(int64_t)acc_row(r, half) * K + xt * 32] = acc[xt][r];
+        bsum += __shfl_xor(bsum, 32);                                    // the two k groups of a column
+        if (half == 0) part_b[(int64_t)chunk * P + ycol] = bsum;
+    }
+}
+
+// out[e] = sum over chunks of part[chunk][e].  A block handles 16 x 4 consecutive outputs; 16 threads
+// share an output quadruple, each adds every 16th chunk in order, and the 16 sums are added in a fixed
+// tree.  part_w and part_b are contiguous ([chunks][PK] then [chunks][P]), so e runs over both.
+__global__ __launch_bounds__(256) void tall_linear_wgrad_reduce_kernel(const float* __restrict__ part_w,
+                                                                       const float* __restrict__ part_b, int chunks, int PK,
+                                                                       int P, float* __restrict__ dw, float* __restrict__ db) {
+    __shared__ tl_f32x4 sums[16][17];
+    const int el = threadIdx.x & 15, cl = threadIdx.x >> 4;
+    const int e = (blockIdx.x * 16 + el) * 4;
+    const bool weight = e < PK, valid = weight || (db && e - PK < P);
+    tl_f32x4 sum = {0.f, 0.f, 0.f, 0.f};
+    if (valid) {
+        const float* src = weight ? part_w + e : part_b + (e - PK);
+        const int64_t pitch = weight ? PK : P;
+        for (int c = cl; c < chunks; c += 16) sum += *reinterpret_cast<const tl_f32x4*>(src + c * pitch);
+    }
+    sums[cl][el] = sum;
+    __syncthreads();
+#pragma unroll
+    for (int w = 8; w >= 1; w >>= 1) {
+        if (cl < w) sums[cl][el] += sums[cl + w][el];
+        __syncthreads();
+    }
+    if (cl == 0 && valid) *reinterpret_cast<tl_f32x4*>(weight ? dw + e : db + (e - PK)) = sums[0][el];
+}
+
 }  // namespace sswin
 
 using namespace sswin;
@@ -323,6 +488,78 @@ int sswin_tall_linear_forward(const float* x, int64_t N, int K, const float* w, 
     hipLaunchKernelGGL(tall_linear_forward_kernel, dim3((unsigned)(per_group * groups)), dim3(256), lds, s, x, N, K, w, groups,
                        bias, y, P, row_blocks);
     return launch_ok("tall_linear_forward");
+}
+
+}  // extern "C"
+
+static void wgrad_split(int64_t N, int groups, int cus, int64_t* rows_per_chunk, int* chunks) {
+    const int64_t want = std::max<int64_t>(1, cus / groups);
+    int64_t rows = (N + want - 1) / want;
+    rows = std::max<int64_t>(WG_STEP_ROWS, (rows + WG_STEP_ROWS - 1) / WG_STEP_ROWS * WG_STEP_ROWS);
+    *rows_per_chunk = rows;
+    *chunks = (int)std::max<int64_t>(1, (N + rows - 1) / rows);
+}
+
+static int device_cus() {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess &&
+        n > 0)
+        return n;
+    return 256;
+}
+
+extern "C" {
+
+size_t sswin_tall_linear_weight_grad_workspace_bytes(int64_t N, int P, int K) {
+    if (N <= 0 || P <= 0 || K <= 0 || (P % 96) || (K % 32) || K > 96) return 0;
+    int64_t rows;
+    int chunks;
+    wgrad_split(N, P / 96, device_cus(), &rows, &chunks);
+    return (size_t)chunks * ((size_t)P * K + P) * sizeof(float) + 256;
+}
+
+int sswin_tall_linear_weight_grad(const float* dy, const float* x, int64_t N, int P, int K, float* dw, float* db, void* ws,
+                                  size_t ws_bytes, void* stream) {
+    SSWIN_CHECK(N > 0 && P > 0 && K > 0, "tall_linear_weight_grad: bad sizes");
+    SSWIN_CHECK(P % 96 == 0, "tall_linear_weight_grad: %d output channels are not a multiple of 96", P);
+    SSWIN_CHECK(K % 32 == 0 && K <= 96, "tall_linear_weight_grad: %d input channels are not supported (32, 64 or 96)", K);
+    SSWIN_CHECK(dy && x && dw && ws, "tall_linear_weight_grad: null pointer");
+    SSWIN_CHECK(((uintptr_t)dw % 16) == 0 && ((uintptr_t)db % 16) == 0 && ((uintptr_t)ws % 16) == 0,
+                "tall_linear_weight_grad: dw, db and the workspace must be 16-byte aligned");
+    SSWIN_CHECK(ws_bytes >= sswin_tall_linear_weight_grad_workspace_bytes(N, P, K), "tall_linear_weight_grad: workspace too small");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int groups = P / 96, xt = K / 32;
+    int64_t rows;
+    int chunks;
+    wgrad_split(N, groups, device_cus(), &rows, &chunks);
+    float* part_w = static_cast<float*>(ws);
+    float* part_b = part_w + (size_t)chunks * P * K;
+    // LDS: the double-buffered planes of X, or the two rounds of the final sums, whichever is larger
+    const size_t planes = 2 * (size_t)WG_QUARTERS * xt * 3 * 64 * sizeof(tl_u32x4);
+    const size_t sums = 6 * (size_t)(xt * 16 + 1) * 64 * sizeof(float);
+    const size_t lds = std::max(planes, sums);
+    static bool configured = false;
+    if (!configured) {
+        const int max_lds = 96 * 1024;
+        SSWIN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(tall_linear_wgrad_kernel<1>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, max_lds));
+        SSWIN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(tall_linear_wgrad_kernel<2>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, max_lds));
+        SSWIN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(tall_linear_wgrad_kernel<3>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, max_lds));
+        configured = true;
+    }
+    const dim3 grid((unsigned)(chunks * groups)), block(WG_WAVES * 64);
+    switch (xt) {
+        case 1: hipLaunchKernelGGL(tall_linear_wgrad_kernel<1>, grid, block, lds, s, dy, x, N, P, groups, rows, part_w, part_b); break;
+        case 2: hipLaunchKernelGGL(tall_linear_wgrad_kernel<2>, grid, block, lds, s, dy, x, N, P, groups, rows, part_w, part_b); break;
+        default: hipLaunchKernelGGL(tall_linear_wgrad_kernel<3>, grid, block, lds, s, dy, x, N, P, groups, rows, part_w, part_b); break;
+    }
+    if (int rc = launch_ok("tall_linear_weight_grad")) return rc;
+    const int PK = P * K, total4 = (PK + P) / 4;
+    hipLaunchKernelGGL(tall_linear_wgrad_reduce_kernel, dim3((unsigned)((total4 + 15) / 16)), dim3(256), 0, s, part_w, part_b, chunks,
+                       PK, P, dw, db);
+    return launch_ok("tall_linear_weight_grad reduce");
 }
 
 }  // extern "C"

@@ -286,6 +286,34 @@ def _split_linear_forward(x: torch.Tensor, weight: torch.Tensor, bias):
     return y
 
 
+def _split_linear_weight_grad(grad_out: torch.Tensor, x: torch.Tensor, want_bias: bool):
+    """``(grad_out^T @ x, grad_out.sum(0))`` through the library's matrix-core kernel for fp32 (one
+    pass over both operands, partial sums added in a fixed order), or ``(None, None)`` when the shape
+    or dtype is outside what that kernel takes."""
+    if not (x.is_cuda and x.dtype == torch.float32 and grad_out.dtype == torch.float32 and x.dim() == 2
+            and grad_out.dim() == 2 and x.shape[0] > 0):
+        return None, None
+    import ctypes as C
+    from . import _lib
+    lib = _lib.load()
+    n, k = x.shape
+    p = grad_out.shape[1]
+    nbytes = int(lib.sswin_tall_linear_weight_grad_workspace_bytes(n, p, k))
+    if nbytes == 0:
+        return None, None
+    x = x.contiguous()
+    with torch.cuda.device(x.device):
+        dw = torch.empty(p, k, dtype=torch.float32, device=x.device)
+        db = torch.empty(p, dtype=torch.float32, device=x.device) if want_bias else None
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
+        _lib.check(lib.sswin_tall_linear_weight_grad(C.c_void_p(grad_out.data_ptr()), C.c_void_p(x.data_ptr()), n, p, k,
+                                                     C.c_void_p(dw.data_ptr()),
+                                                     C.c_void_p(db.data_ptr() if db is not None else None),
+                                                     C.c_void_p(ws.data_ptr()), nbytes,
+                                                     C.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)))
+    return dw, db
+
+
 class _TallLinear(Function):
     """``x @ W^T + b`` for a very tall ``x`` [N, in] (N = number of voxels).  The fp32 forward runs on
     the bf16 matrix cores with exactly split operands where the shape allows; input gradient and
@@ -308,12 +336,15 @@ class _TallLinear(Function):
         x, weight = ctx.saved_tensors
         grad_out = grad_out.contiguous()
         grad_x = grad_w = grad_b = None
+        want_b = ctx.has_bias and ctx.needs_input_grad[2]
+        if ctx.needs_input_grad[1]:
+            grad_w, grad_b = _split_linear_weight_grad(grad_out, x, want_b)
         with _rocblas_gemm():
             if ctx.needs_input_grad[0]:
                 grad_x = grad_out @ weight
-            if ctx.needs_input_grad[1]:
+            if ctx.needs_input_grad[1] and grad_w is None:
                 grad_w = grad_out.t() @ x
-        if ctx.has_bias and ctx.needs_input_grad[2]:
+        if want_b and grad_b is None:
             grad_b = _column_sum(grad_out)
         return grad_x, grad_w, grad_b
 

@@ -91,9 +91,61 @@ def test_tall_linear_rejects_unsupported_shapes():
         _lib.check(rc)
 
 
+@pytest.mark.parametrize("N,K,P,bias", [
+    (107500, 96, 288, True), (107500, 96, 96, True), (1, 96, 96, True), (63, 32, 96, False), (65, 64, 192, True),
+    (1000, 96, 96, True), (4099, 96, 288, False), (20000, 32, 288, True),
+])
+def test_tall_linear_weight_grad(N, K, P, bias):
+    """dW = dY^T X and db = column sums of dY against float64 on the same fp32 inputs; the same bits on
+    a second call (partial sums are added in a fixed order)."""
+    from sparseswin3d_amd import _lib
+    lib = _lib.load()
+    g = torch.Generator().manual_seed(N + 3 * K + P)
+    x = (torch.randn(N, K, generator=g) * torch.exp2(torch.randint(-4, 5, (N, K), generator=g).float())).cuda()
+    dy = (torch.randn(N, P, generator=g) * torch.exp2(torch.randint(-4, 5, (N, P), generator=g).float())).cuda()
+    nb = int(lib.sswin_tall_linear_weight_grad_workspace_bytes(N, P, K))
+    assert nb > 0
+    ws = torch.empty(nb, dtype=torch.uint8, device="cuda")
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    outs = []
+    for _ in range(2):
+        dw = torch.full((P, K), float("nan"), device="cuda")
+        db = torch.full((P,), float("nan"), device="cuda") if bias else None
+        _lib.check(lib.sswin_tall_linear_weight_grad(C.c_void_p(dy.data_ptr()), C.c_void_p(x.data_ptr()), N, P, K,
+                                                     C.c_void_p(dw.data_ptr()),
+                                                     C.c_void_p(db.data_ptr() if bias else None),
+                                                     C.c_void_p(ws.data_ptr()), nb, stream))
+        torch.cuda.synchronize()
+        outs.append((dw, db))
+    dw, db = outs[0]
+    assert torch.equal(dw, outs[1][0])
+    ref = dy.double().T @ x.double()
+    scale = dy.double().abs().T @ x.double().abs()
+    assert ((dw.double() - ref).abs() / scale).max().item() < TOL
+    if bias:
+        assert torch.equal(db, outs[1][1])
+        refb = dy.double().sum(0)
+        assert ((db.double() - refb).abs() / dy.double().abs().sum(0)).max().item() < TOL
+
+
+def test_tall_linear_weight_grad_unsupported_shapes():
+    from sparseswin3d_amd import _lib
+    lib = _lib.load()
+    assert lib.sswin_tall_linear_weight_grad_workspace_bytes(1000, 100, 96) == 0
+    assert lib.sswin_tall_linear_weight_grad_workspace_bytes(1000, 96, 192) == 0
+    assert lib.sswin_tall_linear_weight_grad_workspace_bytes(1000, 96, 48) == 0
+    assert lib.sswin_tall_linear_weight_grad_workspace_bytes(0, 96, 96) == 0
+    t = torch.zeros(64, 96, device="cuda")
+    rc = lib.sswin_tall_linear_weight_grad(C.c_void_p(t.data_ptr()), C.c_void_p(t.data_ptr()), 64, 96, 48,
+                                           C.c_void_p(t.data_ptr()), None, C.c_void_p(t.data_ptr()), 1024, None)
+    assert rc != 0
+    with pytest.raises(RuntimeError, match="input channels"):
+        _lib.check(rc)
+
+
 def test_module_projection_matches_library_gemm():
-    """tall_linear() of the module: forward through the kernel, gradients through the library; both
-    against nn.Linear in float64."""
+    """tall_linear() of the module (forward, weight and bias gradient through the kernels, input
+    gradient through the library) against nn.Linear in float64."""
     from sparseswin3d_amd.window_attention import tall_linear
     torch.manual_seed(5)
     layer = torch.nn.Linear(96, 288).cuda()
