@@ -243,6 +243,13 @@ int sswin_tall_linear_supported(int P, int K);
 int sswin_tall_linear_forward(const float* x, int64_t N, int K, const float* w, const float* bias,
                               int P, float* y, void* stream);
 
+/* dx[N,K] = dy[N,P] w[P,K]: input gradient of the same layers (autograd of nn.Linear,
+ * swin3d_base.py:606-610).  fp32, P and K multiples of 96 (sswin_tall_linear_input_grad_supported
+ * tells); same split-operand arithmetic as the forward.  dy 16-byte aligned.  Asynchronous. */
+int sswin_tall_linear_input_grad_supported(int P, int K);
+int sswin_tall_linear_input_grad(const float* dy, int64_t N, int P, const float* w, int K, float* dx,
+                                 void* stream);
+
 /* dw[P,K] = dy[N,P]^T x[N,K] and, when db is not NULL, db[P] = column sums of dy: weight and bias
  * gradient of the same layers (autograd of nn.Linear, swin3d_base.py:606-610).  fp32, P a multiple
  * of 96, K = 32, 64 or 96 (the workspace size is 0 for anything else).  Same split-operand

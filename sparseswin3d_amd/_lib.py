@@ -50,6 +50,8 @@ SIGNATURES = {
     "sswin_bias_table_grad": (_i32, [_vp, _i64, _i64, _vp, _i64, _i32, _i32, _vp, _i32, _i32, _vp, _vp, _vp, _sz, _vp]),
     "sswin_tall_linear_supported": (_i32, [_i32, _i32]),
     "sswin_tall_linear_forward": (_i32, [_vp, _i64, _i32, _vp, _vp, _i32, _vp, _vp]),
+    "sswin_tall_linear_input_grad_supported": (_i32, [_i32, _i32]),
+    "sswin_tall_linear_input_grad": (_i32, [_vp, _i64, _i32, _vp, _i32, _vp, _vp]),
     "sswin_tall_linear_weight_grad_workspace_bytes": (_sz, [_i64, _i32, _i32]),
     "sswin_tall_linear_weight_grad": (_i32, [_vp, _vp, _i64, _i32, _i32, _vp, _vp, _vp, _sz, _vp]),
     "sswin_window_indices": (_i32, [_vp, _i64, _i32, _vp, _vp, _vp, _vp, _vp]),
@@ -65,7 +67,7 @@ SIGNATURES = {
                                                _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i32, _vp]),
 }
 
-ABI_VERSION = 11
+ABI_VERSION = 12
 _lib = None
 
 

@@ -254,6 +254,129 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 }
 
 // ------------------------------------------------------------------------------------------
+// More than 96 input channels: y[N, 96 G] = x[N, 96 C] Wop, C chunks of 96 channels, accumulators kept
+// in registers over the chunks.  The planes of one chunk of W (54 KB) are double buffered in LDS: the
+// values of the next chunk are requested before the products of the current one and split and
+// stored after them, one barrier per chunk.  One workgroup of 8 waves per CU, one 32-row tile per
+// wave; the lane's 48 values of the next chunk of X are in flight during the products.
+// TRANSPOSED: Wop[k][col] = w[k * out + col] (input gradient dX = dY W of the layer, W [P, K] as
+// stored); otherwise Wop[k][col] = w[col * in + k] (the forward with W [P, K]).
+// ------------------------------------------------------------------------------------------
+constexpr int CH_KS = 6, CH_ITEMS = CH_KS * 3 * 64, CH_SLOTS = (CH_ITEMS + 511) / 512;
+
+template <bool TRANSPOSED>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void tall_linear_chunked_kernel(
+    const float* __restrict__ x, int64_t N, int in, const float* __restrict__ w, int groups, const float* __restrict__ bias,
+    float* __restrict__ y, int out, int64_t row_tiles) {
+    extern __shared__ __attribute__((aligned(16))) tl_u32x4 w_s[];      // [buffer 2][k step 6][tile 3][plane 3][lane 64]
+    constexpr int BUF = CH_KS * 9 * 64;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int half = lane >> 5, l32 = lane & 31;
+    const int chunks = in / 96;
+    int cg, slot;
+    group_and_slot(groups, cg, slot);
+    const int64_t first = (int64_t)slot * 8 + wave, stride = (int64_t)(gridDim.x / groups) * 8;
+    // every wave of the workgroup runs the same number of rounds (barriers inside)
+    const int64_t wg_first = (int64_t)slot * 8;
+    const int rounds = wg_first < row_tiles ? (int)((row_tiles - wg_first + stride - 1) / stride) : 0;
+
+    // --- the chunk of W that comes next: raw values in registers, then planes in LDS
+    float wraw[CH_SLOTS][8];
+    auto w_request = [&](int chunk) {
+#pragma unroll
+        for (int q = 0; q < CH_SLOTS; ++q) {
+            const int it = threadIdx.x + q * 512;
+            if (it < CH_ITEMS) {
+                const int ln = it & 63, ct = (it >> 6) % 3, ks = (it >> 6) / 3;
+                const int col = cg * TL_COLS + ct * 32 + (ln & 31), k0 = chunk * 96 + ks * 16 + (ln >> 5) * 8;
+                if (TRANSPOSED) {
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) wraw[q][e] = w[(int64_t)(k0 + e) * out + col];
+                } else {
+                    const tl_f32x4* src = reinterpret_cast<const tl_f32x4*>(w + (int64_t)col * in + k0);
+                    const tl_f32x4 c0 = src[0], c1 = src[1];
+                    wraw[q][0] = c0.x; wraw[q][1] = c0.y; wraw[q][2] = c0.z; wraw[q][3] = c0.w;
+                    wraw[q][4] = c1.x; wraw[q][5] = c1.y; wraw[q][6] = c1.z; wraw[q][7] = c1.w;
+                }
+            }
+        }
+    };
+    auto w_store = [&](tl_u32x4* buf) {
+#pragma unroll
+        for (int q = 0; q < CH_SLOTS; ++q) {
+            const int it = threadIdx.x + q * 512;
+            if (it < CH_ITEMS) {
+                const Split2 s0 = split2(wraw[q][0], wraw[q][1]), s1 = split2(wraw[q][2], wraw[q][3]);
+                const Split2 s2 = split2(wraw[q][4], wraw[q][5]), s3 = split2(wraw[q][6], wraw[q][7]);
+                tl_u32x4* dst = buf + (it >> 6) * 3 * 64 + (it & 63);
+                dst[0] = tl_u32x4{s0.h, s1.h, s2.h, s3.h};
+                dst[64] = tl_u32x4{s0.m, s1.m, s2.m, s3.m};
+                dst[128] = tl_u32x4{s0.l, s1.l, s2.l, s3.l};
+            }
+        }
+    };
+    // --- the lane's 48 values of one chunk of its row (row l % 32 of the tile, k group l / 32)
+    tl_f32x4 xn[CH_KS][2];
+    auto x_request = [&](int64_t tile, int chunk) {
+        int64_t row = tile * 32 + l32;
+        row = row < N ? row : N - 1;                                     // padding rows read the last row
+        const tl_f32x4* xp = reinterpret_cast<const tl_f32x4*>(x + row * in + chunk * 96 + half * 8);
+#pragma unroll
+        for (int ks = 0; ks < CH_KS; ++ks) xn[ks][0] = xp[ks * 4], xn[ks][1] = xp[ks * 4 + 1];
+    };
+    float bcol[3];
+#pragma unroll
+    for (int ct = 0; ct < 3; ++ct) bcol[ct] = bias ? bias[cg * TL_COLS + ct * 32 + l32] : 0.f;
+
+    if (rounds > 0) {
+        w_request(0);
+        w_store(w_s);
+        x_request(first < row_tiles ? first : row_tiles - 1, 0);
+    }
+    __syncthreads();
+    int it = 0;                                                          // chunk iterations so far: buffer it & 1 is current
+    for (int r = 0; r < rounds; ++r) {
+        const int64_t tile = first + (int64_t)r * stride;
+        const int64_t my_tile = tile < row_tiles ? tile : row_tiles - 1; // a wave past the end repeats the last tile, stores nothing
+        f32x16 acc[3];
+#pragma unroll
+        for (int ct = 0; ct < 3; ++ct) acc[ct] = f32x16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        for (int c = 0; c < chunks; ++c, ++it) {
+            tl_f32x4 xc[CH_KS][2];
+#pragma unroll
+            for (int ks = 0; ks < CH_KS; ++ks) xc[ks][0] = xn[ks][0], xc[ks][1] = xn[ks][1];
+            const bool last = r + 1 == rounds && c + 1 == chunks;
+            const int next_c = c + 1 < chunks ? c + 1 : 0;
+            if (!last) {
+                w_request(next_c);
+                int64_t nt = c + 1 < chunks ? my_tile : tile + stride;
+                x_request(nt < row_tiles ? nt : row_tiles - 1, next_c);
+            }
+            const tl_u32x4* cur = w_s + (it & 1) * BUF + lane;
+#pragma unroll
+            for (int ks = 0; ks < CH_KS; ++ks) {
+                k_step(split8(xc[ks][0], xc[ks][1]), cur + ks * 9 * 64, acc);
+                __builtin_amdgcn_sched_barrier(0);                       // keeps the operands of later steps out of registers
+            }
+            if (!last) w_store(w_s + ((it + 1) & 1) * BUF);
+            __syncthreads();
+        }
+        if (tile < row_tiles) {
+            const int64_t row0 = tile * 32;
+#pragma unroll
+            for (int ct = 0; ct < 3; ++ct) {
+                float* yp = y + (int64_t)cg * TL_COLS + ct * 32 + l32;
+#pragma unroll
+                for (int rr = 0; rr < 16; ++rr) {
+                    const int64_t orow = row0 + acc_row(rr, half);
+                    if (orow < N) yp[orow * out] = acc[ct][rr] + bcol[ct];
+                }
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
 // Weight and bias gradient of the same layers: dW[P,K] = dY^T X, db[P] = column sums of dY, for
 // dY [N,P] and X [N,K] (autograd of the nn.Linear at swin3d_base.py:606-610).
 //
@@ -426,7 +549,48 @@ static int staged_lds_bytes(int ksteps) {
     return ksteps * 9 * 64 * (int)sizeof(tl_u32x4) + 8 * 32 * (ksteps * 16 + 4) * (int)sizeof(float);
 }
 
+static int device_cus() {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess &&
+        n > 0)
+        return n;
+    return 256;
+}
+
+template <bool TRANSPOSED>
+static int launch_chunked(const float* x, int64_t N, int in, const float* w, const float* bias, int out, float* y, int cus,
+                          hipStream_t s, const char* what) {
+    const size_t lds = 2 * (size_t)CH_KS * 9 * 64 * sizeof(tl_u32x4);
+    static bool configured = false;
+    if (!configured) {
+        SSWIN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(tall_linear_chunked_kernel<TRANSPOSED>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds));
+        configured = true;
+    }
+    const int groups = out / TL_COLS;
+    const int64_t row_tiles = (N + 31) / 32;
+    const int64_t per_group = std::min<int64_t>((row_tiles + 7) / 8, std::max<int64_t>(1, cus / groups));
+    hipLaunchKernelGGL(tall_linear_chunked_kernel<TRANSPOSED>, dim3((unsigned)(per_group * groups)), dim3(512), lds, s, x, N, in, w,
+                       groups, bias, y, out, row_tiles);
+    return launch_ok(what);
+}
+
 extern "C" {
+
+int sswin_tall_linear_input_grad_supported(int P, int K) {
+    return P > 0 && K > 0 && (P % 96) == 0 && (K % TL_COLS) == 0;
+}
+
+int sswin_tall_linear_input_grad(const float* dy, int64_t N, int P, const float* w, int K, float* dx, void* stream) {
+    SSWIN_CHECK(N >= 0 && K > 0 && P > 0, "tall_linear_input_grad: bad sizes");
+    SSWIN_CHECK(P % 96 == 0, "tall_linear_input_grad: %d output channels are not a multiple of 96", P);
+    SSWIN_CHECK(K % TL_COLS == 0, "tall_linear_input_grad: %d input channels are not a multiple of %d", K, TL_COLS);
+    if (N == 0) return 0;
+    SSWIN_CHECK(dy && w && dx, "tall_linear_input_grad: null pointer");
+    SSWIN_CHECK(((uintptr_t)dy % 16) == 0, "tall_linear_input_grad: dy must be 16-byte aligned");
+    return launch_chunked<true>(dy, N, P, w, nullptr, K, dx, device_cus(), static_cast<hipStream_t>(stream),
+                                "tall_linear_input_grad");
+}
 
 int sswin_tall_linear_supported(int P, int K) {
     return P > 0 && K > 0 && (P % TL_COLS) == 0 && (K % 16) == 0 && K <= TL_MAX_K;
@@ -498,14 +662,6 @@ static void wgrad_split(int64_t N, int groups, int cus, int64_t* rows_per_chunk,
     rows = std::max<int64_t>(WG_STEP_ROWS, (rows + WG_STEP_ROWS - 1) / WG_STEP_ROWS * WG_STEP_ROWS);
     *rows_per_chunk = rows;
     *chunks = (int)std::max<int64_t>(1, (N + rows - 1) / rows);
-}
-
-static int device_cus() {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) == hipSuccess && hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess &&
-        n > 0)
-        return n;
-    return 256;
 }
 
 extern "C" {

@@ -286,6 +286,30 @@ def _split_linear_forward(x: torch.Tensor, weight: torch.Tensor, bias):
     return y
 
 
+def _split_linear_input_grad(grad_out: torch.Tensor, weight: torch.Tensor):
+    """``grad_out @ W`` through the library's matrix-core kernel for fp32, where it beats the library
+    GEMM (at least 192 output channels of the layer, i.e. the qkv projection), else None."""
+    if not (grad_out.is_cuda and grad_out.dtype == torch.float32 and weight.dtype == torch.float32
+            and grad_out.dim() == 2 and grad_out.shape[0] > 0):
+        return None
+    import ctypes as C
+    from . import _lib
+    lib = _lib.load()
+    n, p = grad_out.shape
+    k = weight.shape[1]
+    if p < 192 or not lib.sswin_tall_linear_input_grad_supported(p, k):
+        return None
+    weight = weight.contiguous()
+    if grad_out.data_ptr() % 16:
+        grad_out = grad_out.clone()
+    with torch.cuda.device(grad_out.device):
+        dx = torch.empty(n, k, dtype=torch.float32, device=grad_out.device)
+        _lib.check(lib.sswin_tall_linear_input_grad(C.c_void_p(grad_out.data_ptr()), n, p, C.c_void_p(weight.data_ptr()), k,
+                                                    C.c_void_p(dx.data_ptr()),
+                                                    C.c_void_p(torch.cuda.current_stream(grad_out.device).cuda_stream)))
+    return dx
+
+
 def _split_linear_weight_grad(grad_out: torch.Tensor, x: torch.Tensor, want_bias: bool):
     """``(grad_out^T @ x, grad_out.sum(0))`` through the library's matrix-core kernel for fp32 (one
     pass over both operands, partial sums added in a fixed order), or ``(None, None)`` when the shape
@@ -316,9 +340,9 @@ def _split_linear_weight_grad(grad_out: torch.Tensor, x: torch.Tensor, want_bias
 
 class _TallLinear(Function):
     """``x @ W^T + b`` for a very tall ``x`` [N, in] (N = number of voxels).  The fp32 forward runs on
-    the bf16 matrix cores with exactly split operands where the shape allows; input gradient and
-    weight gradient are library GEMMs, routed to the BLAS backend that handles tall-skinny shapes
-    best (see :func:`_rocblas_gemm`)."""
+    the bf16 matrix cores with exactly split operands where the shape allows, and so do the weight
+    and bias gradient and the input gradient of wide layers; everything else is a library GEMM, routed
+    to the BLAS backend that handles tall-skinny shapes best (see :func:`_rocblas_gemm`)."""
 
     @staticmethod
     def forward(ctx, x, weight, bias):
@@ -339,8 +363,10 @@ class _TallLinear(Function):
         want_b = ctx.has_bias and ctx.needs_input_grad[2]
         if ctx.needs_input_grad[1]:
             grad_w, grad_b = _split_linear_weight_grad(grad_out, x, want_b)
+        if ctx.needs_input_grad[0]:
+            grad_x = _split_linear_input_grad(grad_out, weight)
         with _rocblas_gemm():
-            if ctx.needs_input_grad[0]:
+            if ctx.needs_input_grad[0] and grad_x is None:
                 grad_x = grad_out @ weight
             if ctx.needs_input_grad[1] and grad_w is None:
                 grad_w = grad_out.t() @ x

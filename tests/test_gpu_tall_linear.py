@@ -128,6 +128,43 @@ def test_tall_linear_weight_grad(N, K, P, bias):
         assert ((db.double() - refb).abs() / dy.double().abs().sum(0)).max().item() < TOL
 
 
+@pytest.mark.parametrize("N,P,K", [
+    (107500, 288, 96),              # qkv of stage 1
+    (25900, 576, 192),              # qkv of stage 2
+    (107500, 96, 96), (1, 288, 96), (31, 192, 96), (257, 96, 192), (4097, 288, 96), (300, 384, 288),
+])
+def test_tall_linear_input_grad(N, P, K):
+    """dX = dY W against float64 on the same fp32 inputs."""
+    from sparseswin3d_amd import _lib
+    lib = _lib.load()
+    assert lib.sswin_tall_linear_input_grad_supported(P, K)
+    g = torch.Generator().manual_seed(N + P + 5 * K)
+    dy = (torch.randn(N, P, generator=g) * torch.exp2(torch.randint(-6, 7, (N, P), generator=g).float())).cuda()
+    w = (torch.randn(P, K, generator=g) * 0.1).cuda()
+    dx = torch.full((N, K), float("nan"), device="cuda")
+    _lib.check(lib.sswin_tall_linear_input_grad(C.c_void_p(dy.data_ptr()), N, P, C.c_void_p(w.data_ptr()), K,
+                                                C.c_void_p(dx.data_ptr()),
+                                                C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+    torch.cuda.synchronize()
+    ref = dy.double() @ w.double()
+    scale = dy.double().abs() @ w.double().abs()
+    assert not torch.isnan(dx).any()
+    assert ((dx.double() - ref).abs() / scale).max().item() < TOL
+
+
+def test_tall_linear_input_grad_unsupported_shapes():
+    from sparseswin3d_amd import _lib
+    lib = _lib.load()
+    assert lib.sswin_tall_linear_input_grad_supported(100, 96) == 0
+    assert lib.sswin_tall_linear_input_grad_supported(96, 64) == 0
+    t = torch.zeros(64, 96, device="cuda")
+    rc = lib.sswin_tall_linear_input_grad(C.c_void_p(t.data_ptr()), 64, 96, C.c_void_p(t.data_ptr()), 64,
+                                          C.c_void_p(t.data_ptr()), None)
+    assert rc != 0
+    with pytest.raises(RuntimeError, match="input channels"):
+        _lib.check(rc)
+
+
 def test_tall_linear_weight_grad_unsupported_shapes():
     from sparseswin3d_amd import _lib
     lib = _lib.load()
@@ -144,8 +181,8 @@ def test_tall_linear_weight_grad_unsupported_shapes():
 
 
 def test_module_projection_matches_library_gemm():
-    """tall_linear() of the module (forward, weight and bias gradient through the kernels, input
-    gradient through the library) against nn.Linear in float64."""
+    """tall_linear() of the module (forward and all three gradients through the kernels) against
+    nn.Linear in float64."""
     from sparseswin3d_amd.window_attention import tall_linear
     torch.manual_seed(5)
     layer = torch.nn.Linear(96, 288).cuda()
