@@ -290,6 +290,7 @@ def kernel_table(wl, reps=20, only=None):
         return [], dict(N=N, E=E, A=A, G=G, c_max=c_max)
     table = measure(r_entries, "resident") + measure(f_entries, "fused") + measure(entries, "operators")
     table += measure(stage_entries(wl), "stage")
+    table += measure(projection_entries(wl), "projections")
     return table, dict(N=N, E=E, A=A, G=G, c_max=c_max)
 
 
@@ -324,6 +325,47 @@ def stage_entries(wl):
         ("torch roll + partition (reference form)", torch_partition, 24 * N, 0),
         ("torch index_add mean pool", torch_pool, 4 * D * (N + M), 0),
     ]
+
+
+def projection_entries(wl):
+    """The qkv and proj nn.Linear of one attention call (fp32 on the bf16 matrix cores with split
+    operands), and the library GEMMs they replace (calls = 0)."""
+    from sparseswin3d_amd import window_attention as wa
+    N, D = wl["N"], wl["dim"]
+    dev = wl["feats"].device
+    x = torch.randn(N, D, device=dev)
+    entries = []
+    for name, P in (("qkv", 3 * D), ("proj", D)):
+        w = torch.randn(P, D, device=dev) * 0.1
+        b = torch.randn(P, device=dev)
+        dy = torch.randn(N, P, device=dev)
+        io = 4 * N * (D + P)
+        entries += [
+            (f"{name} forward", (lambda w=w, b=b: wa._split_linear_forward(x, w, b)), io + 4 * P * D, 1),
+            (f"{name} weight+bias gradient", (lambda dy=dy: wa._split_linear_weight_grad(dy, x, True)), io + 4 * P * D, 1),
+        ]
+        def lib_dx(dy=dy, w=w):
+            with wa._rocblas_gemm():
+                return dy @ w
+
+        if P >= 192:
+            entries.append((f"{name} input gradient", (lambda dy=dy, w=w: wa._split_linear_input_grad(dy, w)), io + 4 * P * D, 1))
+        else:
+            entries.append((f"{name} input gradient (library GEMM)", lib_dx, io + 4 * P * D, 1))
+
+        def lib_fwd(w=w, b=b):
+            with wa._rocblas_gemm():
+                return torch.nn.functional.linear(x, w, b)
+
+        def lib_wgrad(dy=dy):
+            with wa._rocblas_gemm():
+                return dy.t() @ x, wa._column_sum(dy)
+
+        entries += [(f"{name} forward, library GEMM", lib_fwd, io + 4 * P * D, 0),
+                    (f"{name} weight+bias gradient, library GEMM + column sums", lib_wgrad, io + 4 * P * D, 0)]
+        if P >= 192:
+            entries.append((f"{name} input gradient, library GEMM", lib_dx, io + 4 * P * D, 0))
+    return entries
 
 
 # ------------------------------------------------------------------------------------------
@@ -436,10 +478,12 @@ def main():
         table, sizes = kernel_table(wl)
         log(f"{'kernel':36s} {'ms':>9s} {'calls':>5s} {'alg MB':>9s} {'GB/s':>9s} {'% HBM':>7s}")
         summary = {}
-        for path in ("resident", "fused", "operators", "stage"):
+        titles = {"stage": "-- index glue of one stage (window indices, mask, stride-2 merge) --",
+                  "projections": "-- qkv and proj layers of one attention call (dense [N, C] GEMMs) --"}
+        scope = {"stage": "once per stage", "projections": "one attention fwd+bwd"}
+        for path in ("resident", "fused", "operators", "stage", "projections"):
             rows_ = [r for r in table if r["path"] == path]
-            log(f"-- {path} path, one attention forward+backward --" if path != "stage" else
-                "-- index glue of one stage (window indices, mask, stride-2 merge) --")
+            log(titles.get(path, f"-- {path} path, one attention forward+backward --"))
             for r in rows_:
                 log(f"{r['kernel']:36s} {r['ms']:9.4f} {r['calls']:5d} {r['algorithmic_bytes'] / 1e6:9.1f} "
                     f"{(r['achieved_gbps'] or 0):9.1f} {100 * (r['frac'] or 0):7.2f}")
@@ -447,7 +491,7 @@ def main():
             alg = sum(r["algorithmic_bytes"] * r["calls"] for r in rows_)
             summary[path] = dict(ms=round(ms_, 4), algorithmic_bytes=alg,
                                  frac=round(alg / ms_ / 1e6 / HBM_PEAK_GBPS, 4))
-            log(f"{path} kernels, {'one attention fwd+bwd' if path != 'stage' else 'once per stage'}: {ms_:.3f} ms for {alg / 1e6:.1f} MB algorithmic "
+            log(f"{path} kernels, {scope.get(path, 'one attention fwd+bwd')}: {ms_:.3f} ms for {alg / 1e6:.1f} MB algorithmic "
                 f"= {alg / ms_ / 1e6:.1f} GB/s = {100 * alg / ms_ / 1e6 / HBM_PEAK_GBPS:.2f}% of HBM peak")
         # the step runs the window-resident path: its slowest kernel is the dominant one
         # (the token plan is a sequence of small launches, not a kernel)
