@@ -557,13 +557,13 @@ __global__ __launch_bounds__(256) void rpb_grad_reduce_kernel(const float* __res
 // ------------------------------------------------------------------------------------------
 constexpr int RPBT_MAX_ROWS = 1024;
 
+// dynamic LDS: [wave 4][half 2][rows_pad] floats, then [wave 4][buffer 2][128] position codes
 __global__ __launch_bounds__(256) void rpb_table_partial_kernel(FusedGroups gt, const int32_t* __restrict__ tok_pos,
                                                                 int H, const int32_t* __restrict__ code, int offset0,
-                                                                int rows, const float* __restrict__ ds,
+                                                                int rows, int rows_pad, const float* __restrict__ ds,
                                                                 int64_t windows, int wslices, int rsplit,
                                                                 float* __restrict__ partial) {
-    __shared__ float tables[4][2][RPBT_MAX_ROWS];
-    __shared__ int32_t codes[4][128];
+    extern __shared__ __attribute__((aligned(16))) float rpbt_lds[];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int half = lane >> 5, l32 = lane & 31;
     const int64_t p = (int64_t)blockIdx.x * 4 + wave;           // wavefront id = s * H + h
@@ -573,30 +573,42 @@ __global__ __launch_bounds__(256) void rpb_table_partial_kernel(FusedGroups gt, 
     const int64_t sl = p / H;
     const int64_t ws = sl % wslices;                            // windows ws, ws + wslices, ...
     const int rs = (int)(sl / wslices);                         // rows rs, rs + rsplit, ... of each of them
-    float* mine = tables[wave][half];
-    int32_t* cw = codes[wave];
+    float* tables = rpbt_lds + wave * 2 * rows_pad;
+    float* mine = tables + half * rows_pad;
+    int32_t* codes = reinterpret_cast<int32_t*>(rpbt_lds + 8 * rows_pad) + wave * 256;
     for (int e = l32; e < rows; e += 32) mine[e] = 0.f;
     // A slice takes every wslices-th window (crowded windows are neighbours in plan order, so
     // dealing them out evens the load) and, when windows are few and large, every rsplit-th row of
-    // them.  The next window's header is fetched early.
-    int c_n = 0, T_n = 0, sq_n = 0;
-    if (ws < windows) {
-        const int64_t g = ws * H + h;
-        c_n = gt.c[g];
-        T_n = gt.T[g];
-        sq_n = gt.sq[g];
-    }
-    for (int64_t k = ws; k < windows; k += wslices) {
-        const int c = c_n, Tk = T_n;
-        const float* blk = ds + sq_n;
-        if (k + wslices < windows) {
-            const int64_t g = (k + wslices) * H + h;
-            c_n = gt.c[g];
-            T_n = gt.T[g];
-            sq_n = gt.sq[g];
+    // them.  Headers are fetched two windows ahead and the position codes of the next window (two
+    // dependent loads) are in flight while the current one is added.
+    int c_c = 0, sq_c = 0, c_n = 0, T_n = 0, sq_n = 0;
+    auto header = [&](int64_t k, int& c, int& T, int& sq) {
+        if (k < windows) {
+            const int64_t g = k * H + h;
+            c = gt.c[g];
+            T = gt.T[g];
+            sq = gt.sq[g];
+        } else {
+            c = 0;
         }
-        __builtin_amdgcn_wave_barrier();
-        for (int t = lane; t < c; t += 64) cw[t] = code[tok_pos[Tk + t]];
+    };
+    {
+        int T_c = 0;
+        header(ws, c_c, T_c, sq_c);
+        header(ws + wslices, c_n, T_n, sq_n);
+        for (int t = lane; t < c_c; t += 64) codes[t] = code[tok_pos[T_c + t]];
+    }
+    int par = 0;
+    for (int64_t k = ws; k < windows; k += wslices, par ^= 1) {
+        const int c = c_c;
+        const float* blk = ds + sq_c;
+        const int32_t* cw = codes + par * 128;
+        int cn[2] = {0, 0};
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+            if (lane + 64 * u < c_n) cn[u] = code[tok_pos[T_n + lane + 64 * u]];
+        const int c_next = c_n, sq_next = sq_n;
+        header(k + 2 * wslices, c_n, T_n, sq_n);
         __builtin_amdgcn_wave_barrier();
         // item = (row i, chunk of 32 columns): all lanes of an item hit different table rows.
         // The two halves of the wavefront take alternate items and add into separate copies of
@@ -625,10 +637,17 @@ __global__ __launch_bounds__(256) void rpb_table_partial_kernel(FusedGroups gt, 
             for (int u = 0; u < 8; ++u)
                 if (row[u] >= 0) mine[row[u]] += v[u];
         }
+        int32_t* cwn = codes + (par ^ 1) * 128;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+            if (lane + 64 * u < c_next) cwn[lane + 64 * u] = cn[u];
+        __builtin_amdgcn_wave_barrier();
+        c_c = c_next;
+        sq_c = sq_next;
     }
     __builtin_amdgcn_wave_barrier();
     float* out = partial + ((int64_t)h * slices + sl) * rows;
-    for (int e = lane; e < rows; e += 64) out[e] = tables[wave][0][e] + tables[wave][1][e];
+    for (int e = lane; e < rows; e += 64) out[e] = tables[e] + tables[rows_pad + e];
 }
 
 // d_table[row, h] = sum over slices of partial[h][slice][row].  One workgroup per 16 table rows
@@ -894,8 +913,10 @@ int sswin_bias_table_grad(const int32_t* plan, int64_t g_cap, int64_t G, const i
     const int slices = wslices * rsplit;
     float* partial = static_cast<float*>(ws);
     const int64_t waves = (int64_t)slices * H;
-    hipLaunchKernelGGL(rpb_table_partial_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), 0, s, gt, tokens + 3 * N, H,
-                       code, offset0, table_rows, ds, windows, wslices, rsplit, partial);
+    const int rows_pad = (table_rows + 31) / 32 * 32;
+    const size_t lds = (size_t)8 * rows_pad * sizeof(float) + 4 * 256 * sizeof(int32_t);
+    hipLaunchKernelGGL(rpb_table_partial_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), lds, s, gt, tokens + 3 * N, H,
+                       code, offset0, table_rows, rows_pad, ds, windows, wslices, rsplit, partial);
     hipLaunchKernelGGL(rpb_table_reduce_kernel, dim3((unsigned)((table_rows + 15) / 16), (unsigned)H), dim3(1024), 0, s,
                        partial, slices, table_rows, H, d_table);
     return launch_ok("bias table gradient");
