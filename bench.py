@@ -278,7 +278,7 @@ def kernel_table(wl, reps=20, only=None):
         # device-to-device copy of known size that calibrates the FETCH_SIZE / WRITE_SIZE counters
         src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device=dev)
         dst = torch.empty_like(src)
-        picked = [e for e in r_entries + f_entries + entries if only in e[0]]
+        picked = [e for e in r_entries + f_entries + entries + projection_entries(wl) if only in e[0]]
         for name, fn, nbytes, calls in picked:
             log(f"profiling {name}: {reps} launches, algorithmic bytes {nbytes}")
             for _ in range(reps):

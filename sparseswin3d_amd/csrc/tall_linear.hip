@@ -135,7 +135,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     const float* __restrict__ x, int64_t N, int K, const float* __restrict__ w, int groups, const float* __restrict__ bias,
     float* __restrict__ y, int P, int64_t row_blocks) {
     extern __shared__ __attribute__((aligned(16))) tl_u32x4 w_s[];      // [k step][tile][plane][lane]
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave: a scalar
     const int half = lane >> 5, l32 = lane & 31;
     const int ksteps = K / 16;
     int cg, slot;
@@ -182,13 +182,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 // (pitch K + 4 floats, so 8 rows hit 8 different bank groups) and takes its operands from there.
 // One workgroup of 8 waves per CU shares the planes of W: K <= 96 fits 160 KB of LDS.
 constexpr int TL_STAGED_MAX_KS = 6;
-template <int KS>
+// SMALL: fewer than 32 rows in all (one ragged tile, guarded).  Otherwise a last ragged tile is moved
+// back to end at row N: it recomputes a few rows of its neighbour (same inputs, same arithmetic, the
+// same bits stored twice) and every tile takes the unguarded path.
+template <int KS, bool SMALL>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void tall_linear_forward_staged_kernel(
     const float* __restrict__ x, int64_t N, const float* __restrict__ w, int groups, const float* __restrict__ bias,
     float* __restrict__ y, int P, int64_t row_tiles) {
     constexpr int K = KS * 16, PITCH = K + 4, C4 = K / 4, NI = 2 * KS;   // 16-byte chunks per row; loads per lane and tile
     extern __shared__ __attribute__((aligned(16))) tl_u32x4 w_s[];      // [k step][tile][plane][lane], then the X tiles
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave: a scalar
     const int half = lane >> 5, l32 = lane & 31;
     int cg, slot;
     group_and_slot(groups, cg, slot);
@@ -201,25 +204,34 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
     for (int ct = 0; ct < 3; ++ct) bcol[ct] = bias ? bias[cg * TL_COLS + ct * 32 + l32] : 0.f;
 
+    // A load instruction covers 64 / GW rows x GW 16-byte chunks (GW x 16 contiguous bytes per row), so
+    // that global and LDS addresses are a per-lane part, computed once, plus a compile-time part.
+    constexpr int GW = (C4 % 8 == 0) ? 8 : 4, RPI = 64 / GW, CGS = C4 / GW;   // rows per instruction, chunk groups per row
+    static_assert(NI == (32 / RPI) * CGS, "loads per tile");
+    const int lr = lane / GW, lc = lane % GW;
+    const uint32_t g_lane = (uint32_t)(lr * K + lc * 4);                 // floats, within the tile
+    const uint32_t s_lane = (uint32_t)(lr * PITCH + lc * 4);
+    const uint32_t y_lane = (uint32_t)(4 * half * P + l32);              // accumulator rows start at 4 * half
     tl_f32x4 xn[NI];
+    auto tile_row0 = [&](int64_t t) { return SMALL ? 0 : (t * 32 + 32 <= N ? t * 32 : N - 32); };
     auto fetch = [&](int64_t t) {
-        const int64_t e0 = t * 32 * K, end = N * K;                      // the tile is 32 K consecutive floats
-        const tl_f32x4* xp = reinterpret_cast<const tl_f32x4*>(x + e0);
+        const float* xt = x + tile_row0(t) * K;                          // uniform; the tile is 32 K consecutive floats
 #pragma unroll
         for (int i = 0; i < NI; ++i) {
-            const int q = i * 64 + lane;
-            xn[i] = e0 + q * 4 < end ? xp[q] : tl_f32x4{0.f, 0.f, 0.f, 0.f};
+            const tl_f32x4* src = reinterpret_cast<const tl_f32x4*>(xt + ((i / CGS) * RPI * K + (i % CGS) * GW * 4) + g_lane);
+            if (SMALL)
+                xn[i] = (i / CGS) * RPI + lr < N ? *src : tl_f32x4{0.f, 0.f, 0.f, 0.f};
+            else
+                xn[i] = *src;
         }
     };
     if (first < row_tiles) fetch(first);
     for (int64_t t = first; t < row_tiles; t += stride) {
-        const int64_t row0 = t * 32;
+        const int64_t row0 = tile_row0(t);
         __builtin_amdgcn_wave_barrier();                                 // the previous tile's operand reads are done
 #pragma unroll
-        for (int i = 0; i < NI; ++i) {
-            const int q = i * 64 + lane;
-            *reinterpret_cast<tl_f32x4*>(xs + (q / C4) * PITCH + (q % C4) * 4) = xn[i];
-        }
+        for (int i = 0; i < NI; ++i)
+            *reinterpret_cast<tl_f32x4*>(xs + ((i / CGS) * RPI * PITCH + (i % CGS) * GW * 4) + s_lane) = xn[i];
         __builtin_amdgcn_wave_barrier();
         if (t + stride < row_tiles) fetch(t + stride);
         f32x16 acc[3];
@@ -241,15 +253,14 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             k_products(a[ks & 1], b[ks & 1], acc);
             __builtin_amdgcn_sched_barrier(0);                           // keeps the operands of later steps out of registers
         }
+        // accumulator register r of lane l: row 8 (r / 4) + 4 half + r % 4, column l % 32
+        float* yt = y + row0 * P + cg * TL_COLS;                         // uniform
 #pragma unroll
-        for (int ct = 0; ct < 3; ++ct) {
-            float* yp = y + (int64_t)cg * TL_COLS + ct * 32 + l32;
+        for (int ct = 0; ct < 3; ++ct)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                const int64_t orow = row0 + acc_row(r, half);
-                if (orow < N) yp[orow * P] = acc[ct][r] + bcol[ct];
-            }
-        }
+            for (int r = 0; r < 16; ++r)
+                if (!SMALL || acc_row(r, half) < N)                      // the bias last: the small terms are summed first
+                    (yt + (8 * (r >> 2) + (r & 3)) * P + ct * 32)[y_lane] = acc[ct][r] + bcol[ct];
     }
 }
 
@@ -270,7 +281,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     float* __restrict__ y, int out, int64_t row_tiles) {
     extern __shared__ __attribute__((aligned(16))) tl_u32x4 w_s[];      // [buffer 2][k step 6][tile 3][plane 3][lane 64]
     constexpr int BUF = CH_KS * 9 * 64;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave: a scalar
     const int half = lane >> 5, l32 = lane & 31;
     const int chunks = in / 96;
     int cg, slot;
@@ -394,17 +405,6 @@ constexpr int WG_QUARTERS = 4, WG_WAVES = 12, WG_STEP_ROWS = 16 * WG_QUARTERS;
 struct Raw8 {
     float v[8];
 };
-// 8 rows (slot e of k group kg = row r0 + 8 kg + e) of column `col`; rows past N read as zero
-__device__ __forceinline__ Raw8 load_rows8(const float* __restrict__ base, int64_t pitch, int64_t r0, int64_t N, int col,
-                                           int half) {
-    Raw8 o;
-#pragma unroll
-    for (int e = 0; e < 8; ++e) {
-        const int64_t row = r0 + half * 8 + e;
-        o.v[e] = row < N ? base[row * pitch + col] : 0.f;
-    }
-    return o;
-}
 __device__ __forceinline__ APlanes split_raw8(const Raw8& r) {
     const Split2 s0 = split2(r.v[0], r.v[1]), s1 = split2(r.v[2], r.v[3]), s2 = split2(r.v[4], r.v[5]), s3 = split2(r.v[6], r.v[7]);
     APlanes a;
@@ -422,7 +422,7 @@ __global__ __launch_bounds__(WG_WAVES * 64) __attribute__((amdgpu_waves_per_eu(3
     constexpr int K = XT * 32;
     // X planes: [buffer 2][quarter 4][tile XT][plane 3][lane 64] x 16 bytes; reused for the final sums
     extern __shared__ __attribute__((aligned(16))) tl_u32x4 lds[];
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave: a scalar
     const int half = lane >> 5, l32 = lane & 31;
     const int quarter = wave / 3, t = wave % 3;                          // t: this wave's column tile of dY (and of X)
     int g, chunk;
@@ -439,10 +439,26 @@ __global__ __launch_bounds__(WG_WAVES * 64) __attribute__((amdgpu_waves_per_eu(3
     float bsum = 0.f;
     // rows are requested two steps ahead (loaded HBM latency is about two steps of products)
     Raw8 ry[2], rx[2];
+    // addresses: a uniform part (scalar arithmetic) plus a per-lane offset computed once
+    const uint32_t y_lane = (uint32_t)(half * 8 * P + ycol), x_lane = (uint32_t)(half * 8 * K + xcol);
     auto fetch = [&](int s, Raw8& y8, Raw8& x8) {
         const int64_t r0 = row_begin + (int64_t)s * WG_STEP_ROWS + quarter * 16;
-        y8 = load_rows8(dy, P, r0, row_end, ycol, half);
-        if (t < XT) x8 = load_rows8(x, K, r0, row_end, xcol, half);
+        const float* yb = dy + r0 * P;
+        const float* xb = x + r0 * K;
+        if (r0 + 16 <= row_end) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                y8.v[e] = (yb + e * P)[y_lane];
+                if (t < XT) x8.v[e] = (xb + e * K)[x_lane];
+            }
+        } else {                                                         // the ragged end of the rows: zeros past it
+            const int nvalid = (int)(row_end - r0) - half * 8;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                y8.v[e] = e < nvalid ? (yb + e * P)[y_lane] : 0.f;
+                if (t < XT) x8.v[e] = e < nvalid ? (xb + e * K)[x_lane] : 0.f;
+            }
+        }
     };
     auto step = [&](int s, Raw8& y8, Raw8& x8) {
         tl_u32x4* buf = lds + (s & 1) * BUF + quarter * XT * 3 * 64;
@@ -619,14 +635,20 @@ int sswin_tall_linear_forward(const float* x, int64_t N, int K, const float* w, 
         const int max_lds = TL_MAX_K / 16 * 9 * 64 * (int)sizeof(tl_u32x4);
         SSWIN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(tall_linear_forward_kernel),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, max_lds));
-        const void* staged[] = {reinterpret_cast<const void*>(tall_linear_forward_staged_kernel<1>),
-                                reinterpret_cast<const void*>(tall_linear_forward_staged_kernel<2>),
-                                reinterpret_cast<const void*>(tall_linear_forward_staged_kernel<3>),
-                                reinterpret_cast<const void*>(tall_linear_forward_staged_kernel<4>),
-                                reinterpret_cast<const void*>(tall_linear_forward_staged_kernel<5>),
-                                reinterpret_cast<const void*>(tall_linear_forward_staged_kernel<6>)};
-        for (int ks = 1; ks <= TL_STAGED_MAX_KS; ++ks)
-            SSWIN_HIP(hipFuncSetAttribute(staged[ks - 1], hipFuncAttributeMaxDynamicSharedMemorySize, staged_lds_bytes(ks)));
+        const void* staged[] = {reinterpret_cast<const void*>(tall_linear_forward_staged_kernel<1, false>),
+                                reinterpret_cast<const void*>(tall_linear_forward_staged_kernel<2, false>),
+                                reinterpret_cast<const void*>(tall_linear_forward_staged_kernel<3, false>),
+                                reinterpret_cast<const void*>(tall_linear_forward_staged_kernel<4, false>),
+                                reinterpret_cast<const void*>(tall_linear_forward_staged_kernel<5, false>),
+                                reinterpret_cast<const void*>(tall_linear_forward_staged_kernel<6, false>),
+                                reinterpret_cast<const void*>(tall_linear_forward_staged_kernel<1, true>),
+                                reinterpret_cast<const void*>(tall_linear_forward_staged_kernel<2, true>),
+                                reinterpret_cast<const void*>(tall_linear_forward_staged_kernel<3, true>),
+                                reinterpret_cast<const void*>(tall_linear_forward_staged_kernel<4, true>),
+                                reinterpret_cast<const void*>(tall_linear_forward_staged_kernel<5, true>),
+                                reinterpret_cast<const void*>(tall_linear_forward_staged_kernel<6, true>)};
+        for (int q = 0; q < 12; ++q)
+            SSWIN_HIP(hipFuncSetAttribute(staged[q], hipFuncAttributeMaxDynamicSharedMemorySize, staged_lds_bytes(q % 6 + 1)));
         configured = true;
     }
     if (ksteps <= TL_STAGED_MAX_KS) {
@@ -636,8 +658,12 @@ int sswin_tall_linear_forward(const float* x, int64_t N, int K, const float* w, 
         const size_t lds = staged_lds_bytes(ksteps);
 #define SSWIN_TL_STAGED(KS)                                                                                                  \
     case KS:                                                                                                                 \
-        hipLaunchKernelGGL(tall_linear_forward_staged_kernel<KS>, grid, block, lds, s, x, N, w, groups, bias, y, P,          \
-                           row_tiles);                                                                                       \
+        if (N < 32)                                                                                                          \
+            hipLaunchKernelGGL((tall_linear_forward_staged_kernel<KS, true>), grid, block, lds, s, x, N, w, groups, bias, y, \
+                               P, row_tiles);                                                                                \
+        else                                                                                                                 \
+            hipLaunchKernelGGL((tall_linear_forward_staged_kernel<KS, false>), grid, block, lds, s, x, N, w, groups, bias,   \
+                               y, P, row_tiles);                                                                             \
         break;
         switch (ksteps) {
             SSWIN_TL_STAGED(1) SSWIN_TL_STAGED(2) SSWIN_TL_STAGED(3) SSWIN_TL_STAGED(4) SSWIN_TL_STAGED(5) SSWIN_TL_STAGED(6)
