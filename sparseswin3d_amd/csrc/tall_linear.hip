@@ -238,19 +238,38 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 #pragma unroll
         for (int ct = 0; ct < 3; ++ct) acc[ct] = f32x16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
         const float* xr = xs + l32 * PITCH + half * 8;
-        // the operands of step ks + 1 are read and split while the products of step ks run
+        // Software pipeline over the k steps: during the 18 products of step ks the planes of W for step
+        // ks + 1 and the 8 values of X for step ks + 2 are read from LDS, and the values of step ks + 1
+        // (read one step earlier) are split, three vector instructions after every MFMA, so that the
+        // vector ALU works in the shadow of the matrix core.
         APlanes a[2];
         BPlanes b[2];
-        a[0] = split8(*reinterpret_cast<const tl_f32x4*>(xr), *reinterpret_cast<const tl_f32x4*>(xr + 4));
+        tl_f32x4 raw[2][2];
+        raw[0][0] = *reinterpret_cast<const tl_f32x4*>(xr);
+        raw[0][1] = *reinterpret_cast<const tl_f32x4*>(xr + 4);
         b[0] = read_b(w_s + lane);
+        if (KS > 1) {
+            raw[1][0] = *reinterpret_cast<const tl_f32x4*>(xr + 16);
+            raw[1][1] = *reinterpret_cast<const tl_f32x4*>(xr + 20);
+        }
+        a[0] = split8(raw[0][0], raw[0][1]);
+        __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks) {
-            if (ks + 1 < KS) {
-                b[(ks + 1) & 1] = read_b(w_s + (ks + 1) * 9 * 64 + lane);
-                a[(ks + 1) & 1] = split8(*reinterpret_cast<const tl_f32x4*>(xr + (ks + 1) * 16),
-                                         *reinterpret_cast<const tl_f32x4*>(xr + (ks + 1) * 16 + 4));
+            if (ks + 1 < KS) b[(ks + 1) & 1] = read_b(w_s + (ks + 1) * 9 * 64 + lane);
+            if (ks + 2 < KS) {
+                raw[ks & 1][0] = *reinterpret_cast<const tl_f32x4*>(xr + (ks + 2) * 16);
+                raw[ks & 1][1] = *reinterpret_cast<const tl_f32x4*>(xr + (ks + 2) * 16 + 4);
             }
             k_products(a[ks & 1], b[ks & 1], acc);
+            if (ks + 1 < KS) a[(ks + 1) & 1] = split8(raw[(ks + 1) & 1][0], raw[(ks + 1) & 1][1]);
+            // order inside the step: the LDS reads, then MFMA / vector / vector / vector ...
+            __builtin_amdgcn_sched_group_barrier(0x100, 11, 0);
+#pragma unroll
+            for (int q = 0; q < 18; ++q) {
+                __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+                __builtin_amdgcn_sched_group_barrier(0x002, 3, 0);
+            }
             __builtin_amdgcn_sched_barrier(0);                           // keeps the operands of later steps out of registers
         }
         // accumulator register r of lane l: row 8 (r / 4) + 4 half + r % 4, column l % 32
