@@ -407,6 +407,115 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
 }
 
 // ------------------------------------------------------------------------------------------
+// 96 < input channels <= 288 without chunk barriers: the planes of all of W for the workgroup's 96 columns
+// stay in LDS (9 KB per k step, at most 17 steps = 153 KB); with 18 steps (288 channels: the input
+// gradient of the qkv layer of a 96-channel stage) the planes of the last step stay in registers, 36
+// per lane.  After the fill nothing is shared any more: every wave streams its 32-row tiles on its
+// own, the lane's 48 values of the next 96 channels in flight during the products.
+// ------------------------------------------------------------------------------------------
+constexpr int WIDE_LDS_KS = 17, WIDE_MAX_KS = 18;
+
+template <bool TRANSPOSED>
+__global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void tall_linear_wide_kernel(
+    const float* __restrict__ x, int64_t N, int in, const float* __restrict__ w, int groups, const float* __restrict__ bias,
+    float* __restrict__ y, int out, int64_t row_tiles) {
+    extern __shared__ __attribute__((aligned(16))) tl_u32x4 w_s[];      // [k step][tile 3][plane 3][lane 64]
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int half = lane >> 5, l32 = lane & 31;
+    const int ksteps = in / 16, chunks = in / 96;
+    const int lds_ks = ksteps < WIDE_LDS_KS ? ksteps : WIDE_LDS_KS;
+    int cg, slot;
+    group_and_slot(groups, cg, slot);
+    const int64_t first = (int64_t)slot * 8 + wave, stride = (int64_t)(gridDim.x / groups) * 8;
+
+    // 8 values of Wop for (column, k0 .. k0 + 7), split into planes
+    auto w_planes = [&](int col, int k0, tl_u32x4& h, tl_u32x4& m, tl_u32x4& l) {
+        float v[8];
+        if (TRANSPOSED) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = w[(int64_t)(k0 + e) * out + col];
+        } else {
+            const tl_f32x4* src = reinterpret_cast<const tl_f32x4*>(w + (int64_t)col * in + k0);
+            const tl_f32x4 c0 = src[0], c1 = src[1];
+            v[0] = c0.x; v[1] = c0.y; v[2] = c0.z; v[3] = c0.w; v[4] = c1.x; v[5] = c1.y; v[6] = c1.z; v[7] = c1.w;
+        }
+        const Split2 s0 = split2(v[0], v[1]), s1 = split2(v[2], v[3]), s2 = split2(v[4], v[5]), s3 = split2(v[6], v[7]);
+        h = tl_u32x4{s0.h, s1.h, s2.h, s3.h};
+        m = tl_u32x4{s0.m, s1.m, s2.m, s3.m};
+        l = tl_u32x4{s0.l, s1.l, s2.l, s3.l};
+    };
+    for (int it = threadIdx.x; it < lds_ks * 3 * 64; it += 512) {
+        const int ln = it & 63, ct = (it >> 6) % 3, ks = (it >> 6) / 3;
+        tl_u32x4 h, m, l;
+        w_planes(cg * TL_COLS + ct * 32 + (ln & 31), ks * 16 + (ln >> 5) * 8, h, m, l);
+        tl_u32x4* dst = w_s + (it >> 6) * 3 * 64 + ln;
+        dst[0] = h;
+        dst[64] = m;
+        dst[128] = l;
+    }
+    BPlanes breg;                                                        // planes of k step 17, this lane's operand slots
+    if (ksteps > WIDE_LDS_KS) {
+#pragma unroll
+        for (int ct = 0; ct < 3; ++ct) {
+            tl_u32x4 h, m, l;
+            w_planes(cg * TL_COLS + ct * 32 + l32, WIDE_LDS_KS * 16 + half * 8, h, m, l);
+            breg.h[ct] = as_bf16x8(h);
+            breg.m[ct] = as_bf16x8(m);
+            breg.l[ct] = as_bf16x8(l);
+        }
+    }
+    float bcol[3];
+#pragma unroll
+    for (int ct = 0; ct < 3; ++ct) bcol[ct] = bias ? bias[cg * TL_COLS + ct * 32 + l32] : 0.f;
+    __syncthreads();
+
+    // the lane's 48 values of 96 channels of its row (row l % 32 of the tile, k group l / 32)
+    tl_f32x4 xn[CH_KS][2];
+    auto x_request = [&](int64_t tile, int chunk) {
+        int64_t row = tile * 32 + l32;
+        row = row < N ? row : N - 1;                                     // padding rows read the last row
+        const tl_f32x4* xp = reinterpret_cast<const tl_f32x4*>(x + row * in + chunk * 96 + half * 8);
+#pragma unroll
+        for (int ks = 0; ks < CH_KS; ++ks) xn[ks][0] = xp[ks * 4], xn[ks][1] = xp[ks * 4 + 1];
+    };
+    if (first < row_tiles) x_request(first, 0);
+    for (int64_t tile = first; tile < row_tiles; tile += stride) {
+        f32x16 acc[3];
+#pragma unroll
+        for (int ct = 0; ct < 3; ++ct) acc[ct] = f32x16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        for (int c = 0; c < chunks; ++c) {
+            tl_f32x4 xc[CH_KS][2];
+#pragma unroll
+            for (int ks = 0; ks < CH_KS; ++ks) xc[ks][0] = xn[ks][0], xc[ks][1] = xn[ks][1];
+            if (c + 1 < chunks)
+                x_request(tile, c + 1);
+            else if (tile + stride < row_tiles)
+                x_request(tile + stride, 0);
+            const tl_u32x4* cur = w_s + c * CH_KS * 9 * 64 + lane;
+#pragma unroll
+            for (int ks = 0; ks < CH_KS; ++ks) {
+                const APlanes a = split8(xc[ks][0], xc[ks][1]);
+                if (c * CH_KS + ks < WIDE_LDS_KS)
+                    k_step(a, cur + ks * 9 * 64, acc);
+                else
+                    k_products(a, breg, acc);
+                __builtin_amdgcn_sched_barrier(0);                       // keeps the operands of later steps out of registers
+            }
+        }
+        const int64_t row0 = tile * 32;
+#pragma unroll
+        for (int ct = 0; ct < 3; ++ct) {
+            float* yp = y + (int64_t)cg * TL_COLS + ct * 32 + l32;
+#pragma unroll
+            for (int rr = 0; rr < 16; ++rr) {
+                const int64_t orow = row0 + acc_row(rr, half);
+                if (orow < N) yp[orow * out] = acc[ct][rr] + bcol[ct];
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
 // Weight and bias gradient of the same layers: dW[P,K] = dY^T X, db[P] = column sums of dY, for
 // dY [N,P] and X [N,K] (autograd of the nn.Linear at swin3d_base.py:606-610).
 //
@@ -595,6 +704,23 @@ static int device_cus() {
 template <bool TRANSPOSED>
 static int launch_chunked(const float* x, int64_t N, int in, const float* w, const float* bias, int out, float* y, int cus,
                           hipStream_t s, const char* what) {
+    if (in / 16 <= WIDE_MAX_KS) {                                        // all of W stays on the CU
+        const int lds_ks = std::min(in / 16, WIDE_LDS_KS);
+        const size_t lds = (size_t)lds_ks * 9 * 64 * sizeof(tl_u32x4);
+        static bool configured_wide = false;
+        if (!configured_wide) {
+            SSWIN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(tall_linear_wide_kernel<TRANSPOSED>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize,
+                                          WIDE_LDS_KS * 9 * 64 * (int)sizeof(tl_u32x4)));
+            configured_wide = true;
+        }
+        const int groups = out / TL_COLS;
+        const int64_t row_tiles = (N + 31) / 32;
+        const int64_t per_group = std::min<int64_t>((row_tiles + 7) / 8, std::max<int64_t>(1, cus / groups));
+        hipLaunchKernelGGL(tall_linear_wide_kernel<TRANSPOSED>, dim3((unsigned)(per_group * groups)), dim3(512), lds, s, x, N, in,
+                           w, groups, bias, y, out, row_tiles);
+        return launch_ok(what);
+    }
     const size_t lds = 2 * (size_t)CH_KS * 9 * 64 * sizeof(tl_u32x4);
     static bool configured = false;
     if (!configured) {
