@@ -611,31 +611,38 @@ __global__ __launch_bounds__(256) void rpb_table_partial_kernel(FusedGroups gt, 
         header(k + 2 * wslices, c_n, T_n, sq_n);
         __builtin_amdgcn_wave_barrier();
         // item = (row i, chunk of 32 columns): all lanes of an item hit different table rows.
-        // The two halves of the wavefront take alternate items and add into separate copies of
-        // the table, so plain read-add-write is enough.  Eight items per half are loaded first.
+        // The two halves of the wavefront take alternate rows and add into separate copies of
+        // the table, so plain read-add-write is enough.  Chunk by chunk (the lane's column and its
+        // code stay fixed), eight rows per half loaded first; addresses advance by a constant.
         const int nch = (c + 31) >> 5;
         const int my_rows = c > rs ? (c - rs + rsplit - 1) / rsplit : 0;
-        const int items = my_rows * nch;
-        int ir = half / nch, ch = half - ir * nch;            // ir counts this slice's rows
-        for (int q0 = 0; q0 < items; q0 += 16) {
-            float v[8];
-            int row[8];
+        const int row_step = 2 * rsplit;                        // rows between a half's consecutive items
+        // Loads are unconditional (indices clamped to the block, dead items get row -1): straight-line
+        // code with all eight loads and code reads of a batch in flight together.
+        const bool have = my_rows > half;                       // this half has rows in this window
+        const int kmax = have ? (my_rows - 1 - half) >> 1 : 0;  // its last item
+        const int i0 = have ? rs + rsplit * half : 0;           // its first row
+        for (int ch = 0; ch < nch; ++ch) {
+            const int j = ch * 32 + l32;
+            const bool jlive = have && j < c;
+            const int jc = j < c ? j : 0;
+            const int cj = cw[jc] - offset0;
+            const float* src = blk + i0 * c + jc;
+            for (int k0 = 0; 2 * k0 < my_rows; k0 += 8) {       // items k0 .. k0 + 7 of each half
+                float v[8];
+                int row[8];
 #pragma unroll
-            for (int u = 0; u < 8; ++u) {
-                const int q = q0 + 2 * u + half;
-                const int j = ch * 32 + l32;
-                const int i = rs + rsplit * ir;
-                const bool live = q < items && j < c;
-                v[u] = live ? blk[i * c + j] : 0.f;
-                const unsigned r = live ? (unsigned)(cw[i] - cw[j] + offset0) : 0xffffffffu;
-                row[u] = r < (unsigned)rows ? (int)r : -1;
-                ch += 2;
-                if (ch >= nch) { ch -= nch; ir += 1; }
-                if (ch >= nch) { ch -= nch; ir += 1; }
+                for (int u = 0; u < 8; ++u) {
+                    const int k = k0 + u;
+                    const int kc = k < kmax ? k : kmax;
+                    v[u] = src[kc * row_step * c];
+                    const unsigned r = (unsigned)(cw[i0 + kc * row_step] - cj);
+                    row[u] = jlive && k <= kmax && r < (unsigned)rows ? (int)r : -1;
+                }
+#pragma unroll
+                for (int u = 0; u < 8; ++u)
+                    if (row[u] >= 0) mine[row[u]] += v[u];
             }
-#pragma unroll
-            for (int u = 0; u < 8; ++u)
-                if (row[u] >= 0) mine[row[u]] += v[u];
         }
         int32_t* cwn = codes + (par ^ 1) * 128;
 #pragma unroll
