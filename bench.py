@@ -348,10 +348,7 @@ def projection_entries(wl):
             with wa._rocblas_gemm():
                 return dy @ w
 
-        if P >= 192:
-            entries.append((f"{name} input gradient", (lambda dy=dy, w=w: wa._split_linear_input_grad(dy, w)), io + 4 * P * D, 1))
-        else:
-            entries.append((f"{name} input gradient (library GEMM)", lib_dx, io + 4 * P * D, 1))
+        entries.append((f"{name} input gradient", (lambda dy=dy, w=w: wa._split_linear_input_grad(dy, w)), io + 4 * P * D, 1))
 
         def lib_fwd(w=w, b=b):
             with wa._rocblas_gemm():
@@ -363,8 +360,7 @@ def projection_entries(wl):
 
         entries += [(f"{name} forward, library GEMM", lib_fwd, io + 4 * P * D, 0),
                     (f"{name} weight+bias gradient, library GEMM + column sums", lib_wgrad, io + 4 * P * D, 0)]
-        if P >= 192:
-            entries.append((f"{name} input gradient, library GEMM", lib_dx, io + 4 * P * D, 0))
+        entries.append((f"{name} input gradient, library GEMM", lib_dx, io + 4 * P * D, 0))
     return entries
 
 

@@ -65,14 +65,23 @@ __device__ __forceinline__ APlanes split8(const tl_f32x4& c0, const tl_f32x4& c1
 
 // The workgroup's 96 columns of W, split and laid out in LDS in operand order:
 // [k step][column tile 3][plane 3][lane 64][8 bf16]
-template <int THREADS>
-__device__ __forceinline__ void fill_w_planes(const float* __restrict__ w, int K, int ksteps, int cg, tl_u32x4* w_s) {
+// TRANSPOSED: the operand is W^T of a [K, P] array (w[k * P + col]: the input gradient of a layer whose
+// weight is stored [out, in]); otherwise w[col * K + k].
+template <int THREADS, bool TRANSPOSED = false>
+__device__ __forceinline__ void fill_w_planes(const float* __restrict__ w, int K, int ksteps, int cg, tl_u32x4* w_s, int P = 0) {
     for (int it = threadIdx.x; it < ksteps * 3 * 64; it += THREADS) {
         const int lane = it & 63, ct = (it >> 6) % 3, ks = (it >> 6) / 3;
-        const int col = cg * TL_COLS + ct * 32 + (lane & 31);
-        const tl_f32x4* src = reinterpret_cast<const tl_f32x4*>(w + (int64_t)col * K + ks * 16 + (lane >> 5) * 8);
-        const tl_f32x4 c0 = src[0], c1 = src[1];
-        const Split2 s0 = split2(c0.x, c0.y), s1 = split2(c0.z, c0.w), s2 = split2(c1.x, c1.y), s3 = split2(c1.z, c1.w);
+        const int col = cg * TL_COLS + ct * 32 + (lane & 31), k0 = ks * 16 + (lane >> 5) * 8;
+        float v[8];
+        if (TRANSPOSED) {
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = w[(int64_t)(k0 + e) * P + col];
+        } else {
+            const tl_f32x4* src = reinterpret_cast<const tl_f32x4*>(w + (int64_t)col * K + k0);
+            const tl_f32x4 c0 = src[0], c1 = src[1];
+            v[0] = c0.x; v[1] = c0.y; v[2] = c0.z; v[3] = c0.w; v[4] = c1.x; v[5] = c1.y; v[6] = c1.z; v[7] = c1.w;
+        }
+        const Split2 s0 = split2(v[0], v[1]), s1 = split2(v[2], v[3]), s2 = split2(v[4], v[5]), s3 = split2(v[6], v[7]);
         tl_u32x4* dst = w_s + (ks * 3 + ct) * 3 * 64 + lane;
         dst[0] = tl_u32x4{s0.h, s1.h, s2.h, s3.h};
         dst[64] = tl_u32x4{s0.m, s1.m, s2.m, s3.m};
@@ -185,7 +194,7 @@ constexpr int TL_STAGED_MAX_KS = 6;
 // SMALL: fewer than 32 rows in all (one ragged tile, guarded).  Otherwise a last ragged tile is moved
 // back to end at row N: it recomputes a few rows of its neighbour (same inputs, same arithmetic, the
 // same bits stored twice) and every tile takes the unguarded path.
-template <int KS, bool SMALL>
+template <int KS, bool SMALL, bool TRANSPOSED = false>
 __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) void tall_linear_forward_staged_kernel(
     const float* __restrict__ x, int64_t N, const float* __restrict__ w, int groups, const float* __restrict__ bias,
     float* __restrict__ y, int P, int64_t row_tiles) {
@@ -197,7 +206,7 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     group_and_slot(groups, cg, slot);
     const int64_t first = (int64_t)slot * 8 + wave, stride = (int64_t)(gridDim.x / groups) * 8;
     constexpr int n16 = KS * 9 * 64;
-    fill_w_planes<512>(w, K, KS, cg, w_s);
+    fill_w_planes<512, TRANSPOSED>(w, K, KS, cg, w_s, P);
     float* xs = reinterpret_cast<float*>(w_s + n16) + wave * 32 * PITCH;
     __syncthreads();
     float bcol[3];
@@ -749,8 +758,25 @@ int sswin_tall_linear_input_grad(const float* dy, int64_t N, int P, const float*
     if (N == 0) return 0;
     SSWIN_CHECK(dy && w && dx, "tall_linear_input_grad: null pointer");
     SSWIN_CHECK(((uintptr_t)dy % 16) == 0, "tall_linear_input_grad: dy must be 16-byte aligned");
-    return launch_chunked<true>(dy, N, P, w, nullptr, K, dx, device_cus(), static_cast<hipStream_t>(stream),
-                                "tall_linear_input_grad");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int cus = device_cus();
+    if (P == 96 && N >= 32) {
+        // 96 channels of dY: the staged kernel of the forward with W read transposed
+        SSWIN_CHECK(((uintptr_t)w % 16) == 0, "tall_linear_input_grad: w must be 16-byte aligned");
+        static bool configured = false;
+        if (!configured) {
+            SSWIN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(tall_linear_forward_staged_kernel<6, false, true>),
+                                          hipFuncAttributeMaxDynamicSharedMemorySize, staged_lds_bytes(6)));
+            configured = true;
+        }
+        const int groups = K / TL_COLS;
+        const int64_t row_tiles = (N + 31) / 32;
+        const int64_t per_group = std::min<int64_t>((row_tiles + 7) / 8, std::max<int64_t>(1, cus / groups));
+        hipLaunchKernelGGL((tall_linear_forward_staged_kernel<6, false, true>), dim3((unsigned)(per_group * groups)), dim3(512),
+                           staged_lds_bytes(6), s, dy, N, w, groups, static_cast<const float*>(nullptr), dx, K, row_tiles);
+        return launch_ok("tall_linear_input_grad");
+    }
+    return launch_chunked<true>(dy, N, P, w, nullptr, K, dx, cus, s, "tall_linear_input_grad");
 }
 
 int sswin_tall_linear_supported(int P, int K) {

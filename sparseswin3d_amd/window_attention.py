@@ -287,8 +287,9 @@ def _split_linear_forward(x: torch.Tensor, weight: torch.Tensor, bias):
 
 
 def _split_linear_input_grad(grad_out: torch.Tensor, weight: torch.Tensor):
-    """``grad_out @ W`` through the library's matrix-core kernel for fp32, where it beats the library
-    GEMM (at least 192 output channels of the layer, i.e. the qkv projection), else None."""
+    """``grad_out @ W`` through the library's matrix-core kernels for fp32, where they beat the library
+    GEMM (96 output channels of the layer and at least 32 rows, or at least 192 output channels), else
+    None."""
     if not (grad_out.is_cuda and grad_out.dtype == torch.float32 and weight.dtype == torch.float32
             and grad_out.dim() == 2 and grad_out.shape[0] > 0):
         return None
@@ -297,7 +298,7 @@ def _split_linear_input_grad(grad_out: torch.Tensor, weight: torch.Tensor):
     lib = _lib.load()
     n, p = grad_out.shape
     k = weight.shape[1]
-    if p < 192 or not lib.sswin_tall_linear_input_grad_supported(p, k):
+    if not (p >= 192 or (p == 96 and n >= 32)) or not lib.sswin_tall_linear_input_grad_supported(p, k):
         return None
     weight = weight.contiguous()
     if grad_out.data_ptr() % 16:
