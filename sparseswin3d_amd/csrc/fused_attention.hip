@@ -100,6 +100,9 @@ __global__ __launch_bounds__(TP_BLOCK) void tp_windows_kernel(const uint32_t* __
     __shared__ int32_t lds_b[TP_BLOCK / 64];
     __shared__ int64_t base_a_s;
     __shared__ int32_t base_b_s;
+    // this slot's bitmap words are requested first: the load overlaps the prefix below
+    const int64_t w = (int64_t)blockIdx.x * TP_BLOCK + threadIdx.x;
+    const int64_t c = w < B ? tp_window_count(bits, w, W) : 0;
     // prefix of the earlier blocks
     int64_t pa = 0;
     int32_t pb = 0;
@@ -119,8 +122,6 @@ __global__ __launch_bounds__(TP_BLOCK) void tp_windows_kernel(const uint32_t* __
     const int64_t base_a = base_a_s;
     const int32_t base_b = base_b_s;
 
-    const int64_t w = (int64_t)blockIdx.x * TP_BLOCK + threadIdx.x;
-    const int64_t c = w < B ? tp_window_count(bits, w, W) : 0;
     const int64_t ea = block_exclusive_scan<int64_t, TP_BLOCK / 64>(c | ((c * c) << 32), lds_a, &ta) + base_a;
     const int32_t k = block_exclusive_scan<int32_t, TP_BLOCK / 64>(c > 0 ? 1 : 0, lds_b, &tb) + base_b;
     if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) {
@@ -148,16 +149,20 @@ __global__ __launch_bounds__(TP_BLOCK) void tp_windows_kernel(const uint32_t* __
     if (lane == 0 && cm > 0) atomicMax(&counters[5], cm);
     if (tasks == nullptr) return;
     const int b = live ? min(((int)c - 1) >> 5, 4) : -1;
+    // lanes 0..4 reserve the slots of the five buckets with one atomic each, at the same time
     int slot = 0;
+    unsigned long long members[5];
+#pragma unroll
+    for (int q = 0; q < 5; ++q) members[q] = __ballot(b == q);
+    unsigned long long mine = 0;
+#pragma unroll
+    for (int q = 0; q < 5; ++q) mine = lane == q ? members[q] : mine;
+    int base = 0;
+    if (lane < 5 && mine != 0) base = atomicAdd(&counters[lane], H * __popcll(mine));
 #pragma unroll
     for (int q = 0; q < 5; ++q) {
-        const unsigned long long mine = __ballot(b == q);
-        if (mine == 0) continue;
-        const int leader = __ffsll((long long)mine) - 1;
-        int base = 0;
-        if (lane == leader) base = atomicAdd(&counters[q], H * __popcll(mine));
-        base = __shfl(base, leader, 64);
-        if (b == q) slot = base + H * __popcll(mine & ((1ull << lane) - 1ull));
+        const int base_q = __shfl(base, q, 64);
+        if (b == q) slot = base_q + H * __popcll(members[q] & ((1ull << lane) - 1ull));
     }
     if (live && b < 4) {
         for (int h = 0; h < H; ++h)
