@@ -252,7 +252,8 @@ int sswin_tall_linear_input_grad(const float* dy, int64_t N, int P, const float*
 
 /* dw[P,K] = dy[N,P]^T x[N,K] and, when db is not NULL, db[P] = column sums of dy: weight and bias
  * gradient of the same layers (autograd of nn.Linear, swin3d_base.py:606-610).  fp32, P a multiple
- * of 96, K = 32, 64 or 96 (the workspace size is 0 for anything else).  Same split-operand
+ * of 96, K = 32, 64, 96 or a multiple of 96 up to 768, taken in passes of 96 columns of x (the
+ * workspace size is 0 for anything else).  Same split-operand
  * arithmetic as the forward; partial sums per workgroup are added in a fixed order, so the result
  * is the same on every run.  dw, db and ws 16-byte aligned.  Asynchronous. */
 size_t sswin_tall_linear_weight_grad_workspace_bytes(int64_t N, int P, int K);

@@ -551,12 +551,16 @@ __device__ __forceinline__ APlanes split_raw8(const Raw8& r) {
     return a;
 }
 
-// XT = K / 32 column tiles of X (1..3)
-template <int XT>
+// XT = K / 32 column tiles of X (1..3); PITCHED: x has more columns than this pass takes (row pitch
+// x_pitch), otherwise its rows are K long and the row offsets are compile-time constants
+// PC: the number of columns of dy when it is known at compile time (row offsets become constants), else 0
+template <int XT, bool PITCHED, int PC = 0>
 __global__ __launch_bounds__(WG_WAVES * 64) __attribute__((amdgpu_waves_per_eu(3, 3))) void tall_linear_wgrad_kernel(
-    const float* __restrict__ dy, const float* __restrict__ x, int64_t N, int P, int groups, int64_t rows_per_chunk,
-    float* __restrict__ part_w, float* __restrict__ part_b) {
-    constexpr int K = XT * 32;
+    const float* __restrict__ dy, const float* __restrict__ x, int x_pitch, int64_t N, int P_rt, int groups,
+    int64_t rows_per_chunk, float* __restrict__ part_w, float* __restrict__ part_b) {
+    constexpr int K = XT * 32;                                           // columns of X in this pass (x: their first column)
+    const int xp = PITCHED ? x_pitch : K;
+    const int P = PC ? PC : P_rt;
     // X planes: [buffer 2][quarter 4][tile XT][plane 3][lane 64] x 16 bytes; reused for the final sums
     extern __shared__ __attribute__((aligned(16))) tl_u32x4 lds[];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // wave: a scalar
@@ -577,23 +581,23 @@ __global__ __launch_bounds__(WG_WAVES * 64) __attribute__((amdgpu_waves_per_eu(3
     // rows are requested two steps ahead (loaded HBM latency is about two steps of products)
     Raw8 ry[2], rx[2];
     // addresses: a uniform part (scalar arithmetic) plus a per-lane offset computed once
-    const uint32_t y_lane = (uint32_t)(half * 8 * P + ycol), x_lane = (uint32_t)(half * 8 * K + xcol);
+    const uint32_t y_lane = (uint32_t)(half * 8 * P + ycol), x_lane = (uint32_t)(half * 8 * xp + xcol);
     auto fetch = [&](int s, Raw8& y8, Raw8& x8) {
         const int64_t r0 = row_begin + (int64_t)s * WG_STEP_ROWS + quarter * 16;
         const float* yb = dy + r0 * P;
-        const float* xb = x + r0 * K;
+        const float* xb = x + r0 * xp;
         if (r0 + 16 <= row_end) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 y8.v[e] = (yb + e * P)[y_lane];
-                if (t < XT) x8.v[e] = (xb + e * K)[x_lane];
+                if (t < XT) x8.v[e] = (xb + e * xp)[x_lane];
             }
         } else {                                                         // the ragged end of the rows: zeros past it
             const int nvalid = (int)(row_end - r0) - half * 8;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
                 y8.v[e] = e < nvalid ? (yb + e * P)[y_lane] : 0.f;
-                if (t < XT) x8.v[e] = e < nvalid ? (xb + e * K)[x_lane] : 0.f;
+                if (t < XT) x8.v[e] = e < nvalid ? (xb + e * xp)[x_lane] : 0.f;
             }
         }
     };
@@ -673,7 +677,8 @@ __global__ __launch_bounds__(WG_WAVES * 64) __attribute__((amdgpu_waves_per_eu(3
 // tree.  part_w and part_b are contiguous ([chunks][PK] then [chunks][P]), so e runs over both.
 __global__ __launch_bounds__(256) void tall_linear_wgrad_reduce_kernel(const float* __restrict__ part_w,
                                                                        const float* __restrict__ part_b, int chunks, int PK,
-                                                                       int P, float* __restrict__ dw, float* __restrict__ db) {
+                                                                       int P, int K, float* __restrict__ dw, int dw_pitch,
+                                                                       float* __restrict__ db) {
     __shared__ tl_f32x4 sums[16][17];
     const int el = threadIdx.x & 15, cl = threadIdx.x >> 4;
     const int e = (blockIdx.x * 16 + el) * 4;
@@ -691,7 +696,8 @@ __global__ __launch_bounds__(256) void tall_linear_wgrad_reduce_kernel(const flo
         if (cl < w) sums[cl][el] += sums[cl + w][el];
         __syncthreads();
     }
-    if (cl == 0 && valid) *reinterpret_cast<tl_f32x4*>(weight ? dw + e : db + (e - PK)) = sums[0][el];
+    if (cl == 0 && valid)                                                // dw: this pass's K columns of rows of dw_pitch
+        *reinterpret_cast<tl_f32x4*>(weight ? dw + (int64_t)(e / K) * dw_pitch + e % K : db + (e - PK)) = sums[0][el];
 }
 
 }  // namespace sswin
@@ -863,30 +869,37 @@ static void wgrad_split(int64_t N, int groups, int cus, int64_t* rows_per_chunk,
 
 extern "C" {
 
+static bool wgrad_shape_ok(int P, int K) {
+    // up to 96 input channels in one pass, more in passes of 96
+    return P > 0 && K > 0 && (P % 96) == 0 && (K % 32) == 0 && (K <= 96 || ((K % 96) == 0 && K <= 768));
+}
+
 size_t sswin_tall_linear_weight_grad_workspace_bytes(int64_t N, int P, int K) {
-    if (N <= 0 || P <= 0 || K <= 0 || (P % 96) || (K % 32) || K > 96) return 0;
+    if (N <= 0 || !wgrad_shape_ok(P, K)) return 0;
     int64_t rows;
     int chunks;
     wgrad_split(N, P / 96, device_cus(), &rows, &chunks);
-    return (size_t)chunks * ((size_t)P * K + P) * sizeof(float) + 256;
+    const int kp = std::min(K, 96);
+    return (size_t)chunks * ((size_t)P * kp + P) * sizeof(float) + 256;
 }
 
 int sswin_tall_linear_weight_grad(const float* dy, const float* x, int64_t N, int P, int K, float* dw, float* db, void* ws,
                                   size_t ws_bytes, void* stream) {
     SSWIN_CHECK(N > 0 && P > 0 && K > 0, "tall_linear_weight_grad: bad sizes");
     SSWIN_CHECK(P % 96 == 0, "tall_linear_weight_grad: %d output channels are not a multiple of 96", P);
-    SSWIN_CHECK(K % 32 == 0 && K <= 96, "tall_linear_weight_grad: %d input channels are not supported (32, 64 or 96)", K);
+    SSWIN_CHECK(wgrad_shape_ok(P, K),
+                "tall_linear_weight_grad: %d input channels are not supported (32, 64, 96 or a multiple of 96 up to 768)", K);
     SSWIN_CHECK(dy && x && dw && ws, "tall_linear_weight_grad: null pointer");
     SSWIN_CHECK(((uintptr_t)dw % 16) == 0 && ((uintptr_t)db % 16) == 0 && ((uintptr_t)ws % 16) == 0,
                 "tall_linear_weight_grad: dw, db and the workspace must be 16-byte aligned");
     SSWIN_CHECK(ws_bytes >= sswin_tall_linear_weight_grad_workspace_bytes(N, P, K), "tall_linear_weight_grad: workspace too small");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const int groups = P / 96, xt = K / 32;
+    const int groups = P / 96, kp = std::min(K, 96), xt = kp / 32, passes = K / kp;
     int64_t rows;
     int chunks;
     wgrad_split(N, groups, device_cus(), &rows, &chunks);
     float* part_w = static_cast<float*>(ws);
-    float* part_b = part_w + (size_t)chunks * P * K;
+    float* part_b = part_w + (size_t)chunks * P * kp;
     // LDS: the double-buffered planes of X, or the two rounds of the final sums, whichever is larger
     const size_t planes = 2 * (size_t)WG_QUARTERS * xt * 3 * 64 * sizeof(tl_u32x4);
     const size_t sums = 6 * (size_t)(xt * 16 + 1) * 64 * sizeof(float);
@@ -894,25 +907,38 @@ int sswin_tall_linear_weight_grad(const float* dy, const float* x, int64_t N, in
     static bool configured = false;
     if (!configured) {
         const int max_lds = 96 * 1024;
-        SSWIN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(tall_linear_wgrad_kernel<1>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, max_lds));
-        SSWIN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(tall_linear_wgrad_kernel<2>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, max_lds));
-        SSWIN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(tall_linear_wgrad_kernel<3>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, max_lds));
+        const void* all[] = {reinterpret_cast<const void*>(tall_linear_wgrad_kernel<1, false>),
+                             reinterpret_cast<const void*>(tall_linear_wgrad_kernel<2, false>),
+                             reinterpret_cast<const void*>(tall_linear_wgrad_kernel<3, false>),
+                             reinterpret_cast<const void*>(tall_linear_wgrad_kernel<3, true>),
+                             reinterpret_cast<const void*>(tall_linear_wgrad_kernel<3, false, 96>),
+                             reinterpret_cast<const void*>(tall_linear_wgrad_kernel<3, false, 288>)};
+        for (const void* k : all) SSWIN_HIP(hipFuncSetAttribute(k, hipFuncAttributeMaxDynamicSharedMemorySize, max_lds));
         configured = true;
     }
     const dim3 grid((unsigned)(chunks * groups)), block(WG_WAVES * 64);
-    switch (xt) {
-        case 1: hipLaunchKernelGGL(tall_linear_wgrad_kernel<1>, grid, block, lds, s, dy, x, N, P, groups, rows, part_w, part_b); break;
-        case 2: hipLaunchKernelGGL(tall_linear_wgrad_kernel<2>, grid, block, lds, s, dy, x, N, P, groups, rows, part_w, part_b); break;
-        default: hipLaunchKernelGGL(tall_linear_wgrad_kernel<3>, grid, block, lds, s, dy, x, N, P, groups, rows, part_w, part_b); break;
+    const int PK = P * kp, total4 = (PK + P) / 4;
+    // one pass per 96 columns of X: the partial buffer is reused, the column sums of dy come from the first
+    for (int pass = 0; pass < passes; ++pass) {
+        const float* xp = x + pass * kp;
+        if (passes > 1)
+            hipLaunchKernelGGL((tall_linear_wgrad_kernel<3, true>), grid, block, lds, s, dy, xp, K, N, P, groups, rows, part_w, part_b);
+        else if (xt == 1)
+            hipLaunchKernelGGL((tall_linear_wgrad_kernel<1, false>), grid, block, lds, s, dy, xp, K, N, P, groups, rows, part_w, part_b);
+        else if (xt == 2)
+            hipLaunchKernelGGL((tall_linear_wgrad_kernel<2, false>), grid, block, lds, s, dy, xp, K, N, P, groups, rows, part_w, part_b);
+        else if (P == 96)
+            hipLaunchKernelGGL((tall_linear_wgrad_kernel<3, false, 96>), grid, block, lds, s, dy, xp, K, N, P, groups, rows, part_w, part_b);
+        else if (P == 288)
+            hipLaunchKernelGGL((tall_linear_wgrad_kernel<3, false, 288>), grid, block, lds, s, dy, xp, K, N, P, groups, rows, part_w, part_b);
+        else
+            hipLaunchKernelGGL((tall_linear_wgrad_kernel<3, false>), grid, block, lds, s, dy, xp, K, N, P, groups, rows, part_w, part_b);
+        if (int rc = launch_ok("tall_linear_weight_grad")) return rc;
+        hipLaunchKernelGGL(tall_linear_wgrad_reduce_kernel, dim3((unsigned)((total4 + 15) / 16)), dim3(256), 0, s, part_w, part_b,
+                           chunks, PK, P, kp, dw + pass * kp, K, pass == 0 ? db : nullptr);
+        if (int rc = launch_ok("tall_linear_weight_grad reduce")) return rc;
     }
-    if (int rc = launch_ok("tall_linear_weight_grad")) return rc;
-    const int PK = P * K, total4 = (PK + P) / 4;
-    hipLaunchKernelGGL(tall_linear_wgrad_reduce_kernel, dim3((unsigned)((total4 + 15) / 16)), dim3(256), 0, s, part_w, part_b, chunks,
-                       PK, P, dw, db);
-    return launch_ok("tall_linear_weight_grad reduce");
+    return 0;
 }
 
 }  // extern "C"

@@ -94,6 +94,8 @@ def test_tall_linear_rejects_unsupported_shapes():
 @pytest.mark.parametrize("N,K,P,bias", [
     (107500, 96, 288, True), (107500, 96, 96, True), (1, 96, 96, True), (63, 32, 96, False), (65, 64, 192, True),
     (1000, 96, 96, True), (4099, 96, 288, False), (20000, 32, 288, True),
+    (25900, 192, 576, True),        # qkv of stage 2: two passes of 96 columns of x
+    (3000, 288, 96, True), (130, 384, 192, False),
 ])
 def test_tall_linear_weight_grad(N, K, P, bias):
     """dW = dY^T X and db = column sums of dY against float64 on the same fp32 inputs; the same bits on
@@ -169,7 +171,8 @@ def test_tall_linear_weight_grad_unsupported_shapes():
     from sparseswin3d_amd import _lib
     lib = _lib.load()
     assert lib.sswin_tall_linear_weight_grad_workspace_bytes(1000, 100, 96) == 0
-    assert lib.sswin_tall_linear_weight_grad_workspace_bytes(1000, 96, 192) == 0
+    assert lib.sswin_tall_linear_weight_grad_workspace_bytes(1000, 96, 160) == 0
+    assert lib.sswin_tall_linear_weight_grad_workspace_bytes(1000, 96, 864) == 0
     assert lib.sswin_tall_linear_weight_grad_workspace_bytes(1000, 96, 48) == 0
     assert lib.sswin_tall_linear_weight_grad_workspace_bytes(0, 96, 96) == 0
     t = torch.zeros(64, 96, device="cuda")
