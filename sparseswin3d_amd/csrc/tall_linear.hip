@@ -1,20 +1,28 @@
-// Y = X W^T + b for a very tall fp32 X [N, K] (N = voxels, K = channels <= 192) and a small weight
-// W [P, K]: the qkv and proj projections of the window attention (nn.Linear of
-// sparse_swin/swin3d_base.py:606-610, applied at :658 and :676).
+// The qkv and proj projections of the window attention (nn.Linear of sparse_swin/swin3d_base.py:606-610,
+// applied at :658 and :676) for fp32 tokens: Y = X W^T + b for a very tall X [N, K] (N = voxels) and a
+// small weight W [P, K], the input gradient dX = dY W and the weight / bias gradient dW = dY^T X,
+// db = column sums of dY.
 //
 // On gfx950 the fp32 matrix instruction runs on the vector ALU's own multipliers (64 FLOP per clock
 // and SIMD, and it blocks the ALU while it runs), so an fp32 GEMM cannot get past the packed-FMA rate;
-// the bf16 matrix cores are sixteen times faster and sit idle.  This kernel uses them without giving
+// the bf16 matrix cores are sixteen times faster and sit idle.  These kernels use them without giving
 // up fp32 accuracy: every fp32 operand is split exactly into three bf16 pieces (x = h + m + l, 8 + 8 +
 // 8 significant bits, by truncation and exact subtraction) and a product is the sum of the six
 // piece products whose weight is at least 2^-16 of the leading one (hh, hm, mh, mm, hl, lh), all
 // accumulated in fp32 by v_mfma_f32_32x32x16_bf16.  What is dropped (ml, lm, ll) is below 2^-23 of
-// the product, i.e. at the level of fp32 rounding itself.
+// the product, i.e. at the level of fp32 rounding itself.  Inputs are taken to be finite (the pieces
+// of an infinity are infinity and NaN).
 //
-// Layout: a workgroup owns one group of 96 output columns and keeps the three bf16 planes of those
-// columns of W in LDS in MFMA operand order (split by the workgroup itself when it starts); it
-// walks over blocks of 128 rows, one 32-row tile per wave.  Per 16-wide k step a lane reads its
-// 8 fp32 of X (row l % 32, k group l / 32), splits them, and feeds 3 column tiles x 6 products.
+// Common layout of the row-streaming kernels (forward, input gradient): a workgroup owns one group of
+// 96 output columns and keeps the three bf16 planes of those columns of W in LDS in MFMA operand order
+// (it splits them itself when it starts); its waves walk over 32-row tiles.  Per 16-wide k step a
+// lane holds 8 fp32 of X (row l % 32, k group l / 32), splits them, and feeds 3 column tiles x 6
+// products.  Kernels, by shape:
+//   tall_linear_forward_staged_kernel   K <= 96 (also dX of a 96-column dY, W read transposed)
+//   tall_linear_forward_kernel          96 < K <= 192
+//   tall_linear_wide_kernel             dX for 192..288 columns of dY: all of W on the CU
+//   tall_linear_chunked_kernel          dX for more columns of dY: W in chunks of 96 rows
+//   tall_linear_wgrad_kernel (+ reduce) dW and db, the reduction over the rows
 #include <stdint.h>
 
 #include <algorithm>
