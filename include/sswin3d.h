@@ -216,6 +216,12 @@ int sswin_fused_bias_grad(const int32_t* plan, int64_t g_cap, int64_t G, const i
                           int64_t N, int H, int n, const float* ds, float* d_bias, void* ws,
                           size_t ws_bytes, void* stream);
 
+/* bias[H,n,n] (fp32) from the relative position bias table [table_rows, H] (fp32):
+ * bias[h][p][q] = table[code[p] - code[q] + offset0][h], the gather and permute of
+ * swin3d_base.py:644-647 in one launch (code as for sswin_bias_table_grad).  Asynchronous. */
+int sswin_bias_from_table(const float* table, int table_rows, int H, const int32_t* code, int offset0,
+                          int n, float* bias, void* stream);
+
 /* Gradient of the relative position bias table itself (swin3d_base.py:624-652 gathers the
  * [H,n,n] bias from a [(2w-1)^3, H] table by relative_position_index; autograd scatters back with
  * an index_add).  The index is linear in the two positions: rel(p_i,p_j) = code[p_i] - code[p_j]

@@ -46,6 +46,7 @@ SIGNATURES = {
     "sswin_fused_bias_grad": (_i32, [_vp, _i64, _i64, _vp, _i64, _i32, _i32, _vp, _vp, _vp, _sz, _vp]),
     "sswin_column_sum_workspace_bytes": (_sz, [_i64, _i32]),
     "sswin_column_sum": (_i32, [_vp, _i32, _i64, _i32, _vp, _vp, _sz, _vp]),
+    "sswin_bias_from_table": (_i32, [_vp, _i32, _i32, _vp, _i32, _i32, _vp, _vp]),
     "sswin_bias_table_grad_workspace_bytes": (_sz, [_i64, _i32, _i32]),
     "sswin_bias_table_grad": (_i32, [_vp, _i64, _i64, _vp, _i64, _i32, _i32, _vp, _i32, _i32, _vp, _vp, _vp, _sz, _vp]),
     "sswin_tall_linear_supported": (_i32, [_i32, _i32]),
@@ -67,7 +68,7 @@ SIGNATURES = {
                                                _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i32, _vp]),
 }
 
-ABI_VERSION = 12
+ABI_VERSION = 13
 _lib = None
 
 

@@ -560,6 +560,18 @@ __global__ __launch_bounds__(256) void rpb_grad_reduce_kernel(const float* __res
 // the column each (LDS float atomics would be an order of magnitude slower).  Partial columns are
 // summed in slice order by rpb_table_reduce_kernel.
 // ------------------------------------------------------------------------------------------
+// bias[h][p][q] = table[code[p] - code[q] + offset0][h]: the gather of swin3d_base.py:644-647 and its
+// permute(2, 0, 1) in one pass (entries whose table row is out of range read as zero).
+__global__ __launch_bounds__(256) void rpb_gather_kernel(const float* __restrict__ table, int rows, int H,
+                                                         const int32_t* __restrict__ code, int offset0, int n,
+                                                         float* __restrict__ bias) {
+    const int e = blockIdx.x * 256 + threadIdx.x;
+    if (e >= n * n) return;
+    const int p = e / n, q = e - p * n;
+    const unsigned r = (unsigned)(code[p] - code[q] + offset0);
+    for (int h = 0; h < H; ++h) bias[(int64_t)h * n * n + e] = r < (unsigned)rows ? table[(int64_t)r * H + h] : 0.f;
+}
+
 constexpr int RPBT_MAX_ROWS = 1024;
 
 // dynamic LDS: [wave 4][half 2][rows_pad] floats, then [wave 4][buffer 2][128] position codes
@@ -932,6 +944,15 @@ int sswin_bias_table_grad(const int32_t* plan, int64_t g_cap, int64_t G, const i
     hipLaunchKernelGGL(rpb_table_reduce_kernel, dim3((unsigned)((table_rows + 15) / 16), (unsigned)H), dim3(1024), 0, s,
                        partial, slices, table_rows, H, d_table);
     return launch_ok("bias table gradient");
+}
+
+int sswin_bias_from_table(const float* table, int table_rows, int H, const int32_t* code, int offset0, int n, float* bias,
+                          void* stream) {
+    SSWIN_CHECK(table_rows > 0 && H > 0 && n > 0 && n <= 4096, "bias_from_table: bad sizes");
+    SSWIN_CHECK(table && code && bias, "bias_from_table: null pointer");
+    hipLaunchKernelGGL(rpb_gather_kernel, dim3((unsigned)((n * n + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       table, table_rows, H, code, offset0, n, bias);
+    return launch_ok("bias_from_table");
 }
 
 }  // extern "C"

@@ -199,8 +199,12 @@ class _ResidentWindowAttention(Function):
         if table_index is None:
             bias32 = bias.detach().to(torch.float32).contiguous()
         else:
-            bias32 = (bias.detach().to(torch.float32).index_select(0, table_index.flat).reshape(n, n, H)
-                      .permute(2, 0, 1).contiguous())
+            table32 = bias.detach().to(torch.float32).contiguous()
+            bias32 = torch.empty((H, n, n), dtype=torch.float32, device=d)
+            with torch.cuda.device(d):
+                _lib.check(_lib.load().sswin_bias_from_table(
+                    _ptr(table32), table32.shape[0], H, _ptr(table_index.code), table_index.offset0, n, _ptr(bias32),
+                    C.c_void_p(torch.cuda.current_stream(d).cuda_stream)))
         if mask is not None:
             mask = mask.to(torch.int8).contiguous()
         lib = _lib.load()

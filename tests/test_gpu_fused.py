@@ -242,3 +242,25 @@ def test_bias_table_gradient(mix, H):
     _lib.check(lib.sswin_bias_table_grad(_ptr(tp.plan), tp.g_cap, tp.G, _ptr(tp.tokens), tp.N, H, n, _ptr(ti.code),
                                          ti.offset0, rows, _ptr(ds_d), _ptr(out2), _ptr(ws), nbytes, stream))
     assert torch.equal(out, out2)                       # same bits on every run
+
+
+def test_bias_from_table_matches_the_gather():
+    """sswin_bias_from_table against table[relative_position_index].permute(2, 0, 1)
+    (sparse_swin/swin3d_base.py:644-647): a copy, so bit-exact."""
+    import ctypes as C
+    from sparseswin3d_amd import _lib, fused
+    from sparseswin3d_amd.window_attention import relative_position_index_3d
+    lib = _lib.load()
+    for ws, H in (((5, 5, 5), 3), ((3, 4, 2), 2), ((1, 1, 1), 1)):
+        n = ws[0] * ws[1] * ws[2]
+        rows = (2 * ws[0] - 1) * (2 * ws[1] - 1) * (2 * ws[2] - 1)
+        index = relative_position_index_3d(ws).cuda()
+        ti = fused.BiasTableIndex.build(index, rows)
+        assert ti is not None
+        table = torch.randn(rows, H, device="cuda")
+        out = torch.full((H, n, n), float("nan"), device="cuda")
+        _lib.check(lib.sswin_bias_from_table(C.c_void_p(table.data_ptr()), rows, H, C.c_void_p(ti.code.data_ptr()), ti.offset0,
+                                             n, C.c_void_p(out.data_ptr()),
+                                             C.c_void_p(torch.cuda.current_stream().cuda_stream)))
+        ref = table[index.reshape(-1)].reshape(n, n, H).permute(2, 0, 1)
+        assert torch.equal(out, ref)
