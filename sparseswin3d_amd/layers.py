@@ -19,7 +19,7 @@ from torch.autograd import Function
 from torch.autograd.function import once_differentiable
 
 from . import _lib
-from .window_attention import WindowAttentionSparse, replace_feature
+from .window_attention import WindowAttentionSparse, replace_feature, tall_linear
 
 _DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 
@@ -219,7 +219,7 @@ class PoolDownsample(nn.Module):
         pooled = _PoolWindows.apply(x.features, plan, True)
         out = copy.copy(x)
         out.indices, out.spatial_shape = coords, shape
-        out.features = self.reduction(self.norm(pooled))
+        out.features = tall_linear(self.norm(pooled), self.reduction)
         return out
 
 
@@ -248,7 +248,9 @@ class MLP(nn.Module):
         self.drop2 = nn.Dropout(dropout_rate)
 
     def forward(self, x):
-        return self.drop2(self.linear2(self.drop1(self.fn(self.linear1(x)))))
+        # tall 2-D fp32 inputs on the GPU take the projection kernels of the attention (same results as
+        # nn.Linear to fp32 rounding); anything else is nn.Linear itself
+        return self.drop2(tall_linear(self.drop1(self.fn(tall_linear(x, self.linear1))), self.linear2))
 
 
 class DropPath(nn.Module):
