@@ -241,7 +241,7 @@ int sswin_column_sum(const void* x, int dtype, int64_t N, int P, float* out, voi
 
 /* y[N,P] = x[N,K] w[P,K]^T + bias[P] (bias may be NULL) for dense fp32 row-major arrays: the forward
  * of the qkv and proj nn.Linear (swin3d_base.py:606-610, applied at :658 and :676).  K a multiple of
- * 16, at most 192; P a multiple of 96 (sswin_tall_linear_supported tells).  Runs on the bf16 matrix
+ * 16 up to 192 or of 96 up to 768; P a multiple of 96 (sswin_tall_linear_supported tells).  Runs on the bf16 matrix
  * cores with every fp32 operand split exactly into three bf16 pieces and the six largest piece
  * products summed in fp32: results agree with an fp32 GEMM to its own rounding level.  x and w
  * 16-byte aligned.  Asynchronous, no workspace. */

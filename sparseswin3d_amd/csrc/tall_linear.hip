@@ -794,14 +794,15 @@ int sswin_tall_linear_input_grad(const float* dy, int64_t N, int P, const float*
 }
 
 int sswin_tall_linear_supported(int P, int K) {
-    return P > 0 && K > 0 && (P % TL_COLS) == 0 && (K % 16) == 0 && K <= TL_MAX_K;
+    return P > 0 && K > 0 && (P % TL_COLS) == 0 && (K % 16) == 0 && (K <= TL_MAX_K || ((K % 96) == 0 && K <= 768));
 }
 
 int sswin_tall_linear_forward(const float* x, int64_t N, int K, const float* w, const float* bias, int P, float* y,
                               void* stream) {
     SSWIN_CHECK(N >= 0 && K > 0 && P > 0, "tall_linear_forward: bad sizes");
-    SSWIN_CHECK(K % 16 == 0 && K <= TL_MAX_K, "tall_linear_forward: %d input channels are not supported (a multiple of 16, at most %d)",
-                K, TL_MAX_K);
+    SSWIN_CHECK(K % 16 == 0 && (K <= TL_MAX_K || (K % 96 == 0 && K <= 768)),
+                "tall_linear_forward: %d input channels are not supported (a multiple of 16 up to %d, or of 96 up to 768)", K,
+                TL_MAX_K);
     SSWIN_CHECK(P % TL_COLS == 0, "tall_linear_forward: %d output channels are not a multiple of %d", P, TL_COLS);
     if (N == 0) return 0;
     SSWIN_CHECK(x && w && y, "tall_linear_forward: null pointer");
@@ -856,6 +857,7 @@ int sswin_tall_linear_forward(const float* x, int64_t N, int K, const float* w, 
 #undef SSWIN_TL_STAGED
         return launch_ok("tall_linear_forward");
     }
+    if (K > TL_MAX_K) return launch_chunked<false>(x, N, K, w, bias, P, y, cus, s, "tall_linear_forward");
     const size_t lds = (size_t)ksteps * 9 * 64 * sizeof(tl_u32x4);
     const int64_t row_blocks = (N + 127) / 128;
     const int per_cu = lds <= 64 * 1024 ? 2 : 1;                          // workgroups that fit a CU's LDS

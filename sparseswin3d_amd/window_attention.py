@@ -268,7 +268,7 @@ def _split_linear_forward(x: torch.Tensor, weight: torch.Tensor, bias):
     lib = _lib.load()
     n, k = x.shape
     p = weight.shape[0]
-    if not lib.sswin_tall_linear_supported(p, k):
+    if not lib.sswin_tall_linear_supported(p, k) or (k > 192 and n < 20000):   # few rows, many channels: the library wins
         return None
     x = x.contiguous()
     weight = weight.contiguous()

@@ -36,6 +36,8 @@ def _run(lib, _lib, x, w, b):
     (6500, 192, 192, False),
     (1, 96, 96, True), (31, 16, 96, False), (33, 32, 192, True), (257, 48, 96, True), (1000, 64, 96, False),
     (4097, 80, 288, True), (129, 112, 96, True), (300, 176, 192, True),
+    (107500, 384, 96, True),        # second layer of the block's MLP: four chunks of 96 channels
+    (3000, 288, 96, False), (700, 768, 192, True),
 ])
 def test_tall_linear_forward(N, K, P, bias):
     from sparseswin3d_amd import _lib
@@ -80,7 +82,9 @@ def test_tall_linear_rejects_unsupported_shapes():
     assert lib.sswin_tall_linear_supported(288, 96) == 1
     assert lib.sswin_tall_linear_supported(100, 96) == 0             # columns not a multiple of 96
     assert lib.sswin_tall_linear_supported(96, 100) == 0             # channels not a multiple of 16
-    assert lib.sswin_tall_linear_supported(96, 384) == 0             # too many channels
+    assert lib.sswin_tall_linear_supported(96, 384) == 1             # chunks of 96 channels
+    assert lib.sswin_tall_linear_supported(96, 208) == 0             # above 192: multiples of 96 only
+    assert lib.sswin_tall_linear_supported(96, 864) == 0             # too many channels
     x = torch.zeros(8, 100, device="cuda")
     w = torch.zeros(96, 100, device="cuda")
     y = torch.zeros(8, 96, device="cuda")
