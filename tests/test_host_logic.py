@@ -1,0 +1,38 @@
+"""Host-side logic that needs no GPU: which dense layers the projection kernels take, and that the
+layers they do not take fall through to ``nn.Linear`` unchanged."""
+import torch
+
+
+def test_tall_linear_on_cpu_is_the_plain_layer():
+    from sparseswin3d_amd.window_attention import tall_linear
+    torch.manual_seed(0)
+    layer = torch.nn.Linear(96, 288)
+    x = torch.randn(50, 96, requires_grad=True)
+    y = tall_linear(x, layer)
+    ref = layer(x)
+    assert torch.equal(y, ref)
+    y.sum().backward()
+    assert x.grad is not None and layer.weight.grad is not None
+
+
+def test_mlp_on_cpu_matches_its_definition():
+    """linear, activation, dropout, linear, dropout (the block's feed-forward part)."""
+    from sparseswin3d_amd.layers import MLP
+    torch.manual_seed(1)
+    mlp = MLP(32, 128).eval()
+    x = torch.randn(7, 32)
+    ref = mlp.linear2(torch.nn.functional.gelu(mlp.linear1(x)))
+    assert torch.allclose(mlp(x), ref)
+    x3 = torch.randn(2, 5, 32)                      # not 2-D: nn.Linear itself
+    assert mlp(x3).shape == (2, 5, 32)
+
+
+def test_split_linear_helpers_decline_what_the_kernels_do_not_take():
+    """CPU tensors, 16-bit tensors and empty inputs are left to the library path (None), without loading
+    the HIP library."""
+    from sparseswin3d_amd import window_attention as wa
+    x = torch.randn(40, 96)
+    w = torch.randn(288, 96)
+    assert wa._split_linear_forward(x, w, None) is None
+    assert wa._split_linear_input_grad(torch.randn(40, 288), w) is None
+    assert wa._split_linear_weight_grad(torch.randn(40, 288), x, True) == (None, None)
