@@ -288,8 +288,7 @@ def _split_linear_forward(x: torch.Tensor, weight: torch.Tensor, bias):
 
 def _split_linear_input_grad(grad_out: torch.Tensor, weight: torch.Tensor):
     """``grad_out @ W`` through the library's matrix-core kernels for fp32, where they beat the library
-    GEMM (96 output channels of the layer and at least 32 rows, or at least 192 output channels), else
-    None."""
+    GEMM (see the row thresholds below), else None."""
     if not (grad_out.is_cuda and grad_out.dtype == torch.float32 and weight.dtype == torch.float32
             and grad_out.dim() == 2 and grad_out.shape[0] > 0):
         return None
@@ -298,7 +297,10 @@ def _split_linear_input_grad(grad_out: torch.Tensor, weight: torch.Tensor):
     lib = _lib.load()
     n, p = grad_out.shape
     k = weight.shape[1]
-    if not (p >= 192 or (p == 96 and n >= 32)) or not lib.sswin_tall_linear_input_grad_supported(p, k):
+    # measured against rocBLAS on an MI355X: the 96-column kernel wins from 32 rows on, the kernel that keeps
+    # all of W on the CU (192..288 columns) from about 16 000 rows, the chunked one from about 60 000
+    enough_rows = n >= 32 if p == 96 else n >= 16000 if p <= 288 else n >= 60000
+    if p < 96 or (96 < p < 192) or not enough_rows or not lib.sswin_tall_linear_input_grad_supported(p, k):
         return None
     weight = weight.contiguous()
     if grad_out.data_ptr() % 16:
@@ -323,6 +325,8 @@ def _split_linear_weight_grad(grad_out: torch.Tensor, x: torch.Tensor, want_bias
     lib = _lib.load()
     n, k = x.shape
     p = grad_out.shape[1]
+    if k > 96 and n < 16000:                     # passes of 96 columns over few rows: the library wins
+        return None, None
     nbytes = int(lib.sswin_tall_linear_weight_grad_workspace_bytes(n, p, k))
     if nbytes == 0:
         return None, None
