@@ -445,9 +445,8 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
     group_and_slot(groups, cg, slot);
     const int64_t first = (int64_t)slot * 8 + wave, stride = (int64_t)(gridDim.x / groups) * 8;
 
-    // 8 values of Wop for (column, k0 .. k0 + 7), split into planes
-    auto w_planes = [&](int col, int k0, tl_u32x4& h, tl_u32x4& m, tl_u32x4& l) {
-        float v[8];
+    // 8 values of Wop for (column, k0 .. k0 + 7)
+    auto w_load = [&](int col, int k0, float (&v)[8]) {
         if (TRANSPOSED) {
 #pragma unroll
             for (int e = 0; e < 8; ++e) v[e] = w[(int64_t)(k0 + e) * out + col];
@@ -456,26 +455,45 @@ __global__ __launch_bounds__(512) __attribute__((amdgpu_waves_per_eu(2, 2))) voi
             const tl_f32x4 c0 = src[0], c1 = src[1];
             v[0] = c0.x; v[1] = c0.y; v[2] = c0.z; v[3] = c0.w; v[4] = c1.x; v[5] = c1.y; v[6] = c1.z; v[7] = c1.w;
         }
+    };
+    auto w_split = [&](const float (&v)[8], tl_u32x4& h, tl_u32x4& m, tl_u32x4& l) {
         const Split2 s0 = split2(v[0], v[1]), s1 = split2(v[2], v[3]), s2 = split2(v[4], v[5]), s3 = split2(v[6], v[7]);
         h = tl_u32x4{s0.h, s1.h, s2.h, s3.h};
         m = tl_u32x4{s0.m, s1.m, s2.m, s3.m};
         l = tl_u32x4{s0.l, s1.l, s2.l, s3.l};
     };
-    for (int it = threadIdx.x; it < lds_ks * 3 * 64; it += 512) {
-        const int ln = it & 63, ct = (it >> 6) % 3, ks = (it >> 6) / 3;
-        tl_u32x4 h, m, l;
-        w_planes(cg * TL_COLS + ct * 32 + (ln & 31), ks * 16 + (ln >> 5) * 8, h, m, l);
-        tl_u32x4* dst = w_s + (it >> 6) * 3 * 64 + ln;
-        dst[0] = h;
-        dst[64] = m;
-        dst[128] = l;
+    // The fill is a chain of memory latencies if it goes item by item, so all of a thread's values (at
+    // most 7 items of the LDS part and the 3 of the register part) are requested first.
+    constexpr int FILL_ITEMS = (WIDE_LDS_KS * 3 * 64 + 511) / 512;
+    const int total = lds_ks * 3 * 64;
+    float wv[FILL_ITEMS][8], wr[3][8];
+#pragma unroll
+    for (int q = 0; q < FILL_ITEMS; ++q) {
+        const int it = threadIdx.x + q * 512;
+        if (it < total) w_load(cg * TL_COLS + ((it >> 6) % 3) * 32 + (it & 31), ((it >> 6) / 3) * 16 + ((it & 63) >> 5) * 8, wv[q]);
+    }
+    if (ksteps > WIDE_LDS_KS) {
+#pragma unroll
+        for (int ct = 0; ct < 3; ++ct) w_load(cg * TL_COLS + ct * 32 + l32, WIDE_LDS_KS * 16 + half * 8, wr[ct]);
+    }
+#pragma unroll
+    for (int q = 0; q < FILL_ITEMS; ++q) {
+        const int it = threadIdx.x + q * 512;
+        if (it < total) {
+            tl_u32x4 h, m, l;
+            w_split(wv[q], h, m, l);
+            tl_u32x4* dst = w_s + (it >> 6) * 3 * 64 + (it & 63);
+            dst[0] = h;
+            dst[64] = m;
+            dst[128] = l;
+        }
     }
     BPlanes breg;                                                        // planes of k step 17, this lane's operand slots
     if (ksteps > WIDE_LDS_KS) {
 #pragma unroll
         for (int ct = 0; ct < 3; ++ct) {
             tl_u32x4 h, m, l;
-            w_planes(cg * TL_COLS + ct * 32 + l32, WIDE_LDS_KS * 16 + half * 8, h, m, l);
+            w_split(wr[ct], h, m, l);
             breg.h[ct] = as_bf16x8(h);
             breg.m[ct] = as_bf16x8(m);
             breg.l[ct] = as_bf16x8(l);
