@@ -370,21 +370,23 @@ class _TallLinear(Function):
             grad_w, grad_b = _split_linear_weight_grad(grad_out, x, want_b)
         if ctx.needs_input_grad[0]:
             grad_x = _split_linear_input_grad(grad_out, weight)
+        # a forward that ran under autocast hands back a 16-bit gradient for fp32 x and W: the library
+        # products then run in the gradient's type, as autocast itself would run them
         with _rocblas_gemm():
             if ctx.needs_input_grad[0] and grad_x is None:
-                grad_x = grad_out @ weight
+                grad_x = (grad_out @ weight.to(grad_out.dtype)).to(x.dtype)
             if ctx.needs_input_grad[1] and grad_w is None:
-                grad_w = grad_out.t() @ x
+                grad_w = (grad_out.t() @ x.to(grad_out.dtype)).to(weight.dtype)
         if want_b and grad_b is None:
-            grad_b = _column_sum(grad_out)
+            grad_b = _column_sum(grad_out).to(weight.dtype)
         return grad_x, grad_w, grad_b
 
 
 def tall_linear(x, layer: nn.Linear):
     """Apply an ``nn.Linear`` to a tall 2-D input with the split-reduction weight gradient."""
-    if x.dim() == 2 and x.is_cuda:
+    if x.dim() == 2 and x.is_cuda and not torch.is_autocast_enabled(x.device.type):
         return _TallLinear.apply(x, layer.weight, layer.bias)
-    return layer(x)
+    return layer(x)                                  # CPU tensors, and autocast regions (the split kernels are fp32 only)
 
 
 class _BiasTableGather(Function):

@@ -36,3 +36,29 @@ def test_split_linear_helpers_decline_what_the_kernels_do_not_take():
     assert wa._split_linear_forward(x, w, None) is None
     assert wa._split_linear_input_grad(torch.randn(40, 288), w) is None
     assert wa._split_linear_weight_grad(torch.randn(40, 288), x, True) == (None, None)
+
+
+def test_tall_linear_function_under_autocast_backward_does_not_mix_dtypes():
+    """fp32 x and W, forward under autocast on a shape the split kernels do not take (48 -> 144, the
+    reference's shipped feature_size with enable_amp): the library fallback returns a 16-bit result, and
+    the backward, which runs outside autocast, must still multiply operands of one type."""
+    from sparseswin3d_amd.window_attention import _TallLinear
+    torch.manual_seed(2)
+    layer = torch.nn.Linear(48, 144)
+    x = torch.randn(33, 48, requires_grad=True)
+    with torch.autocast("cpu", dtype=torch.bfloat16):
+        y = _TallLinear.apply(x, layer.weight, layer.bias)
+    assert y.dtype == torch.bfloat16
+    y.float().sum().backward()
+    assert x.grad.dtype == torch.float32 and layer.weight.grad.dtype == torch.float32
+    ref_x = torch.ones(33, 144) @ layer.weight.detach()
+    assert torch.allclose(x.grad, ref_x, rtol=2e-2, atol=2e-2)
+    assert torch.allclose(layer.bias.grad, torch.full((144,), 33.0), rtol=1e-2)
+
+
+def test_tall_linear_leaves_autocast_regions_to_the_layer():
+    from sparseswin3d_amd.window_attention import tall_linear
+    layer = torch.nn.Linear(48, 144)
+    x = torch.randn(9, 48)
+    with torch.autocast("cpu", dtype=torch.bfloat16):
+        assert tall_linear(x, layer).dtype == torch.bfloat16
