@@ -58,6 +58,18 @@ size_t sswin_unique_consecutive_workspace_bytes(int64_t M);
 int sswin_unique_consecutive_indices(const void* keys, int key_dtype, int64_t M, int32_t* out,
                                      void* ws, size_t ws_bytes, void* stream);
 
+/* The same operator for callers that cannot allocate device memory (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc).  It has no counterpart in the reference:
+ * it is sswin_unique_consecutive_indices with the scan's tile sums kept in a 256 KiB device array
+ * built into the library (one copy per GPU, held until the process ends) instead of a caller
+ * workspace.  The caller still passes keys and out.  M may not exceed
+ * SSWIN_UNIQUE_CONSECUTIVE_STATIC_MAX keys (error otherwise).  Calls no hipMalloc / hipFree.
+ * All calls on one GPU share that array: calls that overlap on one GPU (two streams, two threads)
+ * race; nothing has to be cleared between calls.  Asynchronous. */
+#define SSWIN_UNIQUE_CONSECUTIVE_STATIC_MAX 134217728LL
+int sswin_unique_consecutive_indices_static(const void* keys, int key_dtype, int64_t M, int32_t* out,
+                                            void* stream);
+
 /* return_inverse (sparse_swin/ops.cu:718-730, ops.h:40): rank of x[i] among the distinct
  * values of x, and the number of distinct values.  maxnum = -1 means max(x)+1 (costs one
  * extra stream synchronisation).  Values of x must lie in [0, maxnum).

@@ -22,6 +22,7 @@ SIGNATURES = {
     "sswin_sort_indices": (_i32, [_vp, _i64, _vp, _vp, _sz, _vp]),
     "sswin_unique_consecutive_workspace_bytes": (_sz, [_i64]),
     "sswin_unique_consecutive_indices": (_i32, [_vp, _i32, _i64, _vp, _vp, _sz, _vp]),
+    "sswin_unique_consecutive_indices_static": (_i32, [_vp, _i32, _i64, _vp, _vp]),
     "sswin_return_inverse_workspace_bytes": (_sz, [_i64, _i64]),
     "sswin_return_inverse": (_i32, [_vp, _i64, _i64, _vp, _vp, _vp, _sz, _vp]),
     "sswin_qkv_sparse_indices_workspace_bytes": (_sz, [_i64, _i32, _i32]),
@@ -68,7 +69,7 @@ SIGNATURES = {
                                                _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i32, _vp]),
 }
 
-ABI_VERSION = 13
+ABI_VERSION = 14
 _lib = None
 
 

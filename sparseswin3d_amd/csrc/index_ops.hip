@@ -2,6 +2,7 @@
 // return_inverse, qkv_sparse_indices.  All of them are HBM-bound integer work; the kernels
 // are laid out for coalesced 64-lane accesses and use no floating point.
 #include <cstring>
+#include <mutex>
 #include <rocprim/device/device_radix_sort.hpp>
 #include <rocprim/iterator/counting_iterator.hpp>
 
@@ -333,7 +334,7 @@ using namespace sswin;
 extern "C" {
 
 const char* sswin_last_error(void) { return error_buffer(); }
-int sswin_abi_version(void) { return 13; }
+int sswin_abi_version(void) { return 14; }
 
 int sswin_flatten_indices(const int32_t* idx, int ndim, int64_t M, const int32_t* sizes, int32_t* out,
                           void* stream) {
@@ -392,16 +393,9 @@ size_t sswin_unique_consecutive_workspace_bytes(int64_t M) {
     return align_up((size_t)(scan_num_tiles(M > 0 ? M : 1)) * sizeof(int32_t), 256) + 256;
 }
 
-int sswin_unique_consecutive_indices(const void* keys, int key_dtype, int64_t M, int32_t* out, void* ws,
-                                     size_t ws_bytes, void* stream) {
-    SSWIN_CHECK(M >= 0, "unique_consecutive_indices: negative length");
-    if (M == 0) return 0;
-    SSWIN_CHECK(keys && out && ws, "unique_consecutive_indices: null pointer");
-    SSWIN_CHECK(ws_bytes >= sswin_unique_consecutive_workspace_bytes(M),
-                "unique_consecutive_indices: workspace too small");
-    Carver cv(ws, ws_bytes);
-    int32_t* tile_sums = cv.take<int32_t>((size_t)scan_num_tiles(M));
-    hipStream_t s = static_cast<hipStream_t>(stream);
+// tile_sums: device int32 [scan_num_tiles(M)]
+static int unique_consecutive_run(const void* keys, int key_dtype, int64_t M, int32_t* out, int32_t* tile_sums,
+                                  hipStream_t s) {
     switch (key_dtype) {
         case SSWIN_I32:
             if (((uintptr_t)keys % 16) == 0 && ((uintptr_t)out % 16) == 0)
@@ -413,6 +407,63 @@ int sswin_unique_consecutive_indices(const void* keys, int key_dtype, int64_t M,
         case SSWIN_U8: return unique_consecutive_t<uint8_t>(keys, M, out, tile_sums, s);
         default: return fail("unique_consecutive_indices: unsupported key dtype %d", key_dtype);
     }
+}
+
+int sswin_unique_consecutive_indices(const void* keys, int key_dtype, int64_t M, int32_t* out, void* ws,
+                                     size_t ws_bytes, void* stream) {
+    SSWIN_CHECK(M >= 0, "unique_consecutive_indices: negative length");
+    if (M == 0) return 0;
+    SSWIN_CHECK(keys && out && ws, "unique_consecutive_indices: null pointer");
+    SSWIN_CHECK(ws_bytes >= sswin_unique_consecutive_workspace_bytes(M),
+                "unique_consecutive_indices: workspace too small");
+    Carver cv(ws, ws_bytes);
+    int32_t* tile_sums = cv.take<int32_t>((size_t)scan_num_tiles(M));
+    return unique_consecutive_run(keys, key_dtype, M, out, tile_sums, static_cast<hipStream_t>(stream));
+}
+
+// ---- unique_consecutive_indices for callers that cannot allocate ---------------------------------
+// The tile sums of the scan live in a file-scope device array instead of a caller workspace.  In host
+// code the array's name is only a handle for hipGetSymbolAddress: the device address is looked up
+// once per device and that pointer is what the kernels receive.
+constexpr int64_t UC_STATIC_TILES = 65536;                                   // 256 KiB per device
+constexpr int64_t UC_STATIC_MAX_M = UC_STATIC_TILES * SCAN_TILE;             // 134 217 728 keys
+static __device__ __align__(256) int32_t uc_static_scratch[UC_STATIC_TILES];
+
+constexpr int UC_MAX_DEVICES = 64;
+static int32_t* uc_static_ptr[UC_MAX_DEVICES] = {nullptr};
+static std::mutex uc_static_mutex;
+
+// device address of this device's copy of the array (looked up on the first call per device)
+static int uc_static_address(int32_t** out) {
+    int dev = -1;
+    SSWIN_HIP(hipGetDevice(&dev));
+    SSWIN_CHECK(dev >= 0 && dev < UC_MAX_DEVICES, "unique_consecutive_indices_static: device %d out of range", dev);
+    std::lock_guard<std::mutex> lock(uc_static_mutex);
+    if (!uc_static_ptr[dev]) {
+        void* p = nullptr;
+        SSWIN_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(uc_static_scratch)));
+        SSWIN_CHECK(p, "unique_consecutive_indices_static: the scratch array has no device address");
+        uc_static_ptr[dev] = static_cast<int32_t*>(p);
+    }
+    *out = uc_static_ptr[dev];
+    return 0;
+}
+
+static_assert(UC_STATIC_MAX_M == SSWIN_UNIQUE_CONSECUTIVE_STATIC_MAX, "header and library disagree on the limit");
+
+int sswin_unique_consecutive_indices_static(const void* keys, int key_dtype, int64_t M, int32_t* out, void* stream) {
+    SSWIN_CHECK(M >= 0, "unique_consecutive_indices_static: negative length");
+    SSWIN_CHECK(M <= UC_STATIC_MAX_M,
+                "unique_consecutive_indices_static: %lld keys exceed the built-in scratch (%lld keys at most); "
+                "use sswin_unique_consecutive_indices with a workspace",
+                (long long)M, (long long)UC_STATIC_MAX_M);
+    if (M == 0) return 0;
+    SSWIN_CHECK(keys && out, "unique_consecutive_indices_static: null pointer");
+    int32_t* tile_sums = nullptr;
+    if (uc_static_address(&tile_sums)) return 1;
+    // every tile sum the scan reads is written by the reduce launch of the same call, so nothing
+    // has to be cleared between calls
+    return unique_consecutive_run(keys, key_dtype, M, out, tile_sums, static_cast<hipStream_t>(stream));
 }
 
 // ---- return_inverse ---------------------------------------------------------------------------
