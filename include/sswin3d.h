@@ -72,7 +72,8 @@ int sswin_unique_consecutive_indices_static(const void* keys, int key_dtype, int
 
 /* return_inverse (sparse_swin/ops.cu:718-730, ops.h:40): rank of x[i] among the distinct
  * values of x, and the number of distinct values.  maxnum = -1 means max(x)+1 (costs one
- * extra stream synchronisation).  Values of x must lie in [0, maxnum).
+ * extra stream synchronisation).  Values of x must lie in [0, maxnum): others set no bit, get
+ * rank -1, and are reported as an error when count_out is delivered.
  * x, out, ws: device.  count_out: host.  Synchronises `stream` to deliver count_out;
  * pass count_out = NULL to stay asynchronous (only possible with maxnum >= 0).
  * workspace query: pass the same maxnum you will pass to the call, or, for maxnum = -1,
@@ -87,11 +88,14 @@ int sswin_return_inverse(const int32_t* x, int64_t M, int64_t maxnum, int32_t* o
  * voxel order, and the permutations that sort their row-major hashes (shapes
  * {B,H,n,hd} and {B,H,hd,n}).  E = N*H*hd.  (window, pos) pairs must be distinct,
  * window in [0,B), pos in [0,n).  The ordering is that of the exact (non-wrapping) hash.
- * All array arguments: device.  Asynchronous. */
+ * Pairs outside that range, or a pair that occurs twice, never turn into a device address: the
+ * kernels that would use them leave sorted_qv / sorted_k unwritten.  validate != 0 waits for the
+ * stream and reports such input as an error; validate == 0 stays asynchronous and silent.
+ * All array arguments: device. */
 size_t sswin_qkv_sparse_indices_workspace_bytes(int64_t N, int B, int n);
 int sswin_qkv_sparse_indices(const int32_t* indices, int64_t N, int B, int n, int H, int hd,
                              int32_t* idx_qv, int32_t* sorted_qv, int32_t* idx_k,
-                             int32_t* sorted_k, void* ws, size_t ws_bytes, void* stream);
+                             int32_t* sorted_k, void* ws, size_t ws_bytes, int validate, void* stream);
 
 /* ---- per-group offsets ("plan") ----------------------------------------------------- */
 
@@ -184,11 +188,13 @@ int sswin_softmax_last_dim_backward(const int32_t* idx_row, const void* y, const
  *   descriptors inside a bucket is unspecified.
  * totals_out (host, 9 x int64): {groups G, non-empty windows, sum over groups of c*c, max c,
  *   groups in bucket 1..4, groups with c > 128 (no descriptor)}; the last five are 0 without tasks.
- * (window, pos) pairs must be distinct, window in [0,B), pos in [0,n).
+ * (window, pos) pairs must be distinct, window in [0,B), pos in [0,n): indices outside that range
+ * are skipped on the device (nothing is written through them) and reported as an error when the
+ * totals are decoded, and so are pairs that occur twice.
  * synchronize != 0: waits for `stream` and decodes the totals.  synchronize == 0: only enqueues
  * the work and a copy of the raw totals into totals_out (pinned host memory); once the caller
  * has waited for the stream, sswin_token_plan_totals(totals_out, H, g_cap) decodes them in place
- * and performs the capacity checks. */
+ * and performs the checks (range, distinctness, capacity). */
 size_t sswin_token_plan_workspace_bytes(int64_t N, int B, int n);
 int sswin_token_plan(const int32_t* indices, int64_t N, int B, int n, int H, int32_t* tokens,
                      int32_t* plan, int64_t g_cap, int32_t* tasks, int64_t* totals_out, void* ws,

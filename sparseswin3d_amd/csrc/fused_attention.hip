@@ -29,33 +29,60 @@ constexpr int FUSED_GROUPS_PER_WG = 4;
 // ------------------------------------------------------------------------------------------
 // token plan
 //
-// Five launches, no sort:
+// Five phases, no sort:
 //   1. clear the presence bitmap (W = ceil(n/32) words per window slot) and the counters
-//   2. one atomicOr per voxel
+//   2. one atomicOr per voxel (indices outside [0,B) x [0,n) are counted and skipped)
 //   3. per block of 256 window slots: sums of (tokens, tokens^2, non-empty windows)
 //   4. per block: prefix of the earlier blocks' sums, scan inside the block; every non-empty
 //      window learns the rank T of its first token, its rank k among the non-empty windows and
 //      the sum of c*c before it, and writes its H plan rows and task descriptors
 //   5. per voxel: rank = T(window) + number of occupied positions below its own
-// Reduce-then-scan (3, 4) instead of a chained scan: no block waits for another block.
+// Reduce-then-scan (3, 4) instead of a chained scan: no block waits for another block.  One launch
+// per phase.  (All five phases in one cooperative launch with grid-wide barriers in between were
+// measured: a barrier across the eight XCDs costs about 8 us, write-back and invalidation of the
+// per-XCD L2 included, against 3 to 5 us for a launch boundary.)
 // ------------------------------------------------------------------------------------------
 constexpr int TP_BLOCK = 256;
 
-__global__ __launch_bounds__(256) void tp_clear_kernel(uint32_t* __restrict__ p, int64_t n, int64_t* counters) {
-    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) p[i] = 0u;
-    if (blockIdx.x == 0 && threadIdx.x < 8) counters[threadIdx.x] = 0;
+// counters (int32) behind the two 64-bit totals: five buckets, c_max, indices out of range
+constexpr int TPC_CMAX = 5, TPC_RANGE = 6;
+
+struct TokenPlanArgs {
+    const int32_t* ind;      // [N, 2] (window, pos)
+    int64_t N;
+    int B, n, W, H;
+    uint32_t* bits;          // [B * W]
+    int32_t* win_T;          // [B]
+    int64_t* partial_a;      // [blocks]
+    int32_t* partial_b;      // [blocks]
+    int64_t* totals;         // [8]: windows, sum c | sum c*c << 32, then twelve int32 counters
+    int32_t* plan;
+    int64_t g_cap;
+    int4* tasks;
+    int32_t* tokens;         // [5 * N]
+    int blocks;              // ceil(B / 256)
+};
+
+__device__ __forceinline__ int32_t* tp_counters(const TokenPlanArgs& a) { return reinterpret_cast<int32_t*>(a.totals + 2); }
+
+// gtid / gthreads: this thread's index and the number of threads that share the phase
+__device__ __forceinline__ void tp_phase_clear(const TokenPlanArgs& a, int64_t gtid, int64_t gthreads) {
+    const int64_t words = (int64_t)a.B * a.W;
+    for (int64_t i = gtid; i < words; i += gthreads) a.bits[i] = 0u;
+    if (gtid < 8) a.totals[gtid] = 0;
 }
 
-__global__ __launch_bounds__(256) void tp_set_bits_kernel(const int32_t* __restrict__ ind, int64_t N, int W,
-                                                          uint32_t* __restrict__ bits) {
-    const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i < N) {
-        const int2 wp = *reinterpret_cast<const int2*>(ind + 2 * i);
-        atomicOr(&bits[(int64_t)wp.x * W + (wp.y >> 5)], 1u << (wp.y & 31));
+__device__ __forceinline__ void tp_phase_set_bits(const TokenPlanArgs& a, int64_t gtid, int64_t gthreads) {
+    for (int64_t i = gtid; i < a.N; i += gthreads) {
+        const int2 wp = *reinterpret_cast<const int2*>(a.ind + 2 * i);
+        if ((unsigned)wp.x < (unsigned)a.B && (unsigned)wp.y < (unsigned)a.n)
+            atomicOr(&a.bits[(int64_t)wp.x * a.W + (wp.y >> 5)], 1u << (wp.y & 31));
+        else
+            atomicAdd(&tp_counters(a)[TPC_RANGE], 1);
     }
 }
 
-__device__ __forceinline__ int tp_window_count(const uint32_t* __restrict__ bits, int64_t w, int W) {
+__device__ __forceinline__ int tp_window_count(const uint32_t* bits, int64_t w, int W) {
     int c = 0;
     if (W == 4) {
         const uint4 v = *reinterpret_cast<const uint4*>(bits + w * 4);
@@ -66,21 +93,24 @@ __device__ __forceinline__ int tp_window_count(const uint32_t* __restrict__ bits
     return c;
 }
 
+struct TpShared {
+    int64_t a[TP_BLOCK / 64];
+    int32_t b[TP_BLOCK / 64];
+    int64_t base_a;
+    int32_t base_b;
+};
+
 // block sums: partial_a[blk] = sum c | sum c*c << 32, partial_b[blk] = non-empty windows
-__global__ __launch_bounds__(TP_BLOCK) void tp_block_sums_kernel(const uint32_t* __restrict__ bits, int64_t B, int W,
-                                                                 int64_t* __restrict__ partial_a,
-                                                                 int32_t* __restrict__ partial_b) {
-    __shared__ int64_t lds_a[TP_BLOCK / 64];
-    __shared__ int32_t lds_b[TP_BLOCK / 64];
-    const int64_t w = (int64_t)blockIdx.x * TP_BLOCK + threadIdx.x;
-    const int64_t c = w < B ? tp_window_count(bits, w, W) : 0;
+__device__ __forceinline__ void tp_phase_block_sums(const TokenPlanArgs& a, int blk, TpShared& sh) {
+    const int64_t w = (int64_t)blk * TP_BLOCK + threadIdx.x;
+    const int64_t c = w < a.B ? tp_window_count(a.bits, w, a.W) : 0;
     int64_t ta;
     int32_t tb;
-    (void)block_exclusive_scan<int64_t, TP_BLOCK / 64>(c | ((c * c) << 32), lds_a, &ta);
-    (void)block_exclusive_scan<int32_t, TP_BLOCK / 64>(c > 0 ? 1 : 0, lds_b, &tb);
+    (void)block_exclusive_scan<int64_t, TP_BLOCK / 64>(c | ((c * c) << 32), sh.a, &ta);
+    (void)block_exclusive_scan<int32_t, TP_BLOCK / 64>(c > 0 ? 1 : 0, sh.b, &tb);
     if (threadIdx.x == 0) {
-        partial_a[blockIdx.x] = ta;
-        partial_b[blockIdx.x] = tb;
+        a.partial_a[blk] = ta;
+        a.partial_b[blk] = tb;
     }
 }
 
@@ -89,65 +119,58 @@ __global__ __launch_bounds__(TP_BLOCK) void tp_block_sums_kernel(const uint32_t*
 // window, sq_start}.  Slots inside a bucket are handed out with one atomic per wavefront and
 // bucket, so the order of the windows inside a bucket varies from run to run; consumers treat a
 // bucket as an unordered set.
-__global__ __launch_bounds__(TP_BLOCK) void tp_windows_kernel(const uint32_t* __restrict__ bits, int64_t B, int W,
-                                                              int H, const int64_t* __restrict__ partial_a,
-                                                              const int32_t* __restrict__ partial_b,
-                                                              int32_t* __restrict__ win_T, int32_t* __restrict__ plan,
-                                                              int64_t g_cap, int4* __restrict__ tasks,
-                                                              int64_t* __restrict__ totals,
-                                                              int32_t* __restrict__ counters) {
-    __shared__ int64_t lds_a[TP_BLOCK / 64];
-    __shared__ int32_t lds_b[TP_BLOCK / 64];
-    __shared__ int64_t base_a_s;
-    __shared__ int32_t base_b_s;
+__device__ __forceinline__ void tp_phase_windows(const TokenPlanArgs& a, int blk, TpShared& sh) {
+    const int H = a.H;
+    const int64_t g_cap = a.g_cap;
+    int32_t* counters = tp_counters(a);
     // this slot's bitmap words are requested first: the load overlaps the prefix below
-    const int64_t w = (int64_t)blockIdx.x * TP_BLOCK + threadIdx.x;
-    const int64_t c = w < B ? tp_window_count(bits, w, W) : 0;
+    const int64_t w = (int64_t)blk * TP_BLOCK + threadIdx.x;
+    const int64_t c = w < a.B ? tp_window_count(a.bits, w, a.W) : 0;
     // prefix of the earlier blocks
     int64_t pa = 0;
     int32_t pb = 0;
-    for (int64_t i = threadIdx.x; i < blockIdx.x; i += TP_BLOCK) {
-        pa += partial_a[i];
-        pb += partial_b[i];
+    for (int64_t i = threadIdx.x; i < blk; i += TP_BLOCK) {
+        pa += a.partial_a[i];
+        pb += a.partial_b[i];
     }
     int64_t ta;
     int32_t tb;
-    (void)block_exclusive_scan<int64_t, TP_BLOCK / 64>(pa, lds_a, &ta);
-    (void)block_exclusive_scan<int32_t, TP_BLOCK / 64>(pb, lds_b, &tb);
+    (void)block_exclusive_scan<int64_t, TP_BLOCK / 64>(pa, sh.a, &ta);
+    (void)block_exclusive_scan<int32_t, TP_BLOCK / 64>(pb, sh.b, &tb);
     if (threadIdx.x == 0) {
-        base_a_s = ta;
-        base_b_s = tb;
+        sh.base_a = ta;
+        sh.base_b = tb;
     }
     __syncthreads();
-    const int64_t base_a = base_a_s;
-    const int32_t base_b = base_b_s;
+    const int64_t base_a = sh.base_a;
+    const int32_t base_b = sh.base_b;
 
-    const int64_t ea = block_exclusive_scan<int64_t, TP_BLOCK / 64>(c | ((c * c) << 32), lds_a, &ta) + base_a;
-    const int32_t k = block_exclusive_scan<int32_t, TP_BLOCK / 64>(c > 0 ? 1 : 0, lds_b, &tb) + base_b;
-    if (blockIdx.x == gridDim.x - 1 && threadIdx.x == 0) {
-        totals[0] = (int64_t)(base_b + tb);                     // non-empty windows
-        totals[1] = base_a + ta;                                // sum c | sum c*c << 32
+    const int64_t ea = block_exclusive_scan<int64_t, TP_BLOCK / 64>(c | ((c * c) << 32), sh.a, &ta) + base_a;
+    const int32_t k = block_exclusive_scan<int32_t, TP_BLOCK / 64>(c > 0 ? 1 : 0, sh.b, &tb) + base_b;
+    if (blk == a.blocks - 1 && threadIdx.x == 0) {
+        a.totals[0] = (int64_t)(base_b + tb);                   // non-empty windows
+        a.totals[1] = base_a + ta;                              // sum c | sum c*c << 32
     }
     const int32_t T = (int32_t)(ea & 0xffffffffll);
     const int64_t q2 = ea >> 32;
-    if (w < B) win_T[w] = T;
+    if (w < a.B) a.win_T[w] = T;
 
     const int lane = threadIdx.x & 63;
     const bool live = c > 0 && ((int64_t)k + 1) * H <= g_cap;
     if (live) {
         for (int h = 0; h < H; ++h) {
             const int64_t g = (int64_t)k * H + h;
-            plan[g] = (int32_t)c;
-            plan[g_cap + g] = T;
-            plan[2 * g_cap + g] = (int32_t)(q2 * H + (int64_t)h * c * c);
-            plan[3 * g_cap + g] = (int32_t)w;
-            plan[4 * g_cap + g] = h;
+            a.plan[g] = (int32_t)c;
+            a.plan[g_cap + g] = T;
+            a.plan[2 * g_cap + g] = (int32_t)(q2 * H + (int64_t)h * c * c);
+            a.plan[3 * g_cap + g] = (int32_t)w;
+            a.plan[4 * g_cap + g] = h;
         }
     }
     // wave maximum of c, one atomic per wavefront
     const int cm = wave_max_i32((int)c);
-    if (lane == 0 && cm > 0) atomicMax(&counters[5], cm);
-    if (tasks == nullptr) return;
+    if (lane == 0 && cm > 0) atomicMax(&counters[TPC_CMAX], cm);
+    if (a.tasks == nullptr) return;
     const int b = live ? min(((int)c - 1) >> 5, 4) : -1;
     // lanes 0..4 reserve the slots of the five buckets with one atomic each, at the same time
     int slot = 0;
@@ -166,48 +189,72 @@ __global__ __launch_bounds__(TP_BLOCK) void tp_windows_kernel(const uint32_t* __
     }
     if (live && b < 4) {
         for (int h = 0; h < H; ++h)
-            tasks[(int64_t)b * g_cap + slot + h] =
+            a.tasks[(int64_t)b * g_cap + slot + h] =
                 make_int4(T, (int)c | (h << 8), (int)w, (int32_t)(q2 * H + (int64_t)h * c * c));
     }
 }
 
 // per voxel -> entries by token rank: source voxel, first rank and size of its window, pos, window
-__global__ __launch_bounds__(256) void tp_rank_kernel(const int32_t* __restrict__ ind, int64_t N, int W,
-                                                      const uint32_t* __restrict__ bits,
-                                                      const int32_t* __restrict__ win_T,
-                                                      int32_t* __restrict__ order, int32_t* __restrict__ tok_T,
-                                                      int32_t* __restrict__ tok_c, int32_t* __restrict__ tok_pos,
-                                                      int32_t* __restrict__ tok_win) {
-    const int64_t v = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (v >= N) return;
-    const int2 wp = *reinterpret_cast<const int2*>(ind + 2 * v);
-    const int T = win_T[wp.x];
-    const int word = wp.y >> 5;
-    const uint32_t below_mask = (1u << (wp.y & 31)) - 1u;
-    int below = 0, c = 0;
-    if (W == 4) {
-        const uint4 q = *reinterpret_cast<const uint4*>(bits + (int64_t)wp.x * 4);
-        const uint32_t b[4] = {q.x, q.y, q.z, q.w};
+__device__ __forceinline__ void tp_phase_rank(const TokenPlanArgs& a, int64_t gtid, int64_t gthreads) {
+    const int W = a.W;
+    const int64_t N = a.N;
+    int32_t* order = a.tokens;
+    int32_t* tok_T = a.tokens + N;
+    int32_t* tok_c = a.tokens + 2 * N;
+    int32_t* tok_pos = a.tokens + 3 * N;
+    int32_t* tok_win = a.tokens + 4 * N;
+    for (int64_t v = gtid; v < N; v += gthreads) {
+        const int2 wp = *reinterpret_cast<const int2*>(a.ind + 2 * v);
+        if ((unsigned)wp.x >= (unsigned)a.B || (unsigned)wp.y >= (unsigned)a.n) continue;   // counted in phase 2
+        const int T = a.win_T[wp.x];
+        const int word = wp.y >> 5;
+        const uint32_t below_mask = (1u << (wp.y & 31)) - 1u;
+        int below = 0, c = 0;
+        if (W == 4) {
+            const uint4 q = *reinterpret_cast<const uint4*>(a.bits + (int64_t)wp.x * 4);
+            const uint32_t b[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            const int pc = __popc(b[k]);
-            c += pc;
-            below += k < word ? pc : (k == word ? __popc(b[k] & below_mask) : 0);
+            for (int k = 0; k < 4; ++k) {
+                const int pc = __popc(b[k]);
+                c += pc;
+                below += k < word ? pc : (k == word ? __popc(b[k] & below_mask) : 0);
+            }
+        } else {
+            for (int k = 0; k < W; ++k) {
+                const uint32_t x = a.bits[(int64_t)wp.x * W + k];
+                const int pc = __popc(x);
+                c += pc;
+                below += k < word ? pc : (k == word ? __popc(x & below_mask) : 0);
+            }
         }
-    } else {
-        for (int k = 0; k < W; ++k) {
-            const uint32_t x = bits[(int64_t)wp.x * W + k];
-            const int pc = __popc(x);
-            c += pc;
-            below += k < word ? pc : (k == word ? __popc(x & below_mask) : 0);
+        const int r = T + below;
+        if (r < N) {                                            // duplicates cannot push a rank past the end, but stay inside anyway
+            order[r] = (int32_t)v;
+            tok_T[r] = T;
+            tok_c[r] = c;
+            tok_pos[r] = wp.y;
+            tok_win[r] = wp.x;
         }
     }
-    const int r = T + below;
-    order[r] = (int32_t)v;
-    tok_T[r] = T;
-    tok_c[r] = c;
-    tok_pos[r] = wp.y;
-    tok_win[r] = wp.x;
+}
+
+// ---- the five launches ----
+__global__ __launch_bounds__(256) void tp_clear_kernel(TokenPlanArgs a) {
+    tp_phase_clear(a, (int64_t)blockIdx.x * 256 + threadIdx.x, (int64_t)gridDim.x * 256);
+}
+__global__ __launch_bounds__(256) void tp_set_bits_kernel(TokenPlanArgs a) {
+    tp_phase_set_bits(a, (int64_t)blockIdx.x * 256 + threadIdx.x, (int64_t)gridDim.x * 256);
+}
+__global__ __launch_bounds__(TP_BLOCK) void tp_block_sums_kernel(TokenPlanArgs a) {
+    __shared__ TpShared sh;
+    tp_phase_block_sums(a, blockIdx.x, sh);
+}
+__global__ __launch_bounds__(TP_BLOCK) void tp_windows_kernel(TokenPlanArgs a) {
+    __shared__ TpShared sh;
+    tp_phase_windows(a, blockIdx.x, sh);
+}
+__global__ __launch_bounds__(256) void tp_rank_kernel(TokenPlanArgs a) {
+    tp_phase_rank(a, (int64_t)blockIdx.x * 256 + threadIdx.x, (int64_t)gridDim.x * 256);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -766,35 +813,40 @@ int sswin_token_plan(const int32_t* indices, int64_t N, int B, int n, int H, int
     SSWIN_CHECK(ws_bytes >= sswin_token_plan_workspace_bytes(N, B, n), "token_plan: workspace too small");
     hipStream_t s = static_cast<hipStream_t>(stream);
     Carver cv(ws, ws_bytes);
-    const int W = tp_words_per_window(n);
-    const size_t words = (size_t)B * W;
+    TokenPlanArgs a;
+    a.ind = indices;
+    a.N = N;
+    a.B = B;
+    a.n = n;
+    a.W = tp_words_per_window(n);
+    a.H = H;
+    const size_t words = (size_t)B * a.W;
     const int64_t blocks = tp_blocks(B);
-    int64_t* totals_dev = cv.take<int64_t>(8);       // [0] windows, [1] sum c | sum c*c << 32, [2..7] counters
-    uint32_t* bits = cv.take<uint32_t>(words);
-    int32_t* win_T = cv.take<int32_t>((size_t)B);
-    int64_t* partial_a = cv.take<int64_t>((size_t)blocks);
-    int32_t* partial_b = cv.take<int32_t>((size_t)blocks);
+    a.blocks = (int)blocks;
+    a.totals = cv.take<int64_t>(8);       // [0] windows, [1] sum c | sum c*c << 32, [2..7] counters
+    a.bits = cv.take<uint32_t>(words);
+    a.win_T = cv.take<int32_t>((size_t)B);
+    a.partial_a = cv.take<int64_t>((size_t)blocks);
+    a.partial_b = cv.take<int32_t>((size_t)blocks);
     SSWIN_CHECK(cv.ok(), "token_plan: workspace too small");
-    int32_t* counters = reinterpret_cast<int32_t*>(totals_dev + 2);   // five buckets, c_max
-    int32_t* order = tokens;
-    int32_t* tok_T = tokens + N;
-    int32_t* tok_c = tokens + 2 * N;
-    int32_t* tok_pos = tokens + 3 * N;
-    int32_t* tok_win = tokens + 4 * N;
+    a.plan = plan;
+    a.g_cap = g_cap;
+    a.tasks = reinterpret_cast<int4*>(tasks);
+    a.tokens = tokens;
+    totals_out[8] = N;                     // read back by sswin_token_plan_totals (the copy below fills [0..7])
 
-    const unsigned clear_blocks = (unsigned)std::min<size_t>((words + 255) / 256, 2048);
-    hipLaunchKernelGGL(tp_clear_kernel, dim3(clear_blocks), dim3(256), 0, s, bits, (int64_t)words, totals_dev);
-    const unsigned nb = (unsigned)((N + 255) / 256);
-    hipLaunchKernelGGL(tp_set_bits_kernel, dim3(nb), dim3(256), 0, s, indices, N, W, bits);
-    hipLaunchKernelGGL(tp_block_sums_kernel, dim3((unsigned)blocks), dim3(TP_BLOCK), 0, s, bits, (int64_t)B, W,
-                       partial_a, partial_b);
-    hipLaunchKernelGGL(tp_windows_kernel, dim3((unsigned)blocks), dim3(TP_BLOCK), 0, s, bits, (int64_t)B, W, H,
-                       partial_a, partial_b, win_T, plan, g_cap, reinterpret_cast<int4*>(tasks), totals_dev, counters);
-    hipLaunchKernelGGL(tp_rank_kernel, dim3(nb), dim3(256), 0, s, indices, N, W, bits, win_T, order, tok_T, tok_c,
-                       tok_pos, tok_win);
+    {
+        const unsigned clear_blocks = (unsigned)std::min<size_t>((words + 255) / 256, 2048);
+        hipLaunchKernelGGL(tp_clear_kernel, dim3(clear_blocks), dim3(256), 0, s, a);
+        const unsigned nb = (unsigned)std::min<int64_t>((N + 255) / 256, 1 << 20);
+        hipLaunchKernelGGL(tp_set_bits_kernel, dim3(nb), dim3(256), 0, s, a);
+        hipLaunchKernelGGL(tp_block_sums_kernel, dim3((unsigned)blocks), dim3(TP_BLOCK), 0, s, a);
+        hipLaunchKernelGGL(tp_windows_kernel, dim3((unsigned)blocks), dim3(TP_BLOCK), 0, s, a);
+        hipLaunchKernelGGL(tp_rank_kernel, dim3(nb), dim3(256), 0, s, a);
+    }
     if (launch_ok("token plan")) return 1;
     // raw totals: the caller decodes them with sswin_token_plan_totals once the copy has landed
-    SSWIN_HIP(hipMemcpyAsync(totals_out, totals_dev, 8 * sizeof(int64_t), hipMemcpyDeviceToHost, s));
+    SSWIN_HIP(hipMemcpyAsync(totals_out, a.totals, 8 * sizeof(int64_t), hipMemcpyDeviceToHost, s));
     if (!synchronize) return 0;
     SSWIN_HIP(hipStreamSynchronize(s));
     return sswin_token_plan_totals(totals_out, H, g_cap);
@@ -802,12 +854,18 @@ int sswin_token_plan(const int32_t* indices, int64_t N, int B, int n, int H, int
 
 int sswin_token_plan_totals(int64_t* totals, int H, int64_t g_cap) {
     SSWIN_CHECK(totals && H > 0, "token_plan_totals: bad arguments");
-    int64_t raw[8];
+    int64_t raw[9];
     memcpy(raw, totals, sizeof(raw));
     int32_t counters[12];
     memcpy(counters, raw + 2, sizeof(counters));
     const int64_t windows = raw[0];
     const int64_t s2 = raw[1] >> 32;
+    const int64_t distinct = raw[1] & 0xffffffffll;
+    const int64_t N = raw[8];
+    SSWIN_CHECK(counters[TPC_RANGE] == 0,
+                "token_plan: %d voxel indices lie outside [0, batch_size) x [0, positions per window)", counters[TPC_RANGE]);
+    SSWIN_CHECK(distinct == N, "token_plan: (window, pos) pairs must be distinct: %lld voxels share a pair with another",
+                (long long)(N - distinct));
     SSWIN_CHECK(raw[1] >= 0 && s2 * H < (int64_t)INT32_MAX,
                 "token_plan: the attention matrix has 2^31 or more non-zeros, which int32 offsets cannot address");
     SSWIN_CHECK(windows * H <= g_cap, "token_plan: %lld groups exceed the plan capacity %lld",
@@ -815,7 +873,7 @@ int sswin_token_plan_totals(int64_t* totals, int H, int64_t g_cap) {
     totals[0] = windows * H;
     totals[1] = windows;
     totals[2] = s2 * H;
-    totals[3] = counters[5];
+    totals[3] = counters[TPC_CMAX];
     for (int b = 0; b < 5; ++b) totals[4 + b] = counters[b];
     return 0;
 }

@@ -181,23 +181,32 @@ __global__ __launch_bounds__(256) void fill_u32_kernel(uint32_t* __restrict__ p,
     for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) p[i] = v;
 }
 
-__global__ __launch_bounds__(256) void set_bits_kernel(const int32_t* __restrict__ x, int64_t M,
-                                                       uint32_t* __restrict__ bits) {
+// Values outside [0, limit) set no bit (the bitmap has `limit` bits): they are counted in *bad instead.
+__global__ __launch_bounds__(256) void set_bits_kernel(const int32_t* __restrict__ x, int64_t M, int64_t limit,
+                                                       uint32_t* __restrict__ bits, int32_t* __restrict__ bad) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i < M) {
         const uint32_t v = (uint32_t)x[i];
-        atomicOr(&bits[v >> 5], 1u << (v & 31));
+        if ((int64_t)v < limit)
+            atomicOr(&bits[v >> 5], 1u << (v & 31));
+        else
+            atomicAdd(bad, 1);
     }
 }
 
-// (window, pos) pairs -> bit window*n + pos
-__global__ __launch_bounds__(256) void set_bits_pairs_kernel(const int32_t* __restrict__ ind, int64_t N,
-                                                             int n, uint32_t* __restrict__ bits) {
+// (window, pos) pairs -> bit window*n + pos; pairs outside [0,B) x [0,n) set no bit and are counted in *bad
+__global__ __launch_bounds__(256) void set_bits_pairs_kernel(const int32_t* __restrict__ ind, int64_t N, int B,
+                                                             int n, uint32_t* __restrict__ bits,
+                                                             int32_t* __restrict__ bad) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (i < N) {
         const int2 wp = *reinterpret_cast<const int2*>(ind + 2 * i);
-        const uint64_t v = (uint64_t)(uint32_t)wp.x * (uint32_t)n + (uint32_t)wp.y;
-        atomicOr(&bits[v >> 5], 1u << (v & 31));
+        if ((unsigned)wp.x < (unsigned)B && (unsigned)wp.y < (unsigned)n) {
+            const uint64_t v = (uint64_t)(uint32_t)wp.x * (uint32_t)n + (uint32_t)wp.y;
+            atomicOr(&bits[v >> 5], 1u << (v & 31));
+        } else {
+            atomicAdd(bad, 1);
+        }
     }
 }
 
@@ -217,12 +226,15 @@ __device__ __forceinline__ int rank_of_bit(const uint32_t* __restrict__ bits,
     return word_prefix[w] + __popc(below);
 }
 
-__global__ __launch_bounds__(256) void rank_lookup_kernel(const int32_t* __restrict__ x, int64_t M,
+__global__ __launch_bounds__(256) void rank_lookup_kernel(const int32_t* __restrict__ x, int64_t M, int64_t limit,
                                                           const uint32_t* __restrict__ bits,
                                                           const int32_t* __restrict__ word_prefix,
                                                           int32_t* __restrict__ out) {
     const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (i < M) out[i] = rank_of_bit(bits, word_prefix, (uint32_t)x[i]);
+    if (i < M) {
+        const uint32_t v = (uint32_t)x[i];
+        out[i] = (int64_t)v < limit ? rank_of_bit(bits, word_prefix, v) : -1;    // out of range: counted by set_bits_kernel
+    }
 }
 
 // max of int32 array into a single device int (one atomicMax per block)
@@ -243,15 +255,24 @@ __global__ __launch_bounds__(256) void max_i32_kernel(const int32_t* __restrict_
 // ------------------------------------------------------------------------------------------
 // Per voxel: rank r in (window, pos) order, and for rank r the source voxel, the rank T of the
 // first token of its window and the token count c of its window.
-__global__ __launch_bounds__(256) void voxel_rank_kernel(const int32_t* __restrict__ ind, int64_t N, int n,
+// status: [0] pairs out of range, [1] distinct pairs (total of the bitmap scan).  The expansion kernels
+// below run only if status[0] == 0 and status[1] == N: otherwise ranks would repeat or be missing and
+// the destination slots computed from them would be arbitrary.
+__device__ __forceinline__ bool pairs_valid(const int32_t* __restrict__ status, int64_t N) {
+    return status[0] == 0 && (int64_t)status[1] == N;
+}
+
+__global__ __launch_bounds__(256) void voxel_rank_kernel(const int32_t* __restrict__ ind, int64_t N, int B, int n,
                                                          const uint32_t* __restrict__ bits,
                                                          const int32_t* __restrict__ word_prefix,
+                                                         const int32_t* __restrict__ status,
                                                          int32_t* __restrict__ order,   // [N] voxel of rank r
                                                          int32_t* __restrict__ win_T,   // [N] by rank
                                                          int32_t* __restrict__ win_c) { // [N] by rank
     const int64_t v = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (v >= N) return;
+    if (v >= N || !pairs_valid(status, N)) return;
     const int2 wp = *reinterpret_cast<const int2*>(ind + 2 * v);
+    (void)B;
     const uint64_t first = (uint64_t)(uint32_t)wp.x * (uint32_t)n;
     const int r = rank_of_bit(bits, word_prefix, first + (uint32_t)wp.y);
     const int T = rank_of_bit(bits, word_prefix, first);
@@ -291,12 +312,13 @@ __global__ __launch_bounds__(256) void expand_coo_kernel(const int32_t* __restri
 // One thread per (rank, head, channel quad): a 16-byte store, 128 contiguous bytes per hd=32 row.
 __global__ __launch_bounds__(256) void sorted_qv_kernel(const int32_t* __restrict__ order,
                                                         const int32_t* __restrict__ win_T,
-                                                        const int32_t* __restrict__ win_c, int64_t N,
+                                                        const int32_t* __restrict__ win_c,
+                                                        const int32_t* __restrict__ status, int64_t N,
                                                         int H, int hd, int32_t* __restrict__ sorted_qv) {
     const int q = hd >> 2;                                  // channel quads per head
     const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
     const int64_t total = N * H * q;
-    if (t >= total) return;
+    if (t >= total || !pairs_valid(status, N)) return;
     const int cq = (int)(t % q);
     const int64_t rh = t / q;
     const int h = (int)(rh % H);
@@ -312,10 +334,11 @@ __global__ __launch_bounds__(256) void sorted_qv_kernel(const int32_t* __restric
 // for a fixed (head, channel) a wave writes runs of c contiguous ints per window.
 __global__ __launch_bounds__(256) void sorted_k_kernel(const int32_t* __restrict__ order,
                                                        const int32_t* __restrict__ win_T,
-                                                       const int32_t* __restrict__ win_c, int64_t N,
+                                                       const int32_t* __restrict__ win_c,
+                                                       const int32_t* __restrict__ status, int64_t N,
                                                        int H, int hd, int32_t* __restrict__ sorted_k) {
     const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (r >= N) return;
+    if (r >= N || !pairs_valid(status, N)) return;
     const int T = win_T[r], c = win_c[r];
     const int i = (int)(r - T);
     const int h = blockIdx.y;
@@ -334,7 +357,7 @@ using namespace sswin;
 extern "C" {
 
 const char* sswin_last_error(void) { return error_buffer(); }
-int sswin_abi_version(void) { return 14; }
+int sswin_abi_version(void) { return 15; }
 
 int sswin_flatten_indices(const int32_t* idx, int ndim, int64_t M, const int32_t* sizes, int32_t* out,
                           void* stream) {
@@ -488,7 +511,7 @@ int sswin_return_inverse(const int32_t* x, int64_t M, int64_t maxnum, int32_t* o
     SSWIN_CHECK(maxnum != -1 || count_out, "return_inverse: maxnum = -1 needs count_out (synchronous call)");
     hipStream_t s = static_cast<hipStream_t>(stream);
     Carver cv(ws, ws_bytes);
-    int32_t* total_dev = cv.take<int32_t>(2);   // [0] distinct count, [1] max
+    int32_t* total_dev = cv.take<int32_t>(3);   // [0] distinct count, [1] max, [2] values outside [0, maxnum)
     SSWIN_CHECK(cv.ok(), "return_inverse: workspace too small");
     if (maxnum == -1) {
         int32_t* max_dev = total_dev + 1;
@@ -509,18 +532,21 @@ int sswin_return_inverse(const int32_t* x, int64_t M, int64_t maxnum, int32_t* o
     SSWIN_CHECK(cv.ok(), "return_inverse: workspace too small for maxnum %lld", (long long)maxnum);
     const unsigned fill_blocks = (unsigned)std::min<size_t>((words + 255) / 256, 4096);
     hipLaunchKernelGGL(fill_u32_kernel, dim3(fill_blocks), dim3(256), 0, s, bits, (int64_t)words, 0u);
-    hipLaunchKernelGGL(set_bits_kernel, dim3((unsigned)((M + 255) / 256)), dim3(256), 0, s, x, M, bits);
+    hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(256), 0, s, reinterpret_cast<uint32_t*>(total_dev + 2), (int64_t)1, 0u);
+    hipLaunchKernelGGL(set_bits_kernel, dim3((unsigned)((M + 255) / 256)), dim3(256), 0, s, x, M, maxnum, bits,
+                       total_dev + 2);
     PopcLoad ld{bits};
     ExclusiveStore st{word_prefix};
     if (device_exclusive_scan<int32_t>(ld, st, (int64_t)words, tile_sums, total_dev, s, "return_inverse scan")) return 1;
-    hipLaunchKernelGGL(rank_lookup_kernel, dim3((unsigned)((M + 255) / 256)), dim3(256), 0, s, x, M, bits,
+    hipLaunchKernelGGL(rank_lookup_kernel, dim3((unsigned)((M + 255) / 256)), dim3(256), 0, s, x, M, maxnum, bits,
                        word_prefix, out);
     if (launch_ok("return_inverse")) return 1;
     if (count_out) {
-        int32_t cnt = 0;
-        SSWIN_HIP(hipMemcpyAsync(&cnt, total_dev, sizeof(int32_t), hipMemcpyDeviceToHost, s));
+        int32_t back[3] = {0, 0, 0};
+        SSWIN_HIP(hipMemcpyAsync(back, total_dev, sizeof(back), hipMemcpyDeviceToHost, s));
         SSWIN_HIP(hipStreamSynchronize(s));
-        *count_out = cnt;
+        SSWIN_CHECK(back[2] == 0, "return_inverse: %d values lie outside [0, %lld)", back[2], (long long)maxnum);
+        *count_out = back[0];
     }
     return 0;
 }
@@ -529,12 +555,12 @@ int sswin_return_inverse(const int32_t* x, int64_t M, int64_t maxnum, int32_t* o
 size_t sswin_qkv_sparse_indices_workspace_bytes(int64_t N, int B, int n) {
     const size_t words = bitmap_words((int64_t)B * n + n);
     return align_up(words * 4, 256) * 2 + align_up((size_t)scan_num_tiles((int64_t)words) * 4, 256) +
-           3 * align_up((size_t)(N > 0 ? N : 1) * 4, 256) + 1024;
+           3 * align_up((size_t)(N > 0 ? N : 1) * 4, 256) + 256 + 1024;
 }
 
 int sswin_qkv_sparse_indices(const int32_t* indices, int64_t N, int B, int n, int H, int hd,
                              int32_t* idx_qv, int32_t* sorted_qv, int32_t* idx_k, int32_t* sorted_k,
-                             void* ws, size_t ws_bytes, void* stream) {
+                             void* ws, size_t ws_bytes, int validate, void* stream) {
     SSWIN_CHECK(N >= 0 && B > 0 && n > 0 && H > 0 && hd > 0, "qkv_sparse_indices: bad sizes");
     SSWIN_CHECK(hd % 4 == 0, "qkv_sparse_indices: head dim %d must be a multiple of 4", hd);
     const int64_t E = N * H * hd;
@@ -553,25 +579,36 @@ int sswin_qkv_sparse_indices(const int32_t* indices, int64_t N, int B, int n, in
     int32_t* order = cv.take<int32_t>((size_t)N);
     int32_t* win_T = cv.take<int32_t>((size_t)N);
     int32_t* win_c = cv.take<int32_t>((size_t)N);
+    int32_t* status = cv.take<int32_t>(2);        // [0] pairs out of range, [1] distinct pairs
     SSWIN_CHECK(cv.ok(), "qkv_sparse_indices: workspace too small");
 
     const unsigned fill_blocks = (unsigned)std::min<size_t>((words + 255) / 256, 4096);
     hipLaunchKernelGGL(fill_u32_kernel, dim3(fill_blocks), dim3(256), 0, s, bits, (int64_t)words, 0u);
+    hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(256), 0, s, reinterpret_cast<uint32_t*>(status), (int64_t)2, 0u);
     const unsigned nb = (unsigned)((N + 255) / 256);
-    hipLaunchKernelGGL(set_bits_pairs_kernel, dim3(nb), dim3(256), 0, s, indices, N, n, bits);
+    hipLaunchKernelGGL(set_bits_pairs_kernel, dim3(nb), dim3(256), 0, s, indices, N, B, n, bits, status);
     PopcLoad ld{bits};
     ExclusiveStore st{word_prefix};
-    if (device_exclusive_scan<int32_t>(ld, st, (int64_t)words, tile_sums, (int32_t*)nullptr, s, "qkv_sparse_indices scan")) return 1;
-    hipLaunchKernelGGL(voxel_rank_kernel, dim3(nb), dim3(256), 0, s, indices, N, n, bits, word_prefix, order,
+    if (device_exclusive_scan<int32_t>(ld, st, (int64_t)words, tile_sums, status + 1, s, "qkv_sparse_indices scan")) return 1;
+    hipLaunchKernelGGL(voxel_rank_kernel, dim3(nb), dim3(256), 0, s, indices, N, B, n, bits, word_prefix, status, order,
                        win_T, win_c);
     hipLaunchKernelGGL(expand_coo_kernel, dim3((unsigned)((E / 4 + 255) / 256)), dim3(256), 0, s, indices, E, H,
                        hd, idx_qv, idx_k);
     const int64_t qv_threads = N * H * (hd / 4);
     hipLaunchKernelGGL(sorted_qv_kernel, dim3((unsigned)((qv_threads + 255) / 256)), dim3(256), 0, s, order,
-                       win_T, win_c, N, H, hd, sorted_qv);
-    hipLaunchKernelGGL(sorted_k_kernel, dim3(nb, (unsigned)H), dim3(256), 0, s, order, win_T, win_c, N, H, hd,
+                       win_T, win_c, status, N, H, hd, sorted_qv);
+    hipLaunchKernelGGL(sorted_k_kernel, dim3(nb, (unsigned)H), dim3(256), 0, s, order, win_T, win_c, status, N, H, hd,
                        sorted_k);
-    return launch_ok("qkv_sparse_indices");
+    if (launch_ok("qkv_sparse_indices")) return 1;
+    if (validate) {
+        int32_t back[2] = {0, 0};
+        SSWIN_HIP(hipMemcpyAsync(back, status, sizeof(back), hipMemcpyDeviceToHost, s));
+        SSWIN_HIP(hipStreamSynchronize(s));
+        SSWIN_CHECK(back[0] == 0, "qkv_sparse_indices: %d voxel indices lie outside [0, batch_size) x [0, spatial_dim)", back[0]);
+        SSWIN_CHECK(back[1] == N, "qkv_sparse_indices: (window, pos) pairs must be distinct: %lld voxels share a pair with another",
+                    (long long)(N - back[1]));
+    }
+    return 0;
 }
 
 }  // extern "C"

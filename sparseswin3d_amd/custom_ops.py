@@ -152,7 +152,7 @@ def qkv_sparse_indices(indices, batch_size, spatial_dim, num_heads, c):
     with torch.cuda.device(d):
         _lib.check(lib.sswin_qkv_sparse_indices(_ptr(indices), n_vox, int(batch_size), int(spatial_dim),
                                                 int(num_heads), int(c), _ptr(idx_qv), _ptr(sorted_qv),
-                                                _ptr(idx_k), _ptr(sorted_k), _ptr(ws), nbytes, _stream(d)))
+                                                _ptr(idx_k), _ptr(sorted_k), _ptr(ws), nbytes, 1, _stream(d)))
     return idx_qv, sorted_qv, idx_k, sorted_k
 
 

@@ -52,7 +52,8 @@ class TokenPlan:
 
     With ``defer=True`` the constructor only enqueues the kernels and the copy of the totals;
     work enqueued afterwards (the qkv projection) overlaps the host round trip, and
-    :meth:`finish` waits for the totals when they are needed."""
+    :meth:`finish` waits for the totals when they are needed.  :meth:`finish` raises if an index
+    lies outside ``[0, batch_size) x [0, n)`` or a (window, pos) pair occurs twice."""
 
     def __init__(self, indices: torch.Tensor, batch_size: int, n: int, num_heads: int, defer: bool = False,
                  tasks: bool = True):

@@ -42,11 +42,27 @@ def test_token_plan_closed_forms(case):
     else:
         B, n, H = 20000, 125, 3
         ind = random_window_indices(rng, B, n, 120000)
-    tp = TokenPlan(torch.from_numpy(ind).cuda(), B, n, H)
     tokens, plan, A, c_max = _closed_form_plan(ind, n, H)
+    tp = TokenPlan(torch.from_numpy(ind).cuda(), B, n, H)
     assert (tp.G, tp.A, tp.c_max) == (plan.shape[1], A, c_max)
     np.testing.assert_array_equal(tp.tokens.view(5, -1).cpu().numpy(), tokens)
     np.testing.assert_array_equal(tp.plan.view(5, -1)[:, :tp.G].cpu().numpy(), plan)
+
+
+def test_token_plan_rejects_bad_indices():
+    """Indices outside [0,B) x [0,n) and repeated (window, pos) pairs are skipped on the device (every kernel
+    exits normally, nothing is written through them) and reported when the totals are decoded."""
+    from sparseswin3d_amd.fused import TokenPlan
+    rng = np.random.default_rng(5)
+    B, n, H = 40, 125, 3
+    good = random_window_indices(rng, B, n, 900)
+    for bad_row, what in (([B, 3], "outside"), ([-1, 0], "outside"), ([2, n], "outside"), ([5, -7], "outside"),
+                          (list(good[17]), "distinct")):
+        ind = np.concatenate([good[:400], np.array([bad_row], np.int32), good[400:]])
+        with pytest.raises(RuntimeError, match=what):
+            TokenPlan(torch.from_numpy(ind).cuda(), B, n, H)
+    tp = TokenPlan(torch.from_numpy(good).cuda(), B, n, H)     # and the library still works
+    assert tp.G == len(np.unique(good[:, 0])) * H
 
 
 def _modules(dim, heads, dtype):

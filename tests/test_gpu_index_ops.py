@@ -123,6 +123,28 @@ def test_qkv_sparse_indices_ragged_and_last_slot(ops, oracle):
         np.testing.assert_array_equal(g.cpu().numpy(), r)
 
 
+def test_index_ops_report_indices_they_cannot_address(ops):
+    """A window id >= batch_size, a position >= n, a negative entry, a repeated (window, pos) pair, or a value
+    >= maxnum never becomes a device address: the kernels skip it and the operator raises."""
+    rng = np.random.default_rng(11)
+    B, n, H, hd = 30, 125, 3, 32
+    good = random_window_indices(rng, B, n, 700)
+    for bad_row, what in (([B, 0], "outside"), ([0, n], "outside"), ([-3, 5], "outside"), ([4, -1], "outside"),
+                          (list(good[5]), "distinct")):
+        ind = np.concatenate([good[:300], np.array([bad_row], np.int32), good[300:]])
+        with pytest.raises(RuntimeError, match=what):
+            ops.qkv_sparse_indices(dev(ind), B, n, H, hd)
+    x = rng.integers(0, 500, size=2000).astype(np.int32)
+    x[77] = 500
+    with pytest.raises(RuntimeError, match="outside"):
+        ops.return_inverse(dev(x), 500)
+    x[77] = -2
+    with pytest.raises(RuntimeError, match="outside"):
+        ops.return_inverse(dev(x), 500)
+    got = ops.qkv_sparse_indices(dev(good), B, n, H, hd)            # and the library still works afterwards
+    assert got[1].numel() == 700 * H * hd
+
+
 def test_ops_reject_cpu_tensors(ops):
     with pytest.raises(RuntimeError, match="GPU only"):
         ops.flatten_indices(torch.zeros((2, 4), dtype=torch.int32), [3, 3])
