@@ -227,9 +227,9 @@ def kernel_table(wl, reps=20, only=None):
                                                       ptr(out_f), D, 0, ptr(lse), stream))
 
     # The step asks for all gradients at once (sides = 3): one launch in which groups of at most
-    # 32 tokens get dQ from their key-side task and only the larger groups have query-side tasks.
-    # The parts are timed alone for comparison: 6 = the key-side tasks of that launch, restricted
-    # bucket counts = the query-side kernel on the larger groups, 1 / 2 = the per-side kernels.
+    # 64 tokens get dQ from their key-side tasks and only the larger groups have query-side tasks.
+    # The parts are timed alone for comparison: restricted bucket counts = the query-side kernel on
+    # the groups of more than 32 tokens, 1 / 2 = the per-side kernels.
     bc = [int(x) for x in tp.bucket_counts]
     cg = tp.plan[:tp.G].to(torch.int64)                                  # plan row 0: tokens of each group
     rows1, rowsL = int(cg[cg <= 32].sum()), int(cg[cg > 32].sum())       # token-head rows of small / large groups
@@ -257,7 +257,6 @@ def kernel_table(wl, reps=20, only=None):
         ("resident forward", r_fwd, 16 * E + 4 * H * N, 1),
         ("resident backward (dQ,dK,dV,dS)", r_bwd(3), 32 * E + 4 * A + 4 * H * N, 1),
         ("resident backward dQ, groups > 32 tokens", r_bwd(1, only_large), (24 * hd + 4) * rowsL, 0),
-        ("resident backward dK,dV,dS + dQ of small groups", r_bwd(6), 28 * E + 4 * A + 4 * H * N + 4 * hd * rows1, 0),
         ("resident backward dQ, all groups", r_bwd(1), 24 * E + 4 * H * N, 0),
         ("resident backward dK,dV,dS only", r_bwd(2), 28 * E + 4 * A + 4 * H * N, 0),
         ("resident bias table grad", r_table_grad, 4 * A, 1),

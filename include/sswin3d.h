@@ -305,9 +305,10 @@ int sswin_window_attention_forward(int dtype, const int32_t* tasks, int64_t g_ca
  * recomputes P per tile and writes dQ = scale dS K, dK = scale dS^T Q, dV = P^T dO with
  * dS = P (dP - rowsum(dO o O)).  ds_out (fp32 "sq" array in plan order, or NULL) receives dS
  * for the bias gradient.  sides: 1 = dQ only (query-side kernel), 2 = dK and dV (and dS) only
- * (key-side kernel), 3 = all: the key-side kernel then also writes dQ of the groups of at most 32
- * tokens (their dS is already in its registers) and the query-side kernel runs for the larger
- * groups only; 6 = the key-side launch of 3 alone (for profiling).  Asynchronous. */
+ * (key-side kernel), 3 = all in one launch: the key-side tasks then also produce dQ of the groups of
+ * at most 64 tokens (one tile: from the dS already in registers; two tiles: the two key-side tasks of a
+ * group exchange their partial dS K through LDS) and only the larger groups have query-side tasks.
+ * Asynchronous. */
 int sswin_window_attention_backward(int dtype, const int32_t* tasks, int64_t g_cap,
                                     const int64_t* bucket_counts, const int32_t* tokens, int64_t N,
                                     int H, int hd, const void* q_base, int64_t q_stride, int q_col0,

@@ -174,6 +174,28 @@ __device__ __forceinline__ void table_get(const uint32_t* tab, int half, uint32_
         x[4 * q] = t.x; x[4 * q + 1] = t.y; x[4 * q + 2] = t.z; x[4 * q + 3] = t.w;
     }
 }
+// A table kept in the spare columns of a tile: rows are 36 dwords wide and only 32 of them carry
+// values, so the four spare dwords of eight consecutive rows hold 32 entries, entries 4k .. 4k+3
+// in row k.  A tile has room for four such tables (rows 0-7, 8-15, 16-23, 24-31); the 16-byte
+// reads of table_get fall on whole rows' spare columns.  The backward kernels keep their tables
+// there, which leaves LDS for the exchange tiles of the two-tile groups.
+struct PadTab {
+    uint32_t* p;
+    __device__ __forceinline__ void put(int e, uint32_t v) const { p[(e >> 2) * TILE_LD + (e & 3)] = v; }
+    __device__ __forceinline__ uint32_t get(int e) const { return p[(e >> 2) * TILE_LD + (e & 3)]; }
+    __device__ __forceinline__ u32x4_a chunk(int ch) const { return *reinterpret_cast<const u32x4_a*>(p + ch * TILE_LD); }
+};
+__device__ __forceinline__ PadTab pad_tab(float* tile, int k) {
+    return PadTab{reinterpret_cast<uint32_t*>(tile) + 8 * k * TILE_LD + 32};
+}
+__device__ __forceinline__ void table_put(const PadTab& tab, int l32, uint32_t v) { tab.put(l32, v); }
+__device__ __forceinline__ void table_get(const PadTab& tab, int half, uint32_t (&x)[16]) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const u32x4_a t = tab.chunk(2 * q + half);
+        x[4 * q] = t.x; x[4 * q + 1] = t.y; x[4 * q + 2] = t.z; x[4 * q + 3] = t.w;
+    }
+}
 __device__ __forceinline__ uint32_t f2u(float v) { return __builtin_bit_cast(uint32_t, v); }
 __device__ __forceinline__ float u2f(uint32_t v) { return __builtin_bit_cast(float, v); }
 __device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
@@ -363,7 +385,7 @@ __device__ __forceinline__ float chunk_dot(const u32x4_a& x, const u32x4_a& y) {
     return d;
 }
 template <typename T>
-__device__ __forceinline__ void rows_dot_to_table(uint32_t* tab, int lane, const RowLoad<T>& x, const RowLoad<T>& y) {
+__device__ __forceinline__ void rows_dot_to_table(const PadTab& tab, int lane, const RowLoad<T>& x, const RowLoad<T>& y) {
     constexpr int CH = RowLoad<T>::CH, ROWS = RowLoad<T>::ROWS;
 #pragma unroll
     for (int v = 0; v < RowLoad<T>::NI; ++v) {
@@ -371,7 +393,7 @@ __device__ __forceinline__ void rows_dot_to_table(uint32_t* tab, int lane, const
         d += dpp_f32<0xB1>(d);                               // lanes 0..3 of a quad
         d += dpp_f32<0x4E>(d);
         if (CH == 8) d += dpp_f32<0x141>(d);                 // the two quads of 8 lanes
-        if (lane % CH == 0) tab[v * ROWS + lane / CH] = f2u(d);
+        if (lane % CH == 0) tab.put(v * ROWS + lane / CH, f2u(d));
     }
 }
 
@@ -517,7 +539,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 // rows in transit to the operand layout, then dQ; two 32-entry tables.
 template <typename T, bool MASK>
 __device__ __forceinline__ void bwd_q_task(const WAttnCommon& a, int64_t task, float* tile, float* tile_x,
-                                           uint32_t* tab_key, uint32_t* tab_D, const TokenTensor32& tq,
+                                           const TokenTensor32& tq,
                                            const TokenTensor32& tk, const TokenTensor32& tv, const TokenTensor32& to,
                                            const TokenTensor32& tdo, const float* __restrict__ lse,
                                            const TokenTensor32& tdq) {
@@ -526,6 +548,7 @@ __device__ __forceinline__ void bwd_q_task(const WAttnCommon& a, int64_t task, f
     int64_t d;
     int bi;
     if (!locate(a, task, d, bi)) return;
+    const PadTab tab_key = pad_tab(tile, 0), tab_D = pad_tab(tile, 1);
     const GroupCtx g = load_group(a.tasks, d);
     const int c = g.c, h = g.h;
     const int nt = (c + 31) >> 5;
@@ -557,7 +580,7 @@ __device__ __forceinline__ void bwd_q_task(const WAttnCommon& a, int64_t task, f
         __builtin_amdgcn_wave_barrier();
         tile_get_rows(tile_x, l32, half, dob);
     }
-    const float D = u2f(tab_D[l32]);
+    const float D = u2f(tab_D.get(l32));
     const float qscale = a.scale * LOG2E;
 #pragma unroll
     for (int s = 0; s < 16; ++s) qb[s] *= qscale;
@@ -623,20 +646,44 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     WAttnCommon a, TokenTensor32 tq, TokenTensor32 tk, TokenTensor32 tv, TokenTensor32 to, TokenTensor32 tdo,
     const float* __restrict__ lse, TokenTensor32 tdq) {
     __shared__ __attribute__((aligned(16))) float tiles[4][2][TILE_WORDS];
-    __shared__ __attribute__((aligned(16))) uint32_t tabs[4][2][32];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    bwd_q_task<T, MASK>(a, (int64_t)blockIdx.x * 4 + wave, tiles[wave][0], tiles[wave][1], tabs[wave][0], tabs[wave][1],
-                        tq, tk, tv, to, tdo, lse, tdq);
+    bwd_q_task<T, MASK>(a, (int64_t)blockIdx.x * 4 + wave, tiles[wave][0], tiles[wave][1], tq, tk, tv, to, tdo, lse, tdq);
 }
 
 // ------------------------------------------------------------------------------------------
 // backward, key side: dK, dV (and dS for the bias gradient)
 // ------------------------------------------------------------------------------------------
-// DQ1: groups of one tile also get their dQ here (dS is already in registers; transposed through
-// LDS it is the A operand of dQ = dS K), which saves them the whole query-side kernel
-template <typename T, bool MASK, bool DQ1>
-__device__ __forceinline__ void bwd_kv_task(const WAttnCommon& a, int64_t task, float* tile_q, float* tile_do,
-                                            uint32_t* tab_pos, uint32_t* tab_L, uint32_t* tab_D,
+// What a key-side task does about dQ:
+//   KV_ONLY    nothing (the group has query-side tasks of its own)
+//   KV_SINGLE  a group of one tile: dS is already in registers; transposed through LDS it is the A
+//              operand of dQ = dS K, which saves the group its whole query-side task
+//   KV_PAIR    a group of two tiles, its two key-side tasks on neighbouring wavefronts of one
+//              workgroup: each forms dS K for both query tiles, hands the partial result of the other
+//              wavefront's tile over through an LDS exchange tile, and after one workgroup barrier adds
+//              the two partial results of its own tile.  S and dP of the group are then computed once
+//              instead of twice (320 instead of 448 MFMA steps of 32x32x2 per group) and the five
+//              operands are read once.
+enum { KV_ONLY = 0, KV_SINGLE = 1, KV_PAIR = 2 };
+
+// xch: this wavefront's exchange tile (KV_PAIR), xch_peer: the other wavefront's; accumulator layout
+__device__ __forceinline__ void xch_put(float* xch, int lane, const f32x16& v) {
+    f32x4_a* p = reinterpret_cast<f32x4_a*>(xch + lane * 16);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) p[q] = f32x4_a{v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]};
+}
+__device__ __forceinline__ void xch_add(const float* xch, int lane, f32x16& v) {
+    const f32x4_a* p = reinterpret_cast<const f32x4_a*>(xch + lane * 16);
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const f32x4_a t = p[q];
+        v[4 * q] += t.x; v[4 * q + 1] += t.y; v[4 * q + 2] += t.z; v[4 * q + 3] += t.w;
+    }
+}
+
+// `live` = false (KV_PAIR only): a wavefront without a task that still has to meet the barrier.
+template <typename T, bool MASK, int DQ>
+__device__ __forceinline__ void bwd_kv_task(const WAttnCommon& a, int64_t task, bool live, float* tile_q, float* tile_do,
+                                            float* xch, const float* xch_peer,
                                             const TokenTensor32& tq, const TokenTensor32& tk, const TokenTensor32& tv,
                                             const TokenTensor32& to, const TokenTensor32& tdo,
                                             const float* __restrict__ lse, const TokenTensor32& tdk,
@@ -646,7 +693,11 @@ __device__ __forceinline__ void bwd_kv_task(const WAttnCommon& a, int64_t task, 
     const int half = lane >> 5, l32 = lane & 31;
     int64_t d;
     int bj;
-    if (!locate(a, task, d, bj)) return;
+    if (!live || !locate(a, task, d, bj)) {
+        if (DQ == KV_PAIR) __syncthreads();
+        return;
+    }
+    const PadTab tab_pos = pad_tab(tile_q, 0), tab_L = pad_tab(tile_q, 1), tab_D = pad_tab(tile_q, 2);
     const GroupCtx g = load_group(a.tasks, d);
     const int c = g.c, h = g.h;
     const int nt = (c + 31) >> 5;
@@ -659,17 +710,40 @@ __device__ __forceinline__ void bwd_kv_task(const WAttnCommon& a, int64_t task, 
     const uint32_t qpitch = pitch_of<T>(tq), opitch = pitch_of<T>(to), dopitch = pitch_of<T>(tdo);
     const float* lse_g = lse + (int64_t)a.H * g.Tk + h * c;
 
+    // Memory round trips of a task depend on one another (descriptor -> token indices -> rows -> bias), and
+    // a task is short, so everything that can be requested in the same round trip is: the indices of the
+    // first query tile go out with the key indices, and its rows with the K and V rows.
+    struct QIdx {
+        uint32_t vox;        // voxel of query t*32 + l32 (clamped to the last token)
+        int pos;
+        float L2;            // its log-sum-exp in units of log 2; +inf for padding queries: P and dS exactly zero
+    };
+    auto load_qidx = [&](const int t) {
+        const int i = t * 32 + l32;
+        const int i_c = i < c ? i : c - 1;
+        QIdx q;
+        q.vox = order[i_c];
+        q.pos = tok_pos[i_c];
+        q.L2 = i < c ? lse_g[i_c] * LOG2E : INFINITY;
+        return q;
+    };
     // key side: lane l32 owns key bj*32 + l32
     const int j_k = bj * 32 + l32;
     const int j_c = j_k < c ? j_k : c - 1;
     const uint32_t vox_j = order[j_c];
     const int pos_j = tok_pos[j_c];
+    const int t_first = DQ == KV_PAIR ? 1 - bj : 0;           // KV_PAIR: the other wavefront's query tile first
+    QIdx qcur = load_qidx(t_first);
     const int reg_j = MASK ? mrow[pos_j] : 0;
+    RowLoad<T> rq, rdo, ro;
     float kb[16], vb[16];
     {
         RowLoad<T> rk, rv;
         rows_load<T>(head_base<T>(tk, h), pitch_of<T>(tk), vox_j, lane, rk);
         rows_load<T>(head_base<T>(tv, h), pitch_of<T>(tv), vox_j, lane, rv);
+        rows_load<T>(qbase, qpitch, qcur.vox, lane, rq);
+        rows_load<T>(dobase, dopitch, qcur.vox, lane, rdo);
+        rows_load<T>(obase, opitch, qcur.vox, lane, ro);
         rows_to_tile<T>(tile_q, lane, rk);
         rows_to_tile<T>(tile_do, lane, rv);
         __builtin_amdgcn_wave_barrier();
@@ -685,58 +759,57 @@ __device__ __forceinline__ void bwd_kv_task(const WAttnCommon& a, int64_t task, 
 
     f32x16 dk = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     f32x16 dv = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-#pragma unroll 1
-    for (int t = 0; t < nt; ++t) {
-        // query side of tile t: lane l32 owns query t*32 + l32
-        const int i = t * 32 + l32;
-        const int i_c = i < c ? i : c - 1;
-        const uint32_t vox_i = order[i_c];
-        const int pos_i = tok_pos[i_c];
-        // padding queries get L = +inf, which makes their P and dS exactly zero
-        const float L2_i = i < c ? lse_g[i_c] * LOG2E : INFINITY;
-        RowLoad<T> rq, rdo, ro;
-        rows_load<T>(qbase, qpitch, vox_i, lane, rq);
-        rows_load<T>(dobase, dopitch, vox_i, lane, rdo);
-        rows_load<T>(obase, opitch, vox_i, lane, ro);
-        uint32_t pi = (uint32_t)(pos_i * a.n) * 4u;          // byte offset of bias row pos_i (< 2^16)
-        if (MASK) pi |= (uint32_t)mrow[pos_i] << 16;
+    f32x16 dq_own;                                            // KV_PAIR: dS K of this wavefront's own query tile
+    // One query tile t against this task's keys.  What happens to dS K of the tile (dq_tag): 0 = not
+    // formed, 1 = written out as dQ of a one-tile group, 2 = handed to the other wavefront of the pair,
+    // 3 = kept in dq_own.
+    // rq, rdo, ro hold the rows of query tile t (requested by the caller), qi its indices.
+    auto tile_pass = [&](const int t, const QIdx& qi, auto dq_tag) {
+        constexpr int DQ_USE = decltype(dq_tag)::value;
+        uint32_t pi = (uint32_t)(qi.pos * a.n) * 4u;         // byte offset of bias row pos_i (< 2^16)
+        if (MASK) pi |= (uint32_t)mrow[qi.pos] << 16;
         __builtin_amdgcn_wave_barrier();
         table_put(tab_pos, l32, pi);
-        table_put(tab_L, l32, f2u(L2_i));
+        table_put(tab_L, l32, f2u(qi.L2));
         rows_dot_to_table<T>(tab_D, lane, rdo, ro);          // D_i = dO_i . O_i
         rows_to_tile<T>(tile_q, lane, rq);                   // both are read back by row and by column
         rows_to_tile<T>(tile_do, lane, rdo);
         __builtin_amdgcn_wave_barrier();
-        float qa[16], doa[16];
-        tile_get_rows(tile_q, l32, half, qa);
-        tile_get_rows(tile_do, l32, half, doa);
-        f32x16 St = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-        f32x16 dPt = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-        mma_slots<T, 0, 16>(qa, kb, St);
-        mma_slots<T, 0, 16>(doa, vb, dPt);
-
         // P and dS of the tile: rows = queries acc_row(r, half), column = this lane's key.
-        // The bias gathers of all 16 rows are issued first; everything else is fetched from
-        // LDS four rows at a time, right before it is used, to keep the register footprint low.
-        uint32_t pir[16];
-        table_get(tab_pos, half, pir);
+        // The bias gathers of all 16 rows are requested between the two score products (the second
+        // one covers their latency, and the operand registers of the first are free by then);
+        // everything else is fetched from LDS four rows at a time, right before it is used, to keep
+        // the register footprint low.
+        f32x16 St, dPt;
+        {
+            float qa[16];
+            tile_get_rows(tile_q, l32, half, qa);
+            St = mma_slots_first<T, 16>(qa, kb);
+        }
         float bv[16];
         uint32_t differ = 0;                                  // bit r: regions of the row and the key differ
+        {
+            uint32_t pir[16];
+            table_get(tab_pos, half, pir);
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            bv[r] = *reinterpret_cast<const float*>(bias_h + (bcol + (MASK ? (pir[r] & 0xffffu) : pir[r])));
-            if (MASK) differ |= ((int)(pir[r] >> 16) != reg_j ? 1u : 0u) << r;
+            for (int r = 0; r < 16; ++r) {
+                bv[r] = *reinterpret_cast<const float*>(bias_h + (bcol + (MASK ? (pir[r] & 0xffffu) : pir[r])));
+                if (MASK) differ |= ((int)(pir[r] >> 16) != reg_j ? 1u : 0u) << r;
+            }
+        }
+        {
+            float doa[16];
+            tile_get_rows(tile_do, l32, half, doa);
+            dPt = mma_slots_first<T, 16>(doa, vb);
         }
         float* ds_t = ds_g ? ds_g + (int64_t)(t * 32 + 4 * half) * c : nullptr;
         const int ilim = c - t * 32 - 4 * half;
-        const u32x4_a* L4 = reinterpret_cast<const u32x4_a*>(tab_L + 4 * half);
-        const u32x4_a* D4 = reinterpret_cast<const u32x4_a*>(tab_D + 4 * half);
         const float* do_col = tile_do + 4 * half * TILE_LD + l32;
         const float* q_col = tile_q + 4 * half * TILE_LD + l32;
         float dob8[8], qbr8[8];                              // 16-bit tokens: operands of eight slots
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
-            const u32x4_a Lq = L4[2 * q], Dq = D4[2 * q];
+            const u32x4_a Lq = tab_L.chunk(2 * q + half), Dq = tab_D.chunk(2 * q + half);
             const uint32_t Lr[4] = {Lq.x, Lq.y, Lq.z, Lq.w}, Dr[4] = {Dq.x, Dq.y, Dq.z, Dq.w};
             float dob[4], qbr[4];
 #pragma unroll
@@ -756,7 +829,7 @@ __device__ __forceinline__ void bwd_kv_task(const WAttnCommon& a, int64_t task, 
                 if constexpr (std::is_same<T, float>::value) {
                     dv = __builtin_amdgcn_mfma_f32_32x32x2f32(pr, dob[k], dv, 0, 0, 0);     // dV += P^T dO
                     dk = __builtin_amdgcn_mfma_f32_32x32x2f32(ds, qbr[k], dk, 0, 0, 0);     // dK += dS^T Q
-                    if (DQ1) dPt[r] = ds;
+                    if (DQ_USE != 0) dPt[r] = ds;
                 } else {                                     // collected: eight slots per 16-bit step
                     St[r] = pr;
                     dPt[r] = ds;
@@ -776,8 +849,8 @@ __device__ __forceinline__ void bwd_kv_task(const WAttnCommon& a, int64_t task, 
                 }
             }
         }
-        if (DQ1 && nt == 1) {
-            // dS of the only tile (rows = queries by register, column = this lane's key; padding keys
+        if constexpr (DQ_USE != 0) {
+            // dS of this tile (rows = queries by register, column = this lane's key; padding keys
             // zeroed) -> LDS -> one query row per lane; K rows (still scaled by scale * log2 e) go back
             // to LDS for the column reads.  dQ = scale dS K = (dS K_scaled) ln 2.
 #pragma unroll
@@ -792,13 +865,44 @@ __device__ __forceinline__ void bwd_kv_task(const WAttnCommon& a, int64_t task, 
 #pragma unroll
             for (int s = 0; s < 16; ++s) kc[s] = k_col[s * TILE_LD];  // K[key 16 * half + s][channel l32]
             f32x16 dq = mma_slots_first<T, 16>(dsr, kc);
+            if constexpr (DQ_USE == 2) {
+                xch_put(xch, lane, dq);
+                __builtin_amdgcn_wave_barrier();
+            } else if constexpr (DQ_USE == 3) {
+                dq_own = dq;
+                __builtin_amdgcn_wave_barrier();
+            } else {
 #pragma unroll
-            for (int r = 0; r < 16; ++r) dq[r] *= LN2;
-            __builtin_amdgcn_wave_barrier();
-            tile_put_acc(tile_do, l32, half, dq);
-            __builtin_amdgcn_wave_barrier();
-            tile_store_rows<T>(tile_do, const_cast<char*>(head_base<T>(tdq, h)), pitch_of<T>(tdq), vox_j, c, lane);
-            __builtin_amdgcn_wave_barrier();
+                for (int r = 0; r < 16; ++r) dq[r] *= LN2;
+                __builtin_amdgcn_wave_barrier();
+                tile_put_acc(tile_do, l32, half, dq);
+                __builtin_amdgcn_wave_barrier();
+                tile_store_rows<T>(tile_do, const_cast<char*>(head_base<T>(tdq, h)), pitch_of<T>(tdq), vox_j, c, lane);
+                __builtin_amdgcn_wave_barrier();
+            }
+        }
+    };
+    // the indices of the next query tile are requested before the current one is worked on
+    auto request_rows = [&](const QIdx& qi) {
+        rows_load<T>(qbase, qpitch, qi.vox, lane, rq);
+        rows_load<T>(dobase, dopitch, qi.vox, lane, rdo);
+        rows_load<T>(obase, opitch, qi.vox, lane, ro);
+    };
+    if constexpr (DQ == KV_PAIR) {
+        // the other wavefront's query tile first, the own one last (its result stays in registers)
+        const QIdx qown = load_qidx(bj);
+        tile_pass(1 - bj, qcur, std::integral_constant<int, 2>{});
+        request_rows(qown);
+        tile_pass(bj, qown, std::integral_constant<int, 3>{});
+    } else if constexpr (DQ == KV_SINGLE) {
+        tile_pass(0, qcur, std::integral_constant<int, 1>{});     // groups of one tile only
+    } else {
+        tile_pass(0, qcur, std::integral_constant<int, 0>{});
+#pragma unroll 1
+        for (int t = 1; t < nt; ++t) {
+            const QIdx qi = load_qidx(t);
+            request_rows(qi);
+            tile_pass(t, qi, std::integral_constant<int, 0>{});
         }
     }
 #pragma unroll
@@ -809,6 +913,15 @@ __device__ __forceinline__ void bwd_kv_task(const WAttnCommon& a, int64_t task, 
     __builtin_amdgcn_wave_barrier();
     tile_store_rows<T>(tile_q, const_cast<char*>(head_base<T>(tdk, h)), pitch_of<T>(tdk), vox_j, c - bj * 32, lane);
     tile_store_rows<T>(tile_do, const_cast<char*>(head_base<T>(tdv, h)), pitch_of<T>(tdv), vox_j, c - bj * 32, lane);
+    if (DQ == KV_PAIR) {
+        __syncthreads();                                     // both partial results of every pair are in LDS
+        xch_add(xch_peer, lane, dq_own);
+#pragma unroll
+        for (int r = 0; r < 16; ++r) dq_own[r] *= LN2;
+        tile_put_acc(tile_do, l32, half, dq_own);
+        __builtin_amdgcn_wave_barrier();
+        tile_store_rows<T>(tile_do, const_cast<char*>(head_base<T>(tdq, h)), pitch_of<T>(tdq), vox_j, c - bj * 32, lane);
+    }
 }
 
 template <typename T, bool MASK>
@@ -816,31 +929,52 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     WAttnCommon a, TokenTensor32 tq, TokenTensor32 tk, TokenTensor32 tv, TokenTensor32 to, TokenTensor32 tdo,
     const float* __restrict__ lse, TokenTensor32 tdk, TokenTensor32 tdv, float* __restrict__ ds_out) {
     __shared__ __attribute__((aligned(16))) float tiles[4][2][TILE_WORDS];
-    __shared__ __attribute__((aligned(16))) uint32_t tabs[4][3][32];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    bwd_kv_task<T, MASK, false>(a, (int64_t)blockIdx.x * 4 + wave, tiles[wave][0], tiles[wave][1], tabs[wave][0],
-                                tabs[wave][1], tabs[wave][2], tq, tk, tv, to, tdo, lse, tdk, tdv, ds_out, tdk);
+    bwd_kv_task<T, MASK, KV_ONLY>(a, (int64_t)blockIdx.x * 4 + wave, true, tiles[wave][0], tiles[wave][1], nullptr, nullptr,
+                                  tq, tk, tv, to, tdo, lse, tdk, tdv, ds_out, tdk);
 }
 
-// The whole backward in one launch: the query-side tasks of the groups of more than 32 tokens
-// first (tasks 0 .. first[3]), then the key-side tasks of all groups; groups of at most 32 tokens
-// get dQ from their key-side task.  One launch keeps the chip filled while the long tasks run.
+// The whole backward in one launch.  Workgroups (four wavefronts, one task each) are numbered through
+// four segments, each starting at a workgroup boundary:
+//   1. query-side tasks of the groups of three and four tiles
+//   2. their key-side tasks (KV_ONLY)
+//   3. key-side tasks of the groups of two tiles, the two tasks of a group side by side (KV_PAIR)
+//   4. key-side tasks of the groups of one tile (KV_SINGLE)
+// Heaviest tasks first, so the long ones start first and the short ones fill the tail.
+struct BwdSegments {
+    int64_t wg_kv, wg_pair, wg_single;   // first workgroup of segments 2, 3, 4
+    int64_t n_big;                       // tasks per side of the groups of three and four tiles
+    int64_t n_pair;                      // key-side tasks of the groups of two tiles (even)
+};
+
 template <typename T, bool MASK>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void wattn_bwd_all_kernel(
-    WAttnCommon a, TokenTensor32 tq, TokenTensor32 tk, TokenTensor32 tv, TokenTensor32 to, TokenTensor32 tdo,
-    const float* __restrict__ lse, TokenTensor32 tdq, TokenTensor32 tdk, TokenTensor32 tdv,
-    float* __restrict__ ds_out, int key_side_only) {
+    WAttnCommon a, BwdSegments sg, TokenTensor32 tq, TokenTensor32 tk, TokenTensor32 tv, TokenTensor32 to,
+    TokenTensor32 tdo, const float* __restrict__ lse, TokenTensor32 tdq, TokenTensor32 tdk, TokenTensor32 tdv,
+    float* __restrict__ ds_out) {
     __shared__ __attribute__((aligned(16))) float tiles[4][2][TILE_WORDS];
-    __shared__ __attribute__((aligned(16))) uint32_t tabs[4][3][32];
+    __shared__ __attribute__((aligned(16))) float xch[4][64 * 16];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int64_t task = (int64_t)blockIdx.x * 4 + wave;
-    const int64_t nq = key_side_only ? 0 : a.first[3];       // query-side tasks of the larger groups
-    if (task < nq)
-        bwd_q_task<T, MASK>(a, task, tiles[wave][0], tiles[wave][1], tabs[wave][0], tabs[wave][1], tq, tk, tv, to, tdo,
-                            lse, tdq);
-    else
-        bwd_kv_task<T, MASK, true>(a, task - nq, tiles[wave][0], tiles[wave][1], tabs[wave][0], tabs[wave][1],
-                                   tabs[wave][2], tq, tk, tv, to, tdo, lse, tdk, tdv, ds_out, tdq);
+    const int64_t wg = blockIdx.x;
+    float* t0 = tiles[wave][0];
+    float* t1 = tiles[wave][1];
+    if (wg < sg.wg_kv) {
+        const int64_t task = wg * 4 + wave;
+        if (task < sg.n_big) bwd_q_task<T, MASK>(a, task, t0, t1, tq, tk, tv, to, tdo, lse, tdq);
+    } else if (wg < sg.wg_pair) {
+        const int64_t task = (wg - sg.wg_kv) * 4 + wave;
+        if (task < sg.n_big)
+            bwd_kv_task<T, MASK, KV_ONLY>(a, task, true, t0, t1, nullptr, nullptr, tq, tk, tv, to, tdo, lse, tdk, tdv,
+                                          ds_out, tdq);
+    } else if (wg < sg.wg_single) {
+        const int64_t task = (wg - sg.wg_pair) * 4 + wave;
+        bwd_kv_task<T, MASK, KV_PAIR>(a, sg.n_big + task, task < sg.n_pair, t0, t1, xch[wave], xch[wave ^ 1], tq, tk, tv, to,
+                                      tdo, lse, tdk, tdv, ds_out, tdq);
+    } else {
+        const int64_t task = (wg - sg.wg_single) * 4 + wave;
+        bwd_kv_task<T, MASK, KV_SINGLE>(a, sg.n_big + sg.n_pair + task, true, t0, t1, nullptr, nullptr, tq, tk, tv, to, tdo,
+                                        lse, tdk, tdv, ds_out, tdq);
+    }
 }
 
 // ------------------------------------------------------------------------------------------
@@ -864,10 +998,18 @@ static void launch_backward(const WAttnCommon& a, const TokenTensor32& q, const 
                             const TokenTensor32& v, const TokenTensor32& o, const TokenTensor32& d_o, const float* lse,
                             const TokenTensor32& dq, const TokenTensor32& dk, const TokenTensor32& dv, float* ds_out,
                             int sides, hipStream_t s) {
-    if (sides == 3 || sides == 6) {
-        const int64_t tasks = a.first[4] + (sides == 3 ? a.first[3] : 0);
-        hipLaunchKernelGGL((wattn_bwd_all_kernel<T, MASK>), dim3((unsigned)((tasks + 3) / 4)), dim3(256), 0, s, a, q, k, v,
-                           o, d_o, lse, dq, dk, dv, ds_out, sides == 6 ? 1 : 0);
+    if (sides == 3) {
+        BwdSegments sg;
+        sg.n_big = a.first[2];
+        sg.n_pair = a.first[3] - a.first[2];
+        const int64_t n_single = a.first[4] - a.first[3];
+        const int64_t wg_big = (sg.n_big + 3) / 4;
+        sg.wg_kv = wg_big;
+        sg.wg_pair = 2 * wg_big;
+        sg.wg_single = sg.wg_pair + (sg.n_pair + 3) / 4;
+        const int64_t wgs = sg.wg_single + (n_single + 3) / 4;
+        hipLaunchKernelGGL((wattn_bwd_all_kernel<T, MASK>), dim3((unsigned)wgs), dim3(256), 0, s, a, sg, q, k, v, o, d_o, lse,
+                           dq, dk, dv, ds_out);
         return;
     }
     const unsigned blocks = (unsigned)((a.first[4] + 3) / 4);
@@ -990,10 +1132,9 @@ int sswin_window_attention_backward(int dtype, const int32_t* tasks, int64_t g_c
                      n_mask_windows, &total))
         return 1;
     if (total == 0) return 0;
-    SSWIN_CHECK(sides == 1 || sides == 2 || sides == 3 || sides == 6,
-                "window_attention_backward: sides must be 1 (dQ), 2 (dK, dV), 3 (all) or 6 (key-side kernel of 3)");
+    SSWIN_CHECK(sides == 1 || sides == 2 || sides == 3, "window_attention_backward: sides must be 1 (dQ), 2 (dK, dV) or 3 (all)");
     SSWIN_CHECK(q_base && k_base && v_base && o_base && do_base && lse, "window_attention_backward: null pointer");
-    SSWIN_CHECK(!(sides & 5) || dq_base, "window_attention_backward: dq is null");
+    SSWIN_CHECK(!(sides & 1) || dq_base, "window_attention_backward: dq is null");
     SSWIN_CHECK(!(sides & 2) || (dk_base && dv_base), "window_attention_backward: dk or dv is null");
     {
         const char* who = "window_attention_backward";
@@ -1003,7 +1144,7 @@ int sswin_window_attention_backward(int dtype, const int32_t* tasks, int64_t g_c
             check_tensor(who, "o", o_base, o_stride, o_col0, N, H, dtype) ||
             check_tensor(who, "do", do_base, do_stride, do_col0, N, H, dtype))
             return 1;
-        if ((sides & 5) && check_tensor(who, "dq", dq_base, dq_stride, dq_col0, N, H, dtype)) return 1;
+        if ((sides & 1) && check_tensor(who, "dq", dq_base, dq_stride, dq_col0, N, H, dtype)) return 1;
         if ((sides & 2) && (check_tensor(who, "dk", dk_base, dk_stride, dk_col0, N, H, dtype) ||
                             check_tensor(who, "dv", dv_base, dv_stride, dv_col0, N, H, dtype)))
             return 1;
