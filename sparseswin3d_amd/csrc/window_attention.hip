@@ -431,11 +431,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     const int i_c = i_q < c ? i_q : c - 1;
     const uint32_t vox_i = order[i_c];
     const int pos_i = tok_pos[i_c];
+    // The memory round trips of a task depend on one another (descriptor -> token indices -> rows ->
+    // bias) and a task is short, so the indices of the first key tile are requested together with the
+    // query indices, and its K and V rows together with the Q rows.
+    struct KIdx {
+        uint32_t vox;        // voxel of key t*32 + l32 (clamped to the last token)
+        int pos;
+    };
+    auto load_kidx = [&](const int t) {
+        const int j = t * 32 + l32;
+        const int j_c = j < c ? j : c - 1;
+        return KIdx{(uint32_t)order[j_c], tok_pos[j_c]};
+    };
+    KIdx kcur = load_kidx(0);
     const int reg_i = MASK ? mrow[pos_i] : 0;
+    RowLoad<T> rk, rv;
     float qb[16];
     {
         RowLoad<T> rq;
         rows_load<T>(qbase, qpitch, vox_i, lane, rq);
+        rows_load<T>(kbase, kpitch, kcur.vox, lane, rk);
+        rows_load<T>(vbase, vpitch, kcur.vox, lane, rv);
         rows_to_tile<T>(tile_x, lane, rq);
         __builtin_amdgcn_wave_barrier();
         tile_get_rows(tile_x, l32, half, qb);
@@ -451,33 +467,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     f32x16 o;
     // one tile of keys.  The first tile is a separate instantiation: its accumulators start from the
     // instruction's zero operand and nothing has to be rescaled (most groups have one tile only).
-    auto tile_step = [&](auto first_tag, const int t) {
+    // rk, rv hold the K and V rows of key tile t (requested by the caller), ki its indices.
+    auto tile_step = [&](auto first_tag, const int t, const KIdx& ki) {
         constexpr bool FIRST = decltype(first_tag)::value;
-        // key side of tile t: lane l32 owns key t*32 + l32
-        const int j = t * 32 + l32;
-        const int j_c = j < c ? j : c - 1;
-        const uint32_t vox_j = order[j_c];
-        const int pos_j = tok_pos[j_c];
-        RowLoad<T> rk, rv;
-        rows_load<T>(kbase, kpitch, vox_j, lane, rk);
-        rows_load<T>(vbase, vpitch, vox_j, lane, rv);
-        uint32_t pk = (uint32_t)pos_j * 4u;
-        if (MASK) pk |= (uint32_t)mrow[pos_j] << 16;
+        uint32_t pk = (uint32_t)ki.pos * 4u;
+        if (MASK) pk |= (uint32_t)mrow[ki.pos] << 16;
         __builtin_amdgcn_wave_barrier();
         table_put(tab_key, l32, pk);
         rows_to_tile<T>(tile_x, lane, rk);
         rows_to_tile<T>(tile, lane, rv);
         __builtin_amdgcn_wave_barrier();
-        float ka[16];
-        tile_get_rows(tile_x, l32, half, ka);
-        // S^T tile: rows = keys, columns = queries
-        f32x16 S = mma_slots_first<T, 16>(ka, qb);
+        // the bias gathers are requested before the score product, which covers part of their latency
         uint32_t pkr[16];
         table_get(tab_key, half, pkr);
         float bv[16];
 #pragma unroll
         for (int r = 0; r < 16; ++r)
             bv[r] = *reinterpret_cast<const float*>(bias_h + (brow + (MASK ? (pkr[r] & 0xffffu) : pkr[r])));
+        float ka[16];
+        tile_get_rows(tile_x, l32, half, ka);
+        // S^T tile: rows = keys, columns = queries
+        f32x16 S = mma_slots_first<T, 16>(ka, qb);
         float vb[16];
         tile_get_cols(tile, l32, half, vb);                  // V[key acc_row(r, half)][channel l32]
 
@@ -513,9 +523,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         else
             mma_slots<T, 0, 16>(S, vb, o);
     };
-    tile_step(std::true_type{}, 0);
+    tile_step(std::true_type{}, 0, kcur);
 #pragma unroll 1
-    for (int t = 1; t < nt; ++t) tile_step(std::false_type{}, t);
+    for (int t = 1; t < nt; ++t) {
+        kcur = load_kidx(t);
+        rows_load<T>(kbase, kpitch, kcur.vox, lane, rk);
+        rows_load<T>(vbase, vpitch, kcur.vox, lane, rv);
+        tile_step(std::false_type{}, t, kcur);
+    }
     l += __shfl_xor(l, 32, 64);
     l += 1e-8f;
     if (half == 0 && i_q < c) lse[(int64_t)a.H * g.Tk + h * c + i_q] = (m + __builtin_amdgcn_logf(l)) * LN2;
@@ -563,6 +578,10 @@ __device__ __forceinline__ void bwd_q_task(const WAttnCommon& a, int64_t task, f
     const int i_c = i_q < c ? i_q : c - 1;
     const uint32_t vox_i = order[i_c];
     const int pos_i = tok_pos[i_c];
+    // indices of the first key tile: requested in the same round trip as the query indices
+    int jn_c = l32 < c ? l32 : c - 1;
+    uint32_t vox_n = order[jn_c];
+    int pos_n = tok_pos[jn_c];
     const int reg_i = MASK ? mrow[pos_i] : 0;
     const float L2 = lse[(int64_t)a.H * g.Tk + h * c + i_c] * LOG2E;
     float qb[16], dob[16];
@@ -590,15 +609,19 @@ __device__ __forceinline__ void bwd_q_task(const WAttnCommon& a, int64_t task, f
     f32x16 dq = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll 1
     for (int t = 0; t < nt; ++t) {
-        const int j = t * 32 + l32;
-        const int j_c = j < c ? j : c - 1;
-        const uint32_t vox_j = order[j_c];
-        const int pos_j = tok_pos[j_c];
+        const uint32_t vox_j = vox_n;
+        const int pos_j = pos_n;
         RowLoad<T> rk, rv;
         rows_load<T>(kbase, kpitch, vox_j, lane, rk);
         rows_load<T>(vbase, vpitch, vox_j, lane, rv);
         uint32_t pk = (uint32_t)pos_j * 4u;
         if (MASK) pk |= (uint32_t)mrow[pos_j] << 16;
+        {                                                    // indices of the next key tile, a tile ahead
+            const int j = (t + 1) * 32 + l32;
+            jn_c = j < c ? j : c - 1;
+            vox_n = order[jn_c];
+            pos_n = tok_pos[jn_c];
+        }
         __builtin_amdgcn_wave_barrier();
         table_put(tab_key, l32, pk);
         rows_to_tile<T>(tile, lane, rk);                     // K rows, read back by column for dQ
@@ -666,16 +689,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 enum { KV_ONLY = 0, KV_SINGLE = 1, KV_PAIR = 2 };
 
 // xch: this wavefront's exchange tile (KV_PAIR), xch_peer: the other wavefront's; accumulator layout
+// (piece q of lane l at 16-byte slot q*64 + l: neighbouring lanes touch neighbouring slots)
 __device__ __forceinline__ void xch_put(float* xch, int lane, const f32x16& v) {
-    f32x4_a* p = reinterpret_cast<f32x4_a*>(xch + lane * 16);
+    f32x4_a* p = reinterpret_cast<f32x4_a*>(xch) + lane;
 #pragma unroll
-    for (int q = 0; q < 4; ++q) p[q] = f32x4_a{v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]};
+    for (int q = 0; q < 4; ++q) p[q * 64] = f32x4_a{v[4 * q], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3]};
 }
 __device__ __forceinline__ void xch_add(const float* xch, int lane, f32x16& v) {
-    const f32x4_a* p = reinterpret_cast<const f32x4_a*>(xch + lane * 16);
+    const f32x4_a* p = reinterpret_cast<const f32x4_a*>(xch) + lane;
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
-        const f32x4_a t = p[q];
+        const f32x4_a t = p[q * 64];
         v[4 * q] += t.x; v[4 * q + 1] += t.y; v[4 * q + 2] += t.z; v[4 * q + 3] += t.w;
     }
 }

@@ -58,29 +58,37 @@ def box_surfaces_scene(seed: int = 1, grid=(128, 128, 128), n_boxes: int = 8):
     return c.astype(np.int32)
 
 
-def room_scene(seed: int = 2, grid=(256, 256, 96), footprint=(168, 152), wall_height=56,
-               n_furniture: int = 20):
+def room_scene(seed: int = 2, grid=(256, 256, 96), footprint=(168, 152), wall_height=52,
+               n_furniture: int = 20, rough: float = 0.5):
     """A ScanNet-like room voxelised on ``grid`` = (x, y, z) extents, z up.
 
-    Floor plane, four walls and ``n_furniture`` random box surfaces standing on the
-    floor.  Returned coordinates are int32 ``[N, 3]`` ordered (d, h, w) = (x, y, z)
-    in a seeded random order.
+    Floor, four walls and ``n_furniture`` random box surfaces standing on the floor.  The floor
+    and the walls are rough, as scanned surfaces are: a fraction ``rough`` of their voxels sits one
+    voxel further along the surface normal, and the two levels straddle a boundary of the
+    ``floor(coord / 2)`` grid, so that down-sampling keeps about 1/3 of the voxels (a perfectly
+    flat one-voxel sheet would keep 1/4).  Returned coordinates are int32 ``[N, 3]`` ordered
+    (d, h, w) = (x, y, z) in a seeded random order.
     """
     rng = np.random.default_rng(seed)
+    jit = np.random.default_rng(seed + 1000)          # roughness: its own stream, the furniture layout does not move
     gx, gy, gz = grid
     fx, fy = footprint
     ox, oy = (gx - fx) // 2, (gy - fy) // 2
     parts = []
-    # floor
+
+    def level(size):
+        return (jit.random(size) < rough).astype(np.int64)
+
+    # floor at z = 1 or 2
     xx, yy = np.meshgrid(np.arange(ox, ox + fx), np.arange(oy, oy + fy), indexing="ij")
-    parts.append(np.stack([xx.ravel(), yy.ravel(), np.zeros(xx.size, np.int64)], 1))
-    # walls
-    for x in (ox, ox + fx - 1):
+    parts.append(np.stack([xx.ravel(), yy.ravel(), 1 + level(xx.size)], 1))
+    # walls, displaced outwards
+    for x, sign in ((ox, -1), (ox + fx - 1, 1)):
         yy, zz = np.meshgrid(np.arange(oy, oy + fy), np.arange(wall_height), indexing="ij")
-        parts.append(np.stack([np.full(yy.size, x), yy.ravel(), zz.ravel()], 1))
-    for y in (oy, oy + fy - 1):
+        parts.append(np.stack([x + sign * level(yy.size), yy.ravel(), zz.ravel()], 1))
+    for y, sign in ((oy, -1), (oy + fy - 1, 1)):
         xx, zz = np.meshgrid(np.arange(ox, ox + fx), np.arange(wall_height), indexing="ij")
-        parts.append(np.stack([xx.ravel(), np.full(xx.size, y), zz.ravel()], 1))
+        parts.append(np.stack([xx.ravel(), y + sign * level(xx.size), zz.ravel()], 1))
     # furniture: boxes standing on the floor
     for _ in range(n_furniture):
         sx, sy = rng.integers(10, 36, size=2)
@@ -100,6 +108,21 @@ def filled_blob_scene(seed: int = 4, grid=(32, 32, 12), fill: float = 0.9):
     c = np.stack([zz.ravel(), yy.ravel(), xx.ravel()], 1)
     keep = rng.random(len(c)) < fill
     c = c[keep]
+    c = c[rng.permutation(len(c))]
+    return c.astype(np.int32)
+
+
+def volumetric_scene(seed: int = 4, coarse=(30, 30, 10), levels: int = 3, fill: float = 0.9, density: float = 0.5):
+    """A volumetric scene on the fine grid ``coarse * 2**levels``: a fraction ``fill`` of the cells of the
+    coarse grid is solid, and a solid cell holds a fraction ``density`` of its fine voxels (at least one).
+    ``levels`` passes of :func:`downsample_coords` give back exactly the solid coarse cells."""
+    rng = np.random.default_rng(seed)
+    f = 2 ** levels
+    solid = rng.random(coarse) < fill
+    fine = np.repeat(np.repeat(np.repeat(solid, f, 0), f, 1), f, 2) & (rng.random(tuple(g * f for g in coarse)) < density)
+    # every solid cell keeps at least its first fine voxel
+    fine[::f, ::f, ::f] |= solid
+    c = np.argwhere(fine)
     c = c[rng.permutation(len(c))]
     return c.astype(np.int32)
 
@@ -270,8 +293,11 @@ def config3():
 
 
 def config4():
-    # volumetric fill so that most windows hold 100-125 tokens
-    c = filled_blob_scene(seed=4, grid=(30, 30, 10), fill=0.9)
+    # a volumetric scene of about two million voxels on a 240 x 240 x 80 grid, down-sampled by floor(coord / 2)
+    # three times: about 8k voxels, most windows hold 100-125 tokens
+    c = volumetric_scene(seed=4, coarse=(30, 30, 10), levels=3, fill=0.9)
+    for _ in range(3):
+        c, _ = downsample_coords(c, 2)
     c4, _ = with_batch([c])
     return Workload("cfg4_dense8k", c4, (30, 30, 10), 1, 768, 24, dtype="bf16")
 
