@@ -170,16 +170,17 @@ def kernel_table(wl, reps=20, only=None):
 
     entries = [
         # name, callable, algorithmic bytes, calls per attention fwd+bwd
-        ("qkv_sparse_indices", lambda: ops.qkv_sparse_indices(b["idx"], b["slots"], b["n"], H, hd), 8 * N + 40 * E, 1),
+        ("qkv_sparse_indices", lambda: ops.qkv_sparse_indices(b["idx"], b["slots"], b["n"], H, hd, _defer_check=True), 8 * N + 40 * E, 1),
         ("plan_from_indices", lambda: _lib.check(lib.sswin_plan_from_indices(ptr(q.indices), m, hd, ptr(plan), g_cap, totals, ptr(ws), nb, stream)), 0, 2),
         ("block_matmul q_k", mm(0, q.values, kt.values, q.indices, out_s, out_si, A), 2 * s * E + (s + 16) * A + 4 * G, 1),
         ("flatten_indices [3,A]", lambda: ops.flatten_indices(s_idx[:3], s_shape[:3]), 16 * A, 1),
         ("unique_consecutive_indices [A]", lambda: ops.unique_consecutive_indices(flat), 8 * A, 1),
         ("softmax_last_dim_forward", lambda: ops.softmax_last_dim_forward(rows, s_val), 12 * A, 1),
         ("block_matmul qk_v", mm(1, p_val, v.values, v.indices, out_o, out_oi, E), s * A + s * E + (s + 16) * E + 4 * G, 1),
-        ("flatten_indices [4,E] (permute)", lambda: ops.flatten_indices(perm_idx, [o_shape[0], o_shape[2], o_shape[1], o_shape[3]]), 0, 1),
-        ("sort_indices [E] (permute)", lambda: ops.sort_indices(flat_perm), 0, 1),
-        ("return_inverse [N]", lambda: ops.return_inverse(flat_tok, -1), 0, 1),
+        ("permute order from the group structure [E]", lambda: ops.permute_heads_order(o_idx, o_shape), 0, 1),
+        ("flatten_indices [4,E] (generic permute)", lambda: ops.flatten_indices(perm_idx, [o_shape[0], o_shape[2], o_shape[1], o_shape[3]]), 0, 0),
+        ("sort_indices [E] (generic permute)", lambda: ops.sort_indices(flat_perm), 0, 0),
+        ("return_inverse [N]", lambda: ops.return_inverse(flat_tok, b["slots"] * b["n"]), 0, 1),
         ("softmax_last_dim_backward", lambda: ops.softmax_last_dim_backward(rows, p_val, g_s), 16 * A, 1),
         ("grad rc_cr", grad(0, g_o, v.values, tmp_a), 2 * s * E + s * A, 1),
         ("grad rr_rc", grad(1, g_s, kt.values, tmp_e), s * A + 2 * s * E, 2),

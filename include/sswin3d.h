@@ -89,13 +89,16 @@ int sswin_return_inverse(const int32_t* x, int64_t M, int64_t maxnum, int32_t* o
  * {B,H,n,hd} and {B,H,hd,n}).  E = N*H*hd.  (window, pos) pairs must be distinct,
  * window in [0,B), pos in [0,n).  The ordering is that of the exact (non-wrapping) hash.
  * Pairs outside that range, or a pair that occurs twice, never turn into a device address: the
- * kernels that would use them leave sorted_qv / sorted_k unwritten.  validate != 0 waits for the
- * stream and reports such input as an error; validate == 0 stays asynchronous and silent.
+ * kernels that would use them fill sorted_qv / sorted_k with zeros instead.  validate != 0 waits for the
+ * stream and reports such input as an error; validate == 0 stays asynchronous, and status_out (pinned host
+ * int32 [2], or NULL) then receives {pairs out of range, distinct pairs} once the stream has run: the input
+ * was valid iff status_out[0] == 0 and status_out[1] == N.
  * All array arguments: device. */
 size_t sswin_qkv_sparse_indices_workspace_bytes(int64_t N, int B, int n);
 int sswin_qkv_sparse_indices(const int32_t* indices, int64_t N, int B, int n, int H, int hd,
                              int32_t* idx_qv, int32_t* sorted_qv, int32_t* idx_k,
-                             int32_t* sorted_k, void* ws, size_t ws_bytes, int validate, void* stream);
+                             int32_t* sorted_k, void* ws, size_t ws_bytes, int validate, int32_t* status_out,
+                             void* stream);
 
 /* ---- per-group offsets ("plan") ----------------------------------------------------- */
 
@@ -118,6 +121,17 @@ size_t sswin_plan_workspace_bytes(int64_t M, int inner);
 int sswin_plan_from_indices(const int32_t* idx, int64_t M, int inner, int32_t* plan,
                             int64_t g_cap, int64_t* totals_out, void* ws, size_t ws_bytes,
                             void* stream);
+
+/* The order SparseTensor.permute((0, 2, 1, 3)) of sparse_swin/swin3d_base.py:47-59 arrives at by hashing the
+ * permuted indices and sorting them, for a coalesced [B, H, n, C] operand whose heads hold the same
+ * positions in every window (an attention output): perm_out[k] = position in the operand of the k-th
+ * entry of the permuted, sorted operand.  idx: its [4, M] indices; plan / g_cap / G: from
+ * sswin_plan_from_indices(idx, M, C).  C a multiple of 4; perm_out (device int32 [M]) 16-byte aligned.
+ * bad_groups (device int32 [1]) receives the number of groups that do not fit the premise (different
+ * counts or positions than the first head of their window); those groups write nothing, and the caller
+ * falls back to flatten_indices + sort_indices when it is not zero.  Asynchronous. */
+int sswin_permute_heads_order(const int32_t* idx, int64_t M, int C, const int32_t* plan, int64_t g_cap,
+                              int64_t G, int32_t* perm_out, int32_t* bad_groups, void* stream);
 
 /* Same three scans from a given `_c` (what the reference recomputes inside every
  * matmul_grad / qkv_transpose call, sparse_swin/ops.cu:681, 697, 965-968, 986-989,

@@ -26,9 +26,10 @@ SIGNATURES = {
     "sswin_return_inverse_workspace_bytes": (_sz, [_i64, _i64]),
     "sswin_return_inverse": (_i32, [_vp, _i64, _i64, _vp, _vp, _vp, _sz, _vp]),
     "sswin_qkv_sparse_indices_workspace_bytes": (_sz, [_i64, _i32, _i32]),
-    "sswin_qkv_sparse_indices": (_i32, [_vp, _i64, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _vp, _sz, _i32, _vp]),
+    "sswin_qkv_sparse_indices": (_i32, [_vp, _i64, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _vp, _sz, _i32, _vp, _vp]),
     "sswin_plan_workspace_bytes": (_sz, [_i64, _i32]),
     "sswin_plan_from_indices": (_i32, [_vp, _i64, _i32, _vp, _i64, _vp, _vp, _sz, _vp]),
+    "sswin_permute_heads_order": (_i32, [_vp, _i64, _i32, _vp, _i64, _i64, _vp, _vp, _vp]),
     "sswin_scan_counts_workspace_bytes": (_sz, [_i64]),
     "sswin_scan_counts": (_i32, [_vp, _i64, _vp, _vp, _sz, _vp]),
     "sswin_block_matmul": (_i32, [_i32, _i32, _vp, _vp, _vp, _i64, _i32, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp]),
@@ -69,7 +70,7 @@ SIGNATURES = {
                                                _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i32, _vp]),
 }
 
-ABI_VERSION = 15
+ABI_VERSION = 17
 _lib = None
 
 

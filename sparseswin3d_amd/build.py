@@ -32,6 +32,38 @@ def _hipcc() -> str:
     raise RuntimeError("hipcc not found")
 
 
+PYBIND_SRC = os.path.join(CSRC, "custom_ops_pybind.cpp")
+PYBIND_NAME = "custom_ops_pybind"
+
+
+def build_pybind(verbose: bool = False) -> str:
+    """Compile the pybind11 module with the reference's ten operator names over the C ABI
+    (``sparseswin3d_amd/custom_ops_pybind*.so``).  hipcc compiles the one host source directly against
+    PyTorch's HIP-native headers; nothing is translated."""
+    import sysconfig
+
+    import pybind11
+    import torch
+    from torch.utils import cpp_extension
+    hipcc = _hipcc()
+    out = os.path.join(HERE, PYBIND_NAME + sysconfig.get_config_var("EXT_SUFFIX"))
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    includes = [pybind11.get_include(), sysconfig.get_paths()["include"], *cpp_extension.include_paths("cuda")]
+    cmd = [hipcc, "-O2", "-std=c++17", "-fPIC", "-shared", "-x", "c++", "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           f"-DTORCH_EXTENSION_NAME={PYBIND_NAME}", "-DTORCH_API_INCLUDE_EXTENSION_H",
+           f"-D_GLIBCXX_USE_CXX11_ABI={int(torch._C._GLIBCXX_USE_CXX11_ABI)}",
+           *[f"-I{p}" for p in includes], PYBIND_SRC, "-o", out,
+           f"-L{torch_lib}", "-lc10", "-lc10_hip", "-ltorch_cpu", "-ltorch_hip", "-ltorch", "-ltorch_python",
+           f"-L{HERE}", "-lsswin3d", "-Wl,-rpath,$ORIGIN", f"-Wl,-rpath,{torch_lib}",
+           "-Wno-unused-command-line-argument"]
+    r = subprocess.run(cmd, capture_output=True, text=True)
+    if r.returncode != 0:
+        raise RuntimeError(f"hipcc failed for {PYBIND_SRC}:\n{r.stderr[-6000:]}")
+    if verbose and r.stderr.strip():
+        print(r.stderr, file=sys.stderr)
+    return out
+
+
 def build(verbose: bool = False) -> str:
     hipcc = _hipcc()
     objdir = os.path.join(HERE, "build")
@@ -58,3 +90,5 @@ def build(verbose: bool = False) -> str:
 
 if __name__ == "__main__":
     print(build(verbose="-v" in sys.argv))
+    if "--no-pybind" not in sys.argv:
+        print(build_pybind(verbose="-v" in sys.argv))

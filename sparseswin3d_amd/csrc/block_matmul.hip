@@ -221,28 +221,95 @@ __global__ __launch_bounds__(256) void block_product_simple_kernel(const T* __re
 
 // ------------------------------------------------------------------------------------------
 // per-group transposes.  rc: [c x C] -> [C x c];  rr: [c x c] -> [c x c]^T.
-// One workgroup per four groups; writes are contiguous, the strided reads stay inside the
-// group's block (at most a few tens of KB) and are served from cache.
+// One wavefront per group.  A group's block is a few KB: it is read as one contiguous run into a
+// wave-private LDS copy (odd pitch, so a column is spread over the banks) and written back as one
+// contiguous run in transposed order, so both sides of the copy are coalesced.  Blocks that do not fit
+// the LDS copy (more than TR_LDS_BYTES) are read with strides from global memory instead.
 // ------------------------------------------------------------------------------------------
+constexpr int TR_LDS_BYTES = 8192;
+
+// f / d through a multiplication, exact for f * d < 2^32 (blocks here stay below 2^14 entries); d = 1 has no
+// 32-bit multiplier and is marked by 0
+__device__ __forceinline__ uint32_t div_magic(uint32_t d) { return d == 1 ? 0u : (uint32_t)((0x100000000ull + d - 1) / d); }
+__device__ __forceinline__ int div_by(int f, uint32_t magic) { return magic ? (int)__umulhi((uint32_t)f, magic) : f; }
+
 template <typename T, bool IS_RR>
 __global__ __launch_bounds__(256) void block_transpose_kernel(const T* __restrict__ in, const int32_t* __restrict__ cs,
                                                               const int32_t* __restrict__ row_start,
                                                               const int32_t* __restrict__ sq_start, int64_t G,
                                                               int C, T* __restrict__ out) {
-    const int64_t g0 = (int64_t)blockIdx.x * GROUPS_PER_WG;
-    for (int q = 0; q < GROUPS_PER_WG; ++q) {
-        const int64_t g = g0 + q;
+    __shared__ __attribute__((aligned(16))) char lds[GROUPS_PER_WG][TR_LDS_BYTES];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    T* t = reinterpret_cast<T*>(lds[wave]);
+    constexpr int U = 8;                      // loads in flight per lane
+    constexpr int cap = TR_LDS_BYTES / (int)sizeof(T);
+    {
+        const int64_t g = (int64_t)blockIdx.x * GROUPS_PER_WG + wave;
         if (g >= G) return;
         const int c = cs[g];
         const int64_t off = IS_RR ? (int64_t)sq_start[g] : (int64_t)row_start[g] * C;
-        const int rows_out = IS_RR ? c : C;       // out is [rows_out x c]
-        const int ld_in = IS_RR ? c : C;          // in  is [c x ld_in]
-        const int count = rows_out * c;
+        const int rows = c;                   // in is [rows x cols], out is [cols x rows]
+        const int cols = IS_RR ? c : C;
         const T* src = in + off;
         T* dst = out + off;
-        for (int f = threadIdx.x; f < count; f += 256) {
-            const int i = f / c, j = f - i * c;
-            dst[f] = src[(int64_t)j * ld_in + i];
+        const uint32_t m_rows = div_magic((uint32_t)rows);
+        const int pitch = cols | 1;
+        if (rows * pitch <= cap) {
+            const int count = rows * cols;
+            const uint32_t m_cols = div_magic((uint32_t)cols);
+            for (int f0 = lane; f0 < count; f0 += 64 * U) {
+                T v[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int f = f0 + 64 * u;
+                    v[u] = src[f < count ? f : count - 1];
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int f = f0 + 64 * u;
+                    const int i = div_by(f, m_cols), j = f - i * cols;
+                    if (f < count) t[i * pitch + j] = v[u];
+                }
+            }
+            __builtin_amdgcn_wave_barrier();
+            for (int f = lane; f < count; f += 64) {
+                const int jo = div_by(f, m_rows), io = f - jo * rows;
+                dst[f] = t[io * pitch + jo];
+            }
+            return;
+        }
+        // slabs of R input columns (= R output rows), R a power of two: reads are runs of R values per input
+        // row, writes one contiguous run per slab
+        int logR = 6;
+        while (logR > 0 && rows * ((1 << logR) | 1) > cap) --logR;
+        const int R = 1 << logR, rp = R | 1;
+        for (int j0 = 0; j0 < cols; j0 += R) {
+            const int Rc = cols - j0 < R ? cols - j0 : R;
+            const int slab = rows << logR;
+            for (int e0 = lane; e0 < slab; e0 += 64 * U) {
+                T v[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int e = e0 + 64 * u;
+                    const int io = e >> logR, jr = e & (R - 1);
+                    const bool ok = e < slab && jr < Rc;
+                    v[u] = src[ok ? (int64_t)io * cols + j0 + jr : 0];
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int e = e0 + 64 * u;
+                    const int io = e >> logR, jr = e & (R - 1);
+                    if (e < slab && jr < Rc) t[io * rp + jr] = v[u];
+                }
+            }
+            __builtin_amdgcn_wave_barrier();
+            T* d = dst + (int64_t)j0 * rows;
+            const int n_out = Rc * rows;
+            for (int f = lane; f < n_out; f += 64) {
+                const int jr = div_by(f, m_rows), io = f - jr * rows;
+                d[f] = t[io * rp + jr];
+            }
+            __builtin_amdgcn_wave_barrier();
         }
     }
 }

@@ -318,7 +318,11 @@ __global__ __launch_bounds__(256) void sorted_qv_kernel(const int32_t* __restric
     const int q = hd >> 2;                                  // channel quads per head
     const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
     const int64_t total = N * H * q;
-    if (t >= total || !pairs_valid(status, N)) return;
+    if (t >= total) return;
+    if (!pairs_valid(status, N)) {                           // defined (all zero) output for a caller that checks later
+        *reinterpret_cast<int4*>(sorted_qv + t * 4) = make_int4(0, 0, 0, 0);
+        return;
+    }
     const int cq = (int)(t % q);
     const int64_t rh = t / q;
     const int h = (int)(rh % H);
@@ -338,7 +342,12 @@ __global__ __launch_bounds__(256) void sorted_k_kernel(const int32_t* __restrict
                                                        const int32_t* __restrict__ status, int64_t N,
                                                        int H, int hd, int32_t* __restrict__ sorted_k) {
     const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
-    if (r >= N || !pairs_valid(status, N)) return;
+    if (r >= N) return;
+    if (!pairs_valid(status, N)) {
+        int32_t* row = sorted_k + ((int64_t)blockIdx.y * N + r) * hd;
+        for (int ch = 0; ch < hd; ++ch) row[ch] = 0;
+        return;
+    }
     const int T = win_T[r], c = win_c[r];
     const int i = (int)(r - T);
     const int h = blockIdx.y;
@@ -357,7 +366,7 @@ using namespace sswin;
 extern "C" {
 
 const char* sswin_last_error(void) { return error_buffer(); }
-int sswin_abi_version(void) { return 15; }
+int sswin_abi_version(void) { return 17; }
 
 int sswin_flatten_indices(const int32_t* idx, int ndim, int64_t M, const int32_t* sizes, int32_t* out,
                           void* stream) {
@@ -560,7 +569,7 @@ size_t sswin_qkv_sparse_indices_workspace_bytes(int64_t N, int B, int n) {
 
 int sswin_qkv_sparse_indices(const int32_t* indices, int64_t N, int B, int n, int H, int hd,
                              int32_t* idx_qv, int32_t* sorted_qv, int32_t* idx_k, int32_t* sorted_k,
-                             void* ws, size_t ws_bytes, int validate, void* stream) {
+                             void* ws, size_t ws_bytes, int validate, int32_t* status_out, void* stream) {
     SSWIN_CHECK(N >= 0 && B > 0 && n > 0 && H > 0 && hd > 0, "qkv_sparse_indices: bad sizes");
     SSWIN_CHECK(hd % 4 == 0, "qkv_sparse_indices: head dim %d must be a multiple of 4", hd);
     const int64_t E = N * H * hd;
@@ -600,6 +609,9 @@ int sswin_qkv_sparse_indices(const int32_t* indices, int64_t N, int B, int n, in
     hipLaunchKernelGGL(sorted_k_kernel, dim3(nb, (unsigned)H), dim3(256), 0, s, order, win_T, win_c, status, N, H, hd,
                        sorted_k);
     if (launch_ok("qkv_sparse_indices")) return 1;
+    if (status_out) {                                        // the caller checks later: {out of range, distinct pairs}
+        SSWIN_HIP(hipMemcpyAsync(status_out, status, 2 * sizeof(int32_t), hipMemcpyDeviceToHost, s));
+    }
     if (validate) {
         int32_t back[2] = {0, 0};
         SSWIN_HIP(hipMemcpyAsync(back, status, sizeof(back), hipMemcpyDeviceToHost, s));

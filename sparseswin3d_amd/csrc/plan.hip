@@ -166,11 +166,65 @@ struct CountStore {
     }
 };
 
+// ------------------------------------------------------------------------------------------
+// Order of a coalesced [B, H, n, C] operand (dense last dimension) after permute (0, 2, 1, 3).
+// The reference re-hashes the permuted indices and sorts all of them (sparse_swin/swin3d_base.py:47-59).
+// When every head of a window holds the same positions - what an attention output does - the
+// sorted order follows from the plan: row i of head number r of a window that starts at row R0
+// and has Hw heads of c rows each goes to row R0 + i*Hw + r.  One wavefront per group writes its
+// rows' entries and checks the premise (equal counts, equal positions as the window's first head);
+// a group that fails it is counted in *bad and writes nothing.
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void permute_heads_kernel(const int32_t* __restrict__ pos_row, const int32_t* __restrict__ plan,
+                                                            int64_t g_cap, int64_t G, int C, int32_t* __restrict__ perm,
+                                                            int32_t* __restrict__ bad) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int64_t g = (int64_t)blockIdx.x * 4 + wave;
+    if (g >= G) return;
+    const int32_t* win = plan + 3 * g_cap;
+    const int c = plan[g], rs = plan[g_cap + g], w = win[g];
+    int64_t g0 = g, g1 = g;                                   // the window's groups are g0 .. g1
+    while (g0 > 0 && win[g0 - 1] == w) --g0;
+    while (g1 + 1 < G && win[g1 + 1] == w) ++g1;
+    const int heads = (int)(g1 - g0 + 1), r = (int)(g - g0);
+    const int rs0 = plan[g_cap + g0];
+    bool ok = plan[g0] == c && rs == rs0 + r * c;
+    if (ok && r > 0)
+        for (int i = lane; i < c; i += 64) ok = ok && pos_row[(int64_t)(rs + i) * C] == pos_row[(int64_t)(rs0 + i) * C];
+    if (!__all(ok)) {
+        if (lane == 0) atomicAdd(bad, 1);
+        return;
+    }
+    const int q = C >> 2;                                     // 16-byte pieces per row
+    for (int t = lane; t < c * q; t += 64) {
+        const int i = t / q, cq = t - i * q;
+        const int src = (rs + i) * C + 4 * cq;
+        const int64_t dst = (int64_t)(rs0 + i * heads + r) * C + 4 * cq;
+        *reinterpret_cast<int4*>(perm + dst) = make_int4(src, src + 1, src + 2, src + 3);
+    }
+}
+
 }  // namespace sswin
 
 using namespace sswin;
 
 extern "C" {
+
+int sswin_permute_heads_order(const int32_t* idx, int64_t M, int C, const int32_t* plan, int64_t g_cap, int64_t G,
+                              int32_t* perm_out, int32_t* bad_groups, void* stream) {
+    SSWIN_CHECK(C > 0 && C % 4 == 0 && M >= 0 && M % C == 0, "permute_heads_order: bad sizes");
+    SSWIN_CHECK(M < (int64_t)INT32_MAX, "permute_heads_order: too many entries for int32 positions");
+    SSWIN_CHECK(G >= 0 && G <= g_cap, "permute_heads_order: bad group count");
+    SSWIN_CHECK(bad_groups, "permute_heads_order: null pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    hipLaunchKernelGGL(zero_i32_kernel, dim3(1), dim3(64), 0, s, bad_groups, 1);
+    if (G == 0 || M == 0) return launch_ok("permute_heads_order");
+    SSWIN_CHECK(idx && plan && perm_out, "permute_heads_order: null pointer");
+    SSWIN_CHECK(((uintptr_t)perm_out % 16) == 0, "permute_heads_order: perm_out is not 16-byte aligned");
+    hipLaunchKernelGGL(permute_heads_kernel, dim3((unsigned)((G + 3) / 4)), dim3(256), 0, s, idx + 2 * M, plan, g_cap, G, C,
+                       perm_out, bad_groups);
+    return launch_ok("permute_heads_order");
+}
 
 size_t sswin_plan_workspace_bytes(int64_t M, int inner) {
     const int64_t R = inner > 0 ? M / inner : 0;

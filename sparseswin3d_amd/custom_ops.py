@@ -13,6 +13,7 @@ Use in the reference's ``swin3d_base.py`` by replacing its JIT ``load(...)`` cal
 from __future__ import annotations
 
 import ctypes as C
+import weakref
 from collections import OrderedDict
 
 import torch
@@ -131,10 +132,37 @@ def return_inverse(x, maxnum=-1):
     with torch.cuda.device(d):
         _lib.check(lib.sswin_return_inverse(_ptr(x), m, maxnum, _ptr(out), C.byref(count), _ptr(ws), nbytes,
                                             _stream(d)))
+        _check_pending()
     return out, int(count.value)
 
 
-def qkv_sparse_indices(indices, batch_size, spatial_dim, num_heads, c):
+# Input checks whose verdict is still on its way from the GPU: (event, pinned status, voxel count).  An
+# operator that has just waited for the stream anyway looks at them (:func:`_check_pending`).
+_pending = []
+
+
+def _check_pending(wait=False):
+    """Raise for a deferred :func:`qkv_sparse_indices` check whose status has arrived (all of them after
+    ``wait=True`` or after the caller has synchronised the stream)."""
+    keep = []
+    bad = None
+    for event, status, n_vox in _pending:
+        if not (wait or event.query()):
+            keep.append((event, status, n_vox))
+            continue
+        event.synchronize()
+        out_of_range, distinct = int(status[0]), int(status[1])
+        if out_of_range:
+            bad = (f"qkv_sparse_indices: {out_of_range} voxel indices lie outside [0, batch_size) x [0, spatial_dim)")
+        elif distinct != n_vox:
+            bad = (f"qkv_sparse_indices: (window, pos) pairs must be distinct: {n_vox - distinct} voxels share a "
+                   "pair with another")
+    _pending[:] = keep
+    if bad:
+        raise RuntimeError(bad)
+
+
+def qkv_sparse_indices(indices, batch_size, spatial_dim, num_heads, c, _defer_check=False):
     """Element-level COO indices of Q/V and K^T plus their sorting permutations (ops.cu:293-335)."""
     lib = _lib.load()
     d = _dev(indices)
@@ -149,10 +177,21 @@ def qkv_sparse_indices(indices, batch_size, spatial_dim, num_heads, c):
     sorted_k = torch.empty(e, dtype=torch.int32, device=d)
     nbytes = lib.sswin_qkv_sparse_indices_workspace_bytes(n_vox, int(batch_size), int(spatial_dim))
     ws = _ws(nbytes, d)
+    # Indices the kernels cannot address (out of range, repeated pairs) are reported as an error: at once,
+    # or, with _defer_check (what qkv_sparse_cuda passes), by the next operator that waits for the stream;
+    # until then the two permutations of such input are all zero, so nothing reads out of bounds.
+    status = torch.zeros(2, dtype=torch.int32, pin_memory=True) if _defer_check else None
     with torch.cuda.device(d):
+        _check_pending()
         _lib.check(lib.sswin_qkv_sparse_indices(_ptr(indices), n_vox, int(batch_size), int(spatial_dim),
                                                 int(num_heads), int(c), _ptr(idx_qv), _ptr(sorted_qv),
-                                                _ptr(idx_k), _ptr(sorted_k), _ptr(ws), nbytes, 1, _stream(d)))
+                                                _ptr(idx_k), _ptr(sorted_k), _ptr(ws), nbytes,
+                                                0 if _defer_check else 1,
+                                                C.c_void_p(status.data_ptr()) if _defer_check else None, _stream(d)))
+        if _defer_check and n_vox > 0:
+            event = torch.cuda.Event()
+            event.record(torch.cuda.current_stream(d))
+            _pending.append((event, status, n_vox))
     return idx_qv, sorted_qv, idx_k, sorted_k
 
 
@@ -194,10 +233,11 @@ _plan_cache = _PlanCache()
 class _IndexPlanCache:
     """Plans keyed by the index matrix they were derived from.  'q_k' and 'qk_v' of one forward
     pass receive the same sorted Q/V index tensor, so the second call skips the plan kernels and
-    their host synchronisation.  Entries keep the index tensor alive (its address cannot be
-    reused) and remember its version counter (in-place edits invalidate the entry)."""
+    their host synchronisation.  An entry holds only a weak reference to the index tensor: it is
+    valid while that tensor is alive (its address cannot have been handed to another tensor) and
+    unchanged (version counter), and it does not keep the [4, E] matrix in memory."""
 
-    def __init__(self, capacity=4):
+    def __init__(self, capacity=8):
         self.capacity = capacity
         self.entries = OrderedDict()
 
@@ -206,13 +246,18 @@ class _IndexPlanCache:
         return (idx.device.index, idx.data_ptr(), idx.shape[1], inner)
 
     def get(self, idx, inner):
-        hit = self.entries.get(self._key(idx, inner))
-        if hit is None or hit[0]._version != hit[1]:
+        key = self._key(idx, inner)
+        hit = self.entries.get(key)
+        if hit is None:
+            return None
+        alive = hit[0]()
+        if alive is None or alive._version != hit[1]:
+            del self.entries[key]
             return None
         return hit[2:]
 
     def put(self, idx, inner, plan, g_cap, totals):
-        self.entries[self._key(idx, inner)] = (idx, idx._version, plan, g_cap, totals)
+        self.entries[self._key(idx, inner)] = (weakref.ref(idx), idx._version, plan, g_cap, totals)
         while len(self.entries) > self.capacity:
             self.entries.popitem(last=False)
 
@@ -227,6 +272,7 @@ def clear_caches():
     """Drop cached plans (and the tensors they keep alive)."""
     _plan_cache.clear()
     _index_plan_cache.clear()
+    _pending.clear()
 
 
 def _scans_for(c, lib, d):
@@ -288,19 +334,7 @@ def matmul_cuda_naive(mat1_v, mat1_idx, mat1_shape, mat2_v, mat2_idx, mat2_shape
     rows = m // inner
     stream = _stream(d)
     with torch.cuda.device(d):
-        cached = _index_plan_cache.get(tok_idx, inner)
-        if cached is not None:
-            plan, g_cap, (g, sum_c, sum_c2, c_max) = cached
-        else:
-            g_cap = max(1, min(rows, s1[0] * s1[1]))
-            plan = torch.empty(5 * g_cap, dtype=torch.int32, device=d)
-            totals = (C.c_int64 * 4)()
-            nbytes = lib.sswin_plan_workspace_bytes(m, inner)
-            ws = _ws(nbytes, d)
-            _lib.check(lib.sswin_plan_from_indices(_ptr(tok_idx), m, inner, _ptr(plan), g_cap, totals, _ptr(ws),
-                                                   nbytes, stream))
-            g, sum_c, sum_c2, c_max = (int(totals[i]) for i in range(4))
-            _index_plan_cache.put(tok_idx, inner, plan, g_cap, (g, sum_c, sum_c2, c_max))
+        plan, g_cap, (g, sum_c, sum_c2, c_max) = _plan_of(tok_idx, inner, s1[0] * s1[1], lib, d)
         if kind == 0:
             _check(mat2_v.numel() == m, f"'q_k': mat2 holds {mat2_v.numel()} values, expected {m}")
             nnz = sum_c2
@@ -315,7 +349,53 @@ def matmul_cuda_naive(mat1_v, mat1_idx, mat1_shape, mat2_v, mat2_idx, mat2_shape
                                           _ptr(out_val), _ptr(out_idx), nnz, stream))
     c_view = plan[:g]
     _plan_cache.put(c_view, plan, g_cap, (g, sum_c, sum_c2, c_max))
+    if kind == 1:
+        # the product has the group structure of V (same windows, heads, rows and dense extent): a later
+        # permute of it finds the plan without another pass over its indices
+        _index_plan_cache.put(out_idx, inner, plan, g_cap, (g, sum_c, sum_c2, c_max))
     return out_idx, out_val, out_shape, c_view
+
+
+def _plan_of(idx, inner, batch_heads, lib, d):
+    """Plan of a coalesced [4, M] index matrix with dense last dimension ``inner`` (cached)."""
+    cached = _index_plan_cache.get(idx, inner)
+    if cached is not None:
+        return cached
+    m = idx.shape[1]
+    g_cap = max(1, min(m // inner, batch_heads))
+    plan = torch.empty(5 * g_cap, dtype=torch.int32, device=d)
+    totals = (C.c_int64 * 4)()
+    nbytes = lib.sswin_plan_workspace_bytes(m, inner)
+    ws = _ws(nbytes, d)
+    _lib.check(lib.sswin_plan_from_indices(_ptr(idx), m, inner, _ptr(plan), g_cap, totals, _ptr(ws), nbytes, _stream(d)))
+    _check_pending()                                  # the stream has just been waited for
+    out = (plan, g_cap, tuple(int(totals[i]) for i in range(4)))
+    _index_plan_cache.put(idx, inner, *out)
+    return out
+
+
+def permute_heads_order(indices, shape):
+    """Order of a coalesced [B, H, n, C] COO operand after ``permute((0, 2, 1, 3))`` (what
+    ``sort_indices(flatten_indices(indices[[0, 2, 1, 3]], ...))`` returns), derived from the group
+    structure without a sort; ``None`` if the heads of some window do not hold the same positions
+    (the caller then sorts).  Not an operator of the reference's module: a helper of
+    :meth:`SparseTensor.permute`."""
+    lib = _lib.load()
+    d = _dev(indices)
+    inner = int(shape[3])
+    m = indices.shape[1]
+    if indices.dtype != torch.int32 or inner % 4 or m == 0 or m % inner or not indices.is_contiguous():
+        return None
+    with torch.cuda.device(d):
+        plan, g_cap, (g, _, _, _) = _plan_of(indices, inner, int(shape[0]) * int(shape[1]), lib, d)
+        order = torch.empty(m, dtype=torch.int32, device=d)
+        bad = torch.empty(1, dtype=torch.int32, device=d)
+        _lib.check(lib.sswin_permute_heads_order(_ptr(indices), m, inner, _ptr(plan), g_cap, g, _ptr(order), _ptr(bad),
+                                                 _stream(d)))
+        if int(bad.item()) != 0:
+            return None
+        _check_pending()
+    return order
 
 
 def matmul_grad_cuda_naive(mat1_v, mat2_v, _c, C_, mul_type):

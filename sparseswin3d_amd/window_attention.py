@@ -84,7 +84,13 @@ class SparseTensor:
             raise ValueError(f"dims {dims} must be a permutation of the dimensions [0, {len(self.shape) - 1}].")
         new_shape = [self.shape[d] for d in dims]
         new_indices = self.indices[list(dims), :]
-        order = self._sorted_order(new_indices, new_shape)
+        order = None
+        if tuple(dims) == (0, 2, 1, 3) and self.indices.is_cuda:
+            # an attention output: every head of a window holds the same rows, so the sorted order of the
+            # permuted indices follows from the group structure (checked on the device); no hash, no sort
+            order = ops.permute_heads_order(self.indices, self.shape)
+        if order is None:
+            order = self._sorted_order(new_indices, new_shape)
         return SparseTensor(new_indices.index_select(1, order), self.values.index_select(0, order), new_shape)
 
     def __mul__(self, other):
@@ -178,7 +184,7 @@ def qkv_sparse_cuda(qkv: torch.Tensor, indices: torch.Tensor, batch_size: int, s
     """Sorted COO operands Q [B,H,n,hd], K^T [B,H,hd,n], V [B,H,n,hd] from ``qkv`` [N,3,H,hd]."""
     num_heads, c = qkv.shape[2:]
     n = spatial_shape
-    idx_qv, order_qv, idx_k, order_k = ops.qkv_sparse_indices(indices, batch_size, n, num_heads, c)
+    idx_qv, order_qv, idx_k, order_k = ops.qkv_sparse_indices(indices, batch_size, n, num_heads, c, _defer_check=True)
     idx_qv = idx_qv.index_select(1, order_qv)
     idx_k = idx_k.index_select(1, order_k)
     q = SparseTensor(idx_qv, qkv[:, 0].reshape(-1).index_select(0, order_qv), [batch_size, num_heads, n, c])
@@ -521,6 +527,7 @@ class WindowAttentionSparse(nn.Module):
             attn = sp_add_mask(attn, mask)
         attn = softmax_last_dim(attn)
         out = spspmm_block_naive(attn, v, "qk_v").permute((0, 2, 1, 3))      # (window, pos, head, ch)
-        unsort = ops.return_inverse(ops.flatten_indices(x.indices.T.contiguous(), [b, n]), -1)[0]
+        # the keys are below b * n: passing that bound spares return_inverse its search for the maximum
+        unsort = ops.return_inverse(ops.flatten_indices(x.indices.T.contiguous(), [b, n]), b * n)[0]
         x = replace_feature(x, out.values.reshape(x.features.shape).index_select(0, unsort))
         return replace_feature(x, self.proj_drop(tall_linear(x.features, self.proj)))

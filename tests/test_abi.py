@@ -60,3 +60,18 @@ def test_product_does_not_import_the_oracle():
                 text = open(os.path.join(dirpath, f)).read()
                 assert not re.search(r"^\s*(from|import)\s+oracle\b", text, flags=re.M), f"{f} imports the oracle"
                 assert "liboracle" not in text and "cpu_path" not in text, f"{f} reaches into oracle/"
+
+
+def test_pybind_module_exports_the_ten_reference_names_and_refuses_cpu_tensors():
+    """The pybind11 build (reference boundary sparse_swin/ops.cpp:7-18) imports without a GPU."""
+    import pytest
+    import torch
+    from sparseswin3d_amd import custom_ops_pybind as pb
+    names = ["matmul_cuda_naive", "matmul_grad_cuda_naive", "qkv_sparse_indices", "flatten_indices", "sort_indices",
+             "return_inverse", "unique_consecutive_indices", "softmax_last_dim_forward", "softmax_last_dim_backward",
+             "qkv_transpose"]
+    assert sorted(n for n in dir(pb) if not n.startswith("_")) == sorted(names)
+    with pytest.raises(RuntimeError, match="no CPU fallback"):
+        pb.sort_indices(torch.zeros(3, dtype=torch.int32))
+    with pytest.raises(RuntimeError, match="Invalid mul_type"):
+        pb.qkv_transpose(torch.zeros(3), torch.zeros(1, dtype=torch.int32), 4, "cc")

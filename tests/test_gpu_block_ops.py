@@ -237,3 +237,41 @@ def test_empty_operands(ops):
     idx, val, shape, c = ops.matmul_cuda_naive(e_val, e_idx, [4, 2, 125, 32], e_val, e_idx, [4, 2, 32, 125], "q_k")
     assert idx.shape == (4, 0) and val.numel() == 0 and c.numel() == 0 and shape == [4, 2, 125, 125]
     assert ops.softmax_last_dim_forward(torch.empty(0, dtype=torch.int32, device="cuda"), e_val).numel() == 0
+
+
+@pytest.mark.parametrize("mix", sorted(MIXES))
+@pytest.mark.parametrize("H,hd", [(3, 32), (2, 16), (1, 64)])
+def test_permute_of_an_attention_output_without_a_sort(ops, oracle, mix, H, hd):
+    """SparseTensor.permute((0, 2, 1, 3)) (reference swin3d_base.py:47-59) on a 'qk_v' product: the order
+    derived from the group structure equals the stable sort of the permuted hash, bit for bit."""
+    from sparseswin3d_amd.window_attention import SparseTensor
+    B, n, d = build(oracle, mix, H, hd, seed_of("permute", mix, H, hd))
+    idx = dev(d["qi"])                                       # coalesced (window, head, pos, channel)
+    val = dev(np.arange(idx.shape[1], dtype=np.float32))
+    shape = [B, H, n, hd]
+    order = ops.permute_heads_order(idx, shape)
+    assert order is not None
+    perm = d["qi"][[0, 2, 1, 3]]
+    want = oracle.sort_indices(oracle.flatten_indices(np.ascontiguousarray(perm), [B, n, H, hd]))
+    np.testing.assert_array_equal(host(order), want)
+    out = SparseTensor(idx, val, shape).permute((0, 2, 1, 3))
+    np.testing.assert_array_equal(host(out.indices), perm[:, want])
+    np.testing.assert_array_equal(host(out.values), want.astype(np.float64))
+    assert out.shape == [B, n, H, hd]
+
+
+def test_permute_falls_back_to_the_sort_when_heads_differ(ops, oracle):
+    """Heads of one window with different positions: the structure check fails on the device and permute
+    sorts, as the reference always does."""
+    from sparseswin3d_amd.window_attention import SparseTensor
+    # window 0: head 0 holds positions {1, 4}, head 1 holds {1, 5}; window 2: one head only
+    rows = [(0, 0, 1), (0, 0, 4), (0, 1, 1), (0, 1, 5), (2, 0, 3)]
+    hd = 4
+    idx = np.array([[w, h, p, ch] for (w, h, p) in rows for ch in range(hd)], np.int32).T.copy()
+    shape = [3, 2, 8, hd]
+    assert ops.permute_heads_order(dev(idx), shape) is None
+    out = SparseTensor(dev(idx), dev(np.arange(idx.shape[1], dtype=np.float32)), shape).permute((0, 2, 1, 3))
+    perm = idx[[0, 2, 1, 3]]
+    want = oracle.sort_indices(oracle.flatten_indices(np.ascontiguousarray(perm), [3, 8, 2, hd]))
+    np.testing.assert_array_equal(host(out.indices), perm[:, want])
+    np.testing.assert_array_equal(host(out.values), want.astype(np.float64))

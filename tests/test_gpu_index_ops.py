@@ -141,6 +141,14 @@ def test_index_ops_report_indices_they_cannot_address(ops):
     x[77] = -2
     with pytest.raises(RuntimeError, match="outside"):
         ops.return_inverse(dev(x), 500)
+    # through qkv_sparse_cuda the check is deferred: the next operator that waits for the stream raises
+    from sparseswin3d_amd.window_attention import qkv_sparse_cuda, spspmm_block_naive
+    ind = np.concatenate([good[:300], good[5:6], good[300:]])
+    qkv = torch.randn(len(ind), 3, H, hd, device="cuda")
+    q, k_t, v = qkv_sparse_cuda(qkv, dev(ind), B, n)
+    with pytest.raises(RuntimeError, match="distinct"):
+        spspmm_block_naive(q, k_t, "q_k")
+    ops.clear_caches()
     got = ops.qkv_sparse_indices(dev(good), B, n, H, hd)            # and the library still works afterwards
     assert got[1].numel() == 700 * H * hd
 
