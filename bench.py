@@ -35,19 +35,35 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0
 
-# HBM bytes per launch measured with rocprofv3 --pmc (FETCH_SIZE, WRITE_SIZE) for the kernels
-# below on this workload; None = not measured.  Source summaries live in profiles/.
-MEASURED_TRAFFIC_BYTES = {
-    # profiles/wattn_kernels_cfg2_pmc.txt and profiles/fused_tok_kernel_cfg2_pmc.txt:
-    # FETCH_SIZE x 2.0 KiB + WRITE_SIZE x 1.0 KiB per launch
-    "resident forward": 174.2e6,
-    "resident backward (dQ,dK,dV,dS)": 490.7e6,
-    "resident backward dQ, all groups": 258.0e6,
-    "resident backward dK,dV,dS only": 344.5e6,
-    "fused dV=P^T dO": 128.1e6,
-    "fused dK=dS^T Q": 128.1e6,      # same kernel instantiation and operand shapes as dV
-    "fused O=PV": 135.4e6,
-}
+CALIBRATION_BYTES = 256 * 1024 * 1024      # size of the plain copy a profiling run launches beside the kernels
+MFMA_PEAK_TFLOPS = {"f32": 157.3, "bf16": 2500.0, "f16": 2500.0}      # dense, MI355X
+TRAFFIC_JSON = os.path.join(ROOT, "profiles", "traffic.json")
+
+
+def source_digest(rel_paths):
+    """sha256 over the named source files: a traffic figure is valid for the sources it was measured on."""
+    import hashlib
+    h = hashlib.sha256()
+    for rel in sorted(rel_paths):
+        with open(os.path.join(ROOT, rel), "rb") as f:
+            h.update(f.read())
+    return h.hexdigest()[:16]
+
+
+def measured_traffic(workload, kernel):
+    """HBM bytes per launch of `kernel` on `workload` as rocprofv3 --pmc measured them (FETCH_SIZE, WRITE_SIZE,
+    scaled by a calibration copy; written by --pmc-summary into profiles/traffic.json), or None with the
+    reason: not measured, or measured on other kernel sources than the ones in the tree."""
+    try:
+        with open(TRAFFIC_JSON) as f:
+            rec = json.load(f).get(workload, {}).get(kernel)
+    except FileNotFoundError:
+        rec = None
+    if rec is None:
+        return None, "not measured"
+    if source_digest(rec["sources"]) != rec["digest"]:
+        return None, f"stale: {', '.join(rec['sources'])} changed since {rec['summary']} was taken"
+    return rec["bytes"], rec["summary"]
 
 
 def log(*a):
@@ -110,122 +126,156 @@ def event_time_ms(fn, reps, warmup=2):
     return start.elapsed_time(stop) / reps
 
 
+DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+# table name of a kernel -> (substring of its symbol in a rocprofv3 trace, source files it is built from)
+KERNEL_SYMBOLS = {
+    "resident forward": ("wattn_fwd_kernel", ["sparseswin3d_amd/csrc/window_attention.hip"]),
+    "resident backward (dQ,dK,dV,dS)": ("wattn_bwd_all_kernel", ["sparseswin3d_amd/csrc/window_attention.hip"]),
+    "block_matmul q_k": ("block_product_mfma_kernel<float, 0", ["sparseswin3d_amd/csrc/block_matmul.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
+    "block_matmul qk_v": ("block_product_mfma_kernel<float, 1", ["sparseswin3d_amd/csrc/block_matmul.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
+    "grad rc_cr": ("block_product_mfma_kernel<float, 2", ["sparseswin3d_amd/csrc/block_matmul.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
+    "grad rr_rc": ("block_product_mfma_kernel<float, 3", ["sparseswin3d_amd/csrc/block_matmul.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
+    "grad cr_rr": ("block_product_mfma_kernel<float, 4", ["sparseswin3d_amd/csrc/block_matmul.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
+    "transpose rc": ("block_transpose_kernel<float, false", ["sparseswin3d_amd/csrc/block_matmul.hip"]),
+    "transpose rr": ("block_transpose_kernel<float, true", ["sparseswin3d_amd/csrc/block_matmul.hip"]),
+    "softmax_last_dim_forward": ("softmax_rows_kernel<float, false", ["sparseswin3d_amd/csrc/softmax.hip"]),
+    "softmax_last_dim_backward": ("softmax_rows_kernel<float, true", ["sparseswin3d_amd/csrc/softmax.hip"]),
+    "fused dV=P^T dO": ("fused_tok_kernel", ["sparseswin3d_amd/csrc/fused_attention.hip"]),
+    "fused O=PV": ("fused_tok_kernel", ["sparseswin3d_amd/csrc/fused_attention.hip"]),
+}
+
+
 def kernel_table(wl, reps=20, only=None):
-    """Time every operator's kernels alone on the first block's tensors (regular windows)."""
-    from sparseswin3d_amd import _lib, custom_ops as ops
-    from sparseswin3d_amd.window_attention import qkv_sparse_cuda
+    """Time every operator's kernels alone on the first block's tensors (regular windows).  The operator
+    and fused paths are timed for fp32 tokens only; the window-resident kernels in the workload's dtype."""
+    from sparseswin3d_amd import _lib, custom_ops as ops, fused as F
+    from sparseswin3d_amd.window_attention import qkv_sparse_cuda, relative_position_index_3d
     lib = _lib.load()
     b = wl["blocks"][0]
     H, D = wl["heads"], wl["dim"]
     hd = D // H
     N = wl["N"]
     dev = wl["feats"].device
+    tdt = wl["dtype"]
+    code = DTYPE_CODE[tdt]
+    es = 2 if code else 4                                    # bytes per token value
     stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
-    ptr = lambda t: C.c_void_p(t.data_ptr())
-
-    qkv = torch.randn(N, 3, H, hd, device=dev)
-    q, kt, v = qkv_sparse_cuda(qkv, b["idx"], b["slots"], b["n"])
-    s_idx, s_val, s_shape, c = ops.matmul_cuda_naive(q.values, q.indices, q.shape, kt.values, kt.indices, kt.shape, "q_k")
-    flat = ops.flatten_indices(s_idx[:3], s_shape[:3])
-    rows = ops.unique_consecutive_indices(flat)
-    p_val = ops.softmax_last_dim_forward(rows, s_val)
-    o_idx, o_val, o_shape, c2 = ops.matmul_cuda_naive(p_val, s_idx, s_shape, v.values, v.indices, v.shape, "qk_v")
-    E, A, G = q.values.numel(), s_val.numel(), c.numel()
-    s = 4
-
-    # plan once, then the product kernels alone
-    m = E
-    g_cap = max(1, min(m // hd, b["slots"] * H))
-    plan = torch.empty(5 * g_cap, dtype=torch.int32, device=dev)
-    totals = (C.c_int64 * 4)()
-    nb = lib.sswin_plan_workspace_bytes(m, hd)
-    ws = torch.empty(nb, dtype=torch.uint8, device=dev)
-    _lib.check(lib.sswin_plan_from_indices(ptr(q.indices), m, hd, ptr(plan), g_cap, totals, ptr(ws), nb, stream))
-    c_max = int(totals[3])
-    scans = torch.stack([plan.view(5, g_cap)[1, :G], plan.view(5, g_cap)[2, :G]]).reshape(-1).contiguous()
-    cc = plan[:G].contiguous()
-    out_s = torch.empty(A, device=dev)
-    out_si = torch.empty((4, A), dtype=torch.int32, device=dev)
-    out_o = torch.empty(E, device=dev)
-    out_oi = torch.empty((4, E), dtype=torch.int32, device=dev)
-    g_s = torch.randn(A, device=dev)
-    g_o = torch.randn(E, device=dev)
-
-    def mm(kind, a, bb, tok, ov, oi, nnz):
-        return lambda: _lib.check(lib.sswin_block_matmul(kind, 0, ptr(a), ptr(bb), ptr(tok), m, hd, ptr(plan), g_cap, G,
-                                                         c_max, ptr(ov), ptr(oi), nnz, stream))
-
-    def grad(kind, a, bb, out):
-        return lambda: _lib.check(lib.sswin_block_matmul_grad(kind, 0, ptr(a), ptr(bb), ptr(cc), ptr(scans), G, hd,
-                                                              ptr(out), stream))
-
-    def tr(kind, a, out):
-        return lambda: _lib.check(lib.sswin_block_transpose(kind, 0, ptr(a), ptr(cc), ptr(scans), G, hd, ptr(out), stream))
-
-    tmp_e, tmp_a = torch.empty(E, device=dev), torch.empty(A, device=dev)
-    idxT = b["idx"].T.contiguous()
-    flat_tok = ops.flatten_indices(idxT, [b["slots"], b["n"]])
-    perm_idx = o_idx[[0, 2, 1, 3], :].contiguous()
-    flat_perm = ops.flatten_indices(perm_idx, [o_shape[0], o_shape[2], o_shape[1], o_shape[3]])
-
-    entries = [
-        # name, callable, algorithmic bytes, calls per attention fwd+bwd
-        ("qkv_sparse_indices", lambda: ops.qkv_sparse_indices(b["idx"], b["slots"], b["n"], H, hd, _defer_check=True), 8 * N + 40 * E, 1),
-        ("plan_from_indices", lambda: _lib.check(lib.sswin_plan_from_indices(ptr(q.indices), m, hd, ptr(plan), g_cap, totals, ptr(ws), nb, stream)), 0, 2),
-        ("block_matmul q_k", mm(0, q.values, kt.values, q.indices, out_s, out_si, A), 2 * s * E + (s + 16) * A + 4 * G, 1),
-        ("flatten_indices [3,A]", lambda: ops.flatten_indices(s_idx[:3], s_shape[:3]), 16 * A, 1),
-        ("unique_consecutive_indices [A]", lambda: ops.unique_consecutive_indices(flat), 8 * A, 1),
-        ("softmax_last_dim_forward", lambda: ops.softmax_last_dim_forward(rows, s_val), 12 * A, 1),
-        ("block_matmul qk_v", mm(1, p_val, v.values, v.indices, out_o, out_oi, E), s * A + s * E + (s + 16) * E + 4 * G, 1),
-        ("permute order from the group structure [E]", lambda: ops.permute_heads_order(o_idx, o_shape), 0, 1),
-        ("flatten_indices [4,E] (generic permute)", lambda: ops.flatten_indices(perm_idx, [o_shape[0], o_shape[2], o_shape[1], o_shape[3]]), 0, 0),
-        ("sort_indices [E] (generic permute)", lambda: ops.sort_indices(flat_perm), 0, 0),
-        ("return_inverse [N]", lambda: ops.return_inverse(flat_tok, b["slots"] * b["n"]), 0, 1),
-        ("softmax_last_dim_backward", lambda: ops.softmax_last_dim_backward(rows, p_val, g_s), 16 * A, 1),
-        ("grad rc_cr", grad(0, g_o, v.values, tmp_a), 2 * s * E + s * A, 1),
-        ("grad rr_rc", grad(1, g_s, kt.values, tmp_e), s * A + 2 * s * E, 2),
-        ("grad cr_rr", grad(2, q.values, g_s, tmp_e), s * A + 2 * s * E, 1),
-        ("transpose rc", tr(0, q.values, tmp_e), 2 * s * E, 2),
-        ("transpose rr", tr(1, g_s, tmp_a), 2 * s * A, 2),
-    ]
-    # ---- the fused path (what WindowAttentionSparse.forward runs by default) ----
-    from sparseswin3d_amd import fused as F
-    tp = F.TokenPlan(b["idx"], b["slots"], b["n"], H)
-    qkv_c = qkv.contiguous()
-    bias = torch.randn(H, b["n"], b["n"], device=dev)
+    ptr = lambda t: C.c_void_p(t.data_ptr() if t is not None else 0)
     mask = wl["blocks"][1]["mask"]
-    s_f = torch.empty(tp.A, device=dev)
-    rows_f = torch.empty(tp.A, dtype=torch.int32, device=dev)
-    out_f = torch.empty(N, D, device=dev)
-    dqkv = torch.empty_like(qkv_c)
-    dbias = torch.zeros(H, b["n"], b["n"], device=dev)
-    dt = torch.float32
-    bg_bytes = lib.sswin_fused_bias_grad_workspace_bytes(tp.G, H, b["n"])
-    bg_ws = torch.empty(int(bg_bytes), dtype=torch.uint8, device=dev)
-    f_entries = [
-        ("fused token_plan", lambda: F.TokenPlan(b["idx"], b["slots"], b["n"], H), 28 * N + 20 * tp.G, 1),
-        ("fused S=QK^T+bias+mask", lambda: F._tokens_to_sq(tp, dt, True, qkv_c, 3 * D, 0, qkv_c, 3 * D, D, hd, 0.17, bias, mask, s_f, rows_f), 8 * E + 8 * A, 1),
-        ("fused softmax fwd", lambda: ops.softmax_last_dim_forward(rows_f, s_f), 12 * A, 1),
-        ("fused O=PV", lambda: F._sq_to_tokens(tp, dt, False, p_val, qkv_c, 3 * D, 2 * D, out_f, D, 0, hd, 1.0), 4 * A + 8 * E, 1),
-        ("fused dP=dO V^T", lambda: F._tokens_to_sq(tp, dt, False, out_f, D, 0, qkv_c, 3 * D, 2 * D, hd, 1.0, None, None, s_f, None), 8 * E + 4 * A, 1),
-        ("fused dV=P^T dO", lambda: F._sq_to_tokens(tp, dt, True, p_val, out_f, D, 0, dqkv, 3 * D, 2 * D, hd, 1.0), 4 * A + 8 * E, 1),
-        ("fused softmax bwd", lambda: ops.softmax_last_dim_backward(rows_f, p_val, g_s), 16 * A, 1),
-        ("fused dQ=dS K", lambda: F._sq_to_tokens(tp, dt, False, g_s, qkv_c, 3 * D, D, dqkv, 3 * D, 0, hd, 0.17), 4 * A + 8 * E, 1),
-        ("fused dK=dS^T Q", lambda: F._sq_to_tokens(tp, dt, True, g_s, qkv_c, 3 * D, 0, dqkv, 3 * D, D, hd, 0.17), 4 * A + 8 * E, 1),
-        ("fused bias grad", lambda: _lib.check(lib.sswin_fused_bias_grad(ptr(tp.plan), tp.g_cap, tp.G, ptr(tp.tokens), tp.N, H, b["n"], ptr(g_s), ptr(dbias), ptr(bg_ws), bg_bytes, stream)), 4 * A, 1),
-    ]
+    qkv = torch.randn(N, 3, H, hd, device=dev)
+    tp = F.TokenPlan(b["idx"], b["slots"], b["n"], H)
+    E, A, G = N * D, int(tp.A), int(tp.G)
+    sizes = dict(N=N, E=E, A=A, G=G, c_max=int(tp.c_max) if hasattr(tp, "c_max") else None)
+    entries, f_entries = [], []
 
-    # ---- the window-resident kernels (what the step runs for heads of 32 channels) ----
+    if code == 0:
+        q, kt, v = qkv_sparse_cuda(qkv, b["idx"], b["slots"], b["n"])
+        s_idx, s_val, s_shape, c = ops.matmul_cuda_naive(q.values, q.indices, q.shape, kt.values, kt.indices, kt.shape, "q_k")
+        flat = ops.flatten_indices(s_idx[:3], s_shape[:3])
+        rows = ops.unique_consecutive_indices(flat)
+        p_val = ops.softmax_last_dim_forward(rows, s_val)
+        o_idx, o_val, o_shape, c2 = ops.matmul_cuda_naive(p_val, s_idx, s_shape, v.values, v.indices, v.shape, "qk_v")
+        assert (E, A, G) == (q.values.numel(), s_val.numel(), c.numel())
+        s = 4
+
+        # plan once, then the product kernels alone
+        m = E
+        g_cap = max(1, min(m // hd, b["slots"] * H))
+        plan = torch.empty(5 * g_cap, dtype=torch.int32, device=dev)
+        totals = (C.c_int64 * 4)()
+        nb = lib.sswin_plan_workspace_bytes(m, hd)
+        ws = torch.empty(nb, dtype=torch.uint8, device=dev)
+        _lib.check(lib.sswin_plan_from_indices(ptr(q.indices), m, hd, ptr(plan), g_cap, totals, ptr(ws), nb, stream))
+        c_max = int(totals[3])
+        sizes["c_max"] = c_max
+        scans = torch.stack([plan.view(5, g_cap)[1, :G], plan.view(5, g_cap)[2, :G]]).reshape(-1).contiguous()
+        cc = plan[:G].contiguous()
+        out_s = torch.empty(A, device=dev)
+        out_si = torch.empty((4, A), dtype=torch.int32, device=dev)
+        out_o = torch.empty(E, device=dev)
+        out_oi = torch.empty((4, E), dtype=torch.int32, device=dev)
+        g_s = torch.randn(A, device=dev)
+        g_o = torch.randn(E, device=dev)
+
+        def mm(kind, a, bb, tok, ov, oi, nnz):
+            return lambda: _lib.check(lib.sswin_block_matmul(kind, 0, ptr(a), ptr(bb), ptr(tok), m, hd, ptr(plan), g_cap, G,
+                                                             c_max, ptr(ov), ptr(oi), nnz, stream))
+
+        def grad(kind, a, bb, out):
+            return lambda: _lib.check(lib.sswin_block_matmul_grad(kind, 0, ptr(a), ptr(bb), ptr(cc), ptr(scans), G, hd,
+                                                                  ptr(out), stream))
+
+        def tr(kind, a, out):
+            return lambda: _lib.check(lib.sswin_block_transpose(kind, 0, ptr(a), ptr(cc), ptr(scans), G, hd, ptr(out), stream))
+
+        tmp_e, tmp_a = torch.empty(E, device=dev), torch.empty(A, device=dev)
+        idxT = b["idx"].T.contiguous()
+        flat_tok = ops.flatten_indices(idxT, [b["slots"], b["n"]])
+        perm_idx = o_idx[[0, 2, 1, 3], :].contiguous()
+        flat_perm = ops.flatten_indices(perm_idx, [o_shape[0], o_shape[2], o_shape[1], o_shape[3]])
+
+        entries = [
+            # name, callable, algorithmic bytes, calls per attention fwd+bwd
+            ("qkv_sparse_indices", lambda: ops.qkv_sparse_indices(b["idx"], b["slots"], b["n"], H, hd, _defer_check=True), 8 * N + 40 * E, 1),
+            ("plan_from_indices", lambda: _lib.check(lib.sswin_plan_from_indices(ptr(q.indices), m, hd, ptr(plan), g_cap, totals, ptr(ws), nb, stream)), 0, 2),
+            ("block_matmul q_k", mm(0, q.values, kt.values, q.indices, out_s, out_si, A), 2 * s * E + (s + 16) * A + 4 * G, 1),
+            ("flatten_indices [3,A]", lambda: ops.flatten_indices(s_idx[:3], s_shape[:3]), 16 * A, 1),
+            ("unique_consecutive_indices [A]", lambda: ops.unique_consecutive_indices(flat), 8 * A, 1),
+            ("softmax_last_dim_forward", lambda: ops.softmax_last_dim_forward(rows, s_val), 12 * A, 1),
+            ("block_matmul qk_v", mm(1, p_val, v.values, v.indices, out_o, out_oi, E), s * A + s * E + (s + 16) * E + 4 * G, 1),
+            ("permute order from the group structure [E]", lambda: ops.permute_heads_order(o_idx, o_shape), 0, 1),
+            ("flatten_indices [4,E] (generic permute)", lambda: ops.flatten_indices(perm_idx, [o_shape[0], o_shape[2], o_shape[1], o_shape[3]]), 0, 0),
+            ("sort_indices [E] (generic permute)", lambda: ops.sort_indices(flat_perm), 0, 0),
+            ("return_inverse [N]", lambda: ops.return_inverse(flat_tok, b["slots"] * b["n"]), 0, 1),
+            ("softmax_last_dim_backward", lambda: ops.softmax_last_dim_backward(rows, p_val, g_s), 16 * A, 1),
+            ("grad rc_cr", grad(0, g_o, v.values, tmp_a), 2 * s * E + s * A, 1),
+            ("grad rr_rc", grad(1, g_s, kt.values, tmp_e), s * A + 2 * s * E, 2),
+            ("grad cr_rr", grad(2, q.values, g_s, tmp_e), s * A + 2 * s * E, 1),
+            ("transpose rc", tr(0, q.values, tmp_e), 2 * s * E, 2),
+            ("transpose rr", tr(1, g_s, tmp_a), 2 * s * A, 2),
+        ]
+        # ---- the fused path (S and P in memory; what the module runs for heads that are not 32 wide) ----
+        qkv_c = qkv.contiguous()
+        bias = torch.randn(H, b["n"], b["n"], device=dev)
+        s_f = torch.empty(tp.A, device=dev)
+        rows_f = torch.empty(tp.A, dtype=torch.int32, device=dev)
+        out_f = torch.empty(N, D, device=dev)
+        dqkv = torch.empty_like(qkv_c)
+        dbias = torch.zeros(H, b["n"], b["n"], device=dev)
+        dt = torch.float32
+        bg_bytes = lib.sswin_fused_bias_grad_workspace_bytes(tp.G, H, b["n"])
+        bg_ws = torch.empty(int(bg_bytes), dtype=torch.uint8, device=dev)
+        f_entries = [
+            ("fused token_plan", lambda: F.TokenPlan(b["idx"], b["slots"], b["n"], H), 28 * N + 20 * tp.G, 1),
+            ("fused S=QK^T+bias+mask", lambda: F._tokens_to_sq(tp, dt, True, qkv_c, 3 * D, 0, qkv_c, 3 * D, D, hd, 0.17, bias, mask, s_f, rows_f), 8 * E + 8 * A, 1),
+            ("fused softmax fwd", lambda: ops.softmax_last_dim_forward(rows_f, s_f), 12 * A, 1),
+            ("fused O=PV", lambda: F._sq_to_tokens(tp, dt, False, p_val, qkv_c, 3 * D, 2 * D, out_f, D, 0, hd, 1.0), 4 * A + 8 * E, 1),
+            ("fused dP=dO V^T", lambda: F._tokens_to_sq(tp, dt, False, out_f, D, 0, qkv_c, 3 * D, 2 * D, hd, 1.0, None, None, s_f, None), 8 * E + 4 * A, 1),
+            ("fused dV=P^T dO", lambda: F._sq_to_tokens(tp, dt, True, p_val, out_f, D, 0, dqkv, 3 * D, 2 * D, hd, 1.0), 4 * A + 8 * E, 1),
+            ("fused softmax bwd", lambda: ops.softmax_last_dim_backward(rows_f, p_val, g_s), 16 * A, 1),
+            ("fused dQ=dS K", lambda: F._sq_to_tokens(tp, dt, False, g_s, qkv_c, 3 * D, D, dqkv, 3 * D, 0, hd, 0.17), 4 * A + 8 * E, 1),
+            ("fused dK=dS^T Q", lambda: F._sq_to_tokens(tp, dt, True, g_s, qkv_c, 3 * D, 0, dqkv, 3 * D, D, hd, 0.17), 4 * A + 8 * E, 1),
+            ("fused bias grad", lambda: _lib.check(lib.sswin_fused_bias_grad(ptr(tp.plan), tp.g_cap, tp.G, ptr(tp.tokens), tp.N, H, b["n"], ptr(g_s), ptr(dbias), ptr(bg_ws), bg_bytes, stream)), 4 * A, 1),
+        ]
+
+    # ---- the window-resident kernels (what the step runs for heads of 32 channels), in the workload's dtype ----
+    qkv_r = qkv.reshape(N, 3 * D).to(tdt).contiguous()
+    bias_r = torch.randn(H, b["n"], b["n"], device=dev)
+    out_r = torch.empty(N, D, device=dev, dtype=tdt)
+    dqkv_r = torch.empty_like(qkv_r)
+    ds_r = torch.empty(A, device=dev)
     lse = torch.empty(H * N, device=dev)
     mask_p, nmw = ptr(mask), (0 if mask is None else mask.shape[0])
-    qa = (ptr(qkv_c), 3 * D, 0, ptr(qkv_c), 3 * D, D, ptr(qkv_c), 3 * D, 2 * D)
-    da = (ptr(dqkv), 3 * D, 0, ptr(dqkv), 3 * D, D, ptr(dqkv), 3 * D, 2 * D)
-    up_r = torch.randn(N, D, device=dev)
+    qa = (ptr(qkv_r), 3 * D, 0, ptr(qkv_r), 3 * D, D, ptr(qkv_r), 3 * D, 2 * D)
+    da = (ptr(dqkv_r), 3 * D, 0, ptr(dqkv_r), 3 * D, D, ptr(dqkv_r), 3 * D, 2 * D)
+    up_r = torch.randn(N, D, device=dev).to(tdt)
+    Er = es * E // 4                                         # E in units of four bytes of token values
 
     def r_fwd():
-        _lib.check(lib.sswin_window_attention_forward(0, ptr(tp.tasks), tp.g_cap, tp.bucket_counts, ptr(tp.tokens), N, H,
-                                                      hd, *qa, C.c_float(0.17), ptr(bias), b["n"], mask_p, nmw,
-                                                      ptr(out_f), D, 0, ptr(lse), stream))
+        _lib.check(lib.sswin_window_attention_forward(code, ptr(tp.tasks), tp.g_cap, tp.bucket_counts, ptr(tp.tokens), N, H,
+                                                      hd, *qa, C.c_float(0.17), ptr(bias_r), b["n"], mask_p, nmw,
+                                                      ptr(out_r), D, 0, ptr(lse), stream))
 
     # The step asks for all gradients at once (sides = 3): one launch in which groups of at most
     # 64 tokens get dQ from their key-side tasks and only the larger groups have query-side tasks.
@@ -233,65 +283,71 @@ def kernel_table(wl, reps=20, only=None):
     # the groups of more than 32 tokens, 1 / 2 = the per-side kernels.
     bc = [int(x) for x in tp.bucket_counts]
     cg = tp.plan[:tp.G].to(torch.int64)                                  # plan row 0: tokens of each group
-    rows1, rowsL = int(cg[cg <= 32].sum()), int(cg[cg > 32].sum())       # token-head rows of small / large groups
+    rowsL = int(cg[cg > 32].sum())                                       # token-head rows of the large groups
     only_large = [0, bc[1], bc[2], bc[3]]
 
     def r_bwd(sides, counts=None):
         counts = tp.bucket_counts if counts is None else (C.c_int64 * 4)(*counts)
         return lambda: _lib.check(lib.sswin_window_attention_backward(
-            0, ptr(tp.tasks), tp.g_cap, counts, ptr(tp.tokens), N, H, hd, *qa, C.c_float(0.17), ptr(bias),
-            b["n"], mask_p, nmw, ptr(out_f), D, 0, ptr(up_r), D, 0, ptr(lse), *da, ptr(s_f), sides, stream))
+            code, ptr(tp.tasks), tp.g_cap, counts, ptr(tp.tokens), N, H, hd, *qa, C.c_float(0.17), ptr(bias_r),
+            b["n"], mask_p, nmw, ptr(out_r), D, 0, ptr(up_r), D, 0, ptr(lse), *da, ptr(ds_r), sides, stream))
 
-    from sparseswin3d_amd.window_attention import relative_position_index_3d
-    ti = F.BiasTableIndex.build(relative_position_index_3d(wl["blocks"][0]["attn"].window_size).to(dev), 729)
-    d_table = torch.empty(729, H, device=dev)
-    tg_bytes = lib.sswin_bias_table_grad_workspace_bytes(tp.G, H, 729)
+    n_table = int(wl["blocks"][0]["attn"].relative_position_bias_table.shape[0])
+    ti = F.BiasTableIndex.build(relative_position_index_3d(wl["blocks"][0]["attn"].window_size).to(dev), n_table)
+    d_table = torch.empty(n_table, H, device=dev)
+    tg_bytes = lib.sswin_bias_table_grad_workspace_bytes(tp.G, H, n_table)
     tg_ws = torch.empty(int(tg_bytes), dtype=torch.uint8, device=dev)
 
     def r_table_grad():
         _lib.check(lib.sswin_bias_table_grad(ptr(tp.plan), tp.g_cap, tp.G, ptr(tp.tokens), tp.N, H, b["n"], ptr(ti.code),
-                                             ti.offset0, 729, ptr(s_f), ptr(d_table), ptr(tg_ws), tg_bytes, stream))
+                                             ti.offset0, n_table, ptr(ds_r), ptr(d_table), ptr(tg_ws), tg_bytes, stream))
 
-    r_fwd()                                       # lse and out_f must hold a real forward for the backward timings
+    r_fwd()                                       # lse and out_r must hold a real forward for the backward timings
+    # flops of a launch: 2 c^2 hd per product and group = 2 A hd per product (two in the forward, five in the backward)
     r_entries = [
         ("resident token_plan", lambda: F.TokenPlan(b["idx"], b["slots"], b["n"], H), 28 * N + 36 * tp.G, 1),
-        ("resident forward", r_fwd, 16 * E + 4 * H * N, 1),
-        ("resident backward (dQ,dK,dV,dS)", r_bwd(3), 32 * E + 4 * A + 4 * H * N, 1),
-        ("resident backward dQ, groups > 32 tokens", r_bwd(1, only_large), (24 * hd + 4) * rowsL, 0),
-        ("resident backward dQ, all groups", r_bwd(1), 24 * E + 4 * H * N, 0),
-        ("resident backward dK,dV,dS only", r_bwd(2), 28 * E + 4 * A + 4 * H * N, 0),
+        ("resident forward", r_fwd, 16 * Er + 4 * H * N, 1, 4 * A * hd),
+        ("resident backward (dQ,dK,dV,dS)", r_bwd(3), 32 * Er + 4 * A + 4 * H * N, 1, 10 * A * hd),
+        ("resident backward dQ, groups > 32 tokens", r_bwd(1, only_large), (24 * es // 4 * hd + 4) * rowsL, 0),
+        ("resident backward dQ, all groups", r_bwd(1), 24 * Er + 4 * H * N, 0),
+        ("resident backward dK,dV,dS only", r_bwd(2), 28 * Er + 4 * A + 4 * H * N, 0),
         ("resident bias table grad", r_table_grad, 4 * A, 1),
-        ("resident bias grad [H,n,n]", lambda: _lib.check(lib.sswin_fused_bias_grad(ptr(tp.plan), tp.g_cap, tp.G, ptr(tp.tokens), tp.N, H, b["n"], ptr(s_f), ptr(dbias), ptr(bg_ws), bg_bytes, stream)), 4 * A, 0),
     ]
+    if code == 0:
+        r_entries.append(("resident bias grad [H,n,n]", lambda: _lib.check(lib.sswin_fused_bias_grad(
+            ptr(tp.plan), tp.g_cap, tp.G, ptr(tp.tokens), tp.N, H, b["n"], ptr(ds_r), ptr(dbias), ptr(bg_ws), bg_bytes, stream)), 4 * A, 0))
 
     def measure(items, path):
         rows_ = []
-        for name, fn, nbytes, calls in items:
+        for name, fn, nbytes, calls, *flops in items:
             ms = event_time_ms(fn, reps)
             gbps = nbytes / ms / 1e6 if nbytes else None
             rows_.append(dict(kernel=name, path=path, ms=ms, algorithmic_bytes=nbytes, calls=calls,
-                              achieved_gbps=gbps, frac=(gbps / HBM_PEAK_GBPS) if gbps else None))
+                              achieved_gbps=gbps, frac=(gbps / HBM_PEAK_GBPS) if gbps else None,
+                              flops=flops[0] if flops else None))
         return rows_
 
     if only is not None:
         # profiling mode: run the named kernels (substring match) `reps` times each, plus a plain
         # device-to-device copy of known size that calibrates the FETCH_SIZE / WRITE_SIZE counters
-        src = torch.empty(64 * 1024 * 1024, dtype=torch.float32, device=dev)
+        src = torch.empty(CALIBRATION_BYTES // 4, dtype=torch.float32, device=dev).normal_()
         dst = torch.empty_like(src)
-        picked = [e for e in r_entries + f_entries + entries + projection_entries(wl) if only in e[0]]
-        for name, fn, nbytes, calls in picked:
+        picked = [e for e in r_entries + f_entries + entries + (projection_entries(wl) if code == 0 else []) if only in e[0]]
+        for name, fn, nbytes, calls, *_ in picked:
             log(f"profiling {name}: {reps} launches, algorithmic bytes {nbytes}")
             for _ in range(reps):
                 fn()
         for _ in range(reps):
-            dst.copy_(src)
+            _lib.check(lib.sswin_calibration_copy(ptr(dst), ptr(src), CALIBRATION_BYTES, stream))
         torch.cuda.synchronize()
-        log(f"calibration copy: {reps} launches of {src.numel() * 4} bytes read and written")
-        return [], dict(N=N, E=E, A=A, G=G, c_max=c_max)
-    table = measure(r_entries, "resident") + measure(f_entries, "fused") + measure(entries, "operators")
-    table += measure(stage_entries(wl), "stage")
-    table += measure(projection_entries(wl), "projections")
-    return table, dict(N=N, E=E, A=A, G=G, c_max=c_max)
+        log(f"calibration copy: {reps} launches of {CALIBRATION_BYTES} bytes read and written")
+        return [], sizes
+    table = measure(r_entries, "resident")
+    if code == 0:
+        table += measure(f_entries, "fused") + measure(entries, "operators")
+        table += measure(stage_entries(wl), "stage")
+        table += measure(projection_entries(wl), "projections")
+    return table, sizes
 
 
 def stage_entries(wl):
@@ -412,30 +468,120 @@ def cpu_baseline(wl, target_tokens=None, budget_s=15.0, max_repeats=3):
 
 
 # ------------------------------------------------------------------------------------------
+def pmc_summary(dirs, out_name, workload, command, only=None):
+    """Turn the csv output of rocprofv3 --pmc runs of ``bench.py --profile-kernel`` (one run per counter set,
+    each written with ``--output-format csv -d DIR``) into a text summary ``profiles/<out_name>.txt`` and
+    into ``profiles/traffic.json`` (HBM bytes per launch of every kernel of KERNEL_SYMBOLS found in the runs).
+    FETCH_SIZE and WRITE_SIZE are scaled by what they read for the calibration copy of CALIBRATION_BYTES."""
+    import collections
+    import csv
+    import glob
+    acc = collections.defaultdict(list)
+    for d in dirs:
+        for path in glob.glob(os.path.join(d, "**", "*counter_collection.csv"), recursive=True):
+            for r in csv.DictReader(open(path)):
+                acc[(r["Kernel_Name"], r["Counter_Name"])].append(float(r["Counter_Value"]))
+    if not acc:
+        sys.exit(f"no *counter_collection.csv under {dirs}")
+    mean = {k: sum(v) / len(v) for k, v in acc.items()}
+    kernels = sorted({k for k, _ in mean if k.startswith(("void sswin::", "sswin::"))})
+    cal = next((k for k in kernels if "calibration_copy_kernel" in k), None)
+    wanted = only or [sym for sym, _ in KERNEL_SYMBOLS.values()]
+    kernels = [k for k in kernels if k == cal or any(w in k for w in wanted)]
+    unit = {}
+    if cal:
+        for cname in ("FETCH_SIZE", "WRITE_SIZE"):
+            if (cal, cname) in mean:
+                unit[cname] = CALIBRATION_BYTES / mean[(cal, cname)]
+    lines = [f"rocprofv3 --pmc counters, workload {workload}, means per dispatch over the launches of each run.",
+             "Commands (one rocprofv3 run per counter set; --pmc cannot split a set over passes):"]
+    lines += [f"  {c}" for c in command]
+    lines.append(f"Calibration: sswin::calibration_copy_kernel copies {CALIBRATION_BYTES} bytes (read once, written once): " +
+                 ", ".join(f"{c} reads {mean[(cal, c)]:.1f} -> {unit[c]:.1f} bytes per count" for c in unit))
+    lines.append("")
+    try:
+        with open(TRAFFIC_JSON) as f:
+            traffic = json.load(f)
+    except FileNotFoundError:
+        traffic = {}
+    for k in kernels:
+        if k == cal:
+            continue
+        cs = {c: v for (kk, c), v in mean.items() if kk == k}
+        lines.append(k if len(k) < 150 else k[:150] + " ...")
+        nb = None
+        if "FETCH_SIZE" in cs and "WRITE_SIZE" in cs and len(unit) == 2:
+            rd, wr = cs["FETCH_SIZE"] * unit["FETCH_SIZE"], cs["WRITE_SIZE"] * unit["WRITE_SIZE"]
+            nb = rd + wr
+            lines.append(f"    HBM traffic per launch: read {rd / 1e6:.1f} MB + written {wr / 1e6:.1f} MB = {nb / 1e6:.1f} MB")
+        for c in sorted(cs):
+            lines.append(f"    {c:28s} {cs[c]:16.1f}   (n={len(acc[(k, c)])})")
+        if "SQ_WAVES" in cs and "SQ_INSTS_VALU" in cs:
+            w = cs["SQ_WAVES"]
+            lines.append(f"    per wave: {cs['SQ_INSTS_VALU'] / w:.0f} VALU, {cs.get('SQ_INSTS_MFMA', 0) / w:.1f} MFMA, "
+                         f"{cs.get('SQ_INSTS_LDS', 0) / w:.0f} LDS, {cs.get('SQ_INSTS_VMEM_RD', 0) / w:.1f} loads, "
+                         f"{cs.get('SQ_INSTS_VMEM_WR', 0) / w:.1f} stores, {cs.get('SQ_INSTS_SALU', 0) / w:.0f} SALU instructions")
+        if "SQ_VALU_MFMA_BUSY_CYCLES" in cs and "SQ_BUSY_CYCLES" in cs and "GRBM_GUI_ACTIVE" in cs:
+            # MFMA busy cycles are summed over the SIMDs; 256 CUs x 4 SIMDs; GRBM_GUI_ACTIVE is summed over 8 XCDs
+            busy = cs["SQ_VALU_MFMA_BUSY_CYCLES"] / 1024
+            active = cs["GRBM_GUI_ACTIVE"] / 8
+            lines.append(f"    matrix cores busy {busy:.0f} cycles per SIMD of {active:.0f} GPU-active cycles = {100 * busy / active:.1f} %")
+        if "SQ_WAIT_INST_ANY" in cs and "SQ_WAVE_CYCLES" in cs:
+            lines.append(f"    waves waiting for an instruction's operands or issue: {100 * cs['SQ_WAIT_INST_ANY'] / cs['SQ_WAVE_CYCLES']:.1f} % of wave cycles")
+        if "SQ_LDS_BANK_CONFLICT" in cs and "SQ_ACTIVE_INST_LDS" in cs and cs["SQ_ACTIVE_INST_LDS"]:
+            # conflicts are counted in cycles, active time in units of four cycles
+            lines.append(f"    LDS bank conflict cycles / LDS active cycles: {100 * cs['SQ_LDS_BANK_CONFLICT'] / (4 * cs['SQ_ACTIVE_INST_LDS']):.1f} %")
+        lines.append("")
+        if nb is not None:
+            for name, (sym, srcs) in KERNEL_SYMBOLS.items():
+                if sym in k:
+                    traffic.setdefault(workload, {})[name] = dict(bytes=round(nb), summary=f"profiles/{out_name}.txt",
+                                                                  kernel=k[:120], sources=srcs, digest=source_digest(srcs))
+    out = os.path.join(ROOT, "profiles", out_name + ".txt")
+    with open(out, "w") as f:
+        f.write("\n".join(lines))
+    with open(TRAFFIC_JSON, "w") as f:
+        json.dump(traffic, f, indent=1, sort_keys=True)
+    print("\n".join(lines))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=20)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=400)
+    ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4"],
-                    help="cfg2 is the benchmark; the others report the step time only")
+                    help="cfg2 is the benchmark (the configuration the metric is quoted on); the others are "
+                         "reported the same way, without the CPU leg")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel table")
     ap.add_argument("--kernels-json", default=None)
     ap.add_argument("--profile-kernel", default=None, metavar="NAME",
                     help="run only the kernels whose table name contains NAME (for rocprofv3) and exit")
     ap.add_argument("--profile-reps", type=int, default=5)
+    ap.add_argument("--pmc-summary", nargs="+", default=None, metavar="DIR",
+                    help="no GPU work: summarise the rocprofv3 --pmc csv output under these directories into "
+                         "profiles/<--pmc-name>.txt and profiles/traffic.json")
+    ap.add_argument("--pmc-name", default=None)
+    ap.add_argument("--pmc-kernels", nargs="+", default=None, metavar="SUBSTR",
+                    help="kernel symbols to keep in the summary (default: those of KERNEL_SYMBOLS)")
+    ap.add_argument("--pmc-command", action="append", default=[], help="command line(s) quoted in the summary")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (windows are independent; sharding is "
                  "described in DESIGN.md); rerun with --gpus 1")
+    if args.pmc_summary:
+        from sparseswin3d_amd import synth
+        name = {"cfg1": synth.config1, "cfg2": synth.config2, "cfg3": synth.config3, "cfg4": synth.config4}[args.workload]().name
+        pmc_summary(args.pmc_summary, args.pmc_name or f"pmc_{args.workload}", name, args.pmc_command, args.pmc_kernels)
+        return
     if not torch.cuda.is_available():
         sys.exit("bench.py: no HIP GPU visible")
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
     wl = build_workload(device, args.workload)
     if args.workload != "cfg2":
-        args.no_cpu = args.no_kernels = True
+        args.no_cpu = True
     log(f"workload {wl['name']}: N={wl['N']}, blocks: " + "; ".join(str(b["stats"]) for b in wl["blocks"]))
     if args.profile_kernel is not None:
         kernel_table(wl, reps=args.profile_reps, only=args.profile_kernel)
@@ -470,6 +616,7 @@ def main():
 
     roofline = None
     sizes = {}
+    dtype_name = {torch.float32: "f32", torch.bfloat16: "bf16", torch.float16: "f16"}[wl["dtype"]]
     if not args.no_kernels:
         table, sizes = kernel_table(wl)
         log(f"{'kernel':36s} {'ms':>9s} {'calls':>5s} {'alg MB':>9s} {'GB/s':>9s} {'% HBM':>7s}")
@@ -479,6 +626,8 @@ def main():
         scope = {"stage": "once per stage", "projections": "one attention fwd+bwd"}
         for path in ("resident", "fused", "operators", "stage", "projections"):
             rows_ = [r for r in table if r["path"] == path]
+            if not rows_:
+                continue
             log(titles.get(path, f"-- {path} path, one attention forward+backward --"))
             for r in rows_:
                 log(f"{r['kernel']:36s} {r['ms']:9.4f} {r['calls']:5d} {r['algorithmic_bytes'] / 1e6:9.1f} "
@@ -498,12 +647,19 @@ def main():
         step_ms = in_step.get("window_attention_backward") if "backward (dQ,dK,dV,dS)" in dom["kernel"] else None
         ms = step_ms or dom["ms"]
         gbps = dom["algorithmic_bytes"] / ms / 1e6
+        traffic, traffic_note = measured_traffic(wl["name"], dom["kernel"])
         roofline = dict(bound="hbm", kernel=dom["kernel"], achieved=round(gbps, 1),
                         peak=HBM_PEAK_GBPS, unit="GB/s", frac=round(gbps / HBM_PEAK_GBPS, 4),
-                        traffic=MEASURED_TRAFFIC_BYTES.get(dom["kernel"]),
+                        traffic=traffic, traffic_source=traffic_note,
                         algorithmic_bytes=dom["algorithmic_bytes"], ms=round(ms, 4),
-                        ms_alone=round(dom["ms"], 4), timed="inside the step" if step_ms else "alone",
-                        path_summaries=summary)
+                        ms_alone=round(dom["ms"], 4), timed="inside the step" if step_ms else "alone")
+        if dom.get("flops"):
+            # the same launch against the matrix-core roof of the type its products run in
+            tflops = dom["flops"] / ms / 1e9
+            roofline["mfma"] = dict(achieved=round(tflops, 2), peak=MFMA_PEAK_TFLOPS[dtype_name], unit="TFLOP/s",
+                                    frac=round(tflops / MFMA_PEAK_TFLOPS[dtype_name], 4), flops=dom["flops"],
+                                    note="algorithmic flops: 2 c^2 hd per product and group, padding of the 32-token tiles not counted")
+        roofline["path_summaries"] = summary
         if args.kernels_json:
             with open(args.kernels_json, "w") as f:
                 json.dump(dict(sizes=sizes, kernels=table), f, indent=1)
@@ -516,7 +672,7 @@ def main():
     line = {
         "metric": "window-attn tokens/s fwd+bwd on 1 MI355X", "value": value, "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
-        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": "bf16" if wl["dtype"] == torch.bfloat16 else "f32", "data": "synthetic",
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype_name, "data": "synthetic",
         "config": {"workload": f"{wl['name']}: block pair (regular 5^3 windows, then shifted by 2) of "
                                f"WindowAttentionSparse, dim {wl['dim']}, {wl['heads']} heads, forward+backward",
                    "voxels": wl["N"], "attention_calls_per_step": calls, **sizes},

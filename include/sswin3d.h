@@ -38,6 +38,11 @@ const char* sswin_last_error(void);
 /* library ABI version, bumped on any signature change */
 int sswin_abi_version(void);
 
+/* A plain copy of `bytes` bytes (a multiple of 16; src, dst: device, 16-byte aligned, not overlapping): every
+ * byte is read once and written once.  It has no counterpart in the reference: a profiling run launches it
+ * beside the kernels it measures, and what the memory counters read for this known traffic gives their unit. */
+int sswin_calibration_copy(void* dst, const void* src, int64_t bytes, void* stream);
+
 /* ---- index operators -------------------------------------------------------------- */
 
 /* flatten_indices (sparse_swin/ops.cu:232-273, ops.h:38): wrapping int32 row-major hash of a

@@ -15,6 +15,7 @@ _vp, _i64, _i32, _sz = C.c_void_p, C.c_int64, C.c_int, C.c_size_t
 
 # name -> (restype, argtypes); mirrors include/sswin3d.h one to one
 SIGNATURES = {
+    "sswin_calibration_copy": (_i32, [_vp, _vp, _i64, _vp]),
     "sswin_last_error": (C.c_char_p, []),
     "sswin_abi_version": (_i32, []),
     "sswin_flatten_indices": (_i32, [_vp, _i32, _i64, _vp, _vp, _vp]),
@@ -70,7 +71,7 @@ SIGNATURES = {
                                                _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i32, _vp]),
 }
 
-ABI_VERSION = 17
+ABI_VERSION = 18
 _lib = None
 
 

@@ -356,6 +356,18 @@ __global__ __launch_bounds__(256) void sorted_k_kernel(const int32_t* __restrict
     for (int ch = 0; ch < hd; ++ch) sorted_k[base + (int64_t)ch * c] = src + ch;
 }
 
+// four 16-byte pieces per thread, each instruction of a wavefront covering 1 KB of contiguous memory
+__global__ __launch_bounds__(256) void calibration_copy_kernel(const int4* __restrict__ src, int4* __restrict__ dst, int64_t n16) {
+    const int64_t base = (int64_t)blockIdx.x * 1024 + threadIdx.x;
+    int4 v[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+        if (base + 256 * u < n16) v[u] = src[base + 256 * u];
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+        if (base + 256 * u < n16) dst[base + 256 * u] = v[u];
+}
+
 }  // namespace sswin
 
 using namespace sswin;
@@ -366,7 +378,20 @@ using namespace sswin;
 extern "C" {
 
 const char* sswin_last_error(void) { return error_buffer(); }
-int sswin_abi_version(void) { return 17; }
+int sswin_abi_version(void) { return 18; }
+
+int sswin_calibration_copy(void* dst, const void* src, int64_t bytes, void* stream) {
+    SSWIN_CHECK(bytes >= 0 && bytes % 16 == 0, "calibration_copy: size must be a multiple of 16 bytes");
+    if (bytes == 0) return 0;
+    SSWIN_CHECK(dst && src && ((uintptr_t)dst % 16) == 0 && ((uintptr_t)src % 16) == 0,
+                "calibration_copy: pointers must be 16-byte aligned device addresses");
+    const int64_t n16 = bytes / 16;
+    const int64_t blocks = (n16 + 256 * 4 - 1) / (256 * 4);
+    SSWIN_CHECK(blocks < ((int64_t)1 << 31), "calibration_copy: too large");
+    hipLaunchKernelGGL(calibration_copy_kernel, dim3((unsigned)blocks), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       static_cast<const int4*>(src), static_cast<int4*>(dst), n16);
+    return launch_ok("calibration_copy");
+}
 
 int sswin_flatten_indices(const int32_t* idx, int ndim, int64_t M, const int32_t* sizes, int32_t* out,
                           void* stream) {
