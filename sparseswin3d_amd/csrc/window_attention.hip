@@ -400,24 +400,51 @@ __device__ __forceinline__ void rows_dot_to_table(const PadTab& tab, int lane, c
 // ------------------------------------------------------------------------------------------
 // forward: rows = 32 queries of a group, tiles = its keys
 // ------------------------------------------------------------------------------------------
-template <typename T, bool MASK>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void wattn_fwd_kernel(WAttnCommon a, TokenTensor32 tq, TokenTensor32 tk,
-                                                        TokenTensor32 tv, TokenTensor32 to,
-                                                        float* __restrict__ lse) {
-    __shared__ __attribute__((aligned(16))) float tiles[4][2][TILE_WORDS];
-    __shared__ __attribute__((aligned(16))) uint32_t tabs[4][2][32];
-    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+// What a forward task needs before it can ask for token rows: its group, its block of 32 queries, and the
+// voxels and window positions of its queries and of its first key tile.  Fetching them takes two dependent
+// memory round trips (descriptor, then indices); they are fetched in one place so that a caller can fetch them ahead of the task.
+struct KIdx {
+    uint32_t vox;        // voxel of key t*32 + l32 (clamped to the last token)
+    int pos;
+};
+struct FwdIdx {
+    uint32_t vox_i;      // voxel of query bi*32 + l32 (clamped to the last token)
+    int pos_i;
+    KIdx k0;
+};
+__device__ __forceinline__ GroupCtx decode_group(const int4& t) {
+    GroupCtx g;
+    g.Tk = __builtin_amdgcn_readfirstlane(t.x);
+    g.c = __builtin_amdgcn_readfirstlane(t.y & 0xff);
+    g.h = __builtin_amdgcn_readfirstlane(t.y >> 8);
+    g.w = __builtin_amdgcn_readfirstlane(t.z);
+    g.sq = __builtin_amdgcn_readfirstlane(t.w);
+    return g;
+}
+__device__ __forceinline__ FwdIdx fwd_indices(const WAttnCommon& a, const GroupCtx& g, int bi, int l32) {
+    const int32_t* order = a.order + g.Tk;
+    const int32_t* tok_pos = a.tok_pos + g.Tk;
+    const int i_q = bi * 32 + l32;
+    const int i_c = i_q < g.c ? i_q : g.c - 1;
+    const int j_c = l32 < g.c ? l32 : g.c - 1;
+    FwdIdx x;
+    x.vox_i = order[i_c];
+    x.pos_i = tok_pos[i_c];
+    x.k0 = KIdx{(uint32_t)order[j_c], tok_pos[j_c]};
+    return x;
+}
+
+// One forward task on one wavefront.  `mid` runs once between the last key tile and the write-out (a hook for
+// work that should overlap the write-out; the plain kernel passes nothing).
+template <typename T, bool MASK, typename Mid>
+__device__ __forceinline__ void fwd_task(const WAttnCommon& a, const GroupCtx& g, const int bi, const FwdIdx& fi,
+                                         float* tile, float* tile_x, uint32_t* tab_key, uint32_t* tab_alpha,
+                                         const TokenTensor32& tq, const TokenTensor32& tk, const TokenTensor32& tv,
+                                         const TokenTensor32& to, float* __restrict__ lse, Mid&& mid) {
+    const int lane = threadIdx.x & 63;
     const int half = lane >> 5, l32 = lane & 31;
-    int64_t d;
-    int bi;
-    if (!locate(a, (int64_t)blockIdx.x * 4 + wave, d, bi)) return;
-    const GroupCtx g = load_group(a.tasks, d);
     const int c = g.c, h = g.h;
     const int nt = (c + 31) >> 5;
-    float* tile = tiles[wave][0];
-    float* tile_x = tiles[wave][1];
-    uint32_t* tab_key = tabs[wave][0];
-    uint32_t* tab_alpha = tabs[wave][1];
     const int32_t* order = a.order + g.Tk;
     const int32_t* tok_pos = a.tok_pos + g.Tk;
     const int8_t* mrow = MASK ? a.mask + (int64_t)(g.w % a.nmw) * a.n : nullptr;
@@ -428,22 +455,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 
     // query side: lane l32 owns query bi*32 + l32 (both halves), clamped to the last token
     const int i_q = bi * 32 + l32;
-    const int i_c = i_q < c ? i_q : c - 1;
-    const uint32_t vox_i = order[i_c];
-    const int pos_i = tok_pos[i_c];
+    const uint32_t vox_i = fi.vox_i;
+    const int pos_i = fi.pos_i;
     // The memory round trips of a task depend on one another (descriptor -> token indices -> rows ->
     // bias) and a task is short, so the indices of the first key tile are requested together with the
     // query indices, and its K and V rows together with the Q rows.
-    struct KIdx {
-        uint32_t vox;        // voxel of key t*32 + l32 (clamped to the last token)
-        int pos;
-    };
     auto load_kidx = [&](const int t) {
         const int j = t * 32 + l32;
         const int j_c = j < c ? j : c - 1;
         return KIdx{(uint32_t)order[j_c], tok_pos[j_c]};
     };
-    KIdx kcur = load_kidx(0);
+    KIdx kcur = fi.k0;
     const int reg_i = MASK ? mrow[pos_i] : 0;
     RowLoad<T> rk, rv;
     float qb[16];
@@ -452,6 +474,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         rows_load<T>(qbase, qpitch, vox_i, lane, rq);
         rows_load<T>(kbase, kpitch, kcur.vox, lane, rk);
         rows_load<T>(vbase, vpitch, kcur.vox, lane, rv);
+        __builtin_amdgcn_wave_barrier();
         rows_to_tile<T>(tile_x, lane, rq);
         __builtin_amdgcn_wave_barrier();
         tile_get_rows(tile_x, l32, half, qb);
@@ -513,15 +536,34 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             for (int r = 0; r < 16; ++r) o[r] *= u2f(ar[r]);
         }
         m = mt;
+        if constexpr (std::is_same<T, float>::value) {
+            // P V by blocks of eight key rows (registers 4q .. 4q + 3 hold rows 8q + k and 8q + k + 4 of the two
+            // lane halves): a block that lies wholly behind the last key is padding and is skipped, exponentials
+            // and matrix steps alike (windows of 5^3 positions hold 20 to 30 tokens on average)
+            const int kleft = c - t * 32;
+            if constexpr (FIRST) o = f32x16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-            S[r] = exp2_fast(S[r] - m);
-            l += S[r];
+            for (int q = 0; q < 4; ++q) {
+                if (q > 0 && 8 * q >= kleft) break;
+#pragma unroll
+                for (int k = 0; k < 4; ++k) {
+                    const int r = 4 * q + k;
+                    const float pr = exp2_fast(S[r] - m);
+                    l += pr;
+                    o = __builtin_amdgcn_mfma_f32_32x32x2f32(pr, vb[r], o, 0, 0, 0);
+                }
+            }
+        } else {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                S[r] = exp2_fast(S[r] - m);
+                l += S[r];
+            }
+            if constexpr (FIRST)
+                o = mma_slots_first<T, 16>(S, vb);
+            else
+                mma_slots<T, 0, 16>(S, vb, o);
         }
-        if constexpr (FIRST)
-            o = mma_slots_first<T, 16>(S, vb);
-        else
-            mma_slots<T, 0, 16>(S, vb, o);
     };
     tile_step(std::true_type{}, 0, kcur);
 #pragma unroll 1
@@ -531,6 +573,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         rows_load<T>(vbase, vpitch, kcur.vox, lane, rv);
         tile_step(std::false_type{}, t, kcur);
     }
+    mid();
     l += __shfl_xor(l, 32, 64);
     l += 1e-8f;
     if (half == 0 && i_q < c) lse[(int64_t)a.H * g.Tk + h * c + i_q] = (m + __builtin_amdgcn_logf(l)) * LN2;
@@ -545,6 +588,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     tile_put_acc(tile, l32, half, o);
     __builtin_amdgcn_wave_barrier();
     tile_store_rows<T>(tile, const_cast<char*>(head_base<T>(to, h)), pitch_of<T>(to), vox_i, c - bi * 32, lane);
+}
+
+
+template <typename T, bool MASK>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void wattn_fwd_kernel(WAttnCommon a, TokenTensor32 tq, TokenTensor32 tk,
+                                                        TokenTensor32 tv, TokenTensor32 to,
+                                                        float* __restrict__ lse) {
+    __shared__ __attribute__((aligned(16))) float tiles[4][2][TILE_WORDS];
+    __shared__ __attribute__((aligned(16))) uint32_t tabs[4][2][32];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    int64_t d;
+    int bi;
+    if (!locate(a, (int64_t)blockIdx.x * 4 + wave, d, bi)) return;
+    const GroupCtx g = load_group(a.tasks, d);
+    const FwdIdx fi = fwd_indices(a, g, bi, lane & 31);
+    fwd_task<T, MASK>(a, g, bi, fi, tiles[wave][0], tiles[wave][1], tabs[wave][0], tabs[wave][1], tq, tk, tv, to, lse, [] {});
 }
 
 // ------------------------------------------------------------------------------------------
@@ -645,6 +704,8 @@ __device__ __forceinline__ void bwd_q_task(const WAttnCommon& a, int64_t task, f
         const int jlim = c - t * 32 - 4 * half;
 #pragma unroll
         for (int r = 0; r < 16; ++r) {
+            // fp32: a block of eight key rows wholly behind the last key is padding and is skipped
+            if (std::is_same<T, float>::value && (r & 3) == 0 && r > 0 && 2 * r >= c - t * 32) break;
             float s = fmaf(bv[r], LOG2E, St[r]);
             if (MASK && (int)(pkr[r] >> 16) != reg_i) s += -100.0f * LOG2E;
             const float pr = (8 * (r >> 2) + (r & 3)) < jlim ? exp2_fast(s - L2) : 0.f;
@@ -831,8 +892,22 @@ __device__ __forceinline__ void bwd_kv_task(const WAttnCommon& a, int64_t task, 
         const float* do_col = tile_do + 4 * half * TILE_LD + l32;
         const float* q_col = tile_q + 4 * half * TILE_LD + l32;
         float dob8[8], qbr8[8];                              // 16-bit tokens: operands of eight slots
+        const int qleft = c - t * 32;                         // queries of this tile
 #pragma unroll
         for (int q = 0; q < 4; ++q) {
+            if constexpr (std::is_same<T, float>::value) {
+                // a block of eight query rows that lies wholly behind the last query is padding: P and dS
+                // are zero there, so its exponentials, LDS reads and matrix steps are skipped
+                if (q > 0 && 8 * q >= qleft) {
+                    if (DQ_USE != 0) {
+#pragma unroll
+                        for (int qq = q; qq < 4; ++qq)
+#pragma unroll
+                            for (int k = 0; k < 4; ++k) dPt[4 * qq + k] = 0.f;
+                    }
+                    break;
+                }
+            }
             const u32x4_a Lq = tab_L.chunk(2 * q + half), Dq = tab_D.chunk(2 * q + half);
             const uint32_t Lr[4] = {Lq.x, Lq.y, Lq.z, Lq.w}, Dr[4] = {Dq.x, Dq.y, Dq.z, Dq.w};
             float dob[4], qbr[4];
@@ -888,7 +963,21 @@ __device__ __forceinline__ void bwd_kv_task(const WAttnCommon& a, int64_t task, 
             const float* k_col = tile_q + 16 * half * TILE_LD + l32;
 #pragma unroll
             for (int s = 0; s < 16; ++s) kc[s] = k_col[s * TILE_LD];  // K[key 16 * half + s][channel l32]
-            f32x16 dq = mma_slots_first<T, 16>(dsr, kc);
+            f32x16 dq;
+            if constexpr (std::is_same<T, float>::value) {
+                // slot s carries keys s and 16 + s of this task's tile: slots behind the last key are padding
+                const int kleft = c - bj * 32;
+                dq = f32x16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+                for (int sb = 0; sb < 4; ++sb) {
+                    if (sb > 0 && 4 * sb >= kleft) break;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k)
+                        dq = __builtin_amdgcn_mfma_f32_32x32x2f32(dsr[4 * sb + k], kc[4 * sb + k], dq, 0, 0, 0);
+                }
+            } else {
+                dq = mma_slots_first<T, 16>(dsr, kc);
+            }
             if constexpr (DQ_USE == 2) {
                 xch_put(xch, lane, dq);
                 __builtin_amdgcn_wave_barrier();
