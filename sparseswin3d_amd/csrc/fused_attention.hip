@@ -32,10 +32,13 @@ constexpr int FUSED_GROUPS_PER_WG = 4;
 // Five phases, no sort:
 //   1. clear the presence bitmap (W = ceil(n/32) words per window slot) and the counters
 //   2. one atomicOr per voxel (indices outside [0,B) x [0,n) are counted and skipped)
-//   3. per block of 256 window slots: sums of (tokens, tokens^2, non-empty windows)
+//   3. per block of 256 window slots: sums of (tokens, tokens^2, non-empty windows, windows per
+//      tile-count bucket) and the largest window
 //   4. per block: prefix of the earlier blocks' sums, scan inside the block; every non-empty
-//      window learns the rank T of its first token, its rank k among the non-empty windows and
-//      the sum of c*c before it, and writes its H plan rows and task descriptors
+//      window learns the rank T of its first token, its rank k among the non-empty windows, the
+//      sum of c*c before it and its rank inside its bucket, and writes its H plan rows and task
+//      descriptors (no atomics: one counter per bucket, bumped once per wavefront from eight XCDs,
+//      made this phase 13 us instead of 5)
 //   5. per voxel: rank = T(window) + number of occupied positions below its own
 // Reduce-then-scan (3, 4) instead of a chained scan: no block waits for another block.  One launch
 // per phase.  (All five phases in one cooperative launch with grid-wide barriers in between were
@@ -53,7 +56,7 @@ struct TokenPlanArgs {
     int B, n, W, H;
     uint32_t* bits;          // [B * W]
     int32_t* win_T;          // [B]
-    int64_t* partial_a;      // [blocks]
+    int64_t* partial_a;      // [3 * blocks]
     int32_t* partial_b;      // [blocks]
     int64_t* totals;         // [8]: windows, sum c | sum c*c << 32, then twelve int32 counters
     int32_t* plan;
@@ -95,30 +98,54 @@ __device__ __forceinline__ int tp_window_count(const uint32_t* bits, int64_t w, 
 
 struct TpShared {
     int64_t a[TP_BLOCK / 64];
-    int32_t b[TP_BLOCK / 64];
-    int64_t base_a;
-    int32_t base_b;
+    int64_t base[3];
+    int32_t m[TP_BLOCK / 64];
+    int32_t base_m;
 };
 
-// block sums: partial_a[blk] = sum c | sum c*c << 32, partial_b[blk] = non-empty windows
+// What a window slot adds to the three running sums (each an int64 of packed fields):
+//   sum c | sum c*c << 32
+//   windows of one, two, three tiles                (21 bits each: fewer than 2^21 window slots)
+//   windows of four tiles, of more, non-empty ones  (21 bits each)
+__device__ __forceinline__ int tp_bucket(int64_t c) { return c > 0 ? min(((int)c - 1) >> 5, 4) : -1; }
+__device__ __forceinline__ void tp_items(int64_t c, int64_t (&item)[3]) {
+    const int b = tp_bucket(c);
+    item[0] = c | ((c * c) << 32);
+    item[1] = b >= 0 && b < 3 ? (int64_t)1 << (21 * b) : 0;
+    item[2] = (b >= 3 ? (int64_t)1 << (21 * (b - 3)) : 0) | (c > 0 ? (int64_t)1 << 42 : 0);
+}
+__device__ __forceinline__ int tp_block_max(int v, TpShared& sh) {
+    const int wm = wave_max_i32(v);
+    if ((threadIdx.x & 63) == 0) sh.m[threadIdx.x >> 6] = wm;
+    __syncthreads();
+    int m = 0;
+#pragma unroll
+    for (int w = 0; w < TP_BLOCK / 64; ++w) m = max(m, sh.m[w]);
+    __syncthreads();
+    return m;
+}
+
+// block sums: partial_a[3 * blk + k] = the three sums over the block's window slots, partial_b[blk] = largest c
 __device__ __forceinline__ void tp_phase_block_sums(const TokenPlanArgs& a, int blk, TpShared& sh) {
     const int64_t w = (int64_t)blk * TP_BLOCK + threadIdx.x;
     const int64_t c = w < a.B ? tp_window_count(a.bits, w, a.W) : 0;
-    int64_t ta;
-    int32_t tb;
-    (void)block_exclusive_scan<int64_t, TP_BLOCK / 64>(c | ((c * c) << 32), sh.a, &ta);
-    (void)block_exclusive_scan<int32_t, TP_BLOCK / 64>(c > 0 ? 1 : 0, sh.b, &tb);
+    int64_t item[3], total[3];
+    tp_items(c, item);
+#pragma unroll
+    for (int k = 0; k < 3; ++k) (void)block_exclusive_scan<int64_t, TP_BLOCK / 64>(item[k], sh.a, &total[k]);
+    const int cm = tp_block_max((int)c, sh);
     if (threadIdx.x == 0) {
-        a.partial_a[blk] = ta;
-        a.partial_b[blk] = tb;
+#pragma unroll
+        for (int k = 0; k < 3; ++k) a.partial_a[3 * blk + k] = total[k];
+        a.partial_b[blk] = cm;
     }
 }
 
 // Groups are bucketed by their number of 32-token tiles (bucket b: 32*b < c <= 32*(b+1), b = 0..3;
 // counters[4] counts larger groups, which get no descriptor).  Descriptor = {T, c | head << 8,
-// window, sq_start}.  Slots inside a bucket are handed out with one atomic per wavefront and
-// bucket, so the order of the windows inside a bucket varies from run to run; consumers treat a
-// bucket as an unordered set.
+// window, sq_start}.  A window's slot inside its bucket is its rank among the bucket's windows in
+// window order (prefix of the earlier blocks' counts + scan inside the block): no atomics, and the same
+// descriptor order on every run.
 __device__ __forceinline__ void tp_phase_windows(const TokenPlanArgs& a, int blk, TpShared& sh) {
     const int H = a.H;
     const int64_t g_cap = a.g_cap;
@@ -127,35 +154,43 @@ __device__ __forceinline__ void tp_phase_windows(const TokenPlanArgs& a, int blk
     const int64_t w = (int64_t)blk * TP_BLOCK + threadIdx.x;
     const int64_t c = w < a.B ? tp_window_count(a.bits, w, a.W) : 0;
     // prefix of the earlier blocks
-    int64_t pa = 0;
-    int32_t pb = 0;
+    int64_t p[3] = {0, 0, 0};
+    int pm = 0;
     for (int64_t i = threadIdx.x; i < blk; i += TP_BLOCK) {
-        pa += a.partial_a[i];
-        pb += a.partial_b[i];
+#pragma unroll
+        for (int k = 0; k < 3; ++k) p[k] += a.partial_a[3 * i + k];
+        pm = max(pm, a.partial_b[i]);
     }
-    int64_t ta;
-    int32_t tb;
-    (void)block_exclusive_scan<int64_t, TP_BLOCK / 64>(pa, sh.a, &ta);
-    (void)block_exclusive_scan<int32_t, TP_BLOCK / 64>(pb, sh.b, &tb);
+    int64_t total[3];
+#pragma unroll
+    for (int k = 0; k < 3; ++k) (void)block_exclusive_scan<int64_t, TP_BLOCK / 64>(p[k], sh.a, &total[k]);
+    const int bm = tp_block_max(max(pm, (int)c), sh);            // largest c up to and including this block
     if (threadIdx.x == 0) {
-        sh.base_a = ta;
-        sh.base_b = tb;
+#pragma unroll
+        for (int k = 0; k < 3; ++k) sh.base[k] = total[k];
     }
     __syncthreads();
-    const int64_t base_a = sh.base_a;
-    const int32_t base_b = sh.base_b;
-
-    const int64_t ea = block_exclusive_scan<int64_t, TP_BLOCK / 64>(c | ((c * c) << 32), sh.a, &ta) + base_a;
-    const int32_t k = block_exclusive_scan<int32_t, TP_BLOCK / 64>(c > 0 ? 1 : 0, sh.b, &tb) + base_b;
+    int64_t item[3], e[3];
+    tp_items(c, item);
+#pragma unroll
+    for (int k = 0; k < 3; ++k) e[k] = block_exclusive_scan<int64_t, TP_BLOCK / 64>(item[k], sh.a, &total[k]) + sh.base[k];
+    const int32_t k = (int32_t)(e[2] >> 42);                     // non-empty windows before this one
     if (blk == a.blocks - 1 && threadIdx.x == 0) {
-        a.totals[0] = (int64_t)(base_b + tb);                   // non-empty windows
-        a.totals[1] = base_a + ta;                              // sum c | sum c*c << 32
+        const int64_t t1 = sh.base[1] + total[1], t2 = sh.base[2] + total[2];
+        a.totals[0] = t2 >> 42;                                  // non-empty windows
+        a.totals[1] = sh.base[0] + total[0];                     // sum c | sum c*c << 32
+        const int64_t f = (1 << 21) - 1;
+        counters[0] = (int32_t)(t1 & f) * H;
+        counters[1] = (int32_t)((t1 >> 21) & f) * H;
+        counters[2] = (int32_t)((t1 >> 42) & f) * H;
+        counters[3] = (int32_t)(t2 & f) * H;
+        counters[4] = (int32_t)((t2 >> 21) & f) * H;
+        counters[TPC_CMAX] = bm;
     }
-    const int32_t T = (int32_t)(ea & 0xffffffffll);
-    const int64_t q2 = ea >> 32;
+    const int32_t T = (int32_t)(e[0] & 0xffffffffll);
+    const int64_t q2 = e[0] >> 32;
     if (w < a.B) a.win_T[w] = T;
 
-    const int lane = threadIdx.x & 63;
     const bool live = c > 0 && ((int64_t)k + 1) * H <= g_cap;
     if (live) {
         for (int h = 0; h < H; ++h) {
@@ -167,30 +202,15 @@ __device__ __forceinline__ void tp_phase_windows(const TokenPlanArgs& a, int blk
             a.plan[4 * g_cap + g] = h;
         }
     }
-    // wave maximum of c, one atomic per wavefront
-    const int cm = wave_max_i32((int)c);
-    if (lane == 0 && cm > 0) atomicMax(&counters[TPC_CMAX], cm);
     if (a.tasks == nullptr) return;
-    const int b = live ? min(((int)c - 1) >> 5, 4) : -1;
-    // lanes 0..4 reserve the slots of the five buckets with one atomic each, at the same time
-    int slot = 0;
-    unsigned long long members[5];
-#pragma unroll
-    for (int q = 0; q < 5; ++q) members[q] = __ballot(b == q);
-    unsigned long long mine = 0;
-#pragma unroll
-    for (int q = 0; q < 5; ++q) mine = lane == q ? members[q] : mine;
-    int base = 0;
-    if (lane < 5 && mine != 0) base = atomicAdd(&counters[lane], H * __popcll(mine));
-#pragma unroll
-    for (int q = 0; q < 5; ++q) {
-        const int base_q = __shfl(base, q, 64);
-        if (b == q) slot = base_q + H * __popcll(members[q] & ((1ull << lane) - 1ull));
-    }
+    const int b = tp_bucket(c);
     if (live && b < 4) {
-        for (int h = 0; h < H; ++h)
-            a.tasks[(int64_t)b * g_cap + slot + h] =
-                make_int4(T, (int)c | (h << 8), (int)w, (int32_t)(q2 * H + (int64_t)h * c * c));
+        const int64_t f = (1 << 21) - 1;
+        const int64_t slot = (b < 3 ? (e[1] >> (21 * b)) & f : e[2] & f) * H;
+        if (slot + H <= g_cap)
+            for (int h = 0; h < H; ++h)
+                a.tasks[(int64_t)b * g_cap + slot + h] =
+                    make_int4(T, (int)c | (h << 8), (int)w, (int32_t)(q2 * H + (int64_t)h * c * c));
     }
 }
 
@@ -796,7 +816,7 @@ size_t sswin_token_plan_workspace_bytes(int64_t N, int B, int n) {
     (void)N;
     const size_t words = (size_t)B * tp_words_per_window(n);
     const size_t blocks = (size_t)tp_blocks(B);
-    return align_up(words * 4, 256) + align_up((size_t)B * 4, 256) + align_up(blocks * 8, 256) +
+    return align_up(words * 4, 256) + align_up((size_t)B * 4, 256) + align_up(blocks * 24, 256) +
            align_up(blocks * 4, 256) + 1024;
 }
 
@@ -804,6 +824,7 @@ int sswin_token_plan(const int32_t* indices, int64_t N, int B, int n, int H, int
                      int32_t* plan, int64_t g_cap, int32_t* tasks, int64_t* totals_out, void* ws,
                      size_t ws_bytes, int synchronize, void* stream) {
     SSWIN_CHECK(N >= 0 && B > 0 && n > 0 && H > 0 && H < 256, "token_plan: bad sizes");
+    SSWIN_CHECK(B < (1 << 21), "token_plan: %d window slots, the plan counts them in 21 bits", B);
     SSWIN_CHECK(totals_out, "token_plan: totals_out is null");
     for (int i = 0; i < 9; ++i) totals_out[i] = 0;
     if (N == 0) return 0;
@@ -826,7 +847,7 @@ int sswin_token_plan(const int32_t* indices, int64_t N, int B, int n, int H, int
     a.totals = cv.take<int64_t>(8);       // [0] windows, [1] sum c | sum c*c << 32, [2..7] counters
     a.bits = cv.take<uint32_t>(words);
     a.win_T = cv.take<int32_t>((size_t)B);
-    a.partial_a = cv.take<int64_t>((size_t)blocks);
+    a.partial_a = cv.take<int64_t>(3 * (size_t)blocks);
     a.partial_b = cv.take<int32_t>((size_t)blocks);
     SSWIN_CHECK(cv.ok(), "token_plan: workspace too small");
     a.plan = plan;
