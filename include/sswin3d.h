@@ -105,6 +105,31 @@ int sswin_qkv_sparse_indices(const int32_t* indices, int64_t N, int B, int n, in
                              int32_t* sorted_k, void* ws, size_t ws_bytes, int validate, int32_t* status_out,
                              void* stream);
 
+/* ---- sorted operands without the permutations ------------------------------------------------
+ * qkv_sparse_cuda (sparse_swin/swin3d_base.py:483-498) gathers the index matrices and the values of
+ * Q, K^T, V through the two permutations of qkv_sparse_indices, and autograd sends the gradients back
+ * through index_add; the tail of WindowAttention.forward (:672-675) un-sorts the output through another
+ * hash, sort and gather.  All of these are fixed permutations of the N*H*hd values, known from the rank
+ * of every voxel in (window, pos) order.  The three calls below produce the same tensors directly.
+ *
+ * sswin_operand_map: map (device int32 [3N + 2]) = voxel of rank r, rank T of the first token of its window,
+ *   tokens c of its window (each [N], by rank), then {pairs out of range, distinct pairs}.  validate /
+ *   status_out as in sswin_qkv_sparse_indices; with invalid pairs the calls below copy nothing.
+ * sswin_operand_copy: layout 0 (Q, V, attention output): val[hd*(H*T + h*c + i) + ch], layout 1 (K^T):
+ *   val[hd*(H*T + h*c) + ch*c + i]  <->  vox[voxel * vox_stride + vox_col0 + h*hd + ch] (strides in values);
+ *   to_operand != 0 copies voxel rows into the operand, 0 copies the operand into voxel rows.  Each direction is
+ *   the gradient of the other.  dtype: any value dtype.
+ * sswin_sorted_coo_indices: the [4, E] index matrices of Q/V and of K^T in sorted order (either may be NULL),
+ *   equal to idx.index_select(1, sorted) of sswin_qkv_sparse_indices.
+ * All asynchronous unless validate != 0. */
+size_t sswin_operand_map_workspace_bytes(int64_t N, int B, int n);
+int sswin_operand_map(const int32_t* indices, int64_t N, int B, int n, int32_t* map, void* ws, size_t ws_bytes,
+                      int validate, int32_t* status_out, void* stream);
+int sswin_operand_copy(int dtype, int layout, int to_operand, void* vox, int64_t vox_stride, int vox_col0, void* val,
+                       const int32_t* map, int64_t N, int H, int hd, void* stream);
+int sswin_sorted_coo_indices(const int32_t* indices, const int32_t* map, int64_t N, int H, int hd, int32_t* idx_qv,
+                             int32_t* idx_k, void* stream);
+
 /* ---- per-group offsets ("plan") ----------------------------------------------------- */
 
 /* Group structure of a coalesced 4-D COO operand whose last dimension is dense

@@ -28,6 +28,10 @@ SIGNATURES = {
     "sswin_return_inverse": (_i32, [_vp, _i64, _i64, _vp, _vp, _vp, _sz, _vp]),
     "sswin_qkv_sparse_indices_workspace_bytes": (_sz, [_i64, _i32, _i32]),
     "sswin_qkv_sparse_indices": (_i32, [_vp, _i64, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _vp, _sz, _i32, _vp, _vp]),
+    "sswin_operand_map_workspace_bytes": (_sz, [_i64, _i32, _i32]),
+    "sswin_operand_map": (_i32, [_vp, _i64, _i32, _i32, _vp, _vp, _sz, _i32, _vp, _vp]),
+    "sswin_operand_copy": (_i32, [_i32, _i32, _i32, _vp, _i64, _i32, _vp, _vp, _i64, _i32, _i32, _vp]),
+    "sswin_sorted_coo_indices": (_i32, [_vp, _vp, _i64, _i32, _i32, _vp, _vp, _vp]),
     "sswin_plan_workspace_bytes": (_sz, [_i64, _i32]),
     "sswin_plan_from_indices": (_i32, [_vp, _i64, _i32, _vp, _i64, _vp, _vp, _sz, _vp]),
     "sswin_permute_heads_order": (_i32, [_vp, _i64, _i32, _vp, _i64, _i64, _vp, _vp, _vp]),
@@ -71,7 +75,7 @@ SIGNATURES = {
                                                _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i32, _vp]),
 }
 
-ABI_VERSION = 18
+ABI_VERSION = 19
 _lib = None
 
 

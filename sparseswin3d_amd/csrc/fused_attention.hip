@@ -56,7 +56,7 @@ struct TokenPlanArgs {
     int B, n, W, H;
     uint32_t* bits;          // [B * W]
     int32_t* win_T;          // [B]
-    int64_t* partial_a;      // [3 * blocks]
+    int64_t* partial_a;      // [4 * blocks]
     int32_t* partial_b;      // [blocks]
     int64_t* totals;         // [8]: windows, sum c | sum c*c << 32, then twelve int32 counters
     int32_t* plan;
@@ -96,23 +96,32 @@ __device__ __forceinline__ int tp_window_count(const uint32_t* bits, int64_t w, 
     return c;
 }
 
+constexpr int TP_SUMS = 4;      // running sums of the plan, two 32-bit fields each
+
 struct TpShared {
     int64_t a[TP_BLOCK / 64];
-    int64_t base[3];
+    int64_t base[TP_SUMS];
     int32_t m[TP_BLOCK / 64];
     int32_t base_m;
 };
 
-// What a window slot adds to the three running sums (each an int64 of packed fields):
-//   sum c | sum c*c << 32
-//   windows of one, two, three tiles                (21 bits each: fewer than 2^21 window slots)
-//   windows of four tiles, of more, non-empty ones  (21 bits each)
+// What a window slot adds to the four running sums (each an int64 holding two 32-bit fields):
+//   sum c, sum c*c
+//   windows of one tile, of two tiles
+//   windows of three tiles, of four tiles
+//   windows of more than four tiles, non-empty windows
 __device__ __forceinline__ int tp_bucket(int64_t c) { return c > 0 ? min(((int)c - 1) >> 5, 4) : -1; }
-__device__ __forceinline__ void tp_items(int64_t c, int64_t (&item)[3]) {
+__device__ __forceinline__ void tp_items(int64_t c, int64_t (&item)[TP_SUMS]) {
     const int b = tp_bucket(c);
     item[0] = c | ((c * c) << 32);
-    item[1] = b >= 0 && b < 3 ? (int64_t)1 << (21 * b) : 0;
-    item[2] = (b >= 3 ? (int64_t)1 << (21 * (b - 3)) : 0) | (c > 0 ? (int64_t)1 << 42 : 0);
+    item[1] = b == 0 ? 1 : (b == 1 ? (int64_t)1 << 32 : 0);
+    item[2] = b == 2 ? 1 : (b == 3 ? (int64_t)1 << 32 : 0);
+    item[3] = (b == 4 ? 1 : 0) | (c > 0 ? (int64_t)1 << 32 : 0);
+}
+// windows of bucket b counted in the sums s
+__device__ __forceinline__ int64_t tp_bucket_count(const int64_t (&s)[TP_SUMS], int b) {
+    const int64_t word = s[1 + (b >> 1)];
+    return (b & 1) ? word >> 32 : word & 0xffffffffll;
 }
 __device__ __forceinline__ int tp_block_max(int v, TpShared& sh) {
     const int wm = wave_max_i32(v);
@@ -125,18 +134,18 @@ __device__ __forceinline__ int tp_block_max(int v, TpShared& sh) {
     return m;
 }
 
-// block sums: partial_a[3 * blk + k] = the three sums over the block's window slots, partial_b[blk] = largest c
+// block sums: partial_a[TP_SUMS * blk + k] = the sums over the block's window slots, partial_b[blk] = largest c
 __device__ __forceinline__ void tp_phase_block_sums(const TokenPlanArgs& a, int blk, TpShared& sh) {
     const int64_t w = (int64_t)blk * TP_BLOCK + threadIdx.x;
     const int64_t c = w < a.B ? tp_window_count(a.bits, w, a.W) : 0;
-    int64_t item[3], total[3];
+    int64_t item[TP_SUMS], total[TP_SUMS];
     tp_items(c, item);
 #pragma unroll
-    for (int k = 0; k < 3; ++k) (void)block_exclusive_scan<int64_t, TP_BLOCK / 64>(item[k], sh.a, &total[k]);
+    for (int k = 0; k < TP_SUMS; ++k) (void)block_exclusive_scan<int64_t, TP_BLOCK / 64>(item[k], sh.a, &total[k]);
     const int cm = tp_block_max((int)c, sh);
     if (threadIdx.x == 0) {
 #pragma unroll
-        for (int k = 0; k < 3; ++k) a.partial_a[3 * blk + k] = total[k];
+        for (int k = 0; k < TP_SUMS; ++k) a.partial_a[TP_SUMS * blk + k] = total[k];
         a.partial_b[blk] = cm;
     }
 }
@@ -154,37 +163,36 @@ __device__ __forceinline__ void tp_phase_windows(const TokenPlanArgs& a, int blk
     const int64_t w = (int64_t)blk * TP_BLOCK + threadIdx.x;
     const int64_t c = w < a.B ? tp_window_count(a.bits, w, a.W) : 0;
     // prefix of the earlier blocks
-    int64_t p[3] = {0, 0, 0};
+    int64_t p[TP_SUMS] = {0, 0, 0, 0};
     int pm = 0;
     for (int64_t i = threadIdx.x; i < blk; i += TP_BLOCK) {
 #pragma unroll
-        for (int k = 0; k < 3; ++k) p[k] += a.partial_a[3 * i + k];
+        for (int k = 0; k < TP_SUMS; ++k) p[k] += a.partial_a[TP_SUMS * i + k];
         pm = max(pm, a.partial_b[i]);
     }
-    int64_t total[3];
+    int64_t total[TP_SUMS];
 #pragma unroll
-    for (int k = 0; k < 3; ++k) (void)block_exclusive_scan<int64_t, TP_BLOCK / 64>(p[k], sh.a, &total[k]);
+    for (int k = 0; k < TP_SUMS; ++k) (void)block_exclusive_scan<int64_t, TP_BLOCK / 64>(p[k], sh.a, &total[k]);
     const int bm = tp_block_max(max(pm, (int)c), sh);            // largest c up to and including this block
     if (threadIdx.x == 0) {
 #pragma unroll
-        for (int k = 0; k < 3; ++k) sh.base[k] = total[k];
+        for (int k = 0; k < TP_SUMS; ++k) sh.base[k] = total[k];
     }
     __syncthreads();
-    int64_t item[3], e[3];
+    int64_t item[TP_SUMS], e[TP_SUMS];
     tp_items(c, item);
 #pragma unroll
-    for (int k = 0; k < 3; ++k) e[k] = block_exclusive_scan<int64_t, TP_BLOCK / 64>(item[k], sh.a, &total[k]) + sh.base[k];
-    const int32_t k = (int32_t)(e[2] >> 42);                     // non-empty windows before this one
+    for (int k = 0; k < TP_SUMS; ++k)
+        e[k] = block_exclusive_scan<int64_t, TP_BLOCK / 64>(item[k], sh.a, &total[k]) + sh.base[k];
+    const int32_t k = (int32_t)(e[3] >> 32);                     // non-empty windows before this one
     if (blk == a.blocks - 1 && threadIdx.x == 0) {
-        const int64_t t1 = sh.base[1] + total[1], t2 = sh.base[2] + total[2];
-        a.totals[0] = t2 >> 42;                                  // non-empty windows
-        a.totals[1] = sh.base[0] + total[0];                     // sum c | sum c*c << 32
-        const int64_t f = (1 << 21) - 1;
-        counters[0] = (int32_t)(t1 & f) * H;
-        counters[1] = (int32_t)((t1 >> 21) & f) * H;
-        counters[2] = (int32_t)((t1 >> 42) & f) * H;
-        counters[3] = (int32_t)(t2 & f) * H;
-        counters[4] = (int32_t)((t2 >> 21) & f) * H;
+        int64_t all[TP_SUMS];
+#pragma unroll
+        for (int q = 0; q < TP_SUMS; ++q) all[q] = sh.base[q] + total[q];
+        a.totals[0] = all[3] >> 32;                              // non-empty windows
+        a.totals[1] = all[0];                                    // sum c | sum c*c << 32
+#pragma unroll
+        for (int b = 0; b < 5; ++b) counters[b] = (int32_t)(tp_bucket_count(all, b) * H);
         counters[TPC_CMAX] = bm;
     }
     const int32_t T = (int32_t)(e[0] & 0xffffffffll);
@@ -205,8 +213,7 @@ __device__ __forceinline__ void tp_phase_windows(const TokenPlanArgs& a, int blk
     if (a.tasks == nullptr) return;
     const int b = tp_bucket(c);
     if (live && b < 4) {
-        const int64_t f = (1 << 21) - 1;
-        const int64_t slot = (b < 3 ? (e[1] >> (21 * b)) & f : e[2] & f) * H;
+        const int64_t slot = tp_bucket_count(e, b) * H;
         if (slot + H <= g_cap)
             for (int h = 0; h < H; ++h)
                 a.tasks[(int64_t)b * g_cap + slot + h] =
@@ -816,7 +823,7 @@ size_t sswin_token_plan_workspace_bytes(int64_t N, int B, int n) {
     (void)N;
     const size_t words = (size_t)B * tp_words_per_window(n);
     const size_t blocks = (size_t)tp_blocks(B);
-    return align_up(words * 4, 256) + align_up((size_t)B * 4, 256) + align_up(blocks * 24, 256) +
+    return align_up(words * 4, 256) + align_up((size_t)B * 4, 256) + align_up(blocks * 32, 256) +
            align_up(blocks * 4, 256) + 1024;
 }
 
@@ -824,7 +831,6 @@ int sswin_token_plan(const int32_t* indices, int64_t N, int B, int n, int H, int
                      int32_t* plan, int64_t g_cap, int32_t* tasks, int64_t* totals_out, void* ws,
                      size_t ws_bytes, int synchronize, void* stream) {
     SSWIN_CHECK(N >= 0 && B > 0 && n > 0 && H > 0 && H < 256, "token_plan: bad sizes");
-    SSWIN_CHECK(B < (1 << 21), "token_plan: %d window slots, the plan counts them in 21 bits", B);
     SSWIN_CHECK(totals_out, "token_plan: totals_out is null");
     for (int i = 0; i < 9; ++i) totals_out[i] = 0;
     if (N == 0) return 0;
@@ -847,7 +853,7 @@ int sswin_token_plan(const int32_t* indices, int64_t N, int B, int n, int H, int
     a.totals = cv.take<int64_t>(8);       // [0] windows, [1] sum c | sum c*c << 32, [2..7] counters
     a.bits = cv.take<uint32_t>(words);
     a.win_T = cv.take<int32_t>((size_t)B);
-    a.partial_a = cv.take<int64_t>(3 * (size_t)blocks);
+    a.partial_a = cv.take<int64_t>(4 * (size_t)blocks);
     a.partial_b = cv.take<int32_t>((size_t)blocks);
     SSWIN_CHECK(cv.ok(), "token_plan: workspace too small");
     a.plan = plan;

@@ -356,6 +356,120 @@ __global__ __launch_bounds__(256) void sorted_k_kernel(const int32_t* __restrict
     for (int ch = 0; ch < hd; ++ch) sorted_k[base + (int64_t)ch * c] = src + ch;
 }
 
+// ------------------------------------------------------------------------------------------
+// Values between voxel order and operand order.  A token tensor holds, for voxel v, the `hd` channels of head
+// h at vox[v * stride + col0 + h * hd ...]; the sorted COO operands of qkv_sparse_cuda hold them at
+//   Q, V (and any product with their structure):  hd * (H*T + h*c + i) + ch
+//   K^T:                                           hd * (H*T + h*c) + ch * c + i
+// for the voxel of rank T + i in a window of c tokens.  Both are permutations of the N*H*hd values, so the
+// gradient of a copy in one direction is the copy in the other direction: no index_add, no atomics.
+// ------------------------------------------------------------------------------------------
+// One thread per (rank, head, piece of V bytes).  to_operand: voxel rows -> operand; else operand -> voxel rows.
+template <typename V>
+__global__ __launch_bounds__(256) void qv_order_copy_kernel(const int32_t* __restrict__ order, const int32_t* __restrict__ win_T,
+                                                            const int32_t* __restrict__ win_c,
+                                                            const int32_t* __restrict__ status, int64_t N, int H,
+                                                            int pieces, char* __restrict__ vox, int64_t row_bytes,
+                                                            int64_t col0_bytes, char* __restrict__ val, bool to_operand) {
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= N * H * pieces || !pairs_valid(status, N)) return;
+    const int pc = (int)(t % pieces);
+    const int64_t rh = t / pieces;
+    const int h = (int)(rh % H);
+    const int64_t r = rh / H;
+    const int T = win_T[r], c = win_c[r];
+    const int64_t row = (int64_t)H * T + (int64_t)h * c + (r - T);
+    V* pv = reinterpret_cast<V*>(vox + (int64_t)order[r] * row_bytes + col0_bytes) + (int64_t)h * pieces + pc;
+    V* po = reinterpret_cast<V*>(val) + row * pieces + pc;
+    if (to_operand)
+        *po = *pv;
+    else
+        *pv = *po;
+}
+
+// One thread per rank and head (blockIdx.y), walking over the channels: for a fixed channel the lanes of a
+// wavefront touch runs of c consecutive operand values per window; a lane's own voxel row stays in cache
+// over the walk.
+template <typename V>
+__global__ __launch_bounds__(256) void k_order_copy_kernel(const int32_t* __restrict__ order, const int32_t* __restrict__ win_T,
+                                                           const int32_t* __restrict__ win_c,
+                                                           const int32_t* __restrict__ status, int64_t N, int H, int hd,
+                                                           char* __restrict__ vox, int64_t row_bytes, int64_t col0_bytes,
+                                                           char* __restrict__ val, bool to_operand) {
+    const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (r >= N || !pairs_valid(status, N)) return;
+    const int T = win_T[r], c = win_c[r];
+    const int h = blockIdx.y;
+    V* pv = reinterpret_cast<V*>(vox + (int64_t)order[r] * row_bytes + col0_bytes) + (int64_t)h * hd;
+    V* po = reinterpret_cast<V*>(val) + (int64_t)hd * ((int64_t)H * T + (int64_t)h * c) + (r - T);
+    if (to_operand) {
+        for (int ch0 = 0; ch0 < hd; ch0 += 8) {
+            V x[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (ch0 + u < hd) x[u] = pv[ch0 + u];
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (ch0 + u < hd) po[(int64_t)(ch0 + u) * c] = x[u];
+        }
+    } else {
+        for (int ch0 = 0; ch0 < hd; ch0 += 8) {
+            V x[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (ch0 + u < hd) x[u] = po[(int64_t)(ch0 + u) * c];
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                if (ch0 + u < hd) pv[ch0 + u] = x[u];
+        }
+    }
+}
+
+// Index matrices of the sorted operands written in place (what expand + sort + gather arrive at): idx_qv
+// rows (window, head, pos, channel) at hd * (H*T + h*c + i) + ch; idx_k rows (window, head, channel, pos) at
+// hd * (H*T + h*c) + ch * c + i.  One thread per (rank, head, channel quad).
+__global__ __launch_bounds__(256) void sorted_coo_kernel(const int32_t* __restrict__ ind, const int32_t* __restrict__ order,
+                                                         const int32_t* __restrict__ win_T, const int32_t* __restrict__ win_c,
+                                                         const int32_t* __restrict__ status, int64_t N, int H, int hd,
+                                                         int64_t E, int32_t* __restrict__ idx_qv, int32_t* __restrict__ idx_k) {
+    const int q = hd >> 2;
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= N * H * q) return;
+    if (!pairs_valid(status, N)) {                           // defined (all zero) indices for a caller that checks later
+        for (int row = 0; row < 4; ++row) {
+            if (idx_qv) *reinterpret_cast<int4*>(idx_qv + row * E + 4 * t) = make_int4(0, 0, 0, 0);
+            if (idx_k) *reinterpret_cast<int4*>(idx_k + row * E + 4 * t) = make_int4(0, 0, 0, 0);
+        }
+        return;
+    }
+    const int cq = (int)(t % q);
+    const int64_t rh = t / q;
+    const int h = (int)(rh % H);
+    const int64_t r = rh / H;
+    const int T = win_T[r], c = win_c[r];
+    const int i = (int)(r - T);
+    const int2 wp = *reinterpret_cast<const int2*>(ind + 2 * (int64_t)order[r]);
+    const int ch = 4 * cq;
+    if (idx_qv) {
+        const int64_t e = (int64_t)hd * ((int64_t)H * T + (int64_t)h * c + i) + ch;
+        *reinterpret_cast<int4*>(idx_qv + e) = make_int4(wp.x, wp.x, wp.x, wp.x);
+        *reinterpret_cast<int4*>(idx_qv + E + e) = make_int4(h, h, h, h);
+        *reinterpret_cast<int4*>(idx_qv + 2 * E + e) = make_int4(wp.y, wp.y, wp.y, wp.y);
+        *reinterpret_cast<int4*>(idx_qv + 3 * E + e) = make_int4(ch, ch + 1, ch + 2, ch + 3);
+    }
+    if (idx_k) {
+        const int64_t base = (int64_t)hd * ((int64_t)H * T + (int64_t)h * c) + i;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int64_t e = base + (int64_t)(ch + u) * c;
+            idx_k[e] = wp.x;
+            idx_k[E + e] = h;
+            idx_k[2 * E + e] = ch + u;
+            idx_k[3 * E + e] = wp.y;
+        }
+    }
+}
+
 // four 16-byte pieces per thread, each instruction of a wavefront covering 1 KB of contiguous memory
 __global__ __launch_bounds__(256) void calibration_copy_kernel(const int4* __restrict__ src, int4* __restrict__ dst, int64_t n16) {
     const int64_t base = (int64_t)blockIdx.x * 1024 + threadIdx.x;
@@ -378,7 +492,7 @@ using namespace sswin;
 extern "C" {
 
 const char* sswin_last_error(void) { return error_buffer(); }
-int sswin_abi_version(void) { return 18; }
+int sswin_abi_version(void) { return 19; }
 
 int sswin_calibration_copy(void* dst, const void* src, int64_t bytes, void* stream) {
     SSWIN_CHECK(bytes >= 0 && bytes % 16 == 0, "calibration_copy: size must be a multiple of 16 bytes");
@@ -592,6 +706,52 @@ size_t sswin_qkv_sparse_indices_workspace_bytes(int64_t N, int B, int n) {
            3 * align_up((size_t)(N > 0 ? N : 1) * 4, 256) + 256 + 1024;
 }
 
+// ranks of the voxels in (window, pos) order: order / win_T / win_c by rank, status = {pairs out of range,
+// distinct pairs}; all carved from `ws`
+struct VoxelRanks {
+    int32_t *order, *win_T, *win_c, *status;
+};
+// (`map` != NULL: in a caller's array [3N + 2] instead)
+static int build_voxel_ranks(const char* who, const int32_t* indices, int64_t N, int B, int n, void* ws, size_t ws_bytes,
+                             int32_t* map, VoxelRanks* out, hipStream_t s) {
+    Carver cv(ws, ws_bytes);
+    const size_t words = bitmap_words((int64_t)B * n + n);
+    uint32_t* bits = cv.take<uint32_t>(words);
+    int32_t* word_prefix = cv.take<int32_t>(words);
+    int32_t* tile_sums = cv.take<int32_t>((size_t)scan_num_tiles((int64_t)words));
+    out->order = map ? map : cv.take<int32_t>((size_t)N);
+    out->win_T = map ? map + N : cv.take<int32_t>((size_t)N);
+    out->win_c = map ? map + 2 * N : cv.take<int32_t>((size_t)N);
+    out->status = map ? map + 3 * N : cv.take<int32_t>(2);
+    SSWIN_CHECK(cv.ok(), "%s: workspace too small", who);
+    const unsigned fill_blocks = (unsigned)std::min<size_t>((words + 255) / 256, 4096);
+    hipLaunchKernelGGL(fill_u32_kernel, dim3(fill_blocks), dim3(256), 0, s, bits, (int64_t)words, 0u);
+    hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(256), 0, s, reinterpret_cast<uint32_t*>(out->status), (int64_t)2, 0u);
+    const unsigned nb = (unsigned)((N + 255) / 256);
+    hipLaunchKernelGGL(set_bits_pairs_kernel, dim3(nb), dim3(256), 0, s, indices, N, B, n, bits, out->status);
+    PopcLoad ld{bits};
+    ExclusiveStore st{word_prefix};
+    if (device_exclusive_scan<int32_t>(ld, st, (int64_t)words, tile_sums, out->status + 1, s, who)) return 1;
+    hipLaunchKernelGGL(voxel_rank_kernel, dim3(nb), dim3(256), 0, s, indices, N, B, n, bits, word_prefix, out->status,
+                       out->order, out->win_T, out->win_c);
+    return 0;
+}
+
+static int report_pairs(const char* who, const int32_t* status, int64_t N, int validate, int32_t* status_out, hipStream_t s) {
+    if (status_out) {                                        // the caller checks later: {out of range, distinct pairs}
+        SSWIN_HIP(hipMemcpyAsync(status_out, status, 2 * sizeof(int32_t), hipMemcpyDeviceToHost, s));
+    }
+    if (validate) {
+        int32_t back[2] = {0, 0};
+        SSWIN_HIP(hipMemcpyAsync(back, status, sizeof(back), hipMemcpyDeviceToHost, s));
+        SSWIN_HIP(hipStreamSynchronize(s));
+        SSWIN_CHECK(back[0] == 0, "%s: %d voxel indices lie outside [0, batch_size) x [0, spatial_dim)", who, back[0]);
+        SSWIN_CHECK(back[1] == N, "%s: (window, pos) pairs must be distinct: %lld voxels share a pair with another", who,
+                    (long long)(N - back[1]));
+    }
+    return 0;
+}
+
 int sswin_qkv_sparse_indices(const int32_t* indices, int64_t N, int B, int n, int H, int hd,
                              int32_t* idx_qv, int32_t* sorted_qv, int32_t* idx_k, int32_t* sorted_k,
                              void* ws, size_t ws_bytes, int validate, int32_t* status_out, void* stream) {
@@ -605,47 +765,101 @@ int sswin_qkv_sparse_indices(const int32_t* indices, int64_t N, int B, int n, in
     SSWIN_CHECK(ws_bytes >= sswin_qkv_sparse_indices_workspace_bytes(N, B, n),
                 "qkv_sparse_indices: workspace too small");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    Carver cv(ws, ws_bytes);
-    const size_t words = bitmap_words((int64_t)B * n + n);
-    uint32_t* bits = cv.take<uint32_t>(words);
-    int32_t* word_prefix = cv.take<int32_t>(words);
-    int32_t* tile_sums = cv.take<int32_t>((size_t)scan_num_tiles((int64_t)words));
-    int32_t* order = cv.take<int32_t>((size_t)N);
-    int32_t* win_T = cv.take<int32_t>((size_t)N);
-    int32_t* win_c = cv.take<int32_t>((size_t)N);
-    int32_t* status = cv.take<int32_t>(2);        // [0] pairs out of range, [1] distinct pairs
-    SSWIN_CHECK(cv.ok(), "qkv_sparse_indices: workspace too small");
-
-    const unsigned fill_blocks = (unsigned)std::min<size_t>((words + 255) / 256, 4096);
-    hipLaunchKernelGGL(fill_u32_kernel, dim3(fill_blocks), dim3(256), 0, s, bits, (int64_t)words, 0u);
-    hipLaunchKernelGGL(fill_u32_kernel, dim3(1), dim3(256), 0, s, reinterpret_cast<uint32_t*>(status), (int64_t)2, 0u);
+    VoxelRanks vr;
+    if (build_voxel_ranks("qkv_sparse_indices", indices, N, B, n, ws, ws_bytes, nullptr, &vr, s)) return 1;
     const unsigned nb = (unsigned)((N + 255) / 256);
-    hipLaunchKernelGGL(set_bits_pairs_kernel, dim3(nb), dim3(256), 0, s, indices, N, B, n, bits, status);
-    PopcLoad ld{bits};
-    ExclusiveStore st{word_prefix};
-    if (device_exclusive_scan<int32_t>(ld, st, (int64_t)words, tile_sums, status + 1, s, "qkv_sparse_indices scan")) return 1;
-    hipLaunchKernelGGL(voxel_rank_kernel, dim3(nb), dim3(256), 0, s, indices, N, B, n, bits, word_prefix, status, order,
-                       win_T, win_c);
     hipLaunchKernelGGL(expand_coo_kernel, dim3((unsigned)((E / 4 + 255) / 256)), dim3(256), 0, s, indices, E, H,
                        hd, idx_qv, idx_k);
     const int64_t qv_threads = N * H * (hd / 4);
-    hipLaunchKernelGGL(sorted_qv_kernel, dim3((unsigned)((qv_threads + 255) / 256)), dim3(256), 0, s, order,
-                       win_T, win_c, status, N, H, hd, sorted_qv);
-    hipLaunchKernelGGL(sorted_k_kernel, dim3(nb, (unsigned)H), dim3(256), 0, s, order, win_T, win_c, status, N, H, hd,
-                       sorted_k);
+    hipLaunchKernelGGL(sorted_qv_kernel, dim3((unsigned)((qv_threads + 255) / 256)), dim3(256), 0, s, vr.order,
+                       vr.win_T, vr.win_c, vr.status, N, H, hd, sorted_qv);
+    hipLaunchKernelGGL(sorted_k_kernel, dim3(nb, (unsigned)H), dim3(256), 0, s, vr.order, vr.win_T, vr.win_c, vr.status, N, H,
+                       hd, sorted_k);
     if (launch_ok("qkv_sparse_indices")) return 1;
-    if (status_out) {                                        // the caller checks later: {out of range, distinct pairs}
-        SSWIN_HIP(hipMemcpyAsync(status_out, status, 2 * sizeof(int32_t), hipMemcpyDeviceToHost, s));
+    return report_pairs("qkv_sparse_indices", vr.status, N, validate, status_out, s);
+}
+
+// ---- sorted operands without the permutations ---------------------------------------------------
+size_t sswin_operand_map_workspace_bytes(int64_t N, int B, int n) { return sswin_qkv_sparse_indices_workspace_bytes(N, B, n); }
+
+int sswin_operand_map(const int32_t* indices, int64_t N, int B, int n, int32_t* map, void* ws, size_t ws_bytes,
+                      int validate, int32_t* status_out, void* stream) {
+    SSWIN_CHECK(N >= 0 && B > 0 && n > 0, "operand_map: bad sizes");
+    SSWIN_CHECK((int64_t)B * n + n < ((int64_t)1 << 36), "operand_map: B*n too large");
+    if (N == 0) return 0;
+    SSWIN_CHECK(indices && map && ws, "operand_map: null pointer");
+    SSWIN_CHECK(N < (int64_t)INT32_MAX / 4, "operand_map: too many voxels");
+    SSWIN_CHECK(ws_bytes >= sswin_operand_map_workspace_bytes(N, B, n), "operand_map: workspace too small");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    VoxelRanks vr;
+    if (build_voxel_ranks("operand_map", indices, N, B, n, ws, ws_bytes, map, &vr, s)) return 1;
+    if (launch_ok("operand_map")) return 1;
+    return report_pairs("operand_map", vr.status, N, validate, status_out, s);
+}
+
+static int value_bytes(int dtype) { return dtype == SSWIN_F64 ? 8 : dtype == SSWIN_F32 ? 4 : 2; }
+
+int sswin_operand_copy(int dtype, int layout, int to_operand, void* vox, int64_t vox_stride, int vox_col0, void* val,
+                       const int32_t* map, int64_t N, int H, int hd, void* stream) {
+    SSWIN_CHECK(dtype >= SSWIN_F32 && dtype <= SSWIN_F64, "operand_copy: unsupported value dtype %d", dtype);
+    SSWIN_CHECK(layout == 0 || layout == 1, "operand_copy: layout must be 0 (Q, V) or 1 (K^T)");
+    SSWIN_CHECK(N >= 0 && H > 0 && hd > 0 && vox_col0 >= 0 && vox_stride >= (int64_t)vox_col0 + (int64_t)H * hd,
+                "operand_copy: bad sizes");
+    if (N == 0) return 0;
+    SSWIN_CHECK(vox && val && map, "operand_copy: null pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int esz = value_bytes(dtype);
+    const int32_t *order = map, *win_T = map + N, *win_c = map + 2 * N, *status = map + 3 * N;
+    const int64_t row_bytes = vox_stride * esz, col0_bytes = (int64_t)vox_col0 * esz;
+    char* v = static_cast<char*>(vox);
+    char* o = static_cast<char*>(val);
+    if (layout == 0) {
+        const int head_bytes = hd * esz;
+        const bool wide = head_bytes % 16 == 0 && row_bytes % 16 == 0 && col0_bytes % 16 == 0 && ((uintptr_t)vox % 16) == 0 &&
+                          ((uintptr_t)val % 16) == 0;
+        const int pieces = wide ? head_bytes / 16 : hd;
+        const int64_t threads = N * H * pieces;
+        const dim3 grid((unsigned)((threads + 255) / 256));
+        if (wide)
+            hipLaunchKernelGGL(qv_order_copy_kernel<int4>, grid, dim3(256), 0, s, order, win_T, win_c, status, N, H, pieces, v,
+                               row_bytes, col0_bytes, o, to_operand != 0);
+        else if (esz == 8)
+            hipLaunchKernelGGL(qv_order_copy_kernel<int64_t>, grid, dim3(256), 0, s, order, win_T, win_c, status, N, H, pieces, v,
+                               row_bytes, col0_bytes, o, to_operand != 0);
+        else if (esz == 4)
+            hipLaunchKernelGGL(qv_order_copy_kernel<int32_t>, grid, dim3(256), 0, s, order, win_T, win_c, status, N, H, pieces, v,
+                               row_bytes, col0_bytes, o, to_operand != 0);
+        else
+            hipLaunchKernelGGL(qv_order_copy_kernel<int16_t>, grid, dim3(256), 0, s, order, win_T, win_c, status, N, H, pieces, v,
+                               row_bytes, col0_bytes, o, to_operand != 0);
+    } else {
+        const dim3 grid((unsigned)((N + 255) / 256), (unsigned)H);
+        if (esz == 8)
+            hipLaunchKernelGGL(k_order_copy_kernel<int64_t>, grid, dim3(256), 0, s, order, win_T, win_c, status, N, H, hd, v,
+                               row_bytes, col0_bytes, o, to_operand != 0);
+        else if (esz == 4)
+            hipLaunchKernelGGL(k_order_copy_kernel<int32_t>, grid, dim3(256), 0, s, order, win_T, win_c, status, N, H, hd, v,
+                               row_bytes, col0_bytes, o, to_operand != 0);
+        else
+            hipLaunchKernelGGL(k_order_copy_kernel<int16_t>, grid, dim3(256), 0, s, order, win_T, win_c, status, N, H, hd, v,
+                               row_bytes, col0_bytes, o, to_operand != 0);
     }
-    if (validate) {
-        int32_t back[2] = {0, 0};
-        SSWIN_HIP(hipMemcpyAsync(back, status, sizeof(back), hipMemcpyDeviceToHost, s));
-        SSWIN_HIP(hipStreamSynchronize(s));
-        SSWIN_CHECK(back[0] == 0, "qkv_sparse_indices: %d voxel indices lie outside [0, batch_size) x [0, spatial_dim)", back[0]);
-        SSWIN_CHECK(back[1] == N, "qkv_sparse_indices: (window, pos) pairs must be distinct: %lld voxels share a pair with another",
-                    (long long)(N - back[1]));
-    }
-    return 0;
+    return launch_ok("operand_copy");
+}
+
+int sswin_sorted_coo_indices(const int32_t* indices, const int32_t* map, int64_t N, int H, int hd, int32_t* idx_qv,
+                             int32_t* idx_k, void* stream) {
+    SSWIN_CHECK(N >= 0 && H > 0 && hd > 0 && hd % 4 == 0, "sorted_coo_indices: bad sizes (head dim a multiple of 4)");
+    const int64_t E = N * H * hd;
+    SSWIN_CHECK(E < (int64_t)INT32_MAX, "sorted_coo_indices: N*H*hd = %lld does not fit int32", (long long)E);
+    if (N == 0) return 0;
+    SSWIN_CHECK(indices && map && (idx_qv || idx_k), "sorted_coo_indices: null pointer");
+    SSWIN_CHECK((!idx_qv || ((uintptr_t)idx_qv % 16) == 0) && (!idx_k || ((uintptr_t)idx_k % 16) == 0),
+                "sorted_coo_indices: index matrices must be 16-byte aligned");
+    const int64_t threads = N * H * (hd / 4);
+    hipLaunchKernelGGL(sorted_coo_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       indices, map, map + N, map + 2 * N, map + 3 * N, N, H, hd, E, idx_qv, idx_k);
+    return launch_ok("sorted_coo_indices");
 }
 
 }  // extern "C"

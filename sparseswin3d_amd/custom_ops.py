@@ -136,6 +136,68 @@ def return_inverse(x, maxnum=-1):
     return out, int(count.value)
 
 
+# ------------------------------------------------------------------------------------------
+# Sorted operands without the permutations (helpers of qkv_sparse_cuda and of the module's tail; not
+# operators of the reference's module)
+# ------------------------------------------------------------------------------------------
+def operand_map(indices, batch_size, spatial_dim):
+    """Rank of every voxel in (window, pos) order as an int32 tensor [3N + 2] (voxel of rank r, first rank
+    and size of its window, then the validity pair); input for :func:`operand_copy` and
+    :func:`sorted_coo_indices`.  Invalid (window, pos) pairs are reported by the next operator that waits
+    for the stream, as for ``qkv_sparse_indices(..., _defer_check=True)``."""
+    lib = _lib.load()
+    d = _dev(indices)
+    _check(indices.dim() == 2 and indices.shape[1] == 2, "operand_map: indices must be [N, 2]")
+    _check(indices.dtype == torch.int32, "operand_map: indices must be int32")
+    indices = indices.contiguous()
+    n_vox = indices.shape[0]
+    out = torch.empty(3 * n_vox + 2, dtype=torch.int32, device=d)
+    nbytes = lib.sswin_operand_map_workspace_bytes(n_vox, int(batch_size), int(spatial_dim))
+    ws = _ws(nbytes, d)
+    status = torch.zeros(2, dtype=torch.int32, pin_memory=True)
+    with torch.cuda.device(d):
+        _check_pending()
+        _lib.check(lib.sswin_operand_map(_ptr(indices), n_vox, int(batch_size), int(spatial_dim), _ptr(out), _ptr(ws),
+                                         nbytes, 0, C.c_void_p(status.data_ptr()), _stream(d)))
+        if n_vox > 0:
+            event = torch.cuda.Event()
+            event.record(torch.cuda.current_stream(d))
+            _pending.append((event, status, n_vox))
+    return out
+
+
+def operand_copy(vox, col0, val, omap, num_heads, c, layout, to_operand):
+    """Copy between a token tensor ``vox`` [N, stride] (columns ``col0 + h*c + ch``) and a sorted operand's
+    value array ``val`` [N*H*c]: layout 0 = Q/V order, 1 = K^T order; ``to_operand`` gives the direction."""
+    lib = _lib.load()
+    d = _dev(vox, val, omap)
+    _check(vox.dim() == 2 and vox.stride(1) == 1 and val.is_contiguous() and vox.dtype == val.dtype,
+           "operand_copy: vox must be [N, stride] with unit column stride and val contiguous of the same dtype")
+    _check(vox.dtype in _DTYPE_CODE, f"unsupported value dtype {vox.dtype}")
+    n_vox = vox.shape[0]
+    _check(omap.numel() == 3 * n_vox + 2 and val.numel() == n_vox * num_heads * c, "operand_copy: sizes do not match")
+    with torch.cuda.device(d):
+        _lib.check(lib.sswin_operand_copy(_DTYPE_CODE[vox.dtype], int(layout), 1 if to_operand else 0, _ptr(vox),
+                                          vox.stride(0), int(col0), _ptr(val), _ptr(omap), n_vox, int(num_heads), int(c),
+                                          _stream(d)))
+
+
+def sorted_coo_indices(indices, omap, num_heads, c):
+    """The sorted [4, E] index matrices of Q/V and of K^T (``idx.index_select(1, order)`` of
+    :func:`qkv_sparse_indices`), written directly."""
+    lib = _lib.load()
+    d = _dev(indices, omap)
+    indices = indices.contiguous()
+    n_vox = indices.shape[0]
+    e = n_vox * num_heads * c
+    idx_qv = torch.empty((4, e), dtype=torch.int32, device=d)
+    idx_k = torch.empty((4, e), dtype=torch.int32, device=d)
+    with torch.cuda.device(d):
+        _lib.check(lib.sswin_sorted_coo_indices(_ptr(indices), _ptr(omap), n_vox, int(num_heads), int(c), _ptr(idx_qv),
+                                                _ptr(idx_k), _stream(d)))
+    return idx_qv, idx_k
+
+
 # Input checks whose verdict is still on its way from the GPU: (event, pinned status, voxel count).  An
 # operator that has just waited for the stream anyway looks at them (:func:`_check_pending`).
 _pending = []

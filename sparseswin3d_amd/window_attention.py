@@ -180,16 +180,73 @@ def softmax_last_dim(mat: SparseTensor) -> SparseTensor:
 # ------------------------------------------------------------------------------------------
 # glue around the operators
 # ------------------------------------------------------------------------------------------
+class _SortedOperandValues(Function):
+    """Values of Q, K^T, V in sorted operand order from ``qkv`` [N, 3, H, hd].  The reference gathers them
+    through the permutations of ``qkv_sparse_indices`` (swin3d_base.py:483-498) and autograd returns the
+    gradients through ``index_add``; the same permutations applied directly, in both directions."""
+
+    @staticmethod
+    def forward(ctx, qkv, omap):
+        n_vox, _, num_heads, c = qkv.shape
+        flat = qkv.contiguous().view(n_vox, 3 * num_heads * c)
+        out = [torch.empty(n_vox * num_heads * c, dtype=qkv.dtype, device=qkv.device) for _ in range(3)]
+        for slot, (val, layout) in enumerate(zip(out, (0, 1, 0))):
+            ops.operand_copy(flat, slot * num_heads * c, val, omap, num_heads, c, layout, True)
+        ctx.save_for_backward(omap)
+        ctx.shape = qkv.shape
+        return tuple(out)
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, d_q, d_k, d_v):
+        (omap,) = ctx.saved_tensors
+        n_vox, _, num_heads, c = ctx.shape
+        d_qkv = torch.empty(ctx.shape, dtype=d_q.dtype, device=d_q.device)
+        flat = d_qkv.view(n_vox, 3 * num_heads * c)
+        for slot, (val, layout) in enumerate(zip((d_q, d_k, d_v), (0, 1, 0))):
+            ops.operand_copy(flat, slot * num_heads * c, val.contiguous(), omap, num_heads, c, layout, False)
+        return d_qkv, None
+
+
+class _OperandToVoxels(Function):
+    """Values of a [B, H, n, hd] product in Q/V order -> token rows [N, H*hd] in voxel order: what
+    ``permute((0, 2, 1, 3))``, ``return_inverse`` and ``index_select`` arrive at in the reference
+    (swin3d_base.py:672-675)."""
+
+    @staticmethod
+    def forward(ctx, val, omap, num_heads, c):
+        n_vox = (omap.numel() - 2) // 3
+        out = torch.empty(n_vox, num_heads * c, dtype=val.dtype, device=val.device)
+        ops.operand_copy(out, 0, val.contiguous(), omap, num_heads, c, 0, False)
+        ctx.save_for_backward(omap)
+        ctx.heads = (num_heads, c)
+        return out
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad):
+        (omap,) = ctx.saved_tensors
+        num_heads, c = ctx.heads
+        grad = grad.contiguous()
+        d_val = torch.empty(grad.numel(), dtype=grad.dtype, device=grad.device)
+        ops.operand_copy(grad, 0, d_val, omap, num_heads, c, 0, True)
+        return d_val, None, None, None
+
+
 def qkv_sparse_cuda(qkv: torch.Tensor, indices: torch.Tensor, batch_size: int, spatial_shape):
-    """Sorted COO operands Q [B,H,n,hd], K^T [B,H,hd,n], V [B,H,n,hd] from ``qkv`` [N,3,H,hd]."""
+    """Sorted COO operands Q [B,H,n,hd], K^T [B,H,hd,n], V [B,H,n,hd] from ``qkv`` [N,3,H,hd]
+    (reference swin3d_base.py:483-498: same tensors; the index matrices and values are written in sorted
+    order directly instead of being expanded, hashed, sorted and gathered).  The returned tensors carry
+    ``operand_map``, which :class:`_OperandToVoxels` takes to bring a product back to voxel order."""
     num_heads, c = qkv.shape[2:]
     n = spatial_shape
-    idx_qv, order_qv, idx_k, order_k = ops.qkv_sparse_indices(indices, batch_size, n, num_heads, c, _defer_check=True)
-    idx_qv = idx_qv.index_select(1, order_qv)
-    idx_k = idx_k.index_select(1, order_k)
-    q = SparseTensor(idx_qv, qkv[:, 0].reshape(-1).index_select(0, order_qv), [batch_size, num_heads, n, c])
-    k_t = SparseTensor(idx_k, qkv[:, 1].reshape(-1).index_select(0, order_k), [batch_size, num_heads, c, n])
-    v = SparseTensor(idx_qv, qkv[:, 2].reshape(-1).index_select(0, order_qv), [batch_size, num_heads, n, c])
+    omap = ops.operand_map(indices, batch_size, n)
+    idx_qv, idx_k = ops.sorted_coo_indices(indices, omap, num_heads, c)
+    q_val, k_val, v_val = _SortedOperandValues.apply(qkv, omap)
+    q = SparseTensor(idx_qv, q_val, [batch_size, num_heads, n, c])
+    k_t = SparseTensor(idx_k, k_val, [batch_size, num_heads, c, n])
+    v = SparseTensor(idx_qv, v_val, [batch_size, num_heads, n, c])
+    q.operand_map = k_t.operand_map = v.operand_map = omap
     return q, k_t, v
 
 
@@ -526,8 +583,14 @@ class WindowAttentionSparse(nn.Module):
         if mask is not None:
             attn = sp_add_mask(attn, mask)
         attn = softmax_last_dim(attn)
-        out = spspmm_block_naive(attn, v, "qk_v").permute((0, 2, 1, 3))      # (window, pos, head, ch)
-        # the keys are below b * n: passing that bound spares return_inverse its search for the maximum
-        unsort = ops.return_inverse(ops.flatten_indices(x.indices.T.contiguous(), [b, n]), b * n)[0]
-        x = replace_feature(x, out.values.reshape(x.features.shape).index_select(0, unsort))
+        out = spspmm_block_naive(attn, v, "qk_v")
+        omap = getattr(v, "operand_map", None)
+        if omap is not None:
+            # the product has V's structure: one copy takes its values from operand order to voxel rows
+            x = replace_feature(x, _OperandToVoxels.apply(out.values, omap, self.num_heads, c // self.num_heads))
+        else:
+            out = out.permute((0, 2, 1, 3))                                  # (window, pos, head, ch)
+            # the keys are below b * n: passing that bound spares return_inverse its search for the maximum
+            unsort = ops.return_inverse(ops.flatten_indices(x.indices.T.contiguous(), [b, n]), b * n)[0]
+            x = replace_feature(x, out.values.reshape(x.features.shape).index_select(0, unsort))
         return replace_feature(x, self.proj_drop(tall_linear(x.features, self.proj)))
