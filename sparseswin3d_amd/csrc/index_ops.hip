@@ -425,21 +425,89 @@ __global__ __launch_bounds__(256) void k_order_copy_kernel(const int32_t* __rest
     }
 }
 
+// The same through LDS for head slices of whole 16-byte pieces: a workgroup takes 64 consecutive ranks of one
+// head (blockIdx.y); voxel rows are touched in whole slices (hd * sizeof(V) contiguous bytes, 16 per lane) and
+// the operand in runs of consecutive ranks per channel, so both sides of the copy are coalesced.
+template <typename V, int HD>
+__global__ __launch_bounds__(256) void k_order_copy_lds_kernel(const int32_t* __restrict__ order, const int32_t* __restrict__ win_T,
+                                                               const int32_t* __restrict__ win_c,
+                                                               const int32_t* __restrict__ status, int64_t N, int H,
+                                                               char* __restrict__ vox, int64_t row_bytes, int64_t col0_bytes,
+                                                               char* __restrict__ val, bool to_operand) {
+    constexpr int PER16 = 16 / (int)sizeof(V);               // values per 16-byte piece
+    constexpr int PIECES = HD / PER16;                       // pieces per head slice
+    constexpr int ROWS_PER_PASS = 256 / PIECES;
+    __shared__ V tile[64][HD + 1];
+    __shared__ int64_t s_base[64];                           // operand position of (rank, channel 0)
+    __shared__ int32_t s_c[64];
+    __shared__ int32_t s_vox[64];
+    if (!pairs_valid(status, N)) return;
+    const int64_t r0 = (int64_t)blockIdx.x * 64;
+    const int h = blockIdx.y;
+    const int tid = threadIdx.x;
+    if (tid < 64) {
+        const int64_t r = r0 + tid;
+        if (r < N) {
+            const int T = win_T[r], c = win_c[r];
+            s_base[tid] = (int64_t)HD * ((int64_t)H * T + (int64_t)h * c) + (r - T);
+            s_c[tid] = c;
+            s_vox[tid] = order[r];
+        } else {
+            s_c[tid] = 0;
+        }
+    }
+    __syncthreads();
+    V* o = reinterpret_cast<V*>(val);
+    const int lane_r = tid & 63, ch0 = tid >> 6;             // operand side: 64 ranks x 4 channels per pass
+    const int piece = tid % PIECES, prow = tid / PIECES;     // voxel side: rows x 16-byte pieces
+    if (to_operand) {
+        for (int rr = prow; rr < 64; rr += ROWS_PER_PASS) {
+            if (s_c[rr] == 0) continue;
+            const int4 x = *reinterpret_cast<const int4*>(vox + (int64_t)s_vox[rr] * row_bytes + col0_bytes +
+                                                          ((int64_t)h * HD + piece * PER16) * sizeof(V));
+            const V* xv = reinterpret_cast<const V*>(&x);
+#pragma unroll
+            for (int u = 0; u < PER16; ++u) tile[rr][piece * PER16 + u] = xv[u];
+        }
+        __syncthreads();
+        const int c = s_c[lane_r];
+        if (c > 0) {
+            const int64_t base = s_base[lane_r];
+#pragma unroll 4
+            for (int ch = ch0; ch < HD; ch += 4) o[base + (int64_t)ch * c] = tile[lane_r][ch];
+        }
+    } else {
+        const int c = s_c[lane_r];
+        if (c > 0) {
+            const int64_t base = s_base[lane_r];
+#pragma unroll 4
+            for (int ch = ch0; ch < HD; ch += 4) tile[lane_r][ch] = o[base + (int64_t)ch * c];
+        }
+        __syncthreads();
+        for (int rr = prow; rr < 64; rr += ROWS_PER_PASS) {
+            if (s_c[rr] == 0) continue;
+            int4 x;
+            V* xv = reinterpret_cast<V*>(&x);
+#pragma unroll
+            for (int u = 0; u < PER16; ++u) xv[u] = tile[rr][piece * PER16 + u];
+            *reinterpret_cast<int4*>(vox + (int64_t)s_vox[rr] * row_bytes + col0_bytes +
+                                     ((int64_t)h * HD + piece * PER16) * sizeof(V)) = x;
+        }
+    }
+}
+
 // Index matrices of the sorted operands written in place (what expand + sort + gather arrive at): idx_qv
 // rows (window, head, pos, channel) at hd * (H*T + h*c + i) + ch; idx_k rows (window, head, channel, pos) at
-// hd * (H*T + h*c) + ch * c + i.  One thread per (rank, head, channel quad).
+// hd * (H*T + h*c) + ch * c + i.  idx_qv: one thread per (rank, head, channel quad), 16-byte stores.
 __global__ __launch_bounds__(256) void sorted_coo_kernel(const int32_t* __restrict__ ind, const int32_t* __restrict__ order,
                                                          const int32_t* __restrict__ win_T, const int32_t* __restrict__ win_c,
                                                          const int32_t* __restrict__ status, int64_t N, int H, int hd,
-                                                         int64_t E, int32_t* __restrict__ idx_qv, int32_t* __restrict__ idx_k) {
+                                                         int64_t E, int32_t* __restrict__ idx_qv) {
     const int q = hd >> 2;
     const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (t >= N * H * q) return;
     if (!pairs_valid(status, N)) {                           // defined (all zero) indices for a caller that checks later
-        for (int row = 0; row < 4; ++row) {
-            if (idx_qv) *reinterpret_cast<int4*>(idx_qv + row * E + 4 * t) = make_int4(0, 0, 0, 0);
-            if (idx_k) *reinterpret_cast<int4*>(idx_k + row * E + 4 * t) = make_int4(0, 0, 0, 0);
-        }
+        for (int row = 0; row < 4; ++row) *reinterpret_cast<int4*>(idx_qv + row * E + 4 * t) = make_int4(0, 0, 0, 0);
         return;
     }
     const int cq = (int)(t % q);
@@ -450,23 +518,37 @@ __global__ __launch_bounds__(256) void sorted_coo_kernel(const int32_t* __restri
     const int i = (int)(r - T);
     const int2 wp = *reinterpret_cast<const int2*>(ind + 2 * (int64_t)order[r]);
     const int ch = 4 * cq;
-    if (idx_qv) {
-        const int64_t e = (int64_t)hd * ((int64_t)H * T + (int64_t)h * c + i) + ch;
-        *reinterpret_cast<int4*>(idx_qv + e) = make_int4(wp.x, wp.x, wp.x, wp.x);
-        *reinterpret_cast<int4*>(idx_qv + E + e) = make_int4(h, h, h, h);
-        *reinterpret_cast<int4*>(idx_qv + 2 * E + e) = make_int4(wp.y, wp.y, wp.y, wp.y);
-        *reinterpret_cast<int4*>(idx_qv + 3 * E + e) = make_int4(ch, ch + 1, ch + 2, ch + 3);
+    const int64_t e = (int64_t)hd * ((int64_t)H * T + (int64_t)h * c + i) + ch;
+    *reinterpret_cast<int4*>(idx_qv + e) = make_int4(wp.x, wp.x, wp.x, wp.x);
+    *reinterpret_cast<int4*>(idx_qv + E + e) = make_int4(h, h, h, h);
+    *reinterpret_cast<int4*>(idx_qv + 2 * E + e) = make_int4(wp.y, wp.y, wp.y, wp.y);
+    *reinterpret_cast<int4*>(idx_qv + 3 * E + e) = make_int4(ch, ch + 1, ch + 2, ch + 3);
+}
+
+// idx_k: one thread per rank and head (blockIdx.y), walking over the channels, so that the lanes of a wavefront
+// write runs of consecutive positions
+__global__ __launch_bounds__(256) void sorted_coo_k_kernel(const int32_t* __restrict__ ind, const int32_t* __restrict__ order,
+                                                           const int32_t* __restrict__ win_T, const int32_t* __restrict__ win_c,
+                                                           const int32_t* __restrict__ status, int64_t N, int H, int hd,
+                                                           int64_t E, int32_t* __restrict__ idx_k) {
+    const int64_t r = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (r >= N) return;
+    const int h = blockIdx.y;
+    if (!pairs_valid(status, N)) {                           // defined (all zero) indices for a caller that checks later
+        for (int row = 0; row < 4; ++row)
+            for (int ch = 0; ch < hd; ++ch) idx_k[row * E + ((int64_t)h * N + r) * hd + ch] = 0;
+        return;
     }
-    if (idx_k) {
-        const int64_t base = (int64_t)hd * ((int64_t)H * T + (int64_t)h * c) + i;
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int64_t e = base + (int64_t)(ch + u) * c;
-            idx_k[e] = wp.x;
-            idx_k[E + e] = h;
-            idx_k[2 * E + e] = ch + u;
-            idx_k[3 * E + e] = wp.y;
-        }
+    const int T = win_T[r], c = win_c[r];
+    const int2 wp = *reinterpret_cast<const int2*>(ind + 2 * (int64_t)order[r]);
+    const int64_t base = (int64_t)hd * ((int64_t)H * T + (int64_t)h * c) + (r - T);
+#pragma unroll 4
+    for (int ch = 0; ch < hd; ++ch) {
+        const int64_t e = base + (int64_t)ch * c;
+        idx_k[e] = wp.x;
+        idx_k[E + e] = h;
+        idx_k[2 * E + e] = ch;
+        idx_k[3 * E + e] = wp.y;
     }
 }
 
@@ -833,6 +915,28 @@ int sswin_operand_copy(int dtype, int layout, int to_operand, void* vox, int64_t
             hipLaunchKernelGGL(qv_order_copy_kernel<int16_t>, grid, dim3(256), 0, s, order, win_T, win_c, status, N, H, pieces, v,
                                row_bytes, col0_bytes, o, to_operand != 0);
     } else {
+        const bool wide = row_bytes % 16 == 0 && col0_bytes % 16 == 0 && ((uintptr_t)vox % 16) == 0 && (hd * esz) % 16 == 0;
+        const dim3 grid64((unsigned)((N + 63) / 64), (unsigned)H);
+#define SSWIN_K_LDS(V, HD)                                                                                              \
+    hipLaunchKernelGGL((k_order_copy_lds_kernel<V, HD>), grid64, dim3(256), 0, s, order, win_T, win_c, status, N, H, v,   \
+                       row_bytes, col0_bytes, o, to_operand != 0)
+        if (wide && esz == 4 && hd == 32) {
+            SSWIN_K_LDS(int32_t, 32);
+            return launch_ok("operand_copy");
+        }
+        if (wide && esz == 4 && hd == 16) {
+            SSWIN_K_LDS(int32_t, 16);
+            return launch_ok("operand_copy");
+        }
+        if (wide && esz == 2 && hd == 32) {
+            SSWIN_K_LDS(int16_t, 32);
+            return launch_ok("operand_copy");
+        }
+        if (wide && esz == 2 && hd == 16) {
+            SSWIN_K_LDS(int16_t, 16);
+            return launch_ok("operand_copy");
+        }
+#undef SSWIN_K_LDS
         const dim3 grid((unsigned)((N + 255) / 256), (unsigned)H);
         if (esz == 8)
             hipLaunchKernelGGL(k_order_copy_kernel<int64_t>, grid, dim3(256), 0, s, order, win_T, win_c, status, N, H, hd, v,
@@ -857,8 +961,13 @@ int sswin_sorted_coo_indices(const int32_t* indices, const int32_t* map, int64_t
     SSWIN_CHECK((!idx_qv || ((uintptr_t)idx_qv % 16) == 0) && (!idx_k || ((uintptr_t)idx_k % 16) == 0),
                 "sorted_coo_indices: index matrices must be 16-byte aligned");
     const int64_t threads = N * H * (hd / 4);
-    hipLaunchKernelGGL(sorted_coo_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, static_cast<hipStream_t>(stream),
-                       indices, map, map + N, map + 2 * N, map + 3 * N, N, H, hd, E, idx_qv, idx_k);
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (idx_qv)
+        hipLaunchKernelGGL(sorted_coo_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, s, indices, map, map + N,
+                           map + 2 * N, map + 3 * N, N, H, hd, E, idx_qv);
+    if (idx_k)
+        hipLaunchKernelGGL(sorted_coo_k_kernel, dim3((unsigned)((N + 255) / 256), (unsigned)H), dim3(256), 0, s, indices, map,
+                           map + N, map + 2 * N, map + 3 * N, N, H, hd, E, idx_k);
     return launch_ok("sorted_coo_indices");
 }
 
