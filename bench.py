@@ -215,19 +215,29 @@ def kernel_table(wl, reps=20, only=None):
         perm_idx = o_idx[[0, 2, 1, 3], :].contiguous()
         flat_perm = ops.flatten_indices(perm_idx, [o_shape[0], o_shape[2], o_shape[1], o_shape[3]])
 
+        # operands straight from the voxel ranks (what qkv_sparse_cuda and the module's tail run)
+        omap = ops.operand_map(b["idx"], b["slots"], b["n"])
+        feat_rows = torch.randn(N, D, device=dev)
+        qkv_rows = qkv.view(N, 3 * D)
+        val_e = torch.empty(E, device=dev)
+
         entries = [
-            # name, callable, algorithmic bytes, calls per attention fwd+bwd
-            ("qkv_sparse_indices", lambda: ops.qkv_sparse_indices(b["idx"], b["slots"], b["n"], H, hd, _defer_check=True), 8 * N + 40 * E, 1),
-            ("plan_from_indices", lambda: _lib.check(lib.sswin_plan_from_indices(ptr(q.indices), m, hd, ptr(plan), g_cap, totals, ptr(ws), nb, stream)), 0, 2),
+            # name, callable, algorithmic bytes, calls per attention fwd+bwd of the module (0: not on the module's path)
+            ("operand_map [N]", lambda: ops.operand_map(b["idx"], b["slots"], b["n"]), 20 * N, 1),
+            ("sorted_coo_indices [4,E] x 2", lambda: ops.sorted_coo_indices(b["idx"], omap, H, hd), 32 * E + 20 * N, 1),
+            ("operand_copy Q/V order", lambda: ops.operand_copy(qkv_rows, 2 * D, val_e, omap, H, hd, 0, True), 2 * s * E, 6),
+            ("operand_copy K^T order", lambda: ops.operand_copy(qkv_rows, D, val_e, omap, H, hd, 1, True), 2 * s * E, 2),
+            ("qkv_sparse_indices (reference operator)", lambda: ops.qkv_sparse_indices(b["idx"], b["slots"], b["n"], H, hd, _defer_check=True), 8 * N + 40 * E, 0),
+            ("plan_from_indices", lambda: _lib.check(lib.sswin_plan_from_indices(ptr(q.indices), m, hd, ptr(plan), g_cap, totals, ptr(ws), nb, stream)), 0, 1),
             ("block_matmul q_k", mm(0, q.values, kt.values, q.indices, out_s, out_si, A), 2 * s * E + (s + 16) * A + 4 * G, 1),
             ("flatten_indices [3,A]", lambda: ops.flatten_indices(s_idx[:3], s_shape[:3]), 16 * A, 1),
             ("unique_consecutive_indices [A]", lambda: ops.unique_consecutive_indices(flat), 8 * A, 1),
             ("softmax_last_dim_forward", lambda: ops.softmax_last_dim_forward(rows, s_val), 12 * A, 1),
             ("block_matmul qk_v", mm(1, p_val, v.values, v.indices, out_o, out_oi, E), s * A + s * E + (s + 16) * E + 4 * G, 1),
-            ("permute order from the group structure [E]", lambda: ops.permute_heads_order(o_idx, o_shape), 0, 1),
+            ("permute order from the group structure [E]", lambda: ops.permute_heads_order(o_idx, o_shape), 0, 0),
             ("flatten_indices [4,E] (generic permute)", lambda: ops.flatten_indices(perm_idx, [o_shape[0], o_shape[2], o_shape[1], o_shape[3]]), 0, 0),
             ("sort_indices [E] (generic permute)", lambda: ops.sort_indices(flat_perm), 0, 0),
-            ("return_inverse [N]", lambda: ops.return_inverse(flat_tok, b["slots"] * b["n"]), 0, 1),
+            ("return_inverse [N]", lambda: ops.return_inverse(flat_tok, b["slots"] * b["n"]), 0, 0),
             ("softmax_last_dim_backward", lambda: ops.softmax_last_dim_backward(rows, p_val, g_s), 16 * A, 1),
             ("grad rc_cr", grad(0, g_o, v.values, tmp_a), 2 * s * E + s * A, 1),
             ("grad rr_rc", grad(1, g_s, kt.values, tmp_e), s * A + 2 * s * E, 2),
@@ -348,6 +358,30 @@ def kernel_table(wl, reps=20, only=None):
         table += measure(stage_entries(wl), "stage")
         table += measure(projection_entries(wl), "projections")
     return table, sizes
+
+
+def module_times(wl, reps=10):
+    """One attention module call, forward + backward (projections and torch glue included), on each of the
+    three paths: HIP events around the whole call, regular windows."""
+    from sparseswin3d_amd.window_attention import SparseVoxelTensor
+    if wl["dtype"] != torch.float32:
+        return {}
+    b = wl["blocks"][0]
+    attn = b["attn"]
+    keep = (attn.fused, attn.resident)
+
+    def once():
+        attn.zero_grad(set_to_none=True)
+        x = wl["feats"].detach().requires_grad_(True)
+        out = attn(SparseVoxelTensor(x, b["idx"], (b["n"],), b["slots"]), None).features
+        out.backward(wl["upstream"])
+
+    out = {}
+    for name, fused_, resident in (("resident", True, True), ("fused", True, False), ("operators", False, None)):
+        attn.fused, attn.resident = fused_, resident
+        out[name] = round(event_time_ms(once, reps), 4)
+    attn.fused, attn.resident = keep
+    return out
 
 
 def stage_entries(wl):
@@ -660,6 +694,8 @@ def main():
                                     frac=round(tflops / MFMA_PEAK_TFLOPS[dtype_name], 4), flops=dom["flops"],
                                     note="algorithmic flops: 2 c^2 hd per product and group, padding of the 32-token tiles not counted")
         roofline["path_summaries"] = summary
+        roofline["module_call_ms"] = module_times(wl)
+        log(f"one module call forward+backward by path (ms, projections and glue included): {roofline['module_call_ms']}")
         if args.kernels_json:
             with open(args.kernels_json, "w") as f:
                 json.dump(dict(sizes=sizes, kernels=table), f, indent=1)

@@ -591,6 +591,138 @@ __device__ __forceinline__ void fwd_task(const WAttnCommon& a, const GroupCtx& g
 }
 
 
+// ------------------------------------------------------------------------------------------
+// forward of a group of at most 16 tokens (fp32) on 16 x 16 tiles: v_mfma_f32_16x16x4_f32 instead of the
+// 32 x 32 x 2 instruction, whose tile would be three quarters padding for such a group.  S^T = K Q^T takes 8
+// matrix steps of 32 cycles instead of 16 of 64, P V two blocks of 4 steps instead of up to 8 steps of 64, and the
+// softmax works on 4 scores per lane instead of 16.
+// Lane l: column col = l % 16, slice g = l / 16.  An operand's reduction index may be permuted freely as long
+// as A and B use the same permutation: for S^T slice g carries channels 8g .. 8g + 7 (two 16-byte LDS reads
+// per operand), for P V it carries keys 4g .. 4g + 3 - exactly the keys whose scores the lane's accumulator
+// holds, so P goes from the accumulator into the second product without leaving its registers.
+// ------------------------------------------------------------------------------------------
+typedef float f32x4_v __attribute__((ext_vector_type(4)));
+
+template <bool MASK>
+__device__ __forceinline__ void fwd_task_small(const WAttnCommon& a, const GroupCtx& g, const FwdIdx& fi, float* tile,
+                                               float* tile_x, uint32_t* tab_key, uint32_t* tab_inv,
+                                               const TokenTensor32& tq, const TokenTensor32& tk, const TokenTensor32& tv,
+                                               const TokenTensor32& to, float* __restrict__ lse) {
+    const int lane = threadIdx.x & 63;
+    const int col = lane & 15, sl = lane >> 4;
+    const int c = g.c, h = g.h;
+    const int8_t* mrow = MASK ? a.mask + (int64_t)(g.w % a.nmw) * a.n : nullptr;
+    // token col of the group (clamped): query of this lane's column and one of its keys' rows
+    const uint32_t vox = (uint32_t)__shfl((int)fi.vox_i, col, 64);       // lanes 0-31 of fi hold tokens 0-31
+    const int pos = __shfl(fi.pos_i, col, 64);
+    const int reg = MASK ? mrow[pos] : 0;
+    u32x4_a rq[2], rk[2], rv[2];
+    const char* qbase = head_base<float>(tq, h);
+    const char* kbase = head_base<float>(tk, h);
+    const char* vbase = head_base<float>(tv, h);
+    const uint32_t qpitch = pitch_of<float>(tq), kpitch = pitch_of<float>(tk), vpitch = pitch_of<float>(tv);
+#pragma unroll
+    for (int v = 0; v < 2; ++v) {                            // eight rows per instruction, 16 bytes per lane
+        const uint32_t vr = (uint32_t)__shfl((int)vox, v * 8 + lane / 8, 64);
+        const uint32_t off = (uint32_t)(lane % 8) * 16u;
+        rq[v] = *reinterpret_cast<const u32x4_a*>(qbase + (__umul24(vr, qpitch) + off));
+        rk[v] = *reinterpret_cast<const u32x4_a*>(kbase + (__umul24(vr, kpitch) + off));
+        rv[v] = *reinterpret_cast<const u32x4_a*>(vbase + (__umul24(vr, vpitch) + off));
+    }
+    uint32_t pk = (uint32_t)pos * 4u;
+    if (MASK) pk |= (uint32_t)reg << 16;
+    __builtin_amdgcn_wave_barrier();
+    if (sl == 0) tab_key[col] = pk;
+    float* tile_k = tile_x + 16 * TILE_LD;                   // rows 16-31 of the second tile hold K
+#pragma unroll
+    for (int v = 0; v < 2; ++v) {
+        const int at = (v * 8 + lane / 8) * TILE_LD + (lane % 8) * 4;
+        *reinterpret_cast<u32x4_a*>(tile_x + at) = rq[v];
+        *reinterpret_cast<u32x4_a*>(tile_k + at) = rk[v];
+        *reinterpret_cast<u32x4_a*>(tile + at) = rv[v];
+    }
+    __builtin_amdgcn_wave_barrier();
+    // bias gathers first: keys 4 sl .. 4 sl + 3 of query col
+    const u32x4_a pkq = *reinterpret_cast<const u32x4_a*>(tab_key + 4 * sl);
+    const uint32_t pkr[4] = {pkq.x, pkq.y, pkq.z, pkq.w};
+    const char* bias_h = reinterpret_cast<const char*>(a.bias + (int64_t)h * a.n * a.n);
+    const uint32_t brow = (uint32_t)(pos * a.n) * 4u;
+    float bv[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) bv[r] = *reinterpret_cast<const float*>(bias_h + (brow + (MASK ? (pkr[r] & 0xffffu) : pkr[r])));
+    float qb[8], ka[8];
+    {
+        const f32x4_a* pq = reinterpret_cast<const f32x4_a*>(tile_x + col * TILE_LD + 8 * sl);
+        const f32x4_a* pk4 = reinterpret_cast<const f32x4_a*>(tile_k + col * TILE_LD + 8 * sl);
+#pragma unroll
+        for (int v = 0; v < 2; ++v) {
+            const f32x4_a x = pq[v], y = pk4[v];
+            qb[4 * v] = x.x; qb[4 * v + 1] = x.y; qb[4 * v + 2] = x.z; qb[4 * v + 3] = x.w;
+            ka[4 * v] = y.x; ka[4 * v + 1] = y.y; ka[4 * v + 2] = y.z; ka[4 * v + 3] = y.w;
+        }
+    }
+    const float qscale = a.scale * LOG2E;
+    f32x4_v S = {0, 0, 0, 0};                                // S^T[key 4 sl + r][query col]
+#pragma unroll
+    for (int m = 0; m < 8; ++m) S = __builtin_amdgcn_mfma_f32_16x16x4f32(ka[m], qb[m] * qscale, S, 0, 0, 0);
+    float vb[2][4];                                          // V[key 4 sl + r][channel 16 b + col]
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        vb[0][r] = tile[(4 * sl + r) * TILE_LD + col];
+        vb[1][r] = tile[(4 * sl + r) * TILE_LD + 16 + col];
+    }
+    float mx = 0.f;                                          // the operator's max(0, rowmax)
+    float sc[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        float x = fmaf(bv[r], LOG2E, S[r]);
+        if (MASK && (int)(pkr[r] >> 16) != reg) x += -100.0f * LOG2E;
+        x = 4 * sl + r < c ? x : -INFINITY;
+        sc[r] = x;
+        mx = fmaxf(mx, x);
+    }
+    mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+    mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+    float l = 0.f;
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        sc[r] = exp2_fast(sc[r] - mx);
+        l += sc[r];
+    }
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    l += 1e-8f;
+    if (sl == 0 && col < c) lse[(int64_t)a.H * g.Tk + h * c + col] = (mx + __builtin_amdgcn_logf(l)) * LN2;
+    f32x4_v o0 = {0, 0, 0, 0}, o1 = {0, 0, 0, 0};            // O[query 4 sl + r][channel col], [16 + col]
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+        if (m > 0 && m >= c) break;                          // step m carries keys m, 4 + m, 8 + m, 12 + m
+        // step m of slice sl carries key 4 sl + m: A = P[query col][that key], B = V[that key][channel]
+        o0 = __builtin_amdgcn_mfma_f32_16x16x4f32(sc[m], vb[0][m], o0, 0, 0, 0);
+        o1 = __builtin_amdgcn_mfma_f32_16x16x4f32(sc[m], vb[1][m], o1, 0, 0, 0);
+    }
+    __builtin_amdgcn_wave_barrier();
+    if (sl == 0) tab_inv[col] = f2u(1.0f / l);
+    __builtin_amdgcn_wave_barrier();
+    const u32x4_a iv = *reinterpret_cast<const u32x4_a*>(tab_inv + 4 * sl);
+    const float inv[4] = {u2f(iv.x), u2f(iv.y), u2f(iv.z), u2f(iv.w)};
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        tile[(4 * sl + r) * TILE_LD + col] = o0[r] * inv[r];
+        tile[(4 * sl + r) * TILE_LD + 16 + col] = o1[r] * inv[r];
+    }
+    __builtin_amdgcn_wave_barrier();
+    char* obase = const_cast<char*>(head_base<float>(to, h));
+    const uint32_t opitch = pitch_of<float>(to);
+#pragma unroll
+    for (int v = 0; v < 2; ++v) {
+        const int R = v * 8 + lane / 8;
+        const uint32_t vr = (uint32_t)__shfl((int)vox, R, 64);
+        const u32x4_a x = *reinterpret_cast<const u32x4_a*>(tile + R * TILE_LD + (lane % 8) * 4);
+        if (R < c) *reinterpret_cast<u32x4_a*>(obase + (__umul24(vr, opitch) + (uint32_t)(lane % 8) * 16u)) = x;
+    }
+}
+
 template <typename T, bool MASK>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void wattn_fwd_kernel(WAttnCommon a, TokenTensor32 tq, TokenTensor32 tk,
                                                         TokenTensor32 tv, TokenTensor32 to,
@@ -603,6 +735,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     if (!locate(a, (int64_t)blockIdx.x * 4 + wave, d, bi)) return;
     const GroupCtx g = load_group(a.tasks, d);
     const FwdIdx fi = fwd_indices(a, g, bi, lane & 31);
+    if constexpr (std::is_same<T, float>::value) {
+        if (g.c <= 16) {
+            fwd_task_small<MASK>(a, g, fi, tiles[wave][0], tiles[wave][1], tabs[wave][0], tabs[wave][1], tq, tk, tv, to, lse);
+            return;
+        }
+    }
     fwd_task<T, MASK>(a, g, bi, fi, tiles[wave][0], tiles[wave][1], tabs[wave][0], tabs[wave][1], tq, tk, tv, to, lse, [] {});
 }
 
