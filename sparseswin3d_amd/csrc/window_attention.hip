@@ -903,6 +903,168 @@ __device__ __forceinline__ void xch_add(const float* xch, int lane, f32x16& v) {
     }
 }
 
+// ------------------------------------------------------------------------------------------
+// backward of a group of at most 16 tokens (fp32) on 16 x 16 tiles (v_mfma_f32_16x16x4_f32; lane l: column
+// col = l % 16, slice sl = l / 16; see the forward).  S and dP are formed with queries as rows
+// (accumulator rows 4 sl + r) and keys as columns (col), so the lane's P and dS are the A operand of
+// dV = P^T dO and dK = dS^T Q as they stand (step m of slice sl carries query 4 sl + m); dQ = dS K takes dS
+// through a 16 x 16 LDS transpose.  40 matrix steps of 32 cycles instead of 80 of 64, ten row loads instead
+// of twenty, a softmax pass over 4 values per lane instead of 16.
+// LDS: rows 0-15 of tile_q hold Q, rows 16-31 K; rows 0-15 of tile_do hold dO, rows 16-31 V, later dS.
+// ------------------------------------------------------------------------------------------
+template <bool MASK>
+__device__ __forceinline__ void bwd_task_small(const WAttnCommon& a, const GroupCtx& g, float* tile_q, float* tile_do,
+                                               const TokenTensor32& tq, const TokenTensor32& tk, const TokenTensor32& tv,
+                                               const TokenTensor32& to, const TokenTensor32& tdo,
+                                               const float* __restrict__ lse, const TokenTensor32& tdq,
+                                               const TokenTensor32& tdk, const TokenTensor32& tdv,
+                                               float* __restrict__ ds_out) {
+    const int lane = threadIdx.x & 63;
+    const int col = lane & 15, sl = lane >> 4;
+    const int c = g.c, h = g.h;
+    const int8_t* mrow = MASK ? a.mask + (int64_t)(g.w % a.nmw) * a.n : nullptr;
+    const PadTab tab_pos = pad_tab(tile_q, 0), tab_L = pad_tab(tile_q, 1), tab_D = pad_tab(tile_q, 2);
+    // token col of the group (clamped to the last one): key of this lane's column
+    const int t_c = col < c ? col : c - 1;
+    const uint32_t vox = (uint32_t)a.order[g.Tk + t_c];
+    const int pos = a.tok_pos[g.Tk + t_c];
+    const float L2 = col < c ? lse[(int64_t)a.H * g.Tk + h * c + t_c] * LOG2E : INFINITY;   // padding queries: P = 0
+    const int reg = MASK ? mrow[pos] : 0;
+    u32x4_a rq[2], rk[2], rv[2], rdo[2], ro[2];
+#pragma unroll
+    for (int v = 0; v < 2; ++v) {                            // eight rows per instruction, 16 bytes per lane
+        const uint32_t vr = (uint32_t)__shfl((int)vox, v * 8 + lane / 8, 64);
+        const uint32_t off = (uint32_t)(lane % 8) * 16u;
+        rk[v] = *reinterpret_cast<const u32x4_a*>(head_base<float>(tk, h) + (__umul24(vr, pitch_of<float>(tk)) + off));
+        rv[v] = *reinterpret_cast<const u32x4_a*>(head_base<float>(tv, h) + (__umul24(vr, pitch_of<float>(tv)) + off));
+        rq[v] = *reinterpret_cast<const u32x4_a*>(head_base<float>(tq, h) + (__umul24(vr, pitch_of<float>(tq)) + off));
+        rdo[v] = *reinterpret_cast<const u32x4_a*>(head_base<float>(tdo, h) + (__umul24(vr, pitch_of<float>(tdo)) + off));
+        ro[v] = *reinterpret_cast<const u32x4_a*>(head_base<float>(to, h) + (__umul24(vr, pitch_of<float>(to)) + off));
+    }
+    uint32_t pi = (uint32_t)(pos * a.n) * 4u;                // byte offset of bias row pos (< 2^16)
+    if (MASK) pi |= (uint32_t)reg << 16;
+    float* tile_k = tile_q + 16 * TILE_LD;
+    float* tile_v = tile_do + 16 * TILE_LD;
+    __builtin_amdgcn_wave_barrier();
+    if (sl == 0) {
+        tab_pos.put(col, pi);
+        tab_L.put(col, f2u(L2));
+    }
+#pragma unroll
+    for (int v = 0; v < 2; ++v) {
+        const int at = (v * 8 + lane / 8) * TILE_LD + (lane % 8) * 4;
+        *reinterpret_cast<u32x4_a*>(tile_q + at) = rq[v];
+        *reinterpret_cast<u32x4_a*>(tile_k + at) = rk[v];
+        *reinterpret_cast<u32x4_a*>(tile_do + at) = rdo[v];
+        *reinterpret_cast<u32x4_a*>(tile_v + at) = rv[v];
+        float d = chunk_dot<float>(rdo[v], ro[v]);           // D_i = dO_i . O_i, summed over the 8 lanes of a row
+        d += dpp_f32<0xB1>(d);
+        d += dpp_f32<0x4E>(d);
+        d += dpp_f32<0x141>(d);
+        if (lane % 8 == 0) tab_D.put(v * 8 + lane / 8, f2u(d));
+    }
+    __builtin_amdgcn_wave_barrier();
+    // bias[h][pos of query 4 sl + r][pos of key col]: gathers first, the products cover their latency
+    const u32x4_a piq = tab_pos.chunk(sl);
+    const uint32_t pir[4] = {piq.x, piq.y, piq.z, piq.w};
+    const char* bias_h = reinterpret_cast<const char*>(a.bias + (int64_t)h * a.n * a.n);
+    const uint32_t bcol = (uint32_t)pos * 4u;
+    float bv[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) bv[r] = *reinterpret_cast<const float*>(bias_h + (bcol + (MASK ? (pir[r] & 0xffffu) : pir[r])));
+    auto row8 = [&](const float* t, float (&x)[8]) {         // channels 8 sl .. 8 sl + 7 of row col
+        const f32x4_a* p4 = reinterpret_cast<const f32x4_a*>(t + col * TILE_LD + 8 * sl);
+        const f32x4_a u = p4[0], w = p4[1];
+        x[0] = u.x; x[1] = u.y; x[2] = u.z; x[3] = u.w; x[4] = w.x; x[5] = w.y; x[6] = w.z; x[7] = w.w;
+    };
+    f32x4_v S = {0, 0, 0, 0}, dP = {0, 0, 0, 0};            // [query 4 sl + r][key col]
+    {
+        float qa[8], kb[8];
+        row8(tile_q, qa);
+        row8(tile_k, kb);
+#pragma unroll
+        for (int m = 0; m < 8; ++m) S = __builtin_amdgcn_mfma_f32_16x16x4f32(qa[m], kb[m], S, 0, 0, 0);
+        float doa[8], vb[8];
+        row8(tile_do, doa);
+        row8(tile_v, vb);
+#pragma unroll
+        for (int m = 0; m < 8; ++m) dP = __builtin_amdgcn_mfma_f32_16x16x4f32(doa[m], vb[m], dP, 0, 0, 0);
+    }
+    const u32x4_a Lq = tab_L.chunk(sl), Dq = tab_D.chunk(sl);
+    const float Lr[4] = {u2f(Lq.x), u2f(Lq.y), u2f(Lq.z), u2f(Lq.w)};
+    const float Dr[4] = {u2f(Dq.x), u2f(Dq.y), u2f(Dq.z), u2f(Dq.w)};
+    const float sscale = a.scale * LOG2E;
+    float pr[4], ds[4];
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        float x = fmaf(S[r], sscale, bv[r] * LOG2E);
+        if (MASK && (int)(pir[r] >> 16) != reg) x += -100.0f * LOG2E;
+        pr[r] = col < c ? exp2_fast(x - Lr[r]) : 0.f;        // padding keys and (L = inf) padding queries: 0
+        ds[r] = pr[r] * (dP[r] - Dr[r]);
+    }
+    if (ds_out && col < c) {
+        float* ds_g = ds_out + g.sq + col;
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            if (4 * sl + r < c) ds_g[(4 * sl + r) * c] = ds[r];
+    }
+    // dV = P^T dO, dK = dS^T Q: step m of slice sl carries query 4 sl + m
+    f32x4_v dv0 = {0, 0, 0, 0}, dv1 = {0, 0, 0, 0}, dk0 = {0, 0, 0, 0}, dk1 = {0, 0, 0, 0};
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+        if (m > 0 && m >= c) break;
+        const float* rdo_ = tile_do + (4 * sl + m) * TILE_LD + col;
+        const float* rq_ = tile_q + (4 * sl + m) * TILE_LD + col;
+        dv0 = __builtin_amdgcn_mfma_f32_16x16x4f32(pr[m], rdo_[0], dv0, 0, 0, 0);
+        dv1 = __builtin_amdgcn_mfma_f32_16x16x4f32(pr[m], rdo_[16], dv1, 0, 0, 0);
+        dk0 = __builtin_amdgcn_mfma_f32_16x16x4f32(ds[m], rq_[0], dk0, 0, 0, 0);
+        dk1 = __builtin_amdgcn_mfma_f32_16x16x4f32(ds[m], rq_[16], dk1, 0, 0, 0);
+    }
+    // dQ = dS K: dS[query][key] through LDS (the V rows are no longer needed), read back a query row per column
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int r = 0; r < 4; ++r) tile_v[(4 * sl + r) * TILE_LD + col] = ds[r];
+    __builtin_amdgcn_wave_barrier();
+    const f32x4_a dsq = *reinterpret_cast<const f32x4_a*>(tile_v + col * TILE_LD + 4 * sl);   // dS[query col][keys 4 sl ..]
+    const float dsr[4] = {dsq.x, dsq.y, dsq.z, dsq.w};
+    f32x4_v dq0 = {0, 0, 0, 0}, dq1 = {0, 0, 0, 0};
+#pragma unroll
+    for (int m = 0; m < 4; ++m) {
+        if (m > 0 && m >= c) break;
+        const float* rk_ = tile_k + (4 * sl + m) * TILE_LD + col;
+        dq0 = __builtin_amdgcn_mfma_f32_16x16x4f32(dsr[m], rk_[0], dq0, 0, 0, 0);
+        dq1 = __builtin_amdgcn_mfma_f32_16x16x4f32(dsr[m], rk_[16], dq1, 0, 0, 0);
+    }
+    // accumulators (rows 4 sl + r, channels col and 16 + col) -> LDS rows -> 16-byte row stores
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int r = 0; r < 4; ++r) {
+        const int at = (4 * sl + r) * TILE_LD + col;
+        tile_q[at] = dq0[r] * a.scale;                       // Q, K, dO rows have all been read
+        tile_q[at + 16] = dq1[r] * a.scale;
+        tile_k[at] = dk0[r] * a.scale;
+        tile_k[at + 16] = dk1[r] * a.scale;
+        tile_do[at] = dv0[r];
+        tile_do[at + 16] = dv1[r];
+    }
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int v = 0; v < 2; ++v) {
+        const int R = v * 8 + lane / 8;
+        const uint32_t vr = (uint32_t)__shfl((int)vox, R, 64);
+        const int at = R * TILE_LD + (lane % 8) * 4;
+        const uint32_t off = (uint32_t)(lane % 8) * 16u;
+        if (R < c) {
+            *reinterpret_cast<u32x4_a*>(const_cast<char*>(head_base<float>(tdq, h)) + (__umul24(vr, pitch_of<float>(tdq)) + off)) =
+                *reinterpret_cast<const u32x4_a*>(tile_q + at);
+            *reinterpret_cast<u32x4_a*>(const_cast<char*>(head_base<float>(tdk, h)) + (__umul24(vr, pitch_of<float>(tdk)) + off)) =
+                *reinterpret_cast<const u32x4_a*>(tile_k + at);
+            *reinterpret_cast<u32x4_a*>(const_cast<char*>(head_base<float>(tdv, h)) + (__umul24(vr, pitch_of<float>(tdv)) + off)) =
+                *reinterpret_cast<const u32x4_a*>(tile_do + at);
+        }
+    }
+}
+
 // `live` = false (KV_PAIR only): a wavefront without a task that still has to meet the barrier.
 template <typename T, bool MASK, int DQ>
 __device__ __forceinline__ void bwd_kv_task(const WAttnCommon& a, int64_t task, bool live, float* tile_q, float* tile_do,
@@ -922,6 +1084,12 @@ __device__ __forceinline__ void bwd_kv_task(const WAttnCommon& a, int64_t task, 
     }
     const PadTab tab_pos = pad_tab(tile_q, 0), tab_L = pad_tab(tile_q, 1), tab_D = pad_tab(tile_q, 2);
     const GroupCtx g = load_group(a.tasks, d);
+    if constexpr (DQ == KV_SINGLE && std::is_same<T, float>::value) {
+        if (g.c <= 16) {
+            bwd_task_small<MASK>(a, g, tile_q, tile_do, tq, tk, tv, to, tdo, lse, tdq, tdk, tdv, ds_out);
+            return;
+        }
+    }
     const int c = g.c, h = g.h;
     const int nt = (c + 31) >> 5;
     const int32_t* order = a.order + g.Tk;

@@ -201,7 +201,9 @@ def test_resident_kernels_on_ragged_windows(mix, use_mask):
         other[cols] = False
         assert np.isnan(got[:, other]).all()                 # the other side is not touched
         if sides != 1:
-            assert torch.equal(ds2, ds)                          # the same dS, bit for bit
+            # the same dS (groups of at most 16 tokens take another kernel path in the one-launch backward, so
+            # the two agree to rounding, not bit for bit)
+            close(ds2.cpu().numpy(), ds.cpu().numpy(), 1e-5, "dS of the key-side kernel")
     # bias gradient from the stored dS
     d_bias = torch.zeros(H, n, n, device="cuda")
     nbytes = lib.sswin_fused_bias_grad_workspace_bytes(tp.G, H, n)
