@@ -69,6 +69,37 @@ def test_window_attention_forward_backward(shift, dim, heads, path):
           leaves["relative_position_bias_table"].grad.numpy(), 1e-5, "d bias table")
 
 
+def test_window_7_heads_of_16_channels_runs_the_operator_path():
+    """The reference's own ScanNet setting: windows of 7^3 = 343 positions, shift 3, 48 channels in 3 heads of 16.
+    Windows above 128 positions are outside the fused kernels, so the module takes the operator path by itself
+    (``fused`` left at its default); forward and backward against the fp64 CPU path."""
+    from sparseswin3d_amd import synth
+    from sparseswin3d_amd.window_attention import SparseVoxelTensor, WindowAttentionSparse
+    torch.manual_seed(4)
+    c4, grid = _scene(seed=11, grid=(42, 42, 42), boxes=3)
+    ws, shift = (7, 7, 7), (3, 3, 3)
+    win_idx, nw, n = synth.window_indices(c4, grid, ws, shift)
+    assert n == 343
+    N = len(win_idx)
+    attn = WindowAttentionSparse(48, 3, ws, qkv_bias=True).cuda()
+    with torch.no_grad():
+        attn.relative_position_bias_table.normal_(0, 0.5)
+    mask_np = synth.shift_region_mask(synth.padded_shape(grid, ws), ws, shift)
+    feats, upstream = torch.randn(N, 48), torch.randn(N, 48)
+    x = SparseVoxelTensor(feats.cuda().requires_grad_(True), torch.from_numpy(win_idx).cuda(), (n,), nw)
+    feats_gpu = x.features
+    out = attn(x, torch.from_numpy(mask_np).cuda()).features
+    out.backward(upstream.cuda())
+    f64 = feats.double().requires_grad_(True)
+    ref, leaves = _cpu_attention(attn, f64, win_idx, n, mask_np)
+    ref.backward(upstream.double())
+    close(out.detach().cpu().numpy(), ref.detach().numpy(), 1e-5, "attention output")
+    close(feats_gpu.grad.cpu().numpy(), f64.grad.numpy(), 1e-5, "d features")
+    close(attn.qkv.weight.grad.cpu().numpy(), leaves["qkv.weight"].grad.numpy(), 1e-5, "d qkv.weight")
+    close(attn.relative_position_bias_table.grad.cpu().numpy(),
+          leaves["relative_position_bias_table"].grad.numpy(), 1e-5, "d bias table")
+
+
 def test_window_attention_matches_dense_swin_on_full_windows():
     """All windows full: the sparse path must equal textbook dense window attention."""
     from oracle import cpu_path
