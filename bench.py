@@ -579,6 +579,47 @@ def pmc_summary(dirs, out_name, workload, command, only=None):
     print("\n".join(lines))
 
 
+def trace_summary(dirs, out_name, command):
+    """Turn the ``*kernel_stats.csv`` of ``rocprofv3 --kernel-trace --stats`` runs of this script (one directory
+    per workload, named ..._<workload>) into the text summary ``profiles/<out_name>.txt``: time per step and
+    kernel.  The step count is read off the backward launch (one per attention call, two calls per step)."""
+    import csv
+    import glob
+    lines = ["rocprofv3 kernel traces of the benchmark step (step = regular + shifted block pair, forward + backward).",
+             "Commands (from the repository root, TMPDIR=/tmp):"]
+    lines += [f"  {c}" for c in command]
+    lines.append("Durations in microseconds; kernels shorter than 1 us per step are left out of the tables.")
+    for d in dirs:
+        paths = glob.glob(os.path.join(d, "**", "*kernel_stats.csv"), recursive=True)
+        if not paths:
+            sys.exit(f"no *kernel_stats.csv under {d}")
+        rows = list(csv.DictReader(open(paths[0])))
+        bwd = sum(int(r["Calls"]) for r in rows if "wattn_bwd_all_kernel" in r["Name"])
+        steps = max(bwd // 2, 1)
+        tot = sum(float(r["TotalDurationNs"]) for r in rows)
+        groups = {"library GEMMs (Cijk_*)": 0.0, "kernels of this library (sswin::*)": 0.0, "PyTorch element-wise / copies": 0.0}
+        lines += ["", f"{os.path.basename(d.rstrip('/'))}: {steps} steps, GPU kernel time {tot / 1e3 / steps:.1f} us per step "
+                      f"over {sum(int(r['Calls']) for r in rows) / steps:.0f} dispatches",
+                  " calls/step   us/step    avg us      %  kernel"]
+        for r in sorted(rows, key=lambda r: -float(r["TotalDurationNs"])):
+            t, name = float(r["TotalDurationNs"]), r["Name"]
+            key = ("library GEMMs (Cijk_*)" if name.startswith("Cijk") else
+                   "kernels of this library (sswin::*)" if "sswin::" in name else "PyTorch element-wise / copies")
+            groups[key] += t
+            if t / 1e3 / steps < 1.0:
+                continue
+            short = name.replace("void ", "")
+            if "sswin::" in short:
+                short = short.split("(")[0]
+            lines.append(f"{int(r['Calls']) / steps:11.1f}  {t / 1e3 / steps:8.1f}  {float(r['AverageNs']) / 1e3:8.1f}  "
+                         f"{100 * t / tot:5.2f}  {short[:100]}")
+        lines.append("per step: " + ", ".join(f"{k} {v / 1e3 / steps:.0f} us" for k, v in groups.items()))
+    out = os.path.join(ROOT, "profiles", out_name + ".txt")
+    with open(out, "w") as f:
+        f.write("\n".join(lines) + "\n")
+    print("\n".join(lines))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -596,6 +637,9 @@ def main():
     ap.add_argument("--pmc-summary", nargs="+", default=None, metavar="DIR",
                     help="no GPU work: summarise the rocprofv3 --pmc csv output under these directories into "
                          "profiles/<--pmc-name>.txt and profiles/traffic.json")
+    ap.add_argument("--trace-summary", nargs="+", default=None, metavar="DIR",
+                    help="no GPU work: summarise the kernel_stats.csv of rocprofv3 --kernel-trace --stats runs of this "
+                         "script into profiles/<--pmc-name>.txt")
     ap.add_argument("--pmc-name", default=None)
     ap.add_argument("--pmc-kernels", nargs="+", default=None, metavar="SUBSTR",
                     help="kernel symbols to keep in the summary (default: those of KERNEL_SYMBOLS)")
@@ -604,6 +648,9 @@ def main():
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (windows are independent; sharding is "
                  "described in DESIGN.md); rerun with --gpus 1")
+    if args.trace_summary:
+        trace_summary(args.trace_summary, args.pmc_name or "bench_step_kernel_trace", args.pmc_command)
+        return
     if args.pmc_summary:
         from sparseswin3d_amd import synth
         name = {"cfg1": synth.config1, "cfg2": synth.config2, "cfg3": synth.config3, "cfg4": synth.config4}[args.workload]().name

@@ -1356,7 +1356,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
 // The whole backward in one launch.  Workgroups (four wavefronts, one task each) are numbered through
 // four segments, each starting at a workgroup boundary:
 //   1. query-side tasks of the groups of three and four tiles
-//   2. their key-side tasks (KV_ONLY)
+//   2. their key-side tasks (KV_ONLY); 1 and 2 are interleaved in runs of eight workgroups (see the kernel)
 //   3. key-side tasks of the groups of two tiles, the two tasks of a group side by side (KV_PAIR)
 //   4. key-side tasks of the groups of one tile (KV_SINGLE)
 // Heaviest tasks first, so the long ones start first and the short ones fill the tail.
@@ -1377,14 +1377,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     const int64_t wg = blockIdx.x;
     float* t0 = tiles[wave][0];
     float* t1 = tiles[wave][1];
-    if (wg < sg.wg_kv) {
-        const int64_t task = wg * 4 + wave;
-        if (task < sg.n_big) bwd_q_task<T, MASK>(a, task, t0, t1, tq, tk, tv, to, tdo, lse, tdq);
-    } else if (wg < sg.wg_pair) {
-        const int64_t task = (wg - sg.wg_kv) * 4 + wave;
-        if (task < sg.n_big)
-            bwd_kv_task<T, MASK, KV_ONLY>(a, task, true, t0, t1, nullptr, nullptr, tq, tk, tv, to, tdo, lse, tdk, tdv,
-                                          ds_out, tdq);
+    if (wg < sg.wg_pair) {
+        // Segments 1 and 2 interleaved in runs of eight workgroups: workgroups 16 k .. 16 k + 7 take the query side
+        // of eight consecutive task quadruples, workgroups 16 k + 8 .. 16 k + 15 the key side of the same ones.
+        // Workgroups are dealt to the eight XCDs round robin, so both sides of a group run on one XCD at about the
+        // same time and the second one finds the group's rows in that XCD's L2.
+        const int64_t quad = (wg >> 4) * 8 + (wg & 7);
+        const int64_t task = quad * 4 + wave;
+        if (task < sg.n_big) {
+            if ((wg & 8) == 0)
+                bwd_q_task<T, MASK>(a, task, t0, t1, tq, tk, tv, to, tdo, lse, tdq);
+            else
+                bwd_kv_task<T, MASK, KV_ONLY>(a, task, true, t0, t1, nullptr, nullptr, tq, tk, tv, to, tdo, lse, tdk, tdv,
+                                              ds_out, tdq);
+        }
     } else if (wg < sg.wg_single) {
         const int64_t task = (wg - sg.wg_pair) * 4 + wave;
         bwd_kv_task<T, MASK, KV_PAIR>(a, sg.n_big + task, task < sg.n_pair, t0, t1, xch[wave], xch[wave ^ 1], tq, tk, tv, to,
@@ -1424,7 +1430,7 @@ static void launch_backward(const WAttnCommon& a, const TokenTensor32& q, const 
         const int64_t n_single = a.first[4] - a.first[3];
         const int64_t wg_big = (sg.n_big + 3) / 4;
         sg.wg_kv = wg_big;
-        sg.wg_pair = 2 * wg_big;
+        sg.wg_pair = 16 * ((wg_big + 7) / 8);              // both sides, interleaved in runs of eight workgroups
         sg.wg_single = sg.wg_pair + (sg.n_pair + 3) / 4;
         const int64_t wgs = sg.wg_single + (n_single + 3) / 4;
         hipLaunchKernelGGL((wattn_bwd_all_kernel<T, MASK>), dim3((unsigned)wgs), dim3(256), 0, s, a, sg, q, k, v, o, d_o, lse,
