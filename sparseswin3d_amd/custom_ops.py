@@ -297,7 +297,9 @@ class _IndexPlanCache:
     pass receive the same sorted Q/V index tensor, so the second call skips the plan kernels and
     their host synchronisation.  An entry holds only a weak reference to the index tensor: it is
     valid while that tensor is alive (its address cannot have been handed to another tensor) and
-    unchanged (version counter), and it does not keep the [4, E] matrix in memory."""
+    unchanged (version counter), and it does not keep the [4, E] matrix in memory.  A plan enters the
+    cache only after the host has waited for the stream that built it (the totals are read back), so a
+    hit from another stream reads finished data."""
 
     def __init__(self, capacity=8):
         self.capacity = capacity
