@@ -48,17 +48,50 @@ __device__ __forceinline__ int axis_region(int v, int extent, int ws, int s) {
     return v < extent - ws ? 0 : (v < extent - s ? 1 : 2);
 }
 
-__device__ __forceinline__ int mask_region(const Grid3& g, int n, int64_t i) {
-    const int pos = (int)(i % n);
-    int w = (int)(i / n);
-    const int wx = w % g.nwin[2];
-    w /= g.nwin[2];
-    const int wy = w % g.nwin[1], wz = w / g.nwin[1];
-    const int px = pos % g.win[2], py = (pos / g.win[2]) % g.win[1], pz = pos / (g.win[2] * g.win[1]);
-    const int rz = axis_region(wz * g.win[0] + pz, g.dim[0], g.win[0], g.shift[0]);
-    const int ry = axis_region(wy * g.win[1] + py, g.dim[1], g.win[1], g.shift[1]);
-    const int rx = axis_region(wx * g.win[2] + px, g.dim[2], g.win[2], g.shift[2]);
+// Region id of entry i = window * n + pos and of the three entries behind it.  The (window, position) pair is
+// decomposed once per thread (five 32-bit divisions; the quotient i / n in 64 bits only when the array is
+// that large) and then advanced by carries: position -> (pz, py, px), window -> (wz, wy, wx).
+struct MaskCursor {
+    int wz, wy, wx, pz, py, px;
+};
+__device__ __forceinline__ MaskCursor mask_cursor(const Grid3& g, int n, int64_t i, bool small) {
+    uint32_t w, pos;
+    if (small) {
+        w = (uint32_t)i / (uint32_t)n;
+        pos = (uint32_t)i - w * (uint32_t)n;
+    } else {
+        w = (uint32_t)(i / n);
+        pos = (uint32_t)(i - (int64_t)w * n);
+    }
+    MaskCursor c;
+    const uint32_t wyz = w / (uint32_t)g.nwin[2];
+    c.wx = (int)(w - wyz * (uint32_t)g.nwin[2]);
+    c.wz = (int)(wyz / (uint32_t)g.nwin[1]);
+    c.wy = (int)(wyz - (uint32_t)c.wz * (uint32_t)g.nwin[1]);
+    const uint32_t pzy = pos / (uint32_t)g.win[2];
+    c.px = (int)(pos - pzy * (uint32_t)g.win[2]);
+    c.pz = (int)(pzy / (uint32_t)g.win[1]);
+    c.py = (int)(pzy - (uint32_t)c.pz * (uint32_t)g.win[1]);
+    return c;
+}
+__device__ __forceinline__ int mask_region(const Grid3& g, const MaskCursor& c) {
+    const int rz = axis_region(c.wz * g.win[0] + c.pz, g.dim[0], g.win[0], g.shift[0]);
+    const int ry = axis_region(c.wy * g.win[1] + c.py, g.dim[1], g.win[1], g.shift[1]);
+    const int rx = axis_region(c.wx * g.win[2] + c.px, g.dim[2], g.win[2], g.shift[2]);
     return 9 * rz + 3 * ry + rx;
+}
+__device__ __forceinline__ void mask_advance(const Grid3& g, MaskCursor& c) {
+    if (++c.px < g.win[2]) return;
+    c.px = 0;
+    if (++c.py < g.win[1]) return;
+    c.py = 0;
+    if (++c.pz < g.win[0]) return;
+    c.pz = 0;                                                // next window
+    if (++c.wx < g.nwin[2]) return;
+    c.wx = 0;
+    if (++c.wy < g.nwin[1]) return;
+    c.wy = 0;
+    ++c.wz;
 }
 
 // four consecutive entries per thread, one 32-bit store (the array is 4-byte aligned); the last
@@ -66,13 +99,20 @@ __device__ __forceinline__ int mask_region(const Grid3& g, int n, int64_t i) {
 __global__ __launch_bounds__(256) void shift_mask_kernel(Grid3 g, int n, int64_t total, int8_t* __restrict__ mask) {
     const int64_t i = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= total) return;
+    MaskCursor c = mask_cursor(g, n, i, total < ((int64_t)1 << 31));
     if (i + 4 <= total) {
         uint32_t v = 0;
 #pragma unroll
-        for (int k = 0; k < 4; ++k) v |= (uint32_t)mask_region(g, n, i + k) << (8 * k);
+        for (int k = 0; k < 4; ++k) {
+            v |= (uint32_t)mask_region(g, c) << (8 * k);
+            mask_advance(g, c);
+        }
         *reinterpret_cast<uint32_t*>(mask + i) = v;
     } else {
-        for (int64_t k = i; k < total; ++k) mask[k] = (int8_t)mask_region(g, n, k);
+        for (int64_t k = i; k < total; ++k) {
+            mask[k] = (int8_t)mask_region(g, c);
+            mask_advance(g, c);
+        }
     }
 }
 
