@@ -230,8 +230,9 @@ def kernel_table(wl, reps=20, only=None):
             ("qkv_sparse_indices (reference operator)", lambda: ops.qkv_sparse_indices(b["idx"], b["slots"], b["n"], H, hd, _defer_check=True), 8 * N + 40 * E, 0),
             ("plan_from_indices", lambda: _lib.check(lib.sswin_plan_from_indices(ptr(q.indices), m, hd, ptr(plan), g_cap, totals, ptr(ws), nb, stream)), 0, 1),
             ("block_matmul q_k", mm(0, q.values, kt.values, q.indices, out_s, out_si, A), 2 * s * E + (s + 16) * A + 4 * G, 1),
-            ("flatten_indices [3,A]", lambda: ops.flatten_indices(s_idx[:3], s_shape[:3]), 16 * A, 1),
-            ("unique_consecutive_indices [A]", lambda: ops.unique_consecutive_indices(flat), 8 * A, 1),
+            ("softmax rows from the group sizes [A]", lambda: ops.softmax_rows_from_counts(c, A), 4 * A + 12 * G, 1),
+            ("flatten_indices [3,A] (generic softmax rows)", lambda: ops.flatten_indices(s_idx[:3], s_shape[:3]), 16 * A, 0),
+            ("unique_consecutive_indices [A] (generic softmax rows)", lambda: ops.unique_consecutive_indices(flat), 8 * A, 0),
             ("softmax_last_dim_forward", lambda: ops.softmax_last_dim_forward(rows, s_val), 12 * A, 1),
             ("block_matmul qk_v", mm(1, p_val, v.values, v.indices, out_o, out_oi, E), s * A + s * E + (s + 16) * E + 4 * G, 1),
             ("permute order from the group structure [E]", lambda: ops.permute_heads_order(o_idx, o_shape), 0, 0),

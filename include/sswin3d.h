@@ -163,6 +163,13 @@ int sswin_plan_from_indices(const int32_t* idx, int64_t M, int inner, int32_t* p
 int sswin_permute_heads_order(const int32_t* idx, int64_t M, int C, const int32_t* plan, int64_t g_cap,
                               int64_t G, int32_t* perm_out, int32_t* bad_groups, void* stream);
 
+/* Row ids of the sparse softmax for a [B, H, n, n] product in sorted order: rows_out[sq_start[g] + i*c + j] =
+ * row_start[g] + i.  Equal to unique_consecutive_indices(flatten_indices(idx[:3])) of that product
+ * (sparse_swin/swin3d_base.py:140-150), without reading its index matrix.  c: device int32 [G] (windows of fewer than
+ * 4096 tokens), scans: device int32 [2*G] as sswin_scan_counts writes them, rows_out: device int32 [sum c*c].
+ * Asynchronous. */
+int sswin_softmax_rows_from_counts(const int32_t* c, const int32_t* scans, int64_t G, int32_t* rows_out, void* stream);
+
 /* Same three scans from a given `_c` (what the reference recomputes inside every
  * matmul_grad / qkv_transpose call, sparse_swin/ops.cu:681, 697, 965-968, 986-989,
  * 1007-1010).  c: device int32 [G].  scans: device int32 [2*G]: row 0 = exclusive scan of c,

@@ -204,6 +204,30 @@ __global__ __launch_bounds__(256) void permute_heads_kernel(const int32_t* __res
     }
 }
 
+// ------------------------------------------------------------------------------------------
+// Row ids of a [B, H, n, n] product in sorted COO order: entry sq_start[g] + i*c + j belongs to attention row
+// row_start[g] + i.  The reference hashes the first three index rows and runs unique_consecutive over the
+// hash (sparse_swin/swin3d_base.py:140-150); every attention row of every group is non-empty, so the
+// running id is the row number.  One wavefront per group.
+// ------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void rows_from_counts_kernel(const int32_t* __restrict__ cs, const int32_t* __restrict__ row_start,
+                                                               const int32_t* __restrict__ sq_start, int64_t G,
+                                                               int32_t* __restrict__ rows) {
+    const int64_t g = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (g >= G) return;
+    const int lane = threadIdx.x & 63;
+    const int c = cs[g], rs = row_start[g];
+    int32_t* out = rows + sq_start[g];
+    const int count = c * c;
+    const float inv = 1.0f / (float)c;
+    for (int f = lane; f < count; f += 64) {
+        int i = (int)((float)f * inv);                        // f / c up to one, corrected below (f < 2^24)
+        i -= i * c > f ? 1 : 0;
+        i += (i + 1) * c <= f ? 1 : 0;
+        out[f] = rs + i;
+    }
+}
+
 }  // namespace sswin
 
 using namespace sswin;
@@ -268,6 +292,15 @@ int sswin_plan_from_indices(const int32_t* idx, int64_t M, int inner, int32_t* p
     totals_out[3] = (int32_t)(host[1] & 0xffffffffll);
     SSWIN_CHECK(G <= g_cap, "plan: %lld groups exceed the plan capacity %lld", (long long)G, (long long)g_cap);
     return 0;
+}
+
+int sswin_softmax_rows_from_counts(const int32_t* c, const int32_t* scans, int64_t G, int32_t* rows_out, void* stream) {
+    SSWIN_CHECK(G >= 0, "softmax_rows_from_counts: negative group count");
+    if (G == 0) return 0;
+    SSWIN_CHECK(c && scans && rows_out, "softmax_rows_from_counts: null pointer");
+    hipLaunchKernelGGL(rows_from_counts_kernel, dim3((unsigned)((G + 3) / 4)), dim3(256), 0, static_cast<hipStream_t>(stream), c,
+                       scans, scans + G, G, rows_out);
+    return launch_ok("softmax_rows_from_counts");
 }
 
 size_t sswin_scan_counts_workspace_bytes(int64_t G) {

@@ -462,6 +462,22 @@ def permute_heads_order(indices, shape):
     return order
 
 
+def softmax_rows_from_counts(_c, nnz):
+    """Row ids of the sparse softmax over a 'q_k' product with group sizes ``_c`` and ``nnz`` entries: what
+    ``unique_consecutive_indices(flatten_indices(idx[:3], shape[:3]))`` returns for it, from the group sizes alone.
+    Not an operator of the reference's module: a helper of :func:`softmax_last_dim`."""
+    lib = _lib.load()
+    d = _dev(_c)
+    _check(_c.dtype == torch.int32 and _c.dim() == 1, "_c must be int32 [G]")
+    c = _c.contiguous()
+    rows = torch.empty(int(nnz), dtype=torch.int32, device=d)
+    with torch.cuda.device(d):
+        scans, sum_c2 = _scans_for(c, lib, d)
+        _check(sum_c2 is None or sum_c2 == nnz, f"softmax_rows_from_counts: {nnz} entries, the groups hold {sum_c2}")
+        _lib.check(lib.sswin_softmax_rows_from_counts(_ptr(c), _ptr(scans), c.numel(), _ptr(rows), _stream(d)))
+    return rows
+
+
 def matmul_grad_cuda_naive(mat1_v, mat2_v, _c, C_, mul_type):
     """Value-only block products of the backward pass (reference ops.cu:945-1031, 1092-1114)."""
     lib = _lib.load()

@@ -57,7 +57,7 @@ def replace_feature(out, new_features):
 class SparseTensor:
     """4-D COO tensor: ``indices`` int32 [4, nnz], ``values`` [nnz], ``shape`` list of 4."""
 
-    def __init__(self, indices, values, shape):
+    def __init__(self, indices, values, shape, group_counts=None):
         assert indices.shape[0] == 4, "Invalid shape"
         assert indices.ndim == 2, "Invalid shape"
         assert values.ndim == 1, "Invalid shape"
@@ -65,6 +65,9 @@ class SparseTensor:
         self.indices = indices
         self.values = values
         self.shape = shape
+        # tokens per (window, head) group when the tensor is a 'q_k' product (or shares its index matrix):
+        # lets softmax_last_dim number the attention rows without hashing the index matrix
+        self.group_counts = group_counts
 
     def __repr__(self):
         return f"SparseTensor(indices={self.indices}, values={self.values}, shape={self.shape})"
@@ -95,7 +98,7 @@ class SparseTensor:
 
     def __mul__(self, other):
         if isinstance(other, (int, float)):
-            return SparseTensor(self.indices, self.values * other, self.shape)
+            return SparseTensor(self.indices, self.values * other, self.shape, self.group_counts)
         raise NotImplementedError
 
 
@@ -121,12 +124,12 @@ class _spspmm_block_naive(Function):
         ctx.save_for_backward(mat2_v, mat1_v, counts)
         ctx.mul_type = mul_type
         ctx.inner = mat1_shape[-1] if mul_type == "q_k" else mat2_shape[-1]
-        ctx.mark_non_differentiable(mat3_idx)
-        return mat3_idx, mat3_v, mat3_shape
+        ctx.mark_non_differentiable(mat3_idx, counts)
+        return mat3_idx, mat3_v, mat3_shape, counts
 
     @staticmethod
     @once_differentiable
-    def backward(ctx, _grad_idx, grad_v, _grad_shape):
+    def backward(ctx, _grad_idx, grad_v, _grad_shape, _grad_counts):
         grad_v = grad_v.contiguous()
         mat2_v, mat1_v, counts = ctx.saved_tensors
         inner = ctx.inner
@@ -148,9 +151,9 @@ class _spspmm_block_naive(Function):
 
 def spspmm_block_naive(mat1: SparseTensor, mat2: SparseTensor, mul_type="q_k") -> SparseTensor:
     _check_mul_type(mul_type)
-    idx, val, shape = _spspmm_block_naive.apply(mat1.values, mat1.indices, mat1.shape,
-                                                mat2.values, mat2.indices, mat2.shape, mul_type)
-    return SparseTensor(idx, val, shape)
+    idx, val, shape, counts = _spspmm_block_naive.apply(mat1.values, mat1.indices, mat1.shape,
+                                                        mat2.values, mat2.indices, mat2.shape, mul_type)
+    return SparseTensor(idx, val, shape, counts if mul_type == "q_k" else None)
 
 
 # ------------------------------------------------------------------------------------------
@@ -158,8 +161,12 @@ def spspmm_block_naive(mat1: SparseTensor, mat2: SparseTensor, mul_type="q_k") -
 # ------------------------------------------------------------------------------------------
 class _softmax_last_dim(Function):
     @staticmethod
-    def forward(ctx, mat_v, mat_idx, mat_shape):
-        rows = ops.unique_consecutive_indices(ops.flatten_indices(mat_idx, mat_shape))
+    def forward(ctx, mat_v, mat_idx, mat_shape, group_counts=None):
+        if group_counts is not None:
+            # a 'q_k' product: its attention rows are numbered from the group sizes (same ids, no hash of the indices)
+            rows = ops.softmax_rows_from_counts(group_counts, mat_v.numel())
+        else:
+            rows = ops.unique_consecutive_indices(ops.flatten_indices(mat_idx, mat_shape))
         out = ops.softmax_last_dim_forward(rows, mat_v)
         ctx.save_for_backward(out, rows)
         return out
@@ -168,13 +175,13 @@ class _softmax_last_dim(Function):
     @once_differentiable
     def backward(ctx, grad_mat):
         out, rows = ctx.saved_tensors
-        return ops.softmax_last_dim_backward(rows, out, grad_mat.contiguous()), None, None
+        return ops.softmax_last_dim_backward(rows, out, grad_mat.contiguous()), None, None, None
 
 
 def softmax_last_dim(mat: SparseTensor) -> SparseTensor:
     dtype = mat.values.dtype
-    out = _softmax_last_dim.apply(mat.values.float(), mat.indices[:3], mat.shape[:-1])
-    return SparseTensor(mat.indices, out.to(dtype), mat.shape)
+    out = _softmax_last_dim.apply(mat.values.float(), mat.indices[:3], mat.shape[:-1], mat.group_counts)
+    return SparseTensor(mat.indices, out.to(dtype), mat.shape, mat.group_counts)
 
 
 # ------------------------------------------------------------------------------------------
@@ -254,7 +261,7 @@ def sp_add_rpb(sparse: SparseTensor, dense: torch.Tensor) -> SparseTensor:
     """``values += dense[head, pos_i, pos_j]`` for a dense bias [H, n, n]."""
     i = sparse.indices
     flat = i[1] * (dense.shape[1] * dense.shape[2]) + i[2] * dense.shape[2] + i[3]
-    return SparseTensor(i, sparse.values + dense.reshape(-1).index_select(0, flat), sparse.shape)
+    return SparseTensor(i, sparse.values + dense.reshape(-1).index_select(0, flat), sparse.shape, sparse.group_counts)
 
 
 def sp_add_mask(sparse: SparseTensor, dense: torch.Tensor) -> SparseTensor:
@@ -263,7 +270,7 @@ def sp_add_mask(sparse: SparseTensor, dense: torch.Tensor) -> SparseTensor:
     row = (i[0] % dense.shape[0]) * dense.shape[1]
     flat = dense.reshape(-1)
     differ = flat.index_select(0, row + i[3]) != flat.index_select(0, row + i[2])
-    return SparseTensor(i, sparse.values + differ.to(sparse.values.dtype) * -100.0, sparse.shape)
+    return SparseTensor(i, sparse.values + differ.to(sparse.values.dtype) * -100.0, sparse.shape, sparse.group_counts)
 
 
 def trunc_normal_(tensor, mean=0.0, std=1.0, a=-2.0, b=2.0):

@@ -275,3 +275,20 @@ def test_permute_falls_back_to_the_sort_when_heads_differ(ops, oracle):
     want = oracle.sort_indices(oracle.flatten_indices(np.ascontiguousarray(perm), [3, 8, 2, hd]))
     np.testing.assert_array_equal(host(out.indices), perm[:, want])
     np.testing.assert_array_equal(host(out.values), want.astype(np.float64))
+
+
+@pytest.mark.parametrize("mix", sorted(MIXES))
+@pytest.mark.parametrize("H,hd", [(3, 32), (2, 16)])
+def test_softmax_rows_from_the_group_sizes(ops, oracle, mix, H, hd):
+    """Row ids of the softmax over a 'q_k' product (reference swin3d_base.py:140-150: hash of the first three index rows,
+    then unique_consecutive) from the group sizes alone: bit-exact against the oracle's hash + unique_consecutive, and
+    softmax_last_dim gives the same result either way."""
+    from sparseswin3d_amd.window_attention import SparseTensor, softmax_last_dim
+    B, n, d = build(oracle, mix, H, hd, seed_of("rows", mix, H, hd))
+    f = run_forward(ops, oracle, d, torch.float32)
+    want = oracle.unique_consecutive_indices(oracle.flatten_indices(f["r_idx"][:3], f["r_shape"][:3]))
+    rows = ops.softmax_rows_from_counts(f["c1"], f["s_val"].numel())
+    np.testing.assert_array_equal(host(rows), want)
+    with_counts = softmax_last_dim(SparseTensor(f["s_idx"], f["s_val"], f["s_shape"], f["c1"]))
+    generic = softmax_last_dim(SparseTensor(f["s_idx"], f["s_val"], f["s_shape"]))
+    assert torch.equal(with_counts.values, generic.values)
