@@ -647,8 +647,8 @@ def main():
     ap.add_argument("--pmc-command", action="append", default=[], help="command line(s) quoted in the summary")
     args = ap.parse_args()
     if args.gpus != 1:
-        sys.exit("bench.py: this build runs on one GPU only (windows are independent; sharding is "
-                 "described in DESIGN.md); rerun with --gpus 1")
+        sys.exit("bench.py: this build runs on one GPU only (windows are independent attention problems, so the path "
+                 "would shard by window ranges with no exchange); rerun with --gpus 1")
     if args.trace_summary:
         trace_summary(args.trace_summary, args.pmc_name or "bench_step_kernel_trace", args.pmc_command)
         return
