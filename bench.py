@@ -221,6 +221,11 @@ def kernel_table(wl, reps=20, only=None):
         qkv_rows = qkv.view(N, 3 * D)
         val_e = torch.empty(E, device=dev)
 
+        gp = ops.group_plan(c)
+        bias_d = torch.randn(H, b["n"], b["n"], device=dev)
+        n_table_o = int(wl["blocks"][0]["attn"].relative_position_bias_table.shape[0])
+        ti_o = F.BiasTableIndex.build(relative_position_index_3d(wl["blocks"][0]["attn"].window_size).to(dev), n_table_o)
+
         entries = [
             # name, callable, algorithmic bytes, calls per attention fwd+bwd of the module (0: not on the module's path)
             ("operand_map [N]", lambda: ops.operand_map(b["idx"], b["slots"], b["n"]), 20 * N, 1),
@@ -230,6 +235,8 @@ def kernel_table(wl, reps=20, only=None):
             ("qkv_sparse_indices (reference operator)", lambda: ops.qkv_sparse_indices(b["idx"], b["slots"], b["n"], H, hd, _defer_check=True), 8 * N + 40 * E, 0),
             ("plan_from_indices", lambda: _lib.check(lib.sswin_plan_from_indices(ptr(q.indices), m, hd, ptr(plan), g_cap, totals, ptr(ws), nb, stream)), 0, 1),
             ("block_matmul q_k", mm(0, q.values, kt.values, q.indices, out_s, out_si, A), 2 * s * E + (s + 16) * A + 4 * G, 1),
+            ("bias + mask add, one pass [A]", lambda: ops.group_add_bias_mask(s_val, s_idx, gp, b["n"], bias_d, mask), 2 * s * A + 8 * G, 1),
+            ("bias table gradient from the product's groups", lambda: ops.group_bias_table_grad(g_s, s_idx, gp, H, b["n"], ti_o.code, ti_o.offset0, n_table_o), 4 * A, 1),
             ("softmax rows from the group sizes [A]", lambda: ops.softmax_rows_from_counts(c, A), 4 * A + 12 * G, 1),
             ("flatten_indices [3,A] (generic softmax rows)", lambda: ops.flatten_indices(s_idx[:3], s_shape[:3]), 16 * A, 0),
             ("unique_consecutive_indices [A] (generic softmax rows)", lambda: ops.unique_consecutive_indices(flat), 8 * A, 0),

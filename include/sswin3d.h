@@ -170,6 +170,23 @@ int sswin_permute_heads_order(const int32_t* idx, int64_t M, int C, const int32_
  * Asynchronous. */
 int sswin_softmax_rows_from_counts(const int32_t* c, const int32_t* scans, int64_t G, int32_t* rows_out, void* stream);
 
+/* values + bias[head, pos_i, pos_j], and -100 more where the mask regions of the two positions differ, for a
+ * [B, H, n, n] 'q_k' product in sorted order (sp_add_rpb and sp_add_mask, sparse_swin/swin3d_base.py:557-581), from the
+ * product's plan (as sswin_plan_from_indices writes it) instead of a linear index per entry.  values / out: [A] of
+ * `dtype`; idx: the product's [4, A] indices (rows 2 and 3 are read at 2c places per group); bias: fp32 [H, n, n]
+ * (rounded to `dtype` before the addition, as the reference's dense bias is); mask: int8 [n_mask_windows, n] region ids
+ * or NULL; c_max: largest group (at most 512 tokens).  Asynchronous. */
+int sswin_group_add_bias_mask(int dtype, const void* values, const int32_t* idx, int64_t A, const int32_t* plan, int64_t g_cap,
+                              int64_t G, int c_max, int n, const float* bias, const int8_t* mask, int n_mask_windows,
+                              void* out, void* stream);
+
+/* Window position of every attention row of a [B, H, n, n] product in sorted order: out[row_start[g] + i] = idx[2] at
+ * the first entry of row i of group g (plan as sswin_plan_from_indices writes it; out: device int32 [sum c]).  With
+ * this array in place of the token positions and the plan's row_start in place of the windows' first ranks,
+ * sswin_bias_table_grad takes the gradient of such a product's values (tokens = out, N = 0).  Asynchronous. */
+int sswin_group_row_positions(const int32_t* idx, int64_t A, const int32_t* plan, int64_t g_cap, int64_t G, int32_t* out,
+                              void* stream);
+
 /* Same three scans from a given `_c` (what the reference recomputes inside every
  * matmul_grad / qkv_transpose call, sparse_swin/ops.cu:681, 697, 965-968, 986-989,
  * 1007-1010).  c: device int32 [G].  scans: device int32 [2*G]: row 0 = exclusive scan of c,
@@ -295,7 +312,7 @@ int sswin_bias_from_table(const float* table, int table_rows, int H, const int32
  * [H,n,n] bias from a [(2w-1)^3, H] table by relative_position_index; autograd scatters back with
  * an index_add).  The index is linear in the two positions: rel(p_i,p_j) = code[p_i] - code[p_j]
  * + offset0 (code: device int32 [n]).  d_table (fp32 [table_rows, H]) is overwritten.
- * table_rows <= 1024, n <= 128.  No atomics, fixed summation order.  Asynchronous (the G == 0 case records a memset: do not capture it). */
+ * table_rows <= 4096, n <= 384 (up to 160 KB of LDS for the largest tables).  No atomics, fixed summation order.  Asynchronous (the G == 0 case records a memset: do not capture it). */
 size_t sswin_bias_table_grad_workspace_bytes(int64_t G, int H, int table_rows);
 int sswin_bias_table_grad(const int32_t* plan, int64_t g_cap, int64_t G, const int32_t* tokens,
                           int64_t N, int H, int n, const int32_t* code, int offset0, int table_rows,

@@ -646,9 +646,11 @@ __global__ __launch_bounds__(256) void rpb_gather_kernel(const float* __restrict
     for (int h = 0; h < H; ++h) bias[(int64_t)h * n * n + e] = r < (unsigned)rows ? table[(int64_t)r * H + h] : 0.f;
 }
 
-constexpr int RPBT_MAX_ROWS = 1024;
+constexpr int RPBT_MAX_ROWS = 4096;
 
-// dynamic LDS: [wave 4][half 2][rows_pad] floats, then [wave 4][buffer 2][128] position codes
+// dynamic LDS: [wave 4][half 2][rows_pad] floats, then [wave 4][buffer 2][64 * CN] position codes; windows
+// of at most 64 * CN tokens (CN = 2: windows of 5^3 positions; CN = 6: up to 384 tokens, windows of 7^3)
+template <int CN>
 __global__ __launch_bounds__(256) void rpb_table_partial_kernel(FusedGroups gt, const int32_t* __restrict__ tok_pos,
                                                                 int H, const int32_t* __restrict__ code, int offset0,
                                                                 int rows, int rows_pad, const float* __restrict__ ds,
@@ -666,7 +668,7 @@ __global__ __launch_bounds__(256) void rpb_table_partial_kernel(FusedGroups gt, 
     const int rs = (int)(sl / wslices);                         // rows rs, rs + rsplit, ... of each of them
     float* tables = rpbt_lds + wave * 2 * rows_pad;
     float* mine = tables + half * rows_pad;
-    int32_t* codes = reinterpret_cast<int32_t*>(rpbt_lds + 8 * rows_pad) + wave * 256;
+    int32_t* codes = reinterpret_cast<int32_t*>(rpbt_lds + 8 * rows_pad) + wave * (2 * 64 * CN);
     for (int e = l32; e < rows; e += 32) mine[e] = 0.f;
     // A slice takes every wslices-th window (crowded windows are neighbours in plan order, so
     // dealing them out evens the load) and, when windows are few and large, every rsplit-th row of
@@ -693,11 +695,10 @@ __global__ __launch_bounds__(256) void rpb_table_partial_kernel(FusedGroups gt, 
     for (int64_t k = ws; k < windows; k += wslices, par ^= 1) {
         const int c = c_c;
         const float* blk = ds + sq_c;
-        const int32_t* cw = codes + par * 128;
-        int cn[2] = {0, 0};
+        const int32_t* cw = codes + par * (64 * CN);
+        int cn[CN];
 #pragma unroll
-        for (int u = 0; u < 2; ++u)
-            if (lane + 64 * u < c_n) cn[u] = code[tok_pos[T_n + lane + 64 * u]];
+        for (int u = 0; u < CN; ++u) cn[u] = lane + 64 * u < c_n ? code[tok_pos[T_n + lane + 64 * u]] : 0;
         const int c_next = c_n, sq_next = sq_n;
         header(k + 2 * wslices, c_n, T_n, sq_n);
         __builtin_amdgcn_wave_barrier();
@@ -735,9 +736,9 @@ __global__ __launch_bounds__(256) void rpb_table_partial_kernel(FusedGroups gt, 
                     if (row[u] >= 0) mine[row[u]] += v[u];
             }
         }
-        int32_t* cwn = codes + (par ^ 1) * 128;
+        int32_t* cwn = codes + (par ^ 1) * (64 * CN);
 #pragma unroll
-        for (int u = 0; u < 2; ++u)
+        for (int u = 0; u < CN; ++u)
             if (lane + 64 * u < c_next) cwn[lane + 64 * u] = cn[u];
         __builtin_amdgcn_wave_barrier();
         c_c = c_next;
@@ -1004,7 +1005,8 @@ size_t sswin_bias_table_grad_workspace_bytes(int64_t G, int H, int table_rows) {
 int sswin_bias_table_grad(const int32_t* plan, int64_t g_cap, int64_t G, const int32_t* tokens, int64_t N, int H,
                           int n, const int32_t* code, int offset0, int table_rows, const float* ds, float* d_table,
                           void* ws, size_t ws_bytes, void* stream) {
-    SSWIN_CHECK(G >= 0 && G <= g_cap && H > 0 && n > 0 && n <= 128, "bias_table_grad: bad sizes");
+    SSWIN_CHECK(G >= 0 && G <= g_cap && H > 0 && n > 0, "bias_table_grad: bad sizes");
+    SSWIN_CHECK(n <= 384, "bias_table_grad: windows of %d positions are not supported (384 at most)", n);
     SSWIN_CHECK(table_rows > 0 && table_rows <= RPBT_MAX_ROWS, "bias_table_grad: a table of %d rows is not supported (%d at most)",
                 table_rows, RPBT_MAX_ROWS);
     SSWIN_CHECK(d_table, "bias_table_grad: null pointer");
@@ -1023,9 +1025,23 @@ int sswin_bias_table_grad(const int32_t* plan, int64_t g_cap, int64_t G, const i
     float* partial = static_cast<float*>(ws);
     const int64_t waves = (int64_t)slices * H;
     const int rows_pad = (table_rows + 31) / 32 * 32;
-    const size_t lds = (size_t)8 * rows_pad * sizeof(float) + 4 * 256 * sizeof(int32_t);
-    hipLaunchKernelGGL(rpb_table_partial_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), lds, s, gt, tokens + 3 * N, H,
-                       code, offset0, table_rows, rows_pad, ds, windows, wslices, rsplit, partial);
+    const int cn = n <= 128 ? 2 : 6;
+    const size_t lds = (size_t)8 * rows_pad * sizeof(float) + (size_t)4 * 2 * 64 * cn * sizeof(int32_t);
+    SSWIN_CHECK(lds <= 160 * 1024, "bias_table_grad: a table of %d rows needs %zu bytes of LDS (160 KB at most)", table_rows, lds);
+    static bool configured = false;
+    if (!configured) {                                       // more than the default 64 KB of dynamic LDS
+        SSWIN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(rpb_table_partial_kernel<2>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        SSWIN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(rpb_table_partial_kernel<6>),
+                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
+        configured = true;
+    }
+    if (cn == 2)
+        hipLaunchKernelGGL(rpb_table_partial_kernel<2>, dim3((unsigned)((waves + 3) / 4)), dim3(256), lds, s, gt, tokens + 3 * N,
+                           H, code, offset0, table_rows, rows_pad, ds, windows, wslices, rsplit, partial);
+    else
+        hipLaunchKernelGGL(rpb_table_partial_kernel<6>, dim3((unsigned)((waves + 3) / 4)), dim3(256), lds, s, gt, tokens + 3 * N,
+                           H, code, offset0, table_rows, rows_pad, ds, windows, wslices, rsplit, partial);
     hipLaunchKernelGGL(rpb_table_reduce_kernel, dim3((unsigned)((table_rows + 15) / 16), (unsigned)H), dim3(1024), 0, s,
                        partial, slices, table_rows, H, d_table);
     return launch_ok("bias table gradient");

@@ -228,6 +228,19 @@ __global__ __launch_bounds__(256) void rows_from_counts_kernel(const int32_t* __
     }
 }
 
+// position (third index row) of every attention row of a [B, H, n, n] product: out[row_start[g] + i] = the index at
+// the first entry of row i of group g
+__global__ __launch_bounds__(256) void group_row_positions_kernel(const int32_t* __restrict__ idx_pi, const int32_t* __restrict__ cs,
+                                                                  const int32_t* __restrict__ row_start,
+                                                                  const int32_t* __restrict__ sq_start, int64_t G,
+                                                                  int32_t* __restrict__ out) {
+    const int64_t g = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (g >= G) return;
+    const int c = cs[g];
+    const int64_t sq = sq_start[g];
+    for (int i = threadIdx.x & 63; i < c; i += 64) out[row_start[g] + i] = idx_pi[sq + (int64_t)i * c];
+}
+
 }  // namespace sswin
 
 using namespace sswin;
@@ -301,6 +314,16 @@ int sswin_softmax_rows_from_counts(const int32_t* c, const int32_t* scans, int64
     hipLaunchKernelGGL(rows_from_counts_kernel, dim3((unsigned)((G + 3) / 4)), dim3(256), 0, static_cast<hipStream_t>(stream), c,
                        scans, scans + G, G, rows_out);
     return launch_ok("softmax_rows_from_counts");
+}
+
+int sswin_group_row_positions(const int32_t* idx, int64_t A, const int32_t* plan, int64_t g_cap, int64_t G, int32_t* out,
+                              void* stream) {
+    SSWIN_CHECK(A >= 0 && G >= 0 && G <= g_cap, "group_row_positions: bad sizes");
+    if (G == 0 || A == 0) return 0;
+    SSWIN_CHECK(idx && plan && out, "group_row_positions: null pointer");
+    hipLaunchKernelGGL(group_row_positions_kernel, dim3((unsigned)((G + 3) / 4)), dim3(256), 0, static_cast<hipStream_t>(stream),
+                       idx + 2 * A, plan, plan + g_cap, plan + 2 * g_cap, G, out);
+    return launch_ok("group_row_positions");
 }
 
 size_t sswin_scan_counts_workspace_bytes(int64_t G) {

@@ -172,6 +172,55 @@ static int launch_softmax(const int32_t* idx_row, const void* v, const void* g, 
     return launch_ok(BWD ? "softmax backward" : "softmax forward");
 }
 
+// ------------------------------------------------------------------------------------------
+// values + bias[head, pos_i, pos_j] (+ -100 where the mask regions of the two positions differ) for a
+// [B, H, n, n] product in sorted order, group by group: what sp_add_rpb and sp_add_mask of
+// sparse_swin/swin3d_base.py:557-581 compute through a linear index per entry and two gathers.  A group's
+// row positions are the third index row at the first entry of each of its rows, its column positions the
+// fourth index row along its first row: 2c index reads per group instead of 4c^2.  One wavefront per group;
+// the two roundings of the reference (after the bias, after the mask) are kept for 16-bit values.
+// ------------------------------------------------------------------------------------------
+constexpr int GBM_MAX_C = 512;
+
+template <typename T>
+__global__ __launch_bounds__(256) void group_bias_mask_kernel(const T* __restrict__ val, const int32_t* __restrict__ idx_pi,
+                                                              const int32_t* __restrict__ idx_pj,
+                                                              const int32_t* __restrict__ cs, const int32_t* __restrict__ sq_start,
+                                                              const int32_t* __restrict__ window,
+                                                              const int32_t* __restrict__ head, int64_t G, int n,
+                                                              const float* __restrict__ bias, const int8_t* __restrict__ mask,
+                                                              int nmw, T* __restrict__ out) {
+    using AccT = typename acc_of<T>::type;
+    __shared__ int32_t pos_s[4][2][GBM_MAX_C];               // position | region << 16 of the rows and of the columns
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int64_t g = (int64_t)blockIdx.x * 4 + wave;
+    if (g >= G) return;
+    const int c = cs[g], h = head[g];
+    const int64_t sq = sq_start[g];
+    const int8_t* mrow = mask ? mask + (int64_t)(window[g] % nmw) * n : nullptr;
+    int32_t* pi = pos_s[wave][0];
+    int32_t* pj = pos_s[wave][1];
+    for (int t = lane; t < c; t += 64) {
+        const int a = idx_pi[sq + (int64_t)t * c], b = idx_pj[sq + t];
+        pi[t] = a | (mrow ? (int)mrow[a] << 16 : 0);
+        pj[t] = b | (mrow ? (int)mrow[b] << 16 : 0);
+    }
+    __builtin_amdgcn_wave_barrier();
+    const float* bias_h = bias + (int64_t)h * n * n;
+    const T* src = val + sq;
+    T* dst = out + sq;
+    const int count = c * c;
+    const float inv = 1.0f / (float)c;
+    for (int f = lane; f < count; f += 64) {
+        int i = (int)((float)f * inv);                        // f / c up to one, corrected below (f < 2^24)
+        i -= i * c > f ? 1 : 0;
+        i += (i + 1) * c <= f ? 1 : 0;
+        const int a = pi[i], b = pj[f - i * c];
+        const T with_bias = from_acc<T>(to_acc(src[f]) + to_acc(from_acc<T>((AccT)bias_h[(a & 0xffff) * n + (b & 0xffff)])));
+        dst[f] = mrow ? from_acc<T>(to_acc(with_bias) + ((a >> 16) != (b >> 16) ? (AccT)-100 : (AccT)0)) : with_bias;
+    }
+}
+
 }  // namespace sswin
 
 using namespace sswin;
@@ -201,6 +250,32 @@ int sswin_softmax_last_dim_backward(const int32_t* idx_row, const void* y, const
     if (dtype == SSWIN_F32) return launch_softmax<float, true>(idx_row, y, grad, A, out, s);
     if (dtype == SSWIN_F64) return launch_softmax<double, true>(idx_row, y, grad, A, out, s);
     return fail("softmax backward: values must be float32 or float64 (dtype code %d)", dtype);
+}
+
+int sswin_group_add_bias_mask(int dtype, const void* values, const int32_t* idx, int64_t A, const int32_t* plan, int64_t g_cap,
+                              int64_t G, int c_max, int n, const float* bias, const int8_t* mask, int n_mask_windows,
+                              void* out, void* stream) {
+    SSWIN_CHECK(A >= 0 && G >= 0 && G <= g_cap && n > 0 && n < (1 << 15), "group_add_bias_mask: bad sizes");
+    if (A == 0 || G == 0) return 0;
+    SSWIN_CHECK(values && idx && plan && bias && out, "group_add_bias_mask: null pointer");
+    SSWIN_CHECK(c_max > 0 && c_max <= GBM_MAX_C, "group_add_bias_mask: windows of %d tokens are not supported (%d at most)", c_max,
+                GBM_MAX_C);
+    SSWIN_CHECK(!mask || n_mask_windows > 0, "group_add_bias_mask: mask without window count");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const dim3 grid((unsigned)((G + 3) / 4));
+    const int32_t *cs = plan, *sq = plan + 2 * g_cap, *win = plan + 3 * g_cap, *head = plan + 4 * g_cap;
+#define SSWIN_GBM(T)                                                                                                         \
+    hipLaunchKernelGGL(group_bias_mask_kernel<T>, grid, dim3(256), 0, s, static_cast<const T*>(values), idx + 2 * A, idx + 3 * A, \
+                       cs, sq, win, head, G, n, bias, mask, n_mask_windows, static_cast<T*>(out))
+    switch (dtype) {
+        case SSWIN_F32: SSWIN_GBM(float); break;
+        case SSWIN_F64: SSWIN_GBM(double); break;
+        case SSWIN_F16: SSWIN_GBM(__half); break;
+        case SSWIN_BF16: SSWIN_GBM(__hip_bfloat16); break;
+        default: return fail("group_add_bias_mask: unsupported value dtype %d", dtype);
+    }
+#undef SSWIN_GBM
+    return launch_ok("group_add_bias_mask");
 }
 
 }  // extern "C"

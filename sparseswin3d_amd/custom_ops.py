@@ -478,6 +478,61 @@ def softmax_rows_from_counts(_c, nnz):
     return rows
 
 
+class GroupPlan:
+    """The plan behind a ``_c`` that :func:`matmul_cuda_naive` returned (group sizes, offsets, windows, heads), held
+    by reference so that a backward pass finds it however many plans have been made since."""
+
+    def __init__(self, plan, g_cap, groups, rows, c_max):
+        self.plan, self.g_cap, self.groups, self.rows, self.c_max = plan, g_cap, groups, rows, c_max
+
+
+def group_plan(_c):
+    """:class:`GroupPlan` of a ``_c`` from :func:`matmul_cuda_naive`, or None if the plan is no longer cached."""
+    hit = _plan_cache.get(_c)
+    if hit is None:
+        return None
+    plan, g_cap, totals, _ = hit
+    return GroupPlan(plan, g_cap, int(totals[0]), int(totals[1]), int(totals[3]))
+
+
+def group_add_bias_mask(values, idx, gp, n, bias32, mask):
+    """``values + bias[head, pos_i, pos_j]`` (and ``-100`` where the int8 mask regions of the two positions differ) for a
+    'q_k' product with indices ``idx`` and :class:`GroupPlan` ``gp``: sp_add_rpb followed by sp_add_mask."""
+    lib = _lib.load()
+    d = _dev(values, idx, bias32)
+    _check(values.dtype in _DTYPE_CODE and bias32.dtype == torch.float32 and idx.dtype == torch.int32, "group_add_bias_mask: dtypes")
+    _check(mask is None or mask.dtype == torch.int8, "group_add_bias_mask: the mask must hold int8 region ids")
+    values, idx, bias32 = values.contiguous(), idx.contiguous(), bias32.contiguous()
+    mask = None if mask is None else mask.contiguous()
+    out = torch.empty_like(values)
+    with torch.cuda.device(d):
+        _lib.check(lib.sswin_group_add_bias_mask(_DTYPE_CODE[values.dtype], _ptr(values), _ptr(idx), values.numel(), _ptr(gp.plan),
+                                                 gp.g_cap, gp.groups, gp.c_max, int(n), _ptr(bias32),
+                                                 _ptr(mask) if mask is not None else None,
+                                                 0 if mask is None else mask.shape[0], _ptr(out), _stream(d)))
+    return out
+
+
+def group_bias_table_grad(grad_values, idx, gp, num_heads, n, code, offset0, table_rows):
+    """Gradient of the relative position bias table [table_rows, H] from the gradient of a 'q_k' product's values
+    (fp32), summed in a fixed order."""
+    lib = _lib.load()
+    d = _dev(grad_values, idx)
+    _check(grad_values.dtype == torch.float32, "group_bias_table_grad: the gradient must be float32")
+    grad_values, idx = grad_values.contiguous(), idx.contiguous()
+    d_table = torch.empty((table_rows, num_heads), dtype=torch.float32, device=d)
+    with torch.cuda.device(d):
+        rows = torch.empty(max(gp.rows, 1), dtype=torch.int32, device=d)
+        _lib.check(lib.sswin_group_row_positions(_ptr(idx), idx.shape[1], _ptr(gp.plan), gp.g_cap, gp.groups, _ptr(rows),
+                                                 _stream(d)))
+        nbytes = lib.sswin_bias_table_grad_workspace_bytes(gp.groups, int(num_heads), int(table_rows))
+        ws = _ws(nbytes, d)
+        _lib.check(lib.sswin_bias_table_grad(_ptr(gp.plan), gp.g_cap, gp.groups, _ptr(rows), 0, int(num_heads), int(n), _ptr(code),
+                                             int(offset0), int(table_rows), _ptr(grad_values), _ptr(d_table), _ptr(ws), nbytes,
+                                             _stream(d)))
+    return d_table
+
+
 def matmul_grad_cuda_naive(mat1_v, mat2_v, _c, C_, mul_type):
     """Value-only block products of the backward pass (reference ops.cu:945-1031, 1092-1114)."""
     lib = _lib.load()

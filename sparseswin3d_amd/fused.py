@@ -281,7 +281,7 @@ class BiasTableIndex:
     @staticmethod
     def build(index: torch.Tensor, table_rows: int):
         n = index.shape[0]
-        if index.dim() != 2 or index.shape[1] != n or n > 128 or table_rows > 1024 or n == 0:
+        if index.dim() != 2 or index.shape[1] != n or n > 384 or table_rows > 4096 or n == 0:
             return None
         idx = index.to(torch.int64)
         code = idx[:, 0]

@@ -273,6 +273,53 @@ def sp_add_mask(sparse: SparseTensor, dense: torch.Tensor) -> SparseTensor:
     return SparseTensor(i, sparse.values + differ.to(sparse.values.dtype) * -100.0, sparse.shape, sparse.group_counts)
 
 
+class _GroupBiasMask(Function):
+    """``sp_add_mask(sp_add_rpb(attn, bias), mask)`` for a 'q_k' product whose bias comes from a relative position
+    table with a linear index: one pass over the values forward (positions read per group, not per entry), the table
+    gradient summed in a fixed order backward (the reference's composition goes through a linear index per entry, two
+    gathers, and an ``index_add`` into the dense bias)."""
+
+    @staticmethod
+    def forward(ctx, values, table, idx, gp, n, mask, table_index):
+        from . import _lib
+        import ctypes as C
+        num_heads = table.shape[1]
+        table32 = table.detach().to(torch.float32).contiguous()
+        bias32 = torch.empty((num_heads, n, n), dtype=torch.float32, device=values.device)
+        with torch.cuda.device(values.device):
+            _lib.check(_lib.load().sswin_bias_from_table(
+                C.c_void_p(table32.data_ptr()), table32.shape[0], num_heads, C.c_void_p(table_index.code.data_ptr()),
+                table_index.offset0, n, C.c_void_p(bias32.data_ptr()),
+                C.c_void_p(torch.cuda.current_stream(values.device).cuda_stream)))
+        ctx.save_for_backward(idx)
+        ctx.meta = (gp, n, table_index, table.shape[0], num_heads, table.dtype)
+        return ops.group_add_bias_mask(values, idx, gp, n, bias32, mask)
+
+    @staticmethod
+    @once_differentiable
+    def backward(ctx, grad):
+        (idx,) = ctx.saved_tensors
+        gp, n, table_index, table_rows, num_heads, table_dtype = ctx.meta
+        d_table = None
+        if ctx.needs_input_grad[1]:
+            d_table = ops.group_bias_table_grad(grad.float(), idx, gp, num_heads, n, table_index.code, table_index.offset0,
+                                                table_rows).to(table_dtype)
+        return grad, d_table, None, None, None, None, None
+
+
+def sp_add_table_bias_and_mask(sparse: SparseTensor, table: torch.Tensor, table_index, mask) -> SparseTensor:
+    """``sp_add_rpb`` with the bias gathered from ``table`` [rows, H], then ``sp_add_mask``, in one pass (a 'q_k'
+    product with its group sizes attached, int8 mask or None); None if the input is not of that kind."""
+    if sparse.group_counts is None or table_index is None or (mask is not None and mask.dtype != torch.int8):
+        return None
+    gp = ops.group_plan(sparse.group_counts)
+    n = sparse.shape[2]
+    if gp is None or gp.c_max > 512 or n > 384:
+        return None
+    out = _GroupBiasMask.apply(sparse.values, table, sparse.indices, gp, n, mask, table_index)
+    return SparseTensor(sparse.indices, out, sparse.shape, sparse.group_counts)
+
+
 def trunc_normal_(tensor, mean=0.0, std=1.0, a=-2.0, b=2.0):
     """Truncated-normal initialisation (inverse-CDF sampling, clamp to [a, b])."""
     if std <= 0:
@@ -586,9 +633,13 @@ class WindowAttentionSparse(nn.Module):
             return replace_feature(x, self.proj_drop(tall_linear(x.features, self.proj)))
         q, k_t, v = qkv_sparse_cuda(qkv, x.indices, b, n)
         attn = spspmm_block_naive(q * self.scale, k_t, "q_k")
-        attn = sp_add_rpb(attn, self.relative_position_bias(n, attn.values.dtype))
-        if mask is not None:
-            attn = sp_add_mask(attn, mask)
+        biased = sp_add_table_bias_and_mask(attn, self.relative_position_bias_table, self._table_index(n), mask)
+        if biased is not None:
+            attn = biased
+        else:
+            attn = sp_add_rpb(attn, self.relative_position_bias(n, attn.values.dtype))
+            if mask is not None:
+                attn = sp_add_mask(attn, mask)
         attn = softmax_last_dim(attn)
         out = spspmm_block_naive(attn, v, "qk_v")
         omap = getattr(v, "operand_map", None)

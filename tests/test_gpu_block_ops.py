@@ -292,3 +292,45 @@ def test_softmax_rows_from_the_group_sizes(ops, oracle, mix, H, hd):
     with_counts = softmax_last_dim(SparseTensor(f["s_idx"], f["s_val"], f["s_shape"], f["c1"]))
     generic = softmax_last_dim(SparseTensor(f["s_idx"], f["s_val"], f["s_shape"]))
     assert torch.equal(with_counts.values, generic.values)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window,mix,use_mask", [((5, 5, 5), "mixed", True), ((5, 5, 5), "edges", False), ((7, 7, 7), "full", True)])
+def test_table_bias_and_mask_in_one_pass(ops, oracle, window, mix, use_mask, dtype):
+    """sp_add_rpb + sp_add_mask of the reference (swin3d_base.py:557-581) against the single pass over a 'q_k' product:
+    same values bit for bit (the reference's two roundings are kept), same gradient of the values, table gradient
+    within fp32 rel 1e-5 of autograd's index_add (another summation order)."""
+    from sparseswin3d_amd.window_attention import (SparseTensor, WindowAttentionSparse, sp_add_mask, sp_add_rpb,
+                                                   sp_add_table_bias_and_mask)
+    H, hd = 3, 16
+    n = window[0] * window[1] * window[2]
+    rng = np.random.default_rng(seed_of("bias", window, mix))
+    counts = MIXES[mix] + ([300, 129] if n > 125 else [])
+    ind = ragged_window_indices(rng, counts, n)
+    B = len(counts)
+    d = qkv_operands(oracle, ind, B, n, H, hd, rng, dtype=np.float64)
+    f = run_forward(ops, oracle, d, torch.float32)
+    attn_mod = WindowAttentionSparse(H * hd, H, window, qkv_bias=False).cuda()
+    with torch.no_grad():
+        attn_mod.relative_position_bias_table.normal_(0, 0.5)
+    mask = dev(rng.integers(0, 27, size=(5, n)).astype(np.int8)) if use_mask else None
+    vals = f["s_val"].to(dtype)
+    up = torch.randn_like(vals)
+
+    v1 = vals.clone().requires_grad_(True)
+    fast = sp_add_table_bias_and_mask(SparseTensor(f["s_idx"], v1, f["s_shape"], f["c1"]),
+                                      attn_mod.relative_position_bias_table, attn_mod._table_index(n), mask)
+    assert fast is not None
+    fast.values.backward(up)
+    g_table_fast = attn_mod.relative_position_bias_table.grad.clone()
+    attn_mod.relative_position_bias_table.grad = None
+
+    v2 = vals.clone().requires_grad_(True)
+    ref = sp_add_rpb(SparseTensor(f["s_idx"], v2, f["s_shape"]), attn_mod.relative_position_bias(n, dtype))
+    if mask is not None:
+        ref = sp_add_mask(ref, mask)
+    ref.values.backward(up)
+    assert torch.equal(fast.values, ref.values)
+    assert torch.equal(v1.grad, v2.grad)
+    close(host(g_table_fast), host(attn_mod.relative_position_bias_table.grad), 1e-5 if dtype == torch.float32 else 2e-2,
+          "d bias table")
