@@ -177,11 +177,13 @@ static int launch_softmax(const int32_t* idx_row, const void* v, const void* g, 
 // [B, H, n, n] product in sorted order, group by group: what sp_add_rpb and sp_add_mask of
 // sparse_swin/swin3d_base.py:557-581 compute through a linear index per entry and two gathers.  A group's
 // row positions are the third index row at the first entry of each of its rows, its column positions the
-// fourth index row along its first row: 2c index reads per group instead of 4c^2.  One wavefront per group;
+// fourth index row along its first row: 2c index reads per group instead of 4c^2.  One wavefront per 32 rows of a group;
 // the two roundings of the reference (after the bias, after the mask) are kept for 16-bit values.
 // ------------------------------------------------------------------------------------------
 constexpr int GBM_MAX_C = 512;
+constexpr int GBM_ROWS = 32;                                 // attention rows of a group per wavefront
 
+// grid: x = four groups (one per wavefront), y = block of GBM_ROWS rows of the group
 template <typename T>
 __global__ __launch_bounds__(256) void group_bias_mask_kernel(const T* __restrict__ val, const int32_t* __restrict__ idx_pi,
                                                               const int32_t* __restrict__ idx_pj,
@@ -191,33 +193,56 @@ __global__ __launch_bounds__(256) void group_bias_mask_kernel(const T* __restric
                                                               const float* __restrict__ bias, const int8_t* __restrict__ mask,
                                                               int nmw, T* __restrict__ out) {
     using AccT = typename acc_of<T>::type;
-    __shared__ int32_t pos_s[4][2][GBM_MAX_C];               // position | region << 16 of the rows and of the columns
+    __shared__ int32_t pos_j[4][GBM_MAX_C];                  // position | region << 16 of the columns
+    __shared__ int32_t pos_i[4][GBM_ROWS];                   // ... of this block's rows
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int64_t g = (int64_t)blockIdx.x * 4 + wave;
     if (g >= G) return;
-    const int c = cs[g], h = head[g];
+    const int c = cs[g];
+    const int i0 = blockIdx.y * GBM_ROWS;
+    if (i0 >= c) return;
+    const int rows = c - i0 < GBM_ROWS ? c - i0 : GBM_ROWS;
+    const int h = head[g];
     const int64_t sq = sq_start[g];
     const int8_t* mrow = mask ? mask + (int64_t)(window[g] % nmw) * n : nullptr;
-    int32_t* pi = pos_s[wave][0];
-    int32_t* pj = pos_s[wave][1];
+    int32_t* pj = pos_j[wave];
+    int32_t* pi = pos_i[wave];
     for (int t = lane; t < c; t += 64) {
-        const int a = idx_pi[sq + (int64_t)t * c], b = idx_pj[sq + t];
-        pi[t] = a | (mrow ? (int)mrow[a] << 16 : 0);
+        const int b = idx_pj[sq + t];
         pj[t] = b | (mrow ? (int)mrow[b] << 16 : 0);
+    }
+    if (lane < rows) {
+        const int a = idx_pi[sq + (int64_t)(i0 + lane) * c];
+        pi[lane] = a | (mrow ? (int)mrow[a] << 16 : 0);
     }
     __builtin_amdgcn_wave_barrier();
     const float* bias_h = bias + (int64_t)h * n * n;
-    const T* src = val + sq;
-    T* dst = out + sq;
-    const int count = c * c;
+    const T* src = val + sq + (int64_t)i0 * c;
+    T* dst = out + sq + (int64_t)i0 * c;
+    const int count = rows * c;
     const float inv = 1.0f / (float)c;
-    for (int f = lane; f < count; f += 64) {
-        int i = (int)((float)f * inv);                        // f / c up to one, corrected below (f < 2^24)
-        i -= i * c > f ? 1 : 0;
-        i += (i + 1) * c <= f ? 1 : 0;
-        const int a = pi[i], b = pj[f - i * c];
-        const T with_bias = from_acc<T>(to_acc(src[f]) + to_acc(from_acc<T>((AccT)bias_h[(a & 0xffff) * n + (b & 0xffff)])));
-        dst[f] = mrow ? from_acc<T>(to_acc(with_bias) + ((a >> 16) != (b >> 16) ? (AccT)-100 : (AccT)0)) : with_bias;
+    for (int f0 = lane; f0 < count; f0 += 256) {             // four entries per lane in flight
+        T v[4];
+        int pa[4], pb[4];
+        float bb[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int f = f0 + 64 * u < count ? f0 + 64 * u : count - 1;
+            v[u] = src[f];
+            int i = (int)((float)f * inv);                    // f / c up to one, corrected below (f < 2^24)
+            i -= i * c > f ? 1 : 0;
+            i += (i + 1) * c <= f ? 1 : 0;
+            pa[u] = pi[i];
+            pb[u] = pj[f - i * c];
+            bb[u] = bias_h[(pa[u] & 0xffff) * n + (pb[u] & 0xffff)];
+        }
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+            const int f = f0 + 64 * u;
+            if (f >= count) break;
+            const T with_bias = from_acc<T>(to_acc(v[u]) + to_acc(from_acc<T>((AccT)bb[u])));
+            dst[f] = mrow ? from_acc<T>(to_acc(with_bias) + ((pa[u] >> 16) != (pb[u] >> 16) ? (AccT)-100 : (AccT)0)) : with_bias;
+        }
     }
 }
 
@@ -262,7 +287,7 @@ int sswin_group_add_bias_mask(int dtype, const void* values, const int32_t* idx,
                 GBM_MAX_C);
     SSWIN_CHECK(!mask || n_mask_windows > 0, "group_add_bias_mask: mask without window count");
     hipStream_t s = static_cast<hipStream_t>(stream);
-    const dim3 grid((unsigned)((G + 3) / 4));
+    const dim3 grid((unsigned)((G + 3) / 4), (unsigned)((c_max + GBM_ROWS - 1) / GBM_ROWS));
     const int32_t *cs = plan, *sq = plan + 2 * g_cap, *win = plan + 3 * g_cap, *head = plan + 4 * g_cap;
 #define SSWIN_GBM(T)                                                                                                         \
     hipLaunchKernelGGL(group_bias_mask_kernel<T>, grid, dim3(256), 0, s, static_cast<const T*>(values), idx + 2 * A, idx + 3 * A, \
