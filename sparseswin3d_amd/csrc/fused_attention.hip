@@ -15,6 +15,7 @@
 // token tensors are [N, row_stride] arrays addressed as row order[T_k + i], column col0 + h*hd + ch.
 // The softmax between the two products is the ordinary sparse row softmax; its row ids are a
 // by-product of the first kernel.
+#include <type_traits>
 #include <algorithm>
 #include <cstring>
 
@@ -631,8 +632,8 @@ __global__ __launch_bounds__(256) void rpb_grad_reduce_kernel(const float* __res
 // wavefront (h, s) walks its slice of the windows in plan order, reads the [c x c] blocks of dS
 // row by row: the entries of one row of dS go to different table rows, so a half wavefront adds a
 // row chunk with plain read-add-write, and the two halves work on alternate rows with a copy of
-// the column each (LDS float atomics would be an order of magnitude slower).  Partial columns are
-// summed in slice order by rpb_table_reduce_kernel.
+// the column each (ds_add_f32 instead: 0.15 ms against 0.04 on 12 M entries, the LDS adds one lane at a
+// time).  Partial columns are summed in slice order by rpb_table_reduce_kernel.
 // ------------------------------------------------------------------------------------------
 // bias[h][p][q] = table[code[p] - code[q] + offset0][h]: the gather of swin3d_base.py:644-647 and its
 // permute(2, 0, 1) in one pass (entries whose table row is out of range read as zero).
@@ -648,101 +649,182 @@ __global__ __launch_bounds__(256) void rpb_gather_kernel(const float* __restrict
 
 constexpr int RPBT_MAX_ROWS = 4096;
 
-// dynamic LDS: [wave 4][half 2][rows_pad] floats, then [wave 4][buffer 2][64 * CN] position codes; windows
-// of at most 64 * CN tokens (CN = 2: windows of 5^3 positions; CN = 6: up to 384 tokens, windows of 7^3)
-template <int CN>
+// f(integral_constant<U>) for U = U0 .. U1 - 1 while it returns true
+template <int U0, int U1, typename F>
+__device__ __forceinline__ void static_steps(F&& f) {
+    if constexpr (U0 < U1) {
+        if (f(std::integral_constant<int, U0>())) static_steps<U0 + 1, U1>(f);
+    }
+}
+constexpr int RPBT_U = 16;                                      // steps of a batch: one per lane of a DPP row
+// dynamic LDS: [wave 4][half 2][rows_pad] floats, then the [n] codes of the window positions
+//
+// A step adds one row of a chunk of 32 columns per half wavefront: the entries of a row go to different table
+// rows, and the halves (rows i and i + 1) add into separate copies of the table, so plain read-add-write is
+// enough and the sums have a fixed order.  RPBT_U steps (2 RPBT_U rows of one chunk) make a batch.  All loads of a
+// batch (its entries of dS, the positions of its rows and columns) follow from the window's header, so a
+// cursor runs two batches ahead of the adds and the batches wait in three register slots taken in turn (a
+// slot is never copied: a copy would wait for its loads).
 __global__ __launch_bounds__(256) void rpb_table_partial_kernel(FusedGroups gt, const int32_t* __restrict__ tok_pos,
-                                                                int H, const int32_t* __restrict__ code, int offset0,
-                                                                int rows, int rows_pad, const float* __restrict__ ds,
-                                                                int64_t windows, int wslices, int rsplit,
-                                                                float* __restrict__ partial) {
+                                                                int H, const int32_t* __restrict__ code, int n,
+                                                                int offset0, int rows, int rows_pad,
+                                                                const float* __restrict__ ds, int64_t windows,
+                                                                int wslices, int rsplit, float* __restrict__ partial) {
     extern __shared__ __attribute__((aligned(16))) float rpbt_lds[];
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int half = lane >> 5, l32 = lane & 31;
+    int32_t* code_lds = reinterpret_cast<int32_t*>(rpbt_lds + 8 * rows_pad);
+    for (int e = threadIdx.x; e < n; e += 256) code_lds[e] = code[e];
+    __syncthreads();
     const int64_t p = (int64_t)blockIdx.x * 4 + wave;           // wavefront id = s * H + h
     const int slices = wslices * rsplit;
     if (p >= (int64_t)slices * H) return;
     const int h = (int)(p % H);
     const int64_t sl = p / H;
     const int64_t ws = sl % wslices;                            // windows ws, ws + wslices, ...
-    const int rs = (int)(sl / wslices);                         // rows rs, rs + rsplit, ... of each of them
+    const int rs = (int)(sl / wslices);                         // which of the rsplit wavefronts of this window slice
     float* tables = rpbt_lds + wave * 2 * rows_pad;
     float* mine = tables + half * rows_pad;
-    int32_t* codes = reinterpret_cast<int32_t*>(rpbt_lds + 8 * rows_pad) + wave * (2 * 64 * CN);
     for (int e = l32; e < rows; e += 32) mine[e] = 0.f;
-    // A slice takes every wslices-th window (crowded windows are neighbours in plan order, so
-    // dealing them out evens the load) and, when windows are few and large, every rsplit-th row of
-    // them.  Headers are fetched two windows ahead and the position codes of the next window (two
-    // dependent loads) are in flight while the current one is added.
-    int c_c = 0, sq_c = 0, c_n = 0, T_n = 0, sq_n = 0;
-    auto header = [&](int64_t k, int& c, int& T, int& sq) {
+
+    // A slice takes every wslices-th window (crowded windows are neighbours in plan order, so dealing them out
+    // evens the load); the batches of its windows are dealt to the rsplit wavefronts of the slice.
+    // The headers of 64 windows of the slice at a time sit in the lanes (lane l: the l-th of them).
+    int hw_c = 0, hw_T = 0, hw_sq = 0;
+    auto load_headers = [&](int m_first) __attribute__((always_inline)) {
+        const int64_t k = ws + ((int64_t)m_first + lane) * wslices;
+        hw_c = 0;
         if (k < windows) {
             const int64_t g = k * H + h;
-            c = gt.c[g];
-            T = gt.T[g];
-            sq = gt.sq[g];
-        } else {
-            c = 0;
+            hw_c = gt.c[g];
+            hw_T = gt.T[g];
+            hw_sq = gt.sq[g];
         }
     };
-    {
-        int T_c = 0;
-        header(ws, c_c, T_c, sq_c);
-        header(ws + wslices, c_n, T_n, sq_n);
-        for (int t = lane; t < c_c; t += 64) codes[t] = code[tok_pos[T_c + t]];
-    }
-    int par = 0;
-    for (int64_t k = ws; k < windows; k += wslices, par ^= 1) {
-        const int c = c_c;
-        const float* blk = ds + sq_c;
-        const int32_t* cw = codes + par * (64 * CN);
-        int cn[CN];
-#pragma unroll
-        for (int u = 0; u < CN; ++u) cn[u] = lane + 64 * u < c_n ? code[tok_pos[T_n + lane + 64 * u]] : 0;
-        const int c_next = c_n, sq_next = sq_n;
-        header(k + 2 * wslices, c_n, T_n, sq_n);
-        __builtin_amdgcn_wave_barrier();
-        // item = (row i, chunk of 32 columns): all lanes of an item hit different table rows.
-        // The two halves of the wavefront take alternate rows and add into separate copies of
-        // the table, so plain read-add-write is enough.  Chunk by chunk (the lane's column and its
-        // code stay fixed), eight rows per half loaded first; addresses advance by a constant.
-        const int nch = (c + 31) >> 5;
-        const int my_rows = c > rs ? (c - rs + rsplit - 1) / rsplit : 0;
-        const int row_step = 2 * rsplit;                        // rows between a half's consecutive items
-        // Loads are unconditional (indices clamped to the block, dead items get row -1): straight-line
-        // code with all eight loads and code reads of a batch in flight together.
-        const bool have = my_rows > half;                       // this half has rows in this window
-        const int kmax = have ? (my_rows - 1 - half) >> 1 : 0;  // its last item
-        const int i0 = have ? rs + rsplit * half : 0;           // its first row
-        for (int ch = 0; ch < nch; ++ch) {
-            const int j = ch * 32 + l32;
-            const bool jlive = have && j < c;
-            const int jc = j < c ? j : 0;
-            const int cj = cw[jc] - offset0;
-            const float* src = blk + i0 * c + jc;
-            for (int k0 = 0; 2 * k0 < my_rows; k0 += 8) {       // items k0 .. k0 + 7 of each half
-                float v[8];
-                int row[8];
-#pragma unroll
-                for (int u = 0; u < 8; ++u) {
-                    const int k = k0 + u;
-                    const int kc = k < kmax ? k : kmax;
-                    v[u] = src[kc * row_step * c];
-                    const unsigned r = (unsigned)(cw[i0 + kc * row_step] - cj);
-                    row[u] = jlive && k <= kmax && r < (unsigned)rows ? (int)r : -1;
-                }
-#pragma unroll
-                for (int u = 0; u < 8; ++u)
-                    if (row[u] >= 0) mine[row[u]] += v[u];
+    constexpr int BR = 2 * RPBT_U;                              // rows of a batch
+    struct Cursor {
+        int m, m0, rot, c, T, sq, ch, ib;
+        bool valid;
+    };
+    // The batches of a window, numbered chunk by chunk inside a block of BR rows, then block by block, are dealt to
+    // the rsplit wavefronts of the slice: this one takes the numbers rot, rot + rsplit, ...; rot moves on by one
+    // with every window.  A count of chunks beyond the window's chunks carries into the row blocks.
+    auto carry = [&](Cursor cur) __attribute__((always_inline)) -> Cursor {
+        const int nch = (cur.c + 31) >> 5;
+        if (nch <= 1) {
+            cur.ib += BR * cur.ch;
+            cur.ch = 0;
+        } else {
+            while (cur.ch >= nch) {
+                cur.ch -= nch;
+                cur.ib += BR;
             }
         }
-        int32_t* cwn = codes + (par ^ 1) * (64 * CN);
+        return cur;
+    };
+    // first batch of window cur.m and after among the 64 windows whose headers are loaded, or none.  (Loading
+    // headers here, inside the pipeline, would put a wait for all loads in flight on every path.)
+    auto seek = [&](Cursor cur) __attribute__((always_inline)) -> Cursor {
+        for (;;) {
+            if (cur.m - cur.m0 == 64)                           // a batch nobody adds, at a safe address
+                return Cursor{cur.m, cur.m0, cur.rot, 1, 0, 0, 0, 0, false};
+            cur.c = __builtin_amdgcn_readlane(hw_c, cur.m - cur.m0);
+            cur.ch = cur.rot;
+            cur.ib = 0;
+            cur = carry(cur);
+            if (cur.ib < cur.c) {
+                cur.T = __builtin_amdgcn_readlane(hw_T, cur.m - cur.m0);
+                cur.sq = __builtin_amdgcn_readlane(hw_sq, cur.m - cur.m0);
+                return cur;
+            }
+            ++cur.m;
+            cur.rot = cur.rot + 1 == rsplit ? 0 : cur.rot + 1;
+        }
+    };
+    auto advance = [&](Cursor cur) __attribute__((always_inline)) -> Cursor {
+        if (!cur.valid) return cur;
+        cur.ch += rsplit;
+        cur = carry(cur);
+        if (cur.ib < cur.c) return cur;
+        ++cur.m;
+        cur.rot = cur.rot + 1 == rsplit ? 0 : cur.rot + 1;
+        return seek(cur);
+    };
+    struct Slot {
+        float v[RPBT_U];
+        int pj, pi;         // positions of this lane's column and of row ib + 2 (lane & 15) + half
+        int c, ch, ib;
+        bool valid;
+    };
+    const uint32_t table_off = (uint32_t)((wave * 2 + half) * rows_pad) * 4u;   // byte offset of this half's table
+    const uint32_t trash_off = table_off + (uint32_t)(rows_pad - 32 + l32) * 4u;   // a spare row per lane: rows_pad >= rows + 32
+    auto issue = [&](Slot& s, const Cursor& cur) __attribute__((always_inline)) {
+        // the loads are issued in any case: the waits of the other slots count on them
+        s.valid = cur.valid;
+        const uint32_t c = (uint32_t)cur.c;
+        s.c = cur.c;
+        s.ch = cur.ch;
+        s.ib = cur.ib;
+        const uint32_t j = (uint32_t)(cur.ch * 32 + l32);
+        const uint32_t jc = j < c ? j : 0u;
+        const float* src = ds + cur.sq;
+        const uint32_t last = (c - 1u) * c + jc;
+        const uint32_t first = (uint32_t)(cur.ib + half) * c + jc;
+        // unconditional loads, rows beyond the window clamped to its last row and dropped later
 #pragma unroll
-        for (int u = 0; u < CN; ++u)
-            if (lane + 64 * u < c_next) cwn[lane + 64 * u] = cn[u];
-        __builtin_amdgcn_wave_barrier();
-        c_c = c_next;
-        sq_c = sq_next;
+        for (int u = 0; u < RPBT_U; ++u) {
+            const uint32_t off = first + (uint32_t)(2 * u) * c;
+            s.v[u] = src[off < last ? off : last];
+        }
+        const uint32_t ir = (uint32_t)(cur.ib + 2 * (lane & 15) + half);
+        s.pj = tok_pos[(uint32_t)cur.T + jc];
+        s.pi = tok_pos[(uint32_t)cur.T + (ir < c ? ir : c - 1u)];
+    };
+    // Step u of a batch: rows ib + 2u (first half of the wavefront) and ib + 2u + 1 (second half).  Lane l holds
+    // the code of row ib + 2 (l & 15) + half, times four, so one DPP broadcast inside each 16 lanes (lane u
+    // of them) hands every lane the code of its half's row.  Dead rows and columns carry codes that put the byte
+    // offset beyond the table: those entries land in the spare row, without a branch.
+    auto consume = [&](const Slot& s) __attribute__((always_inline)) {
+        const int c = s.c;
+        const bool jlive = s.ch * 32 + l32 < c;
+        const bool rlive = s.ib + 2 * (lane & 15) + half < c;
+        const int cjb = jlive ? (code_lds[s.pj] - offset0) * 4 - (int)table_off : -(1 << 30);
+        const int crow4 = rlive ? code_lds[s.pi] * 4 : (1 << 30);
+        static_steps<0, RPBT_U>([&](auto uc) __attribute__((always_inline)) {
+            constexpr int u = decltype(uc)::value;
+            if (s.ib + 2 * u >= c) return false;
+            const int ci4 = __builtin_amdgcn_update_dpp(0, crow4, 0x150 + u, 0xf, 0xf, false);   // row_newbcast:u
+            const uint32_t raw = (uint32_t)(ci4 - cjb);
+            const uint32_t off = raw < trash_off ? raw : trash_off;
+            float* dst = reinterpret_cast<float*>(reinterpret_cast<char*>(rpbt_lds) + off);
+            *dst += s.v[u];
+            return true;
+        });
+    };
+    int rot = rs;
+    for (int m0 = 0; ws + (int64_t)m0 * wslices < windows; m0 += 64) {
+        load_headers(m0);
+        Cursor cur = seek(Cursor{m0, m0, rot, 1, 0, 0, 0, 0, true});
+        Slot sa, sb, sc;
+        issue(sa, cur);
+        cur = advance(cur);
+        issue(sb, cur);
+        cur = advance(cur);
+        for (;;) {
+            if (!sa.valid) break;
+            issue(sc, cur);
+            cur = advance(cur);
+            consume(sa);
+            if (!sb.valid) break;
+            issue(sa, cur);
+            cur = advance(cur);
+            consume(sb);
+            if (!sc.valid) break;
+            issue(sb, cur);
+            cur = advance(cur);
+            consume(sc);
+        }
+        rot = cur.rot;
     }
     __builtin_amdgcn_wave_barrier();
     float* out = partial + ((int64_t)h * slices + sl) * rows;
@@ -981,18 +1063,15 @@ int sswin_fused_bias_grad(const int32_t* plan, int64_t g_cap, int64_t G, const i
     return launch_ok("fused bias gradient");
 }
 
-// slices = window slices x row split: about sixteen wavefronts per CU over all heads, at least two
-// windows per window slice; few large windows are also split by rows (up to 8 ways)
-// About 4096 wavefronts (what the chip holds at once with this kernel's LDS footprint).  Rows of a
-// window are always dealt to three wavefronts: a crowded window (up to four column chunks per row)
-// otherwise makes its wavefront the straggler of the launch (cfg2: 0.051 -> 0.044 ms).
+// slices = window slices x wavefronts per window slice.  About 3072 wavefronts (three per SIMD: what a
+// wavefront waits for is its own chain of LDS read-add-writes, so a few of them share a SIMD well), eight per
+// window slice: the batches of a crowded window (up to 3 x 3 of them for 89 tokens) spread over all eight.
+// Measured on cfg2 (the two launches): 2048 wavefronts / 4 per slice 0.038 ms, 3072 / 8 0.036, 4096 / 8 0.040.
 static void table_grad_slices(int64_t windows, int H, int* wslices, int* rsplit) {
-    const int rsplit_min = 3;
-    const int64_t want = std::max<int64_t>(1, 4096 / (std::max(H, 1) * rsplit_min));
-    const int64_t useful = std::max<int64_t>(1, (windows + 1) / 2);
-    *wslices = (int)std::min<int64_t>(want, useful);
-    const int64_t waves = (int64_t)*wslices * H;
-    *rsplit = (int)std::max<int64_t>(rsplit_min, std::min<int64_t>(8, 2048 / std::max<int64_t>(waves, 1)));
+    constexpr int64_t WAVES = 3072, PER_SLICE = 8;
+    const int64_t want = std::max<int64_t>(1, WAVES / (std::max(H, 1) * PER_SLICE));
+    *wslices = (int)std::min<int64_t>(want, std::max<int64_t>(1, windows));
+    *rsplit = (int)PER_SLICE;
 }
 
 size_t sswin_bias_table_grad_workspace_bytes(int64_t G, int H, int table_rows) {
@@ -1024,24 +1103,17 @@ int sswin_bias_table_grad(const int32_t* plan, int64_t g_cap, int64_t G, const i
     const int slices = wslices * rsplit;
     float* partial = static_cast<float*>(ws);
     const int64_t waves = (int64_t)slices * H;
-    const int rows_pad = (table_rows + 31) / 32 * 32;
-    const int cn = n <= 128 ? 2 : 6;
-    const size_t lds = (size_t)8 * rows_pad * sizeof(float) + (size_t)4 * 2 * 64 * cn * sizeof(int32_t);
+    const int rows_pad = (table_rows + 31) / 32 * 32 + 32;  // 32 spare rows
+    const size_t lds = (size_t)8 * rows_pad * sizeof(float) + (size_t)n * sizeof(int32_t);
     SSWIN_CHECK(lds <= 160 * 1024, "bias_table_grad: a table of %d rows needs %zu bytes of LDS (160 KB at most)", table_rows, lds);
     static bool configured = false;
     if (!configured) {                                       // more than the default 64 KB of dynamic LDS
-        SSWIN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(rpb_table_partial_kernel<2>),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        SSWIN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(rpb_table_partial_kernel<6>),
+        SSWIN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(rpb_table_partial_kernel),
                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
         configured = true;
     }
-    if (cn == 2)
-        hipLaunchKernelGGL(rpb_table_partial_kernel<2>, dim3((unsigned)((waves + 3) / 4)), dim3(256), lds, s, gt, tokens + 3 * N,
-                           H, code, offset0, table_rows, rows_pad, ds, windows, wslices, rsplit, partial);
-    else
-        hipLaunchKernelGGL(rpb_table_partial_kernel<6>, dim3((unsigned)((waves + 3) / 4)), dim3(256), lds, s, gt, tokens + 3 * N,
-                           H, code, offset0, table_rows, rows_pad, ds, windows, wslices, rsplit, partial);
+    hipLaunchKernelGGL(rpb_table_partial_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), lds, s, gt, tokens + 3 * N, H,
+                       code, n, offset0, table_rows, rows_pad, ds, windows, wslices, rsplit, partial);
     hipLaunchKernelGGL(rpb_table_reduce_kernel, dim3((unsigned)((table_rows + 15) / 16), (unsigned)H), dim3(1024), 0, s,
                        partial, slices, table_rows, H, d_table);
     return launch_ok("bias table gradient");

@@ -305,7 +305,9 @@ __device__ __forceinline__ void rows_load(const char* __restrict__ base, uint32_
 #pragma unroll
     for (int v = 0; v < RowLoad<T>::NI; ++v) {
         const uint32_t vox = (uint32_t)__shfl((int)vox_lane, v * ROWS + lane / CH, 64);
-        r.v[v] = *reinterpret_cast<const u32x4_a*>(base + (__umul24(vox, pitch) + (uint32_t)(lane % CH) * 16u));
+        // streaming hint: a row slice is read by one task (two for a group of several tiles)
+        r.v[v] = __builtin_nontemporal_load(
+            reinterpret_cast<const u32x4_a*>(base + (__umul24(vox, pitch) + (uint32_t)(lane % CH) * 16u)));
     }
 }
 template <typename T>
