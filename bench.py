@@ -100,14 +100,18 @@ def build_workload(device, name="cfg2"):
 
 
 def run_step(wl):
-    from sparseswin3d_amd.window_attention import SparseVoxelTensor
+    from sparseswin3d_amd.window_attention import SparseVoxelTensor, replace_feature
     for blk in wl["blocks"]:                                  # as a training step does: fresh gradients
         blk["attn"].zero_grad(set_to_none=True)
     x = wl["feats"].detach().requires_grad_(True)
+    # as a stage does: the token plans of all its blocks are enqueued before the first block runs (they need the
+    # window indices only), so the totals of the later ones are on the host when their block asks
+    views = [SparseVoxelTensor(x, b["idx"], (b["n"],), b["slots"]) for b in wl["blocks"]]
+    for b, t in zip(wl["blocks"], views):
+        b["attn"].prefetch_plan(t)
     h = x
-    for b in wl["blocks"]:
-        t = SparseVoxelTensor(h, b["idx"], (b["n"],), b["slots"])
-        h = b["attn"](t, b["mask"]).features
+    for b, t in zip(wl["blocks"], views):
+        h = b["attn"](replace_feature(t, h), b["mask"]).features
     h.backward(wl["upstream"])
     return x.grad
 

@@ -294,8 +294,8 @@ class SwinTransformerBlock(nn.Module):
         self.norm2 = norm_layer(dim)
         self.mlp = MLP(hidden_size=dim, mlp_dim=int(dim * mlp_ratio), act=act_layer, dropout_rate=drop)
 
-    def forward_part1(self, x, mask_matrix):
-        x = replace_feature(x, self.norm1(x.features))
+    def window_view(self, x):
+        """``x`` seen as (window, position) tokens for this block's shift, and whether the block is shifted."""
         d, h, w = x.spatial_shape
         window_size, shift_size = get_window_size((d, h, w), self.window_size, self.shift_size)
         shifted = any(s > 0 for s in shift_size)
@@ -316,7 +316,17 @@ class SwinTransformerBlock(nn.Module):
             view.plan_cache = {}
             if cache is not None:
                 cache[key] = view
-        view = replace_feature(view, x.features)
+        return replace_feature(view, x.features), shifted
+
+    def prefetch(self, x):
+        """Enqueue this block's window indices and token plan (see ``WindowAttentionSparse.prefetch_plan``);
+        needs ``x.window_cache``."""
+        if getattr(x, "window_cache", None) is not None:
+            self.attn.prefetch_plan(self.window_view(x)[0])
+
+    def forward_part1(self, x, mask_matrix):
+        x = replace_feature(x, self.norm1(x.features))
+        view, shifted = self.window_view(x)
         out = self.attn(view, mask=mask_matrix if shifted else None)
         return replace_feature(x, out.features)
 
@@ -364,6 +374,10 @@ class BasicLayer(nn.Module):
         attn_mask = compute_mask(padded, window_size, shift_size, x.features.device)
         x = copy.copy(x)
         x.window_cache = {}                      # (window, shift) -> window indices and token plans of this stage
+        # the plans need the voxel indices only: all of them are enqueued now, so that only the first block waits
+        # for totals from the GPU
+        for blk in self.blocks:
+            blk.prefetch(x)
         for blk in self.blocks:
             x = blk(x, attn_mask)
         x.window_cache = None

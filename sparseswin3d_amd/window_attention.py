@@ -603,6 +603,25 @@ class WindowAttentionSparse(nn.Module):
         bias = _BiasTableGather.apply(table, *cached).reshape(n, n, -1)
         return bias.permute(2, 0, 1).contiguous().to(dtype)
 
+    def prefetch_plan(self, x):
+        """Enqueue the token plan of ``x``'s window indices now and keep it in ``x.plan_cache`` (created if
+        missing), so that its totals have reached the host by the time :meth:`forward` asks for them.  A stage
+        calls this for all its blocks before the first one runs.  Returns the plan, or None when this input
+        does not take the fused path."""
+        if not self.fused:
+            return None
+        from . import fused
+        n = x.spatial_shape[0]
+        if not fused.supports(x.features, n):
+            return None
+        cache = getattr(x, "plan_cache", None)
+        if cache is None:
+            cache = x.plan_cache = {}
+        plan = cache.get(self.num_heads)
+        if plan is None:
+            plan = cache[self.num_heads] = fused.TokenPlan(x.indices, x.batch_size, n, self.num_heads, defer=True)
+        return plan
+
     def forward(self, x, mask):
         n = x.spatial_shape[0]
         b = x.batch_size
