@@ -145,6 +145,7 @@ KERNEL_SYMBOLS = {
     "transpose rr": ("block_transpose_kernel<float, true", ["sparseswin3d_amd/csrc/block_matmul.hip"]),
     "softmax_last_dim_forward": ("softmax_rows_kernel<float, false", ["sparseswin3d_amd/csrc/softmax.hip"]),
     "softmax_last_dim_backward": ("softmax_rows_kernel<float, true", ["sparseswin3d_amd/csrc/softmax.hip"]),
+    "resident bias table grad": ("rpb_table_partial_kernel", ["sparseswin3d_amd/csrc/fused_attention.hip"]),
     "fused dV=P^T dO": ("fused_tok_kernel", ["sparseswin3d_amd/csrc/fused_attention.hip"]),
     "fused O=PV": ("fused_tok_kernel", ["sparseswin3d_amd/csrc/fused_attention.hip"]),
 }
