@@ -73,6 +73,14 @@ class SparseTensor:
         return f"SparseTensor(indices={self.indices}, values={self.values}, shape={self.shape})"
 
     def _sorted_order(self, indices, shape):
+        # the row-major hash is int32 (sparse_swin/ops.cu:264): beyond 2^31 it wraps and the sorted order is
+        # undefined, in the reference as well; refuse instead of returning a mis-ordered tensor
+        cells = 1
+        for extent in shape:
+            cells *= int(extent)
+        if cells > 2 ** 31:
+            raise RuntimeError(f"SparseTensor of shape {list(shape)}: its {cells} cells do not fit the int32 hash "
+                               "that orders the entries (coalesce / permute); split the batch")
         return ops.sort_indices(ops.flatten_indices(indices, shape))
 
     def coalesce(self):

@@ -62,3 +62,16 @@ def test_tall_linear_leaves_autocast_regions_to_the_layer():
     x = torch.randn(9, 48)
     with torch.autocast("cpu", dtype=torch.bfloat16):
         assert tall_linear(x, layer).dtype == torch.bfloat16
+
+
+def test_sparse_tensor_refuses_shapes_beyond_the_int32_hash():
+    # the reference's row-major hash (sparse_swin/ops.cu:264) is int32; past 2^31 cells the order of
+    # coalesce / permute is undefined there, here it is an error raised before any kernel runs
+    import pytest
+    from sparseswin3d_amd.window_attention import SparseTensor
+    idx = torch.zeros(4, 2, dtype=torch.int32)
+    t = SparseTensor(idx, torch.zeros(2), [216320, 125, 3, 32])
+    with pytest.raises(RuntimeError, match="int32 hash"):
+        t.coalesce()
+    with pytest.raises(RuntimeError, match="int32 hash"):
+        t.permute((0, 2, 1, 3))
