@@ -757,7 +757,7 @@ __global__ __launch_bounds__(256) void rpb_table_partial_kernel(FusedGroups gt, 
         bool valid;
     };
     const uint32_t table_off = (uint32_t)((wave * 2 + half) * rows_pad) * 4u;   // byte offset of this half's table
-    const uint32_t trash_off = table_off + (uint32_t)(rows_pad - 32 + l32) * 4u;   // a spare row per lane: rows_pad >= rows + 32
+    const uint32_t trash_rel = (uint32_t)(rows_pad - 32 + l32) * 4u;            // a spare row per lane: rows_pad >= rows + 32
     auto issue = [&](Slot& s, const Cursor& cur) __attribute__((always_inline)) {
         // the loads are issued in any case: the waits of the other slots count on them
         s.valid = cur.valid;
@@ -783,19 +783,19 @@ __global__ __launch_bounds__(256) void rpb_table_partial_kernel(FusedGroups gt, 
     // Step u of a batch: rows ib + 2u (first half of the wavefront) and ib + 2u + 1 (second half).  Lane l holds
     // the code of row ib + 2 (l & 15) + half, times four, so one DPP broadcast inside each 16 lanes (lane u
     // of them) hands every lane the code of its half's row.  Dead rows and columns carry codes that put the byte
-    // offset beyond the table: those entries land in the spare row, without a branch.
+    // offset beyond the table, as a table row below zero does: those entries land in a spare row, without a branch.
     auto consume = [&](const Slot& s) __attribute__((always_inline)) {
         const int c = s.c;
         const bool jlive = s.ch * 32 + l32 < c;
         const bool rlive = s.ib + 2 * (lane & 15) + half < c;
-        const int cjb = jlive ? (code_lds[s.pj] - offset0) * 4 - (int)table_off : -(1 << 30);
+        const int cjb = jlive ? (code_lds[s.pj] - offset0) * 4 : -(1 << 30);
         const int crow4 = rlive ? code_lds[s.pi] * 4 : (1 << 30);
         static_steps<0, RPBT_U>([&](auto uc) __attribute__((always_inline)) {
             constexpr int u = decltype(uc)::value;
             if (s.ib + 2 * u >= c) return false;
             const int ci4 = __builtin_amdgcn_update_dpp(0, crow4, 0x150 + u, 0xf, 0xf, false);   // row_newbcast:u
-            const uint32_t raw = (uint32_t)(ci4 - cjb);
-            const uint32_t off = raw < trash_off ? raw : trash_off;
+            const uint32_t rel = (uint32_t)(ci4 - cjb);          // table row times four; negative or dead: huge
+            const uint32_t off = (rel < trash_rel ? rel : trash_rel) + table_off;
             float* dst = reinterpret_cast<float*>(reinterpret_cast<char*>(rpbt_lds) + off);
             *dst += s.v[u];
             return true;
