@@ -226,7 +226,7 @@ __global__ __launch_bounds__(256) void block_product_simple_kernel(const T* __re
 // contiguous run in transposed order, so both sides of the copy are coalesced.  Blocks that do not fit
 // the LDS copy (more than TR_LDS_BYTES) are read with strides from global memory instead.
 // ------------------------------------------------------------------------------------------
-constexpr int TR_LDS_BYTES = 8192;
+constexpr int TR_LDS_BYTES = 6144;      // six workgroups per CU; 8192: rc 0.0207, rr 0.0353 ms on cfg2, 6144: 0.0195, 0.0345, 4096: 0.0225, 0.039
 
 // f / d through a multiplication, exact for f * d < 2^32 (blocks here stay below 2^14 entries); d = 1 has no
 // 32-bit multiplier and is marked by 0
