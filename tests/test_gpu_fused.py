@@ -214,7 +214,7 @@ def test_resident_kernels_on_ragged_windows(mix, use_mask):
     close(d_bias.cpu().numpy(), bias_r.grad.numpy(), 1e-5, "d bias")
 
 
-@pytest.mark.parametrize("mix,H", [("tiny", 1), ("mixed", 3), ("full", 2), ("many", 3)])
+@pytest.mark.parametrize("mix,H", [("tiny", 1), ("mixed", 3), ("full", 2), ("many", 3), ("crowd", 3)])
 def test_bias_table_gradient(mix, H):
     """d_table[rel(p_i, p_j), h] = sum of dS: the table-gradient kernel against a numpy scatter."""
     import ctypes as C
@@ -223,7 +223,10 @@ def test_bias_table_gradient(mix, H):
     from sparseswin3d_amd.window_attention import relative_position_index_3d
     rng = np.random.default_rng(len(mix) + H)
     mixes = {"tiny": [1, 2, 3, 1, 5, 4], "mixed": [1, 40, 2, 125, 0, 0, 17, 32, 90, 3, 3, 3, 3, 64, 65, 70],
-             "full": [125, 124, 100, 7], "many": list(rng.integers(0, 60, size=700))}
+             "full": [125, 124, 100, 7], "many": list(rng.integers(0, 60, size=700)),
+             # more than 64 windows per window slice of the kernel (128 slices for three heads): a wavefront
+             # fetches window headers more than once
+             "crowd": list(rng.integers(0, 5, size=9000))}
     counts = [int(c) for c in mixes[mix]]
     n, rows = 125, 729
     ind = ragged_window_indices(rng, counts, n)
