@@ -207,11 +207,23 @@ def bench_encoder(device, args):
 
 
 # ------------------------------------------------------------------------------------------
-def event_time_ms(fn, reps, warmup=2):
+_QUEUE_FILL = []
+
+
+def event_time_ms(fn, reps, warmup=2, queue_ahead=False):
+    """Mean GPU time of `fn` between two HIP events over `reps` calls.  `queue_ahead`: about a millisecond of plain
+    copies is enqueued in front of the first event, so the host has all `reps` calls in the queue before the GPU
+    reaches them; without it a call shorter than its own enqueue cost (about 20 us from Python) is timed at that
+    cost."""
     for _ in range(warmup):
         fn()
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     torch.cuda.synchronize()
+    if queue_ahead:
+        if not _QUEUE_FILL:
+            _QUEUE_FILL.extend(torch.empty(CALIBRATION_BYTES // 4, dtype=torch.int32, device="cuda") for _ in range(2))
+        for _ in range(max(2, reps * 2 // 5)):                # 0.1 ms each: 40 us per call to come
+            _QUEUE_FILL[1].copy_(_QUEUE_FILL[0])
     start.record()
     for _ in range(reps):
         fn()
@@ -433,7 +445,7 @@ def kernel_table(wl, reps=20, only=None):
     def measure(items, path):
         rows_ = []
         for name, fn, nbytes, calls, *flops in items:
-            ms = event_time_ms(fn, reps)
+            ms = event_time_ms(fn, reps, queue_ahead=True)
             gbps = nbytes / ms / 1e6 if nbytes else None
             rows_.append(dict(kernel=name, path=path, ms=ms, algorithmic_bytes=nbytes, calls=calls,
                               achieved_gbps=gbps, frac=(gbps / HBM_PEAK_GBPS) if gbps else None,
