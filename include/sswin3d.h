@@ -180,6 +180,15 @@ int sswin_group_add_bias_mask(int dtype, const void* values, const int32_t* idx,
                               int64_t G, int c_max, int n, const float* bias, const int8_t* mask, int n_mask_windows,
                               void* out, void* stream);
 
+/* The same with the bias taken from the relative position table itself: bias of positions p, q =
+ * table[code[p] - code[q] + offset0][head] (the gather of sparse_swin/swin3d_base.py:644-647 folded in; table: fp32
+ * [table_rows, H], code: device int32 [n], both as sswin_bias_from_table takes them; codes and table rows below 2^15).
+ * The table is a few KB where the gathered bias of 7^3 windows is 1.4 MB.  Asynchronous. */
+int sswin_group_add_table_bias_mask(int dtype, const void* values, const int32_t* idx, int64_t A, const int32_t* plan,
+                                    int64_t g_cap, int64_t G, int c_max, int n, const float* table, int table_rows, int H,
+                                    const int32_t* code, int offset0, const int8_t* mask, int n_mask_windows, void* out,
+                                    void* stream);
+
 /* Window position of every attention row of a [B, H, n, n] product in sorted order: out[row_start[g] + i] = idx[2] at
  * the first entry of row i of group g (plan as sswin_plan_from_indices writes it; out: device int32 [sum c]).  With
  * this array in place of the token positions and the plan's row_start in place of the windows' first ranks,

@@ -37,6 +37,8 @@ SIGNATURES = {
     "sswin_permute_heads_order": (_i32, [_vp, _i64, _i32, _vp, _i64, _i64, _vp, _vp, _vp]),
     "sswin_softmax_rows_from_counts": (_i32, [_vp, _vp, _i64, _vp, _vp]),
     "sswin_group_add_bias_mask": (_i32, [_i32, _vp, _vp, _i64, _vp, _i64, _i64, _i32, _i32, _vp, _vp, _i32, _vp, _vp]),
+    "sswin_group_add_table_bias_mask": (_i32, [_i32, _vp, _vp, _i64, _vp, _i64, _i64, _i32, _i32, _vp, _i32, _i32, _vp, _i32, _vp,
+                                               _i32, _vp, _vp]),
     "sswin_group_row_positions": (_i32, [_vp, _i64, _vp, _i64, _i64, _vp, _vp]),
     "sswin_scan_counts_workspace_bytes": (_sz, [_i64]),
     "sswin_scan_counts": (_i32, [_vp, _i64, _vp, _vp, _sz, _vp]),
@@ -78,7 +80,7 @@ SIGNATURES = {
                                                _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i32, _vp]),
 }
 
-ABI_VERSION = 21
+ABI_VERSION = 22
 _lib = None
 
 

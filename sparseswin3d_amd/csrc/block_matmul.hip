@@ -224,7 +224,7 @@ __global__ __launch_bounds__(256) void block_product_simple_kernel(const T* __re
 // One wavefront per group.  A group's block is a few KB: it is read as one contiguous run into a
 // wave-private LDS copy (odd pitch, so a column is spread over the banks) and written back as one
 // contiguous run in transposed order, so both sides of the copy are coalesced.  Blocks that do not fit
-// the LDS copy (more than TR_LDS_BYTES) are read with strides from global memory instead.
+// the LDS copy (more than TR_LDS_BYTES) go through it tile by tile.
 // ------------------------------------------------------------------------------------------
 constexpr int TR_LDS_BYTES = 6144;      // six workgroups per CU; 8192: rc 0.0207, rr 0.0353 ms on cfg2, 6144: 0.0195, 0.0345, 4096: 0.0225, 0.039
 
@@ -278,38 +278,50 @@ __global__ __launch_bounds__(256) void block_transpose_kernel(const T* __restric
             }
             return;
         }
-        // slabs of R input columns (= R output rows), R a power of two: reads are runs of R values per input
-        // row, writes one contiguous run per slab
-        int logR = 6;
-        while (logR > 0 && rows * ((1 << logR) | 1) > cap) --logR;
-        const int R = 1 << logR, rp = R | 1;
-        for (int j0 = 0; j0 < cols; j0 += R) {
-            const int Rc = cols - j0 < R ? cols - j0 : R;
-            const int slab = rows << logR;
-            for (int e0 = lane; e0 < slab; e0 += 64 * U) {
-                T v[U];
+        // larger blocks: tiles of TS x TS values through the LDS copy (pitch TS + 1).  A tile is read as runs of
+        // TS values of TS input rows and written as runs of TS values of TS output rows; the loads of the next
+        // tile are issued before the current one passes through LDS (two register sets taken in turn: a copy
+        // of loaded registers would wait for them).
+        constexpr int TS = sizeof(T) <= 4 ? 32 : 16;
+        constexpr int PER = TS * TS / 64;                     // values of a tile per lane
+        static_assert((TS + 1) * TS * (int)sizeof(T) <= TR_LDS_BYTES, "a tile fits the LDS copy");
+        const int tcols = (cols + TS - 1) / TS;
+        const int tiles = ((rows + TS - 1) / TS) * tcols;
+        auto fetch = [&](int tile, T (&v)[PER]) __attribute__((always_inline)) {
+            const int bi = tile / tcols, bj = tile - bi * tcols;
 #pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const int e = e0 + 64 * u;
-                    const int io = e >> logR, jr = e & (R - 1);
-                    const bool ok = e < slab && jr < Rc;
-                    v[u] = src[ok ? (int64_t)io * cols + j0 + jr : 0];
-                }
+            for (int u = 0; u < PER; ++u) {
+                const int e = lane + 64 * u;
+                const int gi = bi * TS + e / TS, gj = bj * TS + e % TS;
+                const bool ok = gi < rows && gj < cols;
+                v[u] = src[ok ? (int64_t)gi * cols + gj : 0];
+            }
+        };
+        auto emit = [&](int tile, const T (&v)[PER]) __attribute__((always_inline)) {
+            const int bi = tile / tcols, bj = tile - bi * tcols;
+            __builtin_amdgcn_wave_barrier();
 #pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const int e = e0 + 64 * u;
-                    const int io = e >> logR, jr = e & (R - 1);
-                    if (e < slab && jr < Rc) t[io * rp + jr] = v[u];
-                }
+            for (int u = 0; u < PER; ++u) {
+                const int e = lane + 64 * u;
+                t[(e / TS) * (TS + 1) + e % TS] = v[u];
             }
             __builtin_amdgcn_wave_barrier();
-            T* d = dst + (int64_t)j0 * rows;
-            const int n_out = Rc * rows;
-            for (int f = lane; f < n_out; f += 64) {
-                const int jr = div_by(f, m_rows), io = f - jr * rows;
-                d[f] = t[io * rp + jr];
+#pragma unroll
+            for (int u = 0; u < PER; ++u) {
+                const int e = lane + 64 * u;
+                const int orow = e / TS, ocol = e % TS;           // inside the output tile: row = input column
+                const int gi = bj * TS + orow, gj = bi * TS + ocol;
+                if (gi < cols && gj < rows) dst[(int64_t)gi * rows + gj] = t[ocol * (TS + 1) + orow];
             }
-            __builtin_amdgcn_wave_barrier();
+        };
+        T va[PER], vb[PER];
+        fetch(0, va);
+        for (int tile = 0; tile < tiles; tile += 2) {
+            if (tile + 1 < tiles) fetch(tile + 1, vb);
+            emit(tile, va);
+            if (tile + 1 >= tiles) break;
+            if (tile + 2 < tiles) fetch(tile + 2, va);
+            emit(tile + 1, vb);
         }
     }
 }

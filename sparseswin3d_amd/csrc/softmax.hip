@@ -182,15 +182,20 @@ static int launch_softmax(const int32_t* idx_row, const void* v, const void* g, 
 // ------------------------------------------------------------------------------------------
 constexpr int GBM_MAX_C = 512;
 constexpr int GBM_ROWS = 32;                                 // attention rows of a group per wavefront
+constexpr int GBM_U = 8;                                     // rows in flight per lane (4: 118 us, 8: 112, 16: 107 on 7^3 windows; 38, 38, 41 on 5^3)
 
-// grid: x = four groups (one per wavefront), y = block of GBM_ROWS rows of the group
-template <typename T>
+// grid: x = four groups (one per wavefront), y = block of GBM_ROWS rows of the group.
+// TABLE: `bias` is the relative position table [rows, H] itself and `code` the linear index of a position
+// (bias of positions p, q = table[code[p] - code[q] + offset0]): the table is a few KB where the gathered [H, n, n]
+// bias of 7^3 windows is 1.4 MB, so the gathers stay in the L1.
+template <typename T, bool TABLE>
 __global__ __launch_bounds__(256) void group_bias_mask_kernel(const T* __restrict__ val, const int32_t* __restrict__ idx_pi,
                                                               const int32_t* __restrict__ idx_pj,
                                                               const int32_t* __restrict__ cs, const int32_t* __restrict__ sq_start,
                                                               const int32_t* __restrict__ window,
                                                               const int32_t* __restrict__ head, int64_t G, int n,
-                                                              const float* __restrict__ bias, const int8_t* __restrict__ mask,
+                                                              const float* __restrict__ bias, const int32_t* __restrict__ code,
+                                                              int offset0, int H, const int8_t* __restrict__ mask,
                                                               int nmw, T* __restrict__ out) {
     using AccT = typename acc_of<T>::type;
     __shared__ int32_t pos_j[4][GBM_MAX_C];                  // position | region << 16 of the columns
@@ -207,41 +212,48 @@ __global__ __launch_bounds__(256) void group_bias_mask_kernel(const T* __restric
     const int8_t* mrow = mask ? mask + (int64_t)(window[g] % nmw) * n : nullptr;
     int32_t* pj = pos_j[wave];
     int32_t* pi = pos_i[wave];
+    // low half: the position (TABLE: its code), high half: its mask region
     for (int t = lane; t < c; t += 64) {
         const int b = idx_pj[sq + t];
-        pj[t] = b | (mrow ? (int)mrow[b] << 16 : 0);
+        pj[t] = (TABLE ? code[b] : b) | (mrow ? (int)mrow[b] << 16 : 0);
     }
     if (lane < rows) {
         const int a = idx_pi[sq + (int64_t)(i0 + lane) * c];
-        pi[lane] = a | (mrow ? (int)mrow[a] << 16 : 0);
+        pi[lane] = (TABLE ? code[a] : a) | (mrow ? (int)mrow[a] << 16 : 0);
     }
     __builtin_amdgcn_wave_barrier();
-    const float* bias_h = bias + (int64_t)h * n * n;
+    const float* bias_h = TABLE ? bias + h : bias + (int64_t)h * n * n;
     const T* src = val + sq + (int64_t)i0 * c;
     T* dst = out + sq + (int64_t)i0 * c;
-    const int count = rows * c;
-    const float inv = 1.0f / (float)c;
-    for (int f0 = lane; f0 < count; f0 += 256) {             // four entries per lane in flight
-        T v[4];
-        int pa[4], pb[4];
-        float bb[4];
+    // Row by row, a lane keeps its column: the column's code and region are read once per chunk of columns, the
+    // row's are one LDS broadcast, and no entry needs a division.  Rows of at most 32 entries go two to a wavefront.
+    const int cw = c <= 32 ? 32 : 64;                        // lanes per row
+    const int rstep = c <= 32 ? 2 : 1;                       // rows per step
+    const int jl = lane & (cw - 1), rl = c <= 32 ? lane >> 5 : 0;
+    for (int j0 = 0; j0 < c; j0 += cw) {
+        const int j = j0 + jl;
+        const bool jok = j < c;
+        const int pbv = pj[jok ? j : 0];
+        const int pb_lo = pbv & 0xffff, pb_hi = pbv >> 16;
+        for (int i = rl; i < rows; i += GBM_U * rstep) {     // GBM_U steps in flight
+            T v[GBM_U];
+            int pa[GBM_U];
+            float bb[GBM_U];
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int f = f0 + 64 * u < count ? f0 + 64 * u : count - 1;
-            v[u] = src[f];
-            int i = (int)((float)f * inv);                    // f / c up to one, corrected below (f < 2^24)
-            i -= i * c > f ? 1 : 0;
-            i += (i + 1) * c <= f ? 1 : 0;
-            pa[u] = pi[i];
-            pb[u] = pj[f - i * c];
-            bb[u] = bias_h[(pa[u] & 0xffff) * n + (pb[u] & 0xffff)];
-        }
+            for (int u = 0; u < GBM_U; ++u) {
+                const int ii = i + u * rstep;
+                const int ic = ii < rows ? ii : rows - 1;
+                v[u] = src[jok ? ic * c + j : 0];
+                pa[u] = pi[ic];
+                bb[u] = TABLE ? bias_h[((pa[u] & 0xffff) - pb_lo + offset0) * H] : bias_h[(pa[u] & 0xffff) * n + pb_lo];
+            }
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            const int f = f0 + 64 * u;
-            if (f >= count) break;
-            const T with_bias = from_acc<T>(to_acc(v[u]) + to_acc(from_acc<T>((AccT)bb[u])));
-            dst[f] = mrow ? from_acc<T>(to_acc(with_bias) + ((pa[u] >> 16) != (pb[u] >> 16) ? (AccT)-100 : (AccT)0)) : with_bias;
+            for (int u = 0; u < GBM_U; ++u) {
+                const int ii = i + u * rstep;
+                if (ii >= rows || !jok) continue;
+                const T with_bias = from_acc<T>(to_acc(v[u]) + to_acc(from_acc<T>((AccT)bb[u])));
+                dst[ii * c + j] = mrow ? from_acc<T>(to_acc(with_bias) + ((pa[u] >> 16) != pb_hi ? (AccT)-100 : (AccT)0)) : with_bias;
+            }
         }
     }
 }
@@ -277,30 +289,55 @@ int sswin_softmax_last_dim_backward(const int32_t* idx_row, const void* y, const
     return fail("softmax backward: values must be float32 or float64 (dtype code %d)", dtype);
 }
 
-int sswin_group_add_bias_mask(int dtype, const void* values, const int32_t* idx, int64_t A, const int32_t* plan, int64_t g_cap,
-                              int64_t G, int c_max, int n, const float* bias, const int8_t* mask, int n_mask_windows,
-                              void* out, void* stream) {
-    SSWIN_CHECK(A >= 0 && G >= 0 && G <= g_cap && n > 0 && n < (1 << 15), "group_add_bias_mask: bad sizes");
+static int launch_group_bias_mask(const char* who, bool table_form, int dtype, const void* values, const int32_t* idx,
+                                  int64_t A, const int32_t* plan, int64_t g_cap, int64_t G, int c_max, int n, const float* bias,
+                                  const int32_t* code, int offset0, int H, const int8_t* mask, int n_mask_windows, void* out,
+                                  void* stream) {
+    SSWIN_CHECK(A >= 0 && G >= 0 && G <= g_cap && n > 0 && n < (1 << 15), "%s: bad sizes", who);
     if (A == 0 || G == 0) return 0;
-    SSWIN_CHECK(values && idx && plan && bias && out, "group_add_bias_mask: null pointer");
-    SSWIN_CHECK(c_max > 0 && c_max <= GBM_MAX_C, "group_add_bias_mask: windows of %d tokens are not supported (%d at most)", c_max,
-                GBM_MAX_C);
-    SSWIN_CHECK(!mask || n_mask_windows > 0, "group_add_bias_mask: mask without window count");
+    SSWIN_CHECK(values && idx && plan && bias && out, "%s: null pointer", who);
+    SSWIN_CHECK(c_max > 0 && c_max <= GBM_MAX_C, "%s: windows of %d tokens are not supported (%d at most)", who, c_max, GBM_MAX_C);
+    SSWIN_CHECK(!mask || n_mask_windows > 0, "%s: mask without window count", who);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const dim3 grid((unsigned)((G + 3) / 4), (unsigned)((c_max + GBM_ROWS - 1) / GBM_ROWS));
     const int32_t *cs = plan, *sq = plan + 2 * g_cap, *win = plan + 3 * g_cap, *head = plan + 4 * g_cap;
-#define SSWIN_GBM(T)                                                                                                         \
-    hipLaunchKernelGGL(group_bias_mask_kernel<T>, grid, dim3(256), 0, s, static_cast<const T*>(values), idx + 2 * A, idx + 3 * A, \
-                       cs, sq, win, head, G, n, bias, mask, n_mask_windows, static_cast<T*>(out))
+#define SSWIN_GBM(T)                                                                                                   \
+    do {                                                                                                               \
+        if (table_form)                                                                                                \
+            hipLaunchKernelGGL((group_bias_mask_kernel<T, true>), grid, dim3(256), 0, s, static_cast<const T*>(values), \
+                               idx + 2 * A, idx + 3 * A, cs, sq, win, head, G, n, bias, code, offset0, H, mask,        \
+                               n_mask_windows, static_cast<T*>(out));                                                  \
+        else                                                                                                           \
+            hipLaunchKernelGGL((group_bias_mask_kernel<T, false>), grid, dim3(256), 0, s, static_cast<const T*>(values), \
+                               idx + 2 * A, idx + 3 * A, cs, sq, win, head, G, n, bias, code, offset0, H, mask,        \
+                               n_mask_windows, static_cast<T*>(out));                                                  \
+    } while (0)
     switch (dtype) {
         case SSWIN_F32: SSWIN_GBM(float); break;
         case SSWIN_F64: SSWIN_GBM(double); break;
         case SSWIN_F16: SSWIN_GBM(__half); break;
         case SSWIN_BF16: SSWIN_GBM(__hip_bfloat16); break;
-        default: return fail("group_add_bias_mask: unsupported value dtype %d", dtype);
+        default: return fail("%s: unsupported value dtype %d", who, dtype);
     }
 #undef SSWIN_GBM
-    return launch_ok("group_add_bias_mask");
+    return launch_ok(who);
+}
+
+int sswin_group_add_bias_mask(int dtype, const void* values, const int32_t* idx, int64_t A, const int32_t* plan, int64_t g_cap,
+                              int64_t G, int c_max, int n, const float* bias, const int8_t* mask, int n_mask_windows,
+                              void* out, void* stream) {
+    return launch_group_bias_mask("group_add_bias_mask", false, dtype, values, idx, A, plan, g_cap, G, c_max, n, bias, nullptr, 0,
+                                  1, mask, n_mask_windows, out, stream);
+}
+
+int sswin_group_add_table_bias_mask(int dtype, const void* values, const int32_t* idx, int64_t A, const int32_t* plan,
+                                    int64_t g_cap, int64_t G, int c_max, int n, const float* table, int table_rows, int H,
+                                    const int32_t* code, int offset0, const int8_t* mask, int n_mask_windows, void* out,
+                                    void* stream) {
+    SSWIN_CHECK(table_rows > 0 && table_rows < (1 << 15) && H > 0 && (A == 0 || G == 0 || code),
+                "group_add_table_bias_mask: bad table");
+    return launch_group_bias_mask("group_add_table_bias_mask", true, dtype, values, idx, A, plan, g_cap, G, c_max, n, table, code,
+                                  offset0, H, mask, n_mask_windows, out, stream);
 }
 
 }  // extern "C"

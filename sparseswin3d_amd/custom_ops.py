@@ -513,6 +513,26 @@ def group_add_bias_mask(values, idx, gp, n, bias32, mask):
     return out
 
 
+def group_add_table_bias_mask(values, idx, gp, n, table32, code, offset0, mask):
+    """:func:`group_add_bias_mask` with the bias taken from the relative position table ``table32`` [rows, H] itself:
+    bias of positions p, q = ``table32[code[p] - code[q] + offset0, head]``."""
+    lib = _lib.load()
+    d = _dev(values, idx, table32, code)
+    _check(values.dtype in _DTYPE_CODE and table32.dtype == torch.float32 and idx.dtype == torch.int32 and code.dtype == torch.int32,
+           "group_add_table_bias_mask: dtypes")
+    _check(mask is None or mask.dtype == torch.int8, "group_add_table_bias_mask: the mask must hold int8 region ids")
+    _check(table32.dim() == 2 and code.numel() >= n, "group_add_table_bias_mask: table [rows, H] and one code per position")
+    values, idx, table32, code = values.contiguous(), idx.contiguous(), table32.contiguous(), code.contiguous()
+    mask = None if mask is None else mask.contiguous()
+    out = torch.empty_like(values)
+    with torch.cuda.device(d):
+        _lib.check(lib.sswin_group_add_table_bias_mask(
+            _DTYPE_CODE[values.dtype], _ptr(values), _ptr(idx), values.numel(), _ptr(gp.plan), gp.g_cap, gp.groups, gp.c_max, int(n),
+            _ptr(table32), table32.shape[0], table32.shape[1], _ptr(code), int(offset0),
+            _ptr(mask) if mask is not None else None, 0 if mask is None else mask.shape[0], _ptr(out), _stream(d)))
+    return out
+
+
 def group_bias_table_grad(grad_values, idx, gp, num_heads, n, code, offset0, table_rows):
     """Gradient of the relative position bias table [table_rows, H] from the gradient of a 'q_k' product's values
     (fp32), summed in a fixed order."""

@@ -289,18 +289,21 @@ class _GroupBiasMask(Function):
 
     @staticmethod
     def forward(ctx, values, table, idx, gp, n, mask, table_index):
-        from . import _lib
-        import ctypes as C
         num_heads = table.shape[1]
         table32 = table.detach().to(torch.float32).contiguous()
+        ctx.save_for_backward(idx)
+        ctx.meta = (gp, n, table_index, table.shape[0], num_heads, table.dtype)
+        if table.shape[0] < (1 << 15):
+            # the kernel reads the table itself (a few KB; the gathered [H, n, n] bias of 7^3 windows is 1.4 MB)
+            return ops.group_add_table_bias_mask(values, idx, gp, n, table32, table_index.code, table_index.offset0, mask)
+        from . import _lib
+        import ctypes as C
         bias32 = torch.empty((num_heads, n, n), dtype=torch.float32, device=values.device)
         with torch.cuda.device(values.device):
             _lib.check(_lib.load().sswin_bias_from_table(
                 C.c_void_p(table32.data_ptr()), table32.shape[0], num_heads, C.c_void_p(table_index.code.data_ptr()),
                 table_index.offset0, n, C.c_void_p(bias32.data_ptr()),
                 C.c_void_p(torch.cuda.current_stream(values.device).cuda_stream)))
-        ctx.save_for_backward(idx)
-        ctx.meta = (gp, n, table_index, table.shape[0], num_heads, table.dtype)
         return ops.group_add_bias_mask(values, idx, gp, n, bias32, mask)
 
     @staticmethod

@@ -334,3 +334,7 @@ def test_table_bias_and_mask_in_one_pass(ops, oracle, window, mix, use_mask, dty
     assert torch.equal(v1.grad, v2.grad)
     close(host(g_table_fast), host(attn_mod.relative_position_bias_table.grad), 1e-5 if dtype == torch.float32 else 2e-2,
           "d bias table")
+    # the entry point that takes the gathered [H, n, n] bias gives the same bits as the one that reads the table
+    gp = ops.group_plan(f["c1"])
+    dense = attn_mod.relative_position_bias(n, torch.float32).detach()
+    assert torch.equal(ops.group_add_bias_mask(vals, f["s_idx"], gp, n, dense, mask), fast.values.detach())
