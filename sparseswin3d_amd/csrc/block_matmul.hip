@@ -122,22 +122,25 @@ __global__ __launch_bounds__(256) void block_product_mfma_kernel(const T* __rest
         const T* B = m2 + d.b_off;
         f32x16 acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
         for (int kc = 0; kc < d.K; kc += 32) {
-            const int kb = kc + half * 16;
-            const int left = d.K - kb;                          // values of k left for this lane half
+            // the (at most 32) values of k of this round are split evenly between the two lane halves, so a
+            // reduction over 16 channels takes eight matrix steps, not sixteen with one half feeding zeros
+            const int chunk = d.K - kc < 32 ? d.K - kc : 32;
+            const int kh = (chunk + 1) >> 1;                    // uniform: steps that carry data
+            const int kb = kc + half * kh;
+            const int left = half ? chunk - kh : kh;            // values of k of this lane half
             float a[16], b[16];
-            load_run16<T>(A + (int64_t)i_a * d.K + kb, i_a < d.I ? clamp16(left) : 0, a);
+            load_run16<T>(A + (int64_t)i_a * d.K + kb, i_a < d.I ? left : 0, a);
             if (b_is_kmajor<MODE>()) {
                 const T* bp = B + (int64_t)kb * d.J + j_b;
                 const bool jin = j_b < d.J;
 #pragma unroll
                 for (int s = 0; s < 16; ++s) b[s] = (jin && s < left) ? to_acc(bp[(int64_t)s * d.J]) : 0.f;
             } else {
-                load_run16<T>(B + (int64_t)j_b * d.K + kb, j_b < d.J ? clamp16(left) : 0, b);
+                load_run16<T>(B + (int64_t)j_b * d.K + kb, j_b < d.J ? left : 0, b);
             }
-            const int steps = d.K - kc;                          // uniform: steps that carry data
 #pragma unroll
             for (int s = 0; s < 16; ++s)
-                if (s < steps) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], acc, 0, 0, 0);
+                if (s < kh) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], acc, 0, 0, 0);
         }
 
         if (j_b < d.J) {

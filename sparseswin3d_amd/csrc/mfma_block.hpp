@@ -31,6 +31,15 @@ __device__ __forceinline__ void load_run16(const T* __restrict__ p, int valid, f
 #pragma unroll
             for (int s = 0; s < 16; ++s) x[s] = to_acc(p[s]);
         }
+    } else if (valid == 8 && std::is_same<T, float>::value) {   // half of a 16-channel reduction
+        const f32x4_u* q = reinterpret_cast<const f32x4_u*>(p);
+#pragma unroll
+        for (int v = 0; v < 2; ++v) {
+            const f32x4_u t = q[v];
+            x[4 * v] = t.x; x[4 * v + 1] = t.y; x[4 * v + 2] = t.z; x[4 * v + 3] = t.w;
+        }
+#pragma unroll
+        for (int s = 8; s < 16; ++s) x[s] = 0.f;
     } else {
 #pragma unroll
         for (int s = 0; s < 16; ++s) x[s] = s < valid ? to_acc(p[s]) : 0.f;
