@@ -133,11 +133,16 @@ class _spspmm_block_naive(Function):
         ctx.mul_type = mul_type
         ctx.inner = mat1_shape[-1] if mul_type == "q_k" else mat2_shape[-1]
         ctx.mark_non_differentiable(mat3_idx, counts)
+        # without this autograd hands backward a zero tensor for every output that has no gradient, the [4, nnz]
+        # index matrix included (a 360 MB fill for 7^3 windows)
+        ctx.set_materialize_grads(False)
         return mat3_idx, mat3_v, mat3_shape, counts
 
     @staticmethod
     @once_differentiable
     def backward(ctx, _grad_idx, grad_v, _grad_shape, _grad_counts):
+        if grad_v is None:
+            return None, None, None, None, None, None, None
         grad_v = grad_v.contiguous()
         mat2_v, mat1_v, counts = ctx.saved_tensors
         inner = ctx.inner
