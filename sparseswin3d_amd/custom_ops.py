@@ -269,13 +269,26 @@ class _PlanCache:
     def __init__(self, capacity=32):
         self.capacity = capacity
         self.entries = OrderedDict()
+        self.scans = {}                              # key -> contiguous [2 * G] scans of a plan with g_cap > G
 
     def put(self, c_view, plan, g_cap, totals):
         key = (c_view.device.index, c_view.data_ptr(), c_view.numel())
         self.entries[key] = (plan, g_cap, totals, c_view._version)
+        self.scans.pop(key, None)
         self.entries.move_to_end(key)
         while len(self.entries) > self.capacity:
-            self.entries.popitem(last=False)
+            self.scans.pop(self.entries.popitem(last=False)[0], None)
+
+    def packed_scans(self, c, hit):
+        """The two scan rows of a cached plan side by side (the layout the kernels take), packed once per plan."""
+        key = (c.device.index, c.data_ptr(), c.numel())
+        packed = self.scans.get(key)
+        if packed is None:
+            plan, g_cap = hit[0], hit[1]
+            rows = plan.view(5, g_cap)
+            g = c.numel()
+            packed = self.scans[key] = torch.stack([rows[1, :g], rows[2, :g]]).reshape(-1)
+        return packed
 
     def get(self, c):
         key = (c.device.index, c.data_ptr(), c.numel())
@@ -287,6 +300,7 @@ class _PlanCache:
 
     def clear(self):
         self.entries.clear()
+        self.scans.clear()
 
 
 _plan_cache = _PlanCache()
@@ -348,7 +362,7 @@ def _scans_for(c, lib, d):
         rows = plan.view(5, g_cap)
         if g_cap == g:
             return rows[1:3].reshape(-1), totals[2]
-        return torch.stack([rows[1, :g], rows[2, :g]]).reshape(-1), totals[2]
+        return _plan_cache.packed_scans(c, hit), totals[2]
     scans = torch.empty(2 * max(g, 1), dtype=torch.int32, device=d)
     nbytes = lib.sswin_scan_counts_workspace_bytes(g)
     ws = _ws(nbytes, d)
