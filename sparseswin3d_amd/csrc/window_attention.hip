@@ -298,16 +298,20 @@ struct RowLoad {
 };
 
 // vox_lane: voxel of row l32, held by lanes l32 and l32 + 32
-template <typename T>
+// STREAM: the rows belong to a group of one tile, so no other task reads them: loaded with the streaming hint (the
+// key-side task of one-tile groups in the backward: 0.1203 -> 0.1187 ms on cfg2, 0.096 -> 0.095 on cfg3).  Rows of
+// larger groups are read by up to eight tasks and must stay cached: with the hint on all loads the bf16 backward of
+// 100-125-token windows went from 0.097 to 0.156 ms and the forward from 0.049 to 0.062; in the forward the hint for
+// one-tile groups alone was no gain either (cfg2 0.0568 against 0.0572 ms, cfg3 0.0441 against 0.0425).
+template <typename T, bool STREAM = false>
 __device__ __forceinline__ void rows_load(const char* __restrict__ base, uint32_t pitch, uint32_t vox_lane, int lane,
                                           RowLoad<T>& r) {
     constexpr int CH = RowLoad<T>::CH, ROWS = RowLoad<T>::ROWS;
 #pragma unroll
     for (int v = 0; v < RowLoad<T>::NI; ++v) {
         const uint32_t vox = (uint32_t)__shfl((int)vox_lane, v * ROWS + lane / CH, 64);
-        // streaming hint: a row slice is read by one task (two for a group of several tiles)
-        r.v[v] = __builtin_nontemporal_load(
-            reinterpret_cast<const u32x4_a*>(base + (__umul24(vox, pitch) + (uint32_t)(lane % CH) * 16u)));
+        const u32x4_a* p = reinterpret_cast<const u32x4_a*>(base + (__umul24(vox, pitch) + (uint32_t)(lane % CH) * 16u));
+        r.v[v] = STREAM ? __builtin_nontemporal_load(p) : *p;
     }
 }
 template <typename T>
@@ -1132,11 +1136,12 @@ __device__ __forceinline__ void bwd_kv_task(const WAttnCommon& a, int64_t task, 
     float kb[16], vb[16];
     {
         RowLoad<T> rk, rv;
-        rows_load<T>(head_base<T>(tk, h), pitch_of<T>(tk), vox_j, lane, rk);
-        rows_load<T>(head_base<T>(tv, h), pitch_of<T>(tv), vox_j, lane, rv);
-        rows_load<T>(qbase, qpitch, qcur.vox, lane, rq);
-        rows_load<T>(dobase, dopitch, qcur.vox, lane, rdo);
-        rows_load<T>(obase, opitch, qcur.vox, lane, ro);
+        constexpr bool ONCE = DQ == KV_SINGLE;                // a group of one tile: nobody else reads these rows
+        rows_load<T, ONCE>(head_base<T>(tk, h), pitch_of<T>(tk), vox_j, lane, rk);
+        rows_load<T, ONCE>(head_base<T>(tv, h), pitch_of<T>(tv), vox_j, lane, rv);
+        rows_load<T, ONCE>(qbase, qpitch, qcur.vox, lane, rq);
+        rows_load<T, ONCE>(dobase, dopitch, qcur.vox, lane, rdo);
+        rows_load<T, ONCE>(obase, opitch, qcur.vox, lane, ro);
         rows_to_tile<T>(tile_q, lane, rk);
         rows_to_tile<T>(tile_do, lane, rv);
         __builtin_amdgcn_wave_barrier();
