@@ -381,7 +381,8 @@ def kernel_table(wl, reps=20, only=None):
             ("fused softmax bwd", lambda: ops.softmax_last_dim_backward(rows_f, p_val, g_s), 16 * A, 1),
             ("fused dQ=dS K", lambda: F._sq_to_tokens(tp, dt, False, g_s, qkv_c, 3 * D, D, dqkv, 3 * D, 0, hd, 0.17), 4 * A + 8 * E, 1),
             ("fused dK=dS^T Q", lambda: F._sq_to_tokens(tp, dt, True, g_s, qkv_c, 3 * D, 0, dqkv, 3 * D, D, hd, 0.17), 4 * A + 8 * E, 1),
-            ("fused bias grad", lambda: _lib.check(lib.sswin_fused_bias_grad(ptr(tp.plan), tp.g_cap, tp.G, ptr(tp.tokens), tp.N, H, b["n"], ptr(g_s), ptr(dbias), ptr(bg_ws), bg_bytes, stream)), 4 * A, 1),
+            ("fused bias table grad", lambda: _lib.check(lib.sswin_bias_table_grad(ptr(tp.plan), tp.g_cap, tp.G, ptr(tp.tokens), tp.N, H, b["n"], ptr(ti.code), ti.offset0, n_table, ptr(g_s), ptr(d_table), ptr(tg_ws), tg_bytes, stream)), 4 * A, 1),
+            ("fused bias grad [H,n,n]", lambda: _lib.check(lib.sswin_fused_bias_grad(ptr(tp.plan), tp.g_cap, tp.G, ptr(tp.tokens), tp.N, H, b["n"], ptr(g_s), ptr(dbias), ptr(bg_ws), bg_bytes, stream)), 4 * A, 0),
         ]
 
     # ---- the window-resident kernels (what the step runs for heads of 32 channels), in the workload's dtype ----

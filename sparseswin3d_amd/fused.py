@@ -119,17 +119,55 @@ def _sq_to_tokens(tp, dtype, a_kmajor, sq, b, b_stride, b_col0, o, o_stride, o_c
         _ptr(sq), _ptr(b), b_stride, b_col0, _ptr(o), o_stride, o_col0, C.c_float(scale), stream))
 
 
+def _bias32(bias, table_index, H, n, d):
+    """The fp32 [H, n, n] bias the kernels read: ``bias`` itself, or gathered from the [rows, H] table."""
+    if table_index is None:
+        return bias.detach().to(torch.float32).contiguous()
+    table32 = bias.detach().to(torch.float32).contiguous()
+    bias32 = torch.empty((H, n, n), dtype=torch.float32, device=d)
+    with torch.cuda.device(d):
+        _lib.check(_lib.load().sswin_bias_from_table(
+            _ptr(table32), table32.shape[0], H, _ptr(table_index.code), table_index.offset0, n, _ptr(bias32),
+            C.c_void_p(torch.cuda.current_stream(d).cuda_stream)))
+    return bias32
+
+
+def _bias_gradient(tp, H, d_s, bias_meta, table_index):
+    """Gradient of the [H, n, n] bias, or of the [rows, H] table when ``table_index`` is given, from dS
+    (one [c x c] block per group)."""
+    lib = _lib.load()
+    d = d_s.device
+    bias_dtype, bias_shape = bias_meta
+    stream = C.c_void_p(torch.cuda.current_stream(d).cuda_stream)
+    if table_index is None:
+        d_bias32 = torch.zeros(bias_shape, dtype=torch.float32, device=d)
+        nbytes = lib.sswin_fused_bias_grad_workspace_bytes(tp.G, H, tp.n)
+        ws = torch.empty(int(nbytes), dtype=torch.uint8, device=d)
+        _lib.check(lib.sswin_fused_bias_grad(_ptr(tp.plan), tp.g_cap, tp.G, _ptr(tp.tokens), tp.N, H, tp.n,
+                                             _ptr(d_s), _ptr(d_bias32), _ptr(ws), nbytes, stream))
+    else:
+        rows = bias_shape[0]
+        d_bias32 = torch.empty(bias_shape, dtype=torch.float32, device=d)
+        nbytes = lib.sswin_bias_table_grad_workspace_bytes(tp.G, H, rows)
+        ws = torch.empty(int(nbytes), dtype=torch.uint8, device=d)
+        _lib.check(lib.sswin_bias_table_grad(_ptr(tp.plan), tp.g_cap, tp.G, _ptr(tp.tokens), tp.N, H, tp.n,
+                                             _ptr(table_index.code), table_index.offset0, rows, _ptr(d_s),
+                                             _ptr(d_bias32), _ptr(ws), nbytes, stream))
+    return d_bias32.to(bias_dtype)
+
+
 class _FusedWindowAttention(Function):
     @staticmethod
-    def forward(ctx, qkv, bias, indices, mask, batch_size, n, scale, plan):
-        # qkv [N, 3, H, hd]; bias fp32 [H, n, n]; indices int32 [N, 2]; mask int8 [nW, n] or None
+    def forward(ctx, qkv, bias, indices, mask, batch_size, n, scale, plan, table_index):
+        # qkv [N, 3, H, hd]; bias fp32 [H, n, n], or with ``table_index`` the [rows, H] bias table; indices int32
+        # [N, 2]; mask int8 [nW, n] or None
         qkv = qkv.contiguous()
         N, _, H, hd = qkv.shape
         D = H * hd
         dtype = qkv.dtype
         tp = (plan or TokenPlan(indices, batch_size, n, H)).finish()
         d = qkv.device
-        bias32 = bias.detach().to(torch.float32).contiguous()
+        bias32 = _bias32(bias, table_index, H, n, d)
         if mask is not None:
             mask = mask.to(torch.int8).contiguous()
         with torch.cuda.device(d):
@@ -140,7 +178,7 @@ class _FusedWindowAttention(Function):
             out = torch.empty((N, D), dtype=dtype, device=d)
             _sq_to_tokens(tp, dtype, False, p, qkv, 3 * D, 2 * D, out, D, 0, hd, 1.0)
         ctx.save_for_backward(qkv, p, rows)
-        ctx.tp, ctx.scale, ctx.bias_meta = tp, scale, (bias.dtype, bias.shape)
+        ctx.tp, ctx.scale, ctx.bias_meta, ctx.table_index = tp, scale, (bias.dtype, bias.shape), table_index
         return out
 
     @staticmethod
@@ -164,17 +202,8 @@ class _FusedWindowAttention(Function):
             # dQ = scale * dS K ; dK = scale * dS^T Q
             _sq_to_tokens(tp, dtype, False, d_s, qkv, 3 * D, D, d_qkv, 3 * D, 0, hd, scale)
             _sq_to_tokens(tp, dtype, True, d_s, qkv, 3 * D, 0, d_qkv, 3 * D, D, hd, scale)
-            d_bias = None
-            if ctx.needs_input_grad[1]:
-                bias_dtype, bias_shape = ctx.bias_meta
-                d_bias32 = torch.zeros(bias_shape, dtype=torch.float32, device=d)
-                stream = C.c_void_p(torch.cuda.current_stream(d).cuda_stream)
-                nbytes = lib.sswin_fused_bias_grad_workspace_bytes(tp.G, H, tp.n)
-                ws = torch.empty(int(nbytes), dtype=torch.uint8, device=d)
-                _lib.check(lib.sswin_fused_bias_grad(_ptr(tp.plan), tp.g_cap, tp.G, _ptr(tp.tokens), tp.N, H, tp.n,
-                                                     _ptr(d_s), _ptr(d_bias32), _ptr(ws), nbytes, stream))
-                d_bias = d_bias32.to(bias_dtype)
-        return d_qkv, d_bias, None, None, None, None, None, None
+            d_bias = _bias_gradient(tp, H, d_s, ctx.bias_meta, ctx.table_index) if ctx.needs_input_grad[1] else None
+        return d_qkv, d_bias, None, None, None, None, None, None, None
 
 
 def _token_args(t, stride, col0):
@@ -197,15 +226,7 @@ class _ResidentWindowAttention(Function):
         tp = (plan or TokenPlan(indices, batch_size, n, H)).finish()
         if tp.oversize_groups:
             raise RuntimeError(f"window-resident attention: {tp.oversize_groups} groups hold more than 128 tokens")
-        if table_index is None:
-            bias32 = bias.detach().to(torch.float32).contiguous()
-        else:
-            table32 = bias.detach().to(torch.float32).contiguous()
-            bias32 = torch.empty((H, n, n), dtype=torch.float32, device=d)
-            with torch.cuda.device(d):
-                _lib.check(_lib.load().sswin_bias_from_table(
-                    _ptr(table32), table32.shape[0], H, _ptr(table_index.code), table_index.offset0, n, _ptr(bias32),
-                    C.c_void_p(torch.cuda.current_stream(d).cuda_stream)))
+        bias32 = _bias32(bias, table_index, H, n, d)
         if mask is not None:
             mask = mask.to(torch.int8).contiguous()
         lib = _lib.load()
@@ -247,25 +268,7 @@ class _ResidentWindowAttention(Function):
                     *_token_args(out, D, 0), *_token_args(grad_out, D, 0), _ptr(lse),
                     *_token_args(d_qkv, 3 * D, 0), *_token_args(d_qkv, 3 * D, D), *_token_args(d_qkv, 3 * D, 2 * D),
                     _ptr(d_s), 3, stream))
-            d_bias = None
-            if want_bias:
-                bias_dtype, bias_shape = ctx.bias_meta
-                ti = ctx.table_index
-                if ti is None:
-                    d_bias32 = torch.zeros(bias_shape, dtype=torch.float32, device=d)
-                    nbytes = lib.sswin_fused_bias_grad_workspace_bytes(tp.G, H, tp.n)
-                    ws = torch.empty(int(nbytes), dtype=torch.uint8, device=d)
-                    _lib.check(lib.sswin_fused_bias_grad(_ptr(tp.plan), tp.g_cap, tp.G, _ptr(tp.tokens), tp.N, H,
-                                                         tp.n, _ptr(d_s), _ptr(d_bias32), _ptr(ws), nbytes, stream))
-                else:
-                    rows = bias_shape[0]
-                    d_bias32 = torch.empty(bias_shape, dtype=torch.float32, device=d)
-                    nbytes = lib.sswin_bias_table_grad_workspace_bytes(tp.G, H, rows)
-                    ws = torch.empty(int(nbytes), dtype=torch.uint8, device=d)
-                    _lib.check(lib.sswin_bias_table_grad(_ptr(tp.plan), tp.g_cap, tp.G, _ptr(tp.tokens), tp.N, H, tp.n,
-                                                         _ptr(ti.code), ti.offset0, rows, _ptr(d_s), _ptr(d_bias32),
-                                                         _ptr(ws), nbytes, stream))
-                d_bias = d_bias32.to(bias_dtype)
+            d_bias = _bias_gradient(tp, H, d_s, ctx.bias_meta, ctx.table_index) if want_bias else None
         return d_qkv, d_bias, None, None, None, None, None, None, None
 
 
@@ -303,15 +306,12 @@ def fused_window_attention(qkv, bias, indices, mask, batch_size, n, scale, resid
     ``resident`` selects the window-resident kernels (default: whenever they apply, i.e. heads
     of 32 channels); otherwise the block products with the attention matrix in HBM are used.
     ``plan``: a :class:`TokenPlan` of ``indices`` made earlier (possibly still in flight).
-    ``table_index`` (resident path only): a :class:`BiasTableIndex`; ``bias`` is then the
-    [rows, H] bias table and its gradient is computed without the [H, n, n] detour."""
+    ``table_index``: a :class:`BiasTableIndex`; ``bias`` is then the [rows, H] bias table and its
+    gradient is computed without the [H, n, n] detour."""
     if resident is None:
         resident = supports_resident(qkv, n)
-    if resident:
-        return _ResidentWindowAttention.apply(qkv, bias, indices, mask, batch_size, n, scale, plan, table_index)
-    if table_index is not None:
-        raise ValueError("table_index needs the window-resident kernels")
-    return _FusedWindowAttention.apply(qkv, bias, indices, mask, batch_size, n, scale, plan)
+    fn = _ResidentWindowAttention if resident else _FusedWindowAttention
+    return fn.apply(qkv, bias, indices, mask, batch_size, n, scale, plan, table_index)
 
 
 def supports_resident(qkv: torch.Tensor, n: int) -> bool:

@@ -657,10 +657,10 @@ class WindowAttentionSparse(nn.Module):
         qkv = tall_linear(x.features, self.qkv).reshape(-1, 3, self.num_heads, c // self.num_heads)
         if plan is not None:
             resident = fused.supports_resident(qkv, n) if self.resident is None else self.resident
-            table_index = self._table_index(n) if resident else None
+            table_index = self._table_index(n)
             if table_index is not None:
                 out = fused.fused_window_attention(qkv, self.relative_position_bias_table, x.indices, mask, b, n,
-                                                   self.scale, True, plan, table_index)
+                                                   self.scale, resident, plan, table_index)
             else:
                 out = fused.fused_window_attention(qkv, self.relative_position_bias(n, torch.float32), x.indices,
                                                    mask, b, n, self.scale, resident, plan)
