@@ -64,8 +64,11 @@ struct GroupTable {
     const int32_t* head;       // [G] or null
 };
 
+#ifndef BP_WAVES
+#define BP_WAVES 5
+#endif
 template <typename T, int MODE, bool EMIT>
-__global__ __launch_bounds__(256) void block_product_mfma_kernel(const T* __restrict__ m1, const T* __restrict__ m2,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MODE >= 2 ? BP_WAVES : 4, MODE >= 2 ? BP_WAVES : 4))) void block_product_mfma_kernel(const T* __restrict__ m1, const T* __restrict__ m2,
                                                                  GroupTable gt, int64_t G, int C,
                                                                  const int32_t* __restrict__ tok_pos,
                                                                  T* __restrict__ out, int32_t* __restrict__ out_idx,

@@ -343,7 +343,7 @@ __device__ __forceinline__ void locate_task(const TaskSet& ts, int t, int& q, in
 //   EPI = false: plain product (dP = dO V^T)
 // ------------------------------------------------------------------------------------------
 template <typename T, bool EPI>
-__global__ __launch_bounds__(256) void fused_sq_kernel(FusedGroups gt, const int32_t* __restrict__ order,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void fused_sq_kernel(FusedGroups gt, const int32_t* __restrict__ order,
                                                        const int32_t* __restrict__ tok_pos, int H, int hd,
                                                        TokenTensor ta, TokenTensor tb, float scale_a,
                                                        const float* __restrict__ bias, int n,
@@ -453,7 +453,7 @@ __global__ __launch_bounds__(256) void fused_sq_kernel(FusedGroups gt, const int
 //   A_KMAJOR = true : A(i, k) = sq[k*c + i]   (dV = P^T dO, dK = dS^T Q)
 // ------------------------------------------------------------------------------------------
 template <typename T, bool A_KMAJOR>
-__global__ __launch_bounds__(256) void fused_tok_kernel(FusedGroups gt, const int32_t* __restrict__ order, int hd,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void fused_tok_kernel(FusedGroups gt, const int32_t* __restrict__ order, int hd,
                                                         const float* __restrict__ sq, TokenTensor tb,
                                                         TokenTensor to, float scale_out) {
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -467,9 +467,15 @@ __global__ __launch_bounds__(256) void fused_tok_kernel(FusedGroups gt, const in
     for (int t = wave; t < total; t += 4) {
         int q, c, bi, bj;
         locate_task(ts, t, q, c, bi, bj);
+        // a task belongs to the whole wavefront: its parameters go to scalar registers, and the block of the
+        // attention matrix is addressed by a scalar base plus 32-bit lane offsets (c <= 32767, so c * c * 4 fits)
+        q = __builtin_amdgcn_readfirstlane(q);
+        c = __builtin_amdgcn_readfirstlane(c);
+        bi = __builtin_amdgcn_readfirstlane(bi);
+        bj = __builtin_amdgcn_readfirstlane(bj);
         const int64_t g = g0 + q;
-        const int Tk = gt.T[g], h = gt.head[g];
-        const float* S = sq + gt.sq[g];
+        const int Tk = __builtin_amdgcn_readfirstlane(gt.T[g]), h = __builtin_amdgcn_readfirstlane(gt.head[g]);
+        const float* S = sq + __builtin_amdgcn_readfirstlane(gt.sq[g]);
         const int i_a = bi * 32 + l32, j_b = bj * 32 + l32;
         const bool a_in = i_a < c, b_in = j_b < hd;
         const int i_c = a_in ? i_a : c - 1, j_c = b_in ? j_b : hd - 1;     // clamped: loads need no predicate
@@ -492,10 +498,11 @@ __global__ __launch_bounds__(256) void fused_tok_kernel(FusedGroups gt, const in
             }
             if (kc + 32 <= c) {                                    // full chunk (uniform)
                 if (!A_KMAJOR) {
-                    load_run16_full<float>(S + (int64_t)i_c * c + kb, a);
+                    load_run16_full<float>(S + (uint32_t)(i_c * c + kb), a);
                 } else {
+                    const uint32_t o0 = (uint32_t)(kb * c + i_c);
 #pragma unroll
-                    for (int s = 0; s < 16; ++s) a[s] = S[(int64_t)(kb + s) * c + i_c];
+                    for (int s = 0; s < 16; ++s) a[s] = S[o0 + (uint32_t)(s * c)];
                 }
 #pragma unroll
                 for (int s = 0; s < 16; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], acc, 0, 0, 0);
@@ -504,7 +511,7 @@ __global__ __launch_bounds__(256) void fused_tok_kernel(FusedGroups gt, const in
 #pragma unroll
                 for (int s = 0; s < 16; ++s) {
                     const int k = kb + s < c ? kb + s : c - 1;
-                    const float v = A_KMAJOR ? S[(int64_t)k * c + i_c] : S[(int64_t)i_c * c + k];
+                    const float v = S[A_KMAJOR ? (uint32_t)(k * c + i_c) : (uint32_t)(i_c * c + k)];
                     a[s] = s < left ? v : 0.f;                     // zero A kills the clamped B rows
                 }
                 const int steps = c - kc;
