@@ -100,15 +100,15 @@ def build_workload(device, name="cfg2"):
 
 
 def run_step(wl):
-    from sparseswin3d_amd.window_attention import SparseVoxelTensor, replace_feature
+    from sparseswin3d_amd.window_attention import SparseVoxelTensor, prefetch_plans, replace_feature
     for blk in wl["blocks"]:                                  # as a training step does: fresh gradients
         blk["attn"].zero_grad(set_to_none=True)
     x = wl["feats"].detach().requires_grad_(True)
     # as a stage does: the token plans of all its blocks are enqueued before the first block runs (they need the
-    # window indices only), so the totals of the later ones are on the host when their block asks
+    # window indices only) and share their launches, so the totals of the later ones are on the host when their
+    # block asks
     views = [SparseVoxelTensor(x, b["idx"], (b["n"],), b["slots"]) for b in wl["blocks"]]
-    for b, t in zip(wl["blocks"], views):
-        b["attn"].prefetch_plan(t)
+    prefetch_plans([(b["attn"], t) for b, t in zip(wl["blocks"], views)])
     h = x
     for b, t in zip(wl["blocks"], views):
         h = b["attn"](replace_feature(t, h), b["mask"]).features
@@ -432,6 +432,10 @@ def kernel_table(wl, reps=20, only=None):
     # flops of a launch: 2 c^2 hd per product and group = 2 A hd per product (two in the forward, five in the backward)
     r_entries = [
         ("resident token_plan", lambda: F.TokenPlan(b["idx"], b["slots"], b["n"], H), 28 * N + 36 * tp.G, 1),
+        # what a stage does: the plans of its two partitions from shared launches, nobody waiting for the totals;
+        # the row is the GPU time of both plans (no host round trip inside), bytes of both
+        ("token plans of both blocks, one batch, deferred", lambda: F.TokenPlan.batch(
+            [(bb["idx"], bb["slots"], bb["n"], H) for bb in wl["blocks"][:2]]), 2 * (28 * N + 36 * tp.G), 0),
         ("resident forward", r_fwd, 16 * Er + 4 * H * N, 1, 4 * A * hd),
         ("resident backward (dQ,dK,dV,dS)", r_bwd(3), 32 * Er + 4 * A + 4 * H * N, 1, 10 * A * hd),
         ("resident backward dQ, groups > 32 tokens", r_bwd(1, only_large), (24 * es // 4 * hd + 4) * rowsL, 0),

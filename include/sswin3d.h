@@ -278,6 +278,27 @@ int sswin_token_plan(const int32_t* indices, int64_t N, int B, int n, int H, int
                      size_t ws_bytes, int synchronize, void* stream);
 int sswin_token_plan_totals(int64_t* totals, int H, int64_t g_cap);
 
+/* Up to four token plans in one set of launches: the regular and the shifted block of a stage
+ * (sparse_swin/swin3d_base.py:889-905 runs them one after the other, each with its own
+ * coalesce / sort chain, ops.cu:781-784, 836-841) partition the same voxels differently, and one plan
+ * is a few microseconds of work per launch.  Every descriptor holds the arguments of one
+ * sswin_token_plan call with synchronize == 0 and gives the same results; plans with N == 0 are
+ * skipped (totals all zero).  After waiting for `stream`, decode each totals_out with
+ * sswin_token_plan_totals.  Rejects count > 4. */
+typedef struct sswin_token_plan_desc {
+    const int32_t* indices;
+    int64_t N;
+    int32_t B, n, H, reserved;
+    int32_t* tokens;
+    int32_t* plan;
+    int64_t g_cap;
+    int32_t* tasks;
+    int64_t* totals_out;
+    void* ws;
+    size_t ws_bytes;
+} sswin_token_plan_desc;
+int sswin_token_plan_batch(const sswin_token_plan_desc* descs, int count, void* stream);
+
 /* Token tensors are dense [N, stride] arrays of `dtype`; element (voxel v, head h, channel ch) is
  * base[v*stride + col0 + h*hd + ch].  "sq" arrays are fp32 arrays of all [c x c] blocks.
  *

@@ -13,6 +13,13 @@ LIB_PATH = os.path.join(_HERE, "libsswin3d.so")
 
 _vp, _i64, _i32, _sz = C.c_void_p, C.c_int64, C.c_int, C.c_size_t
 
+class TokenPlanDesc(C.Structure):
+    """``sswin_token_plan_desc`` of include/sswin3d.h: the arguments of one deferred sswin_token_plan call."""
+    _fields_ = [("indices", _vp), ("N", _i64), ("B", C.c_int32), ("n", C.c_int32), ("H", C.c_int32),
+                ("reserved", C.c_int32), ("tokens", _vp), ("plan", _vp), ("g_cap", _i64), ("tasks", _vp),
+                ("totals_out", _vp), ("ws", _vp), ("ws_bytes", _sz)]
+
+
 # name -> (restype, argtypes); mirrors include/sswin3d.h one to one
 SIGNATURES = {
     "sswin_calibration_copy": (_i32, [_vp, _vp, _i64, _vp]),
@@ -50,6 +57,7 @@ SIGNATURES = {
     "sswin_token_plan_workspace_bytes": (_sz, [_i64, _i32, _i32]),
     "sswin_token_plan": (_i32, [_vp, _i64, _i32, _i32, _i32, _vp, _vp, _i64, _vp, _vp, _vp, _sz, _i32, _vp]),
     "sswin_token_plan_totals": (_i32, [_vp, _i32, _i64]),
+    "sswin_token_plan_batch": (_i32, [_vp, _i32, _vp]),
     "sswin_fused_tokens_to_sq": (_i32, [_i32, _i32, _vp, _i64, _i64, _vp, _i64, _i32, _i32, _vp, _i64, _i32,
                                         _vp, _i64, _i32, C.c_float, _vp, _i32, _vp, _i32, _vp, _vp, _vp]),
     "sswin_fused_sq_to_tokens": (_i32, [_i32, _i32, _vp, _i64, _i64, _vp, _i64, _i32, _vp, _vp, _i64, _i32,
@@ -80,7 +88,7 @@ SIGNATURES = {
                                                _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i32, _vp]),
 }
 
-ABI_VERSION = 22
+ABI_VERSION = 23
 _lib = None
 
 

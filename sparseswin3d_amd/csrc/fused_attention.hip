@@ -267,22 +267,33 @@ __device__ __forceinline__ void tp_phase_rank(const TokenPlanArgs& a, int64_t gt
 }
 
 // ---- the five launches ----
-__global__ __launch_bounds__(256) void tp_clear_kernel(TokenPlanArgs a) {
-    tp_phase_clear(a, (int64_t)blockIdx.x * 256 + threadIdx.x, (int64_t)gridDim.x * 256);
+// Each launch works on up to TP_MAX_BATCH independent plans at once (blockIdx.y picks the plan): the phases of
+// one plan are a few microseconds each and mostly launch boundary, so the plans of the blocks of a stage share
+// their launches.  The grid's x extent is the largest any plan of the batch needs; the per-voxel and per-word
+// phases walk their plan with a grid stride, the per-block phases leave when the plan has fewer blocks.
+constexpr int TP_MAX_BATCH = 4;
+struct TokenPlanBatch {
+    TokenPlanArgs p[TP_MAX_BATCH];
+};
+
+__global__ __launch_bounds__(256) void tp_clear_kernel(TokenPlanBatch b) {
+    tp_phase_clear(b.p[blockIdx.y], (int64_t)blockIdx.x * 256 + threadIdx.x, (int64_t)gridDim.x * 256);
 }
-__global__ __launch_bounds__(256) void tp_set_bits_kernel(TokenPlanArgs a) {
-    tp_phase_set_bits(a, (int64_t)blockIdx.x * 256 + threadIdx.x, (int64_t)gridDim.x * 256);
+__global__ __launch_bounds__(256) void tp_set_bits_kernel(TokenPlanBatch b) {
+    tp_phase_set_bits(b.p[blockIdx.y], (int64_t)blockIdx.x * 256 + threadIdx.x, (int64_t)gridDim.x * 256);
 }
-__global__ __launch_bounds__(TP_BLOCK) void tp_block_sums_kernel(TokenPlanArgs a) {
+__global__ __launch_bounds__(TP_BLOCK) void tp_block_sums_kernel(TokenPlanBatch b) {
     __shared__ TpShared sh;
-    tp_phase_block_sums(a, blockIdx.x, sh);
+    const TokenPlanArgs& a = b.p[blockIdx.y];
+    if ((int)blockIdx.x < a.blocks) tp_phase_block_sums(a, blockIdx.x, sh);
 }
-__global__ __launch_bounds__(TP_BLOCK) void tp_windows_kernel(TokenPlanArgs a) {
+__global__ __launch_bounds__(TP_BLOCK) void tp_windows_kernel(TokenPlanBatch b) {
     __shared__ TpShared sh;
-    tp_phase_windows(a, blockIdx.x, sh);
+    const TokenPlanArgs& a = b.p[blockIdx.y];
+    if ((int)blockIdx.x < a.blocks) tp_phase_windows(a, blockIdx.x, sh);
 }
-__global__ __launch_bounds__(256) void tp_rank_kernel(TokenPlanArgs a) {
-    tp_phase_rank(a, (int64_t)blockIdx.x * 256 + threadIdx.x, (int64_t)gridDim.x * 256);
+__global__ __launch_bounds__(256) void tp_rank_kernel(TokenPlanBatch b) {
+    tp_phase_rank(b.p[blockIdx.y], (int64_t)blockIdx.x * 256 + threadIdx.x, (int64_t)gridDim.x * 256);
 }
 
 // ------------------------------------------------------------------------------------------
@@ -917,20 +928,16 @@ size_t sswin_token_plan_workspace_bytes(int64_t N, int B, int n) {
            align_up(blocks * 4, 256) + 1024;
 }
 
-int sswin_token_plan(const int32_t* indices, int64_t N, int B, int n, int H, int32_t* tokens,
-                     int32_t* plan, int64_t g_cap, int32_t* tasks, int64_t* totals_out, void* ws,
-                     size_t ws_bytes, int synchronize, void* stream) {
-    SSWIN_CHECK(N >= 0 && B > 0 && n > 0 && H > 0 && H < 256, "token_plan: bad sizes");
-    SSWIN_CHECK(totals_out, "token_plan: totals_out is null");
-    for (int i = 0; i < 9; ++i) totals_out[i] = 0;
-    if (N == 0) return 0;
-    SSWIN_CHECK(indices && tokens && plan && ws, "token_plan: null pointer");
+// Checks one plan's arguments and carves its workspace; `a` is ready to launch afterwards.
+static int token_plan_args(const int32_t* indices, int64_t N, int B, int n, int H, int32_t* tokens, int32_t* plan,
+                           int64_t g_cap, int32_t* tasks, int64_t* totals_out, void* ws, size_t ws_bytes,
+                           TokenPlanArgs& a) {
+    SSWIN_CHECK(N > 0 && B > 0 && n > 0 && H > 0 && H < 256, "token_plan: bad sizes");
+    SSWIN_CHECK(indices && tokens && plan && ws && totals_out, "token_plan: null pointer");
     SSWIN_CHECK(N < (int64_t)INT32_MAX, "token_plan: too many voxels");
     SSWIN_CHECK(g_cap > 0, "token_plan: g_cap must be positive");
     SSWIN_CHECK(ws_bytes >= sswin_token_plan_workspace_bytes(N, B, n), "token_plan: workspace too small");
-    hipStream_t s = static_cast<hipStream_t>(stream);
     Carver cv(ws, ws_bytes);
-    TokenPlanArgs a;
     a.ind = indices;
     a.N = N;
     a.B = B;
@@ -950,23 +957,74 @@ int sswin_token_plan(const int32_t* indices, int64_t N, int B, int n, int H, int
     a.g_cap = g_cap;
     a.tasks = reinterpret_cast<int4*>(tasks);
     a.tokens = tokens;
-    totals_out[8] = N;                     // read back by sswin_token_plan_totals (the copy below fills [0..7])
+    return 0;
+}
 
-    {
-        const unsigned clear_blocks = (unsigned)std::min<size_t>((words + 255) / 256, 2048);
-        hipLaunchKernelGGL(tp_clear_kernel, dim3(clear_blocks), dim3(256), 0, s, a);
-        const unsigned nb = (unsigned)std::min<int64_t>((N + 255) / 256, 1 << 20);
-        hipLaunchKernelGGL(tp_set_bits_kernel, dim3(nb), dim3(256), 0, s, a);
-        hipLaunchKernelGGL(tp_block_sums_kernel, dim3((unsigned)blocks), dim3(TP_BLOCK), 0, s, a);
-        hipLaunchKernelGGL(tp_windows_kernel, dim3((unsigned)blocks), dim3(TP_BLOCK), 0, s, a);
-        hipLaunchKernelGGL(tp_rank_kernel, dim3(nb), dim3(256), 0, s, a);
+// The five launches for `count` plans (1..TP_MAX_BATCH) and the copies of their raw totals to the host.
+static int token_plan_launch(const TokenPlanArgs* args, int64_t* const* totals_out, int count, hipStream_t s) {
+    TokenPlanBatch b;
+    size_t words = 0;
+    int64_t voxels = 0;
+    int blocks = 0;
+    for (int k = 0; k < TP_MAX_BATCH; ++k) {
+        b.p[k] = args[k < count ? k : 0];  // unused slots repeat the first plan; no block ever reads them
+        if (k >= count) continue;
+        words = std::max(words, (size_t)args[k].B * args[k].W);
+        voxels = std::max(voxels, args[k].N);
+        blocks = std::max(blocks, args[k].blocks);
     }
+    const unsigned y = (unsigned)count;
+    const unsigned clear_blocks = (unsigned)std::min<size_t>((words + 255) / 256, 2048);
+    const unsigned nb = (unsigned)std::min<int64_t>((voxels + 255) / 256, 1 << 20);
+    hipLaunchKernelGGL(tp_clear_kernel, dim3(clear_blocks, y), dim3(256), 0, s, b);
+    hipLaunchKernelGGL(tp_set_bits_kernel, dim3(nb, y), dim3(256), 0, s, b);
+    hipLaunchKernelGGL(tp_block_sums_kernel, dim3((unsigned)blocks, y), dim3(TP_BLOCK), 0, s, b);
+    hipLaunchKernelGGL(tp_windows_kernel, dim3((unsigned)blocks, y), dim3(TP_BLOCK), 0, s, b);
+    hipLaunchKernelGGL(tp_rank_kernel, dim3(nb, y), dim3(256), 0, s, b);
     if (launch_ok("token plan")) return 1;
-    // raw totals: the caller decodes them with sswin_token_plan_totals once the copy has landed
-    SSWIN_HIP(hipMemcpyAsync(totals_out, a.totals, 8 * sizeof(int64_t), hipMemcpyDeviceToHost, s));
+    // raw totals: the caller decodes them with sswin_token_plan_totals once the copies have landed
+    for (int k = 0; k < count; ++k)
+        SSWIN_HIP(hipMemcpyAsync(totals_out[k], args[k].totals, 8 * sizeof(int64_t), hipMemcpyDeviceToHost, s));
+    return 0;
+}
+
+int sswin_token_plan(const int32_t* indices, int64_t N, int B, int n, int H, int32_t* tokens,
+                     int32_t* plan, int64_t g_cap, int32_t* tasks, int64_t* totals_out, void* ws,
+                     size_t ws_bytes, int synchronize, void* stream) {
+    SSWIN_CHECK(N >= 0 && B > 0 && n > 0 && H > 0 && H < 256, "token_plan: bad sizes");
+    SSWIN_CHECK(totals_out, "token_plan: totals_out is null");
+    for (int i = 0; i < 9; ++i) totals_out[i] = 0;
+    if (N == 0) return 0;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    TokenPlanArgs a;
+    if (token_plan_args(indices, N, B, n, H, tokens, plan, g_cap, tasks, totals_out, ws, ws_bytes, a)) return 1;
+    totals_out[8] = N;                     // read back by sswin_token_plan_totals (the copy fills [0..7])
+    if (token_plan_launch(&a, &totals_out, 1, s)) return 1;
     if (!synchronize) return 0;
     SSWIN_HIP(hipStreamSynchronize(s));
     return sswin_token_plan_totals(totals_out, H, g_cap);
+}
+
+int sswin_token_plan_batch(const sswin_token_plan_desc* descs, int count, void* stream) {
+    SSWIN_CHECK(count >= 0 && count <= TP_MAX_BATCH, "token_plan_batch: between 0 and %d plans per call", TP_MAX_BATCH);
+    SSWIN_CHECK(count == 0 || descs, "token_plan_batch: descs is null");
+    TokenPlanArgs args[TP_MAX_BATCH];
+    int64_t* totals[TP_MAX_BATCH];
+    int live = 0;
+    for (int k = 0; k < count; ++k) {
+        const sswin_token_plan_desc& d = descs[k];
+        SSWIN_CHECK(d.N >= 0 && d.B > 0 && d.n > 0 && d.H > 0 && d.H < 256, "token_plan_batch: bad sizes in plan %d", k);
+        SSWIN_CHECK(d.totals_out, "token_plan_batch: totals_out of plan %d is null", k);
+        for (int i = 0; i < 9; ++i) d.totals_out[i] = 0;
+        if (d.N == 0) continue;            // an empty plan: all totals zero, nothing to launch
+        if (token_plan_args(d.indices, d.N, d.B, d.n, d.H, d.tokens, d.plan, d.g_cap, d.tasks, d.totals_out, d.ws,
+                            d.ws_bytes, args[live]))
+            return 1;
+        d.totals_out[8] = d.N;
+        totals[live++] = d.totals_out;
+    }
+    if (live == 0) return 0;
+    return token_plan_launch(args, totals, live, static_cast<hipStream_t>(stream));
 }
 
 int sswin_token_plan_totals(int64_t* totals, int H, int64_t g_cap) {

@@ -55,8 +55,25 @@ class TokenPlan:
     :meth:`finish` waits for the totals when they are needed.  :meth:`finish` raises if an index
     lies outside ``[0, batch_size) x [0, n)`` or a (window, pos) pair occurs twice."""
 
+    MAX_BATCH = 4            # plans per sswin_token_plan_batch call
+
     def __init__(self, indices: torch.Tensor, batch_size: int, n: int, num_heads: int, defer: bool = False,
                  tasks: bool = True):
+        self._allocate(indices, batch_size, n, num_heads, tasks)
+        lib = _lib.load()
+        d = self.device
+        with torch.cuda.device(d):
+            stream = C.c_void_p(torch.cuda.current_stream(d).cuda_stream)
+            _lib.check(lib.sswin_token_plan(_ptr(self._indices), self.N, self.B, self.n, self.H, _ptr(self.tokens),
+                                            _ptr(self.plan), self.g_cap, _ptr(self.tasks),
+                                            C.c_void_p(self._totals.data_ptr()), _ptr(self._ws), self._ws.numel(), 0,
+                                            stream))
+            self._event = torch.cuda.Event()
+            self._event.record(torch.cuda.current_stream(d))
+        if not defer:
+            self.finish()
+
+    def _allocate(self, indices, batch_size, n, num_heads, tasks):
         lib = _lib.load()
         if indices.device.type != "cuda":
             raise RuntimeError("TokenPlan runs on the GPU only; there is no CPU fallback")
@@ -77,14 +94,39 @@ class TokenPlan:
         with torch.cuda.device(d):
             nbytes = lib.sswin_token_plan_workspace_bytes(N, self.B, self.n)
             self._ws = torch.empty(int(nbytes), dtype=torch.uint8, device=d)
-            stream = C.c_void_p(torch.cuda.current_stream(d).cuda_stream)
-            _lib.check(lib.sswin_token_plan(_ptr(indices), N, self.B, self.n, self.H, _ptr(self.tokens),
-                                            _ptr(self.plan), self.g_cap, _ptr(self.tasks),
-                                            C.c_void_p(self._totals.data_ptr()), _ptr(self._ws), nbytes, 0, stream))
-            self._event = torch.cuda.Event()
-            self._event.record(torch.cuda.current_stream(d))
-        if not defer:
-            self.finish()
+
+    @classmethod
+    def batch(cls, specs):
+        """Deferred plans for several index sets on one device, built by shared launches (the regular and the
+        shifted block of a stage).  ``specs``: tuples ``(indices, batch_size, n, num_heads)`` or
+        ``(..., tasks)``; returns the plans in the same order, each to be completed with :meth:`finish`."""
+        plans = []
+        for spec in specs:
+            p = cls.__new__(cls)
+            p._allocate(*spec[:4], spec[4] if len(spec) > 4 else True)
+            plans.append(p)
+        if not plans:
+            return plans
+        d = plans[0].device
+        if any(p.device != d for p in plans):
+            raise RuntimeError("TokenPlan.batch: all index sets must live on one device")
+        lib = _lib.load()
+        with torch.cuda.device(d):
+            stream = torch.cuda.current_stream(d)
+            for k in range(0, len(plans), cls.MAX_BATCH):
+                chunk = plans[k:k + cls.MAX_BATCH]
+                descs = (_lib.TokenPlanDesc * len(chunk))()
+                for desc, p in zip(descs, chunk):
+                    desc.indices, desc.N, desc.B, desc.n, desc.H = p._indices.data_ptr(), p.N, p.B, p.n, p.H
+                    desc.tokens, desc.plan, desc.g_cap = p.tokens.data_ptr(), p.plan.data_ptr(), p.g_cap
+                    desc.tasks = p.tasks.data_ptr() if p.tasks is not None else None
+                    desc.totals_out, desc.ws, desc.ws_bytes = p._totals.data_ptr(), p._ws.data_ptr(), p._ws.numel()
+                _lib.check(lib.sswin_token_plan_batch(descs, len(chunk), C.c_void_p(stream.cuda_stream)))
+            event = torch.cuda.Event()
+            event.record(stream)
+        for p in plans:
+            p._event = event
+        return plans
 
     def finish(self):
         """Wait for the totals (once) and decode them."""

@@ -19,7 +19,7 @@ from torch.autograd import Function
 from torch.autograd.function import once_differentiable
 
 from . import _lib
-from .window_attention import WindowAttentionSparse, replace_feature, tall_linear
+from .window_attention import WindowAttentionSparse, prefetch_plans, replace_feature, tall_linear
 
 _DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 
@@ -324,6 +324,12 @@ class SwinTransformerBlock(nn.Module):
         if getattr(x, "window_cache", None) is not None:
             self.attn.prefetch_plan(self.window_view(x)[0])
 
+    @staticmethod
+    def prefetch_all(blocks, x):
+        """The same for all blocks of a stage at once: their token plans share one set of launches."""
+        if getattr(x, "window_cache", None) is not None:
+            prefetch_plans([(blk.attn, blk.window_view(x)[0]) for blk in blocks])
+
     def forward_part1(self, x, mask_matrix):
         x = replace_feature(x, self.norm1(x.features))
         view, shifted = self.window_view(x)
@@ -376,8 +382,7 @@ class BasicLayer(nn.Module):
         x.window_cache = {}                      # (window, shift) -> window indices and token plans of this stage
         # the plans need the voxel indices only: all of them are enqueued now, so that only the first block waits
         # for totals from the GPU
-        for blk in self.blocks:
-            blk.prefetch(x)
+        SwinTransformerBlock.prefetch_all(self.blocks, x)
         for blk in self.blocks:
             x = blk(x, attn_mask)
         x.window_cache = None

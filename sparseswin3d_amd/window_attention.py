@@ -621,22 +621,10 @@ class WindowAttentionSparse(nn.Module):
 
     def prefetch_plan(self, x):
         """Enqueue the token plan of ``x``'s window indices now and keep it in ``x.plan_cache`` (created if
-        missing), so that its totals have reached the host by the time :meth:`forward` asks for them.  A stage
-        calls this for all its blocks before the first one runs.  Returns the plan, or None when this input
-        does not take the fused path."""
-        if not self.fused:
-            return None
-        from . import fused
-        n = x.spatial_shape[0]
-        if not fused.supports(x.features, n):
-            return None
-        cache = getattr(x, "plan_cache", None)
-        if cache is None:
-            cache = x.plan_cache = {}
-        plan = cache.get(self.num_heads)
-        if plan is None:
-            plan = cache[self.num_heads] = fused.TokenPlan(x.indices, x.batch_size, n, self.num_heads, defer=True)
-        return plan
+        missing), so that its totals have reached the host by the time :meth:`forward` asks for them.
+        Returns the plan, or None when this input does not take the fused path.  :func:`prefetch_plans` does
+        the same for several blocks with shared launches."""
+        return prefetch_plans([(self, x)])[0]
 
     def forward(self, x, mask):
         n = x.spatial_shape[0]
@@ -687,3 +675,36 @@ class WindowAttentionSparse(nn.Module):
             unsort = ops.return_inverse(ops.flatten_indices(x.indices.T.contiguous(), [b, n]), b * n)[0]
             x = replace_feature(x, out.values.reshape(x.features.shape).index_select(0, unsort))
         return replace_feature(x, self.proj_drop(tall_linear(x.features, self.proj)))
+
+
+def prefetch_plans(pairs):
+    """Token plans for several ``(WindowAttentionSparse, window view)`` pairs, enqueued now by shared launches and
+    kept in each view's ``plan_cache``: a stage calls this for all its blocks before the first one runs, so the
+    plans' totals have reached the host by the time the blocks ask for them, and the regular and the shifted
+    partition cost one set of launches instead of two.  Returns one plan per pair (None where the module or the
+    input does not take the fused path); pairs that share a view and a head count share a plan."""
+    from . import fused
+    out, missing = [None] * len(pairs), {}
+    for k, (attn, x) in enumerate(pairs):
+        n = x.spatial_shape[0]
+        if not attn.fused or not fused.supports(x.features, n):
+            continue
+        cache = getattr(x, "plan_cache", None)
+        if cache is None:
+            cache = x.plan_cache = {}
+        plan = cache.get(attn.num_heads)
+        if plan is not None:
+            out[k] = plan
+        else:
+            missing.setdefault((id(cache), attn.num_heads), (cache, x, n, attn.num_heads, []))[4].append(k)
+    todo = list(missing.values())
+    if len(todo) == 1:
+        cache, x, n, heads, ks = todo[0]
+        plans = [fused.TokenPlan(x.indices, x.batch_size, n, heads, defer=True)]
+    else:
+        plans = fused.TokenPlan.batch([(x.indices, x.batch_size, n, heads) for _, x, n, heads, _ in todo])
+    for (cache, _, _, heads, ks), plan in zip(todo, plans):
+        cache[heads] = plan
+        for k in ks:
+            out[k] = plan
+    return out

@@ -49,6 +49,49 @@ def test_token_plan_closed_forms(case):
     np.testing.assert_array_equal(tp.plan.view(5, -1)[:, :tp.G].cpu().numpy(), plan)
 
 
+def test_token_plans_in_one_batch_equal_single_plans():
+    """Several plans built by shared launches (different voxel counts, window counts, window sizes, head counts,
+    one of them empty, one without task descriptors) hold the same bits as plans built one by one; a bad index in
+    one plan of a batch is reported for that plan only."""
+    from sparseswin3d_amd import _lib
+    from sparseswin3d_amd.fused import TokenPlan
+    rng = np.random.default_rng(11)
+    specs = [(random_window_indices(rng, 50, 125, 1500), 50, 125, 3, True),
+             (ragged_window_indices(rng, [1, 0, 125, 2, 0, 0, 33, 64, 5, 17, 1, 1, 100], 125), 13, 125, 6, True),
+             (random_window_indices(rng, 20000, 125, 120000), 20000, 125, 3, True),
+             (np.zeros((0, 2), np.int32), 7, 27, 2, True),
+             (random_window_indices(rng, 3000, 8, 9000), 3000, 8, 1, False),
+             (random_window_indices(rng, 700, 64, 20000), 700, 64, 4, True)]
+    dev = [(torch.from_numpy(ind).cuda(), B, n, H, tasks) for ind, B, n, H, tasks in specs]
+    plans = TokenPlan.batch(dev)                         # six plans: two library calls
+    assert len(plans) == len(specs)
+    for spec, tp in zip(dev, plans):
+        tp.finish()
+        one = TokenPlan(*spec[:4], tasks=spec[4])
+        assert (tp.G, tp.windows, tp.A, tp.c_max, list(tp.bucket_counts)) == \
+               (one.G, one.windows, one.A, one.c_max, list(one.bucket_counts))
+        assert torch.equal(tp.tokens, one.tokens)
+        assert torch.equal(tp.plan.view(5, -1)[:, :tp.G], one.plan.view(5, -1)[:, :one.G])
+        if spec[4] and tp.G:
+            # descriptors of a bucket, as sets: their order inside a bucket is the same here, but not promised
+            a, b = tp.tasks.view(4, tp.g_cap, 4), one.tasks.view(4, one.g_cap, 4)
+            for k in range(4):
+                m = int(tp.bucket_counts[k])
+                assert torch.equal(a[k, :m], b[k, :m])
+    # errors stay with their plan
+    good = specs[0][0]
+    bad = np.concatenate([good[:400], np.array([[50, 3]], np.int32), good[400:]])
+    p_bad, p_good = TokenPlan.batch([(torch.from_numpy(bad).cuda(), 50, 125, 3), dev[1][:4]])
+    with pytest.raises(RuntimeError, match="outside"):
+        p_bad.finish()
+    assert p_good.finish().G == plans[1].G
+    # more than four descriptors in one library call are refused
+    descs = (_lib.TokenPlanDesc * 5)()
+    assert _lib.load().sswin_token_plan_batch(descs, 5, None) != 0
+    assert b"between 0 and 4" in _lib.load().sswin_last_error()
+    assert _lib.load().sswin_token_plan_batch(None, 0, None) == 0
+
+
 def test_token_plan_rejects_bad_indices():
     """Indices outside [0,B) x [0,n) and repeated (window, pos) pairs are skipped on the device (every kernel
     exits normally, nothing is written through them) and reported when the totals are decoded."""

@@ -106,9 +106,9 @@ def test_stage_with_downsample_and_shared_plans(monkeypatch):
     real = fused.TokenPlan
 
     class Counting(real):
-        def __init__(self, *a, **k):
-            made.append(k.get("tasks", True))
-            super().__init__(*a, **k)
+        def _allocate(self, indices, batch_size, n, num_heads, tasks):
+            made.append(tasks)
+            super()._allocate(indices, batch_size, n, num_heads, tasks)
 
     monkeypatch.setattr(fused, "TokenPlan", Counting)
     torch.manual_seed(3)
