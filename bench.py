@@ -138,7 +138,7 @@ def run_encoder(wl):
     """One forward pass of the four stages: per stage the window indices and the shift mask from the voxel grid
     kernels, the attention, then the stride-2 merge.  Returns the voxel count of every stage."""
     from sparseswin3d_amd import layers
-    from sparseswin3d_amd.window_attention import SparseVoxelTensor
+    from sparseswin3d_amd.window_attention import SparseVoxelTensor, prefetch_plans
     ws, sh = (5, 5, 5), (2, 2, 2)
     coords, shape, feats = wl["coords4"], wl["spatial_shape"], wl["feats"]
     counts = []
@@ -149,11 +149,15 @@ def run_encoder(wl):
             idx = layers.sparse_window_indices(coords, wl["batch_size"], dims, ws, sh)
             mask = layers.compute_mask(list(dims), list(ws), list(sh), coords.device)
             slots = wl["batch_size"] * (dims[0] // 5) * (dims[1] // 5) * (dims[2] // 5)
-            out = attn(SparseVoxelTensor(feats, idx, (125,), slots), mask).features
-            if k == len(wl["stages"]) - 1:
+            view = SparseVoxelTensor(feats, idx, (125,), slots)
+            last = k == len(wl["stages"]) - 1
+            # as BasicLayer does: the plan of the attention and the plan of the merge behind it share their launches
+            x = SparseVoxelTensor(feats, coords, shape, wl["batch_size"])
+            merge_plan = prefetch_plans([(attn, view)], [] if last else [layers.downsample_plan_request(x, 2)])[1:]
+            out = attn(view, mask).features
+            if last:
                 break
-            x = SparseVoxelTensor(out, coords, shape, wl["batch_size"])
-            plan, coords, shape = layers.downsample_plan(x, 2)
+            plan, coords, shape = layers.downsample_plan(x, 2, merge_plan[0])
             pooled = layers._PoolWindows.apply(out, plan, True)
             feats = torch.cat([pooled, pooled], 1)
     return counts

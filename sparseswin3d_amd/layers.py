@@ -181,16 +181,30 @@ class _PoolWindows(Function):
         return g_in, None, None
 
 
-def downsample_plan(x, factor: int = 2):
+def downsample_plan_request(x, factor: int = 2):
+    """What the token plan of the ``floor(coord / factor)`` merge is built from: the arguments
+    ``(indices, window slots, positions per window, heads = 1, tasks = False)`` of ``TokenPlan`` /
+    ``TokenPlan.batch``.  It depends on the voxel coordinates only, so a stage can enqueue it together with
+    the plans of its attention blocks and hand the plan to :func:`downsample_plan` later."""
+    f = int(factor)
+    dims = [-(-int(e) // f) * f for e in x.spatial_shape]
+    idx = sparse_window_indices(x.indices, x.batch_size, dims, (f, f, f))
+    slots = x.batch_size * (dims[0] // f) * (dims[1] // f) * (dims[2] // f)
+    return idx, slots, f * f * f, 1, False
+
+
+def downsample_plan(x, factor: int = 2, plan=None):
     """Token plan of the ``floor(coord / factor)`` merge: windows of ``factor``^3 cells, one head.
-    Returns ``(plan, merged coordinates int32 [M, 4], merged spatial shape)``."""
+    Returns ``(plan, merged coordinates int32 [M, 4], merged spatial shape)``.  ``plan``: a plan made earlier
+    from :func:`downsample_plan_request` of the same voxels (possibly still in flight)."""
     from .fused import TokenPlan
     f = int(factor)
     dims = [-(-int(e) // f) * f for e in x.spatial_shape]
     win = (f, f, f)
-    idx = sparse_window_indices(x.indices, x.batch_size, dims, win)
-    slots = x.batch_size * (dims[0] // f) * (dims[1] // f) * (dims[2] // f)
-    plan = TokenPlan(idx, slots, f * f * f, 1, tasks=False)
+    if plan is None:
+        req = downsample_plan_request(x, f)
+        plan = TokenPlan(*req[:4], tasks=req[4])
+    plan.finish()
     coords = torch.empty((plan.windows, 4), dtype=torch.int32, device=x.indices.device)
     with torch.cuda.device(coords.device):
         _lib.check(_lib.load().sswin_window_coords(_ptr(plan.plan), plan.g_cap, plan.windows, _i32x3(dims), _i32x3(win),
@@ -214,8 +228,12 @@ class PoolDownsample(nn.Module):
         self.norm = norm_layer(dim) if norm_layer is not None else nn.Identity()
         self.reduction = nn.Linear(dim, 2 * dim, bias=False)
 
-    def forward(self, x):
-        plan, coords, shape = downsample_plan(x, 2)
+    def plan_request(self, x):
+        """Arguments of the token plan this merge needs for ``x``'s voxels (see :func:`downsample_plan_request`)."""
+        return downsample_plan_request(x, 2)
+
+    def forward(self, x, plan=None):
+        plan, coords, shape = downsample_plan(x, 2, plan)
         pooled = _PoolWindows.apply(x.features, plan, True)
         out = copy.copy(x)
         out.indices, out.spatial_shape = coords, shape
@@ -325,10 +343,12 @@ class SwinTransformerBlock(nn.Module):
             self.attn.prefetch_plan(self.window_view(x)[0])
 
     @staticmethod
-    def prefetch_all(blocks, x):
-        """The same for all blocks of a stage at once: their token plans share one set of launches."""
-        if getattr(x, "window_cache", None) is not None:
-            prefetch_plans([(blk.attn, blk.window_view(x)[0]) for blk in blocks])
+    def prefetch_all(blocks, x, extra=()):
+        """The same for all blocks of a stage at once: their token plans share one set of launches.  ``extra``:
+        further ``TokenPlan`` argument tuples to build in the same launches; their plans are returned."""
+        if getattr(x, "window_cache", None) is None:
+            return prefetch_plans([], extra)
+        return prefetch_plans([(blk.attn, blk.window_view(x)[0]) for blk in blocks], extra)[len(blocks):]
 
     def forward_part1(self, x, mask_matrix):
         x = replace_feature(x, self.norm1(x.features))
@@ -382,10 +402,15 @@ class BasicLayer(nn.Module):
         x.window_cache = {}                      # (window, shift) -> window indices and token plans of this stage
         # the plans need the voxel indices only: all of them are enqueued now, so that only the first block waits
         # for totals from the GPU
-        SwinTransformerBlock.prefetch_all(self.blocks, x)
+        # (and the plan of the stride-2 merge behind the blocks, when the merge can say what it needs)
+        merge_plan = None
+        if self.downsample is not None and hasattr(self.downsample, "plan_request"):
+            merge_plan, = SwinTransformerBlock.prefetch_all(self.blocks, x, [self.downsample.plan_request(x)])
+        else:
+            SwinTransformerBlock.prefetch_all(self.blocks, x)
         for blk in self.blocks:
             x = blk(x, attn_mask)
         x.window_cache = None
         if self.downsample is not None:
-            x = self.downsample(x)
+            x = self.downsample(x, merge_plan) if merge_plan is not None else self.downsample(x)
         return x

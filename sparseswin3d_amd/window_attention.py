@@ -677,13 +677,16 @@ class WindowAttentionSparse(nn.Module):
         return replace_feature(x, self.proj_drop(tall_linear(x.features, self.proj)))
 
 
-def prefetch_plans(pairs):
+def prefetch_plans(pairs, extra=()):
     """Token plans for several ``(WindowAttentionSparse, window view)`` pairs, enqueued now by shared launches and
     kept in each view's ``plan_cache``: a stage calls this for all its blocks before the first one runs, so the
     plans' totals have reached the host by the time the blocks ask for them, and the regular and the shifted
     partition cost one set of launches instead of two.  Returns one plan per pair (None where the module or the
-    input does not take the fused path); pairs that share a view and a head count share a plan."""
+    input does not take the fused path); pairs that share a view and a head count share a plan.  ``extra``:
+    argument tuples of further ``TokenPlan``s (the stride-2 merge of the stage) built in the same launches;
+    their plans follow the pairs' in the returned list."""
     from . import fused
+    extra = list(extra)
     out, missing = [None] * len(pairs), {}
     for k, (attn, x) in enumerate(pairs):
         n = x.spatial_shape[0]
@@ -698,13 +701,9 @@ def prefetch_plans(pairs):
         else:
             missing.setdefault((id(cache), attn.num_heads), (cache, x, n, attn.num_heads, []))[4].append(k)
     todo = list(missing.values())
-    if len(todo) == 1:
-        cache, x, n, heads, ks = todo[0]
-        plans = [fused.TokenPlan(x.indices, x.batch_size, n, heads, defer=True)]
-    else:
-        plans = fused.TokenPlan.batch([(x.indices, x.batch_size, n, heads) for _, x, n, heads, _ in todo])
+    plans = fused.TokenPlan.batch([(x.indices, x.batch_size, n, heads) for _, x, n, heads, _ in todo] + extra)
     for (cache, _, _, heads, ks), plan in zip(todo, plans):
         cache[heads] = plan
         for k in ks:
             out[k] = plan
-    return out
+    return out + plans[len(todo):]
