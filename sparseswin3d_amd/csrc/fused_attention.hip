@@ -64,7 +64,7 @@ struct TokenPlanArgs {
     int64_t g_cap;
     int4* tasks;
     int32_t* tokens;         // [5 * N]
-    int blocks;              // ceil(B / 256)
+    int blocks;              // ceil(B / window slots per block) of the launch the plan goes into
 };
 
 __device__ __forceinline__ int32_t* tp_counters(const TokenPlanArgs& a) { return reinterpret_cast<int32_t*>(a.totals + 2); }
@@ -135,15 +135,33 @@ __device__ __forceinline__ int tp_block_max(int v, TpShared& sh) {
     return m;
 }
 
+// A thread of the per-block phases owns ITEMS consecutive window slots, a block TP_BLOCK * ITEMS of them.  Plans
+// with millions of window slots, nearly all of them empty (the 2 x 2 x 2 cells of a stride-2 merge), take ITEMS = 4:
+// the cost of these phases is the block-wide scans (ten per block), so four slots per thread cut it four times and
+// the number of blocks, whose partial sums every later block adds up, with it.  (Measured instead and dropped:
+// blocks of 1 024 threads, windows phase 158 us against 35; a single-workgroup scan of the partial sums between
+// the two phases, 56 us for 12 288 blocks; eight slots per thread, windows phase 25 us against 22.)
+constexpr int TP_ITEMS_WIDE = 4;
+constexpr int64_t TP_WIDE_FROM = 1 << 16;     // window slots from which a plan's launches take ITEMS = 4
+
 // block sums: partial_a[TP_SUMS * blk + k] = the sums over the block's window slots, partial_b[blk] = largest c
+template <int ITEMS>
 __device__ __forceinline__ void tp_phase_block_sums(const TokenPlanArgs& a, int blk, TpShared& sh) {
-    const int64_t w = (int64_t)blk * TP_BLOCK + threadIdx.x;
-    const int64_t c = w < a.B ? tp_window_count(a.bits, w, a.W) : 0;
-    int64_t item[TP_SUMS], total[TP_SUMS];
-    tp_items(c, item);
+    const int64_t w0 = ((int64_t)blk * TP_BLOCK + threadIdx.x) * ITEMS;
+    int64_t sum[TP_SUMS] = {0, 0, 0, 0}, total[TP_SUMS];
+    int cmax = 0;
 #pragma unroll
-    for (int k = 0; k < TP_SUMS; ++k) (void)block_exclusive_scan<int64_t, TP_BLOCK / 64>(item[k], sh.a, &total[k]);
-    const int cm = tp_block_max((int)c, sh);
+    for (int u = 0; u < ITEMS; ++u) {
+        const int64_t c = w0 + u < a.B ? tp_window_count(a.bits, w0 + u, a.W) : 0;
+        int64_t item[TP_SUMS];
+        tp_items(c, item);
+#pragma unroll
+        for (int k = 0; k < TP_SUMS; ++k) sum[k] += item[k];
+        cmax = max(cmax, (int)c);
+    }
+#pragma unroll
+    for (int k = 0; k < TP_SUMS; ++k) (void)block_exclusive_scan<int64_t, TP_BLOCK / 64>(sum[k], sh.a, &total[k]);
+    const int cm = tp_block_max(cmax, sh);
     if (threadIdx.x == 0) {
 #pragma unroll
         for (int k = 0; k < TP_SUMS; ++k) a.partial_a[TP_SUMS * blk + k] = total[k];
@@ -156,13 +174,20 @@ __device__ __forceinline__ void tp_phase_block_sums(const TokenPlanArgs& a, int 
 // window, sq_start}.  A window's slot inside its bucket is its rank among the bucket's windows in
 // window order (prefix of the earlier blocks' counts + scan inside the block): no atomics, and the same
 // descriptor order on every run.
+template <int ITEMS>
 __device__ __forceinline__ void tp_phase_windows(const TokenPlanArgs& a, int blk, TpShared& sh) {
     const int H = a.H;
     const int64_t g_cap = a.g_cap;
     int32_t* counters = tp_counters(a);
-    // this slot's bitmap words are requested first: the load overlaps the prefix below
-    const int64_t w = (int64_t)blk * TP_BLOCK + threadIdx.x;
-    const int64_t c = w < a.B ? tp_window_count(a.bits, w, a.W) : 0;
+    // this thread's bitmap words are requested first: the loads overlap the prefix below
+    const int64_t w0 = ((int64_t)blk * TP_BLOCK + threadIdx.x) * ITEMS;
+    int64_t c[ITEMS];
+    int cmax = 0;
+#pragma unroll
+    for (int u = 0; u < ITEMS; ++u) {
+        c[u] = w0 + u < a.B ? tp_window_count(a.bits, w0 + u, a.W) : 0;
+        cmax = max(cmax, (int)c[u]);
+    }
     // prefix of the earlier blocks
     int64_t p[TP_SUMS] = {0, 0, 0, 0};
     int pm = 0;
@@ -174,18 +199,24 @@ __device__ __forceinline__ void tp_phase_windows(const TokenPlanArgs& a, int blk
     int64_t total[TP_SUMS];
 #pragma unroll
     for (int k = 0; k < TP_SUMS; ++k) (void)block_exclusive_scan<int64_t, TP_BLOCK / 64>(p[k], sh.a, &total[k]);
-    const int bm = tp_block_max(max(pm, (int)c), sh);            // largest c up to and including this block
+    const int bm = tp_block_max(max(pm, cmax), sh);              // largest c up to and including this block
     if (threadIdx.x == 0) {
 #pragma unroll
         for (int k = 0; k < TP_SUMS; ++k) sh.base[k] = total[k];
     }
     __syncthreads();
-    int64_t item[TP_SUMS], e[TP_SUMS];
-    tp_items(c, item);
+    // running sums in front of this thread's first slot: scan of the threads' sums, then slot by slot
+    int64_t sum[TP_SUMS] = {0, 0, 0, 0}, e[TP_SUMS];
+#pragma unroll
+    for (int u = 0; u < ITEMS; ++u) {
+        int64_t item[TP_SUMS];
+        tp_items(c[u], item);
+#pragma unroll
+        for (int k = 0; k < TP_SUMS; ++k) sum[k] += item[k];
+    }
 #pragma unroll
     for (int k = 0; k < TP_SUMS; ++k)
-        e[k] = block_exclusive_scan<int64_t, TP_BLOCK / 64>(item[k], sh.a, &total[k]) + sh.base[k];
-    const int32_t k = (int32_t)(e[3] >> 32);                     // non-empty windows before this one
+        e[k] = block_exclusive_scan<int64_t, TP_BLOCK / 64>(sum[k], sh.a, &total[k]) + sh.base[k];
     if (blk == a.blocks - 1 && threadIdx.x == 0) {
         int64_t all[TP_SUMS];
 #pragma unroll
@@ -196,29 +227,39 @@ __device__ __forceinline__ void tp_phase_windows(const TokenPlanArgs& a, int blk
         for (int b = 0; b < 5; ++b) counters[b] = (int32_t)(tp_bucket_count(all, b) * H);
         counters[TPC_CMAX] = bm;
     }
-    const int32_t T = (int32_t)(e[0] & 0xffffffffll);
-    const int64_t q2 = e[0] >> 32;
-    if (w < a.B) a.win_T[w] = T;
+#pragma unroll
+    for (int u = 0; u < ITEMS; ++u) {
+        const int64_t w = w0 + u, cu = c[u];
+        const int32_t k = (int32_t)(e[3] >> 32);                 // non-empty windows before this one
+        const int32_t T = (int32_t)(e[0] & 0xffffffffll);
+        const int64_t q2 = e[0] >> 32;
+        if (w < a.B) a.win_T[w] = T;
 
-    const bool live = c > 0 && ((int64_t)k + 1) * H <= g_cap;
-    if (live) {
-        for (int h = 0; h < H; ++h) {
-            const int64_t g = (int64_t)k * H + h;
-            a.plan[g] = (int32_t)c;
-            a.plan[g_cap + g] = T;
-            a.plan[2 * g_cap + g] = (int32_t)(q2 * H + (int64_t)h * c * c);
-            a.plan[3 * g_cap + g] = (int32_t)w;
-            a.plan[4 * g_cap + g] = h;
+        const bool live = cu > 0 && ((int64_t)k + 1) * H <= g_cap;
+        if (live) {
+            for (int h = 0; h < H; ++h) {
+                const int64_t g = (int64_t)k * H + h;
+                a.plan[g] = (int32_t)cu;
+                a.plan[g_cap + g] = T;
+                a.plan[2 * g_cap + g] = (int32_t)(q2 * H + (int64_t)h * cu * cu);
+                a.plan[3 * g_cap + g] = (int32_t)w;
+                a.plan[4 * g_cap + g] = h;
+            }
         }
-    }
-    if (a.tasks == nullptr) return;
-    const int b = tp_bucket(c);
-    if (live && b < 4) {
-        const int64_t slot = tp_bucket_count(e, b) * H;
-        if (slot + H <= g_cap)
-            for (int h = 0; h < H; ++h)
-                a.tasks[(int64_t)b * g_cap + slot + h] =
-                    make_int4(T, (int)c | (h << 8), (int)w, (int32_t)(q2 * H + (int64_t)h * c * c));
+        const int b = tp_bucket(cu);
+        if (a.tasks != nullptr && live && b < 4) {
+            const int64_t slot = tp_bucket_count(e, b) * H;
+            if (slot + H <= g_cap)
+                for (int h = 0; h < H; ++h)
+                    a.tasks[(int64_t)b * g_cap + slot + h] =
+                        make_int4(T, (int)cu | (h << 8), (int)w, (int32_t)(q2 * H + (int64_t)h * cu * cu));
+        }
+        if (ITEMS > 1) {                                         // on to the thread's next slot
+            int64_t item[TP_SUMS];
+            tp_items(cu, item);
+#pragma unroll
+            for (int q = 0; q < TP_SUMS; ++q) e[q] += item[q];
+        }
     }
 }
 
@@ -282,15 +323,17 @@ __global__ __launch_bounds__(256) void tp_clear_kernel(TokenPlanBatch b) {
 __global__ __launch_bounds__(256) void tp_set_bits_kernel(TokenPlanBatch b) {
     tp_phase_set_bits(b.p[blockIdx.y], (int64_t)blockIdx.x * 256 + threadIdx.x, (int64_t)gridDim.x * 256);
 }
+template <int ITEMS>
 __global__ __launch_bounds__(TP_BLOCK) void tp_block_sums_kernel(TokenPlanBatch b) {
     __shared__ TpShared sh;
     const TokenPlanArgs& a = b.p[blockIdx.y];
-    if ((int)blockIdx.x < a.blocks) tp_phase_block_sums(a, blockIdx.x, sh);
+    if ((int)blockIdx.x < a.blocks) tp_phase_block_sums<ITEMS>(a, blockIdx.x, sh);
 }
+template <int ITEMS>
 __global__ __launch_bounds__(TP_BLOCK) void tp_windows_kernel(TokenPlanBatch b) {
     __shared__ TpShared sh;
     const TokenPlanArgs& a = b.p[blockIdx.y];
-    if ((int)blockIdx.x < a.blocks) tp_phase_windows(a, blockIdx.x, sh);
+    if ((int)blockIdx.x < a.blocks) tp_phase_windows<ITEMS>(a, blockIdx.x, sh);
 }
 __global__ __launch_bounds__(256) void tp_rank_kernel(TokenPlanBatch b) {
     tp_phase_rank(b.p[blockIdx.y], (int64_t)blockIdx.x * 256 + threadIdx.x, (int64_t)gridDim.x * 256);
@@ -973,13 +1016,27 @@ static int token_plan_launch(const TokenPlanArgs* args, int64_t* const* totals_o
         voxels = std::max(voxels, args[k].N);
         blocks = std::max(blocks, args[k].blocks);
     }
+    // all plans of a launch share the slots per thread: four as soon as one of them has that many window slots
+    int64_t slots = 0;
+    for (int k = 0; k < count; ++k) slots = std::max<int64_t>(slots, args[k].B);
+    const int items = slots >= TP_WIDE_FROM ? TP_ITEMS_WIDE : 1;
+    blocks = 0;
+    for (int k = 0; k < TP_MAX_BATCH; ++k) {
+        b.p[k].blocks = (int)(((int64_t)b.p[k].B + TP_BLOCK * items - 1) / (TP_BLOCK * items));
+        if (k < count) blocks = std::max(blocks, b.p[k].blocks);
+    }
     const unsigned y = (unsigned)count;
     const unsigned clear_blocks = (unsigned)std::min<size_t>((words + 255) / 256, 2048);
     const unsigned nb = (unsigned)std::min<int64_t>((voxels + 255) / 256, 1 << 20);
     hipLaunchKernelGGL(tp_clear_kernel, dim3(clear_blocks, y), dim3(256), 0, s, b);
     hipLaunchKernelGGL(tp_set_bits_kernel, dim3(nb, y), dim3(256), 0, s, b);
-    hipLaunchKernelGGL(tp_block_sums_kernel, dim3((unsigned)blocks, y), dim3(TP_BLOCK), 0, s, b);
-    hipLaunchKernelGGL(tp_windows_kernel, dim3((unsigned)blocks, y), dim3(TP_BLOCK), 0, s, b);
+    if (items == TP_ITEMS_WIDE) {
+        hipLaunchKernelGGL(tp_block_sums_kernel<TP_ITEMS_WIDE>, dim3((unsigned)blocks, y), dim3(TP_BLOCK), 0, s, b);
+        hipLaunchKernelGGL(tp_windows_kernel<TP_ITEMS_WIDE>, dim3((unsigned)blocks, y), dim3(TP_BLOCK), 0, s, b);
+    } else {
+        hipLaunchKernelGGL(tp_block_sums_kernel<1>, dim3((unsigned)blocks, y), dim3(TP_BLOCK), 0, s, b);
+        hipLaunchKernelGGL(tp_windows_kernel<1>, dim3((unsigned)blocks, y), dim3(TP_BLOCK), 0, s, b);
+    }
     hipLaunchKernelGGL(tp_rank_kernel, dim3(nb, y), dim3(256), 0, s, b);
     if (launch_ok("token plan")) return 1;
     // raw totals: the caller decodes them with sswin_token_plan_totals once the copies have landed

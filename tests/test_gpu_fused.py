@@ -25,7 +25,7 @@ def _closed_form_plan(ind, n, H):
     return tokens, np.stack([g_c, g_T, g_sq, g_w, g_h]), int((counts.astype(np.int64) ** 2).sum()) * H, int(counts.max())
 
 
-@pytest.mark.parametrize("case", ["random", "ragged", "single", "big"])
+@pytest.mark.parametrize("case", ["random", "ragged", "single", "big", "wide"])
 def test_token_plan_closed_forms(case):
     from sparseswin3d_amd.fused import TokenPlan
     rng = np.random.default_rng(len(case))
@@ -39,9 +39,12 @@ def test_token_plan_closed_forms(case):
     elif case == "single":
         B, n, H = 4, 27, 1
         ind = np.array([[3, 26]], np.int32)
-    else:
+    elif case == "big":
         B, n, H = 20000, 125, 3
         ind = random_window_indices(rng, B, n, 120000)
+    else:                            # enough window slots for the per-block phases to take blocks of 1 024 slots
+        B, n, H = 300000, 8, 1
+        ind = random_window_indices(rng, B, n, 250000)
     tokens, plan, A, c_max = _closed_form_plan(ind, n, H)
     tp = TokenPlan(torch.from_numpy(ind).cuda(), B, n, H)
     assert (tp.G, tp.A, tp.c_max) == (plan.shape[1], A, c_max)
@@ -61,16 +64,17 @@ def test_token_plans_in_one_batch_equal_single_plans():
              (random_window_indices(rng, 20000, 125, 120000), 20000, 125, 3, True),
              (np.zeros((0, 2), np.int32), 7, 27, 2, True),
              (random_window_indices(rng, 3000, 8, 9000), 3000, 8, 1, False),
-             (random_window_indices(rng, 700, 64, 20000), 700, 64, 4, True)]
+             (random_window_indices(rng, 700, 64, 20000), 700, 64, 4, True),
+             (random_window_indices(rng, 270000, 27, 90000), 270000, 27, 2, True)]   # its call uses the wide blocks
     dev = [(torch.from_numpy(ind).cuda(), B, n, H, tasks) for ind, B, n, H, tasks in specs]
-    plans = TokenPlan.batch(dev)                         # six plans: two library calls
+    plans = TokenPlan.batch(dev)                         # seven plans: two library calls
     assert len(plans) == len(specs)
     for spec, tp in zip(dev, plans):
         tp.finish()
         one = TokenPlan(*spec[:4], tasks=spec[4])
         assert (tp.G, tp.windows, tp.A, tp.c_max, list(tp.bucket_counts)) == \
                (one.G, one.windows, one.A, one.c_max, list(one.bucket_counts))
-        assert torch.equal(tp.tokens, one.tokens)
+        assert torch.equal(tp.tokens[:5 * tp.N], one.tokens[:5 * one.N])
         assert torch.equal(tp.plan.view(5, -1)[:, :tp.G], one.plan.view(5, -1)[:, :one.G])
         if spec[4] and tp.G:
             # descriptors of a bucket, as sets: their order inside a bucket is the same here, but not promised
