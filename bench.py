@@ -333,6 +333,7 @@ def kernel_table(wl, reps=20, only=None):
         val_e = torch.empty(E, device=dev)
 
         gp = ops.group_plan(c)
+        row_pos = ops.group_row_positions(s_idx, gp)
         bias_d = torch.randn(H, b["n"], b["n"], device=dev)
         n_table_o = int(wl["blocks"][0]["attn"].relative_position_bias_table.shape[0])
         ti_o = F.BiasTableIndex.build(relative_position_index_3d(wl["blocks"][0]["attn"].window_size).to(dev), n_table_o)
@@ -340,19 +341,24 @@ def kernel_table(wl, reps=20, only=None):
         entries = [
             # name, callable, algorithmic bytes, calls per attention fwd+bwd of the module (0: not on the module's path)
             ("operand_map [N]", lambda: ops.operand_map(b["idx"], b["slots"], b["n"]), 20 * N, 1),
-            ("sorted_coo_indices [4,E] x 2", lambda: ops.sorted_coo_indices(b["idx"], omap, H, hd), 32 * E + 20 * N, 1),
+            # the module asks for the Q/V matrix only; K^T's and the products' index matrices are written when somebody
+            # reads them (rows with 0 calls below: what the reference's operators always write)
+            ("sorted_coo_indices [4,E], Q/V", lambda: ops.sorted_coo_indices(b["idx"], omap, H, hd, k=False), 16 * E + 20 * N, 1),
+            ("sorted_coo_indices [4,E] x 2 (with K^T's)", lambda: ops.sorted_coo_indices(b["idx"], omap, H, hd), 32 * E + 20 * N, 0),
             ("operand_copy Q/V order", lambda: ops.operand_copy(qkv_rows, 2 * D, val_e, omap, H, hd, 0, True), 2 * s * E, 6),
             ("operand_copy K^T order", lambda: ops.operand_copy(qkv_rows, D, val_e, omap, H, hd, 1, True), 2 * s * E, 2),
             ("qkv_sparse_indices (reference operator)", lambda: ops.qkv_sparse_indices(b["idx"], b["slots"], b["n"], H, hd, _defer_check=True), 8 * N + 40 * E, 0),
             ("plan_from_indices", lambda: _lib.check(lib.sswin_plan_from_indices(ptr(q.indices), m, hd, ptr(plan), g_cap, totals, ptr(ws), nb, stream)), 0, 1),
-            ("block_matmul q_k", mm(0, q.values, kt.values, q.indices, out_s, out_si, A), 2 * s * E + (s + 16) * A + 4 * G, 1),
-            ("bias + mask add, one pass [A]", lambda: ops.group_add_bias_mask(s_val, s_idx, gp, b["n"], bias_d, mask), 2 * s * A + 8 * G, 1),
-            ("bias table gradient from the product's groups", lambda: ops.group_bias_table_grad(g_s, s_idx, gp, H, b["n"], ti_o.code, ti_o.offset0, n_table_o), 4 * A, 1),
+            ("block_matmul q_k, values", mm(0, q.values, kt.values, q.indices, out_s, None, A), 2 * s * E + s * A + 4 * G, 1),
+            ("block_matmul q_k (values + index matrix)", mm(0, q.values, kt.values, q.indices, out_s, out_si, A), 2 * s * E + (s + 16) * A + 4 * G, 0),
+            ("bias + mask add, one pass [A]", lambda: ops.group_add_bias_mask(s_val, row_pos, gp, b["n"], bias_d, mask), 2 * s * A + 8 * G, 1),
+            ("bias table gradient from the product's groups", lambda: ops.group_bias_table_grad(g_s, row_pos, gp, H, b["n"], ti_o.code, ti_o.offset0, n_table_o), 4 * A, 1),
             ("softmax rows from the group sizes [A]", lambda: ops.softmax_rows_from_counts(c, A), 4 * A + 12 * G, 1),
             ("flatten_indices [3,A] (generic softmax rows)", lambda: ops.flatten_indices(s_idx[:3], s_shape[:3]), 16 * A, 0),
             ("unique_consecutive_indices [A] (generic softmax rows)", lambda: ops.unique_consecutive_indices(flat), 8 * A, 0),
             ("softmax_last_dim_forward", lambda: ops.softmax_last_dim_forward(rows, s_val), 12 * A, 1),
-            ("block_matmul qk_v", mm(1, p_val, v.values, v.indices, out_o, out_oi, E), s * A + s * E + (s + 16) * E + 4 * G, 1),
+            ("block_matmul qk_v, values", mm(1, p_val, v.values, v.indices, out_o, None, E), s * A + 2 * s * E + 4 * G, 1),
+            ("block_matmul qk_v (values + index matrix)", mm(1, p_val, v.values, v.indices, out_o, out_oi, E), s * A + s * E + (s + 16) * E + 4 * G, 0),
             ("permute order from the group structure [E]", lambda: ops.permute_heads_order(o_idx, o_shape), 0, 0),
             ("flatten_indices [4,E] (generic permute)", lambda: ops.flatten_indices(perm_idx, [o_shape[0], o_shape[2], o_shape[1], o_shape[3]]), 0, 0),
             ("sort_indices [E] (generic permute)", lambda: ops.sort_indices(flat_perm), 0, 0),

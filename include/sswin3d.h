@@ -173,10 +173,12 @@ int sswin_softmax_rows_from_counts(const int32_t* c, const int32_t* scans, int64
 /* values + bias[head, pos_i, pos_j], and -100 more where the mask regions of the two positions differ, for a
  * [B, H, n, n] 'q_k' product in sorted order (sp_add_rpb and sp_add_mask, sparse_swin/swin3d_base.py:557-581), from the
  * product's plan (as sswin_plan_from_indices writes it) instead of a linear index per entry.  values / out: [A] of
- * `dtype`; idx: the product's [4, A] indices (rows 2 and 3 are read at 2c places per group); bias: fp32 [H, n, n]
+ * `dtype`; row_pos: device int32 [sum c], the window position of every token row in group order (from
+ * sswin_group_row_positions on the product's indices, or every C-th entry of row 2 of the Q operand's indices: the
+ * product's own index matrix is not read); bias: fp32 [H, n, n]
  * (rounded to `dtype` before the addition, as the reference's dense bias is); mask: int8 [n_mask_windows, n] region ids
  * or NULL; c_max: largest group (at most 512 tokens).  Asynchronous. */
-int sswin_group_add_bias_mask(int dtype, const void* values, const int32_t* idx, int64_t A, const int32_t* plan, int64_t g_cap,
+int sswin_group_add_bias_mask(int dtype, const void* values, const int32_t* row_pos, int64_t A, const int32_t* plan, int64_t g_cap,
                               int64_t G, int c_max, int n, const float* bias, const int8_t* mask, int n_mask_windows,
                               void* out, void* stream);
 
@@ -184,7 +186,7 @@ int sswin_group_add_bias_mask(int dtype, const void* values, const int32_t* idx,
  * table[code[p] - code[q] + offset0][head] (the gather of sparse_swin/swin3d_base.py:644-647 folded in; table: fp32
  * [table_rows, H], code: device int32 [n], both as sswin_bias_from_table takes them; codes and table rows below 2^15).
  * The table is a few KB where the gathered bias of 7^3 windows is 1.4 MB.  Asynchronous. */
-int sswin_group_add_table_bias_mask(int dtype, const void* values, const int32_t* idx, int64_t A, const int32_t* plan,
+int sswin_group_add_table_bias_mask(int dtype, const void* values, const int32_t* row_pos, int64_t A, const int32_t* plan,
                                     int64_t g_cap, int64_t G, int c_max, int n, const float* table, int table_rows, int H,
                                     const int32_t* code, int offset0, const int8_t* mask, int n_mask_windows, void* out,
                                     void* stream);
@@ -215,7 +217,9 @@ int sswin_scan_counts(const int32_t* c, int64_t G, int32_t* scans, void* ws, siz
  *                         out_val [sum c*C], out_idx [4, sum c*C] = (window, head, pos_i, channel)
  * `plan`/`g_cap`/`G`/`c_max` come from sswin_plan_from_indices on `tok_idx`, the [4, M] index matrix
  * of the operand that carries the token rows (Q for q_k, V for qk_v), M = sum c*C; its row 2
- * provides pos.  All array arguments: device.  Asynchronous. */
+ * provides pos.  out_idx == NULL: values only (a caller that composes the operators and never reads the product's
+ * index matrix saves its 16 bytes per entry); out_val == NULL: index rows only (mat1_v, mat2_v and dtype are then
+ * ignored), so the two halves can be asked for at different times.  All array arguments: device.  Asynchronous. */
 int sswin_block_matmul(int kind, int dtype, const void* mat1_v, const void* mat2_v,
                        const int32_t* tok_idx, int64_t M, int C, const int32_t* plan,
                        int64_t g_cap, int64_t G, int64_t c_max, void* out_val,

@@ -88,7 +88,7 @@ SIGNATURES = {
                                                _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i32, _vp]),
 }
 
-ABI_VERSION = 23
+ABI_VERSION = 24
 _lib = None
 
 

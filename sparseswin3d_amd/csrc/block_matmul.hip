@@ -468,13 +468,27 @@ int sswin_block_matmul(int kind, int dtype, const void* mat1_v, const void* mat2
                 "Invalid mul_type code %d. Expected 'q_k' or 'qk_v'.", kind);
     SSWIN_CHECK(C > 0 && M >= 0 && G >= 0 && G <= g_cap, "block_matmul: bad sizes");
     if (G == 0 || out_nnz == 0) return 0;
-    SSWIN_CHECK(mat1_v && mat2_v && tok_idx && plan && out_val && out_idx, "block_matmul: null pointer");
+    SSWIN_CHECK(tok_idx && plan && (out_val || out_idx), "block_matmul: null pointer");
+    SSWIN_CHECK(!out_val || (mat1_v && mat2_v), "block_matmul: null operand");
     SSWIN_CHECK(out_nnz < (int64_t)INT32_MAX, "block_matmul: output nnz does not fit int32 offsets");
     SSWIN_CHECK(c_max >= 1 && c_max <= MAX_POS,
                 "block_matmul: largest group holds %lld tokens; supported range is [1, %d]", (long long)c_max, MAX_POS);
     GroupTable gt{plan, plan + g_cap, plan + 2 * g_cap, plan + 3 * g_cap, plan + 4 * g_cap};
     const int32_t* tok_pos = tok_idx + 2 * M;
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (!out_val) {                                          // index rows only
+        const unsigned blocks = (unsigned)((G + GROUPS_PER_WG - 1) / GROUPS_PER_WG);
+        if (kind == SSWIN_MUL_Q_K)
+            hipLaunchKernelGGL((emit_coo_kernel<true>), dim3(blocks), dim3(256), 0, s, gt, G, C, tok_pos, out_idx, out_nnz);
+        else
+            hipLaunchKernelGGL((emit_coo_kernel<false>), dim3(blocks), dim3(256), 0, s, gt, G, C, tok_pos, out_idx, out_nnz);
+        return launch_ok("block product indices");
+    }
+    if (!out_idx) {                                          // values only
+        if (kind == SSWIN_MUL_Q_K)
+            return dispatch_product<MODE_QK, false>(dtype, mat1_v, mat2_v, gt, G, C, tok_pos, out_val, nullptr, out_nnz, s);
+        return dispatch_product<MODE_PV, false>(dtype, mat1_v, mat2_v, gt, G, C, tok_pos, out_val, nullptr, out_nnz, s);
+    }
     if (kind == SSWIN_MUL_Q_K)
         return dispatch_product<MODE_QK, true>(dtype, mat1_v, mat2_v, gt, G, C, tok_pos, out_val, out_idx, out_nnz, s);
     return dispatch_product<MODE_PV, true>(dtype, mat1_v, mat2_v, gt, G, C, tok_pos, out_val, out_idx, out_nnz, s);

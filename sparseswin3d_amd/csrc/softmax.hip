@@ -189,9 +189,9 @@ constexpr int GBM_U = 8;                                     // rows in flight p
 // (bias of positions p, q = table[code[p] - code[q] + offset0]): the table is a few KB where the gathered [H, n, n]
 // bias of 7^3 windows is 1.4 MB, so the gathers stay in the L1.
 template <typename T, bool TABLE>
-__global__ __launch_bounds__(256) void group_bias_mask_kernel(const T* __restrict__ val, const int32_t* __restrict__ idx_pi,
-                                                              const int32_t* __restrict__ idx_pj,
-                                                              const int32_t* __restrict__ cs, const int32_t* __restrict__ sq_start,
+__global__ __launch_bounds__(256) void group_bias_mask_kernel(const T* __restrict__ val, const int32_t* __restrict__ row_pos,
+                                                              const int32_t* __restrict__ cs, const int32_t* __restrict__ row_start,
+                                                              const int32_t* __restrict__ sq_start,
                                                               const int32_t* __restrict__ window,
                                                               const int32_t* __restrict__ head, int64_t G, int n,
                                                               const float* __restrict__ bias, const int32_t* __restrict__ code,
@@ -209,16 +209,17 @@ __global__ __launch_bounds__(256) void group_bias_mask_kernel(const T* __restric
     const int rows = c - i0 < GBM_ROWS ? c - i0 : GBM_ROWS;
     const int h = head[g];
     const int64_t sq = sq_start[g];
+    const int32_t* gpos = row_pos + row_start[g];            // window positions of the group's c tokens
     const int8_t* mrow = mask ? mask + (int64_t)(window[g] % nmw) * n : nullptr;
     int32_t* pj = pos_j[wave];
     int32_t* pi = pos_i[wave];
     // low half: the position (TABLE: its code), high half: its mask region
     for (int t = lane; t < c; t += 64) {
-        const int b = idx_pj[sq + t];
+        const int b = gpos[t];
         pj[t] = (TABLE ? code[b] : b) | (mrow ? (int)mrow[b] << 16 : 0);
     }
     if (lane < rows) {
-        const int a = idx_pi[sq + (int64_t)(i0 + lane) * c];
+        const int a = gpos[i0 + lane];
         pi[lane] = (TABLE ? code[a] : a) | (mrow ? (int)mrow[a] << 16 : 0);
     }
     __builtin_amdgcn_wave_barrier();
@@ -289,27 +290,27 @@ int sswin_softmax_last_dim_backward(const int32_t* idx_row, const void* y, const
     return fail("softmax backward: values must be float32 or float64 (dtype code %d)", dtype);
 }
 
-static int launch_group_bias_mask(const char* who, bool table_form, int dtype, const void* values, const int32_t* idx,
+static int launch_group_bias_mask(const char* who, bool table_form, int dtype, const void* values, const int32_t* row_pos,
                                   int64_t A, const int32_t* plan, int64_t g_cap, int64_t G, int c_max, int n, const float* bias,
                                   const int32_t* code, int offset0, int H, const int8_t* mask, int n_mask_windows, void* out,
                                   void* stream) {
     SSWIN_CHECK(A >= 0 && G >= 0 && G <= g_cap && n > 0 && n < (1 << 15), "%s: bad sizes", who);
     if (A == 0 || G == 0) return 0;
-    SSWIN_CHECK(values && idx && plan && bias && out, "%s: null pointer", who);
+    SSWIN_CHECK(values && row_pos && plan && bias && out, "%s: null pointer", who);
     SSWIN_CHECK(c_max > 0 && c_max <= GBM_MAX_C, "%s: windows of %d tokens are not supported (%d at most)", who, c_max, GBM_MAX_C);
     SSWIN_CHECK(!mask || n_mask_windows > 0, "%s: mask without window count", who);
     hipStream_t s = static_cast<hipStream_t>(stream);
     const dim3 grid((unsigned)((G + 3) / 4), (unsigned)((c_max + GBM_ROWS - 1) / GBM_ROWS));
-    const int32_t *cs = plan, *sq = plan + 2 * g_cap, *win = plan + 3 * g_cap, *head = plan + 4 * g_cap;
+    const int32_t *cs = plan, *rs = plan + g_cap, *sq = plan + 2 * g_cap, *win = plan + 3 * g_cap, *head = plan + 4 * g_cap;
 #define SSWIN_GBM(T)                                                                                                   \
     do {                                                                                                               \
         if (table_form)                                                                                                \
             hipLaunchKernelGGL((group_bias_mask_kernel<T, true>), grid, dim3(256), 0, s, static_cast<const T*>(values), \
-                               idx + 2 * A, idx + 3 * A, cs, sq, win, head, G, n, bias, code, offset0, H, mask,        \
+                               row_pos, cs, rs, sq, win, head, G, n, bias, code, offset0, H, mask,                     \
                                n_mask_windows, static_cast<T*>(out));                                                  \
         else                                                                                                           \
             hipLaunchKernelGGL((group_bias_mask_kernel<T, false>), grid, dim3(256), 0, s, static_cast<const T*>(values), \
-                               idx + 2 * A, idx + 3 * A, cs, sq, win, head, G, n, bias, code, offset0, H, mask,        \
+                               row_pos, cs, rs, sq, win, head, G, n, bias, code, offset0, H, mask,                     \
                                n_mask_windows, static_cast<T*>(out));                                                  \
     } while (0)
     switch (dtype) {
@@ -323,20 +324,20 @@ static int launch_group_bias_mask(const char* who, bool table_form, int dtype, c
     return launch_ok(who);
 }
 
-int sswin_group_add_bias_mask(int dtype, const void* values, const int32_t* idx, int64_t A, const int32_t* plan, int64_t g_cap,
+int sswin_group_add_bias_mask(int dtype, const void* values, const int32_t* row_pos, int64_t A, const int32_t* plan, int64_t g_cap,
                               int64_t G, int c_max, int n, const float* bias, const int8_t* mask, int n_mask_windows,
                               void* out, void* stream) {
-    return launch_group_bias_mask("group_add_bias_mask", false, dtype, values, idx, A, plan, g_cap, G, c_max, n, bias, nullptr, 0,
+    return launch_group_bias_mask("group_add_bias_mask", false, dtype, values, row_pos, A, plan, g_cap, G, c_max, n, bias, nullptr, 0,
                                   1, mask, n_mask_windows, out, stream);
 }
 
-int sswin_group_add_table_bias_mask(int dtype, const void* values, const int32_t* idx, int64_t A, const int32_t* plan,
+int sswin_group_add_table_bias_mask(int dtype, const void* values, const int32_t* row_pos, int64_t A, const int32_t* plan,
                                     int64_t g_cap, int64_t G, int c_max, int n, const float* table, int table_rows, int H,
                                     const int32_t* code, int offset0, const int8_t* mask, int n_mask_windows, void* out,
                                     void* stream) {
     SSWIN_CHECK(table_rows > 0 && table_rows < (1 << 15) && H > 0 && (A == 0 || G == 0 || code),
                 "group_add_table_bias_mask: bad table");
-    return launch_group_bias_mask("group_add_table_bias_mask", true, dtype, values, idx, A, plan, g_cap, G, c_max, n, table, code,
+    return launch_group_bias_mask("group_add_table_bias_mask", true, dtype, values, row_pos, A, plan, g_cap, G, c_max, n, table, code,
                                   offset0, H, mask, n_mask_windows, out, stream);
 }
 

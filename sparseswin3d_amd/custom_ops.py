@@ -182,19 +182,20 @@ def operand_copy(vox, col0, val, omap, num_heads, c, layout, to_operand):
                                           _stream(d)))
 
 
-def sorted_coo_indices(indices, omap, num_heads, c):
+def sorted_coo_indices(indices, omap, num_heads, c, qv=True, k=True):
     """The sorted [4, E] index matrices of Q/V and of K^T (``idx.index_select(1, order)`` of
-    :func:`qkv_sparse_indices`), written directly."""
+    :func:`qkv_sparse_indices`), written directly.  ``qv=False`` / ``k=False``: None in place of that matrix."""
     lib = _lib.load()
     d = _dev(indices, omap)
     indices = indices.contiguous()
     n_vox = indices.shape[0]
     e = n_vox * num_heads * c
-    idx_qv = torch.empty((4, e), dtype=torch.int32, device=d)
-    idx_k = torch.empty((4, e), dtype=torch.int32, device=d)
-    with torch.cuda.device(d):
-        _lib.check(lib.sswin_sorted_coo_indices(_ptr(indices), _ptr(omap), n_vox, int(num_heads), int(c), _ptr(idx_qv),
-                                                _ptr(idx_k), _stream(d)))
+    idx_qv = torch.empty((4, e), dtype=torch.int32, device=d) if qv else None
+    idx_k = torch.empty((4, e), dtype=torch.int32, device=d) if k else None
+    if qv or k:
+        with torch.cuda.device(d):
+            _lib.check(lib.sswin_sorted_coo_indices(_ptr(indices), _ptr(omap), n_vox, int(num_heads), int(c),
+                                                    _ptr(idx_qv) if qv else None, _ptr(idx_k) if k else None, _stream(d)))
     return idx_qv, idx_k
 
 
@@ -378,35 +379,51 @@ def matmul_cuda_naive(mat1_v, mat1_idx, mat1_shape, mat2_v, mat2_idx, mat2_shape
 
     Returns ``(indices int32 [4, nnz], values [nnz], shape list[4], _c int32 [G])``.
     """
-    lib = _lib.load()
     _check(mat1_idx.dim() == 2, "Expected mat1_idx.dim() == 2 to be true, but got false.")
     _check(mat2_idx.dim() == 2, "Expected mat2_idx.dim() == 2 to be true, but got false.")
-    _check(mat1_v.dim() == 1, "Expected mat1_v.dim() == 1 to be true, but got false.")
-    _check(mat2_v.dim() == 1, "Expected mat2_v.dim() == 1 to be true, but got false.")
+    return block_product(mat1_v, mat1_idx, mat1_shape, mat2_v, mat2_idx, mat2_shape, mul_type)
+
+
+def block_product(mat1_v, mat1_idx, mat1_shape, mat2_v, mat2_idx, mat2_shape, mul_type, values=True, indices=True):
+    """:func:`matmul_cuda_naive` with either half of the result optional: ``indices=False`` returns None in place of
+    the product's [4, nnz] index matrix (a composition of the operators that never reads it saves its 16 bytes per
+    entry), ``values=False`` returns None in place of the values (then the value arrays may be None), so that the
+    index matrix can be produced later, when somebody asks for it.  The index matrix of the operand that carries no
+    token rows (``mat2_idx`` of 'q_k', ``mat1_idx`` of 'qk_v') may be None: the product reads nothing from it."""
+    lib = _lib.load()
     _check(mul_type in _MUL, f"Invalid mul_type: {mul_type}. Expected 'q_k' or 'qk_v'.")
-    _check(mat1_v.dtype == mat2_v.dtype, f"mat1 dtype {mat1_v.dtype} does not match mat2 dtype {mat2_v.dtype}")
-    _check(mat1_idx.dtype == mat2_idx.dtype,
-           f"mat1 dtype {mat1_idx.dtype} does not match mat2 dtype {mat2_idx.dtype}")
-    _check(mat1_idx.dtype == torch.int32, f"mat1 dtype is not int32, but {mat1_idx.dtype}")
+    _check(values or indices, "block_product: nothing asked for")
+    kind = _MUL[mul_type]
+    tok_idx, other_idx = (mat1_idx, mat2_idx) if kind == 0 else (mat2_idx, mat1_idx)
+    _check(tok_idx is not None and tok_idx.dim() == 2, "the operand with the token rows needs its [4, M] index matrix")
+    if values:
+        _check(mat1_v.dim() == 1, "Expected mat1_v.dim() == 1 to be true, but got false.")
+        _check(mat2_v.dim() == 1, "Expected mat2_v.dim() == 1 to be true, but got false.")
+        _check(mat1_v.dtype == mat2_v.dtype, f"mat1 dtype {mat1_v.dtype} does not match mat2 dtype {mat2_v.dtype}")
+        _check(mat1_v.dtype in _DTYPE_CODE, f"unsupported value dtype {mat1_v.dtype}")
+    if other_idx is not None:
+        _check(mat1_idx.dtype == mat2_idx.dtype,
+               f"mat1 dtype {mat1_idx.dtype} does not match mat2 dtype {mat2_idx.dtype}")
+    _check(tok_idx.dtype == torch.int32, f"mat1 dtype is not int32, but {tok_idx.dtype}")
     s1, s2 = [int(v) for v in mat1_shape], [int(v) for v in mat2_shape]
     _check(len(s1) == 4 and len(s2) == 4 and s1[0] == s2[0] and s1[1] == s2[1] and s1[3] == s2[2],
            f"Invalid shapes: mat1_shape {s1} and mat2_shape {s2}. Expected sizes: 4. Expected "
            "mat1_shape[0] == mat2_shape[0], mat1_shape[1] == mat2_shape[1], mat1_shape[3] == mat2_shape[2].")
-    _check(mat1_v.dtype in _DTYPE_CODE, f"unsupported value dtype {mat1_v.dtype}")
-    d = _dev(mat1_v, mat1_idx, mat2_v, mat2_idx)
-    _check(mat1_idx.shape[0] == 4 and mat2_idx.shape[0] == 4, "index matrices must have 4 rows")
-    _check(mat1_idx.shape[1] == mat1_v.numel() and mat2_idx.shape[1] == mat2_v.numel(),
-           "index and value counts differ")
-    mat1_v, mat2_v = mat1_v.contiguous(), mat2_v.contiguous()
-    mat1_idx, mat2_idx = mat1_idx.contiguous(), mat2_idx.contiguous()
+    d = _dev(*(t for t in (mat1_v, mat1_idx, mat2_v, mat2_idx) if t is not None))
+    _check(tok_idx.shape[0] == 4 and (other_idx is None or other_idx.shape[0] == 4), "index matrices must have 4 rows")
+    if values:
+        for v, i in ((mat1_v, mat1_idx), (mat2_v, mat2_idx)):
+            _check(i is None or i.shape[1] == v.numel(), "index and value counts differ")
+        mat1_v, mat2_v = mat1_v.contiguous(), mat2_v.contiguous()
+    tok_idx = tok_idx.contiguous()
+    value_dtype = mat1_v.dtype if values else torch.float32
 
-    kind = _MUL[mul_type]
-    tok_idx = mat1_idx if kind == 0 else mat2_idx
     inner = s1[3] if kind == 0 else s2[3]
     m = tok_idx.shape[1]
     out_shape = [s1[0], s1[1], s1[2], s2[3]]
     if m == 0:
-        return (torch.empty((4, 0), dtype=torch.int32, device=d), torch.empty(0, dtype=mat1_v.dtype, device=d),
+        return (torch.empty((4, 0), dtype=torch.int32, device=d) if indices else None,
+                torch.empty(0, dtype=value_dtype, device=d) if values else None,
                 out_shape, torch.empty(0, dtype=torch.int32, device=d))
     _check(m % inner == 0, f"operand nnz {m} is not a multiple of its dense last dimension {inner}")
     rows = m // inner
@@ -414,20 +431,21 @@ def matmul_cuda_naive(mat1_v, mat1_idx, mat1_shape, mat2_v, mat2_idx, mat2_shape
     with torch.cuda.device(d):
         plan, g_cap, (g, sum_c, sum_c2, c_max) = _plan_of(tok_idx, inner, s1[0] * s1[1], lib, d)
         if kind == 0:
-            _check(mat2_v.numel() == m, f"'q_k': mat2 holds {mat2_v.numel()} values, expected {m}")
+            _check(not values or mat2_v.numel() == m, f"'q_k': mat2 holds {mat2_v.numel() if values else 0} values, expected {m}")
             nnz = sum_c2
         else:
-            _check(mat1_v.numel() == sum_c2,
-                   f"'qk_v': mat1 holds {mat1_v.numel()} values, expected sum of c*c = {sum_c2}")
+            _check(not values or mat1_v.numel() == sum_c2,
+                   f"'qk_v': mat1 holds {mat1_v.numel() if values else 0} values, expected sum of c*c = {sum_c2}")
             nnz = m
-        out_idx = torch.empty((4, nnz), dtype=torch.int32, device=d)
-        out_val = torch.empty(nnz, dtype=mat1_v.dtype, device=d)
-        _lib.check(lib.sswin_block_matmul(kind, _DTYPE_CODE[mat1_v.dtype], _ptr(mat1_v), _ptr(mat2_v),
-                                          _ptr(tok_idx), m, inner, _ptr(plan), g_cap, g, c_max,
-                                          _ptr(out_val), _ptr(out_idx), nnz, stream))
+        out_idx = torch.empty((4, nnz), dtype=torch.int32, device=d) if indices else None
+        out_val = torch.empty(nnz, dtype=value_dtype, device=d) if values else None
+        _lib.check(lib.sswin_block_matmul(kind, _DTYPE_CODE[value_dtype], _ptr(mat1_v) if values else None,
+                                          _ptr(mat2_v) if values else None, _ptr(tok_idx), m, inner, _ptr(plan), g_cap, g,
+                                          c_max, _ptr(out_val) if values else None, _ptr(out_idx) if indices else None,
+                                          nnz, stream))
     c_view = plan[:g]
     _plan_cache.put(c_view, plan, g_cap, (g, sum_c, sum_c2, c_max))
-    if kind == 1:
+    if kind == 1 and indices:
         # the product has the group structure of V (same windows, heads, rows and dense extent): a later
         # permute of it finds the plan without another pass over its indices
         _index_plan_cache.put(out_idx, inner, plan, g_cap, (g, sum_c, sum_c2, c_max))
@@ -509,14 +527,31 @@ def group_plan(_c):
     return GroupPlan(plan, g_cap, int(totals[0]), int(totals[1]), int(totals[3]))
 
 
-def group_add_bias_mask(values, idx, gp, n, bias32, mask):
-    """``values + bias[head, pos_i, pos_j]`` (and ``-100`` where the int8 mask regions of the two positions differ) for a
-    'q_k' product with indices ``idx`` and :class:`GroupPlan` ``gp``: sp_add_rpb followed by sp_add_mask."""
+def group_row_positions(idx, gp):
+    """Window position of every attention row of a 'q_k' product with indices ``idx`` [4, A] and :class:`GroupPlan`
+    ``gp``, in group order: int32 [sum c].  (Every ``C``-th entry of row 2 of the Q operand's index matrix holds the
+    same numbers.)"""
     lib = _lib.load()
-    d = _dev(values, idx, bias32)
-    _check(values.dtype in _DTYPE_CODE and bias32.dtype == torch.float32 and idx.dtype == torch.int32, "group_add_bias_mask: dtypes")
+    d = _dev(idx)
+    _check(idx.dtype == torch.int32 and idx.dim() == 2 and idx.shape[0] == 4, "group_row_positions: idx must be int32 [4, A]")
+    idx = idx.contiguous()
+    rows = torch.empty(max(gp.rows, 1), dtype=torch.int32, device=d)
+    with torch.cuda.device(d):
+        _lib.check(lib.sswin_group_row_positions(_ptr(idx), idx.shape[1], _ptr(gp.plan), gp.g_cap, gp.groups, _ptr(rows),
+                                                 _stream(d)))
+    return rows
+
+
+def group_add_bias_mask(values, row_pos, gp, n, bias32, mask):
+    """``values + bias[head, pos_i, pos_j]`` (and ``-100`` where the int8 mask regions of the two positions differ) for a
+    'q_k' product with row positions ``row_pos`` (:func:`group_row_positions`) and :class:`GroupPlan` ``gp``:
+    sp_add_rpb followed by sp_add_mask."""
+    lib = _lib.load()
+    d = _dev(values, row_pos, bias32)
+    _check(values.dtype in _DTYPE_CODE and bias32.dtype == torch.float32 and row_pos.dtype == torch.int32, "group_add_bias_mask: dtypes")
+    _check(row_pos.dim() == 1 and row_pos.numel() >= gp.rows, "group_add_bias_mask: one position per token row")
     _check(mask is None or mask.dtype == torch.int8, "group_add_bias_mask: the mask must hold int8 region ids")
-    values, idx, bias32 = values.contiguous(), idx.contiguous(), bias32.contiguous()
+    values, idx, bias32 = values.contiguous(), row_pos.contiguous(), bias32.contiguous()
     mask = None if mask is None else mask.contiguous()
     out = torch.empty_like(values)
     with torch.cuda.device(d):
@@ -527,16 +562,17 @@ def group_add_bias_mask(values, idx, gp, n, bias32, mask):
     return out
 
 
-def group_add_table_bias_mask(values, idx, gp, n, table32, code, offset0, mask):
+def group_add_table_bias_mask(values, row_pos, gp, n, table32, code, offset0, mask):
     """:func:`group_add_bias_mask` with the bias taken from the relative position table ``table32`` [rows, H] itself:
     bias of positions p, q = ``table32[code[p] - code[q] + offset0, head]``."""
     lib = _lib.load()
-    d = _dev(values, idx, table32, code)
-    _check(values.dtype in _DTYPE_CODE and table32.dtype == torch.float32 and idx.dtype == torch.int32 and code.dtype == torch.int32,
+    d = _dev(values, row_pos, table32, code)
+    _check(values.dtype in _DTYPE_CODE and table32.dtype == torch.float32 and row_pos.dtype == torch.int32 and code.dtype == torch.int32,
            "group_add_table_bias_mask: dtypes")
+    _check(row_pos.dim() == 1 and row_pos.numel() >= gp.rows, "group_add_table_bias_mask: one position per token row")
     _check(mask is None or mask.dtype == torch.int8, "group_add_table_bias_mask: the mask must hold int8 region ids")
     _check(table32.dim() == 2 and code.numel() >= n, "group_add_table_bias_mask: table [rows, H] and one code per position")
-    values, idx, table32, code = values.contiguous(), idx.contiguous(), table32.contiguous(), code.contiguous()
+    values, idx, table32, code = values.contiguous(), row_pos.contiguous(), table32.contiguous(), code.contiguous()
     mask = None if mask is None else mask.contiguous()
     out = torch.empty_like(values)
     with torch.cuda.device(d):
@@ -547,18 +583,17 @@ def group_add_table_bias_mask(values, idx, gp, n, table32, code, offset0, mask):
     return out
 
 
-def group_bias_table_grad(grad_values, idx, gp, num_heads, n, code, offset0, table_rows):
+def group_bias_table_grad(grad_values, row_pos, gp, num_heads, n, code, offset0, table_rows):
     """Gradient of the relative position bias table [table_rows, H] from the gradient of a 'q_k' product's values
-    (fp32), summed in a fixed order."""
+    (fp32) and its row positions (:func:`group_row_positions`), summed in a fixed order."""
     lib = _lib.load()
-    d = _dev(grad_values, idx)
+    d = _dev(grad_values, row_pos)
     _check(grad_values.dtype == torch.float32, "group_bias_table_grad: the gradient must be float32")
-    grad_values, idx = grad_values.contiguous(), idx.contiguous()
+    _check(row_pos.dtype == torch.int32 and row_pos.dim() == 1 and row_pos.numel() >= gp.rows,
+           "group_bias_table_grad: one int32 position per token row")
+    grad_values, rows = grad_values.contiguous(), row_pos.contiguous()
     d_table = torch.empty((table_rows, num_heads), dtype=torch.float32, device=d)
     with torch.cuda.device(d):
-        rows = torch.empty(max(gp.rows, 1), dtype=torch.int32, device=d)
-        _lib.check(lib.sswin_group_row_positions(_ptr(idx), idx.shape[1], _ptr(gp.plan), gp.g_cap, gp.groups, _ptr(rows),
-                                                 _stream(d)))
         nbytes = lib.sswin_bias_table_grad_workspace_bytes(gp.groups, int(num_heads), int(table_rows))
         ws = _ws(nbytes, d)
         _lib.check(lib.sswin_bias_table_grad(_ptr(gp.plan), gp.g_cap, gp.groups, _ptr(rows), 0, int(num_heads), int(n), _ptr(code),

@@ -54,20 +54,56 @@ def replace_feature(out, new_features):
     return out.replace_feature(new_features)
 
 
+class _LazyIndices:
+    """The [4, nnz] index matrix of a block product, written by the library the first time somebody reads it.  The
+    matrix is a function of the token operand's indices alone, and a composition of the operators that goes from
+    product to product by the group sizes never reads it (16 bytes per entry, 164 MB for the attention of 100 000
+    voxels)."""
+
+    def __init__(self, fn):
+        self.fn, self.value = fn, None
+
+    def get(self):
+        if self.value is None:
+            self.value, self.fn = self.fn(), None
+        return self.value
+
+
 class SparseTensor:
     """4-D COO tensor: ``indices`` int32 [4, nnz], ``values`` [nnz], ``shape`` list of 4."""
 
-    def __init__(self, indices, values, shape, group_counts=None):
-        assert indices.shape[0] == 4, "Invalid shape"
-        assert indices.ndim == 2, "Invalid shape"
+    def __init__(self, indices, values, shape, group_counts=None, row_positions=None):
+        if not isinstance(indices, _LazyIndices):
+            assert indices.shape[0] == 4, "Invalid shape"
+            assert indices.ndim == 2, "Invalid shape"
         assert values.ndim == 1, "Invalid shape"
         assert len(shape) == 4, "Invalid shape"
-        self.indices = indices
+        self._idx = indices
         self.values = values
         self.shape = shape
         # tokens per (window, head) group when the tensor is a 'q_k' product (or shares its index matrix):
         # lets softmax_last_dim number the attention rows without hashing the index matrix
         self.group_counts = group_counts
+        # window position of every token row in group order (int32 [sum c]) when the tensor is a 'q_k' product:
+        # what the bias and mask kernels need of the index matrix
+        self.row_positions = row_positions
+
+    @property
+    def indices(self):
+        if isinstance(self._idx, _LazyIndices):
+            self._idx = self._idx.get()
+        return self._idx
+
+    @indices.setter
+    def indices(self, value):
+        self._idx = value
+
+    def index_source(self):
+        """The index matrix, or the object that will produce it: what a tensor with the same structure is built from
+        without forcing the matrix into existence."""
+        if isinstance(self._idx, _LazyIndices) and self._idx.value is not None:
+            self._idx = self._idx.value
+        return self._idx
 
     def __repr__(self):
         return f"SparseTensor(indices={self.indices}, values={self.values}, shape={self.shape})"
@@ -106,7 +142,8 @@ class SparseTensor:
 
     def __mul__(self, other):
         if isinstance(other, (int, float)):
-            return SparseTensor(self.indices, self.values * other, self.shape, self.group_counts)
+            return SparseTensor(self.index_source(), self.values * other, self.shape, self.group_counts,
+                                self.row_positions)
         raise NotImplementedError
 
 
@@ -125,14 +162,14 @@ class _spspmm_block_naive(Function):
     """Window-blocked sparse x sparse product; gradients flow to both value arrays."""
 
     @staticmethod
-    def forward(ctx, mat1_v, mat1_idx, mat1_shape, mat2_v, mat2_idx, mat2_shape, mul_type):
+    def forward(ctx, mat1_v, mat1_idx, mat1_shape, mat2_v, mat2_idx, mat2_shape, mul_type, want_indices=True):
         _check_mul_type(mul_type)
-        mat3_idx, mat3_v, mat3_shape, counts = ops.matmul_cuda_naive(
-            mat1_v, mat1_idx, mat1_shape, mat2_v, mat2_idx, mat2_shape, mul_type)
+        mat3_idx, mat3_v, mat3_shape, counts = ops.block_product(
+            mat1_v, mat1_idx, mat1_shape, mat2_v, mat2_idx, mat2_shape, mul_type, indices=want_indices)
         ctx.save_for_backward(mat2_v, mat1_v, counts)
         ctx.mul_type = mul_type
         ctx.inner = mat1_shape[-1] if mul_type == "q_k" else mat2_shape[-1]
-        ctx.mark_non_differentiable(mat3_idx, counts)
+        ctx.mark_non_differentiable(*(t for t in (mat3_idx, counts) if t is not None))
         # without this autograd hands backward a zero tensor for every output that has no gradient, the [4, nnz]
         # index matrix included (a 360 MB fill for 7^3 windows)
         ctx.set_materialize_grads(False)
@@ -142,7 +179,7 @@ class _spspmm_block_naive(Function):
     @once_differentiable
     def backward(ctx, _grad_idx, grad_v, _grad_shape, _grad_counts):
         if grad_v is None:
-            return None, None, None, None, None, None, None
+            return None, None, None, None, None, None, None, None
         grad_v = grad_v.contiguous()
         mat2_v, mat1_v, counts = ctx.saved_tensors
         inner = ctx.inner
@@ -159,14 +196,33 @@ class _spspmm_block_naive(Function):
             mat1_t = ops.qkv_transpose(mat1_v, counts, inner, "rr")
             grad_t = ops.qkv_transpose(grad_v, counts, inner, "rc")
             grad_mat2 = ops.matmul_grad_cuda_naive(mat1_t, grad_t, counts, inner, "rr_rc")
-        return grad_mat1, None, None, grad_mat2, None, None, None
+        return grad_mat1, None, None, grad_mat2, None, None, None, None
 
 
 def spspmm_block_naive(mat1: SparseTensor, mat2: SparseTensor, mul_type="q_k") -> SparseTensor:
+    """Window-blocked product of two sparse tensors.  On the GPU the result's index matrix is written when it is
+    first read (``result.indices``): the products, the bias / mask pass and the softmax of the attention go by the
+    group sizes and never ask for it."""
     _check_mul_type(mul_type)
-    idx, val, shape, counts = _spspmm_block_naive.apply(mat1.values, mat1.indices, mat1.shape,
-                                                        mat2.values, mat2.indices, mat2.shape, mul_type)
-    return SparseTensor(idx, val, shape, counts if mul_type == "q_k" else None)
+    # only the operand with the token rows (Q for 'q_k', V for 'qk_v') is read for its indices; the other one's may
+    # still be unwritten and stay so
+    idx1 = mat1.indices if mul_type == "q_k" else _written_indices(mat1)
+    idx2 = mat2.indices if mul_type == "qk_v" else _written_indices(mat2)
+    lazy = mat1.values.is_cuda
+    idx, val, shape, counts = _spspmm_block_naive.apply(mat1.values, idx1, mat1.shape, mat2.values, idx2, mat2.shape,
+                                                        mul_type, not lazy)
+    if lazy:
+        s1, s2 = list(mat1.shape), list(mat2.shape)
+        idx = _LazyIndices(lambda: ops.block_product(None, idx1, s1, None, idx2, s2, mul_type, values=False)[0])
+    if mul_type != "q_k":
+        return SparseTensor(idx, val, shape)
+    inner = int(mat1.shape[-1])
+    return SparseTensor(idx, val, shape, counts, idx1[2, ::inner].contiguous() if lazy else None)
+
+
+def _written_indices(mat: SparseTensor):
+    src = mat.index_source()
+    return None if isinstance(src, _LazyIndices) else src
 
 
 # ------------------------------------------------------------------------------------------
@@ -193,8 +249,9 @@ class _softmax_last_dim(Function):
 
 def softmax_last_dim(mat: SparseTensor) -> SparseTensor:
     dtype = mat.values.dtype
-    out = _softmax_last_dim.apply(mat.values.float(), mat.indices[:3], mat.shape[:-1], mat.group_counts)
-    return SparseTensor(mat.indices, out.to(dtype), mat.shape, mat.group_counts)
+    out = _softmax_last_dim.apply(mat.values.float(), None if mat.group_counts is not None else mat.indices[:3],
+                                  mat.shape[:-1], mat.group_counts)
+    return SparseTensor(mat.index_source(), out.to(dtype), mat.shape, mat.group_counts, mat.row_positions)
 
 
 # ------------------------------------------------------------------------------------------
@@ -261,7 +318,10 @@ def qkv_sparse_cuda(qkv: torch.Tensor, indices: torch.Tensor, batch_size: int, s
     num_heads, c = qkv.shape[2:]
     n = spatial_shape
     omap = ops.operand_map(indices, batch_size, n)
-    idx_qv, idx_k = ops.sorted_coo_indices(indices, omap, num_heads, c)
+    # the index matrix of K^T is read by nobody in the attention (the 'q_k' product takes its structure from Q):
+    # it is written when it is first asked for
+    idx_qv, _ = ops.sorted_coo_indices(indices, omap, num_heads, c, k=False)
+    idx_k = _LazyIndices(lambda: ops.sorted_coo_indices(indices, omap, num_heads, c, qv=False)[1])
     q_val, k_val, v_val = _SortedOperandValues.apply(qkv, omap)
     q = SparseTensor(idx_qv, q_val, [batch_size, num_heads, n, c])
     k_t = SparseTensor(idx_k, k_val, [batch_size, num_heads, c, n])
@@ -293,7 +353,9 @@ class _GroupBiasMask(Function):
     gathers, and an ``index_add`` into the dense bias)."""
 
     @staticmethod
-    def forward(ctx, values, table, idx, gp, n, mask, table_index):
+    def forward(ctx, values, table, row_pos, gp, n, mask, table_index):
+        # row_pos: window position of every token row in group order (int32 [sum c])
+        idx = row_pos
         num_heads = table.shape[1]
         table32 = table.detach().to(torch.float32).contiguous()
         ctx.save_for_backward(idx)
@@ -332,8 +394,9 @@ def sp_add_table_bias_and_mask(sparse: SparseTensor, table: torch.Tensor, table_
     n = sparse.shape[2]
     if gp is None or gp.c_max > 512 or n > 384:
         return None
-    out = _GroupBiasMask.apply(sparse.values, table, sparse.indices, gp, n, mask, table_index)
-    return SparseTensor(sparse.indices, out, sparse.shape, sparse.group_counts)
+    row_pos = sparse.row_positions if sparse.row_positions is not None else ops.group_row_positions(sparse.indices, gp)
+    out = _GroupBiasMask.apply(sparse.values, table, row_pos, gp, n, mask, table_index)
+    return SparseTensor(sparse.index_source(), out, sparse.shape, sparse.group_counts, row_pos)
 
 
 def trunc_normal_(tensor, mean=0.0, std=1.0, a=-2.0, b=2.0):

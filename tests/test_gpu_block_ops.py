@@ -294,6 +294,41 @@ def test_softmax_rows_from_the_group_sizes(ops, oracle, mix, H, hd):
     assert torch.equal(with_counts.values, generic.values)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16])
+@pytest.mark.parametrize("mix,H,hd", [("mixed", 3, 32), ("edges", 2, 16)])
+def test_index_matrices_written_on_demand(ops, oracle, mix, H, hd, dtype):
+    """spspmm_block_naive leaves the product's [4, nnz] index matrix unwritten until it is read: the attention
+    (q_k -> bias -> softmax -> qk_v) goes through without it, and reading it afterwards gives the matrix the
+    operator returns.  The library's values-only and indices-only halves equal the full call bit for bit."""
+    from sparseswin3d_amd.window_attention import SparseTensor, _LazyIndices, softmax_last_dim, spspmm_block_naive
+    B, n, d = build(oracle, mix, H, hd, seed=seed_of("lazy", mix, H, hd))
+    f = run_forward(ops, oracle, d, dtype)
+    q = SparseTensor(f["qi"], f["q"], d["q_shape"])
+    kt = SparseTensor(_LazyIndices(lambda: f["ki"]), f["kt"], d["k_shape"])        # K^T's matrix: never needed
+    v = SparseTensor(f["qi"], f["v"], d["q_shape"])
+    s = spspmm_block_naive(q * 0.5, kt, "q_k")
+    p = softmax_last_dim(s)
+    o = spspmm_block_naive(p, v, "qk_v")
+    for t in (kt, s, p, o):
+        assert isinstance(t._idx, _LazyIndices) and t._idx.value is None
+    assert torch.equal(s.row_positions, f["qi"][2, ::hd])
+    full_idx, full_val, _, _ = ops.matmul_cuda_naive(f["q"] * 0.5, f["qi"], d["q_shape"], f["kt"], f["ki"], d["k_shape"], "q_k")
+    assert torch.equal(s.values, full_val)
+    assert torch.equal(s.indices, full_idx) and p.indices is s.indices             # one matrix, written once
+    o_idx, o_val, _, _ = ops.matmul_cuda_naive(p.values.to(dtype), full_idx, s.shape, f["v"], f["qi"], d["q_shape"], "qk_v")
+    assert torch.equal(o.values, o_val) and torch.equal(o.indices, o_idx)
+    np.testing.assert_array_equal(host(o.indices), oracle.matmul_cuda_naive(
+        host(p.values), f["r_idx"], f["r_shape"], f["v64"], d["qi"], d["q_shape"], "qk_v")[0])
+    # the two halves through the operator module
+    only_idx, none_val, _, c = ops.block_product(None, f["qi"], d["q_shape"], None, None, d["k_shape"], "q_k", values=False)
+    none_idx, only_val, _, _ = ops.block_product(f["q"] * 0.5, f["qi"], d["q_shape"], f["kt"], None, d["k_shape"], "q_k",
+                                                 indices=False)
+    assert none_val is None and none_idx is None
+    assert torch.equal(only_idx, full_idx) and torch.equal(only_val, full_val) and torch.equal(c, f["c1"])
+    with pytest.raises(RuntimeError, match="nothing asked for"):
+        ops.block_product(f["q"], f["qi"], d["q_shape"], f["kt"], f["ki"], d["k_shape"], "q_k", values=False, indices=False)
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("window,mix,use_mask", [((5, 5, 5), "mixed", True), ((5, 5, 5), "edges", False), ((7, 7, 7), "full", True)])
 def test_table_bias_and_mask_in_one_pass(ops, oracle, window, mix, use_mask, dtype):
@@ -337,4 +372,6 @@ def test_table_bias_and_mask_in_one_pass(ops, oracle, window, mix, use_mask, dty
     # the entry point that takes the gathered [H, n, n] bias gives the same bits as the one that reads the table
     gp = ops.group_plan(f["c1"])
     dense = attn_mod.relative_position_bias(n, torch.float32).detach()
-    assert torch.equal(ops.group_add_bias_mask(vals, f["s_idx"], gp, n, dense, mask), fast.values.detach())
+    row_pos = ops.group_row_positions(f["s_idx"], gp)
+    assert torch.equal(row_pos[:gp.rows], f["qi"][2, ::hd])            # = the Q operand's position row, one entry per token
+    assert torch.equal(ops.group_add_bias_mask(vals, row_pos, gp, n, dense, mask), fast.values.detach())
