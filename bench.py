@@ -340,7 +340,9 @@ def kernel_table(wl, reps=20, only=None):
 
         entries = [
             # name, callable, algorithmic bytes, calls per attention fwd+bwd of the module (0: not on the module's path)
-            ("operand_map [N]", lambda: ops.operand_map(b["idx"], b["slots"], b["n"]), 20 * N, 1),
+            # the module takes the operand map and the products' group table from one token plan
+            ("token_plan (operand map + group table)", lambda: F.TokenPlan(b["idx"], b["slots"], b["n"], H, tasks=False), 28 * N + 20 * G, 1),
+            ("operand_map [N] (on its own)", lambda: ops.operand_map(b["idx"], b["slots"], b["n"]), 20 * N, 0),
             # the module asks for the Q/V matrix only; K^T's and the products' index matrices are written when somebody
             # reads them (rows with 0 calls below: what the reference's operators always write)
             ("sorted_coo_indices [4,E], Q/V", lambda: ops.sorted_coo_indices(b["idx"], omap, H, hd, k=False), 16 * E + 20 * N, 1),
@@ -348,7 +350,7 @@ def kernel_table(wl, reps=20, only=None):
             ("operand_copy Q/V order", lambda: ops.operand_copy(qkv_rows, 2 * D, val_e, omap, H, hd, 0, True), 2 * s * E, 6),
             ("operand_copy K^T order", lambda: ops.operand_copy(qkv_rows, D, val_e, omap, H, hd, 1, True), 2 * s * E, 2),
             ("qkv_sparse_indices (reference operator)", lambda: ops.qkv_sparse_indices(b["idx"], b["slots"], b["n"], H, hd, _defer_check=True), 8 * N + 40 * E, 0),
-            ("plan_from_indices", lambda: _lib.check(lib.sswin_plan_from_indices(ptr(q.indices), m, hd, ptr(plan), g_cap, totals, ptr(ws), nb, stream)), 0, 1),
+            ("plan_from_indices (group table from a [4,E] index matrix)", lambda: _lib.check(lib.sswin_plan_from_indices(ptr(q.indices), m, hd, ptr(plan), g_cap, totals, ptr(ws), nb, stream)), 0, 0),
             ("block_matmul q_k, values", mm(0, q.values, kt.values, q.indices, out_s, None, A), 2 * s * E + s * A + 4 * G, 1),
             ("block_matmul q_k (values + index matrix)", mm(0, q.values, kt.values, q.indices, out_s, out_si, A), 2 * s * E + (s + 16) * A + 4 * G, 0),
             ("bias + mask add, one pass [A]", lambda: ops.group_add_bias_mask(s_val, row_pos, gp, b["n"], bias_d, mask), 2 * s * A + 8 * G, 1),

@@ -347,6 +347,14 @@ class _IndexPlanCache:
 _index_plan_cache = _IndexPlanCache()
 
 
+def register_index_plan(idx, inner, plan, g_cap, groups, rows, nnz_sq, c_max):
+    """Tell the block products the plan of a sorted [4, M] index matrix ``idx`` (dense last dimension ``inner``) that
+    the caller has derived by other means: ``plan`` int32 [5 * g_cap] = rows c, row_start, sq_start, window, head of
+    the ``groups`` (window, head) groups, ``rows`` = sum of c, ``nnz_sq`` = sum of c*c, ``c_max`` = largest c.  The
+    stream that wrote ``plan`` must have been waited for.  The products of ``idx`` then skip the pass over it."""
+    _index_plan_cache.put(idx, int(inner), plan, int(g_cap), (int(groups), int(rows), int(nnz_sq), int(c_max)))
+
+
 def clear_caches():
     """Drop cached plans (and the tensors they keep alive)."""
     _plan_cache.clear()

@@ -317,17 +317,46 @@ def qkv_sparse_cuda(qkv: torch.Tensor, indices: torch.Tensor, batch_size: int, s
     ``operand_map``, which :class:`_OperandToVoxels` takes to bring a product back to voxel order."""
     num_heads, c = qkv.shape[2:]
     n = spatial_shape
-    omap = ops.operand_map(indices, batch_size, n)
+    plan = None
+    if qkv.is_cuda and indices.shape[0] > 0 and indices.dtype == torch.int32 and num_heads < 256:
+        # One token plan gives both what the operands need (voxel, first rank and size of its window by rank: the
+        # operand map) and what the block products need (sizes and offsets of the (window, head) groups), so neither
+        # the operand map's own ranking nor the products' pass over the [4, E] index matrix runs.  Invalid
+        # (window, pos) pairs raise here.
+        from . import fused
+        plan = fused.TokenPlan(indices, batch_size, n, num_heads, tasks=False)
+        omap = torch.cat([plan.tokens[:3 * plan.N], _valid_status(plan.N, indices.device)])
+    else:
+        omap = ops.operand_map(indices, batch_size, n)
     # the index matrix of K^T is read by nobody in the attention (the 'q_k' product takes its structure from Q):
     # it is written when it is first asked for
     idx_qv, _ = ops.sorted_coo_indices(indices, omap, num_heads, c, k=False)
     idx_k = _LazyIndices(lambda: ops.sorted_coo_indices(indices, omap, num_heads, c, qv=False)[1])
+    if plan is not None and plan.G > 0:
+        # group table of the products: the token plan's, with the row offset of a group in place of the first rank
+        # of its window (row_start = H * T + head * c)
+        table = plan.plan.view(5, plan.g_cap)
+        table[1].mul_(num_heads).addcmul_(table[4], table[0])
+        ops.register_index_plan(idx_qv, c, plan.plan, plan.g_cap, plan.G, num_heads * plan.N, plan.A, plan.c_max)
     q_val, k_val, v_val = _SortedOperandValues.apply(qkv, omap)
     q = SparseTensor(idx_qv, q_val, [batch_size, num_heads, n, c])
     k_t = SparseTensor(idx_k, k_val, [batch_size, num_heads, c, n])
     v = SparseTensor(idx_qv, v_val, [batch_size, num_heads, n, c])
     q.operand_map = k_t.operand_map = v.operand_map = omap
     return q, k_t, v
+
+
+_STATUS_OK = {}
+
+
+def _valid_status(n_vox: int, device):
+    """The validity pair {pairs out of range = 0, distinct pairs = N} that ends an operand map."""
+    key = (device, n_vox)
+    if key not in _STATUS_OK:
+        if len(_STATUS_OK) > 64:
+            _STATUS_OK.clear()
+        _STATUS_OK[key] = torch.tensor([0, n_vox], dtype=torch.int32, device=device)
+    return _STATUS_OK[key]
 
 
 def sp_add_rpb(sparse: SparseTensor, dense: torch.Tensor) -> SparseTensor:

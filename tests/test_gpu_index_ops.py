@@ -141,13 +141,17 @@ def test_index_ops_report_indices_they_cannot_address(ops):
     x[77] = -2
     with pytest.raises(RuntimeError, match="outside"):
         ops.return_inverse(dev(x), 500)
-    # through qkv_sparse_cuda the check is deferred: the next operator that waits for the stream raises
-    from sparseswin3d_amd.window_attention import qkv_sparse_cuda, spspmm_block_naive
+    # qkv_sparse_cuda builds its operands from a token plan, which reports the same faults
+    from sparseswin3d_amd.window_attention import qkv_sparse_cuda
     ind = np.concatenate([good[:300], good[5:6], good[300:]])
     qkv = torch.randn(len(ind), 3, H, hd, device="cuda")
-    q, k_t, v = qkv_sparse_cuda(qkv, dev(ind), B, n)
     with pytest.raises(RuntimeError, match="distinct"):
-        spspmm_block_naive(q, k_t, "q_k")
+        qkv_sparse_cuda(qkv, dev(ind), B, n)
+    # the operand map on its own defers the check: the next operator that waits for the stream raises
+    omap = ops.operand_map(dev(ind), B, n)
+    ops.sorted_coo_indices(dev(ind), omap, H, hd)
+    with pytest.raises(RuntimeError, match="distinct"):
+        ops.return_inverse(dev(x.clip(0, 499)), 500)
     ops.clear_caches()
     got = ops.qkv_sparse_indices(dev(good), B, n, H, hd)            # and the library still works afterwards
     assert got[1].numel() == 700 * H * hd
