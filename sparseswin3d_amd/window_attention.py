@@ -310,15 +310,18 @@ class _OperandToVoxels(Function):
         return d_val, None, None, None
 
 
-def qkv_sparse_cuda(qkv: torch.Tensor, indices: torch.Tensor, batch_size: int, spatial_shape):
+def qkv_sparse_cuda(qkv: torch.Tensor, indices: torch.Tensor, batch_size: int, spatial_shape, plan=None):
     """Sorted COO operands Q [B,H,n,hd], K^T [B,H,hd,n], V [B,H,n,hd] from ``qkv`` [N,3,H,hd]
     (reference swin3d_base.py:483-498: same tensors; the index matrices and values are written in sorted
     order directly instead of being expanded, hashed, sorted and gathered).  The returned tensors carry
     ``operand_map``, which :class:`_OperandToVoxels` takes to bring a product back to voxel order."""
     num_heads, c = qkv.shape[2:]
     n = spatial_shape
-    plan = None
-    if qkv.is_cuda and indices.shape[0] > 0 and indices.dtype == torch.int32 and num_heads < 256:
+    if plan is not None:
+        # a token plan of these indices made earlier (possibly still in flight, possibly shared with other modules)
+        plan.finish()
+        omap = torch.cat([plan.tokens[:3 * plan.N], _valid_status(plan.N, indices.device)])
+    elif qkv.is_cuda and indices.shape[0] > 0 and indices.dtype == torch.int32 and num_heads < 256:
         # One token plan gives both what the operands need (voxel, first rank and size of its window by rank: the
         # operand map) and what the block products need (sizes and offsets of the (window, head) groups), so neither
         # the operand map's own ranking nor the products' pass over the [4, E] index matrix runs.  Invalid
@@ -335,9 +338,9 @@ def qkv_sparse_cuda(qkv: torch.Tensor, indices: torch.Tensor, batch_size: int, s
     if plan is not None and plan.G > 0:
         # group table of the products: the token plan's, with the row offset of a group in place of the first rank
         # of its window (row_start = H * T + head * c)
-        table = plan.plan.view(5, plan.g_cap)
+        table = plan.plan.clone().view(5, plan.g_cap)
         table[1].mul_(num_heads).addcmul_(table[4], table[0])
-        ops.register_index_plan(idx_qv, c, plan.plan, plan.g_cap, plan.G, num_heads * plan.N, plan.A, plan.c_max)
+        ops.register_index_plan(idx_qv, c, table.view(-1), plan.g_cap, plan.G, num_heads * plan.N, plan.A, plan.c_max)
     q_val, k_val, v_val = _SortedOperandValues.apply(qkv, omap)
     q = SparseTensor(idx_qv, q_val, [batch_size, num_heads, n, c])
     k_t = SparseTensor(idx_k, k_val, [batch_size, num_heads, c, n])
@@ -714,8 +717,8 @@ class WindowAttentionSparse(nn.Module):
     def prefetch_plan(self, x):
         """Enqueue the token plan of ``x``'s window indices now and keep it in ``x.plan_cache`` (created if
         missing), so that its totals have reached the host by the time :meth:`forward` asks for them.
-        Returns the plan, or None when this input does not take the fused path.  :func:`prefetch_plans` does
-        the same for several blocks with shared launches."""
+        Returns the plan, or None for inputs that are not on the GPU.  :func:`prefetch_plans` does the same for
+        several blocks with shared launches."""
         return prefetch_plans([(self, x)])[0]
 
     def forward(self, x, mask):
@@ -723,19 +726,18 @@ class WindowAttentionSparse(nn.Module):
         b = x.batch_size
         c = x.features.shape[-1]
         plan = None
-        if self.fused:
-            from . import fused
-            if fused.supports(x.features, n):
-                # the token plan is enqueued first; the projection below runs while its totals travel.
-                # A stage hands the same window indices to several blocks: they share one plan.
-                cache = getattr(x, "plan_cache", None)
-                plan = cache.get(self.num_heads) if cache is not None else None
-                if plan is None:
-                    plan = fused.TokenPlan(x.indices, b, n, self.num_heads, defer=True)
-                    if cache is not None:
-                        cache[self.num_heads] = plan
+        from . import fused
+        if _takes_token_plan(self, x):
+            # the token plan is enqueued first; the projection below runs while its totals travel.
+            # A stage hands the same window indices to several blocks: they share one plan.
+            cache = getattr(x, "plan_cache", None)
+            plan = cache.get(self.num_heads) if cache is not None else None
+            if plan is None:
+                plan = fused.TokenPlan(x.indices, b, n, self.num_heads, defer=True)
+                if cache is not None:
+                    cache[self.num_heads] = plan
         qkv = tall_linear(x.features, self.qkv).reshape(-1, 3, self.num_heads, c // self.num_heads)
-        if plan is not None:
+        if plan is not None and self.fused and fused.supports(x.features, n):
             resident = fused.supports_resident(qkv, n) if self.resident is None else self.resident
             table_index = self._table_index(n)
             if table_index is not None:
@@ -746,7 +748,7 @@ class WindowAttentionSparse(nn.Module):
                                                    mask, b, n, self.scale, resident, plan)
             x = replace_feature(x, out)
             return replace_feature(x, self.proj_drop(tall_linear(x.features, self.proj)))
-        q, k_t, v = qkv_sparse_cuda(qkv, x.indices, b, n)
+        q, k_t, v = qkv_sparse_cuda(qkv, x.indices, b, n, plan)
         attn = spspmm_block_naive(q * self.scale, k_t, "q_k")
         biased = sp_add_table_bias_and_mask(attn, self.relative_position_bias_table, self._table_index(n), mask)
         if biased is not None:
@@ -769,12 +771,20 @@ class WindowAttentionSparse(nn.Module):
         return replace_feature(x, self.proj_drop(tall_linear(x.features, self.proj)))
 
 
+def _takes_token_plan(attn, x) -> bool:
+    """Every path of the module starts from a token plan of the window indices (the window-resident and fused
+    kernels walk it, the operator path takes its operand map and group table from it) when these are int32 on the
+    GPU."""
+    return x.features.is_cuda and x.indices.is_cuda and x.indices.dtype == torch.int32 and x.indices.shape[0] > 0 \
+        and attn.num_heads < 256
+
+
 def prefetch_plans(pairs, extra=()):
     """Token plans for several ``(WindowAttentionSparse, window view)`` pairs, enqueued now by shared launches and
     kept in each view's ``plan_cache``: a stage calls this for all its blocks before the first one runs, so the
     plans' totals have reached the host by the time the blocks ask for them, and the regular and the shifted
-    partition cost one set of launches instead of two.  Returns one plan per pair (None where the module or the
-    input does not take the fused path); pairs that share a view and a head count share a plan.  ``extra``:
+    partition cost one set of launches instead of two.  Returns one plan per pair (None for inputs that are not on
+    the GPU); pairs that share a view and a head count share a plan.  ``extra``:
     argument tuples of further ``TokenPlan``s (the stride-2 merge of the stage) built in the same launches;
     their plans follow the pairs' in the returned list."""
     from . import fused
@@ -782,7 +792,7 @@ def prefetch_plans(pairs, extra=()):
     out, missing = [None] * len(pairs), {}
     for k, (attn, x) in enumerate(pairs):
         n = x.spatial_shape[0]
-        if not attn.fused or not fused.supports(x.features, n):
+        if not _takes_token_plan(attn, x):
             continue
         cache = getattr(x, "plan_cache", None)
         if cache is None:
