@@ -242,8 +242,9 @@ DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 KERNEL_SYMBOLS = {
     "resident forward": ("wattn_fwd_kernel", ["sparseswin3d_amd/csrc/window_attention.hip"]),
     "resident backward (dQ,dK,dV,dS)": ("wattn_bwd_all_kernel", ["sparseswin3d_amd/csrc/window_attention.hip"]),
-    "block_matmul q_k": ("block_product_mfma_kernel<float, 0", ["sparseswin3d_amd/csrc/block_matmul.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
-    "block_matmul qk_v": ("block_product_mfma_kernel<float, 1", ["sparseswin3d_amd/csrc/block_matmul.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
+    "block_matmul q_k, values": ("block_product_mfma_kernel<float, 0", ["sparseswin3d_amd/csrc/block_matmul.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
+    "block_matmul qk_v, values": ("block_product_mfma_kernel<float, 1, false", ["sparseswin3d_amd/csrc/block_matmul.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
+    "block_matmul qk_v (values + index matrix)": ("block_product_mfma_kernel<float, 1, true", ["sparseswin3d_amd/csrc/block_matmul.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
     "grad rc_cr": ("block_product_mfma_kernel<float, 2", ["sparseswin3d_amd/csrc/block_matmul.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
     "grad rr_rc": ("block_product_mfma_kernel<float, 3", ["sparseswin3d_amd/csrc/block_matmul.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
     "grad cr_rr": ("block_product_mfma_kernel<float, 4", ["sparseswin3d_amd/csrc/block_matmul.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
@@ -277,6 +278,11 @@ def kernel_table(wl, reps=20, only=None):
     qkv = torch.randn(N, 3, H, hd, device=dev)
     tp = F.TokenPlan(b["idx"], b["slots"], b["n"], H)
     E, A, G = N * D, int(tp.A), int(tp.G)
+
+    def staged_plan():
+        # the plans of the regular and the shifted partition in one set of launches, totals not waited for
+        F.TokenPlan.batch([(bb["idx"], bb["slots"], bb["n"], H) for bb in wl["blocks"][:2]])
+    staged_plan.per_call_share = 1.0 / len(wl["blocks"][:2])
     sizes = dict(N=N, E=E, A=A, G=G, c_max=int(tp.c_max) if hasattr(tp, "c_max") else None)
     entries, f_entries = [], []
 
@@ -341,7 +347,8 @@ def kernel_table(wl, reps=20, only=None):
         entries = [
             # name, callable, algorithmic bytes, calls per attention fwd+bwd of the module (0: not on the module's path)
             # the module takes the operand map and the products' group table from one token plan
-            ("token_plan (operand map + group table)", lambda: F.TokenPlan(b["idx"], b["slots"], b["n"], H, tasks=False), 28 * N + 20 * G, 1),
+            ("token plan, one of a stage's two (operand map + group table)", staged_plan, 28 * N + 20 * G, 1),
+            ("token_plan built and waited for on its own", lambda: F.TokenPlan(b["idx"], b["slots"], b["n"], H, tasks=False), 28 * N + 20 * G, 0),
             ("operand_map [N] (on its own)", lambda: ops.operand_map(b["idx"], b["slots"], b["n"]), 20 * N, 0),
             # the module asks for the Q/V matrix only; K^T's and the products' index matrices are written when somebody
             # reads them (rows with 0 calls below: what the reference's operators always write)
@@ -384,7 +391,7 @@ def kernel_table(wl, reps=20, only=None):
         bg_bytes = lib.sswin_fused_bias_grad_workspace_bytes(tp.G, H, b["n"])
         bg_ws = torch.empty(int(bg_bytes), dtype=torch.uint8, device=dev)
         f_entries = [
-            ("fused token_plan", lambda: F.TokenPlan(b["idx"], b["slots"], b["n"], H), 28 * N + 20 * tp.G, 1),
+            ("fused token plan, one of a stage's two", staged_plan, 28 * N + 20 * tp.G, 1),
             ("fused S=QK^T+bias+mask", lambda: F._tokens_to_sq(tp, dt, True, qkv_c, 3 * D, 0, qkv_c, 3 * D, D, hd, 0.17, bias, mask, s_f, rows_f), 8 * E + 8 * A, 1),
             ("fused softmax fwd", lambda: ops.softmax_last_dim_forward(rows_f, s_f), 12 * A, 1),
             ("fused O=PV", lambda: F._sq_to_tokens(tp, dt, False, p_val, qkv_c, 3 * D, 2 * D, out_f, D, 0, hd, 1.0), 4 * A + 8 * E, 1),
@@ -443,11 +450,10 @@ def kernel_table(wl, reps=20, only=None):
     r_fwd()                                       # lse and out_r must hold a real forward for the backward timings
     # flops of a launch: 2 c^2 hd per product and group = 2 A hd per product (two in the forward, five in the backward)
     r_entries = [
-        ("resident token_plan", lambda: F.TokenPlan(b["idx"], b["slots"], b["n"], H), 28 * N + 36 * tp.G, 1),
-        # what a stage does: the plans of its two partitions from shared launches, nobody waiting for the totals;
-        # the row is the GPU time of both plans (no host round trip inside), bytes of both
-        ("token plans of both blocks, one batch, deferred", lambda: F.TokenPlan.batch(
-            [(bb["idx"], bb["slots"], bb["n"], H) for bb in wl["blocks"][:2]]), 2 * (28 * N + 36 * tp.G), 0),
+        # what a stage (and the step) does: the plans of its two partitions from shared launches, nobody waiting for
+        # the totals; the row is half the GPU time of the two plans
+        ("resident token plan, one of a stage's two", staged_plan, 28 * N + 36 * tp.G, 1),
+        ("token_plan built and waited for on its own", lambda: F.TokenPlan(b["idx"], b["slots"], b["n"], H), 28 * N + 36 * tp.G, 0),
         ("resident forward", r_fwd, 16 * Er + 4 * H * N, 1, 4 * A * hd),
         ("resident backward (dQ,dK,dV,dS)", r_bwd(3), 32 * Er + 4 * A + 4 * H * N, 1, 10 * A * hd),
         ("resident backward dQ, groups > 32 tokens", r_bwd(1, only_large), (24 * es // 4 * hd + 4) * rowsL, 0),
@@ -462,7 +468,7 @@ def kernel_table(wl, reps=20, only=None):
     def measure(items, path):
         rows_ = []
         for name, fn, nbytes, calls, *flops in items:
-            ms = event_time_ms(fn, reps, queue_ahead=True)
+            ms = event_time_ms(fn, reps, queue_ahead=True) * getattr(fn, "per_call_share", 1.0)
             gbps = nbytes / ms / 1e6 if nbytes else None
             rows_.append(dict(kernel=name, path=path, ms=ms, algorithmic_bytes=nbytes, calls=calls,
                               achieved_gbps=gbps, frac=(gbps / HBM_PEAK_GBPS) if gbps else None,
