@@ -185,3 +185,35 @@ def test_index_helpers_round_trip():
     assert torch.equal(x.indices, idx)
     m = compute_mask(list(grid), [5, 5, 5], [2, 2, 2], "cuda").cpu().numpy()
     np.testing.assert_array_equal(m, synth.shift_region_mask(grid, (5, 5, 5), (2, 2, 2)))
+
+
+def test_three_paths_share_one_prefetched_token_plan():
+    """Modules on different paths that see the same window view take the one plan a stage has prefetched: the
+    operator path derives its operand map and group table from it without changing it, so the order in which the
+    paths run does not matter and each gives what it gives with a plan of its own."""
+    from sparseswin3d_amd import fused, synth
+    from sparseswin3d_amd.window_attention import SparseVoxelTensor, WindowAttentionSparse, prefetch_plans
+    torch.manual_seed(4)
+    c4, grid = _scene(seed=9)
+    win_idx, nw, n = synth.window_indices(c4, grid, (5, 5, 5), (2, 2, 2))
+    mask = torch.from_numpy(synth.shift_region_mask(synth.padded_shape(grid, (5, 5, 5)), (5, 5, 5), (2, 2, 2))).cuda()
+    feats = torch.randn(len(win_idx), 96).cuda()
+    idx = torch.from_numpy(win_idx).cuda()
+    mods = {}
+    for path in ("operators", "resident", "fused"):
+        torch.manual_seed(1)
+        mods[path] = WindowAttentionSparse(96, 3, (5, 5, 5), qkv_bias=True).cuda()
+        set_path(mods[path], path)
+    alone = {p: m(SparseVoxelTensor(feats, idx, (n,), nw), mask).features for p, m in mods.items()}
+
+    view = SparseVoxelTensor(feats, idx, (n,), nw)
+    plans = prefetch_plans([(m, view) for m in mods.values()])
+    assert plans[0] is plans[1] is plans[2] and isinstance(plans[0], fused.TokenPlan)
+    before = None
+    for path in ("operators", "resident", "operators", "fused"):
+        out = mods[path](view, mask).features
+        assert view.plan_cache[3] is plans[0]
+        assert torch.equal(out, alone[path]), path
+        table = plans[0].plan.clone()
+        assert before is None or torch.equal(table, before)        # nobody wrote into the shared plan
+        before = table
