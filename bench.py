@@ -545,9 +545,13 @@ def stage_entries(wl):
         out = torch.zeros(M, D, device=c4.device).index_add_(0, inv, x.features[plan.tokens[:N].long()])
         return out / plan.plan[:M, None]
 
+    def fresh_mask():
+        layers._MASKS.clear()
+        return layers.compute_mask(list(pd), list(ws), list(sh), c4.device)
+
     return [
         ("stage window indices (pad+roll+partition)", lambda: layers.sparse_window_indices(c4, wl["batch_size"], pd, ws, sh), 24 * N, 1),
-        ("stage shift mask", lambda: layers.compute_mask(list(pd), list(ws), list(sh), c4.device), windows * n, 1),
+        ("stage shift mask (first pass of a stage; kept per shape afterwards)", fresh_mask, windows * n, 1),
         ("stage merge plan (2x2x2 cells, coords)", lambda: layers.downsample_plan(x, 2), 16 * N + 20 * N + 16 * M, 1),
         ("stage merge mean pool", lambda: layers._PoolWindows.apply(x.features, plan, True), 4 * D * (N + M), 1),
         ("torch roll + partition (reference form)", torch_partition, 24 * N, 0),

@@ -9,6 +9,7 @@ torch modules; the attention itself runs in the HIP operators.
 """
 from __future__ import annotations
 
+import collections
 import copy
 import ctypes as C
 from typing import List, Sequence
@@ -123,6 +124,16 @@ def compute_mask(dims: List[int], window_size: List[int], shift_size: List[int],
     device = torch.device(device)
     if device.type != "cuda":
         raise RuntimeError("compute_mask runs on the GPU only; there is no CPU fallback")
+    if device.index is None:
+        device = torch.device("cuda", torch.cuda.current_device())
+    # the mask is a function of the three shapes alone, and a stage asks for the same one in every forward pass:
+    # the last few are kept (per device and stream, read-only by convention), 256 MB at most
+    key = (tuple(int(e) for e in dims), tuple(int(e) for e in window_size), tuple(int(e) for e in shift_size),
+           device.index, torch.cuda.current_stream(device).cuda_stream)
+    mask = _MASKS.get(key)
+    if mask is not None:
+        _MASKS.move_to_end(key)
+        return mask
     windows = 1
     for extent, w in zip(dims, window_size):
         windows *= extent // w
@@ -131,7 +142,14 @@ def compute_mask(dims: List[int], window_size: List[int], shift_size: List[int],
     with torch.cuda.device(device):
         _lib.check(_lib.load().sswin_shift_mask(_i32x3(dims), _i32x3(window_size), _i32x3(shift_size), _ptr(mask),
                                                 _stream(device)))
+    _MASKS[key] = mask
+    while len(_MASKS) > 8 or (len(_MASKS) > 1 and sum(m.numel() for m in _MASKS.values()) > _MASK_CACHE_BYTES):
+        _MASKS.popitem(last=False)
     return mask
+
+
+_MASKS = collections.OrderedDict()
+_MASK_CACHE_BYTES = 256 << 20
 
 
 def sparse_window_indices(indices: torch.Tensor, batch_size: int, dims: Sequence[int], window_size: Sequence[int],

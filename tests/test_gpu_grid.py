@@ -140,3 +140,21 @@ def test_stage_with_downsample_and_shared_plans(monkeypatch):
     np.testing.assert_array_equal(y.indices.cpu().numpy(), ref_coords)
     assert list(y.spatial_shape) == [(g + 1) // 2 for g in grid] and y.features.shape[1] == 192
     close(y.features.detach().cpu().numpy(), ref.numpy(), 1e-4, "stage output after four blocks and the merge")
+
+
+def test_shift_masks_are_kept_per_shape():
+    """compute_mask returns the stored mask for shapes it has seen on this stream, a new one for others, and keeps
+    at most eight."""
+    from sparseswin3d_amd import layers
+    layers._MASKS.clear()
+    a = layers.compute_mask([10, 10, 10], [5, 5, 5], [2, 2, 2], "cuda")
+    assert layers.compute_mask([10, 10, 10], [5, 5, 5], [2, 2, 2], torch.device("cuda", 0)) is a
+    b = layers.compute_mask([10, 10, 15], [5, 5, 5], [2, 2, 2], "cuda")
+    assert b is not a and b.shape == (12, 125) and a.shape == (8, 125)
+    c = layers.compute_mask([10, 10, 10], [5, 5, 5], [2, 0, 2], "cuda")
+    assert c is not a and not torch.equal(c, a)
+    for k in range(9):
+        layers.compute_mask([5, 5, 5 * (k + 1)], [5, 5, 5], [2, 2, 2], "cuda")
+    assert len(layers._MASKS) == 8
+    again = layers.compute_mask([10, 10, 10], [5, 5, 5], [2, 2, 2], "cuda")        # dropped meanwhile: built anew
+    assert again is not a and torch.equal(again, a)
