@@ -288,11 +288,14 @@ int sswin_token_plan_totals(int64_t* totals, int H, int64_t g_cap);
  * is a few microseconds of work per launch.  Every descriptor holds the arguments of one
  * sswin_token_plan call with synchronize == 0 and gives the same results; plans with N == 0 are
  * skipped (totals all zero).  After waiting for `stream`, decode each totals_out with
- * sswin_token_plan_totals.  Rejects count > 4. */
+ * sswin_token_plan_totals.  Rejects count > 4.
+ * flags: SSWIN_PLAN_ORDER_ONLY writes only the first row of `tokens` (voxel of rank r; `tokens` may then hold N
+ * entries): what the stride-2 merge reads (sswin_pool_windows), four scattered stores per voxel fewer. */
+#define SSWIN_PLAN_ORDER_ONLY 1
 typedef struct sswin_token_plan_desc {
     const int32_t* indices;
     int64_t N;
-    int32_t B, n, H, reserved;
+    int32_t B, n, H, flags;
     int32_t* tokens;
     int32_t* plan;
     int64_t g_cap;

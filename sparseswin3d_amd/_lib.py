@@ -16,7 +16,7 @@ _vp, _i64, _i32, _sz = C.c_void_p, C.c_int64, C.c_int, C.c_size_t
 class TokenPlanDesc(C.Structure):
     """``sswin_token_plan_desc`` of include/sswin3d.h: the arguments of one deferred sswin_token_plan call."""
     _fields_ = [("indices", _vp), ("N", _i64), ("B", C.c_int32), ("n", C.c_int32), ("H", C.c_int32),
-                ("reserved", C.c_int32), ("tokens", _vp), ("plan", _vp), ("g_cap", _i64), ("tasks", _vp),
+                ("flags", C.c_int32), ("tokens", _vp), ("plan", _vp), ("g_cap", _i64), ("tasks", _vp),
                 ("totals_out", _vp), ("ws", _vp), ("ws_bytes", _sz)]
 
 
@@ -88,7 +88,7 @@ SIGNATURES = {
                                                _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i32, _vp]),
 }
 
-ABI_VERSION = 24
+ABI_VERSION = 25
 _lib = None
 
 

@@ -65,6 +65,7 @@ struct TokenPlanArgs {
     int4* tasks;
     int32_t* tokens;         // [5 * N]
     int blocks;              // ceil(B / window slots per block) of the launch the plan goes into
+    int order_only;          // tokens holds its first row only (voxel of rank r)
 };
 
 __device__ __forceinline__ int32_t* tp_counters(const TokenPlanArgs& a) { return reinterpret_cast<int32_t*>(a.totals + 2); }
@@ -299,6 +300,7 @@ __device__ __forceinline__ void tp_phase_rank(const TokenPlanArgs& a, int64_t gt
         const int r = T + below;
         if (r < N) {                                            // duplicates cannot push a rank past the end, but stay inside anyway
             order[r] = (int32_t)v;
+            if (a.order_only) continue;
             tok_T[r] = T;
             tok_c[r] = c;
             tok_pos[r] = wp.y;
@@ -973,8 +975,10 @@ size_t sswin_token_plan_workspace_bytes(int64_t N, int B, int n) {
 
 // Checks one plan's arguments and carves its workspace; `a` is ready to launch afterwards.
 static int token_plan_args(const int32_t* indices, int64_t N, int B, int n, int H, int32_t* tokens, int32_t* plan,
-                           int64_t g_cap, int32_t* tasks, int64_t* totals_out, void* ws, size_t ws_bytes,
+                           int64_t g_cap, int32_t* tasks, int64_t* totals_out, void* ws, size_t ws_bytes, int flags,
                            TokenPlanArgs& a) {
+    SSWIN_CHECK((flags & ~SSWIN_PLAN_ORDER_ONLY) == 0, "token_plan: unknown flags %d", flags);
+    a.order_only = (flags & SSWIN_PLAN_ORDER_ONLY) ? 1 : 0;
     SSWIN_CHECK(N > 0 && B > 0 && n > 0 && H > 0 && H < 256, "token_plan: bad sizes");
     SSWIN_CHECK(indices && tokens && plan && ws && totals_out, "token_plan: null pointer");
     SSWIN_CHECK(N < (int64_t)INT32_MAX, "token_plan: too many voxels");
@@ -1054,7 +1058,7 @@ int sswin_token_plan(const int32_t* indices, int64_t N, int B, int n, int H, int
     if (N == 0) return 0;
     hipStream_t s = static_cast<hipStream_t>(stream);
     TokenPlanArgs a;
-    if (token_plan_args(indices, N, B, n, H, tokens, plan, g_cap, tasks, totals_out, ws, ws_bytes, a)) return 1;
+    if (token_plan_args(indices, N, B, n, H, tokens, plan, g_cap, tasks, totals_out, ws, ws_bytes, 0, a)) return 1;
     totals_out[8] = N;                     // read back by sswin_token_plan_totals (the copy fills [0..7])
     if (token_plan_launch(&a, &totals_out, 1, s)) return 1;
     if (!synchronize) return 0;
@@ -1075,7 +1079,7 @@ int sswin_token_plan_batch(const sswin_token_plan_desc* descs, int count, void* 
         for (int i = 0; i < 9; ++i) d.totals_out[i] = 0;
         if (d.N == 0) continue;            // an empty plan: all totals zero, nothing to launch
         if (token_plan_args(d.indices, d.N, d.B, d.n, d.H, d.tokens, d.plan, d.g_cap, d.tasks, d.totals_out, d.ws,
-                            d.ws_bytes, args[live]))
+                            d.ws_bytes, d.flags, args[live]))
             return 1;
         d.totals_out[8] = d.N;
         totals[live++] = d.totals_out;

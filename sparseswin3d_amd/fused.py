@@ -58,7 +58,13 @@ class TokenPlan:
     MAX_BATCH = 4            # plans per sswin_token_plan_batch call
 
     def __init__(self, indices: torch.Tensor, batch_size: int, n: int, num_heads: int, defer: bool = False,
-                 tasks: bool = True):
+                 tasks: bool = True, order_only: bool = False):
+        if order_only:
+            # only the batch entry point knows the flag
+            self.__dict__.update(TokenPlan.batch([(indices, batch_size, n, num_heads, tasks, True)])[0].__dict__)
+            if not defer:
+                self.finish()
+            return
         self._allocate(indices, batch_size, n, num_heads, tasks)
         lib = _lib.load()
         d = self.device
@@ -73,7 +79,7 @@ class TokenPlan:
         if not defer:
             self.finish()
 
-    def _allocate(self, indices, batch_size, n, num_heads, tasks):
+    def _allocate(self, indices, batch_size, n, num_heads, tasks, order_only=False):
         lib = _lib.load()
         if indices.device.type != "cuda":
             raise RuntimeError("TokenPlan runs on the GPU only; there is no CPU fallback")
@@ -84,7 +90,9 @@ class TokenPlan:
         N = indices.shape[0]
         self.N, self.H, self.n, self.B = N, int(num_heads), int(n), int(batch_size)
         self.g_cap = max(1, min(N, self.B) * self.H)
-        self.tokens = torch.empty(5 * max(N, 1), dtype=torch.int32, device=d)
+        # order_only: the plan of a stride-2 merge, whose consumers read the voxel of every rank and nothing else
+        self.order_only = bool(order_only)
+        self.tokens = torch.empty((1 if order_only else 5) * max(N, 1), dtype=torch.int32, device=d)
         self.plan = torch.empty(5 * self.g_cap, dtype=torch.int32, device=d)
         # group descriptors of the window-resident kernels, bucketed by ceil(c / 32)
         self.tasks = torch.empty(16 * self.g_cap, dtype=torch.int32, device=d) if tasks else None
@@ -98,12 +106,13 @@ class TokenPlan:
     @classmethod
     def batch(cls, specs):
         """Deferred plans for several index sets on one device, built by shared launches (the regular and the
-        shifted block of a stage).  ``specs``: tuples ``(indices, batch_size, n, num_heads)`` or
-        ``(..., tasks)``; returns the plans in the same order, each to be completed with :meth:`finish`."""
+        shifted block of a stage).  ``specs``: tuples ``(indices, batch_size, n, num_heads)``,
+        ``(..., tasks)`` or ``(..., tasks, order_only)``; returns the plans in the same order, each to be completed
+        with :meth:`finish`."""
         plans = []
         for spec in specs:
             p = cls.__new__(cls)
-            p._allocate(*spec[:4], spec[4] if len(spec) > 4 else True)
+            p._allocate(*spec[:4], spec[4] if len(spec) > 4 else True, spec[5] if len(spec) > 5 else False)
             plans.append(p)
         if not plans:
             return plans
@@ -118,6 +127,7 @@ class TokenPlan:
                 descs = (_lib.TokenPlanDesc * len(chunk))()
                 for desc, p in zip(descs, chunk):
                     desc.indices, desc.N, desc.B, desc.n, desc.H = p._indices.data_ptr(), p.N, p.B, p.n, p.H
+                    desc.flags = 1 if p.order_only else 0
                     desc.tokens, desc.plan, desc.g_cap = p.tokens.data_ptr(), p.plan.data_ptr(), p.g_cap
                     desc.tasks = p.tasks.data_ptr() if p.tasks is not None else None
                     desc.totals_out, desc.ws, desc.ws_bytes = p._totals.data_ptr(), p._ws.data_ptr(), p._ws.numel()

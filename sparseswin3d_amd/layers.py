@@ -201,14 +201,14 @@ class _PoolWindows(Function):
 
 def downsample_plan_request(x, factor: int = 2):
     """What the token plan of the ``floor(coord / factor)`` merge is built from: the arguments
-    ``(indices, window slots, positions per window, heads = 1, tasks = False)`` of ``TokenPlan`` /
-    ``TokenPlan.batch``.  It depends on the voxel coordinates only, so a stage can enqueue it together with
+    ``(indices, window slots, positions per window, heads = 1, tasks = False, order_only = True)`` of
+    ``TokenPlan`` / ``TokenPlan.batch``.  It depends on the voxel coordinates only, so a stage can enqueue it together with
     the plans of its attention blocks and hand the plan to :func:`downsample_plan` later."""
     f = int(factor)
     dims = [-(-int(e) // f) * f for e in x.spatial_shape]
     idx = sparse_window_indices(x.indices, x.batch_size, dims, (f, f, f))
     slots = x.batch_size * (dims[0] // f) * (dims[1] // f) * (dims[2] // f)
-    return idx, slots, f * f * f, 1, False
+    return idx, slots, f * f * f, 1, False, True
 
 
 def downsample_plan(x, factor: int = 2, plan=None):
@@ -221,7 +221,7 @@ def downsample_plan(x, factor: int = 2, plan=None):
     win = (f, f, f)
     if plan is None:
         req = downsample_plan_request(x, f)
-        plan = TokenPlan(*req[:4], tasks=req[4])
+        plan = TokenPlan(*req[:4], tasks=req[4], order_only=req[5])
     plan.finish()
     coords = torch.empty((plan.windows, 4), dtype=torch.int32, device=x.indices.device)
     with torch.cuda.device(coords.device):

@@ -82,6 +82,17 @@ def test_token_plans_in_one_batch_equal_single_plans():
             for k in range(4):
                 m = int(tp.bucket_counts[k])
                 assert torch.equal(a[k, :m], b[k, :m])
+    # a plan that keeps the voxel order only (what the stride-2 merge reads) holds the same first row and group table
+    lean = TokenPlan(dev[4][0], 3000, 8, 1, tasks=False, order_only=True)
+    assert lean.tokens.numel() == lean.N and torch.equal(lean.tokens, plans[4].tokens[:lean.N])
+    assert torch.equal(lean.plan.view(5, -1)[:, :lean.G], plans[4].plan.view(5, -1)[:, :lean.G])
+    descs = (_lib.TokenPlanDesc * 1)()
+    descs[0].N, descs[0].B, descs[0].n, descs[0].H, descs[0].flags = 4, 4, 8, 1, 6
+    totals = torch.zeros(9, dtype=torch.int64)               # the library clears it before it looks at the rest
+    descs[0].totals_out = totals.data_ptr()
+    descs[0].indices = descs[0].tokens = descs[0].plan = descs[0].ws = dev[4][0].data_ptr()    # never reached
+    descs[0].g_cap, descs[0].ws_bytes = 4, 1 << 20
+    assert _lib.load().sswin_token_plan_batch(descs, 1, None) != 0 and b"flags" in _lib.load().sswin_last_error()
     # errors stay with their plan
     good = specs[0][0]
     bad = np.concatenate([good[:400], np.array([[50, 3]], np.int32), good[400:]])

@@ -106,9 +106,10 @@ def test_stage_with_downsample_and_shared_plans(monkeypatch):
     real = fused.TokenPlan
 
     class Counting(real):
-        def _allocate(self, indices, batch_size, n, num_heads, tasks):
+        def _allocate(self, indices, batch_size, n, num_heads, tasks, order_only=False):
             made.append(tasks)
-            super()._allocate(indices, batch_size, n, num_heads, tasks)
+            assert order_only == (not tasks)             # the merge's plan is the one that keeps the voxel order only
+            super()._allocate(indices, batch_size, n, num_heads, tasks, order_only)
 
     monkeypatch.setattr(fused, "TokenPlan", Counting)
     torch.manual_seed(3)
