@@ -59,23 +59,20 @@ class TokenPlan:
 
     def __init__(self, indices: torch.Tensor, batch_size: int, n: int, num_heads: int, defer: bool = False,
                  tasks: bool = True, order_only: bool = False):
+        self._allocate(indices, batch_size, n, num_heads, tasks, order_only)
         if order_only:
-            # only the batch entry point knows the flag
-            self.__dict__.update(TokenPlan.batch([(indices, batch_size, n, num_heads, tasks, True)])[0].__dict__)
-            if not defer:
-                self.finish()
-            return
-        self._allocate(indices, batch_size, n, num_heads, tasks)
-        lib = _lib.load()
-        d = self.device
-        with torch.cuda.device(d):
-            stream = C.c_void_p(torch.cuda.current_stream(d).cuda_stream)
-            _lib.check(lib.sswin_token_plan(_ptr(self._indices), self.N, self.B, self.n, self.H, _ptr(self.tokens),
-                                            _ptr(self.plan), self.g_cap, _ptr(self.tasks),
-                                            C.c_void_p(self._totals.data_ptr()), _ptr(self._ws), self._ws.numel(), 0,
-                                            stream))
-            self._event = torch.cuda.Event()
-            self._event.record(torch.cuda.current_stream(d))
+            self._enqueue([self])                    # the flag exists in the batch entry point only
+        else:
+            lib = _lib.load()
+            d = self.device
+            with torch.cuda.device(d):
+                stream = C.c_void_p(torch.cuda.current_stream(d).cuda_stream)
+                _lib.check(lib.sswin_token_plan(_ptr(self._indices), self.N, self.B, self.n, self.H, _ptr(self.tokens),
+                                                _ptr(self.plan), self.g_cap, _ptr(self.tasks),
+                                                C.c_void_p(self._totals.data_ptr()), _ptr(self._ws), self._ws.numel(),
+                                                0, stream))
+                self._event = torch.cuda.Event()
+                self._event.record(torch.cuda.current_stream(d))
         if not defer:
             self.finish()
 
@@ -114,16 +111,21 @@ class TokenPlan:
             p = cls.__new__(cls)
             p._allocate(*spec[:4], spec[4] if len(spec) > 4 else True, spec[5] if len(spec) > 5 else False)
             plans.append(p)
-        if not plans:
-            return plans
+        if plans:
+            cls._enqueue(plans)
+        return plans
+
+    @staticmethod
+    def _enqueue(plans):
+        """Launch allocated plans through the batch entry point, MAX_BATCH per call; they share one event."""
         d = plans[0].device
         if any(p.device != d for p in plans):
             raise RuntimeError("TokenPlan.batch: all index sets must live on one device")
         lib = _lib.load()
         with torch.cuda.device(d):
             stream = torch.cuda.current_stream(d)
-            for k in range(0, len(plans), cls.MAX_BATCH):
-                chunk = plans[k:k + cls.MAX_BATCH]
+            for k in range(0, len(plans), TokenPlan.MAX_BATCH):
+                chunk = plans[k:k + TokenPlan.MAX_BATCH]
                 descs = (_lib.TokenPlanDesc * len(chunk))()
                 for desc, p in zip(descs, chunk):
                     desc.indices, desc.N, desc.B, desc.n, desc.H = p._indices.data_ptr(), p.N, p.B, p.n, p.H
@@ -136,7 +138,6 @@ class TokenPlan:
             event.record(stream)
         for p in plans:
             p._event = event
-        return plans
 
     def finish(self):
         """Wait for the totals (once) and decode them."""
