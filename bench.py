@@ -724,10 +724,12 @@ def pmc_summary(dirs, out_name, workload, command, only=None):
 def trace_summary(dirs, out_name, command):
     """Turn the ``*kernel_stats.csv`` of ``rocprofv3 --kernel-trace --stats`` runs of this script (one directory
     per workload, named ..._<workload>) into the text summary ``profiles/<out_name>.txt``: time per step and
-    kernel.  The step count is read off the backward launch (one per attention call, two calls per step)."""
+    kernel.  The step count is read off the backward launch (one per attention call, two calls per step); a trace
+    without backward launches is the forward pass of the four-stage encoder (four forward launches per pass)."""
     import csv
     import glob
-    lines = ["rocprofv3 kernel traces of the benchmark step (step = regular + shifted block pair, forward + backward).",
+    lines = ["rocprofv3 kernel traces of the benchmark step (step = regular + shifted block pair, forward + backward; "
+             "cfg5: one forward pass of the four-stage encoder).",
              "Commands (from the repository root, TMPDIR=/tmp):"]
     lines += [f"  {c}" for c in command]
     lines.append("Durations in microseconds; kernels shorter than 1 us per step are left out of the tables.")
@@ -738,6 +740,8 @@ def trace_summary(dirs, out_name, command):
         rows = list(csv.DictReader(open(paths[0])))
         bwd = sum(int(r["Calls"]) for r in rows if "wattn_bwd_all_kernel" in r["Name"])
         steps = max(bwd // 2, 1)
+        if bwd == 0:                                 # the forward-only encoder: four attention launches per pass
+            steps = max(sum(int(r["Calls"]) for r in rows if "wattn_fwd_kernel" in r["Name"]) // 4, 1)
         tot = sum(float(r["TotalDurationNs"]) for r in rows)
         groups = {"library GEMMs (Cijk_*)": 0.0, "kernels of this library (sswin::*)": 0.0, "PyTorch element-wise / copies": 0.0}
         lines += ["", f"{os.path.basename(d.rstrip('/'))}: {steps} steps, GPU kernel time {tot / 1e3 / steps:.1f} us per step "
