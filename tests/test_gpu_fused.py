@@ -25,7 +25,7 @@ def _closed_form_plan(ind, n, H):
     return tokens, np.stack([g_c, g_T, g_sq, g_w, g_h]), int((counts.astype(np.int64) ** 2).sum()) * H, int(counts.max())
 
 
-@pytest.mark.parametrize("case", ["random", "ragged", "single", "big", "wide"])
+@pytest.mark.parametrize("case", ["random", "ragged", "single", "big", "wide", "wide125"])
 def test_token_plan_closed_forms(case):
     from sparseswin3d_amd.fused import TokenPlan
     rng = np.random.default_rng(len(case))
@@ -42,9 +42,12 @@ def test_token_plan_closed_forms(case):
     elif case == "big":
         B, n, H = 20000, 125, 3
         ind = random_window_indices(rng, B, n, 120000)
-    else:                            # enough window slots for the per-block phases to take blocks of 1 024 slots
+    elif case == "wide":             # enough window slots for the per-block phases to take four slots per thread
         B, n, H = 300000, 8, 1
         ind = random_window_indices(rng, B, n, 250000)
+    else:                            # the same with four bitmap words per slot and several heads
+        B, n, H = 70000, 125, 3
+        ind = random_window_indices(rng, B, n, 150000)
     tokens, plan, A, c_max = _closed_form_plan(ind, n, H)
     tp = TokenPlan(torch.from_numpy(ind).cuda(), B, n, H)
     assert (tp.G, tp.A, tp.c_max) == (plan.shape[1], A, c_max)
