@@ -75,3 +75,29 @@ def test_sparse_tensor_refuses_shapes_beyond_the_int32_hash():
         t.coalesce()
     with pytest.raises(RuntimeError, match="int32 hash"):
         t.permute((0, 2, 1, 3))
+
+
+def test_sparse_tensor_index_matrix_on_demand():
+    """A SparseTensor built around a producer of its index matrix calls it once, the first time ``indices`` is read;
+    tensors derived from it share the produced matrix; ``index_source`` hands the producer on without calling it."""
+    import torch
+    from sparseswin3d_amd.window_attention import SparseTensor, _LazyIndices
+    calls = []
+    matrix = torch.arange(12, dtype=torch.int32).reshape(4, 3)
+
+    def produce():
+        calls.append(1)
+        return matrix
+
+    t = SparseTensor(_LazyIndices(produce), torch.ones(3), [1, 1, 3, 3], group_counts=torch.tensor([3]),
+                     row_positions=torch.tensor([0, 1, 2]))
+    scaled = t * 2.0
+    assert not calls and isinstance(t.index_source(), _LazyIndices) and scaled.index_source() is t.index_source()
+    assert scaled.group_counts is t.group_counts and scaled.row_positions is t.row_positions
+    assert t.indices is matrix and calls == [1]
+    assert scaled.indices is matrix and t.indices is matrix and calls == [1]
+    assert t.index_source() is matrix
+    eager = SparseTensor(matrix, torch.ones(3), [1, 1, 3, 3])
+    assert eager.indices is matrix and eager.index_source() is matrix and eager.row_positions is None
+    eager.indices = matrix + 1
+    assert torch.equal(eager.indices, matrix + 1)
