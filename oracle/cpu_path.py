@@ -46,13 +46,21 @@ def window_order(win_idx: np.ndarray, n: int):
     return perm, wins, counts
 
 
+def _abs_score_grad_hook(probe, h, p):
+    def hook(g):
+        probe["abs_ds"][h].index_put_((p[:, None], p[None, :]), g.detach().abs().to(probe["abs_ds"].dtype), accumulate=True)
+    return hook
+
+
 def window_attention_cpu(features: torch.Tensor, win_idx: np.ndarray, n: int, num_heads: int,
                          qkv_w, qkv_b, proj_w, proj_b, rpb: torch.Tensor, mask: np.ndarray | None,
-                         softmax: str = "ops") -> torch.Tensor:
+                         softmax: str = "ops", probe: dict | None = None) -> torch.Tensor:
     """Forward of the attention module on the CPU; differentiable w.r.t. every tensor input.
 
     features [N, D]; win_idx int32 [N, 2] = (window, pos); rpb [H, n, n] (already gathered from
     the bias table); mask int8 [nW, n] region ids or None.  Returns [N, D] in input voxel order.
+    ``probe``: a dict with a zero tensor ``abs_ds`` [H, n, n]; the backward pass adds |d score| of every
+    attention entry to its (head, pos_i, pos_j) cell, which is the magnitude the bias gradient is a sum over.
     """
     N, D = features.shape
     H, hd = num_heads, D // num_heads
@@ -85,6 +93,8 @@ def window_attention_cpu(features: torch.Tensor, win_idx: np.ndarray, n: int, nu
             s = s + rpb[h].index_select(0, p).index_select(1, p)
             if mask_t is not None:
                 s = s + penalty
+            if probe is not None and s.requires_grad:
+                s.register_hook(_abs_score_grad_hook(probe, h, p))
             scores.append(s.reshape(-1))
             row_ids.append(torch.arange(row_base, row_base + c).repeat_interleave(c))
             row_base += c

@@ -34,3 +34,17 @@ def oracle():
     import oracle as orc
     orc.build()
     return orc
+
+
+def pytest_terminal_summary(terminalreporter):
+    """The values checks that came closest to their bound, and the largest relative errors seen."""
+    try:
+        from helpers import CHECK_LOG
+    except Exception:
+        return
+    if not CHECK_LOG:
+        return
+    tr = terminalreporter
+    tr.write_line(f"values checks: {len(CHECK_LOG)}; closest to their bound:")
+    for what, ratio, rel, rtol in sorted(CHECK_LOG, key=lambda r: -r[1])[:8]:
+        tr.write_line(f"  {what:<44s} |err|/bound {ratio:6.3f}   worst relative error {rel:.2e}   rtol {rtol:g}")

@@ -36,20 +36,80 @@ def qkv_operands(orc, ind, B, n, H, hd, rng, dtype=np.float32, scale=1.0):
                 sorted_qv=sqv, sorted_k=sk, idx_qv=iqv, idx_k=ik)
 
 
-def close(out, ref, rtol, what=""):
-    """|out - ref| <= rtol * (|ref| + max|ref|): relative to the element, with an absolute
-    floor tied to the array's scale so that cancellation near zero does not count."""
+# every values check of a session: (what, worst |err| / bound, worst pure relative error over the elements that carry
+# at least a thousandth of their own scale); conftest prints the tightest ones at the end of the run
+CHECK_LOG = []
+
+
+def close(out, ref, rtol, what="", mag=None, seg=None):
+    """Values check with a bound that follows the conditioning of each element:
+
+        |out - ref| <= rtol * scale_of_the_element
+
+    ``mag``  the element's condition magnitude, e.g. sum_k |a_ik * b_kj| for a product (computed by
+             running the same fp64 oracle on the absolute values of the operands): a result that has
+             lost a low-order term of its sum fails, cancellation inside the sum does not;
+    ``seg``  segment ids of a flat array (the softmax row of every entry): scale = |ref| + the largest
+             |ref| of the element's own segment;
+    neither: arrays with two or more axes use their rows (last axis) as segments: a token's own output
+             row, an output channel's own weight row.  A flat array needs ``mag`` or ``seg``
+             (``seg="all"`` = one segment, for small homogeneous vectors such as a bias gradient).
+    """
     out = np.asarray(out, dtype=np.float64)
     ref = np.asarray(ref, dtype=np.float64)
     assert out.shape == ref.shape, f"{what}: shape {out.shape} vs {ref.shape}"
     if ref.size == 0:
         return
-    scale = np.abs(ref).max()
+    aref = np.abs(ref)
+    if mag is not None:
+        scale = np.maximum(np.abs(np.asarray(mag, dtype=np.float64)).reshape(ref.shape), aref)
+    elif isinstance(seg, str):
+        assert seg == "all"
+        scale = aref + aref.max()
+    elif seg is not None:
+        seg = np.asarray(seg).reshape(-1)
+        top = np.zeros(int(seg.max()) + 1)
+        np.maximum.at(top, seg, aref.reshape(-1))
+        scale = aref + top[seg].reshape(ref.shape)
+    else:
+        assert ref.ndim >= 2, f"{what}: a flat array needs mag= or seg="
+        scale = aref + aref.max(axis=-1, keepdims=True)
     err = np.abs(out - ref)
-    bound = rtol * (np.abs(ref) + scale)
-    worst = np.argmax(err - bound)
-    assert (err <= bound).all(), (f"{what}: worst element {worst}: out={out.flat[worst]!r} "
-                                  f"ref={ref.flat[worst]!r} err={err.flat[worst]:.3e} bound={bound.flat[worst]:.3e}")
+    bound = rtol * scale
+    with np.errstate(divide="ignore", invalid="ignore"):
+        ratio = np.where(bound > 0, err / bound, np.where(err > 0, np.inf, 0.0))
+        carrying = aref >= 1e-3 * scale
+        rel = float((err[carrying] / aref[carrying]).max()) if carrying.any() else 0.0
+    worst = int(np.argmax(ratio))
+    CHECK_LOG.append((what, float(ratio.flat[worst]), rel, rtol))
+    print(f"[values] {what}: worst |err|/bound {ratio.flat[worst]:.3f}, worst relative error {rel:.2e} (rtol {rtol:g})")
+    assert ratio.flat[worst] <= 1.0, (f"{what}: worst element {worst}: out={out.flat[worst]!r} "
+                                      f"ref={ref.flat[worst]!r} err={err.flat[worst]:.3e} bound={bound.flat[worst]:.3e}")
+
+
+def product_mag(orc, fn, *args):
+    """The oracle's product ``fn`` on the absolute values of its floating-point operands: sum_k |a_ik| |b_kj| per
+    output element, the quantity a relative tolerance of a sum refers to."""
+    conv = [np.abs(a) if isinstance(a, np.ndarray) and a.dtype.kind == "f" else a for a in args]
+    res = getattr(orc, fn)(*conv)
+    return res[1] if isinstance(res, tuple) else res
+
+
+class BiasGradMagnitude:
+    """sum |dS| over the attention entries that share a row of the relative position bias table: the magnitude the
+    table gradient (a sum of dS over those entries) is conditioned by.  ``probe`` goes to the CPU path."""
+
+    def __init__(self, heads, n):
+        import torch
+        self.probe = {"abs_ds": torch.zeros(heads, n, n, dtype=torch.float64)}
+
+    def table(self, relative_position_index, table_rows):
+        import torch
+        a = self.probe["abs_ds"]
+        H, n, _ = a.shape
+        mag = torch.zeros(table_rows, H, dtype=torch.float64)
+        mag.index_add_(0, relative_position_index[:n, :n].reshape(-1).long().cpu(), a.permute(1, 2, 0).reshape(-1, H))
+        return mag.numpy()
 
 
 PATHS = ["resident", "fused", "operators"]

@@ -1,14 +1,16 @@
 """End-to-end parity of WindowAttentionSparse / SwinTransformerBlock / BasicLayer on the GPU
 against the PyTorch-CPU path (per-window torch.mm + scatter softmax + autograd).
 
-Tolerance: fp32 values and gradients within rel 1e-5 of the fp64 CPU path (helpers.close)."""
+Tolerance: fp32 values and gradients within rel 1e-5 of the fp64 CPU path, each element measured against its own
+value plus the largest value of its own row (a token's output row, an output channel's weight row), the bias table
+gradient against the sum of |dS| over the attention entries it sums (helpers.close)."""
 import copy
 
 import numpy as np
 import pytest
 import torch
 
-from helpers import PATHS, close, set_path
+from helpers import PATHS, BiasGradMagnitude, close, set_path
 
 pytestmark = pytest.mark.gpu
 
@@ -28,8 +30,10 @@ def _cpu_attention(attn, feats64, win_idx, n, mask, softmax="ops"):
     qkv_b = p.get("qkv.bias")
     table = leaves["relative_position_bias_table"]
     rpb = table[p["relative_position_index"][:n, :n].reshape(-1).long()].reshape(n, n, -1).permute(2, 0, 1)
+    mag = BiasGradMagnitude(attn.num_heads, n)
     out = cpu_path.window_attention_cpu(feats64, win_idx, n, attn.num_heads, leaves["qkv.weight"], qkv_b,
-                                        leaves["proj.weight"], leaves["proj.bias"], rpb, mask, softmax)
+                                        leaves["proj.weight"], leaves["proj.bias"], rpb, mask, softmax, probe=mag.probe)
+    leaves["table_mag"] = lambda: mag.table(p["relative_position_index"], table.shape[0])     # after backward
     return out, leaves
 
 
@@ -66,7 +70,7 @@ def test_window_attention_forward_backward(shift, dim, heads, path):
     close(attn.qkv.weight.grad.cpu().numpy(), leaves["qkv.weight"].grad.numpy(), 1e-5, "d qkv.weight")
     close(attn.proj.weight.grad.cpu().numpy(), leaves["proj.weight"].grad.numpy(), 1e-5, "d proj.weight")
     close(attn.relative_position_bias_table.grad.cpu().numpy(),
-          leaves["relative_position_bias_table"].grad.numpy(), 1e-5, "d bias table")
+          leaves["relative_position_bias_table"].grad.numpy(), 1e-5, "d bias table", mag=leaves["table_mag"]())
 
 
 def test_window_7_heads_of_16_channels_runs_the_operator_path():
@@ -97,7 +101,7 @@ def test_window_7_heads_of_16_channels_runs_the_operator_path():
     close(feats_gpu.grad.cpu().numpy(), f64.grad.numpy(), 1e-5, "d features")
     close(attn.qkv.weight.grad.cpu().numpy(), leaves["qkv.weight"].grad.numpy(), 1e-5, "d qkv.weight")
     close(attn.relative_position_bias_table.grad.cpu().numpy(),
-          leaves["relative_position_bias_table"].grad.numpy(), 1e-5, "d bias table")
+          leaves["relative_position_bias_table"].grad.numpy(), 1e-5, "d bias table", mag=leaves["table_mag"]())
 
 
 def test_window_attention_matches_dense_swin_on_full_windows():

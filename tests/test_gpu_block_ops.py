@@ -1,13 +1,14 @@
 """GPU parity of the window-blocked products, transposes and the sparse softmax against the
 CPU oracle.  Indices and offsets: bit-exact.  Values: fp32 within rel 1e-5 of the fp64 oracle,
-fp16/bf16 within rel 2e-2 (relative error measured as in helpers.close)."""
+fp16/bf16 within rel 2e-2; a product's error is measured against sum_k |a_ik b_kj| of its element, a softmax
+entry's against its own value plus the largest value of its row (helpers.close)."""
 import zlib
 
 import numpy as np
 import pytest
 import torch
 
-from helpers import close, qkv_operands, ragged_window_indices, random_window_indices
+from helpers import close, product_mag, qkv_operands, ragged_window_indices, random_window_indices
 
 pytestmark = pytest.mark.gpu
 
@@ -58,8 +59,9 @@ def run_forward(ops, oracle, d, dtype):
     # oracle consumes the same (rounded) inputs in fp64
     q64, kt64, v64 = host(q), host(kt), host(v)
     r_idx, r_val, r_shape, r_c = oracle.matmul_cuda_naive(q64, d["qi"], d["q_shape"], kt64, d["ki"], d["k_shape"], "q_k")
+    r_mag = product_mag(oracle, "matmul_cuda_naive", q64, d["qi"], d["q_shape"], kt64, d["ki"], d["k_shape"], "q_k")
     return dict(q=q, kt=kt, v=v, qi=qi, ki=ki, s_idx=s_idx, s_val=s_val, s_shape=s_shape, c1=c1,
-                q64=q64, kt64=kt64, v64=v64, r_idx=r_idx, r_val=r_val, r_shape=r_shape, r_c=r_c)
+                q64=q64, kt64=kt64, v64=v64, r_idx=r_idx, r_val=r_val, r_shape=r_shape, r_c=r_c, r_mag=r_mag)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.float16, torch.bfloat16])
@@ -73,7 +75,7 @@ def test_q_k_and_qk_v(ops, oracle, mix, H, hd, dtype):
     assert f["s_shape"] == f["r_shape"] == [B, H, n, n]
     np.testing.assert_array_equal(host(f["c1"]), f["r_c"])
     np.testing.assert_array_equal(host(f["s_idx"]), f["r_idx"])
-    close(host(f["s_val"]), f["r_val"], RTOL[dtype], "q_k values")
+    close(host(f["s_val"]), f["r_val"], RTOL[dtype], "q_k values", mag=f["r_mag"])
     # --- qk_v, fed with the oracle's attention so both sides multiply the same numbers
     rows = oracle.unique_consecutive_indices(oracle.flatten_indices(f["r_idx"][:3], f["r_shape"][:3]))
     p64 = oracle.softmax_last_dim_forward(rows, f["r_val"])
@@ -84,7 +86,8 @@ def test_q_k_and_qk_v(ops, oracle, mix, H, hd, dtype):
     assert o_shape == ro_shape == [B, H, n, hd]
     np.testing.assert_array_equal(host(c2), ro_c)
     np.testing.assert_array_equal(host(o_idx), ro_idx)
-    close(host(o_val), ro_val, RTOL[dtype], "qk_v values")
+    o_mag = product_mag(oracle, "matmul_cuda_naive", host(p), f["r_idx"], f["r_shape"], f["v64"], d["qi"], d["q_shape"], "qk_v")
+    close(host(o_val), ro_val, RTOL[dtype], "qk_v values", mag=o_mag)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16])
@@ -102,7 +105,7 @@ def test_matmul_grad(ops, oracle, mix, H, hd, kind, dtype):
     out = ops.matmul_grad_cuda_naive(m1, m2, dev(c), hd, kind)
     ref = oracle.matmul_grad_cuda_naive(host(m1), host(m2), c, hd, kind)
     assert out.dtype == dtype
-    close(host(out), ref, RTOL[dtype], kind)
+    close(host(out), ref, RTOL[dtype], kind, mag=product_mag(oracle, "matmul_grad_cuda_naive", host(m1), host(m2), c, hd, kind))
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.float16])
@@ -134,7 +137,7 @@ def test_backward_identities_through_transposes(ops, oracle):
     # plain algebra per group
     cs = f["r_c"]
     q64, kt64 = f["q64"], f["kt64"]
-    dq_ref, dkt_ref = [], []
+    dq_ref, dkt_ref, dq_mag, dkt_mag = [], [], [], []
     po = mo = 0
     for cg in cs:
         cg = int(cg)
@@ -143,10 +146,12 @@ def test_backward_identities_through_transposes(ops, oracle):
         dS = g_np[po:po + cg * cg].astype(np.float64).reshape(cg, cg)
         dq_ref.append((dS @ Kt.T).ravel())
         dkt_ref.append((Q.T @ dS).ravel())
+        dq_mag.append((np.abs(dS) @ np.abs(Kt.T)).ravel())
+        dkt_mag.append((np.abs(Q.T) @ np.abs(dS)).ravel())
         po += cg * cg
         mo += cg * C_
-    close(host(dq), np.concatenate(dq_ref), 1e-5, "dQ")
-    close(host(dkt), np.concatenate(dkt_ref), 1e-5, "dK^T")
+    close(host(dq), np.concatenate(dq_ref), 1e-5, "dQ", mag=np.concatenate(dq_mag))
+    close(host(dkt), np.concatenate(dkt_ref), 1e-5, "dK^T", mag=np.concatenate(dkt_mag))
 
 
 # ------------------------------------------------------------------------------------------ softmax
@@ -172,11 +177,11 @@ def test_softmax_forward_backward(ops, oracle, mix, dtype):
     v64 = host(dev(v, dtype))
     y = ops.softmax_last_dim_forward(dev(rows), dev(v, dtype))
     y_ref = oracle.softmax_last_dim_forward(rows, v64)
-    close(host(y), y_ref, RTOL[dtype] if dtype == torch.float64 else 1e-5, "softmax fwd")
+    close(host(y), y_ref, RTOL[dtype] if dtype == torch.float64 else 1e-5, "softmax fwd", seg=rows)
     g = rng.standard_normal(len(rows))
     gx = ops.softmax_last_dim_backward(dev(rows), y, dev(g, dtype))
     gx_ref = oracle.softmax_last_dim_backward(rows, host(y), host(dev(g, dtype)))
-    close(host(gx), gx_ref, RTOL[dtype] if dtype == torch.float64 else 1e-5, "softmax bwd")
+    close(host(gx), gx_ref, RTOL[dtype] if dtype == torch.float64 else 1e-5, "softmax bwd", seg=rows)
 
 
 def test_softmax_all_negative_rows_keep_zero_max(ops, oracle):
@@ -185,7 +190,7 @@ def test_softmax_all_negative_rows_keep_zero_max(ops, oracle):
     v = np.array([-1, -2, -3, -4, -30, -31, -32, -33, -5], np.float32)
     y = ops.softmax_last_dim_forward(dev(rows), dev(v)).cpu().numpy().astype(np.float64)
     ref = oracle.softmax_last_dim_forward(rows, v.astype(np.float64))
-    close(y, ref, 1e-5, "negative rows")
+    close(y, ref, 1e-5, "negative rows", seg=rows)
     assert abs(y[4:8].sum() - 1.0) > 1e-6          # the 1e-8 term is visible for exp(-30)-sized sums
 
 
@@ -196,10 +201,10 @@ def test_softmax_views_inside_an_allocation(ops, oracle):
     v = rng.standard_normal(len(rows) + 1).astype(np.float32)
     rows_d = dev(np.concatenate([[0], rows]).astype(np.int32))[1:]
     y = ops.softmax_last_dim_forward(rows_d, dev(v)[1:])
-    close(host(y), oracle.softmax_last_dim_forward(rows, v[1:].astype(np.float64)), 1e-5, "views fwd")
+    close(host(y), oracle.softmax_last_dim_forward(rows, v[1:].astype(np.float64)), 1e-5, "views fwd", seg=rows)
     g = rng.standard_normal(len(rows) + 1).astype(np.float32)
     gx = ops.softmax_last_dim_backward(rows_d, y, dev(g)[1:])
-    close(host(gx), oracle.softmax_last_dim_backward(rows, host(y), g[1:].astype(np.float64)), 1e-5, "views bwd")
+    close(host(gx), oracle.softmax_last_dim_backward(rows, host(y), g[1:].astype(np.float64)), 1e-5, "views bwd", seg=rows)
 
 
 def test_softmax_deterministic(ops):

@@ -8,12 +8,14 @@ Two kinds of check per configuration:
     plus size-independent properties (row sums of the attention, linearity of the backward in
     the upstream gradient, invariance to the order of the voxels).
 
-Tolerances: fp32 rel 1e-5, bf16 rel 2e-2 (helpers.close)."""
+Tolerances: fp32 rel 1e-5, bf16 rel 2e-2, measured per element against its condition magnitude: sum_k |a_ik b_kj|
+for products, the element's own softmax row, a token's own row of the module outputs, sum |dS| for the bias table
+gradient (helpers.close)."""
 import numpy as np
 import pytest
 import torch
 
-from helpers import PATHS, close, qkv_operands, set_path
+from helpers import PATHS, BiasGradMagnitude, close, product_mag, qkv_operands, set_path
 
 pytestmark = pytest.mark.gpu
 
@@ -78,7 +80,8 @@ def test_operator_chain_full_size(ops, oracle, cfg, shift, dtype):
     assert s_shape == r_shape
     np.testing.assert_array_equal(host(c), r_c)
     np.testing.assert_array_equal(host(s_idx), r_idx)
-    close(host(s_val), r_val, rtol, "q_k values")
+    close(host(s_val), r_val, rtol, "q_k values",
+          mag=product_mag(oracle, "matmul_cuda_naive", q64, d["qi"], d["q_shape"], kt64, d["ki"], d["k_shape"], "q_k"))
 
     # I2 + I4: softmax row ids
     rows = ops.unique_consecutive_indices(ops.flatten_indices(s_idx[:3].contiguous(), s_shape[:3]))
@@ -89,7 +92,7 @@ def test_operator_chain_full_size(ops, oracle, cfg, shift, dtype):
     s32 = dev(r_val, torch.float32)
     p = ops.softmax_last_dim_forward(rows, s32)
     r_p = oracle.softmax_last_dim_forward(r_rows, host(s32))
-    close(host(p), r_p, 1e-5, "softmax forward")
+    close(host(p), r_p, 1e-5, "softmax forward", seg=r_rows)
     # every attention row sums to se / (se + 1e-8), se = sum of exp(v - max(0, rowmax)): 1 up to 1e-8 unless a
     # whole row is far below zero (a window of one token with a negative score)
     sums = np.bincount(r_rows, weights=host(p))
@@ -100,7 +103,7 @@ def test_operator_chain_full_size(ops, oracle, cfg, shift, dtype):
     assert np.all(np.abs(sums[row_max >= 0] - 1.0) < 1e-5)
     gp = dev(rng.standard_normal(len(r_val)), torch.float32)
     gs = ops.softmax_last_dim_backward(rows, p, gp)
-    close(host(gs), oracle.softmax_last_dim_backward(r_rows, host(p), host(gp)), 1e-5, "softmax backward")
+    close(host(gs), oracle.softmax_last_dim_backward(r_rows, host(p), host(gp)), 1e-5, "softmax backward", seg=r_rows)
     zero = np.bincount(r_rows, weights=host(gs))
     assert np.all(np.abs(zero) < 1e-4 * max(1.0, np.abs(host(gs)).max()))   # softmax gradient rows sum to 0
 
@@ -111,14 +114,16 @@ def test_operator_chain_full_size(ops, oracle, cfg, shift, dtype):
     assert o_shape == ro_shape
     np.testing.assert_array_equal(host(c2), ro_c)
     np.testing.assert_array_equal(host(o_idx), ro_idx)
-    close(host(o_val), ro_val, rtol, "qk_v values")
+    close(host(o_val), ro_val, rtol, "qk_v values",
+          mag=product_mag(oracle, "matmul_cuda_naive", host(pd), r_idx, r_shape, v64, d["qi"], d["q_shape"], "qk_v"))
     del o_idx, ro_idx, s_idx, r_idx
 
     # M3 / M4: the three gradient products and the two transposes
     go = dev(rng.standard_normal(len(ro_val)), dtype)
     for kind, a, b in (("rc_cr", go, kt), ("rr_rc", pd, go), ("cr_rr", kt, pd)):
         out = ops.matmul_grad_cuda_naive(a, b, c, hd, kind)
-        close(host(out), oracle.matmul_grad_cuda_naive(host(a), host(b), r_c, hd, kind), rtol, kind)
+        close(host(out), oracle.matmul_grad_cuda_naive(host(a), host(b), r_c, hd, kind), rtol, kind,
+              mag=product_mag(oracle, "matmul_grad_cuda_naive", host(a), host(b), r_c, hd, kind))
     np.testing.assert_array_equal(host(ops.qkv_transpose(v, c, hd, "rc")), oracle.qkv_transpose(v64, r_c, hd, "rc"))
     np.testing.assert_array_equal(host(ops.qkv_transpose(pd, c, hd, "rr")), oracle.qkv_transpose(host(pd), r_c, hd, "rr"))
 
@@ -154,8 +159,10 @@ def _cpu(attn, feats64, idx, n, mask):
               ("qkv.weight", "qkv.bias", "proj.weight", "proj.bias", "relative_position_bias_table")}
     table = leaves["relative_position_bias_table"]
     rpb = table[p["relative_position_index"][:n, :n].reshape(-1).long()].reshape(n, n, -1).permute(2, 0, 1)
+    mag = BiasGradMagnitude(attn.num_heads, n)
     out = cpu_path.window_attention_cpu(feats64, idx, n, attn.num_heads, leaves["qkv.weight"], leaves["qkv.bias"],
-                                        leaves["proj.weight"], leaves["proj.bias"], rpb, mask, "ops")
+                                        leaves["proj.weight"], leaves["proj.bias"], rpb, mask, "ops", probe=mag.probe)
+    leaves["table_mag"] = lambda: mag.table(p["relative_position_index"], table.shape[0])     # after backward
     return out, leaves
 
 
@@ -204,10 +211,10 @@ def test_shifted_forward_backward_against_cpu_path(cfg, path):
     close(host(out), ref.detach().numpy(), 1e-5, "forward")
     close(host(gf), f64.grad.numpy(), 1e-5, "d features")
     close(host(attn.qkv.weight.grad), leaves["qkv.weight"].grad.numpy(), 1e-5, "d qkv.weight")
-    close(host(attn.qkv.bias.grad), leaves["qkv.bias"].grad.numpy(), 1e-5, "d qkv.bias")
+    close(host(attn.qkv.bias.grad), leaves["qkv.bias"].grad.numpy(), 1e-5, "d qkv.bias", seg="all")
     close(host(attn.proj.weight.grad), leaves["proj.weight"].grad.numpy(), 1e-5, "d proj.weight")
     close(host(attn.relative_position_bias_table.grad), leaves["relative_position_bias_table"].grad.numpy(), 1e-5,
-          "d bias table")
+          "d bias table", mag=leaves["table_mag"]())
 
 
 @pytest.mark.parametrize("path", PATHS)
@@ -227,7 +234,7 @@ def test_cfg4_bf16_dense_windows_against_cpu_fp64(path):
     close(host(out), ref.detach().numpy(), 2e-2, "forward")
     close(host(gf), f64.grad.numpy(), 2e-2, "d features")
     close(host(attn.relative_position_bias_table.grad), leaves["relative_position_bias_table"].grad.numpy(), 2e-2,
-          "d bias table")
+          "d bias table", mag=leaves["table_mag"]())
 
 
 def test_cfg5_four_stage_encoder_bf16_forward():

@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import close, qkv_operands, ragged_window_indices
+from helpers import close, product_mag, qkv_operands, ragged_window_indices
 
 pytestmark = pytest.mark.gpu
 
@@ -83,7 +83,8 @@ def test_products_softmax_gradients_transposes(mods, oracle, case):
     assert list(s_shape) == r_shape
     np.testing.assert_array_equal(host(s_idx), r_idx)
     np.testing.assert_array_equal(host(c), r_c)
-    close(host(s_val), r_val, 1e-5, "q_k")
+    close(host(s_val), r_val, 1e-5, "q_k",
+          mag=product_mag(oracle, "matmul_cuda_naive", host(q), d["qi"], d["q_shape"], host(kt), d["ki"], d["k_shape"], "q_k"))
     c_idx, c_val, _, c_c = ct.matmul_cuda_naive(q, qi, d["q_shape"], kt, ki, d["k_shape"], "q_k")
     same(s_idx, c_idx), same(s_val, c_val), same(c, c_c)
 
@@ -91,11 +92,11 @@ def test_products_softmax_gradients_transposes(mods, oracle, case):
     r_rows = oracle.unique_consecutive_indices(oracle.flatten_indices(r_idx[:3], r_shape[:3]))
     np.testing.assert_array_equal(host(rows), r_rows)
     p = pb.softmax_last_dim_forward(rows, s_val)
-    close(host(p), oracle.softmax_last_dim_forward(r_rows, host(s_val)), 1e-5, "softmax forward")
+    close(host(p), oracle.softmax_last_dim_forward(r_rows, host(s_val)), 1e-5, "softmax forward", seg=r_rows)
     same(p, ct.softmax_last_dim_forward(rows, s_val))
     gp = dev(np.random.default_rng(5).standard_normal(p.numel()), torch.float32)
     gs = pb.softmax_last_dim_backward(rows, p, gp)
-    close(host(gs), oracle.softmax_last_dim_backward(r_rows, host(p), host(gp)), 1e-5, "softmax backward")
+    close(host(gs), oracle.softmax_last_dim_backward(r_rows, host(p), host(gp)), 1e-5, "softmax backward", seg=r_rows)
     same(gs, ct.softmax_last_dim_backward(rows, p, gp))
 
     o_idx, o_val, o_shape, c2 = pb.matmul_cuda_naive(p, s_idx, list(s_shape), v, qi, d["q_shape"], "qk_v")
@@ -103,12 +104,14 @@ def test_products_softmax_gradients_transposes(mods, oracle, case):
     assert list(o_shape) == ro_shape
     np.testing.assert_array_equal(host(o_idx), ro_idx)
     np.testing.assert_array_equal(host(c2), ro_c)
-    close(host(o_val), ro_val, 1e-5, "qk_v")
+    close(host(o_val), ro_val, 1e-5, "qk_v",
+          mag=product_mag(oracle, "matmul_cuda_naive", host(p), r_idx, r_shape, host(v), d["qi"], d["q_shape"], "qk_v"))
 
     g_o = dev(np.random.default_rng(6).standard_normal(o_val.numel()), torch.float32)
     for kind, a, b in (("rc_cr", g_o, v), ("rr_rc", gs, kt), ("cr_rr", q, gs)):
         out = pb.matmul_grad_cuda_naive(a, b, c, HD, kind)
-        close(host(out), oracle.matmul_grad_cuda_naive(host(a), host(b), r_c, HD, kind), 1e-5, kind)
+        close(host(out), oracle.matmul_grad_cuda_naive(host(a), host(b), r_c, HD, kind), 1e-5, kind,
+              mag=product_mag(oracle, "matmul_grad_cuda_naive", host(a), host(b), r_c, HD, kind))
         same(out, ct.matmul_grad_cuda_naive(a, b, c, HD, kind))
     for kind, a in (("rc", v), ("rr", p)):
         out = pb.qkv_transpose(a, c, HD, kind)
