@@ -356,7 +356,7 @@ def kernel_table(wl, reps=20, only=None):
             ("sorted_coo_indices [4,E] x 2 (with K^T's)", lambda: ops.sorted_coo_indices(b["idx"], omap, H, hd), 32 * E + 20 * N, 0),
             ("operand_copy Q/V order", lambda: ops.operand_copy(qkv_rows, 2 * D, val_e, omap, H, hd, 0, True), 2 * s * E, 6),
             ("operand_copy K^T order", lambda: ops.operand_copy(qkv_rows, D, val_e, omap, H, hd, 1, True), 2 * s * E, 2),
-            ("qkv_sparse_indices (reference operator)", lambda: ops.qkv_sparse_indices(b["idx"], b["slots"], b["n"], H, hd, _defer_check=True), 8 * N + 40 * E, 0),
+            ("qkv_sparse_indices (reference operator)", lambda: ops.qkv_sparse_indices(b["idx"], b["slots"], b["n"], H, hd), 8 * N + 40 * E, 0),
             ("plan_from_indices (group table from a [4,E] index matrix)", lambda: _lib.check(lib.sswin_plan_from_indices(ptr(q.indices), m, hd, ptr(plan), g_cap, totals, ptr(ws), nb, stream)), 0, 0),
             ("block_matmul q_k, values", mm(0, q.values, kt.values, q.indices, out_s, None, A), 2 * s * E + s * A + 4 * G, 1),
             ("block_matmul q_k (values + index matrix)", mm(0, q.values, kt.values, q.indices, out_s, out_si, A), 2 * s * E + (s + 16) * A + 4 * G, 0),

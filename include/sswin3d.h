@@ -264,9 +264,13 @@ int sswin_softmax_last_dim_backward(const int32_t* idx_row, const void* y, const
  *   window; pos; window.
  * plan (device int32 [5*g_cap]): rows c, T (rank of the window's first token), sq_start
  *   (exclusive scan of c*c over groups), window, head — groups ordered (window, head).
- * tasks (device int32 [4][g_cap][4], or NULL): group descriptors {T, c | head << 8, window,
- *   sq_start} bucketed by ceil(c/32) = 1..4 for sswin_window_attention_*; the order of the
- *   descriptors inside a bucket is unspecified.
+ * tasks (device int32, sswin_token_plan_task_ints(N, g_cap, H) entries, or NULL): group descriptors
+ *   [4][g_cap][4] {T, c | head << 8, window, sq_start} bucketed by ceil(c/32) = 1..4 for
+ *   sswin_window_attention_* (a window's H descriptors side by side, windows of a bucket in window
+ *   order), followed by the token records [N/32 + g_cap/H + 4][32][2]: one record {voxel, pos} x 32 per
+ *   (window, tile of 32 tokens), bucket of four tiles first, inside a bucket by window, then tile;
+ *   entries behind a window's last token repeat it.  A task of the attention kernels finds its
+ *   descriptor and its tokens from its own number alone (one memory round trip instead of two).
  * totals_out (host, 9 x int64): {groups G, non-empty windows, sum over groups of c*c, max c,
  *   groups in bucket 1..4, groups with c > 128 (no descriptor)}; the last five are 0 without tasks.
  * (window, pos) pairs must be distinct, window in [0,B), pos in [0,n): indices outside that range
@@ -277,6 +281,7 @@ int sswin_softmax_last_dim_backward(const int32_t* idx_row, const void* y, const
  * has waited for the stream, sswin_token_plan_totals(totals_out, H, g_cap) decodes them in place
  * and performs the checks (range, distinctness, capacity). */
 size_t sswin_token_plan_workspace_bytes(int64_t N, int B, int n);
+size_t sswin_token_plan_task_ints(int64_t N, int64_t g_cap, int H);
 int sswin_token_plan(const int32_t* indices, int64_t N, int B, int n, int H, int32_t* tokens,
                      int32_t* plan, int64_t g_cap, int32_t* tasks, int64_t* totals_out, void* ws,
                      size_t ws_bytes, int synchronize, void* stream);

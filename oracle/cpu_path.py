@@ -46,12 +46,6 @@ def window_order(win_idx: np.ndarray, n: int):
     return perm, wins, counts
 
 
-def _abs_score_grad_hook(probe, h, p):
-    def hook(g):
-        probe["abs_ds"][h].index_put_((p[:, None], p[None, :]), g.detach().abs().to(probe["abs_ds"].dtype), accumulate=True)
-    return hook
-
-
 def window_attention_cpu(features: torch.Tensor, win_idx: np.ndarray, n: int, num_heads: int,
                          qkv_w, qkv_b, proj_w, proj_b, rpb: torch.Tensor, mask: np.ndarray | None,
                          softmax: str = "ops", probe: dict | None = None) -> torch.Tensor:
@@ -59,8 +53,10 @@ def window_attention_cpu(features: torch.Tensor, win_idx: np.ndarray, n: int, nu
 
     features [N, D]; win_idx int32 [N, 2] = (window, pos); rpb [H, n, n] (already gathered from
     the bias table); mask int8 [nW, n] region ids or None.  Returns [N, D] in input voxel order.
-    ``probe``: a dict with a zero tensor ``abs_ds`` [H, n, n]; the backward pass adds |d score| of every
-    attention entry to its (head, pos_i, pos_j) cell, which is the magnitude the bias gradient is a sum over.
+    ``probe``: an empty dict; it receives what the conditioning of the score gradient dS = P (dP - D),
+    dP = dO V^T, D = dO . O, is made of: ``P`` (the attention values), ``cells`` (index (head, pos_i, pos_j) of every
+    entry in an [H, n, n] array), ``sizes`` (tokens per window), ``V`` and ``O`` in window order and, during the
+    backward pass, ``dO`` (the gradient that reaches O).
     """
     N, D = features.shape
     H, hd = num_heads, D // num_heads
@@ -79,7 +75,7 @@ def window_attention_cpu(features: torch.Tensor, win_idx: np.ndarray, n: int, nu
     sizes = [int(c) for c in counts]
     q_w, k_w, v_w = q.split(sizes), k.split(sizes), v.split(sizes)
 
-    scores, row_ids = [], []
+    scores, row_ids, cells = [], [], []
     start = 0
     row_base = 0
     for k_win, (w, c) in enumerate(zip(wins, counts)):
@@ -93,8 +89,8 @@ def window_attention_cpu(features: torch.Tensor, win_idx: np.ndarray, n: int, nu
             s = s + rpb[h].index_select(0, p).index_select(1, p)
             if mask_t is not None:
                 s = s + penalty
-            if probe is not None and s.requires_grad:
-                s.register_hook(_abs_score_grad_hook(probe, h, p))
+            if probe is not None:
+                cells.append(((h * n + p[:, None]) * n + p[None, :]).reshape(-1))
             scores.append(s.reshape(-1))
             row_ids.append(torch.arange(row_base, row_base + c).repeat_interleave(c))
             row_base += c
@@ -103,6 +99,8 @@ def window_attention_cpu(features: torch.Tensor, win_idx: np.ndarray, n: int, nu
     idx_row = torch.cat(row_ids)
     sm = sparse_softmax_ops if softmax == "ops" else sparse_softmax_readme
     attn = sm(vals, idx_row, row_base)
+    if probe is not None:
+        probe.update(P=attn.detach(), cells=torch.cat(cells), sizes=sizes, V=v.detach())
 
     outs = []
     blocks = attn.split([c * c for c in sizes for _ in range(H)])
@@ -110,6 +108,10 @@ def window_attention_cpu(features: torch.Tensor, win_idx: np.ndarray, n: int, nu
         per_head = [torch.mm(blocks[k_win * H + h].reshape(c, c), v_w[k_win][:, h]) for h in range(H)]
         outs.append(torch.stack(per_head, 1).reshape(c, D))      # (token, head, channel)
     out_sorted = torch.cat(outs, 0)
+    if probe is not None:
+        probe["O"] = out_sorted.detach()
+        if out_sorted.requires_grad:
+            out_sorted.register_hook(lambda g: probe.__setitem__("dO", g.detach()))
     inv = np.empty_like(perm)
     inv[perm] = np.arange(N)
     out = out_sorted.index_select(0, torch.from_numpy(inv))

@@ -54,6 +54,7 @@ SIGNATURES = {
     "sswin_block_transpose": (_i32, [_i32, _i32, _vp, _vp, _vp, _i64, _i32, _vp, _vp]),
     "sswin_softmax_last_dim_forward": (_i32, [_vp, _vp, _i32, _i64, _vp, _vp]),
     "sswin_softmax_last_dim_backward": (_i32, [_vp, _vp, _vp, _i32, _i64, _vp, _vp]),
+    "sswin_token_plan_task_ints": (_sz, [_i64, _i64, _i32]),
     "sswin_token_plan_workspace_bytes": (_sz, [_i64, _i32, _i32]),
     "sswin_token_plan": (_i32, [_vp, _i64, _i32, _i32, _i32, _vp, _vp, _i64, _vp, _vp, _vp, _sz, _i32, _vp]),
     "sswin_token_plan_totals": (_i32, [_vp, _i32, _i64]),
@@ -88,7 +89,7 @@ SIGNATURES = {
                                                _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i32, _vp]),
 }
 
-ABI_VERSION = 25
+ABI_VERSION = 26
 _lib = None
 
 

@@ -15,7 +15,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 OUT = os.path.join(HERE, "libsswin3d.so")
 SOURCES = ["index_ops.hip", "plan.hip", "block_matmul.hip", "softmax.hip", "fused_attention.hip",
-           "window_attention.hip", "column_sum.hip", "voxel_grid.hip", "tall_linear.hip"]
+           "window_attention.hip", "window_attention_x16.hip", "column_sum.hip", "voxel_grid.hip", "tall_linear.hip"]
 ARCH = "gfx950"
 # packed FP32 instructions are switched off for all device code on purpose
 FLAGS = ["-O3", "-std=c++17", "-fPIC", f"--offload-arch={ARCH}",

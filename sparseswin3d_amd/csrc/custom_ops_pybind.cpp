@@ -269,23 +269,27 @@ at::Tensor unique_consecutive_indices(const at::Tensor& nums) {
 }
 
 namespace {
+bool is_16bit(const at::Tensor& t) { return t.scalar_type() == at::kHalf || t.scalar_type() == at::kBFloat16; }
 void check_softmax(const at::Tensor& indices, const at::Tensor& values, const char* who) {
     TORCH_CHECK(indices.scalar_type() == at::kInt, who, ": row ids must be int32");
-    TORCH_CHECK(values.scalar_type() == at::kFloat || values.scalar_type() == at::kDouble, who, ": values must be fp32 or fp64");
+    TORCH_CHECK(values.scalar_type() == at::kFloat || values.scalar_type() == at::kDouble || is_16bit(values), who,
+                ": values must be fp32, fp64, fp16 or bf16");
     TORCH_CHECK(indices.numel() == values.numel(), who, ": ", indices.numel(), " row ids for ", values.numel(), " values");
     on_gpu(values, who);
 }
 }  // namespace
 
-// ops.h:43-45, ops.cu:128-167
+// ops.h:43-45, ops.cu:128-167.  16-bit values (the reference dispatches AT_DISPATCH_FLOATING_TYPES_AND_HALF, ops.cu:140)
+// are computed in fp32 and rounded once at the end.
 at::Tensor softmax_last_dim_forward(const at::Tensor& indices, const at::Tensor& values) {
     check_softmax(indices, values, "softmax_last_dim_forward");
     c10::hip::HIPGuardMasqueradingAsCUDA guard(values.device());
-    const at::Tensor rows = indices.contiguous(), v = values.contiguous();
+    const at::Tensor rows = indices.contiguous();
+    const at::Tensor v = is_16bit(values) ? values.to(at::kFloat).contiguous() : values.contiguous();
     at::Tensor out = at::empty_like(v);
     SSWIN_OK(sswin_softmax_last_dim_forward(rows.data_ptr<int32_t>(), v.data_ptr(), value_code(v), v.numel(), out.data_ptr(),
                                             current_stream(v)));
-    return out;
+    return is_16bit(values) ? out.to(values.scalar_type()) : out;
 }
 
 // ops.h:47-50, ops.cu:169-194
@@ -294,22 +298,32 @@ at::Tensor softmax_last_dim_backward(const at::Tensor& indices, const at::Tensor
     TORCH_CHECK(grad_values.scalar_type() == values.scalar_type() && grad_values.numel() == values.numel(),
                 "softmax_last_dim_backward: gradient and output differ in dtype or size");
     c10::hip::HIPGuardMasqueradingAsCUDA guard(values.device());
-    const at::Tensor rows = indices.contiguous(), y = values.contiguous(), g = grad_values.contiguous();
+    const bool narrow = is_16bit(values);
+    const at::Tensor rows = indices.contiguous();
+    const at::Tensor y = narrow ? values.to(at::kFloat).contiguous() : values.contiguous();
+    const at::Tensor g = narrow ? grad_values.to(at::kFloat).contiguous() : grad_values.contiguous();
     at::Tensor out = at::empty_like(y);
     SSWIN_OK(sswin_softmax_last_dim_backward(rows.data_ptr<int32_t>(), y.data_ptr(), g.data_ptr(), value_code(y), y.numel(),
                                              out.data_ptr(), current_stream(y)));
-    return out;
+    return narrow ? out.to(values.scalar_type()) : out;
 }
 
+// the ten names of the reference's module (ops.cpp:7-18), positional arguments as in ops.h
 PYBIND11_MODULE(TORCH_EXTENSION_NAME, m) {
-    m.def("matmul_cuda_naive", &matmul_cuda_naive, "Compute matmul");
-    m.def("matmul_grad_cuda_naive", &matmul_grad_cuda_naive, "Compute grad matmul");
-    m.def("qkv_sparse_indices", &qkv_sparse_indices, "Compute indices");
-    m.def("flatten_indices", &flatten_indices_impl, "Flatten indices");
-    m.def("sort_indices", &sort_indices_impl, "Sort indices");
-    m.def("return_inverse", &return_inverse_impl, "Return indices based on unique");
-    m.def("unique_consecutive_indices", &unique_consecutive_indices, "Return indices for unique_consecutive");
-    m.def("softmax_last_dim_forward", &softmax_last_dim_forward, "Softmax Forward");
-    m.def("softmax_last_dim_backward", &softmax_last_dim_backward, "Softmax Backward");
-    m.def("qkv_transpose", &qkv_transpose, "Custom Trasnpose for qkv");
+    m.def("matmul_cuda_naive", &matmul_cuda_naive,
+          "(mat1_v, mat1_idx, mat1_shape, mat2_v, mat2_idx, mat2_shape, mul_type 'q_k'|'qk_v') -> (idx, val, shape, group sizes): "
+          "window-blocked COO product on the matrix cores");
+    m.def("matmul_grad_cuda_naive", &matmul_grad_cuda_naive,
+          "(mat1_v, mat2_v, group sizes, C, mul_type 'rc_cr'|'rr_rc'|'cr_rr') -> values of the gradient product");
+    m.def("qkv_sparse_indices", &qkv_sparse_indices,
+          "(indices [N,2], batch_size, spatial_dim, num_heads, c) -> (Q/V index matrix, its sort order, K^T index matrix, its "
+          "sort order), from a presence bitmap instead of a sort");
+    m.def("flatten_indices", &flatten_indices_impl, "(indices [ndim,M], sizes) -> row-major int32 key per column");
+    m.def("sort_indices", &sort_indices_impl, "(keys) -> stable ascending argsort, int32");
+    m.def("return_inverse", &return_inverse_impl, "(keys, maxnum) -> (rank of every key among the distinct keys, their number)");
+    m.def("unique_consecutive_indices", &unique_consecutive_indices, "(keys) -> 0-based rank of the run each key belongs to");
+    m.def("softmax_last_dim_forward", &softmax_last_dim_forward,
+          "(row ids, values) -> exp(v - max(0, rowmax)) / (rowsum + 1e-8) per row");
+    m.def("softmax_last_dim_backward", &softmax_last_dim_backward, "(row ids, softmax output, gradient) -> y (g - sum_row g y)");
+    m.def("qkv_transpose", &qkv_transpose, "(values, group sizes, C, 'rc'|'rr') -> every group's block transposed");
 }

@@ -63,6 +63,9 @@ struct TokenPlanArgs {
     int32_t* plan;
     int64_t g_cap;
     int4* tasks;
+    int2* recs;              // token records behind the descriptors (or null): [rec_cap][32] {voxel, pos}
+    int64_t rec_cap;
+    int32_t* win_rec;        // [B] bucket << 28 | rank of the window inside its bucket, -1 without records
     int32_t* tokens;         // [5 * N]
     int blocks;              // ceil(B / window slots per block) of the launch the plan goes into
     int order_only;          // tokens holds its first row only (voxel of rank r)
@@ -248,13 +251,17 @@ __device__ __forceinline__ void tp_phase_windows(const TokenPlanArgs& a, int blk
             }
         }
         const int b = tp_bucket(cu);
+        int32_t wrec = -1;
         if (a.tasks != nullptr && live && b < 4) {
             const int64_t slot = tp_bucket_count(e, b) * H;
-            if (slot + H <= g_cap)
+            if (slot + H <= g_cap) {
                 for (int h = 0; h < H; ++h)
                     a.tasks[(int64_t)b * g_cap + slot + h] =
                         make_int4(T, (int)cu | (h << 8), (int)w, (int32_t)(q2 * H + (int64_t)h * cu * cu));
+                wrec = (int32_t)((b << 28) | (int32_t)tp_bucket_count(e, b));
+            }
         }
+        if (a.recs != nullptr && w < a.B) a.win_rec[w] = wrec;
         if (ITEMS > 1) {                                         // on to the thread's next slot
             int64_t item[TP_SUMS];
             tp_items(cu, item);
@@ -305,6 +312,26 @@ __device__ __forceinline__ void tp_phase_rank(const TokenPlanArgs& a, int64_t gt
             tok_c[r] = c;
             tok_pos[r] = wp.y;
             tok_win[r] = wp.x;
+        }
+        if (a.recs != nullptr) {
+            // Token records of the window-resident kernels: one record of 32 {voxel, pos} entries per (window, tile
+            // of 32 tokens), at the position of the tile's task inside its bucket, so that a task finds its tokens
+            // from its own number, in the same round trip as its group descriptor.  The entries behind the last
+            // token of a window repeat that token (what the kernels feed their padding rows with).
+            const int32_t wr = a.win_rec[wp.x];
+            if (wr >= 0) {
+                const int b = wr >> 28, nt = b + 1;
+                const int32_t* counters = tp_counters(a);
+                int64_t first = 0;                               // records of the buckets of more tiles come first
+                for (int bb = 3; bb > b; --bb) first += (int64_t)(counters[bb] / a.H) * (bb + 1);
+                const int64_t rec = first + (int64_t)(wr & 0x0fffffff) * nt + (below >> 5);
+                if (rec < a.rec_cap && below < c) {
+                    const int2 entry = make_int2((int)v, wp.y);
+                    a.recs[rec * 32 + (below & 31)] = entry;
+                    if (below == c - 1)
+                        for (int k = (below & 31) + 1; k < 32; ++k) a.recs[rec * 32 + k] = entry;
+                }
+            }
         }
     }
 }
@@ -969,8 +996,15 @@ size_t sswin_token_plan_workspace_bytes(int64_t N, int B, int n) {
     (void)N;
     const size_t words = (size_t)B * tp_words_per_window(n);
     const size_t blocks = (size_t)tp_blocks(B);
-    return align_up(words * 4, 256) + align_up((size_t)B * 4, 256) + align_up(blocks * 32, 256) +
+    return align_up(words * 4, 256) + 2 * align_up((size_t)B * 4, 256) + align_up(blocks * 32, 256) +
            align_up(blocks * 4, 256) + 1024;
+}
+
+// `tasks` holds the group descriptors [4][g_cap] (int4) and, behind them, the token records [rec_cap][32] (int2)
+static int64_t tp_rec_cap(int64_t N, int64_t g_cap, int H) { return N / 32 + g_cap / H + 4; }
+size_t sswin_token_plan_task_ints(int64_t N, int64_t g_cap, int H) {
+    if (N < 0 || g_cap <= 0 || H <= 0) return 0;
+    return (size_t)(16 * g_cap + 64 * tp_rec_cap(N, g_cap, H));
 }
 
 // Checks one plan's arguments and carves its workspace; `a` is ready to launch afterwards.
@@ -997,12 +1031,15 @@ static int token_plan_args(const int32_t* indices, int64_t N, int B, int n, int 
     a.totals = cv.take<int64_t>(8);       // [0] windows, [1] sum c | sum c*c << 32, [2..7] counters
     a.bits = cv.take<uint32_t>(words);
     a.win_T = cv.take<int32_t>((size_t)B);
+    a.win_rec = cv.take<int32_t>((size_t)B);
     a.partial_a = cv.take<int64_t>(4 * (size_t)blocks);
     a.partial_b = cv.take<int32_t>((size_t)blocks);
     SSWIN_CHECK(cv.ok(), "token_plan: workspace too small");
     a.plan = plan;
     a.g_cap = g_cap;
     a.tasks = reinterpret_cast<int4*>(tasks);
+    a.recs = tasks && !a.order_only ? reinterpret_cast<int2*>(tasks + 16 * g_cap) : nullptr;
+    a.rec_cap = tp_rec_cap(N, g_cap, H);
     a.tokens = tokens;
     return 0;
 }
@@ -1232,11 +1269,13 @@ int sswin_bias_table_grad(const int32_t* plan, int64_t g_cap, int64_t G, const i
     const int rows_pad = (table_rows + 31) / 32 * 32 + 32;  // 32 spare rows
     const size_t lds = (size_t)8 * rows_pad * sizeof(float) + (size_t)n * sizeof(int32_t);
     SSWIN_CHECK(lds <= 160 * 1024, "bias_table_grad: a table of %d rows needs %zu bytes of LDS (160 KB at most)", table_rows, lds);
-    static bool configured = false;
-    if (!configured) {                                       // more than the default 64 KB of dynamic LDS
-        SSWIN_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(rpb_table_partial_kernel),
-                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024));
-        configured = true;
+    if (lds > 64 * 1024) {
+        // more than the default 64 KB of dynamic LDS: asked for with every such launch (cheap, and correct for any
+        // number of host threads and devices)
+        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(rpb_table_partial_kernel),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        SSWIN_CHECK(e == hipSuccess, "bias_table_grad: the request for %zu bytes of LDS per workgroup was refused: %s", lds,
+                    hipGetErrorString(e));
     }
     hipLaunchKernelGGL(rpb_table_partial_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), lds, s, gt, tokens + 3 * N, H,
                        code, n, offset0, table_rows, rows_pad, ds, windows, wslices, rsplit, partial);

@@ -189,8 +189,18 @@ __global__ __launch_bounds__(256) void permute_heads_kernel(const int32_t* __res
     const int heads = (int)(g1 - g0 + 1), r = (int)(g - g0);
     const int rs0 = plan[g_cap + g0];
     bool ok = plan[g0] == c && rs == rs0 + r * c;
-    if (ok && r > 0)
-        for (int i = lane; i < c; i += 64) ok = ok && pos_row[(int64_t)(rs + i) * C] == pos_row[(int64_t)(rs0 + i) * C];
+    // the tensor must be coalesced for the derived order to be the sorted one: (window, head) keys ascend from group
+    // to group and positions ascend inside a group (a tensor that is not goes through the sort, as in the reference)
+    if (g > 0) {
+        const int32_t* head = plan + 4 * g_cap;
+        ok = ok && (win[g - 1] < w || (win[g - 1] == w && head[g - 1] < head[g]));
+    }
+    if (ok)
+        for (int i = lane; i < c; i += 64) {
+            const int p = pos_row[(int64_t)(rs + i) * C];
+            if (r > 0) ok = ok && p == pos_row[(int64_t)(rs0 + i) * C];
+            if (i > 0) ok = ok && p > pos_row[(int64_t)(rs + i - 1) * C];
+        }
     if (!__all(ok)) {
         if (lane == 0) atomicAdd(bad, 1);
         return;

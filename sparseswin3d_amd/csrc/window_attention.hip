@@ -40,368 +40,12 @@
 
 #include <type_traits>
 
-#include "mfma_block.hpp"
-#include "sswin_common.hpp"
+#include <stdlib.h>
+
+#include "wattn_common.hpp"
+#include "wattn_x16.hpp"
 
 namespace sswin {
-
-struct TokenTensor32 {      // rows addressed by voxel, columns col0 + h*32 + ch
-    const void* base;
-    int64_t stride;
-    int col0;
-};
-
-struct WAttnCommon {
-    const int4* tasks;      // [4][g_cap] descriptors {T, c | head << 8, window, sq_start} by bucket
-    int64_t g_cap;
-    int64_t first[5];       // first task id of bucket 3, 2, 1, 0 (heaviest first) and the task total
-    const int32_t* order;   // voxel of token rank r
-    const int32_t* tok_pos; // position inside the window of token rank r
-    int H, n;
-    float scale;
-    const float* bias;      // [H, n, n]
-    const int8_t* mask;     // [nmw, n] region ids or null
-    int nmw;
-};
-
-struct GroupCtx {
-    int Tk, c, h, w, sq;
-};
-
-// task id -> (group descriptor, 32-row block inside the group); false past the last task
-__device__ __forceinline__ bool locate(const WAttnCommon& a, int64_t task, int64_t& d, int& blk) {
-    if (task >= a.first[4]) return false;
-    int q = 0;                                   // 0 = bucket 3 (four tiles) ... 3 = bucket 0 (one tile)
-#pragma unroll
-    for (int k = 1; k < 4; ++k) q += task >= a.first[k] ? 1 : 0;
-    const int nt = 4 - q;
-    const int64_t local = task - a.first[q];
-    const int64_t grp = local / nt;
-    blk = (int)(local - grp * nt);
-    d = (int64_t)(nt - 1) * a.g_cap + grp;
-    return true;
-}
-
-__device__ __forceinline__ GroupCtx load_group(const int4* __restrict__ tasks, int64_t d) {
-    const int4 t = tasks[d];
-    GroupCtx g;
-    g.Tk = __builtin_amdgcn_readfirstlane(t.x);
-    g.c = __builtin_amdgcn_readfirstlane(t.y & 0xff);
-    g.h = __builtin_amdgcn_readfirstlane(t.y >> 8);
-    g.w = __builtin_amdgcn_readfirstlane(t.z);
-    g.sq = __builtin_amdgcn_readfirstlane(t.w);
-    return g;
-}
-
-// ------------------------------------------------------------------------------------------
-// Addressing.  Every token tensor is reached as  uniform byte base (tensor base + head columns)
-// + 32-bit byte offset of the row: one full-rate 24-bit multiply per token and no 64-bit vector
-// arithmetic.  The host checks that row offsets fit 32 bits and that rows are 16-byte aligned.
-// ------------------------------------------------------------------------------------------
-typedef float f32x4_a __attribute__((ext_vector_type(4)));               // naturally aligned
-typedef uint32_t u32x4_a __attribute__((ext_vector_type(4)));
-
-constexpr float LOG2E = 1.4426950408889634f;
-constexpr float LN2 = 0.6931471805599453f;
-
-template <typename T>
-__device__ __forceinline__ const char* head_base(const TokenTensor32& t, int h) {
-    return static_cast<const char*>(t.base) + (int64_t)(t.col0 + h * 32) * sizeof(T);
-}
-template <typename T>
-__device__ __forceinline__ uint32_t pitch_of(const TokenTensor32& t) { return (uint32_t)t.stride * (uint32_t)sizeof(T); }
-
-__device__ __forceinline__ void unpack2(uint32_t u, float& lo, float& hi, __half) {
-    const __half2 h2 = __builtin_bit_cast(__half2, u);
-    lo = __low2float(h2);
-    hi = __high2float(h2);
-}
-__device__ __forceinline__ void unpack2(uint32_t u, float& lo, float& hi, __hip_bfloat16) {
-    lo = __builtin_bit_cast(float, u << 16);
-    hi = __builtin_bit_cast(float, u & 0xffff0000u);
-}
-__device__ __forceinline__ uint32_t pack2(float lo, float hi, __half) {
-    return __builtin_bit_cast(uint32_t, __floats2half2_rn(lo, hi));
-}
-__device__ __forceinline__ uint32_t pack2(float lo, float hi, __hip_bfloat16) {
-    const uint32_t a = __builtin_bit_cast(uint16_t, __float2bfloat16(lo));
-    const uint32_t b = __builtin_bit_cast(uint16_t, __float2bfloat16(hi));
-    return a | (b << 16);
-}
-
-// ------------------------------------------------------------------------------------------
-// Wave-private LDS.  A "tile" holds 32 token rows of 32 fp32 channels at a pitch of 36 dwords
-// (16-byte rows stay aligned, and 16-byte accesses of neighbouring rows fall into different
-// banks); it turns the row-major global loads into the column-major MFMA operand of the second
-// product and the accumulators back into rows for wide stores.  A "table" holds one 32-bit value
-// per token of the tile; the 16 entries a lane needs (rows acc_row(r, half)) are four runs of
-// four, fetched with four 16-byte reads.  Only the owning wavefront touches its tiles and tables;
-// LDS operations of one wavefront execute in order, so no barrier is involved.
-// ------------------------------------------------------------------------------------------
-constexpr int TILE_LD = 36;
-constexpr int TILE_WORDS = 32 * TILE_LD;
-
-__device__ __forceinline__ void tile_put_rows(float* tile, int l32, int half, const float (&x)[16]) {
-    f32x4_a* p = reinterpret_cast<f32x4_a*>(tile + l32 * TILE_LD + half * 16);
-#pragma unroll
-    for (int v = 0; v < 4; ++v) p[v] = f32x4_a{x[4 * v], x[4 * v + 1], x[4 * v + 2], x[4 * v + 3]};
-}
-__device__ __forceinline__ void tile_get_rows(const float* tile, int l32, int half, float (&x)[16]) {
-    const f32x4_a* p = reinterpret_cast<const f32x4_a*>(tile + l32 * TILE_LD + half * 16);
-#pragma unroll
-    for (int v = 0; v < 4; ++v) {
-        const f32x4_a t = p[v];
-        x[4 * v] = t.x; x[4 * v + 1] = t.y; x[4 * v + 2] = t.z; x[4 * v + 3] = t.w;
-    }
-}
-// x[r] = tile[row acc_row(r, half)][column l32]
-__device__ __forceinline__ void tile_get_cols(const float* tile, int l32, int half, float (&x)[16]) {
-    const float* p = tile + 4 * half * TILE_LD + l32;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) x[r] = p[(8 * (r >> 2) + (r & 3)) * TILE_LD];
-}
-__device__ __forceinline__ void tile_put_acc(float* tile, int l32, int half, const f32x16& acc) {
-    float* p = tile + 4 * half * TILE_LD + l32;
-#pragma unroll
-    for (int r = 0; r < 16; ++r) p[(8 * (r >> 2) + (r & 3)) * TILE_LD] = acc[r];
-}
-__device__ __forceinline__ void table_put(uint32_t* tab, int l32, uint32_t v) { tab[l32] = v; }
-__device__ __forceinline__ void table_get(const uint32_t* tab, int half, uint32_t (&x)[16]) {
-    const u32x4_a* p = reinterpret_cast<const u32x4_a*>(tab + 4 * half);
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        const u32x4_a t = p[2 * q];
-        x[4 * q] = t.x; x[4 * q + 1] = t.y; x[4 * q + 2] = t.z; x[4 * q + 3] = t.w;
-    }
-}
-// A table kept in the spare columns of a tile: rows are 36 dwords wide and only 32 of them carry
-// values, so the four spare dwords of eight consecutive rows hold 32 entries, entries 4k .. 4k+3
-// in row k.  A tile has room for four such tables (rows 0-7, 8-15, 16-23, 24-31); the 16-byte
-// reads of table_get fall on whole rows' spare columns.  The backward kernels keep their tables
-// there, which leaves LDS for the exchange tiles of the two-tile groups.
-struct PadTab {
-    uint32_t* p;
-    __device__ __forceinline__ void put(int e, uint32_t v) const { p[(e >> 2) * TILE_LD + (e & 3)] = v; }
-    __device__ __forceinline__ uint32_t get(int e) const { return p[(e >> 2) * TILE_LD + (e & 3)]; }
-    __device__ __forceinline__ u32x4_a chunk(int ch) const { return *reinterpret_cast<const u32x4_a*>(p + ch * TILE_LD); }
-};
-__device__ __forceinline__ PadTab pad_tab(float* tile, int k) {
-    return PadTab{reinterpret_cast<uint32_t*>(tile) + 8 * k * TILE_LD + 32};
-}
-__device__ __forceinline__ void table_put(const PadTab& tab, int l32, uint32_t v) { tab.put(l32, v); }
-__device__ __forceinline__ void table_get(const PadTab& tab, int half, uint32_t (&x)[16]) {
-#pragma unroll
-    for (int q = 0; q < 4; ++q) {
-        const u32x4_a t = tab.chunk(2 * q + half);
-        x[4 * q] = t.x; x[4 * q + 1] = t.y; x[4 * q + 2] = t.z; x[4 * q + 3] = t.w;
-    }
-}
-__device__ __forceinline__ uint32_t f2u(float v) { return __builtin_bit_cast(uint32_t, v); }
-__device__ __forceinline__ float u2f(uint32_t v) { return __builtin_bit_cast(float, v); }
-__device__ __forceinline__ float exp2_fast(float x) { return __builtin_amdgcn_exp2f(x); }
-
-// ------------------------------------------------------------------------------------------
-// One MFMA product step over the reduction slots a lane holds.  fp32 tokens: one
-// v_mfma_f32_32x32x2_f32 per slot (the lane pair l, l + 32 supplies k = 2 values).  16-bit tokens:
-// the operands are rounded to the token type and eight slots go into one v_mfma_f32_32x32x16
-// (k = 16: eight slots of lanes 0-31, eight of lanes 32-63) - an eighth of the matrix-core
-// passes.  A and B use the same slot -> reduction index mapping, which is all a product needs.
-// ------------------------------------------------------------------------------------------
-template <typename T> struct LowPrec;
-template <> struct LowPrec<__hip_bfloat16> {
-    typedef __bf16 elem;
-    typedef __bf16 vec __attribute__((ext_vector_type(8)));
-    static __device__ __forceinline__ f32x16 mma(vec a, vec b, f32x16 c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, b, c, 0, 0, 0);
-    }
-};
-template <> struct LowPrec<__half> {
-    typedef _Float16 elem;
-    typedef _Float16 vec __attribute__((ext_vector_type(8)));
-    static __device__ __forceinline__ f32x16 mma(vec a, vec b, f32x16 c) {
-        return __builtin_amdgcn_mfma_f32_32x32x16_f16(a, b, c, 0, 0, 0);
-    }
-};
-// the same, starting from the instruction's zero operand instead of a cleared accumulator
-template <typename T, int N, typename A, typename B>
-__device__ __forceinline__ f32x16 mma_slots_first(const A& a, const B& b) {
-    const f32x16 zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-    f32x16 acc;
-    if constexpr (std::is_same<T, float>::value) {
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[0], b[0], zero, 0, 0, 0);
-#pragma unroll
-        for (int s = 1; s < N; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], acc, 0, 0, 0);
-    } else {
-        typename LowPrec<T>::vec va, vb;
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            va[i] = (typename LowPrec<T>::elem)a[i];
-            vb[i] = (typename LowPrec<T>::elem)b[i];
-        }
-        acc = LowPrec<T>::mma(va, vb, zero);
-#pragma unroll
-        for (int m = 1; m < N / 8; ++m) {
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                va[i] = (typename LowPrec<T>::elem)a[8 * m + i];
-                vb[i] = (typename LowPrec<T>::elem)b[8 * m + i];
-            }
-            acc = LowPrec<T>::mma(va, vb, acc);
-        }
-    }
-    return acc;
-}
-// eight slots: a[OFF .. OFF + 8) against b[0 .. 8)
-template <typename T, int OFF, typename A, typename B>
-__device__ __forceinline__ void mma_slots8_off(const A& a, const B& b, f32x16& acc) {
-    typename LowPrec<T>::vec va, vb;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        va[i] = (typename LowPrec<T>::elem)a[OFF + i];
-        vb[i] = (typename LowPrec<T>::elem)b[i];
-    }
-    acc = LowPrec<T>::mma(va, vb, acc);
-}
-template <typename T, int OFF, int N, typename A, typename B>
-__device__ __forceinline__ void mma_slots(const A& a, const B& b, f32x16& acc) {
-    if constexpr (std::is_same<T, float>::value) {
-#pragma unroll
-        for (int s = 0; s < N; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[OFF + s], b[OFF + s], acc, 0, 0, 0);
-    } else {
-        static_assert(N % 8 == 0, "16-bit products take eight slots per step");
-#pragma unroll
-        for (int m = 0; m < N / 8; ++m) {
-            typename LowPrec<T>::vec va, vb;
-#pragma unroll
-            for (int i = 0; i < 8; ++i) {
-                va[i] = (typename LowPrec<T>::elem)a[OFF + 8 * m + i];
-                vb[i] = (typename LowPrec<T>::elem)b[OFF + 8 * m + i];
-            }
-            acc = LowPrec<T>::mma(va, vb, acc);
-        }
-    }
-}
-
-// ------------------------------------------------------------------------------------------
-// Coalesced token rows.  A head's slice of a token row is 32 channels = CH chunks of 16 bytes
-// (8 for fp32, 4 for 16-bit values).  One load instruction fetches 64 / CH whole slices: lane l
-// reads chunk l % CH of the row l / CH of its group, so the lanes of a slice read one contiguous
-// 128- or 64-byte piece and the memory pipeline sees a quarter of the requests a row-per-lane
-// load makes.  The pieces are turned into the row-per-lane MFMA operand through an LDS tile.
-// ------------------------------------------------------------------------------------------
-template <typename T>
-struct RowLoad {
-    static constexpr int CH = 32 * (int)sizeof(T) / 16;      // chunks per row slice
-    static constexpr int ROWS = 64 / CH;                     // rows per instruction
-    static constexpr int NI = 32 / ROWS;                     // instructions per 32 rows
-    u32x4_a v[NI];
-};
-
-// vox_lane: voxel of row l32, held by lanes l32 and l32 + 32
-// STREAM: the rows belong to a group of one tile, so no other task reads them: loaded with the streaming hint (the
-// key-side task of one-tile groups in the backward: 0.1203 -> 0.1187 ms on cfg2, 0.096 -> 0.095 on cfg3).  Rows of
-// larger groups are read by up to eight tasks and must stay cached: with the hint on all loads the bf16 backward of
-// 100-125-token windows went from 0.097 to 0.156 ms and the forward from 0.049 to 0.062; in the forward the hint for
-// one-tile groups alone was no gain either (cfg2 0.0568 against 0.0572 ms, cfg3 0.0441 against 0.0425).
-template <typename T, bool STREAM = false>
-__device__ __forceinline__ void rows_load(const char* __restrict__ base, uint32_t pitch, uint32_t vox_lane, int lane,
-                                          RowLoad<T>& r) {
-    constexpr int CH = RowLoad<T>::CH, ROWS = RowLoad<T>::ROWS;
-#pragma unroll
-    for (int v = 0; v < RowLoad<T>::NI; ++v) {
-        const uint32_t vox = (uint32_t)__shfl((int)vox_lane, v * ROWS + lane / CH, 64);
-        const u32x4_a* p = reinterpret_cast<const u32x4_a*>(base + (__umul24(vox, pitch) + (uint32_t)(lane % CH) * 16u));
-        r.v[v] = STREAM ? __builtin_nontemporal_load(p) : *p;
-    }
-}
-template <typename T>
-__device__ __forceinline__ void rows_to_tile(float* tile, int lane, const RowLoad<T>& r);
-template <>
-__device__ __forceinline__ void rows_to_tile<float>(float* tile, int lane, const RowLoad<float>& r) {
-#pragma unroll
-    for (int v = 0; v < RowLoad<float>::NI; ++v)
-        *reinterpret_cast<u32x4_a*>(tile + (v * 8 + lane / 8) * TILE_LD + (lane % 8) * 4) = r.v[v];
-}
-template <typename T>
-__device__ __forceinline__ void rows_to_tile(float* tile, int lane, const RowLoad<T>& r) {
-#pragma unroll
-    for (int v = 0; v < RowLoad<T>::NI; ++v) {
-        float x[8];
-        unpack2(r.v[v].x, x[0], x[1], T());
-        unpack2(r.v[v].y, x[2], x[3], T());
-        unpack2(r.v[v].z, x[4], x[5], T());
-        unpack2(r.v[v].w, x[6], x[7], T());
-        f32x4_a* p = reinterpret_cast<f32x4_a*>(tile + (v * 16 + lane / 4) * TILE_LD + (lane % 4) * 8);
-        p[0] = f32x4_a{x[0], x[1], x[2], x[3]};
-        p[1] = f32x4_a{x[4], x[5], x[6], x[7]};
-    }
-}
-// tile rows -> global rows, the same lane assignment; rows at or beyond `rows` are padding
-template <typename T>
-__device__ __forceinline__ void tile_store_rows(const float* tile, char* __restrict__ base, uint32_t pitch,
-                                                uint32_t vox_lane, int rows, int lane);
-template <>
-__device__ __forceinline__ void tile_store_rows<float>(const float* tile, char* __restrict__ base, uint32_t pitch,
-                                                       uint32_t vox_lane, int rows, int lane) {
-#pragma unroll
-    for (int v = 0; v < 4; ++v) {
-        const int R = v * 8 + lane / 8;
-        const uint32_t vox = (uint32_t)__shfl((int)vox_lane, R, 64);
-        const u32x4_a x = *reinterpret_cast<const u32x4_a*>(tile + R * TILE_LD + (lane % 8) * 4);
-        if (R < rows) *reinterpret_cast<u32x4_a*>(base + (__umul24(vox, pitch) + (uint32_t)(lane % 8) * 16u)) = x;
-    }
-}
-template <typename T>
-__device__ __forceinline__ void tile_store_rows(const float* tile, char* __restrict__ base, uint32_t pitch,
-                                                uint32_t vox_lane, int rows, int lane) {
-#pragma unroll
-    for (int v = 0; v < 2; ++v) {
-        const int R = v * 16 + lane / 4;
-        const uint32_t vox = (uint32_t)__shfl((int)vox_lane, R, 64);
-        const f32x4_a* p = reinterpret_cast<const f32x4_a*>(tile + R * TILE_LD + (lane % 4) * 8);
-        const f32x4_a lo = p[0], hi = p[1];
-        const u32x4_a x = {pack2(lo.x, lo.y, T()), pack2(lo.z, lo.w, T()), pack2(hi.x, hi.y, T()), pack2(hi.z, hi.w, T())};
-        if (R < rows) *reinterpret_cast<u32x4_a*>(base + (__umul24(vox, pitch) + (uint32_t)(lane % 4) * 16u)) = x;
-    }
-}
-
-// table[row] = x_row . y_row for the 32 rows two loads hold: per-chunk dot products, summed over
-// the CH lanes of a row by DPP steps inside groups of 4 and 8 lanes
-template <typename T>
-__device__ __forceinline__ float chunk_dot(const u32x4_a& x, const u32x4_a& y);
-template <>
-__device__ __forceinline__ float chunk_dot<float>(const u32x4_a& x, const u32x4_a& y) {
-    float d = u2f(x.x) * u2f(y.x);
-    d = fmaf(u2f(x.y), u2f(y.y), d);
-    d = fmaf(u2f(x.z), u2f(y.z), d);
-    return fmaf(u2f(x.w), u2f(y.w), d);
-}
-template <typename T>
-__device__ __forceinline__ float chunk_dot(const u32x4_a& x, const u32x4_a& y) {
-    const uint32_t xs[4] = {x.x, x.y, x.z, x.w}, ys[4] = {y.x, y.y, y.z, y.w};
-    float d = 0.f;
-#pragma unroll
-    for (int k = 0; k < 4; ++k) {
-        float a0, a1, b0, b1;
-        unpack2(xs[k], a0, a1, T());
-        unpack2(ys[k], b0, b1, T());
-        d = fmaf(a0, b0, d);
-        d = fmaf(a1, b1, d);
-    }
-    return d;
-}
-template <typename T>
-__device__ __forceinline__ void rows_dot_to_table(const PadTab& tab, int lane, const RowLoad<T>& x, const RowLoad<T>& y) {
-    constexpr int CH = RowLoad<T>::CH, ROWS = RowLoad<T>::ROWS;
-#pragma unroll
-    for (int v = 0; v < RowLoad<T>::NI; ++v) {
-        float d = chunk_dot<T>(x.v[v], y.v[v]);
-        d += dpp_f32<0xB1>(d);                               // lanes 0..3 of a quad
-        d += dpp_f32<0x4E>(d);
-        if (CH == 8) d += dpp_f32<0x141>(d);                 // the two quads of 8 lanes
-        if (lane % CH == 0) tab.put(v * ROWS + lane / CH, f2u(d));
-    }
-}
 
 // ------------------------------------------------------------------------------------------
 // forward: rows = 32 queries of a group, tiles = its keys
@@ -427,32 +71,27 @@ __device__ __forceinline__ GroupCtx decode_group(const int4& t) {
     g.sq = __builtin_amdgcn_readfirstlane(t.w);
     return g;
 }
-__device__ __forceinline__ FwdIdx fwd_indices(const WAttnCommon& a, const GroupCtx& g, int bi, int l32) {
-    const int32_t* order = a.order + g.Tk;
-    const int32_t* tok_pos = a.tok_pos + g.Tk;
-    const int i_q = bi * 32 + l32;
-    const int i_c = i_q < g.c ? i_q : g.c - 1;
-    const int j_c = l32 < g.c ? l32 : g.c - 1;
+// rec: the task's own token record, rec0: the record of the group's first tile
+__device__ __forceinline__ FwdIdx fwd_indices(const WAttnCommon& a, int64_t rec, int64_t rec0, int l32) {
+    const int2 eq = token_entry(a, rec, l32), ek = token_entry(a, rec0, l32);
     FwdIdx x;
-    x.vox_i = order[i_c];
-    x.pos_i = tok_pos[i_c];
-    x.k0 = KIdx{(uint32_t)order[j_c], tok_pos[j_c]};
+    x.vox_i = (uint32_t)eq.x;
+    x.pos_i = eq.y;
+    x.k0 = KIdx{(uint32_t)ek.x, ek.y};
     return x;
 }
 
 // One forward task on one wavefront.  `mid` runs once between the last key tile and the write-out (a hook for
 // work that should overlap the write-out; the plain kernel passes nothing).
 template <typename T, bool MASK, typename Mid>
-__device__ __forceinline__ void fwd_task(const WAttnCommon& a, const GroupCtx& g, const int bi, const FwdIdx& fi,
-                                         float* tile, float* tile_x, uint32_t* tab_key, uint32_t* tab_alpha,
+__device__ __forceinline__ void fwd_task(const WAttnCommon& a, const GroupCtx& g, const int bi, const int64_t rec0,
+                                         const FwdIdx& fi, float* tile, float* tile_x, uint32_t* tab_key, uint32_t* tab_alpha,
                                          const TokenTensor32& tq, const TokenTensor32& tk, const TokenTensor32& tv,
                                          const TokenTensor32& to, float* __restrict__ lse, Mid&& mid) {
     const int lane = threadIdx.x & 63;
     const int half = lane >> 5, l32 = lane & 31;
     const int c = g.c, h = g.h;
     const int nt = (c + 31) >> 5;
-    const int32_t* order = a.order + g.Tk;
-    const int32_t* tok_pos = a.tok_pos + g.Tk;
     const int8_t* mrow = MASK ? a.mask + (int64_t)(g.w % a.nmw) * a.n : nullptr;
     const char* qbase = head_base<T>(tq, h);
     const char* kbase = head_base<T>(tk, h);
@@ -467,9 +106,8 @@ __device__ __forceinline__ void fwd_task(const WAttnCommon& a, const GroupCtx& g
     // bias) and a task is short, so the indices of the first key tile are requested together with the
     // query indices, and its K and V rows together with the Q rows.
     auto load_kidx = [&](const int t) {
-        const int j = t * 32 + l32;
-        const int j_c = j < c ? j : c - 1;
-        return KIdx{(uint32_t)order[j_c], tok_pos[j_c]};
+        const int2 e = token_entry(a, rec0 + t, l32);
+        return KIdx{(uint32_t)e.x, e.y};
     };
     KIdx kcur = fi.k0;
     const int reg_i = MASK ? mrow[pos_i] : 0;
@@ -736,18 +374,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     __shared__ __attribute__((aligned(16))) float tiles[4][2][TILE_WORDS];
     __shared__ __attribute__((aligned(16))) uint32_t tabs[4][2][32];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
-    int64_t d;
+    int64_t d, rec;
     int bi;
-    if (!locate(a, (int64_t)blockIdx.x * 4 + wave, d, bi)) return;
-    const GroupCtx g = load_group(a.tasks, d);
-    const FwdIdx fi = fwd_indices(a, g, bi, lane & 31);
+    if (!locate(a, (int64_t)blockIdx.x * 4 + wave, d, bi, rec)) return;
+    const int4 desc = a.tasks[d];                            // descriptor and token records travel together
+    const FwdIdx fi = fwd_indices(a, rec, rec - bi, lane & 31);
+    const GroupCtx g = decode_group(desc);
     if constexpr (std::is_same<T, float>::value) {
         if (g.c <= 16) {
             fwd_task_small<MASK>(a, g, fi, tiles[wave][0], tiles[wave][1], tabs[wave][0], tabs[wave][1], tq, tk, tv, to, lse);
             return;
         }
     }
-    fwd_task<T, MASK>(a, g, bi, fi, tiles[wave][0], tiles[wave][1], tabs[wave][0], tabs[wave][1], tq, tk, tv, to, lse, [] {});
+    fwd_task<T, MASK>(a, g, bi, rec - bi, fi, tiles[wave][0], tiles[wave][1], tabs[wave][0], tabs[wave][1], tq, tk, tv, to, lse,
+                      [] {});
 }
 
 // ------------------------------------------------------------------------------------------
@@ -763,15 +403,17 @@ __device__ __forceinline__ void bwd_q_task(const WAttnCommon& a, int64_t task, f
                                            const TokenTensor32& tdq) {
     const int lane = threadIdx.x & 63;
     const int half = lane >> 5, l32 = lane & 31;
-    int64_t d;
+    int64_t d, rec;
     int bi;
-    if (!locate(a, task, d, bi)) return;
+    if (!locate(a, task, d, bi, rec)) return;
     const PadTab tab_key = pad_tab(tile, 0), tab_D = pad_tab(tile, 1);
-    const GroupCtx g = load_group(a.tasks, d);
+    // the descriptor, the queries' indices and those of the first key tile: one round trip
+    const int4 desc = a.tasks[d];
+    const int64_t rec0 = rec - bi;
+    const int2 e_q = token_entry(a, rec, l32), e_k0 = token_entry(a, rec0, l32);
+    const GroupCtx g = decode_group(desc);
     const int c = g.c, h = g.h;
     const int nt = (c + 31) >> 5;
-    const int32_t* order = a.order + g.Tk;
-    const int32_t* tok_pos = a.tok_pos + g.Tk;
     const int8_t* mrow = MASK ? a.mask + (int64_t)(g.w % a.nmw) * a.n : nullptr;
     const char* kbase = head_base<T>(tk, h);
     const char* vbase = head_base<T>(tv, h);
@@ -779,12 +421,10 @@ __device__ __forceinline__ void bwd_q_task(const WAttnCommon& a, int64_t task, f
 
     const int i_q = bi * 32 + l32;
     const int i_c = i_q < c ? i_q : c - 1;
-    const uint32_t vox_i = order[i_c];
-    const int pos_i = tok_pos[i_c];
-    // indices of the first key tile: requested in the same round trip as the query indices
-    int jn_c = l32 < c ? l32 : c - 1;
-    uint32_t vox_n = order[jn_c];
-    int pos_n = tok_pos[jn_c];
+    const uint32_t vox_i = (uint32_t)e_q.x;
+    const int pos_i = e_q.y;
+    uint32_t vox_n = (uint32_t)e_k0.x;
+    int pos_n = e_k0.y;
     const int reg_i = MASK ? mrow[pos_i] : 0;
     const float L2 = lse[(int64_t)a.H * g.Tk + h * c + i_c] * LOG2E;
     float qb[16], dob[16];
@@ -819,11 +459,10 @@ __device__ __forceinline__ void bwd_q_task(const WAttnCommon& a, int64_t task, f
         rows_load<T>(vbase, vpitch, vox_j, lane, rv);
         uint32_t pk = (uint32_t)pos_j * 4u;
         if (MASK) pk |= (uint32_t)mrow[pos_j] << 16;
-        {                                                    // indices of the next key tile, a tile ahead
-            const int j = (t + 1) * 32 + l32;
-            jn_c = j < c ? j : c - 1;
-            vox_n = order[jn_c];
-            pos_n = tok_pos[jn_c];
+        if (t + 1 < nt) {                                    // indices of the next key tile, a tile ahead
+            const int2 e = token_entry(a, rec0 + t + 1, l32);
+            vox_n = (uint32_t)e.x;
+            pos_n = e.y;
         }
         __builtin_amdgcn_wave_barrier();
         table_put(tab_key, l32, pk);
@@ -919,7 +558,8 @@ __device__ __forceinline__ void xch_add(const float* xch, int lane, f32x16& v) {
 // LDS: rows 0-15 of tile_q hold Q, rows 16-31 K; rows 0-15 of tile_do hold dO, rows 16-31 V, later dS.
 // ------------------------------------------------------------------------------------------
 template <bool MASK>
-__device__ __forceinline__ void bwd_task_small(const WAttnCommon& a, const GroupCtx& g, float* tile_q, float* tile_do,
+__device__ __forceinline__ void bwd_task_small(const WAttnCommon& a, const GroupCtx& g, const int2 entry, float* tile_q,
+                                               float* tile_do,
                                                const TokenTensor32& tq, const TokenTensor32& tk, const TokenTensor32& tv,
                                                const TokenTensor32& to, const TokenTensor32& tdo,
                                                const float* __restrict__ lse, const TokenTensor32& tdq,
@@ -930,10 +570,11 @@ __device__ __forceinline__ void bwd_task_small(const WAttnCommon& a, const Group
     const int c = g.c, h = g.h;
     const int8_t* mrow = MASK ? a.mask + (int64_t)(g.w % a.nmw) * a.n : nullptr;
     const PadTab tab_pos = pad_tab(tile_q, 0), tab_L = pad_tab(tile_q, 1), tab_D = pad_tab(tile_q, 2);
-    // token col of the group (clamped to the last one): key of this lane's column
+    // token col of the group (the last one again behind it): key of this lane's column; `entry` is the record's
+    // entry lane % 32
     const int t_c = col < c ? col : c - 1;
-    const uint32_t vox = (uint32_t)a.order[g.Tk + t_c];
-    const int pos = a.tok_pos[g.Tk + t_c];
+    const uint32_t vox = (uint32_t)__shfl(entry.x, col, 64);
+    const int pos = __shfl(entry.y, col, 64);
     const float L2 = col < c ? lse[(int64_t)a.H * g.Tk + h * c + t_c] * LOG2E : INFINITY;   // padding queries: P = 0
     const int reg = MASK ? mrow[pos] : 0;
     u32x4_a rq[2], rk[2], rv[2], rdo[2], ro[2];
@@ -1082,24 +723,27 @@ __device__ __forceinline__ void bwd_kv_task(const WAttnCommon& a, int64_t task, 
                                             const TokenTensor32& tdq) {
     const int lane = threadIdx.x & 63;
     const int half = lane >> 5, l32 = lane & 31;
-    int64_t d;
+    int64_t d, rec;
     int bj;
-    if (!live || !locate(a, task, d, bj)) {
+    if (!live || !locate(a, task, d, bj, rec)) {
         if (DQ == KV_PAIR) __syncthreads();
         return;
     }
     const PadTab tab_pos = pad_tab(tile_q, 0), tab_L = pad_tab(tile_q, 1), tab_D = pad_tab(tile_q, 2);
-    const GroupCtx g = load_group(a.tasks, d);
+    // the descriptor, the keys' indices and those of the first query tile: one round trip
+    const int t_first = DQ == KV_PAIR ? 1 - bj : 0;           // KV_PAIR: the other wavefront's query tile first
+    const int4 desc = a.tasks[d];
+    const int64_t rec0 = rec - bj;
+    const int2 e_k = token_entry(a, rec, l32), e_q0 = token_entry(a, rec0 + t_first, l32);
+    const GroupCtx g = decode_group(desc);
     if constexpr (DQ == KV_SINGLE && std::is_same<T, float>::value) {
         if (g.c <= 16) {
-            bwd_task_small<MASK>(a, g, tile_q, tile_do, tq, tk, tv, to, tdo, lse, tdq, tdk, tdv, ds_out);
+            bwd_task_small<MASK>(a, g, e_k, tile_q, tile_do, tq, tk, tv, to, tdo, lse, tdq, tdk, tdv, ds_out);
             return;
         }
     }
     const int c = g.c, h = g.h;
     const int nt = (c + 31) >> 5;
-    const int32_t* order = a.order + g.Tk;
-    const int32_t* tok_pos = a.tok_pos + g.Tk;
     const int8_t* mrow = MASK ? a.mask + (int64_t)(g.w % a.nmw) * a.n : nullptr;
     const char* qbase = head_base<T>(tq, h);
     const char* obase = head_base<T>(to, h);
@@ -1115,22 +759,21 @@ __device__ __forceinline__ void bwd_kv_task(const WAttnCommon& a, int64_t task, 
         int pos;
         float L2;            // its log-sum-exp in units of log 2; +inf for padding queries: P and dS exactly zero
     };
-    auto load_qidx = [&](const int t) {
+    auto make_qidx = [&](const int t, const int2 e) {
         const int i = t * 32 + l32;
         const int i_c = i < c ? i : c - 1;
         QIdx q;
-        q.vox = order[i_c];
-        q.pos = tok_pos[i_c];
+        q.vox = (uint32_t)e.x;
+        q.pos = e.y;
         q.L2 = i < c ? lse_g[i_c] * LOG2E : INFINITY;
         return q;
     };
+    auto load_qidx = [&](const int t) { return make_qidx(t, token_entry(a, rec0 + t, l32)); };
     // key side: lane l32 owns key bj*32 + l32
     const int j_k = bj * 32 + l32;
-    const int j_c = j_k < c ? j_k : c - 1;
-    const uint32_t vox_j = order[j_c];
-    const int pos_j = tok_pos[j_c];
-    const int t_first = DQ == KV_PAIR ? 1 - bj : 0;           // KV_PAIR: the other wavefront's query tile first
-    QIdx qcur = load_qidx(t_first);
+    const uint32_t vox_j = (uint32_t)e_k.x;
+    const int pos_j = e_k.y;
+    QIdx qcur = make_qidx(t_first, e_q0);
     const int reg_j = MASK ? mrow[pos_j] : 0;
     RowLoad<T> rq, rdo, ro;
     float kb[16], vb[16];
@@ -1360,19 +1003,6 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
                                   tq, tk, tv, to, tdo, lse, tdk, tdv, ds_out, tdk);
 }
 
-// The whole backward in one launch.  Workgroups (four wavefronts, one task each) are numbered through
-// four segments, each starting at a workgroup boundary:
-//   1. query-side tasks of the groups of three and four tiles
-//   2. their key-side tasks (KV_ONLY); 1 and 2 are interleaved in runs of eight workgroups (see the kernel)
-//   3. key-side tasks of the groups of two tiles, the two tasks of a group side by side (KV_PAIR)
-//   4. key-side tasks of the groups of one tile (KV_SINGLE)
-// Heaviest tasks first, so the long ones start first and the short ones fill the tail.
-struct BwdSegments {
-    int64_t wg_kv, wg_pair, wg_single;   // first workgroup of segments 2, 3, 4
-    int64_t n_big;                       // tasks per side of the groups of three and four tiles
-    int64_t n_pair;                      // key-side tasks of the groups of two tiles (even)
-};
-
 template <typename T, bool MASK>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void wattn_bwd_all_kernel(
     WAttnCommon a, BwdSegments sg, TokenTensor32 tq, TokenTensor32 tk, TokenTensor32 tv, TokenTensor32 to,
@@ -1431,16 +1061,8 @@ static void launch_backward(const WAttnCommon& a, const TokenTensor32& q, const 
                             const TokenTensor32& dq, const TokenTensor32& dk, const TokenTensor32& dv, float* ds_out,
                             int sides, hipStream_t s) {
     if (sides == 3) {
-        BwdSegments sg;
-        sg.n_big = a.first[2];
-        sg.n_pair = a.first[3] - a.first[2];
-        const int64_t n_single = a.first[4] - a.first[3];
-        const int64_t wg_big = (sg.n_big + 3) / 4;
-        sg.wg_kv = wg_big;
-        sg.wg_pair = 16 * ((wg_big + 7) / 8);              // both sides, interleaved in runs of eight workgroups
-        sg.wg_single = sg.wg_pair + (sg.n_pair + 3) / 4;
-        const int64_t wgs = sg.wg_single + (n_single + 3) / 4;
-        hipLaunchKernelGGL((wattn_bwd_all_kernel<T, MASK>), dim3((unsigned)wgs), dim3(256), 0, s, a, sg, q, k, v, o, d_o, lse,
+        const BwdSegments sg = make_segments(a);
+        hipLaunchKernelGGL((wattn_bwd_all_kernel<T, MASK>), dim3((unsigned)sg.wgs), dim3(256), 0, s, a, sg, q, k, v, o, d_o, lse,
                            dq, dk, dv, ds_out);
         return;
     }
@@ -1476,6 +1098,17 @@ static int check_tensor(const char* who, const char* name, const void* base, int
     return 0;
 }
 
+// Which kernels run a call.  fp32 tokens: the kernels of this file (fp32 matrix instructions, fp32 LDS tiles);
+// 16-bit tokens: the 16-bit-operand kernels of window_attention_x16.hip.  SSWIN_WATTN=x16 or SSWIN_WATTN=fp32mfma in
+// the environment forces one family for every type (fp32 tokens on the 16-bit operands are split into two fp16
+// pieces); read at every call.
+static bool legacy_kernels(int dtype) {
+    const char* e = getenv("SSWIN_WATTN");
+    if (e && e[0] == 'x') return false;
+    if (e && e[0] == 'f') return true;
+    return dtype == SSWIN_F32;
+}
+
 static WAttnCommon make_common(const int32_t* tasks, int64_t g_cap, const int64_t* counts, const int32_t* tokens,
                                int64_t N, int H, int n, float scale, const float* bias, const int8_t* mask, int nmw) {
     WAttnCommon a;
@@ -1485,6 +1118,9 @@ static WAttnCommon make_common(const int32_t* tasks, int64_t g_cap, const int64_
     for (int q = 0; q < 4; ++q) a.first[q + 1] = a.first[q] + counts[3 - q] * (4 - q);
     a.order = tokens;
     a.tok_pos = tokens + 3 * N;
+    a.recs = reinterpret_cast<const int2*>(tasks + 16 * g_cap);
+    a.rec_first[0] = 0;
+    for (int q = 0; q < 3; ++q) a.rec_first[q + 1] = a.rec_first[q] + counts[3 - q] / H * (4 - q);
     a.H = H;
     a.n = n;
     a.scale = scale;
@@ -1542,6 +1178,10 @@ int sswin_window_attention_forward(int dtype, const int32_t* tasks, int64_t g_ca
     const TokenTensor32 q{q_base, q_stride, q_col0}, k{k_base, k_stride, k_col0}, v{v_base, v_stride, v_col0},
         o{o_base, o_stride, o_col0};
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (!legacy_kernels(dtype)) {
+        x16::forward(dtype, a, q, k, v, o, lse, s);
+        return launch_ok("window attention forward");
+    }
     switch (dtype) {
         case SSWIN_F32: return run_forward<float>(a, q, k, v, o, lse, s);
         case SSWIN_F16: return run_forward<__half>(a, q, k, v, o, lse, s);
@@ -1586,6 +1226,10 @@ int sswin_window_attention_backward(int dtype, const int32_t* tasks, int64_t g_c
         o{o_base, o_stride, o_col0}, d_o{do_base, do_stride, do_col0}, dq{dq_base, dq_stride, dq_col0},
         dk{dk_base, dk_stride, dk_col0}, dv{dv_base, dv_stride, dv_col0};
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (!legacy_kernels(dtype)) {
+        x16::backward(dtype, a, q, k, v, o, d_o, lse, dq, dk, dv, ds_out, sides, s);
+        return launch_ok("window attention backward");
+    }
     switch (dtype) {
         case SSWIN_F32: return run_backward<float>(a, q, k, v, o, d_o, lse, dq, dk, dv, ds_out, sides, s);
         case SSWIN_F16: return run_backward<__half>(a, q, k, v, o, d_o, lse, dq, dk, dv, ds_out, sides, s);

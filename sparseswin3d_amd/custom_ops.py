@@ -143,8 +143,8 @@ def return_inverse(x, maxnum=-1):
 def operand_map(indices, batch_size, spatial_dim):
     """Rank of every voxel in (window, pos) order as an int32 tensor [3N + 2] (voxel of rank r, first rank
     and size of its window, then the validity pair); input for :func:`operand_copy` and
-    :func:`sorted_coo_indices`.  Invalid (window, pos) pairs are reported by the next operator that waits
-    for the stream, as for ``qkv_sparse_indices(..., _defer_check=True)``."""
+    :func:`sorted_coo_indices`.  Invalid (window, pos) pairs (out of range, repeated) are skipped on the device and
+    reported by the next operator of this module that waits for the stream (:func:`_check_pending`)."""
     lib = _lib.load()
     d = _dev(indices)
     _check(indices.dim() == 2 and indices.shape[1] == 2, "operand_map: indices must be [N, 2]")
@@ -199,13 +199,13 @@ def sorted_coo_indices(indices, omap, num_heads, c, qv=True, k=True):
     return idx_qv, idx_k
 
 
-# Input checks whose verdict is still on its way from the GPU: (event, pinned status, voxel count).  An
-# operator that has just waited for the stream anyway looks at them (:func:`_check_pending`).
+# Input checks of :func:`operand_map` whose verdict is still on its way from the GPU: (event, pinned status,
+# voxel count).  An operator that has just waited for the stream anyway looks at them (:func:`_check_pending`).
 _pending = []
 
 
 def _check_pending(wait=False):
-    """Raise for a deferred :func:`qkv_sparse_indices` check whose status has arrived (all of them after
+    """Raise for a deferred :func:`operand_map` check whose status has arrived (all of them after
     ``wait=True`` or after the caller has synchronised the stream)."""
     keep = []
     bad = None
@@ -216,16 +216,16 @@ def _check_pending(wait=False):
         event.synchronize()
         out_of_range, distinct = int(status[0]), int(status[1])
         if out_of_range:
-            bad = (f"qkv_sparse_indices: {out_of_range} voxel indices lie outside [0, batch_size) x [0, spatial_dim)")
+            bad = (f"operand_map: {out_of_range} voxel indices lie outside [0, batch_size) x [0, spatial_dim)")
         elif distinct != n_vox:
-            bad = (f"qkv_sparse_indices: (window, pos) pairs must be distinct: {n_vox - distinct} voxels share a "
+            bad = (f"operand_map: (window, pos) pairs must be distinct: {n_vox - distinct} voxels share a "
                    "pair with another")
     _pending[:] = keep
     if bad:
         raise RuntimeError(bad)
 
 
-def qkv_sparse_indices(indices, batch_size, spatial_dim, num_heads, c, _defer_check=False):
+def qkv_sparse_indices(indices, batch_size, spatial_dim, num_heads, c):
     """Element-level COO indices of Q/V and K^T plus their sorting permutations (ops.cu:293-335)."""
     lib = _lib.load()
     d = _dev(indices)
@@ -240,21 +240,13 @@ def qkv_sparse_indices(indices, batch_size, spatial_dim, num_heads, c, _defer_ch
     sorted_k = torch.empty(e, dtype=torch.int32, device=d)
     nbytes = lib.sswin_qkv_sparse_indices_workspace_bytes(n_vox, int(batch_size), int(spatial_dim))
     ws = _ws(nbytes, d)
-    # Indices the kernels cannot address (out of range, repeated pairs) are reported as an error: at once,
-    # or, with _defer_check (what qkv_sparse_cuda passes), by the next operator that waits for the stream;
-    # until then the two permutations of such input are all zero, so nothing reads out of bounds.
-    status = torch.zeros(2, dtype=torch.int32, pin_memory=True) if _defer_check else None
+    # Indices the kernels cannot address (out of range, repeated pairs) are reported as an error by this call (it
+    # waits for the stream); the two permutations of such input are all zero, so nothing reads out of bounds.
     with torch.cuda.device(d):
         _check_pending()
         _lib.check(lib.sswin_qkv_sparse_indices(_ptr(indices), n_vox, int(batch_size), int(spatial_dim),
                                                 int(num_heads), int(c), _ptr(idx_qv), _ptr(sorted_qv),
-                                                _ptr(idx_k), _ptr(sorted_k), _ptr(ws), nbytes,
-                                                0 if _defer_check else 1,
-                                                C.c_void_p(status.data_ptr()) if _defer_check else None, _stream(d)))
-        if _defer_check and n_vox > 0:
-            event = torch.cuda.Event()
-            event.record(torch.cuda.current_stream(d))
-            _pending.append((event, status, n_vox))
+                                                _ptr(idx_k), _ptr(sorted_k), _ptr(ws), nbytes, 1, None, _stream(d)))
     return idx_qv, sorted_qv, idx_k, sorted_k
 
 

@@ -92,7 +92,9 @@ class TokenPlan:
         self.tokens = torch.empty((1 if order_only else 5) * max(N, 1), dtype=torch.int32, device=d)
         self.plan = torch.empty(5 * self.g_cap, dtype=torch.int32, device=d)
         # group descriptors of the window-resident kernels, bucketed by ceil(c / 32)
-        self.tasks = torch.empty(16 * self.g_cap, dtype=torch.int32, device=d) if tasks else None
+        # (and behind them the token records, one per window and tile of 32 tokens)
+        self.tasks = (torch.empty(int(lib.sswin_token_plan_task_ints(N, self.g_cap, self.H)), dtype=torch.int32, device=d)
+                      if tasks else None)
         self.device = d
         self._totals = torch.zeros(9, dtype=torch.int64, pin_memory=True)
         self._indices = indices                      # kept alive until the kernels have run
@@ -371,7 +373,9 @@ def supports_resident(qkv: torch.Tensor, n: int) -> bool:
     return supports(qkv, n) and qkv.shape[-1] == 32 and n <= 128
 
 
-def supports(qkv: torch.Tensor, n: int) -> bool:
-    """The fused path covers fp32/fp16/bf16 on the GPU and windows of at most 128 positions
-    (bias-gradient LDS table); everything else takes the operator-by-operator path."""
-    return qkv.is_cuda and qkv.dtype in _DTYPE_CODE and n * n * 4 <= 64 * 1024
+def supports(qkv: torch.Tensor, n: int, table: bool = False) -> bool:
+    """The fused path covers fp32/fp16/bf16 on the GPU.  Windows: at most 128 positions when the bias gradient is
+    formed as an [H, n, n] array (its LDS table), at most 384 (7^3 = 343 included) when it goes straight to the
+    relative position table (``table``: the module has a :class:`BiasTableIndex`).  Everything else takes the
+    operator-by-operator path."""
+    return qkv.is_cuda and qkv.dtype in _DTYPE_CODE and (n <= 384 if table else n * n * 4 <= 64 * 1024)

@@ -116,11 +116,15 @@ def window_partition(x: torch.Tensor, window_size: List[int]) -> torch.Tensor:
     return x.permute(0, 1, 3, 5, 2, 4, 6, 7).contiguous().view(-1, wd * wh * ww, c)
 
 
-def compute_mask(dims: List[int], window_size: List[int], shift_size: List[int], device) -> torch.Tensor:
+def compute_mask(dims: List[int], window_size: List[int], shift_size: List[int], device, private: bool = False) -> torch.Tensor:
     """int8 [windows, tokens per window] region ids (27 regions) of the shifted grid.
 
     The reference assigns 27 slices of a dense volume and partitions it (ref ``:416-452``);
-    here one kernel evaluates the region of every (window, position) directly."""
+    here one kernel evaluates the region of every (window, position) directly.
+
+    The returned tensor is shared: every call with the same shapes, device and stream gets the same tensor
+    (``private=True`` returns a copy of its own).  A caller that writes into a shared mask is detected by the tensor's
+    version counter at the next call, which then builds the mask again."""
     device = torch.device(device)
     if device.type != "cuda":
         raise RuntimeError("compute_mask runs on the GPU only; there is no CPU fallback")
@@ -131,9 +135,9 @@ def compute_mask(dims: List[int], window_size: List[int], shift_size: List[int],
     key = (tuple(int(e) for e in dims), tuple(int(e) for e in window_size), tuple(int(e) for e in shift_size),
            device.index, torch.cuda.current_stream(device).cuda_stream)
     mask = _MASKS.get(key)
-    if mask is not None:
+    if mask is not None and mask._version == 0:              # written to by a caller: not the mask any more
         _MASKS.move_to_end(key)
-        return mask
+        return mask.clone() if private else mask
     windows = 1
     for extent, w in zip(dims, window_size):
         windows *= extent // w
@@ -145,7 +149,7 @@ def compute_mask(dims: List[int], window_size: List[int], shift_size: List[int],
     _MASKS[key] = mask
     while len(_MASKS) > 8 or (len(_MASKS) > 1 and sum(m.numel() for m in _MASKS.values()) > _MASK_CACHE_BYTES):
         _MASKS.popitem(last=False)
-    return mask
+    return mask.clone() if private else mask
 
 
 _MASKS = collections.OrderedDict()

@@ -737,9 +737,9 @@ class WindowAttentionSparse(nn.Module):
                 if cache is not None:
                     cache[self.num_heads] = plan
         qkv = tall_linear(x.features, self.qkv).reshape(-1, 3, self.num_heads, c // self.num_heads)
-        if plan is not None and self.fused and fused.supports(x.features, n):
+        table_index = self._table_index(n) if plan is not None and self.fused else None
+        if plan is not None and self.fused and fused.supports(x.features, n, table_index is not None):
             resident = fused.supports_resident(qkv, n) if self.resident is None else self.resident
-            table_index = self._table_index(n)
             if table_index is not None:
                 out = fused.fused_window_attention(qkv, self.relative_position_bias_table, x.indices, mask, b, n,
                                                    self.scale, resident, plan, table_index)

@@ -6,7 +6,7 @@ import os
 import numpy as np
 import pytest
 
-from helpers import close, product_mag
+from helpers import softmax_bwd_mag, close, product_mag
 
 GOLD = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "tiny_ops.npz")
 
@@ -43,7 +43,8 @@ def test_oracle_reproduces_golden(oracle, gold):
     o_idx, o_val, _, _ = oracle.matmul_cuda_naive(g["p"], s_idx, [B, H, n, n], v, qi, [B, H, n, hd], "qk_v")
     np.testing.assert_array_equal(o_idx, g["o_idx"])
     close(o_val, g["o_val"], 1e-12, "oracle qk_v", seg="all")
-    close(oracle.softmax_last_dim_backward(rows, g["p"], g["d_p"]), g["d_s"], 1e-12, "oracle softmax backward", seg=rows)
+    close(oracle.softmax_last_dim_backward(rows, g["p"], g["d_p"]), g["d_s"], 1e-12, "oracle softmax backward",
+          mag=softmax_bwd_mag(rows, g["p"], g["d_p"]))
     out, cnt = oracle.return_inverse(g["tok"], -1)
     np.testing.assert_array_equal(out, g["unsort"])
     assert cnt == int(g["n_unique"]) == len(g["ind"])
@@ -87,7 +88,7 @@ def test_hip_operators_reproduce_golden(oracle, gold):
     close(d_v.cpu().numpy(), g["d_v"], 1e-5, "dV",
           mag=gmag(oracle.qkv_transpose(f64(g["p"]), cc, hd, "rr"), oracle.qkv_transpose(f64(g["g_o"]), cc, hd, "rc"), "rr_rc"))
     d_s = ops.softmax_last_dim_backward(rows, dev(g["p"], f32), dev(g["d_p"], f32))
-    close(d_s.cpu().numpy(), g["d_s"], 1e-5, "dS", seg=g["rows"])
+    close(d_s.cpu().numpy(), g["d_s"], 1e-5, "dS", mag=softmax_bwd_mag(g["rows"], f64(g["p"]), f64(g["d_p"])))
     d_q = ops.matmul_grad_cuda_naive(dev(g["d_s"], f32), dev(kt, f32), c, hd, "rr_rc")
     close(d_q.cpu().numpy(), g["d_q"], 1e-5, "dQ", mag=gmag(g["d_s"], kt, "rr_rc"))
     d_kt = ops.matmul_grad_cuda_naive(ops.qkv_transpose(dev(q, f32), c, hd, "rc"),

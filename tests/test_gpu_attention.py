@@ -73,10 +73,13 @@ def test_window_attention_forward_backward(shift, dim, heads, path):
           leaves["relative_position_bias_table"].grad.numpy(), 1e-5, "d bias table", mag=leaves["table_mag"]())
 
 
-def test_window_7_heads_of_16_channels_runs_the_operator_path():
-    """The reference's own ScanNet setting: windows of 7^3 = 343 positions, shift 3, 48 channels in 3 heads of 16.
-    Windows above 128 positions are outside the fused kernels, so the module takes the operator path by itself
-    (``fused`` left at its default); forward and backward against the fp64 CPU path."""
+@pytest.mark.parametrize("path", ["fused", "operators"])
+def test_window_7_heads_of_16_channels(path):
+    """The reference's own ScanNet setting (config/scannet/semseg-swin-0-base.py:11-31): windows of 7^3 = 343
+    positions, shift 3, 48 channels in 3 heads of 16.  Heads of 16 channels and windows above 128 positions are
+    outside the window-resident kernels; the module's default is the fused path (block products that read the token
+    rows through the token plan, attention matrix in memory, bias gradient straight into the table), the operator
+    path is the reference's own composition.  Forward and backward against the fp64 CPU path."""
     from sparseswin3d_amd import synth
     from sparseswin3d_amd.window_attention import SparseVoxelTensor, WindowAttentionSparse
     torch.manual_seed(4)
@@ -86,6 +89,8 @@ def test_window_7_heads_of_16_channels_runs_the_operator_path():
     assert n == 343
     N = len(win_idx)
     attn = WindowAttentionSparse(48, 3, ws, qkv_bias=True).cuda()
+    if path == "operators":
+        set_path(attn, path)                                 # "fused" is what the module picks by itself here
     with torch.no_grad():
         attn.relative_position_bias_table.normal_(0, 0.5)
     mask_np = synth.shift_region_mask(synth.padded_shape(grid, ws), ws, shift)

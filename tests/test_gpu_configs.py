@@ -15,7 +15,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import PATHS, BiasGradMagnitude, close, product_mag, qkv_operands, set_path
+from helpers import softmax_bwd_mag, PATHS, BiasGradMagnitude, close, product_mag, qkv_operands, set_path
 
 pytestmark = pytest.mark.gpu
 
@@ -103,7 +103,8 @@ def test_operator_chain_full_size(ops, oracle, cfg, shift, dtype):
     assert np.all(np.abs(sums[row_max >= 0] - 1.0) < 1e-5)
     gp = dev(rng.standard_normal(len(r_val)), torch.float32)
     gs = ops.softmax_last_dim_backward(rows, p, gp)
-    close(host(gs), oracle.softmax_last_dim_backward(r_rows, host(p), host(gp)), 1e-5, "softmax backward", seg=r_rows)
+    close(host(gs), oracle.softmax_last_dim_backward(r_rows, host(p), host(gp)), 1e-5, "softmax backward",
+          mag=softmax_bwd_mag(r_rows, host(p), host(gp)))
     zero = np.bincount(r_rows, weights=host(gs))
     assert np.all(np.abs(zero) < 1e-4 * max(1.0, np.abs(host(gs)).max()))   # softmax gradient rows sum to 0
 
@@ -192,13 +193,14 @@ def test_cfg1_forward_against_cpu_path(path):
     close(host(out), ref.numpy(), 1e-5, "cfg1 forward")
 
 
-@pytest.mark.parametrize("cfg,path", [("cfg2", "resident"), ("cfg2", "fused"), ("cfg3", "resident"), ("cfg3", "fused"),
-                                      ("cfg3", "operators")])
-def test_shifted_forward_backward_against_cpu_path(cfg, path):
-    """Configurations 2 (second block of the pair) and 3: shifted windows with the region mask,
-    fp32 forward + backward with N(0,1) upstream gradients."""
+@pytest.mark.parametrize("cfg,path,shift", [("cfg2", "resident", 2), ("cfg2", "fused", 2), ("cfg2", "operators", 2),
+                                            ("cfg2", "resident", 0), ("cfg3", "resident", 2), ("cfg3", "fused", 2),
+                                            ("cfg3", "operators", 2)])
+def test_forward_backward_against_cpu_path(cfg, path, shift):
+    """Configurations 2 (both blocks of the pair: regular windows, then shifted windows with the region mask) and 3
+    (shifted): fp32 forward + backward with N(0,1) upstream gradients, at full size."""
     w = _workload(cfg)
-    idx, B, n, mask = _windows(w, (2, 2, 2))
+    idx, B, n, mask = _windows(w, (shift, shift, shift))
     attn = _attention(w.dim, w.heads, torch.float32)
     set_path(attn, path)
     torch.manual_seed(2)

@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import PATHS, close, ragged_window_indices, random_window_indices, set_path
+from helpers import score_grad_mag, PATHS, close, ragged_window_indices, random_window_indices, set_path
 
 pytestmark = pytest.mark.gpu
 
@@ -81,10 +81,29 @@ def test_token_plans_in_one_batch_equal_single_plans():
         assert torch.equal(tp.plan.view(5, -1)[:, :tp.G], one.plan.view(5, -1)[:, :one.G])
         if spec[4] and tp.G:
             # descriptors of a bucket, as sets: their order inside a bucket is the same here, but not promised
-            a, b = tp.tasks.view(4, tp.g_cap, 4), one.tasks.view(4, one.g_cap, 4)
+            a, b = tp.tasks[:16 * tp.g_cap].view(4, tp.g_cap, 4), one.tasks[:16 * one.g_cap].view(4, one.g_cap, 4)
             for k in range(4):
                 m = int(tp.bucket_counts[k])
                 assert torch.equal(a[k, :m], b[k, :m])
+            # the token records behind the descriptors: one per (window, tile of 32 tokens), the bucket of four tiles
+            # first, inside a bucket by window, then tile; entry l = (voxel, pos) of token 32 tile + l of the window,
+            # the window's last token again behind it
+            H = spec[3]
+            n_rec = sum(int(tp.bucket_counts[k]) // H * (k + 1) for k in range(4))
+            ra = tp.tasks[16 * tp.g_cap:16 * tp.g_cap + 64 * n_rec].view(n_rec, 32, 2).cpu().numpy()
+            rb = one.tasks[16 * one.g_cap:16 * one.g_cap + 64 * n_rec].view(n_rec, 32, 2).cpu().numpy()
+            np.testing.assert_array_equal(ra, rb)
+            tok = tp.tokens.view(5, -1).cpu().numpy()
+            desc = a.cpu().numpy()
+            first = 0
+            for k in (3, 2, 1, 0):
+                for wslot in range(int(tp.bucket_counts[k]) // H):
+                    T, c = int(desc[k, wslot * H, 0]), int(desc[k, wslot * H, 1]) & 0xff
+                    for tile in range(k + 1):
+                        ranks = T + np.minimum(32 * tile + np.arange(32), c - 1)
+                        want = np.stack([tok[0, ranks], tok[3, ranks]], 1)
+                        np.testing.assert_array_equal(ra[first + wslot * (k + 1) + tile], want)
+                first += int(tp.bucket_counts[k]) // H * (k + 1)
     # a plan that keeps the voxel order only (what the stride-2 merge reads) holds the same first row and group table
     lean = TokenPlan(dev[4][0], 3000, 8, 1, tasks=False, order_only=True)
     assert lean.tokens.numel() == lean.N and torch.equal(lean.tokens, plans[4].tokens[:lean.N])
@@ -180,13 +199,16 @@ def test_fused_16bit_against_cpu_fp64(dtype, path):
     close(out.detach().double().cpu().numpy(), ref.numpy(), 2e-2, f"{path} {dtype}")
 
 
+@pytest.mark.parametrize("family", ["fp32mfma", "x16"])
 @pytest.mark.parametrize("mix", ["tiny", "edges", "full", "mixed"])
 @pytest.mark.parametrize("use_mask", [False, True], ids=["nomask", "mask"])
-def test_resident_kernels_on_ragged_windows(mix, use_mask):
+def test_resident_kernels_on_ragged_windows(mix, use_mask, family, monkeypatch):
     """Window-resident forward/backward through the C ABI on hand-picked occupancies (1 token,
     around the 32/64/96 tile edges, full 125-token windows, empty slots) against dense fp64
-    attention per window; also checks the bucket counts of the task list."""
+    attention per window; also checks the bucket counts of the task list.  Both kernel families on fp32 tokens:
+    the fp32 matrix instructions and the 16-bit operands with every value split into two fp16 pieces."""
     import ctypes as C
+    monkeypatch.setenv("SSWIN_WATTN", family)
     from sparseswin3d_amd import _lib
     from sparseswin3d_amd.fused import TokenPlan, _ptr
     mixes = {"tiny": [1, 2, 3, 1, 5, 4], "edges": [31, 32, 33, 0, 63, 64, 65, 1, 95, 96, 97],
@@ -231,6 +253,10 @@ def test_resident_kernels_on_ragged_windows(mix, use_mask):
     ref = torch.zeros(N, D, dtype=torch.float64)
     order = np.lexsort((ind[:, 1], ind[:, 0]))
     pieces = []
+    bias_mag = torch.zeros(H, n, n, dtype=torch.float64)
+    plan_h = tp.plan.view(5, -1)[:, :tp.G].cpu().numpy()       # rows: c, first row, first entry, window, head
+    sq_of = {(int(plan_h[3, g]), int(plan_h[4, g])): int(plan_h[2, g]) for g in range(tp.G)}
+    ds_ref, ds_mag = np.zeros(tp.A), np.zeros(tp.A)
     for w in np.unique(ind[:, 0]):
         vox = torch.from_numpy(order[ind[order, 0] == w])
         pos = torch.from_numpy(ind[vox.numpy(), 1].astype(np.int64))
@@ -243,6 +269,17 @@ def test_resident_kernels_on_ragged_windows(mix, use_mask):
         e = (s - m).exp()
         p = e / (e.sum(-1, keepdim=True) + 1e-8)
         pieces.append((vox, torch.einsum("hij,jhc->ihc", p, x[:, 2]).reshape(len(vox), D)))
+        with torch.no_grad():           # dS = P (dP - D) itself and what it is conditioned by, per entry and per bias cell
+            dO_w = do32.double().cpu()[vox].reshape(len(vox), H, hd)
+            O_w = pieces[-1][1].reshape(len(vox), H, hd)
+            cw = len(vox)
+            for hh in range(H):
+                mag_wh = score_grad_mag(p[hh], dO_w[:, hh], x[:, 2, hh], O_w[:, hh])
+                bias_mag[hh][pos[:, None], pos[None, :]] += mag_wh
+                dP = dO_w[:, hh] @ x[:, 2, hh].t()
+                sq0 = sq_of[(int(w), hh)]
+                ds_ref[sq0:sq0 + cw * cw] = (p[hh] * (dP - (dO_w[:, hh] * O_w[:, hh]).sum(-1, keepdim=True))).reshape(-1).numpy()
+                ds_mag[sq0:sq0 + cw * cw] = mag_wh.reshape(-1).numpy()
     ref = torch.zeros(N, D, dtype=torch.float64).index_put((torch.cat([v for v, _ in pieces]),),
                                                             torch.cat([o for _, o in pieces]))
     ref.backward(do32.double().cpu())
@@ -257,17 +294,16 @@ def test_resident_kernels_on_ragged_windows(mix, use_mask):
             _ptr(q32), 3 * D, 2 * D, C.c_float(scale), _ptr(b32), n, _ptr(m_dev), nmw, _ptr(out), D, 0, _ptr(do32), D, 0,
             _ptr(lse), _ptr(part), 3 * D, 0, _ptr(part), 3 * D, D, _ptr(part), 3 * D, 2 * D, _ptr(ds2), sides, stream))
         got, want_g = part.cpu().numpy(), qkv_r.grad.numpy()
-        close(got[:, cols], want_g[:, cols], 1e-5, f"sides={sides}")
+        # a token's dQ alone can be zero where dK and dV are not (a window of one token: dS = P (dP - D) = 0 from two
+        # equal numbers of ordinary size): measured against the token's whole gradient row
+        close(got[:, cols], want_g[:, cols], 1e-5, f"sides={sides}",
+              mag=np.abs(want_g[:, cols]) + np.abs(want_g).max(axis=1, keepdims=True))
         other = np.ones(3 * D, bool)
         other[cols] = False
         assert np.isnan(got[:, other]).all()                 # the other side is not touched
         if sides != 1:
-            # the same dS (groups of at most 16 tokens take another kernel path in the one-launch backward, so
-            # the two agree to rounding, not bit for bit)
-            c_g = tp.plan.view(5, -1)[0, :tp.G].cpu().numpy()
-            row_len = np.repeat(c_g, c_g)                     # every attention row of a group holds c entries
-            close(ds2.cpu().numpy(), ds.cpu().numpy(), 1e-5, "dS of the key-side kernel",
-                  seg=np.repeat(np.arange(len(row_len)), row_len))
+            close(ds2.cpu().numpy(), ds_ref, 1e-5, "dS of the key-side kernel", mag=ds_mag)
+    close(ds.cpu().numpy(), ds_ref, 1e-5, "dS of the one-launch backward", mag=ds_mag)
     # bias gradient from the stored dS
     d_bias = torch.zeros(H, n, n, device="cuda")
     nbytes = lib.sswin_fused_bias_grad_workspace_bytes(tp.G, H, n)
@@ -275,16 +311,7 @@ def test_resident_kernels_on_ragged_windows(mix, use_mask):
     _lib.check(lib.sswin_fused_bias_grad(_ptr(tp.plan), tp.g_cap, tp.G, _ptr(tp.tokens), N, H, n, _ptr(ds), _ptr(d_bias),
                                          _ptr(ws), nbytes, stream))
     assert not torch.isnan(ds).any()
-    # measured against sum |dS| over the entries a bias cell sums (dS itself was compared above)
-    plan_h = tp.plan.view(5, -1)[:, :tp.G].cpu().numpy()
-    pos_h = tp.tokens.view(5, -1)[3].cpu().numpy()
-    ds_h = np.abs(ds.cpu().numpy().astype(np.float64))
-    mag = np.zeros((H, n, n))
-    for g in range(tp.G):
-        c, T, sq, _, h = (int(v) for v in plan_h[:, g])
-        pg = pos_h[T:T + c]
-        np.add.at(mag[h], (pg[:, None], pg[None, :]), ds_h[sq:sq + c * c].reshape(c, c))
-    close(d_bias.cpu().numpy(), bias_r.grad.numpy(), 1e-5, "d bias", mag=mag)
+    close(d_bias.cpu().numpy(), bias_r.grad.numpy(), 1e-5, "d bias", mag=bias_mag.numpy())
 
 
 @pytest.mark.parametrize("mix,H", [("tiny", 1), ("mixed", 3), ("full", 2), ("many", 3), ("crowd", 3)])

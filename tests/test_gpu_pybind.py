@@ -7,7 +7,7 @@ import numpy as np
 import pytest
 import torch
 
-from helpers import close, product_mag, qkv_operands, ragged_window_indices
+from helpers import softmax_bwd_mag, close, product_mag, qkv_operands, ragged_window_indices
 
 pytestmark = pytest.mark.gpu
 
@@ -96,7 +96,8 @@ def test_products_softmax_gradients_transposes(mods, oracle, case):
     same(p, ct.softmax_last_dim_forward(rows, s_val))
     gp = dev(np.random.default_rng(5).standard_normal(p.numel()), torch.float32)
     gs = pb.softmax_last_dim_backward(rows, p, gp)
-    close(host(gs), oracle.softmax_last_dim_backward(r_rows, host(p), host(gp)), 1e-5, "softmax backward", seg=r_rows)
+    close(host(gs), oracle.softmax_last_dim_backward(r_rows, host(p), host(gp)), 1e-5, "softmax backward",
+          mag=softmax_bwd_mag(r_rows, host(p), host(gp)))
     same(gs, ct.softmax_last_dim_backward(rows, p, gp))
 
     o_idx, o_val, o_shape, c2 = pb.matmul_cuda_naive(p, s_idx, list(s_shape), v, qi, d["q_shape"], "qk_v")
@@ -117,6 +118,27 @@ def test_products_softmax_gradients_transposes(mods, oracle, case):
         out = pb.qkv_transpose(a, c, HD, kind)
         np.testing.assert_array_equal(host(out), oracle.qkv_transpose(host(a), r_c, HD, kind))
         same(out, ct.qkv_transpose(a, c, HD, kind))
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+def test_softmax_takes_16_bit_values(mods, oracle, dtype):
+    """The reference dispatches its softmax over the floating types and half (ops.cu:140, 155, 183): 16-bit values are
+    computed in fp32 and rounded once, the same as the ctypes module."""
+    pb, ct = mods
+    rng = np.random.default_rng(8)
+    rows_np = np.repeat(np.arange(40), rng.integers(1, 60, 40)).astype(np.int32)
+    rows = dev(rows_np)
+    v = dev(rng.standard_normal(len(rows_np)) * 2.0, dtype)
+    g = dev(rng.standard_normal(len(rows_np)), dtype)
+    y = pb.softmax_last_dim_forward(rows, v)
+    assert y.dtype == dtype
+    close(host(y), oracle.softmax_last_dim_forward(rows_np, host(v)), 2e-2, f"softmax forward {dtype}", seg=rows_np)
+    same(y, ct.softmax_last_dim_forward(rows, v))
+    gx = pb.softmax_last_dim_backward(rows, y, g)
+    assert gx.dtype == dtype
+    close(host(gx), oracle.softmax_last_dim_backward(rows_np, host(y), host(g)), 2e-2, f"softmax backward {dtype}",
+          mag=softmax_bwd_mag(rows_np, host(y), host(g)))
+    same(gx, ct.softmax_last_dim_backward(rows, y, g))
 
 
 def test_error_behaviour(mods):

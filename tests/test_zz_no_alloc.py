@@ -32,11 +32,20 @@ def _both(lib, keys_np, code):
     _lib.check(lib.sswin_unique_consecutive_indices(C.c_void_p(keys.data_ptr()), code, m, C.c_void_p(want.data_ptr()),
                                                     C.c_void_p(ws.data_ptr()), nbytes, stream))
     got = torch.full((m,), -2, dtype=torch.int32, device=dev)
+    # a first call may load the code object; the second one must leave the device's free memory as it was (the
+    # driver's own count: an allocation inside the library would show there, not in PyTorch's allocator)
+    _lib.check(lib.sswin_unique_consecutive_indices_static(C.c_void_p(keys.data_ptr()), code, m,
+                                                           C.c_void_p(got.data_ptr()), stream))
+    torch.cuda.synchronize()
+    got.fill_(-2)
+    torch.cuda.synchronize()
+    free_before = torch.cuda.mem_get_info(dev)[0]
     before = torch.cuda.memory_allocated(dev)
     _lib.check(lib.sswin_unique_consecutive_indices_static(C.c_void_p(keys.data_ptr()), code, m,
                                                            C.c_void_p(got.data_ptr()), stream))
-    assert torch.cuda.memory_allocated(dev) == before
     torch.cuda.synchronize()
+    assert torch.cuda.memory_allocated(dev) == before
+    assert torch.cuda.mem_get_info(dev)[0] == free_before
     return got.cpu().numpy(), want.cpu().numpy()
 
 
