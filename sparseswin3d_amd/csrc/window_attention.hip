@@ -525,11 +525,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 //   KV_SINGLE  a group of one tile: dS is already in registers; transposed through LDS it is the A
 //              operand of dQ = dS K, which saves the group its whole query-side task
 //   KV_PAIR    a group of two tiles, its two key-side tasks on neighbouring wavefronts of one
-//              workgroup: each forms dS K for both query tiles, hands the partial result of the other
-//              wavefront's tile over through an LDS exchange tile, and after one workgroup barrier adds
-//              the two partial results of its own tile.  S and dP of the group are then computed once
-//              instead of twice (320 instead of 448 MFMA steps of 32x32x2 per group) and the five
-//              operands are read once.
+//              workgroup: each forms dS K for both query tiles, query tile 0 first, and puts the partial
+//              result into its LDS exchange tile; after a workgroup barrier the wavefront that owns the
+//              query tile adds the two parts.  S and dP of the group are then computed once instead of
+//              twice (320 instead of 448 MFMA steps of 32x32x2 per group), and because both wavefronts
+//              ask for the same query tile at the same time its rows leave memory once.
 enum { KV_ONLY = 0, KV_SINGLE = 1, KV_PAIR = 2 };
 
 // xch: this wavefront's exchange tile (KV_PAIR), xch_peer: the other wavefront's; accumulator layout
@@ -726,12 +726,13 @@ __device__ __forceinline__ void bwd_kv_task(const WAttnCommon& a, int64_t task, 
     int64_t d, rec;
     int bj;
     if (!live || !locate(a, task, d, bj, rec)) {
-        if (DQ == KV_PAIR) __syncthreads();
+        if (DQ == KV_PAIR)
+            for (int k = 0; k < 4; ++k) __syncthreads();     // the barriers of a live pair (pair_dq, twice)
         return;
     }
     const PadTab tab_pos = pad_tab(tile_q, 0), tab_L = pad_tab(tile_q, 1), tab_D = pad_tab(tile_q, 2);
     // the descriptor, the keys' indices and those of the first query tile: one round trip
-    const int t_first = DQ == KV_PAIR ? 1 - bj : 0;           // KV_PAIR: the other wavefront's query tile first
+    const int t_first = 0;
     const int4 desc = a.tasks[d];
     const int64_t rec0 = rec - bj;
     const int2 e_k = token_entry(a, rec, l32), e_q0 = token_entry(a, rec0 + t_first, l32);
@@ -800,10 +801,8 @@ __device__ __forceinline__ void bwd_kv_task(const WAttnCommon& a, int64_t task, 
 
     f32x16 dk = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     f32x16 dv = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
-    f32x16 dq_own;                                            // KV_PAIR: dS K of this wavefront's own query tile
     // One query tile t against this task's keys.  What happens to dS K of the tile (dq_tag): 0 = not
-    // formed, 1 = written out as dQ of a one-tile group, 2 = handed to the other wavefront of the pair,
-    // 3 = kept in dq_own.
+    // formed, 1 = written out as dQ of a one-tile group, 2 = put into this wavefront's exchange tile (KV_PAIR).
     // rq, rdo, ro hold the rows of query tile t (requested by the caller), qi its indices.
     auto tile_pass = [&](const int t, const QIdx& qi, auto dq_tag) {
         constexpr int DQ_USE = decltype(dq_tag)::value;
@@ -937,9 +936,6 @@ __device__ __forceinline__ void bwd_kv_task(const WAttnCommon& a, int64_t task, 
             if constexpr (DQ_USE == 2) {
                 xch_put(xch, lane, dq);
                 __builtin_amdgcn_wave_barrier();
-            } else if constexpr (DQ_USE == 3) {
-                dq_own = dq;
-                __builtin_amdgcn_wave_barrier();
             } else {
 #pragma unroll
                 for (int r = 0; r < 16; ++r) dq[r] *= LN2;
@@ -957,12 +953,34 @@ __device__ __forceinline__ void bwd_kv_task(const WAttnCommon& a, int64_t task, 
         rows_load<T>(dobase, dopitch, qi.vox, lane, rdo);
         rows_load<T>(obase, opitch, qi.vox, lane, ro);
     };
+    // KV_PAIR: the wavefront that owns query tile `own` adds the two partial products dS K of that tile, which both
+    // wavefronts have put into their exchange tiles, and writes dQ.  Workgroup barriers before (both parts are there)
+    // and after the reads (the exchange tiles may be written again).
+    auto pair_dq = [&](const bool own) {
+        __syncthreads();
+        f32x16 dq = f32x16{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        if (own) {
+            xch_add(xch, lane, dq);
+            xch_add(xch_peer, lane, dq);
+        }
+        __syncthreads();
+        if (own) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) dq[r] *= LN2;
+            tile_put_acc(tile_do, l32, half, dq);
+            __builtin_amdgcn_wave_barrier();
+            tile_store_rows<T>(tile_do, const_cast<char*>(head_base<T>(tdq, h)), pitch_of<T>(tdq), vox_j, c - bj * 32, lane);
+            __builtin_amdgcn_wave_barrier();
+        }
+    };
     if constexpr (DQ == KV_PAIR) {
-        // the other wavefront's query tile first, the own one last (its result stays in registers)
-        const QIdx qown = load_qidx(bj);
-        tile_pass(1 - bj, qcur, std::integral_constant<int, 2>{});
-        request_rows(qown);
-        tile_pass(bj, qown, std::integral_constant<int, 3>{});
+        // Both wavefronts of the pair take query tile 0 first and tile 1 second, so their requests for a tile's rows
+        // go out together and meet in the compute unit's cache: the rows leave memory once, not twice.
+        const QIdx q1 = load_qidx(1);
+        tile_pass(0, qcur, std::integral_constant<int, 2>{});
+        request_rows(q1);
+        pair_dq(bj == 0);
+        tile_pass(1, q1, std::integral_constant<int, 2>{});
     } else if constexpr (DQ == KV_SINGLE) {
         tile_pass(0, qcur, std::integral_constant<int, 1>{});     // groups of one tile only
     } else {
@@ -982,15 +1000,7 @@ __device__ __forceinline__ void bwd_kv_task(const WAttnCommon& a, int64_t task, 
     __builtin_amdgcn_wave_barrier();
     tile_store_rows<T>(tile_q, const_cast<char*>(head_base<T>(tdk, h)), pitch_of<T>(tdk), vox_j, c - bj * 32, lane);
     tile_store_rows<T>(tile_do, const_cast<char*>(head_base<T>(tdv, h)), pitch_of<T>(tdv), vox_j, c - bj * 32, lane);
-    if (DQ == KV_PAIR) {
-        __syncthreads();                                     // both partial results of every pair are in LDS
-        xch_add(xch_peer, lane, dq_own);
-#pragma unroll
-        for (int r = 0; r < 16; ++r) dq_own[r] *= LN2;
-        tile_put_acc(tile_do, l32, half, dq_own);
-        __builtin_amdgcn_wave_barrier();
-        tile_store_rows<T>(tile_do, const_cast<char*>(head_base<T>(tdq, h)), pitch_of<T>(tdq), vox_j, c - bj * 32, lane);
-    }
+    if constexpr (DQ == KV_PAIR) pair_dq(bj == 1);
 }
 
 template <typename T, bool MASK>
