@@ -165,7 +165,7 @@ def run_encoder(wl):
 
 def bench_encoder(device, args):
     """`--workload cfg5`: the forward pass of the four-stage encoder, timed as a whole."""
-    from sparseswin3d_amd import fused
+    from sparseswin3d_amd import _lib
     wl = build_encoder(device)
     counts = run_encoder(wl)
     log(f"workload {wl['name']}: voxels per stage {counts}")
@@ -177,13 +177,13 @@ def bench_encoder(device, args):
         run_encoder(wl)
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / args.steps
-    fused.launch_timer = []
+    _lib.launch_timer = []
     for _ in range(5):
         run_encoder(wl)
     torch.cuda.synchronize()
     per_stage = [[] for _ in wl["stages"]]
-    fw = [(a, b) for name, a, b in fused.launch_timer if name == "window_attention_forward"]
-    fused.launch_timer = None
+    fw = [(a, b) for name, _, a, b in _lib.launch_timer if name == "window_attention_forward"]
+    _lib.launch_timer = None
     for i, (a, b) in enumerate(fw):
         per_stage[i % len(per_stage)].append(a.elapsed_time(b))
     stage_ms = [sum(v) / len(v) for v in per_stage]
@@ -240,14 +240,22 @@ DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 
 # table name of a kernel -> (substring of its symbol in a rocprofv3 trace, source files it is built from)
 KERNEL_SYMBOLS = {
-    "resident forward": ("wattn_fwd_kernel", ["sparseswin3d_amd/csrc/window_attention.hip"]),
-    "resident backward (dQ,dK,dV,dS)": ("wattn_bwd_all_kernel", ["sparseswin3d_amd/csrc/window_attention.hip"]),
+    # fp32 tokens run the kernels of window_attention.hip (wattn_*), 16-bit tokens those of window_attention_x16.hip (wattn16_*)
+    "resident forward": ("_fwd_kernel", ["sparseswin3d_amd/csrc/window_attention.hip", "sparseswin3d_amd/csrc/window_attention_x16.hip",
+                                         "sparseswin3d_amd/csrc/wattn_common.hpp"]),
+    "resident backward (dQ,dK,dV,dS)": ("_bwd_all_kernel", ["sparseswin3d_amd/csrc/window_attention.hip",
+                                                            "sparseswin3d_amd/csrc/window_attention_x16.hip",
+                                                            "sparseswin3d_amd/csrc/wattn_common.hpp"]),
     "block_matmul q_k, values": ("block_product_mfma_kernel<float, 0", ["sparseswin3d_amd/csrc/block_matmul.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
     "block_matmul qk_v, values": ("block_product_mfma_kernel<float, 1, false", ["sparseswin3d_amd/csrc/block_matmul.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
     "block_matmul qk_v (values + index matrix)": ("block_product_mfma_kernel<float, 1, true", ["sparseswin3d_amd/csrc/block_matmul.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
     "grad rc_cr": ("block_product_mfma_kernel<float, 2", ["sparseswin3d_amd/csrc/block_matmul.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
     "grad rr_rc": ("block_product_mfma_kernel<float, 3", ["sparseswin3d_amd/csrc/block_matmul.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
     "grad cr_rr": ("block_product_mfma_kernel<float, 4", ["sparseswin3d_amd/csrc/block_matmul.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
+    "grad tr_rc (dV = P^T dO)": ("block_product_mfma_kernel<float, 5", ["sparseswin3d_amd/csrc/block_matmul.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
+    "grad tc_rr (dK^T = Q^T dS)": ("block_product_mfma_kernel<float, 6", ["sparseswin3d_amd/csrc/block_matmul.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
+    "operand_copy_qkv": ("qkv_order_copy_kernel", ["sparseswin3d_amd/csrc/index_ops.hip"]),
+    "bias + mask add, one pass [A]": ("group_bias_mask_kernel", ["sparseswin3d_amd/csrc/softmax.hip"]),
     "transpose rc": ("block_transpose_kernel<float, false", ["sparseswin3d_amd/csrc/block_matmul.hip"]),
     "transpose rr": ("block_transpose_kernel<float, true", ["sparseswin3d_amd/csrc/block_matmul.hip"]),
     "softmax_last_dim_forward": ("softmax_rows_kernel<float, false", ["sparseswin3d_amd/csrc/softmax.hip"]),
@@ -256,6 +264,59 @@ KERNEL_SYMBOLS = {
     "fused dV=P^T dO": ("fused_tok_kernel", ["sparseswin3d_amd/csrc/fused_attention.hip"]),
     "fused O=PV": ("fused_tok_kernel", ["sparseswin3d_amd/csrc/fused_attention.hip"]),
 }
+
+
+# operator-path table row -> (library entry point, leading integer arguments or None for any) of the launch it times
+OPERATOR_LAUNCHES = {
+    "token plan, one of a stage's two (operand map + group table)": ("sswin_token_plan", None),
+    "sorted_coo_indices [4,E], Q/V": ("sswin_sorted_coo_indices", None),
+    "operand_copy_qkv, voxel rows -> Q*scale, K^T, V": ("sswin_operand_copy_qkv", (0, 1)),
+    "operand_copy_qkv, gradients -> voxel rows": ("sswin_operand_copy_qkv", (0, 0)),
+    "operand_copy Q/V order, operand -> voxel rows": ("sswin_operand_copy", (0, 0, 0)),
+    "operand_copy Q/V order, voxel rows -> operand": ("sswin_operand_copy", (0, 0, 1)),
+    "block_matmul q_k, values": ("sswin_block_matmul", (0, 0)),
+    "bias + mask add, one pass [A]": ("sswin_group_add_table_bias_mask", None),
+    "bias table gradient from the product's groups": ("sswin_bias_table_grad", None),
+    "softmax rows from the group sizes [A]": ("sswin_softmax_rows_from_counts", None),
+    "softmax_last_dim_forward": ("sswin_softmax_last_dim_forward", None),
+    "block_matmul qk_v, values": ("sswin_block_matmul", (1, 0)),
+    "softmax_last_dim_backward": ("sswin_softmax_last_dim_backward", None),
+    "grad rc_cr": ("sswin_block_matmul_grad", (0, 0)),
+    "grad rr_rc": ("sswin_block_matmul_grad", (1, 0)),
+    "grad tr_rc (dV = P^T dO)": ("sswin_block_matmul_grad", (3, 0)),
+    "grad tc_rr (dK^T = Q^T dS)": ("sswin_block_matmul_grad", (4, 0)),
+}
+
+
+def operators_in_module(wl, reps=5):
+    """Every library launch of one attention module call (forward + backward, regular windows) on the operator path,
+    timed where it runs: HIP events around each launch on its stream.  Returns {(entry point, leading integer
+    arguments): (mean ms, launches per call)}."""
+    from sparseswin3d_amd import _lib
+    from sparseswin3d_amd.window_attention import SparseVoxelTensor
+    b = wl["blocks"][0]
+    attn = b["attn"]
+    keep = (attn.fused, attn.resident)
+    attn.fused, attn.resident = False, None
+
+    def once():
+        attn.zero_grad(set_to_none=True)
+        x = wl["feats"].detach().requires_grad_(True)
+        attn(SparseVoxelTensor(x, b["idx"], (b["n"],), b["slots"]), None).features.backward(wl["upstream"])
+
+    for _ in range(3):
+        once()
+    torch.cuda.synchronize()
+    _lib.launch_timer = []
+    for _ in range(reps):
+        once()
+    torch.cuda.synchronize()
+    acc = {}
+    for name, ints, start, stop in _lib.launch_timer:
+        acc.setdefault((name, ints), []).append(start.elapsed_time(stop))
+    _lib.launch_timer = None
+    attn.fused, attn.resident = keep
+    return {k: (sum(v) / len(v), len(v) / reps) for k, v in acc.items()}
 
 
 def kernel_table(wl, reps=20, only=None):
@@ -336,12 +397,14 @@ def kernel_table(wl, reps=20, only=None):
         omap = ops.operand_map(b["idx"], b["slots"], b["n"])
         feat_rows = torch.randn(N, D, device=dev)
         qkv_rows = qkv.view(N, 3 * D)
-        val_e = torch.empty(E, device=dev)
+        val_e, val_e2, val_e3 = (torch.empty(E, device=dev) for _ in range(3))
+        qkv_rows_out = torch.empty_like(qkv_rows)
 
         gp = ops.group_plan(c)
         row_pos = ops.group_row_positions(s_idx, gp)
         bias_d = torch.randn(H, b["n"], b["n"], device=dev)
         n_table_o = int(wl["blocks"][0]["attn"].relative_position_bias_table.shape[0])
+        table_o = wl["blocks"][0]["attn"].relative_position_bias_table.detach().float().contiguous()
         ti_o = F.BiasTableIndex.build(relative_position_index_3d(wl["blocks"][0]["attn"].window_size).to(dev), n_table_o)
 
         entries = [
@@ -354,13 +417,19 @@ def kernel_table(wl, reps=20, only=None):
             # reads them (rows with 0 calls below: what the reference's operators always write)
             ("sorted_coo_indices [4,E], Q/V", lambda: ops.sorted_coo_indices(b["idx"], omap, H, hd, k=False), 16 * E + 20 * N, 1),
             ("sorted_coo_indices [4,E] x 2 (with K^T's)", lambda: ops.sorted_coo_indices(b["idx"], omap, H, hd), 32 * E + 20 * N, 0),
-            ("operand_copy Q/V order", lambda: ops.operand_copy(qkv_rows, 2 * D, val_e, omap, H, hd, 0, True), 2 * s * E, 6),
-            ("operand_copy K^T order", lambda: ops.operand_copy(qkv_rows, D, val_e, omap, H, hd, 1, True), 2 * s * E, 2),
+            # the module copies Q (times the attention scale), K^T and V in one launch each way, and the attention output
+            # to voxel rows (and its gradient back) with one Q/V-order copy each
+            ("operand_copy_qkv, voxel rows -> Q*scale, K^T, V", lambda: ops.operand_copy_qkv(qkv_rows, val_e, val_e2, val_e3, omap, H, hd, True, 0.17), 6 * s * E, 1),
+            ("operand_copy_qkv, gradients -> voxel rows", lambda: ops.operand_copy_qkv(qkv_rows_out, val_e, val_e2, val_e3, omap, H, hd, False, 0.17), 6 * s * E, 1),
+            ("operand_copy Q/V order, operand -> voxel rows", lambda: ops.operand_copy(feat_rows, 0, val_e, omap, H, hd, 0, False), 2 * s * E, 1),
+            ("operand_copy Q/V order, voxel rows -> operand", lambda: ops.operand_copy(qkv_rows, 2 * D, val_e, omap, H, hd, 0, True), 2 * s * E, 1),
+            ("operand_copy K^T order", lambda: ops.operand_copy(qkv_rows, D, val_e, omap, H, hd, 1, True), 2 * s * E, 0),
             ("qkv_sparse_indices (reference operator)", lambda: ops.qkv_sparse_indices(b["idx"], b["slots"], b["n"], H, hd), 8 * N + 40 * E, 0),
             ("plan_from_indices (group table from a [4,E] index matrix)", lambda: _lib.check(lib.sswin_plan_from_indices(ptr(q.indices), m, hd, ptr(plan), g_cap, totals, ptr(ws), nb, stream)), 0, 0),
             ("block_matmul q_k, values", mm(0, q.values, kt.values, q.indices, out_s, None, A), 2 * s * E + s * A + 4 * G, 1),
             ("block_matmul q_k (values + index matrix)", mm(0, q.values, kt.values, q.indices, out_s, out_si, A), 2 * s * E + (s + 16) * A + 4 * G, 0),
-            ("bias + mask add, one pass [A]", lambda: ops.group_add_bias_mask(s_val, row_pos, gp, b["n"], bias_d, mask), 2 * s * A + 8 * G, 1),
+            ("bias + mask add, one pass [A]", lambda: ops.group_add_table_bias_mask(s_val, row_pos, gp, b["n"], table_o, ti_o.code, ti_o.offset0, mask), 2 * s * A + 8 * G, 1),
+            ("bias + mask add from a gathered [H,n,n] bias", lambda: ops.group_add_bias_mask(s_val, row_pos, gp, b["n"], bias_d, mask), 2 * s * A + 8 * G, 0),
             ("bias table gradient from the product's groups", lambda: ops.group_bias_table_grad(g_s, row_pos, gp, H, b["n"], ti_o.code, ti_o.offset0, n_table_o), 4 * A, 1),
             ("softmax rows from the group sizes [A]", lambda: ops.softmax_rows_from_counts(c, A), 4 * A + 12 * G, 1),
             ("flatten_indices [3,A] (generic softmax rows)", lambda: ops.flatten_indices(s_idx[:3], s_shape[:3]), 16 * A, 0),
@@ -374,10 +443,14 @@ def kernel_table(wl, reps=20, only=None):
             ("return_inverse [N]", lambda: ops.return_inverse(flat_tok, b["slots"] * b["n"]), 0, 0),
             ("softmax_last_dim_backward", lambda: ops.softmax_last_dim_backward(rows, p_val, g_s), 16 * A, 1),
             ("grad rc_cr", grad(0, g_o, v.values, tmp_a), 2 * s * E + s * A, 1),
-            ("grad rr_rc", grad(1, g_s, kt.values, tmp_e), s * A + 2 * s * E, 2),
-            ("grad cr_rr", grad(2, q.values, g_s, tmp_e), s * A + 2 * s * E, 1),
-            ("transpose rc", tr(0, q.values, tmp_e), 2 * s * E, 2),
-            ("transpose rr", tr(1, g_s, tmp_a), 2 * s * A, 2),
+            ("grad rr_rc", grad(1, g_s, kt.values, tmp_e), s * A + 2 * s * E, 1),
+            # the second gradient of each product reads the operands as the forward pass left them; the reference's
+            # composition (two transposed copies, then cr_rr / rr_rc) is what the rows with 0 calls time
+            ("grad tr_rc (dV = P^T dO)", grad(3, p_val, g_o, tmp_e), s * A + 2 * s * E, 1),
+            ("grad tc_rr (dK^T = Q^T dS)", grad(4, q.values, g_s, tmp_e), s * A + 2 * s * E, 1),
+            ("grad cr_rr", grad(2, q.values, g_s, tmp_e), s * A + 2 * s * E, 0),
+            ("transpose rc", tr(0, q.values, tmp_e), 2 * s * E, 0),
+            ("transpose rr", tr(1, g_s, tmp_a), 2 * s * A, 0),
         ]
         # ---- the fused path (S and P in memory; what the module runs for heads that are not 32 wide) ----
         qkv_c = qkv.contiguous()
@@ -492,7 +565,23 @@ def kernel_table(wl, reps=20, only=None):
         return [], sizes
     table = measure(r_entries, "resident")
     if code == 0:
-        table += measure(f_entries, "fused") + measure(entries, "operators")
+        op_rows = measure(entries, "operators")
+        # the same launches inside a module call: what the path's summary is made of
+        timed = operators_in_module(wl)
+        seen = set()
+        for row in op_rows:
+            fn, ints = OPERATOR_LAUNCHES.get(row["kernel"], (None, None))
+            hits = [(k, v) for k, v in timed.items() if k[0] == fn and (ints is None or k[1] == ints)]
+            if hits and row["calls"]:
+                seen.update(k for k, _ in hits)
+                launches = sum(v[1] for _, v in hits)
+                row["ms_in_module"] = sum(v[0] * v[1] for _, v in hits) / launches
+                row["calls"] = int(round(launches))
+        stray = {k: v for k, v in timed.items() if k not in seen and "tall_linear" not in k[0] and "column_sum" not in k[0]}
+        for (fn, ints), (ms, launches) in stray.items():        # a launch of the call that no table row stands for
+            op_rows.append(dict(kernel=f"{fn}{ints} (in the module call only)", path="operators", ms=ms, ms_in_module=ms,
+                                algorithmic_bytes=0, calls=int(round(launches)), achieved_gbps=None, frac=None, flops=None))
+        table += measure(f_entries, "fused") + op_rows
         table += measure(stage_entries(wl), "stage")
         table += measure(projection_entries(wl), "projections")
     return table, sizes
@@ -831,15 +920,15 @@ def main():
 
     # the attention launches inside real steps: HIP events on the launch stream around each
     # library call (a few extra steps after the timed region, so the events do not perturb `value`)
-    from sparseswin3d_amd import fused
-    fused.launch_timer = []
+    from sparseswin3d_amd import _lib
+    _lib.launch_timer = []
     for _ in range(max(3, min(10, args.steps))):
         run_step(wl)
     torch.cuda.synchronize()
     in_step = {}
-    for name, start, stop in fused.launch_timer:
+    for name, _, start, stop in _lib.launch_timer:
         in_step.setdefault(name, []).append(start.elapsed_time(stop))
-    fused.launch_timer = None
+    _lib.launch_timer = None
     in_step = {k: sum(v) / len(v) for k, v in in_step.items()}
     log("attention launches inside a step (HIP events, mean over both blocks): " +
         ", ".join(f"{k} {v:.4f} ms" for k, v in in_step.items()))
@@ -860,12 +949,20 @@ def main():
                 continue
             log(titles.get(path, f"-- {path} path, one attention forward+backward --"))
             for r in rows_:
+                inm = r.get("ms_in_module")
                 log(f"{r['kernel']:36s} {r['ms']:9.4f} {r['calls']:5d} {r['algorithmic_bytes'] / 1e6:9.1f} "
-                    f"{(r['achieved_gbps'] or 0):9.1f} {100 * (r['frac'] or 0):7.2f}")
-            ms_ = sum(r["ms"] * r["calls"] for r in rows_)
+                    f"{(r['achieved_gbps'] or 0):9.1f} {100 * (r['frac'] or 0):7.2f}" +
+                    (f"   in the module call {inm:.4f} ms = {100 * r['algorithmic_bytes'] / inm / 1e6 / HBM_PEAK_GBPS:.2f} %" if inm else ""))
+            # the operator path is summed from the durations inside a module call (events around every launch of
+            # the call), the other paths from the launches timed alone
+            ms_ = sum(r.get("ms_in_module", r["ms"]) * r["calls"] for r in rows_)
             alg = sum(r["algorithmic_bytes"] * r["calls"] for r in rows_)
             summary[path] = dict(ms=round(ms_, 4), algorithmic_bytes=alg,
                                  frac=round(alg / ms_ / 1e6 / HBM_PEAK_GBPS, 4))
+            if path == "operators":
+                alone = sum(r["ms"] * r["calls"] for r in rows_)
+                summary[path].update(timed="inside a module call", ms_alone=round(alone, 4),
+                                     frac_alone=round(alg / alone / 1e6 / HBM_PEAK_GBPS, 4))
             log(f"{path} kernels, {scope.get(path, 'one attention fwd+bwd')}: {ms_:.3f} ms for {alg / 1e6:.1f} MB algorithmic "
                 f"= {alg / ms_ / 1e6:.1f} GB/s = {100 * alg / ms_ / 1e6 / HBM_PEAK_GBPS:.2f}% of HBM peak")
         # the step runs the window-resident path: its slowest kernel is the dominant one

@@ -31,7 +31,7 @@ enum { SSWIN_F32 = 0, SSWIN_F16 = 1, SSWIN_BF16 = 2, SSWIN_F64 = 3 };
 enum { SSWIN_I32 = 0, SSWIN_I64 = 1, SSWIN_I16 = 2, SSWIN_I8 = 3, SSWIN_U8 = 4 };
 /* block product kinds */
 enum { SSWIN_MUL_Q_K = 0, SSWIN_MUL_QK_V = 1 };
-enum { SSWIN_GRAD_RC_CR = 0, SSWIN_GRAD_RR_RC = 1, SSWIN_GRAD_CR_RR = 2 };
+enum { SSWIN_GRAD_RC_CR = 0, SSWIN_GRAD_RR_RC = 1, SSWIN_GRAD_CR_RR = 2, SSWIN_GRAD_TR_RC = 3, SSWIN_GRAD_TC_RR = 4 };
 enum { SSWIN_TRANSPOSE_RC = 0, SSWIN_TRANSPOSE_RR = 1 };
 
 const char* sswin_last_error(void);
@@ -118,7 +118,9 @@ int sswin_qkv_sparse_indices(const int32_t* indices, int64_t N, int B, int n, in
  * sswin_operand_copy: layout 0 (Q, V, attention output): val[hd*(H*T + h*c + i) + ch], layout 1 (K^T):
  *   val[hd*(H*T + h*c) + ch*c + i]  <->  vox[voxel * vox_stride + vox_col0 + h*hd + ch] (strides in values);
  *   to_operand != 0 copies voxel rows into the operand, 0 copies the operand into voxel rows.  Each direction is
- *   the gradient of the other.  dtype: any value dtype.
+ *   the gradient of the other.  dtype: any value dtype.  scale != 1 (layout 0 only): every copied value is multiplied
+ *   by it on the way, in the accumulation type of dtype and rounded once (the `q * self.scale` of
+ *   sparse_swin/swin3d_base.py:660 and, with to_operand == 0, its gradient) instead of a pass of its own.
  * sswin_sorted_coo_indices: the [4, E] index matrices of Q/V and of K^T in sorted order (either may be NULL),
  *   equal to idx.index_select(1, sorted) of sswin_qkv_sparse_indices.
  * All asynchronous unless validate != 0. */
@@ -126,7 +128,13 @@ size_t sswin_operand_map_workspace_bytes(int64_t N, int B, int n);
 int sswin_operand_map(const int32_t* indices, int64_t N, int B, int n, int32_t* map, void* ws, size_t ws_bytes,
                       int validate, int32_t* status_out, void* stream);
 int sswin_operand_copy(int dtype, int layout, int to_operand, void* vox, int64_t vox_stride, int vox_col0, void* val,
-                       const int32_t* map, int64_t N, int H, int hd, void* stream);
+                       const int32_t* map, int64_t N, int H, int hd, double scale, void* stream);
+/* The three copies of one attention call in one launch: vox is a [N, 3, H, hd] projection output (Q, K, V slices of a
+ * voxel row H*hd values apart, Q at vox_col0); Q goes to / comes from val_q in Q/V order times q_scale, K val_k in K^T
+ * order, V val_v in Q/V order (the gathers of sparse_swin/swin3d_base.py:492-498 and `q * self.scale`, :660; with
+ * to_operand == 0 their gradients). */
+int sswin_operand_copy_qkv(int dtype, int to_operand, void* vox, int64_t vox_stride, int vox_col0, void* val_q, void* val_k,
+                           void* val_v, const int32_t* map, int64_t N, int H, int hd, double q_scale, void* stream);
 int sswin_sorted_coo_indices(const int32_t* indices, const int32_t* map, int64_t N, int H, int hd, int32_t* idx_qv,
                              int32_t* idx_k, void* stream);
 
@@ -230,6 +238,11 @@ int sswin_block_matmul(int kind, int dtype, const void* mat1_v, const void* mat2
  *  SSWIN_GRAD_RC_CR: out[c x c] = m1[c x C] . m2[c x C]^T
  *  SSWIN_GRAD_RR_RC: out[c x C] = m1[c x c] . m2[C x c]^T
  *  SSWIN_GRAD_CR_RR: out[C x c] = m1[C x c] . m2[c x c]^T
+ * Two more kinds have no operator of their own in the reference: they are what its Python backward
+ * (sparse_swin/swin3d_base.py:121-134) composes from two qkv_transpose calls and one of the products above, read
+ * from the untransposed operands instead (the transposed copies are never written):
+ *  SSWIN_GRAD_TR_RC: out[c x C] = m1[c x c]^T . m2[c x C]     = RR_RC(transpose_rr(m1), transpose_rc(m2))
+ *  SSWIN_GRAD_TC_RR: out[C x c] = m1[c x C]^T . m2[c x c]     = CR_RR(transpose_rc(m1), transpose_rr(m2))
  * c: device int32 [G]; scans: device, from sswin_scan_counts.  Asynchronous. */
 int sswin_block_matmul_grad(int kind, int dtype, const void* m1, const void* m2,
                             const int32_t* c, const int32_t* scans, int64_t G, int C,

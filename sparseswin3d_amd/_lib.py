@@ -37,7 +37,8 @@ SIGNATURES = {
     "sswin_qkv_sparse_indices": (_i32, [_vp, _i64, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _vp, _sz, _i32, _vp, _vp]),
     "sswin_operand_map_workspace_bytes": (_sz, [_i64, _i32, _i32]),
     "sswin_operand_map": (_i32, [_vp, _i64, _i32, _i32, _vp, _vp, _sz, _i32, _vp, _vp]),
-    "sswin_operand_copy": (_i32, [_i32, _i32, _i32, _vp, _i64, _i32, _vp, _vp, _i64, _i32, _i32, _vp]),
+    "sswin_operand_copy_qkv": (_i32, [_i32, _i32, _vp, _i64, _i32, _vp, _vp, _vp, _vp, _i64, _i32, _i32, C.c_double, _vp]),
+    "sswin_operand_copy": (_i32, [_i32, _i32, _i32, _vp, _i64, _i32, _vp, _vp, _i64, _i32, _i32, C.c_double, _vp]),
     "sswin_sorted_coo_indices": (_i32, [_vp, _vp, _i64, _i32, _i32, _vp, _vp, _vp]),
     "sswin_plan_workspace_bytes": (_sz, [_i64, _i32]),
     "sswin_plan_from_indices": (_i32, [_vp, _i64, _i32, _vp, _i64, _vp, _vp, _sz, _vp]),
@@ -89,8 +90,39 @@ SIGNATURES = {
                                                _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i32, _vp]),
 }
 
-ABI_VERSION = 26
+ABI_VERSION = 27
 _lib = None
+
+# A list turns on timing of the library's launches: every call that takes a stream is bracketed by events on that
+# stream and leaves (name, leading integer arguments, start event, stop event) here.  A benchmark uses it to time the
+# kernels where they run, inside a module call or a step; None (the default) costs nothing.
+launch_timer = None
+
+
+class _TimedLibrary:
+    """The loaded library with every stream-taking entry point bracketed by events (see ``launch_timer``)."""
+
+    def __init__(self, lib):
+        self._lib = lib
+
+    def __getattr__(self, name):
+        fn = getattr(self._lib, name)
+        sig = SIGNATURES.get(name)
+        if launch_timer is None or sig is None or sig[0] is not _i32 or not sig[1] or sig[1][-1] is not _vp:
+            return fn
+
+        def call(*args):
+            import torch
+            handle = getattr(args[-1], "value", None)
+            stream = torch.cuda.ExternalStream(handle) if handle else torch.cuda.current_stream()
+            start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            start.record(stream)
+            status = fn(*args)
+            stop.record(stream)
+            if launch_timer is not None:
+                launch_timer.append((name, tuple(a for a in args[:3] if isinstance(a, int)), start, stop))
+            return status
+        return call
 
 
 class LibraryMissing(RuntimeError):
@@ -101,7 +133,7 @@ def load():
     """Load the HIP library once.  Raises :class:`LibraryMissing` if it has not been built."""
     global _lib
     if _lib is not None:
-        return _lib
+        return _lib if launch_timer is None else _TimedLibrary(_lib)
     if not os.path.exists(LIB_PATH):
         raise LibraryMissing(
             f"{LIB_PATH} not found: build it with `python -m sparseswin3d_amd.build` "
@@ -122,6 +154,34 @@ def load():
         raise RuntimeError(f"libsswin3d ABI {lib.sswin_abi_version()} != binding ABI {ABI_VERSION}; rebuild")
     _lib = lib
     return lib
+
+
+class _NoSwitch:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def on_device(device):
+    """Context manager that makes ``device`` the current one for a library call; when it is current already (the
+    usual case) nothing is switched: ``torch.cuda.device`` costs several microseconds on the host per use, a
+    noticeable share of an operator that takes twenty on the GPU."""
+    import torch
+    if device.index is None or device.index == torch.cuda.current_device():
+        return _NO_SWITCH
+    return torch.cuda.device(device)
+
+
+def stream_handle(device):
+    """The current HIP stream of ``device`` as the ``void*`` the library takes."""
+    import torch
+    index = device.index if device.index is not None else torch.cuda.current_device()
+    return C.c_void_p(torch._C._cuda_getCurrentRawStream(index))
 
 
 def check(status: int):

@@ -12,6 +12,10 @@
 //   RC_CR     m1  mat      m2  mat, j-major   sq           c  c  C
 //   RR_RC     m1  sq       m2  mat, j-major   mat [c x C]  c  C  c
 //   CR_RR     m1  mat[Cxc] m2  sq,  j-major   mat [C x c]  C  c  c
+//   TR_RC     m1^T, m1 sq  m2  mat, k-major   mat [c x C]  c  C  c     (A stored k-major: [K x I])
+//   TC_RR     m1^T, m1 mat m2  sq,  k-major   mat [C x c]  C  c  c     (A stored k-major: [K x I])
+// The last two are the second gradient of each product taken from the operands as the forward pass left them:
+// TR_RC(P, dO) = RR_RC(P^T, (dO)^T stored [C x c]) and TC_RR(Q, dS) = CR_RR(Q^T, dS^T), without the transposed copies.
 //
 // Execution model (gfx950, wave64): the unit of work is one 32 x 32 output block of one group,
 // computed by ONE wavefront with v_mfma_f32_32x32x2_f32.  Operands go from global memory
@@ -34,12 +38,16 @@
 
 namespace sswin {
 
-enum { MODE_QK = 0, MODE_PV = 1, MODE_RC_CR = 2, MODE_RR_RC = 3, MODE_CR_RR = 4 };
+enum { MODE_QK = 0, MODE_PV = 1, MODE_RC_CR = 2, MODE_RR_RC = 3, MODE_CR_RR = 4, MODE_TR_RC = 5, MODE_TC_RR = 6 };
 
 constexpr int GROUPS_PER_WG = 4;
 constexpr int MAX_POS = 1024;          // largest window occupancy the simple kernel's LDS table holds
 
-template <int MODE> __host__ __device__ constexpr bool b_is_kmajor() { return MODE == MODE_QK || MODE == MODE_PV; }
+template <int MODE> __host__ __device__ constexpr bool b_is_kmajor() { return MODE == MODE_QK || MODE == MODE_PV || MODE >= MODE_TR_RC; }
+template <int MODE> __host__ __device__ constexpr bool a_is_kmajor() { return MODE >= MODE_TR_RC; }
+// shapes of the output block: I rows, J columns
+template <int MODE> __host__ __device__ constexpr bool rows_are_channels() { return MODE == MODE_CR_RR || MODE == MODE_TC_RR; }
+template <int MODE> __host__ __device__ constexpr bool cols_are_channels() { return MODE == MODE_PV || MODE == MODE_RR_RC || MODE == MODE_TR_RC; }
 
 struct GroupDims {
     int I, J, K;
@@ -51,7 +59,7 @@ __device__ __forceinline__ GroupDims group_dims(int c, int C, int64_t rs, int64_
     GroupDims d;
     const int64_t mat = rs * C;
     if (MODE == MODE_QK || MODE == MODE_RC_CR) { d.I = c; d.J = c; d.K = C; d.a_off = mat; d.b_off = mat; d.o_off = ss; }
-    else if (MODE == MODE_PV || MODE == MODE_RR_RC) { d.I = c; d.J = C; d.K = c; d.a_off = ss; d.b_off = mat; d.o_off = mat; }
+    else if (cols_are_channels<MODE>()) { d.I = c; d.J = C; d.K = c; d.a_off = ss; d.b_off = mat; d.o_off = mat; }
     else { d.I = C; d.J = c; d.K = c; d.a_off = mat; d.b_off = ss; d.o_off = mat; }
     return d;
 }
@@ -67,26 +75,40 @@ struct GroupTable {
 #ifndef BP_WAVES
 #define BP_WAVES 5
 #endif
+#ifndef BP_WAVES_FWD
+#define BP_WAVES_FWD 4
+#endif
 template <typename T, int MODE, bool EMIT>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MODE >= 2 ? BP_WAVES : 4, MODE >= 2 ? BP_WAVES : 4))) void block_product_mfma_kernel(const T* __restrict__ m1, const T* __restrict__ m2,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MODE >= 2 ? BP_WAVES : BP_WAVES_FWD, MODE >= 2 ? BP_WAVES : BP_WAVES_FWD))) void block_product_mfma_kernel(const T* __restrict__ m1, const T* __restrict__ m2,
                                                                  GroupTable gt, int64_t G, int C,
                                                                  const int32_t* __restrict__ tok_pos,
                                                                  T* __restrict__ out, int32_t* __restrict__ out_idx,
                                                                  int64_t out_nnz) {
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    // the wavefront's number as a scalar: everything that follows from it (its task, the group's size and offsets,
+    // the operand bases) stays in scalar registers and the loads take a scalar base with a 32-bit lane offset
+    // (measured on cfg2: 'q_k' 47.5 -> 44 us, 'qk_v' 41 -> 37, 'tr_rc' / 'tc_rr' 40 -> 35; the products whose operands
+    // are both read along their rows lose by it, 'rr_rc' 41 -> 51 us, and keep the lane-held number)
+    const int wave = (b_is_kmajor<MODE>() || a_is_kmajor<MODE>()) ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : threadIdx.x >> 6;
+    const int lane = threadIdx.x & 63;
     const int half = lane >> 5, l32 = lane & 31;
     const int64_t g0 = (int64_t)blockIdx.x * GROUPS_PER_WG;
 
     // blocks of the workgroup's four groups
-    int cq[GROUPS_PER_WG], nbj[GROUPS_PER_WG], first[GROUPS_PER_WG + 1];
+    // sizes and offsets of the four groups leave in one round of loads (the offsets do not wait for the sizes)
+    int cq[GROUPS_PER_WG], nbj[GROUPS_PER_WG], first[GROUPS_PER_WG + 1], rsq[GROUPS_PER_WG], ssq[GROUPS_PER_WG];
     first[0] = 0;
 #pragma unroll
     for (int q = 0; q < GROUPS_PER_WG; ++q) {
         const int64_t g = g0 + q;
-        const int c = g < G ? gt.c[g] : 0;
-        cq[q] = c;
-        const int I = MODE == MODE_CR_RR ? C : c;
-        const int J = (MODE == MODE_PV || MODE == MODE_RR_RC) ? C : c;
+        cq[q] = g < G ? gt.c[g] : 0;
+        rsq[q] = g < G ? gt.row_start[g] : 0;
+        ssq[q] = g < G ? gt.sq_start[g] : 0;
+    }
+#pragma unroll
+    for (int q = 0; q < GROUPS_PER_WG; ++q) {
+        const int c = cq[q];
+        const int I = rows_are_channels<MODE>() ? C : c;
+        const int J = cols_are_channels<MODE>() ? C : c;
         nbj[q] = (J + 31) >> 5;
         first[q + 1] = first[q] + (c > 0 ? ((I + 31) >> 5) * nbj[q] : 0);
     }
@@ -96,14 +118,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MODE >= 2 ?
         int q = 0;
 #pragma unroll
         for (int qq = 1; qq < GROUPS_PER_WG; ++qq) q += (t >= first[qq]) ? 1 : 0;
-        int c = cq[0], nj = nbj[0], f0 = first[0];
+        int c = cq[0], nj = nbj[0], f0 = first[0], rs_ = rsq[0], ss_ = ssq[0];
 #pragma unroll
         for (int qq = 1; qq < GROUPS_PER_WG; ++qq)
-            if (q == qq) { c = cq[qq]; nj = nbj[qq]; f0 = first[qq]; }
+            if (q == qq) { c = cq[qq]; nj = nbj[qq]; f0 = first[qq]; rs_ = rsq[qq]; ss_ = ssq[qq]; }
         const int64_t g = g0 + q;
         const int local = t - f0;
         const int bi = local / nj, bj = local - bi * nj;
-        const int64_t rs = gt.row_start[g], ss = gt.sq_start[g];
+        const int64_t rs = rs_, ss = ss_;
         const GroupDims d = group_dims<MODE>(c, C, rs, ss);
         const int i_a = bi * 32 + l32;           // operand row of A this lane feeds
         const int j_b = bj * 32 + l32;           // operand column of B this lane feeds
@@ -132,12 +154,32 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MODE >= 2 ?
             const int kb = kc + half * kh;
             const int left = half ? chunk - kh : kh;            // values of k of this lane half
             float a[16], b[16];
-            load_run16<T>(A + (int64_t)i_a * d.K + kb, i_a < d.I ? left : 0, a);
+            // A k-major operand is read one row of k per step: element (kc + s) * width + (half * kh * width + column),
+            // a scalar part plus a lane part.  Every lane loads from inside the block (offset clamped to its last
+            // element) and drops what it has no use for: one select per value instead of a branch around each load.
+            if (a_is_kmajor<MODE>()) {
+                const unsigned lane_part = (unsigned)(half * kh * d.I + (i_a < d.I ? i_a : d.I - 1));
+                const unsigned last = (unsigned)(d.K * d.I - 1);
+                const bool iin = i_a < d.I;
+#pragma unroll
+                for (int s = 0; s < 16; ++s) {
+                    const unsigned off = (unsigned)((kc + s) * d.I) + lane_part;
+                    const float x = to_acc(A[off < last ? off : last]);
+                    a[s] = (iin && s < left) ? x : 0.f;
+                }
+            } else {
+                load_run16<T>(A + (int64_t)i_a * d.K + kb, i_a < d.I ? left : 0, a);
+            }
             if (b_is_kmajor<MODE>()) {
-                const T* bp = B + (int64_t)kb * d.J + j_b;
+                const unsigned lane_part = (unsigned)(half * kh * d.J + (j_b < d.J ? j_b : d.J - 1));
+                const unsigned last = (unsigned)(d.K * d.J - 1);
                 const bool jin = j_b < d.J;
 #pragma unroll
-                for (int s = 0; s < 16; ++s) b[s] = (jin && s < left) ? to_acc(bp[(int64_t)s * d.J]) : 0.f;
+                for (int s = 0; s < 16; ++s) {
+                    const unsigned off = (unsigned)((kc + s) * d.J) + lane_part;
+                    const float x = to_acc(B[off < last ? off : last]);
+                    b[s] = (jin && s < left) ? x : 0.f;
+                }
             } else {
                 load_run16<T>(B + (int64_t)j_b * d.K + kb, j_b < d.J ? left : 0, b);
             }
@@ -211,7 +253,7 @@ __global__ __launch_bounds__(256) void block_product_simple_kernel(const T* __re
         const int i = f / d.J, j = f - i * d.J;
         AccT sum = 0;
         for (int k = 0; k < d.K; ++k) {
-            const AccT a = to_acc(A[(int64_t)i * d.K + k]);
+            const AccT a = a_is_kmajor<MODE>() ? to_acc(A[(int64_t)k * d.I + i]) : to_acc(A[(int64_t)i * d.K + k]);
             const AccT b = b_is_kmajor<MODE>() ? to_acc(B[(int64_t)k * d.J + j]) : to_acc(B[(int64_t)j * d.K + k]);
             sum += a * b;
         }
@@ -496,8 +538,8 @@ int sswin_block_matmul(int kind, int dtype, const void* mat1_v, const void* mat2
 
 int sswin_block_matmul_grad(int kind, int dtype, const void* m1, const void* m2, const int32_t* c,
                             const int32_t* scans, int64_t G, int C, void* out, void* stream) {
-    SSWIN_CHECK(kind >= SSWIN_GRAD_RC_CR && kind <= SSWIN_GRAD_CR_RR,
-                "Invalid mul_type code %d. Expected 'rc_cr', 'rr_rc' or 'cr_rr'.", kind);
+    SSWIN_CHECK(kind >= SSWIN_GRAD_RC_CR && kind <= SSWIN_GRAD_TC_RR,
+                "Invalid mul_type code %d. Expected 'rc_cr', 'rr_rc', 'cr_rr', 'tr_rc' or 'tc_rr'.", kind);
     SSWIN_CHECK(C > 0 && G >= 0, "block_matmul_grad: bad sizes");
     if (G == 0) return 0;
     SSWIN_CHECK(m1 && m2 && c && scans && out, "block_matmul_grad: null pointer");
@@ -506,7 +548,9 @@ int sswin_block_matmul_grad(int kind, int dtype, const void* m1, const void* m2,
     switch (kind) {
         case SSWIN_GRAD_RC_CR: return dispatch_product<MODE_RC_CR, false>(dtype, m1, m2, gt, G, C, nullptr, out, nullptr, 0, s);
         case SSWIN_GRAD_RR_RC: return dispatch_product<MODE_RR_RC, false>(dtype, m1, m2, gt, G, C, nullptr, out, nullptr, 0, s);
-        default: return dispatch_product<MODE_CR_RR, false>(dtype, m1, m2, gt, G, C, nullptr, out, nullptr, 0, s);
+        case SSWIN_GRAD_CR_RR: return dispatch_product<MODE_CR_RR, false>(dtype, m1, m2, gt, G, C, nullptr, out, nullptr, 0, s);
+        case SSWIN_GRAD_TR_RC: return dispatch_product<MODE_TR_RC, false>(dtype, m1, m2, gt, G, C, nullptr, out, nullptr, 0, s);
+        default: return dispatch_product<MODE_TC_RR, false>(dtype, m1, m2, gt, G, C, nullptr, out, nullptr, 0, s);
     }
 }
 

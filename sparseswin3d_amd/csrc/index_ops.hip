@@ -387,6 +387,52 @@ __global__ __launch_bounds__(256) void qv_order_copy_kernel(const int32_t* __res
         *pv = *po;
 }
 
+// The same copy with every value multiplied by `scale` on the way (the `q * scale` of the attention module and, in the
+// other direction, its gradient): one thread per (rank, head, piece of VEC values); the product is taken in the
+// accumulation type of T and rounded once, as an elementwise multiply of the copied array would.
+template <typename T, int VEC>
+__global__ __launch_bounds__(256) void qv_order_scale_kernel(const int32_t* __restrict__ order, const int32_t* __restrict__ win_T,
+                                                             const int32_t* __restrict__ win_c,
+                                                             const int32_t* __restrict__ status, int64_t N, int H,
+                                                             int pieces, char* __restrict__ vox, int64_t row_bytes,
+                                                             int64_t col0_bytes, char* __restrict__ val, bool to_operand,
+                                                             typename acc_of<T>::type scale) {
+    struct __attribute__((aligned(sizeof(T) * VEC))) Piece { T v[VEC]; };
+    const int64_t t = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (t >= N * H * pieces || !pairs_valid(status, N)) return;
+    const int pc = (int)(t % pieces);
+    const int64_t rh = t / pieces;
+    const int h = (int)(rh % H);
+    const int64_t r = rh / H;
+    const int T0 = win_T[r], c = win_c[r];
+    const int64_t row = (int64_t)H * T0 + (int64_t)h * c + (r - T0);
+    Piece* pv = reinterpret_cast<Piece*>(vox + (int64_t)order[r] * row_bytes + col0_bytes) + (int64_t)h * pieces + pc;
+    Piece* po = reinterpret_cast<Piece*>(val) + row * pieces + pc;
+    Piece x = to_operand ? *pv : *po;
+#pragma unroll
+    for (int u = 0; u < VEC; ++u) x.v[u] = from_acc<T>(to_acc(x.v[u]) * scale);
+    if (to_operand)
+        *po = x;
+    else
+        *pv = x;
+}
+
+template <typename T>
+static void launch_qv_scale(bool wide, const int32_t* order, const int32_t* win_T, const int32_t* win_c, const int32_t* status,
+                            int64_t N, int H, int hd, char* v, int64_t row_bytes, int64_t col0_bytes, char* o, bool to_operand,
+                            double scale, hipStream_t s) {
+    constexpr int VEC = 16 / (int)sizeof(T);
+    using A = typename acc_of<T>::type;
+    if (wide) {
+        const int pieces = hd / VEC;
+        hipLaunchKernelGGL((qv_order_scale_kernel<T, VEC>), dim3((unsigned)((N * H * pieces + 255) / 256)), dim3(256), 0, s, order,
+                           win_T, win_c, status, N, H, pieces, v, row_bytes, col0_bytes, o, to_operand, (A)scale);
+    } else {
+        hipLaunchKernelGGL((qv_order_scale_kernel<T, 1>), dim3((unsigned)((N * H * hd + 255) / 256)), dim3(256), 0, s, order,
+                           win_T, win_c, status, N, H, hd, v, row_bytes, col0_bytes, o, to_operand, (A)scale);
+    }
+}
+
 // One thread per rank and head (blockIdx.y), walking over the channels: for a fixed channel the lanes of a
 // wavefront touch runs of c consecutive operand values per window; a lane's own voxel row stays in cache
 // over the walk.
@@ -496,6 +542,98 @@ __global__ __launch_bounds__(256) void k_order_copy_lds_kernel(const int32_t* __
     }
 }
 
+// Q, K^T and V of one [N, 3, H, HD] token tensor in one launch (Q times `scale` on the way), or the three gradients back
+// into it: the K^T copy above with the rows of Q and V of the same 64 ranks and head taken along.  A rank's Q / V slice
+// is one contiguous run in the operand (HD values at HD * (H*T + h*c + i)), so it goes piece by piece without LDS.
+template <typename T, int HD>
+__global__ __launch_bounds__(256) void qkv_order_copy_kernel(const int32_t* __restrict__ order, const int32_t* __restrict__ win_T,
+                                                             const int32_t* __restrict__ win_c,
+                                                             const int32_t* __restrict__ status, int64_t N, int H,
+                                                             char* __restrict__ vox, int64_t row_bytes, int64_t col0_bytes,
+                                                             char* __restrict__ val_q, char* __restrict__ val_k,
+                                                             char* __restrict__ val_v, bool to_operand, float scale) {
+    constexpr int PER16 = 16 / (int)sizeof(T);
+    constexpr int PIECES = HD / PER16;
+    constexpr int ROWS_PER_PASS = 256 / PIECES;
+    __shared__ T tile[64][HD + 1];
+    __shared__ int64_t s_base[64];                           // operand position of (rank, channel 0) in K^T order
+    __shared__ int64_t s_row[64];                            // the same in Q/V order
+    __shared__ int32_t s_c[64];
+    __shared__ int32_t s_vox[64];
+    if (!pairs_valid(status, N)) return;
+    const int64_t r0 = (int64_t)blockIdx.x * 64;
+    const int h = blockIdx.y;
+    const int tid = threadIdx.x;
+    if (tid < 64) {
+        const int64_t r = r0 + tid;
+        if (r < N) {
+            const int T0 = win_T[r], c = win_c[r];
+            s_base[tid] = (int64_t)HD * ((int64_t)H * T0 + (int64_t)h * c) + (r - T0);
+            s_row[tid] = (int64_t)HD * ((int64_t)H * T0 + (int64_t)h * c + (r - T0));
+            s_c[tid] = c;
+            s_vox[tid] = order[r];
+        } else {
+            s_c[tid] = 0;
+        }
+    }
+    __syncthreads();
+    T* ok = reinterpret_cast<T*>(val_k);
+    const int lane_r = tid & 63, ch0 = tid >> 6;
+    const int piece = tid % PIECES, prow = tid / PIECES;
+    const int64_t head_bytes = (int64_t)H * HD * sizeof(T);  // Q, K, V slices of a voxel row lie this far apart
+    const int64_t in_row = ((int64_t)h * HD + piece * PER16) * sizeof(T);
+    if (to_operand) {
+        for (int rr = prow; rr < 64; rr += ROWS_PER_PASS) {
+            if (s_c[rr] == 0) continue;
+            const char* src = vox + (int64_t)s_vox[rr] * row_bytes + col0_bytes + in_row;
+            int4 xq = *reinterpret_cast<const int4*>(src);
+            const int4 xk = *reinterpret_cast<const int4*>(src + head_bytes);
+            const int4 xv = *reinterpret_cast<const int4*>(src + 2 * head_bytes);
+            const T* kv = reinterpret_cast<const T*>(&xk);
+#pragma unroll
+            for (int u = 0; u < PER16; ++u) tile[rr][piece * PER16 + u] = kv[u];
+            T* qv = reinterpret_cast<T*>(&xq);
+#pragma unroll
+            for (int u = 0; u < PER16; ++u) qv[u] = from_acc<T>(to_acc(qv[u]) * scale);
+            const int64_t dst = (s_row[rr] + piece * PER16) * sizeof(T);
+            *reinterpret_cast<int4*>(val_q + dst) = xq;
+            *reinterpret_cast<int4*>(val_v + dst) = xv;
+        }
+        __syncthreads();
+        const int c = s_c[lane_r];
+        if (c > 0) {
+            const int64_t base = s_base[lane_r];
+#pragma unroll 4
+            for (int ch = ch0; ch < HD; ch += 4) ok[base + (int64_t)ch * c] = tile[lane_r][ch];
+        }
+    } else {
+        const int c = s_c[lane_r];
+        if (c > 0) {
+            const int64_t base = s_base[lane_r];
+#pragma unroll 4
+            for (int ch = ch0; ch < HD; ch += 4) tile[lane_r][ch] = ok[base + (int64_t)ch * c];
+        }
+        __syncthreads();
+        for (int rr = prow; rr < 64; rr += ROWS_PER_PASS) {
+            if (s_c[rr] == 0) continue;
+            const int64_t from = (s_row[rr] + piece * PER16) * sizeof(T);
+            int4 xq = *reinterpret_cast<const int4*>(val_q + from);
+            const int4 xv = *reinterpret_cast<const int4*>(val_v + from);
+            T* qv = reinterpret_cast<T*>(&xq);
+#pragma unroll
+            for (int u = 0; u < PER16; ++u) qv[u] = from_acc<T>(to_acc(qv[u]) * scale);
+            int4 xk;
+            T* kv = reinterpret_cast<T*>(&xk);
+#pragma unroll
+            for (int u = 0; u < PER16; ++u) kv[u] = tile[rr][piece * PER16 + u];
+            char* dst = vox + (int64_t)s_vox[rr] * row_bytes + col0_bytes + in_row;
+            *reinterpret_cast<int4*>(dst) = xq;
+            *reinterpret_cast<int4*>(dst + head_bytes) = xk;
+            *reinterpret_cast<int4*>(dst + 2 * head_bytes) = xv;
+        }
+    }
+}
+
 // Index matrices of the sorted operands written in place (what expand + sort + gather arrive at): idx_qv
 // rows (window, head, pos, channel) at hd * (H*T + h*c + i) + ch; idx_k rows (window, head, channel, pos) at
 // hd * (H*T + h*c) + ch * c + i.  idx_qv: one thread per (rank, head, channel quad), 16-byte stores.
@@ -574,7 +712,7 @@ using namespace sswin;
 extern "C" {
 
 const char* sswin_last_error(void) { return error_buffer(); }
-int sswin_abi_version(void) { return 26; }
+int sswin_abi_version(void) { return 27; }
 
 int sswin_calibration_copy(void* dst, const void* src, int64_t bytes, void* stream) {
     SSWIN_CHECK(bytes >= 0 && bytes % 16 == 0, "calibration_copy: size must be a multiple of 16 bytes");
@@ -882,9 +1020,10 @@ int sswin_operand_map(const int32_t* indices, int64_t N, int B, int n, int32_t* 
 static int value_bytes(int dtype) { return dtype == SSWIN_F64 ? 8 : dtype == SSWIN_F32 ? 4 : 2; }
 
 int sswin_operand_copy(int dtype, int layout, int to_operand, void* vox, int64_t vox_stride, int vox_col0, void* val,
-                       const int32_t* map, int64_t N, int H, int hd, void* stream) {
+                       const int32_t* map, int64_t N, int H, int hd, double scale, void* stream) {
     SSWIN_CHECK(dtype >= SSWIN_F32 && dtype <= SSWIN_F64, "operand_copy: unsupported value dtype %d", dtype);
     SSWIN_CHECK(layout == 0 || layout == 1, "operand_copy: layout must be 0 (Q, V) or 1 (K^T)");
+    SSWIN_CHECK(scale == 1.0 || layout == 0, "operand_copy: only the Q/V order takes a scale");
     SSWIN_CHECK(N >= 0 && H > 0 && hd > 0 && vox_col0 >= 0 && vox_stride >= (int64_t)vox_col0 + (int64_t)H * hd,
                 "operand_copy: bad sizes");
     if (N == 0) return 0;
@@ -899,6 +1038,16 @@ int sswin_operand_copy(int dtype, int layout, int to_operand, void* vox, int64_t
         const int head_bytes = hd * esz;
         const bool wide = head_bytes % 16 == 0 && row_bytes % 16 == 0 && col0_bytes % 16 == 0 && ((uintptr_t)vox % 16) == 0 &&
                           ((uintptr_t)val % 16) == 0;
+        if (scale != 1.0) {
+            const bool up = to_operand != 0;
+            switch (dtype) {
+                case SSWIN_F32: launch_qv_scale<float>(wide, order, win_T, win_c, status, N, H, hd, v, row_bytes, col0_bytes, o, up, scale, s); break;
+                case SSWIN_F16: launch_qv_scale<__half>(wide, order, win_T, win_c, status, N, H, hd, v, row_bytes, col0_bytes, o, up, scale, s); break;
+                case SSWIN_BF16: launch_qv_scale<__hip_bfloat16>(wide, order, win_T, win_c, status, N, H, hd, v, row_bytes, col0_bytes, o, up, scale, s); break;
+                default: launch_qv_scale<double>(wide, order, win_T, win_c, status, N, H, hd, v, row_bytes, col0_bytes, o, up, scale, s); break;
+            }
+            return launch_ok("operand_copy");
+        }
         const int pieces = wide ? head_bytes / 16 : hd;
         const int64_t threads = N * H * pieces;
         const dim3 grid((unsigned)((threads + 255) / 256));
@@ -949,6 +1098,41 @@ int sswin_operand_copy(int dtype, int layout, int to_operand, void* vox, int64_t
                                row_bytes, col0_bytes, o, to_operand != 0);
     }
     return launch_ok("operand_copy");
+}
+
+int sswin_operand_copy_qkv(int dtype, int to_operand, void* vox, int64_t vox_stride, int vox_col0, void* val_q, void* val_k,
+                           void* val_v, const int32_t* map, int64_t N, int H, int hd, double q_scale, void* stream) {
+    SSWIN_CHECK(dtype >= SSWIN_F32 && dtype <= SSWIN_F64, "operand_copy_qkv: unsupported value dtype %d", dtype);
+    SSWIN_CHECK(N >= 0 && H > 0 && hd > 0 && vox_col0 >= 0 && vox_stride >= (int64_t)vox_col0 + 3 * (int64_t)H * hd,
+                "operand_copy_qkv: bad sizes");
+    if (N == 0) return 0;
+    SSWIN_CHECK(vox && val_q && val_k && val_v && map, "operand_copy_qkv: null pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const int esz = value_bytes(dtype);
+    const int64_t row_bytes = vox_stride * esz, col0_bytes = (int64_t)vox_col0 * esz;
+    const bool wide = dtype != SSWIN_F64 && (hd == 32 || hd == 16) && row_bytes % 16 == 0 && col0_bytes % 16 == 0 &&
+                      ((int64_t)H * hd * esz) % 16 == 0 && ((uintptr_t)vox % 16) == 0 && ((uintptr_t)val_q % 16) == 0 &&
+                      ((uintptr_t)val_v % 16) == 0;
+    if (!wide) {                                             // any other shape: the three copies one by one
+        const int D = H * hd;
+        if (sswin_operand_copy(dtype, 0, to_operand, vox, vox_stride, vox_col0, val_q, map, N, H, hd, q_scale, stream)) return 1;
+        if (sswin_operand_copy(dtype, 1, to_operand, vox, vox_stride, vox_col0 + D, val_k, map, N, H, hd, 1.0, stream)) return 1;
+        return sswin_operand_copy(dtype, 0, to_operand, vox, vox_stride, vox_col0 + 2 * D, val_v, map, N, H, hd, 1.0, stream);
+    }
+    const int32_t *order = map, *win_T = map + N, *win_c = map + 2 * N, *status = map + 3 * N;
+    const dim3 grid((unsigned)((N + 63) / 64), (unsigned)H);
+#define SSWIN_QKV(T, HD)                                                                                                  \
+    hipLaunchKernelGGL((qkv_order_copy_kernel<T, HD>), grid, dim3(256), 0, s, order, win_T, win_c, status, N, H,            \
+                       static_cast<char*>(vox), row_bytes, col0_bytes, static_cast<char*>(val_q), static_cast<char*>(val_k), \
+                       static_cast<char*>(val_v), to_operand != 0, (float)q_scale)
+    if (dtype == SSWIN_F32 && hd == 32) SSWIN_QKV(float, 32);
+    else if (dtype == SSWIN_F32) SSWIN_QKV(float, 16);
+    else if (dtype == SSWIN_F16 && hd == 32) SSWIN_QKV(__half, 32);
+    else if (dtype == SSWIN_F16) SSWIN_QKV(__half, 16);
+    else if (hd == 32) SSWIN_QKV(__hip_bfloat16, 32);
+    else SSWIN_QKV(__hip_bfloat16, 16);
+#undef SSWIN_QKV
+    return launch_ok("operand_copy_qkv");
 }
 
 int sswin_sorted_coo_indices(const int32_t* indices, const int32_t* map, int64_t N, int H, int hd, int32_t* idx_qv,

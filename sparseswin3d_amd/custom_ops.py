@@ -42,7 +42,7 @@ def _dev(*tensors):
 
 
 def _stream(device):
-    return C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+    return _lib.stream_handle(device)
 
 
 def _ptr(t):
@@ -72,7 +72,7 @@ def flatten_indices(indices, sizes):
     indices = indices.contiguous()
     m = indices.shape[1]
     out = torch.empty(m, dtype=torch.int32, device=d)
-    with torch.cuda.device(d):
+    with _lib.on_device(d):
         _lib.check(lib.sswin_flatten_indices(_ptr(indices), ndim, m, _host_i32(sizes), _ptr(out), _stream(d)))
     return out
 
@@ -87,7 +87,7 @@ def sort_indices(flattened_indices):
     out = torch.empty(m, dtype=torch.int32, device=d)
     nbytes = lib.sswin_sort_indices_workspace_bytes(m)
     ws = _ws(nbytes, d)
-    with torch.cuda.device(d):
+    with _lib.on_device(d):
         _lib.check(lib.sswin_sort_indices(_ptr(keys), m, _ptr(out), _ptr(ws), nbytes, _stream(d)))
     return out
 
@@ -103,7 +103,7 @@ def unique_consecutive_indices(nums):
     out = torch.empty(m, dtype=torch.int32, device=d)
     nbytes = lib.sswin_unique_consecutive_workspace_bytes(m)
     ws = _ws(nbytes, d)
-    with torch.cuda.device(d):
+    with _lib.on_device(d):
         _lib.check(lib.sswin_unique_consecutive_indices(_ptr(nums), _KEY_CODE[nums.dtype], m, _ptr(out),
                                                         _ptr(ws), nbytes, _stream(d)))
     return out
@@ -129,7 +129,7 @@ def return_inverse(x, maxnum=-1):
     nbytes = lib.sswin_return_inverse_workspace_bytes(m, bound)
     ws = _ws(nbytes, d)
     count = C.c_int64(0)
-    with torch.cuda.device(d):
+    with _lib.on_device(d):
         _lib.check(lib.sswin_return_inverse(_ptr(x), m, maxnum, _ptr(out), C.byref(count), _ptr(ws), nbytes,
                                             _stream(d)))
         _check_pending()
@@ -155,7 +155,7 @@ def operand_map(indices, batch_size, spatial_dim):
     nbytes = lib.sswin_operand_map_workspace_bytes(n_vox, int(batch_size), int(spatial_dim))
     ws = _ws(nbytes, d)
     status = torch.zeros(2, dtype=torch.int32, pin_memory=True)
-    with torch.cuda.device(d):
+    with _lib.on_device(d):
         _check_pending()
         _lib.check(lib.sswin_operand_map(_ptr(indices), n_vox, int(batch_size), int(spatial_dim), _ptr(out), _ptr(ws),
                                          nbytes, 0, C.c_void_p(status.data_ptr()), _stream(d)))
@@ -166,9 +166,10 @@ def operand_map(indices, batch_size, spatial_dim):
     return out
 
 
-def operand_copy(vox, col0, val, omap, num_heads, c, layout, to_operand):
+def operand_copy(vox, col0, val, omap, num_heads, c, layout, to_operand, scale=1.0):
     """Copy between a token tensor ``vox`` [N, stride] (columns ``col0 + h*c + ch``) and a sorted operand's
-    value array ``val`` [N*H*c]: layout 0 = Q/V order, 1 = K^T order; ``to_operand`` gives the direction."""
+    value array ``val`` [N*H*c]: layout 0 = Q/V order, 1 = K^T order; ``to_operand`` gives the direction.
+    ``scale`` (Q/V order only): the values are multiplied by it on the way."""
     lib = _lib.load()
     d = _dev(vox, val, omap)
     _check(vox.dim() == 2 and vox.stride(1) == 1 and val.is_contiguous() and vox.dtype == val.dtype,
@@ -176,10 +177,28 @@ def operand_copy(vox, col0, val, omap, num_heads, c, layout, to_operand):
     _check(vox.dtype in _DTYPE_CODE, f"unsupported value dtype {vox.dtype}")
     n_vox = vox.shape[0]
     _check(omap.numel() == 3 * n_vox + 2 and val.numel() == n_vox * num_heads * c, "operand_copy: sizes do not match")
-    with torch.cuda.device(d):
+    with _lib.on_device(d):
         _lib.check(lib.sswin_operand_copy(_DTYPE_CODE[vox.dtype], int(layout), 1 if to_operand else 0, _ptr(vox),
                                           vox.stride(0), int(col0), _ptr(val), _ptr(omap), n_vox, int(num_heads), int(c),
-                                          _stream(d)))
+                                          float(scale), _stream(d)))
+
+
+def operand_copy_qkv(vox, val_q, val_k, val_v, omap, num_heads, c, to_operand, q_scale=1.0):
+    """The three operand copies of one attention call in one launch: ``vox`` [N, 3*H*c] (a projection output, Q | K | V)
+    to or from ``val_q`` (Q/V order, times ``q_scale``), ``val_k`` (K^T order), ``val_v`` (Q/V order)."""
+    lib = _lib.load()
+    d = _dev(vox, val_q, val_k, val_v, omap)
+    n_vox = vox.shape[0]
+    _check(vox.dim() == 2 and vox.stride(1) == 1 and vox.shape[1] == 3 * num_heads * c, "operand_copy_qkv: vox must be [N, 3*H*c]")
+    _check(vox.dtype in _DTYPE_CODE, f"unsupported value dtype {vox.dtype}")
+    for val in (val_q, val_k, val_v):
+        _check(val.is_contiguous() and val.dtype == vox.dtype and val.numel() == n_vox * num_heads * c,
+               "operand_copy_qkv: operands must be contiguous [N*H*c] arrays of vox's dtype")
+    _check(omap.numel() == 3 * n_vox + 2, "operand_copy_qkv: sizes do not match")
+    with _lib.on_device(d):
+        _lib.check(lib.sswin_operand_copy_qkv(_DTYPE_CODE[vox.dtype], 1 if to_operand else 0, _ptr(vox), vox.stride(0), 0,
+                                              _ptr(val_q), _ptr(val_k), _ptr(val_v), _ptr(omap), n_vox, int(num_heads), int(c),
+                                              float(q_scale), _stream(d)))
 
 
 def sorted_coo_indices(indices, omap, num_heads, c, qv=True, k=True):
@@ -193,7 +212,7 @@ def sorted_coo_indices(indices, omap, num_heads, c, qv=True, k=True):
     idx_qv = torch.empty((4, e), dtype=torch.int32, device=d) if qv else None
     idx_k = torch.empty((4, e), dtype=torch.int32, device=d) if k else None
     if qv or k:
-        with torch.cuda.device(d):
+        with _lib.on_device(d):
             _lib.check(lib.sswin_sorted_coo_indices(_ptr(indices), _ptr(omap), n_vox, int(num_heads), int(c),
                                                     _ptr(idx_qv) if qv else None, _ptr(idx_k) if k else None, _stream(d)))
     return idx_qv, idx_k
@@ -242,7 +261,7 @@ def qkv_sparse_indices(indices, batch_size, spatial_dim, num_heads, c):
     ws = _ws(nbytes, d)
     # Indices the kernels cannot address (out of range, repeated pairs) are reported as an error by this call (it
     # waits for the stream); the two permutations of such input are all zero, so nothing reads out of bounds.
-    with torch.cuda.device(d):
+    with _lib.on_device(d):
         _check_pending()
         _lib.check(lib.sswin_qkv_sparse_indices(_ptr(indices), n_vox, int(batch_size), int(spatial_dim),
                                                 int(num_heads), int(c), _ptr(idx_qv), _ptr(sorted_qv),
@@ -428,7 +447,7 @@ def block_product(mat1_v, mat1_idx, mat1_shape, mat2_v, mat2_idx, mat2_shape, mu
     _check(m % inner == 0, f"operand nnz {m} is not a multiple of its dense last dimension {inner}")
     rows = m // inner
     stream = _stream(d)
-    with torch.cuda.device(d):
+    with _lib.on_device(d):
         plan, g_cap, (g, sum_c, sum_c2, c_max) = _plan_of(tok_idx, inner, s1[0] * s1[1], lib, d)
         if kind == 0:
             _check(not values or mat2_v.numel() == m, f"'q_k': mat2 holds {mat2_v.numel() if values else 0} values, expected {m}")
@@ -482,7 +501,7 @@ def permute_heads_order(indices, shape):
     m = indices.shape[1]
     if indices.dtype != torch.int32 or inner % 4 or m == 0 or m % inner or not indices.is_contiguous():
         return None
-    with torch.cuda.device(d):
+    with _lib.on_device(d):
         plan, g_cap, (g, _, _, _) = _plan_of(indices, inner, int(shape[0]) * int(shape[1]), lib, d)
         order = torch.empty(m, dtype=torch.int32, device=d)
         bad = torch.empty(1, dtype=torch.int32, device=d)
@@ -503,7 +522,7 @@ def softmax_rows_from_counts(_c, nnz):
     _check(_c.dtype == torch.int32 and _c.dim() == 1, "_c must be int32 [G]")
     c = _c.contiguous()
     rows = torch.empty(int(nnz), dtype=torch.int32, device=d)
-    with torch.cuda.device(d):
+    with _lib.on_device(d):
         scans, sum_c2 = _scans_for(c, lib, d)
         _check(sum_c2 is None or sum_c2 == nnz, f"softmax_rows_from_counts: {nnz} entries, the groups hold {sum_c2}")
         _lib.check(lib.sswin_softmax_rows_from_counts(_ptr(c), _ptr(scans), c.numel(), _ptr(rows), _stream(d)))
@@ -536,7 +555,7 @@ def group_row_positions(idx, gp):
     _check(idx.dtype == torch.int32 and idx.dim() == 2 and idx.shape[0] == 4, "group_row_positions: idx must be int32 [4, A]")
     idx = idx.contiguous()
     rows = torch.empty(max(gp.rows, 1), dtype=torch.int32, device=d)
-    with torch.cuda.device(d):
+    with _lib.on_device(d):
         _lib.check(lib.sswin_group_row_positions(_ptr(idx), idx.shape[1], _ptr(gp.plan), gp.g_cap, gp.groups, _ptr(rows),
                                                  _stream(d)))
     return rows
@@ -554,7 +573,7 @@ def group_add_bias_mask(values, row_pos, gp, n, bias32, mask):
     values, idx, bias32 = values.contiguous(), row_pos.contiguous(), bias32.contiguous()
     mask = None if mask is None else mask.contiguous()
     out = torch.empty_like(values)
-    with torch.cuda.device(d):
+    with _lib.on_device(d):
         _lib.check(lib.sswin_group_add_bias_mask(_DTYPE_CODE[values.dtype], _ptr(values), _ptr(idx), values.numel(), _ptr(gp.plan),
                                                  gp.g_cap, gp.groups, gp.c_max, int(n), _ptr(bias32),
                                                  _ptr(mask) if mask is not None else None,
@@ -575,7 +594,7 @@ def group_add_table_bias_mask(values, row_pos, gp, n, table32, code, offset0, ma
     values, idx, table32, code = values.contiguous(), row_pos.contiguous(), table32.contiguous(), code.contiguous()
     mask = None if mask is None else mask.contiguous()
     out = torch.empty_like(values)
-    with torch.cuda.device(d):
+    with _lib.on_device(d):
         _lib.check(lib.sswin_group_add_table_bias_mask(
             _DTYPE_CODE[values.dtype], _ptr(values), _ptr(idx), values.numel(), _ptr(gp.plan), gp.g_cap, gp.groups, gp.c_max, int(n),
             _ptr(table32), table32.shape[0], table32.shape[1], _ptr(code), int(offset0),
@@ -593,7 +612,7 @@ def group_bias_table_grad(grad_values, row_pos, gp, num_heads, n, code, offset0,
            "group_bias_table_grad: one int32 position per token row")
     grad_values, rows = grad_values.contiguous(), row_pos.contiguous()
     d_table = torch.empty((table_rows, num_heads), dtype=torch.float32, device=d)
-    with torch.cuda.device(d):
+    with _lib.on_device(d):
         nbytes = lib.sswin_bias_table_grad_workspace_bytes(gp.groups, int(num_heads), int(table_rows))
         ws = _ws(nbytes, d)
         _lib.check(lib.sswin_bias_table_grad(_ptr(gp.plan), gp.g_cap, gp.groups, _ptr(rows), 0, int(num_heads), int(n), _ptr(code),
@@ -613,7 +632,7 @@ def matmul_grad_cuda_naive(mat1_v, mat2_v, _c, C_, mul_type):
     mat1_v, mat2_v, _c = mat1_v.contiguous(), mat2_v.contiguous(), _c.contiguous()
     g, C_ = _c.numel(), int(C_)
     kind = _GRAD[mul_type]
-    with torch.cuda.device(d):
+    with _lib.on_device(d):
         scans, sum_c2 = _scans_for(_c, lib, d)
         if kind == 0:
             if sum_c2 is None:      # output size is data dependent: one read-back (reference ops.cu:968)
@@ -631,6 +650,34 @@ def matmul_grad_cuda_naive(mat1_v, mat2_v, _c, C_, mul_type):
     return out
 
 
+_GRAD_UNTRANSPOSED = {"tr_rc": 3, "tc_rr": 4}
+
+
+def matmul_grad_untransposed(mat1_v, mat2_v, _c, C_, mul_type):
+    """The second gradient of a block product from the operands as the forward pass left them (no counterpart among
+    the reference's operators; its Python backward, swin3d_base.py:121-134, transposes both operands first):
+    ``'tr_rc'``: out [c x C] = mat1[c x c]^T . mat2[c x C], equal to
+    ``matmul_grad_cuda_naive(qkv_transpose(mat1, 'rr'), qkv_transpose(mat2, 'rc'), 'rr_rc')``;
+    ``'tc_rr'``: out [C x c] = mat1[c x C]^T . mat2[c x c], equal to
+    ``matmul_grad_cuda_naive(qkv_transpose(mat1, 'rc'), qkv_transpose(mat2, 'rr'), 'cr_rr')``."""
+    lib = _lib.load()
+    _check(mul_type in _GRAD_UNTRANSPOSED, f"Invalid mul_type: {mul_type}. Expected 'tr_rc' or 'tc_rr'.")
+    _check(mat1_v.dtype == mat2_v.dtype, f"mat1 dtype {mat1_v.dtype} does not match mat2 dtype {mat2_v.dtype}")
+    _check(mat1_v.dtype in _DTYPE_CODE, f"unsupported value dtype {mat1_v.dtype}")
+    _check(_c.dtype == torch.int32, "_c must be int32")
+    d = _dev(mat1_v, mat2_v, _c)
+    mat1_v, mat2_v, _c = mat1_v.contiguous(), mat2_v.contiguous(), _c.contiguous()
+    g = _c.numel()
+    kind = _GRAD_UNTRANSPOSED[mul_type]
+    out = torch.empty_like(mat2_v if kind == 3 else mat1_v)
+    with _lib.on_device(d):
+        scans, _ = _scans_for(_c, lib, d)
+        if g > 0 and out.numel() > 0:
+            _lib.check(lib.sswin_block_matmul_grad(kind, _DTYPE_CODE[mat1_v.dtype], _ptr(mat1_v), _ptr(mat2_v),
+                                                   _ptr(_c), _ptr(scans), g, int(C_), _ptr(out), _stream(d)))
+    return out
+
+
 def qkv_transpose(mat1_v, _c, C_, mul_type):
     """Per-group transposes ``'rc'`` / ``'rr'`` (reference ops.cu:663-715, 1117-1132)."""
     lib = _lib.load()
@@ -641,7 +688,7 @@ def qkv_transpose(mat1_v, _c, C_, mul_type):
     mat1_v, _c = mat1_v.contiguous(), _c.contiguous()
     g = _c.numel()
     out = torch.empty_like(mat1_v)
-    with torch.cuda.device(d):
+    with _lib.on_device(d):
         scans, _ = _scans_for(_c, lib, d)
         if g > 0 and mat1_v.numel() > 0:
             _lib.check(lib.sswin_block_transpose(_TRANSPOSE[mul_type], _DTYPE_CODE[mat1_v.dtype], _ptr(mat1_v),
@@ -673,7 +720,7 @@ def softmax_last_dim_forward(indices, values):
     lib = _lib.load()
     d, dtype, work, indices, (values,) = _softmax_args(indices, values)
     out = torch.empty_like(values)
-    with torch.cuda.device(d):
+    with _lib.on_device(d):
         _lib.check(lib.sswin_softmax_last_dim_forward(_ptr(indices), _ptr(values), _DTYPE_CODE[work],
                                                       values.numel(), _ptr(out), _stream(d)))
     return out.to(dtype)
@@ -684,7 +731,7 @@ def softmax_last_dim_backward(indices, values, grad_values):
     lib = _lib.load()
     d, dtype, work, indices, (values, grad_values) = _softmax_args(indices, values, grad_values)
     out = torch.empty_like(values)
-    with torch.cuda.device(d):
+    with _lib.on_device(d):
         _lib.check(lib.sswin_softmax_last_dim_backward(_ptr(indices), _ptr(values), _ptr(grad_values),
                                                        _DTYPE_CODE[work], values.numel(), _ptr(out), _stream(d)))
     return out.to(dtype)

@@ -30,21 +30,18 @@ def _ptr(t):
     return C.c_void_p(t.data_ptr() if t is not None else 0)
 
 
-launch_timer = None      # a list turns on timing: entries (name, start event, stop event) of the attention launches
-
-
 @contextlib.contextmanager
 def _timed(name, device):
-    """Brackets one library launch with events on the stream it is enqueued on (only while
-    ``launch_timer`` is a list; a benchmark uses it to time the kernels inside a real step)."""
-    if launch_timer is None:
+    """Brackets one attention launch with events on the stream it is enqueued on, under a name of its own (only while
+    ``_lib.launch_timer`` is a list; a benchmark uses it to time the kernels inside a real step)."""
+    if _lib.launch_timer is None:
         yield
         return
     start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
     start.record(torch.cuda.current_stream(device))
     yield
     stop.record(torch.cuda.current_stream(device))
-    launch_timer.append((name, start, stop))
+    _lib.launch_timer.append((name, (), start, stop))
 
 
 class TokenPlan:
@@ -65,8 +62,8 @@ class TokenPlan:
         else:
             lib = _lib.load()
             d = self.device
-            with torch.cuda.device(d):
-                stream = C.c_void_p(torch.cuda.current_stream(d).cuda_stream)
+            with _lib.on_device(d):
+                stream = _lib.stream_handle(d)
                 _lib.check(lib.sswin_token_plan(_ptr(self._indices), self.N, self.B, self.n, self.H, _ptr(self.tokens),
                                                 _ptr(self.plan), self.g_cap, _ptr(self.tasks),
                                                 C.c_void_p(self._totals.data_ptr()), _ptr(self._ws), self._ws.numel(),
@@ -98,7 +95,7 @@ class TokenPlan:
         self.device = d
         self._totals = torch.zeros(9, dtype=torch.int64, pin_memory=True)
         self._indices = indices                      # kept alive until the kernels have run
-        with torch.cuda.device(d):
+        with _lib.on_device(d):
             nbytes = lib.sswin_token_plan_workspace_bytes(N, self.B, self.n)
             self._ws = torch.empty(int(nbytes), dtype=torch.uint8, device=d)
 
@@ -124,7 +121,7 @@ class TokenPlan:
         if any(p.device != d for p in plans):
             raise RuntimeError("TokenPlan.batch: all index sets must live on one device")
         lib = _lib.load()
-        with torch.cuda.device(d):
+        with _lib.on_device(d):
             stream = torch.cuda.current_stream(d)
             for k in range(0, len(plans), TokenPlan.MAX_BATCH):
                 chunk = plans[k:k + TokenPlan.MAX_BATCH]
@@ -159,7 +156,7 @@ class TokenPlan:
 
 def _tokens_to_sq(tp, dtype, epilogue, a, a_stride, a_col0, b, b_stride, b_col0, hd, scale, bias, mask, out, rows):
     lib = _lib.load()
-    stream = C.c_void_p(torch.cuda.current_stream(tp.device).cuda_stream)
+    stream = _lib.stream_handle(tp.device)
     _lib.check(lib.sswin_fused_tokens_to_sq(
         _DTYPE_CODE[dtype], 1 if epilogue else 0, _ptr(tp.plan), tp.g_cap, tp.G, _ptr(tp.tokens), tp.N, tp.H, hd,
         _ptr(a), a_stride, a_col0, _ptr(b), b_stride, b_col0, C.c_float(scale), _ptr(bias), tp.n, _ptr(mask),
@@ -168,7 +165,7 @@ def _tokens_to_sq(tp, dtype, epilogue, a, a_stride, a_col0, b, b_stride, b_col0,
 
 def _sq_to_tokens(tp, dtype, a_kmajor, sq, b, b_stride, b_col0, o, o_stride, o_col0, hd, scale):
     lib = _lib.load()
-    stream = C.c_void_p(torch.cuda.current_stream(tp.device).cuda_stream)
+    stream = _lib.stream_handle(tp.device)
     _lib.check(lib.sswin_fused_sq_to_tokens(
         _DTYPE_CODE[dtype], 1 if a_kmajor else 0, _ptr(tp.plan), tp.g_cap, tp.G, _ptr(tp.tokens), tp.N, hd,
         _ptr(sq), _ptr(b), b_stride, b_col0, _ptr(o), o_stride, o_col0, C.c_float(scale), stream))
@@ -180,10 +177,10 @@ def _bias32(bias, table_index, H, n, d):
         return bias.detach().to(torch.float32).contiguous()
     table32 = bias.detach().to(torch.float32).contiguous()
     bias32 = torch.empty((H, n, n), dtype=torch.float32, device=d)
-    with torch.cuda.device(d):
+    with _lib.on_device(d):
         _lib.check(_lib.load().sswin_bias_from_table(
             _ptr(table32), table32.shape[0], H, _ptr(table_index.code), table_index.offset0, n, _ptr(bias32),
-            C.c_void_p(torch.cuda.current_stream(d).cuda_stream)))
+            _lib.stream_handle(d)))
     return bias32
 
 
@@ -193,7 +190,7 @@ def _bias_gradient(tp, H, d_s, bias_meta, table_index):
     lib = _lib.load()
     d = d_s.device
     bias_dtype, bias_shape = bias_meta
-    stream = C.c_void_p(torch.cuda.current_stream(d).cuda_stream)
+    stream = _lib.stream_handle(d)
     if table_index is None:
         d_bias32 = torch.zeros(bias_shape, dtype=torch.float32, device=d)
         nbytes = lib.sswin_fused_bias_grad_workspace_bytes(tp.G, H, tp.n)
@@ -225,7 +222,7 @@ class _FusedWindowAttention(Function):
         bias32 = _bias32(bias, table_index, H, n, d)
         if mask is not None:
             mask = mask.to(torch.int8).contiguous()
-        with torch.cuda.device(d):
+        with _lib.on_device(d):
             s = torch.empty(tp.A, dtype=torch.float32, device=d)
             rows = torch.empty(tp.A, dtype=torch.int32, device=d)
             _tokens_to_sq(tp, dtype, True, qkv, 3 * D, 0, qkv, 3 * D, D, hd, scale, bias32, mask, s, rows)
@@ -247,7 +244,7 @@ class _FusedWindowAttention(Function):
         d = qkv.device
         grad_out = grad_out.contiguous().to(dtype)
         lib = _lib.load()
-        with torch.cuda.device(d):
+        with _lib.on_device(d):
             d_qkv = torch.empty_like(qkv)
             d_p = torch.empty(tp.A, dtype=torch.float32, device=d)
             # dP = dO V^T ; dV = P^T dO
@@ -285,10 +282,10 @@ class _ResidentWindowAttention(Function):
         if mask is not None:
             mask = mask.to(torch.int8).contiguous()
         lib = _lib.load()
-        with torch.cuda.device(d):
+        with _lib.on_device(d):
             out = torch.empty((N, D), dtype=dtype, device=d)
             lse = torch.empty(max(H * N, 1), dtype=torch.float32, device=d)
-            stream = C.c_void_p(torch.cuda.current_stream(d).cuda_stream)
+            stream = _lib.stream_handle(d)
             with _timed("window_attention_forward", d):
                 _lib.check(lib.sswin_window_attention_forward(
                     _DTYPE_CODE[dtype], _ptr(tp.tasks), tp.g_cap, tp.bucket_counts, _ptr(tp.tokens), N, H, hd,
@@ -310,11 +307,11 @@ class _ResidentWindowAttention(Function):
         d = qkv.device
         grad_out = grad_out.contiguous().to(dtype)
         lib = _lib.load()
-        with torch.cuda.device(d):
+        with _lib.on_device(d):
             d_qkv = torch.empty_like(qkv)
             want_bias = ctx.needs_input_grad[1]
             d_s = torch.empty(max(tp.A, 1), dtype=torch.float32, device=d) if want_bias else None
-            stream = C.c_void_p(torch.cuda.current_stream(d).cuda_stream)
+            stream = _lib.stream_handle(d)
             with _timed("window_attention_backward", d):
                 _lib.check(lib.sswin_window_attention_backward(
                     _DTYPE_CODE[dtype], _ptr(tp.tasks), tp.g_cap, tp.bucket_counts, _ptr(tp.tokens), N, H, hd,

@@ -34,7 +34,7 @@ def _i32x3(v):
 
 
 def _stream(device):
-    return C.c_void_p(torch.cuda.current_stream(device).cuda_stream)
+    return _lib.stream_handle(device)
 
 
 def get_window_size(x_size, window_size, shift_size=None):
@@ -143,7 +143,7 @@ def compute_mask(dims: List[int], window_size: List[int], shift_size: List[int],
         windows *= extent // w
     n = window_size[0] * window_size[1] * window_size[2]
     mask = torch.empty((windows, n), dtype=torch.int8, device=device)
-    with torch.cuda.device(device):
+    with _lib.on_device(device):
         _lib.check(_lib.load().sswin_shift_mask(_i32x3(dims), _i32x3(window_size), _i32x3(shift_size), _ptr(mask),
                                                 _stream(device)))
     _MASKS[key] = mask
@@ -167,7 +167,7 @@ def sparse_window_indices(indices: torch.Tensor, batch_size: int, dims: Sequence
         raise RuntimeError("sparse_window_indices: indices must be int32 [N, 4]")
     indices = indices.contiguous()
     out = torch.empty((indices.shape[0], 2), dtype=torch.int32, device=indices.device)
-    with torch.cuda.device(indices.device):
+    with _lib.on_device(indices.device):
         _lib.check(_lib.load().sswin_window_indices(_ptr(indices), indices.shape[0], int(batch_size), _i32x3(dims),
                                                     _i32x3(window_size), _i32x3(shift_size), _ptr(out),
                                                     _stream(indices.device)))
@@ -182,7 +182,7 @@ class _PoolWindows(Function):
         features = features.contiguous()
         M, channels = plan.windows, features.shape[1]
         out = torch.empty((M, channels), dtype=features.dtype, device=features.device)
-        with torch.cuda.device(features.device):
+        with _lib.on_device(features.device):
             _lib.check(_lib.load().sswin_pool_windows(
                 _DTYPE_CODE[features.dtype], 0, 1 if mean else 0, _ptr(plan.plan), plan.g_cap, M, _ptr(plan.tokens),
                 plan.N, _ptr(features), channels, channels, _ptr(out), channels, _stream(features.device)))
@@ -196,7 +196,7 @@ class _PoolWindows(Function):
         grad = grad.contiguous()
         channels = grad.shape[1]
         g_in = torch.empty((plan.N, channels), dtype=grad.dtype, device=grad.device)
-        with torch.cuda.device(grad.device):
+        with _lib.on_device(grad.device):
             _lib.check(_lib.load().sswin_pool_windows(
                 _DTYPE_CODE[grad.dtype], 1, 1 if ctx.mean else 0, _ptr(plan.plan), plan.g_cap, plan.windows,
                 _ptr(plan.tokens), plan.N, _ptr(grad), channels, channels, _ptr(g_in), channels, _stream(grad.device)))
@@ -228,7 +228,7 @@ def downsample_plan(x, factor: int = 2, plan=None):
         plan = TokenPlan(*req[:4], tasks=req[4], order_only=req[5])
     plan.finish()
     coords = torch.empty((plan.windows, 4), dtype=torch.int32, device=x.indices.device)
-    with torch.cuda.device(coords.device):
+    with _lib.on_device(coords.device):
         _lib.check(_lib.load().sswin_window_coords(_ptr(plan.plan), plan.g_cap, plan.windows, _i32x3(dims), _i32x3(win),
                                                    _ptr(coords), _stream(coords.device)))
     return plan, coords, [e // f for e in dims]

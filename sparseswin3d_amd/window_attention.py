@@ -28,6 +28,7 @@ import torch.nn as nn
 from torch.autograd import Function
 from torch.autograd.function import once_differentiable
 
+from . import _lib
 from . import custom_ops as ops
 
 
@@ -158,6 +159,12 @@ def _check_mul_type(mul_type):
         raise ValueError(f"Invalid value for 'mul': {mul_type}. Must be 'q_k' or 'qk_v'.")
 
 
+# The reference's backward of a block product (swin3d_base.py:121-134) transposes both operands of the second gradient
+# with ``qkv_transpose`` and multiplies the copies.  True: do the same (four transposed copies per attention); False
+# (default): the product reads the operands as they are (``ops.matmul_grad_untransposed``, same sums in the same order).
+TRANSPOSED_COPIES = False
+
+
 class _spspmm_block_naive(Function):
     """Window-blocked sparse x sparse product; gradients flow to both value arrays."""
 
@@ -187,15 +194,21 @@ class _spspmm_block_naive(Function):
             # S = Q K:  dQ = dS K^T (K^T is stored [C x c], so it is read along its rows);
             #           dK^T = Q^T dS, assembled from the two transposed operands.
             grad_mat1 = ops.matmul_grad_cuda_naive(grad_v, mat2_v, counts, inner, "rr_rc")
-            mat1_t = ops.qkv_transpose(mat1_v, counts, inner, "rc")
-            grad_t = ops.qkv_transpose(grad_v, counts, inner, "rr")
-            grad_mat2 = ops.matmul_grad_cuda_naive(mat1_t, grad_t, counts, inner, "cr_rr")
+            if TRANSPOSED_COPIES:
+                mat1_t = ops.qkv_transpose(mat1_v, counts, inner, "rc")
+                grad_t = ops.qkv_transpose(grad_v, counts, inner, "rr")
+                grad_mat2 = ops.matmul_grad_cuda_naive(mat1_t, grad_t, counts, inner, "cr_rr")
+            else:
+                grad_mat2 = ops.matmul_grad_untransposed(mat1_v, grad_v, counts, inner, "tc_rr")
         else:
             # O = P V:  dP = dO V^T;  dV = P^T dO.
             grad_mat1 = ops.matmul_grad_cuda_naive(grad_v, mat2_v, counts, inner, "rc_cr")
-            mat1_t = ops.qkv_transpose(mat1_v, counts, inner, "rr")
-            grad_t = ops.qkv_transpose(grad_v, counts, inner, "rc")
-            grad_mat2 = ops.matmul_grad_cuda_naive(mat1_t, grad_t, counts, inner, "rr_rc")
+            if TRANSPOSED_COPIES:
+                mat1_t = ops.qkv_transpose(mat1_v, counts, inner, "rr")
+                grad_t = ops.qkv_transpose(grad_v, counts, inner, "rc")
+                grad_mat2 = ops.matmul_grad_cuda_naive(mat1_t, grad_t, counts, inner, "rr_rc")
+            else:
+                grad_mat2 = ops.matmul_grad_untransposed(mat1_v, grad_v, counts, inner, "tr_rc")
         return grad_mat1, None, None, grad_mat2, None, None, None, None
 
 
@@ -263,14 +276,15 @@ class _SortedOperandValues(Function):
     gradients through ``index_add``; the same permutations applied directly, in both directions."""
 
     @staticmethod
-    def forward(ctx, qkv, omap):
+    def forward(ctx, qkv, omap, q_scale=1.0):
         n_vox, _, num_heads, c = qkv.shape
         flat = qkv.contiguous().view(n_vox, 3 * num_heads * c)
         out = [torch.empty(n_vox * num_heads * c, dtype=qkv.dtype, device=qkv.device) for _ in range(3)]
-        for slot, (val, layout) in enumerate(zip(out, (0, 1, 0))):
-            ops.operand_copy(flat, slot * num_heads * c, val, omap, num_heads, c, layout, True)
+        # one launch for the three; Q takes its factor on the way (the module's `q * self.scale`, swin3d_base.py:660)
+        ops.operand_copy_qkv(flat, *out, omap, num_heads, c, True, q_scale)
         ctx.save_for_backward(omap)
         ctx.shape = qkv.shape
+        ctx.q_scale = q_scale
         return tuple(out)
 
     @staticmethod
@@ -280,9 +294,8 @@ class _SortedOperandValues(Function):
         n_vox, _, num_heads, c = ctx.shape
         d_qkv = torch.empty(ctx.shape, dtype=d_q.dtype, device=d_q.device)
         flat = d_qkv.view(n_vox, 3 * num_heads * c)
-        for slot, (val, layout) in enumerate(zip((d_q, d_k, d_v), (0, 1, 0))):
-            ops.operand_copy(flat, slot * num_heads * c, val.contiguous(), omap, num_heads, c, layout, False)
-        return d_qkv, None
+        ops.operand_copy_qkv(flat, d_q.contiguous(), d_k.contiguous(), d_v.contiguous(), omap, num_heads, c, False, ctx.q_scale)
+        return d_qkv, None, None
 
 
 class _OperandToVoxels(Function):
@@ -310,11 +323,12 @@ class _OperandToVoxels(Function):
         return d_val, None, None, None
 
 
-def qkv_sparse_cuda(qkv: torch.Tensor, indices: torch.Tensor, batch_size: int, spatial_shape, plan=None):
+def qkv_sparse_cuda(qkv: torch.Tensor, indices: torch.Tensor, batch_size: int, spatial_shape, plan=None, q_scale=1.0):
     """Sorted COO operands Q [B,H,n,hd], K^T [B,H,hd,n], V [B,H,n,hd] from ``qkv`` [N,3,H,hd]
     (reference swin3d_base.py:483-498: same tensors; the index matrices and values are written in sorted
     order directly instead of being expanded, hashed, sorted and gathered).  The returned tensors carry
-    ``operand_map``, which :class:`_OperandToVoxels` takes to bring a product back to voxel order."""
+    ``operand_map``, which :class:`_OperandToVoxels` takes to bring a product back to voxel order.
+    ``q_scale``: Q's values come out multiplied by it (``q * q_scale`` without a pass of its own)."""
     num_heads, c = qkv.shape[2:]
     n = spatial_shape
     if plan is not None:
@@ -341,7 +355,7 @@ def qkv_sparse_cuda(qkv: torch.Tensor, indices: torch.Tensor, batch_size: int, s
         table = plan.plan.clone().view(5, plan.g_cap)
         table[1].mul_(num_heads).addcmul_(table[4], table[0])
         ops.register_index_plan(idx_qv, c, table.view(-1), plan.g_cap, plan.G, num_heads * plan.N, plan.A, plan.c_max)
-    q_val, k_val, v_val = _SortedOperandValues.apply(qkv, omap)
+    q_val, k_val, v_val = _SortedOperandValues.apply(qkv, omap, float(q_scale))
     q = SparseTensor(idx_qv, q_val, [batch_size, num_heads, n, c])
     k_t = SparseTensor(idx_k, k_val, [batch_size, num_heads, c, n])
     v = SparseTensor(idx_qv, v_val, [batch_size, num_heads, n, c])
@@ -398,11 +412,11 @@ class _GroupBiasMask(Function):
         from . import _lib
         import ctypes as C
         bias32 = torch.empty((num_heads, n, n), dtype=torch.float32, device=values.device)
-        with torch.cuda.device(values.device):
+        with _lib.on_device(values.device):
             _lib.check(_lib.load().sswin_bias_from_table(
                 C.c_void_p(table32.data_ptr()), table32.shape[0], num_heads, C.c_void_p(table_index.code.data_ptr()),
                 table_index.offset0, n, C.c_void_p(bias32.data_ptr()),
-                C.c_void_p(torch.cuda.current_stream(values.device).cuda_stream)))
+                _lib.stream_handle(values.device)))
         return ops.group_add_bias_mask(values, idx, gp, n, bias32, mask)
 
     @staticmethod
@@ -475,13 +489,13 @@ def _column_sum(t: torch.Tensor) -> torch.Tensor:
     from . import _lib
     lib = _lib.load()
     t = t.contiguous()
-    with torch.cuda.device(t.device):
+    with _lib.on_device(t.device):
         out = torch.empty(p, dtype=torch.float32, device=t.device)
         nbytes = lib.sswin_column_sum_workspace_bytes(t.shape[0], p)
         ws = torch.empty(int(nbytes), dtype=torch.uint8, device=t.device)
         _lib.check(lib.sswin_column_sum(C.c_void_p(t.data_ptr()), _SUM_DTYPE[t.dtype], t.shape[0], p,
                                         C.c_void_p(out.data_ptr()), C.c_void_p(ws.data_ptr()), nbytes,
-                                        C.c_void_p(torch.cuda.current_stream(t.device).cuda_stream)))
+                                        _lib.stream_handle(t.device)))
     return out.to(t.dtype)
 
 
@@ -504,13 +518,13 @@ def _split_linear_forward(x: torch.Tensor, weight: torch.Tensor, bias):
         x = x.clone()
     if weight.data_ptr() % 16:
         weight = weight.clone()
-    with torch.cuda.device(x.device):
+    with _lib.on_device(x.device):
         y = torch.empty(n, p, dtype=torch.float32, device=x.device)
         b = bias.contiguous() if bias is not None else None
         _lib.check(lib.sswin_tall_linear_forward(C.c_void_p(x.data_ptr()), n, k, C.c_void_p(weight.data_ptr()),
                                                  C.c_void_p(b.data_ptr() if b is not None else None), p,
                                                  C.c_void_p(y.data_ptr()),
-                                                 C.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)))
+                                                 _lib.stream_handle(x.device)))
     return y
 
 
@@ -533,11 +547,11 @@ def _split_linear_input_grad(grad_out: torch.Tensor, weight: torch.Tensor):
     weight = weight.contiguous()
     if grad_out.data_ptr() % 16:
         grad_out = grad_out.clone()
-    with torch.cuda.device(grad_out.device):
+    with _lib.on_device(grad_out.device):
         dx = torch.empty(n, k, dtype=torch.float32, device=grad_out.device)
         _lib.check(lib.sswin_tall_linear_input_grad(C.c_void_p(grad_out.data_ptr()), n, p, C.c_void_p(weight.data_ptr()), k,
                                                     C.c_void_p(dx.data_ptr()),
-                                                    C.c_void_p(torch.cuda.current_stream(grad_out.device).cuda_stream)))
+                                                    _lib.stream_handle(grad_out.device)))
     return dx
 
 
@@ -559,7 +573,7 @@ def _split_linear_weight_grad(grad_out: torch.Tensor, x: torch.Tensor, want_bias
     if nbytes == 0:
         return None, None
     x = x.contiguous()
-    with torch.cuda.device(x.device):
+    with _lib.on_device(x.device):
         dw = torch.empty(p, k, dtype=torch.float32, device=x.device)
         db = torch.empty(p, dtype=torch.float32, device=x.device) if want_bias else None
         ws = torch.empty(nbytes, dtype=torch.uint8, device=x.device)
@@ -567,7 +581,7 @@ def _split_linear_weight_grad(grad_out: torch.Tensor, x: torch.Tensor, want_bias
                                                      C.c_void_p(dw.data_ptr()),
                                                      C.c_void_p(db.data_ptr() if db is not None else None),
                                                      C.c_void_p(ws.data_ptr()), nbytes,
-                                                     C.c_void_p(torch.cuda.current_stream(x.device).cuda_stream)))
+                                                     _lib.stream_handle(x.device)))
     return dw, db
 
 
@@ -748,8 +762,8 @@ class WindowAttentionSparse(nn.Module):
                                                    mask, b, n, self.scale, resident, plan)
             x = replace_feature(x, out)
             return replace_feature(x, self.proj_drop(tall_linear(x.features, self.proj)))
-        q, k_t, v = qkv_sparse_cuda(qkv, x.indices, b, n, plan)
-        attn = spspmm_block_naive(q * self.scale, k_t, "q_k")
+        q, k_t, v = qkv_sparse_cuda(qkv, x.indices, b, n, plan, q_scale=self.scale)         # q = q * self.scale
+        attn = spspmm_block_naive(q, k_t, "q_k")
         biased = sp_add_table_bias_and_mask(attn, self.relative_position_bias_table, self._table_index(n), mask)
         if biased is not None:
             attn = biased

@@ -121,6 +121,30 @@ def test_qkv_transpose(ops, oracle, mix, hd, kind, dtype):
     np.testing.assert_array_equal(host(out), ref)          # pure data movement: exact
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16])
+@pytest.mark.parametrize("mix,H,hd", [("tiny", 2, 32), ("edges", 2, 32), ("mixed", 3, 32), ("full", 1, 32),
+                                      ("mixed", 1, 16), ("edges", 1, 64)])
+@pytest.mark.parametrize("kind", ["tr_rc", "tc_rr"])
+def test_matmul_grad_from_untransposed_operands(ops, oracle, mix, H, hd, kind, dtype):
+    """The second gradient of each product read from the operands as the forward pass left them: equal, bit for bit,
+    to the reference's composition of two transposes and a product (swin3d_base.py:123-125, 131-133), and within the
+    product tolerance of the oracle's composition in fp64."""
+    rng = np.random.default_rng(seed_of(mix, H, hd, kind))
+    c = np.repeat(np.array([x for x in MIXES[mix] if x > 0], np.int32), H)
+    mat = int((c.astype(np.int64) * hd).sum())
+    sq = int((c.astype(np.int64) ** 2).sum())
+    n1, n2, t1, t2, prod = {"tr_rc": (sq, mat, "rr", "rc", "rr_rc"), "tc_rr": (mat, sq, "rc", "rr", "cr_rr")}[kind]
+    m1 = dev(rng.standard_normal(n1), dtype)
+    m2 = dev(rng.standard_normal(n2), dtype)
+    cd = dev(c)
+    out = ops.matmul_grad_untransposed(m1, m2, cd, hd, kind)
+    composed = ops.matmul_grad_cuda_naive(ops.qkv_transpose(m1, cd, hd, t1), ops.qkv_transpose(m2, cd, hd, t2), cd, hd, prod)
+    assert out.dtype == dtype and torch.equal(out, composed)
+    r1, r2 = oracle.qkv_transpose(host(m1), c, hd, t1), oracle.qkv_transpose(host(m2), c, hd, t2)
+    ref = oracle.matmul_grad_cuda_naive(r1, r2, c, hd, prod)
+    close(host(out), ref, RTOL[dtype], kind, mag=product_mag(oracle, "matmul_grad_cuda_naive", r1, r2, c, hd, prod))
+
+
 def test_backward_identities_through_transposes(ops, oracle):
     """The backward of 'q_k' as the reference's autograd Function composes it
     (sparse_swin/swin3d_base.py:119-126) against plain per-group matrix algebra in fp64."""
@@ -152,6 +176,7 @@ def test_backward_identities_through_transposes(ops, oracle):
         mo += cg * C_
     close(host(dq), np.concatenate(dq_ref), 1e-5, "dQ", mag=np.concatenate(dq_mag))
     close(host(dkt), np.concatenate(dkt_ref), 1e-5, "dK^T", mag=np.concatenate(dkt_mag))
+    assert torch.equal(ops.matmul_grad_untransposed(f["q"], g, c, C_, "tc_rr"), dkt)
 
 
 # ------------------------------------------------------------------------------------------ softmax

@@ -71,6 +71,57 @@ def test_operand_to_voxels_equals_permute_and_unsort(oracle, H, hd):
     assert torch.equal(g_fast, g_slow)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16, torch.float64])
+@pytest.mark.parametrize("hd", [32, 6])
+def test_copy_with_a_factor_equals_copy_then_multiply(dtype, hd):
+    """``operand_copy(..., scale)`` in both directions: the module's ``q * self.scale`` (swin3d_base.py:660) and its
+    gradient, folded into the copies; bit-equal to the copy followed by the tensor multiply."""
+    from sparseswin3d_amd import custom_ops as ops
+    rng = np.random.default_rng(11)
+    ind = ragged_window_indices(rng, [4, 0, 27, 9, 1], 27)
+    N, H = len(ind), 3
+    scale = hd ** -0.5
+    omap = ops.operand_map(dev(ind), 5, 27)
+    vox = torch.randn(N, 3 * H * hd, device="cuda", dtype=dtype)
+    plain = torch.empty(N * H * hd, device="cuda", dtype=dtype)
+    scaled = torch.empty_like(plain)
+    ops.operand_copy(vox, H * hd, plain, omap, H, hd, 0, True)
+    ops.operand_copy(vox, H * hd, scaled, omap, H, hd, 0, True, scale)
+    assert torch.equal(scaled, plain * scale)
+    back, back_scaled = torch.zeros_like(vox), torch.zeros_like(vox)
+    ops.operand_copy(back, 0, plain, omap, H, hd, 0, False)
+    ops.operand_copy(back_scaled, 0, plain, omap, H, hd, 0, False, scale)
+    assert torch.equal(back_scaled, back * scale)
+    with pytest.raises(RuntimeError, match="only the Q/V order takes a scale"):
+        ops.operand_copy(vox, H * hd, scaled, omap, H, hd, 1, True, scale)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16, torch.bfloat16, torch.float64])
+@pytest.mark.parametrize("hd", [32, 16, 6])
+def test_three_copies_in_one_launch(dtype, hd):
+    """``operand_copy_qkv`` against the three single copies it stands for, in both directions, bit for bit."""
+    from sparseswin3d_amd import custom_ops as ops
+    rng = np.random.default_rng(12)
+    counts = [4, 0, 27, 9, 1] + [int(x) for x in rng.integers(0, 28, 40)]
+    ind = ragged_window_indices(rng, counts, 27)
+    N, H = len(ind), 3
+    D = H * hd
+    scale = hd ** -0.5
+    omap = ops.operand_map(dev(ind), len(counts), 27)
+    vox = torch.randn(N, 3 * D, device="cuda", dtype=dtype)
+    one = [torch.empty(N * D, device="cuda", dtype=dtype) for _ in range(3)]
+    three = [torch.empty_like(t) for t in one]
+    ops.operand_copy_qkv(vox, *one, omap, H, hd, True, scale)
+    for slot, layout in enumerate((0, 1, 0)):
+        ops.operand_copy(vox, slot * D, three[slot], omap, H, hd, layout, True, scale if slot == 0 else 1.0)
+        assert torch.equal(one[slot], three[slot]), slot
+    back_one, back_three = torch.zeros_like(vox), torch.zeros_like(vox)
+    ops.operand_copy_qkv(back_one, *one, omap, H, hd, False, scale)
+    for slot, layout in enumerate((0, 1, 0)):
+        ops.operand_copy(back_three, slot * D, one[slot], omap, H, hd, layout, False, scale if slot == 0 else 1.0)
+    assert torch.equal(back_one, back_three)
+
+
 def test_strided_token_tensor_and_empty_input():
     from sparseswin3d_amd import custom_ops as ops
     rng = np.random.default_rng(3)
