@@ -177,13 +177,13 @@ def bench_encoder(device, args):
         run_encoder(wl)
     torch.cuda.synchronize()
     dt = (time.perf_counter() - t0) / args.steps
-    _lib.launch_timer = []
+    _lib.launch_timer, _lib.launch_timer_only = [], {"sswin_window_attention_forward"}
     for _ in range(5):
         run_encoder(wl)
     torch.cuda.synchronize()
     per_stage = [[] for _ in wl["stages"]]
-    fw = [(a, b) for name, _, a, b in _lib.launch_timer if name == "window_attention_forward"]
-    _lib.launch_timer = None
+    fw = [(a, b) for name, _, a, b in _lib.launch_timer if name == "sswin_window_attention_forward"]
+    _lib.launch_timer = _lib.launch_timer_only = None
     for i, (a, b) in enumerate(fw):
         per_stage[i % len(per_stage)].append(a.elapsed_time(b))
     stage_ms = [sum(v) / len(v) for v in per_stage]
@@ -553,7 +553,9 @@ def kernel_table(wl, reps=20, only=None):
         # device-to-device copy of known size that calibrates the FETCH_SIZE / WRITE_SIZE counters
         src = torch.empty(CALIBRATION_BYTES // 4, dtype=torch.float32, device=dev).normal_()
         dst = torch.empty_like(src)
-        picked = [e for e in r_entries + f_entries + entries + (projection_entries(wl) if code == 0 else []) if only in e[0]]
+        names = [o for o in only.split(",") if o]
+        picked = [e for e in r_entries + f_entries + entries + (projection_entries(wl) if code == 0 else [])
+                  if any(o in e[0] for o in names)]
         for name, fn, nbytes, calls, *_ in picked:
             log(f"profiling {name}: {reps} launches, algorithmic bytes {nbytes}")
             for _ in range(reps):
@@ -867,7 +869,7 @@ def main():
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel table")
     ap.add_argument("--kernels-json", default=None)
     ap.add_argument("--profile-kernel", default=None, metavar="NAME",
-                    help="run only the kernels whose table name contains NAME (for rocprofv3) and exit")
+                    help="run only the kernels whose table name contains NAME (several: comma separated; for rocprofv3) and exit")
     ap.add_argument("--profile-reps", type=int, default=5)
     ap.add_argument("--pmc-summary", nargs="+", default=None, metavar="DIR",
                     help="no GPU work: summarise the rocprofv3 --pmc csv output under these directories into "
@@ -922,13 +924,14 @@ def main():
     # library call (a few extra steps after the timed region, so the events do not perturb `value`)
     from sparseswin3d_amd import _lib
     _lib.launch_timer = []
+    _lib.launch_timer_only = {"sswin_window_attention_forward", "sswin_window_attention_backward"}
     for _ in range(max(3, min(10, args.steps))):
         run_step(wl)
     torch.cuda.synchronize()
     in_step = {}
     for name, _, start, stop in _lib.launch_timer:
-        in_step.setdefault(name, []).append(start.elapsed_time(stop))
-    _lib.launch_timer = None
+        in_step.setdefault(name.replace("sswin_", ""), []).append(start.elapsed_time(stop))
+    _lib.launch_timer = _lib.launch_timer_only = None
     in_step = {k: sum(v) / len(v) for k, v in in_step.items()}
     log("attention launches inside a step (HIP events, mean over both blocks): " +
         ", ".join(f"{k} {v:.4f} ms" for k, v in in_step.items()))

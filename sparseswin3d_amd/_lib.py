@@ -97,6 +97,7 @@ _lib = None
 # stream and leaves (name, leading integer arguments, start event, stop event) here.  A benchmark uses it to time the
 # kernels where they run, inside a module call or a step; None (the default) costs nothing.
 launch_timer = None
+launch_timer_only = None        # a set of entry point names restricts the timing to them (fewer events between the kernels)
 
 
 class _TimedLibrary:
@@ -108,7 +109,8 @@ class _TimedLibrary:
     def __getattr__(self, name):
         fn = getattr(self._lib, name)
         sig = SIGNATURES.get(name)
-        if launch_timer is None or sig is None or sig[0] is not _i32 or not sig[1] or sig[1][-1] is not _vp:
+        if launch_timer is None or sig is None or sig[0] is not _i32 or not sig[1] or sig[1][-1] is not _vp or \
+                (launch_timer_only is not None and name not in launch_timer_only):
             return fn
 
         def call(*args):

@@ -384,20 +384,34 @@ __device__ __forceinline__ void rows_dot_to_table(const PadTab& tab, int lane, c
 //   3. key-side tasks of the groups of two tiles, the two tasks of a group side by side (KV_PAIR)
 //   4. key-side tasks of the groups of one tile (KV_SINGLE)
 // Heaviest tasks first, so the long ones start first and the short ones fill the tail.
+// Workgroups are dealt to the eight XCDs round robin: workgroup b runs on XCD b % 8, and every XCD has an L2 of its own.
+// xcd_run_order turns the workgroup number into a work number such that every XCD takes whole runs of XCD_RUN consecutive
+// work numbers, one after the other: neighbours in the work order (the heads of a window, the two sides of a group) run on
+// one XCD at about the same time and share what they read.  With 16-bit tokens the 64-byte slices of two heads of a
+// token share a 128-byte line: dealt to different XCDs, every line leaves memory twice (measured on 24 heads of bf16
+// tokens: 176 MB read for 62 MB of rows).  The launch holds xcd_run_grid(n) workgroups; work numbers >= n do nothing.
+constexpr int XCD_RUN = 16;
+__device__ __forceinline__ int64_t xcd_run_order(int64_t b) {
+    const int64_t k = b >> 3;
+    return ((k / XCD_RUN) * 8 + (b & 7)) * XCD_RUN + k % XCD_RUN;
+}
+inline int64_t xcd_run_grid(int64_t n) { return (n + 8 * XCD_RUN - 1) / (8 * XCD_RUN) * (8 * XCD_RUN); }
+
 struct BwdSegments {
     int64_t wg_kv, wg_pair, wg_single;   // first workgroup of segments 2, 3, 4
     int64_t n_big;                       // tasks per side of the groups of three and four tiles
     int64_t n_pair;                      // key-side tasks of the groups of two tiles (even)
     int64_t wgs;                         // workgroups of the launch
 };
-inline BwdSegments make_segments(const WAttnCommon& a) {
+// pairs: segments 1 and 2 interleaved workgroup by workgroup (work order of xcd_run_order) instead of in runs of eight
+inline BwdSegments make_segments(const WAttnCommon& a, bool pairs = false) {
     BwdSegments sg;
     sg.n_big = a.first[2];
     sg.n_pair = a.first[3] - a.first[2];
     const int64_t n_single = a.first[4] - a.first[3];
     const int64_t wg_big = (sg.n_big + 3) / 4;
     sg.wg_kv = wg_big;
-    sg.wg_pair = 16 * ((wg_big + 7) / 8);                  // both sides, interleaved in runs of eight workgroups
+    sg.wg_pair = pairs ? 2 * wg_big : 16 * ((wg_big + 7) / 8);   // both sides, interleaved
     sg.wg_single = sg.wg_pair + (sg.n_pair + 3) / 4;
     sg.wgs = sg.wg_single + (n_single + 3) / 4;
     return sg;

@@ -461,7 +461,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
     int64_t d, rec;
     int bi;
-    if (!locate(a, (int64_t)blockIdx.x * 4 + wave, d, bi, rec)) return;
+    if (!locate(a, xcd_run_order(blockIdx.x) * 4 + wave, d, bi, rec)) return;
     // the descriptor, the queries' indices and those of the first key tile: one round trip
     const int4 desc = a.tasks[d];
     const int l32 = threadIdx.x & 31;
@@ -894,7 +894,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     const float* __restrict__ lse, TokenTensor32 tdq) {
     __shared__ __attribute__((aligned(16))) float tiles[4][2][TILE_WORDS];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    bwd_q_task<T, MASK>(a, (int64_t)blockIdx.x * 4 + wave, tiles[wave][0], tiles[wave][1], tq, tk, tv, to, tdo, lse, tdq);
+    bwd_q_task<T, MASK>(a, xcd_run_order(blockIdx.x) * 4 + wave, tiles[wave][0], tiles[wave][1], tq, tk, tv, to, tdo, lse, tdq);
 }
 
 template <typename T, bool MASK>
@@ -903,7 +903,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     const float* __restrict__ lse, TokenTensor32 tdk, TokenTensor32 tdv, float* __restrict__ ds_out) {
     __shared__ __attribute__((aligned(16))) float tiles[4][2][TILE_WORDS];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    bwd_kv_task<T, MASK, KV_ONLY>(a, (int64_t)blockIdx.x * 4 + wave, true, tiles[wave][0], tiles[wave][1], nullptr, nullptr,
+    bwd_kv_task<T, MASK, KV_ONLY>(a, xcd_run_order(blockIdx.x) * 4 + wave, true, tiles[wave][0], tiles[wave][1], nullptr, nullptr,
                                   tq, tk, tv, to, tdo, lse, tdk, tdv, ds_out, tdk);
 }
 
@@ -916,16 +916,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
     __shared__ __attribute__((aligned(16))) float tiles[4][2][TILE_WORDS];
     __shared__ __attribute__((aligned(16))) float xch[4][64 * 16];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-    const int64_t wg = blockIdx.x;
+    const int64_t wg = xcd_run_order(blockIdx.x);
+    if (wg >= sg.wgs) return;
     float* t0 = tiles[wave][0];
     float* t1 = tiles[wave][1];
     if (wg < sg.wg_pair) {
-        // query side and key side of the larger groups interleaved in runs of eight workgroups: both sides of a
-        // group run on one XCD at about the same time and share its L2
-        const int64_t quad = (wg >> 4) * 8 + (wg & 7);
+        // query side and key side of the larger groups side by side in the work order: both sides of a group, and
+        // the heads of a window, run on one XCD at about the same time and share its L2
+        const int64_t quad = wg >> 1;
         const int64_t task = quad * 4 + wave;
         if (task < sg.n_big) {
-            if ((wg & 8) == 0)
+            if ((wg & 1) == 0)
                 bwd_q_task<T, MASK>(a, task, t0, t1, tq, tk, tv, to, tdo, lse, tdq);
             else
                 bwd_kv_task<T, MASK, KV_ONLY>(a, task, true, t0, t1, nullptr, nullptr, tq, tk, tv, to, tdo, lse, tdk, tdv,
@@ -947,12 +948,12 @@ static void launch_backward(const WAttnCommon& a, const TokenTensor32& q, const 
                             const TokenTensor32& o, const TokenTensor32& d_o, const float* lse, const TokenTensor32& dq,
                             const TokenTensor32& dk, const TokenTensor32& dv, float* ds_out, int sides, hipStream_t s) {
     if (sides == 3) {
-        const BwdSegments sg = make_segments(a);
-        hipLaunchKernelGGL((wattn16_bwd_all_kernel<T, MASK>), dim3((unsigned)sg.wgs), dim3(256), 0, s, a, sg, q, k, v, o, d_o,
-                           lse, dq, dk, dv, ds_out);
+        const BwdSegments sg = make_segments(a, true);
+        hipLaunchKernelGGL((wattn16_bwd_all_kernel<T, MASK>), dim3((unsigned)xcd_run_grid(sg.wgs)), dim3(256), 0, s, a, sg, q, k,
+                           v, o, d_o, lse, dq, dk, dv, ds_out);
         return;
     }
-    const unsigned blocks = (unsigned)((a.first[4] + 3) / 4);
+    const unsigned blocks = (unsigned)xcd_run_grid((a.first[4] + 3) / 4);
     if (sides & 1)
         hipLaunchKernelGGL((wattn16_bwd_q_kernel<T, MASK>), dim3(blocks), dim3(256), 0, s, a, q, k, v, o, d_o, lse, dq);
     if (sides & 2)
@@ -963,7 +964,7 @@ static void launch_backward(const WAttnCommon& a, const TokenTensor32& q, const 
 template <typename T>
 static void forward_t(const WAttnCommon& a, const TokenTensor32& q, const TokenTensor32& k, const TokenTensor32& v,
                       const TokenTensor32& o, float* lse, hipStream_t s) {
-    const unsigned blocks = (unsigned)((a.first[4] + 3) / 4);
+    const unsigned blocks = (unsigned)xcd_run_grid((a.first[4] + 3) / 4);
     if (a.mask)
         hipLaunchKernelGGL((wattn16_fwd_kernel<T, true>), dim3(blocks), dim3(256), 0, s, a, q, k, v, o, lse);
     else

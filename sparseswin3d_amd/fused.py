@@ -13,7 +13,6 @@ materialised in HBM (P is needed by the backward pass).
 """
 from __future__ import annotations
 
-import contextlib
 import ctypes as C
 
 import torch
@@ -28,20 +27,6 @@ _DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
 
 def _ptr(t):
     return C.c_void_p(t.data_ptr() if t is not None else 0)
-
-
-@contextlib.contextmanager
-def _timed(name, device):
-    """Brackets one attention launch with events on the stream it is enqueued on, under a name of its own (only while
-    ``_lib.launch_timer`` is a list; a benchmark uses it to time the kernels inside a real step)."""
-    if _lib.launch_timer is None:
-        yield
-        return
-    start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
-    start.record(torch.cuda.current_stream(device))
-    yield
-    stop.record(torch.cuda.current_stream(device))
-    _lib.launch_timer.append((name, (), start, stop))
 
 
 class TokenPlan:
@@ -286,12 +271,11 @@ class _ResidentWindowAttention(Function):
             out = torch.empty((N, D), dtype=dtype, device=d)
             lse = torch.empty(max(H * N, 1), dtype=torch.float32, device=d)
             stream = _lib.stream_handle(d)
-            with _timed("window_attention_forward", d):
-                _lib.check(lib.sswin_window_attention_forward(
-                    _DTYPE_CODE[dtype], _ptr(tp.tasks), tp.g_cap, tp.bucket_counts, _ptr(tp.tokens), N, H, hd,
-                    *_token_args(qkv, 3 * D, 0), *_token_args(qkv, 3 * D, D), *_token_args(qkv, 3 * D, 2 * D),
-                    C.c_float(scale), _ptr(bias32), n, _ptr(mask), 0 if mask is None else mask.shape[0],
-                    *_token_args(out, D, 0), _ptr(lse), stream))
+            _lib.check(lib.sswin_window_attention_forward(
+                _DTYPE_CODE[dtype], _ptr(tp.tasks), tp.g_cap, tp.bucket_counts, _ptr(tp.tokens), N, H, hd,
+                *_token_args(qkv, 3 * D, 0), *_token_args(qkv, 3 * D, D), *_token_args(qkv, 3 * D, 2 * D),
+                C.c_float(scale), _ptr(bias32), n, _ptr(mask), 0 if mask is None else mask.shape[0],
+                *_token_args(out, D, 0), _ptr(lse), stream))
         ctx.save_for_backward(qkv, out, lse, bias32, mask)
         ctx.tp, ctx.scale, ctx.bias_meta, ctx.table_index = tp, scale, (bias.dtype, bias.shape), table_index
         return out
@@ -312,14 +296,13 @@ class _ResidentWindowAttention(Function):
             want_bias = ctx.needs_input_grad[1]
             d_s = torch.empty(max(tp.A, 1), dtype=torch.float32, device=d) if want_bias else None
             stream = _lib.stream_handle(d)
-            with _timed("window_attention_backward", d):
-                _lib.check(lib.sswin_window_attention_backward(
-                    _DTYPE_CODE[dtype], _ptr(tp.tasks), tp.g_cap, tp.bucket_counts, _ptr(tp.tokens), N, H, hd,
-                    *_token_args(qkv, 3 * D, 0), *_token_args(qkv, 3 * D, D), *_token_args(qkv, 3 * D, 2 * D),
-                    C.c_float(scale), _ptr(bias32), tp.n, _ptr(mask), 0 if mask is None else mask.shape[0],
-                    *_token_args(out, D, 0), *_token_args(grad_out, D, 0), _ptr(lse),
-                    *_token_args(d_qkv, 3 * D, 0), *_token_args(d_qkv, 3 * D, D), *_token_args(d_qkv, 3 * D, 2 * D),
-                    _ptr(d_s), 3, stream))
+            _lib.check(lib.sswin_window_attention_backward(
+                _DTYPE_CODE[dtype], _ptr(tp.tasks), tp.g_cap, tp.bucket_counts, _ptr(tp.tokens), N, H, hd,
+                *_token_args(qkv, 3 * D, 0), *_token_args(qkv, 3 * D, D), *_token_args(qkv, 3 * D, 2 * D),
+                C.c_float(scale), _ptr(bias32), tp.n, _ptr(mask), 0 if mask is None else mask.shape[0],
+                *_token_args(out, D, 0), *_token_args(grad_out, D, 0), _ptr(lse),
+                *_token_args(d_qkv, 3 * D, 0), *_token_args(d_qkv, 3 * D, D), *_token_args(d_qkv, 3 * D, 2 * D),
+                _ptr(d_s), 3, stream))
             d_bias = _bias_gradient(tp, H, d_s, ctx.bias_meta, ctx.table_index) if want_bias else None
         return d_qkv, d_bias, None, None, None, None, None, None, None
 
