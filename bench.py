@@ -74,7 +74,8 @@ def log(*a):
 def build_workload(device, name="cfg2"):
     from sparseswin3d_amd import synth
     from sparseswin3d_amd.window_attention import WindowAttentionSparse
-    w = {"cfg1": synth.config1, "cfg2": synth.config2, "cfg3": synth.config3, "cfg4": synth.config4}[name]()
+    w = {"cfg1": synth.config1, "cfg2": synth.config2, "cfg3": synth.config3, "cfg4": synth.config4,
+         "ref7": synth.config_ref7}[name]()
     dtype = torch.bfloat16 if w.dtype == "bf16" else torch.float32
     ws = w.window
     shift = tuple(s // 2 for s in ws)
@@ -477,6 +478,9 @@ def kernel_table(wl, reps=20, only=None):
             ("fused bias grad [H,n,n]", lambda: _lib.check(lib.sswin_fused_bias_grad(ptr(tp.plan), tp.g_cap, tp.G, ptr(tp.tokens), tp.N, H, b["n"], ptr(g_s), ptr(dbias), ptr(bg_ws), bg_bytes, stream)), 4 * A, 0),
         ]
 
+        if b["n"] > 128:                                    # the dense-bias gradient takes windows of at most 128 positions
+            f_entries = [e for e in f_entries if e[0] != "fused bias grad [H,n,n]"]
+
     # ---- the window-resident kernels (what the step runs for heads of 32 channels), in the workload's dtype ----
     qkv_r = qkv.reshape(N, 3 * D).to(tdt).contiguous()
     bias_r = torch.randn(H, b["n"], b["n"], device=dev)
@@ -520,7 +524,9 @@ def kernel_table(wl, reps=20, only=None):
         _lib.check(lib.sswin_bias_table_grad(ptr(tp.plan), tp.g_cap, tp.G, ptr(tp.tokens), tp.N, H, b["n"], ptr(ti.code),
                                              ti.offset0, n_table, ptr(ds_r), ptr(d_table), ptr(tg_ws), tg_bytes, stream))
 
-    r_fwd()                                       # lse and out_r must hold a real forward for the backward timings
+    resident_ok = hd == 32 and int(tp.c_max) <= 128       # otherwise the module runs the fused path
+    if resident_ok:
+        r_fwd()                                   # lse and out_r must hold a real forward for the backward timings
     # flops of a launch: 2 c^2 hd per product and group = 2 A hd per product (two in the forward, five in the backward)
     r_entries = [
         # what a stage (and the step) does: the plans of its two partitions from shared launches, nobody waiting for
@@ -537,6 +543,8 @@ def kernel_table(wl, reps=20, only=None):
     if code == 0:
         r_entries.append(("resident bias grad [H,n,n]", lambda: _lib.check(lib.sswin_fused_bias_grad(
             ptr(tp.plan), tp.g_cap, tp.G, ptr(tp.tokens), tp.N, H, b["n"], ptr(ds_r), ptr(dbias), ptr(bg_ws), bg_bytes, stream)), 4 * A, 0))
+    if not resident_ok:
+        r_entries = r_entries[:2]
 
     def measure(items, path):
         rows_ = []
@@ -606,7 +614,10 @@ def module_times(wl, reps=10):
         out.backward(wl["upstream"])
 
     out = {}
-    for name, fused_, resident in (("resident", True, True), ("fused", True, False), ("operators", False, None)):
+    hd = wl["dim"] // wl["heads"]
+    for name, fused_, resident in (("resident", True, True), ("fused", "always", False), ("operators", False, None)):
+        if name == "resident" and (hd != 32 or b["stats"]["c_max"] > 128):
+            continue                                          # the resident kernels do not take this shape
         attn.fused, attn.resident = fused_, resident
         out[name] = round(event_time_ms(once, reps), 4)
     attn.fused, attn.resident = keep
@@ -663,15 +674,20 @@ def projection_entries(wl):
         b = torch.randn(P, device=dev)
         dy = torch.randn(N, P, device=dev)
         io = 4 * N * (D + P)
-        entries += [
-            (f"{name} forward", (lambda w=w, b=b: wa._split_linear_forward(x, w, b)), io + 4 * P * D, 1),
-            (f"{name} weight+bias gradient", (lambda dy=dy: wa._split_linear_weight_grad(dy, x, True)), io + 4 * P * D, 1),
-        ]
+        # what the module runs: this library's kernels where they take the shape (calls = 1), else the library GEMM
+        own_f = wa._split_linear_forward(x, w, b) is not None
+        own_w = wa._split_linear_weight_grad(dy, x, True)[0] is not None
+        own_x = wa._split_linear_input_grad(dy, w) is not None
+        if own_f:
+            entries.append((f"{name} forward", (lambda w=w, b=b: wa._split_linear_forward(x, w, b)), io + 4 * P * D, 1))
+        if own_w:
+            entries.append((f"{name} weight+bias gradient", (lambda dy=dy: wa._split_linear_weight_grad(dy, x, True)), io + 4 * P * D, 1))
         def lib_dx(dy=dy, w=w):
             with wa._rocblas_gemm():
                 return dy @ w
 
-        entries.append((f"{name} input gradient", (lambda dy=dy, w=w: wa._split_linear_input_grad(dy, w)), io + 4 * P * D, 1))
+        if own_x:
+            entries.append((f"{name} input gradient", (lambda dy=dy, w=w: wa._split_linear_input_grad(dy, w)), io + 4 * P * D, 1))
 
         def lib_fwd(w=w, b=b):
             with wa._rocblas_gemm():
@@ -681,9 +697,9 @@ def projection_entries(wl):
             with wa._rocblas_gemm():
                 return dy.t() @ x, wa._column_sum(dy)
 
-        entries += [(f"{name} forward, library GEMM", lib_fwd, io + 4 * P * D, 0),
-                    (f"{name} weight+bias gradient, library GEMM + column sums", lib_wgrad, io + 4 * P * D, 0)]
-        entries.append((f"{name} input gradient, library GEMM", lib_dx, io + 4 * P * D, 0))
+        entries += [(f"{name} forward, library GEMM", lib_fwd, io + 4 * P * D, 0 if own_f else 1),
+                    (f"{name} weight+bias gradient, library GEMM + column sums", lib_wgrad, io + 4 * P * D, 0 if own_w else 1)]
+        entries.append((f"{name} input gradient, library GEMM", lib_dx, io + 4 * P * D, 0 if own_x else 1))
     return entries
 
 
@@ -775,14 +791,15 @@ def pmc_summary(dirs, out_name, workload, command, only=None):
         if k == cal:
             continue
         cs = {c: v for (kk, c), v in mean.items() if kk == k}
-        lines.append(k if len(k) < 150 else k[:150] + " ...")
+        lines.append(k if len(k) < 110 else k[:110] + " ...")
         nb = None
         if "FETCH_SIZE" in cs and "WRITE_SIZE" in cs and len(unit) == 2:
             rd, wr = cs["FETCH_SIZE"] * unit["FETCH_SIZE"], cs["WRITE_SIZE"] * unit["WRITE_SIZE"]
             nb = rd + wr
             lines.append(f"    HBM traffic per launch: read {rd / 1e6:.1f} MB + written {wr / 1e6:.1f} MB = {nb / 1e6:.1f} MB")
-        for c in sorted(cs):
-            lines.append(f"    {c:28s} {cs[c]:16.1f}   (n={len(acc[(k, c)])})")
+        raw = [f"{c}={cs[c]:.0f}" for c in sorted(cs)]
+        for i in range(0, len(raw), 5):                         # the counters themselves, five to a line
+            lines.append("    " + "  ".join(raw[i:i + 5]))
         if "SQ_WAVES" in cs and "SQ_INSTS_VALU" in cs:
             w = cs["SQ_WAVES"]
             lines.append(f"    per wave: {cs['SQ_INSTS_VALU'] / w:.0f} VALU, {cs.get('SQ_INSTS_MFMA', 0) / w:.1f} MFMA, "
@@ -804,6 +821,12 @@ def pmc_summary(dirs, out_name, workload, command, only=None):
                 if sym in k:
                     traffic.setdefault(workload, {})[name] = dict(bytes=round(nb), summary=f"profiles/{out_name}.txt",
                                                                   kernel=k[:120], sources=srcs, digest=source_digest(srcs))
+    # figures taken on other sources than the tree's are dropped
+    for w in list(traffic):
+        for name in list(traffic[w]):
+            rec = traffic[w][name]
+            if source_digest(rec["sources"]) != rec["digest"]:
+                del traffic[w][name]
     out = os.path.join(ROOT, "profiles", out_name + ".txt")
     with open(out, "w") as f:
         f.write("\n".join(lines))
@@ -829,10 +852,10 @@ def trace_summary(dirs, out_name, command):
         if not paths:
             sys.exit(f"no *kernel_stats.csv under {d}")
         rows = list(csv.DictReader(open(paths[0])))
-        bwd = sum(int(r["Calls"]) for r in rows if "wattn_bwd_all_kernel" in r["Name"])
+        bwd = sum(int(r["Calls"]) for r in rows if "_bwd_all_kernel" in r["Name"])
         steps = max(bwd // 2, 1)
         if bwd == 0:                                 # the forward-only encoder: four attention launches per pass
-            steps = max(sum(int(r["Calls"]) for r in rows if "wattn_fwd_kernel" in r["Name"]) // 4, 1)
+            steps = max(sum(int(r["Calls"]) for r in rows if "_fwd_kernel<" in r["Name"] and "wattn" in r["Name"]) // 4, 1)
         tot = sum(float(r["TotalDurationNs"]) for r in rows)
         groups = {"library GEMMs (Cijk_*)": 0.0, "kernels of this library (sswin::*)": 0.0, "PyTorch element-wise / copies": 0.0}
         lines += ["", f"{os.path.basename(d.rstrip('/'))}: {steps} steps, GPU kernel time {tot / 1e3 / steps:.1f} us per step "
@@ -862,9 +885,11 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=400)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5"],
+    ap.add_argument("--workload", default="cfg2", choices=["cfg1", "cfg2", "cfg3", "cfg4", "cfg5", "ref7"],
                     help="cfg2 is the benchmark (the configuration the metric is quoted on); cfg1, cfg3 and cfg4 are "
-                         "reported the same way, without the CPU leg; cfg5 is the forward pass of the four-stage encoder")
+                         "reported the same way, without the CPU leg; cfg5 is the forward pass of the four-stage encoder; "
+                         "ref7 is the room of cfg2 in the reference's own setting (window 7, 3 heads of 16 channels), which "
+                         "runs on the fused path")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-kernels", action="store_true", help="skip the per-kernel table")
     ap.add_argument("--kernels-json", default=None)
@@ -890,7 +915,8 @@ def main():
         return
     if args.pmc_summary:
         from sparseswin3d_amd import synth
-        name = {"cfg1": synth.config1, "cfg2": synth.config2, "cfg3": synth.config3, "cfg4": synth.config4}[args.workload]().name
+        name = {"cfg1": synth.config1, "cfg2": synth.config2, "cfg3": synth.config3, "cfg4": synth.config4,
+                "ref7": synth.config_ref7}[args.workload]().name
         pmc_summary(args.pmc_summary, args.pmc_name or f"pmc_{args.workload}", name, args.pmc_command, args.pmc_kernels)
         return
     if not torch.cuda.is_available():
@@ -970,25 +996,43 @@ def main():
                 f"= {alg / ms_ / 1e6:.1f} GB/s = {100 * alg / ms_ / 1e6 / HBM_PEAK_GBPS:.2f}% of HBM peak")
         # the step runs the window-resident path: its slowest kernel is the dominant one
         # (the token plan is a sequence of small launches, not a kernel)
-        dom = max((r for r in table if r["path"] == "resident" and "token_plan" not in r["kernel"]),
-                  key=lambda r: r["ms"] * r["calls"])
+        # the path the step runs (the module's own choice): resident where its kernels apply, else fused for windows of
+        # at most 128 positions, else the operator path
+        from sparseswin3d_amd import fused as fused_mod
+        run_path = "resident" if any(r["kernel"] == "resident forward" for r in table) else \
+            "fused" if fused_mod.pays(wl["blocks"][0]["n"]) else "operators"
+        dom = max((r for r in table if r["path"] == run_path and "token plan" not in r["kernel"] and "token_plan" not in r["kernel"]),
+                  key=lambda r: r.get("ms_in_module", r["ms"]) * r["calls"])
         # its duration inside the step (events above) is what the roofline entry uses; the same
         # launch repeated back to back on its own (the table) runs 10-20 % slower
         step_ms = in_step.get("window_attention_backward") if "backward (dQ,dK,dV,dS)" in dom["kernel"] else None
-        ms = step_ms or dom["ms"]
+        ms = step_ms or dom.get("ms_in_module") or dom["ms"]
         gbps = dom["algorithmic_bytes"] / ms / 1e6
         traffic, traffic_note = measured_traffic(wl["name"], dom["kernel"])
         roofline = dict(bound="hbm", kernel=dom["kernel"], achieved=round(gbps, 1),
                         peak=HBM_PEAK_GBPS, unit="GB/s", frac=round(gbps / HBM_PEAK_GBPS, 4),
                         traffic=traffic, traffic_source=traffic_note,
                         algorithmic_bytes=dom["algorithmic_bytes"], ms=round(ms, 4),
-                        ms_alone=round(dom["ms"], 4), timed="inside the step" if step_ms else "alone")
+                        ms_alone=round(dom["ms"], 4), path=run_path,
+                        timed="inside the step" if step_ms else "inside a module call" if dom.get("ms_in_module") else "alone")
         if dom.get("flops"):
             # the same launch against the matrix-core roof of the type its products run in
             tflops = dom["flops"] / ms / 1e9
             roofline["mfma"] = dict(achieved=round(tflops, 2), peak=MFMA_PEAK_TFLOPS[dtype_name], unit="TFLOP/s",
                                     frac=round(tflops / MFMA_PEAK_TFLOPS[dtype_name], 4), flops=dom["flops"],
                                     note="algorithmic flops: 2 c^2 hd per product and group, padding of the 32-token tiles not counted")
+        # the sparse softmax on its own (forward and backward), as the operator path runs it
+        for key, row_name in (("softmax_fwd", "softmax_last_dim_forward"), ("softmax_bwd", "softmax_last_dim_backward")):
+            row = next((r for r in table if r["kernel"] == row_name and r["path"] == "operators"), None)
+            if row:
+                t_bytes, t_note = measured_traffic(wl["name"], row_name)
+                ms_ = row.get("ms_in_module", row["ms"])
+                roofline[key] = dict(kernel=row_name, ms=round(ms_, 4), ms_alone=round(row["ms"], 4),
+                                     algorithmic_bytes=row["algorithmic_bytes"],
+                                     achieved=round(row["algorithmic_bytes"] / ms_ / 1e6, 1), unit="GB/s",
+                                     frac=round(row["algorithmic_bytes"] / ms_ / 1e6 / HBM_PEAK_GBPS, 4),
+                                     traffic=t_bytes, traffic_source=t_note,
+                                     timed="inside a module call" if "ms_in_module" in row else "alone")
         roofline["path_summaries"] = summary
         roofline["module_call_ms"] = module_times(wl)
         log(f"one module call forward+backward by path (ms, projections and glue included): {roofline['module_call_ms']}")
@@ -1005,8 +1049,8 @@ def main():
         "metric": "window-attn tokens/s fwd+bwd on 1 MI355X", "value": value, "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms_per_step,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": dtype_name, "data": "synthetic",
-        "config": {"workload": f"{wl['name']}: block pair (regular 5^3 windows, then shifted by 2) of "
-                               f"WindowAttentionSparse, dim {wl['dim']}, {wl['heads']} heads, forward+backward",
+        "config": {"workload": f"{wl['name']}: block pair (regular {wl['window'][0]}^3 windows, then shifted by "
+                               f"{wl['shift'][0]}) of WindowAttentionSparse, dim {wl['dim']}, {wl['heads']} heads, forward+backward",
                    "voxels": wl["N"], "attention_calls_per_step": calls, **sizes},
         "roofline": roofline, "cpu_baseline": cpu,
     }

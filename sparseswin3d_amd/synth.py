@@ -302,6 +302,14 @@ def config4():
     return Workload("cfg4_dense8k", c4, (30, 30, 10), 1, 768, 24, dtype="bf16")
 
 
+def config_ref7():
+    """The room of configuration 2 in the reference's own attention setting (config/scannet/semseg-swin-0-base.py:11-31:
+    window 7, 48 channels in 3 heads of 16)."""
+    c = room_scene(seed=2)
+    c4, _ = with_batch([c])
+    return Workload("ref7_room100k_window7_heads16", c4, (256, 256, 96), 1, 48, 3, window=(7, 7, 7))
+
+
 def config5_rooms(n_rooms: int = 4):
     rooms = [room_scene(seed=50 + i) for i in range(n_rooms)]
     c4, offsets = with_batch(rooms)
