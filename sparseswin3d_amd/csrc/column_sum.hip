@@ -113,8 +113,8 @@ int sswin_column_sum(const void* x, int dtype, int64_t N, int P, float* out, voi
     SSWIN_CHECK(out, "column_sum: null pointer");
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (N == 0) {
-        SSWIN_HIP(hipMemsetAsync(out, 0, (size_t)P * sizeof(float), s));
-        return 0;
+        zero_fill(out, (int64_t)P, s);
+        return launch_ok("column_sum");
     }
     SSWIN_CHECK(x && ws, "column_sum: null pointer");
     SSWIN_CHECK(((uintptr_t)x % 16) == 0, "column_sum: the matrix is not 16-byte aligned");

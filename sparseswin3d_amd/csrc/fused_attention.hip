@@ -1254,8 +1254,8 @@ int sswin_bias_table_grad(const int32_t* plan, int64_t g_cap, int64_t G, const i
     SSWIN_CHECK(d_table, "bias_table_grad: null pointer");
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (G == 0) {
-        SSWIN_HIP(hipMemsetAsync(d_table, 0, (size_t)table_rows * H * sizeof(float), s));
-        return 0;
+        zero_fill(d_table, (int64_t)table_rows * H, s);
+        return launch_ok("bias_table_grad");
     }
     SSWIN_CHECK(plan && tokens && code && ds && ws, "bias_table_grad: null pointer");
     SSWIN_CHECK(ws_bytes >= sswin_bias_table_grad_workspace_bytes(G, H, table_rows), "bias_table_grad: workspace too small");

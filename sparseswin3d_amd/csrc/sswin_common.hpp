@@ -139,4 +139,17 @@ template <> __device__ __forceinline__ __hip_bfloat16 from_acc<__hip_bfloat16>(f
     return __float2bfloat16(v);
 }
 
+// Zeros by a kernel instead of hipMemsetAsync: callers may capture these entry points into a HIP graph, and memset
+// nodes have given wrong results on replays of a captured graph.
+template <typename T>
+__global__ __launch_bounds__(256) void zero_fill_kernel(T* __restrict__ p, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x; i < n; i += (int64_t)gridDim.x * 256) p[i] = T(0);
+}
+template <typename T>
+inline void zero_fill(T* p, int64_t n, hipStream_t s) {
+    if (n <= 0) return;
+    const unsigned blocks = (unsigned)((n + 255) / 256 < 1024 ? (n + 255) / 256 : 1024);
+    hipLaunchKernelGGL((zero_fill_kernel<T>), dim3(blocks), dim3(256), 0, s, p, n);
+}
+
 }  // namespace sswin

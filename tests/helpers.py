@@ -78,7 +78,7 @@ def close(out, ref, rtol, what="", mag=None, seg=None):
     bound = rtol * scale + 1e-30                             # fp32 results below about 1e-38 underflow
     with np.errstate(divide="ignore", invalid="ignore"):
         ratio = np.where(bound > 0, err / bound, np.where(err > 0, np.inf, 0.0))
-        carrying = aref >= 0.1 * scale                       # elements of the size of their own scale
+        carrying = (aref >= 0.1 * scale) & (aref > 0)        # elements of the size of their own scale
         rel = float((err[carrying] / aref[carrying]).max()) if carrying.any() else 0.0
     worst = int(np.argmax(ratio))
     CHECK_LOG.append((what, float(ratio.flat[worst]), rel, rtol))

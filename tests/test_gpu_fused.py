@@ -381,3 +381,19 @@ def test_bias_from_table_matches_the_gather():
                                              C.c_void_p(torch.cuda.current_stream().cuda_stream)))
         ref = table[index.reshape(-1)].reshape(n, n, H).permute(2, 0, 1)
         assert torch.equal(out, ref)
+
+
+def test_sums_over_nothing_are_zero():
+    """The two reductions with an early exit for empty input (column sums of a matrix without rows, the bias-table
+    gradient of a product without groups) write zeros, through a kernel rather than a memset node."""
+    import ctypes as C
+    from sparseswin3d_amd import _lib
+    lib = _lib.load()
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    out = torch.full((96,), 7.0, device="cuda")
+    _lib.check(lib.sswin_column_sum(None, 0, 0, 96, C.c_void_p(out.data_ptr()), None, 0, stream))
+    assert torch.count_nonzero(out) == 0
+    table = torch.full((729, 3), 7.0, device="cuda")
+    _lib.check(lib.sswin_bias_table_grad(None, 0, 0, None, 0, 3, 125, None, 0, 729, None, C.c_void_p(table.data_ptr()),
+                                         None, 0, stream))
+    assert torch.count_nonzero(table) == 0
