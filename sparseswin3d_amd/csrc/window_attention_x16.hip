@@ -33,6 +33,13 @@
 #include "wattn_common.hpp"
 #include "wattn_x16.hpp"
 
+#ifndef X16_BWD_WAVES
+#define X16_BWD_WAVES 3
+#endif
+#ifndef X16_FWD_WAVES
+#define X16_FWD_WAVES 4
+#endif
+
 namespace sswin {
 namespace x16 {
 
@@ -455,7 +462,7 @@ __device__ __forceinline__ void fwd_task(const WAttnCommon& a, const GroupCtx& g
 }
 
 template <typename T, bool MASK>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void wattn16_fwd_kernel(
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(X16_FWD_WAVES, X16_FWD_WAVES))) void wattn16_fwd_kernel(
     WAttnCommon a, TokenTensor32 tq, TokenTensor32 tk, TokenTensor32 tv, TokenTensor32 to, float* __restrict__ lse) {
     __shared__ __attribute__((aligned(16))) float tiles[4][2][TILE_WORDS];
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -909,7 +916,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) voi
 
 // The whole backward in one launch (segments as described at BwdSegments).
 template <typename T, bool MASK>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(3, 3))) void wattn16_bwd_all_kernel(
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(X16_BWD_WAVES, X16_BWD_WAVES))) void wattn16_bwd_all_kernel(
     WAttnCommon a, BwdSegments sg, TokenTensor32 tq, TokenTensor32 tk, TokenTensor32 tv, TokenTensor32 to,
     TokenTensor32 tdo, const float* __restrict__ lse, TokenTensor32 tdq, TokenTensor32 tdk, TokenTensor32 tdv,
     float* __restrict__ ds_out) {
