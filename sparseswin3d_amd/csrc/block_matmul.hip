@@ -75,6 +75,10 @@ struct GroupTable {
 #ifndef BP_WAVES
 #define BP_WAVES 5
 #endif
+#ifndef BP_BUFFERED
+#define BP_BUFFERED 1
+#endif
+typedef uint32_t u32x4_b __attribute__((ext_vector_type(4)));
 #ifndef BP_WAVES_FWD
 #define BP_WAVES_FWD 4
 #endif
@@ -88,10 +92,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MODE >= 2 ?
     // the operand bases) stays in scalar registers and the loads take a scalar base with a 32-bit lane offset
     // (measured on cfg2: 'q_k' 47.5 -> 44 us, 'qk_v' 41 -> 37, 'tr_rc' / 'tc_rr' 40 -> 35; the products whose operands
     // are both read along their rows lose by it, 'rr_rc' 41 -> 51 us, and keep the lane-held number)
-    const int wave = (b_is_kmajor<MODE>() || a_is_kmajor<MODE>()) ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : threadIdx.x >> 6;
+    const int wave = (b_is_kmajor<MODE>() || a_is_kmajor<MODE>() || (BP_BUFFERED && std::is_same<T, float>::value && !EMIT))
+                         ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : threadIdx.x >> 6;
     const int lane = threadIdx.x & 63;
     const int half = lane >> 5, l32 = lane & 31;
     const int64_t g0 = (int64_t)blockIdx.x * GROUPS_PER_WG;
+    // float values without index rows, task state in scalars: blocks addressed through buffer descriptors
+    constexpr bool BUFFERED = BP_BUFFERED && std::is_same<T, float>::value && !EMIT;
 
     // blocks of the workgroup's four groups
     // sizes and offsets of the four groups leave in one round of loads (the offsets do not wait for the sizes)
@@ -146,6 +153,71 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MODE >= 2 ?
         const T* A = m1 + d.a_off;
         const T* B = m2 + d.b_off;
         f32x16 acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        if constexpr (BUFFERED) {
+            // Every block is addressed through a buffer descriptor of exactly its size (base and size are scalars):
+            // a lane whose row, column or reduction index lies outside the block forms an offset beyond it, loads
+            // zero and has its store dropped by the bounds check of the memory pipeline, so ragged blocks need no
+            // clamp, select or branch, and an access costs one vector add for its offset.
+            constexpr uint32_t OUTSIDE = 0x80000000u;
+            const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(A), 0, d.I * d.K * 4, 0x00020000);
+            const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(B), 0, d.K * d.J * 4, 0x00020000);
+            const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(out + d.o_off, 0, d.I * d.J * 4, 0x00020000);
+            for (int kc = 0; kc < d.K; kc += 32) {
+                const int chunk = d.K - kc < 32 ? d.K - kc : 32;
+                const int kh = (chunk + 1) >> 1;
+                const int left = half ? chunk - kh : kh;
+                uint32_t a[16], b[16];
+                if (a_is_kmajor<MODE>()) {
+                    // element (kc + half * kh + s, i): rows of k behind the block's last one are outside by themselves
+                    const uint32_t v0 = i_a < d.I ? (uint32_t)(half * kh * d.I + i_a) * 4u : OUTSIDE;
+#pragma unroll
+                    for (int s = 0; s < 16; ++s) a[s] = __builtin_amdgcn_raw_buffer_load_b32(ra, v0 + (uint32_t)((kc + s) * d.I * 4), 0, 0);
+                } else {
+                    // a row per lane: 16 consecutive values of row i; values of k behind the row's end belong to the
+                    // next row and are masked through their offsets
+                    const uint32_t v0 = i_a < d.I ? (uint32_t)(i_a * d.K + kc + half * kh) * 4u : OUTSIDE;
+                    if (chunk == 32) {
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) {
+                            const u32x4_b t = __builtin_amdgcn_raw_buffer_load_b128(ra, v0 + 16u * v, 0, 0);
+                            a[4 * v] = t.x; a[4 * v + 1] = t.y; a[4 * v + 2] = t.z; a[4 * v + 3] = t.w;
+                        }
+                    } else {
+#pragma unroll
+                        for (int s = 0; s < 16; ++s) a[s] = __builtin_amdgcn_raw_buffer_load_b32(ra, s < left ? v0 + 4u * s : OUTSIDE, 0, 0);
+                    }
+                }
+                if (b_is_kmajor<MODE>()) {
+                    const uint32_t v0 = j_b < d.J ? (uint32_t)(half * kh * d.J + j_b) * 4u : OUTSIDE;
+#pragma unroll
+                    for (int s = 0; s < 16; ++s) b[s] = __builtin_amdgcn_raw_buffer_load_b32(rb, v0 + (uint32_t)((kc + s) * d.J * 4), 0, 0);
+                } else {
+                    const uint32_t v0 = j_b < d.J ? (uint32_t)(j_b * d.K + kc + half * kh) * 4u : OUTSIDE;
+                    if (chunk == 32) {
+#pragma unroll
+                        for (int v = 0; v < 4; ++v) {
+                            const u32x4_b t = __builtin_amdgcn_raw_buffer_load_b128(rb, v0 + 16u * v, 0, 0);
+                            b[4 * v] = t.x; b[4 * v + 1] = t.y; b[4 * v + 2] = t.z; b[4 * v + 3] = t.w;
+                        }
+                    } else {
+#pragma unroll
+                        for (int s = 0; s < 16; ++s) b[s] = __builtin_amdgcn_raw_buffer_load_b32(rb, s < left ? v0 + 4u * s : OUTSIDE, 0, 0);
+                    }
+                }
+#pragma unroll
+                for (int s = 0; s < 16; ++s)
+                    if (s < kh)
+                        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_bit_cast(float, a[s]), __builtin_bit_cast(float, b[s]), acc, 0, 0, 0);
+            }
+            const uint32_t o0 = j_b < d.J ? (uint32_t)((bi * 32 + 4 * half) * d.J + j_b) * 4u : OUTSIDE;
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float v = acc[r];                      // (a bit_cast of the vector element itself reads element 0)
+                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), ro,
+                                                      o0 + (uint32_t)((8 * (r >> 2) + (r & 3)) * d.J * 4), 0, 0);
+            }
+            continue;
+        }
         for (int kc = 0; kc < d.K; kc += 32) {
             // the (at most 32) values of k of this round are split evenly between the two lane halves, so a
             // reduction over 16 channels takes eight matrix steps, not sixteen with one half feeding zeros
