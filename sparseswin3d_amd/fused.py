@@ -29,6 +29,9 @@ def _ptr(t):
     return C.c_void_p(t.data_ptr() if t is not None else 0)
 
 
+_PINNED_TOTALS = []      # pinned host buffers of finished plans, reused
+
+
 class TokenPlan:
     """Token order and per-group table of one set of (window, pos) voxel indices.
 
@@ -78,7 +81,7 @@ class TokenPlan:
         self.tasks = (torch.empty(int(lib.sswin_token_plan_task_ints(N, self.g_cap, self.H)), dtype=torch.int32, device=d)
                       if tasks else None)
         self.device = d
-        self._totals = torch.zeros(9, dtype=torch.int64, pin_memory=True)
+        self._totals = _PINNED_TOTALS.pop() if _PINNED_TOTALS else torch.zeros(9, dtype=torch.int64, pin_memory=True)
         self._indices = indices                      # kept alive until the kernels have run
         with _lib.on_device(d):
             nbytes = lib.sswin_token_plan_workspace_bytes(N, self.B, self.n)
@@ -132,6 +135,9 @@ class TokenPlan:
         if self.N > 0:
             _lib.check(_lib.load().sswin_token_plan_totals(C.c_void_p(self._totals.data_ptr()), self.H, self.g_cap))
         totals = self._totals.tolist()
+        if len(_PINNED_TOTALS) < 64:                 # the pinned buffer goes back for the next plan (allocating one costs
+            _PINNED_TOTALS.append(self._totals)      # the host tens of microseconds); the library writes all nine entries
+        self._totals = None
         self.G, self.windows, self.A, self.c_max = (int(totals[i]) for i in range(4))
         self.bucket_counts = (C.c_int64 * 4)(*(int(totals[4 + b]) for b in range(4)))
         self.oversize_groups = int(totals[8])
