@@ -92,13 +92,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MODE >= 2 ?
     // the operand bases) stays in scalar registers and the loads take a scalar base with a 32-bit lane offset
     // (measured on cfg2: 'q_k' 47.5 -> 44 us, 'qk_v' 41 -> 37, 'tr_rc' / 'tc_rr' 40 -> 35; the products whose operands
     // are both read along their rows lose by it, 'rr_rc' 41 -> 51 us, and keep the lane-held number)
-    const int wave = (b_is_kmajor<MODE>() || a_is_kmajor<MODE>() || (BP_BUFFERED && std::is_same<T, float>::value && !EMIT))
+    const int wave = (b_is_kmajor<MODE>() || a_is_kmajor<MODE>() || (BP_BUFFERED && !std::is_same<T, double>::value && !EMIT))
                          ? __builtin_amdgcn_readfirstlane(threadIdx.x >> 6) : threadIdx.x >> 6;
     const int lane = threadIdx.x & 63;
     const int half = lane >> 5, l32 = lane & 31;
     const int64_t g0 = (int64_t)blockIdx.x * GROUPS_PER_WG;
-    // float values without index rows, task state in scalars: blocks addressed through buffer descriptors
-    constexpr bool BUFFERED = BP_BUFFERED && std::is_same<T, float>::value && !EMIT;
+    // values without index rows, task state in scalars: blocks addressed through buffer descriptors
+    constexpr bool BUFFERED = BP_BUFFERED && !std::is_same<T, double>::value && !EMIT;
 
     // blocks of the workgroup's four groups
     // sizes and offsets of the four groups leave in one round of loads (the offsets do not wait for the sizes)
@@ -159,62 +159,92 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MODE >= 2 ?
             // zero and has its store dropped by the bounds check of the memory pipeline, so ragged blocks need no
             // clamp, select or branch, and an access costs one vector add for its offset.
             constexpr uint32_t OUTSIDE = 0x80000000u;
-            const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(A), 0, d.I * d.K * 4, 0x00020000);
-            const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(B), 0, d.K * d.J * 4, 0x00020000);
-            const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(out + d.o_off, 0, d.I * d.J * 4, 0x00020000);
+            constexpr uint32_t ES = (uint32_t)sizeof(T);               // 4 (float) or 2 (half, bfloat16)
+            const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(A), 0, d.I * d.K * (int)ES, 0x00020000);
+            const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(B), 0, d.K * d.J * (int)ES, 0x00020000);
+            const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(out + d.o_off, 0, d.I * d.J * (int)ES, 0x00020000);
+            auto load1 = [](const __amdgpu_buffer_rsrc_t& r, uint32_t off) __attribute__((always_inline)) -> float {
+                if constexpr (ES == 4) {
+                    const uint32_t u = __builtin_amdgcn_raw_buffer_load_b32(r, off, 0, 0);
+                    return __builtin_bit_cast(float, u);
+                } else {
+                    const uint16_t u = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(r, off, 0, 0);
+                    return to_acc(__builtin_bit_cast(T, u));
+                }
+            };
+            // 16 consecutive values from byte offset off (all inside or all outside the block)
+            auto load16 = [](const __amdgpu_buffer_rsrc_t& r, uint32_t off, float (&x)[16]) __attribute__((always_inline)) {
+                if constexpr (ES == 4) {
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        const u32x4_b t = __builtin_amdgcn_raw_buffer_load_b128(r, off + 16u * v, 0, 0);
+                        const uint32_t w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) x[4 * v + e] = __builtin_bit_cast(float, w[e]);
+                    }
+                } else {
+#pragma unroll
+                    for (int v = 0; v < 2; ++v) {
+                        const u32x4_b t = __builtin_amdgcn_raw_buffer_load_b128(r, off + 16u * v, 0, 0);
+                        const uint32_t w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            const uint16_t lo = (uint16_t)(w[e] & 0xffffu), hi = (uint16_t)(w[e] >> 16);
+                            x[8 * v + 2 * e] = to_acc(__builtin_bit_cast(T, lo));
+                            x[8 * v + 2 * e + 1] = to_acc(__builtin_bit_cast(T, hi));
+                        }
+                    }
+                }
+            };
             for (int kc = 0; kc < d.K; kc += 32) {
                 const int chunk = d.K - kc < 32 ? d.K - kc : 32;
                 const int kh = (chunk + 1) >> 1;
                 const int left = half ? chunk - kh : kh;
-                uint32_t a[16], b[16];
+                float a[16], b[16];
                 if (a_is_kmajor<MODE>()) {
                     // element (kc + half * kh + s, i): rows of k behind the block's last one are outside by themselves
-                    const uint32_t v0 = i_a < d.I ? (uint32_t)(half * kh * d.I + i_a) * 4u : OUTSIDE;
+                    const uint32_t v0 = i_a < d.I ? (uint32_t)(half * kh * d.I + i_a) * ES : OUTSIDE;
 #pragma unroll
-                    for (int s = 0; s < 16; ++s) a[s] = __builtin_amdgcn_raw_buffer_load_b32(ra, v0 + (uint32_t)((kc + s) * d.I * 4), 0, 0);
+                    for (int s = 0; s < 16; ++s) a[s] = load1(ra, v0 + (uint32_t)((kc + s) * d.I) * ES);
                 } else {
                     // a row per lane: 16 consecutive values of row i; values of k behind the row's end belong to the
                     // next row and are masked through their offsets
-                    const uint32_t v0 = i_a < d.I ? (uint32_t)(i_a * d.K + kc + half * kh) * 4u : OUTSIDE;
-                    if (chunk == 32) {
-#pragma unroll
-                        for (int v = 0; v < 4; ++v) {
-                            const u32x4_b t = __builtin_amdgcn_raw_buffer_load_b128(ra, v0 + 16u * v, 0, 0);
-                            a[4 * v] = t.x; a[4 * v + 1] = t.y; a[4 * v + 2] = t.z; a[4 * v + 3] = t.w;
-                        }
+                    const uint32_t v0 = i_a < d.I ? (uint32_t)(i_a * d.K + kc + half * kh) * ES : OUTSIDE;
+                    if (chunk == 32 && (ES == 4 || d.K % 8 == 0)) {      // 16-byte loads need rows that start at a multiple of 4 bytes
+                        load16(ra, v0, a);
                     } else {
 #pragma unroll
-                        for (int s = 0; s < 16; ++s) a[s] = __builtin_amdgcn_raw_buffer_load_b32(ra, s < left ? v0 + 4u * s : OUTSIDE, 0, 0);
+                        for (int s = 0; s < 16; ++s) a[s] = load1(ra, s < left ? v0 + ES * s : OUTSIDE);
                     }
                 }
                 if (b_is_kmajor<MODE>()) {
-                    const uint32_t v0 = j_b < d.J ? (uint32_t)(half * kh * d.J + j_b) * 4u : OUTSIDE;
+                    const uint32_t v0 = j_b < d.J ? (uint32_t)(half * kh * d.J + j_b) * ES : OUTSIDE;
 #pragma unroll
-                    for (int s = 0; s < 16; ++s) b[s] = __builtin_amdgcn_raw_buffer_load_b32(rb, v0 + (uint32_t)((kc + s) * d.J * 4), 0, 0);
+                    for (int s = 0; s < 16; ++s) b[s] = load1(rb, v0 + (uint32_t)((kc + s) * d.J) * ES);
                 } else {
-                    const uint32_t v0 = j_b < d.J ? (uint32_t)(j_b * d.K + kc + half * kh) * 4u : OUTSIDE;
-                    if (chunk == 32) {
-#pragma unroll
-                        for (int v = 0; v < 4; ++v) {
-                            const u32x4_b t = __builtin_amdgcn_raw_buffer_load_b128(rb, v0 + 16u * v, 0, 0);
-                            b[4 * v] = t.x; b[4 * v + 1] = t.y; b[4 * v + 2] = t.z; b[4 * v + 3] = t.w;
-                        }
+                    const uint32_t v0 = j_b < d.J ? (uint32_t)(j_b * d.K + kc + half * kh) * ES : OUTSIDE;
+                    if (chunk == 32 && (ES == 4 || d.K % 8 == 0)) {
+                        load16(rb, v0, b);
                     } else {
 #pragma unroll
-                        for (int s = 0; s < 16; ++s) b[s] = __builtin_amdgcn_raw_buffer_load_b32(rb, s < left ? v0 + 4u * s : OUTSIDE, 0, 0);
+                        for (int s = 0; s < 16; ++s) b[s] = load1(rb, s < left ? v0 + ES * s : OUTSIDE);
                     }
                 }
 #pragma unroll
                 for (int s = 0; s < 16; ++s)
-                    if (s < kh)
-                        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(__builtin_bit_cast(float, a[s]), __builtin_bit_cast(float, b[s]), acc, 0, 0, 0);
+                    if (s < kh) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], acc, 0, 0, 0);
             }
-            const uint32_t o0 = j_b < d.J ? (uint32_t)((bi * 32 + 4 * half) * d.J + j_b) * 4u : OUTSIDE;
+            const uint32_t o0 = j_b < d.J ? (uint32_t)((bi * 32 + 4 * half) * d.J + j_b) * ES : OUTSIDE;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const float v = acc[r];                      // (a bit_cast of the vector element itself reads element 0)
-                __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), ro,
-                                                      o0 + (uint32_t)((8 * (r >> 2) + (r & 3)) * d.J * 4), 0, 0);
+                const uint32_t off = o0 + (uint32_t)((8 * (r >> 2) + (r & 3)) * d.J) * ES;
+                if constexpr (ES == 4) {
+                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), ro, off, 0, 0);
+                } else {
+                    const T t = from_acc<T>(v);
+                    __builtin_amdgcn_raw_buffer_store_b16((short)__builtin_bit_cast(uint16_t, t), ro, off, 0, 0);
+                }
             }
             continue;
         }
