@@ -236,3 +236,29 @@ def test_three_paths_share_one_prefetched_token_plan():
         table = plans[0].plan.clone()
         assert before is None or torch.equal(table, before)        # nobody wrote into the shared plan
         before = table
+
+
+def test_operator_path_backward_with_and_without_transposed_copies():
+    """The operator path's backward reads the operands of the second gradients untransposed by default; with
+    ``window_attention.TRANSPOSED_COPIES`` it composes them as the reference does (qkv_transpose x 2 + product,
+    swin3d_base.py:121-134).  Same sums in the same order: all gradients bit-equal."""
+    from sparseswin3d_amd import synth, window_attention as wa
+    torch.manual_seed(3)
+    c4, grid = _scene()
+    win_idx, nw, n = synth.window_indices(c4, grid, (5, 5, 5), (2, 2, 2))
+    mask = torch.from_numpy(synth.shift_region_mask(synth.padded_shape(grid, (5, 5, 5)), (5, 5, 5), (2, 2, 2))).cuda()
+    attn = wa.WindowAttentionSparse(96, 3, (5, 5, 5), qkv_bias=True).cuda()
+    set_path(attn, "operators")
+    feats, up = torch.randn(len(win_idx), 96, device="cuda"), torch.randn(len(win_idx), 96, device="cuda")
+    grads = []
+    try:
+        for flag in (False, True):
+            wa.TRANSPOSED_COPIES = flag
+            attn.zero_grad(set_to_none=True)
+            x = feats.clone().requires_grad_(True)
+            attn(wa.SparseVoxelTensor(x, torch.from_numpy(win_idx).cuda(), (n,), nw), mask).features.backward(up)
+            grads.append([x.grad.clone()] + [p.grad.clone() for p in attn.parameters()])
+    finally:
+        wa.TRANSPOSED_COPIES = False
+    for a, b in zip(*grads):
+        assert torch.equal(a, b)
