@@ -389,7 +389,7 @@ __global__ __launch_bounds__(256) void block_transpose_kernel(const T* __restric
                                                               const int32_t* __restrict__ sq_start, int64_t G,
                                                               int C, T* __restrict__ out) {
     __shared__ __attribute__((aligned(16))) char lds[GROUPS_PER_WG][TR_LDS_BYTES];
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     T* t = reinterpret_cast<T*>(lds[wave]);
     constexpr int U = 8;                      // loads in flight per lane
     constexpr int cap = TR_LDS_BYTES / (int)sizeof(T);
@@ -498,7 +498,7 @@ __global__ __launch_bounds__(256) void emit_coo_kernel(GroupTable gt, int64_t G,
                                                        const int32_t* __restrict__ tok_pos,
                                                        int32_t* __restrict__ out_idx, int64_t out_nnz) {
     __shared__ int pos_s[GROUPS_PER_WG][MAX_POS];
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int64_t g = (int64_t)blockIdx.x * GROUPS_PER_WG + wave;
     if (g >= G) return;
     const int c = gt.c[g];

@@ -432,7 +432,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
                                                        const float* __restrict__ bias, int n,
                                                        const int8_t* __restrict__ mask, int n_mask_windows,
                                                        float* __restrict__ out, int32_t* __restrict__ row_ids) {
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int half = lane >> 5, l32 = lane & 31;
     const int64_t g0 = (int64_t)blockIdx.x * FUSED_GROUPS_PER_WG;
     const TaskSet ts = make_tasks(gt, g0, true, hd);
@@ -539,7 +539,7 @@ template <typename T, bool A_KMAJOR>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void fused_tok_kernel(FusedGroups gt, const int32_t* __restrict__ order, int hd,
                                                         const float* __restrict__ sq, TokenTensor tb,
                                                         TokenTensor to, float scale_out) {
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int half = lane >> 5, l32 = lane & 31;
     const int64_t g0 = (int64_t)blockIdx.x * FUSED_GROUPS_PER_WG;
     const TaskSet ts = make_tasks(gt, g0, false, hd);

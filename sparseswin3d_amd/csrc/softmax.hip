@@ -200,7 +200,7 @@ __global__ __launch_bounds__(256) void group_bias_mask_kernel(const T* __restric
     using AccT = typename acc_of<T>::type;
     __shared__ int32_t pos_j[4][GBM_MAX_C];                  // position | region << 16 of the columns
     __shared__ int32_t pos_i[4][GBM_ROWS];                   // ... of this block's rows
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int64_t g = (int64_t)blockIdx.x * 4 + wave;
     if (g >= G) return;
     const int c = cs[g];
