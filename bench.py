@@ -383,7 +383,7 @@ def kernel_table(wl, reps=20, only=None):
 
         def grad(kind, a, bb, out):
             return lambda: _lib.check(lib.sswin_block_matmul_grad(kind, 0, ptr(a), ptr(bb), ptr(cc), ptr(scans), G, hd,
-                                                                  ptr(out), stream))
+                                                                  E, ptr(out), stream))
 
         def tr(kind, a, out):
             return lambda: _lib.check(lib.sswin_block_transpose(kind, 0, ptr(a), ptr(cc), ptr(scans), G, hd, ptr(out), stream))

@@ -243,10 +243,12 @@ int sswin_block_matmul(int kind, int dtype, const void* mat1_v, const void* mat2
  * from the untransposed operands instead (the transposed copies are never written):
  *  SSWIN_GRAD_TR_RC: out[c x C] = m1[c x c]^T . m2[c x C]     = RR_RC(transpose_rr(m1), transpose_rc(m2))
  *  SSWIN_GRAD_TC_RR: out[C x c] = m1[c x C]^T . m2[c x c]     = CR_RR(transpose_rc(m1), transpose_rr(m2))
- * c: device int32 [G]; scans: device, from sswin_scan_counts.  Asynchronous. */
+ * c: device int32 [G]; scans: device, from sswin_scan_counts; mat_nnz: number of values of the [c x C] operand or
+ * result (sum of c*C over the groups, a host number: the numel of that tensor), from which the launch is sized for
+ * the mean group.  Asynchronous. */
 int sswin_block_matmul_grad(int kind, int dtype, const void* m1, const void* m2,
                             const int32_t* c, const int32_t* scans, int64_t G, int C,
-                            void* out, void* stream);
+                            int64_t mat_nnz, void* out, void* stream);
 
 /* qkv_transpose (sparse_swin/ops.cu:518-557, 663-715, 1117-1132, ops.h:30-35):
  *  SSWIN_TRANSPOSE_RC: per group [c x C] -> [C x c];  SSWIN_TRANSPOSE_RR: [c x c] -> transposed.
@@ -344,7 +346,7 @@ int sswin_fused_tokens_to_sq(int dtype, int epilogue, const int32_t* plan, int64
  * Replaces 'qk_v' + permute + un-sort (swin3d_base.py:672-675) and the backward products with
  * their transposes (:119-134).  Asynchronous. */
 int sswin_fused_sq_to_tokens(int dtype, int a_kmajor, const int32_t* plan, int64_t g_cap, int64_t G,
-                             const int32_t* tokens, int64_t N, int hd, const float* sq,
+                             const int32_t* tokens, int64_t N, int H, int hd, const float* sq,
                              const void* b_base, int64_t b_stride, int b_col0, void* o_base,
                              int64_t o_stride, int o_col0, float scale_out, void* stream);
 

@@ -51,7 +51,7 @@ SIGNATURES = {
     "sswin_scan_counts_workspace_bytes": (_sz, [_i64]),
     "sswin_scan_counts": (_i32, [_vp, _i64, _vp, _vp, _sz, _vp]),
     "sswin_block_matmul": (_i32, [_i32, _i32, _vp, _vp, _vp, _i64, _i32, _vp, _i64, _i64, _i64, _vp, _vp, _i64, _vp]),
-    "sswin_block_matmul_grad": (_i32, [_i32, _i32, _vp, _vp, _vp, _vp, _i64, _i32, _vp, _vp]),
+    "sswin_block_matmul_grad": (_i32, [_i32, _i32, _vp, _vp, _vp, _vp, _i64, _i32, _i64, _vp, _vp]),
     "sswin_block_transpose": (_i32, [_i32, _i32, _vp, _vp, _vp, _i64, _i32, _vp, _vp]),
     "sswin_softmax_last_dim_forward": (_i32, [_vp, _vp, _i32, _i64, _vp, _vp]),
     "sswin_softmax_last_dim_backward": (_i32, [_vp, _vp, _vp, _i32, _i64, _vp, _vp]),
@@ -62,7 +62,7 @@ SIGNATURES = {
     "sswin_token_plan_batch": (_i32, [_vp, _i32, _vp]),
     "sswin_fused_tokens_to_sq": (_i32, [_i32, _i32, _vp, _i64, _i64, _vp, _i64, _i32, _i32, _vp, _i64, _i32,
                                         _vp, _i64, _i32, C.c_float, _vp, _i32, _vp, _i32, _vp, _vp, _vp]),
-    "sswin_fused_sq_to_tokens": (_i32, [_i32, _i32, _vp, _i64, _i64, _vp, _i64, _i32, _vp, _vp, _i64, _i32,
+    "sswin_fused_sq_to_tokens": (_i32, [_i32, _i32, _vp, _i64, _i64, _vp, _i64, _i32, _i32, _vp, _vp, _i64, _i32,
                                         _vp, _i64, _i32, C.c_float, _vp]),
     "sswin_fused_bias_grad_workspace_bytes": (_sz, [_i64, _i32, _i32]),
     "sswin_fused_bias_grad": (_i32, [_vp, _i64, _i64, _vp, _i64, _i32, _i32, _vp, _vp, _vp, _sz, _vp]),
@@ -90,7 +90,7 @@ SIGNATURES = {
                                                _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i32, _vp]),
 }
 
-ABI_VERSION = 27
+ABI_VERSION = 28
 _lib = None
 
 # A list turns on timing of the library's launches: every call that takes a stream is bracketed by events on that

@@ -121,7 +121,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MODE >= 2 ?
     }
     const int total = first[GROUPS_PER_WG];
 
-    for (int t = wave; t < total; t += 4) {
+    // gridDim.y workgroups share the four groups' blocks (launches of large windows: a group of 227 tokens has 64 blocks)
+    for (int t = wave + 4 * (int)blockIdx.y; t < total; t += 4 * (int)gridDim.y) {
         int q = 0;
 #pragma unroll
         for (int qq = 1; qq < GROUPS_PER_WG; ++qq) q += (t >= first[qq]) ? 1 : 0;
@@ -196,6 +197,27 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MODE >= 2 ?
                     }
                 }
             };
+            // 8 consecutive values (a reduction over 16 channels: each lane half feeds eight of them)
+            auto load8 = [](const __amdgpu_buffer_rsrc_t& r, uint32_t off, float (&x)[16]) __attribute__((always_inline)) {
+                if constexpr (ES == 4) {
+#pragma unroll
+                    for (int v = 0; v < 2; ++v) {
+                        const u32x4_b t = __builtin_amdgcn_raw_buffer_load_b128(r, off + 16u * v, 0, 0);
+                        const uint32_t w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) x[4 * v + e] = __builtin_bit_cast(float, w[e]);
+                    }
+                } else {
+                    const u32x4_b t = __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
+                    const uint32_t w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) {
+                        const uint16_t lo = (uint16_t)(w[e] & 0xffffu), hi = (uint16_t)(w[e] >> 16);
+                        x[2 * e] = to_acc(__builtin_bit_cast(T, lo));
+                        x[2 * e + 1] = to_acc(__builtin_bit_cast(T, hi));
+                    }
+                }
+            };
             for (int kc = 0; kc < d.K; kc += 32) {
                 const int chunk = d.K - kc < 32 ? d.K - kc : 32;
                 const int kh = (chunk + 1) >> 1;
@@ -205,13 +227,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MODE >= 2 ?
                     // element (kc + half * kh + s, i): rows of k behind the block's last one are outside by themselves
                     const uint32_t v0 = i_a < d.I ? (uint32_t)(half * kh * d.I + i_a) * ES : OUTSIDE;
 #pragma unroll
-                    for (int s = 0; s < 16; ++s) a[s] = load1(ra, v0 + (uint32_t)((kc + s) * d.I) * ES);
+                    for (int s = 0; s < 8; ++s) a[s] = load1(ra, v0 + (uint32_t)((kc + s) * d.I) * ES);
+                    if (kh > 8) {
+#pragma unroll
+                        for (int s = 8; s < 16; ++s) a[s] = load1(ra, v0 + (uint32_t)((kc + s) * d.I) * ES);
+                    }
                 } else {
                     // a row per lane: 16 consecutive values of row i; values of k behind the row's end belong to the
                     // next row and are masked through their offsets
                     const uint32_t v0 = i_a < d.I ? (uint32_t)(i_a * d.K + kc + half * kh) * ES : OUTSIDE;
                     if (chunk == 32 && (ES == 4 || d.K % 8 == 0)) {      // 16-byte loads need rows that start at a multiple of 4 bytes
                         load16(ra, v0, a);
+                    } else if (chunk == 16 && (ES == 4 || d.K % 8 == 0)) {
+                        load8(ra, v0, a);
                     } else {
 #pragma unroll
                         for (int s = 0; s < 16; ++s) a[s] = load1(ra, s < left ? v0 + ES * s : OUTSIDE);
@@ -220,11 +248,17 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MODE >= 2 ?
                 if (b_is_kmajor<MODE>()) {
                     const uint32_t v0 = j_b < d.J ? (uint32_t)(half * kh * d.J + j_b) * ES : OUTSIDE;
 #pragma unroll
-                    for (int s = 0; s < 16; ++s) b[s] = load1(rb, v0 + (uint32_t)((kc + s) * d.J) * ES);
+                    for (int s = 0; s < 8; ++s) b[s] = load1(rb, v0 + (uint32_t)((kc + s) * d.J) * ES);
+                    if (kh > 8) {
+#pragma unroll
+                        for (int s = 8; s < 16; ++s) b[s] = load1(rb, v0 + (uint32_t)((kc + s) * d.J) * ES);
+                    }
                 } else {
                     const uint32_t v0 = j_b < d.J ? (uint32_t)(j_b * d.K + kc + half * kh) * ES : OUTSIDE;
                     if (chunk == 32 && (ES == 4 || d.K % 8 == 0)) {
                         load16(rb, v0, b);
+                    } else if (chunk == 16 && (ES == 4 || d.K % 8 == 0)) {
+                        load8(rb, v0, b);
                     } else {
 #pragma unroll
                         for (int s = 0; s < 16; ++s) b[s] = load1(rb, s < left ? v0 + ES * s : OUTSIDE);
@@ -544,8 +578,15 @@ __global__ __launch_bounds__(256) void emit_coo_kernel(GroupTable gt, int64_t G,
     }
 }
 
+template <int MODE>
+static unsigned task_slices(int64_t G, int C, int64_t mat_nnz) {
+    if (G <= 0 || C <= 0 || mat_nnz <= 0) return 1;
+    const double mean_c = (double)mat_nnz / ((double)C * (double)G);
+    return block_task_slices(mean_c, C, !(rows_are_channels<MODE>() || cols_are_channels<MODE>()), GROUPS_PER_WG);
+}
+
 template <typename T, int MODE, bool EMIT>
-static int launch_product(const void* m1, const void* m2, const GroupTable& gt, int64_t G, int C,
+static int launch_product(const void* m1, const void* m2, const GroupTable& gt, int64_t G, int C, int64_t mat_nnz,
                           const int32_t* tok_pos, void* out, int32_t* out_idx, int64_t out_nnz,
                           hipStream_t s) {
     if (G == 0) return 0;
@@ -557,7 +598,7 @@ static int launch_product(const void* m1, const void* m2, const GroupTable& gt, 
             // 'q_k' writes its four index rows from a streaming kernel (measured faster than carrying
             // them through the MFMA kernel); 'qk_v' keeps them in the product kernel
             constexpr bool split = EMIT && MODE == MODE_QK;
-            hipLaunchKernelGGL((block_product_mfma_kernel<T, MODE, EMIT && !split>), dim3(blocks), dim3(256), 0, s,
+            hipLaunchKernelGGL((block_product_mfma_kernel<T, MODE, EMIT && !split>), dim3(blocks, task_slices<MODE>(G, C, mat_nnz)), dim3(256), 0, s,
                                static_cast<const T*>(m1), static_cast<const T*>(m2), gt, G, C, tok_pos,
                                static_cast<T*>(out), out_idx, out_nnz);
             if (split)
@@ -575,13 +616,13 @@ static int launch_product(const void* m1, const void* m2, const GroupTable& gt, 
 
 template <int MODE, bool EMIT>
 static int dispatch_product(int dtype, const void* m1, const void* m2, const GroupTable& gt, int64_t G, int C,
-                            const int32_t* tok_pos, void* out, int32_t* out_idx, int64_t out_nnz,
+                            int64_t mat_nnz, const int32_t* tok_pos, void* out, int32_t* out_idx, int64_t out_nnz,
                             hipStream_t s) {
     switch (dtype) {
-        case SSWIN_F32: return launch_product<float, MODE, EMIT>(m1, m2, gt, G, C, tok_pos, out, out_idx, out_nnz, s);
-        case SSWIN_F16: return launch_product<__half, MODE, EMIT>(m1, m2, gt, G, C, tok_pos, out, out_idx, out_nnz, s);
-        case SSWIN_BF16: return launch_product<__hip_bfloat16, MODE, EMIT>(m1, m2, gt, G, C, tok_pos, out, out_idx, out_nnz, s);
-        case SSWIN_F64: return launch_product<double, MODE, EMIT>(m1, m2, gt, G, C, tok_pos, out, out_idx, out_nnz, s);
+        case SSWIN_F32: return launch_product<float, MODE, EMIT>(m1, m2, gt, G, C, mat_nnz, tok_pos, out, out_idx, out_nnz, s);
+        case SSWIN_F16: return launch_product<__half, MODE, EMIT>(m1, m2, gt, G, C, mat_nnz, tok_pos, out, out_idx, out_nnz, s);
+        case SSWIN_BF16: return launch_product<__hip_bfloat16, MODE, EMIT>(m1, m2, gt, G, C, mat_nnz, tok_pos, out, out_idx, out_nnz, s);
+        case SSWIN_F64: return launch_product<double, MODE, EMIT>(m1, m2, gt, G, C, mat_nnz, tok_pos, out, out_idx, out_nnz, s);
         default: return fail("unsupported value dtype %d", dtype);
     }
 }
@@ -630,29 +671,29 @@ int sswin_block_matmul(int kind, int dtype, const void* mat1_v, const void* mat2
     }
     if (!out_idx) {                                          // values only
         if (kind == SSWIN_MUL_Q_K)
-            return dispatch_product<MODE_QK, false>(dtype, mat1_v, mat2_v, gt, G, C, tok_pos, out_val, nullptr, out_nnz, s);
-        return dispatch_product<MODE_PV, false>(dtype, mat1_v, mat2_v, gt, G, C, tok_pos, out_val, nullptr, out_nnz, s);
+            return dispatch_product<MODE_QK, false>(dtype, mat1_v, mat2_v, gt, G, C, M, tok_pos, out_val, nullptr, out_nnz, s);
+        return dispatch_product<MODE_PV, false>(dtype, mat1_v, mat2_v, gt, G, C, M, tok_pos, out_val, nullptr, out_nnz, s);
     }
     if (kind == SSWIN_MUL_Q_K)
-        return dispatch_product<MODE_QK, true>(dtype, mat1_v, mat2_v, gt, G, C, tok_pos, out_val, out_idx, out_nnz, s);
-    return dispatch_product<MODE_PV, true>(dtype, mat1_v, mat2_v, gt, G, C, tok_pos, out_val, out_idx, out_nnz, s);
+        return dispatch_product<MODE_QK, true>(dtype, mat1_v, mat2_v, gt, G, C, M, tok_pos, out_val, out_idx, out_nnz, s);
+    return dispatch_product<MODE_PV, true>(dtype, mat1_v, mat2_v, gt, G, C, M, tok_pos, out_val, out_idx, out_nnz, s);
 }
 
 int sswin_block_matmul_grad(int kind, int dtype, const void* m1, const void* m2, const int32_t* c,
-                            const int32_t* scans, int64_t G, int C, void* out, void* stream) {
+                            const int32_t* scans, int64_t G, int C, int64_t mat_nnz, void* out, void* stream) {
     SSWIN_CHECK(kind >= SSWIN_GRAD_RC_CR && kind <= SSWIN_GRAD_TC_RR,
                 "Invalid mul_type code %d. Expected 'rc_cr', 'rr_rc', 'cr_rr', 'tr_rc' or 'tc_rr'.", kind);
-    SSWIN_CHECK(C > 0 && G >= 0, "block_matmul_grad: bad sizes");
+    SSWIN_CHECK(C > 0 && G >= 0 && mat_nnz >= 0, "block_matmul_grad: bad sizes");
     if (G == 0) return 0;
     SSWIN_CHECK(m1 && m2 && c && scans && out, "block_matmul_grad: null pointer");
     GroupTable gt{c, scans, scans + G, nullptr, nullptr};
     hipStream_t s = static_cast<hipStream_t>(stream);
     switch (kind) {
-        case SSWIN_GRAD_RC_CR: return dispatch_product<MODE_RC_CR, false>(dtype, m1, m2, gt, G, C, nullptr, out, nullptr, 0, s);
-        case SSWIN_GRAD_RR_RC: return dispatch_product<MODE_RR_RC, false>(dtype, m1, m2, gt, G, C, nullptr, out, nullptr, 0, s);
-        case SSWIN_GRAD_CR_RR: return dispatch_product<MODE_CR_RR, false>(dtype, m1, m2, gt, G, C, nullptr, out, nullptr, 0, s);
-        case SSWIN_GRAD_TR_RC: return dispatch_product<MODE_TR_RC, false>(dtype, m1, m2, gt, G, C, nullptr, out, nullptr, 0, s);
-        default: return dispatch_product<MODE_TC_RR, false>(dtype, m1, m2, gt, G, C, nullptr, out, nullptr, 0, s);
+        case SSWIN_GRAD_RC_CR: return dispatch_product<MODE_RC_CR, false>(dtype, m1, m2, gt, G, C, mat_nnz, nullptr, out, nullptr, 0, s);
+        case SSWIN_GRAD_RR_RC: return dispatch_product<MODE_RR_RC, false>(dtype, m1, m2, gt, G, C, mat_nnz, nullptr, out, nullptr, 0, s);
+        case SSWIN_GRAD_CR_RR: return dispatch_product<MODE_CR_RR, false>(dtype, m1, m2, gt, G, C, mat_nnz, nullptr, out, nullptr, 0, s);
+        case SSWIN_GRAD_TR_RC: return dispatch_product<MODE_TR_RC, false>(dtype, m1, m2, gt, G, C, mat_nnz, nullptr, out, nullptr, 0, s);
+        default: return dispatch_product<MODE_TC_RR, false>(dtype, m1, m2, gt, G, C, mat_nnz, nullptr, out, nullptr, 0, s);
     }
 }
 

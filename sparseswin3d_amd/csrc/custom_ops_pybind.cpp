@@ -155,7 +155,8 @@ at::Tensor matmul_grad_cuda_naive(const at::Tensor& mat1_v, const at::Tensor& ma
     }
     at::Tensor out = at::empty({out_n}, v1.options());
     SSWIN_OK(sswin_block_matmul_grad(kind, value_code(v1), v1.data_ptr(), v2.data_ptr(), c.data_ptr<int32_t>(),
-                                     scans.data_ptr<int32_t>(), G, C, out.data_ptr(), stream));
+                                     scans.data_ptr<int32_t>(), G, C, kind == SSWIN_GRAD_RC_CR ? v1.numel() : out_n,
+                                     out.data_ptr(), stream));
     return out;
 }
 

@@ -440,7 +440,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     const T* A = static_cast<const T*>(ta.base);
     const T* B = static_cast<const T*>(tb.base);
 
-    for (int t = wave; t < total; t += 4) {
+    for (int t = wave + 4 * (int)blockIdx.y; t < total; t += 4 * (int)gridDim.y) {   // gridDim.y workgroups share the groups' blocks
         int q, c, bi, bj;
         locate_task(ts, t, q, c, bi, bj);
         const int64_t g = g0 + q;
@@ -481,17 +481,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 #pragma unroll
                 for (int s = 0; s < 16; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], acc, 0, 0, 0);
             } else {
-                const int left = hd - kb;
-                load_run16<T>(pa + kb, clamp16(left), a);
-                load_run16<T>(pb + kb, clamp16(left), b);
+                // the channels left are split evenly between the two lane halves: a head of 16 channels takes eight
+                // matrix steps, not sixteen with one half feeding zeros
+                const int chunk = hd - kc;
+                const int kh = (chunk + 1) >> 1;
+                const int left = half ? chunk - kh : kh;
+                load_run16<T>(pa + kc + half * kh, left, a);
+                load_run16<T>(pb + kc + half * kh, left, b);
                 if (scale_a != 1.0f) {
 #pragma unroll
                     for (int s = 0; s < 16; ++s) a[s] *= scale_a;
                 }
-                const int steps = hd - kc;
 #pragma unroll
                 for (int s = 0; s < 16; ++s)
-                    if (s < steps) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], acc, 0, 0, 0);
+                    if (s < kh) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], acc, 0, 0, 0);
             }
         }
 
@@ -547,7 +550,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     const T* B = static_cast<const T*>(tb.base);
     T* O = static_cast<T*>(const_cast<void*>(to.base));
 
-    for (int t = wave; t < total; t += 4) {
+    for (int t = wave + 4 * (int)blockIdx.y; t < total; t += 4 * (int)gridDim.y) {   // gridDim.y workgroups share the groups' blocks
         int q, c, bi, bj;
         locate_task(ts, t, q, c, bi, bj);
         // a task belongs to the whole wavefront: its parameters go to scalar registers, and the block of the
@@ -953,28 +956,30 @@ __global__ __launch_bounds__(1024) void rpb_table_reduce_kernel(const float* __r
 }
 
 template <typename T>
-static int launch_sq(bool epi, const FusedGroups& gt, const int32_t* order, const int32_t* tok_pos, int H, int hd,
+static int launch_sq(bool epi, const FusedGroups& gt, double mean_c, const int32_t* order, const int32_t* tok_pos, int H, int hd,
                      const TokenTensor& ta, const TokenTensor& tb, float scale_a, const float* bias, int n,
                      const int8_t* mask, int nmw, float* out, int32_t* row_ids, hipStream_t s) {
-    const unsigned blocks = (unsigned)((gt.G + FUSED_GROUPS_PER_WG - 1) / FUSED_GROUPS_PER_WG);
+    const dim3 grid((unsigned)((gt.G + FUSED_GROUPS_PER_WG - 1) / FUSED_GROUPS_PER_WG),
+                    block_task_slices(mean_c, hd, true, FUSED_GROUPS_PER_WG));
     if (epi)
-        hipLaunchKernelGGL((fused_sq_kernel<T, true>), dim3(blocks), dim3(256), 0, s, gt, order, tok_pos, H, hd, ta,
+        hipLaunchKernelGGL((fused_sq_kernel<T, true>), grid, dim3(256), 0, s, gt, order, tok_pos, H, hd, ta,
                            tb, scale_a, bias, n, mask, nmw, out, row_ids);
     else
-        hipLaunchKernelGGL((fused_sq_kernel<T, false>), dim3(blocks), dim3(256), 0, s, gt, order, tok_pos, H, hd, ta,
+        hipLaunchKernelGGL((fused_sq_kernel<T, false>), grid, dim3(256), 0, s, gt, order, tok_pos, H, hd, ta,
                            tb, scale_a, bias, n, mask, nmw, out, row_ids);
     return launch_ok("fused tokens->sq product");
 }
 
 template <typename T>
-static int launch_tok(bool a_kmajor, const FusedGroups& gt, const int32_t* order, int hd, const float* sq,
+static int launch_tok(bool a_kmajor, const FusedGroups& gt, double mean_c, const int32_t* order, int hd, const float* sq,
                       const TokenTensor& tb, const TokenTensor& to, float scale_out, hipStream_t s) {
-    const unsigned blocks = (unsigned)((gt.G + FUSED_GROUPS_PER_WG - 1) / FUSED_GROUPS_PER_WG);
+    const dim3 grid((unsigned)((gt.G + FUSED_GROUPS_PER_WG - 1) / FUSED_GROUPS_PER_WG),
+                    block_task_slices(mean_c, hd, false, FUSED_GROUPS_PER_WG));
     if (a_kmajor)
-        hipLaunchKernelGGL((fused_tok_kernel<T, true>), dim3(blocks), dim3(256), 0, s, gt, order, hd, sq, tb, to,
+        hipLaunchKernelGGL((fused_tok_kernel<T, true>), grid, dim3(256), 0, s, gt, order, hd, sq, tb, to,
                            scale_out);
     else
-        hipLaunchKernelGGL((fused_tok_kernel<T, false>), dim3(blocks), dim3(256), 0, s, gt, order, hd, sq, tb, to,
+        hipLaunchKernelGGL((fused_tok_kernel<T, false>), grid, dim3(256), 0, s, gt, order, hd, sq, tb, to,
                            scale_out);
     return launch_ok("fused sq->tokens product");
 }
@@ -1166,28 +1171,30 @@ int sswin_fused_tokens_to_sq(int dtype, int epilogue, const int32_t* plan, int64
     hipStream_t s = static_cast<hipStream_t>(stream);
     const int32_t* order = tokens;
     const int32_t* tok_pos = tokens + 3 * N;
+    const double mean_c = (double)N * H / (double)G;          // every voxel is a token of one window, in each of its H groups
     switch (dtype) {
-        case SSWIN_F32: return launch_sq<float>(epilogue, gt, order, tok_pos, H, hd, ta, tb, scale_a, bias, n, mask, n_mask_windows, out, row_ids, s);
-        case SSWIN_F16: return launch_sq<__half>(epilogue, gt, order, tok_pos, H, hd, ta, tb, scale_a, bias, n, mask, n_mask_windows, out, row_ids, s);
-        case SSWIN_BF16: return launch_sq<__hip_bfloat16>(epilogue, gt, order, tok_pos, H, hd, ta, tb, scale_a, bias, n, mask, n_mask_windows, out, row_ids, s);
+        case SSWIN_F32: return launch_sq<float>(epilogue, gt, mean_c, order, tok_pos, H, hd, ta, tb, scale_a, bias, n, mask, n_mask_windows, out, row_ids, s);
+        case SSWIN_F16: return launch_sq<__half>(epilogue, gt, mean_c, order, tok_pos, H, hd, ta, tb, scale_a, bias, n, mask, n_mask_windows, out, row_ids, s);
+        case SSWIN_BF16: return launch_sq<__hip_bfloat16>(epilogue, gt, mean_c, order, tok_pos, H, hd, ta, tb, scale_a, bias, n, mask, n_mask_windows, out, row_ids, s);
         default: return fail("fused_tokens_to_sq: unsupported token dtype %d", dtype);
     }
 }
 
 int sswin_fused_sq_to_tokens(int dtype, int a_kmajor, const int32_t* plan, int64_t g_cap, int64_t G,
-                             const int32_t* tokens, int64_t N, int hd, const float* sq, const void* b_base,
+                             const int32_t* tokens, int64_t N, int H, int hd, const float* sq, const void* b_base,
                              int64_t b_stride, int b_col0, void* o_base, int64_t o_stride, int o_col0,
                              float scale_out, void* stream) {
-    SSWIN_CHECK(G >= 0 && G <= g_cap && N >= 0 && hd > 0, "fused_sq_to_tokens: bad sizes");
+    SSWIN_CHECK(G >= 0 && G <= g_cap && N >= 0 && H > 0 && hd > 0, "fused_sq_to_tokens: bad sizes");
     if (G == 0) return 0;
     SSWIN_CHECK(plan && tokens && sq && b_base && o_base, "fused_sq_to_tokens: null pointer");
     const FusedGroups gt = groups_of(plan, g_cap, G);
     const TokenTensor tb{b_base, b_stride, b_col0}, to{o_base, o_stride, o_col0};
     hipStream_t s = static_cast<hipStream_t>(stream);
+    const double mean_c = (double)N * H / (double)G;
     switch (dtype) {
-        case SSWIN_F32: return launch_tok<float>(a_kmajor, gt, tokens, hd, sq, tb, to, scale_out, s);
-        case SSWIN_F16: return launch_tok<__half>(a_kmajor, gt, tokens, hd, sq, tb, to, scale_out, s);
-        case SSWIN_BF16: return launch_tok<__hip_bfloat16>(a_kmajor, gt, tokens, hd, sq, tb, to, scale_out, s);
+        case SSWIN_F32: return launch_tok<float>(a_kmajor, gt, mean_c, tokens, hd, sq, tb, to, scale_out, s);
+        case SSWIN_F16: return launch_tok<__half>(a_kmajor, gt, mean_c, tokens, hd, sq, tb, to, scale_out, s);
+        case SSWIN_BF16: return launch_tok<__hip_bfloat16>(a_kmajor, gt, mean_c, tokens, hd, sq, tb, to, scale_out, s);
         default: return fail("fused_sq_to_tokens: unsupported token dtype %d", dtype);
     }
 }

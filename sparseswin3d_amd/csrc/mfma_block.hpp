@@ -62,6 +62,20 @@ __device__ __forceinline__ void load_run16_full(const T* __restrict__ p, float (
     }
 }
 
+// Workgroups that share the 32 x 32 blocks of a workgroup's groups (the y extent of a block-product launch), from the
+// mean group size.  A workgroup deals the blocks of `groups_per_wg` consecutive groups to its wavefronts, which take
+// them one after the other, so windows of many blocks (7^3 positions: up to 64 blocks per group) would leave a few
+// workgroups running long after the rest.  About 2.5 blocks per workgroup and slice measured best on windows of 5^3
+// (30 tokens a group on average), 7^3 (60) and dense 5^3 windows (110).  square: the blocks tile a [c x c] result,
+// otherwise a [c x C] one.
+inline unsigned block_task_slices(double mean_c, int C, bool square, int groups_per_wg) {
+    if (!(mean_c > 0)) return 1;
+    const double nb = mean_c / 32.0 + 0.5;                              // 32-wide blocks along a side of c tokens
+    const double per_group = square ? nb * nb : nb * (double)((C + 31) / 32);
+    const int y = (int)(groups_per_wg * per_group / 2.5 + 0.5);
+    return (unsigned)(y < 1 ? 1 : (y > 8 ? 8 : y));
+}
+
 __device__ __forceinline__ int clamp16(int v) { return v < 0 ? 0 : (v > 16 ? 16 : v); }
 
 __device__ __forceinline__ int acc_row(int r, int half) { return 8 * (r >> 2) + 4 * half + (r & 3); }

@@ -646,7 +646,8 @@ def matmul_grad_cuda_naive(mat1_v, mat2_v, _c, C_, mul_type):
         out = torch.empty(total, dtype=mat1_v.dtype, device=d)
         if g > 0 and total > 0:
             _lib.check(lib.sswin_block_matmul_grad(kind, _DTYPE_CODE[mat1_v.dtype], _ptr(mat1_v), _ptr(mat2_v),
-                                                   _ptr(_c), _ptr(scans), g, C_, _ptr(out), _stream(d)))
+                                                   _ptr(_c), _ptr(scans), g, C_,
+                                                   mat1_v.numel() if kind == 0 else total, _ptr(out), _stream(d)))
     return out
 
 
@@ -674,7 +675,8 @@ def matmul_grad_untransposed(mat1_v, mat2_v, _c, C_, mul_type):
         scans, _ = _scans_for(_c, lib, d)
         if g > 0 and out.numel() > 0:
             _lib.check(lib.sswin_block_matmul_grad(kind, _DTYPE_CODE[mat1_v.dtype], _ptr(mat1_v), _ptr(mat2_v),
-                                                   _ptr(_c), _ptr(scans), g, int(C_), _ptr(out), _stream(d)))
+                                                   _ptr(_c), _ptr(scans), g, int(C_), out.numel(), _ptr(out),
+                                                   _stream(d)))
     return out
 
 

@@ -158,7 +158,7 @@ def _sq_to_tokens(tp, dtype, a_kmajor, sq, b, b_stride, b_col0, o, o_stride, o_c
     lib = _lib.load()
     stream = _lib.stream_handle(tp.device)
     _lib.check(lib.sswin_fused_sq_to_tokens(
-        _DTYPE_CODE[dtype], 1 if a_kmajor else 0, _ptr(tp.plan), tp.g_cap, tp.G, _ptr(tp.tokens), tp.N, hd,
+        _DTYPE_CODE[dtype], 1 if a_kmajor else 0, _ptr(tp.plan), tp.g_cap, tp.G, _ptr(tp.tokens), tp.N, tp.H, hd,
         _ptr(sq), _ptr(b), b_stride, b_col0, _ptr(o), o_stride, o_col0, C.c_float(scale), stream))
 
 

@@ -40,11 +40,14 @@ MIXES = {
     "edges": [31, 32, 33, 0, 63, 64, 65, 1],
     "full": [125, 124, 100, 7],
     "mixed": [1, 40, 2, 125, 0, 0, 17, 32, 90, 3, 3, 3, 3, 64],
+    "wide": [227, 130, 60, 200, 33],      # windows of 7^3 positions: up to 64 blocks of 32 x 32 per group
 }
+POSITIONS = {"wide": 343}
 
 
-def build(oracle, mix, H, hd, seed, n=125):
+def build(oracle, mix, H, hd, seed, n=None):
     rng = np.random.default_rng(seed)
+    n = POSITIONS.get(mix, 125) if n is None else n
     counts = MIXES[mix]
     ind = ragged_window_indices(rng, counts, n)
     B = len(counts)
@@ -66,7 +69,7 @@ def run_forward(ops, oracle, d, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("mix,H,hd", [("tiny", 2, 32), ("edges", 3, 32), ("full", 1, 32), ("mixed", 3, 32),
-                                      ("mixed", 2, 16), ("edges", 1, 64)])
+                                      ("mixed", 2, 16), ("edges", 1, 64), ("wide", 2, 16), ("wide", 1, 48)])
 def test_q_k_and_qk_v(ops, oracle, mix, H, hd, dtype):
     B, n, d = build(oracle, mix, H, hd, seed=seed_of(mix, H, hd))
     f = run_forward(ops, oracle, d, dtype)
@@ -92,7 +95,7 @@ def test_q_k_and_qk_v(ops, oracle, mix, H, hd, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16])
 @pytest.mark.parametrize("mix,H,hd", [("tiny", 2, 32), ("edges", 2, 32), ("mixed", 3, 32), ("full", 1, 32),
-                                      ("mixed", 1, 16), ("edges", 1, 64)])
+                                      ("mixed", 1, 16), ("edges", 1, 64), ("wide", 2, 16), ("wide", 1, 48)])
 @pytest.mark.parametrize("kind", ["rc_cr", "rr_rc", "cr_rr"])
 def test_matmul_grad(ops, oracle, mix, H, hd, kind, dtype):
     rng = np.random.default_rng(seed_of(mix, H, hd, kind))
@@ -123,7 +126,7 @@ def test_qkv_transpose(ops, oracle, mix, hd, kind, dtype):
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64, torch.bfloat16])
 @pytest.mark.parametrize("mix,H,hd", [("tiny", 2, 32), ("edges", 2, 32), ("mixed", 3, 32), ("full", 1, 32),
-                                      ("mixed", 1, 16), ("edges", 1, 64)])
+                                      ("mixed", 1, 16), ("edges", 1, 64), ("wide", 2, 16), ("wide", 1, 48)])
 @pytest.mark.parametrize("kind", ["tr_rc", "tc_rr"])
 def test_matmul_grad_from_untransposed_operands(ops, oracle, mix, H, hd, kind, dtype):
     """The second gradient of each product read from the operands as the forward pass left them: equal, bit for bit,
