@@ -615,7 +615,7 @@ def module_times(wl, reps=10):
 
     out = {}
     hd = wl["dim"] // wl["heads"]
-    for name, fused_, resident in (("resident", True, True), ("fused", "always", False), ("operators", False, None)):
+    for name, fused_, resident in (("resident", True, True), ("fused", True, False), ("operators", False, None)):
         if name == "resident" and (hd != 32 or b["stats"]["c_max"] > 128):
             continue                                          # the resident kernels do not take this shape
         attn.fused, attn.resident = fused_, resident
@@ -996,11 +996,8 @@ def main():
                 f"= {alg / ms_ / 1e6:.1f} GB/s = {100 * alg / ms_ / 1e6 / HBM_PEAK_GBPS:.2f}% of HBM peak")
         # the step runs the window-resident path: its slowest kernel is the dominant one
         # (the token plan is a sequence of small launches, not a kernel)
-        # the path the step runs (the module's own choice): resident where its kernels apply, else fused for windows of
-        # at most 128 positions, else the operator path
-        from sparseswin3d_amd import fused as fused_mod
-        run_path = "resident" if any(r["kernel"] == "resident forward" for r in table) else \
-            "fused" if fused_mod.pays(wl["blocks"][0]["n"]) else "operators"
+        # the path the step runs (the module's own choice): resident where its kernels apply, else fused
+        run_path = "resident" if any(r["kernel"] == "resident forward" for r in table) else "fused"
         dom = max((r for r in table if r["path"] == run_path and "token plan" not in r["kernel"] and "token_plan" not in r["kernel"]),
                   key=lambda r: r.get("ms_in_module", r["ms"]) * r["calls"])
         # its duration inside the step (events above) is what the roofline entry uses; the same

@@ -174,9 +174,10 @@ int sswin_permute_heads_order(const int32_t* idx, int64_t M, int C, const int32_
 /* Row ids of the sparse softmax for a [B, H, n, n] product in sorted order: rows_out[sq_start[g] + i*c + j] =
  * row_start[g] + i.  Equal to unique_consecutive_indices(flatten_indices(idx[:3])) of that product
  * (sparse_swin/swin3d_base.py:140-150), without reading its index matrix.  c: device int32 [G] (windows of fewer than
- * 4096 tokens), scans: device int32 [2*G] as sswin_scan_counts writes them, rows_out: device int32 [sum c*c].
- * Asynchronous. */
-int sswin_softmax_rows_from_counts(const int32_t* c, const int32_t* scans, int64_t G, int32_t* rows_out, void* stream);
+ * 4096 tokens), scans: device int32 [2*G] as sswin_scan_counts writes them, rows_out: device int32 [A], A = sum c*c
+ * (a host number; the launch is sized from the mean group A / G).  Asynchronous. */
+int sswin_softmax_rows_from_counts(const int32_t* c, const int32_t* scans, int64_t G, int64_t A, int32_t* rows_out,
+                                   void* stream);
 
 /* values + bias[head, pos_i, pos_j], and -100 more where the mask regions of the two positions differ, for a
  * [B, H, n, n] 'q_k' product in sorted order (sp_add_rpb and sp_add_mask, sparse_swin/swin3d_base.py:557-581), from the

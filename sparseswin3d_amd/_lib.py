@@ -43,7 +43,7 @@ SIGNATURES = {
     "sswin_plan_workspace_bytes": (_sz, [_i64, _i32]),
     "sswin_plan_from_indices": (_i32, [_vp, _i64, _i32, _vp, _i64, _vp, _vp, _sz, _vp]),
     "sswin_permute_heads_order": (_i32, [_vp, _i64, _i32, _vp, _i64, _i64, _vp, _vp, _vp]),
-    "sswin_softmax_rows_from_counts": (_i32, [_vp, _vp, _i64, _vp, _vp]),
+    "sswin_softmax_rows_from_counts": (_i32, [_vp, _vp, _i64, _i64, _vp, _vp]),
     "sswin_group_add_bias_mask": (_i32, [_i32, _vp, _vp, _i64, _vp, _i64, _i64, _i32, _i32, _vp, _vp, _i32, _vp, _vp]),
     "sswin_group_add_table_bias_mask": (_i32, [_i32, _vp, _vp, _i64, _vp, _i64, _i64, _i32, _i32, _vp, _i32, _i32, _vp, _i32, _vp,
                                                _i32, _vp, _vp]),

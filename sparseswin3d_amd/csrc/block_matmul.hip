@@ -78,7 +78,6 @@ struct GroupTable {
 #ifndef BP_BUFFERED
 #define BP_BUFFERED 1
 #endif
-typedef uint32_t u32x4_b __attribute__((ext_vector_type(4)));
 #ifndef BP_WAVES_FWD
 #define BP_WAVES_FWD 4
 #endif
@@ -155,69 +154,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MODE >= 2 ?
         const T* B = m2 + d.b_off;
         f32x16 acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
         if constexpr (BUFFERED) {
-            // Every block is addressed through a buffer descriptor of exactly its size (base and size are scalars):
-            // a lane whose row, column or reduction index lies outside the block forms an offset beyond it, loads
-            // zero and has its store dropped by the bounds check of the memory pipeline, so ragged blocks need no
-            // clamp, select or branch, and an access costs one vector add for its offset.
-            constexpr uint32_t OUTSIDE = 0x80000000u;
+            // every block through a buffer descriptor of exactly its size (buf_of and the loads of mfma_block.hpp)
+            constexpr uint32_t OUTSIDE = BUF_OUTSIDE;
             constexpr uint32_t ES = (uint32_t)sizeof(T);               // 4 (float) or 2 (half, bfloat16)
-            const __amdgpu_buffer_rsrc_t ra = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(A), 0, d.I * d.K * (int)ES, 0x00020000);
-            const __amdgpu_buffer_rsrc_t rb = __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(B), 0, d.K * d.J * (int)ES, 0x00020000);
-            const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(out + d.o_off, 0, d.I * d.J * (int)ES, 0x00020000);
-            auto load1 = [](const __amdgpu_buffer_rsrc_t& r, uint32_t off) __attribute__((always_inline)) -> float {
-                if constexpr (ES == 4) {
-                    const uint32_t u = __builtin_amdgcn_raw_buffer_load_b32(r, off, 0, 0);
-                    return __builtin_bit_cast(float, u);
-                } else {
-                    const uint16_t u = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(r, off, 0, 0);
-                    return to_acc(__builtin_bit_cast(T, u));
-                }
-            };
-            // 16 consecutive values from byte offset off (all inside or all outside the block)
-            auto load16 = [](const __amdgpu_buffer_rsrc_t& r, uint32_t off, float (&x)[16]) __attribute__((always_inline)) {
-                if constexpr (ES == 4) {
-#pragma unroll
-                    for (int v = 0; v < 4; ++v) {
-                        const u32x4_b t = __builtin_amdgcn_raw_buffer_load_b128(r, off + 16u * v, 0, 0);
-                        const uint32_t w[4] = {t.x, t.y, t.z, t.w};
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) x[4 * v + e] = __builtin_bit_cast(float, w[e]);
-                    }
-                } else {
-#pragma unroll
-                    for (int v = 0; v < 2; ++v) {
-                        const u32x4_b t = __builtin_amdgcn_raw_buffer_load_b128(r, off + 16u * v, 0, 0);
-                        const uint32_t w[4] = {t.x, t.y, t.z, t.w};
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) {
-                            const uint16_t lo = (uint16_t)(w[e] & 0xffffu), hi = (uint16_t)(w[e] >> 16);
-                            x[8 * v + 2 * e] = to_acc(__builtin_bit_cast(T, lo));
-                            x[8 * v + 2 * e + 1] = to_acc(__builtin_bit_cast(T, hi));
-                        }
-                    }
-                }
-            };
-            // 8 consecutive values (a reduction over 16 channels: each lane half feeds eight of them)
-            auto load8 = [](const __amdgpu_buffer_rsrc_t& r, uint32_t off, float (&x)[16]) __attribute__((always_inline)) {
-                if constexpr (ES == 4) {
-#pragma unroll
-                    for (int v = 0; v < 2; ++v) {
-                        const u32x4_b t = __builtin_amdgcn_raw_buffer_load_b128(r, off + 16u * v, 0, 0);
-                        const uint32_t w[4] = {t.x, t.y, t.z, t.w};
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) x[4 * v + e] = __builtin_bit_cast(float, w[e]);
-                    }
-                } else {
-                    const u32x4_b t = __builtin_amdgcn_raw_buffer_load_b128(r, off, 0, 0);
-                    const uint32_t w[4] = {t.x, t.y, t.z, t.w};
-#pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        const uint16_t lo = (uint16_t)(w[e] & 0xffffu), hi = (uint16_t)(w[e] >> 16);
-                        x[2 * e] = to_acc(__builtin_bit_cast(T, lo));
-                        x[2 * e + 1] = to_acc(__builtin_bit_cast(T, hi));
-                    }
-                }
-            };
+            const __amdgpu_buffer_rsrc_t ra = buf_of(A, (uint32_t)(d.I * d.K) * ES);
+            const __amdgpu_buffer_rsrc_t rb = buf_of(B, (uint32_t)(d.K * d.J) * ES);
+            const __amdgpu_buffer_rsrc_t ro = buf_of(out + d.o_off, (uint32_t)(d.I * d.J) * ES);
             for (int kc = 0; kc < d.K; kc += 32) {
                 const int chunk = d.K - kc < 32 ? d.K - kc : 32;
                 const int kh = (chunk + 1) >> 1;
@@ -227,41 +169,41 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MODE >= 2 ?
                     // element (kc + half * kh + s, i): rows of k behind the block's last one are outside by themselves
                     const uint32_t v0 = i_a < d.I ? (uint32_t)(half * kh * d.I + i_a) * ES : OUTSIDE;
 #pragma unroll
-                    for (int s = 0; s < 8; ++s) a[s] = load1(ra, v0 + (uint32_t)((kc + s) * d.I) * ES);
+                    for (int s = 0; s < 8; ++s) a[s] = buf_load1<T>(ra, v0 + (uint32_t)((kc + s) * d.I) * ES);
                     if (kh > 8) {
 #pragma unroll
-                        for (int s = 8; s < 16; ++s) a[s] = load1(ra, v0 + (uint32_t)((kc + s) * d.I) * ES);
+                        for (int s = 8; s < 16; ++s) a[s] = buf_load1<T>(ra, v0 + (uint32_t)((kc + s) * d.I) * ES);
                     }
                 } else {
                     // a row per lane: 16 consecutive values of row i; values of k behind the row's end belong to the
                     // next row and are masked through their offsets
                     const uint32_t v0 = i_a < d.I ? (uint32_t)(i_a * d.K + kc + half * kh) * ES : OUTSIDE;
                     if (chunk == 32 && (ES == 4 || d.K % 8 == 0)) {      // 16-byte loads need rows that start at a multiple of 4 bytes
-                        load16(ra, v0, a);
+                        buf_load_run<T, 16>(ra, v0, a);
                     } else if (chunk == 16 && (ES == 4 || d.K % 8 == 0)) {
-                        load8(ra, v0, a);
+                        buf_load_run<T, 8>(ra, v0, a);
                     } else {
 #pragma unroll
-                        for (int s = 0; s < 16; ++s) a[s] = load1(ra, s < left ? v0 + ES * s : OUTSIDE);
+                        for (int s = 0; s < 16; ++s) a[s] = buf_load1<T>(ra, s < left ? v0 + ES * s : OUTSIDE);
                     }
                 }
                 if (b_is_kmajor<MODE>()) {
                     const uint32_t v0 = j_b < d.J ? (uint32_t)(half * kh * d.J + j_b) * ES : OUTSIDE;
 #pragma unroll
-                    for (int s = 0; s < 8; ++s) b[s] = load1(rb, v0 + (uint32_t)((kc + s) * d.J) * ES);
+                    for (int s = 0; s < 8; ++s) b[s] = buf_load1<T>(rb, v0 + (uint32_t)((kc + s) * d.J) * ES);
                     if (kh > 8) {
 #pragma unroll
-                        for (int s = 8; s < 16; ++s) b[s] = load1(rb, v0 + (uint32_t)((kc + s) * d.J) * ES);
+                        for (int s = 8; s < 16; ++s) b[s] = buf_load1<T>(rb, v0 + (uint32_t)((kc + s) * d.J) * ES);
                     }
                 } else {
                     const uint32_t v0 = j_b < d.J ? (uint32_t)(j_b * d.K + kc + half * kh) * ES : OUTSIDE;
                     if (chunk == 32 && (ES == 4 || d.K % 8 == 0)) {
-                        load16(rb, v0, b);
+                        buf_load_run<T, 16>(rb, v0, b);
                     } else if (chunk == 16 && (ES == 4 || d.K % 8 == 0)) {
-                        load8(rb, v0, b);
+                        buf_load_run<T, 8>(rb, v0, b);
                     } else {
 #pragma unroll
-                        for (int s = 0; s < 16; ++s) b[s] = load1(rb, s < left ? v0 + ES * s : OUTSIDE);
+                        for (int s = 0; s < 16; ++s) b[s] = buf_load1<T>(rb, s < left ? v0 + ES * s : OUTSIDE);
                     }
                 }
 #pragma unroll
@@ -271,14 +213,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MODE >= 2 ?
             const uint32_t o0 = j_b < d.J ? (uint32_t)((bi * 32 + 4 * half) * d.J + j_b) * ES : OUTSIDE;
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
-                const float v = acc[r];                      // (a bit_cast of the vector element itself reads element 0)
-                const uint32_t off = o0 + (uint32_t)((8 * (r >> 2) + (r & 3)) * d.J) * ES;
-                if constexpr (ES == 4) {
-                    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), ro, off, 0, 0);
-                } else {
-                    const T t = from_acc<T>(v);
-                    __builtin_amdgcn_raw_buffer_store_b16((short)__builtin_bit_cast(uint16_t, t), ro, off, 0, 0);
-                }
+                const float v = acc[r];                      // a scalar copy: a bit_cast of the vector element itself reads element 0
+                buf_store1<T>(ro, o0 + (uint32_t)((8 * (r >> 2) + (r & 3)) * d.J) * ES, v);
             }
             continue;
         }

@@ -17,6 +17,7 @@
 // by-product of the first kernel.
 #include <type_traits>
 #include <algorithm>
+#include <cstdlib>
 #include <cstring>
 
 #include "mfma_block.hpp"
@@ -387,46 +388,283 @@ struct TokenTensor {         // rows addressed by voxel, columns col0 + h*hd + c
 };
 
 // work distribution: four consecutive groups per workgroup, their 32-row x 32-column blocks dealt
-// round robin to the four wavefronts
-struct TaskSet {
-    int c[FUSED_GROUPS_PER_WG], nbj[FUSED_GROUPS_PER_WG], first[FUSED_GROUPS_PER_WG + 1];
+// round robin to the four wavefronts of the gridDim.y workgroups that share them.  Lane q < 4 of every wavefront
+// holds the fields of group g0 + q (one load per field for all four groups, and nothing waits for a second round);
+// a task reads its group's fields from that lane into scalar registers.
+struct GroupLanes {
+    int c, T, sq, h, w;
 };
+template <bool WINDOW>
+__device__ __forceinline__ GroupLanes load_groups(const FusedGroups& gt, int64_t g0, int lane) {
+    const int64_t g = g0 + (lane & (FUSED_GROUPS_PER_WG - 1));
+    const bool in = g < gt.G;
+    GroupLanes f;
+    f.c = in ? gt.c[g] : 0;
+    f.T = in ? gt.T[g] : 0;
+    f.sq = in ? gt.sq[g] : 0;
+    f.h = in ? gt.head[g] : 0;
+    f.w = WINDOW && in ? gt.window[g] : 0;
+    return f;
+}
 
-__device__ __forceinline__ TaskSet make_tasks(const FusedGroups& gt, int64_t g0, bool square, int hd) {
+// blocks of a group of c tokens: [c x c] results (square) or [c x hd]
+__device__ __forceinline__ int blocks_across(int c, bool square, int hd) { return square ? (c + 31) >> 5 : (hd + 31) >> 5; }
+
+struct TaskSet {
+    int first[FUSED_GROUPS_PER_WG + 1];     // first[q]: blocks of the groups in front of group q (scalars)
+};
+__device__ __forceinline__ TaskSet make_tasks(const GroupLanes& f, bool square, int hd) {
     TaskSet t;
     t.first[0] = 0;
 #pragma unroll
     for (int q = 0; q < FUSED_GROUPS_PER_WG; ++q) {
-        const int64_t g = g0 + q;
-        const int c = g < gt.G ? gt.c[g] : 0;
-        t.c[q] = c;
-        t.nbj[q] = square ? (c + 31) >> 5 : (hd + 31) >> 5;
-        t.first[q + 1] = t.first[q] + (c > 0 ? ((c + 31) >> 5) * t.nbj[q] : 0);
+        const int c = __builtin_amdgcn_readlane(f.c, q);
+        t.first[q + 1] = t.first[q] + ((c + 31) >> 5) * blocks_across(c, square, hd);
     }
     return t;
 }
 
-__device__ __forceinline__ void locate_task(const TaskSet& ts, int t, int& q, int& c, int& bi, int& bj) {
-    q = 0;
+// a task belongs to the whole wavefront: its parameters are scalars
+struct Task {
+    int c, bi, bj, T, sq, h, w;
+};
+__device__ __forceinline__ Task locate_task(const TaskSet& ts, const GroupLanes& f, int t, bool square, int hd) {
+    int q = 0, f0 = 0;
 #pragma unroll
-    for (int qq = 1; qq < FUSED_GROUPS_PER_WG; ++qq) q += (t >= ts.first[qq]) ? 1 : 0;
-    c = ts.c[0];
-    int nj = ts.nbj[0], f0 = ts.first[0];
-#pragma unroll
-    for (int qq = 1; qq < FUSED_GROUPS_PER_WG; ++qq)
-        if (q == qq) { c = ts.c[qq]; nj = ts.nbj[qq]; f0 = ts.first[qq]; }
-    const int local = t - f0;
-    bi = local / nj;
-    bj = local - bi * nj;
+    for (int qq = 1; qq < FUSED_GROUPS_PER_WG; ++qq) {
+        const bool behind = t >= ts.first[qq];
+        q += behind ? 1 : 0;
+        f0 = behind ? ts.first[qq] : f0;
+    }
+    Task k;
+    k.c = __builtin_amdgcn_readlane(f.c, q);
+    k.T = __builtin_amdgcn_readlane(f.T, q);
+    k.sq = __builtin_amdgcn_readlane(f.sq, q);
+    k.h = __builtin_amdgcn_readlane(f.h, q);
+    k.w = __builtin_amdgcn_readlane(f.w, q);
+    const int nj = blocks_across(k.c, square, hd), local = t - f0;
+    k.bi = local / nj;
+    k.bj = local - k.bi * nj;
+    return k;
+}
+
+// Token rows through a buffer descriptor over the whole tensor, shifted to the head's first channel: element
+// (voxel v, channel ch of head h) is at byte offset v * stride * sizeof(T) + ch * sizeof(T).  `span` = bytes of the
+// whole [N, stride] tensor (at most 2^31: the launcher checks).
+template <typename T>
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t head_rows(const TokenTensor& t, int h, int hd, uint32_t span) {
+    const uint32_t shift = (uint32_t)(t.col0 + h * hd) * (uint32_t)sizeof(T);
+    return buf_of(static_cast<const T*>(t.base) + t.col0 + h * hd, span - shift);
 }
 
 // ------------------------------------------------------------------------------------------
 // tokens x tokens -> sq :  out[i, j] = sum_ch A[token i, ch] * B[token j, ch]   (K = hd)
 //   EPI = true : S = scale*acc + bias[h, pos_i, pos_j] + (mask region differs ? -100 : 0), row ids
 //   EPI = false: plain product (dP = dO V^T)
+// Rows of tokens behind the window's last one are read as zeros and their results dropped by the bounds checks
+// of the buffer descriptors (mfma_block.hpp).
 // ------------------------------------------------------------------------------------------
 template <typename T, bool EPI>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void fused_sq_kernel(FusedGroups gt, const int32_t* __restrict__ order,
+                                                       const int32_t* __restrict__ tok_pos, int H, int hd,
+                                                       TokenTensor ta, TokenTensor tb, uint32_t a_span, uint32_t b_span, float scale_a,
+                                                       const float* __restrict__ bias, int n,
+                                                       const int8_t* __restrict__ mask, int n_mask_windows,
+                                                       float* __restrict__ out, int32_t* __restrict__ row_ids) {
+    constexpr uint32_t ES = (uint32_t)sizeof(T);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int half = lane >> 5, l32 = lane & 31;
+    const int64_t g0 = (int64_t)blockIdx.x * FUSED_GROUPS_PER_WG;
+    const GroupLanes gl = load_groups<EPI>(gt, g0, lane);
+    const TaskSet ts = make_tasks(gl, true, hd);
+    const int total = ts.first[FUSED_GROUPS_PER_WG];
+    const uint32_t a_pitch = (uint32_t)ta.stride * ES, b_pitch = (uint32_t)tb.stride * ES;
+
+    for (int t = wave + 4 * (int)blockIdx.y; t < total; t += 4 * (int)gridDim.y) {   // gridDim.y workgroups share the groups' blocks
+        const Task k = locate_task(ts, gl, t, true, hd);
+        const int c = k.c, Tk = k.T, h = k.h, bi = k.bi, bj = k.bj;
+        const int i_a = bi * 32 + l32, j_b = bj * 32 + l32;
+        const bool a_in = i_a < c, b_in = j_b < c;
+        const int32_t* ord = order + Tk;
+        const int vox_i = ord[a_in ? i_a : c - 1], vox_j = ord[b_in ? j_b : c - 1];
+        // epilogue inputs: one load per lane (row token, column token); the 16 rows a lane stores
+        // are fetched from the row lanes with cross-lane reads in the epilogue
+        int pos_a = 0, pos_j = 0, m_a = 0, m_j = 0;
+        if (EPI) {
+            pos_a = tok_pos[Tk + (a_in ? i_a : c - 1)];
+            pos_j = tok_pos[Tk + (b_in ? j_b : c - 1)];
+            if (mask) {
+                const int8_t* mrow = mask + (int64_t)(k.w % n_mask_windows) * n;
+                m_a = mrow[pos_a];
+                m_j = mrow[pos_j];
+            }
+        }
+        const __amdgpu_buffer_rsrc_t ra = head_rows<T>(ta, h, hd, a_span), rb = head_rows<T>(tb, h, hd, b_span);
+        const uint32_t row_a = a_in ? (uint32_t)vox_i * a_pitch : BUF_OUTSIDE;
+        const uint32_t row_b = b_in ? (uint32_t)vox_j * b_pitch : BUF_OUTSIDE;
+
+        f32x16 acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        for (int kc = 0; kc < hd; kc += 32) {
+            // the channels of a chunk are split evenly between the two lane halves: a head of 16 channels takes
+            // eight matrix steps, not sixteen with one half feeding zeros
+            const int chunk = hd - kc < 32 ? hd - kc : 32;
+            const int kh = (chunk + 1) >> 1;
+            const int left = half ? chunk - kh : kh;
+            const uint32_t ch0 = (uint32_t)(kc + half * kh) * ES;
+            float a[16], b[16];
+            if (chunk == 32) {
+                buf_load_run<T, 16>(ra, row_a + ch0, a);
+                buf_load_run<T, 16>(rb, row_b + ch0, b);
+            } else if (chunk == 16) {
+                buf_load_run<T, 8>(ra, row_a + ch0, a);
+                buf_load_run<T, 8>(rb, row_b + ch0, b);
+            } else {
+#pragma unroll
+                for (int s = 0; s < 16; ++s) {
+                    a[s] = buf_load1<T>(ra, s < left ? row_a + ch0 + ES * s : BUF_OUTSIDE);
+                    b[s] = buf_load1<T>(rb, s < left ? row_b + ch0 + ES * s : BUF_OUTSIDE);
+                }
+            }
+            if (scale_a != 1.0f) {
+#pragma unroll
+                for (int s = 0; s < 16; ++s) a[s] *= scale_a;
+            }
+#pragma unroll
+            for (int s = 0; s < 16; ++s)
+                if (s < kh) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], acc, 0, 0, 0);
+        }
+
+        {
+            // entry (i, j) of the block at byte offset (i * c + j) * 4: rows behind the last one are outside by themselves
+            const __amdgpu_buffer_rsrc_t ro = buf_of(out + k.sq, (uint32_t)(c * c) * 4u);
+            const __amdgpu_buffer_rsrc_t rr = buf_of(row_ids ? row_ids + k.sq : nullptr, row_ids ? (uint32_t)(c * c) * 4u : 0u);
+            const uint32_t o0 = b_in ? (uint32_t)((bi * 32 + 4 * half) * c + j_b) * 4u : BUF_OUTSIDE;
+            const float* brow = EPI ? bias + (int64_t)h * n * n + pos_j : nullptr;
+            const int rid0 = H * Tk + h * c + bi * 32 + 4 * half;
+            // bias values of the 16 rows are gathered before any of them is used, so that the
+            // gather latencies overlap instead of adding up
+            float bv[16];
+            int m_i[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                bv[r] = 0.f;
+                m_i[r] = 0;
+                if (EPI) {                                          // all lanes take part in the shuffles
+                    const int il = acc_row(r, half);
+                    bv[r] = brow[__shfl(pos_a, il, 64) * n];
+                    if (mask) m_i[r] = __shfl(m_a, il, 64);
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int row = 8 * (r >> 2) + (r & 3);             // + 4 * half: the row of the block
+                float v = acc[r];
+                if (EPI) {
+                    v += bv[r];
+                    if (mask && m_i[r] != m_j) v += -100.0f;
+                    if (row_ids) __builtin_amdgcn_raw_buffer_store_b32((uint32_t)(rid0 + row), rr, o0 + (uint32_t)(row * c) * 4u, 0, 0);
+                }
+                buf_store1<float>(ro, o0 + (uint32_t)(row * c) * 4u, v);
+            }
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// sq x tokens -> tokens :  out[token i, ch] = scale * sum_k A(i, k) * B[token k, ch]   (K = c)
+//   A_KMAJOR = false: A(i, k) = sq[i*c + k]   (O = P V, dQ = dS K)
+//   A_KMAJOR = true : A(i, k) = sq[k*c + i]   (dV = P^T dO, dK = dS^T Q)
+// ------------------------------------------------------------------------------------------
+template <typename T, bool A_KMAJOR>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void fused_tok_kernel(FusedGroups gt, const int32_t* __restrict__ order, int hd,
+                                                        const float* __restrict__ sq, TokenTensor tb,
+                                                        TokenTensor to, uint32_t b_span, uint32_t o_span, float scale_out) {
+    constexpr uint32_t ES = (uint32_t)sizeof(T);
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int half = lane >> 5, l32 = lane & 31;
+    const int64_t g0 = (int64_t)blockIdx.x * FUSED_GROUPS_PER_WG;
+    const GroupLanes gl = load_groups<false>(gt, g0, lane);
+    const TaskSet ts = make_tasks(gl, false, hd);
+    const int total = ts.first[FUSED_GROUPS_PER_WG];
+    const uint32_t b_pitch = (uint32_t)tb.stride * ES, o_pitch = (uint32_t)to.stride * ES;
+
+    for (int t = wave + 4 * (int)blockIdx.y; t < total; t += 4 * (int)gridDim.y) {   // gridDim.y workgroups share the groups' blocks
+        const Task k = locate_task(ts, gl, t, false, hd);
+        const int c = k.c, Tk = k.T, h = k.h, bi = k.bi, bj = k.bj;
+        const int i_a = bi * 32 + l32, j_b = bj * 32 + l32;
+        const bool a_in = i_a < c, b_in = j_b < hd;
+        const int32_t* ord = order + Tk;
+        // voxel of this lane's row token (the 16 rows a lane stores are fetched with cross-lane reads) and the
+        // voxels of the first 32 reduction tokens
+        const int vox_a = ord[a_in ? i_a : c - 1];
+        int ord_l = ord[l32 < c ? l32 : c - 1];
+        const __amdgpu_buffer_rsrc_t rs = buf_of(sq + k.sq, (uint32_t)(c * c) * 4u);
+        const __amdgpu_buffer_rsrc_t rb = head_rows<T>(tb, h, hd, b_span), ro = head_rows<T>(to, h, hd, o_span);
+        const uint32_t col = (uint32_t)j_b * ES;
+
+        f32x16 acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+        for (int kc = 0; kc < c; kc += 32) {
+            const int chunk = c - kc < 32 ? c - kc : 32;
+            const int kh = (chunk + 1) >> 1;                        // reduction tokens per lane half (uniform)
+            const int left = half ? chunk - kh : kh;
+            // voxels of the next chunk's tokens: requested now, so that its rows do not wait for them
+            const int ord_cur = ord_l;
+            if (kc + 32 < c) ord_l = ord[kc + 32 + l32 < c ? kc + 32 + l32 : c - 1];
+            float a[16], b[16];
+            // B: row of token kc + half * kh + s, this lane's channel
+            auto b_load = [&](const int s) __attribute__((always_inline)) {
+                const int vox = __shfl(ord_cur, half * kh + s, 64);
+                b[s] = buf_load1<T>(rb, (b_in && s < left) ? (uint32_t)vox * b_pitch + col : BUF_OUTSIDE);
+            };
+#pragma unroll
+            for (int s = 0; s < 8; ++s) b_load(s);
+            if (kh > 8) {
+#pragma unroll
+                for (int s = 8; s < 16; ++s) b_load(s);
+            }
+            if (!A_KMAJOR) {
+                // a row per lane: values of k behind the row's end belong to the next row and are masked through their offsets
+                const uint32_t v0 = a_in ? (uint32_t)(i_a * c + kc + half * kh) * 4u : BUF_OUTSIDE;
+                if (chunk == 32) {
+                    buf_load_run<float, 16>(rs, v0, a);
+                } else {
+#pragma unroll
+                    for (int s = 0; s < 16; ++s) a[s] = buf_load1<float>(rs, s < left ? v0 + 4u * s : BUF_OUTSIDE);
+                }
+            } else {
+                // element (kc + half * kh + s, i): rows of k behind the block's last one are outside by themselves
+                const uint32_t v0 = a_in ? (uint32_t)(half * kh * c + i_a) * 4u : BUF_OUTSIDE;
+#pragma unroll
+                for (int s = 0; s < 8; ++s) a[s] = buf_load1<float>(rs, v0 + (uint32_t)((kc + s) * c) * 4u);
+                if (kh > 8) {
+#pragma unroll
+                    for (int s = 8; s < 16; ++s) a[s] = buf_load1<float>(rs, v0 + (uint32_t)((kc + s) * c) * 4u);
+                }
+            }
+#pragma unroll
+            for (int s = 0; s < 16; ++s)
+                if (s < kh) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], acc, 0, 0, 0);
+        }
+
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int il = acc_row(r, half);
+            const int vox = __shfl(vox_a, il, 64);
+            const float v = acc[r] * scale_out;
+            buf_store1<T>(ro, (b_in && bi * 32 + il < c) ? (uint32_t)vox * o_pitch + col : BUF_OUTSIDE, v);
+        }
+    }
+}
+
+// ------------------------------------------------------------------------------------------
+// The same two products with 64-bit addresses, for token tensors that a buffer descriptor cannot cover (more than
+// 2^31 bytes, or 16-bit rows that do not start at a multiple of four bytes).
+// tokens x tokens -> sq :  out[i, j] = sum_ch A[token i, ch] * B[token j, ch]   (K = hd)
+//   EPI = true : S = scale*acc + bias[h, pos_i, pos_j] + (mask region differs ? -100 : 0), row ids
+//   EPI = false: plain product (dP = dO V^T)
+// ------------------------------------------------------------------------------------------
+template <typename T, bool EPI>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void fused_sq_wide_kernel(FusedGroups gt, const int32_t* __restrict__ order,
                                                        const int32_t* __restrict__ tok_pos, int H, int hd,
                                                        TokenTensor ta, TokenTensor tb, float scale_a,
                                                        const float* __restrict__ bias, int n,
@@ -435,17 +673,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int half = lane >> 5, l32 = lane & 31;
     const int64_t g0 = (int64_t)blockIdx.x * FUSED_GROUPS_PER_WG;
-    const TaskSet ts = make_tasks(gt, g0, true, hd);
+    const GroupLanes gl = load_groups<EPI>(gt, g0, lane);
+    const TaskSet ts = make_tasks(gl, true, hd);
     const int total = ts.first[FUSED_GROUPS_PER_WG];
     const T* A = static_cast<const T*>(ta.base);
     const T* B = static_cast<const T*>(tb.base);
 
     for (int t = wave + 4 * (int)blockIdx.y; t < total; t += 4 * (int)gridDim.y) {   // gridDim.y workgroups share the groups' blocks
-        int q, c, bi, bj;
-        locate_task(ts, t, q, c, bi, bj);
-        const int64_t g = g0 + q;
-        const int Tk = gt.T[g], h = gt.head[g];
-        const int64_t sq0 = gt.sq[g];
+        const Task k = locate_task(ts, gl, t, true, hd);
+        const int c = k.c, bi = k.bi, bj = k.bj, Tk = k.T, h = k.h;
+        const int64_t sq0 = k.sq;
         const int i_a = bi * 32 + l32, j_b = bj * 32 + l32;
         const bool a_in = i_a < c, b_in = j_b < c;
         // rows past the end of the window are clamped to its last token: their products are finite
@@ -461,7 +698,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             pos_a = tok_pos[Tk + i_c];
             pos_j = tok_pos[Tk + j_c];
             if (mask) {
-                const int8_t* mrow = mask + (int64_t)(gt.window[g] % n_mask_windows) * n;
+                const int8_t* mrow = mask + (int64_t)(k.w % n_mask_windows) * n;
                 m_a = mrow[pos_a];
                 m_j = mrow[pos_j];
             }
@@ -539,29 +776,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 //   A_KMAJOR = true : A(i, k) = sq[k*c + i]   (dV = P^T dO, dK = dS^T Q)
 // ------------------------------------------------------------------------------------------
 template <typename T, bool A_KMAJOR>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void fused_tok_kernel(FusedGroups gt, const int32_t* __restrict__ order, int hd,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void fused_tok_wide_kernel(FusedGroups gt, const int32_t* __restrict__ order, int hd,
                                                         const float* __restrict__ sq, TokenTensor tb,
                                                         TokenTensor to, float scale_out) {
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int half = lane >> 5, l32 = lane & 31;
     const int64_t g0 = (int64_t)blockIdx.x * FUSED_GROUPS_PER_WG;
-    const TaskSet ts = make_tasks(gt, g0, false, hd);
+    const GroupLanes gl = load_groups<false>(gt, g0, lane);
+    const TaskSet ts = make_tasks(gl, false, hd);
     const int total = ts.first[FUSED_GROUPS_PER_WG];
     const T* B = static_cast<const T*>(tb.base);
     T* O = static_cast<T*>(const_cast<void*>(to.base));
 
     for (int t = wave + 4 * (int)blockIdx.y; t < total; t += 4 * (int)gridDim.y) {   // gridDim.y workgroups share the groups' blocks
-        int q, c, bi, bj;
-        locate_task(ts, t, q, c, bi, bj);
-        // a task belongs to the whole wavefront: its parameters go to scalar registers, and the block of the
-        // attention matrix is addressed by a scalar base plus 32-bit lane offsets (c <= 32767, so c * c * 4 fits)
-        q = __builtin_amdgcn_readfirstlane(q);
-        c = __builtin_amdgcn_readfirstlane(c);
-        bi = __builtin_amdgcn_readfirstlane(bi);
-        bj = __builtin_amdgcn_readfirstlane(bj);
-        const int64_t g = g0 + q;
-        const int Tk = __builtin_amdgcn_readfirstlane(gt.T[g]), h = __builtin_amdgcn_readfirstlane(gt.head[g]);
-        const float* S = sq + __builtin_amdgcn_readfirstlane(gt.sq[g]);
+        // the block of the attention matrix is addressed by a scalar base plus 32-bit lane offsets (c <= 32767, so
+        // c * c * 4 fits)
+        const Task k = locate_task(ts, gl, t, false, hd);
+        const int c = k.c, bi = k.bi, bj = k.bj, Tk = k.T, h = k.h;
+        const float* S = sq + k.sq;
         const int i_a = bi * 32 + l32, j_b = bj * 32 + l32;
         const bool a_in = i_a < c, b_in = j_b < hd;
         const int i_c = a_in ? i_a : c - 1, j_c = b_in ? j_b : hd - 1;     // clamped: loads need no predicate
@@ -955,32 +1187,65 @@ __global__ __launch_bounds__(1024) void rpb_table_reduce_kernel(const float* __r
     }
 }
 
+// Whether the rows of a token tensor can go through a buffer descriptor: the tensor spans at most 2^31 bytes and, for
+// 16-bit values, every head's row slice starts at a multiple of four bytes (what the 16-byte loads need).
+// SSWIN_FUSED_WIDE=1 in the environment sends everything to the kernels with 64-bit addresses.
 template <typename T>
-static int launch_sq(bool epi, const FusedGroups& gt, double mean_c, const int32_t* order, const int32_t* tok_pos, int H, int hd,
+static bool rows_fit_descriptor(const TokenTensor& t, int64_t N, int hd, uint32_t* span) {
+    const int64_t bytes = N * t.stride * (int64_t)sizeof(T);
+    *span = (uint32_t)bytes;
+    if (bytes > ((int64_t)1 << 31) || t.stride <= 0) return false;
+    if (sizeof(T) == 2 && (((uintptr_t)t.base & 3) || (t.stride & 1) || (t.col0 & 1) || (hd & 1))) return false;
+    const char* e = getenv("SSWIN_FUSED_WIDE");
+    return !(e && e[0] == '1');
+}
+
+template <typename T>
+static int launch_sq(bool epi, const FusedGroups& gt, int64_t N, double mean_c, const int32_t* order, const int32_t* tok_pos, int H, int hd,
                      const TokenTensor& ta, const TokenTensor& tb, float scale_a, const float* bias, int n,
                      const int8_t* mask, int nmw, float* out, int32_t* row_ids, hipStream_t s) {
     const dim3 grid((unsigned)((gt.G + FUSED_GROUPS_PER_WG - 1) / FUSED_GROUPS_PER_WG),
                     block_task_slices(mean_c, hd, true, FUSED_GROUPS_PER_WG));
-    if (epi)
-        hipLaunchKernelGGL((fused_sq_kernel<T, true>), grid, dim3(256), 0, s, gt, order, tok_pos, H, hd, ta,
+    uint32_t a_span, b_span;
+    const bool fit_a = rows_fit_descriptor<T>(ta, N, hd, &a_span), fit_b = rows_fit_descriptor<T>(tb, N, hd, &b_span);
+    if (fit_a && fit_b) {
+        if (epi)
+            hipLaunchKernelGGL((fused_sq_kernel<T, true>), grid, dim3(256), 0, s, gt, order, tok_pos, H, hd, ta,
+                               tb, a_span, b_span, scale_a, bias, n, mask, nmw, out, row_ids);
+        else
+            hipLaunchKernelGGL((fused_sq_kernel<T, false>), grid, dim3(256), 0, s, gt, order, tok_pos, H, hd, ta,
+                               tb, a_span, b_span, scale_a, bias, n, mask, nmw, out, row_ids);
+    } else if (epi) {
+        hipLaunchKernelGGL((fused_sq_wide_kernel<T, true>), grid, dim3(256), 0, s, gt, order, tok_pos, H, hd, ta,
                            tb, scale_a, bias, n, mask, nmw, out, row_ids);
-    else
-        hipLaunchKernelGGL((fused_sq_kernel<T, false>), grid, dim3(256), 0, s, gt, order, tok_pos, H, hd, ta,
+    } else {
+        hipLaunchKernelGGL((fused_sq_wide_kernel<T, false>), grid, dim3(256), 0, s, gt, order, tok_pos, H, hd, ta,
                            tb, scale_a, bias, n, mask, nmw, out, row_ids);
+    }
     return launch_ok("fused tokens->sq product");
 }
 
 template <typename T>
-static int launch_tok(bool a_kmajor, const FusedGroups& gt, double mean_c, const int32_t* order, int hd, const float* sq,
+static int launch_tok(bool a_kmajor, const FusedGroups& gt, int64_t N, double mean_c, const int32_t* order, int hd, const float* sq,
                       const TokenTensor& tb, const TokenTensor& to, float scale_out, hipStream_t s) {
     const dim3 grid((unsigned)((gt.G + FUSED_GROUPS_PER_WG - 1) / FUSED_GROUPS_PER_WG),
                     block_task_slices(mean_c, hd, false, FUSED_GROUPS_PER_WG));
-    if (a_kmajor)
-        hipLaunchKernelGGL((fused_tok_kernel<T, true>), grid, dim3(256), 0, s, gt, order, hd, sq, tb, to,
+    uint32_t b_span, o_span;
+    const bool fit_b = rows_fit_descriptor<T>(tb, N, hd, &b_span), fit_o = rows_fit_descriptor<T>(to, N, hd, &o_span);
+    if (fit_b && fit_o) {
+        if (a_kmajor)
+            hipLaunchKernelGGL((fused_tok_kernel<T, true>), grid, dim3(256), 0, s, gt, order, hd, sq, tb, to, b_span,
+                               o_span, scale_out);
+        else
+            hipLaunchKernelGGL((fused_tok_kernel<T, false>), grid, dim3(256), 0, s, gt, order, hd, sq, tb, to, b_span,
+                               o_span, scale_out);
+    } else if (a_kmajor) {
+        hipLaunchKernelGGL((fused_tok_wide_kernel<T, true>), grid, dim3(256), 0, s, gt, order, hd, sq, tb, to,
                            scale_out);
-    else
-        hipLaunchKernelGGL((fused_tok_kernel<T, false>), grid, dim3(256), 0, s, gt, order, hd, sq, tb, to,
+    } else {
+        hipLaunchKernelGGL((fused_tok_wide_kernel<T, false>), grid, dim3(256), 0, s, gt, order, hd, sq, tb, to,
                            scale_out);
+    }
     return launch_ok("fused sq->tokens product");
 }
 
@@ -1173,9 +1438,9 @@ int sswin_fused_tokens_to_sq(int dtype, int epilogue, const int32_t* plan, int64
     const int32_t* tok_pos = tokens + 3 * N;
     const double mean_c = (double)N * H / (double)G;          // every voxel is a token of one window, in each of its H groups
     switch (dtype) {
-        case SSWIN_F32: return launch_sq<float>(epilogue, gt, mean_c, order, tok_pos, H, hd, ta, tb, scale_a, bias, n, mask, n_mask_windows, out, row_ids, s);
-        case SSWIN_F16: return launch_sq<__half>(epilogue, gt, mean_c, order, tok_pos, H, hd, ta, tb, scale_a, bias, n, mask, n_mask_windows, out, row_ids, s);
-        case SSWIN_BF16: return launch_sq<__hip_bfloat16>(epilogue, gt, mean_c, order, tok_pos, H, hd, ta, tb, scale_a, bias, n, mask, n_mask_windows, out, row_ids, s);
+        case SSWIN_F32: return launch_sq<float>(epilogue, gt, N, mean_c, order, tok_pos, H, hd, ta, tb, scale_a, bias, n, mask, n_mask_windows, out, row_ids, s);
+        case SSWIN_F16: return launch_sq<__half>(epilogue, gt, N, mean_c, order, tok_pos, H, hd, ta, tb, scale_a, bias, n, mask, n_mask_windows, out, row_ids, s);
+        case SSWIN_BF16: return launch_sq<__hip_bfloat16>(epilogue, gt, N, mean_c, order, tok_pos, H, hd, ta, tb, scale_a, bias, n, mask, n_mask_windows, out, row_ids, s);
         default: return fail("fused_tokens_to_sq: unsupported token dtype %d", dtype);
     }
 }
@@ -1192,9 +1457,9 @@ int sswin_fused_sq_to_tokens(int dtype, int a_kmajor, const int32_t* plan, int64
     hipStream_t s = static_cast<hipStream_t>(stream);
     const double mean_c = (double)N * H / (double)G;
     switch (dtype) {
-        case SSWIN_F32: return launch_tok<float>(a_kmajor, gt, mean_c, tokens, hd, sq, tb, to, scale_out, s);
-        case SSWIN_F16: return launch_tok<__half>(a_kmajor, gt, mean_c, tokens, hd, sq, tb, to, scale_out, s);
-        case SSWIN_BF16: return launch_tok<__hip_bfloat16>(a_kmajor, gt, mean_c, tokens, hd, sq, tb, to, scale_out, s);
+        case SSWIN_F32: return launch_tok<float>(a_kmajor, gt, N, mean_c, tokens, hd, sq, tb, to, scale_out, s);
+        case SSWIN_F16: return launch_tok<__half>(a_kmajor, gt, N, mean_c, tokens, hd, sq, tb, to, scale_out, s);
+        case SSWIN_BF16: return launch_tok<__hip_bfloat16>(a_kmajor, gt, N, mean_c, tokens, hd, sq, tb, to, scale_out, s);
         default: return fail("fused_sq_to_tokens: unsupported token dtype %d", dtype);
     }
 }

@@ -7,6 +7,8 @@
 // (row 8*(r/4) + 4*(l/32) + r%4, column l % 32).
 #pragma once
 
+#include <stdint.h>
+
 #include <type_traits>
 
 #include "sswin_common.hpp"
@@ -74,6 +76,58 @@ inline unsigned block_task_slices(double mean_c, int C, bool square, int groups_
     const double per_group = square ? nb * nb : nb * (double)((C + 31) / 32);
     const int y = (int)(groups_per_wg * per_group / 2.5 + 0.5);
     return (unsigned)(y < 1 ? 1 : (y > 8 ? 8 : y));
+}
+
+// ---- blocks addressed through buffer descriptors ----
+// A descriptor of exactly a block's size (base and size are scalars) lets the memory pipeline do the bounds checks: a
+// lane whose row, column or reduction index lies outside the block forms the offset BUF_OUTSIDE, loads zero and has
+// its store dropped, so ragged blocks need no clamp, select or branch, and an access costs one vector add for its
+// offset.  Sizes stay at or below 2^31 bytes so that BUF_OUTSIDE plus any offset inside the block is still outside.
+typedef uint32_t u32x4_b __attribute__((ext_vector_type(4)));
+constexpr uint32_t BUF_OUTSIDE = 0x80000000u;
+
+template <typename T>
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t buf_of(const T* base, uint32_t bytes) {
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<T*>(base), 0, (int)bytes, 0x00020000);
+}
+// one value of a float, half or bfloat16 array at byte offset off
+template <typename T>
+__device__ __forceinline__ float buf_load1(const __amdgpu_buffer_rsrc_t& r, uint32_t off) {
+    if constexpr (sizeof(T) == 4) {
+        return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, off, 0, 0));
+    } else {
+        const uint16_t u = (uint16_t)__builtin_amdgcn_raw_buffer_load_b16(r, off, 0, 0);
+        return to_acc(__builtin_bit_cast(T, u));
+    }
+}
+// N consecutive values (8 or 16) from byte offset off, all inside or all outside the buffer, in 16-byte loads
+template <typename T, int N>
+__device__ __forceinline__ void buf_load_run(const __amdgpu_buffer_rsrc_t& r, uint32_t off, float (&x)[16]) {
+    constexpr int PER = 16 / (int)sizeof(T);                 // values per load
+#pragma unroll
+    for (int v = 0; v < N / PER; ++v) {
+        const u32x4_b t = __builtin_amdgcn_raw_buffer_load_b128(r, off + 16u * v, 0, 0);
+        const uint32_t w[4] = {t.x, t.y, t.z, t.w};
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if constexpr (sizeof(T) == 4) {
+                x[4 * v + e] = __builtin_bit_cast(float, w[e]);
+            } else {
+                const uint16_t lo = (uint16_t)(w[e] & 0xffffu), hi = (uint16_t)(w[e] >> 16);
+                x[8 * v + 2 * e] = to_acc(__builtin_bit_cast(T, lo));
+                x[8 * v + 2 * e + 1] = to_acc(__builtin_bit_cast(T, hi));
+            }
+        }
+    }
+}
+template <typename T>
+__device__ __forceinline__ void buf_store1(const __amdgpu_buffer_rsrc_t& r, uint32_t off, float v) {
+    if constexpr (sizeof(T) == 4) {
+        __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(uint32_t, v), r, off, 0, 0);
+    } else {
+        const T t = from_acc<T>(v);
+        __builtin_amdgcn_raw_buffer_store_b16((short)__builtin_bit_cast(uint16_t, t), r, off, 0, 0);
+    }
 }
 
 __device__ __forceinline__ int clamp16(int v) { return v < 0 ? 0 : (v > 16 ? 16 : v); }

@@ -230,7 +230,9 @@ __global__ __launch_bounds__(256) void rows_from_counts_kernel(const int32_t* __
     int32_t* out = rows + sq_start[g];
     const int count = c * c;
     const float inv = 1.0f / (float)c;
-    for (int f = lane; f < count; f += 64) {
+    // gridDim.y wavefronts share a group's entries: one wavefront alone would write the 51 529 entries of a
+    // 227-token window in 805 rounds
+    for (int f = lane + 64 * (int)blockIdx.y; f < count; f += 64 * (int)gridDim.y) {
         int i = (int)((float)f * inv);                        // f / c up to one, corrected below (f < 2^24)
         i -= i * c > f ? 1 : 0;
         i += (i + 1) * c <= f ? 1 : 0;
@@ -317,12 +319,18 @@ int sswin_plan_from_indices(const int32_t* idx, int64_t M, int inner, int32_t* p
     return 0;
 }
 
-int sswin_softmax_rows_from_counts(const int32_t* c, const int32_t* scans, int64_t G, int32_t* rows_out, void* stream) {
-    SSWIN_CHECK(G >= 0, "softmax_rows_from_counts: negative group count");
-    if (G == 0) return 0;
+int sswin_softmax_rows_from_counts(const int32_t* c, const int32_t* scans, int64_t G, int64_t A, int32_t* rows_out,
+                                   void* stream) {
+    SSWIN_CHECK(G >= 0 && A >= 0, "softmax_rows_from_counts: negative size");
+    if (G == 0 || A == 0) return 0;
     SSWIN_CHECK(c && scans && rows_out, "softmax_rows_from_counts: null pointer");
-    hipLaunchKernelGGL(rows_from_counts_kernel, dim3((unsigned)((G + 3) / 4)), dim3(256), 0, static_cast<hipStream_t>(stream), c,
-                       scans, scans + G, G, rows_out);
+    // wavefronts per group from the mean number of entries of a group: about 256 entries (four rounds) per wavefront
+    // measured best (windows of 5^3: 14.9 -> 12.4 us, of 7^3: 45.6 -> 24.2 us; 128 and 512 entries: 14.3 / 13.4 us
+    // and 24.5 / 25.0 us)
+    const int64_t per = 256;
+    const int64_t y = (A / G + per / 2) / per;
+    hipLaunchKernelGGL(rows_from_counts_kernel, dim3((unsigned)((G + 3) / 4), (unsigned)(y < 1 ? 1 : (y > 16 ? 16 : y))), dim3(256), 0,
+                       static_cast<hipStream_t>(stream), c, scans, scans + G, G, rows_out);
     return launch_ok("softmax_rows_from_counts");
 }
 

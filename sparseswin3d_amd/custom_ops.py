@@ -525,7 +525,7 @@ def softmax_rows_from_counts(_c, nnz):
     with _lib.on_device(d):
         scans, sum_c2 = _scans_for(c, lib, d)
         _check(sum_c2 is None or sum_c2 == nnz, f"softmax_rows_from_counts: {nnz} entries, the groups hold {sum_c2}")
-        _lib.check(lib.sswin_softmax_rows_from_counts(_ptr(c), _ptr(scans), c.numel(), _ptr(rows), _stream(d)))
+        _lib.check(lib.sswin_softmax_rows_from_counts(_ptr(c), _ptr(scans), c.numel(), int(nnz), _ptr(rows), _stream(d)))
     return rows
 
 

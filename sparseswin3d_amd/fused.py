@@ -359,14 +359,6 @@ def supports_resident(qkv: torch.Tensor, n: int) -> bool:
     return supports(qkv, n) and qkv.shape[-1] == 32 and n <= 128
 
 
-def pays(n: int) -> bool:
-    """Whether the module should take the fused path by itself where it is supported: yes for windows of at most 128
-    positions.  For larger windows the operator path is the faster one (a room of 112 000 voxels in windows of 7^3
-    positions, 3 heads of 16 channels: module call 2.08 ms on the fused path, 1.54 ms on the operator path);
-    ``WindowAttentionSparse.fused = "always"`` takes the fused path wherever it is supported."""
-    return n <= 128
-
-
 def supports(qkv: torch.Tensor, n: int, table: bool = False) -> bool:
     """The fused path covers fp32/fp16/bf16 on the GPU.  Windows: at most 128 positions when the bias gradient is
     formed as an [H, n, n] array (its LDS table), at most 384 (7^3 = 343 included) when it goes straight to the

@@ -681,10 +681,10 @@ class WindowAttentionSparse(nn.Module):
     """Window multi-head self attention with relative position bias on sparse windows.
 
     ``fused`` (class or instance attribute, default True) selects the fused HIP path of
-    :mod:`sparseswin3d_amd.fused` where it is supported and the faster one (windows of at most 128
-    positions); ``fused = "always"`` takes it wherever it is supported (windows up to 384 positions
-    with a relative position table, 7^3 included); with ``fused = False`` the forward pass is the
-    operator-by-operator composition of the reference.  ``resident`` picks between the two
+    :mod:`sparseswin3d_amd.fused` wherever it is supported (windows up to 384 positions with a relative
+    position table, 7^3 included; measured faster than the operator path there too: 1.05 against 1.19 ms per
+    module call on a room of 112 000 voxels, 3 heads of 16 channels); with ``fused = False`` the forward pass is
+    the operator-by-operator composition of the reference.  ``resident`` picks between the two
     fused variants: True = window-resident kernels (attention matrix kept in registers, heads
     of 32 channels only), False = block products with the attention matrix in HBM, None =
     resident whenever it applies.  All paths give the same result.
@@ -754,8 +754,7 @@ class WindowAttentionSparse(nn.Module):
                     cache[self.num_heads] = plan
         qkv = tall_linear(x.features, self.qkv).reshape(-1, 3, self.num_heads, c // self.num_heads)
         table_index = self._table_index(n) if plan is not None and self.fused else None
-        if plan is not None and self.fused and fused.supports(x.features, n, table_index is not None) and \
-                (self.fused == "always" or fused.pays(n)):
+        if plan is not None and self.fused and fused.supports(x.features, n, table_index is not None):
             resident = fused.supports_resident(qkv, n) if self.resident is None else self.resident
             if table_index is not None:
                 out = fused.fused_window_attention(qkv, self.relative_position_bias_table, x.indices, mask, b, n,

@@ -155,5 +155,5 @@ def set_path(attn, path):
     """Select the implementation behind WindowAttentionSparse.forward: "resident" = window-resident
     kernels, "fused" = block products with the attention matrix in memory, "operators" = the
     operator-by-operator composition of the reference."""
-    attn.fused = "always" if path != "operators" else False
+    attn.fused = path != "operators"
     attn.resident = {"resident": True, "fused": False, "operators": None}[path]

@@ -77,10 +77,9 @@ def test_window_attention_forward_backward(shift, dim, heads, path):
 def test_window_7_heads_of_16_channels(path):
     """The reference's own ScanNet setting (config/scannet/semseg-swin-0-base.py:11-31): windows of 7^3 = 343
     positions, shift 3, 48 channels in 3 heads of 16.  Heads of 16 channels and windows above 128 positions are
-    outside the window-resident kernels.  The module's default for windows this large is the operator path (the
-    reference's own composition, the faster one here); ``fused = "always"`` takes the fused path (block products
-    that read the token rows through the token plan, attention matrix in memory, bias gradient straight into the
-    table).  Forward and backward of both against the fp64 CPU path."""
+    outside the window-resident kernels: the module takes the fused path (block products that read the token rows
+    through the token plan, attention matrix in memory, bias gradient straight into the table), which the test checks,
+    and ``fused = False`` the reference's own composition.  Forward and backward of both against the fp64 CPU path."""
     from sparseswin3d_amd import synth
     from sparseswin3d_amd.window_attention import SparseVoxelTensor, WindowAttentionSparse
     torch.manual_seed(4)
@@ -91,11 +90,12 @@ def test_window_7_heads_of_16_channels(path):
     N = len(win_idx)
     attn = WindowAttentionSparse(48, 3, ws, qkv_bias=True).cuda()
     if path == "fused":
-        attn.fused, attn.resident = "always", False
         seen = []
         from sparseswin3d_amd import fused as fused_mod
         real = fused_mod.fused_window_attention
         fused_mod.fused_window_attention = lambda *a, **k: (seen.append(1), real(*a, **k))[1]
+    else:
+        attn.fused = False
     with torch.no_grad():
         attn.relative_position_bias_table.normal_(0, 0.5)
     mask_np = synth.shift_region_mask(synth.padded_shape(grid, ws), ws, shift)

@@ -178,6 +178,32 @@ def test_fused_equals_operator_path(shift):
             close(a, b, 1e-5, f"{path}: {what}")
 
 
+@pytest.mark.parametrize("dtype,dim,heads", [(torch.float32, 96, 3), (torch.float32, 48, 3), (torch.bfloat16, 64, 2)])
+def test_fused_products_with_32_and_64_bit_addresses(dtype, dim, heads, monkeypatch):
+    """The fused-path products address token rows through buffer descriptors; tensors beyond 2^31 bytes take kernels
+    with 64-bit addresses (SSWIN_FUSED_WIDE=1 sends everything there).  The two split the last tokens of a reduction
+    between the lane halves differently, so the sums agree to rounding, not bit for bit."""
+    from sparseswin3d_amd import synth
+    from sparseswin3d_amd.window_attention import SparseVoxelTensor
+    c4, _ = synth.with_batch([synth.box_surfaces_scene(seed=5, grid=(40, 40, 40), n_boxes=4)])
+    idx, nw, n = synth.window_indices(c4, (40, 40, 40), (5, 5, 5), (2, 2, 2))
+    mask = torch.from_numpy(synth.shift_region_mask((40, 40, 40), (5, 5, 5), (2, 2, 2))).cuda()
+    attn = _modules(dim, heads, dtype)
+    set_path(attn, "fused")
+    feats = torch.randn(len(idx), dim, device="cuda").to(dtype)
+    up = torch.randn(len(idx), dim, device="cuda").to(dtype)
+    res = []
+    for wide in ("0", "1"):
+        monkeypatch.setenv("SSWIN_FUSED_WIDE", wide)
+        attn.zero_grad()
+        f = feats.clone().requires_grad_(True)
+        out = attn(SparseVoxelTensor(f, torch.from_numpy(idx).cuda(), (n,), nw), mask).features
+        out.backward(up)
+        res.append([t.detach().double().cpu().numpy() for t in (out, f.grad, attn.qkv.weight.grad, attn.relative_position_bias_table.grad)])
+    for a, b, what in zip(res[0], res[1], ("out", "d feats", "d qkv.w", "d bias table")):
+        close(a, b, 1e-5 if dtype == torch.float32 else 2e-2, f"descriptor against 64-bit addresses: {what}")
+
+
 @pytest.mark.parametrize("path", ["resident", "fused"])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_fused_16bit_against_cpu_fp64(dtype, path):
