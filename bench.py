@@ -457,7 +457,7 @@ def kernel_table(wl, reps=20, only=None):
         qkv_c = qkv.contiguous()
         bias = torch.randn(H, b["n"], b["n"], device=dev)
         s_f = torch.empty(tp.A, device=dev)
-        rows_f = torch.empty(tp.A, dtype=torch.int32, device=dev)
+        p_f = torch.empty(tp.A, device=dev)
         out_f = torch.empty(N, D, device=dev)
         dqkv = torch.empty_like(qkv_c)
         dbias = torch.zeros(H, b["n"], b["n"], device=dev)
@@ -466,12 +466,12 @@ def kernel_table(wl, reps=20, only=None):
         bg_ws = torch.empty(int(bg_bytes), dtype=torch.uint8, device=dev)
         f_entries = [
             ("fused token plan, one of a stage's two", staged_plan, 28 * N + 20 * tp.G, 1),
-            ("fused S=QK^T+bias+mask", lambda: F._tokens_to_sq(tp, dt, True, qkv_c, 3 * D, 0, qkv_c, 3 * D, D, hd, 0.17, bias, mask, s_f, rows_f), 8 * E + 8 * A, 1),
-            ("fused softmax fwd", lambda: ops.softmax_last_dim_forward(rows_f, s_f), 12 * A, 1),
+            ("fused S=QK^T+bias+mask", lambda: F._tokens_to_sq(tp, dt, True, qkv_c, 3 * D, 0, qkv_c, 3 * D, D, hd, 0.17, bias, mask, s_f, None), 8 * E + 4 * A, 1),
+            ("fused softmax fwd (rows from the group table)", lambda: F._group_softmax(tp, False, s_f, None, p_f), 8 * A, 1),
             ("fused O=PV", lambda: F._sq_to_tokens(tp, dt, False, p_val, qkv_c, 3 * D, 2 * D, out_f, D, 0, hd, 1.0), 4 * A + 8 * E, 1),
             ("fused dP=dO V^T", lambda: F._tokens_to_sq(tp, dt, False, out_f, D, 0, qkv_c, 3 * D, 2 * D, hd, 1.0, None, None, s_f, None), 8 * E + 4 * A, 1),
             ("fused dV=P^T dO", lambda: F._sq_to_tokens(tp, dt, True, p_val, out_f, D, 0, dqkv, 3 * D, 2 * D, hd, 1.0), 4 * A + 8 * E, 1),
-            ("fused softmax bwd", lambda: ops.softmax_last_dim_backward(rows_f, p_val, g_s), 16 * A, 1),
+            ("fused softmax bwd (rows from the group table)", lambda: F._group_softmax(tp, True, p_val, g_s, p_f), 12 * A, 1),
             ("fused dQ=dS K", lambda: F._sq_to_tokens(tp, dt, False, g_s, qkv_c, 3 * D, D, dqkv, 3 * D, 0, hd, 0.17), 4 * A + 8 * E, 1),
             ("fused dK=dS^T Q", lambda: F._sq_to_tokens(tp, dt, True, g_s, qkv_c, 3 * D, 0, dqkv, 3 * D, D, hd, 0.17), 4 * A + 8 * E, 1),
             ("fused bias table grad", lambda: _lib.check(lib.sswin_bias_table_grad(ptr(tp.plan), tp.g_cap, tp.G, ptr(tp.tokens), tp.N, H, b["n"], ptr(ti.code), ti.offset0, n_table, ptr(g_s), ptr(d_table), ptr(tg_ws), tg_bytes, stream)), 4 * A, 1),

@@ -351,6 +351,15 @@ int sswin_fused_sq_to_tokens(int dtype, int a_kmajor, const int32_t* plan, int64
                              const void* b_base, int64_t b_stride, int b_col0, void* o_base,
                              int64_t o_stride, int o_col0, float scale_out, void* stream);
 
+/* The sparse row softmax over the rows of the groups' [c x c] blocks, forward (backward == 0: out = softmax of
+ * x_or_y, grad ignored) or backward (out = y (g - sum_j g_j y_j) with y = x_or_y, g = grad).  The arithmetic of
+ * softmax_last_dim_forward / _backward (sparse_swin/ops.cu:128-194: zero-initialised maximum, + 1e-8 in the
+ * denominator); the rows come from the group table instead of a row id per entry (swin3d_base.py:140-150 builds those
+ * ids with flatten_indices + unique_consecutive).  fp32 sq arrays; out may be x_or_y or grad (in place).  N, H: voxels
+ * and heads of the plan (the launch is sized from the mean group N*H/G); c_max <= 384.  Asynchronous. */
+int sswin_group_softmax(int backward, const int32_t* plan, int64_t g_cap, int64_t G, int64_t N, int H,
+                        int c_max, const float* x_or_y, const float* grad, float* out, void* stream);
+
 /* d_bias[h, pos_i, pos_j] += ds over all windows (the backward of swin3d_base.py:557-566, which
  * autograd performs as an index_add).  d_bias: fp32 [H,n,n], accumulated into (zero it first).
  * n*n*4 bytes must fit 64 KiB of LDS.  No atomics: every table row is owned by one wavefront

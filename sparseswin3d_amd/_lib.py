@@ -64,6 +64,7 @@ SIGNATURES = {
                                         _vp, _i64, _i32, C.c_float, _vp, _i32, _vp, _i32, _vp, _vp, _vp]),
     "sswin_fused_sq_to_tokens": (_i32, [_i32, _i32, _vp, _i64, _i64, _vp, _i64, _i32, _i32, _vp, _vp, _i64, _i32,
                                         _vp, _i64, _i32, C.c_float, _vp]),
+    "sswin_group_softmax": (_i32, [_i32, _vp, _i64, _i64, _i64, _i32, _i32, _vp, _vp, _vp, _vp]),
     "sswin_fused_bias_grad_workspace_bytes": (_sz, [_i64, _i32, _i32]),
     "sswin_fused_bias_grad": (_i32, [_vp, _i64, _i64, _vp, _i64, _i32, _i32, _vp, _vp, _vp, _sz, _vp]),
     "sswin_column_sum_workspace_bytes": (_sz, [_i64, _i32]),

@@ -657,6 +657,107 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 }
 
 // ------------------------------------------------------------------------------------------
+// sq -> sq: the sparse row softmax of the operator set (ops.cu:128-194: m = max(0, row maximum),
+// y = exp(x - m) / (sum + 1e-8); backward gx = y (g - sum_j g_j y_j)) over the rows of the groups' [c x c] blocks.
+// The rows are known from the group table, so no row ids are written by the score product or read here (4 of the
+// 12 / 16 bytes per entry of the id-driven kernel).  A task = 32 rows of a group; LPR lanes share a row (16, 32 or
+// all 64, the smallest that holds the row in at most six values per lane), so a wavefront works on 4, 2 or 1 rows
+// at a time and reduces with DPP moves inside 16 lanes plus one or two cross-lane reads.  In place (out == the
+// input, or == grad in the backward) is fine: a wavefront reads the values of a row before it writes any of them.
+// ------------------------------------------------------------------------------------------
+template <int LPR>
+__device__ __forceinline__ float seg_sum(float v) {
+    v = row16_sum(v);
+    if (LPR >= 32) v += __shfl_xor(v, 16, 64);
+    if (LPR >= 64) v += __shfl_xor(v, 32, 64);
+    return v;
+}
+// B steps of a task are requested together (a step alone would wait for its loads before the next one asks for its own)
+template <int LPR>
+__device__ __forceinline__ int seg_max_i32(int v) {
+    v = max(v, dpp_i32<0xB1>(v));
+    v = max(v, dpp_i32<0x4E>(v));
+    v = max(v, dpp_i32<0x141>(v));
+    v = max(v, dpp_i32<0x140>(v));
+    if (LPR >= 32) v = max(v, __shfl_xor(v, 16, 64));
+    if (LPR >= 64) v = max(v, __shfl_xor(v, 32, 64));
+    return v;
+}
+
+template <bool BWD, int LPR, int U, int B>
+__device__ __forceinline__ void group_softmax_rows(const __amdgpu_buffer_rsrc_t& rx, const __amdgpu_buffer_rsrc_t& rg,
+                                                   const __amdgpu_buffer_rsrc_t& ro, int c, int row0, int rows, int lane) {
+    constexpr int RPS = 64 / LPR;                              // rows per step
+    const int j0 = lane & (LPR - 1), rl = lane / LPR;
+    for (int r0 = 0; r0 < rows; r0 += RPS * B) {
+        float x[B][U], g[B][U];
+        uint32_t off[B][U];
+#pragma unroll
+        for (int b = 0; b < B; ++b) {
+            const int r = r0 + b * RPS + rl;
+            const uint32_t base = (uint32_t)((row0 + r) * c) * 4u;
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int j = j0 + LPR * u;
+                off[b][u] = (j < c && r < rows) ? base + 4u * (uint32_t)j : BUF_OUTSIDE;
+                x[b][u] = buf_load1<float>(rx, off[b][u]);
+                if (BWD) g[b][u] = buf_load1<float>(rg, off[b][u]);
+            }
+        }
+#pragma unroll
+        for (int b = 0; b < B; ++b) {
+            if (!BWD) {
+                // m = max(0, row maximum): values below zero do not matter, and the bit patterns of floats from zero
+                // upwards are ordered like integers, so the maximum is taken over max(bits, 0) with integer
+                // instructions (a negative float is a negative integer; loads outside the row gave zero)
+                int mb = 0;
+#pragma unroll
+                for (int u = 0; u < U; ++u) mb = max(mb, __builtin_bit_cast(int, x[b][u]));
+                const float m = __builtin_bit_cast(float, seg_max_i32<LPR>(mb));
+                float sum = 0.f;
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    x[b][u] = off[b][u] != BUF_OUTSIDE ? __builtin_amdgcn_exp2f((x[b][u] - m) * 1.44269504088896f) : 0.f;   // x - m <= 0: no range problem
+                    sum += x[b][u];
+                }
+                const float inv = __builtin_amdgcn_rcpf(seg_sum<LPR>(sum) + 1e-8f);   // 1 ulp: inside the tolerance of a product of two roundings
+#pragma unroll
+                for (int u = 0; u < U; ++u) buf_store1<float>(ro, off[b][u], x[b][u] * inv);
+            } else {
+                float dot = 0.f;
+#pragma unroll
+                for (int u = 0; u < U; ++u) dot += x[b][u] * g[b][u];   // loads outside the row are zero
+                dot = seg_sum<LPR>(dot);
+#pragma unroll
+                for (int u = 0; u < U; ++u) buf_store1<float>(ro, off[b][u], x[b][u] * (g[b][u] - dot));
+            }
+        }
+    }
+}
+
+template <bool BWD>
+__global__ __launch_bounds__(256) void group_softmax_kernel(FusedGroups gt, const float* __restrict__ xs,
+                                                            const float* __restrict__ gs, float* __restrict__ out) {
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int64_t g0 = (int64_t)blockIdx.x * FUSED_GROUPS_PER_WG;
+    const GroupLanes gl = load_groups<false>(gt, g0, lane);
+    const TaskSet ts = make_tasks(gl, false, 1);                // one task per 32 rows of a group
+    const int total = ts.first[FUSED_GROUPS_PER_WG];
+    for (int t = wave + 4 * (int)blockIdx.y; t < total; t += 4 * (int)gridDim.y) {
+        const Task k = locate_task(ts, gl, t, false, 1);
+        const int c = k.c, row0 = k.bi * 32;
+        const int rows = c - row0 < 32 ? c - row0 : 32;
+        const uint32_t bytes = (uint32_t)(c * c) * 4u;
+        const __amdgpu_buffer_rsrc_t rx = buf_of(xs + k.sq, bytes), rg = buf_of(BWD ? gs + k.sq : xs + k.sq, bytes);
+        const __amdgpu_buffer_rsrc_t ro = buf_of(out + k.sq, bytes);
+        if (c <= 16) group_softmax_rows<BWD, 16, 1, 8>(rx, rg, ro, c, row0, rows, lane);
+        else if (c <= 32) group_softmax_rows<BWD, 32, 1, 16>(rx, rg, ro, c, row0, rows, lane);
+        else if (c <= 128) group_softmax_rows<BWD, 64, 2, 8>(rx, rg, ro, c, row0, rows, lane);
+        else group_softmax_rows<BWD, 64, 6, 2>(rx, rg, ro, c, row0, rows, lane);
+    }
+}
+
+// ------------------------------------------------------------------------------------------
 // The same two products with 64-bit addresses, for token tensors that a buffer descriptor cannot cover (more than
 // 2^31 bytes, or 16-bit rows that do not start at a multiple of four bytes).
 // tokens x tokens -> sq :  out[i, j] = sum_ch A[token i, ch] * B[token j, ch]   (K = hd)
@@ -1462,6 +1563,23 @@ int sswin_fused_sq_to_tokens(int dtype, int a_kmajor, const int32_t* plan, int64
         case SSWIN_BF16: return launch_tok<__hip_bfloat16>(a_kmajor, gt, N, mean_c, tokens, hd, sq, tb, to, scale_out, s);
         default: return fail("fused_sq_to_tokens: unsupported token dtype %d", dtype);
     }
+}
+
+int sswin_group_softmax(int backward, const int32_t* plan, int64_t g_cap, int64_t G, int64_t N, int H, int c_max,
+                        const float* x_or_y, const float* grad, float* out, void* stream) {
+    SSWIN_CHECK(G >= 0 && G <= g_cap && N >= 0 && H > 0, "group_softmax: bad sizes");
+    if (G == 0) return 0;
+    SSWIN_CHECK(plan && x_or_y && out && (!backward || grad), "group_softmax: null pointer");
+    SSWIN_CHECK(c_max > 0 && c_max <= 384, "group_softmax: windows of %d tokens are not supported (384 at most)", c_max);
+    const FusedGroups gt = groups_of(plan, g_cap, G);
+    const dim3 grid((unsigned)((G + FUSED_GROUPS_PER_WG - 1) / FUSED_GROUPS_PER_WG),
+                    block_task_slices((double)N * H / (double)G, 1, false, FUSED_GROUPS_PER_WG));
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (backward)
+        hipLaunchKernelGGL((group_softmax_kernel<true>), grid, dim3(256), 0, s, gt, x_or_y, grad, out);
+    else
+        hipLaunchKernelGGL((group_softmax_kernel<false>), grid, dim3(256), 0, s, gt, x_or_y, grad, out);
+    return launch_ok("group softmax");
 }
 
 static int bias_grad_slices(int64_t windows, int H) {

@@ -57,15 +57,15 @@ struct Carver {
 // device: wave64 cross-lane primitives.  Reductions inside a 16-lane DPP row use DPP
 // modifiers (no LDS traffic); the two cross-row steps use ds_bpermute via __shfl_xor.
 // ------------------------------------------------------------------------------------------
+// (the controls used here give every lane a source lane, so no lane keeps an old value: the move form without one
+// lets the compiler fold the cross-lane read into the instruction that uses it)
 template <int CTRL>
 __device__ __forceinline__ float dpp_f32(float v) {
-    return __builtin_bit_cast(
-        float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, v), __builtin_bit_cast(int, v),
-                                           CTRL, 0xf, 0xf, false));
+    return __builtin_bit_cast(float, __builtin_amdgcn_mov_dpp(__builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
 }
 template <int CTRL>
 __device__ __forceinline__ int dpp_i32(int v) {
-    return __builtin_amdgcn_update_dpp(v, v, CTRL, 0xf, 0xf, false);
+    return __builtin_amdgcn_mov_dpp(v, CTRL, 0xf, 0xf, true);
 }
 
 // DPP controls: quad_perm[1,0,3,2]=0xB1, quad_perm[2,3,0,1]=0x4E, row_half_mirror=0x141,

@@ -162,6 +162,13 @@ def _sq_to_tokens(tp, dtype, a_kmajor, sq, b, b_stride, b_col0, o, o_stride, o_c
         _ptr(sq), _ptr(b), b_stride, b_col0, _ptr(o), o_stride, o_col0, C.c_float(scale), stream))
 
 
+def _group_softmax(tp, backward, x_or_y, grad, out):
+    """Row softmax (or its backward) over the [c x c] blocks of the plan's groups; ``out`` may be one of the inputs."""
+    _lib.check(_lib.load().sswin_group_softmax(
+        1 if backward else 0, _ptr(tp.plan), tp.g_cap, tp.G, tp.N, tp.H, tp.c_max, _ptr(x_or_y), _ptr(grad), _ptr(out),
+        _lib.stream_handle(tp.device)))
+
+
 def _bias32(bias, table_index, H, n, d):
     """The fp32 [H, n, n] bias the kernels read: ``bias`` itself, or gathered from the [rows, H] table."""
     if table_index is None:
@@ -214,20 +221,19 @@ class _FusedWindowAttention(Function):
         if mask is not None:
             mask = mask.to(torch.int8).contiguous()
         with _lib.on_device(d):
-            s = torch.empty(tp.A, dtype=torch.float32, device=d)
-            rows = torch.empty(tp.A, dtype=torch.int32, device=d)
-            _tokens_to_sq(tp, dtype, True, qkv, 3 * D, 0, qkv, 3 * D, D, hd, scale, bias32, mask, s, rows)
-            p = ops.softmax_last_dim_forward(rows, s)
+            p = torch.empty(tp.A, dtype=torch.float32, device=d)
+            _tokens_to_sq(tp, dtype, True, qkv, 3 * D, 0, qkv, 3 * D, D, hd, scale, bias32, mask, p, None)
+            _group_softmax(tp, False, p, None, p)                  # S -> P in place, rows from the group table
             out = torch.empty((N, D), dtype=dtype, device=d)
             _sq_to_tokens(tp, dtype, False, p, qkv, 3 * D, 2 * D, out, D, 0, hd, 1.0)
-        ctx.save_for_backward(qkv, p, rows)
+        ctx.save_for_backward(qkv, p)
         ctx.tp, ctx.scale, ctx.bias_meta, ctx.table_index = tp, scale, (bias.dtype, bias.shape), table_index
         return out
 
     @staticmethod
     @once_differentiable
     def backward(ctx, grad_out):
-        qkv, p, rows = ctx.saved_tensors
+        qkv, p = ctx.saved_tensors
         tp, scale = ctx.tp, ctx.scale
         N, _, H, hd = qkv.shape
         D = H * hd
@@ -237,11 +243,11 @@ class _FusedWindowAttention(Function):
         lib = _lib.load()
         with _lib.on_device(d):
             d_qkv = torch.empty_like(qkv)
-            d_p = torch.empty(tp.A, dtype=torch.float32, device=d)
+            d_s = torch.empty(tp.A, dtype=torch.float32, device=d)
             # dP = dO V^T ; dV = P^T dO
-            _tokens_to_sq(tp, dtype, False, grad_out, D, 0, qkv, 3 * D, 2 * D, hd, 1.0, None, None, d_p, None)
+            _tokens_to_sq(tp, dtype, False, grad_out, D, 0, qkv, 3 * D, 2 * D, hd, 1.0, None, None, d_s, None)
             _sq_to_tokens(tp, dtype, True, p, grad_out, D, 0, d_qkv, 3 * D, 2 * D, hd, 1.0)
-            d_s = ops.softmax_last_dim_backward(rows, p, d_p)
+            _group_softmax(tp, True, p, d_s, d_s)                  # dP -> dS in place
             # dQ = scale * dS K ; dK = scale * dS^T Q
             _sq_to_tokens(tp, dtype, False, d_s, qkv, 3 * D, D, d_qkv, 3 * D, 0, hd, scale)
             _sq_to_tokens(tp, dtype, True, d_s, qkv, 3 * D, 0, d_qkv, 3 * D, D, hd, scale)

@@ -204,6 +204,46 @@ def test_fused_products_with_32_and_64_bit_addresses(dtype, dim, heads, monkeypa
         close(a, b, 1e-5 if dtype == torch.float32 else 2e-2, f"descriptor against 64-bit addresses: {what}")
 
 
+@pytest.mark.parametrize("H", [1, 3])
+def test_softmax_over_the_rows_of_the_groups(oracle, H):
+    """The fused path's softmax takes its rows from the group table.  Against the fp64 oracle of the operator
+    (zero-initialised maximum, + 1e-8), forward and backward, out of place and in place, on group sizes around the
+    edges of its three lane layouts (16, 32, 64 lanes per row; 2 and 6 values per lane) and with rows that are all
+    negative (their maximum stays 0, ops.cu:128-167)."""
+    from helpers import softmax_bwd_mag
+    from sparseswin3d_amd import fused
+    rng = np.random.default_rng(77 + H)
+    counts = [1, 16, 17, 0, 32, 33, 64, 65, 128, 129, 300, 5, 2, 343]
+    n = 343
+    ind = ragged_window_indices(rng, counts, n)
+    tp = fused.TokenPlan(torch.from_numpy(ind).cuda(), len(counts), n, H)
+    plan = tp.plan.view(5, -1)[:, :tp.G].cpu().numpy()
+    rows = np.empty(tp.A, np.int32)
+    r0 = 0
+    for c, sq in zip(plan[0], plan[2]):
+        rows[sq:sq + c * c] = r0 + np.repeat(np.arange(c), c)
+        r0 += c
+    x = rng.standard_normal(tp.A).astype(np.float32) * 3
+    x[rows % 7 == 3] = -np.abs(x[rows % 7 == 3]) - 1.0          # whole rows below zero
+    g = rng.standard_normal(tp.A).astype(np.float32)
+    xd, gd = torch.from_numpy(x).cuda(), torch.from_numpy(g).cuda()
+    y = torch.empty_like(xd)
+    fused._group_softmax(tp, False, xd, None, y)
+    ref_y = oracle.softmax_last_dim_forward(rows, x.astype(np.float64))
+    close(y.cpu().numpy(), ref_y, 1e-5, "group softmax forward", seg=rows)
+    y2 = xd.clone()
+    fused._group_softmax(tp, False, y2, None, y2)
+    assert torch.equal(y, y2)
+    gx = torch.empty_like(xd)
+    fused._group_softmax(tp, True, y, gd, gx)
+    yh = y.double().cpu().numpy()
+    ref_gx = oracle.softmax_last_dim_backward(rows, yh, g.astype(np.float64))
+    close(gx.cpu().numpy(), ref_gx, 1e-5, "group softmax backward", mag=softmax_bwd_mag(rows, yh, g))
+    g2 = gd.clone()
+    fused._group_softmax(tp, True, y, g2, g2)
+    assert torch.equal(gx, g2)
+
+
 @pytest.mark.parametrize("path", ["resident", "fused"])
 @pytest.mark.parametrize("dtype", [torch.bfloat16, torch.float16])
 def test_fused_16bit_against_cpu_fp64(dtype, path):
