@@ -262,8 +262,12 @@ KERNEL_SYMBOLS = {
     "softmax_last_dim_forward": ("softmax_rows_kernel<float, false", ["sparseswin3d_amd/csrc/softmax.hip"]),
     "softmax_last_dim_backward": ("softmax_rows_kernel<float, true", ["sparseswin3d_amd/csrc/softmax.hip"]),
     "resident bias table grad": ("rpb_table_partial_kernel", ["sparseswin3d_amd/csrc/fused_attention.hip"]),
-    "fused dV=P^T dO": ("fused_tok_kernel", ["sparseswin3d_amd/csrc/fused_attention.hip"]),
-    "fused O=PV": ("fused_tok_kernel", ["sparseswin3d_amd/csrc/fused_attention.hip"]),
+    "fused S=QK^T+bias+mask": ("fused_sq_kernel<float, true", ["sparseswin3d_amd/csrc/fused_attention.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
+    "fused dP=dO V^T": ("fused_sq_kernel<float, false", ["sparseswin3d_amd/csrc/fused_attention.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
+    "fused dV=P^T dO": ("fused_tok_kernel<float, true", ["sparseswin3d_amd/csrc/fused_attention.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
+    "fused O=PV": ("fused_tok_kernel<float, false", ["sparseswin3d_amd/csrc/fused_attention.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
+    "fused softmax fwd (rows from the group table)": ("group_softmax_kernel<false", ["sparseswin3d_amd/csrc/fused_attention.hip"]),
+    "fused softmax bwd (rows from the group table)": ("group_softmax_kernel<true", ["sparseswin3d_amd/csrc/fused_attention.hip"]),
 }
 
 
