@@ -1620,8 +1620,17 @@ int sswin_fused_bias_grad(const int32_t* plan, int64_t g_cap, int64_t G, const i
 // wavefront waits for is its own chain of LDS read-add-writes, so a few of them share a SIMD well), eight per
 // window slice: the batches of a crowded window (up to 3 x 3 of them for 89 tokens) spread over all eight.
 // Measured on cfg2 (the two launches): 2048 wavefronts / 4 per slice 0.038 ms, 3072 / 8 0.036, 4096 / 8 0.040.
-static void table_grad_slices(int64_t windows, int H, int* wslices, int* rsplit) {
-    constexpr int64_t WAVES = 3072, PER_SLICE = 8;
+// A table of more than 1 664 rows (windows of 7^3 positions: 2 197) leaves room for two workgroups per compute unit
+// only, a larger one for one: the launch then holds 2 048 or 1 024 wavefronts, so that all of them are resident at once
+// (3 072 wavefronts on two workgroups per unit ran as one full round and a half-empty second one).
+static size_t table_grad_lds(int table_rows, int n) {
+    const int rows_pad = (table_rows + 31) / 32 * 32 + 32;  // 32 spare rows
+    return (size_t)8 * rows_pad * sizeof(float) + (size_t)n * sizeof(int32_t);
+}
+static void table_grad_slices(int64_t windows, int H, int table_rows, int* wslices, int* rsplit) {
+    constexpr int64_t PER_SLICE = 8;
+    const int64_t resident = std::max<int64_t>(1, std::min<int64_t>(3, (int64_t)(160 * 1024) / (int64_t)table_grad_lds(table_rows, 384)));
+    const int64_t WAVES = 1024 * resident;
     const int64_t want = std::max<int64_t>(1, WAVES / (std::max(H, 1) * PER_SLICE));
     *wslices = (int)std::min<int64_t>(want, std::max<int64_t>(1, windows));
     *rsplit = (int)PER_SLICE;
@@ -1630,7 +1639,7 @@ static void table_grad_slices(int64_t windows, int H, int* wslices, int* rsplit)
 size_t sswin_bias_table_grad_workspace_bytes(int64_t G, int H, int table_rows) {
     const int64_t windows = H > 0 ? G / H : 0;
     int wslices, rsplit;
-    table_grad_slices(windows, H, &wslices, &rsplit);
+    table_grad_slices(windows, H, table_rows, &wslices, &rsplit);
     return (size_t)wslices * rsplit * H * table_rows * sizeof(float) + 256;
 }
 
@@ -1652,12 +1661,12 @@ int sswin_bias_table_grad(const int32_t* plan, int64_t g_cap, int64_t G, const i
     const FusedGroups gt = groups_of(plan, g_cap, G);
     const int64_t windows = G / H;
     int wslices, rsplit;
-    table_grad_slices(windows, H, &wslices, &rsplit);
+    table_grad_slices(windows, H, table_rows, &wslices, &rsplit);
     const int slices = wslices * rsplit;
     float* partial = static_cast<float*>(ws);
     const int64_t waves = (int64_t)slices * H;
     const int rows_pad = (table_rows + 31) / 32 * 32 + 32;  // 32 spare rows
-    const size_t lds = (size_t)8 * rows_pad * sizeof(float) + (size_t)n * sizeof(int32_t);
+    const size_t lds = table_grad_lds(table_rows, n);
     SSWIN_CHECK(lds <= 160 * 1024, "bias_table_grad: a table of %d rows needs %zu bytes of LDS (160 KB at most)", table_rows, lds);
     if (lds > 64 * 1024) {
         // more than the default 64 KB of dynamic LDS: asked for with every such launch (cheap, and correct for any
