@@ -262,12 +262,11 @@ KERNEL_SYMBOLS = {
     "softmax_last_dim_forward": ("softmax_rows_kernel<float, false", ["sparseswin3d_amd/csrc/softmax.hip"]),
     "softmax_last_dim_backward": ("softmax_rows_kernel<float, true", ["sparseswin3d_amd/csrc/softmax.hip"]),
     "resident bias table grad": ("rpb_table_partial_kernel", ["sparseswin3d_amd/csrc/fused_attention.hip"]),
-    "fused S=QK^T+bias+mask": ("fused_sq_kernel<float, true", ["sparseswin3d_amd/csrc/fused_attention.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
-    "fused dP=dO V^T": ("fused_sq_kernel<float, false", ["sparseswin3d_amd/csrc/fused_attention.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
+    "fused S=QK^T+bias+mask": ("fused_sq_kernel<float, 1", ["sparseswin3d_amd/csrc/fused_attention.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
+    "fused dS=P(dO V^T - dO.O)": ("fused_sq_kernel<float, 2", ["sparseswin3d_amd/csrc/fused_attention.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
     "fused dV=P^T dO": ("fused_tok_kernel<float, true", ["sparseswin3d_amd/csrc/fused_attention.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
     "fused O=PV": ("fused_tok_kernel<float, false", ["sparseswin3d_amd/csrc/fused_attention.hip", "sparseswin3d_amd/csrc/mfma_block.hpp"]),
     "fused softmax fwd (rows from the group table)": ("group_softmax_kernel<false", ["sparseswin3d_amd/csrc/fused_attention.hip"]),
-    "fused softmax bwd (rows from the group table)": ("group_softmax_kernel<true", ["sparseswin3d_amd/csrc/fused_attention.hip"]),
 }
 
 
@@ -473,9 +472,10 @@ def kernel_table(wl, reps=20, only=None):
             ("fused S=QK^T+bias+mask", lambda: F._tokens_to_sq(tp, dt, True, qkv_c, 3 * D, 0, qkv_c, 3 * D, D, hd, 0.17, bias, mask, s_f, None), 8 * E + 4 * A, 1),
             ("fused softmax fwd (rows from the group table)", lambda: F._group_softmax(tp, False, s_f, None, p_f), 8 * A, 1),
             ("fused O=PV", lambda: F._sq_to_tokens(tp, dt, False, p_val, qkv_c, 3 * D, 2 * D, out_f, D, 0, hd, 1.0), 4 * A + 8 * E, 1),
-            ("fused dP=dO V^T", lambda: F._tokens_to_sq(tp, dt, False, out_f, D, 0, qkv_c, 3 * D, 2 * D, hd, 1.0, None, None, s_f, None), 8 * E + 4 * A, 1),
+            ("fused dS=P(dO V^T - dO.O)", lambda: F._score_grad(tp, dt, out_f, D, 0, qkv_c, 3 * D, 2 * D, out_f, D, 0, hd, p_val, s_f), 12 * E + 8 * A, 1),
+            ("fused dP=dO V^T (the product alone)", lambda: F._tokens_to_sq(tp, dt, False, out_f, D, 0, qkv_c, 3 * D, 2 * D, hd, 1.0, None, None, s_f, None), 8 * E + 4 * A, 0),
             ("fused dV=P^T dO", lambda: F._sq_to_tokens(tp, dt, True, p_val, out_f, D, 0, dqkv, 3 * D, 2 * D, hd, 1.0), 4 * A + 8 * E, 1),
-            ("fused softmax bwd (rows from the group table)", lambda: F._group_softmax(tp, True, p_val, g_s, p_f), 12 * A, 1),
+            ("fused softmax bwd (rows from the group table; alone)", lambda: F._group_softmax(tp, True, p_val, g_s, p_f), 12 * A, 0),
             ("fused dQ=dS K", lambda: F._sq_to_tokens(tp, dt, False, g_s, qkv_c, 3 * D, D, dqkv, 3 * D, 0, hd, 0.17), 4 * A + 8 * E, 1),
             ("fused dK=dS^T Q", lambda: F._sq_to_tokens(tp, dt, True, g_s, qkv_c, 3 * D, 0, dqkv, 3 * D, D, hd, 0.17), 4 * A + 8 * E, 1),
             ("fused bias table grad", lambda: _lib.check(lib.sswin_bias_table_grad(ptr(tp.plan), tp.g_cap, tp.G, ptr(tp.tokens), tp.N, H, b["n"], ptr(ti.code), ti.offset0, n_table, ptr(g_s), ptr(d_table), ptr(tg_ws), tg_bytes, stream)), 4 * A, 1),

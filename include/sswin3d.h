@@ -351,6 +351,17 @@ int sswin_fused_sq_to_tokens(int dtype, int a_kmajor, const int32_t* plan, int64
                              const void* b_base, int64_t b_stride, int b_col0, void* o_base,
                              int64_t o_stride, int o_col0, float scale_out, void* stream);
 
+/* Gradient of the scores from the gradient of the attention output, in one launch:
+ *   ds[g][i][j] = p[g][i][j] * (sum_ch dO[token i, ch] * V[token j, ch] - D_i),   D_i = sum_ch dO[token i, ch] * O[token i, ch],
+ * which is the product dP = dO V^T (swin3d_base.py:119-134) followed by the softmax backward (ops.cu:169-194):
+ * sum_j p_ij dP_ij = dO_i . O_i because O = P V, so dP is never written.  dO, V, O: token tensors as above; p: the
+ * attention matrix of the forward pass, ds: fp32 sq arrays.  c_max <= 384.  Token tensors that a 32-bit offset cannot
+ * cover run the product and sswin_group_softmax one after the other instead.  Asynchronous. */
+int sswin_fused_score_grad(int dtype, const int32_t* plan, int64_t g_cap, int64_t G, const int32_t* tokens,
+                           int64_t N, int H, int hd, int c_max, const void* do_base, int64_t do_stride,
+                           int do_col0, const void* v_base, int64_t v_stride, int v_col0, const void* o_base,
+                           int64_t o_stride, int o_col0, const float* p, float* ds, void* stream);
+
 /* The sparse row softmax over the rows of the groups' [c x c] blocks, forward (backward == 0: out = softmax of
  * x_or_y, grad ignored) or backward (out = y (g - sum_j g_j y_j) with y = x_or_y, g = grad).  The arithmetic of
  * softmax_last_dim_forward / _backward (sparse_swin/ops.cu:128-194: zero-initialised maximum, + 1e-8 in the

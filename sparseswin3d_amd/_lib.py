@@ -64,6 +64,8 @@ SIGNATURES = {
                                         _vp, _i64, _i32, C.c_float, _vp, _i32, _vp, _i32, _vp, _vp, _vp]),
     "sswin_fused_sq_to_tokens": (_i32, [_i32, _i32, _vp, _i64, _i64, _vp, _i64, _i32, _i32, _vp, _vp, _i64, _i32,
                                         _vp, _i64, _i32, C.c_float, _vp]),
+    "sswin_fused_score_grad": (_i32, [_i32, _vp, _i64, _i64, _vp, _i64, _i32, _i32, _i32, _vp, _i64, _i32, _vp, _i64, _i32,
+                                      _vp, _i64, _i32, _vp, _vp, _vp]),
     "sswin_group_softmax": (_i32, [_i32, _vp, _i64, _i64, _i64, _i32, _i32, _vp, _vp, _vp, _vp]),
     "sswin_fused_bias_grad_workspace_bytes": (_sz, [_i64, _i32, _i32]),
     "sswin_fused_bias_grad": (_i32, [_vp, _i64, _i64, _vp, _i64, _i32, _i32, _vp, _vp, _vp, _sz, _vp]),
@@ -91,7 +93,7 @@ SIGNATURES = {
                                                _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i64, _i32, _vp, _i32, _vp]),
 }
 
-ABI_VERSION = 28
+ABI_VERSION = 29
 _lib = None
 
 # A list turns on timing of the library's launches: every call that takes a stream is bracketed by events on that

@@ -459,15 +459,21 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t head_rows(const TokenTensor& t
 
 // ------------------------------------------------------------------------------------------
 // tokens x tokens -> sq :  out[i, j] = sum_ch A[token i, ch] * B[token j, ch]   (K = hd)
-//   EPI = true : S = scale*acc + bias[h, pos_i, pos_j] + (mask region differs ? -100 : 0), row ids
-//   EPI = false: plain product (dP = dO V^T)
+//   EPI = SQ_SCORES: S = scale*acc + bias[h, pos_i, pos_j] + (mask region differs ? -100 : 0), row ids
+//   EPI = SQ_PLAIN : plain product (dP = dO V^T)
+//   EPI = SQ_SCORE_GRAD: dS = P (dO V^T - D) with D_i = dO_i . O_i (= sum_j P_ij dP_ij, since O = P V): the softmax
+//         backward (ops.cu:169-194) as the epilogue of the product, so dP never reaches memory and no softmax
+//         launch follows.  A = dO, B = V, tc = O (rows like A's), `bias` = P (the sq array of the forward pass).
 // Rows of tokens behind the window's last one are read as zeros and their results dropped by the bounds checks
 // of the buffer descriptors (mfma_block.hpp).
 // ------------------------------------------------------------------------------------------
-template <typename T, bool EPI>
+enum { SQ_PLAIN = 0, SQ_SCORES = 1, SQ_SCORE_GRAD = 2 };
+
+template <typename T, int EPI>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void fused_sq_kernel(FusedGroups gt, const int32_t* __restrict__ order,
                                                        const int32_t* __restrict__ tok_pos, int H, int hd,
-                                                       TokenTensor ta, TokenTensor tb, uint32_t a_span, uint32_t b_span, float scale_a,
+                                                       TokenTensor ta, TokenTensor tb, TokenTensor tc, uint32_t a_span, uint32_t b_span,
+                                                       uint32_t c_span, float scale_a,
                                                        const float* __restrict__ bias, int n,
                                                        const int8_t* __restrict__ mask, int n_mask_windows,
                                                        float* __restrict__ out, int32_t* __restrict__ row_ids) {
@@ -475,10 +481,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
     const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const int half = lane >> 5, l32 = lane & 31;
     const int64_t g0 = (int64_t)blockIdx.x * FUSED_GROUPS_PER_WG;
-    const GroupLanes gl = load_groups<EPI>(gt, g0, lane);
+    const GroupLanes gl = load_groups<EPI == SQ_SCORES>(gt, g0, lane);
     const TaskSet ts = make_tasks(gl, true, hd);
     const int total = ts.first[FUSED_GROUPS_PER_WG];
-    const uint32_t a_pitch = (uint32_t)ta.stride * ES, b_pitch = (uint32_t)tb.stride * ES;
+    const uint32_t a_pitch = (uint32_t)ta.stride * ES, b_pitch = (uint32_t)tb.stride * ES, c_pitch = (uint32_t)tc.stride * ES;
 
     for (int t = wave + 4 * (int)blockIdx.y; t < total; t += 4 * (int)gridDim.y) {   // gridDim.y workgroups share the groups' blocks
         const Task k = locate_task(ts, gl, t, true, hd);
@@ -490,7 +496,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         // epilogue inputs: one load per lane (row token, column token); the 16 rows a lane stores
         // are fetched from the row lanes with cross-lane reads in the epilogue
         int pos_a = 0, pos_j = 0, m_a = 0, m_j = 0;
-        if (EPI) {
+        if (EPI == SQ_SCORES) {
             pos_a = tok_pos[Tk + (a_in ? i_a : c - 1)];
             pos_j = tok_pos[Tk + (b_in ? j_b : c - 1)];
             if (mask) {
@@ -502,6 +508,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         const __amdgpu_buffer_rsrc_t ra = head_rows<T>(ta, h, hd, a_span), rb = head_rows<T>(tb, h, hd, b_span);
         const uint32_t row_a = a_in ? (uint32_t)vox_i * a_pitch : BUF_OUTSIDE;
         const uint32_t row_b = b_in ? (uint32_t)vox_j * b_pitch : BUF_OUTSIDE;
+        // entry (i, j) of the block at byte offset (i * c + j) * 4: rows behind the last one are outside by themselves
+        const uint32_t o0 = b_in ? (uint32_t)((bi * 32 + 4 * half) * c + j_b) * 4u : BUF_OUTSIDE;
+        // score gradient: D collects dO_i . O_i over this lane's channels
+        float d_part = 0.f;
+        __amdgpu_buffer_rsrc_t rc = ra;
+        uint32_t row_c = BUF_OUTSIDE;
+        if (EPI == SQ_SCORE_GRAD) {
+            rc = head_rows<T>(tc, h, hd, c_span);
+            row_c = a_in ? (uint32_t)vox_i * c_pitch : BUF_OUTSIDE;
+        }
 
         f32x16 acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
         for (int kc = 0; kc < hd; kc += 32) {
@@ -525,6 +541,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
                     b[s] = buf_load1<T>(rb, s < left ? row_b + ch0 + ES * s : BUF_OUTSIDE);
                 }
             }
+            if (EPI == SQ_SCORE_GRAD) {
+                float o[16];
+                if (chunk == 32) {
+                    buf_load_run<T, 16>(rc, row_c + ch0, o);
+                } else if (chunk == 16) {
+                    buf_load_run<T, 8>(rc, row_c + ch0, o);
+                } else {
+#pragma unroll
+                    for (int s = 0; s < 16; ++s) o[s] = buf_load1<T>(rc, s < left ? row_c + ch0 + ES * s : BUF_OUTSIDE);
+                }
+#pragma unroll
+                for (int s = 0; s < 16; ++s)
+                    if (s < kh) d_part = fmaf(a[s], o[s], d_part);
+            }
             if (scale_a != 1.0f) {
 #pragma unroll
                 for (int s = 0; s < 16; ++s) a[s] *= scale_a;
@@ -534,11 +564,24 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
                 if (s < kh) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a[s], b[s], acc, 0, 0, 0);
         }
 
-        {
-            // entry (i, j) of the block at byte offset (i * c + j) * 4: rows behind the last one are outside by themselves
+        if constexpr (EPI == SQ_SCORE_GRAD) {
+            // the block of P (requested behind the matrix steps: sixteen more registers in flight beside the operands
+            // would spill); D of row i_a: the two lane halves hold the two halves of its channels
+            const __amdgpu_buffer_rsrc_t rp = buf_of(bias + k.sq, (uint32_t)(c * c) * 4u);
+            float pv[16];
+#pragma unroll
+            for (int r = 0; r < 16; ++r) pv[r] = buf_load1<float>(rp, o0 + (uint32_t)((8 * (r >> 2) + (r & 3)) * c) * 4u);
+            const float d_row = d_part + __shfl_xor(d_part, 32, 64);
+            const __amdgpu_buffer_rsrc_t ro = buf_of(out + k.sq, (uint32_t)(c * c) * 4u);
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const float d_r = __shfl(d_row, acc_row(r, half), 64);
+                const float v = acc[r];
+                buf_store1<float>(ro, o0 + (uint32_t)((8 * (r >> 2) + (r & 3)) * c) * 4u, pv[r] * (v - d_r));
+            }
+        } else {
             const __amdgpu_buffer_rsrc_t ro = buf_of(out + k.sq, (uint32_t)(c * c) * 4u);
             const __amdgpu_buffer_rsrc_t rr = buf_of(row_ids ? row_ids + k.sq : nullptr, row_ids ? (uint32_t)(c * c) * 4u : 0u);
-            const uint32_t o0 = b_in ? (uint32_t)((bi * 32 + 4 * half) * c + j_b) * 4u : BUF_OUTSIDE;
             const float* brow = EPI ? bias + (int64_t)h * n * n + pos_j : nullptr;
             const int rid0 = H * Tk + h * c + bi * 32 + 4 * half;
             // bias values of the 16 rows are gathered before any of them is used, so that the
@@ -1301,27 +1344,36 @@ static bool rows_fit_descriptor(const TokenTensor& t, int64_t N, int hd, uint32_
     return !(e && e[0] == '1');
 }
 
+// epi: SQ_PLAIN, SQ_SCORES or SQ_SCORE_GRAD (then tc = O rows and bias = P).  *fused_done says whether the epilogue
+// ran inside the product (always for the first two; the score gradient only on the descriptor kernel: otherwise
+// the plain product is written and the caller runs the softmax backward over it).
 template <typename T>
-static int launch_sq(bool epi, const FusedGroups& gt, int64_t N, double mean_c, const int32_t* order, const int32_t* tok_pos, int H, int hd,
-                     const TokenTensor& ta, const TokenTensor& tb, float scale_a, const float* bias, int n,
-                     const int8_t* mask, int nmw, float* out, int32_t* row_ids, hipStream_t s) {
+static int launch_sq(int epi, const FusedGroups& gt, int64_t N, double mean_c, const int32_t* order, const int32_t* tok_pos, int H, int hd,
+                     const TokenTensor& ta, const TokenTensor& tb, const TokenTensor& tc, float scale_a, const float* bias, int n,
+                     const int8_t* mask, int nmw, float* out, int32_t* row_ids, hipStream_t s, bool* fused_done) {
     const dim3 grid((unsigned)((gt.G + FUSED_GROUPS_PER_WG - 1) / FUSED_GROUPS_PER_WG),
                     block_task_slices(mean_c, hd, true, FUSED_GROUPS_PER_WG));
-    uint32_t a_span, b_span;
+    uint32_t a_span, b_span, c_span = 0;
     const bool fit_a = rows_fit_descriptor<T>(ta, N, hd, &a_span), fit_b = rows_fit_descriptor<T>(tb, N, hd, &b_span);
-    if (fit_a && fit_b) {
-        if (epi)
-            hipLaunchKernelGGL((fused_sq_kernel<T, true>), grid, dim3(256), 0, s, gt, order, tok_pos, H, hd, ta,
-                               tb, a_span, b_span, scale_a, bias, n, mask, nmw, out, row_ids);
+    const bool fit_c = epi != SQ_SCORE_GRAD || rows_fit_descriptor<T>(tc, N, hd, &c_span);
+    if (fused_done) *fused_done = true;
+    if (fit_a && fit_b && fit_c) {
+        if (epi == SQ_SCORES)
+            hipLaunchKernelGGL((fused_sq_kernel<T, SQ_SCORES>), grid, dim3(256), 0, s, gt, order, tok_pos, H, hd, ta,
+                               tb, tc, a_span, b_span, c_span, scale_a, bias, n, mask, nmw, out, row_ids);
+        else if (epi == SQ_SCORE_GRAD)
+            hipLaunchKernelGGL((fused_sq_kernel<T, SQ_SCORE_GRAD>), grid, dim3(256), 0, s, gt, order, tok_pos, H, hd, ta,
+                               tb, tc, a_span, b_span, c_span, scale_a, bias, n, mask, nmw, out, row_ids);
         else
-            hipLaunchKernelGGL((fused_sq_kernel<T, false>), grid, dim3(256), 0, s, gt, order, tok_pos, H, hd, ta,
-                               tb, a_span, b_span, scale_a, bias, n, mask, nmw, out, row_ids);
-    } else if (epi) {
+            hipLaunchKernelGGL((fused_sq_kernel<T, SQ_PLAIN>), grid, dim3(256), 0, s, gt, order, tok_pos, H, hd, ta,
+                               tb, tc, a_span, b_span, c_span, scale_a, bias, n, mask, nmw, out, row_ids);
+    } else if (epi == SQ_SCORES) {
         hipLaunchKernelGGL((fused_sq_wide_kernel<T, true>), grid, dim3(256), 0, s, gt, order, tok_pos, H, hd, ta,
                            tb, scale_a, bias, n, mask, nmw, out, row_ids);
     } else {
+        if (fused_done) *fused_done = epi != SQ_SCORE_GRAD;
         hipLaunchKernelGGL((fused_sq_wide_kernel<T, false>), grid, dim3(256), 0, s, gt, order, tok_pos, H, hd, ta,
-                           tb, scale_a, bias, n, mask, nmw, out, row_ids);
+                           tb, scale_a, nullptr, n, nullptr, 0, out, nullptr);
     }
     return launch_ok("fused tokens->sq product");
 }
@@ -1539,9 +1591,9 @@ int sswin_fused_tokens_to_sq(int dtype, int epilogue, const int32_t* plan, int64
     const int32_t* tok_pos = tokens + 3 * N;
     const double mean_c = (double)N * H / (double)G;          // every voxel is a token of one window, in each of its H groups
     switch (dtype) {
-        case SSWIN_F32: return launch_sq<float>(epilogue, gt, N, mean_c, order, tok_pos, H, hd, ta, tb, scale_a, bias, n, mask, n_mask_windows, out, row_ids, s);
-        case SSWIN_F16: return launch_sq<__half>(epilogue, gt, N, mean_c, order, tok_pos, H, hd, ta, tb, scale_a, bias, n, mask, n_mask_windows, out, row_ids, s);
-        case SSWIN_BF16: return launch_sq<__hip_bfloat16>(epilogue, gt, N, mean_c, order, tok_pos, H, hd, ta, tb, scale_a, bias, n, mask, n_mask_windows, out, row_ids, s);
+        case SSWIN_F32: return launch_sq<float>(epilogue ? SQ_SCORES : SQ_PLAIN, gt, N, mean_c, order, tok_pos, H, hd, ta, tb, ta, scale_a, bias, n, mask, n_mask_windows, out, row_ids, s, nullptr);
+        case SSWIN_F16: return launch_sq<__half>(epilogue ? SQ_SCORES : SQ_PLAIN, gt, N, mean_c, order, tok_pos, H, hd, ta, tb, ta, scale_a, bias, n, mask, n_mask_windows, out, row_ids, s, nullptr);
+        case SSWIN_BF16: return launch_sq<__hip_bfloat16>(epilogue ? SQ_SCORES : SQ_PLAIN, gt, N, mean_c, order, tok_pos, H, hd, ta, tb, ta, scale_a, bias, n, mask, n_mask_windows, out, row_ids, s, nullptr);
         default: return fail("fused_tokens_to_sq: unsupported token dtype %d", dtype);
     }
 }
@@ -1580,6 +1632,31 @@ int sswin_group_softmax(int backward, const int32_t* plan, int64_t g_cap, int64_
     else
         hipLaunchKernelGGL((group_softmax_kernel<false>), grid, dim3(256), 0, s, gt, x_or_y, grad, out);
     return launch_ok("group softmax");
+}
+
+int sswin_fused_score_grad(int dtype, const int32_t* plan, int64_t g_cap, int64_t G, const int32_t* tokens, int64_t N,
+                           int H, int hd, int c_max, const void* do_base, int64_t do_stride, int do_col0,
+                           const void* v_base, int64_t v_stride, int v_col0, const void* o_base, int64_t o_stride,
+                           int o_col0, const float* p, float* ds, void* stream) {
+    SSWIN_CHECK(G >= 0 && G <= g_cap && N >= 0 && H > 0 && hd > 0, "fused_score_grad: bad sizes");
+    if (G == 0) return 0;
+    SSWIN_CHECK(plan && tokens && do_base && v_base && o_base && p && ds, "fused_score_grad: null pointer");
+    SSWIN_CHECK(c_max > 0 && c_max <= 384, "fused_score_grad: windows of %d tokens are not supported (384 at most)", c_max);
+    const FusedGroups gt = groups_of(plan, g_cap, G);
+    const TokenTensor ta{do_base, do_stride, do_col0}, tb{v_base, v_stride, v_col0}, tc{o_base, o_stride, o_col0};
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    const double mean_c = (double)N * H / (double)G;
+    bool done = false;
+    int rc;
+    switch (dtype) {
+        case SSWIN_F32: rc = launch_sq<float>(SQ_SCORE_GRAD, gt, N, mean_c, tokens, tokens + 3 * N, H, hd, ta, tb, tc, 1.0f, p, 0, nullptr, 0, ds, nullptr, s, &done); break;
+        case SSWIN_F16: rc = launch_sq<__half>(SQ_SCORE_GRAD, gt, N, mean_c, tokens, tokens + 3 * N, H, hd, ta, tb, tc, 1.0f, p, 0, nullptr, 0, ds, nullptr, s, &done); break;
+        case SSWIN_BF16: rc = launch_sq<__hip_bfloat16>(SQ_SCORE_GRAD, gt, N, mean_c, tokens, tokens + 3 * N, H, hd, ta, tb, tc, 1.0f, p, 0, nullptr, 0, ds, nullptr, s, &done); break;
+        default: return fail("fused_score_grad: unsupported token dtype %d", dtype);
+    }
+    if (rc != 0 || done) return rc;
+    // token tensors beyond the reach of a buffer descriptor: ds holds dP now, the softmax backward runs over it in place
+    return sswin_group_softmax(1, plan, g_cap, G, N, H, c_max, p, ds, ds, stream);
 }
 
 static int bias_grad_slices(int64_t windows, int H) {

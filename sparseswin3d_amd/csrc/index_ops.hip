@@ -712,7 +712,7 @@ using namespace sswin;
 extern "C" {
 
 const char* sswin_last_error(void) { return error_buffer(); }
-int sswin_abi_version(void) { return 28; }
+int sswin_abi_version(void) { return 29; }
 
 int sswin_calibration_copy(void* dst, const void* src, int64_t bytes, void* stream) {
     SSWIN_CHECK(bytes >= 0 && bytes % 16 == 0, "calibration_copy: size must be a multiple of 16 bytes");

@@ -162,6 +162,13 @@ def _sq_to_tokens(tp, dtype, a_kmajor, sq, b, b_stride, b_col0, o, o_stride, o_c
         _ptr(sq), _ptr(b), b_stride, b_col0, _ptr(o), o_stride, o_col0, C.c_float(scale), stream))
 
 
+def _score_grad(tp, dtype, d_o, do_stride, do_col0, v, v_stride, v_col0, o, o_stride, o_col0, hd, p, ds):
+    """dS = P (dO V^T - D), D_i = dO_i . O_i: the product dP and the softmax backward in one launch."""
+    _lib.check(_lib.load().sswin_fused_score_grad(
+        _DTYPE_CODE[dtype], _ptr(tp.plan), tp.g_cap, tp.G, _ptr(tp.tokens), tp.N, tp.H, hd, tp.c_max, _ptr(d_o), do_stride,
+        do_col0, _ptr(v), v_stride, v_col0, _ptr(o), o_stride, o_col0, _ptr(p), _ptr(ds), _lib.stream_handle(tp.device)))
+
+
 def _group_softmax(tp, backward, x_or_y, grad, out):
     """Row softmax (or its backward) over the [c x c] blocks of the plan's groups; ``out`` may be one of the inputs."""
     _lib.check(_lib.load().sswin_group_softmax(
@@ -226,14 +233,14 @@ class _FusedWindowAttention(Function):
             _group_softmax(tp, False, p, None, p)                  # S -> P in place, rows from the group table
             out = torch.empty((N, D), dtype=dtype, device=d)
             _sq_to_tokens(tp, dtype, False, p, qkv, 3 * D, 2 * D, out, D, 0, hd, 1.0)
-        ctx.save_for_backward(qkv, p)
+        ctx.save_for_backward(qkv, p, out)
         ctx.tp, ctx.scale, ctx.bias_meta, ctx.table_index = tp, scale, (bias.dtype, bias.shape), table_index
         return out
 
     @staticmethod
     @once_differentiable
     def backward(ctx, grad_out):
-        qkv, p = ctx.saved_tensors
+        qkv, p, out = ctx.saved_tensors
         tp, scale = ctx.tp, ctx.scale
         N, _, H, hd = qkv.shape
         D = H * hd
@@ -244,10 +251,9 @@ class _FusedWindowAttention(Function):
         with _lib.on_device(d):
             d_qkv = torch.empty_like(qkv)
             d_s = torch.empty(tp.A, dtype=torch.float32, device=d)
-            # dP = dO V^T ; dV = P^T dO
-            _tokens_to_sq(tp, dtype, False, grad_out, D, 0, qkv, 3 * D, 2 * D, hd, 1.0, None, None, d_s, None)
+            # dS = P (dO V^T - dO . O): the softmax backward is the epilogue of the product ; dV = P^T dO
+            _score_grad(tp, dtype, grad_out, D, 0, qkv, 3 * D, 2 * D, out, D, 0, hd, p, d_s)
             _sq_to_tokens(tp, dtype, True, p, grad_out, D, 0, d_qkv, 3 * D, 2 * D, hd, 1.0)
-            _group_softmax(tp, True, p, d_s, d_s)                  # dP -> dS in place
             # dQ = scale * dS K ; dK = scale * dS^T Q
             _sq_to_tokens(tp, dtype, False, d_s, qkv, 3 * D, D, d_qkv, 3 * D, 0, hd, scale)
             _sq_to_tokens(tp, dtype, True, d_s, qkv, 3 * D, 0, d_qkv, 3 * D, D, hd, scale)
