@@ -856,7 +856,9 @@ def trace_summary(dirs, out_name, command):
         if not paths:
             sys.exit(f"no *kernel_stats.csv under {d}")
         rows = list(csv.DictReader(open(paths[0])))
-        bwd = sum(int(r["Calls"]) for r in rows if "_bwd_all_kernel" in r["Name"])
+        # one backward launch per attention call: the resident kernels' or, on the fused path, the score gradient's
+        bwd = sum(int(r["Calls"]) for r in rows if "_bwd_all_kernel" in r["Name"]) or \
+            sum(int(r["Calls"]) for r in rows if "fused_sq_kernel<" in r["Name"] and ", 2>" in r["Name"])
         steps = max(bwd // 2, 1)
         if bwd == 0:                                 # the forward-only encoder: four attention launches per pass
             steps = max(sum(int(r["Calls"]) for r in rows if "_fwd_kernel<" in r["Name"] and "wattn" in r["Name"]) // 4, 1)
