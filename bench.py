@@ -478,7 +478,7 @@ def kernel_table(wl, reps=20, only=None):
             ("fused softmax bwd (rows from the group table; alone)", lambda: F._group_softmax(tp, True, p_val, g_s, p_f), 12 * A, 0),
             ("fused dQ=dS K", lambda: F._sq_to_tokens(tp, dt, False, g_s, qkv_c, 3 * D, D, dqkv, 3 * D, 0, hd, 0.17), 4 * A + 8 * E, 1),
             ("fused dK=dS^T Q", lambda: F._sq_to_tokens(tp, dt, True, g_s, qkv_c, 3 * D, 0, dqkv, 3 * D, D, hd, 0.17), 4 * A + 8 * E, 1),
-            ("fused bias table grad", lambda: _lib.check(lib.sswin_bias_table_grad(ptr(tp.plan), tp.g_cap, tp.G, ptr(tp.tokens), tp.N, H, b["n"], ptr(ti.code), ti.offset0, n_table, ptr(g_s), ptr(d_table), ptr(tg_ws), tg_bytes, stream)), 4 * A, 1),
+            ("fused bias table grad", lambda: F._bias_gradient(tp, H, g_s, (torch.float32, (n_table, H)), ti), 4 * A, 1),
             ("fused bias grad [H,n,n]", lambda: _lib.check(lib.sswin_fused_bias_grad(ptr(tp.plan), tp.g_cap, tp.G, ptr(tp.tokens), tp.N, H, b["n"], ptr(g_s), ptr(dbias), ptr(bg_ws), bg_bytes, stream)), 4 * A, 0),
         ]
 
@@ -524,9 +524,19 @@ def kernel_table(wl, reps=20, only=None):
     tg_bytes = lib.sswin_bias_table_grad_workspace_bytes(tp.G, H, n_table)
     tg_ws = torch.empty(int(tg_bytes), dtype=torch.uint8, device=dev)
 
-    def r_table_grad():
+    def r_table_grad_groups():
         _lib.check(lib.sswin_bias_table_grad(ptr(tp.plan), tp.g_cap, tp.G, ptr(tp.tokens), tp.N, H, b["n"], ptr(ti.code),
                                              ti.offset0, n_table, ptr(ds_r), ptr(d_table), ptr(tg_ws), tg_bytes, stream))
+
+    # what the module calls when every window holds at most 128 tokens: the batches dealt from the task descriptors
+    by_tasks = tp.tasks is not None and b["n"] <= 128 and sum(tp.bucket_counts) == tp.G
+
+    def r_table_grad():
+        if not by_tasks:
+            return r_table_grad_groups()
+        _lib.check(lib.sswin_bias_table_grad_tasks(ptr(tp.tasks), tp.g_cap, tp.bucket_counts, tp.G, ptr(tp.tokens), tp.N, H, b["n"],
+                                                   ptr(ti.code), ti.offset0, n_table, ptr(ds_r), ptr(d_table), ptr(tg_ws), tg_bytes,
+                                                   stream))
 
     resident_ok = hd == 32 and int(tp.c_max) <= 128       # otherwise the module runs the fused path
     if resident_ok:
@@ -543,6 +553,7 @@ def kernel_table(wl, reps=20, only=None):
         ("resident backward dQ, all groups", r_bwd(1), 24 * Er + 4 * H * N, 0),
         ("resident backward dK,dV,dS only", r_bwd(2), 28 * Er + 4 * A + 4 * H * N, 0),
         ("resident bias table grad", r_table_grad, 4 * A, 1),
+        ("bias table grad, batches from the group table", r_table_grad_groups, 4 * A, 0),
     ]
     if code == 0:
         r_entries.append(("resident bias grad [H,n,n]", lambda: _lib.check(lib.sswin_fused_bias_grad(

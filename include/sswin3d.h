@@ -396,6 +396,16 @@ int sswin_bias_table_grad(const int32_t* plan, int64_t g_cap, int64_t G, const i
                           int64_t N, int H, int n, const int32_t* code, int offset0, int table_rows,
                           const float* ds, float* d_table, void* ws, size_t ws_bytes, void* stream);
 
+/* The same gradient with the batches taken from the task descriptors of a token plan (`tasks`, `bucket_counts`: what
+ * sswin_window_attention_forward takes) instead of its group table: the descriptors list the groups by their number
+ * of 32-token tiles, so the 32 x 32 batches of dS can be dealt to the wavefronts evenly.  For plans whose windows all
+ * hold at most 128 tokens (the sum of bucket_counts equals G); same workspace, same result up to the order of the
+ * fp32 sums (fixed from run to run).  No counterpart in the reference (autograd's index_add, swin3d_base.py:557-566). */
+int sswin_bias_table_grad_tasks(const int32_t* tasks, int64_t g_cap, const int64_t* bucket_counts, int64_t G,
+                                const int32_t* tokens, int64_t N, int H, int n, const int32_t* code,
+                                int offset0, int table_rows, const float* ds, float* d_table, void* ws,
+                                size_t ws_bytes, void* stream);
+
 /* Column sums (fp32) of a dense [N, P] matrix of `dtype` (fp32 / fp16 / bf16; P a multiple of 4,
  * rows contiguous): the bias gradient of the qkv / proj nn.Linear (swin3d_base.py:606-610;
  * autograd's grad_out.sum(0)).  Fixed summation order.  Asynchronous (N == 0 records a memset). */

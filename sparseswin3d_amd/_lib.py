@@ -74,6 +74,8 @@ SIGNATURES = {
     "sswin_bias_from_table": (_i32, [_vp, _i32, _i32, _vp, _i32, _i32, _vp, _vp]),
     "sswin_bias_table_grad_workspace_bytes": (_sz, [_i64, _i32, _i32]),
     "sswin_bias_table_grad": (_i32, [_vp, _i64, _i64, _vp, _i64, _i32, _i32, _vp, _i32, _i32, _vp, _vp, _vp, _sz, _vp]),
+    "sswin_bias_table_grad_tasks": (_i32, [_vp, _i64, _vp, _i64, _vp, _i64, _i32, _i32, _vp, _i32, _i32, _vp, _vp, _vp, _sz,
+                                           _vp]),
     "sswin_tall_linear_supported": (_i32, [_i32, _i32]),
     "sswin_tall_linear_forward": (_i32, [_vp, _i64, _i32, _vp, _vp, _i32, _vp, _vp]),
     "sswin_tall_linear_input_grad_supported": (_i32, [_i32, _i32]),

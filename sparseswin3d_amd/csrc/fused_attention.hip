@@ -1134,7 +1134,25 @@ constexpr int RPBT_U = 16;                                      // steps of a ba
 // batch (its entries of dS, the positions of its rows and columns) follow from the window's header, so a
 // cursor runs two batches ahead of the adds and the batches wait in three register slots taken in turn (a
 // slot is never copied: a copy would wait for its loads).
-__global__ __launch_bounds__(256) void rpb_table_partial_kernel(FusedGroups gt, const int32_t* __restrict__ tok_pos,
+//
+// Which batches a wavefront adds (BY_TASKS):
+//   false: from the group table.  A slice of wavefronts takes every wslices-th window and deals the batches of its
+//          windows among its rsplit members (each member walks over all windows of the slice).
+//   true:  from the task descriptors of a token plan, which list the groups by their number of 32-token tiles
+//          (fused TokenPlan, windows of at most 128 tokens).  The batches of a head, numbered bucket by bucket (16, 9,
+//          4 or 1 per group), are dealt to the head's wavefronts in turn: wavefront q adds the batches q, q + Q, ...,
+//          so every wavefront adds the same number of batches to within one (the slices of the group table differ by
+//          the sizes of the windows that fall to them: 1.6 x between the fullest slice and the mean on a room of
+//          112 000 voxels), and nothing is walked: lane l decodes the wavefront's l-th batch and loads its descriptor.
+struct BatchList {
+    const int4* tasks;       // [4][g_cap] descriptors {T, c | head << 8, window, sq}, bucket b = groups of b + 1 tiles
+    int64_t g_cap;
+    int first[4];            // batches of a head in front of bucket b (buckets in the order 3, 2, 1, 0)
+    int total;               // batches of a head
+};
+
+template <bool BY_TASKS>
+__global__ __launch_bounds__(256) void rpb_table_partial_kernel(FusedGroups gt, BatchList bl, const int32_t* __restrict__ tok_pos,
                                                                 int H, const int32_t* __restrict__ code, int n,
                                                                 int offset0, int rows, int rows_pad,
                                                                 const float* __restrict__ ds, int64_t windows,
@@ -1159,15 +1177,35 @@ __global__ __launch_bounds__(256) void rpb_table_partial_kernel(FusedGroups gt, 
     // A slice takes every wslices-th window (crowded windows are neighbours in plan order, so dealing them out
     // evens the load); the batches of its windows are dealt to the rsplit wavefronts of the slice.
     // The headers of 64 windows of the slice at a time sit in the lanes (lane l: the l-th of them).
-    int hw_c = 0, hw_T = 0, hw_sq = 0;
+    int hw_c = 0, hw_T = 0, hw_sq = 0, hw_ch = 0, hw_ib = 0;
     auto load_headers = [&](int m_first) __attribute__((always_inline)) {
-        const int64_t k = ws + ((int64_t)m_first + lane) * wslices;
         hw_c = 0;
-        if (k < windows) {
-            const int64_t g = k * H + h;
-            hw_c = gt.c[g];
-            hw_T = gt.T[g];
-            hw_sq = gt.sq[g];
+        if constexpr (BY_TASKS) {
+            // batch number (m_first + lane) * slices + sl of head h -> bucket, group inside it, chunk and row block
+            const int64_t f64 = ((int64_t)m_first + lane) * slices + sl;
+            if (f64 < bl.total) {
+                const int f = (int)f64;
+                int b = 3, r = f - bl.first[3];
+                if (f >= bl.first[2]) { b = 2; r = f - bl.first[2]; }
+                if (f >= bl.first[1]) { b = 1; r = f - bl.first[1]; }
+                if (f >= bl.first[0]) { b = 0; r = f - bl.first[0]; }
+                const int nb = b + 1, per = nb * nb;
+                const int gi = r / per, rem = r - gi * per;
+                const int4 d = bl.tasks[(int64_t)b * bl.g_cap + (int64_t)gi * H + h];
+                hw_T = d.x;
+                hw_c = d.y & 0xff;
+                hw_sq = d.w;
+                hw_ib = (rem / nb) * 32;
+                hw_ch = rem - (rem / nb) * nb;
+            }
+        } else {
+            const int64_t k = ws + ((int64_t)m_first + lane) * wslices;
+            if (k < windows) {
+                const int64_t g = k * H + h;
+                hw_c = gt.c[g];
+                hw_T = gt.T[g];
+                hw_sq = gt.sq[g];
+            }
         }
     };
     constexpr int BR = 2 * RPBT_U;                              // rows of a batch
@@ -1194,6 +1232,14 @@ __global__ __launch_bounds__(256) void rpb_table_partial_kernel(FusedGroups gt, 
     // first batch of window cur.m and after among the 64 windows whose headers are loaded, or none.  (Loading
     // headers here, inside the pipeline, would put a wait for all loads in flight on every path.)
     auto seek = [&](Cursor cur) __attribute__((always_inline)) -> Cursor {
+        if constexpr (BY_TASKS) {
+            // the batch of lane cur.m - cur.m0, or none (a lane without a batch holds c = 0)
+            const int at = cur.m - cur.m0;
+            const int c_at = at < 64 ? __builtin_amdgcn_readlane(hw_c, at & 63) : 0;
+            if (c_at == 0) return Cursor{cur.m, cur.m0, 0, 1, 0, 0, 0, 0, false};
+            return Cursor{cur.m, cur.m0, 0, c_at, __builtin_amdgcn_readlane(hw_T, at & 63), __builtin_amdgcn_readlane(hw_sq, at & 63),
+                          __builtin_amdgcn_readlane(hw_ch, at & 63), __builtin_amdgcn_readlane(hw_ib, at & 63), true};
+        }
         for (;;) {
             if (cur.m - cur.m0 == 64)                           // a batch nobody adds, at a safe address
                 return Cursor{cur.m, cur.m0, cur.rot, 1, 0, 0, 0, 0, false};
@@ -1212,6 +1258,10 @@ __global__ __launch_bounds__(256) void rpb_table_partial_kernel(FusedGroups gt, 
     };
     auto advance = [&](Cursor cur) __attribute__((always_inline)) -> Cursor {
         if (!cur.valid) return cur;
+        if constexpr (BY_TASKS) {
+            ++cur.m;
+            return seek(cur);
+        }
         cur.ch += rsplit;
         cur = carry(cur);
         if (cur.ib < cur.c) return cur;
@@ -1271,7 +1321,7 @@ __global__ __launch_bounds__(256) void rpb_table_partial_kernel(FusedGroups gt, 
         });
     };
     int rot = rs;
-    for (int m0 = 0; ws + (int64_t)m0 * wslices < windows; m0 += 64) {
+    for (int m0 = 0; BY_TASKS ? (int64_t)m0 * slices + sl < bl.total : ws + (int64_t)m0 * wslices < windows; m0 += 64) {
         load_headers(m0);
         Cursor cur = seek(Cursor{m0, m0, rot, 1, 0, 0, 0, 0, true});
         Slot sa, sb, sc;
@@ -1720,6 +1770,48 @@ size_t sswin_bias_table_grad_workspace_bytes(int64_t G, int H, int table_rows) {
     return (size_t)wslices * rsplit * H * table_rows * sizeof(float) + 256;
 }
 
+// the two launches of the table gradient; bl == nullptr: batches from the group table
+static int launch_table_grad(const FusedGroups& gt, const BatchList* bl, int64_t G, const int32_t* tokens, int64_t N, int H, int n,
+                             const int32_t* code, int offset0, int table_rows, const float* ds, float* d_table, void* ws,
+                             size_t ws_bytes, hipStream_t s) {
+    SSWIN_CHECK(ws_bytes >= sswin_bias_table_grad_workspace_bytes(G, H, table_rows), "bias_table_grad: workspace too small");
+    const int64_t windows = G / H;
+    int wslices, rsplit;
+    table_grad_slices(windows, H, table_rows, &wslices, &rsplit);
+    if (bl) {
+        // dealt batches: a wavefront should have about six of them before it is worth its table (small inputs: 22 000
+        // voxels 18.5 -> 15 us with half the wavefronts; more wavefronts than the walking kernel's never paid)
+        const int per_head = (int)std::max<int64_t>(32, std::min<int64_t>((int64_t)wslices * rsplit, bl->total / 6));
+        wslices = per_head;
+        rsplit = 1;
+    }
+    const int slices = wslices * rsplit;
+    float* partial = static_cast<float*>(ws);
+    const int64_t waves = (int64_t)slices * H;
+    const int rows_pad = (table_rows + 31) / 32 * 32 + 32;  // 32 spare rows
+    const size_t lds = table_grad_lds(table_rows, n);
+    SSWIN_CHECK(lds <= 160 * 1024, "bias_table_grad: a table of %d rows needs %zu bytes of LDS (160 KB at most)", table_rows, lds);
+    if (lds > 64 * 1024) {
+        // more than the default 64 KB of dynamic LDS: asked for with every such launch (cheap, and correct for any
+        // number of host threads and devices)
+        const void* fn = bl ? reinterpret_cast<const void*>(rpb_table_partial_kernel<true>)
+                            : reinterpret_cast<const void*>(rpb_table_partial_kernel<false>);
+        const hipError_t e = hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        SSWIN_CHECK(e == hipSuccess, "bias_table_grad: the request for %zu bytes of LDS per workgroup was refused: %s", lds,
+                    hipGetErrorString(e));
+    }
+    const dim3 grid((unsigned)((waves + 3) / 4));
+    if (bl)
+        hipLaunchKernelGGL(rpb_table_partial_kernel<true>, grid, dim3(256), lds, s, gt, *bl, tokens + 3 * N, H,
+                           code, n, offset0, table_rows, rows_pad, ds, windows, wslices, rsplit, partial);
+    else
+        hipLaunchKernelGGL(rpb_table_partial_kernel<false>, grid, dim3(256), lds, s, gt, BatchList{}, tokens + 3 * N, H,
+                           code, n, offset0, table_rows, rows_pad, ds, windows, wslices, rsplit, partial);
+    hipLaunchKernelGGL(rpb_table_reduce_kernel, dim3((unsigned)((table_rows + 15) / 16), (unsigned)H), dim3(1024), 0, s,
+                       partial, slices, table_rows, H, d_table);
+    return launch_ok("bias table gradient");
+}
+
 int sswin_bias_table_grad(const int32_t* plan, int64_t g_cap, int64_t G, const int32_t* tokens, int64_t N, int H,
                           int n, const int32_t* code, int offset0, int table_rows, const float* ds, float* d_table,
                           void* ws, size_t ws_bytes, void* stream) {
@@ -1734,30 +1826,44 @@ int sswin_bias_table_grad(const int32_t* plan, int64_t g_cap, int64_t G, const i
         return launch_ok("bias_table_grad");
     }
     SSWIN_CHECK(plan && tokens && code && ds && ws, "bias_table_grad: null pointer");
-    SSWIN_CHECK(ws_bytes >= sswin_bias_table_grad_workspace_bytes(G, H, table_rows), "bias_table_grad: workspace too small");
-    const FusedGroups gt = groups_of(plan, g_cap, G);
-    const int64_t windows = G / H;
-    int wslices, rsplit;
-    table_grad_slices(windows, H, table_rows, &wslices, &rsplit);
-    const int slices = wslices * rsplit;
-    float* partial = static_cast<float*>(ws);
-    const int64_t waves = (int64_t)slices * H;
-    const int rows_pad = (table_rows + 31) / 32 * 32 + 32;  // 32 spare rows
-    const size_t lds = table_grad_lds(table_rows, n);
-    SSWIN_CHECK(lds <= 160 * 1024, "bias_table_grad: a table of %d rows needs %zu bytes of LDS (160 KB at most)", table_rows, lds);
-    if (lds > 64 * 1024) {
-        // more than the default 64 KB of dynamic LDS: asked for with every such launch (cheap, and correct for any
-        // number of host threads and devices)
-        const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(rpb_table_partial_kernel),
-                                                 hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        SSWIN_CHECK(e == hipSuccess, "bias_table_grad: the request for %zu bytes of LDS per workgroup was refused: %s", lds,
-                    hipGetErrorString(e));
+    return launch_table_grad(groups_of(plan, g_cap, G), nullptr, G, tokens, N, H, n, code, offset0, table_rows, ds, d_table, ws,
+                             ws_bytes, s);
+}
+
+int sswin_bias_table_grad_tasks(const int32_t* tasks, int64_t g_cap, const int64_t* bucket_counts, int64_t G,
+                                const int32_t* tokens, int64_t N, int H, int n, const int32_t* code, int offset0,
+                                int table_rows, const float* ds, float* d_table, void* ws, size_t ws_bytes, void* stream) {
+    SSWIN_CHECK(G >= 0 && G <= g_cap && H > 0 && n > 0 && n <= 128, "bias_table_grad_tasks: bad sizes");
+    SSWIN_CHECK(table_rows > 0 && table_rows <= RPBT_MAX_ROWS, "bias_table_grad_tasks: a table of %d rows is not supported (%d at most)",
+                table_rows, RPBT_MAX_ROWS);
+    SSWIN_CHECK(d_table && bucket_counts, "bias_table_grad_tasks: null pointer");
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (G == 0) {
+        zero_fill(d_table, (int64_t)table_rows * H, s);
+        return launch_ok("bias_table_grad_tasks");
     }
-    hipLaunchKernelGGL(rpb_table_partial_kernel, dim3((unsigned)((waves + 3) / 4)), dim3(256), lds, s, gt, tokens + 3 * N, H,
-                       code, n, offset0, table_rows, rows_pad, ds, windows, wslices, rsplit, partial);
-    hipLaunchKernelGGL(rpb_table_reduce_kernel, dim3((unsigned)((table_rows + 15) / 16), (unsigned)H), dim3(1024), 0, s,
-                       partial, slices, table_rows, H, d_table);
-    return launch_ok("bias table gradient");
+    SSWIN_CHECK(tasks && tokens && code && ds && ws, "bias_table_grad_tasks: null pointer");
+    int64_t groups = 0;
+    for (int b = 0; b < 4; ++b) {
+        SSWIN_CHECK(bucket_counts[b] >= 0 && bucket_counts[b] % H == 0, "bias_table_grad_tasks: bucket %d holds %lld groups, not a multiple of the %d heads",
+                    b, (long long)bucket_counts[b], H);
+        groups += bucket_counts[b];
+    }
+    SSWIN_CHECK(groups == G, "bias_table_grad_tasks: the buckets hold %lld groups, the plan %lld (windows of more than 128 tokens have no descriptor)",
+                (long long)groups, (long long)G);
+    BatchList bl;
+    bl.tasks = reinterpret_cast<const int4*>(tasks);
+    bl.g_cap = g_cap;
+    int64_t at = 0;
+    for (int b = 3; b >= 0; --b) {
+        bl.first[b] = (int)at;
+        at += bucket_counts[b] / H * (b + 1) * (b + 1);
+    }
+    SSWIN_CHECK(at < ((int64_t)1 << 31), "bias_table_grad_tasks: too many batches");
+    bl.total = (int)at;
+    // the group table is not read on this path: only its size G matters
+    const FusedGroups gt{nullptr, nullptr, nullptr, nullptr, nullptr, G};
+    return launch_table_grad(gt, &bl, G, tokens, N, H, n, code, offset0, table_rows, ds, d_table, ws, ws_bytes, s);
 }
 
 int sswin_bias_from_table(const float* table, int table_rows, int H, const int32_t* code, int offset0, int n, float* bias,

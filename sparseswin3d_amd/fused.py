@@ -207,9 +207,15 @@ def _bias_gradient(tp, H, d_s, bias_meta, table_index):
         d_bias32 = torch.empty(bias_shape, dtype=torch.float32, device=d)
         nbytes = lib.sswin_bias_table_grad_workspace_bytes(tp.G, H, rows)
         ws = torch.empty(int(nbytes), dtype=torch.uint8, device=d)
-        _lib.check(lib.sswin_bias_table_grad(_ptr(tp.plan), tp.g_cap, tp.G, _ptr(tp.tokens), tp.N, H, tp.n,
-                                             _ptr(table_index.code), table_index.offset0, rows, _ptr(d_s),
-                                             _ptr(d_bias32), _ptr(ws), nbytes, stream))
+        if tp.tasks is not None and tp.n <= 128 and sum(tp.bucket_counts) == tp.G:
+            # every group has a task descriptor: the batches of dS are dealt evenly from the descriptor lists
+            _lib.check(lib.sswin_bias_table_grad_tasks(_ptr(tp.tasks), tp.g_cap, tp.bucket_counts, tp.G, _ptr(tp.tokens), tp.N,
+                                                       H, tp.n, _ptr(table_index.code), table_index.offset0, rows,
+                                                       _ptr(d_s), _ptr(d_bias32), _ptr(ws), nbytes, stream))
+        else:
+            _lib.check(lib.sswin_bias_table_grad(_ptr(tp.plan), tp.g_cap, tp.G, _ptr(tp.tokens), tp.N, H, tp.n,
+                                                 _ptr(table_index.code), table_index.offset0, rows, _ptr(d_s),
+                                                 _ptr(d_bias32), _ptr(ws), nbytes, stream))
     return d_bias32.to(bias_dtype)
 
 

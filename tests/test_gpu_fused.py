@@ -425,6 +425,16 @@ def test_bias_table_gradient(mix, H):
     _lib.check(lib.sswin_bias_table_grad(_ptr(tp.plan), tp.g_cap, tp.G, _ptr(tp.tokens), tp.N, H, n, _ptr(ti.code),
                                          ti.offset0, rows, _ptr(ds_d), _ptr(out2), _ptr(ws), nbytes, stream))
     assert torch.equal(out, out2)                       # same bits on every run
+    # the same gradient with the batches dealt from the plan's task descriptors (what the module calls when every
+    # window holds at most 128 tokens): same reference, and the same bits on every run
+    res = []
+    for _ in range(2):
+        o = torch.full((rows, H), float("nan"), device="cuda")
+        _lib.check(lib.sswin_bias_table_grad_tasks(_ptr(tp.tasks), tp.g_cap, tp.bucket_counts, tp.G, _ptr(tp.tokens), tp.N, H, n,
+                                                   _ptr(ti.code), ti.offset0, rows, _ptr(ds_d), _ptr(o), _ptr(ws), nbytes, stream))
+        res.append(o)
+    close(res[0].cpu().numpy(), ref, 1e-5, "d table, batches from the task descriptors", mag=mag)
+    assert torch.equal(res[0], res[1])
 
 
 def test_bias_from_table_matches_the_gather():
