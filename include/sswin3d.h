@@ -328,7 +328,8 @@ typedef struct sswin_token_plan_desc {
 int sswin_token_plan_batch(const sswin_token_plan_desc* descs, int count, void* stream);
 
 /* Token tensors are dense [N, stride] arrays of `dtype`; element (voxel v, head h, channel ch) is
- * base[v*stride + col0 + h*hd + ch].  "sq" arrays are fp32 arrays of all [c x c] blocks.
+ * base[v*stride + col0 + h*hd + ch].  "sq" arrays are fp32 arrays of all [c x c] blocks; a window holds at most
+ * 16 384 tokens (a block is addressed with 32-bit byte offsets below 2^31).
  *
  * tokens x tokens -> sq: out[g][i][j] = sum_ch (scale_a * A[token i, ch]) * B[token j, ch].
  * With epilogue != 0 (the product S = Q K^T of swin3d_base.py:660-668): adds
