@@ -1140,10 +1140,11 @@ constexpr int RPBT_U = 16;                                      // steps of a ba
 //          windows among its rsplit members (each member walks over all windows of the slice).
 //   true:  from the task descriptors of a token plan, which list the groups by their number of 32-token tiles
 //          (fused TokenPlan, windows of at most 128 tokens).  The batches of a head, numbered bucket by bucket (16, 9,
-//          4 or 1 per group), are dealt to the head's wavefronts in turn: wavefront q adds the batches q, q + Q, ...,
-//          so every wavefront adds the same number of batches to within one (the slices of the group table differ by
-//          the sizes of the windows that fall to them: 1.6 x between the fullest slice and the mean on a room of
-//          112 000 voxels), and nothing is walked: lane l decodes the wavefront's l-th batch and loads its descriptor.
+//          4 or 1 per group), are cut into Q runs of equal length, one per wavefront of the head (consecutive
+//          batches: neighbouring blocks of dS, and the same descriptor for the batches of a group), so every
+//          wavefront adds the same number of batches (the slices of the group table differ by the sizes of the windows
+//          that fall to them: 1.6 x between the fullest slice and the mean on a room of 112 000 voxels), and nothing
+//          is walked: lane l decodes the l-th batch of the wavefront's run and loads its descriptor.
 struct BatchList {
     const int4* tasks;       // [4][g_cap] descriptors {T, c | head << 8, window, sq}, bucket b = groups of b + 1 tiles
     int64_t g_cap;
@@ -1178,12 +1179,13 @@ __global__ __launch_bounds__(256) void rpb_table_partial_kernel(FusedGroups gt, 
     // evens the load); the batches of its windows are dealt to the rsplit wavefronts of the slice.
     // The headers of 64 windows of the slice at a time sit in the lanes (lane l: the l-th of them).
     int hw_c = 0, hw_T = 0, hw_sq = 0, hw_ch = 0, hw_ib = 0;
+    const int per_wave = BY_TASKS ? (bl.total + slices - 1) / slices : 0;   // a wavefront's run of consecutive batches
     auto load_headers = [&](int m_first) __attribute__((always_inline)) {
         hw_c = 0;
         if constexpr (BY_TASKS) {
-            // batch number (m_first + lane) * slices + sl of head h -> bucket, group inside it, chunk and row block
-            const int64_t f64 = ((int64_t)m_first + lane) * slices + sl;
-            if (f64 < bl.total) {
+            // batch number sl * per_wave + m_first + lane of head h -> bucket, group inside it, chunk and row block
+            const int64_t f64 = sl * per_wave + m_first + lane;
+            if (m_first + lane < per_wave && f64 < bl.total) {
                 const int f = (int)f64;
                 int b = 3, r = f - bl.first[3];
                 if (f >= bl.first[2]) { b = 2; r = f - bl.first[2]; }
@@ -1321,7 +1323,7 @@ __global__ __launch_bounds__(256) void rpb_table_partial_kernel(FusedGroups gt, 
         });
     };
     int rot = rs;
-    for (int m0 = 0; BY_TASKS ? (int64_t)m0 * slices + sl < bl.total : ws + (int64_t)m0 * wslices < windows; m0 += 64) {
+    for (int m0 = 0; BY_TASKS ? m0 < per_wave && sl * per_wave + m0 < bl.total : ws + (int64_t)m0 * wslices < windows; m0 += 64) {
         load_headers(m0);
         Cursor cur = seek(Cursor{m0, m0, rot, 1, 0, 0, 0, 0, true});
         Slot sa, sb, sc;
