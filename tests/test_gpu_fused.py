@@ -473,3 +473,33 @@ def test_sums_over_nothing_are_zero():
     _lib.check(lib.sswin_bias_table_grad(None, 0, 0, None, 0, 3, 125, None, 0, 729, None, C.c_void_p(table.data_ptr()),
                                          None, 0, stream))
     assert torch.count_nonzero(table) == 0
+    table.fill_(7.0)
+    counts = (C.c_int64 * 4)(0, 0, 0, 0)
+    _lib.check(lib.sswin_bias_table_grad_tasks(None, 0, counts, 0, None, 0, 3, 125, None, 0, 729, None,
+                                               C.c_void_p(table.data_ptr()), None, 0, stream))
+    assert torch.count_nonzero(table) == 0
+    # nothing to do for a plan without groups: no launch, no pointer touched
+    _lib.check(lib.sswin_group_softmax(0, None, 0, 0, 0, 3, 1, None, None, None, stream))
+    _lib.check(lib.sswin_fused_score_grad(0, None, 0, 0, None, 0, 3, 16, 1, None, 0, 0, None, 0, 0, None, 0, 0, None, None, stream))
+
+
+def test_entry_points_of_the_fused_path_reject_what_they_cannot_do():
+    """Error behaviour of the entry points that take sizes the kernels are built around."""
+    import ctypes as C
+    from sparseswin3d_amd import _lib
+    from sparseswin3d_amd.fused import TokenPlan, _ptr
+    lib = _lib.load()
+    stream = C.c_void_p(torch.cuda.current_stream().cuda_stream)
+    rng = np.random.default_rng(1)
+    ind = ragged_window_indices(rng, [3, 40, 7], 125)
+    tp = TokenPlan(torch.from_numpy(ind).cuda(), 3, 125, 2)
+    x = torch.zeros(tp.A, device="cuda")
+    with pytest.raises(RuntimeError, match="384 at most"):
+        _lib.check(lib.sswin_group_softmax(0, _ptr(tp.plan), tp.g_cap, tp.G, tp.N, tp.H, 385, _ptr(x), None, _ptr(x), stream))
+    with pytest.raises(RuntimeError, match="null pointer"):
+        _lib.check(lib.sswin_group_softmax(1, _ptr(tp.plan), tp.g_cap, tp.G, tp.N, tp.H, tp.c_max, _ptr(x), None, _ptr(x), stream))
+    table = torch.zeros(729, 2, device="cuda")
+    short = (C.c_int64 * 4)(2, 0, 0, 0)                      # fewer groups in the buckets than the plan holds
+    with pytest.raises(RuntimeError, match="have no descriptor"):
+        _lib.check(lib.sswin_bias_table_grad_tasks(_ptr(tp.tasks), tp.g_cap, short, tp.G, _ptr(tp.tokens), tp.N, 2, 125,
+                                                   _ptr(x), 0, 729, _ptr(x), _ptr(table), _ptr(x), 1 << 30, stream))
