@@ -519,6 +519,22 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
             row_c = a_in ? (uint32_t)vox_i * c_pitch : BUF_OUTSIDE;
         }
 
+        // scores: the bias values of the 16 rows a lane stores are gathered here, beside the row loads (behind the matrix
+        // steps they were one more memory round trip per task); position and mask region of a row come from its row
+        // lane in one cross-lane read
+        float bv[16];
+        int m_i[16];
+        if (EPI == SQ_SCORES) {
+            const float* brow = bias + (int64_t)h * n * n + pos_j;
+            const int pm_a = pos_a | (m_a << 16);                   // positions stay below 2^15, regions below 2^7
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {                          // all lanes take part in the cross-lane reads
+                const int pm = __shfl(pm_a, acc_row(r, half), 64);
+                bv[r] = brow[(pm & 0xffff) * n];
+                m_i[r] = pm >> 16;
+            }
+        }
+
         f32x16 acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
         for (int kc = 0; kc < hd; kc += 32) {
             // the channels of a chunk are split evenly between the two lane halves: a head of 16 channels takes
@@ -582,22 +598,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
         } else {
             const __amdgpu_buffer_rsrc_t ro = buf_of(out + k.sq, (uint32_t)(c * c) * 4u);
             const __amdgpu_buffer_rsrc_t rr = buf_of(row_ids ? row_ids + k.sq : nullptr, row_ids ? (uint32_t)(c * c) * 4u : 0u);
-            const float* brow = EPI ? bias + (int64_t)h * n * n + pos_j : nullptr;
             const int rid0 = H * Tk + h * c + bi * 32 + 4 * half;
-            // bias values of the 16 rows are gathered before any of them is used, so that the
-            // gather latencies overlap instead of adding up
-            float bv[16];
-            int m_i[16];
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                bv[r] = 0.f;
-                m_i[r] = 0;
-                if (EPI) {                                          // all lanes take part in the shuffles
-                    const int il = acc_row(r, half);
-                    bv[r] = brow[__shfl(pos_a, il, 64) * n];
-                    if (mask) m_i[r] = __shfl(m_a, il, 64);
-                }
-            }
 #pragma unroll
             for (int r = 0; r < 16; ++r) {
                 const int row = 8 * (r >> 2) + (r & 3);             // + 4 * half: the row of the block
