@@ -79,10 +79,10 @@ struct GroupTable {
 #define BP_BUFFERED 1
 #endif
 #ifndef BP_WAVES_FWD
-#define BP_WAVES_FWD 4
+#define BP_WAVES_FWD 5
 #endif
 template <typename T, int MODE, bool EMIT>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(MODE >= 2 ? BP_WAVES : BP_WAVES_FWD, MODE >= 2 ? BP_WAVES : BP_WAVES_FWD))) void block_product_mfma_kernel(const T* __restrict__ m1, const T* __restrict__ m2,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(EMIT ? 4 : MODE >= 2 ? BP_WAVES : BP_WAVES_FWD, EMIT ? 4 : MODE >= 2 ? BP_WAVES : BP_WAVES_FWD))) void block_product_mfma_kernel(const T* __restrict__ m1, const T* __restrict__ m2,
                                                                  GroupTable gt, int64_t G, int C,
                                                                  const int32_t* __restrict__ tok_pos,
                                                                  T* __restrict__ out, int32_t* __restrict__ out_idx,
