@@ -24,6 +24,13 @@
 #include "scan.hpp"
 #include "sswin_common.hpp"
 
+#ifndef FUSED_TOK_WAVES
+#define FUSED_TOK_WAVES 5
+#endif
+#ifndef FUSED_SQ_PLAIN_WAVES
+#define FUSED_SQ_PLAIN_WAVES 4
+#endif
+
 namespace sswin {
 
 constexpr int FUSED_GROUPS_PER_WG = 4;
@@ -470,7 +477,7 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t head_rows(const TokenTensor& t
 enum { SQ_PLAIN = 0, SQ_SCORES = 1, SQ_SCORE_GRAD = 2 };
 
 template <typename T, int EPI>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void fused_sq_kernel(FusedGroups gt, const int32_t* __restrict__ order,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(EPI == SQ_PLAIN ? FUSED_SQ_PLAIN_WAVES : 4, EPI == SQ_PLAIN ? FUSED_SQ_PLAIN_WAVES : 4))) void fused_sq_kernel(FusedGroups gt, const int32_t* __restrict__ order,
                                                        const int32_t* __restrict__ tok_pos, int H, int hd,
                                                        TokenTensor ta, TokenTensor tb, TokenTensor tc, uint32_t a_span, uint32_t b_span,
                                                        uint32_t c_span, float scale_a,
@@ -620,7 +627,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) voi
 //   A_KMAJOR = true : A(i, k) = sq[k*c + i]   (dV = P^T dO, dK = dS^T Q)
 // ------------------------------------------------------------------------------------------
 template <typename T, bool A_KMAJOR>
-__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(4, 4))) void fused_tok_kernel(FusedGroups gt, const int32_t* __restrict__ order, int hd,
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(FUSED_TOK_WAVES, FUSED_TOK_WAVES))) void fused_tok_kernel(FusedGroups gt, const int32_t* __restrict__ order, int hd,
                                                         const float* __restrict__ sq, TokenTensor tb,
                                                         TokenTensor to, uint32_t b_span, uint32_t o_span, float scale_out) {
     constexpr uint32_t ES = (uint32_t)sizeof(T);
