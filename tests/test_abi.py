@@ -30,6 +30,48 @@ def test_library_exports_every_declared_symbol():
     assert lib.sswin_abi_version() == _lib.ABI_VERSION
 
 
+def declared_arguments():
+    """name -> list of argument kinds ("ptr", "i32", "i64", "size", "f32", "f64") parsed from the header."""
+    text = open(os.path.join(ROOT, "include", "sswin3d.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    out = {}
+    for m in re.finditer(r"\b(?:int|size_t|const char\s*\*)\s+(sswin_[a-z0-9_]+)\s*\(([^;{]*?)\)\s*;", text, flags=re.S):
+        name, args = m.group(1), " ".join(m.group(2).split())
+        kinds = []
+        if args not in ("", "void"):
+            for a in args.split(","):
+                a = a.strip()
+                if "*" in a:
+                    kinds.append("ptr")
+                elif a.startswith("int64_t"):
+                    kinds.append("i64")
+                elif a.startswith("size_t"):
+                    kinds.append("size")
+                elif a.startswith("float"):
+                    kinds.append("f32")
+                elif a.startswith("double"):
+                    kinds.append("f64")
+                elif a.startswith("int"):
+                    kinds.append("i32")
+                else:
+                    kinds.append(a)
+        out[name] = kinds
+    return out
+
+
+def test_ctypes_signatures_match_the_header():
+    """Every argument list of the binding has the header's length and kinds: a size added on one side only would
+    shift every later argument."""
+    from sparseswin3d_amd import _lib
+    kind_of = {ctypes.c_void_p: "ptr", ctypes.c_char_p: "ptr", ctypes.c_int32: "i32", ctypes.c_int: "i32", ctypes.c_int64: "i64",
+               ctypes.c_size_t: "size", ctypes.c_float: "f32", ctypes.c_double: "f64"}
+    declared = declared_arguments()
+    assert sorted(declared) == declared_symbols()
+    for name, (_, argtypes) in _lib.SIGNATURES.items():
+        bound = ["ptr" if isinstance(t, type) and issubclass(t, ctypes._Pointer) else kind_of.get(t, str(t)) for t in argtypes]
+        assert bound == declared[name], f"{name}: binding {bound} against header {declared[name]}"
+
+
 def test_argument_errors_are_reported_without_a_gpu():
     from sparseswin3d_amd import _lib
     lib = _lib.load()
