@@ -280,6 +280,7 @@ OPERATOR_LAUNCHES = {
     "operand_copy Q/V order, voxel rows -> operand": ("sswin_operand_copy", (0, 0, 1)),
     "block_matmul q_k, values": ("sswin_block_matmul", (0, 0)),
     "bias + mask add, one pass [A]": ("sswin_group_add_table_bias_mask", None),
+    "bias table gradient (batches from the token plan)": ("sswin_bias_table_grad_tasks", None),
     "bias table gradient from the product's groups": ("sswin_bias_table_grad", None),
     "softmax rows from the group sizes [A]": ("sswin_softmax_rows_from_counts", None),
     "softmax_last_dim_forward": ("sswin_softmax_last_dim_forward", None),
@@ -410,6 +411,7 @@ def kernel_table(wl, reps=20, only=None):
         n_table_o = int(wl["blocks"][0]["attn"].relative_position_bias_table.shape[0])
         table_o = wl["blocks"][0]["attn"].relative_position_bias_table.detach().float().contiguous()
         ti_o = F.BiasTableIndex.build(relative_position_index_3d(wl["blocks"][0]["attn"].window_size).to(dev), n_table_o)
+        dealt_o = tp.tasks is not None and b["n"] <= 128 and sum(tp.bucket_counts) == tp.G   # every window has a task descriptor
 
         entries = [
             # name, callable, algorithmic bytes, calls per attention fwd+bwd of the module (0: not on the module's path)
@@ -434,7 +436,9 @@ def kernel_table(wl, reps=20, only=None):
             ("block_matmul q_k (values + index matrix)", mm(0, q.values, kt.values, q.indices, out_s, out_si, A), 2 * s * E + (s + 16) * A + 4 * G, 0),
             ("bias + mask add, one pass [A]", lambda: ops.group_add_table_bias_mask(s_val, row_pos, gp, b["n"], table_o, ti_o.code, ti_o.offset0, mask), 2 * s * A + 8 * G, 1),
             ("bias + mask add from a gathered [H,n,n] bias", lambda: ops.group_add_bias_mask(s_val, row_pos, gp, b["n"], bias_d, mask), 2 * s * A + 8 * G, 0),
-            ("bias table gradient from the product's groups", lambda: ops.group_bias_table_grad(g_s, row_pos, gp, H, b["n"], ti_o.code, ti_o.offset0, n_table_o), 4 * A, 1),
+            # what the module's backward calls: with a token plan at hand the batches are dealt from its descriptors
+            ("bias table gradient (batches from the token plan)", lambda: F._bias_gradient(tp, H, g_s, (torch.float32, (n_table_o, H)), ti_o), 4 * A, int(dealt_o)),
+            ("bias table gradient from the product's groups", lambda: ops.group_bias_table_grad(g_s, row_pos, gp, H, b["n"], ti_o.code, ti_o.offset0, n_table_o), 4 * A, int(not dealt_o)),
             ("softmax rows from the group sizes [A]", lambda: ops.softmax_rows_from_counts(c, A), 4 * A + 12 * G, 1),
             ("flatten_indices [3,A] (generic softmax rows)", lambda: ops.flatten_indices(s_idx[:3], s_shape[:3]), 16 * A, 0),
             ("unique_consecutive_indices [A] (generic softmax rows)", lambda: ops.unique_consecutive_indices(flat), 8 * A, 0),

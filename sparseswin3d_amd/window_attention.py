@@ -399,13 +399,15 @@ class _GroupBiasMask(Function):
     gathers, and an ``index_add`` into the dense bias)."""
 
     @staticmethod
-    def forward(ctx, values, table, row_pos, gp, n, mask, table_index):
-        # row_pos: window position of every token row in group order (int32 [sum c])
+    def forward(ctx, values, table, row_pos, gp, n, mask, table_index, token_plan=None):
+        # row_pos: window position of every token row in group order (int32 [sum c]); token_plan: the TokenPlan the
+        # product's group table was taken from, if any (its task descriptors let the backward deal the work evenly)
         idx = row_pos
         num_heads = table.shape[1]
         table32 = table.detach().to(torch.float32).contiguous()
         ctx.save_for_backward(idx)
         ctx.meta = (gp, n, table_index, table.shape[0], num_heads, table.dtype)
+        ctx.token_plan = token_plan
         if table.shape[0] < (1 << 15):
             # the kernel reads the table itself (a few KB; the gathered [H, n, n] bias of 7^3 windows is 1.4 MB)
             return ops.group_add_table_bias_mask(values, idx, gp, n, table32, table_index.code, table_index.offset0, mask)
@@ -426,12 +428,20 @@ class _GroupBiasMask(Function):
         gp, n, table_index, table_rows, num_heads, table_dtype = ctx.meta
         d_table = None
         if ctx.needs_input_grad[1]:
-            d_table = ops.group_bias_table_grad(grad.float(), idx, gp, num_heads, n, table_index.code, table_index.offset0,
-                                                table_rows).to(table_dtype)
-        return grad, d_table, None, None, None, None, None
+            from . import fused
+            tp = ctx.token_plan
+            if tp is not None and tp.H == num_heads and tp.A == grad.numel():
+                # the values of the product lie in the plan's group order: the fused path's table gradient applies
+                # as it is (batches dealt from the task descriptors where every window has one)
+                d_table = fused._bias_gradient(tp, num_heads, grad.float().contiguous(), (table_dtype, (table_rows, num_heads)),
+                                               table_index)
+            else:
+                d_table = ops.group_bias_table_grad(grad.float(), idx, gp, num_heads, n, table_index.code,
+                                                    table_index.offset0, table_rows).to(table_dtype)
+        return grad, d_table, None, None, None, None, None, None
 
 
-def sp_add_table_bias_and_mask(sparse: SparseTensor, table: torch.Tensor, table_index, mask) -> SparseTensor:
+def sp_add_table_bias_and_mask(sparse: SparseTensor, table: torch.Tensor, table_index, mask, token_plan=None) -> SparseTensor:
     """``sp_add_rpb`` with the bias gathered from ``table`` [rows, H], then ``sp_add_mask``, in one pass (a 'q_k'
     product with its group sizes attached, int8 mask or None); None if the input is not of that kind."""
     if sparse.group_counts is None or table_index is None or (mask is not None and mask.dtype != torch.int8):
@@ -441,7 +451,7 @@ def sp_add_table_bias_and_mask(sparse: SparseTensor, table: torch.Tensor, table_
     if gp is None or gp.c_max > 512 or n > 384:
         return None
     row_pos = sparse.row_positions if sparse.row_positions is not None else ops.group_row_positions(sparse.indices, gp)
-    out = _GroupBiasMask.apply(sparse.values, table, row_pos, gp, n, mask, table_index)
+    out = _GroupBiasMask.apply(sparse.values, table, row_pos, gp, n, mask, table_index, token_plan)
     return SparseTensor(sparse.index_source(), out, sparse.shape, sparse.group_counts, row_pos)
 
 
@@ -766,7 +776,7 @@ class WindowAttentionSparse(nn.Module):
             return replace_feature(x, self.proj_drop(tall_linear(x.features, self.proj)))
         q, k_t, v = qkv_sparse_cuda(qkv, x.indices, b, n, plan, q_scale=self.scale)         # q = q * self.scale
         attn = spspmm_block_naive(q, k_t, "q_k")
-        biased = sp_add_table_bias_and_mask(attn, self.relative_position_bias_table, self._table_index(n), mask)
+        biased = sp_add_table_bias_and_mask(attn, self.relative_position_bias_table, self._table_index(n), mask, plan)
         if biased is not None:
             attn = biased
         else:
