@@ -1172,11 +1172,11 @@ __global__ __launch_bounds__(256) void rpb_table_partial_kernel(FusedGroups gt, 
     int32_t* code_lds = reinterpret_cast<int32_t*>(rpbt_lds + 8 * rows_pad);
     for (int e = threadIdx.x; e < n; e += 256) code_lds[e] = code[e];
     __syncthreads();
-    const int64_t p = (int64_t)blockIdx.x * 4 + wave;           // wavefront id = s * H + h
-    const int slices = wslices * rsplit;
-    if (p >= (int64_t)slices * H) return;
-    const int h = (int)(p % H);
-    const int64_t sl = p / H;
+    const int64_t p = (int64_t)blockIdx.x * 4 + wave;           // wavefront id = h * slices + sl
+    const int slices = wslices * rsplit;                        // a multiple of four: the wavefronts of a workgroup share a head
+    if (p >= (int64_t)slices * H) return;                       // (the whole workgroup then)
+    const int h = (int)(p / slices);
+    const int64_t sl = p % slices;
     const int64_t ws = sl % wslices;                            // windows ws, ws + wslices, ...
     const int rs = (int)(sl / wslices);                         // which of the rsplit wavefronts of this window slice
     float* tables = rpbt_lds + wave * 2 * rows_pad;
@@ -1355,9 +1355,16 @@ __global__ __launch_bounds__(256) void rpb_table_partial_kernel(FusedGroups gt, 
         }
         rot = cur.rot;
     }
-    __builtin_amdgcn_wave_barrier();
-    float* out = partial + ((int64_t)h * slices + sl) * rows;
-    for (int e = lane; e < rows; e += 64) out[e] = tables[e] + tables[rows_pad + e];
+    // the eight tables of the workgroup (four wavefronts, two halves each) are one head's: summed here in a fixed
+    // order, so a quarter of the partial tables reaches memory and the reduction
+    __syncthreads();
+    float* out = partial + ((int64_t)h * (slices / 4) + sl / 4) * rows;
+    for (int e = threadIdx.x; e < rows; e += 256) {
+        float total = 0.f;
+#pragma unroll
+        for (int t = 0; t < 8; ++t) total += rpbt_lds[t * rows_pad + e];
+        out[e] = total;
+    }
 }
 
 // d_table[row, h] = sum over slices of partial[h][slice][row].  One workgroup per 16 table rows
@@ -1792,7 +1799,7 @@ static int launch_table_grad(const FusedGroups& gt, const BatchList* bl, int64_t
         // dealt batches: a wavefront should have about six of them before it is worth its table (small inputs: 22 000
         // voxels 18.5 -> 15 us with half the wavefronts; more wavefronts than the walking kernel's never paid)
         const int per_head = (int)std::max<int64_t>(32, std::min<int64_t>((int64_t)wslices * rsplit, bl->total / 6));
-        wslices = per_head;
+        wslices = (per_head + 3) / 4 * 4;                          // whole workgroups per head
         rsplit = 1;
     }
     const int slices = wslices * rsplit;
@@ -1818,7 +1825,7 @@ static int launch_table_grad(const FusedGroups& gt, const BatchList* bl, int64_t
         hipLaunchKernelGGL(rpb_table_partial_kernel<false>, grid, dim3(256), lds, s, gt, BatchList{}, tokens + 3 * N, H,
                            code, n, offset0, table_rows, rows_pad, ds, windows, wslices, rsplit, partial);
     hipLaunchKernelGGL(rpb_table_reduce_kernel, dim3((unsigned)((table_rows + 15) / 16), (unsigned)H), dim3(1024), 0, s,
-                       partial, slices, table_rows, H, d_table);
+                       partial, slices / 4, table_rows, H, d_table);
     return launch_ok("bias table gradient");
 }
 
